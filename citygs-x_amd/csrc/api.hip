@@ -1,0 +1,695 @@
+// C ABI of libgsrast.so (declarations and contracts: include/gsrast.h).
+// Host-side orchestration only; kernels live in the other translation units.
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include <map>
+#include <string>
+#include <vector>
+
+#include "../../include/gsrast.h"
+#include "gs_common.h"
+#include "gs_kernels.h"
+
+namespace gs {
+
+static thread_local char g_err[512] = "";
+
+void set_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+}
+
+int check_launch(const char* what, hipStream_t stream, bool sync) {
+  hipError_t e = hipGetLastError();
+  if (e == hipSuccess && sync) {
+    e = hipStreamSynchronize(stream);
+    if (e == hipSuccess) e = hipGetLastError();
+  }
+  if (e != hipSuccess) {
+    set_error("%s: %s", what, hipGetErrorString(e));
+    return 1;
+  }
+  return 0;
+}
+
+// Optional per-stage GPU timing (the role of MyTimerOnGPU,
+// cuda_rasterizer/timers.cu:11-79): when enabled, every stage of the composite
+// entry points is bracketed by an event pair on its stream; pairs are resolved
+// only when the caller collects them, so enabling it adds no synchronisation.
+// Process-wide and not thread safe: meant for benchmarks and profiling.
+struct StageClock {
+  struct Rec {
+    const char* name;
+    hipEvent_t a, b;
+  };
+  bool enabled = false;
+  std::vector<hipEvent_t> pool;
+  std::vector<Rec> pending;
+  hipEvent_t take() {
+    if (!pool.empty()) {
+      hipEvent_t e = pool.back();
+      pool.pop_back();
+      return e;
+    }
+    hipEvent_t e = nullptr;
+    if (hipEventCreate(&e) != hipSuccess) return nullptr;
+    return e;
+  }
+  void begin(const char* name, hipStream_t s) {
+    if (!enabled) return;
+    Rec r{name, take(), take()};
+    if (!r.a || !r.b) return;
+    (void)hipEventRecord(r.a, s);
+    pending.push_back(r);
+  }
+  void end(hipStream_t s) {
+    if (!enabled || pending.empty()) return;
+    (void)hipEventRecord(pending.back().b, s);
+  }
+};
+static StageClock g_clock;
+
+struct StageScope {
+  hipStream_t s;
+  StageScope(const char* name, hipStream_t stream) : s(stream) { g_clock.begin(name, s); }
+  ~StageScope() { g_clock.end(s); }
+};
+
+namespace {
+
+inline char* align_ptr(const char* p, size_t a) {
+  return (char*)(((uintptr_t)p + a - 1) / a * a);
+}
+
+inline void tile_grid(int W, int H, int& gx, int& gy) {
+  gx = (W + GS_TILE_X - 1) / GS_TILE_X;
+  gy = (H + GS_TILE_Y - 1) / GS_TILE_Y;
+}
+
+struct ImageLayout {
+  size_t accum_alpha, n_contrib, n_contrib2loss, ranges, total;
+};
+ImageLayout image_layout(int W, int H) {
+  ImageLayout L;
+  const size_t N = (size_t)W * H;
+  int gx, gy;
+  tile_grid(W, H, gx, gy);
+  size_t off = 0;
+  auto take = [&](size_t b) { size_t o = off; off += align_up(b, 256); return o; };
+  L.accum_alpha = take(N * 4);
+  L.n_contrib = take(N * 4);
+  L.n_contrib2loss = take(N * 4);
+  L.ranges = take((size_t)gx * gy * 8);
+  L.total = off + 256;
+  return L;
+}
+
+struct GeometryLayout {
+  size_t tiles_touched, point_offsets, scan_temp, total;
+};
+GeometryLayout geometry_layout(int P) {
+  GeometryLayout L;
+  const size_t n = (size_t)(P > 0 ? P : 1);
+  size_t off = 0;
+  auto take = [&](size_t b) { size_t o = off; off += align_up(b, 256); return o; };
+  L.tiles_touched = take(n * 4);
+  L.point_offsets = take(n * 4);
+  L.scan_temp = take(scan_temp_bytes((int64_t)n));
+  L.total = off + 256;
+  return L;
+}
+
+struct BinningLayout {
+  size_t point_list, keys, point_list_unsorted, keys_unsorted, sort_temp, total;
+};
+BinningLayout binning_layout(int64_t R) {
+  BinningLayout L;
+  const size_t n = (size_t)(R > 0 ? R : 1);
+  size_t off = 0;
+  auto take = [&](size_t b) { size_t o = off; off += align_up(b, 256); return o; };
+  L.point_list = take(n * 4);
+  L.keys = take(n * 8);
+  L.point_list_unsorted = take(n * 4);
+  L.keys_unsorted = take(n * 8);
+  L.sort_temp = take(sort_temp_bytes((int64_t)n));
+  L.total = off + 256;
+  return L;
+}
+
+int sort_end_bit(int W, int H) {
+  int gx, gy;
+  tile_grid(W, H, gx, gy);
+  return 32 + (int)gs_higher_msb((uint32_t)(gx * gy));
+}
+
+struct EventTimer {
+  hipEvent_t a = nullptr, b = nullptr;
+  bool on = false;
+  int begin(bool enable, hipStream_t s) {
+    on = enable;
+    if (!on) return 0;
+    GS_HIP_TRY(hipEventCreate(&a));
+    GS_HIP_TRY(hipEventCreate(&b));
+    GS_HIP_TRY(hipEventRecord(a, s));
+    return 0;
+  }
+  int end(hipStream_t s, float* ms) {
+    if (!on) return 0;
+    GS_HIP_TRY(hipEventRecord(b, s));
+    GS_HIP_TRY(hipEventSynchronize(b));
+    GS_HIP_TRY(hipEventElapsedTime(ms, a, b));
+    return 0;
+  }
+  ~EventTimer() {
+    if (a) (void)hipEventDestroy(a);
+    if (b) (void)hipEventDestroy(b);
+  }
+};
+
+#define GS_REQUIRE(cond, msg)        \
+  do {                               \
+    if (!(cond)) {                   \
+      gs::set_error("%s", msg);      \
+      return 1;                      \
+    }                                \
+  } while (0)
+
+}  // namespace
+}  // namespace gs
+
+using namespace gs;
+
+extern "C" {
+
+const char* gs_last_error(void) { return g_err; }
+
+int gs_get_block_xy(int* bx, int* by, int* one_dim) {
+  GS_REQUIRE(bx && by && one_dim, "gs_get_block_xy: null output");
+  *bx = GS_TILE_X;
+  *by = GS_TILE_Y;
+  *one_dim = GS_BLOCK_1D;
+  return 0;
+}
+
+uint32_t gs_higher_msb(uint32_t n) {
+  // Smallest b with n < 2^b found by bisection from 16, as the reference's
+  // host helper does; equals bit_length(n) for n >= 1 and 1 for n == 0.
+  uint32_t msb = sizeof(n) * 4;
+  uint32_t step = msb;
+  while (step > 1) {
+    step /= 2;
+    if (n >> msb)
+      msb += step;
+    else
+      msb -= step;
+  }
+  if (n >> msb) msb++;
+  return msb;
+}
+
+int gs_mark_visible(int P, const float* means3D, const float* viewmatrix, const float* projmatrix, uint8_t* present,
+                    gs_stream_t stream) {
+  (void)projmatrix;
+  GS_REQUIRE(P >= 0, "gs_mark_visible: negative P");
+  if (P == 0) return 0;
+  GS_REQUIRE(means3D && viewmatrix && present, "gs_mark_visible: null pointer");
+  launch_mark_visible(P, means3D, viewmatrix, present, (hipStream_t)stream);
+  return check_launch("mark_visible", (hipStream_t)stream, false);
+}
+
+int gs_visible_filter(int P, int M, int width, int height, const float* means3D, const float* scales,
+                      float scale_modifier, const float* rotations, const float* cov3D_precomp,
+                      const float* viewmatrix, const float* projmatrix, float tan_fovx, float tan_fovy,
+                      int prefiltered, int* radii, int debug, gs_stream_t stream) {
+  (void)M;
+  (void)prefiltered;
+  GS_REQUIRE(P >= 0 && width > 0 && height > 0, "gs_visible_filter: bad sizes");
+  if (P == 0) return 0;
+  GS_REQUIRE(means3D && viewmatrix && projmatrix && radii, "gs_visible_filter: null pointer");
+  GS_REQUIRE(cov3D_precomp || (scales && rotations),
+             "gs_visible_filter: need scales+rotations or a precomputed 3D covariance");
+  {
+    StageScope _t("visible_filter", (hipStream_t)stream);
+    launch_visible_filter(P, means3D, scales, scale_modifier, rotations, cov3D_precomp, viewmatrix, projmatrix, width,
+                        height, tan_fovx, tan_fovy, radii, (hipStream_t)stream);
+  }
+  return check_launch("visible_filter", (hipStream_t)stream, debug != 0);
+}
+
+int gs_preprocess_forward(float* means2D, float* depths, int* radii, float* cov3D, float* conic_opacity, float* rgb,
+                          uint8_t* clamped, uint32_t* tiles_touched, int P, int D, int M, int width, int height,
+                          const float* means3D, const float* scales, const float* rotations, const float* shs,
+                          const float* opacities, float scale_modifier, const float* viewmatrix,
+                          const float* projmatrix, const float* cam_pos, float tan_fovx, float tan_fovy,
+                          int prefiltered, int debug, gs_stream_t stream) {
+  (void)prefiltered;
+  GS_REQUIRE(P >= 0 && width > 0 && height > 0, "gs_preprocess_forward: bad sizes");
+  if (P == 0) return 0;
+  GS_REQUIRE(means2D && depths && radii && cov3D && conic_opacity && rgb && clamped,
+             "gs_preprocess_forward: null output");
+  GS_REQUIRE(means3D && scales && rotations && opacities && viewmatrix && projmatrix,
+             "gs_preprocess_forward: null input");
+  const bool sh_mode = shs != nullptr && M > 0;
+  GS_REQUIRE(!sh_mode || (cam_pos != nullptr && D >= 0 && D <= 3 && M >= (D + 1) * (D + 1) && M <= 16),
+             "gs_preprocess_forward: SH mode needs cam_pos, 0<=D<=3 and (D+1)^2 <= M <= 16");
+  PreprocessFwdArgs a;
+  a.P = P; a.D = D; a.M = sh_mode ? M : 0; a.W = width; a.H = height;
+  a.means3D = means3D; a.scales = scales; a.rotations = rotations; a.opacities = opacities;
+  a.shs = sh_mode ? shs : nullptr;
+  a.scale_modifier = scale_modifier;
+  a.viewmatrix = viewmatrix; a.projmatrix = projmatrix; a.campos = cam_pos;
+  a.tanx = tan_fovx; a.tany = tan_fovy;
+  a.radii = radii; a.means2D = means2D; a.depths = depths; a.cov3D = cov3D; a.conic_opacity = conic_opacity;
+  a.rgb = rgb; a.clamped = clamped; a.tiles_touched = tiles_touched;
+  {
+    StageScope _t("preprocess_fwd", (hipStream_t)stream);
+    launch_preprocess_fwd(a, (hipStream_t)stream);
+  }
+  return check_launch("preprocess_forward", (hipStream_t)stream, debug != 0);
+}
+
+int gs_preprocess_backward(const int* radii, const float* cov3D, const uint8_t* clamped, int P, int D, int M,
+                           int width, int height, const float* means3D, const float* scales, const float* rotations,
+                           const float* shs, float scale_modifier, const float* viewmatrix, const float* projmatrix,
+                           const float* campos, float tan_fovx, float tan_fovy, const float* dL_dmean2D,
+                           int mean2D_stride, const float* dL_dconic_opacity, const float* dL_dcolor,
+                           float* dL_dmean3D, float* dL_dcov3D, float* dL_dscale, float* dL_drot, float* dL_dsh,
+                           float* dL_dopacity, int debug, gs_stream_t stream) {
+  GS_REQUIRE(P >= 0 && width > 0 && height > 0, "gs_preprocess_backward: bad sizes");
+  if (P == 0) return 0;
+  GS_REQUIRE(radii && cov3D && means3D && viewmatrix && projmatrix && dL_dmean2D && dL_dconic_opacity && dL_dmean3D,
+             "gs_preprocess_backward: null pointer");
+  GS_REQUIRE(mean2D_stride == 2 || mean2D_stride == 3, "gs_preprocess_backward: mean2D_stride must be 2 or 3");
+  GS_REQUIRE((scales == nullptr) == (rotations == nullptr), "gs_preprocess_backward: scales and rotations go together");
+  GS_REQUIRE(!scales || (dL_dscale && dL_drot), "gs_preprocess_backward: null scale/rotation gradient");
+  const bool sh_mode = shs != nullptr && M > 0 && dL_dsh != nullptr;
+  GS_REQUIRE(!sh_mode || (campos && clamped && dL_dcolor && D >= 0 && D <= 3 && M >= (D + 1) * (D + 1) && M <= 16),
+             "gs_preprocess_backward: SH mode needs campos, clamped, dL_dcolor and (D+1)^2 <= M <= 16");
+  PreprocessBwdArgs a;
+  a.P = P; a.D = D; a.M = sh_mode ? M : 0; a.W = width; a.H = height;
+  a.means3D = means3D; a.radii = radii; a.shs = sh_mode ? shs : nullptr; a.clamped = clamped;
+  a.scales = scales; a.rotations = rotations; a.scale_modifier = scale_modifier;
+  a.cov3D = cov3D; a.viewmatrix = viewmatrix; a.projmatrix = projmatrix; a.campos = campos;
+  a.tanx = tan_fovx; a.tany = tan_fovy;
+  a.dL_dmean2D = dL_dmean2D; a.mean2D_stride = mean2D_stride; a.dL_dconic_opacity = dL_dconic_opacity;
+  a.dL_dcolor = dL_dcolor;
+  a.dL_dmean3D = dL_dmean3D; a.dL_dcov3D = dL_dcov3D; a.dL_dsh = sh_mode ? dL_dsh : nullptr;
+  a.dL_dscale = dL_dscale; a.dL_drot = dL_drot; a.dL_dopacity = dL_dopacity;
+  {
+    StageScope _t("preprocess_bwd", (hipStream_t)stream);
+    launch_preprocess_bwd(a, (hipStream_t)stream);
+  }
+  return check_launch("preprocess_backward", (hipStream_t)stream, debug != 0);
+}
+
+int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resize_fn binningBuffer,
+                      void* binning_user, gs_resize_fn imageBuffer, void* image_user, int P, const float* background,
+                      int width, int height, float focal_x, float focal_y, float cx, float cy,
+                      const float* viewmatrix, const float* cam_pos, const float* all_map, const float* means2D,
+                      const float* depths, const int* radii, const float* conic_opacity, const float* rgb,
+                      const uint8_t* compute_locally, float* out_color, int* n_render, int* n_consider,
+                      int* n_contrib, int* out_observe, float* out_all_map, float* out_plane_depth, int render_geo,
+                      int debug, int* num_rendered, float* elapsed_ms, gs_stream_t stream_) {
+  (void)viewmatrix;
+  (void)cam_pos;
+  hipStream_t stream = (hipStream_t)stream_;
+  GS_REQUIRE(P > 0 && width > 0 && height > 0, "gs_render_forward: P, width and height must be positive");
+  GS_REQUIRE(geometryBuffer && binningBuffer && imageBuffer, "gs_render_forward: null resize callback");
+  GS_REQUIRE(background && means2D && depths && radii && conic_opacity && rgb && compute_locally,
+             "gs_render_forward: null input");
+  GS_REQUIRE(out_color && n_render && n_consider && n_contrib && out_observe && num_rendered,
+             "gs_render_forward: null output");
+  GS_REQUIRE(!render_geo || (all_map && out_all_map && out_plane_depth),
+             "gs_render_forward: render_geo needs all_map, out_all_map and out_plane_depth");
+  const bool dbg = debug != 0;
+  int gx, gy;
+  tile_grid(width, height, gx, gy);
+  const int T = gx * gy;
+
+  const GeometryLayout GL = geometry_layout(P);
+  char* gbase = geometryBuffer(GL.total, geometry_user);
+  GS_REQUIRE(gbase, "gs_render_forward: geometry buffer callback returned NULL");
+  gbase = align_ptr(gbase, 256);
+  uint32_t* tiles_touched = (uint32_t*)(gbase + GL.tiles_touched);
+  uint32_t* point_offsets = (uint32_t*)(gbase + GL.point_offsets);
+  void* scan_temp = gbase + GL.scan_temp;
+
+  const ImageLayout IL = image_layout(width, height);
+  char* ibase = imageBuffer(IL.total, image_user);
+  GS_REQUIRE(ibase, "gs_render_forward: image buffer callback returned NULL");
+  ibase = align_ptr(ibase, 256);
+  float* accum_alpha = (float*)(ibase + IL.accum_alpha);
+  uint32_t* n_contrib_px = (uint32_t*)(ibase + IL.n_contrib);
+  uint32_t* n_contrib2loss_px = (uint32_t*)(ibase + IL.n_contrib2loss);
+  uint32_t* ranges = (uint32_t*)(ibase + IL.ranges);
+
+  {
+    StageScope _t("tile_count", stream);
+    launch_tile_count(P, width, height, radii, means2D, compute_locally, tiles_touched, stream);
+  }
+  if (check_launch("tile_count", stream, dbg)) return 1;
+  {
+    StageScope _t("inclusive_sum", stream);
+    launch_inclusive_sum(P, tiles_touched, point_offsets, scan_temp, stream);
+  }
+  if (check_launch("inclusive_sum", stream, dbg)) return 1;
+
+  uint32_t R_u = 0;
+  GS_HIP_TRY(hipMemcpyAsync(&R_u, point_offsets + (P - 1), sizeof(uint32_t), hipMemcpyDeviceToHost, stream));
+  GS_HIP_TRY(hipStreamSynchronize(stream));
+  if (R_u >= 0x7FFFFFFFu) {
+    set_error("gs_render_forward: %u (Gaussian, tile) instances exceed the supported 2^31-2", R_u);
+    return 1;
+  }
+  const int64_t R = (int64_t)R_u;
+  *num_rendered = (int)R;
+
+  const BinningLayout BL = binning_layout(R);
+  char* bbase = binningBuffer(BL.total, binning_user);
+  GS_REQUIRE(bbase, "gs_render_forward: binning buffer callback returned NULL");
+  bbase = align_ptr(bbase, 256);
+  uint32_t* point_list = (uint32_t*)(bbase + BL.point_list);
+  uint64_t* keys = (uint64_t*)(bbase + BL.keys);
+  uint32_t* point_list_other = (uint32_t*)(bbase + BL.point_list_unsorted);
+  uint64_t* keys_other = (uint64_t*)(bbase + BL.keys_unsorted);
+  void* sort_temp = bbase + BL.sort_temp;
+
+  EventTimer timer;
+  if (timer.begin(elapsed_ms != nullptr, stream)) return 1;
+
+  const int end_bit = sort_end_bit(width, height);
+  // The sort ping-pongs; start from the array pair that makes it finish in
+  // (keys, point_list).
+  const bool odd = sort_result_in_b(end_bit);
+  uint64_t* k_start = odd ? keys_other : keys;
+  uint32_t* v_start = odd ? point_list_other : point_list;
+  uint64_t* k_partner = odd ? keys : keys_other;
+  uint32_t* v_partner = odd ? point_list : point_list_other;
+  if (R > 0) {
+    {
+    StageScope _t("duplicate_with_keys", stream);
+    launch_duplicate_with_keys(P, width, height, means2D, depths, point_offsets, radii, compute_locally, k_start,
+                               v_start, stream);
+  }
+    if (check_launch("duplicate_with_keys", stream, dbg)) return 1;
+    {
+      StageScope _t("sort_pairs", stream);
+      if (launch_sort_pairs_u64(R, k_start, k_partner, v_start, v_partner, end_bit, sort_temp, stream)) return 1;
+    }
+    if (check_launch("sort_pairs", stream, dbg)) return 1;
+  }
+  {
+    StageScope _t("identify_tile_ranges", stream);
+    launch_tile_ranges(R, keys, T, ranges, stream);
+  }
+  if (check_launch("identify_tile_ranges", stream, dbg)) return 1;
+
+  RenderFwdArgs a;
+  a.P = P; a.W = width; a.H = height;
+  a.fx = focal_x; a.fy = focal_y; a.cx = cx; a.cy = cy;
+  a.ranges = ranges; a.point_list = point_list;
+  a.means2D = means2D; a.rgb = rgb; a.all_map = all_map; a.conic_opacity = conic_opacity;
+  a.compute_locally = compute_locally; a.bg = background; a.render_geo = render_geo;
+  a.final_T = accum_alpha; a.n_contrib_px = n_contrib_px; a.n_contrib2loss_px = n_contrib2loss_px;
+  a.out_color = out_color; a.out_observe = out_observe; a.out_all_map = out_all_map;
+  a.out_plane_depth = out_plane_depth;
+  a.n_render = n_render; a.n_consider = n_consider; a.n_contrib_tile = n_contrib;
+  {
+    StageScope _t("render_fwd", stream);
+    launch_render_fwd(a, stream);
+  }
+  if (check_launch("render_forward", stream, dbg)) return 1;
+  if (timer.end(stream, elapsed_ms)) return 1;
+  return 0;
+}
+
+int gs_render_backward(int P, int R, const float* background, int width, int height, float tan_fovx, float tan_fovy,
+                       const char* geom_buffer, const char* binning_buffer, const char* img_buffer,
+                       const uint8_t* compute_locally, const float* dL_dpix, const float* dL_dout_all_map,
+                       const float* dL_dout_plane_depth, float* dL_dmean2D, float* dL_dmean2D_abs,
+                       float* dL_dconic_opacity, float* dL_dcolor, float* dL_dall_map, const float* means2D,
+                       const float* conic_opacity, const float* rgb, const float* all_maps,
+                       const float* all_map_pixels, int render_geo, int debug, float* elapsed_ms,
+                       gs_stream_t stream_) {
+  (void)geom_buffer;
+  hipStream_t stream = (hipStream_t)stream_;
+  GS_REQUIRE(P > 0 && R >= 0 && width > 0 && height > 0, "gs_render_backward: bad sizes");
+  GS_REQUIRE(binning_buffer && img_buffer && compute_locally && background, "gs_render_backward: null buffer");
+  GS_REQUIRE(dL_dpix && dL_dmean2D && dL_dmean2D_abs && dL_dconic_opacity && dL_dcolor && means2D &&
+                 conic_opacity && rgb,
+             "gs_render_backward: null pointer");
+  GS_REQUIRE(!render_geo || (dL_dout_all_map && dL_dout_plane_depth && dL_dall_map && all_maps && all_map_pixels),
+             "gs_render_backward: render_geo needs the geometry-map tensors");
+  const BinningLayout BL = binning_layout(R);
+  const ImageLayout IL = image_layout(width, height);
+  const char* bbase = align_ptr(binning_buffer, 256);
+  const char* ibase = align_ptr(img_buffer, 256);
+  RenderBwdArgs a;
+  a.P = P; a.W = width; a.H = height;
+  a.fy = height / (2.0f * tan_fovy);  // cuda_rasterizer/rasterizer_impl.cu:885-886
+  a.fx = width / (2.0f * tan_fovx);
+  a.bg = background;
+  a.ranges = (const uint32_t*)(ibase + IL.ranges);
+  a.point_list = (const uint32_t*)(bbase + BL.point_list);
+  a.means2D = means2D; a.conic_opacity = conic_opacity; a.rgb = rgb; a.all_map = all_maps;
+  a.all_map_pixels = all_map_pixels;
+  a.final_T = (const float*)(ibase + IL.accum_alpha);
+  a.n_contrib_px = (const uint32_t*)(ibase + IL.n_contrib);
+  a.compute_locally = compute_locally;
+  a.dL_dpix = dL_dpix; a.dL_dout_all_map = dL_dout_all_map; a.dL_dout_plane_depth = dL_dout_plane_depth;
+  a.render_geo = render_geo;
+  a.dL_dmean2D = dL_dmean2D; a.dL_dmean2D_abs = dL_dmean2D_abs; a.dL_dconic_opacity = dL_dconic_opacity;
+  a.dL_dcolors = dL_dcolor; a.dL_dall_map = dL_dall_map;
+  EventTimer timer;
+  if (timer.begin(elapsed_ms != nullptr, stream)) return 1;
+  {
+    StageScope _t("render_bwd", stream);
+    launch_render_bwd(a, stream);
+  }
+  if (check_launch("render_backward", stream, debug != 0)) return 1;
+  if (timer.end(stream, elapsed_ms)) return 1;
+  return 0;
+}
+
+size_t gs_knn_workspace_bytes(int P) { return knn_temp_bytes(P) + 256; }
+
+int gs_knn_dist2(int P, const float* points, float* mean_dists, void* workspace, size_t workspace_bytes,
+                 gs_stream_t stream) {
+  GS_REQUIRE(P >= 0, "gs_knn_dist2: negative P");
+  if (P == 0) return 0;
+  GS_REQUIRE(points && mean_dists && workspace, "gs_knn_dist2: null pointer");
+  GS_REQUIRE(workspace_bytes >= gs_knn_workspace_bytes(P), "gs_knn_dist2: workspace too small");
+  {
+    StageScope _t("knn_dist2", (hipStream_t)stream);
+    if (launch_knn_dist2(P, points, mean_dists, align_ptr((char*)workspace, 256), (hipStream_t)stream)) return 1;
+  }
+  return check_launch("knn_dist2", (hipStream_t)stream, false);
+}
+
+// ------------------------------------------------------------ stage level --
+
+int gs_tile_count(int P, int width, int height, const int* radii, const float* means2D,
+                  const uint8_t* compute_locally, uint32_t* tiles_touched, gs_stream_t stream) {
+  GS_REQUIRE(P >= 0 && width > 0 && height > 0, "gs_tile_count: bad sizes");
+  if (P == 0) return 0;
+  GS_REQUIRE(radii && means2D && compute_locally && tiles_touched, "gs_tile_count: null pointer");
+  launch_tile_count(P, width, height, radii, means2D, compute_locally, tiles_touched, (hipStream_t)stream);
+  return check_launch("tile_count", (hipStream_t)stream, false);
+}
+
+size_t gs_scan_workspace_bytes(int64_t n) { return scan_temp_bytes(n) + 256; }
+
+int gs_inclusive_sum(int64_t n, const uint32_t* in, uint32_t* out, void* workspace, size_t workspace_bytes,
+                     gs_stream_t stream) {
+  GS_REQUIRE(n >= 0, "gs_inclusive_sum: negative n");
+  if (n == 0) return 0;
+  GS_REQUIRE(in && out && workspace, "gs_inclusive_sum: null pointer");
+  GS_REQUIRE(workspace_bytes >= gs_scan_workspace_bytes(n), "gs_inclusive_sum: workspace too small");
+  launch_inclusive_sum(n, in, out, align_ptr((char*)workspace, 256), (hipStream_t)stream);
+  return check_launch("inclusive_sum", (hipStream_t)stream, false);
+}
+
+int gs_duplicate_with_keys(int P, int width, int height, const float* means2D, const float* depths,
+                           const uint32_t* offsets, const int* radii, const uint8_t* compute_locally, uint64_t* keys,
+                           uint32_t* values, gs_stream_t stream) {
+  GS_REQUIRE(P >= 0 && width > 0 && height > 0, "gs_duplicate_with_keys: bad sizes");
+  if (P == 0) return 0;
+  GS_REQUIRE(means2D && depths && offsets && radii && compute_locally && keys && values,
+             "gs_duplicate_with_keys: null pointer");
+  launch_duplicate_with_keys(P, width, height, means2D, depths, offsets, radii, compute_locally, keys, values,
+                             (hipStream_t)stream);
+  return check_launch("duplicate_with_keys", (hipStream_t)stream, false);
+}
+
+size_t gs_sort_workspace_bytes(int64_t n) { return sort_temp_bytes(n) + 256; }
+
+int gs_sort_pairs_u64(int64_t n, uint64_t* keys_in, uint64_t* keys_out, uint32_t* vals_in, uint32_t* vals_out,
+                      int end_bit, void* workspace, size_t workspace_bytes, gs_stream_t stream_) {
+  hipStream_t stream = (hipStream_t)stream_;
+  GS_REQUIRE(n >= 0 && end_bit >= 1 && end_bit <= 64, "gs_sort_pairs_u64: bad n or end_bit");
+  if (n == 0) return 0;
+  GS_REQUIRE(keys_in && keys_out && vals_in && vals_out && workspace, "gs_sort_pairs_u64: null pointer");
+  GS_REQUIRE(workspace_bytes >= gs_sort_workspace_bytes(n), "gs_sort_pairs_u64: workspace too small");
+  void* temp = align_ptr((char*)workspace, 256);
+  if (sort_result_in_b(end_bit)) {
+    if (launch_sort_pairs_u64(n, keys_in, keys_out, vals_in, vals_out, end_bit, temp, stream)) return 1;
+  } else {
+    GS_HIP_TRY(hipMemcpyAsync(keys_out, keys_in, (size_t)n * 8, hipMemcpyDeviceToDevice, stream));
+    GS_HIP_TRY(hipMemcpyAsync(vals_out, vals_in, (size_t)n * 4, hipMemcpyDeviceToDevice, stream));
+    if (launch_sort_pairs_u64(n, keys_out, keys_in, vals_out, vals_in, end_bit, temp, stream)) return 1;
+  }
+  return check_launch("sort_pairs_u64", stream, false);
+}
+
+int gs_sort_pairs_u32(int64_t n, uint32_t* keys_in, uint32_t* keys_out, uint32_t* vals_in, uint32_t* vals_out,
+                      int end_bit, void* workspace, size_t workspace_bytes, gs_stream_t stream_) {
+  hipStream_t stream = (hipStream_t)stream_;
+  GS_REQUIRE(n >= 0 && end_bit >= 1 && end_bit <= 32, "gs_sort_pairs_u32: bad n or end_bit");
+  if (n == 0) return 0;
+  GS_REQUIRE(keys_in && keys_out && vals_in && vals_out && workspace, "gs_sort_pairs_u32: null pointer");
+  GS_REQUIRE(workspace_bytes >= gs_sort_workspace_bytes(n), "gs_sort_pairs_u32: workspace too small");
+  void* temp = align_ptr((char*)workspace, 256);
+  if (sort_result_in_b(end_bit)) {
+    if (launch_sort_pairs_u32(n, keys_in, keys_out, vals_in, vals_out, end_bit, temp, stream)) return 1;
+  } else {
+    GS_HIP_TRY(hipMemcpyAsync(keys_out, keys_in, (size_t)n * 4, hipMemcpyDeviceToDevice, stream));
+    GS_HIP_TRY(hipMemcpyAsync(vals_out, vals_in, (size_t)n * 4, hipMemcpyDeviceToDevice, stream));
+    if (launch_sort_pairs_u32(n, keys_out, keys_in, vals_out, vals_in, end_bit, temp, stream)) return 1;
+  }
+  return check_launch("sort_pairs_u32", stream, false);
+}
+
+int gs_identify_tile_ranges(int64_t L, const uint64_t* keys_sorted, int tiles, uint32_t* ranges, gs_stream_t stream) {
+  GS_REQUIRE(L >= 0 && tiles > 0 && ranges && (L == 0 || keys_sorted), "gs_identify_tile_ranges: bad arguments");
+  launch_tile_ranges(L, keys_sorted, tiles, ranges, (hipStream_t)stream);
+  return check_launch("identify_tile_ranges", (hipStream_t)stream, false);
+}
+
+int gs_render_tiles_forward(int P, int width, int height, float focal_x, float focal_y, float cx, float cy,
+                            const uint32_t* ranges, const uint32_t* point_list, const float* means2D,
+                            const float* rgb, const float* all_map, const float* conic_opacity,
+                            const uint8_t* compute_locally, const float* background, int render_geo, float* final_T,
+                            uint32_t* n_contrib_px, uint32_t* n_contrib2loss_px, float* out_color, int* out_observe,
+                            float* out_all_map, float* out_plane_depth, int* n_render, int* n_consider,
+                            int* n_contrib, gs_stream_t stream) {
+  GS_REQUIRE(P > 0 && width > 0 && height > 0, "gs_render_tiles_forward: bad sizes");
+  GS_REQUIRE(ranges && point_list && means2D && rgb && conic_opacity && compute_locally && background && final_T &&
+                 n_contrib_px && n_contrib2loss_px && out_color && out_observe && n_render && n_consider && n_contrib,
+             "gs_render_tiles_forward: null pointer");
+  GS_REQUIRE(!render_geo || (all_map && out_all_map && out_plane_depth),
+             "gs_render_tiles_forward: render_geo needs all_map, out_all_map and out_plane_depth");
+  RenderFwdArgs a;
+  a.P = P; a.W = width; a.H = height;
+  a.fx = focal_x; a.fy = focal_y; a.cx = cx; a.cy = cy;
+  a.ranges = ranges; a.point_list = point_list;
+  a.means2D = means2D; a.rgb = rgb; a.all_map = all_map; a.conic_opacity = conic_opacity;
+  a.compute_locally = compute_locally; a.bg = background; a.render_geo = render_geo;
+  a.final_T = final_T; a.n_contrib_px = n_contrib_px; a.n_contrib2loss_px = n_contrib2loss_px;
+  a.out_color = out_color; a.out_observe = out_observe; a.out_all_map = out_all_map;
+  a.out_plane_depth = out_plane_depth;
+  a.n_render = n_render; a.n_consider = n_consider; a.n_contrib_tile = n_contrib;
+  launch_render_fwd(a, (hipStream_t)stream);
+  return check_launch("render_tiles_forward", (hipStream_t)stream, false);
+}
+
+int gs_render_tiles_backward(int P, int width, int height, float tan_fovx, float tan_fovy, const float* background,
+                             const uint32_t* ranges, const uint32_t* point_list, const float* means2D,
+                             const float* conic_opacity, const float* rgb, const float* all_maps,
+                             const float* all_map_pixels, const float* final_T, const uint32_t* n_contrib_px,
+                             const uint8_t* compute_locally, const float* dL_dpix, const float* dL_dout_all_map,
+                             const float* dL_dout_plane_depth, int render_geo, float* dL_dmean2D,
+                             float* dL_dmean2D_abs, float* dL_dconic_opacity, float* dL_dcolor, float* dL_dall_map,
+                             gs_stream_t stream) {
+  GS_REQUIRE(P > 0 && width > 0 && height > 0, "gs_render_tiles_backward: bad sizes");
+  GS_REQUIRE(background && ranges && point_list && means2D && conic_opacity && rgb && final_T && n_contrib_px &&
+                 compute_locally && dL_dpix && dL_dmean2D && dL_dmean2D_abs && dL_dconic_opacity && dL_dcolor,
+             "gs_render_tiles_backward: null pointer");
+  GS_REQUIRE(!render_geo || (dL_dout_all_map && dL_dout_plane_depth && dL_dall_map && all_maps && all_map_pixels),
+             "gs_render_tiles_backward: render_geo needs the geometry-map tensors");
+  RenderBwdArgs a;
+  a.P = P; a.W = width; a.H = height;
+  a.fy = height / (2.0f * tan_fovy);
+  a.fx = width / (2.0f * tan_fovx);
+  a.bg = background; a.ranges = ranges; a.point_list = point_list;
+  a.means2D = means2D; a.conic_opacity = conic_opacity; a.rgb = rgb; a.all_map = all_maps;
+  a.all_map_pixels = all_map_pixels; a.final_T = final_T; a.n_contrib_px = n_contrib_px;
+  a.compute_locally = compute_locally;
+  a.dL_dpix = dL_dpix; a.dL_dout_all_map = dL_dout_all_map; a.dL_dout_plane_depth = dL_dout_plane_depth;
+  a.render_geo = render_geo;
+  a.dL_dmean2D = dL_dmean2D; a.dL_dmean2D_abs = dL_dmean2D_abs; a.dL_dconic_opacity = dL_dconic_opacity;
+  a.dL_dcolors = dL_dcolor; a.dL_dall_map = dL_dall_map;
+  launch_render_bwd(a, (hipStream_t)stream);
+  return check_launch("render_tiles_backward", (hipStream_t)stream, false);
+}
+
+int gs_stage_timing_enable(int enable) {
+  g_clock.enabled = enable != 0;
+  return 0;
+}
+
+int gs_stage_timing_collect(char* report, size_t report_bytes) {
+  GS_REQUIRE(report && report_bytes > 0, "gs_stage_timing_collect: null report buffer");
+  std::map<std::string, std::pair<double, long>> acc;
+  std::vector<std::string> order;
+  for (auto& r : g_clock.pending) {
+    float ms = 0.f;
+    GS_HIP_TRY(hipEventSynchronize(r.b));
+    GS_HIP_TRY(hipEventElapsedTime(&ms, r.a, r.b));
+    if (!acc.count(r.name)) order.push_back(r.name);
+    acc[r.name].first += ms;
+    acc[r.name].second += 1;
+    g_clock.pool.push_back(r.a);
+    g_clock.pool.push_back(r.b);
+  }
+  g_clock.pending.clear();
+  size_t used = 0;
+  report[0] = 0;
+  for (auto& name : order) {
+    const int w = snprintf(report + used, report_bytes - used, "%s %.6f %ld\n", name.c_str(), acc[name].first,
+                           acc[name].second);
+    if (w < 0 || (size_t)w >= report_bytes - used) break;
+    used += (size_t)w;
+  }
+  return 0;
+}
+
+int gs_image_state_layout(int width, int height, size_t* accum_alpha, size_t* n_contrib, size_t* n_contrib2loss,
+                          size_t* ranges, size_t* total_bytes) {
+  GS_REQUIRE(width > 0 && height > 0, "gs_image_state_layout: bad sizes");
+  const ImageLayout L = image_layout(width, height);
+  if (accum_alpha) *accum_alpha = L.accum_alpha;
+  if (n_contrib) *n_contrib = L.n_contrib;
+  if (n_contrib2loss) *n_contrib2loss = L.n_contrib2loss;
+  if (ranges) *ranges = L.ranges;
+  if (total_bytes) *total_bytes = L.total;
+  return 0;
+}
+
+int gs_binning_state_layout(int64_t R, int width, int height, size_t* point_list, size_t* point_list_keys,
+                            size_t* point_list_unsorted, size_t* point_list_keys_unsorted, size_t* total_bytes) {
+  (void)width;
+  (void)height;
+  GS_REQUIRE(R >= 0, "gs_binning_state_layout: negative R");
+  const BinningLayout L = binning_layout(R);
+  if (point_list) *point_list = L.point_list;
+  if (point_list_keys) *point_list_keys = L.keys;
+  if (point_list_unsorted) *point_list_unsorted = L.point_list_unsorted;
+  if (point_list_keys_unsorted) *point_list_keys_unsorted = L.keys_unsorted;
+  if (total_bytes) *total_bytes = L.total;
+  return 0;
+}
+
+int gs_geometry_state_layout(int P, size_t* tiles_touched, size_t* point_offsets, size_t* total_bytes) {
+  GS_REQUIRE(P >= 0, "gs_geometry_state_layout: negative P");
+  const GeometryLayout L = geometry_layout(P);
+  if (tiles_touched) *tiles_touched = L.tiles_touched;
+  if (point_offsets) *point_offsets = L.point_offsets;
+  if (total_bytes) *total_bytes = L.total;
+  return 0;
+}
+
+}  // extern "C"

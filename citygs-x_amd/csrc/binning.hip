@@ -1,0 +1,234 @@
+// Tile binning: per-Gaussian tile counts, uint32 prefix sum, (tile|depth) key
+// emission and per-tile range detection
+// (cuda_rasterizer/rasterizer_impl.cu:74-144, :264-288, :633-697).
+// All of it is integer / bit work and must match a CPU bit for bit.
+#include "gs_common.h"
+#include "gs_kernels.h"
+
+namespace gs {
+
+namespace {
+
+constexpr int SCAN_THREADS = 256;
+constexpr int SCAN_ITEMS = 8;
+constexpr int SCAN_TILE = SCAN_THREADS * SCAN_ITEMS;
+
+__device__ __forceinline__ uint32_t wave_inclusive_scan(uint32_t v) {
+  const int lane = threadIdx.x & (GS_WAVE - 1);
+#pragma unroll
+  for (int d = 1; d < GS_WAVE; d <<= 1) {
+    const uint32_t o = __shfl_up(v, d, GS_WAVE);
+    if (lane >= d) v += o;
+  }
+  return v;
+}
+
+// Exclusive prefix of v across the block plus the block total.
+template <int THREADS>
+__device__ __forceinline__ uint32_t block_exclusive_scan(uint32_t v, uint32_t* s_wave /*THREADS/64 + 1*/,
+                                                         uint32_t& total) {
+  constexpr int NW = THREADS / GS_WAVE;
+  const int lane = threadIdx.x & (GS_WAVE - 1), wave = threadIdx.x / GS_WAVE;
+  const uint32_t inc = wave_inclusive_scan(v);
+  if (lane == GS_WAVE - 1) s_wave[wave] = inc;
+  __syncthreads();
+  uint32_t base = 0, tot = 0;
+#pragma unroll
+  for (int w = 0; w < NW; w++) {
+    const uint32_t s = s_wave[w];
+    if (w < wave) base += s;
+    tot += s;
+  }
+  __syncthreads();
+  total = tot;
+  return base + inc - v;
+}
+
+// cuda_rasterizer/rasterizer_impl.cu:264-288.
+__global__ void __launch_bounds__(GS_BLOCK_1D)
+tile_count_kernel(int P, uint32_t gx, uint32_t gy, const int* __restrict__ radii,
+                  const float2* __restrict__ means2D, const uint8_t* __restrict__ compute_locally,
+                  uint32_t* __restrict__ tiles_touched) {
+  const int i = blockIdx.x * GS_BLOCK_1D + threadIdx.x;
+  if (i >= P) return;
+  uint32_t cnt = 0;
+  const int r = radii[i];
+  if (r > 0) {
+    const float2 p = means2D[i];
+    const Rect rc = get_rect(p.x, p.y, r, gx, gy);
+    for (uint32_t y = rc.y0; y < rc.y1; y++)
+      for (uint32_t x = rc.x0; x < rc.x1; x++)
+        if (compute_locally[y * gx + x]) cnt++;
+  }
+  tiles_touched[i] = cnt;
+}
+
+__global__ void __launch_bounds__(SCAN_THREADS)
+scan_block_sums_kernel(int64_t n, const uint32_t* __restrict__ in, uint32_t* __restrict__ block_sums) {
+  __shared__ uint32_t s_wave[SCAN_THREADS / GS_WAVE];
+  const int64_t base = (int64_t)blockIdx.x * SCAN_TILE;
+  uint32_t s = 0;
+#pragma unroll
+  for (int k = 0; k < SCAN_ITEMS; k++) {
+    const int64_t idx = base + (int64_t)k * SCAN_THREADS + threadIdx.x;
+    if (idx < n) s += in[idx];
+  }
+#pragma unroll
+  for (int d = GS_WAVE / 2; d >= 1; d >>= 1) s += __shfl_xor(s, d, GS_WAVE);
+  if ((threadIdx.x & (GS_WAVE - 1)) == 0) s_wave[threadIdx.x / GS_WAVE] = s;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    uint32_t t = 0;
+    for (int w = 0; w < SCAN_THREADS / GS_WAVE; w++) t += s_wave[w];
+    block_sums[blockIdx.x] = t;
+  }
+}
+
+// One block turns the per-tile sums into exclusive prefixes in place.
+__global__ void __launch_bounds__(1024) scan_spine_kernel(int nblocks, uint32_t* __restrict__ block_sums) {
+  __shared__ uint32_t s_wave[1024 / GS_WAVE];
+  uint32_t carry = 0;
+  for (int start = 0; start < nblocks; start += 1024) {
+    const int idx = start + threadIdx.x;
+    const uint32_t v = idx < nblocks ? block_sums[idx] : 0u;
+    uint32_t total;
+    const uint32_t ex = block_exclusive_scan<1024>(v, s_wave, total);
+    if (idx < nblocks) block_sums[idx] = carry + ex;
+    carry += total;
+  }
+}
+
+template <bool EXCLUSIVE>
+__global__ void __launch_bounds__(SCAN_THREADS)
+scan_apply_kernel(int64_t n, const uint32_t* in, const uint32_t* __restrict__ block_prefix, uint32_t* out) {
+  // in and out may be the same array: each thread reads its items before it writes them.
+  __shared__ uint32_t s_wave[SCAN_THREADS / GS_WAVE];
+  // Blocked arrangement: thread t owns SCAN_ITEMS consecutive elements.
+  const int64_t base = (int64_t)blockIdx.x * SCAN_TILE + (int64_t)threadIdx.x * SCAN_ITEMS;
+  uint32_t v[SCAN_ITEMS];
+  uint32_t s = 0;
+#pragma unroll
+  for (int k = 0; k < SCAN_ITEMS; k++) {
+    v[k] = (base + k < n) ? in[base + k] : 0u;
+    s += v[k];
+  }
+  uint32_t total;
+  uint32_t run = block_prefix[blockIdx.x] + block_exclusive_scan<SCAN_THREADS>(s, s_wave, total);
+#pragma unroll
+  for (int k = 0; k < SCAN_ITEMS; k++) {
+    if (EXCLUSIVE) {
+      if (base + k < n) out[base + k] = run;
+      run += v[k];
+    } else {
+      run += v[k];
+      if (base + k < n) out[base + k] = run;
+    }
+  }
+}
+
+// cuda_rasterizer/rasterizer_impl.cu:74-117.
+__global__ void __launch_bounds__(GS_BLOCK_1D)
+duplicate_with_keys_kernel(int P, uint32_t gx, uint32_t gy, const float2* __restrict__ means2D,
+                           const float* __restrict__ depths, const uint32_t* __restrict__ offsets,
+                           const int* __restrict__ radii, const uint8_t* __restrict__ compute_locally,
+                           uint64_t* __restrict__ keys, uint32_t* __restrict__ values) {
+  const int i = blockIdx.x * GS_BLOCK_1D + threadIdx.x;
+  if (i >= P) return;
+  const int r = radii[i];
+  if (r > 0) {
+    uint32_t off = (i == 0) ? 0u : offsets[i - 1];
+    const float2 p = means2D[i];
+    const Rect rc = get_rect(p.x, p.y, r, gx, gy);
+    const uint32_t dbits = __float_as_uint(depths[i]);
+    for (uint32_t y = rc.y0; y < rc.y1; y++)
+      for (uint32_t x = rc.x0; x < rc.x1; x++)
+        if (compute_locally[y * gx + x]) {
+          const uint64_t key = ((uint64_t)(y * gx + x) << 32) | (uint64_t)dbits;
+          keys[off] = key;
+          values[off] = (uint32_t)i;
+          off++;
+        }
+  }
+}
+
+__global__ void fill_u32_kernel(int64_t n, uint32_t v, uint32_t* __restrict__ p) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = v;
+}
+
+// cuda_rasterizer/rasterizer_impl.cu:122-144.
+__global__ void __launch_bounds__(GS_BLOCK_1D)
+tile_ranges_kernel(int64_t L, const uint64_t* __restrict__ keys, uint32_t* __restrict__ ranges) {
+  const int64_t i = (int64_t)blockIdx.x * GS_BLOCK_1D + threadIdx.x;
+  if (i >= L) return;
+  const uint32_t cur = (uint32_t)(keys[i] >> 32);
+  if (i == 0)
+    ranges[2 * cur] = 0;
+  else {
+    const uint32_t prev = (uint32_t)(keys[i - 1] >> 32);
+    if (cur != prev) {
+      ranges[2 * prev + 1] = (uint32_t)i;
+      ranges[2 * cur] = (uint32_t)i;
+    }
+  }
+  if (i == L - 1) ranges[2 * cur + 1] = (uint32_t)L;
+}
+
+}  // namespace
+
+int launch_tile_count(int P, int W, int H, const int* radii, const float* means2D, const uint8_t* compute_locally,
+                      uint32_t* tiles_touched, hipStream_t stream) {
+  if (P <= 0) return 0;
+  const uint32_t gx = (W + GS_TILE_X - 1) / GS_TILE_X, gy = (H + GS_TILE_Y - 1) / GS_TILE_Y;
+  hipLaunchKernelGGL(tile_count_kernel, dim3((P + GS_BLOCK_1D - 1) / GS_BLOCK_1D), dim3(GS_BLOCK_1D), 0, stream, P,
+                     gx, gy, radii, (const float2*)means2D, compute_locally, tiles_touched);
+  return 0;
+}
+
+size_t scan_temp_bytes(int64_t n) {
+  const int64_t nb = (n + SCAN_TILE - 1) / SCAN_TILE;
+  return align_up((size_t)(nb > 0 ? nb : 1) * sizeof(uint32_t), 256);
+}
+
+static int scan_impl(int64_t n, const uint32_t* in, uint32_t* out, void* temp, bool exclusive, hipStream_t stream) {
+  if (n <= 0) return 0;
+  const int nb = (int)((n + SCAN_TILE - 1) / SCAN_TILE);
+  uint32_t* sums = (uint32_t*)temp;
+  hipLaunchKernelGGL(scan_block_sums_kernel, dim3(nb), dim3(SCAN_THREADS), 0, stream, n, in, sums);
+  hipLaunchKernelGGL(scan_spine_kernel, dim3(1), dim3(1024), 0, stream, nb, sums);
+  if (exclusive)
+    hipLaunchKernelGGL(scan_apply_kernel<true>, dim3(nb), dim3(SCAN_THREADS), 0, stream, n, in, sums, out);
+  else
+    hipLaunchKernelGGL(scan_apply_kernel<false>, dim3(nb), dim3(SCAN_THREADS), 0, stream, n, in, sums, out);
+  return 0;
+}
+
+// in and out may alias.
+int launch_inclusive_sum(int64_t n, const uint32_t* in, uint32_t* out, void* temp, hipStream_t stream) {
+  return scan_impl(n, in, out, temp, false, stream);
+}
+
+int launch_exclusive_sum(int64_t n, const uint32_t* in, uint32_t* out, void* temp, hipStream_t stream) {
+  return scan_impl(n, in, out, temp, true, stream);
+}
+
+int launch_duplicate_with_keys(int P, int W, int H, const float* means2D, const float* depths,
+                               const uint32_t* offsets, const int* radii, const uint8_t* compute_locally,
+                               uint64_t* keys, uint32_t* values, hipStream_t stream) {
+  if (P <= 0) return 0;
+  const uint32_t gx = (W + GS_TILE_X - 1) / GS_TILE_X, gy = (H + GS_TILE_Y - 1) / GS_TILE_Y;
+  hipLaunchKernelGGL(duplicate_with_keys_kernel, dim3((P + GS_BLOCK_1D - 1) / GS_BLOCK_1D), dim3(GS_BLOCK_1D), 0,
+                     stream, P, gx, gy, (const float2*)means2D, depths, offsets, radii, compute_locally, keys, values);
+  return 0;
+}
+
+int launch_tile_ranges(int64_t L, const uint64_t* keys_sorted, int T, uint32_t* ranges, hipStream_t stream) {
+  if (T > 0)
+    hipLaunchKernelGGL(fill_u32_kernel, dim3((2 * T + 255) / 256), dim3(256), 0, stream, (int64_t)2 * T, 0u, ranges);
+  if (L > 0)
+    hipLaunchKernelGGL(tile_ranges_kernel, dim3((unsigned)((L + GS_BLOCK_1D - 1) / GS_BLOCK_1D)), dim3(GS_BLOCK_1D), 0,
+                       stream, L, keys_sorted, ranges);
+  return 0;
+}
+
+}  // namespace gs

@@ -1,0 +1,153 @@
+// Shared host/device definitions for the gfx950 Gaussian rasterizer library.
+//
+// Arithmetic policy: every kernel is compiled with -ffp-contract=off, so each
+// fp32 operation rounds once exactly as written; fused multiply-adds appear
+// only where __builtin_fmaf is spelled out.  Division and sqrt are the
+// correctly rounded ones (hipcc default).  This is what makes radii, tile
+// rectangles, depth keys and contributor counts reproducible bit for bit on a
+// CPU.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#define GS_TILE_X 16      // cuda_rasterizer/config.h:17
+#define GS_TILE_Y 16      // cuda_rasterizer/config.h:19
+#define GS_TILE_PIX 256
+#define GS_BLOCK_1D 256   // cuda_rasterizer/config.h:21
+#define GS_N_RGB 3        // cuda_rasterizer/config.h:15
+#define GS_N_MAP 5        // cuda_rasterizer/config.h:24
+#define GS_WAVE 64
+
+namespace gs {
+
+void set_error(const char* fmt, ...);
+int check_launch(const char* what, hipStream_t stream, bool sync);
+
+#define GS_HIP_TRY(expr)                                                            \
+  do {                                                                              \
+    hipError_t _e = (expr);                                                         \
+    if (_e != hipSuccess) {                                                         \
+      gs::set_error("%s failed: %s (%s:%d)", #expr, hipGetErrorString(_e), __FILE__, __LINE__); \
+      return 1;                                                                     \
+    }                                                                               \
+  } while (0)
+
+inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+// ------------------------------------------------------------ device math --
+
+__device__ __forceinline__ int f2i_sat(float v) {
+  // float -> int32 with the conversion instruction's semantics spelled out:
+  // truncate toward zero, clamp to the int32 range, NaN -> 0.
+  if (!(v == v)) return 0;
+  if (v >= 2147483648.0f) return 2147483647;
+  if (v <= -2147483648.0f) return (-2147483647 - 1);
+  return (int)v;
+}
+
+__device__ __forceinline__ uint32_t f2u_sat(float v) {
+  if (!(v == v)) return 0u;
+  if (v >= 4294967296.0f) return 0xFFFFFFFFu;
+  if (v <= 0.0f) return 0u;
+  return (uint32_t)v;
+}
+
+// exp() of the blending loops: n = rint(x*log2e), r = x - n*ln2 (two-constant
+// split), degree-6 polynomial, scale by 2^n.  Only IEEE operations and explicit
+// FMAs, so a CPU evaluates the same bits.  x < -87 -> 0, x > 88 -> +inf.
+__device__ __forceinline__ float gs_expf(float x) {
+  if (!(x == x)) return x;
+  if (x < -87.0f) return 0.0f;
+  if (x > 88.0f) return __builtin_inff();
+  float n = __builtin_rintf(x * 1.44269504088896341f);
+  float r = __builtin_fmaf(n, -0.693145751953125f, x);
+  r = __builtin_fmaf(n, -1.42860682030941723212e-6f, r);
+  float p = 1.9875691500e-4f;
+  p = __builtin_fmaf(p, r, 1.3981999507e-3f);
+  p = __builtin_fmaf(p, r, 8.3334519073e-3f);
+  p = __builtin_fmaf(p, r, 4.1665795894e-2f);
+  p = __builtin_fmaf(p, r, 1.6666665459e-1f);
+  p = __builtin_fmaf(p, r, 5.0000001201e-1f);
+  float r2 = r * r;
+  p = __builtin_fmaf(p, r2, r);
+  p = p + 1.0f;
+  return __builtin_ldexpf(p, (int)n);
+}
+
+// Column-major 3x3 with the product evaluated term by term, left to right
+// (the semantics of the reference's matrix type,
+// third_party/glm/glm/detail/type_mat3x3.inl:486-518).
+struct M3 {
+  float m[3][3];  // m[col][row]
+};
+
+__device__ __forceinline__ M3 m3_cols(float a0, float a1, float a2, float b0, float b1, float b2,
+                                      float c0, float c1, float c2) {
+  M3 r;
+  r.m[0][0] = a0; r.m[0][1] = a1; r.m[0][2] = a2;
+  r.m[1][0] = b0; r.m[1][1] = b1; r.m[1][2] = b2;
+  r.m[2][0] = c0; r.m[2][1] = c1; r.m[2][2] = c2;
+  return r;
+}
+
+__device__ __forceinline__ M3 m3_mul(const M3& A, const M3& B) {
+  M3 R;
+#pragma unroll
+  for (int c = 0; c < 3; c++)
+#pragma unroll
+    for (int r = 0; r < 3; r++)
+      R.m[c][r] = (A.m[0][r] * B.m[c][0] + A.m[1][r] * B.m[c][1]) + A.m[2][r] * B.m[c][2];
+  return R;
+}
+
+__device__ __forceinline__ M3 m3_T(const M3& A) {
+  M3 R;
+#pragma unroll
+  for (int c = 0; c < 3; c++)
+#pragma unroll
+    for (int r = 0; r < 3; r++) R.m[c][r] = A.m[r][c];
+  return R;
+}
+
+__device__ __forceinline__ float dot3(const float* a, const float* b) {
+  return (a[0] * b[0] + a[1] * b[1]) + a[2] * b[2];
+}
+
+// Row-vector transforms by a 4x4 matrix stored row-major
+// (cuda_rasterizer/auxiliary.h:112-151).
+__device__ __forceinline__ void xform4x3(const float* p, const float* M, float* o) {
+#pragma unroll
+  for (int k = 0; k < 3; k++) o[k] = ((M[k] * p[0] + M[4 + k] * p[1]) + M[8 + k] * p[2]) + M[12 + k];
+}
+__device__ __forceinline__ void xform4x4(const float* p, const float* M, float* o) {
+#pragma unroll
+  for (int k = 0; k < 4; k++) o[k] = ((M[k] * p[0] + M[4 + k] * p[1]) + M[8 + k] * p[2]) + M[12 + k];
+}
+__device__ __forceinline__ void xformVec4x3T(const float* v, const float* M, float* o) {
+#pragma unroll
+  for (int k = 0; k < 3; k++) o[k] = (M[4 * k] * v[0] + M[4 * k + 1] * v[1]) + M[4 * k + 2] * v[2];
+}
+
+// cuda_rasterizer/auxiliary.h:52-55 (double intermediates).
+__device__ __forceinline__ float ndc2pix(float v, int S) {
+  return (float)((((double)v + 1.0) * (double)S - 1.0) * 0.5);
+}
+
+struct Rect {
+  uint32_t x0, y0, x1, y1;
+};
+
+// cuda_rasterizer/auxiliary.h:66-76: tile rectangle [min,max) of a splat with
+// integer radius, clamped to the grid.
+__device__ __forceinline__ Rect get_rect(float px, float py, int radius, uint32_t gx, uint32_t gy) {
+  const float rf = (float)radius;
+  Rect r;
+  r.x0 = min(gx, (uint32_t)max(0, f2i_sat((px - rf) / (float)GS_TILE_X)));
+  r.y0 = min(gy, (uint32_t)max(0, f2i_sat((py - rf) / (float)GS_TILE_Y)));
+  r.x1 = min(gx, (uint32_t)max(0, f2i_sat((((px + rf) + (float)GS_TILE_X) - 1.0f) / (float)GS_TILE_X)));
+  r.y1 = min(gy, (uint32_t)max(0, f2i_sat((((py + rf) + (float)GS_TILE_Y) - 1.0f) / (float)GS_TILE_Y)));
+  return r;
+}
+
+}  // namespace gs

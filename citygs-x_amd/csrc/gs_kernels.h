@@ -1,0 +1,112 @@
+// Internal launch interface between the C-ABI layer (api.hip) and the kernel
+// translation units.  All pointers are device pointers unless noted.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+namespace gs {
+
+struct PreprocessFwdArgs {
+  int P, D, M, W, H;
+  const float *means3D, *scales, *rotations, *opacities, *shs;
+  float scale_modifier;
+  const float *viewmatrix, *projmatrix, *campos;
+  float tanx, tany;
+  int* radii;
+  float *means2D, *depths, *cov3D, *conic_opacity, *rgb;
+  uint8_t* clamped;
+  uint32_t* tiles_touched;  // optional
+};
+
+struct PreprocessBwdArgs {
+  int P, D, M, W, H;
+  const float* means3D;
+  const int* radii;
+  const float* shs;
+  const uint8_t* clamped;
+  const float *scales, *rotations;
+  float scale_modifier;
+  const float *cov3D, *viewmatrix, *projmatrix, *campos;
+  float tanx, tany;
+  const float* dL_dmean2D;
+  int mean2D_stride;               // 2 or 3 floats per row
+  const float* dL_dconic_opacity;  // (P,4) packed [x, y, w, opacity]
+  const float* dL_dcolor;          // (P,3), SH mode only
+  float *dL_dmean3D, *dL_dcov3D /*optional*/, *dL_dsh /*optional*/, *dL_dscale, *dL_drot, *dL_dopacity /*optional*/;
+};
+
+int launch_preprocess_fwd(const PreprocessFwdArgs& a, hipStream_t stream);
+int launch_preprocess_bwd(const PreprocessBwdArgs& a, hipStream_t stream);
+int launch_visible_filter(int P, const float* means, const float* scales, float mod, const float* rots,
+                          const float* cov_pre, const float* V, const float* PM, int W, int H, float tanx,
+                          float tany, int* radii, hipStream_t stream);
+int launch_mark_visible(int P, const float* means, const float* V, uint8_t* present, hipStream_t stream);
+
+// ---- binning ----
+int launch_tile_count(int P, int W, int H, const int* radii, const float* means2D, const uint8_t* compute_locally,
+                      uint32_t* tiles_touched, hipStream_t stream);
+size_t scan_temp_bytes(int64_t n);
+int launch_inclusive_sum(int64_t n, const uint32_t* in, uint32_t* out, void* temp, hipStream_t stream);
+int launch_exclusive_sum(int64_t n, const uint32_t* in, uint32_t* out, void* temp, hipStream_t stream);
+int launch_duplicate_with_keys(int P, int W, int H, const float* means2D, const float* depths,
+                               const uint32_t* offsets, const int* radii, const uint8_t* compute_locally,
+                               uint64_t* keys, uint32_t* values, hipStream_t stream);
+int launch_tile_ranges(int64_t L, const uint64_t* keys_sorted, int T, uint32_t* ranges, hipStream_t stream);
+
+// ---- radix sort (stable, LSD, 8-bit digits) ----
+size_t sort_temp_bytes(int64_t n);
+// Sorts on key bits [0, end_bit), ping-ponging between the (a) and (b) arrays
+// starting from (a).  With an odd number of 8-bit passes the sorted result
+// lands in (b), with an even number back in (a): sort_result_in_b() tells.
+inline int sort_num_passes(int end_bit) { return (end_bit + 7) / 8; }
+inline bool sort_result_in_b(int end_bit) { return (sort_num_passes(end_bit) & 1) != 0; }
+int launch_sort_pairs_u64(int64_t n, uint64_t* keys_a, uint64_t* keys_b, uint32_t* vals_a, uint32_t* vals_b,
+                          int end_bit, void* temp, hipStream_t stream);
+int launch_sort_pairs_u32(int64_t n, uint32_t* keys_a, uint32_t* keys_b, uint32_t* vals_a, uint32_t* vals_b,
+                          int end_bit, void* temp, hipStream_t stream);
+
+// ---- tile render ----
+struct RenderFwdArgs {
+  int P, W, H;
+  float fx, fy, cx, cy;
+  const uint32_t* ranges;      // (T,2)
+  const uint32_t* point_list;  // (R)
+  const float *means2D, *rgb, *all_map, *conic_opacity;
+  const uint8_t* compute_locally;
+  const float* bg;
+  int render_geo;
+  float* final_T;
+  uint32_t *n_contrib_px, *n_contrib2loss_px;
+  float* out_color;
+  int* out_observe;
+  float *out_all_map, *out_plane_depth;
+  int *n_render, *n_consider, *n_contrib_tile;
+};
+int launch_render_fwd(const RenderFwdArgs& a, hipStream_t stream);
+
+struct RenderBwdArgs {
+  int P, W, H;
+  float fx, fy;
+  const float* bg;
+  const uint32_t *ranges, *point_list;
+  const float *means2D, *conic_opacity, *rgb, *all_map, *all_map_pixels, *final_T;
+  const uint32_t* n_contrib_px;
+  const uint8_t* compute_locally;
+  const float *dL_dpix, *dL_dout_all_map, *dL_dout_plane_depth;
+  int render_geo;
+  // zero-initialised accumulation targets
+  float* dL_dmean2D;         // (P,2)
+  float* dL_dmean2D_abs;     // (P,3)
+  float* dL_dconic_opacity;  // (P,4) packed [x, y, w, opacity]
+  float* dL_dcolors;         // (P,3)
+  float* dL_dall_map;        // (P,5)
+};
+int launch_render_bwd(const RenderBwdArgs& a, hipStream_t stream);
+
+// ---- k-nearest-neighbour mean squared distance ----
+size_t knn_temp_bytes(int P);
+int launch_knn_dist2(int P, const float* points, float* mean_dist2, void* temp, hipStream_t stream);
+
+}  // namespace gs

@@ -1,0 +1,237 @@
+// Mean squared distance to the three nearest neighbours of every point
+// (simple-knn/simple_knn.cu:185-221, distCUDA2): global bounding box, 30-bit
+// Morton codes, stable sort by code, bounding boxes of runs of 1024 sorted
+// points, then an exact search that visits only boxes closer than the current
+// third-best distance.  The search is exhaustive within that bound, so the
+// three distances equal a brute-force search whatever the visiting order.
+#include <float.h>
+
+#include "gs_common.h"
+#include "gs_kernels.h"
+
+namespace gs {
+
+namespace {
+
+constexpr int KNN_BOX = 1024;  // simple-knn/simple_knn.cu:12
+constexpr int MM_BLOCKS = 512;
+constexpr int MM_THREADS = 256;
+
+struct KnnLayout {
+  size_t partial, minmax, codes_a, codes_b, idx_a, idx_b, sorted_pts, boxes, sort_temp, total;
+};
+
+KnnLayout knn_layout(int P) {
+  KnnLayout L;
+  size_t off = 0;
+  auto take = [&](size_t bytes) {
+    size_t o = off;
+    off += align_up(bytes, 256);
+    return o;
+  };
+  const size_t n = (size_t)(P > 0 ? P : 1);
+  const size_t nb = (n + KNN_BOX - 1) / KNN_BOX;
+  L.partial = take(sizeof(float) * 6 * MM_BLOCKS);
+  L.minmax = take(sizeof(float) * 6);
+  L.codes_a = take(sizeof(uint32_t) * n);
+  L.codes_b = take(sizeof(uint32_t) * n);
+  L.idx_a = take(sizeof(uint32_t) * n);
+  L.idx_b = take(sizeof(uint32_t) * n);
+  L.sorted_pts = take(sizeof(float4) * n);
+  L.boxes = take(sizeof(float) * 6 * nb);
+  L.sort_temp = take(sort_temp_bytes((int64_t)n));
+  L.total = off;
+  return L;
+}
+
+__device__ __forceinline__ void reduce6(float* v, float (*s)[MM_THREADS / GS_WAVE], float* out) {
+  // v[0..2] min, v[3..5] max
+#pragma unroll
+  for (int d = GS_WAVE / 2; d >= 1; d >>= 1) {
+#pragma unroll
+    for (int k = 0; k < 3; k++) {
+      v[k] = fminf(v[k], __shfl_xor(v[k], d, GS_WAVE));
+      v[3 + k] = fmaxf(v[3 + k], __shfl_xor(v[3 + k], d, GS_WAVE));
+    }
+  }
+  const int lane = threadIdx.x & (GS_WAVE - 1), wave = threadIdx.x / GS_WAVE;
+  if (lane == 0) {
+#pragma unroll
+    for (int k = 0; k < 6; k++) s[k][wave] = v[k];
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+#pragma unroll
+    for (int k = 0; k < 3; k++) {
+      float mn = s[k][0], mx = s[3 + k][0];
+      for (int w = 1; w < MM_THREADS / GS_WAVE; w++) {
+        mn = fminf(mn, s[k][w]);
+        mx = fmaxf(mx, s[3 + k][w]);
+      }
+      out[k] = mn;
+      out[3 + k] = mx;
+    }
+  }
+}
+
+// Reduction identity is 0 for both min and max (simple-knn/simple_knn.cu:191).
+__global__ void __launch_bounds__(MM_THREADS) minmax_partial_kernel(int P, const float* __restrict__ pts,
+                                                                     float* __restrict__ partial) {
+  __shared__ float s[6][MM_THREADS / GS_WAVE];
+  float v[6] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  for (int i = blockIdx.x * MM_THREADS + threadIdx.x; i < P; i += MM_BLOCKS * MM_THREADS) {
+#pragma unroll
+    for (int k = 0; k < 3; k++) {
+      const float c = pts[3 * (size_t)i + k];
+      v[k] = fminf(v[k], c);
+      v[3 + k] = fmaxf(v[3 + k], c);
+    }
+  }
+  reduce6(v, s, partial + 6 * blockIdx.x);
+}
+
+__global__ void __launch_bounds__(MM_THREADS) minmax_final_kernel(const float* __restrict__ partial,
+                                                                   float* __restrict__ minmax) {
+  __shared__ float s[6][MM_THREADS / GS_WAVE];
+  float v[6] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  for (int b = threadIdx.x; b < MM_BLOCKS; b += MM_THREADS) {
+#pragma unroll
+    for (int k = 0; k < 3; k++) {
+      v[k] = fminf(v[k], partial[6 * b + k]);
+      v[3 + k] = fmaxf(v[3 + k], partial[6 * b + 3 + k]);
+    }
+  }
+  reduce6(v, s, minmax);
+}
+
+__device__ __forceinline__ uint32_t spread10(uint32_t x) {  // simple-knn/simple_knn.cu:45-52
+  x = (x | (x << 16)) & 0x030000FF;
+  x = (x | (x << 8)) & 0x0300F00F;
+  x = (x | (x << 4)) & 0x030C30C3;
+  x = (x | (x << 2)) & 0x09249249;
+  return x;
+}
+
+__global__ void __launch_bounds__(GS_BLOCK_1D) morton_kernel(int P, const float* __restrict__ pts,
+                                                             const float* __restrict__ minmax,
+                                                             uint32_t* __restrict__ codes, uint32_t* __restrict__ idx) {
+  const int i = blockIdx.x * GS_BLOCK_1D + threadIdx.x;
+  if (i >= P) return;
+  uint32_t c[3];
+#pragma unroll
+  for (int k = 0; k < 3; k++) {
+    const float mn = minmax[k], mx = minmax[3 + k];
+    c[k] = spread10(f2u_sat(((pts[3 * (size_t)i + k] - mn) / (mx - mn)) * (float)((1 << 10) - 1)));
+  }
+  codes[i] = c[0] | (c[1] << 1) | (c[2] << 2);
+  idx[i] = (uint32_t)i;
+}
+
+__global__ void __launch_bounds__(GS_BLOCK_1D) gather_points_kernel(int P, const float* __restrict__ pts,
+                                                                    const uint32_t* __restrict__ idx,
+                                                                    float4* __restrict__ sorted_pts) {
+  const int i = blockIdx.x * GS_BLOCK_1D + threadIdx.x;
+  if (i >= P) return;
+  const size_t g = idx[i];
+  sorted_pts[i] = make_float4(pts[3 * g], pts[3 * g + 1], pts[3 * g + 2], 0.f);
+}
+
+// simple-knn/simple_knn.cu:78-117: one workgroup per run of 1024 sorted points.
+__global__ void __launch_bounds__(MM_THREADS) box_minmax_kernel(int P, const float4* __restrict__ sorted_pts,
+                                                                float* __restrict__ boxes) {
+  __shared__ float s[6][MM_THREADS / GS_WAVE];
+  float v[6] = {FLT_MAX, FLT_MAX, FLT_MAX, -FLT_MAX, -FLT_MAX, -FLT_MAX};
+  const int start = blockIdx.x * KNN_BOX;
+  for (int t = threadIdx.x; t < KNN_BOX; t += MM_THREADS) {
+    const int i = start + t;
+    if (i < P) {
+      const float4 p = sorted_pts[i];
+      v[0] = fminf(v[0], p.x); v[1] = fminf(v[1], p.y); v[2] = fminf(v[2], p.z);
+      v[3] = fmaxf(v[3], p.x); v[4] = fmaxf(v[4], p.y); v[5] = fmaxf(v[5], p.z);
+    }
+  }
+  reduce6(v, s, boxes + 6 * blockIdx.x);
+}
+
+__device__ __forceinline__ void update3(const float4& ref, const float4& p, float* knn) {  // simple_knn.cu:131-145
+  const float dx = p.x - ref.x, dy = p.y - ref.y, dz = p.z - ref.z;
+  float dist = (dx * dx + dy * dy) + dz * dz;
+#pragma unroll
+  for (int j = 0; j < 3; j++) {
+    if (knn[j] > dist) {
+      const float t = knn[j];
+      knn[j] = dist;
+      dist = t;
+    }
+  }
+}
+
+// simple-knn/simple_knn.cu:147-183.
+__global__ void __launch_bounds__(GS_BLOCK_1D) box_mean_dist_kernel(int P, const float4* __restrict__ sorted_pts,
+                                                                    const uint32_t* __restrict__ idx,
+                                                                    const float* __restrict__ boxes, int nboxes,
+                                                                    float* __restrict__ out) {
+  const int k = blockIdx.x * GS_BLOCK_1D + threadIdx.x;
+  if (k >= P) return;
+  const float4 p = sorted_pts[k];
+  float best[3] = {FLT_MAX, FLT_MAX, FLT_MAX};
+  const int lo = max(0, k - 3), hi = min(P - 1, k + 3);
+  for (int i = lo; i <= hi; i++) {
+    if (i == k) continue;
+    update3(p, sorted_pts[i], best);
+  }
+  const float reject = best[2];
+  best[0] = best[1] = best[2] = FLT_MAX;
+  for (int b = 0; b < nboxes; b++) {
+    const float* bx = boxes + 6 * b;
+    float diff[3] = {0.f, 0.f, 0.f};
+    const float pc[3] = {p.x, p.y, p.z};
+#pragma unroll
+    for (int c = 0; c < 3; c++)
+      if (pc[c] < bx[c] || pc[c] > bx[3 + c]) diff[c] = fminf(fabsf(pc[c] - bx[c]), fabsf(pc[c] - bx[3 + c]));
+    const float dist = (diff[0] * diff[0] + diff[1] * diff[1]) + diff[2] * diff[2];
+    if (dist > reject || dist > best[2]) continue;
+    const int e = min(P, (b + 1) * KNN_BOX);
+    for (int i = b * KNN_BOX; i < e; i++) {
+      if (i == k) continue;
+      update3(p, sorted_pts[i], best);
+    }
+  }
+  out[idx[k]] = ((best[0] + best[1]) + best[2]) / 3.0f;
+}
+
+}  // namespace
+
+size_t knn_temp_bytes(int P) { return knn_layout(P).total; }
+
+int launch_knn_dist2(int P, const float* points, float* mean_dist2, void* temp, hipStream_t stream) {
+  if (P <= 0) return 0;
+  const KnnLayout L = knn_layout(P);
+  char* base = (char*)temp;
+  float* partial = (float*)(base + L.partial);
+  float* minmax = (float*)(base + L.minmax);
+  uint32_t* codes_a = (uint32_t*)(base + L.codes_a);
+  uint32_t* codes_b = (uint32_t*)(base + L.codes_b);
+  uint32_t* idx_a = (uint32_t*)(base + L.idx_a);
+  uint32_t* idx_b = (uint32_t*)(base + L.idx_b);
+  float4* sorted_pts = (float4*)(base + L.sorted_pts);
+  float* boxes = (float*)(base + L.boxes);
+  void* sort_temp = base + L.sort_temp;
+  const int blocks = (P + GS_BLOCK_1D - 1) / GS_BLOCK_1D;
+  const int nboxes = (P + KNN_BOX - 1) / KNN_BOX;
+
+  hipLaunchKernelGGL(minmax_partial_kernel, dim3(MM_BLOCKS), dim3(MM_THREADS), 0, stream, P, points, partial);
+  hipLaunchKernelGGL(minmax_final_kernel, dim3(1), dim3(MM_THREADS), 0, stream, partial, minmax);
+  hipLaunchKernelGGL(morton_kernel, dim3(blocks), dim3(GS_BLOCK_1D), 0, stream, P, points, minmax, codes_a, idx_a);
+  const int end_bit = 32;  // 4 passes (even): the sorted pairs come back in the (a) arrays
+  if (launch_sort_pairs_u32(P, codes_a, codes_b, idx_a, idx_b, end_bit, sort_temp, stream)) return 1;
+  const uint32_t* idx_sorted = sort_result_in_b(end_bit) ? idx_b : idx_a;
+  hipLaunchKernelGGL(gather_points_kernel, dim3(blocks), dim3(GS_BLOCK_1D), 0, stream, P, points, idx_sorted,
+                     sorted_pts);
+  hipLaunchKernelGGL(box_minmax_kernel, dim3(nboxes), dim3(MM_THREADS), 0, stream, P, sorted_pts, boxes);
+  hipLaunchKernelGGL(box_mean_dist_kernel, dim3(blocks), dim3(GS_BLOCK_1D), 0, stream, P, sorted_pts, idx_sorted,
+                     boxes, nboxes, mean_dist2);
+  return 0;
+}
+
+}  // namespace gs

@@ -1,0 +1,154 @@
+"""Operator API of CityGS-X's differentiable Gaussian rasterizer on MI355X.
+
+Same names, argument order, shapes, dtypes and gradient contracts as
+submodule_cityx/diff-gaussian-rasterization/diff_gaussian_rasterization/__init__.py
+(GaussianRasterizationSettings :314-327, GaussianRasterizer :329-405,
+preprocess op :46-146, render op :182-303), so gaussian_renderer/__init__.py
+and train.py can call it unchanged.  The native side is libgsrast.so
+(hand-written gfx950 kernels) reached through `_C`.
+
+One addition: passing SH coefficients shaped (P, M, 3) as `shs` makes
+preprocess evaluate colour from spherical harmonics at `sh_degree` and return
+the matching dL/dshs; any other `shs` shape keeps the reference behaviour
+(colour output zero, zero gradient of the same shape as `shs`).
+"""
+from typing import NamedTuple
+
+import torch
+import torch.nn as nn
+
+from . import _C
+
+__all__ = ["GaussianRasterizationSettings", "GaussianRasterizer", "preprocess_gaussians", "render_gaussians"]
+
+
+class GaussianRasterizationSettings(NamedTuple):
+    image_height: int
+    image_width: int
+    tanfovx: float
+    tanfovy: float
+    bg: torch.Tensor
+    scale_modifier: float
+    viewmatrix: torch.Tensor
+    projmatrix: torch.Tensor
+    sh_degree: int
+    campos: torch.Tensor
+    prefiltered: bool
+    render_geo: bool
+    debug: bool
+
+
+# --------------------------------------------------------------- preprocess --
+
+class _PreprocessGaussians(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, means3D, scales, rotations, sh, opacities, raster_settings, cuda_args):
+        rs = raster_settings
+        (num_rendered, means2D, depths, radii, cov3D, conic_opacity, rgb, clamped) = _C.preprocess_gaussians(
+            means3D, scales, rotations, sh, opacities, rs.scale_modifier, rs.viewmatrix, rs.projmatrix, rs.tanfovx,
+            rs.tanfovy, rs.image_height, rs.image_width, rs.sh_degree, rs.campos, rs.prefiltered, rs.debug, cuda_args)
+        ctx.raster_settings = rs
+        ctx.cuda_args = cuda_args
+        ctx.num_rendered = num_rendered
+        ctx.save_for_backward(means3D, scales, rotations, sh, radii, cov3D, clamped)
+        ctx.mark_non_differentiable(radii, depths)
+        return means2D, rgb, conic_opacity, radii, depths
+
+    @staticmethod
+    def backward(ctx, grad_means2D, grad_rgb, grad_conic_opacity, grad_radii, grad_depths):
+        rs = ctx.raster_settings
+        means3D, scales, rotations, sh, radii, cov3D, clamped = ctx.saved_tensors
+        dL_dmeans3D, dL_dscales, dL_drotations, dL_dsh, dL_dopacity = _C.preprocess_gaussians_backward(
+            radii, cov3D, clamped, means3D, scales, rotations, sh, rs.scale_modifier, rs.viewmatrix, rs.projmatrix,
+            rs.tanfovx, rs.tanfovy, rs.image_height, rs.image_width, rs.sh_degree, rs.campos, grad_means2D,
+            grad_conic_opacity, grad_rgb, ctx.num_rendered, rs.debug, ctx.cuda_args)
+        if dL_dsh.shape != sh.shape:
+            dL_dsh = torch.zeros_like(sh)
+        return dL_dmeans3D, dL_dscales, dL_drotations, dL_dsh, dL_dopacity, None, None
+
+
+def preprocess_gaussians(means3D, scales, rotations, sh, opacities, raster_settings, cuda_args):
+    return _PreprocessGaussians.apply(means3D, scales, rotations, sh, opacities, raster_settings, cuda_args)
+
+
+# ------------------------------------------------------------------- render --
+
+class _RenderGaussians(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, means2D, means2D_abs, conic_opacity, rgb, all_maps, depths, radii, compute_locally,
+                extended_compute_locally, raster_settings, cuda_args):
+        rs = raster_settings
+        avoid = bool(cuda_args.get("avoid_pixel_all2all", False)) if cuda_args is not None else False
+        mask = extended_compute_locally if avoid else compute_locally
+        (num_rendered, color, n_render, n_consider, n_contrib, out_observe, out_all_map, out_plane_depth, geomBuffer,
+         binningBuffer, imgBuffer) = _C.render_gaussians(
+            rs.bg, rs.image_height, rs.image_width, means2D, depths, radii, conic_opacity, rgb, mask, rs.viewmatrix,
+            rs.campos, rs.tanfovx, rs.tanfovy, all_maps, rs.render_geo, rs.debug, cuda_args)
+        ctx.raster_settings = rs
+        ctx.cuda_args = cuda_args
+        ctx.num_rendered = num_rendered
+        ctx.save_for_backward(means2D, conic_opacity, rgb, all_maps, out_all_map, geomBuffer, binningBuffer, imgBuffer,
+                              compute_locally)
+        ctx.mark_non_differentiable(n_render, n_consider, n_contrib, out_observe)
+        return color, n_render, n_consider, n_contrib, out_observe, out_all_map, out_plane_depth
+
+    @staticmethod
+    def backward(ctx, grad_color, grad_n_render, grad_n_consider, grad_n_contrib, grad_out_observe, grad_out_all_map,
+                 grad_out_plane_depth):
+        rs = ctx.raster_settings
+        (means2D, conic_opacity, rgb, all_maps, all_map_pixels, geomBuffer, binningBuffer, imgBuffer,
+         compute_locally) = ctx.saved_tensors
+        if grad_color is None:
+            grad_color = torch.zeros_like(all_map_pixels[:3])
+        if rs.render_geo:
+            if grad_out_all_map is None:
+                grad_out_all_map = torch.zeros_like(all_map_pixels)
+            if grad_out_plane_depth is None:
+                grad_out_plane_depth = torch.zeros_like(all_map_pixels[:1])
+        dL_dmeans2D, dL_dmeans2D_abs, dL_dconic_opacity, dL_dcolors, dL_dall_map = _C.render_gaussians_backward(
+            rs.bg, rs.tanfovx, rs.tanfovy, all_map_pixels, all_maps, ctx.num_rendered, geomBuffer, binningBuffer,
+            imgBuffer, compute_locally, grad_color, grad_out_all_map, grad_out_plane_depth, means2D, conic_opacity,
+            rgb, rs.render_geo, rs.debug, ctx.cuda_args)
+        return (dL_dmeans2D, dL_dmeans2D_abs, dL_dconic_opacity, dL_dcolors, dL_dall_map, None, None, None, None, None,
+                None)
+
+
+def render_gaussians(means2D, means2D_abs, conic_opacity, rgb, all_map, depths, radii, compute_locally,
+                     extended_compute_locally, raster_settings, cuda_args):
+    return _RenderGaussians.apply(means2D, means2D_abs, conic_opacity, rgb, all_map, depths, radii, compute_locally,
+                                  extended_compute_locally, raster_settings, cuda_args)
+
+
+# ------------------------------------------------------------------- module --
+
+class GaussianRasterizer(nn.Module):
+    def __init__(self, raster_settings):
+        super().__init__()
+        self.raster_settings = raster_settings
+
+    def markVisible(self, positions):
+        """Boolean mask of points in front of the camera."""
+        with torch.no_grad():
+            rs = self.raster_settings
+            return _C.mark_visible(positions, rs.viewmatrix, rs.projmatrix)
+
+    def preprocess_gaussians(self, means3D, scales, rotations, shs, opacities, cuda_args=None):
+        return preprocess_gaussians(means3D, scales, rotations, shs, opacities, self.raster_settings, cuda_args)
+
+    def visible_filter(self, means3D, scales=None, rotations=None, cov3D_precomp=None):
+        rs = self.raster_settings
+        if scales is None:
+            scales = torch.Tensor([])
+        if rotations is None:
+            rotations = torch.Tensor([])
+        if cov3D_precomp is None:
+            cov3D_precomp = torch.Tensor([])
+        with torch.no_grad():
+            return _C.rasterize_aussians_filter(means3D, scales, rotations, rs.scale_modifier, cov3D_precomp,
+                                                rs.viewmatrix, rs.projmatrix, rs.tanfovx, rs.tanfovy, rs.image_height,
+                                                rs.image_width, rs.prefiltered, rs.debug)
+
+    def render_gaussians(self, means2D, means2D_abs, conic_opacity, rgb, all_map, depths, radii, compute_locally,
+                         extended_compute_locally, cuda_args=None):
+        return render_gaussians(means2D, means2D_abs, conic_opacity, rgb, all_map, depths, radii, compute_locally,
+                                extended_compute_locally, self.raster_settings, cuda_args)

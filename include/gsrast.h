@@ -1,0 +1,220 @@
+/* C ABI of libgsrast.so: the gfx950 Gaussian rasterizer behind CityGS-X's
+ * diff_gaussian_rasterization / simple_knn operator API.
+ *
+ * Conventions
+ *   - Every pointer is a device pointer unless its comment says "host".
+ *   - The library never allocates or frees device memory.  Outputs are caller
+ *     allocated; scratch comes either from a resize callback (render forward,
+ *     like the reference's std::function<char*(size_t)> buffers) or from a
+ *     workspace whose size a *_workspace_bytes() query returns.
+ *   - stream is a hipStream_t (NULL = the default stream).  Calls are
+ *     asynchronous except where stated.
+ *   - Return value 0 = success; otherwise gs_last_error() (thread local)
+ *     describes the failure.
+ *   - debug != 0 synchronises the stream after every launch and reports the
+ *     first HIP error (cuda_rasterizer/auxiliary.h:220-227).
+ *   - Matrices are the (4,4) row-major tensors CityGS-X passes
+ *     (scene/cameras.py:124-140): p_view = [p,1] @ viewmatrix.
+ *
+ * Reference paths: CR/ = submodule_cityx/diff-gaussian-rasterization/cuda_rasterizer/,
+ * DGR/ = submodule_cityx/diff-gaussian-rasterization/, KNN/ = submodule_cityx/simple-knn/.
+ */
+#ifndef GSRAST_H_INCLUDED
+#define GSRAST_H_INCLUDED
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* gs_stream_t;
+
+/* Grows a caller-owned byte buffer to at least nbytes and returns its device
+ * address (host callback).  Replaces std::function<char*(size_t)> of
+ * CR/rasterizer.h:38-40,131-133 / DGR/rasterize_points.cu:31-37. */
+typedef char* (*gs_resize_fn)(size_t nbytes, void* user);
+
+/* Message for the last non-zero return on this thread (host string). */
+const char* gs_last_error(void);
+
+/* Replaces GetBlockXY (DGR/rasterize_points.cu:858-861): tile width, tile
+ * height and 1-D block size, i.e. (16, 16, 256).  Host pointers. */
+int gs_get_block_xy(int* block_x, int* block_y, int* one_dim_block);
+
+/* Replaces Rasterizer::markVisible (CR/rasterizer.h:30-35,
+ * CR/rasterizer_impl.cu:147-159): present[i] = (view-space z > 0). */
+int gs_mark_visible(int P, const float* means3D, const float* viewmatrix, const float* projmatrix,
+                    uint8_t* present, gs_stream_t stream);
+
+/* Replaces Rasterizer::visible_filter (CR/rasterizer.h:40-57,
+ * CR/rasterizer_impl.cu:517-573): radii only.  Either scales+rotations or
+ * cov3D_precomp may be NULL.  No scratch buffers are needed. */
+int gs_visible_filter(int P, int M, int width, int height, const float* means3D, const float* scales,
+                      float scale_modifier, const float* rotations, const float* cov3D_precomp,
+                      const float* viewmatrix, const float* projmatrix, float tan_fovx, float tan_fovy,
+                      int prefiltered, int* radii, int debug, gs_stream_t stream);
+
+/* Replaces Rasterizer::preprocessForward (CR/rasterizer.h:61-84,
+ * CR/rasterizer_impl.cu:336-425).  Shapes: means2D (P,2), depths (P), radii
+ * (P) int32, cov3D (P,6), conic_opacity (P,4), rgb (P,3), clamped (P,3) bytes.
+ * Every output element is written (zeros for culled Gaussians), so outputs
+ * need no initialisation.  shs == NULL or M == 0: colour is left zero, as in
+ * the reference (its SH call is commented out, CR/forward.cu:243-250);
+ * otherwise shs is (P,M,3) and rgb/clamped follow CR/forward.cu:21-72 at
+ * degree D.  tiles_touched (P) uint32 is optional (NULL to skip): the tile
+ * rectangle area of each surviving Gaussian (CR/forward.cu:258).
+ * prefiltered is accepted and ignored (the reference traps the GPU when a
+ * prefiltered Gaussian is culled, CR/auxiliary.h:210-214). */
+int gs_preprocess_forward(float* means2D, float* depths, int* radii, float* cov3D, float* conic_opacity,
+                          float* rgb, uint8_t* clamped, uint32_t* tiles_touched, int P, int D, int M, int width,
+                          int height, const float* means3D, const float* scales, const float* rotations,
+                          const float* shs, const float* opacities, float scale_modifier, const float* viewmatrix,
+                          const float* projmatrix, const float* cam_pos, float tan_fovx, float tan_fovy,
+                          int prefiltered, int debug, gs_stream_t stream);
+
+/* Replaces Rasterizer::preprocessBackward (CR/rasterizer.h:86-111,
+ * CR/rasterizer_impl.cu:427-489) together with the tensor repacking of
+ * PreprocessGaussiansBackwardCUDA (DGR/rasterize_points.cu:181-194):
+ * dL_dconic_opacity is the packed (P,4) gradient [conic.x, conic.y, conic.w,
+ * opacity]; dL_dmean2D has mean2D_stride (2 or 3) floats per row.  Outputs
+ * dL_dmean3D (P,3), dL_dscale (P,3), dL_drot (P,4), dL_dopacity (P) are fully
+ * written.  dL_dsh: NULL in reference-compatible mode; (P,M,3) in SH mode,
+ * where dL_dcolor (P,3) and clamped are read.  dL_dcov3D (P,6) is optional
+ * (NULL: kept in registers). */
+int gs_preprocess_backward(const int* radii, const float* cov3D, const uint8_t* clamped, int P, int D, int M,
+                           int width, int height, const float* means3D, const float* scales,
+                           const float* rotations, const float* shs, float scale_modifier,
+                           const float* viewmatrix, const float* projmatrix, const float* campos, float tan_fovx,
+                           float tan_fovy, const float* dL_dmean2D, int mean2D_stride,
+                           const float* dL_dconic_opacity, const float* dL_dcolor, float* dL_dmean3D,
+                           float* dL_dcov3D, float* dL_dscale, float* dL_drot, float* dL_dsh, float* dL_dopacity,
+                           int debug, gs_stream_t stream);
+
+/* Replaces Rasterizer::renderForward (CR/rasterizer.h:130-160,
+ * CR/rasterizer_impl.cu:586-846): tile count -> prefix sum -> host read-back of
+ * the instance count (the call blocks on the stream there, as the reference
+ * does at :653) -> key emission -> 64-bit radix sort on 32+bits(tiles) bits
+ * -> tile ranges -> blend -> per-tile statistics.
+ * out_color (3,H,W); out_all_map (5,H,W) and out_plane_depth (1,H,W) are
+ * written only when render_geo != 0; out_observe (P) int32 must arrive zeroed;
+ * n_render / n_consider / n_contrib are (tiles) int32, fully written.
+ * *num_rendered (host) receives the instance count R.
+ * elapsed_ms (host, optional): if non-NULL the call times key emission + sort
+ * + blend with events and blocks until done (the forward_render_time the
+ * reference stores at CR/rasterizer_impl.cu:754-755). */
+int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resize_fn binningBuffer,
+                      void* binning_user, gs_resize_fn imageBuffer, void* image_user, int P,
+                      const float* background, int width, int height, float focal_x, float focal_y, float cx,
+                      float cy, const float* viewmatrix, const float* cam_pos, const float* all_map,
+                      const float* means2D, const float* depths, const int* radii, const float* conic_opacity,
+                      const float* rgb, const uint8_t* compute_locally, float* out_color, int* n_render,
+                      int* n_consider, int* n_contrib, int* out_observe, float* out_all_map,
+                      float* out_plane_depth, int render_geo, int debug, int* num_rendered, float* elapsed_ms,
+                      gs_stream_t stream);
+
+/* Replaces Rasterizer::renderBackward (CR/rasterizer.h:162-187,
+ * CR/rasterizer_impl.cu:850-932) plus the repacking of
+ * RenderGaussiansBackwardCUDA (DGR/rasterize_points.cu:428-440).  The three
+ * buffers are the ones gs_render_forward filled.  Gradient outputs must
+ * arrive zeroed (they are atomic accumulation targets): dL_dmean2D (P,2),
+ * dL_dmean2D_abs (P,3), dL_dconic_opacity (P,4) packed [x, y, w, opacity],
+ * dL_dcolor (P,3), dL_dall_map (P,5).  elapsed_ms as above
+ * (backward_render_time, CR/rasterizer_impl.cu:924-926). */
+int gs_render_backward(int P, int R, const float* background, int width, int height, float tan_fovx,
+                       float tan_fovy, const char* geom_buffer, const char* binning_buffer,
+                       const char* img_buffer, const uint8_t* compute_locally, const float* dL_dpix,
+                       const float* dL_dout_all_map, const float* dL_dout_plane_depth, float* dL_dmean2D,
+                       float* dL_dmean2D_abs, float* dL_dconic_opacity, float* dL_dcolor, float* dL_dall_map,
+                       const float* means2D, const float* conic_opacity, const float* rgb, const float* all_maps,
+                       const float* all_map_pixels, int render_geo, int debug, float* elapsed_ms,
+                       gs_stream_t stream);
+
+/* Replaces SimpleKNN::knn / distCUDA2 (KNN/simple_knn.h:17, KNN/simple_knn.cu:185-221,
+ * KNN/spatial.cu:17-35): mean_dists[i] = mean squared distance from point i
+ * to its three nearest other points.  points (P,3).  The reference allocates
+ * its temporaries internally; here the caller passes a workspace of
+ * gs_knn_workspace_bytes(P) bytes. */
+size_t gs_knn_workspace_bytes(int P);
+int gs_knn_dist2(int P, const float* points, float* mean_dists, void* workspace, size_t workspace_bytes,
+                 gs_stream_t stream);
+
+/* ---- Stage-level entry points: the individual steps of renderForward, exposed
+ * so each can be checked and profiled on its own. ---- */
+
+/* updateTileTouched (CR/rasterizer_impl.cu:264-288). */
+int gs_tile_count(int P, int width, int height, const int* radii, const float* means2D,
+                  const uint8_t* compute_locally, uint32_t* tiles_touched, gs_stream_t stream);
+
+/* cub::DeviceScan::InclusiveSum as called at CR/rasterizer_impl.cu:648 (uint32). */
+size_t gs_scan_workspace_bytes(int64_t n);
+int gs_inclusive_sum(int64_t n, const uint32_t* in, uint32_t* out, void* workspace, size_t workspace_bytes,
+                     gs_stream_t stream);
+
+/* duplicateWithKeys (CR/rasterizer_impl.cu:74-117). offsets = inclusive sum of tiles_touched. */
+int gs_duplicate_with_keys(int P, int width, int height, const float* means2D, const float* depths,
+                           const uint32_t* offsets, const int* radii, const uint8_t* compute_locally,
+                           uint64_t* keys, uint32_t* values, gs_stream_t stream);
+
+/* cub::DeviceRadixSort::SortPairs on bits [0, end_bit) (CR/rasterizer_impl.cu:679-684,
+ * KNN/simple_knn.cu:210-213): stable.  The input arrays are clobbered; the
+ * sorted pairs land in keys_out / vals_out. */
+size_t gs_sort_workspace_bytes(int64_t n);
+int gs_sort_pairs_u64(int64_t n, uint64_t* keys_in, uint64_t* keys_out, uint32_t* vals_in, uint32_t* vals_out,
+                      int end_bit, void* workspace, size_t workspace_bytes, gs_stream_t stream);
+int gs_sort_pairs_u32(int64_t n, uint32_t* keys_in, uint32_t* keys_out, uint32_t* vals_in, uint32_t* vals_out,
+                      int end_bit, void* workspace, size_t workspace_bytes, gs_stream_t stream);
+
+/* getHigherMsb (CR/rasterizer_impl.cu:39-54); host function. */
+uint32_t gs_higher_msb(uint32_t n);
+
+/* memset + identifyTileRanges (CR/rasterizer_impl.cu:687-697). ranges is (tiles,2) uint32. */
+int gs_identify_tile_ranges(int64_t L, const uint64_t* keys_sorted, int tiles, uint32_t* ranges,
+                            gs_stream_t stream);
+
+/* FORWARD::render + get_n_render + 2x reduce_data_per_block
+ * (CR/forward.cu:264-437, CR/rasterizer_impl.cu:219-262). */
+int gs_render_tiles_forward(int P, int width, int height, float focal_x, float focal_y, float cx, float cy,
+                            const uint32_t* ranges, const uint32_t* point_list, const float* means2D,
+                            const float* rgb, const float* all_map, const float* conic_opacity,
+                            const uint8_t* compute_locally, const float* background, int render_geo,
+                            float* final_T, uint32_t* n_contrib_px, uint32_t* n_contrib2loss_px, float* out_color,
+                            int* out_observe, float* out_all_map, float* out_plane_depth, int* n_render,
+                            int* n_consider, int* n_contrib, gs_stream_t stream);
+
+/* BACKWARD::render (CR/backward.cu:324-567) on explicit arrays. */
+int gs_render_tiles_backward(int P, int width, int height, float tan_fovx, float tan_fovy,
+                             const float* background, const uint32_t* ranges, const uint32_t* point_list,
+                             const float* means2D, const float* conic_opacity, const float* rgb,
+                             const float* all_maps, const float* all_map_pixels, const float* final_T,
+                             const uint32_t* n_contrib_px, const uint8_t* compute_locally, const float* dL_dpix,
+                             const float* dL_dout_all_map, const float* dL_dout_plane_depth, int render_geo,
+                             float* dL_dmean2D, float* dL_dmean2D_abs, float* dL_dconic_opacity,
+                             float* dL_dcolor, float* dL_dall_map, gs_stream_t stream);
+
+/* Optional per-stage GPU timing, the role of the reference's MyTimerOnGPU
+ * (CR/timers.cu:11-79; stage names at CR/rasterizer_impl.cu:385-752): while
+ * enabled, each stage of the composite entry points (preprocess_fwd,
+ * tile_count, inclusive_sum, duplicate_with_keys, sort_pairs,
+ * identify_tile_ranges, render_fwd, render_bwd, preprocess_bwd, knn_dist2)
+ * is bracketed by an event pair on its stream.  Nothing is synchronised until
+ * gs_stage_timing_collect, which waits for the recorded events and writes one
+ * line per stage, "name total_ms launches", into report (host buffer), then
+ * clears the records.  Process wide, not thread safe. */
+int gs_stage_timing_enable(int enable);
+int gs_stage_timing_collect(char* report, size_t report_bytes);
+
+/* Byte offsets of the arrays inside the buffers gs_render_forward fills
+ * (the role of ImageState / BinningState::fromChunk, CR/rasterizer_impl.cu:182-205),
+ * relative to the 256-byte-aligned start of each buffer.  Host pointers. */
+int gs_image_state_layout(int width, int height, size_t* accum_alpha, size_t* n_contrib, size_t* n_contrib2loss,
+                          size_t* ranges, size_t* total_bytes);
+int gs_binning_state_layout(int64_t R, int width, int height, size_t* point_list, size_t* point_list_keys,
+                            size_t* point_list_unsorted, size_t* point_list_keys_unsorted, size_t* total_bytes);
+int gs_geometry_state_layout(int P, size_t* tiles_touched, size_t* point_offsets, size_t* total_bytes);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* GSRAST_H_INCLUDED */

@@ -1,0 +1,298 @@
+"""ctypes front end of the CPU oracle (libgs_oracle.so).
+
+TEST INFRASTRUCTURE ONLY: imported by tests/, the smoke check and the
+benchmark's CPU-baseline leg.  The product modules never import this file.
+
+All functions take and return numpy arrays (C-contiguous).  Shapes follow the
+reference binding (submodule_cityx/diff-gaussian-rasterization/rasterize_points.cu).
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "libgs_oracle.so")
+
+
+def build(force=False):
+    """Compile the oracle with the Makefile beside this file."""
+    if force or not os.path.exists(_LIB_PATH):
+        subprocess.check_call(["make", "-B", "-C", _HERE, "libgs_oracle.so"])
+    return _LIB_PATH
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            build()
+        _lib = C.CDLL(_LIB_PATH)
+        _lib.oracle_higher_msb.restype = C.c_uint32
+        _lib.oracle_higher_msb.argtypes = [C.c_uint32]
+        _lib.oracle_morton.restype = C.c_uint32
+        _lib.oracle_num_threads.restype = C.c_int
+    return _lib
+
+
+def _p(a):
+    if a is None:
+        return None
+    assert a.flags["C_CONTIGUOUS"]
+    return a.ctypes.data_as(C.c_void_p)
+
+
+def _f32(a):
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
+def _u8(a):
+    return np.ascontiguousarray(np.asarray(a).astype(np.uint8))
+
+
+def num_threads():
+    return lib().oracle_num_threads()
+
+
+def set_num_threads(n):
+    lib().oracle_set_num_threads(C.c_int(n))
+
+
+def expf(x):
+    x = _f32(x).ravel()
+    y = np.empty_like(x)
+    lib().oracle_expf(C.c_int(x.size), _p(x), _p(y))
+    return y
+
+
+def higher_msb(n):
+    return int(lib().oracle_higher_msb(C.c_uint32(n)))
+
+
+def tile_grid(W, H):
+    return (W + 15) // 16, (H + 15) // 16
+
+
+def mark_visible(means, V, PM):
+    means, V, PM = _f32(means), _f32(V), _f32(PM)
+    P = means.shape[0]
+    out = np.zeros(P, np.uint8)
+    lib().oracle_mark_visible(C.c_int(P), _p(means), _p(V), _p(PM), _p(out))
+    return out.astype(bool)
+
+
+def preprocess_fwd(means, scales, rots, opac, shs, V, PM, campos, W, H, tanx, tany, sh_degree=3, mod=1.0):
+    """shs is None / (P,3) (reference-compatible: colour untouched) or (P,M,3) (SH mode)."""
+    means, scales, rots, opac = _f32(means), _f32(scales), _f32(rots), _f32(opac)
+    V, PM, campos = _f32(V), _f32(PM), _f32(campos)
+    P = means.shape[0]
+    sh_mode = shs is not None and np.ndim(shs) == 3
+    M = shs.shape[1] if sh_mode else 0
+    shs_c = _f32(shs) if sh_mode else None
+    o = dict(
+        radii=np.zeros(P, np.int32),
+        means2D=np.zeros((P, 2), np.float32),
+        depths=np.zeros(P, np.float32),
+        cov3D=np.zeros((P, 6), np.float32),
+        conic_opacity=np.zeros((P, 4), np.float32),
+        rgb=np.zeros((P, 3), np.float32),
+        clamped=np.zeros((P, 3), np.uint8),
+        tiles_touched=np.zeros(P, np.uint32),
+    )
+    lib().oracle_preprocess_fwd(
+        C.c_int(P), C.c_int(sh_degree), C.c_int(M), _p(means), _p(scales), C.c_float(mod), _p(rots), _p(opac),
+        _p(shs_c), _p(V), _p(PM), _p(campos), C.c_int(W), C.c_int(H), C.c_float(tanx), C.c_float(tany),
+        _p(o["radii"]), _p(o["means2D"]), _p(o["depths"]), _p(o["cov3D"]), _p(o["conic_opacity"]), _p(o["rgb"]),
+        _p(o["clamped"]), _p(o["tiles_touched"]))
+    return o
+
+
+def visible_filter(means, scales, rots, cov_pre, V, PM, W, H, tanx, tany, mod=1.0):
+    means, V, PM = _f32(means), _f32(V), _f32(PM)
+    P = means.shape[0]
+    scales = _f32(scales) if scales is not None else None
+    rots = _f32(rots) if rots is not None else None
+    cov_pre = _f32(cov_pre) if cov_pre is not None else None
+    radii = np.zeros(P, np.int32)
+    lib().oracle_visible_filter(C.c_int(P), _p(means), _p(scales), C.c_float(mod), _p(rots), _p(cov_pre), _p(V),
+                                _p(PM), C.c_int(W), C.c_int(H), C.c_float(tanx), C.c_float(tany), _p(radii))
+    return radii
+
+
+def tiles_touched(radii, means2D, compute_locally, W, H):
+    radii = np.ascontiguousarray(radii, np.int32)
+    means2D = _f32(means2D)
+    cl = _u8(compute_locally).ravel()
+    P = radii.shape[0]
+    out = np.zeros(P, np.uint32)
+    lib().oracle_tiles_touched(C.c_int(P), C.c_int(W), C.c_int(H), _p(radii), _p(means2D), _p(cl), _p(out))
+    return out
+
+
+def inclusive_sum(x):
+    x = np.ascontiguousarray(x, np.uint32)
+    out = np.empty_like(x)
+    lib().oracle_inclusive_sum(C.c_int(x.size), _p(x), _p(out))
+    return out
+
+
+def duplicate_with_keys(means2D, depths, offsets, radii, compute_locally, W, H):
+    means2D, depths = _f32(means2D), _f32(depths)
+    offsets = np.ascontiguousarray(offsets, np.uint32)
+    radii = np.ascontiguousarray(radii, np.int32)
+    cl = _u8(compute_locally).ravel()
+    P = radii.shape[0]
+    R = int(offsets[-1]) if P else 0
+    keys = np.zeros(R, np.uint64)
+    vals = np.zeros(R, np.uint32)
+    lib().oracle_duplicate_with_keys(C.c_int(P), C.c_int(W), C.c_int(H), _p(means2D), _p(depths), _p(offsets),
+                                     _p(radii), _p(cl), _p(keys), _p(vals))
+    return keys, vals
+
+
+def sort_pairs(keys, vals, end_bit=64):
+    keys = np.ascontiguousarray(keys, np.uint64)
+    vals = np.ascontiguousarray(vals, np.uint32)
+    ko, vo = np.empty_like(keys), np.empty_like(vals)
+    lib().oracle_sort_pairs(C.c_int64(keys.size), _p(keys), _p(vals), _p(ko), _p(vo), C.c_int(end_bit))
+    return ko, vo
+
+
+def sort_pairs_u32(keys, vals):
+    keys = np.ascontiguousarray(keys, np.uint32)
+    vals = np.ascontiguousarray(vals, np.uint32)
+    ko, vo = np.empty_like(keys), np.empty_like(vals)
+    lib().oracle_sort_pairs_u32(C.c_int64(keys.size), _p(keys), _p(vals), _p(ko), _p(vo))
+    return ko, vo
+
+
+def tile_ranges(keys_sorted, T):
+    keys_sorted = np.ascontiguousarray(keys_sorted, np.uint64)
+    ranges = np.zeros((T, 2), np.uint32)
+    lib().oracle_tile_ranges(C.c_int64(keys_sorted.size), _p(keys_sorted), C.c_int(T), _p(ranges))
+    return ranges
+
+
+def bin_and_sort(radii, means2D, depths, compute_locally, W, H):
+    """updateTileTouched -> InclusiveSum -> duplicateWithKeys -> SortPairs -> identifyTileRanges
+    (renderForward, cuda_rasterizer/rasterizer_impl.cu:633-697)."""
+    gx, gy = tile_grid(W, H)
+    tt = tiles_touched(radii, means2D, compute_locally, W, H)
+    offs = inclusive_sum(tt)
+    keys, vals = duplicate_with_keys(means2D, depths, offs, radii, compute_locally, W, H)
+    bit = higher_msb(gx * gy)
+    ks, vs = sort_pairs(keys, vals, 32 + bit)
+    ranges = tile_ranges(ks, gx * gy)
+    return dict(tiles_touched=tt, point_offsets=offs, keys_unsorted=keys, vals_unsorted=vals, keys=ks,
+                point_list=vs, ranges=ranges, num_rendered=int(keys.size))
+
+
+def render_fwd(ranges, point_list, means2D, rgb, all_map, conic_opacity, compute_locally, bg, W, H, tanx, tany,
+               render_geo=True):
+    ranges = np.ascontiguousarray(ranges, np.uint32)
+    point_list = np.ascontiguousarray(point_list, np.uint32)
+    means2D, rgb, all_map, conic_opacity, bg = _f32(means2D), _f32(rgb), _f32(all_map), _f32(conic_opacity), _f32(bg)
+    cl = _u8(compute_locally).ravel()
+    P = means2D.shape[0]
+    o = dict(
+        final_T=np.zeros((H, W), np.float32),
+        n_contrib=np.zeros((H, W), np.uint32),
+        n_contrib2loss=np.zeros((H, W), np.uint32),
+        color=np.zeros((3, H, W), np.float32),
+        out_observe=np.zeros(P, np.int32),
+        out_all_map=np.zeros((5, H, W), np.float32),
+        out_plane_depth=np.zeros((1, H, W), np.float32),
+    )
+    lib().oracle_render_fwd(C.c_int(W), C.c_int(H), C.c_float(tanx), C.c_float(tany), _p(ranges), _p(point_list),
+                            _p(means2D), _p(rgb), _p(all_map), _p(conic_opacity), _p(cl), _p(bg),
+                            C.c_int(int(render_geo)), _p(o["final_T"]), _p(o["n_contrib"]), _p(o["n_contrib2loss"]),
+                            _p(o["color"]), _p(o["out_observe"]), _p(o["out_all_map"]), _p(o["out_plane_depth"]))
+    gx, gy = tile_grid(W, H)
+    T = gx * gy
+    o["n_render"] = np.zeros(T, np.int32)
+    o["n_consider"] = np.zeros(T, np.int32)
+    o["n_contrib_tile"] = np.zeros(T, np.int32)
+    lib().oracle_tile_stats(C.c_int(W), C.c_int(H), _p(ranges), _p(o["n_contrib"]), _p(o["n_contrib2loss"]), _p(cl),
+                            _p(o["n_render"]), _p(o["n_consider"]), _p(o["n_contrib_tile"]))
+    return o
+
+
+def render_bwd(ranges, point_list, means2D, conic_opacity, rgb, all_map, all_map_pixels, final_T, n_contrib,
+               compute_locally, bg, dL_dpix, dL_dout_all_map, dL_dout_plane_depth, W, H, tanx, tany, render_geo=True):
+    ranges = np.ascontiguousarray(ranges, np.uint32)
+    point_list = np.ascontiguousarray(point_list, np.uint32)
+    means2D, rgb, all_map, conic_opacity, bg = _f32(means2D), _f32(rgb), _f32(all_map), _f32(conic_opacity), _f32(bg)
+    all_map_pixels, final_T = _f32(all_map_pixels), _f32(final_T)
+    n_contrib = np.ascontiguousarray(n_contrib, np.uint32)
+    dL_dpix, dL_dout_all_map, dL_dout_plane_depth = _f32(dL_dpix), _f32(dL_dout_all_map), _f32(dL_dout_plane_depth)
+    cl = _u8(compute_locally).ravel()
+    P = means2D.shape[0]
+    o = dict(
+        dL_dmeans2D=np.zeros((P, 3), np.float32),
+        dL_dmeans2D_abs=np.zeros((P, 3), np.float32),
+        dL_dconic=np.zeros((P, 4), np.float32),
+        dL_dopacity=np.zeros((P, 1), np.float32),
+        dL_dcolors=np.zeros((P, 3), np.float32),
+        dL_dall_map=np.zeros((P, 5), np.float32),
+    )
+    lib().oracle_render_bwd(C.c_int(P), C.c_int(W), C.c_int(H), C.c_float(tanx), C.c_float(tany), _p(bg), _p(ranges),
+                            _p(point_list), _p(means2D), _p(conic_opacity), _p(rgb), _p(all_map), _p(all_map_pixels),
+                            _p(final_T), _p(n_contrib), _p(cl), _p(dL_dpix), _p(dL_dout_all_map),
+                            _p(dL_dout_plane_depth), C.c_int(int(render_geo)), _p(o["dL_dmeans2D"]),
+                            _p(o["dL_dmeans2D_abs"]), _p(o["dL_dconic"]), _p(o["dL_dopacity"]), _p(o["dL_dcolors"]),
+                            _p(o["dL_dall_map"]))
+    # packed form returned by the binding (rasterize_points.cu:428-440): [conic.x, conic.y, conic.w, opacity]
+    d = o["dL_dconic"]
+    o["dL_dconic_opacity"] = np.stack([d[:, 0], d[:, 1], d[:, 3], o["dL_dopacity"][:, 0]], axis=1)
+    return o
+
+
+def preprocess_bwd(means, radii, shs, clamped, scales, rots, cov3D, V, PM, campos, W, H, tanx, tany, dL_dmeans2D,
+                   dL_dconic_opacity, dL_dcolor, sh_degree=3, mod=1.0):
+    """dL_dmeans2D (P,2) or (P,3); dL_dconic_opacity (P,4) packed [x, y, w, opacity]
+    (rasterize_points.cu:181-194).  Returns the five gradients of the binding."""
+    means, scales, rots, cov3D = _f32(means), _f32(scales), _f32(rots), _f32(cov3D)
+    V, PM, campos = _f32(V), _f32(PM), _f32(campos)
+    radii = np.ascontiguousarray(radii, np.int32)
+    P = means.shape[0]
+    sh_mode = shs is not None and np.ndim(shs) == 3
+    M = shs.shape[1] if sh_mode else 0
+    shs_c = _f32(shs) if sh_mode else None
+    g2 = np.zeros((P, 3), np.float32)
+    g2[:, :2] = _f32(dL_dmeans2D)[:, :2]
+    gco = _f32(dL_dconic_opacity)
+    gconic = np.zeros((P, 4), np.float32)
+    gconic[:, 0], gconic[:, 1], gconic[:, 3] = gco[:, 0], gco[:, 1], gco[:, 2]
+    gcol = _f32(dL_dcolor) if dL_dcolor is not None else np.zeros((P, 3), np.float32)
+    cl = _u8(clamped) if clamped is not None else np.zeros((P, 3), np.uint8)
+    o = dict(
+        dL_dmeans3D=np.zeros((P, 3), np.float32),
+        dL_dcov3D=np.zeros((P, 6), np.float32),
+        dL_dscales=np.zeros((P, 3), np.float32),
+        dL_drotations=np.zeros((P, 4), np.float32),
+        dL_dsh=np.zeros((P, M, 3) if sh_mode else (P, 3), np.float32),
+        dL_dopacity=gco[:, 3:4].copy(),
+    )
+    lib().oracle_preprocess_bwd(C.c_int(P), C.c_int(sh_degree), C.c_int(M), _p(means), _p(radii), _p(shs_c), _p(cl),
+                                _p(scales), _p(rots), C.c_float(mod), _p(cov3D), _p(V), _p(PM), C.c_int(W), C.c_int(H),
+                                C.c_float(tanx), C.c_float(tany), _p(campos), _p(g2), _p(gconic), _p(gcol),
+                                _p(o["dL_dmeans3D"]), _p(o["dL_dcov3D"]), _p(o["dL_dsh"]) if sh_mode else None,
+                                _p(o["dL_dscales"]), _p(o["dL_drotations"]))
+    return o
+
+
+def knn_dist2(points):
+    points = _f32(points)
+    P = points.shape[0]
+    out = np.zeros(P, np.float32)
+    lib().oracle_knn_dist2(C.c_int(P), _p(points), _p(out))
+    return out
+
+
+def morton(p, mn, mx):
+    p, mn, mx = _f32(p), _f32(mn), _f32(mx)
+    return int(lib().oracle_morton(_p(p), _p(mn), _p(mx)))

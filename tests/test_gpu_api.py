@@ -1,0 +1,201 @@
+"""The Python operator API (GaussianRasterizationSettings / GaussianRasterizer /
+distCUDA2) end to end on the GPU, with the call sequence CityGS-X uses
+(visible_filter -> preprocess -> all_map in torch -> render -> backward), against
+the CPU oracle running the same sequence."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+def _settings(cam, render_geo=True, sh_degree=3, bg=(0.0, 0.0, 0.0)):
+    from diff_gaussian_rasterization import GaussianRasterizationSettings
+    return GaussianRasterizationSettings(
+        image_height=cam.image_height, image_width=cam.image_width, tanfovx=cam.tanfovx, tanfovy=cam.tanfovy,
+        bg=torch.tensor(bg, dtype=torch.float32, device=DEV), scale_modifier=1.0,
+        viewmatrix=cam.world_view_transform.to(DEV), projmatrix=cam.full_proj_transform.to(DEV), sh_degree=sh_degree,
+        campos=cam.camera_center.to(DEV), prefiltered=False, render_geo=render_geo, debug=False)
+
+
+def _cuda_args():
+    return {"mode": "train", "global_rank": "0", "world_size": "1", "iteration": "1", "log_interval": "10",
+            "log_folder": "/tmp", "zhx_debug": "False", "zhx_time": "False", "avoid_pixel_all2all": False,
+            "stats_collector": {}}
+
+
+def _rel(a, b):
+    a, b = np.asarray(a, np.float64), np.asarray(b, np.float64)
+    return np.linalg.norm(a - b) / max(np.linalg.norm(b), 1e-30)
+
+
+def test_block_xy_and_module_surface():
+    import diff_gaussian_rasterization as dgr
+    assert dgr._C.get_block_XY() == (16, 16, 256)
+    with pytest.raises(RuntimeError, match="deprecated"):
+        dgr._C.get_distribution_strategy()
+    with pytest.raises(NotImplementedError):
+        dgr._C.get_local2j_ids_bool()
+
+
+@pytest.mark.parametrize("cfg,P,sh_mode", [(0, 50_000, True), (1, 150_000, True), (1, 150_000, False)])
+def test_full_pipeline_matches_oracle(orc, cfg, P, sh_mode):
+    import gs_scenes
+    from diff_gaussian_rasterization import GaussianRasterizer
+    g, cams = gs_scenes.make_scene(cfg, P=P, n_views=1)
+    cam = cams[0]
+    W, H = cam.image_width, cam.image_height
+    rs = _settings(cam)
+    rast = GaussianRasterizer(rs)
+    leaf = {k: g[k].to(DEV).requires_grad_(True) for k in ("means3D", "scales", "rotations", "opacities", "shs")}
+    mlp_rgb = torch.rand(P, 3, generator=torch.Generator().manual_seed(3)).to(DEV).requires_grad_(True)
+    cuda_args = _cuda_args()
+
+    vis = rast.visible_filter(leaf["means3D"].detach(), leaf["scales"].detach(), leaf["rotations"].detach())
+    shs_arg = leaf["shs"] if sh_mode else mlp_rgb
+    means2D, rgb, conic_opacity, radii, depths = rast.preprocess_gaussians(
+        leaf["means3D"], leaf["scales"], leaf["rotations"], shs_arg, leaf["opacities"], cuda_args)
+    assert means2D.shape == (P, 2) and rgb.shape == (P, 3) and conic_opacity.shape == (P, 4)
+    assert radii.dtype == torch.int32 and radii.shape == (P,) and depths.shape == (P,)
+    assert not radii.requires_grad and not depths.requires_grad
+    assert torch.equal(vis, radii)
+    means2D.retain_grad()
+    all_map = gs_scenes.build_all_map(leaf["means3D"], leaf["scales"], leaf["rotations"], cam)
+    gx, gy = (W + 15) // 16, (H + 15) // 16
+    cl = torch.ones(gy, gx, dtype=torch.bool, device=DEV)
+    means2D_abs = torch.zeros_like(leaf["means3D"], requires_grad=True) + 0
+    means2D_abs.retain_grad()
+    colour_in = rgb if sh_mode else mlp_rgb
+    color, n_render, n_consider, n_contrib, out_observe, out_all_map, out_plane_depth = rast.render_gaussians(
+        means2D, means2D_abs, conic_opacity, colour_in, all_map, depths, radii, cl, cl, cuda_args)
+    assert color.shape == (3, H, W) and out_all_map.shape == (5, H, W) and out_plane_depth.shape == (1, H, W)
+    assert n_render.shape == (gx * gy,) and n_render.dtype == torch.int32 and out_observe.shape == (P,)
+    assert "forward_render_time" in cuda_args["stats_collector"]
+    ug = gs_scenes.upstream_grads(cam)
+    loss = (color * ug["color"].to(DEV)).sum() + (out_all_map * ug["all_map"].to(DEV)).sum() + \
+        (out_plane_depth * ug["plane_depth"].to(DEV)).sum()
+    loss.backward()
+    assert "backward_render_time" in cuda_args["stats_collector"]
+
+    # ---- oracle, same sequence
+    n = lambda t: t.detach().cpu().numpy()
+    pre = orc.preprocess_fwd(n(g["means3D"]), n(g["scales"]), n(g["rotations"]), n(g["opacities"]),
+                             n(g["shs"]) if sh_mode else None, n(cam.world_view_transform), n(cam.full_proj_transform),
+                             n(cam.camera_center), W, H, cam.tanfovx, cam.tanfovy)
+    assert np.array_equal(n(radii), pre["radii"])
+    cl_np = np.ones(gx * gy, bool)
+    b = orc.bin_and_sort(pre["radii"], pre["means2D"], pre["depths"], cl_np, W, H)
+    am = n(all_map)
+    col_np = pre["rgb"] if sh_mode else n(mlp_rgb)
+    f = orc.render_fwd(b["ranges"], b["point_list"], pre["means2D"], col_np, am, pre["conic_opacity"], cl_np,
+                       np.zeros(3, np.float32), W, H, cam.tanfovx, cam.tanfovy)
+    assert np.abs(n(color) - f["color"]).max() <= 1e-4
+    assert np.abs(n(out_all_map) - f["out_all_map"]).max() <= 1e-4
+    assert np.array_equal(n(n_render), f["n_render"])
+    assert np.array_equal(n(n_consider), f["n_consider"])
+    assert np.array_equal(n(n_contrib), f["n_contrib_tile"])
+    assert np.array_equal(n(out_observe), f["out_observe"])
+    rb = orc.render_bwd(b["ranges"], b["point_list"], pre["means2D"], pre["conic_opacity"], col_np, am,
+                        f["out_all_map"], f["final_T"], f["n_contrib"], cl_np, np.zeros(3, np.float32), n(ug["color"]),
+                        n(ug["all_map"]), n(ug["plane_depth"]), W, H, cam.tanfovx, cam.tanfovy)
+    assert _rel(n(means2D.grad), rb["dL_dmeans2D"][:, :2]) <= 1e-3
+    assert _rel(n(means2D_abs.grad), rb["dL_dmeans2D_abs"]) <= 1e-3
+    pb = orc.preprocess_bwd(n(g["means3D"]), pre["radii"], n(g["shs"]) if sh_mode else None, pre["clamped"],
+                            n(g["scales"]), n(g["rotations"]), pre["cov3D"], n(cam.world_view_transform),
+                            n(cam.full_proj_transform), n(cam.camera_center), W, H, cam.tanfovx, cam.tanfovy,
+                            rb["dL_dmeans2D"], rb["dL_dconic_opacity"], rb["dL_dcolors"])
+    # all_map is built in torch from the same leaves, so its autograd path adds to these leaves;
+    # compare the opacity and SH/colour gradients, which only flow through the rasterizer ops
+    assert _rel(n(leaf["opacities"].grad), pb["dL_dopacity"]) <= 1e-3
+    if sh_mode:
+        assert leaf["shs"].grad.shape == (P, 16, 3)
+        assert _rel(n(leaf["shs"].grad), pb["dL_dsh"]) <= 1e-3
+    else:
+        assert mlp_rgb.grad.shape == (P, 3)
+        assert _rel(n(mlp_rgb.grad), rb["dL_dcolors"]) <= 1e-3
+    for k in ("means3D", "scales", "rotations"):
+        assert leaf[k].grad is not None and torch.isfinite(leaf[k].grad).all()
+
+
+def test_rasterizer_only_grads_match_oracle(orc):
+    """all_map detached, so the leaves' gradients come from the two rasterizer ops alone."""
+    import gs_scenes
+    from diff_gaussian_rasterization import GaussianRasterizer
+    P = 120_000
+    g, cams = gs_scenes.make_scene(1, P=P, n_views=1)
+    cam = cams[0]
+    W, H = cam.image_width, cam.image_height
+    rast = GaussianRasterizer(_settings(cam, bg=(0.1, 0.2, 0.3)))
+    leaf = {k: g[k].to(DEV).requires_grad_(True) for k in ("means3D", "scales", "rotations", "opacities", "shs")}
+    ca = _cuda_args()
+    means2D, rgb, co, radii, depths = rast.preprocess_gaussians(leaf["means3D"], leaf["scales"], leaf["rotations"],
+                                                                leaf["shs"], leaf["opacities"], ca)
+    am = gs_scenes.build_all_map(g["means3D"], g["scales"], g["rotations"], cam).to(DEV)
+    gx, gy = (W + 15) // 16, (H + 15) // 16
+    cl = torch.ones(gy, gx, dtype=torch.bool, device=DEV)
+    m2abs = torch.zeros(P, 3, device=DEV, requires_grad=True)
+    color, _, _, _, _, oam, opd = rast.render_gaussians(means2D, m2abs, co, rgb, am, depths, radii, cl, cl, ca)
+    ug = gs_scenes.upstream_grads(cam)
+    ((color * ug["color"].to(DEV)).sum() + (oam * ug["all_map"].to(DEV)).sum() +
+     (opd * ug["plane_depth"].to(DEV)).sum()).backward()
+    n = lambda t: t.detach().cpu().numpy()
+    pre = orc.preprocess_fwd(n(g["means3D"]), n(g["scales"]), n(g["rotations"]), n(g["opacities"]), n(g["shs"]),
+                             n(cam.world_view_transform), n(cam.full_proj_transform), n(cam.camera_center), W, H,
+                             cam.tanfovx, cam.tanfovy)
+    cl_np = np.ones(gx * gy, bool)
+    b = orc.bin_and_sort(pre["radii"], pre["means2D"], pre["depths"], cl_np, W, H)
+    bg = np.array([0.1, 0.2, 0.3], np.float32)
+    f = orc.render_fwd(b["ranges"], b["point_list"], pre["means2D"], pre["rgb"], n(am), pre["conic_opacity"], cl_np, bg,
+                       W, H, cam.tanfovx, cam.tanfovy)
+    rb = orc.render_bwd(b["ranges"], b["point_list"], pre["means2D"], pre["conic_opacity"], pre["rgb"], n(am),
+                        f["out_all_map"], f["final_T"], f["n_contrib"], cl_np, bg, n(ug["color"]), n(ug["all_map"]),
+                        n(ug["plane_depth"]), W, H, cam.tanfovx, cam.tanfovy)
+    pb = orc.preprocess_bwd(n(g["means3D"]), pre["radii"], n(g["shs"]), pre["clamped"], n(g["scales"]),
+                            n(g["rotations"]), pre["cov3D"], n(cam.world_view_transform), n(cam.full_proj_transform),
+                            n(cam.camera_center), W, H, cam.tanfovx, cam.tanfovy, rb["dL_dmeans2D"],
+                            rb["dL_dconic_opacity"], rb["dL_dcolors"])
+    for k, r in (("means3D", "dL_dmeans3D"), ("scales", "dL_dscales"), ("rotations", "dL_drotations"),
+                 ("opacities", "dL_dopacity"), ("shs", "dL_dsh")):
+        assert _rel(n(leaf[k].grad), pb[r]) <= 1e-3, k
+    assert _rel(n(m2abs.grad), rb["dL_dmeans2D_abs"]) <= 1e-3
+
+
+def test_empty_inputs_and_errors():
+    import gs_scenes
+    from diff_gaussian_rasterization import GaussianRasterizer
+    cam = gs_scenes.make_scene(0, P=10)[1][0]
+    rast = GaussianRasterizer(_settings(cam))
+    z = lambda *s: torch.zeros(*s, device=DEV)
+    m2, rgb, co, radii, depths = rast.preprocess_gaussians(z(0, 3), z(0, 3), z(0, 4), z(0, 3), z(0, 1), _cuda_args())
+    assert m2.shape == (0, 2) and radii.shape == (0,)
+    gx, gy = (cam.image_width + 15) // 16, (cam.image_height + 15) // 16
+    cl = torch.ones(gy, gx, dtype=torch.bool, device=DEV)
+    out = rast.render_gaussians(m2, z(0, 3), co, rgb, z(0, 5), depths, radii, cl, cl, _cuda_args())
+    assert out[0].shape == (3, cam.image_height, cam.image_width) and float(out[0].abs().max()) == 0.0
+    assert rast.visible_filter(z(0, 3), z(0, 3), z(0, 4)).shape == (0,)
+    with pytest.raises(RuntimeError, match="num_points, 3"):
+        rast.preprocess_gaussians(z(5, 2), z(5, 3), z(5, 4), z(5, 3), z(5, 1), _cuda_args())
+    with pytest.raises(RuntimeError, match="GPU tensor"):
+        rast.preprocess_gaussians(torch.zeros(5, 3), z(5, 3), z(5, 4), z(5, 3), z(5, 1), _cuda_args())
+
+
+def test_all_gaussians_behind_camera_renders_background():
+    import gs_scenes
+    from diff_gaussian_rasterization import GaussianRasterizer
+    g, cams = gs_scenes.make_scene(0, P=1000)
+    cam = cams[0]
+    rast = GaussianRasterizer(_settings(cam, bg=(0.25, 0.5, 0.75)))
+    means = g["means3D"].clone()
+    means[:, 2] = -100.0  # camera sits at z=-30 looking towards +z
+    m2, rgb, co, radii, depths = rast.preprocess_gaussians(means.to(DEV), g["scales"].to(DEV), g["rotations"].to(DEV),
+                                                           g["shs"].to(DEV), g["opacities"].to(DEV), _cuda_args())
+    assert int(radii.max()) == 0
+    gx, gy = (cam.image_width + 15) // 16, (cam.image_height + 15) // 16
+    cl = torch.ones(gy, gx, dtype=torch.bool, device=DEV)
+    color, n_render, *_ = rast.render_gaussians(m2, torch.zeros(1000, 3, device=DEV), co, rgb,
+                                                torch.zeros(1000, 5, device=DEV), depths, radii, cl, cl, _cuda_args())
+    assert int(n_render.sum()) == 0
+    assert torch.allclose(color[:, 0, 0].cpu(), torch.tensor([0.25, 0.5, 0.75]))
+    assert float((color - color[:, :1, :1]).abs().max()) == 0.0

@@ -1,0 +1,84 @@
+"""GPU radix sort and k-NN against library routines / brute force."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def H():
+    import gpu_harness
+    assert torch.cuda.is_available()
+    return gpu_harness
+
+
+@pytest.mark.parametrize("n", [1, 2, 63, 64, 65, 255, 2047, 2048, 2049, 100_003, 1_500_000])
+@pytest.mark.parametrize("end_bit", [44, 45, 64, 33, 40])
+def test_sort_pairs_u64(H, n, end_bit):
+    rng = np.random.default_rng(n * 131 + end_bit)
+    tile_bits = max(1, end_bit - 32)
+    # few distinct depths per tile so ties exercise stability
+    tiles = rng.integers(0, 1 << min(tile_bits, 12), n, dtype=np.uint64)
+    depth = rng.integers(0, 50, n, dtype=np.uint64) * np.uint64(0x01010101)
+    keys = (tiles << np.uint64(32)) | depth
+    if end_bit < 64:
+        # garbage above end_bit must be ignored by the comparison and carried along unchanged
+        keys |= rng.integers(0, 2, n, dtype=np.uint64) << np.uint64(min(63, end_bit + 3))
+    vals = np.arange(n, dtype=np.uint32)
+    ko, vo = H.sort_pairs_u64(H.as_u64(keys), H.as_u32(vals), end_bit)
+    mask = np.uint64((1 << end_bit) - 1) if end_bit < 64 else np.uint64(0xFFFFFFFFFFFFFFFF)
+    order = np.argsort(keys & mask, kind="stable")
+    assert np.array_equal(H.np_u32(vo), vals[order])
+    assert np.array_equal(H.np_u64(ko), keys[order])
+
+
+@pytest.mark.parametrize("n", [1, 1000, 2048, 4097, 777_777])
+def test_sort_pairs_u32(H, n):
+    rng = np.random.default_rng(n)
+    keys = rng.integers(0, 1 << 30, n, dtype=np.uint32)
+    keys[rng.integers(0, n, n // 3)] = keys[0]
+    vals = rng.permutation(n).astype(np.uint32)
+    ko, vo = H.sort_pairs_u32(H.as_u32(keys), H.as_u32(vals))
+    order = np.argsort(keys, kind="stable")
+    assert np.array_equal(H.np_u32(ko), keys[order])
+    assert np.array_equal(H.np_u32(vo), vals[order])
+
+
+@pytest.mark.parametrize("n", [1, 5, 2047, 2048, 2049, 1_000_001])
+def test_inclusive_sum(H, n):
+    rng = np.random.default_rng(n)
+    x = rng.integers(0, 9, n, dtype=np.uint32)
+    out = torch.empty(n, dtype=torch.int32, device=H.DEV)
+    nb = H.lib.gs_scan_workspace_bytes(n)
+    ws = torch.empty(nb, dtype=torch.uint8, device=H.DEV)
+    H.gn.check(H.lib.gs_inclusive_sum(n, H.ptr(H.as_u32(x)), H.ptr(out), H.ptr(ws), nb, H.stream()), "scan")
+    torch.cuda.synchronize()
+    assert np.array_equal(H.np_u32(out), np.cumsum(x, dtype=np.uint64).astype(np.uint32))
+
+
+def _brute(points):
+    from scipy.spatial import cKDTree
+    d, _ = cKDTree(points.astype(np.float64)).query(points.astype(np.float64), k=4)
+    return (d[:, 1:] ** 2).mean(axis=1)
+
+
+@pytest.mark.parametrize("P,kind", [(7, "uniform"), (1024, "uniform"), (1025, "uniform"), (20_000, "uniform"),
+                                    (20_000, "positive"), (50_000, "clustered"), (300_000, "slab")])
+def test_knn_dist2(H, orc, P, kind):
+    import simple_knn._C as knn
+    rng = np.random.default_rng(P)
+    if kind == "uniform":
+        pts = rng.uniform(-10, 10, (P, 3))
+    elif kind == "positive":
+        pts = rng.uniform(5, 25, (P, 3))  # the zero-initialised bounding box reduction matters here
+    elif kind == "clustered":
+        pts = rng.normal(0, 1, (P, 3)) + rng.integers(0, 4, (P, 1)) * 30.0
+    else:
+        pts = rng.uniform(0, 1, (P, 3)) * np.array([200.0, 200.0, 30.0]) - np.array([100.0, 100.0, 0.0])
+    pts = pts.astype(np.float32)
+    got = knn.distCUDA2(torch.from_numpy(pts).to(H.DEV)).cpu().numpy()
+    ref = orc.knn_dist2(pts)
+    assert np.array_equal(got, ref), f"max abs diff {np.abs(got - ref).max()}"
+    if P <= 50_000:
+        np.testing.assert_allclose(got, _brute(pts), rtol=2e-4, atol=1e-9)

@@ -1,0 +1,215 @@
+"""GPU parity of every stage of the rasterizer against the CPU oracle, through
+the C ABI.  Integer and index outputs must be identical; images within 1e-4
+absolute; gradients within 1e-3 relative L2."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+IMG_TOL = 1e-4
+GRAD_TOL = 1e-3
+
+
+@pytest.fixture(scope="module")
+def H():
+    import gpu_harness
+    assert torch.cuda.is_available()
+    return gpu_harness
+
+
+def _scene(cfg, P):
+    import gs_scenes
+    g, cams = gs_scenes.make_scene(cfg, P=P, n_views=1)
+    return g, cams[0]
+
+
+CASES = [(0, 50_000), (1, 200_000), (3, 60_000)]
+
+
+@pytest.mark.parametrize("cfg,P", CASES)
+@pytest.mark.parametrize("sh_mode", [True, False])
+def test_preprocess_forward(H, orc, cfg, P, sh_mode):
+    g, cam = _scene(cfg, P)
+    got, _ = H.preprocess_fwd(g, cam, sh_mode=sh_mode)
+    ref = H.oracle_preprocess(orc, g, cam, sh_mode=sh_mode)
+    assert np.array_equal(got["radii"].cpu().numpy(), ref["radii"])
+    assert np.array_equal(H.np_u32(got["tiles_touched"]), ref["tiles_touched"])
+    # depth feeds the sort key: bits must agree
+    assert np.array_equal(H.np_u32(got["depths"].view(torch.int32)), ref["depths"].view(np.uint32))
+    assert np.array_equal(got["clamped"].cpu().numpy(), ref["clamped"])
+    for k in ("means2D", "cov3D", "conic_opacity", "rgb"):
+        a, b = got[k].cpu().numpy(), ref[k]
+        assert np.array_equal(a, b), f"{k}: max abs diff {np.abs(a - b).max()}"
+    assert (ref["radii"] > 0).any() and (ref["radii"] == 0).any() or cfg == 0
+
+
+@pytest.mark.parametrize("cfg,P", CASES)
+def test_visible_filter_and_mark_visible(H, orc, cfg, P):
+    import ctypes as C
+    g, cam = _scene(cfg, P)
+    gd = {k: H.dev(v) for k, v in g.items() if torch.is_tensor(v)}
+    V, PM = H.dev(cam.world_view_transform), H.dev(cam.full_proj_transform)
+    W, Hh = cam.image_width, cam.image_height
+    radii = torch.full((P,), 9, dtype=torch.int32, device=H.DEV)
+    H.gn.check(H.lib.gs_visible_filter(P, 0, W, Hh, H.ptr(gd["means3D"]), H.ptr(gd["scales"]), 1.0,
+                                       H.ptr(gd["rotations"]), None, H.ptr(V), H.ptr(PM), cam.tanfovx, cam.tanfovy, 0,
+                                       H.ptr(radii), 1, H.stream()), "gs_visible_filter")
+    n = lambda t: t.numpy()
+    ref = orc.visible_filter(n(g["means3D"]), n(g["scales"]), n(g["rotations"]), None, n(cam.world_view_transform),
+                             n(cam.full_proj_transform), W, Hh, cam.tanfovx, cam.tanfovy)
+    assert np.array_equal(radii.cpu().numpy(), ref)
+    # with a precomputed covariance instead of scale/rotation
+    pre = H.oracle_preprocess(orc, g, cam, sh_mode=False)
+    cov = H.dev(pre["cov3D"])
+    radii2 = torch.full((P,), 9, dtype=torch.int32, device=H.DEV)
+    H.gn.check(H.lib.gs_visible_filter(P, 0, W, Hh, H.ptr(gd["means3D"]), None, 1.0, None, H.ptr(cov), H.ptr(V),
+                                       H.ptr(PM), cam.tanfovx, cam.tanfovy, 0, H.ptr(radii2), 1, H.stream()),
+               "gs_visible_filter")
+    ref2 = orc.visible_filter(n(g["means3D"]), None, None, pre["cov3D"], n(cam.world_view_transform),
+                              n(cam.full_proj_transform), W, Hh, cam.tanfovx, cam.tanfovy)
+    assert np.array_equal(radii2.cpu().numpy(), ref2)
+    present = torch.full((P,), 7, dtype=torch.uint8, device=H.DEV)
+    H.gn.check(H.lib.gs_mark_visible(P, H.ptr(gd["means3D"]), H.ptr(V), H.ptr(PM), H.ptr(present), H.stream()),
+               "gs_mark_visible")
+    assert np.array_equal(present.cpu().numpy().astype(bool),
+                          orc.mark_visible(n(g["means3D"]), n(cam.world_view_transform), n(cam.full_proj_transform)))
+
+
+def _mask(kind, gx, gy):
+    cl = np.ones((gy, gx), bool)
+    if kind == "rows":
+        cl[: gy // 3] = False
+    elif kind == "checker":
+        cl[::2, ::2] = False
+    return cl.ravel()
+
+
+@pytest.mark.parametrize("cfg,P,mask", [(0, 50_000, "all"), (1, 200_000, "all"), (1, 100_000, "rows"),
+                                        (3, 60_000, "checker")])
+def test_binning_stages(H, orc, cfg, P, mask):
+    g, cam = _scene(cfg, P)
+    W, Hh = cam.image_width, cam.image_height
+    gx, gy = H.grid(W, Hh)
+    pre = H.oracle_preprocess(orc, g, cam)
+    cl = _mask(mask, gx, gy)
+    ref = orc.bin_and_sort(pre["radii"], pre["means2D"], pre["depths"], cl, W, Hh)
+    got = H.bin_stages(H.dev(pre["radii"]), H.dev(pre["means2D"]), H.dev(pre["depths"]), H.dev(cl), W, Hh)
+    assert got["num_rendered"] == ref["num_rendered"] > 0
+    for k in ("tiles_touched", "point_offsets", "keys_unsorted", "vals_unsorted", "keys", "point_list", "ranges"):
+        assert np.array_equal(got[k], ref[k]), k
+
+
+def _render_inputs(H, orc, cfg, P, mask="all"):
+    import gs_scenes
+    g, cam = _scene(cfg, P)
+    W, Hh = cam.image_width, cam.image_height
+    gx, gy = H.grid(W, Hh)
+    pre = H.oracle_preprocess(orc, g, cam)
+    cl = _mask(mask, gx, gy)
+    b = orc.bin_and_sort(pre["radii"], pre["means2D"], pre["depths"], cl, W, Hh)
+    am = gs_scenes.build_all_map(g["means3D"], g["scales"], g["rotations"], cam).numpy()
+    return g, cam, pre, cl, b, am
+
+
+@pytest.mark.parametrize("cfg,P,mask,geo,bgv", [(0, 50_000, "all", True, 0.0), (1, 200_000, "all", True, 0.3),
+                                                (1, 100_000, "rows", True, 0.0), (3, 60_000, "all", False, 1.0),
+                                                (3, 60_000, "checker", True, 0.5)])
+def test_render_forward(H, orc, cfg, P, mask, geo, bgv):
+    g, cam, pre, cl, b, am = _render_inputs(H, orc, cfg, P, mask)
+    W, Hh = cam.image_width, cam.image_height
+    bg = np.array([bgv, 0.5 * bgv, 1.0 - bgv], np.float32)
+    ref = orc.render_fwd(b["ranges"], b["point_list"], pre["means2D"], pre["rgb"], am, pre["conic_opacity"], cl, bg, W,
+                         Hh, cam.tanfovx, cam.tanfovy, render_geo=geo)
+    got = H.render_fwd(P, W, Hh, cam.tanfovx, cam.tanfovy, H.as_u32(b["ranges"]), H.as_u32(b["point_list"]),
+                       H.dev(pre["means2D"]), H.dev(pre["rgb"]), H.dev(am), H.dev(pre["conic_opacity"]), H.dev(cl),
+                       H.dev(bg), render_geo=geo)
+    gx, gy = H.grid(W, Hh)
+    # pixels of tiles that are not computed locally are left untouched by both sides
+    pix_local = np.repeat(np.repeat(cl.reshape(gy, gx), 16, 0), 16, 1)[:Hh, :W]
+    for k in ("n_contrib", "n_contrib2loss"):
+        assert np.array_equal(H.np_u32(got[k])[pix_local], ref[k][pix_local]), k
+    assert np.array_equal(got["out_observe"].cpu().numpy(), ref["out_observe"])
+    for k in ("n_render", "n_consider", "n_contrib_tile"):
+        assert np.array_equal(got[k].cpu().numpy(), ref[k]), k
+    assert np.abs(got["final_T"].cpu().numpy() - ref["final_T"])[pix_local].max() <= IMG_TOL
+    keys = ("color", "out_all_map", "out_plane_depth") if geo else ("color",)
+    for k in keys:
+        a, r = got[k].cpu().numpy()[:, pix_local], ref[k][:, pix_local]
+        if k == "out_plane_depth":
+            # a ratio: compare where the denominator is not tiny
+            ok = np.isfinite(r) & (np.abs(r) < 1e4)
+            assert np.abs(a - r)[ok].max() <= IMG_TOL * np.maximum(1.0, np.abs(r[ok])).max(), k
+        else:
+            assert np.abs(a - r).max() <= IMG_TOL, f"{k}: {np.abs(a - r).max()}"
+    if not geo:
+        assert float(got["out_all_map"].abs().max()) == 0.0 and float(got["out_plane_depth"].abs().max()) == 0.0
+
+
+@pytest.mark.parametrize("cfg,P,mask,geo", [(0, 50_000, "all", True), (1, 200_000, "all", True),
+                                            (1, 100_000, "rows", True), (3, 60_000, "all", False)])
+def test_render_backward(H, orc, cfg, P, mask, geo):
+    import gs_scenes
+    g, cam, pre, cl, b, am = _render_inputs(H, orc, cfg, P, mask)
+    W, Hh = cam.image_width, cam.image_height
+    bg = np.array([0.2, 0.4, 0.6], np.float32)
+    f = orc.render_fwd(b["ranges"], b["point_list"], pre["means2D"], pre["rgb"], am, pre["conic_opacity"], cl, bg, W,
+                       Hh, cam.tanfovx, cam.tanfovy, render_geo=geo)
+    ug = gs_scenes.upstream_grads(cam)
+    gpix, gmap, gdep = ug["color"].numpy(), ug["all_map"].numpy(), ug["plane_depth"].numpy()
+    ref = orc.render_bwd(b["ranges"], b["point_list"], pre["means2D"], pre["conic_opacity"], pre["rgb"], am,
+                         f["out_all_map"], f["final_T"], f["n_contrib"], cl, bg, gpix, gmap, gdep, W, Hh, cam.tanfovx,
+                         cam.tanfovy, render_geo=geo)
+    got = H.render_bwd(P, W, Hh, cam.tanfovx, cam.tanfovy, H.dev(bg), H.as_u32(b["ranges"]), H.as_u32(b["point_list"]),
+                       H.dev(pre["means2D"]), H.dev(pre["conic_opacity"]), H.dev(pre["rgb"]), H.dev(am),
+                       H.dev(f["out_all_map"]), H.dev(f["final_T"]), H.as_u32(f["n_contrib"]), H.dev(cl), H.dev(gpix),
+                       H.dev(gmap), H.dev(gdep), render_geo=geo)
+    pairs = [("dL_dmeans2D", ref["dL_dmeans2D"][:, :2]), ("dL_dmeans2D_abs", ref["dL_dmeans2D_abs"]),
+             ("dL_dconic_opacity", ref["dL_dconic_opacity"]), ("dL_dcolors", ref["dL_dcolors"])]
+    if geo:
+        pairs.append(("dL_dall_map", ref["dL_dall_map"]))
+    for k, r in pairs:
+        a = got[k].cpu().numpy()
+        assert np.isfinite(a).all(), k
+        assert H.rel_l2(a, r) <= GRAD_TOL, f"{k}: rel L2 {H.rel_l2(a, r)}"
+    a = got["dL_dmeans2D_abs"].cpu().numpy()
+    assert (a[:, :2] + 1e-3 * np.abs(a[:, :2]) + 1e-6 >= np.abs(got["dL_dmeans2D"].cpu().numpy())).all()
+    assert (a[:, 2] == 0).all()
+    if not geo:
+        assert float(got["dL_dall_map"].abs().max()) == 0.0
+
+
+@pytest.mark.parametrize("cfg,P", CASES)
+@pytest.mark.parametrize("sh_mode", [True, False])
+def test_preprocess_backward(H, orc, cfg, P, sh_mode):
+    g, cam = _scene(cfg, P)
+    W, Hh = cam.image_width, cam.image_height
+    pre = H.oracle_preprocess(orc, g, cam, sh_mode=sh_mode)
+    gen = torch.Generator().manual_seed(5)
+    g2 = torch.randn(P, 2, generator=gen).numpy()
+    gco = torch.randn(P, 4, generator=gen).numpy()
+    gcol = torch.randn(P, 3, generator=gen).numpy()
+    n = lambda t: t.numpy()
+    ref = orc.preprocess_bwd(n(g["means3D"]), pre["radii"], n(g["shs"]) if sh_mode else None, pre["clamped"],
+                             n(g["scales"]), n(g["rotations"]), pre["cov3D"], n(cam.world_view_transform),
+                             n(cam.full_proj_transform), n(cam.camera_center), W, Hh, cam.tanfovx, cam.tanfovy, g2, gco,
+                             gcol)
+    gd = {k: H.dev(v) for k, v in g.items() if torch.is_tensor(v)}
+    V, PM, cp = H.dev(cam.world_view_transform), H.dev(cam.full_proj_transform), H.dev(cam.camera_center)
+    f = lambda *s: torch.full(s, 33.0, device=H.DEV)
+    o = dict(dL_dmeans3D=f(P, 3), dL_dcov3D=f(P, 6), dL_dscales=f(P, 3), dL_drotations=f(P, 4), dL_dsh=f(P, 16, 3),
+             dL_dopacity=f(P, 1))
+    H.gn.check(H.lib.gs_preprocess_backward(
+        H.ptr(H.dev(pre["radii"])), H.ptr(H.dev(pre["cov3D"])), H.ptr(H.dev(pre["clamped"])), P, 3,
+        16 if sh_mode else 0, W, Hh, H.ptr(gd["means3D"]), H.ptr(gd["scales"]), H.ptr(gd["rotations"]),
+        H.ptr(gd["shs"]) if sh_mode else None, 1.0, H.ptr(V), H.ptr(PM), H.ptr(cp), cam.tanfovx, cam.tanfovy,
+        H.ptr(H.dev(g2)), 2, H.ptr(H.dev(gco)), H.ptr(H.dev(gcol)), H.ptr(o["dL_dmeans3D"]), H.ptr(o["dL_dcov3D"]),
+        H.ptr(o["dL_dscales"]), H.ptr(o["dL_drotations"]), H.ptr(o["dL_dsh"]) if sh_mode else None,
+        H.ptr(o["dL_dopacity"]), 1, H.stream()), "gs_preprocess_backward")
+    torch.cuda.synchronize()
+    keys = ["dL_dmeans3D", "dL_dcov3D", "dL_dscales", "dL_drotations", "dL_dopacity"] + (["dL_dsh"] if sh_mode else [])
+    for k in keys:
+        a, r = o[k].cpu().numpy(), ref[k]
+        assert np.isfinite(a).all(), k
+        assert H.rel_l2(a, r) <= GRAD_TOL, f"{k}: rel L2 {H.rel_l2(a, r)}"
+        assert np.array_equal(a, r) or H.rel_l2(a, r) < 1e-6, f"{k} drifted from the op-for-op statement"
