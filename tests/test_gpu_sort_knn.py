@@ -52,7 +52,8 @@ def test_inclusive_sum(H, n):
     out = torch.empty(n, dtype=torch.int32, device=H.DEV)
     nb = H.lib.gs_scan_workspace_bytes(n)
     ws = torch.empty(nb, dtype=torch.uint8, device=H.DEV)
-    H.gn.check(H.lib.gs_inclusive_sum(n, H.ptr(H.as_u32(x)), H.ptr(out), H.ptr(ws), nb, H.stream()), "scan")
+    xin = H.as_u32(x)
+    H.gn.check(H.lib.gs_inclusive_sum(n, H.ptr(xin), H.ptr(out), H.ptr(ws), nb, H.stream()), "scan")
     torch.cuda.synchronize()
     assert np.array_equal(H.np_u32(out), np.cumsum(x, dtype=np.uint64).astype(np.uint32))
 

@@ -199,11 +199,14 @@ def test_preprocess_backward(H, orc, cfg, P, sh_mode):
     f = lambda *s: torch.full(s, 33.0, device=H.DEV)
     o = dict(dL_dmeans3D=f(P, 3), dL_dcov3D=f(P, 6), dL_dscales=f(P, 3), dL_drotations=f(P, 4), dL_dsh=f(P, 16, 3),
              dL_dopacity=f(P, 1))
+    # keep every device tensor referenced until the call has run
+    t_radii, t_cov, t_clamped = H.dev(pre["radii"]), H.dev(pre["cov3D"]), H.dev(pre["clamped"])
+    t_g2, t_gco, t_gcol = H.dev(g2), H.dev(gco), H.dev(gcol)
     H.gn.check(H.lib.gs_preprocess_backward(
-        H.ptr(H.dev(pre["radii"])), H.ptr(H.dev(pre["cov3D"])), H.ptr(H.dev(pre["clamped"])), P, 3,
+        H.ptr(t_radii), H.ptr(t_cov), H.ptr(t_clamped), P, 3,
         16 if sh_mode else 0, W, Hh, H.ptr(gd["means3D"]), H.ptr(gd["scales"]), H.ptr(gd["rotations"]),
         H.ptr(gd["shs"]) if sh_mode else None, 1.0, H.ptr(V), H.ptr(PM), H.ptr(cp), cam.tanfovx, cam.tanfovy,
-        H.ptr(H.dev(g2)), 2, H.ptr(H.dev(gco)), H.ptr(H.dev(gcol)), H.ptr(o["dL_dmeans3D"]), H.ptr(o["dL_dcov3D"]),
+        H.ptr(t_g2), 2, H.ptr(t_gco), H.ptr(t_gcol), H.ptr(o["dL_dmeans3D"]), H.ptr(o["dL_dcov3D"]),
         H.ptr(o["dL_dscales"]), H.ptr(o["dL_drotations"]), H.ptr(o["dL_dsh"]) if sh_mode else None,
         H.ptr(o["dL_dopacity"]), 1, H.stream()), "gs_preprocess_backward")
     torch.cuda.synchronize()
