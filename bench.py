@@ -1,0 +1,188 @@
+#!/usr/bin/env python3
+"""Benchmark of the rasterizer hot path on one MI355X.
+
+A step is one training-style view: preprocess forward -> render forward (tile
+count, scan, key emission, radix sort, tile ranges, blend) -> render backward ->
+preprocess backward, driven through the Python operator API with N(0,1)
+upstream gradients on colour, the 5-channel map and plane depth.  Workload:
+BASELINE config 1 (1M Gaussians, 1152x864, SH degree 3), synthetic, seed 0,
+inputs resident in HBM before the timed region.
+
+Prints one JSON line (see --help for flags).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "citygs-x_amd"))
+
+HBM_PEAK_GBS = 8000.0
+
+# Algorithmic bytes per unit of each HBM-bound stage (G = Gaussian, I = (Gaussian,tile) instance).
+BYTES_PER_GAUSSIAN = {
+    "preprocess_fwd": 307 + 4 * 0,  # 44 B geometry in + 192 B SH in + 56 B geometry out + 12 B rgb + 3 B clamped
+    "tile_count": 16,
+    "inclusive_sum": 8,
+    "preprocess_bwd": 560,
+}
+BYTES_PER_INSTANCE = {"sort_pairs": 152, "identify_tile_ranges": 8}
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--config", type=int, default=1, help="BASELINE config index (1 = the headline workload)")
+    ap.add_argument("--gaussians", type=int, default=None, help="override the Gaussian count (debugging only)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-runs", type=int, default=3)
+    return ap.parse_args()
+
+
+def cpu_baseline(g, cam, am, ug, runs):
+    """Times the CPU oracle on the same view with the host's cores."""
+    import numpy as np
+    from oracle import oracle as orc
+    threads = min(16, os.cpu_count() or 1)
+    orc.set_num_threads(threads)
+    n = lambda t: t.numpy()
+    W, H = cam.image_width, cam.image_height
+    gx, gy = orc.tile_grid(W, H)
+    cl = np.ones(gx * gy, bool)
+    bg = np.zeros(3, np.float32)
+    times = []
+    for _ in range(runs):
+        t0 = time.perf_counter()
+        pre = orc.preprocess_fwd(n(g["means3D"]), n(g["scales"]), n(g["rotations"]), n(g["opacities"]), n(g["shs"]),
+                                 n(cam.world_view_transform), n(cam.full_proj_transform), n(cam.camera_center), W, H,
+                                 cam.tanfovx, cam.tanfovy)
+        b = orc.bin_and_sort(pre["radii"], pre["means2D"], pre["depths"], cl, W, H)
+        f = orc.render_fwd(b["ranges"], b["point_list"], pre["means2D"], pre["rgb"], am, pre["conic_opacity"], cl, bg,
+                           W, H, cam.tanfovx, cam.tanfovy)
+        rb = orc.render_bwd(b["ranges"], b["point_list"], pre["means2D"], pre["conic_opacity"], pre["rgb"], am,
+                            f["out_all_map"], f["final_T"], f["n_contrib"], cl, bg, n(ug["color"]), n(ug["all_map"]),
+                            n(ug["plane_depth"]), W, H, cam.tanfovx, cam.tanfovy)
+        orc.preprocess_bwd(n(g["means3D"]), pre["radii"], n(g["shs"]), pre["clamped"], n(g["scales"]),
+                           n(g["rotations"]), pre["cov3D"], n(cam.world_view_transform), n(cam.full_proj_transform),
+                           n(cam.camera_center), W, H, cam.tanfovx, cam.tanfovy, rb["dL_dmeans2D"],
+                           rb["dL_dconic_opacity"], rb["dL_dcolors"])
+        times.append((time.perf_counter() - t0) * 1e3)
+    times.sort()
+    return {"value": round(times[len(times) // 2], 2), "unit": "ms/view", "cores": threads, "kind": "port",
+            "sample": f"{runs} full views of the same workload (median); C++/OpenMP oracle incl. python glue"}
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only (no collectives are part of it); use --gpus 1",
+              file=sys.stderr)
+        sys.exit(2)
+    import torch
+    import gs_scenes
+    import gsrast_native as gn
+    from diff_gaussian_rasterization import GaussianRasterizationSettings, GaussianRasterizer
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the rasterizer has no CPU path", file=sys.stderr)
+        sys.exit(2)
+    dev = "cuda:0"
+    g, cams = gs_scenes.make_scene(args.config, P=args.gaussians, n_views=1)
+    cam = cams[0]
+    P = g["means3D"].shape[0]
+    W, H = cam.image_width, cam.image_height
+    am_cpu = gs_scenes.build_all_map(g["means3D"], g["scales"], g["rotations"], cam)
+    ug_cpu = gs_scenes.upstream_grads(cam)
+
+    rs = GaussianRasterizationSettings(
+        image_height=H, image_width=W, tanfovx=cam.tanfovx, tanfovy=cam.tanfovy, bg=torch.zeros(3, device=dev),
+        scale_modifier=1.0, viewmatrix=cam.world_view_transform.to(dev), projmatrix=cam.full_proj_transform.to(dev),
+        sh_degree=3, campos=cam.camera_center.to(dev), prefiltered=False, render_geo=True, debug=False)
+    rast = GaussianRasterizer(rs)
+    leaf = {k: g[k].to(dev).requires_grad_(True) for k in ("means3D", "scales", "rotations", "opacities", "shs")}
+    am = am_cpu.to(dev)
+    ug = {k: v.to(dev) for k, v in ug_cpu.items()}
+    gx, gy = (W + 15) // 16, (H + 15) // 16
+    cl = torch.ones(gy, gx, dtype=torch.bool, device=dev)
+    m2abs = torch.zeros(P, 3, device=dev, requires_grad=True)
+    ca = {"avoid_pixel_all2all": False, "stats_collector": {}}
+    info = {}
+
+    def step():
+        for t in leaf.values():
+            t.grad = None
+        m2abs.grad = None
+        means2D, rgb, co, radii, depths = rast.preprocess_gaussians(leaf["means3D"], leaf["scales"],
+                                                                    leaf["rotations"], leaf["shs"],
+                                                                    leaf["opacities"], ca)
+        color, n_render, _, _, _, oam, opd = rast.render_gaussians(means2D, m2abs, co, rgb, am, depths, radii, cl, cl,
+                                                                   ca)
+        torch.autograd.backward([color, oam, opd], [ug["color"], ug["all_map"], ug["plane_depth"]])
+        info["n_render"] = n_render
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    gn.stage_timing(True)
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    gn.stage_timing(False)
+    stages = gn.stage_timing_collect()
+    ms_per_step = (t1 - t0) * 1e3 / args.steps
+    R = int(info["n_render"].sum().item())
+
+    stage_report = {}
+    for name, (tot, cnt) in stages.items():
+        ms = tot / max(cnt, 1)
+        e = {"ms": round(ms, 4), "launches_per_step": cnt / args.steps}
+        nbytes = None
+        if name in BYTES_PER_GAUSSIAN:
+            nbytes = BYTES_PER_GAUSSIAN[name] * P
+        elif name in BYTES_PER_INSTANCE:
+            nbytes = BYTES_PER_INSTANCE[name] * R
+        elif name == "duplicate_with_keys":
+            nbytes = 20 * P + 12 * R
+        if nbytes is not None and ms > 0:
+            e["algorithmic_bytes"] = nbytes
+            e["GBps"] = round(nbytes / (ms * 1e-3) / 1e9, 1)
+            e["frac_of_hbm_peak"] = round(e["GBps"] / HBM_PEAK_GBS, 4)
+        stage_report[name] = e
+
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+    if os.path.exists(tpath):
+        try:
+            traffic = json.load(open(tpath)).get("preprocess_fwd_kernel", {}).get("bytes_per_launch")
+        except (OSError, ValueError):
+            traffic = None
+    pf = stage_report.get("preprocess_fwd", {})
+    roofline = {"kernel": "preprocess_fwd_kernel", "bound": "hbm", "achieved": pf.get("GBps"), "peak": HBM_PEAK_GBS,
+                "unit": "GB/s", "frac": pf.get("frac_of_hbm_peak"), "traffic": traffic,
+                "algorithmic_bytes_per_launch": pf.get("algorithmic_bytes")}
+
+    out = {
+        "metric": "fwd+bwd ms/view @1M Gaussians 1152x864; preprocess+sort HBM GB/s vs peak",
+        "value": round(ms_per_step, 4), "unit": "ms/view", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"BASELINE config {args.config}: {P} Gaussians, {W}x{H}, SH degree 3, render_geo, "
+                               f"1 view per step, seed 0", "instances_R": R, "tiles": gx * gy},
+        "gaussian_views_per_s": round(P / (ms_per_step * 1e-3), 1),
+        "roofline": roofline,
+        "stages": stage_report,
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(g, cam, am_cpu.numpy(), ug_cpu, args.cpu_runs)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()
