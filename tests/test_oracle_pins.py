@@ -1,0 +1,459 @@
+"""Pins for the CPU oracle (oracle/gs_oracle.cpp): closed forms, library
+routines, brute force on tiny inputs and an independent torch restatement with
+autograd.  The reference ships no tests or golden vectors for this path, so
+these are what fixes the oracle's meaning.  CPU only."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import gs_scenes
+from oracle import torch_ref as tr
+
+
+def _cam(W=640, H=480, fov=60.0, eye=(0.0, 0.0, -30.0), tgt=(0, 0, 0), up=(0.0, -1.0, 0.0)):
+    return gs_scenes.look_at_camera(eye, tgt, W, H, fov, up=up)
+
+
+def _rel(a, b):
+    a, b = np.asarray(a, np.float64).ravel(), np.asarray(b, np.float64).ravel()
+    return np.linalg.norm(a - b) / max(np.linalg.norm(b), 1e-30)
+
+
+def _pre(orc, g, cam, **kw):
+    n = lambda t: t.numpy()
+    return orc.preprocess_fwd(n(g["means3D"]), n(g["scales"]), n(g["rotations"]), n(g["opacities"]),
+                              kw.pop("shs", n(g["shs"])), n(cam.world_view_transform), n(cam.full_proj_transform),
+                              n(cam.camera_center), cam.image_width, cam.image_height, cam.tanfovx, cam.tanfovy, **kw)
+
+
+# ------------------------------------------------------------------ scalars --
+
+def test_expf_against_libm(orc):
+    x = np.concatenate([np.linspace(-87, 0, 200001), np.linspace(0, 5, 1001), [-5.541264, -1e-8, 0.0]]).astype(np.float32)
+    y = orc.expf(x)
+    ref = np.exp(x.astype(np.float64))
+    ulp = np.spacing(ref.astype(np.float32)).astype(np.float64)
+    assert np.max(np.abs(y.astype(np.float64) - ref) / ulp) <= 1.5
+    assert orc.expf(np.array([0.0], np.float32))[0] == 1.0
+    assert orc.expf(np.array([-87.5, -1000.0], np.float32)).tolist() == [0.0, 0.0]
+    xs = np.sort(x[x <= 0])
+    assert (np.diff(orc.expf(xs)) >= 0).all()  # monotone: threshold tests cannot flip back and forth
+
+
+def test_higher_msb(orc):
+    for n in [1, 2, 3, 4, 255, 256, 1200, 3888, 4095, 4096, 8160, 65535, 65536, 1 << 20]:
+        assert orc.higher_msb(n) == n.bit_length(), n
+    assert orc.higher_msb(40 * 30) == 11 and orc.higher_msb(72 * 54) == 12 and orc.higher_msb(120 * 68) == 13
+
+
+# --------------------------------------------------------------- preprocess --
+
+def test_preprocess_closed_form_on_axis(orc):
+    """Identity rotation, isotropic scale s, on the optical axis at depth z:
+    cov2D = diag((f s / z)^2 + 0.3), radius = ceil(3 sqrt(.)), pixel = ((0+1) S - 1) / 2."""
+    cam = _cam()
+    W, H = 640, 480
+    f = W / (2 * cam.tanfovx)
+    for s, z in [(0.05, 30.0), (0.5, 10.0), (1.0, 55.0)]:
+        g = dict(means3D=torch.tensor([[0.0, 0.0, z - 30.0]]), scales=torch.full((1, 3), s),
+                 rotations=torch.tensor([[1.0, 0, 0, 0]]), opacities=torch.tensor([[0.7]]), shs=torch.zeros(1, 16, 3))
+        o = _pre(orc, g, cam)
+        var = (f * s / z) ** 2 + 0.3
+        assert o["radii"][0] == math.ceil(3 * math.sqrt(var))
+        np.testing.assert_allclose(o["means2D"][0], [(W - 1) / 2, (H - 1) / 2], rtol=0, atol=1e-3)
+        np.testing.assert_allclose(o["conic_opacity"][0], [1 / var, 0, 1 / var, 0.7], rtol=2e-5, atol=1e-7)
+        np.testing.assert_allclose(o["depths"][0], z, rtol=1e-6)
+        np.testing.assert_allclose(o["cov3D"][0], [s * s, 0, 0, s * s, 0, s * s], rtol=1e-6, atol=1e-12)
+        np.testing.assert_allclose(o["rgb"][0], [0.5, 0.5, 0.5])  # zero SH -> 0.5
+        assert o["tiles_touched"][0] >= 1
+
+
+@pytest.mark.parametrize("cfg", [0, 1])
+def test_preprocess_matches_matrix_form(orc, cfg):
+    g, cams = gs_scenes.make_scene(cfg, P=20_000)
+    cam = cams[0]
+    o = _pre(orc, g, cam)
+    d = lambda t: t.double()
+    r = tr.preprocess(d(g["means3D"]), d(g["scales"]), d(g["rotations"]), d(g["opacities"]),
+                      d(cam.world_view_transform), d(cam.full_proj_transform), cam.image_width, cam.image_height,
+                      cam.tanfovx, cam.tanfovy, shs=d(g["shs"]), campos=d(cam.camera_center))
+    vis = o["radii"] > 0
+    assert vis.sum() > 1000
+    # invariant: dropped <=> behind the camera or empty tile rectangle (det == 0 never happens with the 0.3 filter)
+    assert (r["in_front"].numpy()[vis]).all()
+    for k, tol in (("means2D", 2e-6), ("depths", 1e-6), ("conic_opacity", 2e-5), ("rgb", 1e-5)):
+        assert _rel(o[k][vis], r[k].numpy()[vis]) <= tol, k
+    infront = r["in_front"].numpy()
+    assert _rel(o["cov3D"][infront], np.stack([r["Sigma"][:, i, j].numpy() for i, j in
+                                                ((0, 0), (0, 1), (0, 2), (1, 1), (1, 2), (2, 2))], 1)[infront]) <= 1e-6
+    assert (o["cov3D"][~infront] == 0).all()
+    rf = np.ceil(r["radius_f"].numpy())
+    assert (np.abs(o["radii"][vis] - rf[vis]) <= 1).all() and (o["radii"][vis] == rf[vis]).mean() > 0.999
+    assert np.array_equal(o["clamped"][vis].astype(bool), r["clamped"].numpy()[vis]) or \
+        (o["clamped"][vis].astype(bool) != r["clamped"].numpy()[vis]).mean() < 1e-4
+    # conic is the inverse of the filtered 2D covariance
+    a, b, c = (r["cov2D"][:, i].numpy()[vis] for i in range(3))
+    co = o["conic_opacity"][vis]
+    np.testing.assert_allclose(co[:, 0] * a + co[:, 1] * b, 1.0, atol=1e-4)
+    np.testing.assert_allclose(co[:, 0] * b + co[:, 1] * c, 0.0, atol=1e-4)
+    # visibility prefilter and frustum mark agree with preprocess
+    n = lambda t: t.numpy()
+    vf = orc.visible_filter(n(g["means3D"]), n(g["scales"]), n(g["rotations"]), None, n(cam.world_view_transform),
+                            n(cam.full_proj_transform), cam.image_width, cam.image_height, cam.tanfovx, cam.tanfovy)
+    assert np.array_equal(vf, o["radii"])
+    vf2 = orc.visible_filter(n(g["means3D"]), None, None, o["cov3D"], n(cam.world_view_transform),
+                             n(cam.full_proj_transform), cam.image_width, cam.image_height, cam.tanfovx, cam.tanfovy)
+    assert np.array_equal(vf2[infront], o["radii"][infront])
+    mv = orc.mark_visible(n(g["means3D"]), n(cam.world_view_transform), n(cam.full_proj_transform))
+    assert np.array_equal(mv, infront)
+
+
+def test_reference_compatible_mode_leaves_colour_zero(orc):
+    g, cams = gs_scenes.make_scene(0, P=500)
+    o = _pre(orc, g, cams[0], shs=None)
+    assert (o["rgb"] == 0).all() and (o["clamped"] == 0).all() and (o["radii"] > 0).any()
+
+
+def test_sh_degree0_and_rotation_invariance(orc):
+    g, cams = gs_scenes.make_scene(0, P=200)
+    cam = cams[0]
+    sh = torch.zeros(200, 16, 3)
+    sh[:, 0] = torch.randn(200, 3, generator=torch.Generator().manual_seed(1))
+    o = _pre(orc, g, cam, shs=sh.numpy(), sh_degree=0)
+    vis = o["radii"] > 0
+    np.testing.assert_allclose(o["rgb"][vis], np.maximum(0, 0.5 + tr.C0 * sh[:, 0].numpy()[vis]), atol=1e-6)
+    # band-1 energy: sum_k B_k(d)^2 = C1^2 for every unit direction
+    dirs = torch.nn.functional.normalize(torch.randn(50, 3, dtype=torch.float64), dim=-1)
+    B = tr.sh_basis(dirs, 3)
+    np.testing.assert_allclose((B[:, 1:4] ** 2).sum(-1).numpy(), tr.C1 ** 2, rtol=1e-12)
+    np.testing.assert_allclose((B[:, 4:9] ** 2).sum(-1).numpy(), 5 / (4 * math.pi), rtol=1e-6)
+    np.testing.assert_allclose((B[:, 9:16] ** 2).sum(-1).numpy(), 7 / (4 * math.pi), rtol=1e-6)
+
+
+@pytest.mark.parametrize("cfg,deg", [(0, 3), (1, 3), (1, 1)])
+def test_preprocess_backward_matches_autograd(orc, cfg, deg):
+    P = 3000
+    g, cams = gs_scenes.make_scene(cfg, P=P)
+    cam = cams[0]
+    W, H = cam.image_width, cam.image_height
+    o = _pre(orc, g, cam, sh_degree=deg)
+    vis = torch.from_numpy(o["radii"] > 0)
+    gen = torch.Generator().manual_seed(11)
+    g2 = torch.randn(P, 2, generator=gen, dtype=torch.float64)
+    gco = torch.randn(P, 4, generator=gen, dtype=torch.float64)
+    gcol = torch.randn(P, 3, generator=gen, dtype=torch.float64)
+    leaves = {k: g[k].double().requires_grad_(True) for k in ("means3D", "scales", "rotations", "shs", "opacities")}
+    r = tr.preprocess(leaves["means3D"], leaves["scales"], leaves["rotations"], leaves["opacities"],
+                      cam.world_view_transform.double(), cam.full_proj_transform.double(), W, H, cam.tanfovx,
+                      cam.tanfovy, shs=leaves["shs"], campos=cam.camera_center.double(), degree=deg)
+    m = vis[:, None].double()
+    # Convention between the two ops: the off-diagonal conic gradient that render backward emits is HALF the
+    # derivative with respect to the conic's b entry (backward.cu:557 has the -0.5 factor on a term that enters the
+    # exponent once), and preprocess backward doubles it back (backward.cu:135-137).  So a unit of gco[:,1] is
+    # worth two units of true gradient.
+    conv = torch.tensor([1.0, 2.0, 1.0, 1.0], dtype=torch.float64)
+    loss = (r["ndc"][:, :2] * g2 * m).sum() + (r["conic_opacity"] * gco * conv * m).sum() + (r["rgb"] * gcol * m).sum()
+    loss.backward()
+    n = lambda t: t.numpy()
+    b = orc.preprocess_bwd(n(g["means3D"]), o["radii"], n(g["shs"]), o["clamped"], n(g["scales"]), n(g["rotations"]),
+                           o["cov3D"], n(cam.world_view_transform), n(cam.full_proj_transform), n(cam.camera_center), W,
+                           H, cam.tanfovx, cam.tanfovy, g2.numpy(), gco.numpy(), gcol.numpy(), sh_degree=deg)
+    assert _rel(b["dL_dmeans3D"], leaves["means3D"].grad.numpy()) <= 2e-4
+    assert _rel(b["dL_dscales"], leaves["scales"].grad.numpy()) <= 2e-4
+    assert _rel(b["dL_drotations"], leaves["rotations"].grad.numpy()) <= 2e-4
+    assert _rel(b["dL_dsh"], leaves["shs"].grad.numpy()) <= 1e-5
+    # opacity is a pass-through of the packed gradient (rasterize_points.cu:191-194): not masked by visibility
+    np.testing.assert_array_equal(b["dL_dopacity"][:, 0], gco.numpy()[:, 3].astype(np.float32))
+    assert (b["dL_dmeans3D"][~vis.numpy()] == 0).all() and (b["dL_dsh"][~vis.numpy()] == 0).all()
+
+
+def test_cov3d_gradient_convention_and_finite_differences(orc):
+    """dL/dcov3D doubles the off-diagonal entries (backward.cu:146-152); checked by central differences in
+    float64 on the torch restatement, which the oracle must match."""
+    g, cams = gs_scenes.make_scene(0, P=16)
+    cam = cams[0]
+    W, H = cam.image_width, cam.image_height
+    o = _pre(orc, g, cam)
+    gco = np.zeros((16, 4))
+    gco[:, :3] = np.random.default_rng(0).normal(size=(16, 3))
+    n = lambda t: t.numpy()
+    b = orc.preprocess_bwd(n(g["means3D"]), o["radii"], n(g["shs"]), o["clamped"], n(g["scales"]), n(g["rotations"]),
+                           o["cov3D"], n(cam.world_view_transform), n(cam.full_proj_transform), n(cam.camera_center), W,
+                           H, cam.tanfovx, cam.tanfovy, np.zeros((16, 2)), gco, np.zeros((16, 3)))
+
+    def f(sc):
+        r = tr.preprocess(g["means3D"].double(), sc, g["rotations"].double(), g["opacities"].double(),
+                          cam.world_view_transform.double(), cam.full_proj_transform.double(), W, H, cam.tanfovx,
+                          cam.tanfovy)
+        return float((r["conic_opacity"][:, :3] * torch.from_numpy(gco[:, :3]) * torch.tensor([1.0, 2.0, 1.0])).sum())
+    sc = g["scales"].double()
+    fd = np.zeros((16, 3))
+    for i in range(16):
+        for k in range(3):
+            h = 1e-6 * float(sc[i, k])
+            sp, sm = sc.clone(), sc.clone()
+            sp[i, k] += h
+            sm[i, k] -= h
+            fd[i, k] = (f(sp) - f(sm)) / (2 * h)
+    vis = o["radii"] > 0
+    assert vis.all()
+    assert _rel(b["dL_dscales"], fd) <= 1e-3
+
+
+# ------------------------------------------------------------------ binning --
+
+def test_binning_against_brute_force(orc):
+    g, cams = gs_scenes.make_scene(0, P=4000)
+    cam = cams[0]
+    W, H = cam.image_width, cam.image_height
+    o = _pre(orc, g, cam)
+    gx, gy = orc.tile_grid(W, H)
+    rng = np.random.default_rng(3)
+    for cl in (np.ones(gx * gy, bool), rng.random(gx * gy) < 0.6):
+        b = orc.bin_and_sort(o["radii"], o["means2D"], o["depths"], cl, W, H)
+        # brute force: a tile is touched iff it intersects the pixel square [c - r, c + r] under the reference's
+        # truncating rule, restated with integer tile bounds
+        cnt = np.zeros(len(o["radii"]), np.uint32)
+        keys, vals = [], []
+        for i in np.nonzero(o["radii"] > 0)[0]:
+            px, py = np.float32(o["means2D"][i, 0]), np.float32(o["means2D"][i, 1])
+            r = np.float32(o["radii"][i])
+            x0 = min(gx, max(0, int(np.float32(px - r) / np.float32(16))))
+            y0 = min(gy, max(0, int(np.float32(py - r) / np.float32(16))))
+            x1 = min(gx, max(0, int(np.float32(np.float32(np.float32(px + r) + np.float32(16)) - np.float32(1)) / np.float32(16))))
+            y1 = min(gy, max(0, int(np.float32(np.float32(np.float32(py + r) + np.float32(16)) - np.float32(1)) / np.float32(16))))
+            for y in range(y0, y1):
+                for x in range(x0, x1):
+                    if cl[y * gx + x]:
+                        cnt[i] += 1
+                        keys.append((np.uint64(y * gx + x) << np.uint64(32)) | np.uint64(o["depths"][i:i + 1].view(np.uint32)[0]))
+                        vals.append(i)
+        assert np.array_equal(b["tiles_touched"], cnt)
+        assert np.array_equal(b["point_offsets"], np.cumsum(cnt, dtype=np.uint64).astype(np.uint32))
+        keys, vals = np.array(keys, np.uint64), np.array(vals, np.uint32)
+        assert np.array_equal(b["keys_unsorted"], keys) and np.array_equal(b["vals_unsorted"], vals)
+        order = np.argsort(keys, kind="stable")
+        assert np.array_equal(b["keys"], keys[order]) and np.array_equal(b["point_list"], vals[order])
+        tiles = (b["keys"] >> np.uint64(32)).astype(np.int64)
+        lo = np.searchsorted(tiles, np.arange(gx * gy), side="left")
+        hi = np.searchsorted(tiles, np.arange(gx * gy), side="right")
+        empty = lo == hi
+        assert np.array_equal(b["ranges"][~empty, 0], lo[~empty]) and np.array_equal(b["ranges"][~empty, 1], hi[~empty])
+        assert (b["ranges"][empty] == 0).all()
+        if cl.all():
+            assert np.array_equal(b["tiles_touched"], o["tiles_touched"])  # preprocess's rectangle area
+
+
+def test_sort_is_stable_and_respects_bit_range(orc):
+    rng = np.random.default_rng(5)
+    keys = (rng.integers(0, 16, 5000, dtype=np.uint64) << np.uint64(32)) | rng.integers(0, 4, 5000, dtype=np.uint64)
+    junk = rng.integers(0, 2, 5000, dtype=np.uint64) << np.uint64(50)
+    vals = np.arange(5000, dtype=np.uint32)
+    ko, vo = orc.sort_pairs(keys | junk, vals, 36)
+    order = np.argsort(keys, kind="stable")
+    assert np.array_equal(vo, vals[order]) and np.array_equal(ko, (keys | junk)[order])
+    k32 = rng.integers(0, 100, 3000, dtype=np.uint32)
+    ko, vo = orc.sort_pairs_u32(k32, np.arange(3000, dtype=np.uint32))
+    assert np.array_equal(vo, np.argsort(k32, kind="stable").astype(np.uint32))
+
+
+def test_empty_binning(orc):
+    r = orc.tile_ranges(np.zeros(0, np.uint64), 12)
+    assert r.shape == (12, 2) and (r == 0).all()
+    b = orc.bin_and_sort(np.zeros(5, np.int32), np.zeros((5, 2), np.float32), np.zeros(5, np.float32), np.ones(1200, bool),
+                         640, 480)
+    assert b["num_rendered"] == 0 and (b["ranges"] == 0).all()
+
+
+# ------------------------------------------------------------------- render --
+
+def _one_gaussian(orc, mean, conic, opacity, rgb, amap, bg, W=48, H=32, geo=True):
+    cam = _cam(W, H)
+    gx, gy = orc.tile_grid(W, H)
+    means2D = np.array([mean], np.float32)
+    co = np.array([[conic[0], conic[1], conic[2], opacity]], np.float32)
+    radii = np.array([200], np.int32)
+    b = orc.bin_and_sort(radii, means2D, np.array([5.0], np.float32), np.ones(gx * gy, bool), W, H)
+    f = orc.render_fwd(b["ranges"], b["point_list"], means2D, np.array([rgb], np.float32), np.array([amap], np.float32),
+                       co, np.ones(gx * gy, bool), np.array(bg, np.float32), W, H, cam.tanfovx, cam.tanfovy, geo)
+    return cam, f
+
+
+def test_render_single_gaussian_closed_form(orc):
+    W, H = 48, 32
+    mean, conic, o, rgb, bg = (20.25, 11.5), (0.05, 0.01, 0.08), 0.8, (0.2, 0.6, 0.9), (0.1, 0.3, 0.5)
+    amap = (0.0, 0.0, 1.0, 1.0, 7.0)  # planar Gaussian facing the camera at plane distance 7
+    cam, f = _one_gaussian(orc, mean, conic, o, rgb, amap, bg, W, H)
+    ys, xs = np.mgrid[0:H, 0:W].astype(np.float64)
+    dx, dy = mean[0] - xs, mean[1] - ys
+    power = -0.5 * (conic[0] * dx * dx + conic[2] * dy * dy) - conic[1] * dx * dy
+    alpha = np.minimum(0.99, o * np.exp(power))
+    alpha[alpha < 1 / 255] = 0
+    for ch in range(3):
+        np.testing.assert_allclose(f["color"][ch], rgb[ch] * alpha + (1 - alpha) * bg[ch], atol=2e-6)
+    np.testing.assert_allclose(f["final_T"], 1 - alpha, atol=2e-6)
+    np.testing.assert_allclose(f["out_all_map"][3], 1 - f["final_T"], atol=1e-6)  # alpha channel when all_map[:,3] = 1
+    assert np.array_equal(f["n_contrib"], (alpha > 0).astype(np.uint32))
+    assert np.array_equal(f["n_contrib2loss"], f["n_contrib"])
+    # plane depth: distance / (-n . ray) with n = (0,0,1)  ->  -7 alpha / (alpha + 1e-8)
+    hit = alpha > 0
+    np.testing.assert_allclose(f["out_plane_depth"][0][hit], -7.0, rtol=1e-5)
+    assert f["out_observe"][0] == int(hit.sum())  # T = 1 > 0.5 for every contributing pixel
+    assert f["n_render"].sum() == ((W + 15) // 16) * ((H + 15) // 16)  # radius 200 covers every tile
+
+
+def test_render_depth_order_and_termination(orc):
+    """Two coincident opaque-ish Gaussians: the nearer one is blended first; a stack of opaque Gaussians
+    stops at T < 1e-4 and later ones do not count."""
+    W, H = 16, 16
+    cam = _cam(W, H)
+    n = 12
+    means2D = np.tile(np.array([[8.0, 8.0]], np.float32), (n, 1))
+    co = np.tile(np.array([[1e-4, 0.0, 1e-4, 0.8]], np.float32), (n, 1))
+    depths = np.arange(n, 0, -1).astype(np.float32)  # index n-1 is nearest
+    rgb = np.zeros((n, 3), np.float32)
+    rgb[:, 0] = np.arange(n) / n
+    b = orc.bin_and_sort(np.full(n, 50, np.int32), means2D, depths, np.ones(1, bool), W, H)
+    assert np.array_equal(b["point_list"], np.arange(n - 1, -1, -1))
+    f = orc.render_fwd(b["ranges"], b["point_list"], means2D, rgb, np.zeros((n, 5), np.float32), co, np.ones(1, bool),
+                       np.zeros(3, np.float32), W, H, cam.tanfovx, cam.tanfovy, True)
+    a = 0.8  # at the centre pixel (8,8) the exponent is 0
+    T, col, cnt = 1.0, 0.0, 0
+    for k in range(n - 1, -1, -1):
+        if T * (1 - a) < 1e-4:
+            break
+        col += rgb[k, 0] * a * T
+        T *= 1 - a
+        cnt += 1
+    assert cnt == 5  # 0.2^5 = 3.2e-4 is kept, 0.2^6 = 6.4e-5 stops the pixel
+    assert f["n_contrib"][8, 8] == cnt and f["n_contrib2loss"][8, 8] == cnt
+    np.testing.assert_allclose(f["color"][0, 8, 8], col, rtol=1e-5)
+    np.testing.assert_allclose(f["final_T"][8, 8], T, rtol=1e-5)
+    # out_observe counts pixels where T > 0.5 before blending: only the first (nearest) Gaussian
+    assert f["out_observe"][n - 1] == 256 and f["out_observe"][: n - 1].sum() == 0
+
+
+@pytest.mark.parametrize("seed,geo", [(0, True), (1, True), (2, False)])
+def test_render_forward_backward_match_autograd(orc, seed, geo):
+    W, H, P = 64, 48, 150
+    cam = _cam(W, H)
+    gen = torch.Generator().manual_seed(seed)
+    means2D = torch.rand(P, 2, generator=gen, dtype=torch.float64) * torch.tensor([W, H]) - 0.5
+    s = torch.rand(P, generator=gen, dtype=torch.float64) * 6 + 1.5
+    ang = torch.rand(P, generator=gen, dtype=torch.float64) * math.pi
+    ecc = torch.rand(P, generator=gen, dtype=torch.float64) * 0.6 + 0.4
+    ca, sa = torch.cos(ang), torch.sin(ang)
+    ia, ib = 1 / s ** 2, 1 / (s * ecc) ** 2
+    conic = torch.stack([ca * ca * ia + sa * sa * ib, ca * sa * (ia - ib), sa * sa * ia + ca * ca * ib], -1)
+    opac = torch.rand(P, 1, generator=gen, dtype=torch.float64) * 0.9 + 0.05
+    co = torch.cat([conic, opac], 1)
+    rgb = torch.rand(P, 3, generator=gen, dtype=torch.float64)
+    # camera-facing normals keep the plane-depth denominator (n . ray) away from zero, so the check is
+    # well conditioned in fp32
+    amap = torch.randn(P, 5, generator=gen, dtype=torch.float64)
+    amap[:, :2] *= 0.2
+    amap[:, 2] = 1.0
+    amap[:, :3] = torch.nn.functional.normalize(amap[:, :3], dim=-1)
+    amap[:, 3] = 1.0
+    amap[:, 4] = amap[:, 4].abs() + 1.0
+    depths = torch.rand(P, generator=gen) * 10 + 1
+    radii = torch.ceil(3 * s).int()
+    bg = torch.tensor([0.3, 0.1, 0.7], dtype=torch.float64)
+    gx, gy = orc.tile_grid(W, H)
+    cl = np.ones(gx * gy, bool)
+    f32 = lambda t: t.detach().float().numpy()
+    b = orc.bin_and_sort(radii.numpy(), f32(means2D), depths.numpy(), cl, W, H)
+    fo = orc.render_fwd(b["ranges"], b["point_list"], f32(means2D), f32(rgb), f32(amap), f32(co), cl, f32(bg), W, H,
+                        cam.tanfovx, cam.tanfovy, geo)
+    leaves = [t.clone().requires_grad_(True) for t in (means2D, co, rgb, amap)]
+    ft = tr.render(leaves[0], leaves[1], leaves[2], leaves[3], b["ranges"], b["point_list"], bg, W, H, cam.tanfovx,
+                   cam.tanfovy, geo)
+    assert np.array_equal(fo["n_contrib"], ft["n_contrib"].numpy().astype(np.uint32))
+    np.testing.assert_allclose(fo["color"], ft["color"].detach().numpy(), atol=3e-6)
+    np.testing.assert_allclose(fo["final_T"], ft["final_T"].detach().numpy(), atol=3e-6)
+    if geo:
+        np.testing.assert_allclose(fo["out_all_map"], ft["out_all_map"].detach().numpy(), atol=2e-5)
+        pd_ref = ft["out_plane_depth"].detach().numpy()
+        np.testing.assert_allclose(fo["out_plane_depth"], pd_ref, rtol=1e-4, atol=1e-4)
+    # final_T equals the product of (1 - alpha) of the blended Gaussians; sum over tiles of range lengths = instances
+    assert fo["n_render"].sum() == b["num_rendered"]
+    assert fo["out_observe"].sum() <= fo["n_contrib2loss"].sum()
+    # backward
+    gpix = torch.randn(3, H, W, generator=gen, dtype=torch.float64)
+    gmap = torch.randn(5, H, W, generator=gen, dtype=torch.float64)
+    gdep = torch.randn(1, H, W, generator=gen, dtype=torch.float64)
+    loss = (ft["color"] * gpix).sum()
+    if geo:
+        loss = loss + (ft["out_all_map"] * gmap).sum() + (ft["out_plane_depth"] * gdep).sum()
+    loss.backward()
+    bo = orc.render_bwd(b["ranges"], b["point_list"], f32(means2D), f32(co), f32(rgb), f32(amap), fo["out_all_map"],
+                        fo["final_T"], fo["n_contrib"], cl, f32(bg), f32(gpix), f32(gmap), f32(gdep), W, H, cam.tanfovx,
+                        cam.tanfovy, geo)
+    # the reference reports the mean2D gradient per NDC unit: pixel gradient times (W/2, H/2) (backward.cu:443-444)
+    gm = leaves[0].grad.numpy() * np.array([0.5 * W, 0.5 * H])
+    assert _rel(bo["dL_dmeans2D"][:, :2], gm) <= 1e-4
+    assert (bo["dL_dmeans2D"][:, 2] == 0).all() and (bo["dL_dmeans2D_abs"][:, 2] == 0).all()
+    # off-diagonal conic gradient is emitted at half weight (see test_preprocess_backward_matches_autograd)
+    assert _rel(bo["dL_dconic_opacity"], leaves[1].grad.numpy() * np.array([1.0, 0.5, 1.0, 1.0])) <= 1e-4
+    assert (bo["dL_dconic"][:, 2] == 0).all()
+    assert _rel(bo["dL_dcolors"], leaves[2].grad.numpy()) <= 1e-4
+    if geo:
+        assert _rel(bo["dL_dall_map"], leaves[3].grad.numpy()) <= 1e-4
+    else:
+        assert (bo["dL_dall_map"] == 0).all()
+    assert (bo["dL_dmeans2D_abs"][:, :2] >= np.abs(bo["dL_dmeans2D"][:, :2]) * (1 - 1e-5) - 1e-7).all()
+
+
+def test_render_masked_tiles_are_untouched(orc):
+    g, cams = gs_scenes.make_scene(0, P=3000)
+    cam = cams[0]
+    W, H = cam.image_width, cam.image_height
+    o = _pre(orc, g, cam)
+    gx, gy = orc.tile_grid(W, H)
+    cl = np.ones((gy, gx), bool)
+    cl[:, : gx // 2] = False
+    b = orc.bin_and_sort(o["radii"], o["means2D"], o["depths"], cl.ravel(), W, H)
+    assert (b["ranges"].reshape(gy, gx, 2)[:, : gx // 2] == 0).all()
+    am = gs_scenes.build_all_map(g["means3D"], g["scales"], g["rotations"], cam).numpy()
+    f = orc.render_fwd(b["ranges"], b["point_list"], o["means2D"], o["rgb"], am, o["conic_opacity"], cl.ravel(),
+                       np.ones(3, np.float32), W, H, cam.tanfovx, cam.tanfovy)
+    half = (gx // 2) * 16
+    assert (f["color"][:, :, :half] == 0).all() and (f["color"][:, :, half:] > 0).any()
+    assert (f["n_consider"].reshape(gy, gx)[:, : gx // 2] == 0).all()
+    # per-tile statistics are plain sums
+    nc = f["n_contrib"].astype(np.int64)
+    pad = np.zeros((gy * 16, gx * 16), np.int64)
+    pad[:H, :W] = nc
+    sums = pad.reshape(gy, 16, gx, 16).sum(axis=(1, 3))
+    assert np.array_equal(f["n_consider"].reshape(gy, gx)[:, gx // 2:], sums[:, gx // 2:])
+
+
+# ---------------------------------------------------------------------- knn --
+
+def test_morton_known_answers(orc):
+    mn, mx = np.zeros(3, np.float32), np.ones(3, np.float32)
+    assert orc.morton([1, 0, 0], mn, mx) == 0x09249249          # prepMorton(1023)
+    assert orc.morton([0, 1, 0], mn, mx) == 0x09249249 << 1
+    assert orc.morton([0, 0, 1], mn, mx) == 0x09249249 << 2
+    assert orc.morton([1, 1, 1], mn, mx) == 0x3FFFFFFF
+    assert orc.morton([0, 0, 0], mn, mx) == 0
+    assert orc.morton([0.5, 0, 0], mn, mx) == sum(1 << (3 * b) for b in range(10) if (511 >> b) & 1)
+
+
+@pytest.mark.parametrize("P,kind", [(5, "u"), (1500, "u"), (6000, "pos"), (6000, "line")])
+def test_knn_against_brute_force(orc, P, kind):
+    from scipy.spatial import cKDTree
+    rng = np.random.default_rng(P)
+    if kind == "u":
+        pts = rng.uniform(-5, 5, (P, 3))
+    elif kind == "pos":
+        pts = rng.uniform(10, 12, (P, 3))  # bounding box reduction starts from 0: codes use a tenth of the range
+    else:
+        pts = np.stack([np.linspace(0, 100, P), np.zeros(P), np.zeros(P)], 1) + rng.normal(0, 1e-3, (P, 3))
+    pts = pts.astype(np.float32)
+    got = orc.knn_dist2(pts)
+    p64 = pts.astype(np.float64)
+    d, _ = cKDTree(p64).query(p64, k=4)
+    np.testing.assert_allclose(got, (d[:, 1:] ** 2).mean(1), rtol=3e-5, atol=1e-12)
