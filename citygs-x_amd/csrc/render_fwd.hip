@@ -2,18 +2,23 @@
 // with the per-tile statistics of cuda_rasterizer/rasterizer_impl.cu:219-262
 // folded into the same kernel.
 //
-// One 256-thread workgroup (four 64-lane waves) per 16x16 tile, one pixel per
-// thread.  The tile's depth-sorted Gaussians are staged through LDS in batches
-// of 256: index, centre, conic+opacity, colour and the five geometry channels,
-// so the blending loop reads only LDS (every lane reads the same entry, which
-// the LDS serves as a broadcast).  A batch is skipped as soon as every lane of
-// every wave has saturated (ballot per wave, one flag per wave in LDS).
+// One 256-thread workgroup per 16x16 tile; each of its four 64-lane waves owns
+// an 8x8 pixel quadrant.  The tile's depth-sorted Gaussians are staged through
+// LDS in batches of 256 (index, centre, conic+opacity, colour, the five
+// geometry channels, and a conservative screen-space box).  Per batch every
+// wave builds four 64-bit ballots of the Gaussians whose box meets its
+// quadrant and then walks only the set bits with scalar bit scans, so a
+// Gaussian that cannot touch the quadrant costs the wave nothing.  A wave
+// leaves the walk as soon as all its pixels have saturated, and a batch is
+// not even fetched once all four waves have.
 //
-// The per-pixel arithmetic keeps the operation order of the reference so that
+// The per-pixel arithmetic keeps the operation order of the reference, so
 // contributor counts (and in practice the images) match a CPU evaluation bit
-// for bit; exp() is gs_expf.
+// for bit; exp() is gs_expf.  out_observe increments are summed per wave with
+// a ballot and per workgroup in LDS, then added once per (tile, Gaussian).
 #include "gs_common.h"
 #include "gs_kernels.h"
+#include "render_common.h"
 
 namespace gs {
 
@@ -34,13 +39,16 @@ render_fwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
   __shared__ int s_id[BATCH];
   __shared__ float2 s_xy[BATCH];
   __shared__ float4 s_co[BATCH];
+  __shared__ float4 s_bb[BATCH];
   __shared__ float s_rgb[GS_N_RGB][BATCH];
   __shared__ float s_map[GS_N_MAP][BATCH];
+  __shared__ int s_obs[BATCH];
   __shared__ int s_done[GS_TILE_PIX / GS_WAVE];
   __shared__ int s_red[2][GS_TILE_PIX / GS_WAVE];
 
-  const int tid = threadIdx.y * GS_TILE_X + threadIdx.x;
-  const int lane = tid & (GS_WAVE - 1), wave = tid / GS_WAVE;
+  const int tid = threadIdx.x;
+  const TileThread tt = tile_thread(blockIdx.x, blockIdx.y);
+  const int lane = tt.lane, wave = tt.wave;
   const uint32_t tile = blockIdx.y * gridDim.x + blockIdx.x;
   const uint2 range = ranges[tile];
   if (tid == 0) n_render[tile] = (int)(range.y - range.x);
@@ -51,7 +59,7 @@ render_fwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
     }
     return;
   }
-  const uint32_t px = blockIdx.x * GS_TILE_X + threadIdx.x, py = blockIdx.y * GS_TILE_Y + threadIdx.y;
+  const uint32_t px = tt.px, py = tt.py;
   const bool inside = px < (uint32_t)W && py < (uint32_t)H;
   const size_t pid = (size_t)W * py + px;
   const float pfx = (float)px, pfy = (float)py;
@@ -62,7 +70,7 @@ render_fwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
   const int rounds = (todo + BATCH - 1) / BATCH;
 
   float T = 1.0f;
-  uint32_t contributor = 0, last = 0, n2l = 0;
+  uint32_t last = 0, n2l = 0;
   float C[GS_N_RGB] = {0.f, 0.f, 0.f};
   float Mp[GS_N_MAP] = {0.f, 0.f, 0.f, 0.f, 0.f};
 
@@ -72,12 +80,15 @@ render_fwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
     __syncthreads();
     if (s_done[0] && s_done[1] && s_done[2] && s_done[3]) break;
 
-    const uint32_t progress = (uint32_t)i * BATCH + tid;
-    if (range.x + progress < range.y) {
-      const uint32_t g = point_list[range.x + progress];
+    const int count = todo < BATCH ? todo : BATCH;
+    if (tid < count) {
+      const uint32_t g = point_list[range.x + (uint32_t)i * BATCH + tid];
+      const float2 xy = means2D[g];
+      const float4 co = conic_opacity[g];
       s_id[tid] = (int)g;
-      s_xy[tid] = means2D[g];
-      s_co[tid] = conic_opacity[g];
+      s_xy[tid] = xy;
+      s_co[tid] = co;
+      s_bb[tid] = cull_box(xy, co);
       s_rgb[0][tid] = rgb[3 * (size_t)g];
       s_rgb[1][tid] = rgb[3 * (size_t)g + 1];
       s_rgb[2][tid] = rgb[3 * (size_t)g + 2];
@@ -86,33 +97,71 @@ render_fwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
         for (int ch = 0; ch < GS_N_MAP; ch++) s_map[ch][tid] = all_map[5 * (size_t)g + ch];
       }
     }
+    s_obs[tid] = 0;
     __syncthreads();
 
-    const int count = todo < BATCH ? todo : BATCH;
-    for (int j = 0; !done && j < count; j++) {
-      contributor++;
-      const float2 xy = s_xy[j];
-      const float dx = xy.x - pfx, dy = xy.y - pfy;
-      const float4 co = s_co[j];
-      const float power = -0.5f * (co.x * dx * dx + co.z * dy * dy) - co.y * dx * dy;
-      if (power > 0.0f) continue;
-      const float alpha = fminf(0.99f, co.w * gs_expf(power));
-      if (alpha < 1.0f / 255.0f) continue;
-      const float test_T = T * (1 - alpha);
-      if (test_T < 0.0001f) {
-        done = true;
-        continue;
-      }
-      n2l++;
+    if (!wave_done) {
+      // which Gaussians of the batch can touch this wave's 8x8 quadrant
+      uint64_t rel[BATCH / GS_WAVE];
 #pragma unroll
-      for (int ch = 0; ch < GS_N_RGB; ch++) C[ch] += s_rgb[ch][j] * alpha * T;
-      if (render_geo) {
-#pragma unroll
-        for (int ch = 0; ch < GS_N_MAP; ch++) Mp[ch] += s_map[ch][j] * alpha * T;
+      for (int k = 0; k < BATCH / GS_WAVE; k++) {
+        const int j = k * GS_WAVE + lane;
+        rel[k] = __ballot(j < count && box_hits_wave(s_bb[j], tt));
       }
-      if (T > 0.5f) atomicAdd(&out_observe[s_id[j]], 1);
-      T = test_T;
-      last = contributor;
+      bool alive = true;
+#pragma unroll
+      for (int k = 0; k < BATCH / GS_WAVE; k++) {
+        uint64_t m = alive ? rel[k] : 0ull;
+        while (m != 0ull) {
+          const int j = k * GS_WAVE + (int)__builtin_ctzll(m);
+          m &= m - 1ull;
+          bool blend = false;
+          float alpha = 0.f, test_T = 0.f;
+          if (!done) {
+            const float2 xy = s_xy[j];
+            const float dx = xy.x - pfx, dy = xy.y - pfy;
+            const float4 co = s_co[j];
+            const float power = -0.5f * (co.x * dx * dx + co.z * dy * dy) - co.y * dx * dy;
+            if (!(power > 0.0f)) {
+              alpha = fminf(0.99f, co.w * gs_expf(power));
+              if (!(alpha < 1.0f / 255.0f)) {
+                test_T = T * (1 - alpha);
+                if (test_T < 0.0001f)
+                  done = true;
+                else
+                  blend = true;
+              }
+            }
+          }
+          const uint64_t bmask = __ballot(blend);
+          if (bmask != 0ull) {
+            if (blend) {
+              n2l++;
+#pragma unroll
+              for (int ch = 0; ch < GS_N_RGB; ch++) C[ch] += s_rgb[ch][j] * alpha * T;
+              if (render_geo) {
+#pragma unroll
+                for (int ch = 0; ch < GS_N_MAP; ch++) Mp[ch] += s_map[ch][j] * alpha * T;
+              }
+            }
+            const uint64_t omask = __ballot(blend && T > 0.5f);
+            if (omask != 0ull && lane == 0) atomicAdd(&s_obs[j], (int)__popcll(omask));
+            if (blend) {
+              T = test_T;
+              last = (uint32_t)(i * BATCH + j + 1);
+            }
+          }
+          if (__ballot(!done) == 0ull) {
+            m = 0ull;
+            alive = false;  // every pixel of this wave has saturated
+          }
+        }
+      }
+    }
+    __syncthreads();
+    if (tid < count) {
+      const int c = s_obs[tid];
+      if (c != 0) atomicAdd(&out_observe[s_id[tid]], c);
     }
   }
 
@@ -138,6 +187,7 @@ render_fwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
     a += __shfl_xor(a, d, GS_WAVE);
     b += __shfl_xor(b, d, GS_WAVE);
   }
+  __syncthreads();
   if (lane == 0) {
     s_red[0][wave] = a;
     s_red[1][wave] = b;
@@ -153,12 +203,11 @@ render_fwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
 
 int launch_render_fwd(const RenderFwdArgs& a, hipStream_t stream) {
   const dim3 grid((a.W + GS_TILE_X - 1) / GS_TILE_X, (a.H + GS_TILE_Y - 1) / GS_TILE_Y, 1);
-  const dim3 block(GS_TILE_X, GS_TILE_Y, 1);
-  hipLaunchKernelGGL(render_fwd_kernel, grid, block, 0, stream, (const uint2*)a.ranges, a.point_list, a.W, a.H, a.fx,
-                     a.fy, a.cx, a.cy, (const float2*)a.means2D, a.rgb, a.all_map, (const float4*)a.conic_opacity,
-                     a.compute_locally, a.bg, a.render_geo, a.final_T, a.n_contrib_px, a.n_contrib2loss_px,
-                     a.out_color, a.out_observe, a.out_all_map, a.out_plane_depth, a.n_render, a.n_consider,
-                     a.n_contrib_tile);
+  hipLaunchKernelGGL(render_fwd_kernel, grid, dim3(GS_TILE_PIX), 0, stream, (const uint2*)a.ranges, a.point_list, a.W,
+                     a.H, a.fx, a.fy, a.cx, a.cy, (const float2*)a.means2D, a.rgb, a.all_map,
+                     (const float4*)a.conic_opacity, a.compute_locally, a.bg, a.render_geo, a.final_T, a.n_contrib_px,
+                     a.n_contrib2loss_px, a.out_color, a.out_observe, a.out_all_map, a.out_plane_depth, a.n_render,
+                     a.n_consider, a.n_contrib_tile);
   return 0;
 }
 
