@@ -75,6 +75,24 @@ __device__ __forceinline__ float gs_expf(float x) {
   return __builtin_ldexpf(p, (int)n);
 }
 
+// Same routine without the range checks, for callers that guarantee -87 <= x <= 0
+// (or NaN, which propagates); returns the same bits as gs_expf there.
+__device__ __forceinline__ float gs_expf_core(float x) {
+  float n = __builtin_rintf(x * 1.44269504088896341f);
+  float r = __builtin_fmaf(n, -0.693145751953125f, x);
+  r = __builtin_fmaf(n, -1.42860682030941723212e-6f, r);
+  float p = 1.9875691500e-4f;
+  p = __builtin_fmaf(p, r, 1.3981999507e-3f);
+  p = __builtin_fmaf(p, r, 8.3334519073e-3f);
+  p = __builtin_fmaf(p, r, 4.1665795894e-2f);
+  p = __builtin_fmaf(p, r, 1.6666665459e-1f);
+  p = __builtin_fmaf(p, r, 5.0000001201e-1f);
+  float r2 = r * r;
+  p = __builtin_fmaf(p, r2, r);
+  p = p + 1.0f;
+  return __builtin_ldexpf(p, (int)n);
+}
+
 // Column-major 3x3 with the product evaluated term by term, left to right
 // (the semantics of the reference's matrix type,
 // third_party/glm/glm/detail/type_mat3x3.inl:486-518).

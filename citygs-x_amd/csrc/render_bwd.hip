@@ -44,6 +44,7 @@ render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
   __shared__ float2 s_xy[BATCH];
   __shared__ float4 s_co[BATCH];
   __shared__ float4 s_bb[BATCH];
+  __shared__ float s_floor[BATCH];
   __shared__ float s_rgb[GS_N_RGB][BATCH];
   __shared__ float s_map[GS_N_MAP][BATCH];
   __shared__ float s_acc[NV][BATCH];
@@ -77,7 +78,6 @@ render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
   const int tile_last = max(max(s_max[0], s_max[1]), max(s_max[2], s_max[3]));
   if (tile_last == 0) return;
 
-  float accum_rec[GS_N_RGB] = {0.f, 0.f, 0.f}, accum_map[GS_N_MAP] = {0.f, 0.f, 0.f, 0.f, 0.f};
   float gpix[GS_N_RGB] = {0.f, 0.f, 0.f}, gmap[GS_N_MAP] = {0.f, 0.f, 0.f, 0.f, 0.f};
   if (inside) {
 #pragma unroll
@@ -99,7 +99,9 @@ render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
 #pragma unroll
   for (int ch = 0; ch < GS_N_RGB; ch++) bg_dot += bg[ch] * gpix[ch];
 
+  const float bg_term = T_final * bg_dot;
   float last_alpha = 0.f;
+  float accum_rec[GS_N_RGB] = {0.f, 0.f, 0.f}, accum_map[GS_N_MAP] = {0.f, 0.f, 0.f, 0.f, 0.f};
   float last_color[GS_N_RGB] = {0.f, 0.f, 0.f}, last_map[GS_N_MAP] = {0.f, 0.f, 0.f, 0.f, 0.f};
   const float ddelx_dx = (float)(0.5 * W), ddely_dy = (float)(0.5 * H);
 
@@ -120,7 +122,9 @@ render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
       s_id[tid] = (int)g;
       s_xy[tid] = xy;
       s_co[tid] = co;
-      s_bb[tid] = cull_box(xy, co);
+      float pfl;
+      s_bb[tid] = cull_box(xy, co, pfl);
+      s_floor[tid] = pfl;
       s_rgb[0][tid] = rgb[3 * (size_t)g];
       s_rgb[1][tid] = rgb[3 * (size_t)g + 1];
       s_rgb[2][tid] = rgb[3 * (size_t)g + 2];
@@ -146,22 +150,26 @@ render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
         const int j = k * GS_WAVE + (int)__builtin_ctzll(m);
         m &= m - 1ull;
         const int pos = first_pos - j;
-        bool active = pos < last_contributor;  // false for pixels outside the image (last_contributor = 0)
-        float dx = 0.f, dy = 0.f, G = 0.f, alpha = 0.f;
+        // Same tests as the forward pass, on the same bits: exponent first, exponential only where
+        // alpha >= 1/255 is still possible.
+        bool in = false;
+        float dx = 0.f, dy = 0.f, power = 0.f;
         float4 co = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (active) {
+        if (pos < last_contributor) {  // never true for pixels outside the image (last_contributor = 0)
           const float2 xy = s_xy[j];
           dx = xy.x - pfx;
           dy = xy.y - pfy;
           co = s_co[j];
-          const float power = -0.5f * (co.x * dx * dx + co.z * dy * dy) - co.y * dx * dy;
-          if (power > 0.0f) {
-            active = false;
-          } else {
-            G = gs_expf(power);
-            alpha = fminf(0.99f, co.w * G);
-            if (alpha < 1.0f / 255.0f) active = false;
-          }
+          power = -0.5f * (co.x * dx * dx + co.z * dy * dy) - co.y * dx * dy;
+          in = !(power > 0.0f) && !(power < s_floor[j]);
+        }
+        if (__ballot(in) == 0ull) continue;  // wave-uniform
+        bool active = false;
+        float G = 0.f, alpha = 0.f;
+        if (in) {
+          G = gs_expf_core(power);
+          alpha = fminf(0.99f, co.w * G);
+          active = !(alpha < 1.0f / 255.0f);
         }
         if (__ballot(active) == 0ull) continue;  // wave-uniform
 
@@ -169,30 +177,36 @@ render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
 #pragma unroll
         for (int q = 0; q < NV; q++) v[q] = 0.f;
         if (active) {
-          T = T / (1.f - alpha);
+          // Up to dL/dalpha the operation sequence is exactly the CPU statement's (IEEE reciprocal, explicit
+          // FMAs): upstream gradients of the geometry channels can be many orders of magnitude larger than
+          // the result (plane depth divides by a blended normal that may be nearly perpendicular to the
+          // ray), so these operations decide how far a gradient can drift.  What follows dL/dalpha is
+          // products only.
+          const float rcp1ma = 1.f / (1.f - alpha);
+          T = T * rcp1ma;
           const float w = alpha * T;
+          const float oml = 1.f - last_alpha;
           float dL_dalpha = 0.0f;
 #pragma unroll
           for (int ch = 0; ch < GS_N_RGB; ch++) {
             const float c = s_rgb[ch][j];
-            accum_rec[ch] = last_alpha * last_color[ch] + (1.f - last_alpha) * accum_rec[ch];
+            accum_rec[ch] = __builtin_fmaf(last_alpha, last_color[ch], oml * accum_rec[ch]);
             last_color[ch] = c;
-            dL_dalpha += (c - accum_rec[ch]) * gpix[ch];
+            dL_dalpha = __builtin_fmaf(c - accum_rec[ch], gpix[ch], dL_dalpha);
             v[8 + ch] = w * gpix[ch];
           }
           if (render_geo) {
 #pragma unroll
             for (int ch = 0; ch < GS_N_MAP; ch++) {
               const float c = s_map[ch][j];
-              accum_map[ch] = last_alpha * last_map[ch] + (1.f - last_alpha) * accum_map[ch];
+              accum_map[ch] = __builtin_fmaf(last_alpha, last_map[ch], oml * accum_map[ch]);
               last_map[ch] = c;
-              dL_dalpha += (c - accum_map[ch]) * gmap[ch];
+              dL_dalpha = __builtin_fmaf(c - accum_map[ch], gmap[ch], dL_dalpha);
               v[11 + ch] = w * gmap[ch];
             }
           }
-          dL_dalpha *= T;
           last_alpha = alpha;
-          dL_dalpha += (-T_final / (1.f - alpha)) * bg_dot;
+          dL_dalpha = __builtin_fmaf(dL_dalpha, T, -(bg_term * rcp1ma));
           const float dL_dG = co.w * dL_dalpha;
           const float gdx = G * dx, gdy = G * dy;
           const float dG_ddelx = -gdx * co.x - gdy * co.y;
@@ -201,9 +215,10 @@ render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
           v[1] = dL_dG * dG_ddely * ddely_dy;
           v[2] = fabsf(v[0]);
           v[3] = fabsf(v[1]);
-          v[4] = -0.5f * gdx * dx * dL_dG;
-          v[5] = -0.5f * gdx * dy * dL_dG;
-          v[6] = -0.5f * gdy * dy * dL_dG;
+          const float hg = -0.5f * dL_dG;
+          v[4] = hg * gdx * dx;
+          v[5] = hg * gdx * dy;
+          v[6] = hg * gdy * dy;
           v[7] = G * dL_dalpha;
         }
         float r[4];

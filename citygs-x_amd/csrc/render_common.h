@@ -41,15 +41,22 @@ __device__ __forceinline__ TileThread tile_thread(uint32_t tile_x, uint32_t tile
 // rounding in the per-pixel evaluation can never disagree with it; whenever the
 // box cannot be trusted (non-positive determinant, NaN) it is infinite.  Culling
 // with it only skips work, it never changes a result.
-__device__ __forceinline__ float4 cull_box(float2 xy, float4 co) {
+// power_floor receives the exponent below which alpha < 1/255 is certain (never below -87, where
+// gs_expf returns 0 anyway): pixels with power < power_floor can skip the exponential.
+__device__ __forceinline__ float4 cull_box(float2 xy, float4 co, float& power_floor) {
   const float inf = __builtin_inff();
   float4 bb = make_float4(-inf, -inf, inf, inf);  // xmin, ymin, xmax, ymax
   const float o = co.w;
+  power_floor = -87.0f;
   if (o < 0.0039f) {
     // opacity below 1/255: alpha = o*exp(power) with power <= 0 can never reach 1/255
     return make_float4(inf, inf, -inf, -inf);
   }
   const float det = co.x * co.z - co.y * co.y;
+  if (o < 1.0e30f) {
+    const float tau = __logf(255.0f * o) + 0.01f;
+    if (tau == tau) power_floor = fmaxf(-tau, -87.0f);
+  }
   if (det > 0.0f && o < 1.0e30f) {
     const float tau = __logf(255.0f * o) + 0.01f;
     const float s = 2.0f * tau / det;

@@ -40,6 +40,7 @@ render_fwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
   __shared__ float2 s_xy[BATCH];
   __shared__ float4 s_co[BATCH];
   __shared__ float4 s_bb[BATCH];
+  __shared__ float s_floor[BATCH];
   __shared__ float s_rgb[GS_N_RGB][BATCH];
   __shared__ float s_map[GS_N_MAP][BATCH];
   __shared__ int s_obs[BATCH];
@@ -88,7 +89,9 @@ render_fwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
       s_id[tid] = (int)g;
       s_xy[tid] = xy;
       s_co[tid] = co;
-      s_bb[tid] = cull_box(xy, co);
+      float pfl;
+      s_bb[tid] = cull_box(xy, co, pfl);
+      s_floor[tid] = pfl;
       s_rgb[0][tid] = rgb[3 * (size_t)g];
       s_rgb[1][tid] = rgb[3 * (size_t)g + 1];
       s_rgb[2][tid] = rgb[3 * (size_t)g + 2];
@@ -115,33 +118,41 @@ render_fwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
         while (m != 0ull) {
           const int j = k * GS_WAVE + (int)__builtin_ctzll(m);
           m &= m - 1ull;
-          bool blend = false;
-          float alpha = 0.f, test_T = 0.f;
+          // exponent first; the exponential only for lanes that can still pass the 1/255 test
+          float power = 0.f, o = 0.f;
+          bool in = false;
           if (!done) {
             const float2 xy = s_xy[j];
             const float dx = xy.x - pfx, dy = xy.y - pfy;
             const float4 co = s_co[j];
-            const float power = -0.5f * (co.x * dx * dx + co.z * dy * dy) - co.y * dx * dy;
-            if (!(power > 0.0f)) {
-              alpha = fminf(0.99f, co.w * gs_expf(power));
-              if (!(alpha < 1.0f / 255.0f)) {
-                test_T = T * (1 - alpha);
-                if (test_T < 0.0001f)
-                  done = true;
-                else
-                  blend = true;
-              }
+            o = co.w;
+            power = -0.5f * (co.x * dx * dx + co.z * dy * dy) - co.y * dx * dy;
+            in = !(power > 0.0f) && !(power < s_floor[j]);
+          }
+          if (__ballot(in) == 0ull) continue;
+          bool blend = false;
+          float alpha = 0.f, test_T = 0.f;
+          if (in) {
+            alpha = fminf(0.99f, o * gs_expf_core(power));
+            if (!(alpha < 1.0f / 255.0f)) {
+              test_T = T * (1 - alpha);
+              if (test_T < 0.0001f)
+                done = true;
+              else
+                blend = true;
             }
           }
           const uint64_t bmask = __ballot(blend);
           if (bmask != 0ull) {
             if (blend) {
               n2l++;
+              // weight once, then one fused multiply-add per channel (image values are held to 1e-4, not to the bit)
+              const float w = alpha * T;
 #pragma unroll
-              for (int ch = 0; ch < GS_N_RGB; ch++) C[ch] += s_rgb[ch][j] * alpha * T;
+              for (int ch = 0; ch < GS_N_RGB; ch++) C[ch] = __builtin_fmaf(s_rgb[ch][j], w, C[ch]);
               if (render_geo) {
 #pragma unroll
-                for (int ch = 0; ch < GS_N_MAP; ch++) Mp[ch] += s_map[ch][j] * alpha * T;
+                for (int ch = 0; ch < GS_N_MAP; ch++) Mp[ch] = __builtin_fmaf(s_map[ch][j], w, Mp[ch]);
               }
             }
             const uint64_t omask = __ballot(blend && T > 0.5f);

@@ -12,13 +12,26 @@
 //      DGR/ = submodule_cityx/diff-gaussian-rasterization/,
 //      KNN/ = submodule_cityx/simple-knn/.
 //
-// Two deliberate, documented choices where the reference leaves the bits open
+// Four deliberate, documented choices where the reference leaves the bits open
 // (its CUDA binary contracts FMAs and calls the device expf):
 //   * exp() in the blending loops is orc_expf below, a fixed Cody-Waite +
 //     degree-6 polynomial routine built from fmaf and IEEE ops only, so the
 //     same bits come out on any IEEE machine;
 //   * float->int conversions saturate (NaN -> 0) like the GPU's conversion
-//     instruction does (CR/forward.cu:254, CR/auxiliary.h:66-76).
+//     instruction does (CR/forward.cu:254, CR/auxiliary.h:66-76);
+//   * the per-pixel colour / map accumulation "C += c * alpha * T"
+//     (CR/forward.cu:403-407) is evaluated as w = alpha*T; C = fma(c, w, C):
+//     the form a contracting compiler produces, one rounding per channel.  It
+//     only touches float image values (tolerance 1e-4), never a decision;
+//   * likewise in the backward replay the "colour behind" recurrence and the
+//     dL/dalpha accumulation (CR/backward.cu:497-521) are written with the
+//     FMAs a contracting compiler forms from those source lines:
+//     behind = fma(last_alpha, last_c, (1-last_alpha)*behind);
+//     dL_dalpha = fma(c - behind, g, dL_dalpha);
+//     and the two divisions by (1 - alpha) of CR/backward.cu:488,534 share one
+//     reciprocal: inv = 1/(1-alpha); T *= inv;
+//     dL_dalpha = fma(dL_dalpha, T, -(T_final*bg_dot)*inv).
+//     Algebraically the reference's expressions, with the rounding order fixed.
 //
 // Parity pins (tests/test_oracle_*.py): closed forms, an independent torch
 // restatement with autograd, brute force on tiny inputs, numpy/scipy library
@@ -551,9 +564,11 @@ void oracle_render_fwd(int W, int H, float tanx, float tany, const uint32_t* ran
           const float test_T = Tr * (1 - alpha);
           if (test_T < 0.0001f) break;
           n2l++;
-          for (int ch = 0; ch < N_RGB; ch++) C[ch] += rgb[3 * (size_t)g + ch] * alpha * Tr;
+          // weight first, then one fused multiply-add per channel (see the header note on accumulation)
+          const float wgt = alpha * Tr;
+          for (int ch = 0; ch < N_RGB; ch++) C[ch] = fmaf(rgb[3 * (size_t)g + ch], wgt, C[ch]);
           if (render_geo)
-            for (int ch = 0; ch < N_MAP; ch++) Mp[ch] += all_map[5 * (size_t)g + ch] * alpha * Tr;
+            for (int ch = 0; ch < N_MAP; ch++) Mp[ch] = fmaf(all_map[5 * (size_t)g + ch], wgt, Mp[ch]);
           if (Tr > 0.5f) {
 #pragma omp atomic
             out_observe[g] += 1;
@@ -665,15 +680,16 @@ void oracle_render_bwd(int P, int W, int H, float tanx, float tany, const float*
           const float G = orc_expf(power);
           const float alpha = fminf(0.99f, co[3] * G);
           if (alpha < 1.0f / 255.0f) continue;
-          Tr = Tr / (1.f - alpha);
+          const float inv1ma = 1.f / (1.f - alpha);
+          Tr = Tr * inv1ma;
           const float w = alpha * Tr;
           double* a = acc.data() + (size_t)g * 16;
           float dL_dalpha = 0.0f;
           for (int ch = 0; ch < N_RGB; ch++) {
             const float c = rgb[3 * (size_t)g + ch];
-            accum_rec[ch] = last_alpha * last_color[ch] + (1.f - last_alpha) * accum_rec[ch];
+            accum_rec[ch] = fmaf(last_alpha, last_color[ch], (1.f - last_alpha) * accum_rec[ch]);
             last_color[ch] = c;
-            dL_dalpha += (c - accum_rec[ch]) * gpix[ch];
+            dL_dalpha = fmaf(c - accum_rec[ch], gpix[ch], dL_dalpha);
             const double v = (double)(w * gpix[ch]);
 #pragma omp atomic
             a[8 + ch] += v;
@@ -681,18 +697,17 @@ void oracle_render_bwd(int P, int W, int H, float tanx, float tany, const float*
           if (render_geo)
             for (int ch = 0; ch < N_MAP; ch++) {
               const float c = all_map[5 * (size_t)g + ch];
-              accum_map[ch] = last_alpha * last_map[ch] + (1.f - last_alpha) * accum_map[ch];
+              accum_map[ch] = fmaf(last_alpha, last_map[ch], (1.f - last_alpha) * accum_map[ch]);
               last_map[ch] = c;
-              dL_dalpha += (c - accum_map[ch]) * gmap[ch];
+              dL_dalpha = fmaf(c - accum_map[ch], gmap[ch], dL_dalpha);
               const double v = (double)(w * gmap[ch]);
 #pragma omp atomic
               a[11 + ch] += v;
             }
-          dL_dalpha *= Tr;
           last_alpha = alpha;
           float bg_dot = 0;
           for (int ch = 0; ch < N_RGB; ch++) bg_dot += bg[ch] * gpix[ch];
-          dL_dalpha += (-T_final / (1.f - alpha)) * bg_dot;
+          dL_dalpha = fmaf(dL_dalpha, Tr, -((T_final * bg_dot) * inv1ma));
           const float dL_dG = co[3] * dL_dalpha;
           const float gdx = G * dx, gdy = G * dy;
           const float dG_ddelx = -gdx * co[0] - gdy * co[1];
