@@ -626,6 +626,12 @@ int gs_render_tiles_backward(int P, int width, int height, float tan_fovx, float
   return check_launch("render_tiles_backward", (hipStream_t)stream, false);
 }
 
+int gs_selftest_reductions(const float* in, float* out_wave, float* out_rows, gs_stream_t stream) {
+  GS_REQUIRE(in && out_wave && out_rows, "gs_selftest_reductions: null pointer");
+  launch_reduce_selftest(in, out_wave, out_rows, (hipStream_t)stream);
+  return check_launch("selftest_reductions", (hipStream_t)stream, true);
+}
+
 int gs_stage_timing_enable(int enable) {
   g_clock.enabled = enable != 0;
   return 0;

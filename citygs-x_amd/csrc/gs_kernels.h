@@ -105,6 +105,8 @@ struct RenderBwdArgs {
 };
 int launch_render_bwd(const RenderBwdArgs& a, hipStream_t stream);
 
+int launch_reduce_selftest(const float* in, float* out_wave, float* out_rows, hipStream_t stream);
+
 // ---- k-nearest-neighbour mean squared distance ----
 size_t knn_temp_bytes(int P);
 int launch_knn_dist2(int P, const float* points, float* mean_dist2, void* temp, hipStream_t stream);

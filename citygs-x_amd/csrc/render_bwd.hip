@@ -3,21 +3,24 @@
 // transmittance and contributor count, and per-Gaussian gradients are summed
 // over pixels.
 //
-// Workgroup = one 16x16 tile = four 64-lane waves, one 8x8 quadrant each.
-// Per batch of 256 Gaussians (staged in LDS in back-to-front order):
-//   * every wave ballots which Gaussians can touch its quadrant (conservative
-//     box test) and lie in front of its deepest contributor, and walks only
-//     those with scalar bit scans;
-//   * all lanes of a wave visit the same Gaussian together, so the 16 partial
-//     sums (mean2D x/y, |mean2D| x/y, conic x/y/w, opacity, colour 3, map 5)
-//     are reduced across the 64 lanes with permlane32/16 swaps + DPP row adds
-//     (40 ALU operations, no LDS traffic);
-//   * the four waves add their totals into a 16x256 LDS accumulator with LDS
-//     float atomics, and at the end of the batch each thread flushes one
-//     Gaussian with global float atomics: one atomic per (tile, Gaussian,
-//     component) instead of one per (pixel, Gaussian, component).
-// Summation order therefore differs from a per-pixel atomic order; gradients
-// agree with a CPU evaluation to rounding, not bit for bit.
+// Workgroup = one 16x16 tile = four 64-lane waves; a wave owns an 8x8 quadrant
+// and each of its 16-lane rows a 4x4 pixel block.  Per batch of 256 Gaussians
+// (staged in LDS in back-to-front order):
+//   * a wave ballots, for each of its rows, which Gaussians can touch the
+//     row's block (conservative box test) and lie in front of the row's
+//     deepest contributor; the four rows then walk their own bit lists
+//     concurrently, so one pass of the loop handles up to four Gaussians;
+//   * the 16 partial sums of a Gaussian (mean2D x/y, |mean2D| x/y, conic
+//     x/y/w, opacity, colour 3, map 5) are reduced over the row's 16 lanes by
+//     a transposing DPP reduction (15 additions instead of 64) that leaves
+//     component q in lane q, and one LDS float-atomic instruction adds all of
+//     them into a 16x256 accumulator;
+//   * at the end of the batch each thread flushes one Gaussian with global
+//     float atomics: one atomic per (tile, Gaussian, component) instead of
+//     one per (pixel, Gaussian, component).
+// The per-pixel arithmetic is, operation for operation, the CPU statement's;
+// only the order in which pixels are summed differs, so gradients agree with a
+// CPU evaluation to rounding of the sums, not bit for bit.
 #include "gs_common.h"
 #include "gs_kernels.h"
 #include "render_common.h"
@@ -28,6 +31,7 @@ namespace {
 
 constexpr int BATCH = GS_TILE_PIX;
 constexpr int NV = 16;
+constexpr int CHUNKS = BATCH / 32;
 
 __global__ void __launch_bounds__(GS_TILE_PIX)
 render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__ point_list, int W, int H, float fx,
@@ -47,15 +51,16 @@ render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
   __shared__ float s_floor[BATCH];
   __shared__ float s_rgb[GS_N_RGB][BATCH];
   __shared__ float s_map[GS_N_MAP][BATCH];
-  __shared__ float s_acc[NV][BATCH];
+  __shared__ float s_acc[NV][BATCH + 1];  // +1: the 16 components of one Gaussian fall in 16 different banks
+  __shared__ uint32_t s_list[GS_TILE_PIX / GS_WAVE][4][CHUNKS];
   __shared__ int s_max[GS_TILE_PIX / GS_WAVE];
 
   const int tid = threadIdx.x;
-  const TileThread tt = tile_thread(blockIdx.x, blockIdx.y);
-  const int lane = tt.lane, wave = tt.wave;
+  const RowThread rt = row_thread(blockIdx.x, blockIdx.y);
+  const int lane = rt.lane, wave = rt.wave, row = rt.row, l16 = rt.l16;
   const uint32_t tile = blockIdx.y * gridDim.x + blockIdx.x;
   if (!compute_locally[tile]) return;
-  const uint32_t px = tt.px, py = tt.py;
+  const uint32_t px = rt.px, py = rt.py;
   const bool inside = px < (uint32_t)W && py < (uint32_t)H;
   const size_t pid = (size_t)W * py + px;
   const size_t HW = (size_t)H * W;
@@ -69,10 +74,14 @@ render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
   float T = T_final;
   const int last_contributor = inside ? (int)n_contrib_px[pid] : 0;
 
-  // deepest contributor of this wave and of the whole tile: nothing behind it is ever touched
-  int wave_last = last_contributor;
+  // deepest contributor of each row, of this wave and of the whole tile: nothing behind it is ever touched
+  int row_last = last_contributor;
 #pragma unroll
-  for (int d = GS_WAVE / 2; d >= 1; d >>= 1) wave_last = max(wave_last, __shfl_xor(wave_last, d, GS_WAVE));
+  for (int d = 8; d >= 1; d >>= 1) row_last = max(row_last, __shfl_xor(row_last, d, GS_WAVE));
+  int row_last_of[4];
+#pragma unroll
+  for (int r = 0; r < 4; r++) row_last_of[r] = __builtin_amdgcn_readlane(row_last, 16 * r);
+  const int wave_last = max(max(row_last_of[0], row_last_of[1]), max(row_last_of[2], row_last_of[3]));
   if (lane == 0) s_max[wave] = wave_last;
   __syncthreads();
   const int tile_last = max(max(s_max[0], s_max[1]), max(s_max[2], s_max[3]));
@@ -137,25 +146,44 @@ render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
     for (int q = 0; q < NV; q++) s_acc[q][tid] = 0.f;
     __syncthreads();
 
-    uint64_t rel[BATCH / GS_WAVE];
+    // per-row lists: bit b of word c of row r = slot 32c+b of the batch can touch row r's 4x4 block
 #pragma unroll
     for (int k = 0; k < BATCH / GS_WAVE; k++) {
-      const int j = k * GS_WAVE + lane;
-      rel[k] = __ballot(j < count && (first_pos - j) < wave_last && box_hits_wave(s_bb[j], tt));
+      const int jj = k * GS_WAVE + lane;
+      const bool valid = jj < count;
+      const float4 bb = s_bb[valid ? jj : 0];
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        const uint64_t hit = __ballot(valid && (first_pos - jj) < row_last_of[r] && box_hits_row(bb, rt.qx0, rt.qy0, r));
+        if (lane == 0) {
+          s_list[wave][r][2 * k] = (uint32_t)hit;
+          s_list[wave][r][2 * k + 1] = (uint32_t)(hit >> 32);
+        }
+      }
     }
-#pragma unroll
-    for (int k = 0; k < BATCH / GS_WAVE; k++) {
-      uint64_t m = rel[k];
-      while (m != 0ull) {
-        const int j = k * GS_WAVE + (int)__builtin_ctzll(m);
-        m &= m - 1ull;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+
+    {
+      int kk = 0;
+      uint32_t m = s_list[wave][row][0];
+      for (;;) {
+        if (m == 0u && kk < CHUNKS - 1) {
+          kk++;
+          m = s_list[wave][row][kk];
+        }
+        const bool has = m != 0u;
+        if (__ballot(has || kk < CHUNKS - 1) == 0ull) break;
+        const int j = has ? kk * 32 + (int)__builtin_ctz(m) : 0;
+        m &= m - 1u;
         const int pos = first_pos - j;
         // Same tests as the forward pass, on the same bits: exponent first, exponential only where
         // alpha >= 1/255 is still possible.
         bool in = false;
         float dx = 0.f, dy = 0.f, power = 0.f;
         float4 co = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (pos < last_contributor) {  // never true for pixels outside the image (last_contributor = 0)
+        if (has && pos < last_contributor) {  // never true for pixels outside the image (last_contributor = 0)
           const float2 xy = s_xy[j];
           dx = xy.x - pfx;
           dy = xy.y - pfy;
@@ -221,13 +249,9 @@ render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
           v[6] = hg * gdy * dy;
           v[7] = G * dL_dalpha;
         }
-        float r[4];
-        wave_reduce16(v, r);
-        if ((lane & 15) == 0) {
-          const int row = lane >> 4;  // r[k] in this row is the total of value k + 4*row
-#pragma unroll
-          for (int k2 = 0; k2 < 4; k2++) unsafeAtomicAdd(&s_acc[k2 + 4 * row][j], r[k2]);
-        }
+        // lane q of the row now receives the row's total of component q
+        const float tot = row_transpose_reduce16(v, l16);
+        if (has && tot != 0.f) unsafeAtomicAdd(&s_acc[l16][j], tot);
       }
     }
     __syncthreads();

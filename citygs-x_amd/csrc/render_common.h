@@ -101,4 +101,77 @@ __device__ __forceinline__ void wave_reduce16(const float* v, float* out) {
   }
 }
 
+// ---- 4x4-pixel rows -------------------------------------------------------
+// Inside a wave's 8x8 quadrant every 16-lane DPP row owns a 4x4 pixel block
+// (row r at x offset 4*(r&1), y offset 4*(r>>1); lane l16 of the row is pixel
+// (l16 & 3, l16 >> 2) of the block).  The blend loops let the four rows of a
+// wave walk four different Gaussians at the same time, each row following its
+// own list of Gaussians whose box meets its 4x4 block.
+struct RowThread {
+  int lane, wave, row, l16;
+  uint32_t px, py;
+  float qx0, qy0;  // top-left pixel of the wave's quadrant
+};
+
+__device__ __forceinline__ RowThread row_thread(uint32_t tile_x, uint32_t tile_y) {
+  RowThread t;
+  const int tid = threadIdx.x;
+  t.lane = tid & (GS_WAVE - 1);
+  t.wave = tid / GS_WAVE;
+  t.row = t.lane >> 4;
+  t.l16 = t.lane & 15;
+  const uint32_t x0 = tile_x * GS_TILE_X + (uint32_t)(t.wave & 1) * 8u;
+  const uint32_t y0 = tile_y * GS_TILE_Y + (uint32_t)(t.wave >> 1) * 8u;
+  t.px = x0 + (uint32_t)(t.row & 1) * 4u + (uint32_t)(t.l16 & 3);
+  t.py = y0 + (uint32_t)(t.row >> 1) * 4u + (uint32_t)(t.l16 >> 2);
+  t.qx0 = (float)x0;
+  t.qy0 = (float)y0;
+  return t;
+}
+
+// Box against the 4x4 block of row r of the quadrant at (qx0, qy0).
+__device__ __forceinline__ bool box_hits_row(const float4 bb, float qx0, float qy0, int r) {
+  const float x0 = qx0 + (float)((r & 1) * 4), y0 = qy0 + (float)((r >> 1) * 4);
+  return !(bb.z < x0 || bb.x > x0 + 3.0f || bb.w < y0 || bb.y > y0 + 3.0f);
+}
+
+template <int CTRL, int BANK_MASK>
+__device__ __forceinline__ float dpp_merge(float old, float src) {
+  // lanes of the enabled banks read src through the DPP pattern, the others keep old
+  return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(old), __float_as_int(src), CTRL, 0xF, BANK_MASK, false));
+}
+
+// Transposing reduction inside every 16-lane row: on entry each lane holds 16
+// values, on return lane l16 of a row holds the sum over the row's 16 lanes of
+// value number l16.  Four halving steps (distances 8, 4, 2, 1): at each step a
+// lane keeps half of its values and receives the partner lane's copy of them,
+// so 8 + 4 + 2 + 1 additions replace 16 x 4.
+__device__ __forceinline__ float row_transpose_reduce16(const float* v, int l16) {
+  float a[8], b[4], c[2];
+#pragma unroll
+  for (int i = 0; i < 8; i++) {
+    // lanes 0-7 keep value i and fetch it from lane +8; lanes 8-15 keep value i+8 and fetch it from lane -8
+    const float x = dpp_merge<0x128 /*row_ror:8*/, 0x3>(v[i + 8], v[i]);
+    const float y = dpp_merge<0x128 /*row_ror:8*/, 0xC>(v[i], v[i + 8]);
+    a[i] = x + y;
+  }
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    // lanes with bit 2 clear (banks 0, 2) keep value i, fetched from lane +4; the others keep i+4, from lane -4
+    const float x = dpp_merge<0x104 /*row_shl:4*/, 0x5>(a[i + 4], a[i]);
+    const float y = dpp_merge<0x114 /*row_shr:4*/, 0xA>(a[i], a[i + 4]);
+    b[i] = x + y;
+  }
+  const bool bit1 = (l16 & 2) != 0, bit0 = (l16 & 1) != 0;
+#pragma unroll
+  for (int i = 0; i < 2; i++) {
+    const float lo = dpp_row_add<0x4E>(b[i]);      // quad_perm [2,3,0,1]: + lane^2
+    const float hi = dpp_row_add<0x4E>(b[i + 2]);
+    c[i] = bit1 ? hi : lo;
+  }
+  const float lo = dpp_row_add<0xB1>(c[0]);  // quad_perm [1,0,3,2]: + lane^1
+  const float hi = dpp_row_add<0xB1>(c[1]);
+  return bit0 ? hi : lo;
+}
+
 }  // namespace gs

@@ -2,20 +2,23 @@
 // with the per-tile statistics of cuda_rasterizer/rasterizer_impl.cu:219-262
 // folded into the same kernel.
 //
-// One 256-thread workgroup per 16x16 tile; each of its four 64-lane waves owns
-// an 8x8 pixel quadrant.  The tile's depth-sorted Gaussians are staged through
-// LDS in batches of 256 (index, centre, conic+opacity, colour, the five
-// geometry channels, and a conservative screen-space box).  Per batch every
-// wave builds four 64-bit ballots of the Gaussians whose box meets its
-// quadrant and then walks only the set bits with scalar bit scans, so a
-// Gaussian that cannot touch the quadrant costs the wave nothing.  A wave
-// leaves the walk as soon as all its pixels have saturated, and a batch is
-// not even fetched once all four waves have.
+// One 256-thread workgroup per 16x16 tile; each 64-lane wave owns an 8x8
+// quadrant and each 16-lane row of a wave a 4x4 pixel block.  The tile's
+// depth-sorted Gaussians are staged through LDS in batches of 256 (index,
+// centre, conic+opacity, colour, the five geometry channels, a conservative
+// screen-space box and the exponent below which alpha < 1/255 is certain).
+// Per batch a wave ballots, for each of its four rows, which Gaussians' boxes
+// meet the row's 4x4 block and leaves those bit lists in LDS; the four rows
+// then walk their own lists concurrently (find-first-set on a per-row mask),
+// so one pass of the loop blends up to four different Gaussians and a
+// Gaussian that cannot touch a block costs that row nothing.  Pixels keep
+// their own front-to-back order, which is all the blend needs.  A row stops
+// when its 16 pixels have saturated; a batch is not fetched once all have.
 //
-// The per-pixel arithmetic keeps the operation order of the reference, so
-// contributor counts (and in practice the images) match a CPU evaluation bit
-// for bit; exp() is gs_expf.  out_observe increments are summed per wave with
-// a ballot and per workgroup in LDS, then added once per (tile, Gaussian).
+// The per-pixel arithmetic keeps a fixed operation order, so contributor
+// counts and images match a CPU evaluation bit for bit; exp() is gs_expf.
+// out_observe increments are counted per row with a ballot, summed per
+// workgroup in LDS and added once per (tile, Gaussian).
 #include "gs_common.h"
 #include "gs_kernels.h"
 #include "render_common.h"
@@ -25,6 +28,7 @@ namespace gs {
 namespace {
 
 constexpr int BATCH = GS_TILE_PIX;
+constexpr int CHUNKS = BATCH / 32;  // 32-bit list words per row and batch
 
 __global__ void __launch_bounds__(GS_TILE_PIX)
 render_fwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__ point_list, int W, int H, float fx,
@@ -44,12 +48,13 @@ render_fwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
   __shared__ float s_rgb[GS_N_RGB][BATCH];
   __shared__ float s_map[GS_N_MAP][BATCH];
   __shared__ int s_obs[BATCH];
+  __shared__ uint32_t s_list[GS_TILE_PIX / GS_WAVE][4][CHUNKS];
   __shared__ int s_done[GS_TILE_PIX / GS_WAVE];
   __shared__ int s_red[2][GS_TILE_PIX / GS_WAVE];
 
   const int tid = threadIdx.x;
-  const TileThread tt = tile_thread(blockIdx.x, blockIdx.y);
-  const int lane = tt.lane, wave = tt.wave;
+  const RowThread rt = row_thread(blockIdx.x, blockIdx.y);
+  const int lane = rt.lane, wave = rt.wave, row = rt.row;
   const uint32_t tile = blockIdx.y * gridDim.x + blockIdx.x;
   const uint2 range = ranges[tile];
   if (tid == 0) n_render[tile] = (int)(range.y - range.x);
@@ -60,12 +65,13 @@ render_fwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
     }
     return;
   }
-  const uint32_t px = tt.px, py = tt.py;
+  const uint32_t px = rt.px, py = rt.py;
   const bool inside = px < (uint32_t)W && py < (uint32_t)H;
   const size_t pid = (size_t)W * py + px;
   const float pfx = (float)px, pfy = (float)py;
   const float rayx = (pfx - cx) / fx, rayy = (pfy - cy) / fy;
   bool done = !inside;
+  const int row_shift = 16 * row;
 
   int todo = (int)(range.y - range.x);
   const int rounds = (todo + BATCH - 1) / BATCH;
@@ -76,8 +82,8 @@ render_fwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
   float Mp[GS_N_MAP] = {0.f, 0.f, 0.f, 0.f, 0.f};
 
   for (int i = 0; i < rounds; i++, todo -= BATCH) {
-    const bool wave_done = __ballot(!done) == 0ull;
-    if (lane == 0) s_done[wave] = wave_done;
+    const uint64_t alive_mask = __ballot(!done);
+    if (lane == 0) s_done[wave] = alive_mask == 0ull;
     __syncthreads();
     if (s_done[0] && s_done[1] && s_done[2] && s_done[3]) break;
 
@@ -86,10 +92,10 @@ render_fwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
       const uint32_t g = point_list[range.x + (uint32_t)i * BATCH + tid];
       const float2 xy = means2D[g];
       const float4 co = conic_opacity[g];
+      float pfl;
       s_id[tid] = (int)g;
       s_xy[tid] = xy;
       s_co[tid] = co;
-      float pfl;
       s_bb[tid] = cull_box(xy, co, pfl);
       s_floor[tid] = pfl;
       s_rgb[0][tid] = rgb[3 * (size_t)g];
@@ -103,68 +109,93 @@ render_fwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
     s_obs[tid] = 0;
     __syncthreads();
 
-    if (!wave_done) {
-      // which Gaussians of the batch can touch this wave's 8x8 quadrant
-      uint64_t rel[BATCH / GS_WAVE];
+    if (alive_mask != 0ull) {
+      // per-row lists: bit b of word c of row r = Gaussian 32c+b of the batch can touch row r's 4x4 block
 #pragma unroll
       for (int k = 0; k < BATCH / GS_WAVE; k++) {
-        const int j = k * GS_WAVE + lane;
-        rel[k] = __ballot(j < count && box_hits_wave(s_bb[j], tt));
+        const int jj = k * GS_WAVE + lane;
+        const bool valid = jj < count;
+        const float4 bb = s_bb[valid ? jj : 0];
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+          const bool row_alive = ((alive_mask >> (16 * r)) & 0xFFFFull) != 0ull;
+          const uint64_t b = __ballot(valid && row_alive && box_hits_row(bb, rt.qx0, rt.qy0, r));
+          if (lane == 0) {
+            s_list[wave][r][2 * k] = (uint32_t)b;
+            s_list[wave][r][2 * k + 1] = (uint32_t)(b >> 32);
+          }
+        }
       }
-      bool alive = true;
-#pragma unroll
-      for (int k = 0; k < BATCH / GS_WAVE; k++) {
-        uint64_t m = alive ? rel[k] : 0ull;
-        while (m != 0ull) {
-          const int j = k * GS_WAVE + (int)__builtin_ctzll(m);
-          m &= m - 1ull;
-          // exponent first; the exponential only for lanes that can still pass the 1/255 test
-          float power = 0.f, o = 0.f;
-          bool in = false;
-          if (!done) {
-            const float2 xy = s_xy[j];
-            const float dx = xy.x - pfx, dy = xy.y - pfy;
-            const float4 co = s_co[j];
-            o = co.w;
-            power = -0.5f * (co.x * dx * dx + co.z * dy * dy) - co.y * dx * dy;
-            in = !(power > 0.0f) && !(power < s_floor[j]);
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+
+      int kk = 0;
+      uint32_t m = s_list[wave][row][0];
+      for (;;) {
+        if (m == 0u && kk < CHUNKS - 1) {
+          kk++;
+          m = s_list[wave][row][kk];
+        }
+        const bool has = m != 0u;
+        if (__ballot(has || kk < CHUNKS - 1) == 0ull) break;
+        const int j = has ? kk * 32 + (int)__builtin_ctz(m) : 0;
+        m &= m - 1u;
+
+        // exponent first; the exponential only for lanes that can still pass the 1/255 test
+        float power = 0.f, o = 0.f;
+        bool in = false;
+        if (has && !done) {
+          const float2 xy = s_xy[j];
+          const float dx = xy.x - pfx, dy = xy.y - pfy;
+          const float4 co = s_co[j];
+          o = co.w;
+          power = -0.5f * (co.x * dx * dx + co.z * dy * dy) - co.y * dx * dy;
+          in = !(power > 0.0f) && !(power < s_floor[j]);
+        }
+        if (__ballot(in) == 0ull) continue;
+        bool blend = false, stop = false;
+        float alpha = 0.f, test_T = 0.f;
+        if (in) {
+          alpha = fminf(0.99f, o * gs_expf_core(power));
+          if (!(alpha < 1.0f / 255.0f)) {
+            test_T = T * (1 - alpha);
+            if (test_T < 0.0001f)
+              stop = true;
+            else
+              blend = true;
           }
-          if (__ballot(in) == 0ull) continue;
-          bool blend = false;
-          float alpha = 0.f, test_T = 0.f;
-          if (in) {
-            alpha = fminf(0.99f, o * gs_expf_core(power));
-            if (!(alpha < 1.0f / 255.0f)) {
-              test_T = T * (1 - alpha);
-              if (test_T < 0.0001f)
-                done = true;
-              else
-                blend = true;
+        }
+        const uint64_t bmask = __ballot(blend);
+        if (bmask != 0ull) {
+          if (blend) {
+            n2l++;
+            // weight once, then one fused multiply-add per channel
+            const float w = alpha * T;
+#pragma unroll
+            for (int ch = 0; ch < GS_N_RGB; ch++) C[ch] = __builtin_fmaf(s_rgb[ch][j], w, C[ch]);
+            if (render_geo) {
+#pragma unroll
+              for (int ch = 0; ch < GS_N_MAP; ch++) Mp[ch] = __builtin_fmaf(s_map[ch][j], w, Mp[ch]);
             }
           }
-          const uint64_t bmask = __ballot(blend);
-          if (bmask != 0ull) {
-            if (blend) {
-              n2l++;
-              // weight once, then one fused multiply-add per channel (image values are held to 1e-4, not to the bit)
-              const float w = alpha * T;
-#pragma unroll
-              for (int ch = 0; ch < GS_N_RGB; ch++) C[ch] = __builtin_fmaf(s_rgb[ch][j], w, C[ch]);
-              if (render_geo) {
-#pragma unroll
-                for (int ch = 0; ch < GS_N_MAP; ch++) Mp[ch] = __builtin_fmaf(s_map[ch][j], w, Mp[ch]);
-              }
-            }
-            const uint64_t omask = __ballot(blend && T > 0.5f);
-            if (omask != 0ull && lane == 0) atomicAdd(&s_obs[j], (int)__popcll(omask));
-            if (blend) {
-              T = test_T;
-              last = (uint32_t)(i * BATCH + j + 1);
-            }
+          const uint64_t omask = __ballot(blend && T > 0.5f);
+          if (omask != 0ull) {
+            const int cnt = __popc((uint32_t)(omask >> row_shift) & 0xFFFFu);
+            if (rt.l16 == 0 && cnt != 0) atomicAdd(&s_obs[j], cnt);
           }
-          if (__ballot(!done) == 0ull) {
-            m = 0ull;
-            alive = false;  // every pixel of this wave has saturated
+          if (blend) {
+            T = test_T;
+            last = (uint32_t)(i * BATCH + j + 1);
+          }
+        }
+        if (__ballot(stop) != 0ull) {
+          if (stop) done = true;
+          // a row whose 16 pixels have all saturated drops the rest of its list
+          const uint64_t still = __ballot(!done);
+          if (((uint32_t)(still >> row_shift) & 0xFFFFu) == 0u) {
+            m = 0u;
+            kk = CHUNKS - 1;
           }
         }
       }

@@ -46,6 +46,7 @@ _SIGNATURES = {
     "gs_identify_tile_ranges": (_i, [_i64, _vp, _i, _vp, _vp]),
     "gs_render_tiles_forward": (_i, [_i, _i, _i, _f, _f, _f, _f] + [_vp] * 8 + [_i] + [_vp] * 11),
     "gs_render_tiles_backward": (_i, [_i, _i, _i, _f, _f] + [_vp] * 14 + [_i] + [_vp] * 6),
+    "gs_selftest_reductions": (_i, [_vp, _vp, _vp, _vp]),
     "gs_stage_timing_enable": (_i, [_i]),
     "gs_stage_timing_collect": (_i, [C.c_char_p, _sz]),
     "gs_image_state_layout": (_i, [_i, _i] + [_psz] * 5),

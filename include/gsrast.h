@@ -193,6 +193,12 @@ int gs_render_tiles_backward(int P, int width, int height, float tan_fovx, float
                              float* dL_dmean2D, float* dL_dmean2D_abs, float* dL_dconic_opacity,
                              float* dL_dcolor, float* dL_dall_map, gs_stream_t stream);
 
+/* Diagnostic with no counterpart in the reference: runs the two cross-lane
+ * reductions of the blend kernels on one 64-lane wave.  in is (64,16) floats;
+ * out_wave (16) receives the sums over all 64 lanes, out_rows (4,16) the sums
+ * over each 16-lane row.  Synchronises the stream. */
+int gs_selftest_reductions(const float* in, float* out_wave, float* out_rows, gs_stream_t stream);
+
 /* Optional per-stage GPU timing, the role of the reference's MyTimerOnGPU
  * (CR/timers.cu:11-79; stage names at CR/rasterizer_impl.cu:385-752): while
  * enabled, each stage of the composite entry points (preprocess_fwd,

@@ -83,3 +83,14 @@ def test_knn_dist2(H, orc, P, kind):
     assert np.array_equal(got, ref), f"max abs diff {np.abs(got - ref).max()}"
     if P <= 50_000:
         np.testing.assert_allclose(got, _brute(pts), rtol=2e-4, atol=1e-9)
+
+
+def test_cross_lane_reductions(H):
+    rng = np.random.default_rng(0)
+    x = rng.integers(-8, 9, (64, 16)).astype(np.float32)  # small integers: sums are exact in any order
+    tin = H.dev(x)
+    ow = torch.zeros(16, device=H.DEV)
+    orow = torch.zeros(4, 16, device=H.DEV)
+    H.gn.check(H.lib.gs_selftest_reductions(H.ptr(tin), H.ptr(ow), H.ptr(orow), H.stream()), "selftest")
+    assert np.array_equal(ow.cpu().numpy(), x.sum(0))
+    assert np.array_equal(orow.cpu().numpy(), x.reshape(4, 16, 16).sum(1))
