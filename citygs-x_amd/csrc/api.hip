@@ -124,7 +124,7 @@ GeometryLayout geometry_layout(int P) {
 }
 
 struct BinningLayout {
-  size_t point_list, keys, point_list_unsorted, keys_unsorted, sort_temp, total;
+  size_t point_list, keys, point_list_unsorted, keys_unsorted, emission, emission_other, sort_temp, total;
 };
 BinningLayout binning_layout(int64_t R) {
   BinningLayout L;
@@ -135,6 +135,8 @@ BinningLayout binning_layout(int64_t R) {
   L.keys = take(n * 8);
   L.point_list_unsorted = take(n * 4);
   L.keys_unsorted = take(n * 8);
+  L.emission = take(n * 4);
+  L.emission_other = take(n * 4);
   L.sort_temp = take(sort_temp_bytes((int64_t)n));
   L.total = off + 256;
   return L;
@@ -374,31 +376,35 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
   bbase = align_ptr(bbase, 256);
   uint32_t* point_list = (uint32_t*)(bbase + BL.point_list);
   uint64_t* keys = (uint64_t*)(bbase + BL.keys);
-  uint32_t* point_list_other = (uint32_t*)(bbase + BL.point_list_unsorted);
+  uint32_t* gauss_of_emission = (uint32_t*)(bbase + BL.point_list_unsorted);
   uint64_t* keys_other = (uint64_t*)(bbase + BL.keys_unsorted);
+  uint32_t* emission = (uint32_t*)(bbase + BL.emission);
+  uint32_t* emission_other = (uint32_t*)(bbase + BL.emission_other);
   void* sort_temp = bbase + BL.sort_temp;
 
   EventTimer timer;
   if (timer.begin(elapsed_ms != nullptr, stream)) return 1;
 
   const int end_bit = sort_end_bit(width, height);
-  // The sort ping-pongs; start from the array pair that makes it finish in
-  // (keys, point_list).
+  // The sort carries each instance's index in emission order as its payload (the backward pass files
+  // per-instance gradients under it); the Gaussian ids of the sorted list are gathered afterwards.
+  // It ping-pongs, so start from the array pair that makes it finish in (keys, emission).
   const bool odd = sort_result_in_b(end_bit);
   uint64_t* k_start = odd ? keys_other : keys;
-  uint32_t* v_start = odd ? point_list_other : point_list;
+  uint32_t* e_start = odd ? emission_other : emission;
   uint64_t* k_partner = odd ? keys : keys_other;
-  uint32_t* v_partner = odd ? point_list : point_list_other;
+  uint32_t* e_partner = odd ? emission : emission_other;
   if (R > 0) {
     {
-    StageScope _t("duplicate_with_keys", stream);
-    launch_duplicate_with_keys(P, width, height, means2D, depths, point_offsets, radii, compute_locally, k_start,
-                               v_start, stream);
-  }
+      StageScope _t("duplicate_with_keys", stream);
+      launch_duplicate_with_keys(P, width, height, means2D, depths, point_offsets, radii, compute_locally, k_start,
+                                 gauss_of_emission, e_start, stream);
+    }
     if (check_launch("duplicate_with_keys", stream, dbg)) return 1;
     {
       StageScope _t("sort_pairs", stream);
-      if (launch_sort_pairs_u64(R, k_start, k_partner, v_start, v_partner, end_bit, sort_temp, stream)) return 1;
+      if (launch_sort_pairs_u64(R, k_start, k_partner, e_start, e_partner, end_bit, sort_temp, stream)) return 1;
+      launch_gather_u32(R, emission, gauss_of_emission, point_list, stream);
     }
     if (check_launch("sort_pairs", stream, dbg)) return 1;
   }
@@ -433,12 +439,14 @@ int gs_render_backward(int P, int R, const float* background, int width, int hei
                        const float* dL_dout_plane_depth, float* dL_dmean2D, float* dL_dmean2D_abs,
                        float* dL_dconic_opacity, float* dL_dcolor, float* dL_dall_map, const float* means2D,
                        const float* conic_opacity, const float* rgb, const float* all_maps,
-                       const float* all_map_pixels, int render_geo, int debug, float* elapsed_ms,
-                       gs_stream_t stream_) {
-  (void)geom_buffer;
+                       const float* all_map_pixels, int render_geo, int debug, float* instance_grads,
+                       size_t instance_grads_bytes, float* elapsed_ms, gs_stream_t stream_) {
   hipStream_t stream = (hipStream_t)stream_;
   GS_REQUIRE(P > 0 && R >= 0 && width > 0 && height > 0, "gs_render_backward: bad sizes");
-  GS_REQUIRE(binning_buffer && img_buffer && compute_locally && background, "gs_render_backward: null buffer");
+  GS_REQUIRE(geom_buffer && binning_buffer && img_buffer && compute_locally && background,
+             "gs_render_backward: null buffer");
+  GS_REQUIRE(instance_grads && instance_grads_bytes >= gs_render_backward_workspace_bytes(R),
+             "gs_render_backward: instance_grads workspace missing or too small");
   GS_REQUIRE(dL_dpix && dL_dmean2D && dL_dmean2D_abs && dL_dconic_opacity && dL_dcolor && means2D &&
                  conic_opacity && rgb,
              "gs_render_backward: null pointer");
@@ -446,9 +454,14 @@ int gs_render_backward(int P, int R, const float* background, int width, int hei
              "gs_render_backward: render_geo needs the geometry-map tensors");
   const BinningLayout BL = binning_layout(R);
   const ImageLayout IL = image_layout(width, height);
+  const GeometryLayout GL = geometry_layout(P);
+  const char* gbase = align_ptr(geom_buffer, 256);
   const char* bbase = align_ptr(binning_buffer, 256);
   const char* ibase = align_ptr(img_buffer, 256);
   RenderBwdArgs a;
+  a.emission_sorted = (const uint32_t*)(bbase + BL.emission);
+  a.point_offsets = (const uint32_t*)(gbase + GL.point_offsets);
+  a.instance_grads = (float*)align_ptr((const char*)instance_grads, 256);
   a.P = P; a.W = width; a.H = height;
   a.fy = height / (2.0f * tan_fovy);  // cuda_rasterizer/rasterizer_impl.cu:885-886
   a.fx = width / (2.0f * tan_fovx);
@@ -474,6 +487,8 @@ int gs_render_backward(int P, int R, const float* background, int width, int hei
   if (timer.end(stream, elapsed_ms)) return 1;
   return 0;
 }
+
+size_t gs_render_backward_workspace_bytes(int R) { return (size_t)(R > 0 ? R : 1) * 16 * sizeof(float) + 256; }
 
 size_t gs_knn_workspace_bytes(int P) { return knn_temp_bytes(P) + 256; }
 
@@ -520,7 +535,7 @@ int gs_duplicate_with_keys(int P, int width, int height, const float* means2D, c
   if (P == 0) return 0;
   GS_REQUIRE(means2D && depths && offsets && radii && compute_locally && keys && values,
              "gs_duplicate_with_keys: null pointer");
-  launch_duplicate_with_keys(P, width, height, means2D, depths, offsets, radii, compute_locally, keys, values,
+  launch_duplicate_with_keys(P, width, height, means2D, depths, offsets, radii, compute_locally, keys, values, nullptr,
                              (hipStream_t)stream);
   return check_launch("duplicate_with_keys", (hipStream_t)stream, false);
 }
@@ -601,12 +616,14 @@ int gs_render_tiles_backward(int P, int width, int height, float tan_fovx, float
                              const float* conic_opacity, const float* rgb, const float* all_maps,
                              const float* all_map_pixels, const float* final_T, const uint32_t* n_contrib_px,
                              const uint8_t* compute_locally, const float* dL_dpix, const float* dL_dout_all_map,
-                             const float* dL_dout_plane_depth, int render_geo, float* dL_dmean2D,
+                             const float* dL_dout_plane_depth, int render_geo, const uint32_t* emission_sorted,
+                             const uint32_t* point_offsets, float* instance_grads, float* dL_dmean2D,
                              float* dL_dmean2D_abs, float* dL_dconic_opacity, float* dL_dcolor, float* dL_dall_map,
                              gs_stream_t stream) {
   GS_REQUIRE(P > 0 && width > 0 && height > 0, "gs_render_tiles_backward: bad sizes");
   GS_REQUIRE(background && ranges && point_list && means2D && conic_opacity && rgb && final_T && n_contrib_px &&
-                 compute_locally && dL_dpix && dL_dmean2D && dL_dmean2D_abs && dL_dconic_opacity && dL_dcolor,
+                 compute_locally && dL_dpix && dL_dmean2D && dL_dmean2D_abs && dL_dconic_opacity && dL_dcolor &&
+                 emission_sorted && point_offsets && instance_grads,
              "gs_render_tiles_backward: null pointer");
   GS_REQUIRE(!render_geo || (dL_dout_all_map && dL_dout_plane_depth && dL_dall_map && all_maps && all_map_pixels),
              "gs_render_tiles_backward: render_geo needs the geometry-map tensors");
@@ -620,6 +637,7 @@ int gs_render_tiles_backward(int P, int width, int height, float tan_fovx, float
   a.compute_locally = compute_locally;
   a.dL_dpix = dL_dpix; a.dL_dout_all_map = dL_dout_all_map; a.dL_dout_plane_depth = dL_dout_plane_depth;
   a.render_geo = render_geo;
+  a.emission_sorted = emission_sorted; a.point_offsets = point_offsets; a.instance_grads = instance_grads;
   a.dL_dmean2D = dL_dmean2D; a.dL_dmean2D_abs = dL_dmean2D_abs; a.dL_dconic_opacity = dL_dconic_opacity;
   a.dL_dcolors = dL_dcolor; a.dL_dall_map = dL_dall_map;
   launch_render_bwd(a, (hipStream_t)stream);

@@ -131,7 +131,8 @@ __global__ void __launch_bounds__(GS_BLOCK_1D)
 duplicate_with_keys_kernel(int P, uint32_t gx, uint32_t gy, const float2* __restrict__ means2D,
                            const float* __restrict__ depths, const uint32_t* __restrict__ offsets,
                            const int* __restrict__ radii, const uint8_t* __restrict__ compute_locally,
-                           uint64_t* __restrict__ keys, uint32_t* __restrict__ values) {
+                           uint64_t* __restrict__ keys, uint32_t* __restrict__ values,
+                           uint32_t* __restrict__ emission) {
   const int i = blockIdx.x * GS_BLOCK_1D + threadIdx.x;
   if (i >= P) return;
   const int r = radii[i];
@@ -146,9 +147,18 @@ duplicate_with_keys_kernel(int P, uint32_t gx, uint32_t gy, const float2* __rest
           const uint64_t key = ((uint64_t)(y * gx + x) << 32) | (uint64_t)dbits;
           keys[off] = key;
           values[off] = (uint32_t)i;
+          if (emission) emission[off] = off;  // position in emission order, carried through the sort
           off++;
         }
   }
+}
+
+// point_list[k] = Gaussian of the instance that the sort moved to position k.
+__global__ void __launch_bounds__(GS_BLOCK_1D)
+gather_u32_kernel(int64_t n, const uint32_t* __restrict__ index, const uint32_t* __restrict__ table,
+                  uint32_t* __restrict__ out) {
+  const int64_t i = (int64_t)blockIdx.x * GS_BLOCK_1D + threadIdx.x;
+  if (i < n) out[i] = table[index[i]];
 }
 
 __global__ void fill_u32_kernel(int64_t n, uint32_t v, uint32_t* __restrict__ p) {
@@ -214,11 +224,19 @@ int launch_exclusive_sum(int64_t n, const uint32_t* in, uint32_t* out, void* tem
 
 int launch_duplicate_with_keys(int P, int W, int H, const float* means2D, const float* depths,
                                const uint32_t* offsets, const int* radii, const uint8_t* compute_locally,
-                               uint64_t* keys, uint32_t* values, hipStream_t stream) {
+                               uint64_t* keys, uint32_t* values, uint32_t* emission, hipStream_t stream) {
   if (P <= 0) return 0;
   const uint32_t gx = (W + GS_TILE_X - 1) / GS_TILE_X, gy = (H + GS_TILE_Y - 1) / GS_TILE_Y;
   hipLaunchKernelGGL(duplicate_with_keys_kernel, dim3((P + GS_BLOCK_1D - 1) / GS_BLOCK_1D), dim3(GS_BLOCK_1D), 0,
-                     stream, P, gx, gy, (const float2*)means2D, depths, offsets, radii, compute_locally, keys, values);
+                     stream, P, gx, gy, (const float2*)means2D, depths, offsets, radii, compute_locally, keys, values,
+                     emission);
+  return 0;
+}
+
+int launch_gather_u32(int64_t n, const uint32_t* index, const uint32_t* table, uint32_t* out, hipStream_t stream) {
+  if (n <= 0) return 0;
+  hipLaunchKernelGGL(gather_u32_kernel, dim3((unsigned)((n + GS_BLOCK_1D - 1) / GS_BLOCK_1D)), dim3(GS_BLOCK_1D), 0,
+                     stream, n, index, table, out);
   return 0;
 }
 

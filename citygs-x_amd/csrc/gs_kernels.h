@@ -52,7 +52,9 @@ int launch_inclusive_sum(int64_t n, const uint32_t* in, uint32_t* out, void* tem
 int launch_exclusive_sum(int64_t n, const uint32_t* in, uint32_t* out, void* temp, hipStream_t stream);
 int launch_duplicate_with_keys(int P, int W, int H, const float* means2D, const float* depths,
                                const uint32_t* offsets, const int* radii, const uint8_t* compute_locally,
-                               uint64_t* keys, uint32_t* values, hipStream_t stream);
+                               uint64_t* keys, uint32_t* values, uint32_t* emission /*optional*/,
+                               hipStream_t stream);
+int launch_gather_u32(int64_t n, const uint32_t* index, const uint32_t* table, uint32_t* out, hipStream_t stream);
 int launch_tile_ranges(int64_t L, const uint64_t* keys_sorted, int T, uint32_t* ranges, hipStream_t stream);
 
 // ---- radix sort (stable, LSD, 8-bit digits) ----
@@ -96,7 +98,13 @@ struct RenderBwdArgs {
   const uint8_t* compute_locally;
   const float *dL_dpix, *dL_dout_all_map, *dL_dout_plane_depth;
   int render_geo;
-  // zero-initialised accumulation targets
+  // Per-instance gradient records: instance_grads[e] (16 floats) for the instance with emission index e;
+  // emission_sorted[k] = emission index of the instance at sorted position k; point_offsets = inclusive
+  // prefix sum of tiles touched, i.e. Gaussian i owns emission indices [point_offsets[i-1], point_offsets[i]).
+  const uint32_t* emission_sorted;
+  const uint32_t* point_offsets;
+  float* instance_grads;  // (R,16) scratch, fully written by the blend kernel
+  // outputs, fully written by the per-Gaussian reduction
   float* dL_dmean2D;         // (P,2)
   float* dL_dmean2D_abs;     // (P,3)
   float* dL_dconic_opacity;  // (P,4) packed [x, y, w, opacity]

@@ -15,9 +15,14 @@
 //     a transposing DPP reduction (15 additions instead of 64) that leaves
 //     component q in lane q, and one LDS float-atomic instruction adds all of
 //     them into a 16x256 accumulator;
-//   * at the end of the batch each thread flushes one Gaussian with global
-//     float atomics: one atomic per (tile, Gaussian, component) instead of
-//     one per (pixel, Gaussian, component).
+//   * at the end of the batch each thread stores one (tile, Gaussian)
+//     instance's 16 sums as one 64-byte record, at the instance's index in
+//     emission order (the order key emission wrote them: all instances of a
+//     Gaussian are consecutive there).  No global atomics at all.
+// A second kernel then sums, for every Gaussian, its consecutive records and
+// writes the five gradient tensors: a streaming pass, deterministic from run to
+// run.  (The reference issues 16 global float atomics per pixel and Gaussian,
+// cuda_rasterizer/backward.cu:510-563.)
 // The per-pixel arithmetic is, operation for operation, the CPU statement's;
 // only the order in which pixels are summed differs, so gradients agree with a
 // CPU evaluation to rounding of the sums, not bit for bit.
@@ -41,10 +46,9 @@ render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
                   const float* __restrict__ final_Ts, const uint32_t* __restrict__ n_contrib_px,
                   const uint8_t* __restrict__ compute_locally, const float* __restrict__ dL_dpix,
                   const float* __restrict__ dL_dout_all_map, const float* __restrict__ dL_dout_plane_depth,
-                  int render_geo, float* __restrict__ dL_dmean2D, float* __restrict__ dL_dmean2D_abs,
-                  float* __restrict__ dL_dconic_opacity, float* __restrict__ dL_dcolors,
-                  float* __restrict__ dL_dall_map) {
-  __shared__ int s_id[BATCH];
+                  int render_geo, const uint32_t* __restrict__ emission_sorted,
+                  float4* __restrict__ instance_grads) {
+  __shared__ uint32_t s_emis[BATCH];
   __shared__ float2 s_xy[BATCH];
   __shared__ float4 s_co[BATCH];
   __shared__ float4 s_bb[BATCH];
@@ -59,7 +63,6 @@ render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
   const RowThread rt = row_thread(blockIdx.x, blockIdx.y);
   const int lane = rt.lane, wave = rt.wave, row = rt.row, l16 = rt.l16;
   const uint32_t tile = blockIdx.y * gridDim.x + blockIdx.x;
-  if (!compute_locally[tile]) return;
   const uint32_t px = rt.px, py = rt.py;
   const bool inside = px < (uint32_t)W && py < (uint32_t)H;
   const size_t pid = (size_t)W * py + px;
@@ -69,6 +72,15 @@ render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
   const float rayy = (float)(((double)pfy - H * 0.5) / (double)fy);
   const uint2 range = ranges[tile];
   const int total = (int)(range.y - range.x);
+  if (!compute_locally[tile]) {
+    // normally an empty range; if the forward pass binned this tile under a wider mask its records are zeros
+    for (int p = tid; p < total; p += GS_TILE_PIX) {
+      float4* rec = instance_grads + 4 * (size_t)emission_sorted[range.x + (uint32_t)p];
+      const float4 z = make_float4(0.f, 0.f, 0.f, 0.f);
+      rec[0] = z; rec[1] = z; rec[2] = z; rec[3] = z;
+    }
+    return;
+  }
 
   const float T_final = inside ? final_Ts[pid] : 0.f;
   float T = T_final;
@@ -85,6 +97,13 @@ render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
   if (lane == 0) s_max[wave] = wave_last;
   __syncthreads();
   const int tile_last = max(max(s_max[0], s_max[1]), max(s_max[2], s_max[3]));
+  // Every instance record of the tile is written exactly once: the ones behind the deepest contributor
+  // get zeros here, the others are written at the end of their batch.
+  for (int p = tile_last + tid; p < total; p += GS_TILE_PIX) {
+    float4* rec = instance_grads + 4 * (size_t)emission_sorted[range.x + (uint32_t)p];
+    const float4 z = make_float4(0.f, 0.f, 0.f, 0.f);
+    rec[0] = z; rec[1] = z; rec[2] = z; rec[3] = z;
+  }
   if (tile_last == 0) return;
 
   float gpix[GS_N_RGB] = {0.f, 0.f, 0.f}, gmap[GS_N_MAP] = {0.f, 0.f, 0.f, 0.f, 0.f};
@@ -118,17 +137,17 @@ render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
   // Slot j of batch i holds position start - (i*BATCH + j).
   const int start = tile_last - 1;
   const int rounds = (start + 1 + BATCH - 1) / BATCH;
-  (void)total;
 
   for (int i = 0; i < rounds; i++) {
     const int first_pos = start - i * BATCH;  // position in slot 0
     const int count = first_pos + 1 < BATCH ? first_pos + 1 : BATCH;
     __syncthreads();
     if (tid < count) {
-      const uint32_t g = point_list[range.x + (uint32_t)(first_pos - tid)];
+      const uint32_t k_sorted = range.x + (uint32_t)(first_pos - tid);
+      const uint32_t g = point_list[k_sorted];
       const float2 xy = means2D[g];
       const float4 co = conic_opacity[g];
-      s_id[tid] = (int)g;
+      s_emis[tid] = emission_sorted[k_sorted];
       s_xy[tid] = xy;
       s_co[tid] = co;
       float pfl;
@@ -256,29 +275,50 @@ render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
     }
     __syncthreads();
     if (tid < count) {
-      float a[NV];
-      bool any = false;
-#pragma unroll
-      for (int q = 0; q < NV; q++) {
-        a[q] = s_acc[q][tid];
-        any = any || (a[q] != 0.f);
-      }
-      if (any) {
-        const size_t g = (size_t)s_id[tid];
-        unsafeAtomicAdd(&dL_dmean2D[2 * g], a[0]);
-        unsafeAtomicAdd(&dL_dmean2D[2 * g + 1], a[1]);
-        unsafeAtomicAdd(&dL_dmean2D_abs[3 * g], a[2]);
-        unsafeAtomicAdd(&dL_dmean2D_abs[3 * g + 1], a[3]);
-#pragma unroll
-        for (int c = 0; c < 4; c++) unsafeAtomicAdd(&dL_dconic_opacity[4 * g + c], a[4 + c]);
-#pragma unroll
-        for (int c = 0; c < GS_N_RGB; c++) unsafeAtomicAdd(&dL_dcolors[3 * g + c], a[8 + c]);
-        if (render_geo) {
-#pragma unroll
-          for (int c = 0; c < GS_N_MAP; c++) unsafeAtomicAdd(&dL_dall_map[5 * g + c], a[11 + c]);
-        }
-      }
+      float4* rec = instance_grads + 4 * (size_t)s_emis[tid];
+      rec[0] = make_float4(s_acc[0][tid], s_acc[1][tid], s_acc[2][tid], s_acc[3][tid]);
+      rec[1] = make_float4(s_acc[4][tid], s_acc[5][tid], s_acc[6][tid], s_acc[7][tid]);
+      rec[2] = make_float4(s_acc[8][tid], s_acc[9][tid], s_acc[10][tid], s_acc[11][tid]);
+      rec[3] = make_float4(s_acc[12][tid], s_acc[13][tid], s_acc[14][tid], s_acc[15][tid]);
     }
+  }
+}
+
+// Sums the instance records of every Gaussian (consecutive in emission order) into the gradient
+// tensors.  Record layout: [mean2D.x, mean2D.y, |mean2D|.x, |mean2D|.y, conic.x, conic.y, conic.w,
+// opacity, rgb(3), map(5)].  Every output element is written.
+__global__ void __launch_bounds__(GS_BLOCK_1D)
+reduce_instances_kernel(int P, const uint32_t* __restrict__ point_offsets, const float4* __restrict__ instance_grads,
+                        int render_geo, float2* __restrict__ dL_dmean2D, float* __restrict__ dL_dmean2D_abs,
+                        float4* __restrict__ dL_dconic_opacity, float* __restrict__ dL_dcolors,
+                        float* __restrict__ dL_dall_map) {
+  const int i = blockIdx.x * GS_BLOCK_1D + threadIdx.x;
+  if (i >= P) return;
+  const uint32_t b = i == 0 ? 0u : point_offsets[i - 1], e = point_offsets[i];
+  float4 a0 = make_float4(0.f, 0.f, 0.f, 0.f), a1 = a0, a2 = a0, a3 = a0;
+  for (uint32_t k = b; k < e; k++) {
+    const float4* rec = instance_grads + 4 * (size_t)k;
+    const float4 r0 = rec[0], r1 = rec[1], r2 = rec[2], r3 = rec[3];
+    a0.x += r0.x; a0.y += r0.y; a0.z += r0.z; a0.w += r0.w;
+    a1.x += r1.x; a1.y += r1.y; a1.z += r1.z; a1.w += r1.w;
+    a2.x += r2.x; a2.y += r2.y; a2.z += r2.z; a2.w += r2.w;
+    a3.x += r3.x; a3.y += r3.y; a3.z += r3.z; a3.w += r3.w;
+  }
+  dL_dmean2D[i] = make_float2(a0.x, a0.y);
+  dL_dmean2D_abs[3 * (size_t)i] = a0.z;
+  dL_dmean2D_abs[3 * (size_t)i + 1] = a0.w;
+  dL_dmean2D_abs[3 * (size_t)i + 2] = 0.f;
+  dL_dconic_opacity[i] = a1;
+  dL_dcolors[3 * (size_t)i] = a2.x;
+  dL_dcolors[3 * (size_t)i + 1] = a2.y;
+  dL_dcolors[3 * (size_t)i + 2] = a2.z;
+  if (dL_dall_map) {
+    float* m = dL_dall_map + 5 * (size_t)i;
+    m[0] = render_geo ? a2.w : 0.f;
+    m[1] = render_geo ? a3.x : 0.f;
+    m[2] = render_geo ? a3.y : 0.f;
+    m[3] = render_geo ? a3.z : 0.f;
+    m[4] = render_geo ? a3.w : 0.f;
   }
 }
 
@@ -289,8 +329,11 @@ int launch_render_bwd(const RenderBwdArgs& a, hipStream_t stream) {
   hipLaunchKernelGGL(render_bwd_kernel, grid, dim3(GS_TILE_PIX), 0, stream, (const uint2*)a.ranges, a.point_list, a.W,
                      a.H, a.fx, a.fy, a.bg, (const float2*)a.means2D, (const float4*)a.conic_opacity, a.rgb, a.all_map,
                      a.all_map_pixels, a.final_T, a.n_contrib_px, a.compute_locally, a.dL_dpix, a.dL_dout_all_map,
-                     a.dL_dout_plane_depth, a.render_geo, a.dL_dmean2D, a.dL_dmean2D_abs, a.dL_dconic_opacity,
-                     a.dL_dcolors, a.dL_dall_map);
+                     a.dL_dout_plane_depth, a.render_geo, a.emission_sorted, (float4*)a.instance_grads);
+  hipLaunchKernelGGL(reduce_instances_kernel, dim3((a.P + GS_BLOCK_1D - 1) / GS_BLOCK_1D), dim3(GS_BLOCK_1D), 0,
+                     stream, a.P, a.point_offsets, (const float4*)a.instance_grads, a.render_geo,
+                     (float2*)a.dL_dmean2D, a.dL_dmean2D_abs, (float4*)a.dL_dconic_opacity, a.dL_dcolors,
+                     a.dL_dall_map);
   return 0;
 }
 

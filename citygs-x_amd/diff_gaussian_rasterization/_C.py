@@ -229,12 +229,15 @@ def render_gaussians_backward(background, tan_fovx, tan_fovy, all_map_pixels, al
     H, W = dL_dout_color.shape[1], dL_dout_color.shape[2]
     f32 = dict(dtype=torch.float32, device=dev)
     geo = bool(render_geo)
-    dL_dmeans2D = torch.zeros(P, 2, **f32)
-    dL_dmeans2D_abs = torch.zeros(P, 3, **f32)
-    dL_dconic_opacity = torch.zeros(P, 4, **f32)
-    dL_dcolors = torch.zeros(P, NUM_CHANNELS, **f32)
-    dL_dall_map = torch.zeros(P, NUM_ALL_MAP, **f32)
+    # every element is written by the native reduction, so no zero fill is needed
+    dL_dmeans2D = torch.empty(P, 2, **f32)
+    dL_dmeans2D_abs = torch.empty(P, 3, **f32)
+    dL_dconic_opacity = torch.empty(P, 4, **f32)
+    dL_dcolors = torch.empty(P, NUM_CHANNELS, **f32)
+    dL_dall_map = torch.empty(P, NUM_ALL_MAP, **f32)
     if P != 0:
+        ws_bytes = _lib.gs_render_backward_workspace_bytes(int(R))
+        workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
         bg = _f32c(background, "background")
         gpix = _f32c(dL_dout_color, "dL_dout_color")
         gmap = _f32c(dL_dout_all_map, "dL_dout_all_map") if geo else None
@@ -249,8 +252,8 @@ def render_gaussians_backward(background, tan_fovx, tan_fovy, all_map_pixels, al
                 P, int(R), _ptr(bg), W, H, float(tan_fovx), float(tan_fovy), _ptr(geomBuffer), _ptr(binningBuffer),
                 _ptr(imageBuffer), _ptr(compute_locally.contiguous()), _ptr(gpix), _ptr(gmap), _ptr(gdep),
                 _ptr(dL_dmeans2D), _ptr(dL_dmeans2D_abs), _ptr(dL_dconic_opacity), _ptr(dL_dcolors), _ptr(dL_dall_map),
-                _ptr(means2D), _ptr(co), _ptr(col), _ptr(am), _ptr(amp), int(geo), int(bool(debug)),
-                C.byref(elapsed) if timing else None, _stream(dev)), "render_gaussians_backward")
+                _ptr(means2D), _ptr(co), _ptr(col), _ptr(am), _ptr(amp), int(geo), int(bool(debug)), _ptr(workspace),
+                ws_bytes, C.byref(elapsed) if timing else None, _stream(dev)), "render_gaussians_backward")
         _record_time(args, "backward_render_time", elapsed.value)
     else:
         _record_time(args, "backward_render_time", 0.0)

@@ -33,7 +33,8 @@ _SIGNATURES = {
                                [_vp] * 8 + [_i, _vp]),
     "gs_render_forward": (_i, [RESIZE_FN, _vp, RESIZE_FN, _vp, RESIZE_FN, _vp, _i, _vp, _i, _i, _f, _f, _f, _f] +
                           [_vp] * 16 + [_i, _i, C.POINTER(_i), C.POINTER(_f), _vp]),
-    "gs_render_backward": (_i, [_i, _i, _vp, _i, _i, _f, _f] + [_vp] * 17 + [_i, _i, C.POINTER(_f), _vp]),
+    "gs_render_backward_workspace_bytes": (_sz, [_i]),
+    "gs_render_backward": (_i, [_i, _i, _vp, _i, _i, _f, _f] + [_vp] * 17 + [_i, _i, _vp, _sz, C.POINTER(_f), _vp]),
     "gs_knn_workspace_bytes": (_sz, [_i]),
     "gs_knn_dist2": (_i, [_i, _vp, _vp, _vp, _sz, _vp]),
     "gs_tile_count": (_i, [_i, _i, _i, _vp, _vp, _vp, _vp, _vp]),
@@ -45,7 +46,7 @@ _SIGNATURES = {
     "gs_sort_pairs_u32": (_i, [_i64, _vp, _vp, _vp, _vp, _i, _vp, _sz, _vp]),
     "gs_identify_tile_ranges": (_i, [_i64, _vp, _i, _vp, _vp]),
     "gs_render_tiles_forward": (_i, [_i, _i, _i, _f, _f, _f, _f] + [_vp] * 8 + [_i] + [_vp] * 11),
-    "gs_render_tiles_backward": (_i, [_i, _i, _i, _f, _f] + [_vp] * 14 + [_i] + [_vp] * 6),
+    "gs_render_tiles_backward": (_i, [_i, _i, _i, _f, _f] + [_vp] * 14 + [_i] + [_vp] * 9),
     "gs_selftest_reductions": (_i, [_vp, _vp, _vp, _vp]),
     "gs_stage_timing_enable": (_i, [_i]),
     "gs_stage_timing_collect": (_i, [C.c_char_p, _sz]),

@@ -117,19 +117,25 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
 /* Replaces Rasterizer::renderBackward (CR/rasterizer.h:162-187,
  * CR/rasterizer_impl.cu:850-932) plus the repacking of
  * RenderGaussiansBackwardCUDA (DGR/rasterize_points.cu:428-440).  The three
- * buffers are the ones gs_render_forward filled.  Gradient outputs must
- * arrive zeroed (they are atomic accumulation targets): dL_dmean2D (P,2),
- * dL_dmean2D_abs (P,3), dL_dconic_opacity (P,4) packed [x, y, w, opacity],
- * dL_dcolor (P,3), dL_dall_map (P,5).  elapsed_ms as above
- * (backward_render_time, CR/rasterizer_impl.cu:924-926). */
+ * buffers are the ones gs_render_forward filled (the geometry buffer is read
+ * too: it holds the per-Gaussian instance offsets).  Gradient outputs are
+ * fully written and need no initialisation: dL_dmean2D (P,2), dL_dmean2D_abs
+ * (P,3), dL_dconic_opacity (P,4) packed [x, y, w, opacity], dL_dcolor (P,3),
+ * dL_dall_map (P,5).  Where the reference adds every pixel's contribution
+ * with global float atomics, this implementation writes one 64-byte record
+ * per (tile, Gaussian) instance into instance_grads, a caller-provided scratch
+ * of gs_render_backward_workspace_bytes(R) bytes, and sums each Gaussian's
+ * records in a second kernel (no atomics, run-to-run deterministic).
+ * elapsed_ms as above (backward_render_time, CR/rasterizer_impl.cu:924-926). */
+size_t gs_render_backward_workspace_bytes(int R);
 int gs_render_backward(int P, int R, const float* background, int width, int height, float tan_fovx,
                        float tan_fovy, const char* geom_buffer, const char* binning_buffer,
                        const char* img_buffer, const uint8_t* compute_locally, const float* dL_dpix,
                        const float* dL_dout_all_map, const float* dL_dout_plane_depth, float* dL_dmean2D,
                        float* dL_dmean2D_abs, float* dL_dconic_opacity, float* dL_dcolor, float* dL_dall_map,
                        const float* means2D, const float* conic_opacity, const float* rgb, const float* all_maps,
-                       const float* all_map_pixels, int render_geo, int debug, float* elapsed_ms,
-                       gs_stream_t stream);
+                       const float* all_map_pixels, int render_geo, int debug, float* instance_grads,
+                       size_t instance_grads_bytes, float* elapsed_ms, gs_stream_t stream);
 
 /* Replaces SimpleKNN::knn / distCUDA2 (KNN/simple_knn.h:17, KNN/simple_knn.cu:185-221,
  * KNN/spatial.cu:17-35): mean_dists[i] = mean squared distance from point i
@@ -183,15 +189,18 @@ int gs_render_tiles_forward(int P, int width, int height, float focal_x, float f
                             int* out_observe, float* out_all_map, float* out_plane_depth, int* n_render,
                             int* n_consider, int* n_contrib, gs_stream_t stream);
 
-/* BACKWARD::render (CR/backward.cu:324-567) on explicit arrays. */
+/* BACKWARD::render (CR/backward.cu:324-567) on explicit arrays.  emission_sorted[k] is the index, in
+ * key-emission order, of the instance at sorted position k (the permutation the sort applied);
+ * point_offsets is the inclusive prefix sum of tiles touched; instance_grads is (R,16) float scratch. */
 int gs_render_tiles_backward(int P, int width, int height, float tan_fovx, float tan_fovy,
                              const float* background, const uint32_t* ranges, const uint32_t* point_list,
                              const float* means2D, const float* conic_opacity, const float* rgb,
                              const float* all_maps, const float* all_map_pixels, const float* final_T,
                              const uint32_t* n_contrib_px, const uint8_t* compute_locally, const float* dL_dpix,
                              const float* dL_dout_all_map, const float* dL_dout_plane_depth, int render_geo,
-                             float* dL_dmean2D, float* dL_dmean2D_abs, float* dL_dconic_opacity,
-                             float* dL_dcolor, float* dL_dall_map, gs_stream_t stream);
+                             const uint32_t* emission_sorted, const uint32_t* point_offsets,
+                             float* instance_grads, float* dL_dmean2D, float* dL_dmean2D_abs,
+                             float* dL_dconic_opacity, float* dL_dcolor, float* dL_dall_map, gs_stream_t stream);
 
 /* Diagnostic with no counterpart in the reference: runs the two cross-lane
  * reductions of the blend kernels on one 64-lane wave.  in is (64,16) floats;

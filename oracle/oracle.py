@@ -187,8 +187,11 @@ def bin_and_sort(radii, means2D, depths, compute_locally, W, H):
     bit = higher_msb(gx * gy)
     ks, vs = sort_pairs(keys, vals, 32 + bit)
     ranges = tile_ranges(ks, gx * gy)
+    # the permutation the stable sort applied: sorted position -> index in emission order
+    mask = np.uint64((1 << (32 + bit)) - 1)
+    emission_sorted = np.argsort(keys & mask, kind="stable").astype(np.uint32)
     return dict(tiles_touched=tt, point_offsets=offs, keys_unsorted=keys, vals_unsorted=vals, keys=ks,
-                point_list=vs, ranges=ranges, num_rendered=int(keys.size))
+                point_list=vs, ranges=ranges, num_rendered=int(keys.size), emission_sorted=emission_sorted)
 
 
 def render_fwd(ranges, point_list, means2D, rgb, all_map, conic_opacity, compute_locally, bg, W, H, tanx, tany,

@@ -155,14 +155,17 @@ def render_fwd(P, W, H, tanx, tany, ranges, point_list, means2D, rgb, all_map, c
 
 
 def render_bwd(P, W, H, tanx, tany, bg, ranges, point_list, means2D, conic_opacity, rgb, all_map, all_map_pixels,
-               final_T, n_contrib, cl, gpix, gmap, gdepth, render_geo=True):
-    z = lambda *s: torch.zeros(s, device=DEV)
+               final_T, n_contrib, cl, gpix, gmap, gdepth, emission_sorted, point_offsets, render_geo=True):
+    z = lambda *s: torch.full(s, 44.0, device=DEV)  # outputs must be fully overwritten
     o = dict(dL_dmeans2D=z(P, 2), dL_dmeans2D_abs=z(P, 3), dL_dconic_opacity=z(P, 4), dL_dcolors=z(P, 3),
              dL_dall_map=z(P, 5))
+    R = int(point_list.shape[0])
+    recs = torch.full((max(R, 1), 16), float("nan"), device=DEV)
     gn.check(lib.gs_render_tiles_backward(
         P, W, H, tanx, tany, ptr(bg), ptr(ranges), ptr(point_list), ptr(means2D), ptr(conic_opacity), ptr(rgb),
         ptr(all_map), ptr(all_map_pixels), ptr(final_T), ptr(n_contrib), ptr(cl), ptr(gpix), ptr(gmap), ptr(gdepth),
-        int(render_geo), ptr(o["dL_dmeans2D"]), ptr(o["dL_dmeans2D_abs"]), ptr(o["dL_dconic_opacity"]),
+        int(render_geo), ptr(emission_sorted), ptr(point_offsets), ptr(recs), ptr(o["dL_dmeans2D"]),
+        ptr(o["dL_dmeans2D_abs"]), ptr(o["dL_dconic_opacity"]),
         ptr(o["dL_dcolors"]), ptr(o["dL_dall_map"]), stream()), "gs_render_tiles_backward")
     torch.cuda.synchronize()
     return o

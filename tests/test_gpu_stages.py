@@ -163,7 +163,8 @@ def test_render_backward(H, orc, cfg, P, mask, geo):
     got = H.render_bwd(P, W, Hh, cam.tanfovx, cam.tanfovy, H.dev(bg), H.as_u32(b["ranges"]), H.as_u32(b["point_list"]),
                        H.dev(pre["means2D"]), H.dev(pre["conic_opacity"]), H.dev(pre["rgb"]), H.dev(am),
                        H.dev(f["out_all_map"]), H.dev(f["final_T"]), H.as_u32(f["n_contrib"]), H.dev(cl), H.dev(gpix),
-                       H.dev(gmap), H.dev(gdep), render_geo=geo)
+                       H.dev(gmap), H.dev(gdep), H.as_u32(b["emission_sorted"]), H.as_u32(b["point_offsets"]),
+                       render_geo=geo)
     pairs = [("dL_dmeans2D", ref["dL_dmeans2D"][:, :2]), ("dL_dmeans2D_abs", ref["dL_dmeans2D_abs"]),
              ("dL_dconic_opacity", ref["dL_dconic_opacity"]), ("dL_dcolors", ref["dL_dcolors"])]
     if geo:
