@@ -9,14 +9,21 @@
 // digit bases; then each pass is ONE kernel that reads every pair once and
 // writes it once.  Inside a pass a 4096-pair tile
 //   1. takes a ticket (atomic counter), so tile numbers follow start order;
-//   2. ranks its keys: per wave, lanes holding equal digits are matched with
-//      eight ballots, and a per-wave running counter per digit in LDS gives
-//      each key its rank in wave order (stable);
-//   3. publishes its 256 digit counts (flag "aggregate") and looks back over
-//      the preceding tiles, adding aggregates until it meets a tile whose
-//      inclusive prefix is already published, then publishes its own prefix;
+//   2. ranks its keys: per wave, lanes holding equal digits find each other
+//      through a lane mask per digit in LDS, and a per-wave running counter
+//      per digit gives each key its rank in wave order (stable);
+//   3. publishes its 256 digit counts and finds how many keys of each digit
+//      precede it with a two-level look-back (below);
 //   4. regroups its pairs by digit in LDS and writes each digit run to
 //      consecutive addresses.
+// Look-back: tiles form groups of 16.  A tile adds the counts of the tiles
+// before it in its own group (these need no prefix, only the counts, so
+// nothing chains), then walks back over whole groups: a group entry is
+// either the group's sum ("aggregate", published by the group's last tile as
+// soon as the 16 counts exist) or the inclusive prefix up to the group's end
+// (published by the same tile after its own walk).  One round trip to memory
+// therefore advances the prefix frontier by 16 groups = 256 tiles, instead of
+// one tile per round trip in a plain chain.
 // A tile only ever waits for tiles with smaller tickets, which have already
 // started, so the wait always ends; the spin is bounded anyway and raises an
 // error flag instead of hanging.
@@ -39,9 +46,11 @@ constexpr uint32_t FLAG_AGGREGATE = 1u << 30;
 constexpr uint32_t FLAG_PREFIX = 2u << 30;
 constexpr uint32_t VALUE_MASK = (1u << 30) - 1u;
 constexpr int SPIN_LIMIT = 1 << 22;
+constexpr int GROUP = 16;           // tiles per look-back group
+constexpr int GROUP_LOOKBACK = 16;  // group entries fetched per round trip
 
 // Control block in the workspace: [hist: MAX_PASSES*256][ticket: MAX_PASSES][error: 1][pad to 16]
-// followed by the tile states [passes][ntiles][256].
+// followed by the tile counts [passes][ntiles][256] and the group entries [passes][ngroups][256].
 constexpr size_t CTRL_WORDS = MAX_PASSES * RADIX + 16;
 
 template <typename K>
@@ -64,12 +73,20 @@ sort_histogram_kernel(int64_t n, const K* __restrict__ keys, int passes, int end
 #pragma unroll 4
   for (int k = 0; k < HIST_ITEMS; k++) {
     const int64_t idx = base + (int64_t)k * SORT_THREADS + threadIdx.x;
-    if (idx < n) {
-      const K key = keys[idx];
-      for (int p = 0; p < passes; p++) {
-        const int shift = 8 * p;
-        const int bits = end_bit - shift >= 8 ? 8 : end_bit - shift;
-        atomicAdd(&s_h[p][digit_of(key, shift, (1u << bits) - 1u)], 1u);
+    const bool valid = idx < n;
+    const K key = valid ? keys[idx] : (K)0;
+    for (int p = 0; p < passes; p++) {
+      const int shift = 8 * p;
+      const int bits = end_bit - shift >= 8 ? 8 : end_bit - shift;
+      const uint32_t d = digit_of(key, shift, (1u << bits) - 1u);
+      // A digit shared by the whole wave (float exponent bits, unused high bits) would serialise the LDS
+      // atomic 64 ways: one lane adds the wave's count instead.
+      const uint64_t vm = __ballot(valid);
+      const uint32_t d0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)d);
+      if (vm != 0ull && __ballot(valid && d == d0) == vm && (vm & 1ull)) {
+        if ((threadIdx.x & (GS_WAVE - 1)) == 0) atomicAdd(&s_h[p][d0], (uint32_t)__popcll(vm));
+      } else if (valid) {
+        atomicAdd(&s_h[p][d], 1u);
       }
     }
   }
@@ -99,24 +116,66 @@ __global__ void __launch_bounds__(RADIX) sort_digit_bases_kernel(uint32_t* __res
   h[threadIdx.x] = base + inc - v;
 }
 
+// Sums the entries [first, last] of a 256-wide state array for digit `tid`, newest first, W entries per round
+// trip, until an entry flagged FLAG_PREFIX has been added (or `first` has been passed).  Entries not yet
+// published (flag 0) are polled.  Returns false when the bounded spin ran out.
+template <int W>
+__device__ __forceinline__ bool look_back(const uint32_t* __restrict__ state, int64_t first, int64_t last, int tid,
+                                          uint32_t& sum) {
+  int64_t prev = last;
+  int spins = 0;
+  bool finished = prev < first;
+  while (!finished) {
+    uint32_t s[W];
+#pragma unroll
+    for (int i = 0; i < W; i++) {
+      const int64_t t = prev - i;
+      // before `first` there is nothing: reads as a published prefix of 0, which ends the walk
+      s[i] = t >= first ? __hip_atomic_load(state + (size_t)t * RADIX + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+                        : FLAG_PREFIX;
+    }
+    int consumed = 0;
+#pragma unroll
+    for (int i = 0; i < W; i++) {
+      if (finished || consumed != i) continue;  // stopped at an entry that is not published yet
+      const uint32_t flag = s[i] & ~VALUE_MASK;
+      if (flag == 0u) continue;
+      sum += s[i] & VALUE_MASK;
+      consumed = i + 1;
+      if (flag == FLAG_PREFIX) finished = true;
+    }
+    prev -= consumed;
+    if (!finished && consumed < W) {
+      if (++spins > SPIN_LIMIT) return false;
+      __builtin_amdgcn_s_sleep(1);
+    }
+  }
+  return true;
+}
+
 template <typename K>
 __global__ void __launch_bounds__(SORT_THREADS)
 sort_onesweep_kernel(int64_t n, const K* __restrict__ keys_in, K* __restrict__ keys_out,
                      const uint32_t* __restrict__ vals_in, uint32_t* __restrict__ vals_out, int shift, uint32_t mask,
                      const uint32_t* __restrict__ digit_base, uint32_t* __restrict__ ticket,
-                     uint32_t* __restrict__ tile_state, uint32_t* __restrict__ error_flag) {
+                     uint32_t* __restrict__ tile_state, uint32_t* __restrict__ group_state, int ntiles,
+                     uint32_t* __restrict__ error_flag) {
   __shared__ uint32_t s_wcount[SORT_WAVES][RADIX];
-  __shared__ uint32_t s_dbase[RADIX];
   __shared__ uint32_t s_gbase[RADIX];
   __shared__ uint32_t s_scan[SORT_WAVES];
   __shared__ uint32_t s_tile;
+  // regrouping buffer: keys first, then reused for the values; before that its head holds the lane masks
   __shared__ K s_keys[SORT_TILE];
-  __shared__ uint32_t s_vals[SORT_TILE];
+  static_assert(sizeof(K) * SORT_TILE >= sizeof(unsigned long long) * SORT_WAVES * RADIX, "lane masks must fit");
+  unsigned long long (*s_mask)[RADIX] = reinterpret_cast<unsigned long long (*)[RADIX]>(s_keys);
 
   const int tid = threadIdx.x, lane = tid & (GS_WAVE - 1), wave = tid / GS_WAVE;
   if (tid == 0) s_tile = atomicAdd(ticket, 1u);
 #pragma unroll
-  for (int w = 0; w < SORT_WAVES; w++) s_wcount[w][tid] = 0;
+  for (int w = 0; w < SORT_WAVES; w++) {
+    s_wcount[w][tid] = 0;
+    s_mask[w][tid] = 0ull;
+  }
   __syncthreads();
   const uint32_t tile = s_tile;
   const int64_t tile_start = (int64_t)tile * SORT_TILE;
@@ -126,7 +185,6 @@ sort_onesweep_kernel(int64_t n, const K* __restrict__ keys_in, K* __restrict__ k
 
   K key[SORT_ITEMS];
   uint32_t val[SORT_ITEMS];
-  uint16_t rank[SORT_ITEMS];
 #pragma unroll
   for (int k = 0; k < SORT_ITEMS; k++) {
     const int64_t idx = wave_start + (int64_t)k * GS_WAVE + lane;
@@ -134,48 +192,73 @@ sort_onesweep_kernel(int64_t n, const K* __restrict__ keys_in, K* __restrict__ k
     key[k] = valid ? keys_in[idx] : (K)0;
     val[k] = valid ? vals_in[idx] : 0u;
   }
-  const uint64_t lt_mask = (1ull << lane) - 1ull;
+
+  // Ranking.  LDS operations of one wave execute in program order, which the two steps below rely on; none
+  // of them waits for an earlier one's result, so all items are in flight together.
+  // Step 1: the lanes of the wave that hold the same digit find each other through a 64-bit lane mask per
+  // digit: every lane ORs its bit in, reads the mask back, and clears it for the next item.
+  volatile unsigned long long* vmask = s_mask[wave];
+  volatile uint32_t* vcount = s_wcount[wave];
+  const unsigned long long lane_bit = 1ull << lane;
+  const unsigned long long lt_mask = lane_bit - 1ull;
+  uint32_t match[SORT_ITEMS];  // rank in the wave | valid << 17; later the place in the regrouped tile
+  constexpr int HALF = SORT_ITEMS / 2;  // two batches keep fewer masks live in registers
 #pragma unroll
-  for (int k = 0; k < SORT_ITEMS; k++) {
-    const int64_t idx = wave_start + (int64_t)k * GS_WAVE + lane;
-    const bool valid = idx < n;
-    const uint32_t d = digit_of(key[k], shift, mask);
-    uint64_t same = __ballot(valid);
+  for (int h = 0; h < 2; h++) {
+    unsigned long long same[HALF];
 #pragma unroll
-    for (int b = 0; b < 8; b++) {
-      const bool bit = (d >> b) & 1u;
-      const uint64_t vote = __ballot(valid && bit);
-      same &= bit ? vote : ~vote;
-    }
-    uint32_t r = 0;
-    if (valid) {
-      const uint32_t before = s_wcount[wave][d];
-      r = before + (uint32_t)__popcll(same & lt_mask);
+    for (int j = 0; j < HALF; j++) {
+      const int k = h * HALF + j;
+      const bool valid = wave_start + (int64_t)k * GS_WAVE + lane < n;
+      const uint32_t d = digit_of(key[k], shift, mask);
+      if (valid) atomicOr(&s_mask[wave][d], lane_bit);
       __builtin_amdgcn_wave_barrier();
-      if ((same & lt_mask) == 0ull) s_wcount[wave][d] = before + (uint32_t)__popcll(same);
+      same[j] = valid ? vmask[d] : 0ull;
+      __builtin_amdgcn_wave_barrier();
+      if (valid) vmask[d] = 0ull;
+      __builtin_amdgcn_wave_barrier();
     }
-    __builtin_amdgcn_wave_barrier();
-    rank[k] = (uint16_t)r;
+    // Step 2: a per-wave running count per digit turns the place among the matching lanes into a rank in
+    // wave order (stable): all lanes read the count, the first of the matching lanes adds their number.
+#pragma unroll
+    for (int j = 0; j < HALF; j++) {
+      const int k = h * HALF + j;
+      const bool valid = same[j] != 0ull;
+      const uint32_t d = digit_of(key[k], shift, mask);
+      const unsigned long long lower = same[j] & lt_mask;
+      const uint32_t before = valid ? vcount[d] : 0u;
+      __builtin_amdgcn_wave_barrier();
+      if (valid && lower == 0ull) atomicAdd(&s_wcount[wave][d], (uint32_t)__popcll(same[j]));
+      __builtin_amdgcn_wave_barrier();
+      match[k] = (before + (uint32_t)__popcll(lower)) | (valid ? 1u << 17 : 0u);
+    }
   }
   __syncthreads();
 
   // thread tid owns digit tid
+  uint32_t wcount[SORT_WAVES];
   uint32_t total = 0;
-  {
-    uint32_t run = 0;
 #pragma unroll
-    for (int w = 0; w < SORT_WAVES; w++) {
-      const uint32_t c = s_wcount[w][tid];
-      s_wcount[w][tid] = run;
-      run += c;
-    }
-    total = run;
+  for (int w = 0; w < SORT_WAVES; w++) {
+    wcount[w] = s_wcount[w][tid];
+    total += wcount[w];
   }
-  uint32_t* my_state = tile_state + (size_t)tile * RADIX + tid;
-  __hip_atomic_store(my_state, (tile == 0 ? FLAG_PREFIX : FLAG_AGGREGATE) | total, __ATOMIC_RELAXED,
+  // counts of this tile, for the later tiles of its group
+  __hip_atomic_store(tile_state + (size_t)tile * RADIX + tid, FLAG_AGGREGATE | total, __ATOMIC_RELAXED,
                      __HIP_MEMORY_SCOPE_AGENT);
 
-  // digit prefix inside the tile (needed for the LDS regrouping); overlaps with the look-back latency
+  // Look-back, level 1, issue: fetch the counts of the earlier tiles of the own group now and use them after
+  // the regrouping below, so the round trip to memory overlaps with LDS work.
+  const int64_t group = tile / GROUP;
+  const int in_group = (int)(tile % GROUP);
+  uint32_t earlier[GROUP - 1];
+#pragma unroll
+  for (int i = 0; i < GROUP - 1; i++)
+    earlier[i] = i < in_group ? __hip_atomic_load(tile_state + (size_t)(tile - 1 - i) * RADIX + tid, __ATOMIC_RELAXED,
+                                                  __HIP_MEMORY_SCOPE_AGENT)
+                              : FLAG_AGGREGATE;
+
+  // digit prefix inside the tile, then regroup the keys by digit in LDS
   uint32_t inc = total;
 #pragma unroll
   for (int dd = 1; dd < GS_WAVE; dd <<= 1) {
@@ -189,62 +272,93 @@ sort_onesweep_kernel(int64_t n, const K* __restrict__ keys_in, K* __restrict__ k
   for (int w = 0; w < SORT_WAVES; w++)
     if (w < wave) wbase += s_scan[w];
   const uint32_t ex = wbase + inc - total;
-
-  // decoupled look-back over the preceding tiles
-  uint32_t before_tiles = 0;
-  if (tile != 0) {
-    int64_t prev = (int64_t)tile - 1;
-    int spins = 0;
-    for (;;) {
-      const uint32_t s = __hip_atomic_load(tile_state + (size_t)prev * RADIX + tid, __ATOMIC_RELAXED,
-                                           __HIP_MEMORY_SCOPE_AGENT);
-      const uint32_t flag = s & ~VALUE_MASK;
-      if (flag == 0u) {
-        if (++spins > SPIN_LIMIT) {
-          *error_flag = 1u;
-          break;
-        }
-        __builtin_amdgcn_s_sleep(1);
-        continue;
-      }
-      before_tiles += s & VALUE_MASK;
-      if (flag == FLAG_PREFIX) break;
-      prev--;  // an aggregate: keep walking back (prev >= 0 because tile 0 always publishes a prefix)
+  {
+    // s_wcount[w][d] becomes the place in the regrouped tile of wave w's first key with digit d
+    uint32_t run = ex;
+#pragma unroll
+    for (int w = 0; w < SORT_WAVES; w++) {
+      s_wcount[w][tid] = run;
+      run += wcount[w];
     }
-    __hip_atomic_store(my_state, FLAG_PREFIX | ((before_tiles + total) & VALUE_MASK), __ATOMIC_RELAXED,
-                       __HIP_MEMORY_SCOPE_AGENT);
   }
-  s_dbase[tid] = ex;
-  s_gbase[tid] = digit_base[tid] + before_tiles - ex;
   __syncthreads();
 
 #pragma unroll
   for (int k = 0; k < SORT_ITEMS; k++) {
-    const int64_t idx = wave_start + (int64_t)k * GS_WAVE + lane;
-    if (idx < n) {
-      const uint32_t d = digit_of(key[k], shift, mask);
-      const uint32_t pos = s_dbase[d] + s_wcount[wave][d] + (uint32_t)rank[k];
-      s_keys[pos] = key[k];
-      s_vals[pos] = val[k];
-    }
+    const uint32_t d = digit_of(key[k], shift, mask);
+    const bool valid = match[k] & (1u << 17);
+    const uint32_t pos = s_wcount[wave][d] + (match[k] & 0xFFFFu);
+    if (valid) s_keys[pos] = key[k];
+    match[k] = valid ? pos : 0xFFFFFFFFu;  // now: place in the regrouped tile, or none
   }
   __syncthreads();
-
 #pragma unroll
   for (int k = 0; k < SORT_ITEMS; k++) {
     const int p = k * SORT_THREADS + tid;
-    if (p < tile_count) {
-      const K kk = s_keys[p];
-      const uint32_t dst = s_gbase[digit_of(kk, shift, mask)] + (uint32_t)p;
-      keys_out[dst] = kk;
-      vals_out[dst] = s_vals[p];
+    key[k] = p < tile_count ? s_keys[p] : (K)0;  // from here on: the key at regrouped place p
+  }
+
+  // Look-back, level 1, use: all earlier tiles of the group must have published; poll the late ones
+  uint32_t before_tiles = 0;
+  bool ok = true;
+  uint32_t missing = 0;
+#pragma unroll
+  for (int i = 0; i < GROUP - 1; i++) {
+    before_tiles += earlier[i] & VALUE_MASK;
+    if ((earlier[i] & ~VALUE_MASK) == 0u) missing |= 1u << i;
+  }
+  for (int spins = 0; missing != 0u;) {
+    const int i = __builtin_ctz(missing);
+    const uint32_t v = __hip_atomic_load(tile_state + (size_t)(tile - 1 - i) * RADIX + tid, __ATOMIC_RELAXED,
+                                         __HIP_MEMORY_SCOPE_AGENT);
+    if ((v & ~VALUE_MASK) != 0u) {
+      before_tiles += v & VALUE_MASK;
+      missing &= missing - 1u;
+    } else if (++spins > SPIN_LIMIT) {
+      ok = false;
+      break;
+    } else {
+      __builtin_amdgcn_s_sleep(1);
     }
+  }
+  // level 2: whole groups
+  const bool closes_group = in_group == GROUP - 1;  // an incomplete last group is never looked at
+  if (closes_group)
+    __hip_atomic_store(group_state + (size_t)group * RADIX + tid,
+                       (group == 0 ? FLAG_PREFIX : FLAG_AGGREGATE) | ((before_tiles + total) & VALUE_MASK),
+                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if (group != 0) {
+    ok = look_back<GROUP_LOOKBACK>(group_state, 0, group - 1, tid, before_tiles) && ok;
+    if (closes_group)
+      __hip_atomic_store(group_state + (size_t)group * RADIX + tid, FLAG_PREFIX | ((before_tiles + total) & VALUE_MASK),
+                         __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  if (!ok) *error_flag = 1u;
+  s_gbase[tid] = digit_base[tid] + before_tiles - ex;
+  __syncthreads();  // also: every read of s_keys above is complete, the buffer can take the values
+
+  uint32_t dst[SORT_ITEMS];
+#pragma unroll
+  for (int k = 0; k < SORT_ITEMS; k++) {
+    const int p = k * SORT_THREADS + tid;
+    dst[k] = s_gbase[digit_of(key[k], shift, mask)] + (uint32_t)p;
+    if (p < tile_count) keys_out[dst[k]] = key[k];
+  }
+  uint32_t* s_vals = reinterpret_cast<uint32_t*>(s_keys);
+#pragma unroll
+  for (int k = 0; k < SORT_ITEMS; k++)
+    if (match[k] != 0xFFFFFFFFu) s_vals[match[k]] = val[k];
+  __syncthreads();
+#pragma unroll
+  for (int k = 0; k < SORT_ITEMS; k++) {
+    const int p = k * SORT_THREADS + tid;
+    if (p < tile_count) vals_out[dst[k]] = s_vals[p];
   }
 }
 
 struct SortLayout {
   size_t ctrl_words, state_words, total_bytes;
-  int ntiles;
+  int ntiles, ngroups;
 };
 
 SortLayout sort_layout(int64_t n) {
@@ -252,7 +366,8 @@ SortLayout sort_layout(int64_t n) {
   const int64_t nt = (n + SORT_TILE - 1) / SORT_TILE;
   L.ntiles = (int)(nt > 0 ? nt : 1);
   L.ctrl_words = CTRL_WORDS;
-  L.state_words = (size_t)MAX_PASSES * L.ntiles * RADIX;
+  L.ngroups = (L.ntiles + GROUP - 1) / GROUP;
+  L.state_words = (size_t)MAX_PASSES * (L.ntiles + L.ngroups) * RADIX;
   L.total_bytes = align_up((L.ctrl_words + L.state_words) * sizeof(uint32_t), 256);
   return L;
 }
@@ -276,7 +391,8 @@ int sort_pairs_impl(int64_t n, K* keys_a, K* keys_b, uint32_t* vals_a, uint32_t*
   uint32_t* tickets = ctrl + MAX_PASSES * RADIX;
   uint32_t* error_flag = tickets + MAX_PASSES;
   uint32_t* states = ctrl + L.ctrl_words;
-  const int64_t clear_words = (int64_t)(L.ctrl_words + (size_t)passes * L.ntiles * RADIX);
+  uint32_t* group_states = states + (size_t)passes * L.ntiles * RADIX;
+  const int64_t clear_words = (int64_t)(L.ctrl_words + (size_t)passes * (L.ntiles + L.ngroups) * RADIX);
   hipLaunchKernelGGL(sort_clear_kernel, dim3((unsigned)((clear_words + 255) / 256)), dim3(256), 0, stream, clear_words,
                      ctrl);
   const int hist_blocks = (int)((n + SORT_THREADS * HIST_ITEMS - 1) / (SORT_THREADS * HIST_ITEMS));
@@ -292,7 +408,8 @@ int sort_pairs_impl(int64_t n, K* keys_a, K* keys_b, uint32_t* vals_a, uint32_t*
     const int bits = end_bit - shift >= 8 ? 8 : end_bit - shift;
     const uint32_t mask = (1u << bits) - 1u;
     hipLaunchKernelGGL(sort_onesweep_kernel<K>, dim3(L.ntiles), dim3(SORT_THREADS), 0, stream, n, kin, kout, vin, vout,
-                       shift, mask, hist + p * RADIX, tickets + p, states + (size_t)p * L.ntiles * RADIX, error_flag);
+                       shift, mask, hist + p * RADIX, tickets + p, states + (size_t)p * L.ntiles * RADIX,
+                       group_states + (size_t)p * L.ngroups * RADIX, L.ntiles, error_flag);
     K* tk = kin; kin = kout; kout = tk;
     uint32_t* tv = vin; vin = vout; vout = tv;
   }
