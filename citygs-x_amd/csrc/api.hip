@@ -12,6 +12,9 @@
 #include "gs_common.h"
 #include "gs_kernels.h"
 
+#include <atomic>
+#include <mutex>
+
 namespace gs {
 
 static thread_local char g_err[512] = "";
@@ -308,6 +311,65 @@ int gs_preprocess_backward(const int* radii, const float* cov3D, const uint8_t* 
   return check_launch("preprocess_backward", (hipStream_t)stream, debug != 0);
 }
 
+// Host-visible words through which the scan hands the instance count to the waiting host thread.  Pinned
+// memory is allocated once per process; calls take the words in turn, so calls on different streams or
+// threads do not share one unless more than TOTAL_SLOTS of them are inside gs_render_forward together.
+namespace {
+constexpr uint32_t TOTAL_PENDING = 0xFFFFFFFFu;  // never a valid count (counts stay below 2^31)
+constexpr int TOTAL_SLOTS = 64;
+std::atomic<uint32_t*> g_total_slots{nullptr};
+std::atomic<unsigned> g_total_next{0};
+std::mutex g_total_mutex;
+
+uint32_t* acquire_total_slot() {
+  uint32_t* base = g_total_slots.load(std::memory_order_acquire);
+  if (base == nullptr) {
+    std::lock_guard<std::mutex> lock(g_total_mutex);
+    base = g_total_slots.load(std::memory_order_acquire);
+    if (base == nullptr) {
+      void* p = nullptr;
+      // 64-byte spacing keeps the words on separate lines
+      if (hipHostMalloc(&p, TOTAL_SLOTS * 64, hipHostMallocDefault) != hipSuccess) {
+        (void)hipGetLastError();
+        return nullptr;  // the caller falls back to a copy and a stream wait
+      }
+      base = (uint32_t*)p;
+      g_total_slots.store(base, std::memory_order_release);
+    }
+  }
+  uint32_t* slot = base + 16 * (g_total_next.fetch_add(1, std::memory_order_relaxed) % TOTAL_SLOTS);
+  __atomic_store_n(slot, TOTAL_PENDING, __ATOMIC_RELEASE);
+  return slot;
+}
+
+// Polls the word; looks at the stream now and then so that a failed launch ends the wait with its error.
+int wait_for_total(uint32_t* slot, hipStream_t stream, uint32_t* out) {
+  for (unsigned spins = 0;; spins++) {
+    const uint32_t v = __atomic_load_n(slot, __ATOMIC_ACQUIRE);
+    if (v != TOTAL_PENDING) {
+      *out = v;
+      return 0;
+    }
+    if ((spins & 0x3FFFu) == 0x3FFFu) {
+      const hipError_t q = hipStreamQuery(stream);
+      if (q == hipSuccess) {
+        const uint32_t w = __atomic_load_n(slot, __ATOMIC_ACQUIRE);
+        if (w != TOTAL_PENDING) {
+          *out = w;
+          return 0;
+        }
+        set_error("gs_render_forward: the stream drained without the scan reporting its total");
+        return 1;
+      }
+      if (q != hipErrorNotReady) {
+        set_error("gs_render_forward: waiting for the instance count: %s", hipGetErrorString(q));
+        return 1;
+      }
+    }
+  }
+}
+}  // namespace
+
 int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resize_fn binningBuffer,
                       void* binning_user, gs_resize_fn imageBuffer, void* image_user, int P, const float* background,
                       int width, int height, float focal_x, float focal_y, float cx, float cy,
@@ -349,6 +411,7 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
   uint32_t* n_contrib2loss_px = (uint32_t*)(ibase + IL.n_contrib2loss);
   uint32_t* ranges = (uint32_t*)(ibase + IL.ranges);
 
+  uint32_t* total_slot = acquire_total_slot();
   {
     StageScope _t("tile_count", stream);
     launch_tile_count(P, width, height, radii, means2D, compute_locally, tiles_touched, stream);
@@ -356,13 +419,20 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
   if (check_launch("tile_count", stream, dbg)) return 1;
   {
     StageScope _t("inclusive_sum", stream);
-    launch_inclusive_sum(P, tiles_touched, point_offsets, scan_temp, stream);
+    launch_inclusive_sum(P, tiles_touched, point_offsets, scan_temp, stream, total_slot);
   }
   if (check_launch("inclusive_sum", stream, dbg)) return 1;
 
+  // The instance count decides the size of the binning buffer, so the host needs it here.  The scan writes
+  // it straight into pinned host memory and the host polls that word: no copy, and no sleeping wait whose
+  // wake-up would leave the GPU idle.
   uint32_t R_u = 0;
-  GS_HIP_TRY(hipMemcpyAsync(&R_u, point_offsets + (P - 1), sizeof(uint32_t), hipMemcpyDeviceToHost, stream));
-  GS_HIP_TRY(hipStreamSynchronize(stream));
+  if (total_slot != nullptr) {
+    if (wait_for_total(total_slot, stream, &R_u)) return 1;
+  } else {
+    GS_HIP_TRY(hipMemcpyAsync(&R_u, point_offsets + (P - 1), sizeof(uint32_t), hipMemcpyDeviceToHost, stream));
+    GS_HIP_TRY(hipStreamSynchronize(stream));
+  }
   if (R_u >= 0x7FFFFFFFu) {
     set_error("gs_render_forward: %u (Gaussian, tile) instances exceed the supported 2^31-2", R_u);
     return 1;

@@ -100,7 +100,8 @@ __global__ void __launch_bounds__(1024) scan_spine_kernel(int nblocks, uint32_t*
 
 template <bool EXCLUSIVE>
 __global__ void __launch_bounds__(SCAN_THREADS)
-scan_apply_kernel(int64_t n, const uint32_t* in, const uint32_t* __restrict__ block_prefix, uint32_t* out) {
+scan_apply_kernel(int64_t n, const uint32_t* in, const uint32_t* __restrict__ block_prefix, uint32_t* out,
+                  uint32_t* total_out) {
   // in and out may be the same array: each thread reads its items before it writes them.
   __shared__ uint32_t s_wave[SCAN_THREADS / GS_WAVE];
   // Blocked arrangement: thread t owns SCAN_ITEMS consecutive elements.
@@ -124,6 +125,10 @@ scan_apply_kernel(int64_t n, const uint32_t* in, const uint32_t* __restrict__ bl
       if (base + k < n) out[base + k] = run;
     }
   }
+  // The owner of the last element also hands the grand total to the host, which may be polling this word
+  // (host-visible memory), so the store is made visible system wide.
+  if (total_out != nullptr && n - 1 >= base && n - 1 < base + SCAN_ITEMS)
+    __hip_atomic_store(total_out, run, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
 }
 
 // cuda_rasterizer/rasterizer_impl.cu:74-117.
@@ -200,26 +205,28 @@ size_t scan_temp_bytes(int64_t n) {
   return align_up((size_t)(nb > 0 ? nb : 1) * sizeof(uint32_t), 256);
 }
 
-static int scan_impl(int64_t n, const uint32_t* in, uint32_t* out, void* temp, bool exclusive, hipStream_t stream) {
+static int scan_impl(int64_t n, const uint32_t* in, uint32_t* out, void* temp, bool exclusive, uint32_t* total_out,
+                     hipStream_t stream) {
   if (n <= 0) return 0;
   const int nb = (int)((n + SCAN_TILE - 1) / SCAN_TILE);
   uint32_t* sums = (uint32_t*)temp;
   hipLaunchKernelGGL(scan_block_sums_kernel, dim3(nb), dim3(SCAN_THREADS), 0, stream, n, in, sums);
   hipLaunchKernelGGL(scan_spine_kernel, dim3(1), dim3(1024), 0, stream, nb, sums);
   if (exclusive)
-    hipLaunchKernelGGL(scan_apply_kernel<true>, dim3(nb), dim3(SCAN_THREADS), 0, stream, n, in, sums, out);
+    hipLaunchKernelGGL(scan_apply_kernel<true>, dim3(nb), dim3(SCAN_THREADS), 0, stream, n, in, sums, out, total_out);
   else
-    hipLaunchKernelGGL(scan_apply_kernel<false>, dim3(nb), dim3(SCAN_THREADS), 0, stream, n, in, sums, out);
+    hipLaunchKernelGGL(scan_apply_kernel<false>, dim3(nb), dim3(SCAN_THREADS), 0, stream, n, in, sums, out, total_out);
   return 0;
 }
 
 // in and out may alias.
-int launch_inclusive_sum(int64_t n, const uint32_t* in, uint32_t* out, void* temp, hipStream_t stream) {
-  return scan_impl(n, in, out, temp, false, stream);
+int launch_inclusive_sum(int64_t n, const uint32_t* in, uint32_t* out, void* temp, hipStream_t stream,
+                         uint32_t* total_out) {
+  return scan_impl(n, in, out, temp, false, total_out, stream);
 }
 
 int launch_exclusive_sum(int64_t n, const uint32_t* in, uint32_t* out, void* temp, hipStream_t stream) {
-  return scan_impl(n, in, out, temp, true, stream);
+  return scan_impl(n, in, out, temp, true, nullptr, stream);
 }
 
 int launch_duplicate_with_keys(int P, int W, int H, const float* means2D, const float* depths,

@@ -48,7 +48,9 @@ int launch_mark_visible(int P, const float* means, const float* V, uint8_t* pres
 int launch_tile_count(int P, int W, int H, const int* radii, const float* means2D, const uint8_t* compute_locally,
                       uint32_t* tiles_touched, hipStream_t stream);
 size_t scan_temp_bytes(int64_t n);
-int launch_inclusive_sum(int64_t n, const uint32_t* in, uint32_t* out, void* temp, hipStream_t stream);
+// total_out, when given, is a host-visible word that receives the grand total as well
+int launch_inclusive_sum(int64_t n, const uint32_t* in, uint32_t* out, void* temp, hipStream_t stream,
+                         uint32_t* total_out = nullptr);
 int launch_exclusive_sum(int64_t n, const uint32_t* in, uint32_t* out, void* temp, hipStream_t stream);
 int launch_duplicate_with_keys(int P, int W, int H, const float* means2D, const float* depths,
                                const uint32_t* offsets, const int* radii, const uint8_t* compute_locally,

@@ -162,6 +162,48 @@ __device__ __forceinline__ float sh_channel(int deg, float x, float y, float z, 
   return res + 0.5f;
 }
 
+// 192-byte rows (16 SH coefficients x 3 channels) of the 64 Gaussians of a wave, moved between global memory
+// and LDS with whole-wave 16-byte accesses over the wave's contiguous 12 KB, so every fetched line is used
+// completely; a lane then reads or writes its own row in LDS.  Rows are padded to 13 x 16 bytes, which keeps
+// both access patterns free of bank conflicts.
+constexpr int SH_ROW4 = 13;
+constexpr int SH_WAVE_ROWS4 = GS_WAVE * SH_ROW4;
+
+__device__ __forceinline__ void wave_sync_lds() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// rows whose bit in `need` is clear are not fetched (their LDS rows read as zero)
+__device__ __forceinline__ void wave_rows_load(const float4* __restrict__ g4, uint64_t need, float4* lds, int lane) {
+  float4 v[12];
+#pragma unroll
+  for (int j = 0; j < 12; j++) {
+    const int idx = j * GS_WAVE + lane;
+    const int row = idx / 12;
+    v[j] = ((need >> row) & 1ull) ? g4[idx] : make_float4(0.f, 0.f, 0.f, 0.f);
+  }
+#pragma unroll
+  for (int j = 0; j < 12; j++) {
+    const int idx = j * GS_WAVE + lane;
+    const int row = idx / 12;
+    lds[row * SH_ROW4 + (idx - row * 12)] = v[j];
+  }
+  wave_sync_lds();
+}
+
+// stores the first `rows` rows
+__device__ __forceinline__ void wave_rows_store(float4* __restrict__ g4, int rows, const float4* lds, int lane) {
+  wave_sync_lds();
+#pragma unroll
+  for (int j = 0; j < 12; j++) {
+    const int idx = j * GS_WAVE + lane;
+    const int row = idx / 12;
+    if (row < rows) g4[idx] = lds[row * SH_ROW4 + (idx - row * 12)];
+  }
+}
+
 __global__ void __launch_bounds__(GS_BLOCK_1D)
 preprocess_fwd_kernel(int P, int D, int M, const float* __restrict__ means, const float* __restrict__ scales,
                       float mod, const float* __restrict__ rots, const float* __restrict__ opac,
@@ -199,6 +241,7 @@ preprocess_fwd_kernel(int P, int D, int M, const float* __restrict__ means, cons
     float c[3][16];
     const float* sh = shs + (size_t)i * M * 3;
     if (M == 16) {
+      // direct 16-byte loads: staging the rows through LDS costs this kernel more occupancy than it saves
       const float4* sh4 = reinterpret_cast<const float4*>(sh);
       float flat[48];
 #pragma unroll
@@ -295,14 +338,25 @@ preprocess_bwd_kernel(int P, int D, int M, const float* __restrict__ means, cons
                       const float4* __restrict__ dL_dconic_opacity, const float* __restrict__ dL_dcolor,
                       float* __restrict__ dL_dmean3D, float* __restrict__ dL_dcov3D_out, float* __restrict__ dL_dsh,
                       float* __restrict__ dL_dscale, float* __restrict__ dL_drot, float* __restrict__ dL_dopacity) {
-  const int i = blockIdx.x * GS_BLOCK_1D + threadIdx.x;
-  if (i >= P) return;
+  __shared__ float4 s_rows[GS_BLOCK_1D / GS_WAVE][SH_WAVE_ROWS4];
+  const int lane = threadIdx.x & (GS_WAVE - 1), wave = threadIdx.x / GS_WAVE;
+  const int raw_i = blockIdx.x * GS_BLOCK_1D + threadIdx.x;
+  const bool in_range = raw_i < P;
+  const int i = in_range ? raw_i : P - 1;  // lanes past the end shadow the last Gaussian and store nothing
   const bool sh_mode = (shs != nullptr) && M > 0 && (dL_dsh != nullptr);
+  const bool sh_staged = sh_mode && M == 16;  // coefficient rows and their gradients go through LDS
   const float4 gco = dL_dconic_opacity[i];
-  if (dL_dopacity) dL_dopacity[i] = gco.w;  // passthrough, rasterize_points.cu:191-194
+  if (dL_dopacity && in_range) dL_dopacity[i] = gco.w;  // passthrough, rasterize_points.cu:191-194
   float gm[3] = {0.f, 0.f, 0.f}, gs_[3] = {0.f, 0.f, 0.f}, gq[4] = {0.f, 0.f, 0.f, 0.f};
   float gc[6] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-  const bool live = radii[i] > 0;
+  const bool live = in_range && radii[i] > 0;
+  const size_t wave_first = (size_t)blockIdx.x * GS_BLOCK_1D + (size_t)wave * GS_WAVE;
+  float4* my_row = s_rows[wave] + lane * SH_ROW4;
+  if (sh_staged) {
+    const uint64_t need = __ballot(live);
+    if (need != 0ull)
+      wave_rows_load(reinterpret_cast<const float4*>(shs) + wave_first * 12, need, s_rows[wave], lane);
+  }
   if (live) {
     CamParams cam;
     load_cam(Vg, PMg, camg, cam);
@@ -379,6 +433,21 @@ preprocess_bwd_kernel(int P, int D, int M, const float* __restrict__ means, cons
     if (sh_mode) {
       const float* sh = shs + (size_t)i * M * 3;
       float* gsh = dL_dsh + (size_t)i * M * 3;
+      // the Gaussian's coefficients, in registers; 16-coefficient rows (192 bytes) move as twelve 16-byte words
+      float shv[48];
+      if (M == 16) {
+#pragma unroll
+        for (int j = 0; j < 12; j++) {
+          const float4 v = my_row[j];
+          shv[4 * j] = v.x;
+          shv[4 * j + 1] = v.y;
+          shv[4 * j + 2] = v.z;
+          shv[4 * j + 3] = v.w;
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < 48; e++) shv[e] = e < 3 * M ? sh[e] : 0.f;
+      }
       const float d0[3] = {mean[0] - cam.campos[0], mean[1] - cam.campos[1], mean[2] - cam.campos[2]};
       const float s2 = dot3(d0, d0);
       const float len = sqrtf(s2);
@@ -390,7 +459,7 @@ preprocess_bwd_kernel(int P, int D, int M, const float* __restrict__ means, cons
 #pragma unroll
       for (int k = 0; k < 16; k++) basis[k] = 0.f;
       float dRdx[3] = {0.f, 0.f, 0.f}, dRdy[3] = {0.f, 0.f, 0.f}, dRdz[3] = {0.f, 0.f, 0.f};
-#define SHV(k, ch) sh[3 * (k) + (ch)]
+#define SHV(k, ch) shv[3 * (k) + (ch)]
       basis[0] = kC0;
       if (D > 0) {
         basis[1] = -kC1 * y;
@@ -443,11 +512,18 @@ preprocess_bwd_kernel(int P, int D, int M, const float* __restrict__ means, cons
         }
       }
 #undef SHV
-      for (int k = 0; k < M; k++) {
-        const float bk = k < 16 ? basis[k] : 0.f;
-        gsh[3 * k] = bk * gr[0];
-        gsh[3 * k + 1] = bk * gr[1];
-        gsh[3 * k + 2] = bk * gr[2];
+      if (M == 16) {
+#pragma unroll
+        for (int j = 0; j < 12; j++)
+          my_row[j] = make_float4(basis[(4 * j) / 3] * gr[(4 * j) % 3], basis[(4 * j + 1) / 3] * gr[(4 * j + 1) % 3],
+                                basis[(4 * j + 2) / 3] * gr[(4 * j + 2) % 3], basis[(4 * j + 3) / 3] * gr[(4 * j + 3) % 3]);
+      } else {
+        for (int k = 0; k < M; k++) {
+          const float bk = k < 16 ? basis[k] : 0.f;
+          gsh[3 * k] = bk * gr[0];
+          gsh[3 * k + 1] = bk * gr[1];
+          gsh[3 * k + 2] = bk * gr[2];
+        }
       }
       const float gdir[3] = {dot3(dRdx, gr), dot3(dRdy, gr), dot3(dRdz, gr)};
       const float inv32 = 1.0f / sqrtf(s2 * s2 * s2);
@@ -496,10 +572,22 @@ preprocess_bwd_kernel(int P, int D, int M, const float* __restrict__ means, cons
                2 * y * (dMt.m[1][2] + dMt.m[2][1])) -
               4 * z * (dMt.m[1][1] + dMt.m[0][0]);
     }
-  } else if (sh_mode) {
+  } else if (sh_mode && in_range) {
     float* gsh = dL_dsh + (size_t)i * M * 3;
-    for (int k = 0; k < 3 * M; k++) gsh[k] = 0.f;
+    if (M == 16) {
+#pragma unroll
+      for (int j = 0; j < 12; j++) my_row[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+    } else {
+      for (int k = 0; k < 3 * M; k++) gsh[k] = 0.f;
+    }
   }
+  if (sh_staged) {
+    const long long left = (long long)P - (long long)wave_first;
+    if (left > 0)
+      wave_rows_store(reinterpret_cast<float4*>(dL_dsh) + wave_first * 12, left < GS_WAVE ? (int)left : GS_WAVE,
+                      s_rows[wave], lane);
+  }
+  if (!in_range) return;
   dL_dmean3D[3 * (size_t)i] = gm[0];
   dL_dmean3D[3 * (size_t)i + 1] = gm[1];
   dL_dmean3D[3 * (size_t)i + 2] = gm[2];

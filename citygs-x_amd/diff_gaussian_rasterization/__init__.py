@@ -52,12 +52,21 @@ class _PreprocessGaussians(torch.autograd.Function):
         ctx.num_rendered = num_rendered
         ctx.save_for_backward(means3D, scales, rotations, sh, radii, cov3D, clamped)
         ctx.mark_non_differentiable(radii, depths)
+        # no zero tensors for the outputs nobody differentiates (radii, depths): backward fills in what it needs
+        ctx.set_materialize_grads(False)
         return means2D, rgb, conic_opacity, radii, depths
 
     @staticmethod
     def backward(ctx, grad_means2D, grad_rgb, grad_conic_opacity, grad_radii, grad_depths):
         rs = ctx.raster_settings
         means3D, scales, rotations, sh, radii, cov3D, clamped = ctx.saved_tensors
+        P = means3D.shape[0]
+        if grad_means2D is None:
+            grad_means2D = means3D.new_zeros(P, 2)
+        if grad_rgb is None:
+            grad_rgb = means3D.new_zeros(P, 3)
+        if grad_conic_opacity is None:
+            grad_conic_opacity = means3D.new_zeros(P, 4)
         dL_dmeans3D, dL_dscales, dL_drotations, dL_dsh, dL_dopacity = _C.preprocess_gaussians_backward(
             radii, cov3D, clamped, means3D, scales, rotations, sh, rs.scale_modifier, rs.viewmatrix, rs.projmatrix,
             rs.tanfovx, rs.tanfovy, rs.image_height, rs.image_width, rs.sh_degree, rs.campos, grad_means2D,
@@ -90,6 +99,7 @@ class _RenderGaussians(torch.autograd.Function):
         ctx.save_for_backward(means2D, conic_opacity, rgb, all_maps, out_all_map, geomBuffer, binningBuffer, imgBuffer,
                               compute_locally)
         ctx.mark_non_differentiable(n_render, n_consider, n_contrib, out_observe)
+        ctx.set_materialize_grads(False)  # the four integer outputs never get a zero "gradient" allocated
         return color, n_render, n_consider, n_contrib, out_observe, out_all_map, out_plane_depth
 
     @staticmethod
