@@ -7,7 +7,7 @@
 // and each of its 16-lane rows a 4x4 pixel block.  Per batch of 256 Gaussians
 // (staged in LDS in back-to-front order):
 //   * a wave ballots, for each of its rows, which Gaussians can touch the
-//     row's block (conservative box test) and lie in front of the row's
+//     row's block (inflated alpha >= 1/255 ellipse against the block) and lie in front of the row's
 //     deepest contributor; the four rows then walk their own bit lists
 //     concurrently, so one pass of the loop handles up to four Gaussians;
 //   * the 16 partial sums of a Gaussian (mean2D x/y, |mean2D| x/y, conic
@@ -51,7 +51,7 @@ render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
   __shared__ uint32_t s_emis[BATCH];
   __shared__ float2 s_xy[BATCH];
   __shared__ float4 s_co[BATCH];
-  __shared__ float4 s_bb[BATCH];
+  __shared__ float4 s_cp[BATCH];
   __shared__ float s_floor[BATCH];
   __shared__ float s_rgb[GS_N_RGB][BATCH];
   __shared__ float s_map[GS_N_MAP][BATCH];
@@ -151,7 +151,7 @@ render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
       s_xy[tid] = xy;
       s_co[tid] = co;
       float pfl;
-      s_bb[tid] = cull_box(xy, co, pfl);
+      s_cp[tid] = cull_params(co, pfl);
       s_floor[tid] = pfl;
       s_rgb[0][tid] = rgb[3 * (size_t)g];
       s_rgb[1][tid] = rgb[3 * (size_t)g + 1];
@@ -170,10 +170,13 @@ render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
     for (int k = 0; k < BATCH / GS_WAVE; k++) {
       const int jj = k * GS_WAVE + lane;
       const bool valid = jj < count;
-      const float4 bb = s_bb[valid ? jj : 0];
+      const float2 mu = s_xy[valid ? jj : 0];
+      const float4 cq = s_co[valid ? jj : 0];
+      const float4 cp = s_cp[valid ? jj : 0];
 #pragma unroll
       for (int r = 0; r < 4; r++) {
-        const uint64_t hit = __ballot(valid && (first_pos - jj) < row_last_of[r] && box_hits_row(bb, rt.qx0, rt.qy0, r));
+        const uint64_t hit = __ballot(valid && (first_pos - jj) < row_last_of[r] &&
+                                      ellipse_hits_row(mu, cq, cp, rt.qx0, rt.qy0, r));
         if (lane == 0) {
           s_list[wave][r][2 * k] = (uint32_t)hit;
           s_list[wave][r][2 * k + 1] = (uint32_t)(hit >> 32);

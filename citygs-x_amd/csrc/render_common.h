@@ -67,6 +67,44 @@ __device__ __forceinline__ float4 cull_box(float2 xy, float4 co, float& power_fl
   return bb;
 }
 
+// The same region, tested exactly against a block of pixels instead of through its bounding box.
+// cull_params returns (1/A, 1/C, q_max, 0): alpha >= 1/255 needs q(d) = A dx^2 + 2B dx dy + C dy^2 <= q_max
+// = 2 (tau + 0.01).  q_max is +infinity when the conic cannot be trusted (every block then counts as hit)
+// and negative when the opacity alone rules every pixel out.  power_floor as for cull_box.
+__device__ __forceinline__ float4 cull_params(float4 co, float& power_floor) {
+  const float inf = __builtin_inff();
+  const float o = co.w;
+  power_floor = -87.0f;
+  if (o < 0.0039f) return make_float4(0.f, 0.f, -1.0f, 0.f);
+  float4 cp = make_float4(0.f, 0.f, inf, 0.f);
+  if (o < 1.0e30f) {
+    const float tau = __logf(255.0f * o) + 0.01f;
+    if (tau == tau) {
+      power_floor = fmaxf(-tau, -87.0f);
+      const float det = co.x * co.z - co.y * co.y;
+      const float ia = 1.0f / co.x, ic = 1.0f / co.z;
+      if (det > 0.0f && co.x > 0.0f && co.z > 0.0f && ia < inf && ic < inf) cp = make_float4(ia, ic, 2.0f * tau, 0.f);
+    }
+  }
+  return cp;
+}
+
+// Can any point of the pixel block [bx0, bx0+ext] x [by0, by0+ext] have q <= q_max?  q is convex, so over
+// the block it is smallest either at the centre (inside the block: 0) or on one of the two block edges that
+// face the centre; along an edge it is a parabola whose minimiser is clamped to the edge.  The block is
+// treated as a continuous rectangle, which can only add hits; the 0.01 added to tau covers the rounding
+// differences against the per-pixel evaluation.  NaNs count as hits.
+__device__ __forceinline__ bool ellipse_hits_block(float2 mu, float4 co, float4 cp, float bx0, float by0, float ext) {
+  const float lox = bx0 - mu.x, hix = lox + ext, loy = by0 - mu.y, hiy = loy + ext;
+  const float dxc = fminf(fmaxf(0.f, lox), hix);  // offset of the nearest column / row of the block
+  const float dyc = fminf(fmaxf(0.f, loy), hiy);
+  const float dy1 = fminf(fmaxf(-co.y * dxc * cp.y, loy), hiy);  // best point of the column x = dxc
+  const float q1 = (co.x * dxc * dxc + 2.0f * co.y * dxc * dy1) + co.z * dy1 * dy1;
+  const float dx2 = fminf(fmaxf(-co.y * dyc * cp.x, lox), hix);  // best point of the row y = dyc
+  const float q2 = (co.x * dx2 * dx2 + 2.0f * co.y * dx2 * dyc) + co.z * dyc * dyc;
+  return !(fminf(q1, q2) > cp.z);
+}
+
 __device__ __forceinline__ bool box_hits_wave(const float4 bb, const TileThread& t) {
   return !(bb.z < t.wx0 || bb.x > t.wx1 || bb.w < t.wy0 || bb.y > t.wy1);
 }
@@ -127,6 +165,11 @@ __device__ __forceinline__ RowThread row_thread(uint32_t tile_x, uint32_t tile_y
   t.qx0 = (float)x0;
   t.qy0 = (float)y0;
   return t;
+}
+
+// Ellipse against the 4x4 block of row r of the quadrant at (qx0, qy0).
+__device__ __forceinline__ bool ellipse_hits_row(float2 mu, float4 co, float4 cp, float qx0, float qy0, int r) {
+  return ellipse_hits_block(mu, co, cp, qx0 + (float)((r & 1) * 4), qy0 + (float)((r >> 1) * 4), 3.0f);
 }
 
 // Box against the 4x4 block of row r of the quadrant at (qx0, qy0).

@@ -5,10 +5,11 @@
 // One 256-thread workgroup per 16x16 tile; each 64-lane wave owns an 8x8
 // quadrant and each 16-lane row of a wave a 4x4 pixel block.  The tile's
 // depth-sorted Gaussians are staged through LDS in batches of 256 (index,
-// centre, conic+opacity, colour, the five geometry channels, a conservative
-// screen-space box and the exponent below which alpha < 1/255 is certain).
-// Per batch a wave ballots, for each of its four rows, which Gaussians' boxes
-// meet the row's 4x4 block and leaves those bit lists in LDS; the four rows
+// centre, conic+opacity, colour, the five geometry channels, the culling
+// parameters and the exponent below which alpha < 1/255 is certain).
+// Per batch a wave ballots, for each of its four rows, which Gaussians'
+// alpha >= 1/255 ellipses (slightly inflated) can reach the row's 4x4 block
+// and leaves those bit lists in LDS; the four rows
 // then walk their own lists concurrently (find-first-set on a per-row mask),
 // so one pass of the loop blends up to four different Gaussians and a
 // Gaussian that cannot touch a block costs that row nothing.  Pixels keep
@@ -43,7 +44,7 @@ render_fwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
   __shared__ int s_id[BATCH];
   __shared__ float2 s_xy[BATCH];
   __shared__ float4 s_co[BATCH];
-  __shared__ float4 s_bb[BATCH];
+  __shared__ float4 s_cp[BATCH];
   __shared__ float s_floor[BATCH];
   __shared__ float s_rgb[GS_N_RGB][BATCH];
   __shared__ float s_map[GS_N_MAP][BATCH];
@@ -96,7 +97,7 @@ render_fwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
       s_id[tid] = (int)g;
       s_xy[tid] = xy;
       s_co[tid] = co;
-      s_bb[tid] = cull_box(xy, co, pfl);
+      s_cp[tid] = cull_params(co, pfl);
       s_floor[tid] = pfl;
       s_rgb[0][tid] = rgb[3 * (size_t)g];
       s_rgb[1][tid] = rgb[3 * (size_t)g + 1];
@@ -115,11 +116,13 @@ render_fwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
       for (int k = 0; k < BATCH / GS_WAVE; k++) {
         const int jj = k * GS_WAVE + lane;
         const bool valid = jj < count;
-        const float4 bb = s_bb[valid ? jj : 0];
+        const float2 mu = s_xy[valid ? jj : 0];
+        const float4 cq = s_co[valid ? jj : 0];
+        const float4 cp = s_cp[valid ? jj : 0];
 #pragma unroll
         for (int r = 0; r < 4; r++) {
           const bool row_alive = ((alive_mask >> (16 * r)) & 0xFFFFull) != 0ull;
-          const uint64_t b = __ballot(valid && row_alive && box_hits_row(bb, rt.qx0, rt.qy0, r));
+          const uint64_t b = __ballot(valid && row_alive && ellipse_hits_row(mu, cq, cp, rt.qx0, rt.qy0, r));
           if (lane == 0) {
             s_list[wave][r][2 * k] = (uint32_t)b;
             s_list[wave][r][2 * k + 1] = (uint32_t)(b >> 32);
