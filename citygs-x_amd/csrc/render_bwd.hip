@@ -38,6 +38,7 @@ constexpr int BATCH = GS_TILE_PIX;
 constexpr int NV = 16;
 constexpr int CHUNKS = BATCH / 32;
 
+template <bool RENDER_GEO>
 __global__ void __launch_bounds__(GS_TILE_PIX)
 render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__ point_list, int W, int H, float fx,
                   float fy, const float* __restrict__ bg, const float2* __restrict__ means2D,
@@ -46,8 +47,8 @@ render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
                   const float* __restrict__ final_Ts, const uint32_t* __restrict__ n_contrib_px,
                   const uint8_t* __restrict__ compute_locally, const float* __restrict__ dL_dpix,
                   const float* __restrict__ dL_dout_all_map, const float* __restrict__ dL_dout_plane_depth,
-                  int render_geo, const uint32_t* __restrict__ emission_sorted,
-                  float4* __restrict__ instance_grads) {
+                  const uint32_t* __restrict__ emission_sorted, float4* __restrict__ instance_grads) {
+  constexpr bool render_geo = RENDER_GEO;
   __shared__ uint32_t s_emis[BATCH];
   __shared__ float2 s_xy[BATCH];
   __shared__ float4 s_co[BATCH];
@@ -200,79 +201,78 @@ render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
         const int j = has ? kk * 32 + (int)__builtin_ctz(m) : 0;
         m &= m - 1u;
         const int pos = first_pos - j;
-        // Same tests as the forward pass, on the same bits: exponent first, exponential only where
-        // alpha >= 1/255 is still possible.
-        bool in = false;
-        float dx = 0.f, dy = 0.f, power = 0.f;
-        float4 co = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (has && pos < last_contributor) {  // never true for pixels outside the image (last_contributor = 0)
-          const float2 xy = s_xy[j];
-          dx = xy.x - pfx;
-          dy = xy.y - pfy;
-          co = s_co[j];
-          power = -0.5f * (co.x * dx * dx + co.z * dy * dy) - co.y * dx * dy;
-          in = !(power > 0.0f) && !(power < s_floor[j]);
-        }
+        // Straight-line from here on: every lane evaluates its row's Gaussian, and a lane for which the
+        // Gaussian does not count (behind the pixel's last contributor, outside the power window, alpha
+        // below 1/255) takes part with alpha = 0, G = 0.  Such a step leaves T unchanged (T * 1/(1-0)),
+        // contributes zeros to every sum, and only rotates the recurrence state in a way the next real
+        // step undoes exactly (fma(0, c, 1 * accum) == accum), so results are those of skipping it.
+        // Same tests as the forward pass, on the same bits.
+        const float2 xy = s_xy[j];
+        const float4 co = s_co[j];
+        const float dx = xy.x - pfx, dy = xy.y - pfy;
+        const float power = -0.5f * (co.x * dx * dx + co.z * dy * dy) - co.y * dx * dy;
+        // never true for pixels outside the image (last_contributor = 0)
+        const float floor_j = s_floor[j];
+        // (bitwise on purpose: no short-circuit branches in the loop)
+        const bool in = has & (pos < last_contributor) & !(power > 0.0f) & !(power < floor_j);
         if (__ballot(in) == 0ull) continue;  // wave-uniform
-        bool active = false;
-        float G = 0.f, alpha = 0.f;
-        if (in) {
-          G = gs_expf_core(power);
-          alpha = fminf(0.99f, co.w * G);
-          active = !(alpha < 1.0f / 255.0f);
-        }
+        const float G_raw = gs_expf_core(power);
+        const float alpha_raw = fminf(0.99f, co.w * G_raw);
+        const bool active = in & !(alpha_raw < 1.0f / 255.0f);
         if (__ballot(active) == 0ull) continue;  // wave-uniform
+        const float alpha = active ? alpha_raw : 0.f;
+        const float G = active ? G_raw : 0.f;
 
         float v[NV];
+        // Up to dL/dalpha the operation sequence is exactly the CPU statement's (IEEE reciprocal, explicit
+        // FMAs): upstream gradients of the geometry channels can be many orders of magnitude larger than
+        // the result (plane depth divides by a blended normal that may be nearly perpendicular to the
+        // ray), so these operations decide how far a gradient can drift.  What follows dL/dalpha is
+        // products only.
+        const float rcp1ma = 1.f / (1.f - alpha);
+        T = T * rcp1ma;
+        const float w = alpha * T;
+        const float oml = 1.f - last_alpha;
+        float dL_dalpha = 0.0f;
 #pragma unroll
-        for (int q = 0; q < NV; q++) v[q] = 0.f;
-        if (active) {
-          // Up to dL/dalpha the operation sequence is exactly the CPU statement's (IEEE reciprocal, explicit
-          // FMAs): upstream gradients of the geometry channels can be many orders of magnitude larger than
-          // the result (plane depth divides by a blended normal that may be nearly perpendicular to the
-          // ray), so these operations decide how far a gradient can drift.  What follows dL/dalpha is
-          // products only.
-          const float rcp1ma = 1.f / (1.f - alpha);
-          T = T * rcp1ma;
-          const float w = alpha * T;
-          const float oml = 1.f - last_alpha;
-          float dL_dalpha = 0.0f;
-#pragma unroll
-          for (int ch = 0; ch < GS_N_RGB; ch++) {
-            const float c = s_rgb[ch][j];
-            accum_rec[ch] = __builtin_fmaf(last_alpha, last_color[ch], oml * accum_rec[ch]);
-            last_color[ch] = c;
-            dL_dalpha = __builtin_fmaf(c - accum_rec[ch], gpix[ch], dL_dalpha);
-            v[8 + ch] = w * gpix[ch];
-          }
-          if (render_geo) {
-#pragma unroll
-            for (int ch = 0; ch < GS_N_MAP; ch++) {
-              const float c = s_map[ch][j];
-              accum_map[ch] = __builtin_fmaf(last_alpha, last_map[ch], oml * accum_map[ch]);
-              last_map[ch] = c;
-              dL_dalpha = __builtin_fmaf(c - accum_map[ch], gmap[ch], dL_dalpha);
-              v[11 + ch] = w * gmap[ch];
-            }
-          }
-          last_alpha = alpha;
-          dL_dalpha = __builtin_fmaf(dL_dalpha, T, -(bg_term * rcp1ma));
-          const float dL_dG = co.w * dL_dalpha;
-          const float gdx = G * dx, gdy = G * dy;
-          const float dG_ddelx = -gdx * co.x - gdy * co.y;
-          const float dG_ddely = -gdy * co.z - gdx * co.y;
-          v[0] = dL_dG * dG_ddelx * ddelx_dx;
-          v[1] = dL_dG * dG_ddely * ddely_dy;
-          v[2] = fabsf(v[0]);
-          v[3] = fabsf(v[1]);
-          const float hg = -0.5f * dL_dG;
-          v[4] = hg * gdx * dx;
-          v[5] = hg * gdx * dy;
-          v[6] = hg * gdy * dy;
-          v[7] = G * dL_dalpha;
+        for (int ch = 0; ch < GS_N_RGB; ch++) {
+          const float c = s_rgb[ch][j];
+          accum_rec[ch] = __builtin_fmaf(last_alpha, last_color[ch], oml * accum_rec[ch]);
+          last_color[ch] = c;
+          dL_dalpha = __builtin_fmaf(c - accum_rec[ch], gpix[ch], dL_dalpha);
+          v[8 + ch] = w * gpix[ch];
         }
+        if (render_geo) {
+#pragma unroll
+          for (int ch = 0; ch < GS_N_MAP; ch++) {
+            const float c = s_map[ch][j];
+            accum_map[ch] = __builtin_fmaf(last_alpha, last_map[ch], oml * accum_map[ch]);
+            last_map[ch] = c;
+            dL_dalpha = __builtin_fmaf(c - accum_map[ch], gmap[ch], dL_dalpha);
+            v[11 + ch] = w * gmap[ch];
+          }
+        } else {
+#pragma unroll
+          for (int ch = 0; ch < GS_N_MAP; ch++) v[11 + ch] = 0.f;
+        }
+        last_alpha = alpha;
+        dL_dalpha = __builtin_fmaf(dL_dalpha, T, -(bg_term * rcp1ma));
+        dL_dalpha = active ? dL_dalpha : 0.f;
+        const float dL_dG = co.w * dL_dalpha;
+        const float gdx = G * dx, gdy = G * dy;
+        const float dG_ddelx = -gdx * co.x - gdy * co.y;
+        const float dG_ddely = -gdy * co.z - gdx * co.y;
+        v[0] = dL_dG * dG_ddelx * ddelx_dx;
+        v[1] = dL_dG * dG_ddely * ddely_dy;
+        v[2] = fabsf(v[0]);
+        v[3] = fabsf(v[1]);
+        const float hg = -0.5f * dL_dG;
+        v[4] = hg * gdx * dx;
+        v[5] = hg * gdx * dy;
+        v[6] = hg * gdy * dy;
+        v[7] = G * dL_dalpha;
         // lane q of the row now receives the row's total of component q
-        const float tot = row_transpose_reduce16(v, l16);
+        const float tot = row_transpose_reduce16(v);
         if (has && tot != 0.f) unsafeAtomicAdd(&s_acc[l16][j], tot);
       }
     }
@@ -329,10 +329,18 @@ reduce_instances_kernel(int P, const uint32_t* __restrict__ point_offsets, const
 
 int launch_render_bwd(const RenderBwdArgs& a, hipStream_t stream) {
   const dim3 grid((a.W + GS_TILE_X - 1) / GS_TILE_X, (a.H + GS_TILE_Y - 1) / GS_TILE_Y, 1);
-  hipLaunchKernelGGL(render_bwd_kernel, grid, dim3(GS_TILE_PIX), 0, stream, (const uint2*)a.ranges, a.point_list, a.W,
-                     a.H, a.fx, a.fy, a.bg, (const float2*)a.means2D, (const float4*)a.conic_opacity, a.rgb, a.all_map,
-                     a.all_map_pixels, a.final_T, a.n_contrib_px, a.compute_locally, a.dL_dpix, a.dL_dout_all_map,
-                     a.dL_dout_plane_depth, a.render_geo, a.emission_sorted, (float4*)a.instance_grads);
+  if (a.render_geo)
+    hipLaunchKernelGGL(render_bwd_kernel<true>, grid, dim3(GS_TILE_PIX), 0, stream, (const uint2*)a.ranges,
+                       a.point_list, a.W, a.H, a.fx, a.fy, a.bg, (const float2*)a.means2D,
+                       (const float4*)a.conic_opacity, a.rgb, a.all_map, a.all_map_pixels, a.final_T, a.n_contrib_px,
+                       a.compute_locally, a.dL_dpix, a.dL_dout_all_map, a.dL_dout_plane_depth, a.emission_sorted,
+                       (float4*)a.instance_grads);
+  else
+    hipLaunchKernelGGL(render_bwd_kernel<false>, grid, dim3(GS_TILE_PIX), 0, stream, (const uint2*)a.ranges,
+                       a.point_list, a.W, a.H, a.fx, a.fy, a.bg, (const float2*)a.means2D,
+                       (const float4*)a.conic_opacity, a.rgb, a.all_map, a.all_map_pixels, a.final_T, a.n_contrib_px,
+                       a.compute_locally, a.dL_dpix, a.dL_dout_all_map, a.dL_dout_plane_depth, a.emission_sorted,
+                       (float4*)a.instance_grads);
   hipLaunchKernelGGL(reduce_instances_kernel, dim3((a.P + GS_BLOCK_1D - 1) / GS_BLOCK_1D), dim3(GS_BLOCK_1D), 0,
                      stream, a.P, a.point_offsets, (const float4*)a.instance_grads, a.render_geo,
                      (float2*)a.dL_dmean2D, a.dL_dmean2D_abs, (float4*)a.dL_dconic_opacity, a.dL_dcolors,

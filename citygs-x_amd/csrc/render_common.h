@@ -187,34 +187,64 @@ __device__ __forceinline__ float dpp_merge(float old, float src) {
 // Transposing reduction inside every 16-lane row: on entry each lane holds 16
 // values, on return lane l16 of a row holds the sum over the row's 16 lanes of
 // value number l16.  Four halving steps (distances 8, 4, 2, 1): at each step a
-// lane keeps half of its values and receives the partner lane's copy of them,
-// so 8 + 4 + 2 + 1 additions replace 16 x 4.
-__device__ __forceinline__ float row_transpose_reduce16(const float* v, int l16) {
-  float a[8], b[4], c[2];
-#pragma unroll
-  for (int i = 0; i < 8; i++) {
-    // lanes 0-7 keep value i and fetch it from lane +8; lanes 8-15 keep value i+8 and fetch it from lane -8
-    const float x = dpp_merge<0x128 /*row_ror:8*/, 0x3>(v[i + 8], v[i]);
-    const float y = dpp_merge<0x128 /*row_ror:8*/, 0xC>(v[i], v[i + 8]);
-    a[i] = x + y;
-  }
-#pragma unroll
-  for (int i = 0; i < 4; i++) {
-    // lanes with bit 2 clear (banks 0, 2) keep value i, fetched from lane +4; the others keep i+4, from lane -4
-    const float x = dpp_merge<0x104 /*row_shl:4*/, 0x5>(a[i + 4], a[i]);
-    const float y = dpp_merge<0x114 /*row_shr:4*/, 0xA>(a[i], a[i + 4]);
-    b[i] = x + y;
-  }
-  const bool bit1 = (l16 & 2) != 0, bit0 = (l16 & 1) != 0;
-#pragma unroll
-  for (int i = 0; i < 2; i++) {
-    const float lo = dpp_row_add<0x4E>(b[i]);      // quad_perm [2,3,0,1]: + lane^2
-    const float hi = dpp_row_add<0x4E>(b[i + 2]);
-    c[i] = bit1 ? hi : lo;
-  }
-  const float lo = dpp_row_add<0xB1>(c[0]);  // quad_perm [1,0,3,2]: + lane^1
-  const float hi = dpp_row_add<0xB1>(c[1]);
-  return bit0 ? hi : lo;
+// lane keeps half of its values and adds the partner lane's copy of them, so
+// 8 + 4 + 2 + 1 lane-pair sums replace 16 x 4.  Written as DPP additions whose
+// bank mask selects which lanes of a row take the result, two instructions per
+// kept value in the first two steps (33 VALU instructions in all); v[0..7] are
+// overwritten.  All 64 lanes must be active.
+__device__ __forceinline__ float row_transpose_reduce16(float* v) {
+  const uint64_t bit1_lanes = 0xCCCCCCCCCCCCCCCCull, bit0_lanes = 0xAAAAAAAAAAAAAAAAull;
+  // A DPP operand written by the preceding VALU instruction needs two idle issue slots first; the s_nop 1
+  // between the steps provide them, inside a step no instruction reads a register written less than two
+  // instructions earlier through DPP.
+  asm volatile(
+      "s_nop 1\n\t"
+      // distance 8: lanes 0-7 of a row keep values 0-7, lanes 8-15 keep values 8-15
+      "v_add_f32_dpp %0, %0, %0 row_ror:8 row_mask:0xf bank_mask:0xf\n\t"
+      "v_add_f32_dpp %1, %1, %1 row_ror:8 row_mask:0xf bank_mask:0xf\n\t"
+      "v_add_f32_dpp %2, %2, %2 row_ror:8 row_mask:0xf bank_mask:0xf\n\t"
+      "v_add_f32_dpp %3, %3, %3 row_ror:8 row_mask:0xf bank_mask:0xf\n\t"
+      "v_add_f32_dpp %4, %4, %4 row_ror:8 row_mask:0xf bank_mask:0xf\n\t"
+      "v_add_f32_dpp %5, %5, %5 row_ror:8 row_mask:0xf bank_mask:0xf\n\t"
+      "v_add_f32_dpp %6, %6, %6 row_ror:8 row_mask:0xf bank_mask:0xf\n\t"
+      "v_add_f32_dpp %7, %7, %7 row_ror:8 row_mask:0xf bank_mask:0xf\n\t"
+      "v_add_f32_dpp %0, %8, %8 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+      "v_add_f32_dpp %1, %9, %9 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+      "v_add_f32_dpp %2, %10, %10 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+      "v_add_f32_dpp %3, %11, %11 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+      "v_add_f32_dpp %4, %12, %12 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+      "v_add_f32_dpp %5, %13, %13 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+      "v_add_f32_dpp %6, %14, %14 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+      "v_add_f32_dpp %7, %15, %15 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+      "s_nop 1\n\t"
+      // distance 4: lanes with bit 2 clear (banks 0, 2) keep registers 0-3 and add lane +4's copy,
+      // the others keep registers 4-7 and add lane -4's copy
+      "v_add_f32_dpp %0, %0, %0 row_shl:4 row_mask:0xf bank_mask:0x5\n\t"
+      "v_add_f32_dpp %1, %1, %1 row_shl:4 row_mask:0xf bank_mask:0x5\n\t"
+      "v_add_f32_dpp %2, %2, %2 row_shl:4 row_mask:0xf bank_mask:0x5\n\t"
+      "v_add_f32_dpp %3, %3, %3 row_shl:4 row_mask:0xf bank_mask:0x5\n\t"
+      "v_add_f32_dpp %0, %4, %4 row_shr:4 row_mask:0xf bank_mask:0xa\n\t"
+      "v_add_f32_dpp %1, %5, %5 row_shr:4 row_mask:0xf bank_mask:0xa\n\t"
+      "v_add_f32_dpp %2, %6, %6 row_shr:4 row_mask:0xf bank_mask:0xa\n\t"
+      "v_add_f32_dpp %3, %7, %7 row_shr:4 row_mask:0xf bank_mask:0xa\n\t"
+      "s_nop 1\n\t"
+      // distance 2: + lane^2; lanes with bit 1 set keep registers 2, 3
+      "v_add_f32_dpp %0, %0, %0 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf\n\t"
+      "v_add_f32_dpp %1, %1, %1 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf\n\t"
+      "v_add_f32_dpp %2, %2, %2 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf\n\t"
+      "v_add_f32_dpp %3, %3, %3 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf\n\t"
+      "v_cndmask_b32_e64 %0, %0, %2, %16\n\t"
+      "v_cndmask_b32_e64 %1, %1, %3, %16\n\t"
+      "s_nop 1\n\t"
+      // distance 1: + lane^1; lanes with bit 0 set keep register 1
+      "v_add_f32_dpp %0, %0, %0 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf\n\t"
+      "v_add_f32_dpp %1, %1, %1 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf\n\t"
+      "s_nop 0\n\t"
+      "v_cndmask_b32_e64 %0, %0, %1, %17\n\t"
+      : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]), "+v"(v[4]), "+v"(v[5]), "+v"(v[6]), "+v"(v[7])
+      : "v"(v[8]), "v"(v[9]), "v"(v[10]), "v"(v[11]), "v"(v[12]), "v"(v[13]), "v"(v[14]), "v"(v[15]),
+        "s"(bit1_lanes), "s"(bit0_lanes));
+  return v[0];
 }
 
 }  // namespace gs

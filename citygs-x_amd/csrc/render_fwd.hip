@@ -31,16 +31,18 @@ namespace {
 constexpr int BATCH = GS_TILE_PIX;
 constexpr int CHUNKS = BATCH / 32;  // 32-bit list words per row and batch
 
+template <bool RENDER_GEO>
 __global__ void __launch_bounds__(GS_TILE_PIX)
 render_fwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__ point_list, int W, int H, float fx,
                   float fy, float cx, float cy, const float2* __restrict__ means2D, const float* __restrict__ rgb,
                   const float* __restrict__ all_map, const float4* __restrict__ conic_opacity,
-                  const uint8_t* __restrict__ compute_locally, const float* __restrict__ bg, int render_geo,
+                  const uint8_t* __restrict__ compute_locally, const float* __restrict__ bg,
                   float* __restrict__ final_T, uint32_t* __restrict__ n_contrib_px,
                   uint32_t* __restrict__ n_contrib2loss_px, float* __restrict__ out_color,
                   int* __restrict__ out_observe, float* __restrict__ out_all_map,
                   float* __restrict__ out_plane_depth, int* __restrict__ n_render, int* __restrict__ n_consider,
                   int* __restrict__ n_contrib_tile) {
+  constexpr bool render_geo = RENDER_GEO;
   __shared__ int s_id[BATCH];
   __shared__ float2 s_xy[BATCH];
   __shared__ float4 s_co[BATCH];
@@ -145,52 +147,39 @@ render_fwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
         const int j = has ? kk * 32 + (int)__builtin_ctz(m) : 0;
         m &= m - 1u;
 
-        // exponent first; the exponential only for lanes that can still pass the 1/255 test
-        float power = 0.f, o = 0.f;
-        bool in = false;
-        if (has && !done) {
-          const float2 xy = s_xy[j];
-          const float dx = xy.x - pfx, dy = xy.y - pfy;
-          const float4 co = s_co[j];
-          o = co.w;
-          power = -0.5f * (co.x * dx * dx + co.z * dy * dy) - co.y * dx * dy;
-          in = !(power > 0.0f) && !(power < s_floor[j]);
-        }
+        // Straight-line: every lane evaluates its row's Gaussian; a lane for which it does not count blends
+        // with weight 0, which leaves its sums unchanged bit for bit (fma(c, 0, C) == C).
+        const float2 xy = s_xy[j];
+        const float4 co = s_co[j];
+        const float dx = xy.x - pfx, dy = xy.y - pfy;
+        const float power = -0.5f * (co.x * dx * dx + co.z * dy * dy) - co.y * dx * dy;
+        const float floor_j = s_floor[j];
+        // (bitwise on purpose: no short-circuit branches in the loop)
+        const bool in = has & !done & !(power > 0.0f) & !(power < floor_j);
         if (__ballot(in) == 0ull) continue;
-        bool blend = false, stop = false;
-        float alpha = 0.f, test_T = 0.f;
-        if (in) {
-          alpha = fminf(0.99f, o * gs_expf_core(power));
-          if (!(alpha < 1.0f / 255.0f)) {
-            test_T = T * (1 - alpha);
-            if (test_T < 0.0001f)
-              stop = true;
-            else
-              blend = true;
-          }
-        }
+        const float alpha = fminf(0.99f, co.w * gs_expf_core(power));
+        const bool pass = in & !(alpha < 1.0f / 255.0f);
+        const float test_T = T * (1 - alpha);
+        const bool stop = pass & (test_T < 0.0001f);
+        const bool blend = pass & !stop;
         const uint64_t bmask = __ballot(blend);
         if (bmask != 0ull) {
-          if (blend) {
-            n2l++;
-            // weight once, then one fused multiply-add per channel
-            const float w = alpha * T;
+          if (blend) n2l++;
+          // weight once, then one fused multiply-add per channel
+          const float w = blend ? alpha * T : 0.f;
 #pragma unroll
-            for (int ch = 0; ch < GS_N_RGB; ch++) C[ch] = __builtin_fmaf(s_rgb[ch][j], w, C[ch]);
-            if (render_geo) {
+          for (int ch = 0; ch < GS_N_RGB; ch++) C[ch] = __builtin_fmaf(s_rgb[ch][j], w, C[ch]);
+          if (render_geo) {
 #pragma unroll
-              for (int ch = 0; ch < GS_N_MAP; ch++) Mp[ch] = __builtin_fmaf(s_map[ch][j], w, Mp[ch]);
-            }
+            for (int ch = 0; ch < GS_N_MAP; ch++) Mp[ch] = __builtin_fmaf(s_map[ch][j], w, Mp[ch]);
           }
           const uint64_t omask = __ballot(blend && T > 0.5f);
           if (omask != 0ull) {
             const int cnt = __popc((uint32_t)(omask >> row_shift) & 0xFFFFu);
             if (rt.l16 == 0 && cnt != 0) atomicAdd(&s_obs[j], cnt);
           }
-          if (blend) {
-            T = test_T;
-            last = (uint32_t)(i * BATCH + j + 1);
-          }
+          T = blend ? test_T : T;
+          last = blend ? (uint32_t)(i * BATCH + j + 1) : last;
         }
         if (__ballot(stop) != 0ull) {
           if (stop) done = true;
@@ -248,11 +237,18 @@ render_fwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
 
 int launch_render_fwd(const RenderFwdArgs& a, hipStream_t stream) {
   const dim3 grid((a.W + GS_TILE_X - 1) / GS_TILE_X, (a.H + GS_TILE_Y - 1) / GS_TILE_Y, 1);
-  hipLaunchKernelGGL(render_fwd_kernel, grid, dim3(GS_TILE_PIX), 0, stream, (const uint2*)a.ranges, a.point_list, a.W,
-                     a.H, a.fx, a.fy, a.cx, a.cy, (const float2*)a.means2D, a.rgb, a.all_map,
-                     (const float4*)a.conic_opacity, a.compute_locally, a.bg, a.render_geo, a.final_T, a.n_contrib_px,
-                     a.n_contrib2loss_px, a.out_color, a.out_observe, a.out_all_map, a.out_plane_depth, a.n_render,
-                     a.n_consider, a.n_contrib_tile);
+  if (a.render_geo)
+    hipLaunchKernelGGL(render_fwd_kernel<true>, grid, dim3(GS_TILE_PIX), 0, stream, (const uint2*)a.ranges,
+                       a.point_list, a.W, a.H, a.fx, a.fy, a.cx, a.cy, (const float2*)a.means2D, a.rgb, a.all_map,
+                       (const float4*)a.conic_opacity, a.compute_locally, a.bg, a.final_T, a.n_contrib_px,
+                       a.n_contrib2loss_px, a.out_color, a.out_observe, a.out_all_map, a.out_plane_depth, a.n_render,
+                       a.n_consider, a.n_contrib_tile);
+  else
+    hipLaunchKernelGGL(render_fwd_kernel<false>, grid, dim3(GS_TILE_PIX), 0, stream, (const uint2*)a.ranges,
+                       a.point_list, a.W, a.H, a.fx, a.fy, a.cx, a.cy, (const float2*)a.means2D, a.rgb, a.all_map,
+                       (const float4*)a.conic_opacity, a.compute_locally, a.bg, a.final_T, a.n_contrib_px,
+                       a.n_contrib2loss_px, a.out_color, a.out_observe, a.out_all_map, a.out_plane_depth, a.n_render,
+                       a.n_consider, a.n_contrib_tile);
   return 0;
 }
 

@@ -24,7 +24,7 @@ __global__ void __launch_bounds__(GS_WAVE) reduce_selftest_kernel(const float* _
 #pragma unroll
     for (int k = 0; k < 4; k++) out_wave[k + 4 * row] = r[k];
   }
-  const float t = row_transpose_reduce16(v, lane & 15);
+  const float t = row_transpose_reduce16(v);
   out_rows[(lane >> 4) * 16 + (lane & 15)] = t;
 }
 
