@@ -41,6 +41,9 @@ def parse():
     ap.add_argument("--gaussians", type=int, default=None, help="override the Gaussian count (debugging only)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-runs", type=int, default=3)
+    ap.add_argument("--copy-calibration-mib", type=int, default=0,
+                    help="also run three plain device-to-device copies of this many MiB after the timed regions: "
+                         "a kernel of known traffic against which FETCH_SIZE / WRITE_SIZE counters are scaled")
     return ap.parse_args()
 
 
@@ -147,6 +150,13 @@ def main():
     gn.stage_timing(False)
     stages = gn.stage_timing_collect()
     ms_per_step_instrumented = (t3 - t2) * 1e3 / args.steps
+    if args.copy_calibration_mib > 0:
+        src = torch.empty(args.copy_calibration_mib << 20, dtype=torch.uint8, device=dev).random_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     R = int(info["n_render"].sum().item())
 
     stage_report = {}

@@ -70,11 +70,17 @@ sort_histogram_kernel(int64_t n, const K* __restrict__ keys, int passes, int end
   for (int p = 0; p < passes; p++) s_h[p][threadIdx.x] = 0;
   __syncthreads();
   const int64_t base = (int64_t)blockIdx.x * (SORT_THREADS * HIST_ITEMS);
-#pragma unroll 4
+  K keyv[HIST_ITEMS];  // all loads in flight before the first key is counted
+#pragma unroll
+  for (int k = 0; k < HIST_ITEMS; k++) {
+    const int64_t idx = base + (int64_t)k * SORT_THREADS + threadIdx.x;
+    keyv[k] = idx < n ? keys[idx] : (K)0;
+  }
+#pragma unroll
   for (int k = 0; k < HIST_ITEMS; k++) {
     const int64_t idx = base + (int64_t)k * SORT_THREADS + threadIdx.x;
     const bool valid = idx < n;
-    const K key = valid ? keys[idx] : (K)0;
+    const K key = keyv[k];
     for (int p = 0; p < passes; p++) {
       const int shift = 8 * p;
       const int bits = end_bit - shift >= 8 ? 8 : end_bit - shift;
