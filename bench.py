@@ -28,6 +28,8 @@ BYTES_PER_GAUSSIAN = {
     "tile_count": 16,
     "inclusive_sum": 8,
     "preprocess_bwd": 560,
+    "all_map_fwd": 60,   # means 12 + scales 12 + rotations 16 in, 20 out
+    "all_map_bwd": 88,   # the same 40 + 20 B of upstream gradient in, 12 + 16 out
 }
 BYTES_PER_INSTANCE = {"sort_pairs": 152, "identify_tile_ranges": 8}
 
@@ -147,9 +149,35 @@ def main():
         step()
     torch.cuda.synchronize()
     t3 = time.perf_counter()
+    # the fused geometry-channel op that sits between the two rasterizer ops in the caller (not part of
+    # `value`, whose step uses a precomputed all_map like the earlier measurements): same event pairs
+    from diff_gaussian_rasterization import build_all_map
+    vmat, cpos = cam.world_view_transform.to(dev), cam.camera_center.to(dev)
+    g_am = torch.randn(P, 5, device=dev)
+    # these kernels are shorter than a Python launch: keep the stream busy first so the launches queue up
+    # behind it and the event pairs bracket kernels, not host latency
+    torch.cuda._sleep(int(4e7))
+    for _ in range(args.steps):
+        for k in ("means3D", "rotations"):
+            leaf[k].grad = None
+        build_all_map(leaf["means3D"], leaf["scales"], leaf["rotations"], vmat, cpos).backward(g_am)
+    torch.cuda.synchronize()
     gn.stage_timing(False)
     stages = gn.stage_timing_collect()
     ms_per_step_instrumented = (t3 - t2) * 1e3 / args.steps
+    # the torch lines it replaces, timed the same way for reference
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch_am_ms = []
+    for _ in range(5):
+        for k in ("means3D", "rotations"):
+            leaf[k].grad = None
+        e0.record()
+        gs_scenes.build_all_map(leaf["means3D"], leaf["scales"], leaf["rotations"], cam).backward(g_am)
+        e1.record()
+        torch.cuda.synchronize()
+        torch_am_ms.append(e0.elapsed_time(e1))
+    for t in leaf.values():
+        t.grad = None
     if args.copy_calibration_mib > 0:
         src = torch.empty(args.copy_calibration_mib << 20, dtype=torch.uint8, device=dev).random_()
         dst = torch.empty_like(src)
@@ -199,6 +227,7 @@ def main():
         "roofline": roofline,
         "ms_per_step_with_stage_events": round(ms_per_step_instrumented, 4),
         "stages": stage_report,
+        "all_map_torch_reference_ms": round(sorted(torch_am_ms)[len(torch_am_ms) // 2], 4),
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(g, cam, am_cpu.numpy(), ug_cpu, args.cpu_runs)

@@ -562,6 +562,33 @@ size_t gs_render_backward_workspace_bytes(int R) { return (size_t)(R > 0 ? R : 1
 
 size_t gs_knn_workspace_bytes(int P) { return knn_temp_bytes(P) + 256; }
 
+int gs_all_map_forward(int P, const float* means3D, const float* scales, const float* rotations,
+                       const float* viewmatrix, const float* campos, float* all_map, gs_stream_t stream) {
+  GS_REQUIRE(P >= 0, "gs_all_map_forward: negative P");
+  if (P == 0) return 0;
+  GS_REQUIRE(means3D && scales && rotations && viewmatrix && campos && all_map, "gs_all_map_forward: null pointer");
+  {
+    StageScope _t("all_map_fwd", (hipStream_t)stream);
+    launch_all_map_fwd(P, means3D, scales, rotations, viewmatrix, campos, all_map, (hipStream_t)stream);
+  }
+  return check_launch("all_map_forward", (hipStream_t)stream, false);
+}
+
+int gs_all_map_backward(int P, const float* means3D, const float* scales, const float* rotations,
+                        const float* viewmatrix, const float* campos, const float* dL_dall_map,
+                        float* dL_dmeans3D, float* dL_drotations, gs_stream_t stream) {
+  GS_REQUIRE(P >= 0, "gs_all_map_backward: negative P");
+  if (P == 0) return 0;
+  GS_REQUIRE(means3D && scales && rotations && viewmatrix && campos && dL_dall_map && dL_dmeans3D && dL_drotations,
+             "gs_all_map_backward: null pointer");
+  {
+    StageScope _t("all_map_bwd", (hipStream_t)stream);
+    launch_all_map_bwd(P, means3D, scales, rotations, viewmatrix, campos, dL_dall_map, dL_dmeans3D, dL_drotations,
+                       (hipStream_t)stream);
+  }
+  return check_launch("all_map_backward", (hipStream_t)stream, false);
+}
+
 int gs_knn_dist2(int P, const float* points, float* mean_dists, void* workspace, size_t workspace_bytes,
                  gs_stream_t stream) {
   GS_REQUIRE(P >= 0, "gs_knn_dist2: negative P");

@@ -57,6 +57,11 @@ int launch_duplicate_with_keys(int P, int W, int H, const float* means2D, const 
                                uint64_t* keys, uint32_t* values, uint32_t* emission /*optional*/,
                                hipStream_t stream);
 int launch_gather_u32(int64_t n, const uint32_t* index, const uint32_t* table, uint32_t* out, hipStream_t stream);
+int launch_all_map_fwd(int P, const float* means, const float* scales, const float* rots, const float* V,
+                       const float* campos, float* out, hipStream_t stream);
+int launch_all_map_bwd(int P, const float* means, const float* scales, const float* rots, const float* V,
+                       const float* campos, const float* grad_out, float* dmeans, float* drots,
+                       hipStream_t stream);
 int launch_tile_ranges(int64_t L, const uint64_t* keys_sorted, int T, uint32_t* ranges, hipStream_t stream);
 
 // ---- radix sort (stable, LSD, 8-bit digits) ----

@@ -282,6 +282,42 @@ def rasterize_aussians_filter(means3D, scales, rotations, scale_modifier, cov3D_
     return radii
 
 
+def build_all_map(means3D, scales, rotations, viewmatrix, campos):
+    """The per-Gaussian geometry channels [normal_cam(3), 1, |normal . p_cam|] that the caller of the
+    reference assembles in torch between the two rasterizer ops
+    (gaussian_renderer/__init__.py:1501-1518), as one kernel.  No counterpart in the reference's
+    extension module."""
+    means3D = _f32c(means3D, "means3D")
+    dev = means3D.device
+    P = means3D.shape[0]
+    all_map = torch.empty(P, 5, dtype=torch.float32, device=dev)
+    if P == 0:
+        return all_map
+    sc, rot = _f32c(scales, "scales"), _f32c(rotations, "rotations")
+    vm, cp = _f32c(viewmatrix, "viewmatrix"), _f32c(campos, "campos")
+    _n.check(_n.lib.gs_all_map_forward(P, _ptr(means3D), _ptr(sc), _ptr(rot), _ptr(vm), _ptr(cp), _ptr(all_map),
+                                       _stream(dev)), "build_all_map")
+    return all_map
+
+
+def build_all_map_backward(means3D, scales, rotations, viewmatrix, campos, dL_dall_map):
+    """Gradient of build_all_map with respect to means3D and (unnormalised) rotations."""
+    means3D = _f32c(means3D, "means3D")
+    dev = means3D.device
+    P = means3D.shape[0]
+    dL_dmeans3D = torch.empty(P, 3, dtype=torch.float32, device=dev)
+    dL_drotations = torch.empty(P, 4, dtype=torch.float32, device=dev)
+    if P == 0:
+        return dL_dmeans3D, dL_drotations
+    sc, rot = _f32c(scales, "scales"), _f32c(rotations, "rotations")
+    vm, cp = _f32c(viewmatrix, "viewmatrix"), _f32c(campos, "campos")
+    g = _f32c(dL_dall_map, "dL_dall_map")
+    _n.check(_n.lib.gs_all_map_backward(P, _ptr(means3D), _ptr(sc), _ptr(rot), _ptr(vm), _ptr(cp), _ptr(g),
+                                        _ptr(dL_dmeans3D), _ptr(dL_drotations), _stream(dev)),
+             "build_all_map_backward")
+    return dL_dmeans3D, dL_drotations
+
+
 def get_distribution_strategy(*_args, **_kwargs):
     # Same behaviour as the reference (rasterizer_impl.cu:507-508).
     raise RuntimeError("getDistributionStrategy is deprecated.")

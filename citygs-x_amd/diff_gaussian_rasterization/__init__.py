@@ -19,7 +19,8 @@ import torch.nn as nn
 
 from . import _C
 
-__all__ = ["GaussianRasterizationSettings", "GaussianRasterizer", "preprocess_gaussians", "render_gaussians"]
+__all__ = ["GaussianRasterizationSettings", "GaussianRasterizer", "preprocess_gaussians", "render_gaussians",
+           "build_all_map"]
 
 
 class GaussianRasterizationSettings(NamedTuple):
@@ -127,6 +128,29 @@ def render_gaussians(means2D, means2D_abs, conic_opacity, rgb, all_map, depths, 
                      extended_compute_locally, raster_settings, cuda_args):
     return _RenderGaussians.apply(means2D, means2D_abs, conic_opacity, rgb, all_map, depths, radii, compute_locally,
                                   extended_compute_locally, raster_settings, cuda_args)
+
+
+# ------------------------------------------------------------------ all_map --
+
+class _BuildAllMap(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, means3D, scales, rotations, viewmatrix, campos):
+        ctx.save_for_backward(means3D, scales, rotations, viewmatrix, campos)
+        return _C.build_all_map(means3D, scales, rotations, viewmatrix, campos)
+
+    @staticmethod
+    def backward(ctx, grad_all_map):
+        means3D, scales, rotations, viewmatrix, campos = ctx.saved_tensors
+        dL_dmeans3D, dL_drotations = _C.build_all_map_backward(means3D, scales, rotations, viewmatrix, campos,
+                                                               grad_all_map)
+        return dL_dmeans3D, None, dL_drotations, None, None
+
+
+def build_all_map(means3D, scales, rotations, viewmatrix, campos):
+    """[normal in the camera frame, 1, |normal . p_cam|] per Gaussian: a drop-in for the torch lines
+    gaussian_renderer/__init__.py:1501-1518 (pass the camera's world_view_transform and camera_center).
+    Differentiable in means3D and rotations, like those lines; `scales` only picks the axis."""
+    return _BuildAllMap.apply(means3D, scales, rotations, viewmatrix, campos)
 
 
 # ------------------------------------------------------------------- module --

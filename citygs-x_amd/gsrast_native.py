@@ -35,6 +35,8 @@ _SIGNATURES = {
                           [_vp] * 16 + [_i, _i, C.POINTER(_i), C.POINTER(_f), _vp]),
     "gs_render_backward_workspace_bytes": (_sz, [_i]),
     "gs_render_backward": (_i, [_i, _i, _vp, _i, _i, _f, _f] + [_vp] * 17 + [_i, _i, _vp, _sz, C.POINTER(_f), _vp]),
+    "gs_all_map_forward": (_i, [_i] + [_vp] * 7),
+    "gs_all_map_backward": (_i, [_i] + [_vp] * 9),
     "gs_knn_workspace_bytes": (_sz, [_i]),
     "gs_knn_dist2": (_i, [_i, _vp, _vp, _vp, _sz, _vp]),
     "gs_tile_count": (_i, [_i, _i, _i, _vp, _vp, _vp, _vp, _vp]),

@@ -146,6 +146,20 @@ size_t gs_knn_workspace_bytes(int P);
 int gs_knn_dist2(int P, const float* points, float* mean_dists, void* workspace, size_t workspace_bytes,
                  gs_stream_t stream);
 
+/* Replaces the caller-side torch code that builds the per-Gaussian geometry channels between the two
+ * rasterizer ops (gaussian_renderer/__init__.py:1501-1518: quaternion_to_matrix(normalize(rotations)),
+ * axis of the smallest scale as normal, flipped towards the camera, rotated by viewmatrix[:3,:3];
+ * distance = |normal . p_cam|).  all_map (P,5) = [normal_cam(3), 1, distance].  `scales` only has to order
+ * like the activated scales (the reference takes the argmin of exp(scales)).
+ * The backward entry returns what autograd derives from those lines: dL/dmeans3D (P,3) and
+ * dL/drotations (P,4, with respect to the unnormalised quaternions); scales get no gradient.
+ * Every output element is written. */
+int gs_all_map_forward(int P, const float* means3D, const float* scales, const float* rotations,
+                       const float* viewmatrix, const float* campos, float* all_map, gs_stream_t stream);
+int gs_all_map_backward(int P, const float* means3D, const float* scales, const float* rotations,
+                        const float* viewmatrix, const float* campos, const float* dL_dall_map,
+                        float* dL_dmeans3D, float* dL_drotations, gs_stream_t stream);
+
 /* ---- Stage-level entry points: the individual steps of renderForward, exposed
  * so each can be checked and profiled on its own. ---- */
 

@@ -33,6 +33,9 @@
 //     dL_dalpha = fma(dL_dalpha, T, -(T_final*bg_dot)*inv).
 //     Algebraically the reference's expressions, with the rounding order fixed.
 //
+// oracle_all_map_* restate caller-side torch code (floating-point sums whose order torch leaves open):
+// pinned to rounding against a float64 torch evaluation with autograd, not bit for bit.
+//
 // Parity pins (tests/test_oracle_*.py): closed forms, an independent torch
 // restatement with autograd, brute force on tiny inputs, numpy/scipy library
 // routines.  The reference holds no golden vectors for this path.
@@ -1035,6 +1038,142 @@ uint32_t oracle_morton(const float* p, const float* mn, const float* mx) {
     c[k] = x;
   }
   return c[0] | (c[1] << 1) | (c[2] << 2);
+}
+
+
+// ---------------------------------------------------------------------------
+// Per-Gaussian geometry channels handed to the blend ("all_map"): the caller's
+// torch code at gaussian_renderer/__init__.py:1501-1518, restated per Gaussian.
+//   R = quaternion_to_matrix(normalize(q))      (pytorch3d 0.3.0, environment.yml:156:
+//        two_s = 2 / (q.q); row-major 3x3 with (r,i,j,k) = q;  F.normalize divides by max(|q|, 1e-12))
+//   n = column argmin(scales) of R, negated where n . (campos - mean) < 0
+//   local = n @ V[:3,:3];  p = mean @ V[:3,:3] + V[3,:3];  out = [local, 1, |local . p|]
+// The reference takes the argmin over exp(scales); exp is monotone, so this is the argmin of the
+// scales themselves (first minimum on ties).  torch's reductions and matmul leave the summation
+// order open; sums here run left to right, so agreement with torch is to rounding, not bitwise.
+static inline int allmap_min_axis(const float* s) {
+  int a = 0;
+  if (s[1] < s[a]) a = 1;
+  if (s[2] < s[a]) a = 2;
+  return a;
+}
+
+// column `c` of quaternion_to_matrix for a (not necessarily unit) quaternion q = (r,i,j,k)
+static inline void allmap_column(const float* q, int c, float two_s, float* n) {
+  const float r = q[0], i = q[1], j = q[2], k = q[3];
+  if (c == 0) {
+    n[0] = 1.0f - two_s * (j * j + k * k);
+    n[1] = two_s * (i * j + k * r);
+    n[2] = two_s * (i * k - j * r);
+  } else if (c == 1) {
+    n[0] = two_s * (i * j - k * r);
+    n[1] = 1.0f - two_s * (i * i + k * k);
+    n[2] = two_s * (j * k + i * r);
+  } else {
+    n[0] = two_s * (i * k + j * r);
+    n[1] = two_s * (j * k - i * r);
+    n[2] = 1.0f - two_s * (i * i + j * j);
+  }
+}
+
+void oracle_all_map_fwd(int P, const float* means, const float* scales, const float* rots, const float* V,
+                        const float* campos, float* out) {
+#pragma omp parallel for schedule(static)
+  for (int g = 0; g < P; g++) {
+    const float* q0 = rots + 4 * (size_t)g;
+    const float* m = means + 3 * (size_t)g;
+    const float len = sqrtf(((q0[0] * q0[0] + q0[1] * q0[1]) + q0[2] * q0[2]) + q0[3] * q0[3]);
+    const float den = fmaxf(len, 1e-12f);
+    const float q[4] = {q0[0] / den, q0[1] / den, q0[2] / den, q0[3] / den};
+    const float two_s = 2.0f / (((q[0] * q[0] + q[1] * q[1]) + q[2] * q[2]) + q[3] * q[3]);
+    float n[3];
+    allmap_column(q, allmap_min_axis(scales + 3 * (size_t)g), two_s, n);
+    const float tc[3] = {campos[0] - m[0], campos[1] - m[1], campos[2] - m[2]};
+    if ((n[0] * tc[0] + n[1] * tc[1]) + n[2] * tc[2] < 0.0f) {
+      n[0] = -n[0]; n[1] = -n[1]; n[2] = -n[2];
+    }
+    float loc[3], pc[3];
+    for (int k = 0; k < 3; k++) {
+      loc[k] = (n[0] * V[k] + n[1] * V[4 + k]) + n[2] * V[8 + k];
+      pc[k] = ((m[0] * V[k] + m[1] * V[4 + k]) + m[2] * V[8 + k]) + V[12 + k];
+    }
+    float* o = out + 5 * (size_t)g;
+    o[0] = loc[0]; o[1] = loc[1]; o[2] = loc[2];
+    o[3] = 1.0f;
+    o[4] = fabsf((loc[0] * pc[0] + loc[1] * pc[1]) + loc[2] * pc[2]);
+  }
+}
+
+// Gradient of the above with respect to means and (unnormalised) rotations: what autograd derives
+// from the same torch lines.  scales only choose the axis and the flip only a sign: no gradient.
+void oracle_all_map_bwd(int P, const float* means, const float* scales, const float* rots, const float* V,
+                        const float* campos, const float* gout, float* dmeans, float* drots) {
+#pragma omp parallel for schedule(static)
+  for (int g = 0; g < P; g++) {
+    const float* q0 = rots + 4 * (size_t)g;
+    const float* m = means + 3 * (size_t)g;
+    const float* go = gout + 5 * (size_t)g;
+    const float len = sqrtf(((q0[0] * q0[0] + q0[1] * q0[1]) + q0[2] * q0[2]) + q0[3] * q0[3]);
+    const float den = fmaxf(len, 1e-12f);
+    const float q[4] = {q0[0] / den, q0[1] / den, q0[2] / den, q0[3] / den};
+    const float two_s = 2.0f / (((q[0] * q[0] + q[1] * q[1]) + q[2] * q[2]) + q[3] * q[3]);
+    const int c = allmap_min_axis(scales + 3 * (size_t)g);
+    float n[3];
+    allmap_column(q, c, two_s, n);
+    const float tc[3] = {campos[0] - m[0], campos[1] - m[1], campos[2] - m[2]};
+    const bool flip = (n[0] * tc[0] + n[1] * tc[1]) + n[2] * tc[2] < 0.0f;
+    const float sgn = flip ? -1.0f : 1.0f;
+    float loc[3], pc[3];
+    for (int k = 0; k < 3; k++) {
+      loc[k] = sgn * ((n[0] * V[k] + n[1] * V[4 + k]) + n[2] * V[8 + k]);
+      pc[k] = ((m[0] * V[k] + m[1] * V[4 + k]) + m[2] * V[8 + k]) + V[12 + k];
+    }
+    const float s = (loc[0] * pc[0] + loc[1] * pc[1]) + loc[2] * pc[2];
+    const float gs = go[4] * (s > 0.0f ? 1.0f : (s < 0.0f ? -1.0f : 0.0f));  // d|s| = sign(s)
+    float gl[3], gp[3];
+    for (int k = 0; k < 3; k++) {
+      gl[k] = go[k] + gs * pc[k];
+      gp[k] = gs * loc[k];
+    }
+    float gn[3];
+    for (int a = 0; a < 3; a++) {
+      gn[a] = sgn * ((gl[0] * V[4 * a] + gl[1] * V[4 * a + 1]) + gl[2] * V[4 * a + 2]);
+      dmeans[3 * (size_t)g + a] = (gp[0] * V[4 * a] + gp[1] * V[4 * a + 1]) + gp[2] * V[4 * a + 2];
+    }
+    // column c of R as a function of (r,i,j,k) and two_s = 2/(q.q)
+    const float r = q[0], i = q[1], j = q[2], k = q[3], ts = two_s;
+    float gq[4], gts;
+    if (c == 0) {
+      gq[0] = ts * (k * gn[1] - j * gn[2]);
+      gq[1] = ts * (j * gn[1] + k * gn[2]);
+      gq[2] = ts * ((-2.0f * j * gn[0] + i * gn[1]) - r * gn[2]);
+      gq[3] = ts * ((-2.0f * k * gn[0] + r * gn[1]) + i * gn[2]);
+      gts = (-(j * j + k * k) * gn[0] + (i * j + k * r) * gn[1]) + (i * k - j * r) * gn[2];
+    } else if (c == 1) {
+      gq[0] = ts * (-k * gn[0] + i * gn[2]);
+      gq[1] = ts * ((j * gn[0] - 2.0f * i * gn[1]) + r * gn[2]);
+      gq[2] = ts * (i * gn[0] + k * gn[2]);
+      gq[3] = ts * ((-r * gn[0] - 2.0f * k * gn[1]) + j * gn[2]);
+      gts = ((i * j - k * r) * gn[0] - (i * i + k * k) * gn[1]) + (j * k + i * r) * gn[2];
+    } else {
+      gq[0] = ts * (j * gn[0] - i * gn[1]);
+      gq[1] = ts * ((k * gn[0] - r * gn[1]) - 2.0f * i * gn[2]);
+      gq[2] = ts * ((r * gn[0] + k * gn[1]) - 2.0f * j * gn[2]);
+      gq[3] = ts * (i * gn[0] + j * gn[1]);
+      gts = ((i * k + j * r) * gn[0] + (j * k - i * r) * gn[1]) - (i * i + j * j) * gn[2];
+    }
+    // d two_s / dq = -two_s^2 q
+    const float w = -(ts * ts) * gts;
+    for (int a = 0; a < 4; a++) gq[a] += w * q[a];
+    // F.normalize backward: q_hat = q0 / max(|q0|, eps)
+    float* dq = drots + 4 * (size_t)g;
+    if (len > 1e-12f) {
+      const float dot = ((q[0] * gq[0] + q[1] * gq[1]) + q[2] * gq[2]) + q[3] * gq[3];
+      for (int a = 0; a < 4; a++) dq[a] = (gq[a] - q[a] * dot) / len;
+    } else {
+      for (int a = 0; a < 4; a++) dq[a] = gq[a] / den;
+    }
+  }
 }
 
 }  // extern "C"

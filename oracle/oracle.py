@@ -288,6 +288,26 @@ def preprocess_bwd(means, radii, shs, clamped, scales, rots, cov3D, V, PM, campo
     return o
 
 
+def all_map_fwd(means3D, scales, rotations, viewmatrix, campos):
+    """gaussian_renderer/__init__.py:1501-1518."""
+    means3D, scales, rotations = _f32(means3D), _f32(scales), _f32(rotations)
+    V, cp = _f32(viewmatrix).reshape(16), _f32(campos).reshape(3)
+    P = means3D.shape[0]
+    out = np.zeros((P, 5), np.float32)
+    lib().oracle_all_map_fwd(C.c_int(P), _p(means3D), _p(scales), _p(rotations), _p(V), _p(cp), _p(out))
+    return out
+
+
+def all_map_bwd(means3D, scales, rotations, viewmatrix, campos, grad_out):
+    means3D, scales, rotations, grad_out = _f32(means3D), _f32(scales), _f32(rotations), _f32(grad_out)
+    V, cp = _f32(viewmatrix).reshape(16), _f32(campos).reshape(3)
+    P = means3D.shape[0]
+    dm, dq = np.zeros((P, 3), np.float32), np.zeros((P, 4), np.float32)
+    lib().oracle_all_map_bwd(C.c_int(P), _p(means3D), _p(scales), _p(rotations), _p(V), _p(cp), _p(grad_out), _p(dm),
+                             _p(dq))
+    return dm, dq
+
+
 def knn_dist2(points):
     points = _f32(points)
     P = points.shape[0]

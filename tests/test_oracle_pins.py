@@ -457,3 +457,60 @@ def test_knn_against_brute_force(orc, P, kind):
     p64 = pts.astype(np.float64)
     d, _ = cKDTree(p64).query(p64, k=4)
     np.testing.assert_allclose(got, (d[:, 1:] ** 2).mean(1), rtol=3e-5, atol=1e-12)
+
+
+# ---------------------------------------------------------------- all_map --
+
+def _all_map_case(P=4000, seed=5):
+    import gs_scenes
+    g, cams = gs_scenes.make_scene(0, P=P, n_views=1, seed=seed)
+    return g, cams[0]
+
+
+def test_all_map_forward_matches_float64_torch_and_closed_form(orc):
+    import gs_scenes
+    g, cam = _all_map_case()
+
+    class C64:
+        world_view_transform = cam.world_view_transform.double()
+        camera_center = cam.camera_center.double()
+    ref = gs_scenes.build_all_map(g["means3D"].double(), g["scales"].double(), g["rotations"].double(), C64).numpy()
+    o = orc.all_map_fwd(g["means3D"].numpy(), g["scales"].numpy(), g["rotations"].numpy(),
+                        cam.world_view_transform.numpy(), cam.camera_center.numpy())
+    assert np.abs(o[:, :3] - ref[:, :3]).max() <= 2e-6
+    assert np.all(o[:, 3] == 1.0)
+    assert np.abs(o[:, 4] - ref[:, 4]).max() <= 1e-5 * max(1.0, np.abs(ref[:, 4]).max())
+    # closed form: identity rotation, smallest scale along z, camera = identity at the origin looking at +z
+    m = np.array([[0.5, -0.25, 4.0]], np.float32)
+    s = np.array([[0.3, 0.2, 0.1]], np.float32)
+    q = np.array([[2.0, 0.0, 0.0, 0.0]], np.float32)  # unnormalised on purpose
+    V = np.eye(4, dtype=np.float32)
+    o1 = orc.all_map_fwd(m, s, q, V, np.zeros(3, np.float32))
+    # normal = +z flipped towards the camera at the origin -> (0,0,-1); distance = |n . p| = 4
+    assert np.allclose(o1[0], [0.0, 0.0, -1.0, 1.0, 4.0], atol=1e-6)
+    # smallest scale along x, rotation of 90 degrees about z maps the x axis to +y
+    q90 = np.array([[np.sqrt(0.5), 0.0, 0.0, np.sqrt(0.5)]], np.float32)
+    o2 = orc.all_map_fwd(m, np.array([[0.1, 0.2, 0.3]], np.float32), q90, V, np.zeros(3, np.float32))
+    # n = +y; n . (cam - m) = 0.25 > 0: kept; distance = |-0.25|
+    assert np.allclose(o2[0], [0.0, 1.0, 0.0, 1.0, 0.25], atol=1e-6)
+
+
+def test_all_map_backward_matches_float64_autograd(orc):
+    import gs_scenes
+    g, cam = _all_map_case(seed=6)
+
+    class C64:
+        world_view_transform = cam.world_view_transform.double()
+        camera_center = cam.camera_center.double()
+    m = g["means3D"].double().requires_grad_(True)
+    q = (g["rotations"].double() * 1.7).requires_grad_(True)  # away from unit length: exercises normalize
+    out = gs_scenes.build_all_map(m, g["scales"].double(), q, C64)
+    go = torch.randn(out.shape, generator=torch.Generator().manual_seed(2), dtype=torch.float64)
+    (out * go).sum().backward()
+    dm, dq = orc.all_map_bwd(g["means3D"].numpy(), g["scales"].numpy(), (g["rotations"] * 1.7).numpy(),
+                             cam.world_view_transform.numpy(), cam.camera_center.numpy(), go.float().numpy())
+    rel = lambda a, b: np.linalg.norm(a - b) / np.linalg.norm(b)
+    assert rel(dm, m.grad.numpy()) <= 1e-6
+    assert rel(dq, q.grad.numpy()) <= 1e-6
+    # the rotation gradient is orthogonal to the quaternion (the output does not depend on its length)
+    assert np.abs((dq * (g["rotations"] * 1.7).numpy()).sum(1)).max() <= 1e-4 * np.abs(dq).max()
