@@ -161,6 +161,14 @@ def main():
         for k in ("means3D", "rotations"):
             leaf[k].grad = None
         build_all_map(leaf["means3D"], leaf["scales"], leaf["rotations"], vmat, cpos).backward(g_am)
+    # the optimizer step over the same five parameter tensors (59 M elements), fused into one launch
+    from gs_optim import FusedAdam
+    opt = FusedAdam([{"params": [leaf[k]], "lr": 1e-5, "name": k} for k in leaf], lr=0.0, eps=1e-15)
+    for t in leaf.values():
+        t.grad = torch.randn_like(t) * 1e-3
+    n_adam = sum(t.numel() for t in leaf.values())
+    for _ in range(args.steps):
+        opt.step()
     torch.cuda.synchronize()
     gn.stage_timing(False)
     stages = gn.stage_timing_collect()
@@ -198,6 +206,8 @@ def main():
             nbytes = BYTES_PER_INSTANCE[name] * R
         elif name == "duplicate_with_keys":
             nbytes = 20 * P + 12 * R
+        elif name == "adam_step":
+            nbytes = 28 * n_adam  # p, g, m, v in; p, m, v out
         if nbytes is not None and ms > 0:
             e["algorithmic_bytes"] = nbytes
             e["GBps"] = round(nbytes / (ms * 1e-3) / 1e9, 1)

@@ -562,6 +562,26 @@ size_t gs_render_backward_workspace_bytes(int R) { return (size_t)(R > 0 ? R : 1
 
 size_t gs_knn_workspace_bytes(int P) { return knn_temp_bytes(P) + 256; }
 
+int gs_adam_step(int count, float* const* params, const float* const* grads, float* const* exp_avg,
+                 float* const* exp_avg_sq, const long long* sizes, const double* lrs, const int* steps, double beta1,
+                 double beta2, double eps, float grad_scale, gs_stream_t stream) {
+  GS_REQUIRE(count >= 0, "gs_adam_step: negative count");
+  if (count == 0) return 0;
+  GS_REQUIRE(params && grads && exp_avg && exp_avg_sq && sizes && lrs && steps, "gs_adam_step: null table");
+  for (int i = 0; i < count; i++) {
+    if (sizes[i] <= 0) continue;
+    GS_REQUIRE(params[i] && grads[i] && exp_avg[i] && exp_avg_sq[i], "gs_adam_step: null tensor pointer");
+    GS_REQUIRE(steps[i] >= 1, "gs_adam_step: step numbers start at 1");
+  }
+  GS_REQUIRE(beta1 >= 0.0 && beta1 < 1.0 && beta2 >= 0.0 && beta2 < 1.0, "gs_adam_step: betas must lie in [0, 1)");
+  {
+    StageScope _t("adam_step", (hipStream_t)stream);
+    launch_adam(count, params, grads, exp_avg, exp_avg_sq, sizes, lrs, steps, beta1, beta2, eps, grad_scale,
+                (hipStream_t)stream);
+  }
+  return check_launch("adam_step", (hipStream_t)stream, false);
+}
+
 int gs_all_map_forward(int P, const float* means3D, const float* scales, const float* rotations,
                        const float* viewmatrix, const float* campos, float* all_map, gs_stream_t stream) {
   GS_REQUIRE(P >= 0, "gs_all_map_forward: negative P");

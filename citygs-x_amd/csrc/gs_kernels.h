@@ -57,6 +57,10 @@ int launch_duplicate_with_keys(int P, int W, int H, const float* means2D, const 
                                uint64_t* keys, uint32_t* values, uint32_t* emission /*optional*/,
                                hipStream_t stream);
 int launch_gather_u32(int64_t n, const uint32_t* index, const uint32_t* table, uint32_t* out, hipStream_t stream);
+constexpr int ADAM_MAX_TENSORS = 24;  // tensors per launch (more are split over several launches)
+int launch_adam(int count, float* const* params, const float* const* grads, float* const* exp_avg,
+                float* const* exp_avg_sq, const long long* sizes, const double* lrs, const int* steps, double beta1,
+                double beta2, double eps, float grad_scale, hipStream_t stream);
 int launch_all_map_fwd(int P, const float* means, const float* scales, const float* rots, const float* V,
                        const float* campos, float* out, hipStream_t stream);
 int launch_all_map_bwd(int P, const float* means, const float* scales, const float* rots, const float* V,

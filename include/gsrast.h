@@ -160,6 +160,17 @@ int gs_all_map_backward(int P, const float* means3D, const float* scales, const 
                         const float* viewmatrix, const float* campos, const float* dL_dall_map,
                         float* dL_dmeans3D, float* dL_drotations, gs_stream_t stream);
 
+/* Replaces optimizer.step() of the reference's torch.optim.Adam(lr=0.0, eps=1e-15) with per-group learning
+ * rates (scene/gaussian_model.py:574, stepped at train_internal.py:404-417) for `count` tensors in one
+ * launch: update rule of torch 2.0.0 with betas (beta1, beta2), no weight decay, no amsgrad.
+ * params / grads / exp_avg / exp_avg_sq: host arrays of `count` device pointers (float32, sizes[i] elements
+ * each); hyper-parameters are doubles, as the Python floats of that optimizer are; lrs[i] and steps[i] (the step number after this update, >= 1) per tensor; grad_scale multiplies
+ * every gradient first (1/bsz of train_internal.py:407-410; 1.0 for none).  params, exp_avg and
+ * exp_avg_sq are updated in place; grads are only read.  Tensors with sizes[i] <= 0 are skipped. */
+int gs_adam_step(int count, float* const* params, const float* const* grads, float* const* exp_avg,
+                 float* const* exp_avg_sq, const long long* sizes, const double* lrs, const int* steps, double beta1,
+                 double beta2, double eps, float grad_scale, gs_stream_t stream);
+
 /* ---- Stage-level entry points: the individual steps of renderForward, exposed
  * so each can be checked and profiled on its own. ---- */
 

@@ -308,6 +308,22 @@ def all_map_bwd(means3D, scales, rotations, viewmatrix, campos, grad_out):
     return dm, dq
 
 
+def adam_step(param, grad, exp_avg, exp_avg_sq, lr, step, beta1=0.9, beta2=0.999, eps=1e-15, grad_scale=1.0):
+    """One torch.optim.Adam update (torch 2.0.0 rule, no weight decay / amsgrad; the optimizer of
+    scene/gaussian_model.py:574) in float32 numpy, returning new (param, exp_avg, exp_avg_sq).  Bias corrections
+    are Python floats, as in torch/optim/adam.py."""
+    f = np.float32
+    p, g, m, v = _f32(param), _f32(grad) * f(grad_scale), _f32(exp_avg), _f32(exp_avg_sq)
+    m = m * f(beta1) + f(1.0 - beta1) * g
+    v = v * f(beta2) + (f(1.0 - beta2) * g) * g
+    bc1 = 1.0 - beta1 ** step
+    bc2 = 1.0 - beta2 ** step
+    neg_step = f(-(lr / bc1))
+    denom = np.sqrt(v) / f(np.sqrt(bc2)) + f(eps)
+    p = p + (neg_step * m) / denom
+    return p.astype(np.float32), m.astype(np.float32), v.astype(np.float32)
+
+
 def knn_dist2(points):
     points = _f32(points)
     P = points.shape[0]

@@ -514,3 +514,35 @@ def test_all_map_backward_matches_float64_autograd(orc):
     assert rel(dq, q.grad.numpy()) <= 1e-6
     # the rotation gradient is orthogonal to the quaternion (the output does not depend on its length)
     assert np.abs((dq * (g["rotations"] * 1.7).numpy()).sum(1)).max() <= 1e-4 * np.abs(dq).max()
+
+
+# ------------------------------------------------------------------- Adam --
+
+def test_adam_step_matches_torch_optim_adam(orc):
+    """Library routine: torch.optim.Adam on the CPU, five steps, two parameter groups with their own lr."""
+    gen = torch.Generator().manual_seed(11)
+    shapes, lrs = [(1000, 3), (257,)], [1.6e-4, 5e-3]
+    ps = [torch.randn(s, generator=gen) for s in shapes]
+    tp = [p.clone().requires_grad_(True) for p in ps]
+    opt = torch.optim.Adam([{"params": [tp[0]], "lr": lrs[0]}, {"params": [tp[1]], "lr": lrs[1]}], lr=0.0, eps=1e-15)
+    mine = [(p.numpy().copy(), np.zeros(s, np.float32), np.zeros(s, np.float32)) for p, s in zip(ps, shapes)]
+    for step in range(1, 6):
+        grads = [torch.randn(s, generator=gen) * (10.0 ** (step - 3)) for s in shapes]
+        for p, g in zip(tp, grads):
+            p.grad = g.clone()
+        opt.step()
+        mine = [orc.adam_step(p, g.numpy(), m, v, lr, step) for (p, m, v), g, lr in zip(mine, grads, lrs)]
+        for (p, m, v), t, p0 in zip(mine, tp, ps):
+            st = opt.state[t]
+            rel = lambda a, b: np.linalg.norm(a - b) / max(np.linalg.norm(b), 1e-30)
+            assert rel(m, st["exp_avg"].numpy()) <= 1e-6
+            assert rel(v, st["exp_avg_sq"].numpy()) <= 1e-6
+            assert rel(p - p0.numpy(), t.detach().numpy() - p0.numpy()) <= 1e-5
+    # first step of Adam moves every element with a non-zero gradient by lr (textbook property)
+    p1, _, _ = orc.adam_step(np.zeros(4, np.float32), np.array([3.0, -2.0, 1e-3, 0.0], np.float32),
+                             np.zeros(4, np.float32), np.zeros(4, np.float32), 0.01, 1)
+    assert np.allclose(p1, [-0.01, 0.01, -0.01, 0.0], rtol=1e-5, atol=0)
+    # grad_scale = 1/bsz is the same as dividing the gradient first
+    a = orc.adam_step(ps[0].numpy(), grads[0].numpy(), mine[0][1], mine[0][2], 1e-3, 7, grad_scale=0.25)
+    b = orc.adam_step(ps[0].numpy(), grads[0].numpy() * np.float32(0.25), mine[0][1], mine[0][2], 1e-3, 7)
+    assert all(np.array_equal(x, y) for x, y in zip(a, b))
