@@ -169,10 +169,45 @@ def main():
     n_adam = sum(t.numel() for t in leaf.values())
     for _ in range(args.steps):
         opt.step()
+    # densification statistics of one view: 1 M anchors x 10 offsets, 40 % visible, 60 % selected, 90 % kept
+    import gs_densify
+    gen = torch.Generator(device=dev).manual_seed(5)
+    A_s, k_s = 1_000_000, 10
+    s_vis = torch.rand(A_s, generator=gen, device=dev) < 0.4
+    s_sel = torch.rand(int(s_vis.sum()) * k_s, generator=gen, device=dev) < 0.6
+    s_flt = torch.rand(int(s_sel.sum()), generator=gen, device=dev) < 0.9
+    s_grad = torch.randn(s_flt.numel(), 3, generator=gen, device=dev)
+    s_op = torch.randn(s_sel.numel(), 1, generator=gen, device=dev)
+    s_acc = [torch.zeros(A_s, 1, device=dev), torch.zeros(A_s, 1, device=dev), torch.zeros(A_s * k_s, 1, device=dev),
+             torch.zeros(A_s * k_s, 1, device=dev)]
+    stats_bytes = (A_s + 5 * s_sel.numel() + 13 * s_flt.numel() + 16 * int(s_vis.sum()) + 16 * int(s_flt.sum()))
+    torch.cuda._sleep(int(4e7))
+    for _ in range(args.steps):
+        gs_densify.training_statis(s_acc[0], s_acc[1], s_acc[2], s_acc[3], k_s, s_grad, s_op, s_flt, s_sel, s_vis)
     torch.cuda.synchronize()
     gn.stage_timing(False)
     stages = gn.stage_timing_collect()
     ms_per_step_instrumented = (t3 - t2) * 1e3 / args.steps
+    # the torch statements training_statis consists of, for reference
+    torch_stats_ms = []
+    for _ in range(5):
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        ev0.record()
+        temp = s_op.clone().view(-1)
+        temp[temp < 0] = 0
+        s_acc[0][s_vis] += temp.view(-1, k_s).sum(dim=1, keepdim=True)
+        s_acc[1][s_vis] += 1
+        vis_rep = s_vis.unsqueeze(1).repeat(1, k_s).view(-1)
+        combined = torch.zeros(A_s * k_s, dtype=torch.bool, device=dev)
+        combined[vis_rep] = s_sel
+        temp_mask = combined.clone()
+        combined[temp_mask] = s_flt
+        s_acc[2][combined] += torch.norm(s_grad[s_flt, :2], dim=-1, keepdim=True)
+        s_acc[3][combined] += 1
+        ev1.record()
+        torch.cuda.synchronize()
+        torch_stats_ms.append(ev0.elapsed_time(ev1))
+    del s_acc, s_grad, s_op, s_sel, s_flt, s_vis
     # the torch lines it replaces, timed the same way for reference
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     torch_am_ms = []
@@ -206,6 +241,8 @@ def main():
             nbytes = BYTES_PER_INSTANCE[name] * R
         elif name == "duplicate_with_keys":
             nbytes = 20 * P + 12 * R
+        elif name == "training_stats":
+            nbytes = stats_bytes  # masks, opacities, gradient rows and the read-modify-write of the touched accumulators
         elif name == "adam_step":
             nbytes = 28 * n_adam  # p, g, m, v in; p, m, v out
         if nbytes is not None and ms > 0:
@@ -237,6 +274,7 @@ def main():
         "roofline": roofline,
         "ms_per_step_with_stage_events": round(ms_per_step_instrumented, 4),
         "stages": stage_report,
+        "training_stats_torch_reference_ms": round(sorted(torch_stats_ms)[len(torch_stats_ms) // 2], 4),
         "all_map_torch_reference_ms": round(sorted(torch_am_ms)[len(torch_am_ms) // 2], 4),
     }
     if not args.no_cpu_baseline:

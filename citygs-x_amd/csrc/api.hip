@@ -562,6 +562,39 @@ size_t gs_render_backward_workspace_bytes(int R) { return (size_t)(R > 0 ? R : 1
 
 size_t gs_knn_workspace_bytes(int P) { return knn_temp_bytes(P) + 256; }
 
+size_t gs_training_stats_workspace_bytes(int64_t num_anchors, int64_t num_candidates) {
+  return train_stats_temp_bytes(num_anchors, num_candidates) + 256;
+}
+
+int gs_training_stats(int64_t num_anchors, int n_offsets, int64_t num_candidates, int64_t num_selected,
+                      const uint8_t* anchor_visible_mask, const uint8_t* offset_selection_mask,
+                      const uint8_t* update_filter, const float* viewspace_grad, int grad_stride,
+                      const float* opacity, float* opacity_accum, float* anchor_demon,
+                      float* offset_gradient_accum, float* offset_denom, void* workspace, size_t workspace_bytes,
+                      gs_stream_t stream) {
+  GS_REQUIRE(num_anchors >= 0 && n_offsets > 0 && num_candidates >= 0 && num_selected >= 0,
+             "gs_training_stats: bad sizes");
+  if (num_anchors == 0) return 0;
+  GS_REQUIRE(num_anchors * (int64_t)n_offsets < 0x7FFFFFFFll * GS_BLOCK_1D, "gs_training_stats: too many slots");
+  GS_REQUIRE(num_candidates < 0xFFFFFFFFll && num_anchors < 0xFFFFFFFFll, "gs_training_stats: ranks are 32-bit");
+  GS_REQUIRE(anchor_visible_mask && opacity_accum && anchor_demon && offset_gradient_accum && offset_denom,
+             "gs_training_stats: null pointer");
+  GS_REQUIRE(num_candidates == 0 || (offset_selection_mask && opacity),
+             "gs_training_stats: candidates without mask or opacity");
+  GS_REQUIRE(num_selected == 0 || (update_filter && viewspace_grad && grad_stride >= 2),
+             "gs_training_stats: selected Gaussians without filter or gradient (stride >= 2)");
+  GS_REQUIRE(workspace && workspace_bytes >= gs_training_stats_workspace_bytes(num_anchors, num_candidates),
+             "gs_training_stats: workspace missing or too small");
+  {
+    StageScope _t("training_stats", (hipStream_t)stream);
+    launch_train_stats(num_anchors, n_offsets, num_candidates, num_selected, anchor_visible_mask,
+                       offset_selection_mask, update_filter, viewspace_grad, grad_stride, opacity, opacity_accum,
+                       anchor_demon, offset_gradient_accum, offset_denom, align_ptr((char*)workspace, 256),
+                       (hipStream_t)stream);
+  }
+  return check_launch("training_stats", (hipStream_t)stream, false);
+}
+
 int gs_adam_step(int count, float* const* params, const float* const* grads, float* const* exp_avg,
                  float* const* exp_avg_sq, const long long* sizes, const double* lrs, const int* steps, double beta1,
                  double beta2, double eps, float grad_scale, gs_stream_t stream) {

@@ -63,8 +63,9 @@ tile_count_kernel(int P, uint32_t gx, uint32_t gy, const int* __restrict__ radii
   tiles_touched[i] = cnt;
 }
 
+template <typename T>
 __global__ void __launch_bounds__(SCAN_THREADS)
-scan_block_sums_kernel(int64_t n, const uint32_t* __restrict__ in, uint32_t* __restrict__ block_sums) {
+scan_block_sums_kernel(int64_t n, const T* __restrict__ in, uint32_t* __restrict__ block_sums) {
   __shared__ uint32_t s_wave[SCAN_THREADS / GS_WAVE];
   const int64_t base = (int64_t)blockIdx.x * SCAN_TILE;
   uint32_t s = 0;
@@ -98,9 +99,9 @@ __global__ void __launch_bounds__(1024) scan_spine_kernel(int nblocks, uint32_t*
   }
 }
 
-template <bool EXCLUSIVE>
+template <bool EXCLUSIVE, typename T>
 __global__ void __launch_bounds__(SCAN_THREADS)
-scan_apply_kernel(int64_t n, const uint32_t* in, const uint32_t* __restrict__ block_prefix, uint32_t* out,
+scan_apply_kernel(int64_t n, const T* in, const uint32_t* __restrict__ block_prefix, uint32_t* out,
                   uint32_t* total_out) {
   // in and out may be the same array: each thread reads its items before it writes them.
   __shared__ uint32_t s_wave[SCAN_THREADS / GS_WAVE];
@@ -205,17 +206,18 @@ size_t scan_temp_bytes(int64_t n) {
   return align_up((size_t)(nb > 0 ? nb : 1) * sizeof(uint32_t), 256);
 }
 
-static int scan_impl(int64_t n, const uint32_t* in, uint32_t* out, void* temp, bool exclusive, uint32_t* total_out,
+template <typename T>
+static int scan_impl(int64_t n, const T* in, uint32_t* out, void* temp, bool exclusive, uint32_t* total_out,
                      hipStream_t stream) {
   if (n <= 0) return 0;
   const int nb = (int)((n + SCAN_TILE - 1) / SCAN_TILE);
   uint32_t* sums = (uint32_t*)temp;
-  hipLaunchKernelGGL(scan_block_sums_kernel, dim3(nb), dim3(SCAN_THREADS), 0, stream, n, in, sums);
+  hipLaunchKernelGGL(scan_block_sums_kernel<T>, dim3(nb), dim3(SCAN_THREADS), 0, stream, n, in, sums);
   hipLaunchKernelGGL(scan_spine_kernel, dim3(1), dim3(1024), 0, stream, nb, sums);
   if (exclusive)
-    hipLaunchKernelGGL(scan_apply_kernel<true>, dim3(nb), dim3(SCAN_THREADS), 0, stream, n, in, sums, out, total_out);
+    hipLaunchKernelGGL((scan_apply_kernel<true, T>), dim3(nb), dim3(SCAN_THREADS), 0, stream, n, in, sums, out, total_out);
   else
-    hipLaunchKernelGGL(scan_apply_kernel<false>, dim3(nb), dim3(SCAN_THREADS), 0, stream, n, in, sums, out, total_out);
+    hipLaunchKernelGGL((scan_apply_kernel<false, T>), dim3(nb), dim3(SCAN_THREADS), 0, stream, n, in, sums, out, total_out);
   return 0;
 }
 
@@ -226,6 +228,11 @@ int launch_inclusive_sum(int64_t n, const uint32_t* in, uint32_t* out, void* tem
 }
 
 int launch_exclusive_sum(int64_t n, const uint32_t* in, uint32_t* out, void* temp, hipStream_t stream) {
+  return scan_impl(n, in, out, temp, true, nullptr, stream);
+}
+
+// exclusive ranks of the set bytes of a 0/1 mask
+int launch_exclusive_sum_u8(int64_t n, const uint8_t* in, uint32_t* out, void* temp, hipStream_t stream) {
   return scan_impl(n, in, out, temp, true, nullptr, stream);
 }
 

@@ -48,6 +48,7 @@ int launch_mark_visible(int P, const float* means, const float* V, uint8_t* pres
 int launch_tile_count(int P, int W, int H, const int* radii, const float* means2D, const uint8_t* compute_locally,
                       uint32_t* tiles_touched, hipStream_t stream);
 size_t scan_temp_bytes(int64_t n);
+int launch_exclusive_sum_u8(int64_t n, const uint8_t* in, uint32_t* out, void* temp, hipStream_t stream);
 // total_out, when given, is a host-visible word that receives the grand total as well
 int launch_inclusive_sum(int64_t n, const uint32_t* in, uint32_t* out, void* temp, hipStream_t stream,
                          uint32_t* total_out = nullptr);
@@ -57,6 +58,11 @@ int launch_duplicate_with_keys(int P, int W, int H, const float* means2D, const 
                                uint64_t* keys, uint32_t* values, uint32_t* emission /*optional*/,
                                hipStream_t stream);
 int launch_gather_u32(int64_t n, const uint32_t* index, const uint32_t* table, uint32_t* out, hipStream_t stream);
+size_t train_stats_temp_bytes(long long A, long long Vk);
+int launch_train_stats(long long A, int k, long long Vk, long long M, const uint8_t* visible,
+                       const uint8_t* selected, const uint8_t* update_filter, const float* grad, int grad_stride,
+                       const float* opacity, float* opacity_accum, float* anchor_demon, float* grad_accum,
+                       float* denom, void* temp, hipStream_t stream);
 constexpr int ADAM_MAX_TENSORS = 24;  // tensors per launch (more are split over several launches)
 int launch_adam(int count, float* const* params, const float* const* grads, float* const* exp_avg,
                 float* const* exp_avg_sq, const long long* sizes, const double* lrs, const int* steps, double beta1,

@@ -160,6 +160,24 @@ int gs_all_map_backward(int P, const float* means3D, const float* scales, const 
                         const float* viewmatrix, const float* campos, const float* dL_dall_map,
                         float* dL_dmeans3D, float* dL_drotations, gs_stream_t stream);
 
+/* Replaces the body of GaussianModel.training_statis (scene/gaussian_model.py:1181-1205), the per-view
+ * update of the densification statistics.  num_anchors anchors with n_offsets offsets each;
+ * anchor_visible_mask u8[num_anchors]; offset_selection_mask u8[num_candidates] and opacity
+ * f32[num_candidates] over the candidates of the visible anchors in anchor order (num_candidates =
+ * visible anchors x n_offsets); update_filter u8[num_selected] and viewspace_grad f32[num_selected][grad_stride]
+ * (columns 0 and 1 are used) over the selected candidates in order.  Updated in place:
+ * opacity_accum f32[num_anchors], anchor_demon f32[num_anchors], offset_gradient_accum and offset_denom
+ * f32[num_anchors*n_offsets].  Masks are bytes holding 0 or 1 (torch.bool).  Indices that the masks would
+ * send past num_candidates / num_selected (inconsistent inputs) are ignored rather than read.
+ * workspace: gs_training_stats_workspace_bytes(num_anchors, num_candidates) bytes. */
+size_t gs_training_stats_workspace_bytes(int64_t num_anchors, int64_t num_candidates);
+int gs_training_stats(int64_t num_anchors, int n_offsets, int64_t num_candidates, int64_t num_selected,
+                      const uint8_t* anchor_visible_mask, const uint8_t* offset_selection_mask,
+                      const uint8_t* update_filter, const float* viewspace_grad, int grad_stride,
+                      const float* opacity, float* opacity_accum, float* anchor_demon,
+                      float* offset_gradient_accum, float* offset_denom, void* workspace, size_t workspace_bytes,
+                      gs_stream_t stream);
+
 /* Replaces optimizer.step() of the reference's torch.optim.Adam(lr=0.0, eps=1e-15) with per-group learning
  * rates (scene/gaussian_model.py:574, stepped at train_internal.py:404-417) for `count` tensors in one
  * launch: update rule of torch 2.0.0 with betas (beta1, beta2), no weight decay, no amsgrad.

@@ -308,6 +308,36 @@ def all_map_bwd(means3D, scales, rotations, viewmatrix, campos, grad_out):
     return dm, dq
 
 
+def training_stats(opacity_accum, anchor_demon, grad_accum, denom, k, grad, opacity, update_filter,
+                   offset_selection_mask, anchor_visible_mask):
+    """GaussianModel.training_statis (scene/gaussian_model.py:1181-1205) with the mask gathers and scatters
+    written out as ranks: returns the four updated accumulators (flattened float32)."""
+    oa, ad = _f32(opacity_accum).ravel().copy(), _f32(anchor_demon).ravel().copy()
+    ga, dn = _f32(grad_accum).ravel().copy(), _f32(denom).ravel().copy()
+    vis = np.asarray(anchor_visible_mask).astype(bool).ravel()
+    sel = np.asarray(offset_selection_mask).astype(bool).ravel()
+    flt = np.asarray(update_filter).astype(bool).ravel()
+    op, g = _f32(opacity).ravel(), _f32(grad)
+    rank_vis = np.cumsum(vis) - vis      # exclusive count of visible anchors
+    rank_sel = np.cumsum(sel) - sel      # exclusive count of selected candidates
+    for a in np.nonzero(vis)[0]:
+        first = int(rank_vis[a]) * k
+        s = np.float32(0)
+        for j in range(k):
+            o = op[first + j]
+            s = np.float32(s + (np.float32(0) if o < 0 else o))    # :1183-1187
+        oa[a] += s
+        ad[a] += np.float32(1)                                       # :1190
+        for j in range(k):
+            i = first + j
+            if sel[i]:                                               # combined_mask[anchor_visible] = offset_selection
+                r = int(rank_sel[i])
+                if flt[r]:                                           # combined_mask[temp_mask] = update_filter
+                    ga[a * k + j] += np.sqrt(g[r, 0] * g[r, 0] + g[r, 1] * g[r, 1])   # :1203-1204
+                    dn[a * k + j] += np.float32(1)                                     # :1205
+    return oa, ad, ga, dn
+
+
 def adam_step(param, grad, exp_avg, exp_avg_sq, lr, step, beta1=0.9, beta2=0.999, eps=1e-15, grad_scale=1.0):
     """One torch.optim.Adam update (torch 2.0.0 rule, no weight decay / amsgrad; the optimizer of
     scene/gaussian_model.py:574) in float32 numpy, returning new (param, exp_avg, exp_avg_sq).  Bias corrections

@@ -546,3 +546,49 @@ def test_adam_step_matches_torch_optim_adam(orc):
     a = orc.adam_step(ps[0].numpy(), grads[0].numpy(), mine[0][1], mine[0][2], 1e-3, 7, grad_scale=0.25)
     b = orc.adam_step(ps[0].numpy(), grads[0].numpy() * np.float32(0.25), mine[0][1], mine[0][2], 1e-3, 7)
     assert all(np.array_equal(x, y) for x, y in zip(a, b))
+
+
+# ------------------------------------------------- densification statistics --
+
+def _stats_case(A=300, k=5, seed=0, p_vis=0.6, p_sel=0.7, p_flt=0.8):
+    gen = torch.Generator().manual_seed(seed)
+    vis = torch.rand(A, generator=gen) < p_vis
+    V = int(vis.sum())
+    sel = torch.rand(V * k, generator=gen) < p_sel
+    S = int(sel.sum())
+    flt = torch.rand(S, generator=gen) < p_flt
+    grad = torch.randn(S, 3, generator=gen)
+    opacity = torch.randn(V * k, 1, generator=gen)
+    acc = [torch.rand(A, 1, generator=gen), torch.rand(A, 1, generator=gen).round(),
+           torch.rand(A * k, 1, generator=gen), torch.rand(A * k, 1, generator=gen).round()]
+    return vis, sel, flt, grad, opacity, acc
+
+
+def _stats_by_mask_indexing(acc, k, grad, opacity, flt, sel, vis):
+    """The same update through torch's boolean-mask gathers and scatters (library semantics of x[mask] = y)."""
+    oa, ad, ga, dn = [t.clone() for t in acc]
+    temp = opacity.clone().view(-1)
+    temp[temp < 0] = 0
+    oa[vis] += temp.view(-1, k).sum(dim=1, keepdim=True)
+    ad[vis] += 1
+    vis_rep = vis.unsqueeze(1).repeat(1, k).view(-1)
+    combined = torch.zeros(ga.shape[0], dtype=torch.bool)
+    combined[vis_rep] = sel
+    temp_mask = combined.clone()
+    combined[temp_mask] = flt
+    ga[combined] += torch.norm(grad[flt, :2], dim=-1, keepdim=True)
+    dn[combined] += 1
+    return oa, ad, ga, dn
+
+
+@pytest.mark.parametrize("seed,p", [(0, (0.6, 0.7, 0.8)), (1, (1.0, 1.0, 1.0)), (2, (0.05, 0.3, 0.5)), (3, (0.5, 0.0, 0.5))])
+def test_training_stats_matches_mask_indexing(orc, seed, p):
+    vis, sel, flt, grad, opacity, acc = _stats_case(seed=seed, p_vis=p[0], p_sel=p[1], p_flt=p[2])
+    ref = _stats_by_mask_indexing(acc, 5, grad, opacity, flt, sel, vis)
+    got = orc.training_stats(acc[0].numpy(), acc[1].numpy(), acc[2].numpy(), acc[3].numpy(), 5, grad.numpy(),
+                             opacity.numpy(), flt.numpy(), sel.numpy(), vis.numpy())
+    for g, r in zip(got, ref):
+        assert np.allclose(g, r.numpy().ravel(), rtol=1e-6, atol=1e-7)
+    # counters move by whole numbers, and only where the chain of masks says so
+    assert np.array_equal(got[1] - acc[1].numpy().ravel(), vis.numpy().astype(np.float32))
+    assert int((got[3] - acc[3].numpy().ravel()).sum()) == int(flt.sum())
