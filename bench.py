@@ -184,10 +184,45 @@ def main():
     torch.cuda._sleep(int(4e7))
     for _ in range(args.steps):
         gs_densify.training_statis(s_acc[0], s_acc[1], s_acc[2], s_acc[3], k_s, s_grad, s_op, s_flt, s_sel, s_vis)
+    # the masked L1 + SSIM loss maps on the rendered image, forward and backward
+    import gs_loss
+    gt = torch.rand(3, H, W, device=dev)
+    pm = torch.rand(H, W, device=dev) < 0.9
+    img_l = torch.rand(3, H, W, device=dev, requires_grad=True)
+    torch.cuda._sleep(int(4e7))
+    for _ in range(args.steps):
+        img_l.grad = None
+        l1m, ssm = gs_loss.pixelwise_l1_ssim_with_mask(img_l, gt, pm)
+        torch.autograd.backward([l1m, ssm], [gt, gt])
     torch.cuda.synchronize()
     gn.stage_timing(False)
     stages = gn.stage_timing_collect()
     ms_per_step_instrumented = (t3 - t2) * 1e3 / args.steps
+    # the reference's conv2d formulation of the same maps, forward + backward, for reference
+    import math
+    import torch.nn.functional as F
+    gwin = torch.Tensor([math.exp(-((x - 5) ** 2) / float(2 * 1.5 ** 2)) for x in range(11)])
+    gwin = (gwin / gwin.sum()).unsqueeze(1)
+    win2 = gwin.mm(gwin.t()).float().unsqueeze(0).unsqueeze(0).expand(3, 1, 11, 11).contiguous().to(dev)
+    torch_ssim_ms = []
+    for _ in range(5):
+        img_l.grad = None
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        ev0.record()
+        mu1 = F.conv2d(img_l, win2, padding=5, groups=3)
+        mu2 = F.conv2d(gt, win2, padding=5, groups=3)
+        mu1_sq, mu2_sq, mu12 = mu1.pow(2), mu2.pow(2), mu1 * mu2
+        sg1 = F.conv2d(img_l * img_l, win2, padding=5, groups=3) - mu1_sq
+        sg2 = F.conv2d(gt * gt, win2, padding=5, groups=3) - mu2_sq
+        sg12 = F.conv2d(img_l * gt, win2, padding=5, groups=3) - mu12
+        smap = ((2 * mu12 + 0.01 ** 2) * (2 * sg12 + 0.03 ** 2)) / ((mu1_sq + mu2_sq + 0.01 ** 2) * (sg1 + sg2 + 0.03 ** 2))
+        smap = smap * pm.unsqueeze(0)
+        lmap = torch.abs(img_l - gt) * pm.unsqueeze(0)
+        torch.autograd.backward([lmap, smap], [gt, gt])
+        ev1.record()
+        torch.cuda.synchronize()
+        torch_ssim_ms.append(ev0.elapsed_time(ev1))
+    del gt, pm, img_l, l1m, ssm
     # the torch statements training_statis consists of, for reference
     torch_stats_ms = []
     for _ in range(5):
@@ -241,6 +276,10 @@ def main():
             nbytes = BYTES_PER_INSTANCE[name] * R
         elif name == "duplicate_with_keys":
             nbytes = 20 * P + 12 * R
+        elif name == "ssim_l1_fwd":
+            nbytes = (8 + 8 + 12) * 3 * H * W + H * W  # two images in, two maps + three derivative maps out, mask
+        elif name == "ssim_l1_bwd":
+            nbytes = (8 + 8 + 12 + 4) * 3 * H * W + H * W  # images, two upstream maps, three derivative maps in; one out
         elif name == "training_stats":
             nbytes = stats_bytes  # masks, opacities, gradient rows and the read-modify-write of the touched accumulators
         elif name == "adam_step":
@@ -274,6 +313,7 @@ def main():
         "roofline": roofline,
         "ms_per_step_with_stage_events": round(ms_per_step_instrumented, 4),
         "stages": stage_report,
+        "ssim_l1_torch_reference_ms": round(sorted(torch_ssim_ms)[len(torch_ssim_ms) // 2], 4),
         "training_stats_torch_reference_ms": round(sorted(torch_stats_ms)[len(torch_stats_ms) // 2], 4),
         "all_map_torch_reference_ms": round(sorted(torch_am_ms)[len(torch_am_ms) // 2], 4),
     }

@@ -562,6 +562,39 @@ size_t gs_render_backward_workspace_bytes(int R) { return (size_t)(R > 0 ? R : 1
 
 size_t gs_knn_workspace_bytes(int P) { return knn_temp_bytes(P) + 256; }
 
+int gs_ssim_l1_forward(int channels, int height, int width, const float* img1, const float* img2,
+                       const uint8_t* pixel_mask, float* l1_map, float* ssim_map, float* d_mu, float* d_xx,
+                       float* d_xy, gs_stream_t stream) {
+  GS_REQUIRE(channels >= 0 && height >= 0 && width >= 0, "gs_ssim_l1_forward: negative size");
+  if (channels == 0 || height == 0 || width == 0) return 0;
+  GS_REQUIRE(channels <= 65535, "gs_ssim_l1_forward: too many channels");
+  GS_REQUIRE(img1 && img2 && l1_map && ssim_map, "gs_ssim_l1_forward: null pointer");
+  GS_REQUIRE((d_mu && d_xx && d_xy) || (!d_mu && !d_xx && !d_xy),
+             "gs_ssim_l1_forward: pass all three derivative maps or none");
+  {
+    StageScope _t("ssim_l1_fwd", (hipStream_t)stream);
+    launch_ssim_l1_fwd(channels, height, width, img1, img2, pixel_mask, l1_map, ssim_map, d_mu, d_xx, d_xy,
+                       (hipStream_t)stream);
+  }
+  return check_launch("ssim_l1_forward", (hipStream_t)stream, false);
+}
+
+int gs_ssim_l1_backward(int channels, int height, int width, const float* img1, const float* img2,
+                        const uint8_t* pixel_mask, const float* dL_dl1_map, const float* dL_dssim_map,
+                        const float* d_mu, const float* d_xx, const float* d_xy, float* dL_dimg1,
+                        gs_stream_t stream) {
+  GS_REQUIRE(channels >= 0 && height >= 0 && width >= 0, "gs_ssim_l1_backward: negative size");
+  if (channels == 0 || height == 0 || width == 0) return 0;
+  GS_REQUIRE(channels <= 65535, "gs_ssim_l1_backward: too many channels");
+  GS_REQUIRE(img1 && img2 && d_mu && d_xx && d_xy && dL_dimg1, "gs_ssim_l1_backward: null pointer");
+  {
+    StageScope _t("ssim_l1_bwd", (hipStream_t)stream);
+    launch_ssim_l1_bwd(channels, height, width, img1, img2, pixel_mask, dL_dl1_map, dL_dssim_map, d_mu, d_xx, d_xy,
+                       dL_dimg1, (hipStream_t)stream);
+  }
+  return check_launch("ssim_l1_backward", (hipStream_t)stream, false);
+}
+
 size_t gs_training_stats_workspace_bytes(int64_t num_anchors, int64_t num_candidates) {
   return train_stats_temp_bytes(num_anchors, num_candidates) + 256;
 }

@@ -58,6 +58,11 @@ int launch_duplicate_with_keys(int P, int W, int H, const float* means2D, const 
                                uint64_t* keys, uint32_t* values, uint32_t* emission /*optional*/,
                                hipStream_t stream);
 int launch_gather_u32(int64_t n, const uint32_t* index, const uint32_t* table, uint32_t* out, hipStream_t stream);
+int launch_ssim_l1_fwd(int C, int H, int W, const float* img1, const float* img2, const uint8_t* mask,
+                       float* l1_map, float* ssim_map, float* d_mu, float* d_xx, float* d_xy, hipStream_t stream);
+int launch_ssim_l1_bwd(int C, int H, int W, const float* img1, const float* img2, const uint8_t* mask,
+                       const float* g_l1, const float* g_ssim, const float* d_mu, const float* d_xx,
+                       const float* d_xy, float* dimg1, hipStream_t stream);
 size_t train_stats_temp_bytes(long long A, long long Vk);
 int launch_train_stats(long long A, int k, long long Vk, long long M, const uint8_t* visible,
                        const uint8_t* selected, const uint8_t* update_filter, const float* grad, int grad_stride,

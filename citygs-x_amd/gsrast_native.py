@@ -35,6 +35,8 @@ _SIGNATURES = {
                           [_vp] * 16 + [_i, _i, C.POINTER(_i), C.POINTER(_f), _vp]),
     "gs_render_backward_workspace_bytes": (_sz, [_i]),
     "gs_render_backward": (_i, [_i, _i, _vp, _i, _i, _f, _f] + [_vp] * 17 + [_i, _i, _vp, _sz, C.POINTER(_f), _vp]),
+    "gs_ssim_l1_forward": (_i, [_i, _i, _i] + [_vp] * 9),
+    "gs_ssim_l1_backward": (_i, [_i, _i, _i] + [_vp] * 10),
     "gs_training_stats_workspace_bytes": (_sz, [_i64, _i64]),
     "gs_training_stats": (_i, [_i64, _i, _i64, _i64, _vp, _vp, _vp, _vp, _i] + [_vp] * 6 + [_sz, _vp]),
     "gs_adam_step": (_i, [_i] + [_vp] * 7 + [C.c_double, C.c_double, C.c_double, _f, _vp]),

@@ -160,6 +160,21 @@ int gs_all_map_backward(int P, const float* means3D, const float* scales, const 
                         const float* viewmatrix, const float* campos, const float* dL_dall_map,
                         float* dL_dmeans3D, float* dL_drotations, gs_stream_t stream);
 
+/* Replaces pixelwise_l1_with_mask and pixelwise_ssim_with_mask (utils/loss_utils.py:88-132, 11x11 Gaussian
+ * window of create_window :27-43, zero padding; called at gaussian_renderer/loss_distribution.py:267-279).
+ * img1, img2 and the maps are (channels, height, width) float32; pixel_mask u8[height*width] (0/1) or NULL
+ * for all ones.  l1_map = |img1-img2| * mask, ssim_map = SSIM * mask.  d_mu / d_xx / d_xy (each the size
+ * of a map, or all three NULL when no backward pass will follow) receive the partial derivatives the
+ * backward entry needs.  gs_ssim_l1_backward writes dL/dimg1 for upstream gradients dL_dl1_map and
+ * dL_dssim_map (either may be NULL = zero); img2 is treated as constant (it is the ground truth). */
+int gs_ssim_l1_forward(int channels, int height, int width, const float* img1, const float* img2,
+                       const uint8_t* pixel_mask, float* l1_map, float* ssim_map, float* d_mu, float* d_xx,
+                       float* d_xy, gs_stream_t stream);
+int gs_ssim_l1_backward(int channels, int height, int width, const float* img1, const float* img2,
+                        const uint8_t* pixel_mask, const float* dL_dl1_map, const float* dL_dssim_map,
+                        const float* d_mu, const float* d_xx, const float* d_xy, float* dL_dimg1,
+                        gs_stream_t stream);
+
 /* Replaces the body of GaussianModel.training_statis (scene/gaussian_model.py:1181-1205), the per-view
  * update of the densification statistics.  num_anchors anchors with n_offsets offsets each;
  * anchor_visible_mask u8[num_anchors]; offset_selection_mask u8[num_candidates] and opacity

@@ -1176,4 +1176,117 @@ void oracle_all_map_bwd(int P, const float* means, const float* scales, const fl
   }
 }
 
+
+// ---------------------------------------------------------------------------
+// Per-pixel masked L1 and SSIM maps of the training loss: pixelwise_l1_with_mask and
+// pixelwise_ssim_with_mask (utils/loss_utils.py:88-132), window from create_window (:27-43): an 11x11
+// Gaussian (sigma 1.5) applied per channel with zero padding of 5.  `win` holds the 11 normalised 1-D
+// weights as float32 (the caller builds them as gaussian() does); the 2-D window is their float32 outer
+// product, as torch's mm gives it.  Convolutions are summed row by row, left to right, in float32; torch's
+// conv2d leaves that order open, so agreement with torch is to rounding.
+static void ssim_stats(int H, int W, const float* a, const float* b, const float* w2, int y, int x, float* st) {
+  float m1 = 0.f, m2 = 0.f, e11 = 0.f, e22 = 0.f, e12 = 0.f;
+  for (int dy = -5; dy <= 5; dy++) {
+    const int yy = y + dy;
+    if (yy < 0 || yy >= H) continue;
+    for (int dx = -5; dx <= 5; dx++) {
+      const int xx = x + dx;
+      if (xx < 0 || xx >= W) continue;
+      const float wt = w2[(dy + 5) * 11 + (dx + 5)];
+      const float p = a[(size_t)yy * W + xx], q = b[(size_t)yy * W + xx];
+      m1 += wt * p;
+      m2 += wt * q;
+      e11 += wt * (p * p);
+      e22 += wt * (q * q);
+      e12 += wt * (p * q);
+    }
+  }
+  st[0] = m1; st[1] = m2; st[2] = e11; st[3] = e22; st[4] = e12;
+}
+
+void oracle_ssim_l1_fwd(int C, int H, int W, const float* img1, const float* img2, const uint8_t* mask,
+                        const float* win, float* l1_map, float* ssim_map) {
+  float w2[121];
+  for (int i = 0; i < 11; i++)
+    for (int j = 0; j < 11; j++) w2[i * 11 + j] = win[i] * win[j];
+  const float C1 = (float)(0.01 * 0.01), C2 = (float)(0.03 * 0.03);
+#pragma omp parallel for collapse(2) schedule(static)
+  for (int c = 0; c < C; c++)
+    for (int y = 0; y < H; y++) {
+      const float* a = img1 + (size_t)c * H * W;
+      const float* b = img2 + (size_t)c * H * W;
+      for (int x = 0; x < W; x++) {
+        float st[5];
+        ssim_stats(H, W, a, b, w2, y, x, st);
+        const float mu1 = st[0], mu2 = st[1];
+        const float mu1_sq = mu1 * mu1, mu2_sq = mu2 * mu2, mu12 = mu1 * mu2;
+        const float s1 = st[2] - mu1_sq, s2 = st[3] - mu2_sq, s12 = st[4] - mu12;
+        const float v = ((2 * mu12 + C1) * (2 * s12 + C2)) / ((mu1_sq + mu2_sq + C1) * (s1 + s2 + C2));
+        const float mk = mask ? (float)(mask[(size_t)y * W + x] != 0) : 1.0f;
+        const size_t o = ((size_t)c * H + y) * W + x;
+        ssim_map[o] = v * mk;
+        l1_map[o] = fabsf(a[(size_t)y * W + x] - b[(size_t)y * W + x]) * mk;
+      }
+    }
+}
+
+// d(sum(g_l1 * l1_map) + sum(g_ssim * ssim_map)) / d img1, by the adjoint of the statements above: the three
+// partial derivatives of the SSIM value with respect to the window means of x, x*x and x*y, weighted by
+// mask and upstream gradient, are spread back through the (symmetric) window.
+void oracle_ssim_l1_bwd(int C, int H, int W, const float* img1, const float* img2, const uint8_t* mask,
+                        const float* win, const float* g_l1, const float* g_ssim, float* dimg1) {
+  float w2[121];
+  for (int i = 0; i < 11; i++)
+    for (int j = 0; j < 11; j++) w2[i * 11 + j] = win[i] * win[j];
+  const float C1 = (float)(0.01 * 0.01), C2 = (float)(0.03 * 0.03);
+  const size_t HW = (size_t)H * W;
+  std::vector<float> d_mu((size_t)C * HW), d_e11((size_t)C * HW), d_e12((size_t)C * HW);
+#pragma omp parallel for collapse(2) schedule(static)
+  for (int c = 0; c < C; c++)
+    for (int y = 0; y < H; y++) {
+      const float* a = img1 + (size_t)c * HW;
+      const float* b = img2 + (size_t)c * HW;
+      for (int x = 0; x < W; x++) {
+        float st[5];
+        ssim_stats(H, W, a, b, w2, y, x, st);
+        const float mu1 = st[0], mu2 = st[1];
+        const float A1 = 2 * (mu1 * mu2) + C1, B1 = (mu1 * mu1 + mu2 * mu2) + C1;
+        const float s12 = st[4] - mu1 * mu2;
+        const float A2 = 2 * s12 + C2, B2 = ((st[2] - mu1 * mu1) + (st[3] - mu2 * mu2)) + C2;
+        const float S = (A1 * A2) / (B1 * B2);
+        const float mk = mask ? (float)(mask[(size_t)y * W + x] != 0) : 1.0f;
+        const size_t o = (size_t)c * HW + (size_t)y * W + x;
+        const float gw = g_ssim[o] * mk;
+        d_mu[o] = gw * ((2 * mu2 * (A2 - A1)) / (B1 * B2) - S * (2 * mu1 / B1) + S * (2 * mu1 / B2));
+        d_e11[o] = gw * (-S / B2);
+        d_e12[o] = gw * (2 * A1 / (B1 * B2));
+      }
+    }
+#pragma omp parallel for collapse(2) schedule(static)
+  for (int c = 0; c < C; c++)
+    for (int y = 0; y < H; y++)
+      for (int x = 0; x < W; x++) {
+        float cm = 0.f, c11 = 0.f, c12 = 0.f;
+        for (int dy = -5; dy <= 5; dy++) {
+          const int yy = y + dy;
+          if (yy < 0 || yy >= H) continue;
+          for (int dx = -5; dx <= 5; dx++) {
+            const int xx = x + dx;
+            if (xx < 0 || xx >= W) continue;
+            const float wt = w2[(dy + 5) * 11 + (dx + 5)];
+            const size_t q = (size_t)c * HW + (size_t)yy * W + xx;
+            cm += wt * d_mu[q];
+            c11 += wt * d_e11[q];
+            c12 += wt * d_e12[q];
+          }
+        }
+        const size_t o = (size_t)c * HW + (size_t)y * W + x;
+        const float p = img1[o], q2 = img2[o];
+        const float mk = mask ? (float)(mask[(size_t)y * W + x] != 0) : 1.0f;
+        const float d = p - q2;
+        const float sg = d > 0.f ? 1.0f : (d < 0.f ? -1.0f : 0.0f);
+        dimg1[o] = ((cm + 2 * p * c11) + q2 * c12) + g_l1[o] * mk * sg;
+      }
+}
+
 }  // extern "C"

@@ -308,6 +308,35 @@ def all_map_bwd(means3D, scales, rotations, viewmatrix, campos, grad_out):
     return dm, dq
 
 
+def ssim_window():
+    """The 11 normalised 1-D weights of create_window (utils/loss_utils.py:27-43) as float32: exp in Python
+    floats, stored as float32, divided by their float32 sum."""
+    import math
+    g = np.array([math.exp(-((x - 11 // 2) ** 2) / float(2 * 1.5 ** 2)) for x in range(11)], np.float32)
+    return (g / g.sum(dtype=np.float32)).astype(np.float32)
+
+
+def ssim_l1_fwd(img1, img2, mask=None):
+    """pixelwise_l1_with_mask, pixelwise_ssim_with_mask (utils/loss_utils.py:88-132): (l1_map, ssim_map)."""
+    img1, img2 = _f32(img1), _f32(img2)
+    Cn, H, W = img1.shape
+    m = None if mask is None else _u8(mask).reshape(H, W)
+    l1, ss = np.zeros_like(img1), np.zeros_like(img1)
+    lib().oracle_ssim_l1_fwd(C.c_int(Cn), C.c_int(H), C.c_int(W), _p(img1), _p(img2), _p(m) if m is not None else None,
+                             _p(ssim_window()), _p(l1), _p(ss))
+    return l1, ss
+
+
+def ssim_l1_bwd(img1, img2, mask, g_l1, g_ssim):
+    img1, img2, g_l1, g_ssim = _f32(img1), _f32(img2), _f32(g_l1), _f32(g_ssim)
+    Cn, H, W = img1.shape
+    m = None if mask is None else _u8(mask).reshape(H, W)
+    d = np.zeros_like(img1)
+    lib().oracle_ssim_l1_bwd(C.c_int(Cn), C.c_int(H), C.c_int(W), _p(img1), _p(img2),
+                             _p(m) if m is not None else None, _p(ssim_window()), _p(g_l1), _p(g_ssim), _p(d))
+    return d
+
+
 def training_stats(opacity_accum, anchor_demon, grad_accum, denom, k, grad, opacity, update_filter,
                    offset_selection_mask, anchor_visible_mask):
     """GaussianModel.training_statis (scene/gaussian_model.py:1181-1205) with the mask gathers and scatters

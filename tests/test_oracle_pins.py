@@ -592,3 +592,58 @@ def test_training_stats_matches_mask_indexing(orc, seed, p):
     # counters move by whole numbers, and only where the chain of masks says so
     assert np.array_equal(got[1] - acc[1].numpy().ravel(), vis.numpy().astype(np.float32))
     assert int((got[3] - acc[3].numpy().ravel()).sum()) == int(flt.sum())
+
+
+# ------------------------------------------------------------- L1 + SSIM --
+
+def _ssim_ref64(a, b, mask, window):
+    """The reference statements (utils/loss_utils.py:97-132) with torch's conv2d in float64."""
+    import torch.nn.functional as F
+    Cn = a.shape[0]
+    w1 = torch.tensor(window).double()
+    w = (w1[:, None] @ w1[None, :]).expand(Cn, 1, 11, 11).contiguous()
+    conv = lambda t: F.conv2d(t[None], w, padding=5, groups=Cn)[0]
+    mu1, mu2 = conv(a), conv(b)
+    s1, s2, s12 = conv(a * a) - mu1 ** 2, conv(b * b) - mu2 ** 2, conv(a * b) - mu1 * mu2
+    m = ((2 * mu1 * mu2 + 0.01 ** 2) * (2 * s12 + 0.03 ** 2)) / ((mu1 ** 2 + mu2 ** 2 + 0.01 ** 2) * (s1 + s2 + 0.03 ** 2))
+    return torch.abs(a - b) * mask[None], m * mask[None]
+
+
+def test_ssim_window_is_create_window(orc):
+    w = orc.ssim_window()
+    assert w.dtype == np.float32 and w.shape == (11,)
+    assert abs(float(w.sum()) - 1.0) < 1e-6 and np.array_equal(w, w[::-1]) and w.argmax() == 5
+    assert abs(w[5] / w[4] - np.exp(1.0 / 4.5)) < 1e-6  # sigma = 1.5
+
+
+def test_ssim_l1_forward_and_backward_match_float64_torch(orc):
+    gen = torch.Generator().manual_seed(0)
+    Cn, H, W = 3, 37, 52  # not multiples of the window or of any block size; borders matter
+    a = torch.rand(Cn, H, W, generator=gen)
+    b = (a + 0.2 * torch.randn(Cn, H, W, generator=gen)).clamp(0, 1)
+    mask = torch.rand(H, W, generator=gen) < 0.7
+    ad = a.double().requires_grad_(True)
+    l1r, sr = _ssim_ref64(ad, b.double(), mask, orc.ssim_window())
+    l1, ss = orc.ssim_l1_fwd(a.numpy(), b.numpy(), mask.numpy())
+    assert np.abs(l1 - l1r.detach().numpy()).max() <= 1e-7
+    assert np.abs(ss - sr.detach().numpy()).max() <= 2e-5
+    g1, g2 = torch.randn(Cn, H, W, generator=gen), torch.randn(Cn, H, W, generator=gen)
+    ((l1r * g1.double()).sum() + (sr * g2.double()).sum()).backward()
+    d = orc.ssim_l1_bwd(a.numpy(), b.numpy(), mask.numpy(), g1.numpy(), g2.numpy())
+    assert np.linalg.norm(d - ad.grad.numpy()) / np.linalg.norm(ad.grad.numpy()) <= 1e-5
+
+
+def test_ssim_closed_forms(orc):
+    H, W = 30, 40
+    a = torch.rand(3, H, W, generator=torch.Generator().manual_seed(1)).numpy()
+    l1, ss = orc.ssim_l1_fwd(a, a, None)
+    assert np.all(l1 == 0) and np.all(ss == 1.0)         # an image against itself
+    ca, cb = np.full((1, H, W), 0.3, np.float32), np.full((1, H, W), 0.6, np.float32)
+    l1, ss = orc.ssim_l1_fwd(ca, cb, None)
+    assert np.allclose(l1, 0.3, atol=1e-7)
+    want = (2 * 0.3 * 0.6 + 1e-4) / (0.3 ** 2 + 0.6 ** 2 + 1e-4)   # constants: no variance, full window inside
+    assert np.abs(ss[0, 5:-5, 5:-5] - want).max() <= 1e-4
+    m = np.zeros((H, W), bool)
+    m[3:9, 4:20] = True
+    l1m, ssm = orc.ssim_l1_fwd(ca, cb, m)
+    assert np.all(ssm[0][~m] == 0) and np.all(l1m[0][~m] == 0) and np.array_equal(ssm[0][m], ss[0][m])
