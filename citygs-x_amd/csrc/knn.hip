@@ -14,11 +14,13 @@ namespace gs {
 namespace {
 
 constexpr int KNN_BOX = 1024;  // simple-knn/simple_knn.cu:12
+constexpr int KNN_GROUP = 64;  // boxes per group (one group test replaces this many box tests)
+constexpr int KNN_LEAF = 64;   // points per leaf box inside a box (one leaf test replaces this many distances)
 constexpr int MM_BLOCKS = 512;
 constexpr int MM_THREADS = 256;
 
 struct KnnLayout {
-  size_t partial, minmax, codes_a, codes_b, idx_a, idx_b, sorted_pts, boxes, sort_temp, total;
+  size_t partial, minmax, codes_a, codes_b, idx_a, idx_b, sorted_pts, boxes, groups, leaves, sort_temp, total;
 };
 
 KnnLayout knn_layout(int P) {
@@ -39,6 +41,8 @@ KnnLayout knn_layout(int P) {
   L.idx_b = take(sizeof(uint32_t) * n);
   L.sorted_pts = take(sizeof(float4) * n);
   L.boxes = take(sizeof(float) * 6 * nb);
+  L.leaves = take(sizeof(float) * 6 * ((n + KNN_LEAF - 1) / KNN_LEAF));
+  L.groups = take(sizeof(float) * 6 * ((nb + KNN_GROUP - 1) / KNN_GROUP));
   L.sort_temp = take(sort_temp_bytes((int64_t)n));
   L.total = off;
   return L;
@@ -153,6 +157,65 @@ __global__ void __launch_bounds__(MM_THREADS) box_minmax_kernel(int P, const flo
   reduce6(v, s, boxes + 6 * blockIdx.x);
 }
 
+// Bounding box of every run of KNN_GROUP consecutive boxes: lets the search discard that many boxes with
+// one test.  (Not in the reference, which tests every box for every point; the result is the same set of
+// three nearest neighbours, because a group's box bounds its members' boxes from below.)
+__global__ void __launch_bounds__(GS_WAVE) box_group_kernel(int nboxes, const float* __restrict__ boxes,
+                                                            float* __restrict__ groups) {
+  const int b = blockIdx.x * KNN_GROUP + threadIdx.x;
+  float v[6] = {FLT_MAX, FLT_MAX, FLT_MAX, -FLT_MAX, -FLT_MAX, -FLT_MAX};
+  if (threadIdx.x < KNN_GROUP && b < nboxes) {
+#pragma unroll
+    for (int c = 0; c < 6; c++) v[c] = boxes[6 * b + c];
+  }
+#pragma unroll
+  for (int d = GS_WAVE / 2; d >= 1; d >>= 1) {
+#pragma unroll
+    for (int c = 0; c < 3; c++) {
+      v[c] = fminf(v[c], __shfl_xor(v[c], d, GS_WAVE));
+      v[3 + c] = fmaxf(v[3 + c], __shfl_xor(v[3 + c], d, GS_WAVE));
+    }
+  }
+  if (threadIdx.x == 0) {
+#pragma unroll
+    for (int c = 0; c < 6; c++) groups[6 * blockIdx.x + c] = v[c];
+  }
+}
+
+// Bounding box of every run of KNN_LEAF consecutive sorted points (one wave each): the finest level of the
+// search.  Like the groups, an addition that prunes work without changing which neighbours are found.
+__global__ void __launch_bounds__(GS_BLOCK_1D) leaf_minmax_kernel(int P, const float4* __restrict__ sorted_pts,
+                                                                  float* __restrict__ leaves) {
+  const int i = blockIdx.x * GS_BLOCK_1D + threadIdx.x;
+  float v[6] = {FLT_MAX, FLT_MAX, FLT_MAX, -FLT_MAX, -FLT_MAX, -FLT_MAX};
+  if (i < P) {
+    const float4 p = sorted_pts[i];
+    v[0] = v[3] = p.x; v[1] = v[4] = p.y; v[2] = v[5] = p.z;
+  }
+#pragma unroll
+  for (int d = GS_WAVE / 2; d >= 1; d >>= 1) {
+#pragma unroll
+    for (int c = 0; c < 3; c++) {
+      v[c] = fminf(v[c], __shfl_xor(v[c], d, GS_WAVE));
+      v[3 + c] = fmaxf(v[3 + c], __shfl_xor(v[3 + c], d, GS_WAVE));
+    }
+  }
+  const int leaf = i / KNN_LEAF;
+  if ((threadIdx.x & (GS_WAVE - 1)) == 0 && leaf * KNN_LEAF < P) {
+#pragma unroll
+    for (int c = 0; c < 6; c++) leaves[6 * (size_t)leaf + c] = v[c];
+  }
+}
+
+__device__ __forceinline__ float box_dist2(const float4& p, const float* bx) {  // simple_knn.cu:119-129
+  float diff[3] = {0.f, 0.f, 0.f};
+  const float pc[3] = {p.x, p.y, p.z};
+#pragma unroll
+  for (int c = 0; c < 3; c++)
+    if (pc[c] < bx[c] || pc[c] > bx[3 + c]) diff[c] = fminf(fabsf(pc[c] - bx[c]), fabsf(pc[c] - bx[3 + c]));
+  return (diff[0] * diff[0] + diff[1] * diff[1]) + diff[2] * diff[2];
+}
+
 __device__ __forceinline__ void update3(const float4& ref, const float4& p, float* knn) {  // simple_knn.cu:131-145
   const float dx = p.x - ref.x, dy = p.y - ref.y, dz = p.z - ref.z;
   float dist = (dx * dx + dy * dy) + dz * dz;
@@ -170,6 +233,8 @@ __device__ __forceinline__ void update3(const float4& ref, const float4& p, floa
 __global__ void __launch_bounds__(GS_BLOCK_1D) box_mean_dist_kernel(int P, const float4* __restrict__ sorted_pts,
                                                                     const uint32_t* __restrict__ idx,
                                                                     const float* __restrict__ boxes, int nboxes,
+                                                                    const float* __restrict__ groups,
+                                                                    const float* __restrict__ leaves,
                                                                     float* __restrict__ out) {
   const int k = blockIdx.x * GS_BLOCK_1D + threadIdx.x;
   if (k >= P) return;
@@ -182,19 +247,25 @@ __global__ void __launch_bounds__(GS_BLOCK_1D) box_mean_dist_kernel(int P, const
   }
   const float reject = best[2];
   best[0] = best[1] = best[2] = FLT_MAX;
-  for (int b = 0; b < nboxes; b++) {
-    const float* bx = boxes + 6 * b;
-    float diff[3] = {0.f, 0.f, 0.f};
-    const float pc[3] = {p.x, p.y, p.z};
-#pragma unroll
-    for (int c = 0; c < 3; c++)
-      if (pc[c] < bx[c] || pc[c] > bx[3 + c]) diff[c] = fminf(fabsf(pc[c] - bx[c]), fabsf(pc[c] - bx[3 + c]));
-    const float dist = (diff[0] * diff[0] + diff[1] * diff[1]) + diff[2] * diff[2];
-    if (dist > reject || dist > best[2]) continue;
-    const int e = min(P, (b + 1) * KNN_BOX);
-    for (int i = b * KNN_BOX; i < e; i++) {
-      if (i == k) continue;
-      update3(p, sorted_pts[i], best);
+  const int ngroups = (nboxes + KNN_GROUP - 1) / KNN_GROUP;
+  for (int gi = 0; gi < ngroups; gi++) {
+    // a group that is too far away holds no box that is near enough
+    const float gd = box_dist2(p, groups + 6 * gi);
+    if (gd > reject || gd > best[2]) continue;
+    const int b_end = min(nboxes, (gi + 1) * KNN_GROUP);
+    for (int b = gi * KNN_GROUP; b < b_end; b++) {
+      const float dist = box_dist2(p, boxes + 6 * b);
+      if (dist > reject || dist > best[2]) continue;
+      const int e = min(P, (b + 1) * KNN_BOX);
+      for (int l0 = b * KNN_BOX; l0 < e; l0 += KNN_LEAF) {
+        const float ld = box_dist2(p, leaves + 6 * (size_t)(l0 / KNN_LEAF));
+        if (ld > reject || ld > best[2]) continue;
+        const int le = min(e, l0 + KNN_LEAF);
+        for (int i = l0; i < le; i++) {
+          if (i == k) continue;
+          update3(p, sorted_pts[i], best);
+        }
+      }
     }
   }
   out[idx[k]] = ((best[0] + best[1]) + best[2]) / 3.0f;
@@ -216,6 +287,8 @@ int launch_knn_dist2(int P, const float* points, float* mean_dist2, void* temp, 
   uint32_t* idx_b = (uint32_t*)(base + L.idx_b);
   float4* sorted_pts = (float4*)(base + L.sorted_pts);
   float* boxes = (float*)(base + L.boxes);
+  float* groups = (float*)(base + L.groups);
+  float* leaves = (float*)(base + L.leaves);
   void* sort_temp = base + L.sort_temp;
   const int blocks = (P + GS_BLOCK_1D - 1) / GS_BLOCK_1D;
   const int nboxes = (P + KNN_BOX - 1) / KNN_BOX;
@@ -229,8 +302,11 @@ int launch_knn_dist2(int P, const float* points, float* mean_dist2, void* temp, 
   hipLaunchKernelGGL(gather_points_kernel, dim3(blocks), dim3(GS_BLOCK_1D), 0, stream, P, points, idx_sorted,
                      sorted_pts);
   hipLaunchKernelGGL(box_minmax_kernel, dim3(nboxes), dim3(MM_THREADS), 0, stream, P, sorted_pts, boxes);
+  hipLaunchKernelGGL(leaf_minmax_kernel, dim3(blocks), dim3(GS_BLOCK_1D), 0, stream, P, sorted_pts, leaves);
+  hipLaunchKernelGGL(box_group_kernel, dim3((nboxes + KNN_GROUP - 1) / KNN_GROUP), dim3(GS_WAVE), 0, stream, nboxes,
+                     boxes, groups);
   hipLaunchKernelGGL(box_mean_dist_kernel, dim3(blocks), dim3(GS_BLOCK_1D), 0, stream, P, sorted_pts, idx_sorted,
-                     boxes, nboxes, mean_dist2);
+                     boxes, nboxes, groups, leaves, mean_dist2);
   return 0;
 }
 

@@ -136,3 +136,26 @@ def test_config1_full_size(H):
     for t in pb:
         assert bool(torch.isfinite(t).all())
     assert float(pb[3][dead].abs().max()) == 0.0  # dL/dshs of culled Gaussians
+
+
+def test_knn_large_against_brute_force_on_a_sample():
+    """distCUDA2 on 3 M points; 512 of them checked against an exhaustive search done with torch."""
+    from simple_knn._C import distCUDA2
+    P = 3_000_000
+    g = torch.Generator(device=DEV).manual_seed(12)
+    pts = torch.rand(P, 3, generator=g, device=DEV) * torch.tensor([2000.0, 2000.0, 80.0], device=DEV)
+    pts[:P // 10] = pts[:P // 10] * torch.tensor([0.05, 0.05, 1.0], device=DEV)  # a dense cluster: uneven boxes
+    got = distCUDA2(pts)
+    assert got.shape == (P,) and bool(torch.isfinite(got).all()) and float(got.min()) > 0.0
+    q = torch.randint(0, P, (512,), generator=g, device=DEV)
+    best = torch.full((512, 3), float("inf"), device=DEV)
+    for s in range(0, P, 250_000):
+        blk = pts[s:s + 250_000]
+        d = blk[None, :, :] - pts[q][:, None, :]
+        d2 = (d[..., 0] * d[..., 0] + d[..., 1] * d[..., 1]) + d[..., 2] * d[..., 2]
+        own = (q[:, None] == (torch.arange(blk.shape[0], device=DEV)[None, :] + s))
+        d2 = torch.where(own, torch.full_like(d2, float("inf")), d2)
+        best = torch.cat([best, d2], dim=1).topk(3, dim=1, largest=False).values
+    want = ((best[:, 0] + best[:, 1]) + best[:, 2]) / 3.0
+    # torch may contract its multiply-adds, the search does not: equal up to the last bits of a distance
+    assert float(((got[q] - want).abs() / want).max()) <= 1e-6
