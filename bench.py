@@ -31,7 +31,9 @@ BYTES_PER_GAUSSIAN = {
     "all_map_fwd": 60,   # means 12 + scales 12 + rotations 16 in, 20 out
     "all_map_bwd": 88,   # the same 40 + 20 B of upstream gradient in, 12 + 16 out
 }
-BYTES_PER_INSTANCE = {"sort_pairs": 152, "identify_tile_ranges": 8}
+# sort: one 8 B histogram read + 5 passes (9-bit digits over the 44 key bits) x (12 B read + 12 B write)
+# tile ranges: 8 B key read, plus the gather of the sorted Gaussian ids fused into it (index, table, output: 12 B)
+BYTES_PER_INSTANCE = {"sort_pairs": 128, "identify_tile_ranges": 20}
 
 
 def parse():

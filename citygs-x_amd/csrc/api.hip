@@ -414,7 +414,10 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
   uint32_t* total_slot = acquire_total_slot();
   {
     StageScope _t("tile_count", stream);
-    launch_tile_count(P, width, height, radii, means2D, compute_locally, tiles_touched, stream);
+    // also clears the tile ranges (cudaMemset of CR/rasterizer_impl.cu:687), which nothing reads before
+    // identify_tile_ranges fills them
+    launch_tile_count(P, width, height, radii, means2D, compute_locally, tiles_touched, stream, ranges,
+                      (int64_t)2 * T);
   }
   if (check_launch("tile_count", stream, dbg)) return 1;
   {
@@ -474,13 +477,13 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
     {
       StageScope _t("sort_pairs", stream);
       if (launch_sort_pairs_u64(R, k_start, k_partner, e_start, e_partner, end_bit, sort_temp, stream)) return 1;
-      launch_gather_u32(R, emission, gauss_of_emission, point_list, stream);
     }
     if (check_launch("sort_pairs", stream, dbg)) return 1;
   }
   {
     StageScope _t("identify_tile_ranges", stream);
-    launch_tile_ranges(R, keys, T, ranges, stream);
+    // ... and gathers the Gaussian ids of the sorted instances on the way (point_list)
+    launch_tile_ranges(R, keys, T, ranges, stream, true, emission, gauss_of_emission, point_list);
   }
   if (check_launch("identify_tile_ranges", stream, dbg)) return 1;
 

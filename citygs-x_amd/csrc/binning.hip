@@ -48,8 +48,10 @@ __device__ __forceinline__ uint32_t block_exclusive_scan(uint32_t v, uint32_t* s
 __global__ void __launch_bounds__(GS_BLOCK_1D)
 tile_count_kernel(int P, uint32_t gx, uint32_t gy, const int* __restrict__ radii,
                   const float2* __restrict__ means2D, const uint8_t* __restrict__ compute_locally,
-                  uint32_t* __restrict__ tiles_touched) {
+                  uint32_t* __restrict__ tiles_touched, uint32_t* __restrict__ zero_words, int64_t zero_count) {
   const int i = blockIdx.x * GS_BLOCK_1D + threadIdx.x;
+  // optionally clears another array on the side (the tile ranges of the same call: saves a launch)
+  for (int64_t j = i; j < zero_count; j += (int64_t)gridDim.x * GS_BLOCK_1D) zero_words[j] = 0u;
   if (i >= P) return;
   uint32_t cnt = 0;
   const int r = radii[i];
@@ -174,9 +176,13 @@ __global__ void fill_u32_kernel(int64_t n, uint32_t v, uint32_t* __restrict__ p)
 
 // cuda_rasterizer/rasterizer_impl.cu:122-144.
 __global__ void __launch_bounds__(GS_BLOCK_1D)
-tile_ranges_kernel(int64_t L, const uint64_t* __restrict__ keys, uint32_t* __restrict__ ranges) {
+tile_ranges_kernel(int64_t L, const uint64_t* __restrict__ keys, uint32_t* __restrict__ ranges,
+                   const uint32_t* __restrict__ gather_index, const uint32_t* __restrict__ gather_table,
+                   uint32_t* __restrict__ gather_out) {
   const int64_t i = (int64_t)blockIdx.x * GS_BLOCK_1D + threadIdx.x;
   if (i >= L) return;
+  // optionally also: gather_out[i] = gather_table[gather_index[i]] (the sorted list of Gaussian ids)
+  if (gather_out != nullptr) gather_out[i] = gather_table[gather_index[i]];
   const uint32_t cur = (uint32_t)(keys[i] >> 32);
   if (i == 0)
     ranges[2 * cur] = 0;
@@ -193,11 +199,12 @@ tile_ranges_kernel(int64_t L, const uint64_t* __restrict__ keys, uint32_t* __res
 }  // namespace
 
 int launch_tile_count(int P, int W, int H, const int* radii, const float* means2D, const uint8_t* compute_locally,
-                      uint32_t* tiles_touched, hipStream_t stream) {
+                      uint32_t* tiles_touched, hipStream_t stream, uint32_t* zero_words, int64_t zero_count) {
   if (P <= 0) return 0;
   const uint32_t gx = (W + GS_TILE_X - 1) / GS_TILE_X, gy = (H + GS_TILE_Y - 1) / GS_TILE_Y;
   hipLaunchKernelGGL(tile_count_kernel, dim3((P + GS_BLOCK_1D - 1) / GS_BLOCK_1D), dim3(GS_BLOCK_1D), 0, stream, P,
-                     gx, gy, radii, (const float2*)means2D, compute_locally, tiles_touched);
+                     gx, gy, radii, (const float2*)means2D, compute_locally, tiles_touched, zero_words,
+                     zero_words ? zero_count : 0);
   return 0;
 }
 
@@ -254,12 +261,14 @@ int launch_gather_u32(int64_t n, const uint32_t* index, const uint32_t* table, u
   return 0;
 }
 
-int launch_tile_ranges(int64_t L, const uint64_t* keys_sorted, int T, uint32_t* ranges, hipStream_t stream) {
-  if (T > 0)
+int launch_tile_ranges(int64_t L, const uint64_t* keys_sorted, int T, uint32_t* ranges, hipStream_t stream,
+                       bool already_zero, const uint32_t* gather_index, const uint32_t* gather_table,
+                       uint32_t* gather_out) {
+  if (T > 0 && !already_zero)
     hipLaunchKernelGGL(fill_u32_kernel, dim3((2 * T + 255) / 256), dim3(256), 0, stream, (int64_t)2 * T, 0u, ranges);
   if (L > 0)
     hipLaunchKernelGGL(tile_ranges_kernel, dim3((unsigned)((L + GS_BLOCK_1D - 1) / GS_BLOCK_1D)), dim3(GS_BLOCK_1D), 0,
-                       stream, L, keys_sorted, ranges);
+                       stream, L, keys_sorted, ranges, gather_index, gather_table, gather_out);
   return 0;
 }
 

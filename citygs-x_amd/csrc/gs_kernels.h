@@ -46,7 +46,8 @@ int launch_mark_visible(int P, const float* means, const float* V, uint8_t* pres
 
 // ---- binning ----
 int launch_tile_count(int P, int W, int H, const int* radii, const float* means2D, const uint8_t* compute_locally,
-                      uint32_t* tiles_touched, hipStream_t stream);
+                      uint32_t* tiles_touched, hipStream_t stream,
+                      uint32_t* zero_words = nullptr, int64_t zero_count = 0);
 size_t scan_temp_bytes(int64_t n);
 int launch_exclusive_sum_u8(int64_t n, const uint8_t* in, uint32_t* out, void* temp, hipStream_t stream);
 // total_out, when given, is a host-visible word that receives the grand total as well
@@ -77,14 +78,18 @@ int launch_all_map_fwd(int P, const float* means, const float* scales, const flo
 int launch_all_map_bwd(int P, const float* means, const float* scales, const float* rots, const float* V,
                        const float* campos, const float* grad_out, float* dmeans, float* drots,
                        hipStream_t stream);
-int launch_tile_ranges(int64_t L, const uint64_t* keys_sorted, int T, uint32_t* ranges, hipStream_t stream);
+// already_zero: the caller cleared `ranges` itself; gather_*: also write gather_out[i] = gather_table[gather_index[i]]
+int launch_tile_ranges(int64_t L, const uint64_t* keys_sorted, int T, uint32_t* ranges, hipStream_t stream,
+                       bool already_zero = false, const uint32_t* gather_index = nullptr,
+                       const uint32_t* gather_table = nullptr, uint32_t* gather_out = nullptr);
 
 // ---- radix sort (stable, LSD, 8-bit digits) ----
 size_t sort_temp_bytes(int64_t n);
 // Sorts on key bits [0, end_bit), ping-ponging between the (a) and (b) arrays
 // starting from (a).  With an odd number of 8-bit passes the sorted result
 // lands in (b), with an even number back in (a): sort_result_in_b() tells.
-inline int sort_num_passes(int end_bit) { return (end_bit + 7) / 8; }
+constexpr int SORT_DIGIT_BITS = 9;  // 44-bit tile|depth keys take 5 passes (8-bit digits would need 6)
+inline int sort_num_passes(int end_bit) { return (end_bit + SORT_DIGIT_BITS - 1) / SORT_DIGIT_BITS; }
 inline bool sort_result_in_b(int end_bit) { return (sort_num_passes(end_bit) & 1) != 0; }
 int launch_sort_pairs_u64(int64_t n, uint64_t* keys_a, uint64_t* keys_b, uint32_t* vals_a, uint32_t* vals_b,
                           int end_bit, void* temp, hipStream_t stream);

@@ -1,5 +1,5 @@
 // Stable least-significant-digit radix sort of (key, uint32 value) pairs with
-// 8-bit digits, for 64-bit (tile|depth) keys and 32-bit Morton keys.  Replaces
+// 9-bit digits, for 64-bit (tile|depth) keys and 32-bit Morton keys.  Replaces
 // the library sort the reference calls at cuda_rasterizer/rasterizer_impl.cu:679-684
 // and simple-knn/simple_knn.cu:210-213; stability and the [0, end_bit) bit range
 // are part of the contract because tie order decides blending order.
@@ -12,7 +12,7 @@
 //   2. ranks its keys: per wave, lanes holding equal digits find each other
 //      through a lane mask per digit in LDS, and a per-wave running counter
 //      per digit gives each key its rank in wave order (stable);
-//   3. publishes its 256 digit counts and finds how many keys of each digit
+//   3. publishes its 512 digit counts and finds how many keys of each digit
 //      precede it with a two-level look-back (below);
 //   4. regroups its pairs by digit in LDS and writes each digit run to
 //      consecutive addresses.
@@ -34,11 +34,11 @@ namespace gs {
 
 namespace {
 
-constexpr int SORT_THREADS = 256;
+constexpr int RADIX = 1 << SORT_DIGIT_BITS;
+constexpr int SORT_THREADS = RADIX;  // one thread per digit value
 constexpr int SORT_WAVES = SORT_THREADS / GS_WAVE;
-constexpr int SORT_ITEMS = 16;
+constexpr int SORT_ITEMS = 8;
 constexpr int SORT_TILE = SORT_THREADS * SORT_ITEMS;
-constexpr int RADIX = 256;
 constexpr int MAX_PASSES = 8;
 constexpr int HIST_ITEMS = 16;  // keys per thread in the histogram kernel
 
@@ -82,8 +82,8 @@ sort_histogram_kernel(int64_t n, const K* __restrict__ keys, int passes, int end
     const bool valid = idx < n;
     const K key = keyv[k];
     for (int p = 0; p < passes; p++) {
-      const int shift = 8 * p;
-      const int bits = end_bit - shift >= 8 ? 8 : end_bit - shift;
+      const int shift = SORT_DIGIT_BITS * p;
+      const int bits = end_bit - shift >= SORT_DIGIT_BITS ? SORT_DIGIT_BITS : end_bit - shift;
       const uint32_t d = digit_of(key, shift, (1u << bits) - 1u);
       // A digit shared by the whole wave (float exponent bits, unused high bits) would serialise the LDS
       // atomic 64 ways: one lane adds the wave's count instead.
@@ -170,10 +170,13 @@ sort_onesweep_kernel(int64_t n, const K* __restrict__ keys_in, K* __restrict__ k
   __shared__ uint32_t s_gbase[RADIX];
   __shared__ uint32_t s_scan[SORT_WAVES];
   __shared__ uint32_t s_tile;
-  // regrouping buffer: keys first, then reused for the values; before that its head holds the lane masks
-  __shared__ K s_keys[SORT_TILE];
-  static_assert(sizeof(K) * SORT_TILE >= sizeof(unsigned long long) * SORT_WAVES * RADIX, "lane masks must fit");
-  unsigned long long (*s_mask)[RADIX] = reinterpret_cast<unsigned long long (*)[RADIX]>(s_keys);
+  // regrouping buffer: the lane masks of the ranking first, then the keys, then the values
+  constexpr size_t BUF_BYTES = sizeof(K) * SORT_TILE > sizeof(unsigned long long) * SORT_WAVES * RADIX
+                                   ? sizeof(K) * SORT_TILE
+                                   : sizeof(unsigned long long) * SORT_WAVES * RADIX;
+  __shared__ __attribute__((aligned(16))) unsigned char s_buf[BUF_BYTES];
+  K* s_keys = reinterpret_cast<K*>(s_buf);
+  unsigned long long (*s_mask)[RADIX] = reinterpret_cast<unsigned long long (*)[RADIX]>(s_buf);
 
   const int tid = threadIdx.x, lane = tid & (GS_WAVE - 1), wave = tid / GS_WAVE;
   if (tid == 0) s_tile = atomicAdd(ticket, 1u);
@@ -410,8 +413,8 @@ int sort_pairs_impl(int64_t n, K* keys_a, K* keys_b, uint32_t* vals_a, uint32_t*
   uint32_t* vin = vals_a;
   uint32_t* vout = vals_b;
   for (int p = 0; p < passes; p++) {
-    const int shift = 8 * p;
-    const int bits = end_bit - shift >= 8 ? 8 : end_bit - shift;
+    const int shift = SORT_DIGIT_BITS * p;
+    const int bits = end_bit - shift >= SORT_DIGIT_BITS ? SORT_DIGIT_BITS : end_bit - shift;
     const uint32_t mask = (1u << bits) - 1u;
     hipLaunchKernelGGL(sort_onesweep_kernel<K>, dim3(L.ntiles), dim3(SORT_THREADS), 0, stream, n, kin, kout, vin, vout,
                        shift, mask, hist + p * RADIX, tickets + p, states + (size_t)p * L.ntiles * RADIX,
