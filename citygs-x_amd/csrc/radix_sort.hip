@@ -159,6 +159,32 @@ __device__ __forceinline__ bool look_back(const uint32_t* __restrict__ state, in
   return true;
 }
 
+// Adds up the counts of the earlier tiles of the group, fetched into `earlier` beforehand; entries that had not
+// been published at the time of the fetch are polled.  Returns false when the bounded spin ran out.
+__device__ __forceinline__ bool level1_sum(const uint32_t* earlier, const uint32_t* __restrict__ tile_state,
+                                           uint32_t tile, int tid, uint32_t& sum) {
+  uint32_t missing = 0;
+#pragma unroll
+  for (int i = 0; i < GROUP - 1; i++) {
+    sum += earlier[i] & VALUE_MASK;
+    if ((earlier[i] & ~VALUE_MASK) == 0u) missing |= 1u << i;
+  }
+  for (int spins = 0; missing != 0u;) {
+    const int i = __builtin_ctz(missing);
+    const uint32_t v = __hip_atomic_load(tile_state + (size_t)(tile - 1 - i) * RADIX + tid, __ATOMIC_RELAXED,
+                                         __HIP_MEMORY_SCOPE_AGENT);
+    if ((v & ~VALUE_MASK) != 0u) {
+      sum += v & VALUE_MASK;
+      missing &= missing - 1u;
+    } else if (++spins > SPIN_LIMIT) {
+      return false;
+    } else {
+      __builtin_amdgcn_s_sleep(1);
+    }
+  }
+  return true;
+}
+
 template <typename K>
 __global__ void __launch_bounds__(SORT_THREADS)
 sort_onesweep_kernel(int64_t n, const K* __restrict__ keys_in, K* __restrict__ keys_out,
@@ -185,6 +211,7 @@ sort_onesweep_kernel(int64_t n, const K* __restrict__ keys_in, K* __restrict__ k
     s_wcount[w][tid] = 0;
     s_mask[w][tid] = 0ull;
   }
+  s_gbase[tid] = 0u;  // first the tile's digit histogram, later the global bases
   __syncthreads();
   const uint32_t tile = s_tile;
   const int64_t tile_start = (int64_t)tile * SORT_TILE;
@@ -200,6 +227,47 @@ sort_onesweep_kernel(int64_t n, const K* __restrict__ keys_in, K* __restrict__ k
     const bool valid = idx < n;
     key[k] = valid ? keys_in[idx] : (K)0;
     val[k] = valid ? vals_in[idx] : 0u;
+  }
+
+  // The tile's digit counts first, by plain LDS atomics, so that they can be published before the (longer)
+  // ranking: the later tiles of the group and the group's closing tile wait for nothing else, and this
+  // tile's own look-back loads travel while it ranks and regroups.
+#pragma unroll
+  for (int k = 0; k < SORT_ITEMS; k++) {
+    const bool valid = wave_start + (int64_t)k * GS_WAVE + lane < n;
+    const uint32_t d = digit_of(key[k], shift, mask);
+    // a digit shared by the whole wave would serialise 64 ways: one lane adds the count
+    const uint64_t vm = __ballot(valid);
+    const uint32_t d0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)d);
+    if (vm != 0ull && __ballot(valid && d == d0) == vm && (vm & 1ull)) {
+      if (lane == 0) atomicAdd(&s_gbase[d0], (uint32_t)__popcll(vm));
+    } else if (valid) {
+      atomicAdd(&s_gbase[d], 1u);
+    }
+  }
+  __syncthreads();
+  const uint32_t total = s_gbase[tid];  // thread tid owns digit tid
+  __hip_atomic_store(tile_state + (size_t)tile * RADIX + tid, FLAG_AGGREGATE | total, __ATOMIC_RELAXED,
+                     __HIP_MEMORY_SCOPE_AGENT);
+  // Look-back, level 1, issue: the counts of the earlier tiles of the own group
+  const int64_t group = tile / GROUP;
+  const int in_group = (int)(tile % GROUP);
+  const bool closes_group = in_group == GROUP - 1;  // an incomplete last group is never looked at
+  uint32_t earlier[GROUP - 1];
+#pragma unroll
+  for (int i = 0; i < GROUP - 1; i++)
+    earlier[i] = i < in_group ? __hip_atomic_load(tile_state + (size_t)(tile - 1 - i) * RADIX + tid, __ATOMIC_RELAXED,
+                                                  __HIP_MEMORY_SCOPE_AGENT)
+                              : FLAG_AGGREGATE;
+  uint32_t before_tiles = 0;
+  bool ok = true;
+  // The closing tile of a group resolves level 1 at once and publishes the group's sum: every later group
+  // is waiting for it.  The other tiles come back to their loads after the regrouping.
+  if (closes_group) {
+    ok = level1_sum(earlier, tile_state, tile, tid, before_tiles);
+    __hip_atomic_store(group_state + (size_t)group * RADIX + tid,
+                       (group == 0 ? FLAG_PREFIX : FLAG_AGGREGATE) | ((before_tiles + total) & VALUE_MASK),
+                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
 
   // Ranking.  LDS operations of one wave execute in program order, which the two steps below rely on; none
@@ -244,28 +312,9 @@ sort_onesweep_kernel(int64_t n, const K* __restrict__ keys_in, K* __restrict__ k
   }
   __syncthreads();
 
-  // thread tid owns digit tid
   uint32_t wcount[SORT_WAVES];
-  uint32_t total = 0;
 #pragma unroll
-  for (int w = 0; w < SORT_WAVES; w++) {
-    wcount[w] = s_wcount[w][tid];
-    total += wcount[w];
-  }
-  // counts of this tile, for the later tiles of its group
-  __hip_atomic_store(tile_state + (size_t)tile * RADIX + tid, FLAG_AGGREGATE | total, __ATOMIC_RELAXED,
-                     __HIP_MEMORY_SCOPE_AGENT);
-
-  // Look-back, level 1, issue: fetch the counts of the earlier tiles of the own group now and use them after
-  // the regrouping below, so the round trip to memory overlaps with LDS work.
-  const int64_t group = tile / GROUP;
-  const int in_group = (int)(tile % GROUP);
-  uint32_t earlier[GROUP - 1];
-#pragma unroll
-  for (int i = 0; i < GROUP - 1; i++)
-    earlier[i] = i < in_group ? __hip_atomic_load(tile_state + (size_t)(tile - 1 - i) * RADIX + tid, __ATOMIC_RELAXED,
-                                                  __HIP_MEMORY_SCOPE_AGENT)
-                              : FLAG_AGGREGATE;
+  for (int w = 0; w < SORT_WAVES; w++) wcount[w] = s_wcount[w][tid];
 
   // digit prefix inside the tile, then regroup the keys by digit in LDS
   uint32_t inc = total;
@@ -307,35 +356,9 @@ sort_onesweep_kernel(int64_t n, const K* __restrict__ keys_in, K* __restrict__ k
     key[k] = p < tile_count ? s_keys[p] : (K)0;  // from here on: the key at regrouped place p
   }
 
-  // Look-back, level 1, use: all earlier tiles of the group must have published; poll the late ones
-  uint32_t before_tiles = 0;
-  bool ok = true;
-  uint32_t missing = 0;
-#pragma unroll
-  for (int i = 0; i < GROUP - 1; i++) {
-    before_tiles += earlier[i] & VALUE_MASK;
-    if ((earlier[i] & ~VALUE_MASK) == 0u) missing |= 1u << i;
-  }
-  for (int spins = 0; missing != 0u;) {
-    const int i = __builtin_ctz(missing);
-    const uint32_t v = __hip_atomic_load(tile_state + (size_t)(tile - 1 - i) * RADIX + tid, __ATOMIC_RELAXED,
-                                         __HIP_MEMORY_SCOPE_AGENT);
-    if ((v & ~VALUE_MASK) != 0u) {
-      before_tiles += v & VALUE_MASK;
-      missing &= missing - 1u;
-    } else if (++spins > SPIN_LIMIT) {
-      ok = false;
-      break;
-    } else {
-      __builtin_amdgcn_s_sleep(1);
-    }
-  }
+  // Look-back, level 1, use (the closing tile has done it already)
+  if (!closes_group) ok = level1_sum(earlier, tile_state, tile, tid, before_tiles);
   // level 2: whole groups
-  const bool closes_group = in_group == GROUP - 1;  // an incomplete last group is never looked at
-  if (closes_group)
-    __hip_atomic_store(group_state + (size_t)group * RADIX + tid,
-                       (group == 0 ? FLAG_PREFIX : FLAG_AGGREGATE) | ((before_tiles + total) & VALUE_MASK),
-                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   if (group != 0) {
     ok = look_back<GROUP_LOOKBACK>(group_state, 0, group - 1, tid, before_tiles) && ok;
     if (closes_group)
