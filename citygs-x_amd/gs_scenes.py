@@ -189,3 +189,46 @@ def build_all_map(means3D, scales, rotations, cam):
     out[:, 3] = 1.0
     out[:, 4] = dist
     return out
+
+
+def make_anchor_scene(N, k=10, seed=0, feat_dim=32):
+    """Seeded anchors for the neural-Gaussian generation step: anchor positions, features, offsets,
+    activated scalings (N,6), a camera centre and the three MLPs as nn.Linear-shaped tensors
+    (scene/gaussian_model.py:131-149: Linear(feat_dim+3, feat_dim), ReLU, Linear(feat_dim, out)) drawn with
+    nn.Linear's default range.  Returns a dict; "mlps" is [(W1, b1, W2, b2)] in the order opacity, color, cov."""
+    gen = torch.Generator().manual_seed(1000 + seed)
+    r = lambda *s: torch.rand(*s, generator=gen)
+    n = lambda *s: torch.randn(*s, generator=gen)
+    anchor = (r(N, 3) - 0.5) * torch.tensor([400.0, 400.0, 40.0])
+    feat = n(N, feat_dim) * 0.7
+    offsets = n(N, k, 3) * 0.5
+    scaling = torch.exp(n(N, 6) * 0.4 - 1.0)
+    campos = torch.tensor([10.0, -20.0, 120.0])
+    mlps = []
+    for out in (k, 3 * k, 7 * k):
+        a1, a2 = 1.0 / math.sqrt(feat_dim + 3), 1.0 / math.sqrt(feat_dim)
+        mlps.append(((r(feat_dim, feat_dim + 3) * 2 - 1) * a1, (r(feat_dim) * 2 - 1) * a1,
+                     (r(out, feat_dim) * 2 - 1) * a2, (r(out) * 2 - 1) * a2))
+    return {"anchor": anchor, "feat": feat, "offsets": offsets, "scaling": scaling, "campos": campos, "mlps": mlps}
+
+
+def neural_gaussians_torch(anchor, feat, offsets, scaling, campos, mlps):
+    """generate_neural_gaussians (gaussian_renderer/__init__.py:789-899) in its default configuration, with
+    torch operations in the dtype of its inputs: the comparison the fused operator is measured against."""
+    k = offsets.shape[1]
+    ob_view = anchor - campos
+    ob_view = ob_view / ob_view.norm(dim=1, keepdim=True)
+    x = torch.cat([feat, ob_view], dim=1)
+    run = lambda m: torch.relu(x @ m[0].t() + m[1]) @ m[2].t() + m[3]
+    neural_opacity = torch.tanh(run(mlps[0])).reshape(-1, 1)
+    mask = (neural_opacity > 0.0).view(-1)
+    opacity = neural_opacity[mask]
+    color = torch.sigmoid(run(mlps[1])).reshape(-1, 3)
+    scale_rot = run(mlps[2]).reshape(-1, 7)
+    cat = torch.cat([scaling, anchor], dim=-1).repeat_interleave(k, dim=0)
+    masked = torch.cat([cat, color, scale_rot, offsets.reshape(-1, 3)], dim=-1)[mask]
+    scaling_repeat, repeat_anchor, color, scale_rot, offs = masked.split([6, 3, 3, 7, 3], dim=-1)
+    scal = scaling_repeat[:, 3:] * torch.sigmoid(scale_rot[:, :3])
+    rot = torch.nn.functional.normalize(scale_rot[:, 3:7])
+    xyz = repeat_anchor + offs * scaling_repeat[:, :3]
+    return xyz, color, opacity, scal, rot, neural_opacity, mask

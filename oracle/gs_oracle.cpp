@@ -1289,4 +1289,201 @@ void oracle_ssim_l1_bwd(int C, int H, int W, const float* img1, const float* img
       }
 }
 
+
+// ---------------------------------------------------------------------------
+// Neural-Gaussian generation, generate_neural_gaussians (gaussian_renderer/__init__.py:789-899) in the
+// reference's default configuration (arguments/__init__.py:94-124: feat_dim 32, no feature bank, no
+// appearance embedding, no distance / level inputs, dist2level 'round'): per visible anchor
+//   x = [feat(32), (anchor - campos)/|anchor - campos| (3)]
+//   neural_opacity = tanh(W2o relu(W1o x + b1o) + b2o)            (k values)       :841-853
+//   color = sigmoid(W2c relu(W1c x + b1c) + b2c)                  (k x 3)          :866-870
+//   scale_rot = W2v relu(W1v x + b1v) + b2v                       (k x 7)          :873-877
+// and for every (anchor, offset) with neural_opacity > 0, in that order (:856-858, :886):
+//   xyz = anchor + offset * scaling[0:3];  scaling = scaling[3:6] * sigmoid(scale_rot[0:3]);
+//   rot = scale_rot[3:7] / max(|scale_rot[3:7]|, 1e-12);  color;  opacity = neural_opacity   (:889-896)
+// MLPs as nn.Linear: W1 (32 x 35), b1 (32), W2 (out x 32), b2 (out), row-major [out][in]
+// (scene/gaussian_model.py:131-149).  `scaling` is the activated one, get_scaling (N x 6).
+// Sums run left to right in float32; torch's matmul leaves the order open: agreement to rounding.
+struct MlpView {
+  const float *W1, *b1, *W2, *b2;
+  int out;
+};
+
+static void mlp_forward(const MlpView& m, const float* x, float* hidden, float* out) {
+  for (int h = 0; h < 32; h++) {
+    float a = m.b1[h];
+    for (int i = 0; i < 35; i++) a += m.W1[h * 35 + i] * x[i];
+    hidden[h] = a > 0.f ? a : 0.f;
+  }
+  for (int o = 0; o < m.out; o++) {
+    float a = m.b2[o];
+    for (int h = 0; h < 32; h++) a += m.W2[o * 32 + h] * hidden[h];
+    out[o] = a;
+  }
+}
+
+static void neural_input(const float* anchor, const float* feat, const float* campos, float* x, float* dist) {
+  for (int i = 0; i < 32; i++) x[i] = feat[i];
+  const float v[3] = {anchor[0] - campos[0], anchor[1] - campos[1], anchor[2] - campos[2]};
+  const float d = sqrtf((v[0] * v[0] + v[1] * v[1]) + v[2] * v[2]);
+  x[32] = v[0] / d; x[33] = v[1] / d; x[34] = v[2] / d;
+  *dist = d;
+}
+
+// dense per-slot results: neural_opacity (N*k), mask (N*k), color (N*k*3, after sigmoid), scale_rot (N*k*7)
+void oracle_neural_mlp_fwd(int N, int k, const float* anchor, const float* feat, const float* campos,
+                           const float* W1o, const float* b1o, const float* W2o, const float* b2o,
+                           const float* W1c, const float* b1c, const float* W2c, const float* b2c,
+                           const float* W1v, const float* b1v, const float* W2v, const float* b2v,
+                           float* neural_opacity, uint8_t* mask, float* color, float* scale_rot) {
+  const MlpView mo{W1o, b1o, W2o, b2o, k}, mc{W1c, b1c, W2c, b2c, 3 * k}, mv{W1v, b1v, W2v, b2v, 7 * k};
+#pragma omp parallel for schedule(static)
+  for (int a = 0; a < N; a++) {
+    float x[35], dist, hid[32];
+    neural_input(anchor + 3 * (size_t)a, feat + 32 * (size_t)a, campos, x, &dist);
+    std::vector<float> out(7 * k);
+    mlp_forward(mo, x, hid, out.data());
+    for (int j = 0; j < k; j++) {
+      const float t = tanhf(out[j]);
+      neural_opacity[(size_t)a * k + j] = t;
+      mask[(size_t)a * k + j] = t > 0.f;
+    }
+    mlp_forward(mc, x, hid, out.data());
+    for (int j = 0; j < 3 * k; j++) color[(size_t)a * 3 * k + j] = 1.0f / (1.0f + expf(-out[j]));
+    mlp_forward(mv, x, hid, out.data());
+    for (int j = 0; j < 7 * k; j++) scale_rot[(size_t)a * 7 * k + j] = out[j];
+  }
+}
+
+// compaction and post-processing; returns the number of selected Gaussians
+int oracle_neural_compact(int N, int k, const float* anchor, const float* offsets, const float* scaling,
+                          const float* neural_opacity, const uint8_t* mask, const float* color,
+                          const float* scale_rot, float* xyz, float* col, float* opacity, float* scal, float* rot) {
+  size_t r = 0;
+  for (int a = 0; a < N; a++)
+    for (int j = 0; j < k; j++) {
+      const size_t s = (size_t)a * k + j;
+      if (!mask[s]) continue;
+      const float* sc = scaling + 6 * (size_t)a;
+      for (int c = 0; c < 3; c++) {
+        xyz[3 * r + c] = anchor[3 * (size_t)a + c] + offsets[3 * s + c] * sc[c];
+        col[3 * r + c] = color[3 * s + c];
+        scal[3 * r + c] = sc[3 + c] * (1.0f / (1.0f + expf(-scale_rot[7 * s + c])));
+      }
+      opacity[r] = neural_opacity[s];
+      const float* q = scale_rot + 7 * s + 3;
+      const float len = sqrtf(((q[0] * q[0] + q[1] * q[1]) + q[2] * q[2]) + q[3] * q[3]);
+      const float den = fmaxf(len, 1e-12f);
+      for (int c = 0; c < 4; c++) rot[4 * r + c] = q[c] / den;
+      r++;
+    }
+  return (int)r;
+}
+
+// Backward of both steps.  Upstream gradients are given for the compacted outputs (S rows each); results:
+// d_anchor (N,3), d_feat (N,32), d_offsets (N*k,3), d_scaling (N,6) and the twelve weight gradients
+// (accumulated in double, returned as float32).  neural_opacity itself (the dense output) is taken as
+// non-differentiated, as the reference only uses it detached (scene/gaussian_model.py:1183).
+void oracle_neural_bwd(int N, int k, const float* anchor, const float* feat, const float* offsets,
+                       const float* scaling, const float* campos,
+                       const float* W1o, const float* b1o, const float* W2o, const float* b2o,
+                       const float* W1c, const float* b1c, const float* W2c, const float* b2c,
+                       const float* W1v, const float* b1v, const float* W2v, const float* b2v,
+                       const float* g_xyz, const float* g_col, const float* g_opacity, const float* g_scal,
+                       const float* g_rot, float* d_anchor, float* d_feat, float* d_offsets, float* d_scaling,
+                       float* dW1o, float* db1o, float* dW2o, float* db2o, float* dW1c, float* db1c, float* dW2c,
+                       float* db2c, float* dW1v, float* db1v, float* dW2v, float* db2v) {
+  const MlpView ms[3] = {{W1o, b1o, W2o, b2o, k}, {W1c, b1c, W2c, b2c, 3 * k}, {W1v, b1v, W2v, b2v, 7 * k}};
+  float* dW1s[3] = {dW1o, dW1c, dW1v};
+  float* db1s[3] = {db1o, db1c, db1v};
+  float* dW2s[3] = {dW2o, dW2c, dW2v};
+  float* db2s[3] = {db2o, db2c, db2v};
+  std::vector<std::vector<double>> aW1(3), ab1(3), aW2(3), ab2(3);
+  for (int m = 0; m < 3; m++) {
+    aW1[m].assign(32 * 35, 0.0); ab1[m].assign(32, 0.0);
+    aW2[m].assign((size_t)ms[m].out * 32, 0.0); ab2[m].assign(ms[m].out, 0.0);
+  }
+  size_t r = 0;
+  for (int a = 0; a < N; a++) {
+    float x[35], dist, hid[3][32];
+    neural_input(anchor + 3 * (size_t)a, feat + 32 * (size_t)a, campos, x, &dist);
+    std::vector<float> out[3], gout[3];
+    for (int m = 0; m < 3; m++) {
+      out[m].resize(ms[m].out);
+      gout[m].assign(ms[m].out, 0.f);
+      mlp_forward(ms[m], x, hid[m], out[m].data());
+    }
+    const float* sc = scaling + 6 * (size_t)a;
+    float da[3] = {0.f, 0.f, 0.f}, dsc[6] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    for (int j = 0; j < k; j++) {
+      const size_t s = (size_t)a * k + j;
+      for (int c = 0; c < 3; c++) d_offsets[3 * s + c] = 0.f;
+      const float t = tanhf(out[0][j]);
+      if (!(t > 0.f)) continue;
+      // opacity = tanh(pre)
+      gout[0][j] = g_opacity[r] * (1.0f - t * t);
+      for (int c = 0; c < 3; c++) {
+        const float cs = 1.0f / (1.0f + expf(-out[1][3 * j + c]));
+        gout[1][3 * j + c] = g_col[3 * r + c] * (cs * (1.0f - cs));
+        // xyz = anchor + offset * sc[c]
+        da[c] += g_xyz[3 * r + c];
+        d_offsets[3 * s + c] = g_xyz[3 * r + c] * sc[c];
+        dsc[c] += g_xyz[3 * r + c] * offsets[3 * s + c];
+        // scaling = sc[3+c] * sigmoid(sr[c])
+        const float sg = 1.0f / (1.0f + expf(-out[2][7 * j + c]));
+        dsc[3 + c] += g_scal[3 * r + c] * sg;
+        gout[2][7 * j + c] = g_scal[3 * r + c] * sc[3 + c] * (sg * (1.0f - sg));
+      }
+      // rot = q / max(|q|, eps)
+      const float* q = out[2].data() + 7 * j + 3;
+      const float len = sqrtf(((q[0] * q[0] + q[1] * q[1]) + q[2] * q[2]) + q[3] * q[3]);
+      const float* gr = g_rot + 4 * r;
+      if (len > 1e-12f) {
+        float qh[4], dot = 0.f;
+        for (int c = 0; c < 4; c++) { qh[c] = q[c] / len; dot += qh[c] * gr[c]; }
+        for (int c = 0; c < 4; c++) gout[2][7 * j + 3 + c] = (gr[c] - qh[c] * dot) / len;
+      } else {
+        for (int c = 0; c < 4; c++) gout[2][7 * j + 3 + c] = gr[c] / 1e-12f;
+      }
+      r++;
+    }
+    // through the three MLPs
+    float dx[35];
+    for (int i = 0; i < 35; i++) dx[i] = 0.f;
+    for (int m = 0; m < 3; m++) {
+      float dh[32];
+      for (int h = 0; h < 32; h++) dh[h] = 0.f;
+      for (int o = 0; o < ms[m].out; o++) {
+        const float g = gout[m][o];
+        if (g == 0.f) continue;
+        ab2[m][o] += g;
+        for (int h = 0; h < 32; h++) {
+          aW2[m][(size_t)o * 32 + h] += (double)g * hid[m][h];
+          dh[h] += ms[m].W2[o * 32 + h] * g;
+        }
+      }
+      for (int h = 0; h < 32; h++) {
+        if (!(hid[m][h] > 0.f)) continue;  // ReLU
+        ab1[m][h] += dh[h];
+        for (int i = 0; i < 35; i++) {
+          aW1[m][h * 35 + i] += (double)dh[h] * x[i];
+          dx[i] += ms[m].W1[h * 35 + i] * dh[h];
+        }
+      }
+    }
+    for (int i = 0; i < 32; i++) d_feat[32 * (size_t)a + i] = dx[i];
+    // view direction v/|v|: d v = (g - n (n.g)) / |v|
+    const float nv[3] = {x[32], x[33], x[34]};
+    const float ng = (nv[0] * dx[32] + nv[1] * dx[33]) + nv[2] * dx[34];
+    for (int c = 0; c < 3; c++) d_anchor[3 * (size_t)a + c] = da[c] + (dx[32 + c] - nv[c] * ng) / dist;
+    for (int c = 0; c < 6; c++) d_scaling[6 * (size_t)a + c] = dsc[c];
+  }
+  for (int m = 0; m < 3; m++) {
+    for (int i = 0; i < 32 * 35; i++) dW1s[m][i] = (float)aW1[m][i];
+    for (int i = 0; i < 32; i++) db1s[m][i] = (float)ab1[m][i];
+    for (size_t i = 0; i < (size_t)ms[m].out * 32; i++) dW2s[m][i] = (float)aW2[m][i];
+    for (int i = 0; i < ms[m].out; i++) db2s[m][i] = (float)ab2[m][i];
+  }
+}
+
 }  // extern "C"

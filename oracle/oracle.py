@@ -394,3 +394,49 @@ def knn_dist2(points):
 def morton(p, mn, mx):
     p, mn, mx = _f32(p), _f32(mn), _f32(mx)
     return int(lib().oracle_morton(_p(p), _p(mn), _p(mx)))
+
+
+def _mlp_args(mlps):
+    """mlps: three (W1 (32,35), b1 (32), W2 (out,32), b2 (out)) tuples in the order opacity, color, cov."""
+    flat = []
+    for W1, b1, W2, b2 in mlps:
+        flat += [_f32(W1), _f32(b1), _f32(W2), _f32(b2)]
+    return flat
+
+
+def neural_gaussians_fwd(anchor, feat, offsets, scaling, campos, mlps):
+    """generate_neural_gaussians (gaussian_renderer/__init__.py:789-899), default configuration, on the anchors
+    already selected by visible_mask.  Returns (xyz, color, opacity, scaling, rot, neural_opacity, mask)."""
+    anchor, feat, offsets, scaling = _f32(anchor), _f32(feat), _f32(offsets), _f32(scaling)
+    cp = _f32(campos).reshape(3)
+    N, k = anchor.shape[0], offsets.shape[1]
+    w = _mlp_args(mlps)
+    nop, mask = np.zeros((N * k, 1), np.float32), np.zeros(N * k, np.uint8)
+    col, sr = np.zeros((N * k, 3), np.float32), np.zeros((N * k, 7), np.float32)
+    lib().oracle_neural_mlp_fwd(C.c_int(N), C.c_int(k), _p(anchor), _p(feat), _p(cp), *[_p(x) for x in w], _p(nop),
+                                _p(mask), _p(col), _p(sr))
+    S = int(mask.sum())
+    xyz, c, op = np.zeros((S, 3), np.float32), np.zeros((S, 3), np.float32), np.zeros((S, 1), np.float32)
+    sc, rot = np.zeros((S, 3), np.float32), np.zeros((S, 4), np.float32)
+    lib().oracle_neural_compact.restype = C.c_int
+    got = lib().oracle_neural_compact(C.c_int(N), C.c_int(k), _p(anchor), _p(offsets), _p(scaling), _p(nop), _p(mask),
+                                      _p(col), _p(sr), _p(xyz), _p(c), _p(op), _p(sc), _p(rot))
+    assert got == S
+    return xyz, c, op, sc, rot, nop, mask.astype(bool)
+
+
+def neural_gaussians_bwd(anchor, feat, offsets, scaling, campos, mlps, g_xyz, g_color, g_opacity, g_scaling, g_rot):
+    """Gradients of neural_gaussians_fwd's five compacted outputs: (d_anchor, d_feat, d_offsets, d_scaling,
+    [12 weight gradients in the order of mlps])."""
+    anchor, feat, offsets, scaling = _f32(anchor), _f32(feat), _f32(offsets), _f32(scaling)
+    cp = _f32(campos).reshape(3)
+    N, k = anchor.shape[0], offsets.shape[1]
+    w = _mlp_args(mlps)
+    gs = [_f32(g_xyz), _f32(g_color), _f32(g_opacity), _f32(g_scaling), _f32(g_rot)]
+    da, df = np.zeros((N, 3), np.float32), np.zeros((N, 32), np.float32)
+    do, ds = np.zeros((N, k, 3), np.float32), np.zeros((N, 6), np.float32)
+    dw = [np.zeros_like(x) for x in w]
+    lib().oracle_neural_bwd(C.c_int(N), C.c_int(k), _p(anchor), _p(feat), _p(offsets), _p(scaling), _p(cp),
+                            *[_p(x) for x in w], *[_p(x) for x in gs], _p(da), _p(df), _p(do), _p(ds),
+                            *[_p(x) for x in dw])
+    return da, df, do, ds, dw

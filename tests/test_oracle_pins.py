@@ -647,3 +647,77 @@ def test_ssim_closed_forms(orc):
     m[3:9, 4:20] = True
     l1m, ssm = orc.ssim_l1_fwd(ca, cb, m)
     assert np.all(ssm[0][~m] == 0) and np.all(l1m[0][~m] == 0) and np.array_equal(ssm[0][m], ss[0][m])
+
+
+# ------------------------------------------------- neural-Gaussian generation --
+
+def _anchor_scene_np(N, k, seed):
+    s = gs_scenes.make_anchor_scene(N, k, seed)
+    n = lambda t: t.numpy()
+    mlps = [tuple(n(x) for x in m) for m in s["mlps"]]
+    return s, (n(s["anchor"]), n(s["feat"]), n(s["offsets"]), n(s["scaling"]), n(s["campos"]), mlps)
+
+
+@pytest.mark.parametrize("N,k,seed", [(257, 10, 0), (64, 5, 1), (1, 10, 2)])
+def test_neural_gaussians_forward_matches_float64_torch(orc, N, k, seed):
+    s, args = _anchor_scene_np(N, k, seed)
+    got = orc.neural_gaussians_fwd(*args)
+    d = lambda t: t.double()
+    want = gs_scenes.neural_gaussians_torch(d(s["anchor"]), d(s["feat"]), d(s["offsets"]), d(s["scaling"]),
+                                            d(s["campos"]), [tuple(d(x) for x in m) for m in s["mlps"]])
+    # the selection is a threshold on a float32 value: equal unless an opacity sits within rounding of zero
+    wmask = want[6].numpy()
+    near = np.abs(want[5].numpy().ravel()) < 1e-6
+    assert (got[6] == wmask)[~near].all()
+    if (got[6] == wmask).all():
+        for g, w in zip(got[:6], want[:6]):
+            assert g.shape == tuple(w.shape)
+            assert _rel(g, w.numpy()) < 2e-6
+    assert got[0].shape[0] == int(got[6].sum()) and 0 < got[6].sum() < N * k or N == 1
+    # rotations are unit quaternions, opacities are the positive dense ones in slot order
+    assert np.allclose(np.linalg.norm(got[4], axis=1), 1.0, atol=1e-6)
+    assert np.array_equal(got[2].ravel(), got[5].ravel()[got[6]])
+
+
+def test_neural_gaussians_known_case(orc):
+    """Zero weights: every output is its bias through the activation; one offset switched off by a negative bias."""
+    N, k = 3, 4
+    s, (anchor, feat, offsets, scaling, campos, mlps) = _anchor_scene_np(N, k, 5)
+    z = lambda a: np.zeros_like(a)
+    b_op = np.array([0.5, -0.5, 0.25, 1.0], np.float32)
+    b_col = np.linspace(-1, 1, 3 * k).astype(np.float32)
+    b_cov = np.tile(np.array([0.0, 1.0, -1.0, 2.0, 0.0, 0.0, 0.0], np.float32), k)
+    mlps = [(z(mlps[0][0]), z(mlps[0][1]), z(mlps[0][2]), b_op), (z(mlps[1][0]), z(mlps[1][1]), z(mlps[1][2]), b_col),
+            (z(mlps[2][0]), z(mlps[2][1]), z(mlps[2][2]), b_cov)]
+    xyz, col, op, sc, rot, nop, mask = orc.neural_gaussians_fwd(anchor, feat, offsets, scaling, campos, mlps)
+    assert mask.reshape(N, k).tolist() == [[True, False, True, True]] * N
+    keep = [0, 2, 3]
+    assert np.allclose(op.reshape(N, 3), np.tanh(b_op[keep].astype(np.float64)), rtol=1e-6)
+    sig = lambda v: 1 / (1 + np.exp(-v.astype(np.float64)))
+    assert np.allclose(col.reshape(N, 3, 3), sig(b_col.reshape(k, 3)[keep]), rtol=1e-6)
+    assert np.allclose(rot, [1.0, 0.0, 0.0, 0.0])
+    assert np.allclose(sc.reshape(N, 3, 3), scaling[:, None, 3:] * sig(b_cov[:3])[None, None, :], rtol=1e-6)
+    assert np.allclose(xyz.reshape(N, 3, 3), anchor[:, None, :] + offsets[:, keep, :] * scaling[:, None, :3], rtol=1e-6)
+
+
+@pytest.mark.parametrize("N,k,seed", [(193, 10, 3), (50, 5, 4)])
+def test_neural_gaussians_backward_matches_float64_autograd(orc, N, k, seed):
+    s, args = _anchor_scene_np(N, k, seed)
+    fwd = orc.neural_gaussians_fwd(*args)
+    S = fwd[0].shape[0]
+    gen = torch.Generator().manual_seed(seed)
+    ups = [torch.randn(S, c, generator=gen) for c in (3, 3, 1, 3, 4)]
+    got = orc.neural_gaussians_bwd(*args, *[u.numpy() for u in ups])
+    leaf = lambda t: t.double().requires_grad_(True)
+    anchor, feat, offsets, scaling = leaf(s["anchor"]), leaf(s["feat"]), leaf(s["offsets"]), leaf(s["scaling"])
+    mlps = [tuple(leaf(x) for x in m) for m in s["mlps"]]
+    out = gs_scenes.neural_gaussians_torch(anchor, feat, offsets, scaling, s["campos"].double(), mlps)
+    assert np.array_equal(out[6].numpy(), fwd[6])
+    loss = sum((o * u.double()).sum() for o, u in zip(out[:5], ups))
+    loss.backward()
+    for name, g, w in zip(("anchor", "feat", "offsets", "scaling"), got[:4], (anchor, feat, offsets, scaling)):
+        assert _rel(g, w.grad.numpy()) < 1e-5, name
+    flat = [x for m in mlps for x in m]
+    for i, (g, w) in enumerate(zip(got[4], flat)):
+        assert g.shape == tuple(w.shape)
+        assert _rel(g, w.grad.numpy()) < 1e-5, i
