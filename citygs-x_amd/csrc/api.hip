@@ -651,6 +651,158 @@ int gs_adam_step(int count, float* const* params, const float* const* grads, flo
   return check_launch("adam_step", (hipStream_t)stream, false);
 }
 
+int gs_neural_supported(int n_offsets) { return neural_supported(n_offsets) ? 1 : 0; }
+
+namespace {
+struct NeuralWorkspace {
+  size_t packed, counts, scan, total;
+};
+NeuralWorkspace neural_workspace(int64_t N, int k) {
+  NeuralWorkspace L;
+  size_t off = 0;
+  L.packed = off; off += align_up(neural_packed_floats(k) * sizeof(float), 256);
+  L.counts = off; off += align_up((size_t)(N > 0 ? N : 1), 256);
+  L.scan = off; off += scan_temp_bytes(N);
+  L.total = off;
+  return L;
+}
+}  // namespace
+
+size_t gs_neural_workspace_bytes(int64_t num_anchors, int n_offsets) {
+  return neural_workspace(num_anchors, n_offsets).total + 256;
+}
+
+int gs_neural_opacity_forward(int64_t N, int k, const float* anchor, const float* feat, const float* campos,
+                              const float* const* mlp_params, float* neural_opacity, uint8_t* mask, uint32_t* first,
+                              void* workspace, size_t workspace_bytes, int64_t* num_selected, gs_stream_t stream_) {
+  hipStream_t stream = (hipStream_t)stream_;
+  GS_REQUIRE(N >= 0, "gs_neural_opacity_forward: negative anchor count");
+  GS_REQUIRE(neural_supported(k), "gs_neural_opacity_forward: n_offsets not among the supported values");
+  GS_REQUIRE(num_selected, "gs_neural_opacity_forward: null num_selected");
+  *num_selected = 0;
+  GS_REQUIRE(N * (int64_t)k < 0x7FFFFFFFll, "gs_neural_opacity_forward: anchors x offsets exceed 2^31-1");
+  GS_REQUIRE(mlp_params && campos, "gs_neural_opacity_forward: null pointer");
+  for (int i = 0; i < 12; i++) GS_REQUIRE(mlp_params[i], "gs_neural_opacity_forward: null MLP parameter");
+  GS_REQUIRE(workspace && workspace_bytes >= gs_neural_workspace_bytes(N, k),
+             "gs_neural_opacity_forward: workspace missing or too small");
+  char* base = align_ptr((char*)workspace, 256);
+  const NeuralWorkspace L = neural_workspace(N, k);
+  float* packed = (float*)(base + L.packed);
+  {
+    StageScope _t("neural_pack", stream);
+    launch_neural_pack(k, mlp_params, packed, stream);
+  }
+  if (check_launch("neural_pack", stream, false)) return 1;
+  if (N == 0) return 0;
+  GS_REQUIRE(anchor && feat && neural_opacity && mask && first, "gs_neural_opacity_forward: null pointer");
+  uint8_t* counts = (uint8_t*)(base + L.counts);
+  {
+    StageScope _t("neural_opacity", stream);
+    launch_neural_opacity(N, k, anchor, feat, campos, packed, neural_opacity, mask, counts, stream);
+  }
+  if (check_launch("neural_opacity", stream, false)) return 1;
+  uint32_t* total_slot = acquire_total_slot();
+  {
+    StageScope _t("neural_scan", stream);
+    launch_exclusive_sum_u8(N, counts, first, base + L.scan, stream, total_slot);
+  }
+  if (check_launch("neural_scan", stream, false)) return 1;
+  uint32_t total = 0;
+  if (total_slot != nullptr) {
+    if (wait_for_total(total_slot, stream, &total)) return 1;
+  } else {
+    uint32_t last_first = 0;
+    uint8_t last_count = 0;
+    GS_HIP_TRY(hipMemcpyAsync(&last_first, first + (N - 1), sizeof(uint32_t), hipMemcpyDeviceToHost, stream));
+    GS_HIP_TRY(hipMemcpyAsync(&last_count, counts + (N - 1), 1, hipMemcpyDeviceToHost, stream));
+    GS_HIP_TRY(hipStreamSynchronize(stream));
+    total = last_first + last_count;
+  }
+  *num_selected = (int64_t)total;
+  return 0;
+}
+
+int gs_neural_gaussians_forward(int64_t N, int k, int64_t S, const float* anchor, const float* feat,
+                                const float* offsets, const float* scaling, const float* campos,
+                                const float* neural_opacity, const uint32_t* first, const void* workspace,
+                                size_t workspace_bytes, float* xyz, float* color, float* opacity, float* scaling_out,
+                                float* rot, float* aux, gs_stream_t stream_) {
+  hipStream_t stream = (hipStream_t)stream_;
+  GS_REQUIRE(N >= 0 && S >= 0, "gs_neural_gaussians_forward: negative size");
+  GS_REQUIRE(neural_supported(k), "gs_neural_gaussians_forward: n_offsets not among the supported values");
+  if (N == 0 || S == 0) return 0;
+  GS_REQUIRE(S <= N * (int64_t)k, "gs_neural_gaussians_forward: more selected Gaussians than offsets");
+  GS_REQUIRE(anchor && feat && offsets && scaling && campos && neural_opacity && first,
+             "gs_neural_gaussians_forward: null input");
+  GS_REQUIRE(xyz && color && opacity && scaling_out && rot && aux, "gs_neural_gaussians_forward: null output");
+  GS_REQUIRE(((uintptr_t)rot & 15) == 0 && ((uintptr_t)aux & 15) == 0 && ((uintptr_t)feat & 15) == 0,
+             "gs_neural_gaussians_forward: feat, rot and aux must be 16-byte aligned");
+  GS_REQUIRE(workspace && workspace_bytes >= gs_neural_workspace_bytes(N, k),
+             "gs_neural_gaussians_forward: workspace missing or too small");
+  const float* packed = (const float*)(align_ptr((const char*)workspace, 256) + neural_workspace(N, k).packed);
+  {
+    StageScope _t("neural_gaussians", stream);
+    launch_neural_gaussians(N, k, anchor, feat, offsets, scaling, campos, packed, neural_opacity, first, xyz, color,
+                            opacity, scaling_out, rot, aux, stream);
+  }
+  return check_launch("neural_gaussians", stream, false);
+}
+
+size_t gs_neural_backward_workspace_bytes(int64_t num_anchors, int n_offsets) {
+  return align_up(neural_packed_floats(n_offsets) * sizeof(float), 256) +
+         align_up(neural_partial_floats(n_offsets, num_anchors > 0 ? num_anchors : 1) * sizeof(float), 256) + 256;
+}
+
+int gs_neural_backward(int64_t N, int k, int64_t S, const float* anchor, const float* feat, const float* offsets,
+                       const float* scaling, const float* campos, const float* const* mlp_params,
+                       const float* neural_opacity, const uint32_t* first, const float* color, const float* rot,
+                       const float* aux, const float* dL_dxyz, const float* dL_dcolor, const float* dL_dopacity,
+                       const float* dL_dscaling, const float* dL_drot, float* d_anchor, float* d_feat,
+                       float* d_offsets, float* d_scaling, float* const* d_mlp_params, void* workspace,
+                       size_t workspace_bytes, gs_stream_t stream_) {
+  hipStream_t stream = (hipStream_t)stream_;
+  GS_REQUIRE(N >= 0 && S >= 0, "gs_neural_backward: negative size");
+  GS_REQUIRE(neural_supported(k), "gs_neural_backward: n_offsets not among the supported values");
+  GS_REQUIRE(mlp_params && d_mlp_params && campos, "gs_neural_backward: null pointer");
+  for (int i = 0; i < 12; i++)
+    GS_REQUIRE(mlp_params[i] && d_mlp_params[i], "gs_neural_backward: null MLP parameter or gradient");
+  if (N == 0) {
+    // no anchors: the weight gradients are zero
+    const size_t sizes[4] = {32 * 35, 32, 0, 0};
+    for (int i = 0; i < 12; i++) {
+      const int out = (i / 4 == 0 ? 1 : i / 4 == 1 ? 3 : 7) * k;
+      const size_t n = i % 4 == 2 ? (size_t)out * 32 : i % 4 == 3 ? (size_t)out : sizes[i % 4];
+      GS_HIP_TRY(hipMemsetAsync(d_mlp_params[i], 0, n * sizeof(float), stream));
+    }
+    return 0;
+  }
+  GS_REQUIRE(S <= N * (int64_t)k, "gs_neural_backward: more selected Gaussians than offsets");
+  GS_REQUIRE(anchor && feat && offsets && scaling && neural_opacity && first, "gs_neural_backward: null input");
+  GS_REQUIRE(S == 0 || (color && rot && aux && dL_dxyz && dL_dcolor && dL_dopacity && dL_dscaling && dL_drot),
+             "gs_neural_backward: null saved output or upstream gradient");
+  GS_REQUIRE(d_anchor && d_feat && d_offsets && d_scaling, "gs_neural_backward: null gradient output");
+  GS_REQUIRE(((uintptr_t)rot & 15) == 0 && ((uintptr_t)aux & 15) == 0 && ((uintptr_t)feat & 15) == 0 &&
+                 ((uintptr_t)dL_drot & 15) == 0 && ((uintptr_t)d_feat & 15) == 0,
+             "gs_neural_backward: feat, rot, aux, dL_drot and d_feat must be 16-byte aligned");
+  GS_REQUIRE(workspace && workspace_bytes >= gs_neural_backward_workspace_bytes(N, k),
+             "gs_neural_backward: workspace missing or too small");
+  char* base = align_ptr((char*)workspace, 256);
+  float* packed = (float*)base;
+  float* partials = (float*)(base + align_up(neural_packed_floats(k) * sizeof(float), 256));
+  {
+    StageScope _t("neural_pack", stream);
+    launch_neural_pack(k, mlp_params, packed, stream);
+  }
+  if (check_launch("neural_pack", stream, false)) return 1;
+  {
+    StageScope _t("neural_backward", stream);
+    launch_neural_backward(N, k, anchor, feat, offsets, scaling, campos, packed, neural_opacity, first, color, rot,
+                           aux, dL_dxyz, dL_dcolor, dL_dopacity, dL_dscaling, dL_drot, d_anchor, d_feat, d_offsets,
+                           d_scaling, d_mlp_params, partials, stream);
+  }
+  return check_launch("neural_backward", stream, false);
+}
+
 int gs_all_map_forward(int P, const float* means3D, const float* scales, const float* rotations,
                        const float* viewmatrix, const float* campos, float* all_map, gs_stream_t stream) {
   GS_REQUIRE(P >= 0, "gs_all_map_forward: negative P");

@@ -238,9 +238,10 @@ int launch_exclusive_sum(int64_t n, const uint32_t* in, uint32_t* out, void* tem
   return scan_impl(n, in, out, temp, true, nullptr, stream);
 }
 
-// exclusive ranks of the set bytes of a 0/1 mask
-int launch_exclusive_sum_u8(int64_t n, const uint8_t* in, uint32_t* out, void* temp, hipStream_t stream) {
-  return scan_impl(n, in, out, temp, true, nullptr, stream);
+// exclusive prefix sums of small counts (a 0/1 mask gives the ranks of its set bytes)
+int launch_exclusive_sum_u8(int64_t n, const uint8_t* in, uint32_t* out, void* temp, hipStream_t stream,
+                            uint32_t* total_out) {
+  return scan_impl(n, in, out, temp, true, total_out, stream);
 }
 
 int launch_duplicate_with_keys(int P, int W, int H, const float* means2D, const float* depths,

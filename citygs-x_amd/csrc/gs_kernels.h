@@ -49,7 +49,8 @@ int launch_tile_count(int P, int W, int H, const int* radii, const float* means2
                       uint32_t* tiles_touched, hipStream_t stream,
                       uint32_t* zero_words = nullptr, int64_t zero_count = 0);
 size_t scan_temp_bytes(int64_t n);
-int launch_exclusive_sum_u8(int64_t n, const uint8_t* in, uint32_t* out, void* temp, hipStream_t stream);
+int launch_exclusive_sum_u8(int64_t n, const uint8_t* in, uint32_t* out, void* temp, hipStream_t stream,
+                            uint32_t* total_out = nullptr);
 // total_out, when given, is a host-visible word that receives the grand total as well
 int launch_inclusive_sum(int64_t n, const uint32_t* in, uint32_t* out, void* temp, hipStream_t stream,
                          uint32_t* total_out = nullptr);
@@ -73,6 +74,25 @@ constexpr int ADAM_MAX_TENSORS = 24;  // tensors per launch (more are split over
 int launch_adam(int count, float* const* params, const float* const* grads, float* const* exp_avg,
                 float* const* exp_avg_sq, const long long* sizes, const double* lrs, const int* steps, double beta1,
                 double beta2, double eps, float grad_scale, hipStream_t stream);
+// ---- neural-Gaussian generation (n_offsets = k) ----
+bool neural_supported(int k);
+size_t neural_packed_floats(int k);
+size_t neural_partial_floats(int k, int64_t N);
+int launch_neural_pack(int k, const float* const* params, float* packed, hipStream_t stream);
+int launch_neural_opacity(int64_t N, int k, const float* anchor, const float* feat, const float* campos,
+                          const float* packed, float* neural_opacity, uint8_t* mask, uint8_t* counts,
+                          hipStream_t stream);
+int launch_neural_gaussians(int64_t N, int k, const float* anchor, const float* feat, const float* offsets,
+                            const float* scaling, const float* campos, const float* packed,
+                            const float* neural_opacity, const uint32_t* first, float* xyz, float* color,
+                            float* opacity, float* scal, float* rot, float* aux, hipStream_t stream);
+int launch_neural_backward(int64_t N, int k, const float* anchor, const float* feat, const float* offsets,
+                           const float* scaling, const float* campos, const float* packed,
+                           const float* neural_opacity, const uint32_t* first, const float* color_out,
+                           const float* rot_out, const float* aux, const float* g_xyz, const float* g_color,
+                           const float* g_opacity, const float* g_scal, const float* g_rot, float* d_anchor,
+                           float* d_feat, float* d_offsets, float* d_scaling, float* const* d_params, float* partials,
+                           hipStream_t stream);
 int launch_all_map_fwd(int P, const float* means, const float* scales, const float* rots, const float* V,
                        const float* campos, float* out, hipStream_t stream);
 int launch_all_map_bwd(int P, const float* means, const float* scales, const float* rots, const float* V,

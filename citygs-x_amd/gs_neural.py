@@ -1,0 +1,130 @@
+"""Neural-Gaussian generation of the reference, generate_neural_gaussians (gaussian_renderer/__init__.py:789-899),
+as three kernel launches forward (opacity MLP, scan, color/cov MLPs with the post-processing) and two backward,
+in libgsrast.so.  Covers the reference's default model configuration (arguments/__init__.py:94-124): feat_dim 32,
+no feature bank, no appearance embedding, no distance or level inputs to the MLPs, dist2level other than
+'progressive'; anything else raises NotImplementedError."""
+import ctypes as C
+
+import torch
+
+import gsrast_native as _n
+
+
+def _p(t):
+    return None if t is None else C.c_void_p(t.data_ptr())
+
+
+def _f32(t, name, shape):
+    if t.dtype != torch.float32:
+        raise TypeError(f"{name} must be float32, got {t.dtype}")
+    if not t.is_cuda:
+        raise RuntimeError(f"{name} must be a GPU tensor: there is no CPU path")
+    if tuple(t.shape) != tuple(shape):
+        raise RuntimeError(f"{name} must have shape {tuple(shape)}, got {tuple(t.shape)}")
+    return t.contiguous()
+
+
+def _table(tensors):
+    arr = (C.c_void_p * len(tensors))(*[t.data_ptr() for t in tensors])
+    return arr
+
+
+def _param_shapes(k):
+    shapes = []
+    for out in (k, 3 * k, 7 * k):
+        shapes += [(32, 35), (32,), (out, 32), (out,)]
+    return shapes
+
+
+class _NeuralGaussians(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, anchor, feat, offsets, scaling, campos, *params):
+        if len(params) != 12:
+            raise RuntimeError("expected W1, b1, W2, b2 of the opacity, color and cov MLPs (12 tensors)")
+        N = anchor.shape[0]
+        if offsets.dim() != 3:
+            raise RuntimeError("offsets must be (anchors, n_offsets, 3)")
+        k = offsets.shape[1]
+        if not _n.lib.gs_neural_supported(k):
+            raise NotImplementedError(f"n_offsets = {k} is not among the values the kernels are built for")
+        anchor, feat = _f32(anchor, "anchor", (N, 3)), _f32(feat, "feat", (N, 32))
+        offsets, scaling = _f32(offsets, "offsets", (N, k, 3)), _f32(scaling, "scaling", (N, 6))
+        campos = _f32(campos, "camera_center", (3,))
+        params = [_f32(p, f"MLP parameter {i}", s) for i, (p, s) in enumerate(zip(params, _param_shapes(k)))]
+        dev = anchor.device
+        stream = C.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+        neural_opacity = torch.empty(N * k, 1, dtype=torch.float32, device=dev)
+        mask = torch.empty(N * k, dtype=torch.bool, device=dev)
+        first = torch.empty(max(N, 1), dtype=torch.int32, device=dev)
+        ws_bytes = _n.lib.gs_neural_workspace_bytes(N, k)
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+        table = _table(params)
+        S = C.c_int64(0)
+        _n.check(_n.lib.gs_neural_opacity_forward(N, k, _p(anchor), _p(feat), _p(campos), table, _p(neural_opacity),
+                                                  _p(mask), _p(first), _p(ws), ws_bytes, C.byref(S), stream),
+                 "generate_neural_gaussians")
+        S = S.value
+        xyz, color = torch.empty(S, 3, device=dev), torch.empty(S, 3, device=dev)
+        opacity, scal = torch.empty(S, 1, device=dev), torch.empty(S, 3, device=dev)
+        rot, aux = torch.empty(S, 4, device=dev), torch.empty(S, 4, device=dev)
+        _n.check(_n.lib.gs_neural_gaussians_forward(N, k, S, _p(anchor), _p(feat), _p(offsets), _p(scaling),
+                                                    _p(campos), _p(neural_opacity), _p(first), _p(ws), ws_bytes,
+                                                    _p(xyz), _p(color), _p(opacity), _p(scal), _p(rot), _p(aux),
+                                                    stream), "generate_neural_gaussians")
+        ctx.save_for_backward(anchor, feat, offsets, scaling, campos, neural_opacity, first, color, rot, aux, *params)
+        ctx.sizes = (N, k, S)
+        ctx.mark_non_differentiable(neural_opacity, mask)
+        ctx.set_materialize_grads(False)
+        return xyz, color, opacity, scal, rot, neural_opacity, mask
+
+    @staticmethod
+    def backward(ctx, g_xyz, g_color, g_opacity, g_scal, g_rot, _g_nop, _g_mask):
+        anchor, feat, offsets, scaling, campos, neural_opacity, first, color, rot, aux, *params = ctx.saved_tensors
+        N, k, S = ctx.sizes
+        dev = anchor.device
+        ups = []
+        for g, c in ((g_xyz, 3), (g_color, 3), (g_opacity, 1), (g_scal, 3), (g_rot, 4)):
+            ups.append(torch.zeros(S, c, device=dev) if g is None else _f32(g, "upstream gradient", (S, c)))
+        d_anchor, d_feat = torch.empty_like(anchor), torch.empty_like(feat)
+        d_offsets, d_scaling = torch.empty_like(offsets), torch.empty_like(scaling)
+        d_params = [torch.empty_like(p) for p in params]
+        ws_bytes = _n.lib.gs_neural_backward_workspace_bytes(N, k)
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+        stream = C.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+        _n.check(_n.lib.gs_neural_backward(N, k, S, _p(anchor), _p(feat), _p(offsets), _p(scaling), _p(campos),
+                                           _table(params), _p(neural_opacity), _p(first), _p(color), _p(rot), _p(aux),
+                                           *[_p(u) for u in ups], _p(d_anchor), _p(d_feat), _p(d_offsets),
+                                           _p(d_scaling), _table(d_params), _p(ws), ws_bytes, stream),
+                 "generate_neural_gaussians backward")
+        return (d_anchor, d_feat, d_offsets, d_scaling, None, *d_params)
+
+
+def neural_gaussians(anchor, feat, offsets, scaling, camera_center, mlp_opacity, mlp_color, mlp_cov):
+    """The body of generate_neural_gaussians after the visible_mask gathers (gaussian_renderer/__init__.py:800-896).
+    anchor (N,3), feat (N,32), offsets (N,k,3), scaling (N,6) = get_scaling, camera_center (3); each mlp_* is
+    (W1, b1, W2, b2) as nn.Linear holds them.  Returns (xyz, color, opacity, scaling, rot, neural_opacity, mask);
+    differentiable in everything but the camera centre; neural_opacity and mask carry no gradient (the reference
+    uses them detached, scene/gaussian_model.py:1183)."""
+    return _NeuralGaussians.apply(anchor, feat, offsets, scaling, camera_center, *mlp_opacity, *mlp_color, *mlp_cov)
+
+
+def _linear_pair(seq):
+    """(W1, b1, W2, b2) of a Sequential(Linear, ReLU, Linear[, activation]) (scene/gaussian_model.py:131-149)."""
+    return seq[0].weight, seq[0].bias, seq[2].weight, seq[2].bias
+
+
+def generate_neural_gaussians(viewpoint_camera, pc, visible_mask=None, is_training=False, ape_code=-1):
+    """Same signature and results as gaussian_renderer/__init__.py:789-899."""
+    if (pc.use_feat_bank or pc.appearance_dim > 0 or pc.add_opacity_dist or pc.add_color_dist or pc.add_cov_dist
+            or pc.add_level or pc.dist2level == "progressive"):
+        raise NotImplementedError("generate_neural_gaussians: only the default model configuration (no feature bank, "
+                                  "appearance embedding, distance or level inputs, progressive levels) is built")
+    if visible_mask is None:
+        anchor, feat, offsets, scaling = pc.get_anchor, pc.get_anchor_feat, pc._offset, pc.get_scaling
+    else:
+        anchor, feat = pc.get_anchor[visible_mask], pc.get_anchor_feat[visible_mask]
+        offsets, scaling = pc._offset[visible_mask], pc.get_scaling[visible_mask]
+    out = neural_gaussians(anchor, feat, offsets, scaling, viewpoint_camera.camera_center,
+                           _linear_pair(pc.get_opacity_mlp), _linear_pair(pc.get_color_mlp),
+                           _linear_pair(pc.get_cov_mlp))
+    return out if is_training else out[:5]
