@@ -34,6 +34,15 @@ BYTES_PER_GAUSSIAN = {
 # sort: one 8 B histogram read + 5 passes (9-bit digits over the 44 key bits) x (12 B read + 12 B write)
 # tile ranges: 8 B key read, plus the gather of the sorted Gaussian ids fused into it (index, table, output: 12 B)
 BYTES_PER_INSTANCE = {"sort_pairs": 128, "identify_tile_ranges": 20}
+FP32_MATRIX_PEAK_TFLOPS = 157.3
+# Neural-Gaussian generation with 10 offsets: (bytes per anchor, bytes per selected Gaussian, flops per anchor).
+#   opacity:   feat 128 + anchor 12 in; 10 opacities, 10 mask bytes, 1 count out;      2 (35*32 + 32*10) flops
+#   gaussians: feat, anchor, offsets 120, scaling 24, opacities 40, first 4 in; 72 B per Gaussian out (xyz, color,
+#              opacity, scaling, rot, aux);                                            2 (2*35*32 + 32*100) flops
+#   backward:  the same inputs; per Gaussian 56 B of upstream gradients + color, rot, aux 44 B; per anchor
+#              284 B of gradients out; layer 1 again, dH, dX, dW2, dW1:                34240 flops
+NEURAL_COST = {"neural_opacity": (191, 0, 2880), "neural_gaussians": (328, 72, 10880),
+               "neural_backward": (328 + 284, 100, 34240)}
 
 
 def parse():
@@ -134,6 +143,17 @@ def main():
 
     for _ in range(args.warmup):
         step()
+    # inputs of the neural-Gaussian generation stage (timed further down), and one untimed call
+    import gs_neural
+    N_a, k_a = 200_000, 10
+    sc_a = gs_scenes.make_anchor_scene(N_a, k_a, 7)
+    na = {k: sc_a[k].to(dev).requires_grad_(True) for k in ("anchor", "feat", "offsets", "scaling")}
+    na_cam = sc_a["campos"].to(dev)
+    na_mlps = [tuple(x.to(dev).requires_grad_(True) for x in m) for m in sc_a["mlps"]]
+    na_leaves = list(na.values()) + [x for m in na_mlps for x in m]
+    no = gs_neural.neural_gaussians(na["anchor"], na["feat"], na["offsets"], na["scaling"], na_cam, *na_mlps)
+    torch.autograd.backward(list(no[:5]), [torch.ones_like(o) for o in no[:5]])
+    del no
     torch.cuda.synchronize()
     # timed region: exactly `steps` steps, nothing but the work itself on the stream
     t0 = time.perf_counter()
@@ -196,9 +216,35 @@ def main():
         img_l.grad = None
         l1m, ssm = gs_loss.pixelwise_l1_ssim_with_mask(img_l, gt, pm)
         torch.autograd.backward([l1m, ssm], [gt, gt])
+    del l1m, ssm
+    # neural-Gaussian generation for one view: 200 k visible anchors x 10 offsets through the three MLPs,
+    # forward (opacity MLP, scan, color/cov MLPs + post-processing) and backward
+    torch.cuda._sleep(int(4e7))
+    for _ in range(args.steps):
+        for t in na_leaves:
+            t.grad = None
+        no = gs_neural.neural_gaussians(na["anchor"], na["feat"], na["offsets"], na["scaling"], na_cam, *na_mlps)
+        S_a = no[0].shape[0]
+        if "na_up" not in info:
+            info["na_up"] = [torch.randn_like(o) for o in no[:5]]
+        torch.autograd.backward(list(no[:5]), info["na_up"])
     torch.cuda.synchronize()
     gn.stage_timing(False)
     stages = gn.stage_timing_collect()
+    torch_neural_ms = []
+    for _ in range(5):
+        for t in na_leaves:
+            t.grad = None
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        ev0.record()
+        ro = gs_scenes.neural_gaussians_torch(na["anchor"], na["feat"], na["offsets"], na["scaling"], na_cam, na_mlps)
+        ups = info["na_up"] if ro[0].shape[0] == S_a else [torch.ones_like(o) for o in ro[:5]]
+        torch.autograd.backward(list(ro[:5]), ups)
+        ev1.record()
+        torch.cuda.synchronize()
+        torch_neural_ms.append(ev0.elapsed_time(ev1))
+    del no, ro, ups, na, na_mlps, na_leaves
+    info.pop("na_up")
     ms_per_step_instrumented = (t3 - t2) * 1e3 / args.steps
     # the reference's conv2d formulation of the same maps, forward + backward, for reference
     import math
@@ -224,7 +270,7 @@ def main():
         ev1.record()
         torch.cuda.synchronize()
         torch_ssim_ms.append(ev0.elapsed_time(ev1))
-    del gt, pm, img_l, l1m, ssm
+    del gt, pm, img_l
     # the torch statements training_statis consists of, for reference
     torch_stats_ms = []
     for _ in range(5):
@@ -286,6 +332,13 @@ def main():
             nbytes = stats_bytes  # masks, opacities, gradient rows and the read-modify-write of the touched accumulators
         elif name == "adam_step":
             nbytes = 28 * n_adam  # p, g, m, v in; p, m, v out
+        elif name in NEURAL_COST:
+            per_anchor_b, per_gaussian_b, per_anchor_flop = NEURAL_COST[name]
+            nbytes = per_anchor_b * N_a + per_gaussian_b * S_a
+            e["algorithmic_flops"] = per_anchor_flop * N_a
+            if ms > 0:
+                e["TFLOPs"] = round(per_anchor_flop * N_a / (ms * 1e-3) / 1e12, 2)
+                e["frac_of_fp32_matrix_peak"] = round(e["TFLOPs"] / FP32_MATRIX_PEAK_TFLOPS, 4)
         if nbytes is not None and ms > 0:
             e["algorithmic_bytes"] = nbytes
             e["GBps"] = round(nbytes / (ms * 1e-3) / 1e9, 1)
@@ -318,6 +371,8 @@ def main():
         "ssim_l1_torch_reference_ms": round(sorted(torch_ssim_ms)[len(torch_ssim_ms) // 2], 4),
         "training_stats_torch_reference_ms": round(sorted(torch_stats_ms)[len(torch_stats_ms) // 2], 4),
         "all_map_torch_reference_ms": round(sorted(torch_am_ms)[len(torch_am_ms) // 2], 4),
+        "neural_gaussians_torch_reference_ms": round(sorted(torch_neural_ms)[len(torch_neural_ms) // 2], 4),
+        "neural_gaussians_workload": {"anchors": N_a, "n_offsets": k_a, "selected": S_a},
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(g, cam, am_cpu.numpy(), ug_cpu, args.cpu_runs)

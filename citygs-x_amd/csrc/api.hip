@@ -749,8 +749,10 @@ int gs_neural_gaussians_forward(int64_t N, int k, int64_t S, const float* anchor
 }
 
 size_t gs_neural_backward_workspace_bytes(int64_t num_anchors, int n_offsets) {
+  const int64_t n = num_anchors > 0 ? num_anchors : 1;
   return align_up(neural_packed_floats(n_offsets) * sizeof(float), 256) +
-         align_up(neural_partial_floats(n_offsets, num_anchors > 0 ? num_anchors : 1) * sizeof(float), 256) + 256;
+         align_up(neural_slot_grad_floats(n_offsets, n) * sizeof(float), 256) +
+         align_up(neural_partial_floats(n_offsets, n) * sizeof(float), 256) + 256;
 }
 
 int gs_neural_backward(int64_t N, int k, int64_t S, const float* anchor, const float* feat, const float* offsets,
@@ -788,7 +790,8 @@ int gs_neural_backward(int64_t N, int k, int64_t S, const float* anchor, const f
              "gs_neural_backward: workspace missing or too small");
   char* base = align_ptr((char*)workspace, 256);
   float* packed = (float*)base;
-  float* partials = (float*)(base + align_up(neural_packed_floats(k) * sizeof(float), 256));
+  float* slot_grads = (float*)(base + align_up(neural_packed_floats(k) * sizeof(float), 256));
+  float* partials = (float*)((char*)slot_grads + align_up(neural_slot_grad_floats(k, N) * sizeof(float), 256));
   {
     StageScope _t("neural_pack", stream);
     launch_neural_pack(k, mlp_params, packed, stream);
@@ -798,7 +801,7 @@ int gs_neural_backward(int64_t N, int k, int64_t S, const float* anchor, const f
     StageScope _t("neural_backward", stream);
     launch_neural_backward(N, k, anchor, feat, offsets, scaling, campos, packed, neural_opacity, first, color, rot,
                            aux, dL_dxyz, dL_dcolor, dL_dopacity, dL_dscaling, dL_drot, d_anchor, d_feat, d_offsets,
-                           d_scaling, d_mlp_params, partials, stream);
+                           d_scaling, d_mlp_params, slot_grads, partials, stream);
   }
   return check_launch("neural_backward", stream, false);
 }

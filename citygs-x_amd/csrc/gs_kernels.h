@@ -91,8 +91,9 @@ int launch_neural_backward(int64_t N, int k, const float* anchor, const float* f
                            const float* neural_opacity, const uint32_t* first, const float* color_out,
                            const float* rot_out, const float* aux, const float* g_xyz, const float* g_color,
                            const float* g_opacity, const float* g_scal, const float* g_rot, float* d_anchor,
-                           float* d_feat, float* d_offsets, float* d_scaling, float* const* d_params, float* partials,
-                           hipStream_t stream);
+                           float* d_feat, float* d_offsets, float* d_scaling, float* const* d_params,
+                           float* slot_grads, float* partials, hipStream_t stream);
+size_t neural_slot_grad_floats(int k, int64_t N);
 int launch_all_map_fwd(int P, const float* means, const float* scales, const float* rots, const float* V,
                        const float* campos, float* out, hipStream_t stream);
 int launch_all_map_bwd(int P, const float* means, const float* scales, const float* rots, const float* V,

@@ -19,14 +19,16 @@
 namespace gs {
 namespace {
 
-constexpr int NG_WAVES = 4;          // waves per block
+constexpr int NG_WAVES = 4;          // waves per block of the forward kernels
 constexpr int NG_THREADS = 64 * NG_WAVES;
 constexpr int NG_ANCHORS = 32;       // anchors per wave tile
 constexpr int NG_W1_STEPS = 18;      // 36 input slots: 32 features, 3 view components, 1 constant for the bias
-constexpr int NG_W1_SIZE = NG_W1_STEPS * 64;
-constexpr int NG_TILE = 1024;        // one 32x32 operand tile
+constexpr int NG_SLOTS = 2 * NG_W1_STEPS;
+constexpr int NG_TILE = 1024;        // one 32x32 accumulator tile
+constexpr int WS = 33;               // row stride of the weight arrays in LDS (conflict-free both ways)
 constexpr int SX_STRIDE = 37;
 constexpr int SG_STRIDE = 33;
+constexpr int NG_SLOT_GRADS = 11;    // pre-activation gradients per offset: 1 opacity, 3 color, 7 cov
 
 typedef float v16f __attribute__((ext_vector_type(16)));
 
@@ -45,28 +47,24 @@ struct Shape {
   static constexpr int TILES = T0 + T1 + T2;
   static constexpr int APG = 64 / K;                       // anchors per 64-lane slot group
   static constexpr int GROUPS = (NG_ANCHORS + APG - 1) / APG;
-  // rows of the per-tile output-gradient matrix, each MLP's block padded to an even count
+  // row numbering shared by the output-layer weights and the output-gradient matrix: the three MLPs' output
+  // units one after the other, each block padded to an even count
   static constexpr int G0 = 0, G1 = even_up(OUT0), G2 = G1 + even_up(OUT1), GROWS = G2 + even_up(OUT2);
+  static constexpr int BWD_WAVES = GROWS <= 110 ? 4 : 2;   // waves per block of the backward kernel (LDS)
   __host__ __device__ static constexpr int out(int m) { return m == 0 ? OUT0 : m == 1 ? OUT1 : OUT2; }
   __host__ __device__ static constexpr int tiles(int m) { return m == 0 ? T0 : m == 1 ? T1 : T2; }
   __host__ __device__ static constexpr int first_tile(int m) { return m == 0 ? 0 : m == 1 ? T0 : T0 + T1; }
   __host__ __device__ static constexpr int grow(int m) { return m == 0 ? G0 : m == 1 ? G1 : G2; }
 };
 
-// offsets (in floats) of the packed operand arrays
+// The weights as the kernels keep them in LDS (offsets in floats): W1 transposed with the bias as input slot 35,
+// [m][slot][WS]; W2 by output row, [row][WS], pad rows zero; b2 by output row.  With the odd row stride both
+// the row-wise and the column-wise operand reads of the forward and backward products are conflict-free.
 struct PackLayout {
-  int w1, w2, b2, w2t, w1t, w1tv, total;
+  int w1t, w2, b2, total;
 };
-__host__ __device__ inline PackLayout pack_layout(int tiles) {
-  PackLayout L;
-  L.w1 = 0;                           // [3][18*64]  layer-1 A operand: W1[h][xslot], bias in slot 35
-  L.w2 = 3 * NG_W1_SIZE;              // [tiles][16*64] layer-2 A operand: W2[row][hrow(half, s)]
-  L.b2 = L.w2 + tiles * NG_TILE;      // [tiles][32]
-  L.w2t = L.b2 + tiles * 32;          // [tiles][32 rows][32]  W2 rows, zero padded (A operand of dH = W2^T G)
-  L.w1t = L.w2t + tiles * NG_TILE;    // [3][16*64]  W1[hrow(half, s)][i], i < 32   (A operand of dX)
-  L.w1tv = L.w1t + 3 * NG_TILE;       // [3][16*64]  W1[hrow(half, s)][32 + i], i < 3, else 0
-  L.total = L.w1tv + 3 * NG_TILE;
-  return L;
+__host__ __device__ constexpr PackLayout pack_layout(int grows) {
+  return PackLayout{0, 3 * NG_SLOTS * WS, 3 * NG_SLOTS * WS + grows * WS, 3 * NG_SLOTS * WS + grows * WS + grows};
 }
 
 struct MlpParams {
@@ -79,40 +77,20 @@ struct MlpGrads {
 template <int K>
 __global__ void __launch_bounds__(256) neural_pack_kernel(MlpParams w, float* __restrict__ packed) {
   using S = Shape<K>;
-  const PackLayout L = pack_layout(S::TILES);
+  constexpr PackLayout L = pack_layout(S::GROWS);
   const int e = blockIdx.x * 256 + threadIdx.x;
   if (e >= L.total) return;
   float v = 0.0f;
   if (e < L.w2) {
-    const int m = e / NG_W1_SIZE, r = e % NG_W1_SIZE, s = r >> 6, half = (r >> 5) & 1, h = r & 31;
-    const int slot = xslot(half, s);
-    v = slot < 35 ? w.p[4 * m][h * 35 + slot] : w.p[4 * m + 1][h];
-  } else if (e < L.w1t) {
-    // the three per-tile arrays
-    const int which = e < L.b2 ? 0 : e < L.w2t ? 1 : 2;
-    const int rel = e - (which == 0 ? L.w2 : which == 1 ? L.b2 : L.w2t);
-    const int per = which == 1 ? 32 : NG_TILE;
-    const int t = rel / per, r = rel % per;
-    const int m = t < S::T0 ? 0 : t < S::T0 + S::T1 ? 1 : 2;
-    const int lt = t - S::first_tile(m), out = S::out(m);
-    const float* W2 = w.p[4 * m + 2];
-    if (which == 0) {
-      const int s = r >> 6, half = (r >> 5) & 1, row = 32 * lt + (r & 31);
-      v = row < out ? W2[row * 32 + hrow(half, s)] : 0.0f;
-    } else if (which == 1) {
-      const int row = 32 * lt + r;
-      v = row < out ? w.p[4 * m + 3][row] : 0.0f;
-    } else {
-      const int row = 32 * lt + (r >> 5), h = r & 31;
-      v = row < out ? W2[row * 32 + h] : 0.0f;
-    }
+    const int m = e / (NG_SLOTS * WS), r = e % (NG_SLOTS * WS), slot = r / WS, h = r % WS;
+    if (h < 32) v = slot < 35 ? w.p[4 * m][h * 35 + slot] : w.p[4 * m + 1][h];
   } else {
-    const bool view = e >= L.w1tv;
-    const int rel = e - (view ? L.w1tv : L.w1t);
-    const int m = rel / NG_TILE, r = rel % NG_TILE, s = r >> 6, half = (r >> 5) & 1, i = r & 31;
-    const float* W1 = w.p[4 * m];
-    if (!view) v = W1[hrow(half, s) * 35 + i];
-    else v = i < 3 ? W1[hrow(half, s) * 35 + 32 + i] : 0.0f;
+    const bool bias = e >= L.b2;
+    const int rel = e - (bias ? L.b2 : L.w2);
+    const int row = bias ? rel : rel / WS, h = bias ? 0 : rel % WS;
+    const int m = row < S::G1 ? 0 : row < S::G2 ? 1 : 2;
+    const int o = row - S::grow(m);
+    if (o < S::out(m) && h < 32) v = bias ? w.p[4 * m + 3][o] : w.p[4 * m + 2][o * 32 + h];
   }
   packed[e] = v;
 }
@@ -123,26 +101,41 @@ __device__ __forceinline__ void wave_sync() {
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
-__device__ __forceinline__ float sigmoidf(float x) { return 1.0f / (1.0f + expf(-x)); }
+// hardware exp2 and reciprocal: about 1e-6 relative, far inside what float32 MLP outputs carry
+__device__ __forceinline__ float sigmoidf(float x) { return __frcp_rn(1.0f + __expf(-x)); }
 
 // The 18 layer-1 B operands of this lane: its anchor's features of its half, the view direction and the constant.
 // Also returns the unit view direction and the distance (every lane computes both).
-__device__ __forceinline__ void load_x(float (&xb)[NG_W1_STEPS], float (&nv)[3], float& dist, bool valid, int64_t a,
-                                       int half, const float* __restrict__ anchor, const float* __restrict__ feat,
-                                       const float cam[3]) {
+struct XOperand {
+  float4 f[4];
+  float ax, ay, az;
+};
+__device__ __forceinline__ XOperand fetch_x(bool valid, int64_t a, int half, const float* __restrict__ anchor,
+                                            const float* __restrict__ feat) {
+  XOperand x;
   if (valid) {
     const float4* f = (const float4*)(feat + a * 32 + 16 * half);
 #pragma unroll
-    for (int q = 0; q < 4; q++) {
-      const float4 v = f[q];
-      xb[4 * q] = v.x; xb[4 * q + 1] = v.y; xb[4 * q + 2] = v.z; xb[4 * q + 3] = v.w;
-    }
-    const float vx = anchor[a * 3] - cam[0], vy = anchor[a * 3 + 1] - cam[1], vz = anchor[a * 3 + 2] - cam[2];
+    for (int q = 0; q < 4; q++) x.f[q] = f[q];
+    x.ax = anchor[a * 3]; x.ay = anchor[a * 3 + 1]; x.az = anchor[a * 3 + 2];
+  } else {
+#pragma unroll
+    for (int q = 0; q < 4; q++) x.f[q] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    x.ax = x.ay = x.az = 0.0f;
+  }
+  return x;
+}
+__device__ __forceinline__ void unpack_x(float (&xb)[NG_W1_STEPS], float (&nv)[3], float& dist, const XOperand& x,
+                                         bool valid, int half, const float cam[3]) {
+#pragma unroll
+  for (int q = 0; q < 4; q++) {
+    xb[4 * q] = x.f[q].x; xb[4 * q + 1] = x.f[q].y; xb[4 * q + 2] = x.f[q].z; xb[4 * q + 3] = x.f[q].w;
+  }
+  if (valid) {
+    const float vx = x.ax - cam[0], vy = x.ay - cam[1], vz = x.az - cam[2];
     dist = sqrtf((vx * vx + vy * vy) + vz * vz);
     nv[0] = vx / dist; nv[1] = vy / dist; nv[2] = vz / dist;
   } else {
-#pragma unroll
-    for (int q = 0; q < 16; q++) xb[q] = 0.0f;
     nv[0] = nv[1] = nv[2] = 0.0f;
     dist = 1.0f;
   }
@@ -150,23 +143,38 @@ __device__ __forceinline__ void load_x(float (&xb)[NG_W1_STEPS], float (&nv)[3],
   xb[17] = half ? 1.0f : nv[2];
 }
 
-// relu(W1 x + b1) for the wave's 32 anchors; w1 indexed step * 64 + lane
-__device__ __forceinline__ v16f hidden_layer(const float* w1, const float (&xb)[NG_W1_STEPS], int lane) {
+// relu(W1 x + b1) for the wave's 32 anchors; w1t = this MLP's [slot][WS] array
+__device__ __forceinline__ v16f hidden_layer(const float* w1t, const float (&xb)[NG_W1_STEPS], int al, int half) {
   v16f acc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+  const float* lo = w1t + half * 16 * WS + al;  // slots 16 half + s
+  const float* hi = w1t + (32 + half) * WS + al;  // slots 32 + half, 34 + half
 #pragma unroll
-  for (int s = 0; s < NG_W1_STEPS; s++) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(w1[s * 64 + lane], xb[s], acc, 0, 0, 0);
+  for (int s = 0; s < 16; s++) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(lo[s * WS], xb[s], acc, 0, 0, 0);
+  acc = __builtin_amdgcn_mfma_f32_32x32x2f32(hi[0], xb[16], acc, 0, 0, 0);
+  acc = __builtin_amdgcn_mfma_f32_32x32x2f32(hi[2 * WS], xb[17], acc, 0, 0, 0);
 #pragma unroll
   for (int i = 0; i < 16; i++) acc[i] = acc[i] > 0.0f ? acc[i] : 0.0f;
   return acc;
 }
 
-// one 32-row tile of W2 h + b2; w2 indexed step * 64 + lane, b2 by row
-__device__ __forceinline__ v16f output_tile(const float* w2, const float* b2, const v16f& h, int lane, int half) {
+// rows [32 lt, 32 lt + 32) of W2 h + b2 of an MLP with `out` output units; w2, b2 = the MLP's first row
+template <int OUT>
+__device__ __forceinline__ v16f output_tile(const float* w2, const float* b2, int lt, const v16f& h, int al, int half) {
+  const int row = 32 * lt + al;
+  const bool full = 32 * lt + 32 <= OUT;  // uniform
+  const bool live = full || row < OUT;
+  const float* wr = w2 + (live ? row : OUT - 1) * WS + 4 * half;
   v16f acc;
 #pragma unroll
-  for (int i = 0; i < 16; i++) acc[i] = b2[hrow(half, i)];
+  for (int i = 0; i < 16; i++) {
+    const int r = 32 * lt + hrow(half, i);
+    acc[i] = b2[r < OUT ? r : OUT - 1];
+  }
 #pragma unroll
-  for (int s = 0; s < 16; s++) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(w2[s * 64 + lane], h[s], acc, 0, 0, 0);
+  for (int s = 0; s < 16; s++) {
+    const float v = wr[8 * (s >> 2) + (s & 3)];
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(live ? v : 0.0f, h[s], acc, 0, 0, 0);
+  }
   return acc;
 }
 
@@ -186,14 +194,14 @@ neural_opacity_kernel(int64_t N, int ntiles, const float* __restrict__ anchor, c
                       const float* __restrict__ campos, const float* __restrict__ packed,
                       float* __restrict__ neural_opacity, uint8_t* __restrict__ mask, uint8_t* __restrict__ counts) {
   using S = Shape<K>;
-  const PackLayout L = pack_layout(S::TILES);
-  __shared__ float sW1[NG_W1_SIZE];
-  __shared__ float sW2[NG_TILE];
-  __shared__ float sB2[32];
+  constexpr PackLayout L = pack_layout(S::GROWS);
+  __shared__ float sW1[NG_SLOTS * WS];
+  __shared__ float sW2[S::G1 * WS];
+  __shared__ float sB2[S::G1];
   __shared__ float sOp[NG_WAVES][NG_ANCHORS * K];
-  for (int e = threadIdx.x; e < NG_W1_SIZE; e += NG_THREADS) sW1[e] = packed[L.w1 + e];
-  for (int e = threadIdx.x; e < NG_TILE; e += NG_THREADS) sW2[e] = packed[L.w2 + e];
-  if (threadIdx.x < 32) sB2[threadIdx.x] = packed[L.b2 + threadIdx.x];
+  for (int e = threadIdx.x; e < NG_SLOTS * WS; e += NG_THREADS) sW1[e] = packed[L.w1t + e];
+  for (int e = threadIdx.x; e < S::G1 * WS; e += NG_THREADS) sW2[e] = packed[L.w2 + e];
+  for (int e = threadIdx.x; e < S::G1; e += NG_THREADS) sB2[e] = packed[L.b2 + e];
   __syncthreads();
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, half = lane >> 5, al = lane & 31;
   const float cam[3] = {campos[0], campos[1], campos[2]};
@@ -201,9 +209,9 @@ neural_opacity_kernel(int64_t N, int ntiles, const float* __restrict__ anchor, c
   for (int tile = blockIdx.x * NG_WAVES + wave; tile < ntiles; tile += gridDim.x * NG_WAVES) {
     const int64_t a = (int64_t)tile * NG_ANCHORS + al;
     float xb[NG_W1_STEPS], nv[3], dist;
-    load_x(xb, nv, dist, a < N, a, half, anchor, feat, cam);
-    const v16f h = hidden_layer(sW1, xb, lane);
-    const v16f o = output_tile(sW2, sB2, h, lane, half);
+    unpack_x(xb, nv, dist, fetch_x(a < N, a, half, anchor, feat), a < N, half, cam);
+    const v16f h = hidden_layer(sW1, xb, al, half);
+    const v16f o = output_tile<S::OUT0>(sW2, sB2, 0, h, al, half);
 #pragma unroll
     for (int i = 0; i < 16; i++) {
       const int row = hrow(half, i);
@@ -231,7 +239,8 @@ neural_opacity_kernel(int64_t N, int ntiles, const float* __restrict__ anchor, c
 
 // ---------------------------------------------------------------------------------------------------------
 // Step 2: the color and cov MLPs and the post-processing, written straight to each selected Gaussian's row
-// (first[a] = number of selected offsets of all anchors before a).
+// (first[a] = number of selected offsets of all anchors before a).  Everything an offset needs from memory
+// is requested before the matrix products start, so the loads complete behind them.
 template <int K>
 __global__ void __launch_bounds__(NG_THREADS)
 neural_gaussians_kernel(int64_t N, int ntiles, const float* __restrict__ anchor, const float* __restrict__ feat,
@@ -241,38 +250,51 @@ neural_gaussians_kernel(int64_t N, int ntiles, const float* __restrict__ anchor,
                         float* __restrict__ xyz, float* __restrict__ color, float* __restrict__ opacity,
                         float* __restrict__ scal, float* __restrict__ rot, float* __restrict__ aux) {
   using S = Shape<K>;
-  const PackLayout L = pack_layout(S::TILES);
-  constexpr int NT = S::T1 + S::T2;              // tiles of the two MLPs of this kernel
-  constexpr int ROWS = 32 * S::T1 + S::OUT2;     // rows kept: color tiles whole, cov rows up to 7K
-  __shared__ float sW1[2][NG_W1_SIZE];
-  __shared__ float sW2[NT][NG_TILE];
-  __shared__ float sB2[NT * 32];
+  constexpr PackLayout L = pack_layout(S::GROWS);
+  constexpr int WROWS = S::GROWS - S::G1;        // output rows of the two MLPs of this kernel
+  constexpr int ROWS = 32 * S::T1 + S::OUT2;     // result rows kept: color tiles whole, cov rows up to 7K
+  __shared__ float sW1[2 * NG_SLOTS * WS];
+  __shared__ float sW2[WROWS * WS];
+  __shared__ float sB2[WROWS];
   __shared__ float sOut[NG_WAVES][ROWS * SG_STRIDE];
-  for (int e = threadIdx.x; e < 2 * NG_W1_SIZE; e += NG_THREADS) (&sW1[0][0])[e] = packed[L.w1 + NG_W1_SIZE + e];
-  for (int e = threadIdx.x; e < NT * NG_TILE; e += NG_THREADS) (&sW2[0][0])[e] = packed[L.w2 + S::T0 * NG_TILE + e];
-  for (int e = threadIdx.x; e < NT * 32; e += NG_THREADS) sB2[e] = packed[L.b2 + S::T0 * 32 + e];
+  for (int e = threadIdx.x; e < 2 * NG_SLOTS * WS; e += NG_THREADS) sW1[e] = packed[L.w1t + NG_SLOTS * WS + e];
+  for (int e = threadIdx.x; e < WROWS * WS; e += NG_THREADS) sW2[e] = packed[L.w2 + S::G1 * WS + e];
+  for (int e = threadIdx.x; e < WROWS; e += NG_THREADS) sB2[e] = packed[L.b2 + S::G1 + e];
   __syncthreads();
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, half = lane >> 5, al = lane & 31;
   const float cam[3] = {campos[0], campos[1], campos[2]};
   float* out = sOut[wave];
   for (int tile = blockIdx.x * NG_WAVES + wave; tile < ntiles; tile += gridDim.x * NG_WAVES) {
     const int64_t a = (int64_t)tile * NG_ANCHORS + al;
+    const XOperand xo = fetch_x(a < N, a, half, anchor, feat);
+    // per offset of this lane: opacity and row base, requested before the matrix products start
+    float s_t[S::GROUPS];
+    uint32_t s_first[S::GROUPS];
+#pragma unroll
+    for (int g = 0; g < S::GROUPS; g++) {
+      const int idx = g * S::APG * K + lane;
+      const int ax = idx / K;
+      const int64_t sa = (int64_t)tile * NG_ANCHORS + ax;
+      const bool ok = lane < S::APG * K && ax < NG_ANCHORS && sa < N;
+      s_t[g] = ok ? neural_opacity[sa * K + idx % K] : 0.0f;
+      s_first[g] = ok ? first[sa] : 0u;
+    }
     float xb[NG_W1_STEPS], nv[3], dist;
-    load_x(xb, nv, dist, a < N, a, half, anchor, feat, cam);
+    unpack_x(xb, nv, dist, xo, a < N, half, cam);
     {
-      const v16f h = hidden_layer(sW1[0], xb, lane);
+      const v16f h = hidden_layer(sW1, xb, al, half);
 #pragma unroll
       for (int t = 0; t < S::T1; t++) {
-        const v16f o = output_tile(sW2[t], sB2 + 32 * t, h, lane, half);
+        const v16f o = output_tile<S::OUT1>(sW2, sB2, t, h, al, half);
 #pragma unroll
         for (int i = 0; i < 16; i++) out[(32 * t + hrow(half, i)) * SG_STRIDE + al] = o[i];
       }
     }
     {
-      const v16f h = hidden_layer(sW1[1], xb, lane);
+      const v16f h = hidden_layer(sW1 + NG_SLOTS * WS, xb, al, half);
 #pragma unroll
       for (int t = 0; t < S::T2; t++) {
-        const v16f o = output_tile(sW2[S::T1 + t], sB2 + 32 * (S::T1 + t), h, lane, half);
+        const v16f o = output_tile<S::OUT2>(sW2 + (S::G2 - S::G1) * WS, sB2 + (S::G2 - S::G1), t, h, al, half);
 #pragma unroll
         for (int i = 0; i < 16; i++) {
           const int row = 32 * t + hrow(half, i);
@@ -281,24 +303,22 @@ neural_gaussians_kernel(int64_t N, int ntiles, const float* __restrict__ anchor,
       }
     }
     wave_sync();
-#pragma unroll 1
+#pragma unroll
     for (int g = 0; g < S::GROUPS; g++) {
       const int idx = g * S::APG * K + lane;
       const int ax = idx / K, j = idx % K;
-      const int64_t sa = (int64_t)tile * NG_ANCHORS + ax;
-      const bool ok = lane < S::APG * K && ax < NG_ANCHORS && sa < N;
-      const int64_t slot = sa * K + j;
-      const float t = ok ? neural_opacity[slot] : 0.0f;
+      const float t = s_t[g];
       const bool sel = t > 0.0f;
       const unsigned long long bits = __ballot(sel);
       if (sel) {
-        const int64_t r = (int64_t)first[sa] + count_lanes(bits, lane - j, lane);
+        const int64_t r = (int64_t)s_first[g] + count_lanes(bits, lane - j, lane);
+        const int64_t sa = (int64_t)tile * NG_ANCHORS + ax;
         const float* sc = scaling + sa * 6;
         const float* cv = out + (32 * S::T1 + 7 * j) * SG_STRIDE + ax;
         float sg[3];
 #pragma unroll
         for (int c = 0; c < 3; c++) {
-          xyz[r * 3 + c] = anchor[sa * 3 + c] + offsets[slot * 3 + c] * sc[c];
+          xyz[r * 3 + c] = anchor[sa * 3 + c] + offsets[(sa * K + j) * 3 + c] * sc[c];
           color[r * 3 + c] = sigmoidf(out[(3 * j + c) * SG_STRIDE + ax]);
           sg[c] = sigmoidf(cv[c * SG_STRIDE]);
           scal[r * 3 + c] = sc[3 + c] * sg[c];
@@ -316,20 +336,106 @@ neural_gaussians_kernel(int64_t N, int ntiles, const float* __restrict__ anchor,
 }
 
 // ---------------------------------------------------------------------------------------------------------
-// Backward.  Per wave tile: the gradients of the selected Gaussians become the pre-activation gradients G of
-// the three output layers (a GROWS x 32 matrix in LDS, zero for unselected offsets); then per MLP
+// Backward, first kernel: everything that is per offset.  The gradients of a selected Gaussian's five outputs
+// become the 11 pre-activation gradients of its offset's output units (zero for unselected offsets), written
+// as one record per offset; the direct gradients of offsets, scaling and anchor (xyz = anchor + offset * scaling)
+// are finished here, the per-anchor sums running over an anchor's offsets in order.
+template <int K>
+__global__ void __launch_bounds__(NG_THREADS)
+neural_offset_backward_kernel(int64_t N, int ntiles, const float* __restrict__ offsets,
+                              const float* __restrict__ scaling, const float* __restrict__ neural_opacity,
+                              const uint32_t* __restrict__ first, const float* __restrict__ color_out,
+                              const float* __restrict__ rot_out, const float* __restrict__ aux,
+                              const float* __restrict__ g_xyz, const float* __restrict__ g_color,
+                              const float* __restrict__ g_opacity, const float* __restrict__ g_scal,
+                              const float* __restrict__ g_rot, float* __restrict__ slot_grads,
+                              float* __restrict__ d_anchor, float* __restrict__ d_offsets,
+                              float* __restrict__ d_scaling) {
+  using S = Shape<K>;
+  __shared__ float sC[NG_WAVES][64 * 9];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int tile = blockIdx.x * NG_WAVES + wave;
+  if (tile >= ntiles) return;  // no workgroup barrier below
+  float* con_s = sC[wave];
+#pragma unroll 1
+  for (int g = 0; g < S::GROUPS; g++) {
+    const int idx = g * S::APG * K + lane;
+    const int ax = idx / K, j = idx % K;
+    const int64_t sa = (int64_t)tile * NG_ANCHORS + ax;
+    const bool ok = lane < S::APG * K && ax < NG_ANCHORS && sa < N;
+    const int64_t slot = sa * K + j;
+    const float t = ok ? neural_opacity[slot] : 0.0f;
+    const bool sel = t > 0.0f;
+    const unsigned long long bits = __ballot(sel);
+    float grad[NG_SLOT_GRADS] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+    float con[9] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f}, dof[3] = {0.0f, 0.0f, 0.0f};
+    if (sel) {
+      const int64_t r = (int64_t)first[sa] + count_lanes(bits, lane - j, lane);
+      const float* sc = scaling + sa * 6;
+      grad[0] = g_opacity[r] * (1.0f - t * t);
+      const float4 ax4 = *(const float4*)(aux + r * 4);
+      const float sg[3] = {ax4.x, ax4.y, ax4.z};
+#pragma unroll
+      for (int c = 0; c < 3; c++) {
+        const float cs = color_out[r * 3 + c];
+        grad[1 + c] = g_color[r * 3 + c] * (cs * (1.0f - cs));
+        const float gx = g_xyz[r * 3 + c], gs = g_scal[r * 3 + c];
+        con[c] = gx;
+        dof[c] = gx * sc[c];
+        con[3 + c] = gx * offsets[slot * 3 + c];
+        con[6 + c] = gs * sg[c];
+        grad[4 + c] = gs * sc[3 + c] * (sg[c] * (1.0f - sg[c]));
+      }
+      const float len = ax4.w;
+      const float4 gr = *(const float4*)(g_rot + r * 4);
+      if (len > 1e-12f) {
+        const float4 qh = *(const float4*)(rot_out + r * 4);
+        const float dot = ((qh.x * gr.x + qh.y * gr.y) + qh.z * gr.z) + qh.w * gr.w;
+        grad[7] = (gr.x - qh.x * dot) / len; grad[8] = (gr.y - qh.y * dot) / len;
+        grad[9] = (gr.z - qh.z * dot) / len; grad[10] = (gr.w - qh.w * dot) / len;
+      } else {
+        grad[7] = gr.x / 1e-12f; grad[8] = gr.y / 1e-12f; grad[9] = gr.z / 1e-12f; grad[10] = gr.w / 1e-12f;
+      }
+    }
+    if (ok) {
+#pragma unroll
+      for (int c = 0; c < NG_SLOT_GRADS; c++) slot_grads[slot * NG_SLOT_GRADS + c] = grad[c];
+#pragma unroll
+      for (int c = 0; c < 3; c++) d_offsets[slot * 3 + c] = dof[c];
+    }
+#pragma unroll
+    for (int c = 0; c < 9; c++) con_s[lane * 9 + c] = con[c];
+    wave_sync();
+    for (int item = lane; item < S::APG * 9; item += 64) {
+      const int ga = item / 9, comp = item % 9;
+      const int ax2 = g * S::APG + ga;
+      const int64_t sa2 = (int64_t)tile * NG_ANCHORS + ax2;
+      if (ax2 < NG_ANCHORS && sa2 < N) {
+        float sum = 0.0f;
+#pragma unroll
+        for (int jj = 0; jj < K; jj++) sum += con_s[(ga * K + jj) * 9 + comp];
+        if (comp < 3) d_anchor[sa2 * 3 + comp] = sum;
+        else d_scaling[sa2 * 6 + (comp - 3)] = sum;
+      }
+    }
+    wave_sync();
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// Backward, second kernel: through the MLPs.  Per wave tile, with G the GROWS x 32 matrix of the tile's
+// pre-activation output gradients, and per MLP
 //   H = relu(W1 x + b1) (recomputed), dH = W2^T G, dHpre = dH where H > 0, dX += W1^T dHpre,
 //   dW2 += G H^T, [dW1 | db1] += dHpre [x | 1]^T, db2 += row sums of G,
-// with the weight gradients kept in matrix-core accumulators over all tiles of the wave and reduced over the
-// block at the end (one partial set per block; a second kernel adds the blocks in a fixed order).
+// the weight gradients staying in matrix-core accumulators over all tiles of the wave; they are reduced over the
+// block at the end (one partial set per block; a last kernel adds the blocks in a fixed order).  The next tile's
+// features and gradient records are requested before the current tile's products start.
 template <int K>
 struct BwdLds {
   using S = Shape<K>;
   float g[S::GROWS * SG_STRIDE];
   float hd[2 * 32 * SG_STRIDE];  // H, then dHpre; also the staging area of the final block reduction
   float x[NG_ANCHORS * SX_STRIDE];
-  float c[64 * 9];
-  float da[NG_ANCHORS * 3];
 };
 
 // floats of one block's partial weight gradients: W2 tiles, then W1 (3 MLPs x 2 column tiles), then b2 rows
@@ -339,27 +445,34 @@ __host__ __device__ constexpr int partial_floats() {
 }
 
 template <int K>
-__global__ void __launch_bounds__(NG_THREADS)
-neural_backward_kernel(int64_t N, int ntiles, const float* __restrict__ anchor, const float* __restrict__ feat,
-                       const float* __restrict__ offsets, const float* __restrict__ scaling,
-                       const float* __restrict__ campos, const float* __restrict__ packed,
-                       const float* __restrict__ neural_opacity, const uint32_t* __restrict__ first,
-                       const float* __restrict__ color_out, const float* __restrict__ rot_out,
-                       const float* __restrict__ aux, const float* __restrict__ g_xyz,
-                       const float* __restrict__ g_color, const float* __restrict__ g_opacity,
-                       const float* __restrict__ g_scal, const float* __restrict__ g_rot,
-                       float* __restrict__ d_anchor, float* __restrict__ d_feat, float* __restrict__ d_offsets,
-                       float* __restrict__ d_scaling, float* __restrict__ partials) {
+__global__ void __launch_bounds__(64 * Shape<K>::BWD_WAVES)
+neural_mlp_backward_kernel(int64_t N, int ntiles, const float* __restrict__ anchor, const float* __restrict__ feat,
+                           const float* __restrict__ campos, const float* __restrict__ packed,
+                           const float* __restrict__ slot_grads, float* __restrict__ d_anchor,
+                           float* __restrict__ d_feat, float* __restrict__ partials) {
   using S = Shape<K>;
-  const PackLayout L = pack_layout(S::TILES);
+  constexpr PackLayout L = pack_layout(S::GROWS);
+  constexpr int NW = S::BWD_WAVES, NT = 64 * NW;
   constexpr int B2N = (S::GROWS + 63) / 64;
-  __shared__ BwdLds<K> lds[NG_WAVES];
+  constexpr int TILE_FLOATS = NG_ANCHORS * K * NG_SLOT_GRADS;
+  constexpr int NQ = (TILE_FLOATS / 4 + 63) / 64;  // float4 loads per lane and tile
+  __shared__ BwdLds<K> lds[NW];
+  __shared__ float sW1[3 * NG_SLOTS * WS];
+  __shared__ float sW2[S::GROWS * WS];
+  __shared__ unsigned short sWhere[TILE_FLOATS];  // where in G each float of a tile's records goes
+  for (int e = threadIdx.x; e < 3 * NG_SLOTS * WS; e += NT) sW1[e] = packed[L.w1t + e];
+  for (int e = threadIdx.x; e < S::GROWS * WS; e += NT) sW2[e] = packed[L.w2 + e];
+  for (int e = threadIdx.x; e < TILE_FLOATS; e += NT) {
+    const int slot = e / NG_SLOT_GRADS, comp = e % NG_SLOT_GRADS, ax = slot / K, j = slot % K;
+    const int row = comp == 0 ? S::G0 + j : comp < 4 ? S::G1 + 3 * j + (comp - 1) : S::G2 + 7 * j + (comp - 4);
+    sWhere[e] = (unsigned short)(row * SG_STRIDE + ax);
+  }
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, half = lane >> 5, al = lane & 31;
   const float cam[3] = {campos[0], campos[1], campos[2]};
   BwdLds<K>& W = lds[wave];
   // rows that pad a block of G to an even count are read by the dH products and never written below
   for (int e = lane; e < S::GROWS * SG_STRIDE; e += 64) W.g[e] = 0.0f;
-  wave_sync();
+  __syncthreads();
 
   v16f accW2[S::TILES], accW1[3][2];
   float accB2[B2N];
@@ -374,109 +487,73 @@ neural_backward_kernel(int64_t N, int ntiles, const float* __restrict__ anchor, 
 #pragma unroll
   for (int q = 0; q < B2N; q++) accB2[q] = 0.0f;
 
-  for (int tile = blockIdx.x * NG_WAVES + wave; tile < ntiles; tile += gridDim.x * NG_WAVES) {
+  const int64_t total_floats = N * K * NG_SLOT_GRADS;
+  const int stride = gridDim.x * NW;
+  int tile = blockIdx.x * NW + wave;
+  XOperand xo;
+  float4 gq[NQ];
+  auto fetch_tile = [&](int t) {
+    const int64_t a = (int64_t)t * NG_ANCHORS + al;
+    xo = fetch_x(a < N, a, half, anchor, feat);
+    const int64_t base = (int64_t)t * TILE_FLOATS;
+#pragma unroll
+    for (int q = 0; q < NQ; q++) {
+      const int e = (q * 64 + lane) * 4;
+      // the buffer is padded, so a float4 that straddles the end is readable; its tail is dropped below
+      gq[q] = (e < TILE_FLOATS && base + e < total_floats) ? *(const float4*)(slot_grads + base + e)
+                                                           : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    }
+  };
+  if (tile < ntiles) fetch_tile(tile);
+  for (; tile < ntiles; tile += stride) {
     const int64_t a = (int64_t)tile * NG_ANCHORS + al;
     const bool valid = a < N;
     float xb[NG_W1_STEPS], nv[3], dist;
-    load_x(xb, nv, dist, valid, a, half, anchor, feat, cam);
+    unpack_x(xb, nv, dist, xo, valid, half, cam);
 #pragma unroll
     for (int s = 0; s < NG_W1_STEPS; s++) W.x[al * SX_STRIDE + xslot(half, s)] = xb[s];
-
-    // ---- per offset: output gradients -> G, direct gradients of offsets, scaling and anchor
-#pragma unroll 1
-    for (int g = 0; g < S::GROUPS; g++) {
-      const int idx = g * S::APG * K + lane;
-      const int ax = idx / K, j = idx % K;
-      const int64_t sa = (int64_t)tile * NG_ANCHORS + ax;
-      const bool in_group = lane < S::APG * K && ax < NG_ANCHORS;
-      const bool ok = in_group && sa < N;
-      const int64_t slot = sa * K + j;
-      const float t = ok ? neural_opacity[slot] : 0.0f;
-      const bool sel = t > 0.0f;
-      const unsigned long long bits = __ballot(sel);
-      float go = 0.0f, gc[3] = {0.0f, 0.0f, 0.0f}, gv[7] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
-      float con[9] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f}, dof[3] = {0.0f, 0.0f, 0.0f};
-      if (sel) {
-        const int64_t r = (int64_t)first[sa] + count_lanes(bits, lane - j, lane);
-        const float* sc = scaling + sa * 6;
-        go = g_opacity[r] * (1.0f - t * t);
-        const float4 ax4 = *(const float4*)(aux + r * 4);
-        const float sg[3] = {ax4.x, ax4.y, ax4.z};
+    {
+      const int64_t base = (int64_t)tile * TILE_FLOATS;
 #pragma unroll
-        for (int c = 0; c < 3; c++) {
-          const float cs = color_out[r * 3 + c];
-          gc[c] = g_color[r * 3 + c] * (cs * (1.0f - cs));
-          const float gx = g_xyz[r * 3 + c], gs = g_scal[r * 3 + c];
-          con[c] = gx;
-          dof[c] = gx * sc[c];
-          con[3 + c] = gx * offsets[slot * 3 + c];
-          con[6 + c] = gs * sg[c];
-          gv[c] = gs * sc[3 + c] * (sg[c] * (1.0f - sg[c]));
-        }
-        const float len = ax4.w;
-        const float4 gr = *(const float4*)(g_rot + r * 4);
-        if (len > 1e-12f) {
-          const float4 qh = *(const float4*)(rot_out + r * 4);
-          const float dot = ((qh.x * gr.x + qh.y * gr.y) + qh.z * gr.z) + qh.w * gr.w;
-          gv[3] = (gr.x - qh.x * dot) / len; gv[4] = (gr.y - qh.y * dot) / len;
-          gv[5] = (gr.z - qh.z * dot) / len; gv[6] = (gr.w - qh.w * dot) / len;
-        } else {
-          gv[3] = gr.x / 1e-12f; gv[4] = gr.y / 1e-12f; gv[5] = gr.z / 1e-12f; gv[6] = gr.w / 1e-12f;
+      for (int q = 0; q < NQ; q++) {
+        const int e = (q * 64 + lane) * 4;
+        if (e < TILE_FLOATS) {
+          const float v[4] = {gq[q].x, gq[q].y, gq[q].z, gq[q].w};
+#pragma unroll
+          for (int c = 0; c < 4; c++) W.g[sWhere[e + c]] = base + e + c < total_floats ? v[c] : 0.0f;
         }
       }
-      if (in_group) {
-        W.g[(S::G0 + j) * SG_STRIDE + ax] = go;
-#pragma unroll
-        for (int c = 0; c < 3; c++) W.g[(S::G1 + 3 * j + c) * SG_STRIDE + ax] = gc[c];
-#pragma unroll
-        for (int c = 0; c < 7; c++) W.g[(S::G2 + 7 * j + c) * SG_STRIDE + ax] = gv[c];
-#pragma unroll
-        for (int c = 0; c < 9; c++) W.c[lane * 9 + c] = con[c];
-      }
-      if (ok) {
-#pragma unroll
-        for (int c = 0; c < 3; c++) d_offsets[slot * 3 + c] = dof[c];
-      }
-      wave_sync();
-      // sums over the offsets of an anchor, in offset order
-      for (int item = lane; item < S::APG * 9; item += 64) {
-        const int ga = item / 9, comp = item % 9;
-        const int ax2 = g * S::APG + ga;
-        const int64_t sa2 = (int64_t)tile * NG_ANCHORS + ax2;
-        if (ax2 < NG_ANCHORS && sa2 < N) {
-          float sum = 0.0f;
-#pragma unroll
-          for (int jj = 0; jj < K; jj++) sum += W.c[(ga * K + jj) * 9 + comp];
-          if (comp < 3) W.da[ax2 * 3 + comp] = sum;
-          else d_scaling[sa2 * 6 + (comp - 3)] = sum;
-        }
-      }
-      wave_sync();
     }
+    wave_sync();
+    if (tile + stride < ntiles) fetch_tile(tile + stride);
 
-    // ---- through the MLPs
     v16f dxf = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0}, dxv = dxf;
 #pragma unroll
     for (int m = 0; m < 3; m++) {
-      const v16f h = hidden_layer(packed + L.w1 + m * NG_W1_SIZE, xb, lane);
+      const float* w1t = sW1 + m * NG_SLOTS * WS;
+      const v16f h = hidden_layer(w1t, xb, al, half);
       v16f dh = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+      {
+        // dH = W2^T G over this MLP's rows (pad row included: zero on both sides)
+        const float* w2r = sW2 + (S::grow(m) + half) * WS + al;
+        const float* gr = W.g + (S::grow(m) + half) * SG_STRIDE + al;
 #pragma unroll
-      for (int lt = 0; lt < S::tiles(m); lt++) {
-        const int rows = S::out(m) - 32 * lt < 32 ? S::out(m) - 32 * lt : 32;
-        const float* w2t = packed + L.w2t + (S::first_tile(m) + lt) * NG_TILE;
-        const float* gt = W.g + (S::grow(m) + 32 * lt) * SG_STRIDE;
-#pragma unroll
-        for (int s = 0; s < (rows + 1) / 2; s++)
-          dh = __builtin_amdgcn_mfma_f32_32x32x2f32(w2t[s * 64 + lane], gt[(2 * s + half) * SG_STRIDE + al], dh, 0, 0, 0);
+        for (int s = 0; s < even_up(S::out(m)) / 2; s++)
+          dh = __builtin_amdgcn_mfma_f32_32x32x2f32(w2r[2 * s * WS], gr[2 * s * SG_STRIDE], dh, 0, 0, 0);
       }
 #pragma unroll
       for (int i = 0; i < 16; i++) dh[i] = h[i] > 0.0f ? dh[i] : 0.0f;
-      const float* w1t = packed + L.w1t + m * NG_TILE;
-      const float* w1tv = packed + L.w1tv + m * NG_TILE;
+      {
+        // dX += W1^T dHpre: rows = the 32 features, then the 3 view components
+        const float* wf = w1t + al * WS + 4 * half;
+        const float* wv = w1t + (32 + (al < 3 ? al : 2)) * WS + 4 * half;
 #pragma unroll
-      for (int s = 0; s < 16; s++) {
-        dxf = __builtin_amdgcn_mfma_f32_32x32x2f32(w1t[s * 64 + lane], dh[s], dxf, 0, 0, 0);
-        dxv = __builtin_amdgcn_mfma_f32_32x32x2f32(w1tv[s * 64 + lane], dh[s], dxv, 0, 0, 0);
+        for (int s = 0; s < 16; s++) {
+          const int hc = 8 * (s >> 2) + (s & 3);
+          dxf = __builtin_amdgcn_mfma_f32_32x32x2f32(wf[hc], dh[s], dxf, 0, 0, 0);
+          const float v = wv[hc];
+          dxv = __builtin_amdgcn_mfma_f32_32x32x2f32(al < 3 ? v : 0.0f, dh[s], dxv, 0, 0, 0);
+        }
       }
 #pragma unroll
       for (int i = 0; i < 16; i++) {
@@ -520,15 +597,16 @@ neural_backward_kernel(int64_t N, int ntiles, const float* __restrict__ anchor, 
       for (int q = 0; q < 4; q++)
         *(float4*)(d_feat + a * 32 + 8 * q + 4 * half) = make_float4(dxf[4 * q], dxf[4 * q + 1], dxf[4 * q + 2], dxf[4 * q + 3]);
       if (half == 0) {
+        // the view direction n = v / |v| adds (g - n (n.g)) / |v| to the anchor's direct gradient
         const float ng = (nv[0] * dxv[0] + nv[1] * dxv[1]) + nv[2] * dxv[2];
 #pragma unroll
-        for (int c = 0; c < 3; c++) d_anchor[a * 3 + c] = W.da[al * 3 + c] + (dxv[c] - nv[c] * ng) / dist;
+        for (int c = 0; c < 3; c++) d_anchor[a * 3 + c] = d_anchor[a * 3 + c] + (dxv[c] - nv[c] * ng) / dist;
       }
     }
     wave_sync();
   }
 
-  // ---- reduce the four waves' accumulators, one 32x32 tile at a time, through each wave's staging area
+  // ---- reduce the waves' accumulators, one 32x32 tile at a time, through each wave's staging area
   float* out = partials + (size_t)blockIdx.x * partial_floats<K>();
   constexpr int NACC = S::TILES + 6;
 #pragma unroll
@@ -538,66 +616,87 @@ neural_backward_kernel(int64_t N, int ntiles, const float* __restrict__ anchor, 
 #pragma unroll
     for (int i = 0; i < 16; i++) W.hd[hrow(half, i) * 32 + al] = acc[i];
     __syncthreads();
-    for (int e = threadIdx.x; e < NG_TILE; e += NG_THREADS)
-      out[t * NG_TILE + e] = ((lds[0].hd[e] + lds[1].hd[e]) + lds[2].hd[e]) + lds[3].hd[e];
+    for (int e = threadIdx.x; e < NG_TILE; e += NT) {
+      float sum = lds[0].hd[e];
+#pragma unroll
+      for (int w = 1; w < NW; w++) sum += lds[w].hd[e];
+      out[t * NG_TILE + e] = sum;
+    }
   }
   __syncthreads();
 #pragma unroll
   for (int q = 0; q < B2N; q++) W.hd[q * 64 + lane] = accB2[q];
   __syncthreads();
-  for (int e = threadIdx.x; e < B2N * 64; e += NG_THREADS)
-    out[NACC * NG_TILE + e] = ((lds[0].hd[e] + lds[1].hd[e]) + lds[2].hd[e]) + lds[3].hd[e];
+  for (int e = threadIdx.x; e < B2N * 64; e += NT) {
+    float sum = lds[0].hd[e];
+#pragma unroll
+    for (int w = 1; w < NW; w++) sum += lds[w].hd[e];
+    out[NACC * NG_TILE + e] = sum;
+  }
 }
 
-// Adds the blocks' partial sets in block order and writes the twelve weight gradients.
+// Adds the blocks' partial sets and writes the twelve weight gradients.  16 threads share an output element:
+// each adds every 16th block's value, then the 16 sums are added in thread order (a fixed order for a given
+// launch geometry, so results repeat bit for bit).
 template <int K>
 __global__ void __launch_bounds__(256)
 neural_weight_reduce_kernel(int nblocks, const float* __restrict__ partials, MlpGrads d) {
   using S = Shape<K>;
   constexpr int PER_MLP_1 = 32 * 35 + 32;
   constexpr int TOTAL = 3 * PER_MLP_1 + 33 * (S::OUT0 + S::OUT1 + S::OUT2);
-  const int e = blockIdx.x * 256 + threadIdx.x;
-  if (e >= TOTAL) return;
-  int src;      // index inside a partial set
-  float* dst;
-  if (e < 3 * PER_MLP_1) {
-    const int m = e / PER_MLP_1, r = e % PER_MLP_1;
-    if (r < 32 * 35) {
-      const int h = r / 35, i = r % 35;
-      src = (S::TILES + 2 * m + (i >= 32)) * NG_TILE + h * 32 + (i & 31);
-      dst = d.p[4 * m] + r;
+  __shared__ float s_part[16][17];
+  const int el = threadIdx.x & 15, part = threadIdx.x >> 4;
+  const int e = blockIdx.x * 16 + el;
+  int src = 0;  // index inside a partial set
+  float* dst = nullptr;
+  if (e < TOTAL) {
+    if (e < 3 * PER_MLP_1) {
+      const int m = e / PER_MLP_1, r = e % PER_MLP_1;
+      if (r < 32 * 35) {
+        const int h = r / 35, i = r % 35;
+        src = (S::TILES + 2 * m + (i >= 32)) * NG_TILE + h * 32 + (i & 31);
+        dst = d.p[4 * m] + r;
+      } else {
+        const int h = r - 32 * 35;
+        src = (S::TILES + 2 * m + 1) * NG_TILE + h * 32 + 3;
+        dst = d.p[4 * m + 1] + h;
+      }
     } else {
-      const int h = r - 32 * 35;
-      src = (S::TILES + 2 * m + 1) * NG_TILE + h * 32 + 3;
-      dst = d.p[4 * m + 1] + h;
-    }
-  } else {
-    int r = e - 3 * PER_MLP_1;
-    int m = 0;
-    while (r >= 33 * S::out(m)) { r -= 33 * S::out(m); m++; }
-    const int out = S::out(m);
-    if (r < 32 * out) {
-      const int row = r / 32, h = r % 32;
-      src = (S::first_tile(m) + row / 32) * NG_TILE + (row % 32) * 32 + h;
-      dst = d.p[4 * m + 2] + r;
-    } else {
-      const int row = r - 32 * out;
-      src = (S::TILES + 6) * NG_TILE + S::grow(m) + row;
-      dst = d.p[4 * m + 3] + row;
+      int r = e - 3 * PER_MLP_1;
+      int m = 0;
+      while (r >= 33 * S::out(m)) { r -= 33 * S::out(m); m++; }
+      const int out = S::out(m);
+      if (r < 32 * out) {
+        const int row = r / 32, h = r % 32;
+        src = (S::first_tile(m) + row / 32) * NG_TILE + (row % 32) * 32 + h;
+        dst = d.p[4 * m + 2] + r;
+      } else {
+        const int row = r - 32 * out;
+        src = (S::TILES + 6) * NG_TILE + S::grow(m) + row;
+        dst = d.p[4 * m + 3] + row;
+      }
     }
   }
   float sum = 0.0f;
-  for (int b = 0; b < nblocks; b++) sum += partials[(size_t)b * partial_floats<K>() + src];
-  *dst = sum;
+  if (e < TOTAL)
+    for (int b = part; b < nblocks; b += 16) sum += partials[(size_t)b * partial_floats<K>() + src];
+  s_part[part][el] = sum;
+  __syncthreads();
+  if (part == 0 && e < TOTAL) {
+    float total = s_part[0][el];
+#pragma unroll
+    for (int q = 1; q < 16; q++) total += s_part[q][el];
+    *dst = total;
+  }
 }
 
-int blocks_for(int ntiles, int per_cu) {
+int blocks_for(int ntiles, int waves_per_block, int per_cu) {
   int dev = 0, cus = 256;
   if (hipGetDevice(&dev) == hipSuccess) {
     int v = 0;
     if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0) cus = v;
   }
-  const int want = (ntiles + NG_WAVES - 1) / NG_WAVES;
+  const int want = (ntiles + waves_per_block - 1) / waves_per_block;
   const int cap = cus * per_cu;
   return want < cap ? want : cap;
 }
@@ -608,40 +707,44 @@ struct Launcher {
   static void pack(const float* const* params, float* packed, hipStream_t stream) {
     MlpParams w;
     for (int i = 0; i < 12; i++) w.p[i] = params[i];
-    const int total = pack_layout(S::TILES).total;
+    const int total = pack_layout(S::GROWS).total;
     hipLaunchKernelGGL(neural_pack_kernel<K>, dim3((total + 255) / 256), dim3(256), 0, stream, w, packed);
   }
   static void opacity(int64_t N, const float* anchor, const float* feat, const float* campos, const float* packed,
                       float* neural_opacity, uint8_t* mask, uint8_t* counts, hipStream_t stream) {
     const int ntiles = (int)((N + NG_ANCHORS - 1) / NG_ANCHORS);
-    hipLaunchKernelGGL(neural_opacity_kernel<K>, dim3(blocks_for(ntiles, 4)), dim3(NG_THREADS), 0, stream, N, ntiles,
-                       anchor, feat, campos, packed, neural_opacity, mask, counts);
+    hipLaunchKernelGGL(neural_opacity_kernel<K>, dim3(blocks_for(ntiles, NG_WAVES, 4)), dim3(NG_THREADS), 0, stream,
+                       N, ntiles, anchor, feat, campos, packed, neural_opacity, mask, counts);
   }
   static void gaussians(int64_t N, const float* anchor, const float* feat, const float* offsets, const float* scaling,
                         const float* campos, const float* packed, const float* neural_opacity, const uint32_t* first,
                         float* xyz, float* color, float* opacity, float* scal, float* rot, float* aux,
                         hipStream_t stream) {
     const int ntiles = (int)((N + NG_ANCHORS - 1) / NG_ANCHORS);
-    hipLaunchKernelGGL(neural_gaussians_kernel<K>, dim3(blocks_for(ntiles, 2)), dim3(NG_THREADS), 0, stream, N, ntiles,
-                       anchor, feat, offsets, scaling, campos, packed, neural_opacity, first, xyz, color, opacity,
-                       scal, rot, aux);
+    hipLaunchKernelGGL(neural_gaussians_kernel<K>, dim3(blocks_for(ntiles, NG_WAVES, 2)), dim3(NG_THREADS), 0, stream,
+                       N, ntiles, anchor, feat, offsets, scaling, campos, packed, neural_opacity, first, xyz, color,
+                       opacity, scal, rot, aux);
   }
-  static int backward_blocks(int64_t N) { return blocks_for((int)((N + NG_ANCHORS - 1) / NG_ANCHORS), 1); }
+  static int backward_blocks(int64_t N) {
+    return blocks_for((int)((N + NG_ANCHORS - 1) / NG_ANCHORS), S::BWD_WAVES, 1);
+  }
   static void backward(int64_t N, const float* anchor, const float* feat, const float* offsets, const float* scaling,
                        const float* campos, const float* packed, const float* neural_opacity, const uint32_t* first,
                        const float* color_out, const float* rot_out, const float* aux, const float* g_xyz,
                        const float* g_color, const float* g_opacity, const float* g_scal, const float* g_rot,
                        float* d_anchor, float* d_feat, float* d_offsets, float* d_scaling, float* const* d_params,
-                       float* partials, hipStream_t stream) {
+                       float* slot_grads, float* partials, hipStream_t stream) {
     const int ntiles = (int)((N + NG_ANCHORS - 1) / NG_ANCHORS);
+    hipLaunchKernelGGL(neural_offset_backward_kernel<K>, dim3((ntiles + NG_WAVES - 1) / NG_WAVES), dim3(NG_THREADS), 0,
+                       stream, N, ntiles, offsets, scaling, neural_opacity, first, color_out, rot_out, aux, g_xyz,
+                       g_color, g_opacity, g_scal, g_rot, slot_grads, d_anchor, d_offsets, d_scaling);
     const int nblocks = backward_blocks(N);
-    hipLaunchKernelGGL(neural_backward_kernel<K>, dim3(nblocks), dim3(NG_THREADS), 0, stream, N, ntiles, anchor, feat,
-                       offsets, scaling, campos, packed, neural_opacity, first, color_out, rot_out, aux, g_xyz,
-                       g_color, g_opacity, g_scal, g_rot, d_anchor, d_feat, d_offsets, d_scaling, partials);
+    hipLaunchKernelGGL(neural_mlp_backward_kernel<K>, dim3(nblocks), dim3(64 * S::BWD_WAVES), 0, stream, N, ntiles,
+                       anchor, feat, campos, packed, slot_grads, d_anchor, d_feat, partials);
     MlpGrads d;
     for (int i = 0; i < 12; i++) d.p[i] = d_params[i];
     const int total = 3 * (32 * 35 + 32) + 33 * (S::OUT0 + S::OUT1 + S::OUT2);
-    hipLaunchKernelGGL(neural_weight_reduce_kernel<K>, dim3((total + 255) / 256), dim3(256), 0, stream, nblocks,
+    hipLaunchKernelGGL(neural_weight_reduce_kernel<K>, dim3((total + 15) / 16), dim3(256), 0, stream, nblocks,
                        partials, d);
   }
 };
@@ -663,7 +766,7 @@ bool neural_supported(int k) {
 
 size_t neural_packed_floats(int k) {
   switch (k) {
-#define X(KK) case KK: return (size_t)pack_layout(Shape<KK>::TILES).total;
+#define X(KK) case KK: return (size_t)pack_layout(Shape<KK>::GROWS).total;
     NG_FOR_EACH_K(X)
 #undef X
     default: return 0;
@@ -678,6 +781,9 @@ size_t neural_partial_floats(int k, int64_t N) {
     default: return 0;
   }
 }
+
+// floats of the per-offset gradient records, padded so a 16-byte read at the end stays inside
+size_t neural_slot_grad_floats(int k, int64_t N) { return (size_t)N * (size_t)k * NG_SLOT_GRADS + 4; }
 
 int launch_neural_pack(int k, const float* const* params, float* packed, hipStream_t stream) {
   switch (k) {
@@ -718,11 +824,11 @@ int launch_neural_backward(int64_t N, int k, const float* anchor, const float* f
                            const float* neural_opacity, const uint32_t* first, const float* color_out,
                            const float* rot_out, const float* aux, const float* g_xyz, const float* g_color,
                            const float* g_opacity, const float* g_scal, const float* g_rot, float* d_anchor,
-                           float* d_feat, float* d_offsets, float* d_scaling, float* const* d_params, float* partials,
-                           hipStream_t stream) {
+                           float* d_feat, float* d_offsets, float* d_scaling, float* const* d_params,
+                           float* slot_grads, float* partials, hipStream_t stream) {
   if (N <= 0) return 0;
   switch (k) {
-#define X(KK) case KK: Launcher<KK>::backward(N, anchor, feat, offsets, scaling, campos, packed, neural_opacity, first, color_out, rot_out, aux, g_xyz, g_color, g_opacity, g_scal, g_rot, d_anchor, d_feat, d_offsets, d_scaling, d_params, partials, stream); return 0;
+#define X(KK) case KK: Launcher<KK>::backward(N, anchor, feat, offsets, scaling, campos, packed, neural_opacity, first, color_out, rot_out, aux, g_xyz, g_color, g_opacity, g_scal, g_rot, d_anchor, d_feat, d_offsets, d_scaling, d_params, slot_grads, partials, stream); return 0;
     NG_FOR_EACH_K(X)
 #undef X
     default: return 1;
