@@ -459,9 +459,12 @@ neural_mlp_backward_kernel(int64_t N, int ntiles, const float* __restrict__ anch
   __shared__ BwdLds<K> lds[NW];
   __shared__ float sW1[3 * NG_SLOTS * WS];
   __shared__ float sW2[S::GROWS * WS];
+  __shared__ __align__(16) float sWview[9 * 32];   // W1[h][32 + c] as [m][c][h]: the view-direction columns
   __shared__ unsigned short sWhere[TILE_FLOATS];  // where in G each float of a tile's records goes
   for (int e = threadIdx.x; e < 3 * NG_SLOTS * WS; e += NT) sW1[e] = packed[L.w1t + e];
   for (int e = threadIdx.x; e < S::GROWS * WS; e += NT) sW2[e] = packed[L.w2 + e];
+  for (int e = threadIdx.x; e < 9 * 32; e += NT)
+    sWview[e] = packed[L.w1t + ((e / 96) * NG_SLOTS + 32 + (e / 32) % 3) * WS + e % 32];
   for (int e = threadIdx.x; e < TILE_FLOATS; e += NT) {
     const int slot = e / NG_SLOT_GRADS, comp = e % NG_SLOT_GRADS, ax = slot / K, j = slot % K;
     const int row = comp == 0 ? S::G0 + j : comp < 4 ? S::G1 + 3 * j + (comp - 1) : S::G2 + 7 * j + (comp - 4);
@@ -474,16 +477,21 @@ neural_mlp_backward_kernel(int64_t N, int ntiles, const float* __restrict__ anch
   for (int e = lane; e < S::GROWS * SG_STRIDE; e += 64) W.g[e] = 0.0f;
   __syncthreads();
 
-  v16f accW2[S::TILES], accW1[3][2];
+  // weight-gradient accumulators: the W2 tiles, the 32 feature columns of W1 per MLP, and one tile that holds the
+  // four remaining columns of W1 (view direction, bias) of all three MLPs as its rows 4 m + c
+  v16f accW2[S::TILES], accW1[3], accWx;
   float accB2[B2N];
 #pragma unroll
   for (int t = 0; t < S::TILES; t++)
 #pragma unroll
     for (int i = 0; i < 16; i++) accW2[t][i] = 0.0f;
 #pragma unroll
-  for (int m = 0; m < 3; m++)
+  for (int m = 0; m < 3; m++) {
 #pragma unroll
-    for (int i = 0; i < 16; i++) accW1[m][0][i] = accW1[m][1][i] = 0.0f;
+    for (int i = 0; i < 16; i++) accW1[m][i] = 0.0f;
+  }
+#pragma unroll
+  for (int i = 0; i < 16; i++) accWx[i] = 0.0f;
 #pragma unroll
   for (int q = 0; q < B2N; q++) accB2[q] = 0.0f;
 
@@ -492,9 +500,14 @@ neural_mlp_backward_kernel(int64_t N, int ntiles, const float* __restrict__ anch
   int tile = blockIdx.x * NW + wave;
   XOperand xo;
   float4 gq[NQ];
+  float da[3] = {0.0f, 0.0f, 0.0f};  // the anchor's direct gradient, as the first kernel left it
   auto fetch_tile = [&](int t) {
     const int64_t a = (int64_t)t * NG_ANCHORS + al;
     xo = fetch_x(a < N, a, half, anchor, feat);
+    if (a < N && half == 0) {
+#pragma unroll
+      for (int c = 0; c < 3; c++) da[c] = d_anchor[a * 3 + c];
+    }
     const int64_t base = (int64_t)t * TILE_FLOATS;
 #pragma unroll
     for (int q = 0; q < NQ; q++) {
@@ -508,30 +521,48 @@ neural_mlp_backward_kernel(int64_t N, int ntiles, const float* __restrict__ anch
   for (; tile < ntiles; tile += stride) {
     const int64_t a = (int64_t)tile * NG_ANCHORS + al;
     const bool valid = a < N;
-    float xb[NG_W1_STEPS], nv[3], dist;
-    unpack_x(xb, nv, dist, xo, valid, half, cam);
-#pragma unroll
-    for (int s = 0; s < NG_W1_STEPS; s++) W.x[al * SX_STRIDE + xslot(half, s)] = xb[s];
+    float nv[3], dist;
+    const float da_now[3] = {da[0], da[1], da[2]};
     {
-      const int64_t base = (int64_t)tile * TILE_FLOATS;
+      float xb[NG_W1_STEPS];
+      unpack_x(xb, nv, dist, xo, valid, half, cam);
+#pragma unroll
+      for (int s = 0; s < NG_W1_STEPS; s++) W.x[al * SX_STRIDE + xslot(half, s)] = xb[s];
+      const int64_t left = total_floats - (int64_t)tile * TILE_FLOATS;
+      const int nvalid = left < TILE_FLOATS ? (int)left : TILE_FLOATS;  // floats of this tile that exist
 #pragma unroll
       for (int q = 0; q < NQ; q++) {
         const int e = (q * 64 + lane) * 4;
         if (e < TILE_FLOATS) {
           const float v[4] = {gq[q].x, gq[q].y, gq[q].z, gq[q].w};
 #pragma unroll
-          for (int c = 0; c < 4; c++) W.g[sWhere[e + c]] = base + e + c < total_floats ? v[c] : 0.0f;
+          for (int c = 0; c < 4; c++) W.g[sWhere[e + c]] = e + c < nvalid ? v[c] : 0.0f;
         }
       }
     }
     wave_sync();
-    if (tile + stride < ntiles) fetch_tile(tile + stride);
 
-    v16f dxf = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0}, dxv = dxf;
+    v16f dxf = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+    float dv[3] = {0.0f, 0.0f, 0.0f};  // this half's share of the gradient of the view direction
+    const float* xrow = W.x + al * SX_STRIDE;
 #pragma unroll
     for (int m = 0; m < 3; m++) {
+      // the next tile's loads go out before the last and longest MLP, late enough to keep their registers
+      // free until then and early enough to land behind its products
+      if (m == 2 && tile + stride < ntiles) fetch_tile(tile + stride);
       const float* w1t = sW1 + m * NG_SLOTS * WS;
-      const v16f h = hidden_layer(w1t, xb, al, half);
+      v16f h = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+      {
+        const float* lo = w1t + half * 16 * WS + al;
+        const float* hi = w1t + (32 + half) * WS + al;
+#pragma unroll
+        for (int s = 0; s < 16; s++) h = __builtin_amdgcn_mfma_f32_32x32x2f32(lo[s * WS], xrow[16 * half + s], h, 0, 0, 0);
+        h = __builtin_amdgcn_mfma_f32_32x32x2f32(hi[0], xrow[32 + half], h, 0, 0, 0);
+        h = __builtin_amdgcn_mfma_f32_32x32x2f32(hi[2 * WS], xrow[34 + half], h, 0, 0, 0);
+#pragma unroll
+        for (int i = 0; i < 16; i++) h[i] = h[i] > 0.0f ? h[i] : 0.0f;
+      }
+      __builtin_amdgcn_sched_barrier(0);
       v16f dh = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
       {
         // dH = W2^T G over this MLP's rows (pad row included: zero on both sides)
@@ -543,18 +574,27 @@ neural_mlp_backward_kernel(int64_t N, int ntiles, const float* __restrict__ anch
       }
 #pragma unroll
       for (int i = 0; i < 16; i++) dh[i] = h[i] > 0.0f ? dh[i] : 0.0f;
+      __builtin_amdgcn_sched_barrier(0);
       {
-        // dX += W1^T dHpre: rows = the 32 features, then the 3 view components
+        // dX += W1^T dHpre: the 32 feature rows on the matrix cores, the 3 view rows as plain sums over the 16
+        // hidden units this lane holds (the other 16 sit in the lane of the other half)
         const float* wf = w1t + al * WS + 4 * half;
-        const float* wv = w1t + (32 + (al < 3 ? al : 2)) * WS + 4 * half;
 #pragma unroll
-        for (int s = 0; s < 16; s++) {
-          const int hc = 8 * (s >> 2) + (s & 3);
-          dxf = __builtin_amdgcn_mfma_f32_32x32x2f32(wf[hc], dh[s], dxf, 0, 0, 0);
-          const float v = wv[hc];
-          dxv = __builtin_amdgcn_mfma_f32_32x32x2f32(al < 3 ? v : 0.0f, dh[s], dxv, 0, 0, 0);
-        }
+        for (int s = 0; s < 16; s++)
+          dxf = __builtin_amdgcn_mfma_f32_32x32x2f32(wf[8 * (s >> 2) + (s & 3)], dh[s], dxf, 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int c = 0; c < 3; c++)
+#pragma unroll
+          for (int q = 0; q < 4; q++) {
+            const float4 w = *(const float4*)(sWview + (m * 3 + c) * 32 + 8 * q + 4 * half);
+            dv[c] = __builtin_fmaf(w.x, dh[4 * q], dv[c]);
+            dv[c] = __builtin_fmaf(w.y, dh[4 * q + 1], dv[c]);
+            dv[c] = __builtin_fmaf(w.z, dh[4 * q + 2], dv[c]);
+            dv[c] = __builtin_fmaf(w.w, dh[4 * q + 3], dv[c]);
+          }
       }
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int i = 0; i < 16; i++) {
         W.hd[hrow(half, i) * SG_STRIDE + al] = h[i];
@@ -570,13 +610,17 @@ neural_mlp_backward_kernel(int64_t N, int ntiles, const float* __restrict__ anch
         for (int s = 0; s < 16; s++)
           accW2[S::first_tile(m) + lt] = __builtin_amdgcn_mfma_f32_32x32x2f32(
               gt[2 * s + half], W.hd[al * SG_STRIDE + 2 * s + half], accW2[S::first_tile(m) + lt], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
       }
-#pragma unroll
+      const float* dhrow = W.hd + (32 + al) * SG_STRIDE;
+#pragma unroll 4
       for (int s = 0; s < 16; s++) {
-        const float dhv = W.hd[(32 + al) * SG_STRIDE + 2 * s + half];
-        accW1[m][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(dhv, W.x[(2 * s + half) * SX_STRIDE + al], accW1[m][0], 0, 0, 0);
-        accW1[m][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(dhv, W.x[(2 * s + half) * SX_STRIDE + 32 + (al & 3)],
-                                                          accW1[m][1], 0, 0, 0);
+        const float dhv = dhrow[2 * s + half];
+        const float* xr = W.x + (2 * s + half) * SX_STRIDE;
+        accW1[m] = __builtin_amdgcn_mfma_f32_32x32x2f32(dhv, xr[al], accW1[m], 0, 0, 0);
+        // rows 4 m .. 4 m + 3 of the shared tile take this MLP's view and bias columns, the other rows add zero
+        const float xv = xr[32 + (al & 3)];
+        accWx = __builtin_amdgcn_mfma_f32_32x32x2f32((al >> 2) == m ? xv : 0.0f, dhv, accWx, 0, 0, 0);
       }
       wave_sync();
     }
@@ -592,15 +636,17 @@ neural_mlp_backward_kernel(int64_t N, int ntiles, const float* __restrict__ anch
     }
 
     // ---- per anchor results
+#pragma unroll
+    for (int c = 0; c < 3; c++) dv[c] += __shfl_xor(dv[c], 32);
     if (valid) {
 #pragma unroll
       for (int q = 0; q < 4; q++)
         *(float4*)(d_feat + a * 32 + 8 * q + 4 * half) = make_float4(dxf[4 * q], dxf[4 * q + 1], dxf[4 * q + 2], dxf[4 * q + 3]);
       if (half == 0) {
         // the view direction n = v / |v| adds (g - n (n.g)) / |v| to the anchor's direct gradient
-        const float ng = (nv[0] * dxv[0] + nv[1] * dxv[1]) + nv[2] * dxv[2];
+        const float ng = (nv[0] * dv[0] + nv[1] * dv[1]) + nv[2] * dv[2];
 #pragma unroll
-        for (int c = 0; c < 3; c++) d_anchor[a * 3 + c] = d_anchor[a * 3 + c] + (dxv[c] - nv[c] * ng) / dist;
+        for (int c = 0; c < 3; c++) d_anchor[a * 3 + c] = da_now[c] + (dv[c] - nv[c] * ng) / dist;
       }
     }
     wave_sync();
@@ -608,10 +654,11 @@ neural_mlp_backward_kernel(int64_t N, int ntiles, const float* __restrict__ anch
 
   // ---- reduce the waves' accumulators, one 32x32 tile at a time, through each wave's staging area
   float* out = partials + (size_t)blockIdx.x * partial_floats<K>();
-  constexpr int NACC = S::TILES + 6;
+  constexpr int NACC = S::TILES + 4;
 #pragma unroll
   for (int t = 0; t < NACC; t++) {
-    const v16f& acc = t < S::TILES ? accW2[t] : accW1[(t - S::TILES) >> 1][(t - S::TILES) & 1];
+    const v16f& acc = t < S::TILES ? accW2[t] : t < S::TILES + 3 ? accW1[t - S::TILES] : accWx;
+    float* dst = out + (t < S::TILES ? t : S::TILES + 2 * (t - S::TILES)) * NG_TILE;
     __syncthreads();
 #pragma unroll
     for (int i = 0; i < 16; i++) W.hd[hrow(half, i) * 32 + al] = acc[i];
@@ -620,7 +667,14 @@ neural_mlp_backward_kernel(int64_t N, int ntiles, const float* __restrict__ anch
       float sum = lds[0].hd[e];
 #pragma unroll
       for (int w = 1; w < NW; w++) sum += lds[w].hd[e];
-      out[t * NG_TILE + e] = sum;
+      if (t < S::TILES + 3) {
+        dst[e] = sum;
+      } else if (e < 12 * 32) {
+        // row 4 m + c, column h of the shared tile -> column 32 + c of W1 of MLP m: element h * 32 + c of its
+        // second tile
+        const int row = e >> 5, h = e & 31;
+        out[(S::TILES + 2 * (row >> 2) + 1) * NG_TILE + h * 32 + (row & 3)] = sum;
+      }
     }
   }
   __syncthreads();
@@ -631,7 +685,7 @@ neural_mlp_backward_kernel(int64_t N, int ntiles, const float* __restrict__ anch
     float sum = lds[0].hd[e];
 #pragma unroll
     for (int w = 1; w < NW; w++) sum += lds[w].hd[e];
-    out[NACC * NG_TILE + e] = sum;
+    out[(S::TILES + 6) * NG_TILE + e] = sum;
   }
 }
 
