@@ -102,7 +102,7 @@ __device__ __forceinline__ void wave_sync() {
 }
 
 // hardware exp2 and reciprocal: about 1e-6 relative, far inside what float32 MLP outputs carry
-__device__ __forceinline__ float sigmoidf(float x) { return __frcp_rn(1.0f + __expf(-x)); }
+__device__ __forceinline__ float sigmoidf(float x) { return __builtin_amdgcn_rcpf(1.0f + __expf(-x)); }
 
 // The 18 layer-1 B operands of this lane: its anchor's features of its half, the view direction and the constant.
 // Also returns the unit view direction and the distance (every lane computes both).
@@ -242,7 +242,7 @@ neural_opacity_kernel(int64_t N, int ntiles, const float* __restrict__ anchor, c
 // (first[a] = number of selected offsets of all anchors before a).  Everything an offset needs from memory
 // is requested before the matrix products start, so the loads complete behind them.
 template <int K>
-__global__ void __launch_bounds__(NG_THREADS)
+__global__ void __launch_bounds__(NG_THREADS, 2)
 neural_gaussians_kernel(int64_t N, int ntiles, const float* __restrict__ anchor, const float* __restrict__ feat,
                         const float* __restrict__ offsets, const float* __restrict__ scaling,
                         const float* __restrict__ campos, const float* __restrict__ packed,
@@ -252,11 +252,13 @@ neural_gaussians_kernel(int64_t N, int ntiles, const float* __restrict__ anchor,
   using S = Shape<K>;
   constexpr PackLayout L = pack_layout(S::GROWS);
   constexpr int WROWS = S::GROWS - S::G1;        // output rows of the two MLPs of this kernel
-  constexpr int ROWS = 32 * S::T1 + S::OUT2;     // result rows kept: color tiles whole, cov rows up to 7K
+  constexpr int ROWS = S::OUT1 + S::OUT2;        // result rows kept per anchor: 3K color, 7K cov
+  constexpr int GEO = 10;                        // per anchor: position, scaling (6), row base
   __shared__ float sW1[2 * NG_SLOTS * WS];
   __shared__ float sW2[WROWS * WS];
   __shared__ float sB2[WROWS];
   __shared__ float sOut[NG_WAVES][ROWS * SG_STRIDE];
+  __shared__ float sGeo[NG_WAVES][NG_ANCHORS * GEO];
   for (int e = threadIdx.x; e < 2 * NG_SLOTS * WS; e += NG_THREADS) sW1[e] = packed[L.w1t + NG_SLOTS * WS + e];
   for (int e = threadIdx.x; e < WROWS * WS; e += NG_THREADS) sW2[e] = packed[L.w2 + S::G1 * WS + e];
   for (int e = threadIdx.x; e < WROWS; e += NG_THREADS) sB2[e] = packed[L.b2 + S::G1 + e];
@@ -264,30 +266,53 @@ neural_gaussians_kernel(int64_t N, int ntiles, const float* __restrict__ anchor,
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, half = lane >> 5, al = lane & 31;
   const float cam[3] = {campos[0], campos[1], campos[2]};
   float* out = sOut[wave];
-  for (int tile = blockIdx.x * NG_WAVES + wave; tile < ntiles; tile += gridDim.x * NG_WAVES) {
-    const int64_t a = (int64_t)tile * NG_ANCHORS + al;
-    const XOperand xo = fetch_x(a < N, a, half, anchor, feat);
-    // per offset of this lane: opacity and row base, requested before the matrix products start
-    float s_t[S::GROUPS];
-    uint32_t s_first[S::GROUPS];
+  float* geo = sGeo[wave];
+  // What a tile reads from memory.  Per anchor (lane = anchor; the two halves share the work): features, position,
+  // scaling, row base.  Per offset (lane = offset within a 64-slot group): opacity and offset vector.  The next
+  // tile's set is requested before the current tile's per-offset work, so it arrives behind it.
+  XOperand xo;
+  float p_sc[3], s_t[S::GROUPS], s_of[S::GROUPS][3];
+  uint32_t p_first = 0;
+  auto fetch_tile = [&](int t) {
+    const int64_t a = (int64_t)t * NG_ANCHORS + al;
+    xo = fetch_x(a < N, a, half, anchor, feat);
+#pragma unroll
+    for (int c = 0; c < 3; c++) p_sc[c] = a < N ? scaling[a * 6 + 3 * half + c] : 0.0f;
+    p_first = a < N ? first[a] : 0u;
 #pragma unroll
     for (int g = 0; g < S::GROUPS; g++) {
       const int idx = g * S::APG * K + lane;
-      const int ax = idx / K;
-      const int64_t sa = (int64_t)tile * NG_ANCHORS + ax;
-      const bool ok = lane < S::APG * K && ax < NG_ANCHORS && sa < N;
-      s_t[g] = ok ? neural_opacity[sa * K + idx % K] : 0.0f;
-      s_first[g] = ok ? first[sa] : 0u;
+      const int64_t sa = (int64_t)t * NG_ANCHORS + idx / K;
+      const bool ok = lane < S::APG * K && idx < NG_ANCHORS * K && sa < N;
+      const int64_t slot = (int64_t)t * NG_ANCHORS * K + idx;
+      s_t[g] = ok ? neural_opacity[slot] : 0.0f;
+#pragma unroll
+      for (int c = 0; c < 3; c++) s_of[g][c] = ok ? offsets[slot * 3 + c] : 0.0f;
     }
+  };
+  const int stride = gridDim.x * NG_WAVES;
+  int tile = blockIdx.x * NG_WAVES + wave;
+  if (tile < ntiles) fetch_tile(tile);
+  for (; tile < ntiles; tile += stride) {
+    const int64_t a = (int64_t)tile * NG_ANCHORS + al;
     float xb[NG_W1_STEPS], nv[3], dist;
     unpack_x(xb, nv, dist, xo, a < N, half, cam);
+    if (half == 0) {
+      geo[al * GEO] = xo.ax; geo[al * GEO + 1] = xo.ay; geo[al * GEO + 2] = xo.az;
+      geo[al * GEO + 9] = __uint_as_float(p_first);
+    }
+#pragma unroll
+    for (int c = 0; c < 3; c++) geo[al * GEO + 3 + 3 * half + c] = p_sc[c];
     {
       const v16f h = hidden_layer(sW1, xb, al, half);
 #pragma unroll
       for (int t = 0; t < S::T1; t++) {
         const v16f o = output_tile<S::OUT1>(sW2, sB2, t, h, al, half);
 #pragma unroll
-        for (int i = 0; i < 16; i++) out[(32 * t + hrow(half, i)) * SG_STRIDE + al] = o[i];
+        for (int i = 0; i < 16; i++) {
+          const int row = 32 * t + hrow(half, i);
+          if (row < S::OUT1) out[row * SG_STRIDE + al] = o[i];
+        }
       }
     }
     {
@@ -298,30 +323,38 @@ neural_gaussians_kernel(int64_t N, int ntiles, const float* __restrict__ anchor,
 #pragma unroll
         for (int i = 0; i < 16; i++) {
           const int row = 32 * t + hrow(half, i);
-          if (row < S::OUT2) out[(32 * S::T1 + row) * SG_STRIDE + al] = o[i];
+          if (row < S::OUT2) out[(S::OUT1 + row) * SG_STRIDE + al] = o[i];
         }
       }
     }
     wave_sync();
+    // this tile's per-offset inputs move to fresh registers so the next tile's loads can start now
+    float c_t[S::GROUPS], c_of[S::GROUPS][3];
+#pragma unroll
+    for (int g = 0; g < S::GROUPS; g++) {
+      c_t[g] = s_t[g];
+#pragma unroll
+      for (int c = 0; c < 3; c++) c_of[g][c] = s_of[g][c];
+    }
+    if (tile + stride < ntiles) fetch_tile(tile + stride);
 #pragma unroll
     for (int g = 0; g < S::GROUPS; g++) {
       const int idx = g * S::APG * K + lane;
       const int ax = idx / K, j = idx % K;
-      const float t = s_t[g];
+      const float t = c_t[g];
       const bool sel = t > 0.0f;
       const unsigned long long bits = __ballot(sel);
       if (sel) {
-        const int64_t r = (int64_t)s_first[g] + count_lanes(bits, lane - j, lane);
-        const int64_t sa = (int64_t)tile * NG_ANCHORS + ax;
-        const float* sc = scaling + sa * 6;
-        const float* cv = out + (32 * S::T1 + 7 * j) * SG_STRIDE + ax;
+        const float* ga = geo + ax * GEO;
+        const int64_t r = (int64_t)__float_as_uint(ga[9]) + count_lanes(bits, lane - j, lane);
+        const float* cv = out + (S::OUT1 + 7 * j) * SG_STRIDE + ax;
         float sg[3];
 #pragma unroll
         for (int c = 0; c < 3; c++) {
-          xyz[r * 3 + c] = anchor[sa * 3 + c] + offsets[(sa * K + j) * 3 + c] * sc[c];
+          xyz[r * 3 + c] = ga[c] + c_of[g][c] * ga[3 + c];
           color[r * 3 + c] = sigmoidf(out[(3 * j + c) * SG_STRIDE + ax]);
           sg[c] = sigmoidf(cv[c * SG_STRIDE]);
-          scal[r * 3 + c] = sc[3 + c] * sg[c];
+          scal[r * 3 + c] = ga[6 + c] * sg[c];
         }
         opacity[r] = t;
         const float q0 = cv[3 * SG_STRIDE], q1 = cv[4 * SG_STRIDE], q2 = cv[5 * SG_STRIDE], q3 = cv[6 * SG_STRIDE];
