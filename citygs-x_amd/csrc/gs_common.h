@@ -53,6 +53,15 @@ __device__ __forceinline__ uint32_t f2u_sat(float v) {
   return (uint32_t)v;
 }
 
+// Store for data that is written once and not read again on the GPU for a long while (gradients of leaf
+// parameters on their way to the optimizer): it goes out past the caches, so it does not evict what the next
+// kernel reads.
+__device__ __forceinline__ void store_streaming(float4* p, const float4& v) {
+  typedef float v4f __attribute__((ext_vector_type(4)));
+  const v4f w = {v.x, v.y, v.z, v.w};
+  __builtin_nontemporal_store(w, reinterpret_cast<v4f*>(p));
+}
+
 // exp() of the blending loops: n = rint(x*log2e), r = x - n*ln2 (two-constant
 // split), degree-6 polynomial, scale by 2^n.  Only IEEE operations and explicit
 // FMAs, so a CPU evaluates the same bits.  x < -87 -> 0, x > 88 -> +inf.

@@ -193,14 +193,16 @@ __device__ __forceinline__ void wave_rows_load(const float4* __restrict__ g4, ui
   wave_sync_lds();
 }
 
-// stores the first `rows` rows
+// stores the first `rows` rows, streaming: SH coefficient gradients exist only when the coefficients are leaf
+// parameters, and then the optimizer is their next reader; the position, scale and rotation gradients can feed
+// the caller's backward pass at once and are stored normally
 __device__ __forceinline__ void wave_rows_store(float4* __restrict__ g4, int rows, const float4* lds, int lane) {
   wave_sync_lds();
 #pragma unroll
   for (int j = 0; j < 12; j++) {
     const int idx = j * GS_WAVE + lane;
     const int row = idx / 12;
-    if (row < rows) g4[idx] = lds[row * SH_ROW4 + (idx - row * 12)];
+    if (row < rows) store_streaming(g4 + idx, lds[row * SH_ROW4 + (idx - row * 12)]);
   }
 }
 
