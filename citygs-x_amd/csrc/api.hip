@@ -94,7 +94,7 @@ inline void tile_grid(int W, int H, int& gx, int& gy) {
 }
 
 struct ImageLayout {
-  size_t accum_alpha, n_contrib, n_contrib2loss, ranges, total;
+  size_t accum_alpha, n_contrib, n_contrib2loss, ranges, bucket_table, total;
 };
 ImageLayout image_layout(int W, int H) {
   ImageLayout L;
@@ -107,6 +107,8 @@ ImageLayout image_layout(int W, int H) {
   L.n_contrib = take(N * 4);
   L.n_contrib2loss = take(N * 4);
   L.ranges = take((size_t)gx * gy * 8);
+  // workgroup-by-tile counts of the counting sort by tile (nothing when the grid is too large for it)
+  L.bucket_table = take(gx * gy <= bucket_max_tiles() ? bucket_table_bytes(gx * gy) : 0);
   L.total = off + 256;
   return L;
 }
@@ -338,6 +340,7 @@ uint32_t* acquire_total_slot() {
     }
   }
   uint32_t* slot = base + 16 * (g_total_next.fetch_add(1, std::memory_order_relaxed) % TOTAL_SLOTS);
+  slot[1] = 0u;  // second word of the slot: the longest tile list, written before the total
   __atomic_store_n(slot, TOTAL_PENDING, __ATOMIC_RELEASE);
   return slot;
 }
@@ -369,6 +372,21 @@ int wait_for_total(uint32_t* slot, hipStream_t stream, uint32_t* out) {
   }
 }
 }  // namespace
+
+namespace {
+// list lengths at which the per-tile sort hands over to its large variant and to the radix sort
+std::atomic<int> g_tile_sort_small{TILE_SORT_SMALL};
+std::atomic<int> g_tile_sort_large{TILE_SORT_LARGE};
+}  // namespace
+
+void gs_set_tile_sort_limits(int small_limit, int large_limit) {
+  if (small_limit < 1) small_limit = 1;
+  if (small_limit > TILE_SORT_SMALL) small_limit = TILE_SORT_SMALL;
+  if (large_limit > TILE_SORT_LARGE) large_limit = TILE_SORT_LARGE;
+  if (large_limit > 0 && large_limit < small_limit) large_limit = small_limit;
+  g_tile_sort_small.store(small_limit);
+  g_tile_sort_large.store(large_limit);
+}
 
 int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resize_fn binningBuffer,
                       void* binning_user, gs_resize_fn imageBuffer, void* image_user, int P, const float* background,
@@ -411,8 +429,19 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
   uint32_t* n_contrib2loss_px = (uint32_t*)(ibase + IL.n_contrib2loss);
   uint32_t* ranges = (uint32_t*)(ibase + IL.ranges);
 
+  // Two ways to the sorted per-tile lists.  The default buckets the instances by tile (counting sort) and sorts
+  // every tile's list in LDS; it needs the tile histogram to fit in LDS and every list to fit the per-tile
+  // sort.  Otherwise: emit (tile | depth) keys, radix-sort all of them, find the tile boundaries.
   uint32_t* total_slot = acquire_total_slot();
-  {
+  void* bucket_table = ibase + IL.bucket_table;
+  const bool counted_by_tile = T <= bucket_max_tiles() && total_slot != nullptr && g_tile_sort_large.load() > 0;
+  bool bucketed = counted_by_tile;
+  if (bucketed) {
+    StageScope _t("tile_count", stream);
+    if (launch_bucket_count(P, width, height, radii, means2D, compute_locally, tiles_touched, bucket_table, ranges,
+                            total_slot + 1, stream))
+      return 1;
+  } else {
     StageScope _t("tile_count", stream);
     // also clears the tile ranges (cudaMemset of CR/rasterizer_impl.cu:687), which nothing reads before
     // identify_tile_ranges fills them
@@ -428,10 +457,12 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
 
   // The instance count decides the size of the binning buffer, so the host needs it here.  The scan writes
   // it straight into pinned host memory and the host polls that word: no copy, and no sleeping wait whose
-  // wake-up would leave the GPU idle.
-  uint32_t R_u = 0;
+  // wake-up would leave the GPU idle.  The longest tile list sits in the word beside it, written by a kernel
+  // that ran before the scan.
+  uint32_t R_u = 0, longest = 0;
   if (total_slot != nullptr) {
     if (wait_for_total(total_slot, stream, &R_u)) return 1;
+    longest = __atomic_load_n(total_slot + 1, __ATOMIC_ACQUIRE);
   } else {
     GS_HIP_TRY(hipMemcpyAsync(&R_u, point_offsets + (P - 1), sizeof(uint32_t), hipMemcpyDeviceToHost, stream));
     GS_HIP_TRY(hipStreamSynchronize(stream));
@@ -458,34 +489,53 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
   EventTimer timer;
   if (timer.begin(elapsed_ms != nullptr, stream)) return 1;
 
-  const int end_bit = sort_end_bit(width, height);
-  // The sort carries each instance's index in emission order as its payload (the backward pass files
-  // per-instance gradients under it); the Gaussian ids of the sorted list are gathered afterwards.
-  // It ping-pongs, so start from the array pair that makes it finish in (keys, emission).
-  const bool odd = sort_result_in_b(end_bit);
-  uint64_t* k_start = odd ? keys_other : keys;
-  uint32_t* e_start = odd ? emission_other : emission;
-  uint64_t* k_partner = odd ? keys : keys_other;
-  uint32_t* e_partner = odd ? emission : emission_other;
-  if (R > 0) {
-    {
-      StageScope _t("duplicate_with_keys", stream);
-      launch_duplicate_with_keys(P, width, height, means2D, depths, point_offsets, radii, compute_locally, k_start,
-                                 gauss_of_emission, e_start, stream);
+  if (bucketed && longest > (uint32_t)g_tile_sort_large.load()) bucketed = false;  // a list too long for the LDS sort
+  if (bucketed) {
+    if (R > 0) {
+      {
+        StageScope _t("bucket_scatter", stream);
+        launch_bucket_scatter(P, width, height, means2D, depths, point_offsets, radii, compute_locally, bucket_table,
+                              ranges, keys_other, gauss_of_emission, stream);
+      }
+      if (check_launch("bucket_scatter", stream, dbg)) return 1;
+      {
+        StageScope _t("tile_sort", stream);
+        launch_tile_sort(T, longest, (uint32_t)g_tile_sort_small.load(), ranges, keys_other, gauss_of_emission, keys,
+                         emission, point_list, stream);
+      }
+      if (check_launch("tile_sort", stream, dbg)) return 1;
     }
-    if (check_launch("duplicate_with_keys", stream, dbg)) return 1;
-    {
-      StageScope _t("sort_pairs", stream);
-      if (launch_sort_pairs_u64(R, k_start, k_partner, e_start, e_partner, end_bit, sort_temp, stream)) return 1;
+  } else {
+    const int end_bit = sort_end_bit(width, height);
+    // The sort carries each instance's index in emission order as its payload (the backward pass files
+    // per-instance gradients under it); the Gaussian ids of the sorted list are gathered afterwards.
+    // It ping-pongs, so start from the array pair that makes it finish in (keys, emission).
+    const bool odd = sort_result_in_b(end_bit);
+    uint64_t* k_start = odd ? keys_other : keys;
+    uint32_t* e_start = odd ? emission_other : emission;
+    uint64_t* k_partner = odd ? keys : keys_other;
+    uint32_t* e_partner = odd ? emission : emission_other;
+    if (R > 0) {
+      {
+        StageScope _t("duplicate_with_keys", stream);
+        launch_duplicate_with_keys(P, width, height, means2D, depths, point_offsets, radii, compute_locally, k_start,
+                                   gauss_of_emission, e_start, stream);
+      }
+      if (check_launch("duplicate_with_keys", stream, dbg)) return 1;
+      {
+        StageScope _t("sort_pairs", stream);
+        if (launch_sort_pairs_u64(R, k_start, k_partner, e_start, e_partner, end_bit, sort_temp, stream)) return 1;
+      }
+      if (check_launch("sort_pairs", stream, dbg)) return 1;
     }
-    if (check_launch("sort_pairs", stream, dbg)) return 1;
+    {
+      StageScope _t("identify_tile_ranges", stream);
+      // ... and gathers the Gaussian ids of the sorted instances on the way (point_list).  The ranges were
+      // cleared by the counting kernel of this path, or hold the other path's table and are cleared here.
+      launch_tile_ranges(R, keys, T, ranges, stream, !counted_by_tile, emission, gauss_of_emission, point_list);
+    }
+    if (check_launch("identify_tile_ranges", stream, dbg)) return 1;
   }
-  {
-    StageScope _t("identify_tile_ranges", stream);
-    // ... and gathers the Gaussian ids of the sorted instances on the way (point_list)
-    launch_tile_ranges(R, keys, T, ranges, stream, true, emission, gauss_of_emission, point_list);
-  }
-  if (check_launch("identify_tile_ranges", stream, dbg)) return 1;
 
   RenderFwdArgs a;
   a.P = P; a.W = width; a.H = height;

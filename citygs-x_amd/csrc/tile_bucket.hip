@@ -1,0 +1,305 @@
+// Binning by tile without a global sort.  The list the rasterizer needs is "instances ordered by (tile, depth
+// bits), ties in emission order" (cuda_rasterizer/rasterizer_impl.cu:74-144, :675-697: duplicateWithKeys, a stable
+// radix sort on the (tile << 32 | depth) key, identifyTileRanges).  The tile part of that key takes few values
+// and every tile's list is short, so the same list comes out of
+//   1. a counting sort by tile: per-workgroup tile histograms in LDS, a prefix over workgroups and tiles (which
+//      is also the table of tile ranges), and a scatter of every instance into its tile's segment, in any order;
+//   2. one workgroup per tile sorting its segment in LDS by (depth bits, emission index): the emission index
+//      is unique, so the order does not depend on how the scatter happened to fill the segment, and it is the
+//      order a stable sort on the depth bits would leave.
+// No pass over all instances per digit, no look-back chain.  Lists longer than the LDS variant holds are left to
+// the radix sort (the caller decides from the longest list, which this code reports).
+#include "gs_common.h"
+#include "gs_kernels.h"
+
+namespace gs {
+namespace {
+
+constexpr int BK_THREADS = 1024;        // counting and scatter kernels
+constexpr int BK_MAX_BLOCKS = 256;
+constexpr int BK_MIN_PER_BLOCK = 4096;  // Gaussians per workgroup, at least
+constexpr int TS_THREADS = 256;         // per-tile sort
+
+__host__ __device__ inline int bucket_per_block(int P) {
+  const int per = (P + BK_MAX_BLOCKS - 1) / BK_MAX_BLOCKS;
+  return per < BK_MIN_PER_BLOCK ? BK_MIN_PER_BLOCK : per;
+}
+__host__ __device__ inline int bucket_blocks(int P) {
+  const int per = bucket_per_block(P);
+  return (P + per - 1) / per;
+}
+
+// 1a. Per Gaussian the number of tiles it touches (rasterizer_impl.cu:264-288), per workgroup the number of
+// instances of every tile.  The workgroup's Gaussians are a contiguous chunk; the scatter walks the same chunk.
+__global__ void __launch_bounds__(BK_THREADS)
+bucket_count_kernel(int P, int per_block, uint32_t gx, uint32_t gy, const int* __restrict__ radii,
+                    const float2* __restrict__ means2D, const uint8_t* __restrict__ compute_locally,
+                    uint32_t* __restrict__ tiles_touched, uint32_t* __restrict__ table) {
+  extern __shared__ uint32_t s_hist[];
+  const uint32_t T = gx * gy;
+  for (uint32_t t = threadIdx.x; t < T; t += BK_THREADS) s_hist[t] = 0u;
+  __syncthreads();
+  const int first = blockIdx.x * per_block;
+  const int last = first + per_block < P ? first + per_block : P;
+  for (int i = first + threadIdx.x; i < last; i += BK_THREADS) {
+    uint32_t cnt = 0;
+    const int r = radii[i];
+    if (r > 0) {
+      const float2 p = means2D[i];
+      const Rect rc = get_rect(p.x, p.y, r, gx, gy);
+      for (uint32_t y = rc.y0; y < rc.y1; y++)
+        for (uint32_t x = rc.x0; x < rc.x1; x++)
+          if (compute_locally[y * gx + x]) {
+            atomicAdd(&s_hist[y * gx + x], 1u);
+            cnt++;
+          }
+    }
+    tiles_touched[i] = cnt;
+  }
+  __syncthreads();
+  uint32_t* row = table + (size_t)blockIdx.x * T;
+  for (uint32_t t = threadIdx.x; t < T; t += BK_THREADS) row[t] = s_hist[t];
+}
+
+// 1b. Per tile: the workgroups' counts become exclusive prefixes in place, their sum goes to totals.  A workgroup
+// takes 32 tiles (one 128-byte row segment) by 8 runs of consecutive workgroup rows; a thread holds its run in
+// registers, the runs' sums meet in LDS.
+constexpr int COL_TILES = 32, COL_RUNS = 8, COL_RUN_MAX = BK_MAX_BLOCKS / COL_RUNS;
+__global__ void __launch_bounds__(COL_TILES * COL_RUNS)
+bucket_columns_kernel(int nblocks, uint32_t T, uint32_t* __restrict__ table, uint32_t* __restrict__ totals) {
+  __shared__ uint32_t s_sum[COL_RUNS][COL_TILES];
+  const int tx = threadIdx.x % COL_TILES, run = threadIdx.x / COL_TILES;
+  const uint32_t t = blockIdx.x * COL_TILES + tx;
+  const int len = (nblocks + COL_RUNS - 1) / COL_RUNS;  // <= COL_RUN_MAX
+  const int b0 = run * len;
+  uint32_t c[COL_RUN_MAX];
+  uint32_t sum = 0;
+#pragma unroll
+  for (int k = 0; k < COL_RUN_MAX; k++) {
+    const int b = b0 + k;
+    c[k] = (k < len && b < nblocks && t < T) ? table[(size_t)b * T + t] : 0u;
+    sum += c[k];
+  }
+  s_sum[run][tx] = sum;
+  __syncthreads();
+  uint32_t before = 0, all = 0;
+#pragma unroll
+  for (int r = 0; r < COL_RUNS; r++) {
+    const uint32_t v = s_sum[r][tx];
+    if (r < run) before += v;
+    all += v;
+  }
+  if (t >= T) return;
+#pragma unroll
+  for (int k = 0; k < COL_RUN_MAX; k++) {
+    const int b = b0 + k;
+    if (k < len && b < nblocks) table[(size_t)b * T + t] = before;
+    before += c[k];
+  }
+  if (run == 0) totals[t] = all;
+}
+
+__device__ __forceinline__ uint32_t wave_inclusive_scan_u32(uint32_t v, int lane) {
+#pragma unroll
+  for (int d = 1; d < GS_WAVE; d <<= 1) {
+    const uint32_t o = __shfl_up(v, d, GS_WAVE);
+    if (lane >= d) v += o;
+  }
+  return v;
+}
+
+// 1c. One workgroup: exclusive prefix of the tile totals = the tile ranges (rasterizer_impl.cu:122-144 leaves
+// (0, 0) for a tile without instances), and the longest list, stored where the host can read it.
+__global__ void __launch_bounds__(1024)
+bucket_ranges_kernel(uint32_t T, const uint32_t* __restrict__ totals, uint32_t* __restrict__ ranges,
+                     uint32_t* __restrict__ longest_out) {
+  __shared__ uint32_t s_wave[16], s_max[16];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  uint32_t carry = 0, longest = 0;
+  for (uint32_t start = 0; start < T; start += 1024) {
+    const uint32_t t = start + threadIdx.x;
+    const uint32_t v = t < T ? totals[t] : 0u;
+    longest = v > longest ? v : longest;
+    const uint32_t inc = wave_inclusive_scan_u32(v, lane);
+    if (lane == 63) s_wave[wave] = inc;
+    __syncthreads();
+    uint32_t base = 0, all = 0;
+#pragma unroll
+    for (int w = 0; w < 16; w++) {
+      const uint32_t s = s_wave[w];
+      if (w < wave) base += s;
+      all += s;
+    }
+    __syncthreads();
+    const uint32_t begin = carry + base + inc - v;
+    if (t < T) {
+      ranges[2 * t] = v ? begin : 0u;
+      ranges[2 * t + 1] = v ? begin + v : 0u;
+    }
+    carry += all;
+  }
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) {
+    const uint32_t o = __shfl_xor(longest, d, GS_WAVE);
+    longest = o > longest ? o : longest;
+  }
+  if (lane == 0) s_max[wave] = longest;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    uint32_t m = 0;
+    for (int w = 0; w < 16; w++) m = s_max[w] > m ? s_max[w] : m;
+    __hip_atomic_store(longest_out, m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+  }
+}
+
+// 1d. Every instance goes to its tile's segment: segment start (ranges) + instances of earlier workgroups
+// (table) + a place among this workgroup's own, handed out by an LDS counter.  The record is
+// (depth bits << 32 | emission index); the Gaussian of an emission index goes to a side table
+// (rasterizer_impl.cu:74-117 writes the same pairs in emission order).
+__global__ void __launch_bounds__(BK_THREADS)
+bucket_scatter_kernel(int P, int per_block, uint32_t gx, uint32_t gy, const float2* __restrict__ means2D,
+                      const float* __restrict__ depths, const uint32_t* __restrict__ offsets,
+                      const int* __restrict__ radii, const uint8_t* __restrict__ compute_locally,
+                      const uint32_t* __restrict__ table, const uint32_t* __restrict__ ranges,
+                      uint64_t* __restrict__ records, uint32_t* __restrict__ gauss_of_emission) {
+  extern __shared__ uint32_t s_next[];
+  const uint32_t T = gx * gy;
+  const uint32_t* row = table + (size_t)blockIdx.x * T;
+  for (uint32_t t = threadIdx.x; t < T; t += BK_THREADS) s_next[t] = ranges[2 * t] + row[t];
+  __syncthreads();
+  const int first = blockIdx.x * per_block;
+  const int last = first + per_block < P ? first + per_block : P;
+  for (int i = first + threadIdx.x; i < last; i += BK_THREADS) {
+    const int r = radii[i];
+    if (r <= 0) continue;
+    uint32_t e = (i == 0) ? 0u : offsets[i - 1];
+    const float2 p = means2D[i];
+    const Rect rc = get_rect(p.x, p.y, r, gx, gy);
+    const uint64_t hi = (uint64_t)__float_as_uint(depths[i]) << 32;
+    for (uint32_t y = rc.y0; y < rc.y1; y++)
+      for (uint32_t x = rc.x0; x < rc.x1; x++)
+        if (compute_locally[y * gx + x]) {
+          const uint32_t pos = atomicAdd(&s_next[y * gx + x], 1u);
+          records[pos] = hi | (uint64_t)e;
+          gauss_of_emission[e] = (uint32_t)i;
+          e++;
+        }
+  }
+}
+
+// 2. One workgroup per tile: bitonic sort of the tile's records in LDS, then the three sorted arrays the
+// rasterizer keeps: the reference's key (tile << 32 | depth bits), the emission index (the backward pass files
+// per-instance gradients under it) and the Gaussian id.  Handles lists of min_n < n <= max_n <= CAP records.
+template <int CAP>
+__global__ void __launch_bounds__(TS_THREADS)
+tile_sort_kernel(const uint32_t* __restrict__ ranges, const uint64_t* __restrict__ records,
+                 const uint32_t* __restrict__ gauss_of_emission, uint64_t* __restrict__ keys,
+                 uint32_t* __restrict__ emission, uint32_t* __restrict__ point_list, uint32_t min_n, uint32_t max_n) {
+  __shared__ uint64_t s[CAP];
+  const uint32_t t = blockIdx.x;
+  const uint32_t start = ranges[2 * t];
+  const uint32_t n = ranges[2 * t + 1] - start;
+  if (n <= min_n || n > max_n) return;
+  uint32_t m = 1;
+  while (m < n) m <<= 1;
+  for (uint32_t i = threadIdx.x; i < m; i += TS_THREADS) s[i] = i < n ? records[start + i] : ~0ull;
+  __syncthreads();
+  // Compare-exchange number idx pairs elements lo and lo + j.  A wave owns the same 64 numbers in every step
+  // (idx = thread + 256 r), and for j <= 64 those touch only the wave's own 128 elements, so such steps follow each
+  // other without a workgroup barrier; one is needed only around the steps with j >= 128.
+  for (uint32_t k = 2; k <= m; k <<= 1) {
+    for (uint32_t j = k >> 1; j > 0; j >>= 1) {
+      for (uint32_t idx = threadIdx.x; idx < (m >> 1); idx += TS_THREADS) {
+        const uint32_t lo = 2 * idx - (idx & (j - 1));
+        const uint32_t hi = lo + j;
+        const uint64_t a = s[lo], b = s[hi];
+        const bool ascending = (lo & k) == 0;
+        if ((a > b) == ascending) {
+          s[lo] = b;
+          s[hi] = a;
+        }
+      }
+      const uint32_t next_j = j > 1 ? (j >> 1) : k;  // first step of the next k is j = k (if there is one)
+      if (j >= 128 || (next_j >= 128 && (j > 1 || 2 * k <= m))) {
+        __syncthreads();
+      } else {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      }
+    }
+  }
+  __syncthreads();
+  const uint64_t tile_bits = (uint64_t)t << 32;
+  for (uint32_t i = threadIdx.x; i < n; i += TS_THREADS) {
+    const uint64_t rec = s[i];
+    const uint32_t e = (uint32_t)rec;
+    keys[start + i] = tile_bits | (rec >> 32);
+    emission[start + i] = e;
+    point_list[start + i] = gauss_of_emission[e];
+  }
+}
+
+}  // namespace
+
+// Tiles the LDS histograms of the counting kernels can hold.
+int bucket_max_tiles() { return 32768; }
+
+// workgroup-by-tile counts, then the tile totals
+size_t bucket_table_bytes(int T) { return ((size_t)BK_MAX_BLOCKS + 1) * (size_t)T * sizeof(uint32_t); }
+
+int launch_bucket_count(int P, int W, int H, const int* radii, const float* means2D, const uint8_t* compute_locally,
+                        uint32_t* tiles_touched, void* table, uint32_t* ranges, uint32_t* longest_out,
+                        hipStream_t stream) {
+  if (P <= 0) return 0;
+  const uint32_t gx = (W + GS_TILE_X - 1) / GS_TILE_X, gy = (H + GS_TILE_Y - 1) / GS_TILE_Y;
+  const uint32_t T = gx * gy;
+  const size_t lds = (size_t)T * sizeof(uint32_t);
+  static bool raised = false;  // more than 64 KB of dynamic LDS has to be asked for once per kernel
+  if (!raised) {
+    GS_HIP_TRY(hipFuncSetAttribute((const void*)bucket_count_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                   bucket_max_tiles() * (int)sizeof(uint32_t)));
+    GS_HIP_TRY(hipFuncSetAttribute((const void*)bucket_scatter_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                   bucket_max_tiles() * (int)sizeof(uint32_t)));
+    raised = true;
+  }
+  const int nb = bucket_blocks(P), per = bucket_per_block(P);
+  uint32_t* tab = (uint32_t*)table;
+  uint32_t* totals = tab + (size_t)BK_MAX_BLOCKS * T;
+  hipLaunchKernelGGL(bucket_count_kernel, dim3(nb), dim3(BK_THREADS), lds, stream, P, per, gx, gy, radii,
+                     (const float2*)means2D, compute_locally, tiles_touched, tab);
+  hipLaunchKernelGGL(bucket_columns_kernel, dim3((T + COL_TILES - 1) / COL_TILES), dim3(COL_TILES * COL_RUNS), 0, stream, nb, T,
+                     tab, totals);
+  hipLaunchKernelGGL(bucket_ranges_kernel, dim3(1), dim3(1024), 0, stream, T, totals, ranges, longest_out);
+  return 0;
+}
+
+int launch_bucket_scatter(int P, int W, int H, const float* means2D, const float* depths, const uint32_t* offsets,
+                          const int* radii, const uint8_t* compute_locally, const void* table,
+                          const uint32_t* ranges, uint64_t* records, uint32_t* gauss_of_emission,
+                          hipStream_t stream) {
+  if (P <= 0) return 0;
+  const uint32_t gx = (W + GS_TILE_X - 1) / GS_TILE_X, gy = (H + GS_TILE_Y - 1) / GS_TILE_Y;
+  const size_t lds = (size_t)gx * gy * sizeof(uint32_t);
+  hipLaunchKernelGGL(bucket_scatter_kernel, dim3(bucket_blocks(P)), dim3(BK_THREADS), lds, stream, P,
+                     bucket_per_block(P), gx, gy, (const float2*)means2D, depths, offsets, radii, compute_locally,
+                     (const uint32_t*)table, ranges, records, gauss_of_emission);
+  return 0;
+}
+
+// Sorts every tile's segment; `longest` is the longest list (lists above small_cap take the larger variant,
+// nothing may exceed TILE_SORT_LARGE).
+int launch_tile_sort(int T, uint32_t longest, uint32_t small_cap, const uint32_t* ranges, const uint64_t* records,
+                     const uint32_t* gauss_of_emission, uint64_t* keys, uint32_t* emission, uint32_t* point_list,
+                     hipStream_t stream) {
+  if (T <= 0 || longest == 0) return 0;
+  if (small_cap > (uint32_t)TILE_SORT_SMALL) small_cap = TILE_SORT_SMALL;
+  hipLaunchKernelGGL(tile_sort_kernel<TILE_SORT_SMALL>, dim3(T), dim3(TS_THREADS), 0, stream, ranges, records,
+                     gauss_of_emission, keys, emission, point_list, 0u, small_cap);
+  if (longest > small_cap)
+    hipLaunchKernelGGL(tile_sort_kernel<TILE_SORT_LARGE>, dim3(T), dim3(TS_THREADS), 0, stream, ranges, records,
+                       gauss_of_emission, keys, emission, point_list, small_cap, (uint32_t)TILE_SORT_LARGE);
+  return 0;
+}
+
+}  // namespace gs

@@ -1,0 +1,137 @@
+"""The per-tile lists render_gaussians builds (ranges, sorted keys, point_list), by each of its routes: instances
+bucketed by tile and sorted per tile in LDS (small and large variant), and the radix sort over all (tile | depth)
+keys.  Every route must give the oracle's lists bit for bit, and the backward pass must file its per-instance
+gradients correctly under each."""
+import ctypes as C
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def H():
+    import gpu_harness
+    return gpu_harness
+
+
+@pytest.fixture(autouse=True)
+def _restore_limits():
+    import gsrast_native as gn
+    yield
+    gn.lib.gs_set_tile_sort_limits(2048, 8192)
+
+
+def _mask(kind, gx, gy):
+    cl = torch.ones(gy, gx, dtype=torch.bool)
+    if kind == "rows":
+        cl[: gy // 3] = False
+    elif kind == "checker":
+        yy, xx = torch.meshgrid(torch.arange(gy), torch.arange(gx), indexing="ij")
+        cl = ((yy + xx) % 2 == 0)
+    return cl
+
+
+# (small limit, large limit): defaults; nearly every tile through the large variant; a list longer than the large
+# limit, found after the counting pass (radix route takes over); radix route from the start
+ROUTES = [(2048, 8192), (8, 8192), (8, 40), (8, 0)]
+
+
+@pytest.mark.parametrize("cfg,P,mask", [(0, 30_000, "all"), (1, 120_000, "all"), (1, 60_000, "checker"),
+                                        (3, 40_000, "rows")])
+def test_lists_match_oracle_by_every_route(orc, H, cfg, P, mask):
+    import gs_scenes
+    import gsrast_native as gn
+    from diff_gaussian_rasterization import _C
+    g, cams = gs_scenes.make_scene(cfg, P=P, n_views=1)
+    cam = cams[0]
+    W, Hh = cam.image_width, cam.image_height
+    gx, gy = H.grid(W, Hh)
+    T = gx * gy
+    cl = _mask(mask, gx, gy)
+    o, gd = H.preprocess_fwd(g, cam)
+    vm, cp = cam.world_view_transform.to(DEV), cam.camera_center.to(DEV)
+    am = gs_scenes.build_all_map(gd["means3D"], gd["scales"], gd["rotations"], cam)
+    n = lambda t: t.detach().cpu().numpy()
+    want = orc.bin_and_sort(n(o["radii"]), n(o["means2D"]), n(o["depths"]), cl.numpy().reshape(-1), W, Hh)
+    R_want = int(want["point_list"].shape[0])
+    counts = want["ranges"].reshape(-1, 2).astype(np.int64)
+    longest = int((counts[:, 1] - counts[:, 0]).max())
+    assert longest > 40  # so that the third route really exceeds its large limit
+    ug = gs_scenes.upstream_grads(cam)
+    args = {"stats_collector": {}}
+    grads = []
+    for small, large in ROUTES:
+        gn.lib.gs_set_tile_sort_limits(small, large)
+        out = _C.render_gaussians(torch.zeros(3, device=DEV), Hh, W, o["means2D"], o["depths"], o["radii"],
+                                  o["conic_opacity"], o["rgb"], cl.to(DEV), vm, cp, cam.tanfovx, cam.tanfovy, am,
+                                  True, False, args)
+        R, color, n_render, n_consider, n_contrib, out_observe, oam, opd, geomB, binB, imgB = out
+        assert R == R_want
+        off = [C.c_size_t() for _ in range(5)]
+        gn.check(gn.lib.gs_binning_state_layout(R, W, Hh, *[C.byref(x) for x in off]), "layout")
+        base = (binB.data_ptr() + 255) // 256 * 256 - binB.data_ptr()
+        point_list = binB[base + off[0].value: base + off[0].value + 4 * R].view(torch.int32)
+        keys = binB[base + off[1].value: base + off[1].value + 8 * R].view(torch.int64)
+        ioff = [C.c_size_t() for _ in range(5)]
+        gn.check(gn.lib.gs_image_state_layout(W, Hh, *[C.byref(x) for x in ioff]), "layout")
+        ibase = (imgB.data_ptr() + 255) // 256 * 256 - imgB.data_ptr()
+        ranges = imgB[ibase + ioff[3].value: ibase + ioff[3].value + 8 * T].view(torch.int32)
+        assert np.array_equal(H.np_u32(ranges), want["ranges"].reshape(-1)), (small, large)
+        assert np.array_equal(H.np_u32(point_list), want["point_list"]), (small, large)
+        assert np.array_equal(H.np_u64(keys), want["keys"]), (small, large)
+        assert np.array_equal(n(n_render), (counts[:, 1] - counts[:, 0]).astype(np.int32))
+        back = _C.render_gaussians_backward(torch.zeros(3, device=DEV), cam.tanfovx, cam.tanfovy, oam, am, R, geomB,
+                                            binB, imgB, cl.to(DEV), ug["color"].to(DEV), ug["all_map"].to(DEV),
+                                            ug["plane_depth"].to(DEV), o["means2D"], o["conic_opacity"], o["rgb"],
+                                            True, False, args)
+        grads.append((color, [b.clone() for b in back]))
+    # the lists are identical, so every route gives the same image bit for bit and the same gradients up to the
+    # order of the LDS sums inside a tile
+    # (pixels of tiles that are not computed locally are left untouched, so only the others are compared)
+    px = cl.repeat_interleave(16, 0).repeat_interleave(16, 1)[:Hh, :W].to(DEV)
+    for color, back in grads[1:]:
+        assert torch.equal(color[:, px], grads[0][0][:, px])
+        for a, b in zip(back, grads[0][1]):
+            assert float((a - b).norm()) <= 1e-5 * float(b.norm()) + 1e-12
+    f = orc.render_fwd(want["ranges"], want["point_list"], n(o["means2D"]), n(o["rgb"]), n(am), n(o["conic_opacity"]),
+                       cl.numpy().reshape(-1), np.zeros(3, np.float32), W, Hh, cam.tanfovx, cam.tanfovy)
+    rb = orc.render_bwd(want["ranges"], want["point_list"], n(o["means2D"]), n(o["conic_opacity"]), n(o["rgb"]), n(am),
+                        f["out_all_map"], f["final_T"], f["n_contrib"], cl.numpy().reshape(-1), np.zeros(3, np.float32),
+                        n(ug["color"]), n(ug["all_map"]), n(ug["plane_depth"]), W, Hh, cam.tanfovx, cam.tanfovy)
+    got = n(grads[0][1][0])
+    assert np.linalg.norm(got[:, :2] - rb["dL_dmeans2D"][:, :2]) <= 1e-3 * np.linalg.norm(rb["dL_dmeans2D"][:, :2])
+
+
+def test_equal_depths_keep_emission_order(orc, H):
+    """Many Gaussians at exactly the same depth: within a tile their order is the emission order (Gaussian index),
+    whichever route builds the list."""
+    import gs_scenes
+    import gsrast_native as gn
+    from diff_gaussian_rasterization import _C
+    g, cams = gs_scenes.make_scene(0, P=20_000, n_views=1)
+    cam = cams[0]
+    W, Hh = cam.image_width, cam.image_height
+    gx, gy = H.grid(W, Hh)
+    o, gd = H.preprocess_fwd(g, cam)
+    o["depths"] = (o["depths"] * 4).round() / 4  # few distinct values
+    cl = torch.ones(gy, gx, dtype=torch.bool)
+    n = lambda t: t.detach().cpu().numpy()
+    want = orc.bin_and_sort(n(o["radii"]), n(o["means2D"]), n(o["depths"]), cl.numpy().reshape(-1), W, Hh)
+    vm, cp = cam.world_view_transform.to(DEV), cam.camera_center.to(DEV)
+    am = gs_scenes.build_all_map(gd["means3D"], gd["scales"], gd["rotations"], cam)
+    for small, large in ROUTES:
+        gn.lib.gs_set_tile_sort_limits(small, large)
+        out = _C.render_gaussians(torch.zeros(3, device=DEV), Hh, W, o["means2D"], o["depths"], o["radii"],
+                                  o["conic_opacity"], o["rgb"], cl.to(DEV), vm, cp, cam.tanfovx, cam.tanfovy, am,
+                                  True, False, {"stats_collector": {}})
+        R, binB = out[0], out[9]
+        off = [C.c_size_t() for _ in range(5)]
+        gn.check(gn.lib.gs_binning_state_layout(R, W, Hh, *[C.byref(x) for x in off]), "layout")
+        base = (binB.data_ptr() + 255) // 256 * 256 - binB.data_ptr()
+        point_list = binB[base + off[0].value: base + off[0].value + 4 * R].view(torch.int32)
+        assert np.array_equal(H.np_u32(point_list), want["point_list"]), (small, large)
