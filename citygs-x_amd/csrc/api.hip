@@ -374,17 +374,16 @@ int wait_for_total(uint32_t* slot, hipStream_t stream, uint32_t* out) {
 }  // namespace
 
 namespace {
-// list lengths at which the per-tile sort hands over to its large variant and to the radix sort
-std::atomic<int> g_tile_sort_small{TILE_SORT_SMALL};
+// whether the per-tile sort keeps the records in registers (or in LDS), and the list length up to which any
+// per-tile sort is used
+std::atomic<int> g_tile_sort_registers{1};
 std::atomic<int> g_tile_sort_large{TILE_SORT_LARGE};
 }  // namespace
 
-void gs_set_tile_sort_limits(int small_limit, int large_limit) {
-  if (small_limit < 1) small_limit = 1;
-  if (small_limit > TILE_SORT_SMALL) small_limit = TILE_SORT_SMALL;
+void gs_set_tile_sort_limits(int in_registers, int large_limit) {
   if (large_limit > TILE_SORT_LARGE) large_limit = TILE_SORT_LARGE;
-  if (large_limit > 0 && large_limit < small_limit) large_limit = small_limit;
-  g_tile_sort_small.store(small_limit);
+  if (large_limit < 0) large_limit = 0;
+  g_tile_sort_registers.store(in_registers != 0 ? 1 : 0);
   g_tile_sort_large.store(large_limit);
 }
 
@@ -500,7 +499,7 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
       if (check_launch("bucket_scatter", stream, dbg)) return 1;
       {
         StageScope _t("tile_sort", stream);
-        launch_tile_sort(T, longest, (uint32_t)g_tile_sort_small.load(), ranges, keys_other, gauss_of_emission, keys,
+        launch_tile_sort(T, longest, (uint32_t)g_tile_sort_registers.load(), ranges, keys_other, gauss_of_emission, keys,
                          emission, point_list, stream);
       }
       if (check_launch("tile_sort", stream, dbg)) return 1;

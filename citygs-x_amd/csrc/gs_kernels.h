@@ -60,8 +60,8 @@ int launch_duplicate_with_keys(int P, int W, int H, const float* means2D, const 
                                uint64_t* keys, uint32_t* values, uint32_t* emission /*optional*/,
                                hipStream_t stream);
 // ---- binning by tile: counting sort by tile + per-tile LDS sort (tile_bucket.hip) ----
-constexpr int TILE_SORT_SMALL = 2048;  // records per tile the small per-tile sort holds
-constexpr int TILE_SORT_LARGE = 8192;  // ... and the large one; longer lists go to the radix sort
+constexpr int TILE_SORT_SMALL = 2048;  // records per tile the small LDS variant holds
+constexpr int TILE_SORT_LARGE = 8192;  // longest list any per-tile sort takes; longer lists go to the radix sort
 int bucket_max_tiles();
 size_t bucket_table_bytes(int T);
 // tiles_touched per Gaussian, the workgroup-by-tile table, ranges (2 words per tile) and the longest list
@@ -73,7 +73,7 @@ int launch_bucket_scatter(int P, int W, int H, const float* means2D, const float
                           const int* radii, const uint8_t* compute_locally, const void* table,
                           const uint32_t* ranges, uint64_t* records, uint32_t* gauss_of_emission,
                           hipStream_t stream);
-int launch_tile_sort(int T, uint32_t longest, uint32_t small_cap, const uint32_t* ranges, const uint64_t* records,
+int launch_tile_sort(int T, uint32_t longest, uint32_t in_registers, const uint32_t* ranges, const uint64_t* records,
                      const uint32_t* gauss_of_emission, uint64_t* keys, uint32_t* emission, uint32_t* point_list,
                      hipStream_t stream);
 int launch_gather_u32(int64_t n, const uint32_t* index, const uint32_t* table, uint32_t* out, hipStream_t stream);

@@ -187,7 +187,140 @@ bucket_scatter_kernel(int P, int per_block, uint32_t gx, uint32_t gy, const floa
   }
 }
 
-// 2. One workgroup per tile: bitonic sort of the tile's records in LDS, then the three sorted arrays the
+// 2. Per-tile sort, register variant: one workgroup of four waves per tile.  A wave holds 64 E records, record
+// i = r * 64 + lane in register r of its lane, and the four waves hold consecutive runs of 64 E, so a list of
+// up to 256 E records is sorted with E = 1 .. 32.  In the bitonic network a step pairs i with i ^ j:
+//   j < 64        the partner sits in another lane, same register: one cross-lane read, keep the smaller or larger;
+//   64 <= j < 64E the partner sits in another register of the same lane: no data moves at all;
+//   j >= 64 E     the partner sits in another wave: one exchange through LDS (three such steps in a whole sort).
+// The direction of a step, ((i & k) == 0) ascending, and which of the pair an element keeps are computed from
+// the indices.  Short dependency chains matter more than instruction count here: every tile is resident at once,
+// so the kernel takes as long as its longest tile, and four waves with few records each finish it soonest.
+constexpr int RS_WAVES = 4;
+
+template <int E>
+__device__ __forceinline__ void exchange_step(uint64_t (&v)[E], const uint64_t (&other)[E], uint32_t row0,
+                                              uint32_t lane, uint32_t k, bool lower) {
+#pragma unroll
+  for (int r = 0; r < E; r++) {
+    const uint32_t i = ((row0 + r) << 6) | lane;
+    const bool ascending = (i & k) == 0;
+    const bool keep_min = lower == ascending;
+    const uint64_t a = v[r], b = other[r];
+    const bool a_less = a < b;
+    v[r] = (a_less == keep_min) ? a : b;
+  }
+}
+
+template <int E>
+__device__ __forceinline__ void register_sort(uint64_t (&v)[E], uint32_t wave, uint32_t lane, uint64_t* s_x) {
+  constexpr uint32_t M = 64u * E * RS_WAVES;
+  const uint32_t row0 = wave * E;
+  for (uint32_t k = 2; k <= M; k <<= 1) {
+    for (uint32_t j = k >> 1; j > 0; j >>= 1) {
+      if (j < 64) {
+        uint64_t other[E];
+#pragma unroll
+        for (int r = 0; r < E; r++) {
+          const uint32_t lo = __shfl_xor((uint32_t)v[r], (int)j, 64);
+          const uint32_t hi = __shfl_xor((uint32_t)(v[r] >> 32), (int)j, 64);
+          other[r] = ((uint64_t)hi << 32) | lo;
+        }
+        exchange_step<E>(v, other, row0, lane, k, (lane & j) == 0);
+      } else if (j < 64u * E) {
+        const uint32_t jr = j >> 6;
+#pragma unroll
+        for (int b = 1; b < E; b <<= 1) {
+          if (jr != (uint32_t)b) continue;
+#pragma unroll
+          for (int r = 0; r < E; r++) {
+            if (r & b) continue;
+            const uint32_t i = ((row0 + r) << 6) | lane;
+            const bool ascending = (i & k) == 0;
+            const uint64_t x = v[r], y = v[r | b];
+            const bool swap = (x > y) == ascending;
+            v[r] = swap ? y : x;
+            v[r | b] = swap ? x : y;
+          }
+        }
+      } else {
+        // partner wave = wave ^ jw: everybody posts, everybody reads the partner's post
+        const uint32_t jw = j / (64u * E);
+        __syncthreads();
+#pragma unroll
+        for (int r = 0; r < E; r++) s_x[((wave * E + r) << 6) | lane] = v[r];
+        __syncthreads();
+        uint64_t other[E];
+#pragma unroll
+        for (int r = 0; r < E; r++) other[r] = s_x[(((wave ^ jw) * E + r) << 6) | lane];
+        exchange_step<E>(v, other, row0, lane, k, (wave & jw) == 0);
+      }
+    }
+  }
+}
+
+template <int E>
+__device__ __forceinline__ void register_sort_tile(uint32_t t, uint32_t start, uint32_t n,
+                                                   const uint64_t* __restrict__ records,
+                                                   const uint32_t* __restrict__ gauss_of_emission,
+                                                   uint64_t* __restrict__ keys, uint32_t* __restrict__ emission,
+                                                   uint32_t* __restrict__ point_list, uint64_t* s_x) {
+  const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  uint64_t v[E];
+#pragma unroll
+  for (int r = 0; r < E; r++) {
+    const uint32_t i = ((wave * E + r) << 6) | lane;
+    v[r] = i < n ? records[start + i] : ~0ull;
+  }
+  register_sort<E>(v, wave, lane, s_x);
+  const uint64_t tile_bits = (uint64_t)t << 32;
+#pragma unroll
+  for (int r = 0; r < E; r++) {
+    const uint32_t i = ((wave * E + r) << 6) | lane;
+    if (i < n) {
+      const uint32_t e = (uint32_t)v[r];
+      keys[start + i] = tile_bits | (v[r] >> 32);
+      emission[start + i] = e;
+      point_list[start + i] = gauss_of_emission[e];
+    }
+  }
+}
+
+// Dynamic LDS: 8 bytes per record of the longest list the kernel takes, rounded up to a power of two (at least
+// 256 records).  Two kernels, so that the common one (lists of up to 2048 records) keeps a small register budget.
+#define GS_SORT_CASE(EE) \
+  register_sort_tile<EE>(t, start, n, records, gauss_of_emission, keys, emission, point_list, s_exchange)
+__global__ void __launch_bounds__(64 * RS_WAVES)
+tile_sort_registers_kernel(const uint32_t* __restrict__ ranges, const uint64_t* __restrict__ records,
+                           const uint32_t* __restrict__ gauss_of_emission, uint64_t* __restrict__ keys,
+                           uint32_t* __restrict__ emission, uint32_t* __restrict__ point_list) {
+  extern __shared__ uint64_t s_exchange[];
+  const uint32_t t = blockIdx.x;
+  const uint32_t start = ranges[2 * t];
+  const uint32_t n = ranges[2 * t + 1] - start;
+  if (n == 0 || n > 2048) return;
+  if (n <= 256) GS_SORT_CASE(1);
+  else if (n <= 512) GS_SORT_CASE(2);
+  else if (n <= 1024) GS_SORT_CASE(4);
+  else GS_SORT_CASE(8);
+}
+
+__global__ void __launch_bounds__(64 * RS_WAVES)
+tile_sort_registers_long_kernel(const uint32_t* __restrict__ ranges, const uint64_t* __restrict__ records,
+                                const uint32_t* __restrict__ gauss_of_emission, uint64_t* __restrict__ keys,
+                                uint32_t* __restrict__ emission, uint32_t* __restrict__ point_list) {
+  extern __shared__ uint64_t s_exchange[];
+  const uint32_t t = blockIdx.x;
+  const uint32_t start = ranges[2 * t];
+  const uint32_t n = ranges[2 * t + 1] - start;
+  if (n <= 2048) return;
+  if (n <= 4096) GS_SORT_CASE(16);
+  else GS_SORT_CASE(32);
+}
+#undef GS_SORT_CASE
+
+// 3. The same sort with the records in LDS (kept as the variant the tests can force): one workgroup per tile,
+// bitonic sort of the tile's records in LDS, then the three sorted arrays the
 // rasterizer keeps: the reference's key (tile << 32 | depth bits), the emission index (the backward pass files
 // per-instance gradients under it) and the Gaussian id.  Handles lists of min_n < n <= max_n <= CAP records.
 template <int CAP>
@@ -287,18 +420,29 @@ int launch_bucket_scatter(int P, int W, int H, const float* means2D, const float
   return 0;
 }
 
-// Sorts every tile's segment; `longest` is the longest list (lists above small_cap take the larger variant,
-// nothing may exceed TILE_SORT_LARGE).
-int launch_tile_sort(int T, uint32_t longest, uint32_t small_cap, const uint32_t* ranges, const uint64_t* records,
+// Sorts every tile's segment; `longest` is the longest list (nothing may exceed TILE_SORT_LARGE).  The register
+// variant by default; with in_registers == 0 the LDS variants (small up to TILE_SORT_SMALL, then large).
+int launch_tile_sort(int T, uint32_t longest, uint32_t in_registers, const uint32_t* ranges, const uint64_t* records,
                      const uint32_t* gauss_of_emission, uint64_t* keys, uint32_t* emission, uint32_t* point_list,
                      hipStream_t stream) {
   if (T <= 0 || longest == 0) return 0;
-  if (small_cap > (uint32_t)TILE_SORT_SMALL) small_cap = TILE_SORT_SMALL;
-  hipLaunchKernelGGL(tile_sort_kernel<TILE_SORT_SMALL>, dim3(T), dim3(TS_THREADS), 0, stream, ranges, records,
-                     gauss_of_emission, keys, emission, point_list, 0u, small_cap);
-  if (longest > small_cap)
-    hipLaunchKernelGGL(tile_sort_kernel<TILE_SORT_LARGE>, dim3(T), dim3(TS_THREADS), 0, stream, ranges, records,
-                       gauss_of_emission, keys, emission, point_list, small_cap, (uint32_t)TILE_SORT_LARGE);
+  if (in_registers == 0) {
+    hipLaunchKernelGGL(tile_sort_kernel<TILE_SORT_SMALL>, dim3(T), dim3(TS_THREADS), 0, stream, ranges, records,
+                       gauss_of_emission, keys, emission, point_list, 0u, (uint32_t)TILE_SORT_SMALL);
+    if (longest > (uint32_t)TILE_SORT_SMALL)
+      hipLaunchKernelGGL(tile_sort_kernel<TILE_SORT_LARGE>, dim3(T), dim3(TS_THREADS), 0, stream, ranges, records,
+                         gauss_of_emission, keys, emission, point_list, (uint32_t)TILE_SORT_SMALL,
+                         (uint32_t)TILE_SORT_LARGE);
+    return 0;
+  }
+  uint32_t m = 256;
+  while (m < longest && m < 2048) m <<= 1;
+  hipLaunchKernelGGL(tile_sort_registers_kernel, dim3(T), dim3(64 * RS_WAVES), (size_t)m * sizeof(uint64_t), stream,
+                     ranges, records, gauss_of_emission, keys, emission, point_list);
+  if (longest > 2048)
+    hipLaunchKernelGGL(tile_sort_registers_long_kernel, dim3(T), dim3(64 * RS_WAVES),
+                       (size_t)(longest > 4096 ? 8192 : 4096) * sizeof(uint64_t), stream, ranges, records,
+                       gauss_of_emission, keys, emission, point_list);
   return 0;
 }
 

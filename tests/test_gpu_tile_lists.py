@@ -23,7 +23,7 @@ def H():
 def _restore_limits():
     import gsrast_native as gn
     yield
-    gn.lib.gs_set_tile_sort_limits(2048, 8192)
+    gn.lib.gs_set_tile_sort_limits(1, 8192)
 
 
 def _mask(kind, gx, gy):
@@ -36,9 +36,9 @@ def _mask(kind, gx, gy):
     return cl
 
 
-# (small limit, large limit): defaults; nearly every tile through the large variant; a list longer than the large
-# limit, found after the counting pass (radix route takes over); radix route from the start
-ROUTES = [(2048, 8192), (8, 8192), (8, 40), (8, 0)]
+# (records in registers?, per-tile limit): defaults; every list through the LDS variants; a list longer than the
+# per-tile limit, found after the counting pass (the radix route takes over); the radix route from the start
+ROUTES = [(1, 8192), (0, 8192), (1, 40), (1, 0)]
 
 
 @pytest.mark.parametrize("cfg,P,mask", [(0, 30_000, "all"), (1, 120_000, "all"), (1, 60_000, "checker"),
@@ -135,3 +135,45 @@ def test_equal_depths_keep_emission_order(orc, H):
         base = (binB.data_ptr() + 255) // 256 * 256 - binB.data_ptr()
         point_list = binB[base + off[0].value: base + off[0].value + 4 * R].view(torch.int32)
         assert np.array_equal(H.np_u32(point_list), want["point_list"]), (small, large)
+
+
+@pytest.mark.parametrize("P,expect", [(28_000, "waves4"), (56_000, "waves8"), (110_000, "radix")])
+def test_long_lists(orc, H, P, expect):
+    """A small image under many large Gaussians: lists of several thousand records per tile (16 and 32 records
+    per lane in the register sort), and beyond 8192 the radix route, which then takes over by itself."""
+    import gs_scenes
+    import gsrast_native as gn
+    from diff_gaussian_rasterization import _C
+    g, cams = gs_scenes.make_scene(0, P=P, n_views=1)
+    cam = cams[0]
+    W, Hh = cam.image_width, cam.image_height
+    gx, gy = H.grid(W, Hh)
+    T = gx * gy
+    g["scales"] = g["scales"] + 0.9  # larger splats: more tiles per Gaussian
+    o, gd = H.preprocess_fwd(g, cam)
+    cl = torch.ones(gy, gx, dtype=torch.bool)
+    n = lambda t: t.detach().cpu().numpy()
+    want = orc.bin_and_sort(n(o["radii"]), n(o["means2D"]), n(o["depths"]), cl.numpy().reshape(-1), W, Hh)
+    counts = want["ranges"].reshape(-1, 2).astype(np.int64)
+    longest = int((counts[:, 1] - counts[:, 0]).max())
+    lo, hi = {"waves4": (2048, 4096), "waves8": (4096, 8192), "radix": (8192, 1 << 30)}[expect]
+    assert lo < longest <= hi, longest
+    vm, cp = cam.world_view_transform.to(DEV), cam.camera_center.to(DEV)
+    am = gs_scenes.build_all_map(gd["means3D"], gd["scales"], gd["rotations"], cam)
+    out = _C.render_gaussians(torch.zeros(3, device=DEV), Hh, W, o["means2D"], o["depths"], o["radii"],
+                              o["conic_opacity"], o["rgb"], cl.to(DEV), vm, cp, cam.tanfovx, cam.tanfovy, am, True,
+                              False, {"stats_collector": {}})
+    R, binB, imgB = out[0], out[9], out[10]
+    assert R == want["point_list"].shape[0]
+    off = [C.c_size_t() for _ in range(5)]
+    gn.check(gn.lib.gs_binning_state_layout(R, W, Hh, *[C.byref(x) for x in off]), "layout")
+    base = (binB.data_ptr() + 255) // 256 * 256 - binB.data_ptr()
+    point_list = binB[base + off[0].value: base + off[0].value + 4 * R].view(torch.int32)
+    keys = binB[base + off[1].value: base + off[1].value + 8 * R].view(torch.int64)
+    ioff = [C.c_size_t() for _ in range(5)]
+    gn.check(gn.lib.gs_image_state_layout(W, Hh, *[C.byref(x) for x in ioff]), "layout")
+    ibase = (imgB.data_ptr() + 255) // 256 * 256 - imgB.data_ptr()
+    ranges = imgB[ibase + ioff[3].value: ibase + ioff[3].value + 8 * T].view(torch.int32)
+    assert np.array_equal(H.np_u32(ranges), want["ranges"].reshape(-1))
+    assert np.array_equal(H.np_u64(keys), want["keys"])
+    assert np.array_equal(H.np_u32(point_list), want["point_list"])
