@@ -18,6 +18,7 @@ namespace {
 constexpr int BK_THREADS = 1024;        // counting and scatter kernels
 constexpr int BK_MAX_BLOCKS = 256;
 constexpr int BK_MIN_PER_BLOCK = 4096;  // Gaussians per workgroup, at least
+constexpr int BK_BATCH = 4;             // Gaussians a thread loads ahead
 constexpr int TS_THREADS = 256;         // per-tile sort
 
 __host__ __device__ inline int bucket_per_block(int P) {
@@ -37,24 +38,40 @@ bucket_count_kernel(int P, int per_block, uint32_t gx, uint32_t gy, const int* _
                     uint32_t* __restrict__ tiles_touched, uint32_t* __restrict__ table) {
   extern __shared__ uint32_t s_hist[];
   const uint32_t T = gx * gy;
-  for (uint32_t t = threadIdx.x; t < T; t += BK_THREADS) s_hist[t] = 0u;
+  uint8_t* s_local = reinterpret_cast<uint8_t*>(s_hist + T);  // the tile mask, read once per visited tile
+  for (uint32_t t = threadIdx.x; t < T; t += BK_THREADS) {
+    s_hist[t] = 0u;
+    s_local[t] = compute_locally[t];
+  }
   __syncthreads();
   const int first = blockIdx.x * per_block;
   const int last = first + per_block < P ? first + per_block : P;
-  for (int i = first + threadIdx.x; i < last; i += BK_THREADS) {
-    uint32_t cnt = 0;
-    const int r = radii[i];
-    if (r > 0) {
-      const float2 p = means2D[i];
-      const Rect rc = get_rect(p.x, p.y, r, gx, gy);
-      for (uint32_t y = rc.y0; y < rc.y1; y++)
-        for (uint32_t x = rc.x0; x < rc.x1; x++)
-          if (compute_locally[y * gx + x]) {
-            atomicAdd(&s_hist[y * gx + x], 1u);
-            cnt++;
-          }
+  // four Gaussians per round: their loads go out together, then each is walked
+  for (int i0 = first + threadIdx.x; i0 < last; i0 += BK_BATCH * BK_THREADS) {
+    int r[BK_BATCH];
+    float2 p[BK_BATCH];
+#pragma unroll
+    for (int q = 0; q < BK_BATCH; q++) {
+      const int i = i0 + q * BK_THREADS;
+      r[q] = i < last ? radii[i] : 0;
+      p[q] = i < last ? means2D[i] : make_float2(0.0f, 0.0f);
     }
-    tiles_touched[i] = cnt;
+#pragma unroll
+    for (int q = 0; q < BK_BATCH; q++) {
+      const int i = i0 + q * BK_THREADS;
+      if (i >= last) break;
+      uint32_t cnt = 0;
+      if (r[q] > 0) {
+        const Rect rc = get_rect(p[q].x, p[q].y, r[q], gx, gy);
+        for (uint32_t y = rc.y0; y < rc.y1; y++)
+          for (uint32_t x = rc.x0; x < rc.x1; x++)
+            if (s_local[y * gx + x]) {
+              atomicAdd(&s_hist[y * gx + x], 1u);
+              cnt++;
+            }
+      }
+      tiles_touched[i] = cnt;
+    }
   }
   __syncthreads();
   uint32_t* row = table + (size_t)blockIdx.x * T;
@@ -164,26 +181,43 @@ bucket_scatter_kernel(int P, int per_block, uint32_t gx, uint32_t gy, const floa
                       uint64_t* __restrict__ records, uint32_t* __restrict__ gauss_of_emission) {
   extern __shared__ uint32_t s_next[];
   const uint32_t T = gx * gy;
+  uint8_t* s_local = reinterpret_cast<uint8_t*>(s_next + T);
   const uint32_t* row = table + (size_t)blockIdx.x * T;
-  for (uint32_t t = threadIdx.x; t < T; t += BK_THREADS) s_next[t] = ranges[2 * t] + row[t];
+  for (uint32_t t = threadIdx.x; t < T; t += BK_THREADS) {
+    s_next[t] = ranges[2 * t] + row[t];
+    s_local[t] = compute_locally[t];
+  }
   __syncthreads();
   const int first = blockIdx.x * per_block;
   const int last = first + per_block < P ? first + per_block : P;
-  for (int i = first + threadIdx.x; i < last; i += BK_THREADS) {
-    const int r = radii[i];
-    if (r <= 0) continue;
-    uint32_t e = (i == 0) ? 0u : offsets[i - 1];
-    const float2 p = means2D[i];
-    const Rect rc = get_rect(p.x, p.y, r, gx, gy);
-    const uint64_t hi = (uint64_t)__float_as_uint(depths[i]) << 32;
-    for (uint32_t y = rc.y0; y < rc.y1; y++)
-      for (uint32_t x = rc.x0; x < rc.x1; x++)
-        if (compute_locally[y * gx + x]) {
-          const uint32_t pos = atomicAdd(&s_next[y * gx + x], 1u);
-          records[pos] = hi | (uint64_t)e;
-          gauss_of_emission[e] = (uint32_t)i;
-          e++;
-        }
+  for (int i0 = first + threadIdx.x; i0 < last; i0 += BK_BATCH * BK_THREADS) {
+    int r[BK_BATCH];
+    float2 p[BK_BATCH];
+    uint32_t e0[BK_BATCH], dbits[BK_BATCH];
+#pragma unroll
+    for (int q = 0; q < BK_BATCH; q++) {
+      const int i = i0 + q * BK_THREADS;
+      r[q] = i < last ? radii[i] : 0;
+      p[q] = i < last ? means2D[i] : make_float2(0.0f, 0.0f);
+      dbits[q] = i < last ? __float_as_uint(depths[i]) : 0u;
+      e0[q] = (i < last && i > 0) ? offsets[i - 1] : 0u;
+    }
+#pragma unroll
+    for (int q = 0; q < BK_BATCH; q++) {
+      const int i = i0 + q * BK_THREADS;
+      if (i >= last || r[q] <= 0) continue;
+      uint32_t e = e0[q];
+      const Rect rc = get_rect(p[q].x, p[q].y, r[q], gx, gy);
+      const uint64_t hi = (uint64_t)dbits[q] << 32;
+      for (uint32_t y = rc.y0; y < rc.y1; y++)
+        for (uint32_t x = rc.x0; x < rc.x1; x++)
+          if (s_local[y * gx + x]) {
+            const uint32_t pos = atomicAdd(&s_next[y * gx + x], 1u);
+            records[pos] = hi | (uint64_t)e;
+            gauss_of_emission[e] = (uint32_t)i;
+            e++;
+          }
+    }
   }
 }
 
@@ -376,7 +410,7 @@ tile_sort_kernel(const uint32_t* __restrict__ ranges, const uint64_t* __restrict
 }  // namespace
 
 // Tiles the LDS histograms of the counting kernels can hold.
-int bucket_max_tiles() { return 32768; }
+int bucket_max_tiles() { return 30000; }
 
 // workgroup-by-tile counts, then the tile totals
 size_t bucket_table_bytes(int T) { return ((size_t)BK_MAX_BLOCKS + 1) * (size_t)T * sizeof(uint32_t); }
@@ -387,13 +421,13 @@ int launch_bucket_count(int P, int W, int H, const int* radii, const float* mean
   if (P <= 0) return 0;
   const uint32_t gx = (W + GS_TILE_X - 1) / GS_TILE_X, gy = (H + GS_TILE_Y - 1) / GS_TILE_Y;
   const uint32_t T = gx * gy;
-  const size_t lds = (size_t)T * sizeof(uint32_t);
+  const size_t lds = (size_t)T * (sizeof(uint32_t) + 1);
   static bool raised = false;  // more than 64 KB of dynamic LDS has to be asked for once per kernel
   if (!raised) {
     GS_HIP_TRY(hipFuncSetAttribute((const void*)bucket_count_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                   bucket_max_tiles() * (int)sizeof(uint32_t)));
+                                   bucket_max_tiles() * (int)(sizeof(uint32_t) + 1)));
     GS_HIP_TRY(hipFuncSetAttribute((const void*)bucket_scatter_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                   bucket_max_tiles() * (int)sizeof(uint32_t)));
+                                   bucket_max_tiles() * (int)(sizeof(uint32_t) + 1)));
     raised = true;
   }
   const int nb = bucket_blocks(P), per = bucket_per_block(P);
@@ -413,7 +447,7 @@ int launch_bucket_scatter(int P, int W, int H, const float* means2D, const float
                           hipStream_t stream) {
   if (P <= 0) return 0;
   const uint32_t gx = (W + GS_TILE_X - 1) / GS_TILE_X, gy = (H + GS_TILE_Y - 1) / GS_TILE_Y;
-  const size_t lds = (size_t)gx * gy * sizeof(uint32_t);
+  const size_t lds = (size_t)gx * gy * (sizeof(uint32_t) + 1);
   hipLaunchKernelGGL(bucket_scatter_kernel, dim3(bucket_blocks(P)), dim3(BK_THREADS), lds, stream, P,
                      bucket_per_block(P), gx, gy, (const float2*)means2D, depths, offsets, radii, compute_locally,
                      (const uint32_t*)table, ranges, records, gauss_of_emission);

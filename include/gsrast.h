@@ -94,7 +94,7 @@ int gs_preprocess_backward(const int* radii, const float* cov3D, const uint8_t* 
 
 /* No counterpart in the reference: a test hook.  gs_render_forward builds the per-tile lists either by
  * bucketing the instances by tile and sorting each tile's list on its own (lists of up to 8192 records), or, when
- * a list is longer than that (or the tile grid larger than 32768 tiles), by the reference's own route:
+ * a list is longer than that (or the tile grid larger than 30000 tiles), by the reference's own route:
  * (tile | depth) keys (rasterizer_impl.cu:74-117), one radix sort over all of them (:675-684), identifyTileRanges
  * (:122-144).  All give the same lists bit for bit.  in_registers = 0 makes the per-tile sort keep its records in
  * LDS instead of registers (default 1); large_limit lowers the list length up to which a per-tile sort is used
