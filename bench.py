@@ -33,7 +33,10 @@ BYTES_PER_GAUSSIAN = {
 }
 # sort: one 8 B histogram read + 5 passes (9-bit digits over the 44 key bits) x (12 B read + 12 B write)
 # tile ranges: 8 B key read, plus the gather of the sorted Gaussian ids fused into it (index, table, output: 12 B)
-BYTES_PER_INSTANCE = {"sort_pairs": 128, "identify_tile_ranges": 20}
+# tile_sort: 8 B record + 4 B Gaussian id in, 8 B key + 4 B emission index + 4 B Gaussian id out.
+# sort_pairs: the radix sort (5 passes of 9-bit digits over 44 key bits), timed on its own on keys of the same
+# distribution: the per-tile lists are built without it unless a list exceeds 8192 records.
+BYTES_PER_INSTANCE = {"sort_pairs": 128, "identify_tile_ranges": 20, "tile_sort": 28}
 FP32_MATRIX_PEAK_TFLOPS = 157.3
 # Neural-Gaussian generation with 10 offsets: (bytes per anchor, bytes per selected Gaussian, flops per anchor).
 #   opacity:   feat 128 + anchor 12 in; 10 opacities, 10 mask bytes, 1 count out;      2 (35*32 + 32*10) flops
@@ -217,6 +220,28 @@ def main():
         l1m, ssm = gs_loss.pixelwise_l1_ssim_with_mask(img_l, gt, pm)
         torch.autograd.backward([l1m, ssm], [gt, gt])
     del l1m, ssm
+    # the radix sort on its own: (tile << 32 | depth bits) keys with this view's number of instances per tile, in
+    # random order, 32-bit payload
+    import ctypes as C
+    n_per_tile = info["n_render"].to(torch.int64)
+    R_s = int(n_per_tile.sum().item())
+    gen_s = torch.Generator(device=dev).manual_seed(11)
+    s_tiles = torch.repeat_interleave(torch.arange(n_per_tile.numel(), device=dev), n_per_tile)
+    s_depth = (torch.rand(R_s, generator=gen_s, device=dev) * 99.0 + 1.0).view(torch.int32).to(torch.int64)
+    s_keys = ((s_tiles << 32) | s_depth)[torch.randperm(R_s, generator=gen_s, device=dev)].contiguous()
+    s_vals = torch.arange(R_s, dtype=torch.int32, device=dev)
+    s_kout, s_vout = torch.empty_like(s_keys), torch.empty_like(s_vals)
+    s_ws_bytes = gn.lib.gs_sort_workspace_bytes(R_s)
+    s_ws = torch.empty(s_ws_bytes, dtype=torch.uint8, device=dev)
+    s_end_bit = 32 + gn.lib.gs_higher_msb(gx * gy)
+    s_ptr = lambda t: C.c_void_p(t.data_ptr())
+    torch.cuda._sleep(int(4e7))
+    for _ in range(args.steps):
+        gn.check(gn.lib.gs_sort_pairs_u64(R_s, s_ptr(s_keys), s_ptr(s_kout), s_ptr(s_vals), s_ptr(s_vout), s_end_bit,
+                                          s_ptr(s_ws), s_ws_bytes,
+                                          C.c_void_p(torch.cuda.current_stream().cuda_stream)), "gs_sort_pairs_u64")
+    assert bool((s_kout[1:] >= s_kout[:-1]).all())
+    del s_tiles, s_depth, s_keys, s_vals, s_kout, s_vout, s_ws
     # neural-Gaussian generation for one view: 200 k visible anchors x 10 offsets through the three MLPs,
     # forward (opacity MLP, scan, color/cov MLPs + post-processing) and backward
     torch.cuda._sleep(int(4e7))
@@ -322,7 +347,7 @@ def main():
             nbytes = BYTES_PER_GAUSSIAN[name] * P
         elif name in BYTES_PER_INSTANCE:
             nbytes = BYTES_PER_INSTANCE[name] * R
-        elif name == "duplicate_with_keys":
+        elif name in ("duplicate_with_keys", "bucket_scatter"):
             nbytes = 20 * P + 12 * R
         elif name == "ssim_l1_fwd":
             nbytes = (8 + 8 + 12) * 3 * H * W + H * W  # two images in, two maps + three derivative maps out, mask

@@ -940,6 +940,7 @@ int gs_sort_pairs_u64(int64_t n, uint64_t* keys_in, uint64_t* keys_out, uint32_t
   GS_REQUIRE(keys_in && keys_out && vals_in && vals_out && workspace, "gs_sort_pairs_u64: null pointer");
   GS_REQUIRE(workspace_bytes >= gs_sort_workspace_bytes(n), "gs_sort_pairs_u64: workspace too small");
   void* temp = align_ptr((char*)workspace, 256);
+  StageScope _t("sort_pairs", stream);
   if (sort_result_in_b(end_bit)) {
     if (launch_sort_pairs_u64(n, keys_in, keys_out, vals_in, vals_out, end_bit, temp, stream)) return 1;
   } else {
