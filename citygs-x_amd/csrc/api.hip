@@ -437,8 +437,10 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
   bool bucketed = counted_by_tile;
   if (bucketed) {
     StageScope _t("tile_count", stream);
+    // the histogram's grand total is the instance count: the host gets it from here, and the prefix over the
+    // Gaussians below runs while the host is busy growing the binning buffer
     if (launch_bucket_count(P, width, height, radii, means2D, compute_locally, tiles_touched, bucket_table, ranges,
-                            total_slot + 1, stream))
+                            total_slot, stream))
       return 1;
   } else {
     StageScope _t("tile_count", stream);
@@ -450,14 +452,14 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
   if (check_launch("tile_count", stream, dbg)) return 1;
   {
     StageScope _t("inclusive_sum", stream);
-    launch_inclusive_sum(P, tiles_touched, point_offsets, scan_temp, stream, total_slot);
+    launch_inclusive_sum(P, tiles_touched, point_offsets, scan_temp, stream, bucketed ? nullptr : total_slot);
   }
   if (check_launch("inclusive_sum", stream, dbg)) return 1;
 
   // The instance count decides the size of the binning buffer, so the host needs it here.  The scan writes
   // it straight into pinned host memory and the host polls that word: no copy, and no sleeping wait whose
-  // wake-up would leave the GPU idle.  The longest tile list sits in the word beside it, written by a kernel
-  // that ran before the scan.
+  // wake-up would leave the GPU idle.  On the bucketed route the count and, in the word beside it, the longest
+  // tile list come from the kernel that builds the tile ranges.
   uint32_t R_u = 0, longest = 0;
   if (total_slot != nullptr) {
     if (wait_for_total(total_slot, stream, &R_u)) return 1;

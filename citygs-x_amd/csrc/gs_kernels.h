@@ -64,10 +64,10 @@ constexpr int TILE_SORT_SMALL = 2048;  // records per tile the small LDS variant
 constexpr int TILE_SORT_LARGE = 8192;  // longest list any per-tile sort takes; longer lists go to the radix sort
 int bucket_max_tiles();
 size_t bucket_table_bytes(int T);
-// tiles_touched per Gaussian, the workgroup-by-tile table, ranges (2 words per tile) and the longest list
-// (a host-visible word)
+// tiles_touched per Gaussian, the workgroup-by-tile table, ranges (2 words per tile), and in two host-visible
+// words the number of instances (word 0, written last) and the longest list (word 1)
 int launch_bucket_count(int P, int W, int H, const int* radii, const float* means2D, const uint8_t* compute_locally,
-                        uint32_t* tiles_touched, void* table, uint32_t* ranges, uint32_t* longest_out,
+                        uint32_t* tiles_touched, void* table, uint32_t* ranges, uint32_t* host_words,
                         hipStream_t stream);
 int launch_bucket_scatter(int P, int W, int H, const float* means2D, const float* depths, const uint32_t* offsets,
                           const int* radii, const uint8_t* compute_locally, const void* table,

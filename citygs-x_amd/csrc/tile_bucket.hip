@@ -126,10 +126,11 @@ __device__ __forceinline__ uint32_t wave_inclusive_scan_u32(uint32_t v, int lane
 }
 
 // 1c. One workgroup: exclusive prefix of the tile totals = the tile ranges (rasterizer_impl.cu:122-144 leaves
-// (0, 0) for a tile without instances), and the longest list, stored where the host can read it.
+// (0, 0) for a tile without instances).  The longest list and then the number of instances are stored where the
+// host can read them (host_words[1] and host_words[0]; the host polls word 0, so it is written last).
 __global__ void __launch_bounds__(1024)
 bucket_ranges_kernel(uint32_t T, const uint32_t* __restrict__ totals, uint32_t* __restrict__ ranges,
-                     uint32_t* __restrict__ longest_out) {
+                     uint32_t* __restrict__ host_words) {
   __shared__ uint32_t s_wave[16], s_max[16];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   uint32_t carry = 0, longest = 0;
@@ -165,7 +166,8 @@ bucket_ranges_kernel(uint32_t T, const uint32_t* __restrict__ totals, uint32_t* 
   if (threadIdx.x == 0) {
     uint32_t m = 0;
     for (int w = 0; w < 16; w++) m = s_max[w] > m ? s_max[w] : m;
-    __hip_atomic_store(longest_out, m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    __hip_atomic_store(host_words + 1, m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    __hip_atomic_store(host_words, carry, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
   }
 }
 
@@ -416,7 +418,7 @@ int bucket_max_tiles() { return 30000; }
 size_t bucket_table_bytes(int T) { return ((size_t)BK_MAX_BLOCKS + 1) * (size_t)T * sizeof(uint32_t); }
 
 int launch_bucket_count(int P, int W, int H, const int* radii, const float* means2D, const uint8_t* compute_locally,
-                        uint32_t* tiles_touched, void* table, uint32_t* ranges, uint32_t* longest_out,
+                        uint32_t* tiles_touched, void* table, uint32_t* ranges, uint32_t* host_words,
                         hipStream_t stream) {
   if (P <= 0) return 0;
   const uint32_t gx = (W + GS_TILE_X - 1) / GS_TILE_X, gy = (H + GS_TILE_Y - 1) / GS_TILE_Y;
@@ -437,7 +439,7 @@ int launch_bucket_count(int P, int W, int H, const int* radii, const float* mean
                      (const float2*)means2D, compute_locally, tiles_touched, tab);
   hipLaunchKernelGGL(bucket_columns_kernel, dim3((T + COL_TILES - 1) / COL_TILES), dim3(COL_TILES * COL_RUNS), 0, stream, nb, T,
                      tab, totals);
-  hipLaunchKernelGGL(bucket_ranges_kernel, dim3(1), dim3(1024), 0, stream, T, totals, ranges, longest_out);
+  hipLaunchKernelGGL(bucket_ranges_kernel, dim3(1), dim3(1024), 0, stream, T, totals, ranges, host_words);
   return 0;
 }
 
