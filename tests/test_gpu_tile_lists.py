@@ -177,3 +177,38 @@ def test_long_lists(orc, H, P, expect):
     assert np.array_equal(H.np_u32(ranges), want["ranges"].reshape(-1))
     assert np.array_equal(H.np_u64(keys), want["keys"])
     assert np.array_equal(H.np_u32(point_list), want["point_list"])
+
+
+def test_grid_too_large_for_the_tile_histogram(orc, H):
+    """3840x2160 is 32400 tiles, more than the counting kernels keep in LDS: the radix route is taken from the start."""
+    import gs_scenes
+    import gsrast_native as gn
+    from diff_gaussian_rasterization import _C
+    cam = gs_scenes.look_at_camera((0.0, 0.0, -30.0), (0, 0, 0), 3840, 2160, 60.0, up=(0.0, -1.0, 0.0))
+    g, _ = gs_scenes.make_scene(0, P=20_000, n_views=1)
+    W, Hh = cam.image_width, cam.image_height
+    gx, gy = H.grid(W, Hh)
+    T = gx * gy
+    assert T > 30000
+    o, gd = H.preprocess_fwd(g, cam)
+    cl = torch.ones(gy, gx, dtype=torch.bool)
+    n = lambda t: t.detach().cpu().numpy()
+    want = orc.bin_and_sort(n(o["radii"]), n(o["means2D"]), n(o["depths"]), cl.numpy().reshape(-1), W, Hh)
+    assert want["point_list"].shape[0] > 1000
+    vm, cp = cam.world_view_transform.to(DEV), cam.camera_center.to(DEV)
+    am = gs_scenes.build_all_map(gd["means3D"], gd["scales"], gd["rotations"], cam)
+    out = _C.render_gaussians(torch.zeros(3, device=DEV), Hh, W, o["means2D"], o["depths"], o["radii"],
+                              o["conic_opacity"], o["rgb"], cl.to(DEV), vm, cp, cam.tanfovx, cam.tanfovy, am, True,
+                              False, {"stats_collector": {}})
+    R, binB, imgB = out[0], out[9], out[10]
+    assert R == want["point_list"].shape[0]
+    off = [C.c_size_t() for _ in range(5)]
+    gn.check(gn.lib.gs_binning_state_layout(R, W, Hh, *[C.byref(x) for x in off]), "layout")
+    base = (binB.data_ptr() + 255) // 256 * 256 - binB.data_ptr()
+    point_list = binB[base + off[0].value: base + off[0].value + 4 * R].view(torch.int32)
+    ioff = [C.c_size_t() for _ in range(5)]
+    gn.check(gn.lib.gs_image_state_layout(W, Hh, *[C.byref(x) for x in ioff]), "layout")
+    ibase = (imgB.data_ptr() + 255) // 256 * 256 - imgB.data_ptr()
+    ranges = imgB[ibase + ioff[3].value: ibase + ioff[3].value + 8 * T].view(torch.int32)
+    assert np.array_equal(H.np_u32(ranges), want["ranges"].reshape(-1))
+    assert np.array_equal(H.np_u32(point_list), want["point_list"])
