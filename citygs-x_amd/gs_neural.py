@@ -122,8 +122,10 @@ def generate_neural_gaussians(viewpoint_camera, pc, visible_mask=None, is_traini
     if visible_mask is None:
         anchor, feat, offsets, scaling = pc.get_anchor, pc.get_anchor_feat, pc._offset, pc.get_scaling
     else:
-        anchor, feat = pc.get_anchor[visible_mask], pc.get_anchor_feat[visible_mask]
-        offsets, scaling = pc._offset[visible_mask], pc.get_scaling[visible_mask]
+        # one nonzero() (one host synchronisation) serves the four gathers; x[visible_mask] would run it four times
+        idx = visible_mask.nonzero(as_tuple=True)[0]
+        anchor, feat = pc.get_anchor.index_select(0, idx), pc.get_anchor_feat.index_select(0, idx)
+        offsets, scaling = pc._offset.index_select(0, idx), pc.get_scaling.index_select(0, idx)
     out = neural_gaussians(anchor, feat, offsets, scaling, viewpoint_camera.camera_center,
                            _linear_pair(pc.get_opacity_mlp), _linear_pair(pc.get_color_mlp),
                            _linear_pair(pc.get_cov_mlp))
