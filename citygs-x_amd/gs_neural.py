@@ -1,8 +1,9 @@
 """Neural-Gaussian generation of the reference, generate_neural_gaussians (gaussian_renderer/__init__.py:789-899),
 as three kernel launches forward (opacity MLP, scan, color/cov MLPs with the post-processing) and two backward,
-in libgsrast.so.  Covers the reference's default model configuration (arguments/__init__.py:94-124): feat_dim 32,
-no feature bank, no appearance embedding, no distance or level inputs to the MLPs, dist2level other than
-'progressive'; anything else raises NotImplementedError."""
+in libgsrast.so.  The fused operator is the reference's default model configuration (arguments/__init__.py:94-124):
+feat_dim 32, inputs [feature, view direction]; the drop-in function also serves the appearance embedding and the
+feature bank, which reduce to it; distance or level inputs to the MLPs and dist2level 'progressive' raise
+NotImplementedError."""
 import ctypes as C
 
 import torch
@@ -114,11 +115,15 @@ def _linear_pair(seq):
 
 
 def generate_neural_gaussians(viewpoint_camera, pc, visible_mask=None, is_training=False, ape_code=-1):
-    """Same signature and results as gaussian_renderer/__init__.py:789-899."""
-    if (pc.use_feat_bank or pc.appearance_dim > 0 or pc.add_opacity_dist or pc.add_color_dist or pc.add_cov_dist
-            or pc.add_level or pc.dist2level == "progressive"):
-        raise NotImplementedError("generate_neural_gaussians: only the default model configuration (no feature bank, "
-                                  "appearance embedding, distance or level inputs, progressive levels) is built")
+    """Same signature and results as gaussian_renderer/__init__.py:789-899.  Served: the default configuration,
+    the appearance embedding (appearance_dim > 0: every anchor of a view gets the same embedding row, :830-836,
+    :866-868, so its part of the first color layer is a per-view addition to that layer's bias) and the feature
+    bank (use_feat_bank, :809-823: the view-dependent mix of the feature's resolutions is a few torch lines ahead
+    of the fused operator).  The distance / level inputs and progressive levels raise NotImplementedError."""
+    if (pc.add_opacity_dist or pc.add_color_dist or pc.add_cov_dist or pc.add_level
+            or pc.dist2level == "progressive"):
+        raise NotImplementedError("generate_neural_gaussians: distance or level inputs to the MLPs and progressive "
+                                  "levels are not built")
     if visible_mask is None:
         anchor, feat, offsets, scaling = pc.get_anchor, pc.get_anchor_feat, pc._offset, pc.get_scaling
     else:
@@ -126,7 +131,21 @@ def generate_neural_gaussians(viewpoint_camera, pc, visible_mask=None, is_traini
         idx = visible_mask.nonzero(as_tuple=True)[0]
         anchor, feat = pc.get_anchor.index_select(0, idx), pc.get_anchor_feat.index_select(0, idx)
         offsets, scaling = pc._offset.index_select(0, idx), pc.get_scaling.index_select(0, idx)
+    if pc.use_feat_bank:
+        ob_view = anchor - viewpoint_camera.camera_center
+        ob_view = ob_view / ob_view.norm(dim=1, keepdim=True)
+        bank_weight = pc.get_featurebank_mlp(ob_view).unsqueeze(dim=1)  # [n, 1, 3]
+        f = feat.unsqueeze(dim=-1)
+        f = f[:, ::4, :1].repeat([1, 4, 1]) * bank_weight[:, :, :1] + \
+            f[:, ::2, :1].repeat([1, 2, 1]) * bank_weight[:, :, 1:2] + \
+            f[:, ::1, :1] * bank_weight[:, :, 2:]
+        feat = f.squeeze(dim=-1)
+    color_mlp = _linear_pair(pc.get_color_mlp)
+    if pc.appearance_dim > 0:
+        cam_id = viewpoint_camera.uid if (is_training or ape_code < 0) else ape_code[0]
+        row = pc.get_appearance(torch.tensor([cam_id], dtype=torch.long, device=anchor.device))[0]
+        W1 = color_mlp[0]
+        color_mlp = (W1[:, :35].contiguous(), color_mlp[1] + W1[:, 35:] @ row, color_mlp[2], color_mlp[3])
     out = neural_gaussians(anchor, feat, offsets, scaling, viewpoint_camera.camera_center,
-                           _linear_pair(pc.get_opacity_mlp), _linear_pair(pc.get_color_mlp),
-                           _linear_pair(pc.get_cov_mlp))
+                           _linear_pair(pc.get_opacity_mlp), color_mlp, _linear_pair(pc.get_cov_mlp))
     return out if is_training else out[:5]

@@ -154,6 +154,79 @@ def test_drop_in_signature():
         for lin in (q[0], q[2]):
             assert bool(torch.isfinite(lin.weight.grad).all()) and float(lin.weight.grad.abs().max()) > 0.0
     assert float(pc.get_opacity_mlp[2].weight.grad.abs().max()) == 0.0
-    pc.use_feat_bank = True
+    pc.add_cov_dist = True
     with pytest.raises(NotImplementedError):
         generate_neural_gaussians(cam, pc, vis)
+
+
+def test_drop_in_with_appearance_embedding_and_feature_bank():
+    """appearance_dim > 0 and use_feat_bank, against the reference's statements for them
+    (gaussian_renderer/__init__.py:809-836, :866-870) run by torch."""
+    import types
+    import torch.nn as nn
+    from gs_neural import generate_neural_gaussians
+    N, k, A = 400, 10, 32
+    s = gs_scenes.make_anchor_scene(N, k, 13)
+    torch.manual_seed(4)
+    mlp_op = nn.Sequential(nn.Linear(35, 32), nn.ReLU(True), nn.Linear(32, k), nn.Tanh()).to(DEV)
+    mlp_cov = nn.Sequential(nn.Linear(35, 32), nn.ReLU(True), nn.Linear(32, 7 * k)).to(DEV)
+    mlp_col = nn.Sequential(nn.Linear(35 + A, 32), nn.ReLU(True), nn.Linear(32, 3 * k), nn.Sigmoid()).to(DEV)
+    bank = nn.Sequential(nn.Linear(3, 32), nn.ReLU(True), nn.Linear(32, 3), nn.Softmax(dim=1)).to(DEV)
+    emb = nn.Embedding(7, A).to(DEV)
+    leaf = lambda t: t.to(DEV).requires_grad_(True)
+    pc = types.SimpleNamespace(
+        use_feat_bank=True, appearance_dim=A, add_opacity_dist=False, add_color_dist=False, add_cov_dist=False,
+        add_level=False, dist2level="round", n_offsets=k, get_anchor=leaf(s["anchor"]),
+        get_anchor_feat=leaf(s["feat"]), _offset=leaf(s["offsets"]), get_scaling=leaf(s["scaling"]),
+        get_opacity_mlp=mlp_op, get_color_mlp=mlp_col, get_cov_mlp=mlp_cov, get_featurebank_mlp=bank,
+        get_appearance=emb)
+    cam = types.SimpleNamespace(camera_center=s["campos"].to(DEV), uid=3)
+    vis = (torch.rand(N, generator=torch.Generator().manual_seed(2)) < 0.7).to(DEV)
+
+    def reference():
+        anchor, feat = pc.get_anchor[vis], pc.get_anchor_feat[vis]
+        grid_offsets, grid_scaling = pc._offset[vis], pc.get_scaling[vis]
+        ob_view = anchor - cam.camera_center
+        ob_dist = ob_view.norm(dim=1, keepdim=True)
+        ob_view = ob_view / ob_dist
+        bank_weight = bank(ob_view).unsqueeze(dim=1)
+        feat = feat.unsqueeze(dim=-1)
+        feat = feat[:, ::4, :1].repeat([1, 4, 1]) * bank_weight[:, :, :1] + \
+            feat[:, ::2, :1].repeat([1, 2, 1]) * bank_weight[:, :, 1:2] + feat[:, ::1, :1] * bank_weight[:, :, 2:]
+        feat = feat.squeeze(dim=-1)
+        x = torch.cat([feat, ob_view], dim=1)
+        camera_indicies = torch.ones_like(x[:, 0], dtype=torch.long) * cam.uid
+        appearance = emb(camera_indicies)
+        neural_opacity = mlp_op(x).reshape([-1, 1])
+        mask = (neural_opacity > 0.0).view(-1)
+        opacity = neural_opacity[mask]
+        color = mlp_col(torch.cat([x, appearance], dim=1)).reshape([anchor.shape[0] * k, 3])
+        scale_rot = mlp_cov(x).reshape([anchor.shape[0] * k, 7])
+        offsets = grid_offsets.view([-1, 3])
+        cat = torch.cat([grid_scaling, anchor], dim=-1).repeat_interleave(k, dim=0)
+        masked = torch.cat([cat, color, scale_rot, offsets], dim=-1)[mask]
+        scaling_repeat, repeat_anchor, color, scale_rot, offsets = masked.split([6, 3, 3, 7, 3], dim=-1)
+        scaling = scaling_repeat[:, 3:] * torch.sigmoid(scale_rot[:, :3])
+        rot = torch.nn.functional.normalize(scale_rot[:, 3:7])
+        xyz = repeat_anchor + offsets * scaling_repeat[:, :3]
+        return xyz, color, opacity, scaling, rot, neural_opacity, mask
+
+    params = [pc.get_anchor, pc.get_anchor_feat, pc._offset, pc.get_scaling, emb.weight] + \
+        [p for m in (mlp_op, mlp_col, mlp_cov, bank) for p in m.parameters()]
+    ups = None
+    grads = []
+    for fn in (lambda: generate_neural_gaussians(cam, pc, vis, is_training=True), reference):
+        for p in params:
+            p.grad = None
+        out = fn()
+        if ups is None:
+            ups = [torch.randn_like(o) for o in out[:5]]
+            first = out
+        else:
+            assert torch.equal(out[6], first[6])
+            for o, r in zip(first[:6], out[:6]):
+                assert float((o - r).norm() / r.norm()) <= 5e-6
+        torch.autograd.backward(list(out[:5]), ups)
+        grads.append([p.grad.clone() for p in params])
+    for i, (a, b) in enumerate(zip(*grads)):
+        assert float((a - b).norm()) <= 2e-4 * float(b.norm()) + 1e-12, i
