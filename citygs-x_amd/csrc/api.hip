@@ -393,8 +393,9 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
                       const float* viewmatrix, const float* cam_pos, const float* all_map, const float* means2D,
                       const float* depths, const int* radii, const float* conic_opacity, const float* rgb,
                       const uint8_t* compute_locally, float* out_color, int* n_render, int* n_consider,
-                      int* n_contrib, int* out_observe, float* out_all_map, float* out_plane_depth, int render_geo,
-                      int debug, int* num_rendered, float* elapsed_ms, gs_stream_t stream_) {
+                      int* n_contrib, int* out_observe, float* out_all_map, float* out_plane_depth,
+                      float* out_max_weight_depth, int render_geo, int debug, int* num_rendered, float* elapsed_ms,
+                      gs_stream_t stream_) {
   (void)viewmatrix;
   (void)cam_pos;
   hipStream_t stream = (hipStream_t)stream_;
@@ -547,6 +548,7 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
   a.final_T = accum_alpha; a.n_contrib_px = n_contrib_px; a.n_contrib2loss_px = n_contrib2loss_px;
   a.out_color = out_color; a.out_observe = out_observe; a.out_all_map = out_all_map;
   a.out_plane_depth = out_plane_depth;
+  a.depths = depths; a.out_max_weight_depth = out_max_weight_depth;
   a.n_render = n_render; a.n_consider = n_consider; a.n_contrib_tile = n_contrib;
   {
     StageScope _t("render_fwd", stream);

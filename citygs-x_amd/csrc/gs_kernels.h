@@ -150,6 +150,8 @@ struct RenderFwdArgs {
   int* out_observe;
   float *out_all_map, *out_plane_depth;
   int *n_render, *n_consider, *n_contrib_tile;
+  const float* depths = nullptr;            // only read when out_max_weight_depth is given
+  float* out_max_weight_depth = nullptr;    // optional (H*W)
 };
 int launch_render_fwd(const RenderFwdArgs& a, hipStream_t stream);
 

@@ -31,7 +31,10 @@ namespace {
 constexpr int BATCH = GS_TILE_PIX;
 constexpr int CHUNKS = BATCH / 32;  // 32-bit list words per row and batch
 
-template <bool RENDER_GEO>
+// MAX_DEPTH adds one output with no counterpart in the reference: per pixel, the view-space depth of the Gaussian
+// that blends with the largest weight alpha * T (the front-most one among equals; 0 where nothing blends).  It
+// leaves every other output as it is.
+template <bool RENDER_GEO, bool MAX_DEPTH>
 __global__ void __launch_bounds__(GS_TILE_PIX)
 render_fwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__ point_list, int W, int H, float fx,
                   float fy, float cx, float cy, const float2* __restrict__ means2D, const float* __restrict__ rgb,
@@ -41,8 +44,10 @@ render_fwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
                   uint32_t* __restrict__ n_contrib2loss_px, float* __restrict__ out_color,
                   int* __restrict__ out_observe, float* __restrict__ out_all_map,
                   float* __restrict__ out_plane_depth, int* __restrict__ n_render, int* __restrict__ n_consider,
-                  int* __restrict__ n_contrib_tile) {
+                  int* __restrict__ n_contrib_tile, const float* __restrict__ depths,
+                  float* __restrict__ out_max_weight_depth) {
   constexpr bool render_geo = RENDER_GEO;
+  __shared__ float s_depth[MAX_DEPTH ? BATCH : 1];
   __shared__ int s_id[BATCH];
   __shared__ float2 s_xy[BATCH];
   __shared__ float4 s_co[BATCH];
@@ -83,6 +88,7 @@ render_fwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
   uint32_t last = 0, n2l = 0;
   float C[GS_N_RGB] = {0.f, 0.f, 0.f};
   float Mp[GS_N_MAP] = {0.f, 0.f, 0.f, 0.f, 0.f};
+  float best_w = 0.f, best_depth = 0.f;
 
   for (int i = 0; i < rounds; i++, todo -= BATCH) {
     const uint64_t alive_mask = __ballot(!done);
@@ -108,6 +114,7 @@ render_fwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
 #pragma unroll
         for (int ch = 0; ch < GS_N_MAP; ch++) s_map[ch][tid] = all_map[5 * (size_t)g + ch];
       }
+      if (MAX_DEPTH) s_depth[tid] = depths[g];
     }
     s_obs[tid] = 0;
     __syncthreads();
@@ -173,6 +180,11 @@ render_fwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
 #pragma unroll
             for (int ch = 0; ch < GS_N_MAP; ch++) Mp[ch] = __builtin_fmaf(s_map[ch][j], w, Mp[ch]);
           }
+          if (MAX_DEPTH) {
+            const bool better = w > best_w;  // w is 0 for a lane that does not blend
+            best_depth = better ? s_depth[j] : best_depth;
+            best_w = better ? w : best_w;
+          }
           const uint64_t omask = __ballot(blend && T > 0.5f);
           if (omask != 0ull) {
             const int cnt = __popc((uint32_t)(omask >> row_shift) & 0xFFFFu);
@@ -212,6 +224,7 @@ render_fwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
       const float den_f = (Mp[0] * rayx + Mp[1] * rayy) + Mp[2];
       out_plane_depth[pid] = (float)((double)Mp[4] / -((double)den_f + 1.0e-8));
     }
+    if (MAX_DEPTH) out_max_weight_depth[pid] = best_depth;
   }
 
   // per-tile integer sums of the two per-pixel counters
@@ -235,20 +248,25 @@ render_fwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
 
 }  // namespace
 
-int launch_render_fwd(const RenderFwdArgs& a, hipStream_t stream) {
+template <bool GEO, bool MAXD>
+static void launch_render_fwd_variant(const RenderFwdArgs& a, hipStream_t stream) {
   const dim3 grid((a.W + GS_TILE_X - 1) / GS_TILE_X, (a.H + GS_TILE_Y - 1) / GS_TILE_Y, 1);
-  if (a.render_geo)
-    hipLaunchKernelGGL(render_fwd_kernel<true>, grid, dim3(GS_TILE_PIX), 0, stream, (const uint2*)a.ranges,
-                       a.point_list, a.W, a.H, a.fx, a.fy, a.cx, a.cy, (const float2*)a.means2D, a.rgb, a.all_map,
-                       (const float4*)a.conic_opacity, a.compute_locally, a.bg, a.final_T, a.n_contrib_px,
-                       a.n_contrib2loss_px, a.out_color, a.out_observe, a.out_all_map, a.out_plane_depth, a.n_render,
-                       a.n_consider, a.n_contrib_tile);
-  else
-    hipLaunchKernelGGL(render_fwd_kernel<false>, grid, dim3(GS_TILE_PIX), 0, stream, (const uint2*)a.ranges,
-                       a.point_list, a.W, a.H, a.fx, a.fy, a.cx, a.cy, (const float2*)a.means2D, a.rgb, a.all_map,
-                       (const float4*)a.conic_opacity, a.compute_locally, a.bg, a.final_T, a.n_contrib_px,
-                       a.n_contrib2loss_px, a.out_color, a.out_observe, a.out_all_map, a.out_plane_depth, a.n_render,
-                       a.n_consider, a.n_contrib_tile);
+  hipLaunchKernelGGL((render_fwd_kernel<GEO, MAXD>), grid, dim3(GS_TILE_PIX), 0, stream, (const uint2*)a.ranges,
+                     a.point_list, a.W, a.H, a.fx, a.fy, a.cx, a.cy, (const float2*)a.means2D, a.rgb, a.all_map,
+                     (const float4*)a.conic_opacity, a.compute_locally, a.bg, a.final_T, a.n_contrib_px,
+                     a.n_contrib2loss_px, a.out_color, a.out_observe, a.out_all_map, a.out_plane_depth, a.n_render,
+                     a.n_consider, a.n_contrib_tile, a.depths, a.out_max_weight_depth);
+}
+
+int launch_render_fwd(const RenderFwdArgs& a, hipStream_t stream) {
+  const bool maxd = a.out_max_weight_depth != nullptr;
+  if (a.render_geo) {
+    if (maxd) launch_render_fwd_variant<true, true>(a, stream);
+    else launch_render_fwd_variant<true, false>(a, stream);
+  } else {
+    if (maxd) launch_render_fwd_variant<false, true>(a, stream);
+    else launch_render_fwd_variant<false, false>(a, stream);
+  }
   return 0;
 }
 

@@ -168,7 +168,9 @@ class _GrowBuffer:
 
 def render_gaussians(background, image_height, image_width, means2D, depths, radii, conic_opacity, rgb,
                      compute_locally, viewmatrix, campos, tan_fovx, tan_fovy, all_map, render_geo, debug, args):
-    """rasterize_points.cu:276-364."""
+    """rasterize_points.cu:276-364.  One addition: with args["max_weight_depth"] set, the per-pixel depth of the
+    Gaussian that blends with the largest weight (1, H, W) is left in args["stats_collector"]["max_weight_depth"];
+    the returned tuple is the reference's either way."""
     means2D = _f32c(means2D, "means2D")
     dev = means2D.device
     P = means2D.shape[0]
@@ -199,6 +201,8 @@ def render_gaussians(background, image_height, image_width, means2D, depths, rad
     if cl.dtype != torch.bool or cl.numel() != tiles:
         raise RuntimeError(f"compute_locally must be a bool tensor with {tiles} elements")
     am = _f32c(all_map, "all_map") if geo else None
+    want_mwd = isinstance(args, dict) and bool(args.get("max_weight_depth"))
+    mwd = torch.empty(1, H, W, **f32) if want_mwd else None
     # fp32 arithmetic, as `H / (2.0f * tan_fovy)` at rasterize_points.cu:328-329
     focal_y = np.float32(H) / (np.float32(2.0) * np.float32(tan_fovy))
     focal_x = np.float32(W) / (np.float32(2.0) * np.float32(tan_fovx))
@@ -210,10 +214,13 @@ def render_gaussians(background, image_height, image_width, means2D, depths, rad
             geom.callback, None, binning.callback, None, img.callback, None, P, _ptr(bg), W, H, float(focal_x),
             float(focal_y), float(W * 0.5), float(H * 0.5), _ptr(viewmatrix), _ptr(campos), _ptr(am), _ptr(means2D),
             _ptr(depths), _ptr(radii), _ptr(conic_opacity), _ptr(rgb), _ptr(cl), _ptr(out_color), _ptr(n_render),
-            _ptr(n_consider), _ptr(n_contrib), _ptr(out_observe), _ptr(out_all_map), _ptr(out_plane_depth), int(geo),
+            _ptr(n_consider), _ptr(n_contrib), _ptr(out_observe), _ptr(out_all_map), _ptr(out_plane_depth), _ptr(mwd),
+            int(geo),
             int(bool(debug)), C.byref(num_rendered), C.byref(elapsed) if timing else None, _stream(dev)),
             "render_gaussians")
     _record_time(args, "forward_render_time", elapsed.value)
+    if want_mwd:
+        args.setdefault("stats_collector", {})["max_weight_depth"] = mwd
     return (num_rendered.value, out_color, n_render, n_consider, n_contrib, out_observe, out_all_map, out_plane_depth,
             geom.release(), binning.release(), img.release())
 

@@ -32,7 +32,7 @@ _SIGNATURES = {
     "gs_preprocess_backward": (_i, [_vp] * 3 + [_i] * 5 + [_vp] * 4 + [_f] + [_vp] * 3 + [_f, _f] + [_vp, _i] +
                                [_vp] * 8 + [_i, _vp]),
     "gs_render_forward": (_i, [RESIZE_FN, _vp, RESIZE_FN, _vp, RESIZE_FN, _vp, _i, _vp, _i, _i, _f, _f, _f, _f] +
-                          [_vp] * 16 + [_i, _i, C.POINTER(_i), C.POINTER(_f), _vp]),
+                          [_vp] * 17 + [_i, _i, C.POINTER(_i), C.POINTER(_f), _vp]),
     "gs_render_backward_workspace_bytes": (_sz, [_i]),
     "gs_render_backward": (_i, [_i, _i, _vp, _i, _i, _f, _f] + [_vp] * 17 + [_i, _i, _vp, _sz, C.POINTER(_f), _vp]),
     "gs_ssim_l1_forward": (_i, [_i, _i, _i] + [_vp] * 9),

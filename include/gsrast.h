@@ -110,6 +110,9 @@ void gs_set_tile_sort_limits(int in_registers, int large_limit);
  * written only when render_geo != 0; out_observe (P) int32 must arrive zeroed;
  * n_render / n_consider / n_contrib are (tiles) int32, fully written.
  * *num_rendered (host) receives the instance count R.
+ * out_max_weight_depth (H*W, optional, NULL to skip) has no counterpart in the reference: per pixel the view-space
+ * depth (depths[g]) of the Gaussian that blends with the largest weight alpha * T, the front-most among equals, 0
+ * where nothing blends; asking for it changes no other output.
  * elapsed_ms (host, optional): if non-NULL the call times key emission + sort
  * + blend with events and blocks until done (the forward_render_time the
  * reference stores at CR/rasterizer_impl.cu:754-755). */
@@ -120,8 +123,8 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
                       const float* means2D, const float* depths, const int* radii, const float* conic_opacity,
                       const float* rgb, const uint8_t* compute_locally, float* out_color, int* n_render,
                       int* n_consider, int* n_contrib, int* out_observe, float* out_all_map,
-                      float* out_plane_depth, int render_geo, int debug, int* num_rendered, float* elapsed_ms,
-                      gs_stream_t stream);
+                      float* out_plane_depth, float* out_max_weight_depth, int render_geo, int debug,
+                      int* num_rendered, float* elapsed_ms, gs_stream_t stream);
 
 /* Replaces Rasterizer::renderBackward (CR/rasterizer.h:162-187,
  * CR/rasterizer_impl.cu:850-932) plus the repacking of

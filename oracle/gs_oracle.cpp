@@ -592,6 +592,48 @@ void oracle_render_fwd(int W, int H, float tanx, float tany, const uint32_t* ran
   }
 }
 
+// No counterpart in the reference (an additional output of the blend, defined here): per pixel the view-space
+// depth of the Gaussian that blends with the largest weight alpha * T, the front-most among equal weights, 0 where
+// nothing blends.  Same walk, tests and arithmetic as oracle_render_fwd (CR/forward.cu:330-437).
+void oracle_max_weight_depth(int W, int H, const uint32_t* ranges, const uint32_t* point_list, const float* means2D,
+                             const float* conic_opacity, const float* depths, const uint8_t* compute_locally,
+                             float* out) {
+  uint32_t gx, gy;
+  grid_of(W, H, gx, gy);
+  const int T = (int)(gx * gy);
+#pragma omp parallel for schedule(dynamic, 1)
+  for (int tile = 0; tile < T; tile++) {
+    if (!compute_locally[tile]) continue;
+    const uint32_t r0 = ranges[2 * tile], r1 = ranges[2 * tile + 1];
+    const int tx0 = (tile % (int)gx) * TILE_X, ty0 = (tile / (int)gx) * TILE_Y;
+    for (int ly = 0; ly < TILE_Y; ly++)
+      for (int lx = 0; lx < TILE_X; lx++) {
+        const int px = tx0 + lx, py = ty0 + ly;
+        if (px >= W || py >= H) continue;
+        const float pfx = (float)px, pfy = (float)py;
+        float Tr = 1.0f, best_w = 0.0f, best_d = 0.0f;
+        for (uint32_t k = r0; k < r1; k++) {
+          const uint32_t g = point_list[k];
+          const float dx = means2D[2 * g] - pfx, dy = means2D[2 * g + 1] - pfy;
+          const float* co = conic_opacity + 4 * (size_t)g;
+          const float power = -0.5f * (co[0] * dx * dx + co[2] * dy * dy) - co[1] * dx * dy;
+          if (power > 0.0f) continue;
+          const float alpha = fminf(0.99f, co[3] * orc_expf(power));
+          if (alpha < 1.0f / 255.0f) continue;
+          const float test_T = Tr * (1 - alpha);
+          if (test_T < 0.0001f) break;
+          const float wgt = alpha * Tr;
+          if (wgt > best_w) {
+            best_w = wgt;
+            best_d = depths[g];
+          }
+          Tr = test_T;
+        }
+        out[(size_t)W * py + px] = best_d;
+      }
+  }
+}
+
 // CR/rasterizer_impl.cu:219-262, launched :731-752.  Outputs arrive zeroed
 // (DGR/rasterize_points.cu:315-317); non-local tiles keep n_consider and
 // n_contrib at zero, n_render is written for every tile.

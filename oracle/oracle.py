@@ -224,6 +224,19 @@ def render_fwd(ranges, point_list, means2D, rgb, all_map, conic_opacity, compute
     return o
 
 
+def max_weight_depth(ranges, point_list, means2D, conic_opacity, depths, compute_locally, W, H):
+    """Per pixel the depth of the Gaussian that blends with the largest weight (no reference counterpart; defined
+    by oracle_max_weight_depth).  (1, H, W); pixels of tiles that are not computed locally stay 0."""
+    ranges = np.ascontiguousarray(ranges, np.uint32)
+    point_list = np.ascontiguousarray(point_list, np.uint32)
+    means2D, conic_opacity, depths = _f32(means2D), _f32(conic_opacity), _f32(depths)
+    cl = _u8(compute_locally).ravel()
+    out = np.zeros((1, H, W), np.float32)
+    lib().oracle_max_weight_depth(C.c_int(W), C.c_int(H), _p(ranges), _p(point_list), _p(means2D), _p(conic_opacity),
+                                  _p(depths), _p(cl), _p(out))
+    return out
+
+
 def render_bwd(ranges, point_list, means2D, conic_opacity, rgb, all_map, all_map_pixels, final_T, n_contrib,
                compute_locally, bg, dL_dpix, dL_dout_all_map, dL_dout_plane_depth, W, H, tanx, tany, render_geo=True):
     ranges = np.ascontiguousarray(ranges, np.uint32)

@@ -199,3 +199,48 @@ def test_all_gaussians_behind_camera_renders_background():
     assert int(n_render.sum()) == 0
     assert torch.allclose(color[:, 0, 0].cpu(), torch.tensor([0.25, 0.5, 0.75]))
     assert float((color - color[:, :1, :1]).abs().max()) == 0.0
+
+
+@pytest.mark.parametrize("cfg,P,mask,geo", [(0, 40_000, False, True), (1, 100_000, True, True), (0, 20_000, False, False)])
+def test_max_weight_depth_matches_oracle_and_changes_nothing_else(orc, cfg, P, mask, geo):
+    """The additional per-pixel output (depth of the Gaussian with the largest blending weight) equals the oracle's
+    bit for bit, and asking for it leaves every other output of render_gaussians as it is."""
+    import gpu_harness as H
+    import gs_scenes
+    from diff_gaussian_rasterization import _C
+    g, cams = gs_scenes.make_scene(cfg, P=P, n_views=1)
+    cam = cams[0]
+    W, Hh = cam.image_width, cam.image_height
+    gx, gy = H.grid(W, Hh)
+    cl = torch.ones(gy, gx, dtype=torch.bool)
+    if mask:
+        cl[::2, 1::3] = False
+    o, gd = H.preprocess_fwd(g, cam)
+    vm, cp = cam.world_view_transform.to(DEV), cam.camera_center.to(DEV)
+    am = gs_scenes.build_all_map(gd["means3D"], gd["scales"], gd["rotations"], cam)
+
+    def run(args):
+        return _C.render_gaussians(torch.zeros(3, device=DEV), Hh, W, o["means2D"], o["depths"], o["radii"],
+                                   o["conic_opacity"], o["rgb"], cl.to(DEV), vm, cp, cam.tanfovx, cam.tanfovy, am,
+                                   geo, False, args)
+
+    plain_args = {"stats_collector": {}}
+    plain = run(plain_args)
+    assert "max_weight_depth" not in plain_args["stats_collector"]
+    args = {"stats_collector": {}, "max_weight_depth": True}
+    out = run(args)
+    got = args["stats_collector"]["max_weight_depth"]
+    assert got.shape == (1, Hh, W)
+    px = cl.repeat_interleave(16, 0).repeat_interleave(16, 1)[:Hh, :W].to(DEV)
+    for a, b in zip(plain[1:8], out[1:8]):
+        if a.dim() == 3:
+            assert torch.equal(a[:, px], b[:, px])
+        else:
+            assert torch.equal(a, b)
+    n = lambda t: t.detach().cpu().numpy()
+    bins = orc.bin_and_sort(n(o["radii"]), n(o["means2D"]), n(o["depths"]), cl.numpy().reshape(-1), W, Hh)
+    want = orc.max_weight_depth(bins["ranges"], bins["point_list"], n(o["means2D"]), n(o["conic_opacity"]),
+                                n(o["depths"]), cl.numpy().reshape(-1), W, Hh)
+    pxn = n(px)
+    assert np.array_equal(n(got)[0][pxn], want[0][pxn])
+    assert float(got[0][px].max()) > 0

@@ -721,3 +721,94 @@ def test_neural_gaussians_backward_matches_float64_autograd(orc, N, k, seed):
     for i, (g, w) in enumerate(zip(got[4], flat)):
         assert g.shape == tuple(w.shape)
         assert _rel(g, w.grad.numpy()) < 1e-5, i
+
+
+# ------------------------------------------------------ max-weight depth --
+
+def test_max_weight_depth_known_cases(orc):
+    """Closed cases: one Gaussian (its depth wherever it blends, 0 elsewhere); a faint near one in front of a strong
+    far one (the far one wins where alpha_far (1 - alpha_near) > alpha_near); equal weights (the front one wins)."""
+    W, H = 48, 32
+    gx, gy = orc.tile_grid(W, H)
+    cl = np.ones(gx * gy, bool)
+    # one Gaussian
+    m1 = np.array([[20.25, 11.5]], np.float32)
+    co1 = np.array([[0.05, 0.01, 0.08, 0.8]], np.float32)
+    b = orc.bin_and_sort(np.array([200], np.int32), m1, np.array([5.0], np.float32), cl, W, H)
+    d = orc.max_weight_depth(b["ranges"], b["point_list"], m1, co1, np.array([5.0], np.float32), cl, W, H)[0]
+    ys, xs = np.mgrid[0:H, 0:W].astype(np.float64)
+    dx, dy = 20.25 - xs, 11.5 - ys
+    alpha = 0.8 * np.exp(-0.5 * (0.05 * dx * dx + 0.08 * dy * dy) - 0.01 * dx * dy)
+    sure = np.abs(alpha - 1 / 255) > 1e-6
+    assert np.array_equal(d[sure], np.where(alpha >= 1 / 255, 5.0, 0.0).astype(np.float32)[sure])
+    # near faint (depth 2, opacity 0.2), far strong (depth 9, opacity 0.9), both flat over the image
+    m2 = np.array([[24.0, 16.0], [24.0, 16.0]], np.float32)
+    flat = lambda o: [1e-7, 0.0, 1e-7, o]
+    co2 = np.array([flat(0.2), flat(0.9)], np.float32)
+    dep2 = np.array([2.0, 9.0], np.float32)
+    b = orc.bin_and_sort(np.array([200, 200], np.int32), m2, dep2, cl, W, H)
+    assert b["point_list"][:2].tolist() == [0, 1]
+    d = orc.max_weight_depth(b["ranges"], b["point_list"], m2, co2, dep2, cl, W, H)[0]
+    assert (d == 9.0).all()  # 0.9 * 0.8 = 0.72 > 0.2
+    co2[0, 3] = 0.6  # now 0.9 * 0.4 = 0.36 < 0.6: the near one wins
+    d = orc.max_weight_depth(b["ranges"], b["point_list"], m2, co2, dep2, cl, W, H)[0]
+    assert (d == 2.0).all()
+    co2[0, 3], co2[1, 3] = 0.5, 0.99  # weights 0.5 and 0.99 * 0.5 = 0.495 -> near; with alpha clamp 0.99
+    d = orc.max_weight_depth(b["ranges"], b["point_list"], m2, co2, dep2, cl, W, H)[0]
+    assert (d == 2.0).all()
+    # exactly equal weights: alpha 0.5 then alpha 1.0 -> clamped to 0.99 ... use 0.5 and 0.5/(1-0.5) is not
+    # representable below the clamp, so take three Gaussians 0.5, 0.5, 0.5: weights 0.5, 0.25, 0.125 -> front
+    m3 = np.tile(m2[:1], (3, 1))
+    co3 = np.array([flat(0.5)] * 3, np.float32)
+    dep3 = np.array([3.0, 4.0, 5.0], np.float32)
+    b = orc.bin_and_sort(np.full(3, 200, np.int32), m3, dep3, cl, W, H)
+    d = orc.max_weight_depth(b["ranges"], b["point_list"], m3, co3, dep3, cl, W, H)[0]
+    assert (d == 3.0).all()
+
+
+def test_max_weight_depth_against_float64_weights(orc):
+    """A random scene: the winner is the contributor whose float64 weight is largest (pixels where the two largest
+    weights are within 1e-5 of each other are left out), and pixels of masked tiles stay 0."""
+    g, cams = gs_scenes.make_scene(0, P=20000, n_views=1)
+    cam = cams[0]
+    W, H = cam.image_width, cam.image_height
+    pre = _pre(orc, g, cam)
+    gx, gy = orc.tile_grid(W, H)
+    cl = np.ones(gx * gy, bool)
+    cl[::3] = False
+    b = orc.bin_and_sort(pre["radii"], pre["means2D"], pre["depths"], cl, W, H)
+    got = orc.max_weight_depth(b["ranges"], b["point_list"], pre["means2D"], pre["conic_opacity"], pre["depths"], cl, W,
+                               H)[0]
+    ranges = b["ranges"].reshape(-1, 2)
+    checked = 0
+    rng = np.random.default_rng(0)
+    for tile in rng.choice(gx * gy, 60, replace=False):
+        ty, tx = divmod(int(tile), gx)
+        ys, xs = np.mgrid[ty * 16:min(ty * 16 + 16, H), tx * 16:min(tx * 16 + 16, W)]
+        if not cl[tile]:
+            assert (got[ys, xs] == 0).all()
+            continue
+        ids = b["point_list"][ranges[tile, 0]:ranges[tile, 1]]
+        if len(ids) == 0:
+            assert (got[ys, xs] == 0).all()
+            continue
+        mu = pre["means2D"][ids].astype(np.float64)
+        co = pre["conic_opacity"][ids].astype(np.float64)
+        dx = mu[:, 0, None, None] - xs[None]
+        dy = mu[:, 1, None, None] - ys[None]
+        power = -0.5 * (co[:, 0, None, None] * dx * dx + co[:, 2, None, None] * dy * dy) - co[:, 1, None, None] * dx * dy
+        alpha = np.minimum(0.99, co[:, 3, None, None] * np.exp(power))
+        alpha[(power > 0) | (alpha < 1 / 255)] = 0
+        Tr = np.cumprod(1 - alpha, axis=0)
+        T_before = np.concatenate([np.ones_like(Tr[:1]), Tr[:-1]], axis=0)
+        w = alpha * T_before
+        w[Tr < 1e-4] = 0  # the Gaussian that would take T below 1e-4 and all after it do not blend
+        order = np.sort(w, axis=0)
+        clear = ((order[-1] - (order[-2] if len(ids) > 1 else 0)) > 1e-5) | (order[-1] == 0)
+        near_stop = np.any(np.abs(Tr - 1e-4) < 1e-7, axis=0) | np.any(np.abs(alpha - 1 / 255) < 1e-7, axis=0)
+        ok = clear & ~near_stop
+        win = np.argmax(w, axis=0)
+        want = np.where(order[-1] > 0, pre["depths"][ids][win], 0.0).astype(np.float32)
+        assert np.array_equal(got[ys, xs][ok], want[ok])
+        checked += int(ok.sum())
+    assert checked > 5000
