@@ -684,6 +684,15 @@ int gs_training_stats(int64_t num_anchors, int n_offsets, int64_t num_candidates
   return check_launch("training_stats", (hipStream_t)stream, false);
 }
 
+int gs_max_radii_update(int64_t n, const int* radii, const uint8_t* visibility_filter, float* max_radii2D,
+                        gs_stream_t stream) {
+  GS_REQUIRE(n >= 0, "gs_max_radii_update: negative n");
+  if (n == 0) return 0;
+  GS_REQUIRE(radii && visibility_filter && max_radii2D, "gs_max_radii_update: null pointer");
+  launch_max_radii(n, radii, visibility_filter, max_radii2D, (hipStream_t)stream);
+  return check_launch("max_radii_update", (hipStream_t)stream, false);
+}
+
 int gs_adam_step(int count, float* const* params, const float* const* grads, float* const* exp_avg,
                  float* const* exp_avg_sq, const long long* sizes, const double* lrs, const int* steps, double beta1,
                  double beta2, double eps, float grad_scale, gs_stream_t stream) {

@@ -87,6 +87,7 @@ int launch_train_stats(long long A, int k, long long Vk, long long M, const uint
                        const uint8_t* selected, const uint8_t* update_filter, const float* grad, int grad_stride,
                        const float* opacity, float* opacity_accum, float* anchor_demon, float* grad_accum,
                        float* denom, void* temp, hipStream_t stream);
+int launch_max_radii(long long n, const int* radii, const uint8_t* visible, float* max_radii, hipStream_t stream);
 constexpr int ADAM_MAX_TENSORS = 24;  // tensors per launch (more are split over several launches)
 int launch_adam(int count, float* const* params, const float* const* grads, float* const* exp_avg,
                 float* const* exp_avg_sq, const long long* sizes, const double* lrs, const int* steps, double beta1,

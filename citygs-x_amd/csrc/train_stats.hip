@@ -104,6 +104,24 @@ size_t train_stats_temp_bytes(long long A, long long Vk) {
          align_up(scan_temp_bytes(A > Vk ? A : Vk), 256);
 }
 
+// gaussians.max_radii2D[visibility_filter] = max(gaussians.max_radii2D[visibility_filter], radii[visibility_filter])
+// (densification.py:71-73, add_densification_stats' companion in the Gaussian-splatting training loop).
+namespace {
+__global__ void __launch_bounds__(GS_BLOCK_1D)
+max_radii_kernel(long long n, const int* __restrict__ radii, const uint8_t* __restrict__ visible,
+                 float* __restrict__ max_radii) {
+  const long long i = (long long)blockIdx.x * GS_BLOCK_1D + threadIdx.x;
+  if (i < n && visible[i]) max_radii[i] = fmaxf(max_radii[i], (float)radii[i]);
+}
+}  // namespace
+
+int launch_max_radii(long long n, const int* radii, const uint8_t* visible, float* max_radii, hipStream_t stream) {
+  if (n <= 0) return 0;
+  hipLaunchKernelGGL(max_radii_kernel, dim3((unsigned)((n + GS_BLOCK_1D - 1) / GS_BLOCK_1D)), dim3(GS_BLOCK_1D), 0,
+                     stream, n, radii, visible, max_radii);
+  return 0;
+}
+
 int launch_train_stats(long long A, int k, long long Vk, long long M, const uint8_t* visible,
                        const uint8_t* selected, const uint8_t* update_filter, const float* grad, int grad_stride,
                        const float* opacity, float* opacity_accum, float* anchor_demon, float* grad_accum,

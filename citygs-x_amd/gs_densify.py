@@ -62,3 +62,21 @@ def training_statis(opacity_accum, anchor_demon, offset_gradient_accum, offset_d
                                       p(opacity_accum), p(anchor_demon), p(offset_gradient_accum), p(offset_denom),
                                       C.c_void_p(ws.data_ptr()), nb,
                                       C.c_void_p(torch.cuda.current_stream(dev).cuda_stream)), "training_statis")
+
+
+@torch.no_grad()
+def update_max_radii(max_radii2D, radii, visibility_filter):
+    """max_radii2D[visibility_filter] = max(max_radii2D[visibility_filter], radii[visibility_filter]) in place
+    (densification.py:71-73), one launch."""
+    _f32(max_radii2D, "max_radii2D")
+    n = max_radii2D.numel()
+    if radii.dtype != torch.int32 or not radii.is_cuda or radii.numel() != n:
+        raise RuntimeError("radii must be an int32 GPU tensor with one entry per Gaussian")
+    vis = _u8(visibility_filter, "visibility_filter")
+    if vis.numel() != n:
+        raise RuntimeError("visibility_filter must have one entry per Gaussian")
+    dev = max_radii2D.device
+    _n.check(_n.lib.gs_max_radii_update(n, C.c_void_p(radii.contiguous().data_ptr()), C.c_void_p(vis.data_ptr()),
+                                        C.c_void_p(max_radii2D.data_ptr()),
+                                        C.c_void_p(torch.cuda.current_stream(dev).cuda_stream)), "update_max_radii")
+    return max_radii2D

@@ -248,6 +248,12 @@ int gs_training_stats(int64_t num_anchors, int n_offsets, int64_t num_candidates
                       float* offset_gradient_accum, float* offset_denom, void* workspace, size_t workspace_bytes,
                       gs_stream_t stream);
 
+/* Replaces `gaussians.max_radii2D[visibility_filter] = torch.max(gaussians.max_radii2D[visibility_filter],
+ * radii[visibility_filter])` (densification.py:71-73): the running maximum of the screen-space radius of every
+ * Gaussian, over the views that saw it.  radii int32[n], visibility_filter u8[n] (0/1), max_radii2D float[n]. */
+int gs_max_radii_update(int64_t n, const int* radii, const uint8_t* visibility_filter, float* max_radii2D,
+                        gs_stream_t stream);
+
 /* Replaces optimizer.step() of the reference's torch.optim.Adam(lr=0.0, eps=1e-15) with per-group learning
  * rates (scene/gaussian_model.py:574, stepped at train_internal.py:404-417) for `count` tensors in one
  * launch: update rule of torch 2.0.0 with betas (beta1, beta2), no weight decay, no amsgrad.

@@ -85,3 +85,17 @@ def test_training_stats_rejects_inconsistent_inputs():
         gs_densify.training_statis(torch.zeros(4, 1), torch.zeros(4, 1), torch.zeros(8, 1), torch.zeros(8, 1), 2,
                                    torch.zeros(0, 3), torch.zeros(0, 1), torch.zeros(0, dtype=torch.bool),
                                    torch.zeros(0, dtype=torch.bool), torch.zeros(4, dtype=torch.bool))
+
+
+def test_update_max_radii_matches_torch_statement():
+    import gs_densify
+    gen = torch.Generator().manual_seed(3)
+    n = 100_003
+    m = torch.rand(n, generator=gen) * 40
+    radii = torch.randint(0, 80, (n,), generator=gen, dtype=torch.int32)
+    vis = torch.rand(n, generator=gen) < 0.4
+    want = m.clone()
+    want[vis] = torch.max(want[vis], radii[vis].float())
+    got = gs_densify.update_max_radii(m.to(DEV), radii.to(DEV), vis.to(DEV)).cpu()
+    assert torch.equal(got, want)
+    assert torch.equal(got[~vis], m[~vis])
