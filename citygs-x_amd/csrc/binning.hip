@@ -52,17 +52,18 @@ tile_count_kernel(int P, uint32_t gx, uint32_t gy, const int* __restrict__ radii
   const int i = blockIdx.x * GS_BLOCK_1D + threadIdx.x;
   // optionally clears another array on the side (the tile ranges of the same call: saves a launch)
   for (int64_t j = i; j < zero_count; j += (int64_t)gridDim.x * GS_BLOCK_1D) zero_words[j] = 0u;
-  if (i >= P) return;
-  uint32_t cnt = 0;
-  const int r = radii[i];
-  if (r > 0) {
+  // (no early return: the walk below is a wave-wide operation)
+  const bool live = i < P && radii[i] > 0;
+  Rect rc = {0u, 0u, 0u, 0u};
+  if (live) {
     const float2 p = means2D[i];
-    const Rect rc = get_rect(p.x, p.y, r, gx, gy);
-    for (uint32_t y = rc.y0; y < rc.y1; y++)
-      for (uint32_t x = rc.x0; x < rc.x1; x++)
-        if (compute_locally[y * gx + x]) cnt++;
+    rc = get_rect(p.x, p.y, radii[i], gx, gy);
   }
-  tiles_touched[i] = cnt;
+  struct None { uint32_t unused; } none = {0u};
+  const uint32_t cnt = walk_wave_rects(
+      live, rc, gx, none, [&](uint32_t tile) { return compute_locally[tile] != 0; },
+      [](const None&, uint32_t, uint32_t) {});
+  if (i < P) tiles_touched[i] = cnt;
 }
 
 template <typename T>
@@ -142,23 +143,23 @@ duplicate_with_keys_kernel(int P, uint32_t gx, uint32_t gy, const float2* __rest
                            uint64_t* __restrict__ keys, uint32_t* __restrict__ values,
                            uint32_t* __restrict__ emission) {
   const int i = blockIdx.x * GS_BLOCK_1D + threadIdx.x;
-  if (i >= P) return;
-  const int r = radii[i];
-  if (r > 0) {
-    uint32_t off = (i == 0) ? 0u : offsets[i - 1];
+  const bool live = i < P && radii[i] > 0;
+  Rect rc = {0u, 0u, 0u, 0u};
+  struct Owner { uint32_t first, depth_bits, id; } mine = {0u, 0u, (uint32_t)i};
+  if (live) {
+    mine.first = (i == 0) ? 0u : offsets[i - 1];
     const float2 p = means2D[i];
-    const Rect rc = get_rect(p.x, p.y, r, gx, gy);
-    const uint32_t dbits = __float_as_uint(depths[i]);
-    for (uint32_t y = rc.y0; y < rc.y1; y++)
-      for (uint32_t x = rc.x0; x < rc.x1; x++)
-        if (compute_locally[y * gx + x]) {
-          const uint64_t key = ((uint64_t)(y * gx + x) << 32) | (uint64_t)dbits;
-          keys[off] = key;
-          values[off] = (uint32_t)i;
-          if (emission) emission[off] = off;  // position in emission order, carried through the sort
-          off++;
-        }
+    rc = get_rect(p.x, p.y, radii[i], gx, gy);
+    mine.depth_bits = __float_as_uint(depths[i]);
   }
+  walk_wave_rects(
+      live, rc, gx, mine, [&](uint32_t tile) { return compute_locally[tile] != 0; },
+      [&](const Owner& o, uint32_t tile, uint32_t rank) {
+        const uint32_t e = o.first + rank;
+        keys[e] = ((uint64_t)tile << 32) | (uint64_t)o.depth_bits;
+        values[e] = o.id;
+        if (emission) emission[e] = e;  // position in emission order, carried through the sort
+      });
 }
 
 // point_list[k] = Gaussian of the instance that the sort moved to position k.

@@ -177,4 +177,60 @@ __device__ __forceinline__ Rect get_rect(float px, float py, int radius, uint32_
   return r;
 }
 
+// Walks the tile rectangles of a wave's 64 Gaussians (one per lane; `live` = the lane has one) and calls
+// visit(payload_of_owner, tile, rank) for every tile of a rectangle that is computed locally, rank = number of
+// such tiles before it in the rectangle's row-major order (the order duplicateWithKeys emits them,
+// cuda_rasterizer/rasterizer_impl.cu:95-112).  Returns, to the owner lane, its rectangle's count of local tiles.
+// A rectangle of more than GS_BIG_RECT tiles is walked by the whole wave, 64 tiles at a time, instead of by its
+// owner alone: a street-level view has Gaussians that cover thousands of tiles, and one lane looping over them
+// would hold up everybody.  `mine` is whatever visit needs of the owning Gaussian (a struct of 32-bit words); for a
+// big rectangle it is handed from the owner lane to all lanes while the wave is still convergent.  Every lane of
+// the wave must call this (it uses ballots and cross-lane reads).
+#define GS_BIG_RECT 16
+template <typename Payload, typename Mask, typename Visit>
+__device__ __forceinline__ uint32_t walk_wave_rects(bool live, const Rect& rc, uint32_t gx, const Payload& mine,
+                                                    Mask is_local, Visit visit) {
+  static_assert(sizeof(Payload) % 4 == 0, "payload of 32-bit words");
+  const int lane = threadIdx.x & (GS_WAVE - 1);
+  const uint32_t w = live ? rc.x1 - rc.x0 : 0u, h = live ? rc.y1 - rc.y0 : 0u;
+  const uint32_t area = w * h;
+  uint32_t count = 0;
+  uint64_t big = __ballot(area > GS_BIG_RECT);
+  while (big != 0ull) {
+    const int owner = (int)__builtin_ctzll(big);
+    big &= big - 1ull;
+    const uint32_t ox0 = __shfl(rc.x0, owner, GS_WAVE), oy0 = __shfl(rc.y0, owner, GS_WAVE);
+    const uint32_t ow = __shfl(w, owner, GS_WAVE), on = __shfl(area, owner, GS_WAVE);
+    Payload theirs;
+    {
+      const uint32_t* src = reinterpret_cast<const uint32_t*>(&mine);
+      uint32_t* dst = reinterpret_cast<uint32_t*>(&theirs);
+#pragma unroll
+      for (int k = 0; k < (int)(sizeof(Payload) / 4); k++) dst[k] = __shfl(src[k], owner, GS_WAVE);
+    }
+    uint32_t before = 0;
+    for (uint32_t q0 = 0; q0 < on; q0 += GS_WAVE) {
+      const uint32_t q = q0 + (uint32_t)lane;
+      const uint32_t ry = q / ow, rx = q - ry * ow;
+      const uint32_t tile = (oy0 + ry) * gx + (ox0 + rx);
+      const bool local = q < on && is_local(tile);
+      const uint64_t bits = __ballot(local);
+      if (local) visit(theirs, tile, before + (uint32_t)__popcll(bits & ((1ull << lane) - 1ull)));
+      before += (uint32_t)__popcll(bits);
+    }
+    if (lane == owner) count = before;
+  }
+  if (area != 0u && area <= GS_BIG_RECT) {
+    for (uint32_t y = rc.y0; y < rc.y1; y++)
+      for (uint32_t x = rc.x0; x < rc.x1; x++) {
+        const uint32_t tile = y * gx + x;
+        if (is_local(tile)) {
+          visit(mine, tile, count);
+          count++;
+        }
+      }
+  }
+  return count;
+}
+
 }  // namespace gs

@@ -46,31 +46,27 @@ bucket_count_kernel(int P, int per_block, uint32_t gx, uint32_t gy, const int* _
   __syncthreads();
   const int first = blockIdx.x * per_block;
   const int last = first + per_block < P ? first + per_block : P;
-  // four Gaussians per round: their loads go out together, then each is walked
-  for (int i0 = first + threadIdx.x; i0 < last; i0 += BK_BATCH * BK_THREADS) {
+  // four Gaussians per round: their loads go out together, then each is walked (the loop bounds are the same
+  // for every thread of the workgroup, because the walk is a wave-wide operation)
+  struct None { uint32_t unused; } none = {0u};
+  for (int base = first; base < last; base += BK_BATCH * BK_THREADS) {
     int r[BK_BATCH];
     float2 p[BK_BATCH];
 #pragma unroll
     for (int q = 0; q < BK_BATCH; q++) {
-      const int i = i0 + q * BK_THREADS;
+      const int i = base + (int)threadIdx.x + q * BK_THREADS;
       r[q] = i < last ? radii[i] : 0;
       p[q] = i < last ? means2D[i] : make_float2(0.0f, 0.0f);
     }
 #pragma unroll
     for (int q = 0; q < BK_BATCH; q++) {
-      const int i = i0 + q * BK_THREADS;
-      if (i >= last) break;
-      uint32_t cnt = 0;
-      if (r[q] > 0) {
-        const Rect rc = get_rect(p[q].x, p[q].y, r[q], gx, gy);
-        for (uint32_t y = rc.y0; y < rc.y1; y++)
-          for (uint32_t x = rc.x0; x < rc.x1; x++)
-            if (s_local[y * gx + x]) {
-              atomicAdd(&s_hist[y * gx + x], 1u);
-              cnt++;
-            }
-      }
-      tiles_touched[i] = cnt;
+      const int i = base + (int)threadIdx.x + q * BK_THREADS;
+      const bool live = i < last && r[q] > 0;
+      const Rect rc = live ? get_rect(p[q].x, p[q].y, r[q], gx, gy) : Rect{0u, 0u, 0u, 0u};
+      const uint32_t cnt = walk_wave_rects(
+          live, rc, gx, none, [&](uint32_t tile) { return s_local[tile] != 0; },
+          [&](const None&, uint32_t tile, uint32_t) { atomicAdd(&s_hist[tile], 1u); });
+      if (i < last) tiles_touched[i] = cnt;
     }
   }
   __syncthreads();
@@ -192,13 +188,14 @@ bucket_scatter_kernel(int P, int per_block, uint32_t gx, uint32_t gy, const floa
   __syncthreads();
   const int first = blockIdx.x * per_block;
   const int last = first + per_block < P ? first + per_block : P;
-  for (int i0 = first + threadIdx.x; i0 < last; i0 += BK_BATCH * BK_THREADS) {
+  struct Owner { uint32_t first, depth_bits, id; };
+  for (int base = first; base < last; base += BK_BATCH * BK_THREADS) {
     int r[BK_BATCH];
     float2 p[BK_BATCH];
     uint32_t e0[BK_BATCH], dbits[BK_BATCH];
 #pragma unroll
     for (int q = 0; q < BK_BATCH; q++) {
-      const int i = i0 + q * BK_THREADS;
+      const int i = base + (int)threadIdx.x + q * BK_THREADS;
       r[q] = i < last ? radii[i] : 0;
       p[q] = i < last ? means2D[i] : make_float2(0.0f, 0.0f);
       dbits[q] = i < last ? __float_as_uint(depths[i]) : 0u;
@@ -206,19 +203,18 @@ bucket_scatter_kernel(int P, int per_block, uint32_t gx, uint32_t gy, const floa
     }
 #pragma unroll
     for (int q = 0; q < BK_BATCH; q++) {
-      const int i = i0 + q * BK_THREADS;
-      if (i >= last || r[q] <= 0) continue;
-      uint32_t e = e0[q];
-      const Rect rc = get_rect(p[q].x, p[q].y, r[q], gx, gy);
-      const uint64_t hi = (uint64_t)dbits[q] << 32;
-      for (uint32_t y = rc.y0; y < rc.y1; y++)
-        for (uint32_t x = rc.x0; x < rc.x1; x++)
-          if (s_local[y * gx + x]) {
-            const uint32_t pos = atomicAdd(&s_next[y * gx + x], 1u);
-            records[pos] = hi | (uint64_t)e;
-            gauss_of_emission[e] = (uint32_t)i;
-            e++;
-          }
+      const int i = base + (int)threadIdx.x + q * BK_THREADS;
+      const bool live = i < last && r[q] > 0;
+      const Rect rc = live ? get_rect(p[q].x, p[q].y, r[q], gx, gy) : Rect{0u, 0u, 0u, 0u};
+      const Owner mine = {e0[q], dbits[q], (uint32_t)i};
+      walk_wave_rects(
+          live, rc, gx, mine, [&](uint32_t tile) { return s_local[tile] != 0; },
+          [&](const Owner& o, uint32_t tile, uint32_t rank) {
+            const uint32_t e = o.first + rank;
+            const uint32_t pos = atomicAdd(&s_next[tile], 1u);
+            records[pos] = ((uint64_t)o.depth_bits << 32) | (uint64_t)e;
+            gauss_of_emission[e] = o.id;
+          });
     }
   }
 }
