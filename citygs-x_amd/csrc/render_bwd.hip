@@ -296,16 +296,45 @@ reduce_instances_kernel(int P, const uint32_t* __restrict__ point_offsets, const
                         float4* __restrict__ dL_dconic_opacity, float* __restrict__ dL_dcolors,
                         float* __restrict__ dL_dall_map) {
   const int i = blockIdx.x * GS_BLOCK_1D + threadIdx.x;
-  if (i >= P) return;
-  const uint32_t b = i == 0 ? 0u : point_offsets[i - 1], e = point_offsets[i];
+  const int lane = threadIdx.x & (GS_WAVE - 1);
+  const bool live = i < P;
+  const uint32_t b = (!live || i == 0) ? 0u : point_offsets[i - 1], e = live ? point_offsets[i] : 0u;
+  const uint32_t n = e - b;
   float4 a0 = make_float4(0.f, 0.f, 0.f, 0.f), a1 = a0, a2 = a0, a3 = a0;
-  for (uint32_t k = b; k < e; k++) {
-    const float4* rec = instance_grads + 4 * (size_t)k;
-    const float4 r0 = rec[0], r1 = rec[1], r2 = rec[2], r3 = rec[3];
-    a0.x += r0.x; a0.y += r0.y; a0.z += r0.z; a0.w += r0.w;
-    a1.x += r1.x; a1.y += r1.y; a1.z += r1.z; a1.w += r1.w;
-    a2.x += r2.x; a2.y += r2.y; a2.z += r2.z; a2.w += r2.w;
-    a3.x += r3.x; a3.y += r3.y; a3.z += r3.z; a3.w += r3.w;
+  auto add = [](float4& a, const float4& r) { a.x += r.x; a.y += r.y; a.z += r.z; a.w += r.w; };
+  // A Gaussian with many instances (in a street-level view one can cover thousands of tiles) is summed by the
+  // whole wave: lane l takes records l, l + 64, ..., then the 64 partial sums are added across the lanes in a fixed
+  // order.  Everything else is summed by its own thread, record after record.
+  constexpr uint32_t MANY = 32;
+  uint64_t many = __ballot(n > MANY);
+  while (many != 0ull) {
+    const int owner = (int)__builtin_ctzll(many);
+    many &= many - 1ull;
+    const uint32_t ob = __shfl(b, owner, GS_WAVE), on = __shfl(n, owner, GS_WAVE);
+    float4 p0 = make_float4(0.f, 0.f, 0.f, 0.f), p1 = p0, p2 = p0, p3 = p0;
+    for (uint32_t k = (uint32_t)lane; k < on; k += GS_WAVE) {
+      const float4* rec = instance_grads + 4 * (size_t)(ob + k);
+      add(p0, rec[0]); add(p1, rec[1]); add(p2, rec[2]); add(p3, rec[3]);
+    }
+#pragma unroll
+    for (int d = GS_WAVE / 2; d >= 1; d >>= 1) {
+      float4* parts[4] = {&p0, &p1, &p2, &p3};
+#pragma unroll
+      for (int q = 0; q < 4; q++) {
+        parts[q]->x += __shfl_xor(parts[q]->x, d, GS_WAVE);
+        parts[q]->y += __shfl_xor(parts[q]->y, d, GS_WAVE);
+        parts[q]->z += __shfl_xor(parts[q]->z, d, GS_WAVE);
+        parts[q]->w += __shfl_xor(parts[q]->w, d, GS_WAVE);
+      }
+    }
+    if (lane == owner) { a0 = p0; a1 = p1; a2 = p2; a3 = p3; }
+  }
+  if (!live) return;
+  if (n <= MANY) {
+    for (uint32_t k = b; k < e; k++) {
+      const float4* rec = instance_grads + 4 * (size_t)k;
+      add(a0, rec[0]); add(a1, rec[1]); add(a2, rec[2]); add(a3, rec[3]);
+    }
   }
   dL_dmean2D[i] = make_float2(a0.x, a0.y);
   dL_dmean2D_abs[3 * (size_t)i] = a0.z;
