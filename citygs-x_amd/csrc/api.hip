@@ -491,7 +491,9 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
   EventTimer timer;
   if (timer.begin(elapsed_ms != nullptr, stream)) return 1;
 
-  if (bucketed && longest > (uint32_t)g_tile_sort_large.load()) bucketed = false;  // a list too long for the LDS sort
+  // a list too long for the per-tile sort: beyond 8192 records one tile's sort takes longer than the radix sort
+  // of the whole view
+  if (bucketed && longest > (uint32_t)g_tile_sort_large.load()) bucketed = false;
   if (bucketed) {
     if (R > 0) {
       {

@@ -219,16 +219,17 @@ bucket_scatter_kernel(int P, int per_block, uint32_t gx, uint32_t gy, const floa
   }
 }
 
-// 2. Per-tile sort, register variant: one workgroup of four waves per tile.  A wave holds 64 E records, record
-// i = r * 64 + lane in register r of its lane, and the four waves hold consecutive runs of 64 E, so a list of
-// up to 256 E records is sorted with E = 1 .. 32.  In the bitonic network a step pairs i with i ^ j:
+// 2. Per-tile sort, register variant: one workgroup of W waves per tile (4 for lists of up to 2048 records, 16
+// for longer ones).  A wave holds 64 E records, record i = r * 64 + lane in register r of its lane, and the waves
+// hold consecutive runs of 64 E, so a list of up to 64 E W records is sorted with E = 1 .. 8.  In the bitonic
+// network a step pairs i with i ^ j:
 //   j < 64        the partner sits in another lane, same register: one cross-lane read, keep the smaller or larger;
 //   64 <= j < 64E the partner sits in another register of the same lane: no data moves at all;
-//   j >= 64 E     the partner sits in another wave: one exchange through LDS (three such steps in a whole sort).
+//   j >= 64 E     the partner sits in another wave: one exchange through LDS (3 such steps in a whole sort with
+//                 4 waves, 10 with 16).
 // The direction of a step, ((i & k) == 0) ascending, and which of the pair an element keeps are computed from
 // the indices.  Short dependency chains matter more than instruction count here: every tile is resident at once,
-// so the kernel takes as long as its longest tile, and four waves with few records each finish it soonest.
-constexpr int RS_WAVES = 4;
+// so the kernel takes as long as its longest tile, and many waves with few records each finish it soonest.
 
 template <int E>
 __device__ __forceinline__ void exchange_step(uint64_t (&v)[E], const uint64_t (&other)[E], uint32_t row0,
@@ -244,9 +245,9 @@ __device__ __forceinline__ void exchange_step(uint64_t (&v)[E], const uint64_t (
   }
 }
 
-template <int E>
+template <int E, int W>
 __device__ __forceinline__ void register_sort(uint64_t (&v)[E], uint32_t wave, uint32_t lane, uint64_t* s_x) {
-  constexpr uint32_t M = 64u * E * RS_WAVES;
+  constexpr uint32_t M = 64u * E * W;
   const uint32_t row0 = wave * E;
   for (uint32_t k = 2; k <= M; k <<= 1) {
     for (uint32_t j = k >> 1; j > 0; j >>= 1) {
@@ -291,7 +292,7 @@ __device__ __forceinline__ void register_sort(uint64_t (&v)[E], uint32_t wave, u
   }
 }
 
-template <int E>
+template <int E, int W>
 __device__ __forceinline__ void register_sort_tile(uint32_t t, uint32_t start, uint32_t n,
                                                    const uint64_t* __restrict__ records,
                                                    const uint32_t* __restrict__ gauss_of_emission,
@@ -304,7 +305,7 @@ __device__ __forceinline__ void register_sort_tile(uint32_t t, uint32_t start, u
     const uint32_t i = ((wave * E + r) << 6) | lane;
     v[r] = i < n ? records[start + i] : ~0ull;
   }
-  register_sort<E>(v, wave, lane, s_x);
+  register_sort<E, W>(v, wave, lane, s_x);
   const uint64_t tile_bits = (uint64_t)t << 32;
 #pragma unroll
   for (int r = 0; r < E; r++) {
@@ -319,10 +320,10 @@ __device__ __forceinline__ void register_sort_tile(uint32_t t, uint32_t start, u
 }
 
 // Dynamic LDS: 8 bytes per record of the longest list the kernel takes, rounded up to a power of two (at least
-// 256 records).  Two kernels, so that the common one (lists of up to 2048 records) keeps a small register budget.
-#define GS_SORT_CASE(EE) \
-  register_sort_tile<EE>(t, start, n, records, gauss_of_emission, keys, emission, point_list, s_exchange)
-__global__ void __launch_bounds__(64 * RS_WAVES)
+// 256 records).
+#define GS_SORT_CASE(EE, WW) \
+  register_sort_tile<EE, WW>(t, start, n, records, gauss_of_emission, keys, emission, point_list, s_exchange)
+__global__ void __launch_bounds__(256)
 tile_sort_registers_kernel(const uint32_t* __restrict__ ranges, const uint64_t* __restrict__ records,
                            const uint32_t* __restrict__ gauss_of_emission, uint64_t* __restrict__ keys,
                            uint32_t* __restrict__ emission, uint32_t* __restrict__ point_list) {
@@ -331,13 +332,13 @@ tile_sort_registers_kernel(const uint32_t* __restrict__ ranges, const uint64_t* 
   const uint32_t start = ranges[2 * t];
   const uint32_t n = ranges[2 * t + 1] - start;
   if (n == 0 || n > 2048) return;
-  if (n <= 256) GS_SORT_CASE(1);
-  else if (n <= 512) GS_SORT_CASE(2);
-  else if (n <= 1024) GS_SORT_CASE(4);
-  else GS_SORT_CASE(8);
+  if (n <= 256) GS_SORT_CASE(1, 4);
+  else if (n <= 512) GS_SORT_CASE(2, 4);
+  else if (n <= 1024) GS_SORT_CASE(4, 4);
+  else GS_SORT_CASE(8, 4);
 }
 
-__global__ void __launch_bounds__(64 * RS_WAVES)
+__global__ void __launch_bounds__(1024)
 tile_sort_registers_long_kernel(const uint32_t* __restrict__ ranges, const uint64_t* __restrict__ records,
                                 const uint32_t* __restrict__ gauss_of_emission, uint64_t* __restrict__ keys,
                                 uint32_t* __restrict__ emission, uint32_t* __restrict__ point_list) {
@@ -346,9 +347,10 @@ tile_sort_registers_long_kernel(const uint32_t* __restrict__ ranges, const uint6
   const uint32_t start = ranges[2 * t];
   const uint32_t n = ranges[2 * t + 1] - start;
   if (n <= 2048) return;
-  if (n <= 4096) GS_SORT_CASE(16);
-  else GS_SORT_CASE(32);
+  if (n <= 4096) GS_SORT_CASE(4, 16);
+  else GS_SORT_CASE(8, 16);
 }
+
 #undef GS_SORT_CASE
 
 // 3. The same sort with the records in LDS (kept as the variant the tests can force): one workgroup per tile,
@@ -453,7 +455,8 @@ int launch_bucket_scatter(int P, int W, int H, const float* means2D, const float
 }
 
 // Sorts every tile's segment; `longest` is the longest list (nothing may exceed TILE_SORT_LARGE).  The register
-// variant by default; with in_registers == 0 the LDS variants (small up to TILE_SORT_SMALL, then large).
+// variant by default; with in_registers == 0 the LDS variants (small up to
+// TILE_SORT_SMALL, then large).
 int launch_tile_sort(int T, uint32_t longest, uint32_t in_registers, const uint32_t* ranges, const uint64_t* records,
                      const uint32_t* gauss_of_emission, uint64_t* keys, uint32_t* emission, uint32_t* point_list,
                      hipStream_t stream) {
@@ -469,10 +472,10 @@ int launch_tile_sort(int T, uint32_t longest, uint32_t in_registers, const uint3
   }
   uint32_t m = 256;
   while (m < longest && m < 2048) m <<= 1;
-  hipLaunchKernelGGL(tile_sort_registers_kernel, dim3(T), dim3(64 * RS_WAVES), (size_t)m * sizeof(uint64_t), stream,
-                     ranges, records, gauss_of_emission, keys, emission, point_list);
+  hipLaunchKernelGGL(tile_sort_registers_kernel, dim3(T), dim3(256), (size_t)m * sizeof(uint64_t), stream, ranges,
+                     records, gauss_of_emission, keys, emission, point_list);
   if (longest > 2048)
-    hipLaunchKernelGGL(tile_sort_registers_long_kernel, dim3(T), dim3(64 * RS_WAVES),
+    hipLaunchKernelGGL(tile_sort_registers_long_kernel, dim3(T), dim3(1024),
                        (size_t)(longest > 4096 ? 8192 : 4096) * sizeof(uint64_t), stream, ranges, records,
                        gauss_of_emission, keys, emission, point_list);
   return 0;

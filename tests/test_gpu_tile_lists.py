@@ -139,8 +139,8 @@ def test_equal_depths_keep_emission_order(orc, H):
 
 @pytest.mark.parametrize("P,expect", [(28_000, "waves4"), (56_000, "waves8"), (110_000, "radix")])
 def test_long_lists(orc, H, P, expect):
-    """A small image under many large Gaussians: lists of several thousand records per tile (16 and 32 records
-    per lane in the register sort), and beyond 8192 the radix route, which then takes over by itself."""
+    """A small image under many large Gaussians: lists of several thousand records per tile (sixteen waves per
+    tile, 4 or 8 records per lane), and beyond 8192 the radix route, which then takes over by itself."""
     import gs_scenes
     import gsrast_native as gn
     from diff_gaussian_rasterization import _C
