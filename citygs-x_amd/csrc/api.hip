@@ -340,7 +340,8 @@ uint32_t* acquire_total_slot() {
     }
   }
   uint32_t* slot = base + 16 * (g_total_next.fetch_add(1, std::memory_order_relaxed) % TOTAL_SLOTS);
-  slot[1] = 0u;  // second word of the slot: the longest tile list, written before the total
+  slot[1] = 0u;  // second and third word of the slot: the longest tile list and the number of chunks that the
+  slot[2] = 0u;  // longer lists are sorted in, both written before the total
   __atomic_store_n(slot, TOTAL_PENDING, __ATOMIC_RELEASE);
   return slot;
 }
@@ -374,17 +375,21 @@ int wait_for_total(uint32_t* slot, hipStream_t stream, uint32_t* out) {
 }  // namespace
 
 namespace {
-// whether the per-tile sort keeps the records in registers (or in LDS), and the list length up to which any
-// per-tile sort is used
+// whether the per-tile sort keeps the records in registers (or in LDS), the list length up to which one
+// workgroup sorts a list whole (0: every view takes the radix sort), and the number of chunks up to which the
+// longer lists of a view are sorted in chunks and merged
 std::atomic<int> g_tile_sort_registers{1};
 std::atomic<int> g_tile_sort_large{TILE_SORT_LARGE};
+std::atomic<int> g_tile_sort_chunks{TILE_SORT_MAX_CHUNKS};
 }  // namespace
 
-void gs_set_tile_sort_limits(int in_registers, int large_limit) {
+void gs_set_tile_sort_limits(int in_registers, int large_limit, int max_chunks) {
   if (large_limit > TILE_SORT_LARGE) large_limit = TILE_SORT_LARGE;
   if (large_limit < 0) large_limit = 0;
+  if (max_chunks < 0) max_chunks = 0;
   g_tile_sort_registers.store(in_registers != 0 ? 1 : 0);
   g_tile_sort_large.store(large_limit);
+  g_tile_sort_chunks.store(max_chunks);
 }
 
 int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resize_fn binningBuffer,
@@ -434,14 +439,15 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
   // sort.  Otherwise: emit (tile | depth) keys, radix-sort all of them, find the tile boundaries.
   uint32_t* total_slot = acquire_total_slot();
   void* bucket_table = ibase + IL.bucket_table;
-  const bool counted_by_tile = T <= bucket_max_tiles() && total_slot != nullptr && g_tile_sort_large.load() > 0;
+  const uint32_t sort_limit = (uint32_t)g_tile_sort_large.load();
+  const bool counted_by_tile = T <= bucket_max_tiles() && total_slot != nullptr && sort_limit > 0;
   bool bucketed = counted_by_tile;
   if (bucketed) {
     StageScope _t("tile_count", stream);
     // the histogram's grand total is the instance count: the host gets it from here, and the prefix over the
     // Gaussians below runs while the host is busy growing the binning buffer
     if (launch_bucket_count(P, width, height, radii, means2D, compute_locally, tiles_touched, bucket_table, ranges,
-                            total_slot, stream))
+                            sort_limit, total_slot, stream))
       return 1;
   } else {
     StageScope _t("tile_count", stream);
@@ -461,10 +467,11 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
   // it straight into pinned host memory and the host polls that word: no copy, and no sleeping wait whose
   // wake-up would leave the GPU idle.  On the bucketed route the count and, in the word beside it, the longest
   // tile list come from the kernel that builds the tile ranges.
-  uint32_t R_u = 0, longest = 0;
+  uint32_t R_u = 0, longest = 0, chunks = 0;
   if (total_slot != nullptr) {
     if (wait_for_total(total_slot, stream, &R_u)) return 1;
     longest = __atomic_load_n(total_slot + 1, __ATOMIC_ACQUIRE);
+    chunks = __atomic_load_n(total_slot + 2, __ATOMIC_ACQUIRE);
   } else {
     GS_HIP_TRY(hipMemcpyAsync(&R_u, point_offsets + (P - 1), sizeof(uint32_t), hipMemcpyDeviceToHost, stream));
     GS_HIP_TRY(hipStreamSynchronize(stream));
@@ -491,9 +498,10 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
   EventTimer timer;
   if (timer.begin(elapsed_ms != nullptr, stream)) return 1;
 
-  // a list too long for the per-tile sort: beyond 8192 records one tile's sort takes longer than the radix sort
-  // of the whole view
-  if (bucketed && longest > (uint32_t)g_tile_sort_large.load()) bucketed = false;
+  // A list of more than sort_limit records is sorted in chunks of at most that many and merged.  That serves a
+  // view with a few such lists; the merge looks every record up in every other chunk of its list, and a view
+  // with many long lists is sorted as fast by the radix sort over all its keys, which then takes over.
+  if (bucketed && longest > sort_limit && chunks > (uint32_t)g_tile_sort_chunks.load()) bucketed = false;
   if (bucketed) {
     if (R > 0) {
       {
@@ -504,8 +512,8 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
       if (check_launch("bucket_scatter", stream, dbg)) return 1;
       {
         StageScope _t("tile_sort", stream);
-        launch_tile_sort(T, longest, (uint32_t)g_tile_sort_registers.load(), ranges, keys_other, gauss_of_emission, keys,
-                         emission, point_list, stream);
+        launch_tile_sort(T, longest, sort_limit, chunks, (uint32_t)g_tile_sort_registers.load(), ranges, bucket_table,
+                         keys_other, gauss_of_emission, keys, emission, point_list, stream);
       }
       if (check_launch("tile_sort", stream, dbg)) return 1;
     }

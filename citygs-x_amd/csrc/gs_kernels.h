@@ -61,21 +61,23 @@ int launch_duplicate_with_keys(int P, int W, int H, const float* means2D, const 
                                hipStream_t stream);
 // ---- binning by tile: counting sort by tile + per-tile LDS sort (tile_bucket.hip) ----
 constexpr int TILE_SORT_SMALL = 2048;  // records per tile the small LDS variant holds
-constexpr int TILE_SORT_LARGE = 8192;  // longest list any per-tile sort takes; longer lists go to the radix sort
+constexpr int TILE_SORT_LARGE = 8192;  // longest list one workgroup sorts; longer ones are sorted in chunks and merged
+constexpr int TILE_SORT_MAX_CHUNKS = 32;  // chunks of long lists per view the merge takes; beyond: the radix sort
 int bucket_max_tiles();
 size_t bucket_table_bytes(int T);
-// tiles_touched per Gaussian, the workgroup-by-tile table, ranges (2 words per tile), and in two host-visible
-// words the number of instances (word 0, written last) and the longest list (word 1)
+// tiles_touched per Gaussian, the workgroup-by-tile table, ranges (2 words per tile), and in three host-visible
+// words the number of instances (word 0, written last), the longest list (word 1) and the number of chunks that
+// the lists of more than chunk_limit records are cut into (word 2)
 int launch_bucket_count(int P, int W, int H, const int* radii, const float* means2D, const uint8_t* compute_locally,
-                        uint32_t* tiles_touched, void* table, uint32_t* ranges, uint32_t* host_words,
-                        hipStream_t stream);
+                        uint32_t* tiles_touched, void* table, uint32_t* ranges, uint32_t chunk_limit,
+                        uint32_t* host_words, hipStream_t stream);
 int launch_bucket_scatter(int P, int W, int H, const float* means2D, const float* depths, const uint32_t* offsets,
                           const int* radii, const uint8_t* compute_locally, const void* table,
                           const uint32_t* ranges, uint64_t* records, uint32_t* gauss_of_emission,
                           hipStream_t stream);
-int launch_tile_sort(int T, uint32_t longest, uint32_t in_registers, const uint32_t* ranges, const uint64_t* records,
-                     const uint32_t* gauss_of_emission, uint64_t* keys, uint32_t* emission, uint32_t* point_list,
-                     hipStream_t stream);
+int launch_tile_sort(int T, uint32_t longest, uint32_t limit, uint32_t chunks, uint32_t in_registers,
+                     const uint32_t* ranges, const void* table, uint64_t* records, const uint32_t* gauss_of_emission,
+                     uint64_t* keys, uint32_t* emission, uint32_t* point_list, hipStream_t stream);
 int launch_gather_u32(int64_t n, const uint32_t* index, const uint32_t* table, uint32_t* out, hipStream_t stream);
 int launch_ssim_l1_fwd(int C, int H, int W, const float* img1, const float* img2, const uint8_t* mask,
                        float* l1_map, float* ssim_map, float* d_mu, float* d_xx, float* d_xy, hipStream_t stream);

@@ -122,35 +122,48 @@ __device__ __forceinline__ uint32_t wave_inclusive_scan_u32(uint32_t v, int lane
 }
 
 // 1c. One workgroup: exclusive prefix of the tile totals = the tile ranges (rasterizer_impl.cu:122-144 leaves
-// (0, 0) for a tile without instances).  The longest list and then the number of instances are stored where the
-// host can read them (host_words[1] and host_words[0]; the host polls word 0, so it is written last).
+// (0, 0) for a tile without instances).  A list of more than `limit` records is sorted in chunks that are merged
+// afterwards: chunk_first[t] = number of chunks of the tiles before t (chunk_first[T] = all chunks; a tile within
+// the limit has none).  The longest list, the number of chunks and then the number of instances are stored where
+// the host can read them (host_words[1], [2] and [0]; the host polls word 0, so it is written last).
 __global__ void __launch_bounds__(1024)
-bucket_ranges_kernel(uint32_t T, const uint32_t* __restrict__ totals, uint32_t* __restrict__ ranges,
-                     uint32_t* __restrict__ host_words) {
-  __shared__ uint32_t s_wave[16], s_max[16];
+bucket_ranges_kernel(uint32_t T, uint32_t limit, const uint32_t* __restrict__ totals, uint32_t* __restrict__ ranges,
+                     uint32_t* __restrict__ chunk_first, uint32_t* __restrict__ host_words) {
+  __shared__ uint32_t s_wave[16], s_wave_chunks[16], s_max[16];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  uint32_t carry = 0, longest = 0;
+  uint32_t carry = 0, carry_chunks = 0, longest = 0;
   for (uint32_t start = 0; start < T; start += 1024) {
     const uint32_t t = start + threadIdx.x;
     const uint32_t v = t < T ? totals[t] : 0u;
+    const uint32_t c = v > limit ? (v + limit - 1u) / limit : 0u;
     longest = v > longest ? v : longest;
     const uint32_t inc = wave_inclusive_scan_u32(v, lane);
-    if (lane == 63) s_wave[wave] = inc;
+    const uint32_t inc_chunks = wave_inclusive_scan_u32(c, lane);
+    if (lane == 63) {
+      s_wave[wave] = inc;
+      s_wave_chunks[wave] = inc_chunks;
+    }
     __syncthreads();
-    uint32_t base = 0, all = 0;
+    uint32_t base = 0, all = 0, base_chunks = 0, all_chunks = 0;
 #pragma unroll
     for (int w = 0; w < 16; w++) {
-      const uint32_t s = s_wave[w];
-      if (w < wave) base += s;
+      const uint32_t s = s_wave[w], sc = s_wave_chunks[w];
+      if (w < wave) {
+        base += s;
+        base_chunks += sc;
+      }
       all += s;
+      all_chunks += sc;
     }
     __syncthreads();
     const uint32_t begin = carry + base + inc - v;
     if (t < T) {
       ranges[2 * t] = v ? begin : 0u;
       ranges[2 * t + 1] = v ? begin + v : 0u;
+      chunk_first[t] = carry_chunks + base_chunks + inc_chunks - c;
     }
     carry += all;
+    carry_chunks += all_chunks;
   }
 #pragma unroll
   for (int d = 32; d >= 1; d >>= 1) {
@@ -162,7 +175,9 @@ bucket_ranges_kernel(uint32_t T, const uint32_t* __restrict__ totals, uint32_t* 
   if (threadIdx.x == 0) {
     uint32_t m = 0;
     for (int w = 0; w < 16; w++) m = s_max[w] > m ? s_max[w] : m;
+    chunk_first[T] = carry_chunks;
     __hip_atomic_store(host_words + 1, m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    __hip_atomic_store(host_words + 2, carry_chunks, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
     __hip_atomic_store(host_words, carry, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
   }
 }
@@ -326,12 +341,12 @@ __device__ __forceinline__ void register_sort_tile(uint32_t t, uint32_t start, u
 __global__ void __launch_bounds__(256)
 tile_sort_registers_kernel(const uint32_t* __restrict__ ranges, const uint64_t* __restrict__ records,
                            const uint32_t* __restrict__ gauss_of_emission, uint64_t* __restrict__ keys,
-                           uint32_t* __restrict__ emission, uint32_t* __restrict__ point_list) {
+                           uint32_t* __restrict__ emission, uint32_t* __restrict__ point_list, uint32_t max_n) {
   extern __shared__ uint64_t s_exchange[];
   const uint32_t t = blockIdx.x;
   const uint32_t start = ranges[2 * t];
   const uint32_t n = ranges[2 * t + 1] - start;
-  if (n == 0 || n > 2048) return;
+  if (n == 0 || n > 2048 || n > max_n) return;
   if (n <= 256) GS_SORT_CASE(1, 4);
   else if (n <= 512) GS_SORT_CASE(2, 4);
   else if (n <= 1024) GS_SORT_CASE(4, 4);
@@ -341,14 +356,101 @@ tile_sort_registers_kernel(const uint32_t* __restrict__ ranges, const uint64_t* 
 __global__ void __launch_bounds__(1024)
 tile_sort_registers_long_kernel(const uint32_t* __restrict__ ranges, const uint64_t* __restrict__ records,
                                 const uint32_t* __restrict__ gauss_of_emission, uint64_t* __restrict__ keys,
-                                uint32_t* __restrict__ emission, uint32_t* __restrict__ point_list) {
+                                uint32_t* __restrict__ emission, uint32_t* __restrict__ point_list,
+                                uint32_t max_n) {
   extern __shared__ uint64_t s_exchange[];
   const uint32_t t = blockIdx.x;
   const uint32_t start = ranges[2 * t];
   const uint32_t n = ranges[2 * t + 1] - start;
-  if (n <= 2048) return;
+  if (n <= 2048 || n > max_n) return;
   if (n <= 4096) GS_SORT_CASE(4, 16);
   else GS_SORT_CASE(8, 16);
+}
+
+// 2b. Lists beyond the limit of the per-tile sort: the list is cut into chunk_first[t + 1] - chunk_first[t]
+// chunks of equal size (the last one may be shorter), one workgroup sorts each chunk in place, and the merge
+// below puts every record at its final place.
+struct Chunk { uint32_t tile, list_start, list_n, size, index, count; };
+__device__ __forceinline__ Chunk find_chunk(uint32_t b, uint32_t T, const uint32_t* __restrict__ chunk_first,
+                                            const uint32_t* __restrict__ ranges) {
+  // the tile t with chunk_first[t] <= b < chunk_first[t + 1]
+  uint32_t lo = 0, hi = T;
+  while (hi - lo > 1) {
+    const uint32_t mid = (lo + hi) >> 1;
+    if (chunk_first[mid] <= b) lo = mid; else hi = mid;
+  }
+  Chunk c;
+  c.tile = lo;
+  c.list_start = ranges[2 * lo];
+  c.list_n = ranges[2 * lo + 1] - c.list_start;
+  c.count = chunk_first[lo + 1] - chunk_first[lo];
+  c.index = b - chunk_first[lo];
+  c.size = (c.list_n + c.count - 1u) / c.count;
+  return c;
+}
+
+template <int E, int W>
+__device__ __forceinline__ void register_sort_in_place(uint64_t* __restrict__ records, uint32_t n, uint64_t* s_x) {
+  const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  uint64_t v[E];
+#pragma unroll
+  for (int r = 0; r < E; r++) {
+    const uint32_t i = ((wave * E + r) << 6) | lane;
+    v[r] = i < n ? records[i] : ~0ull;
+  }
+  register_sort<E, W>(v, wave, lane, s_x);
+#pragma unroll
+  for (int r = 0; r < E; r++) {
+    const uint32_t i = ((wave * E + r) << 6) | lane;
+    if (i < n) records[i] = v[r];
+  }
+}
+
+__global__ void __launch_bounds__(1024)
+chunk_sort_kernel(uint32_t T, const uint32_t* __restrict__ chunk_first, const uint32_t* __restrict__ ranges,
+                  uint64_t* __restrict__ records) {
+  extern __shared__ uint64_t s_exchange[];
+  const Chunk c = find_chunk(blockIdx.x, T, chunk_first, ranges);
+  const uint32_t begin = c.index * c.size;
+  if (begin >= c.list_n) return;
+  const uint32_t n = c.list_n - begin < c.size ? c.list_n - begin : c.size;
+  uint64_t* mine = records + c.list_start + begin;
+  if (n <= 4096) register_sort_in_place<4, 16>(mine, n, s_exchange);
+  else register_sort_in_place<8, 16>(mine, n, s_exchange);
+}
+
+// A record's final place in its tile's list: its place in its own chunk plus, for every other chunk of the
+// list, the number of that chunk's records below it (records are distinct: they end in the emission index).
+__global__ void __launch_bounds__(256)
+chunk_merge_kernel(uint32_t T, const uint32_t* __restrict__ chunk_first, const uint32_t* __restrict__ ranges,
+                   const uint64_t* __restrict__ records, const uint32_t* __restrict__ gauss_of_emission,
+                   uint64_t* __restrict__ keys, uint32_t* __restrict__ emission, uint32_t* __restrict__ point_list) {
+  const Chunk c = find_chunk(blockIdx.x, T, chunk_first, ranges);
+  const uint32_t begin = c.index * c.size;
+  if (begin >= c.list_n) return;
+  const uint32_t n = c.list_n - begin < c.size ? c.list_n - begin : c.size;
+  const uint64_t* list = records + c.list_start;
+  const uint64_t tile_bits = (uint64_t)c.tile << 32;
+  for (uint32_t i = threadIdx.x; i < n; i += 256) {
+    const uint64_t rec = list[begin + i];
+    uint32_t place = i;
+    for (uint32_t other = 0; other < c.count; other++) {
+      if (other == c.index) continue;
+      const uint32_t ob = other * c.size;
+      if (ob >= c.list_n) break;
+      const uint32_t on = c.list_n - ob < c.size ? c.list_n - ob : c.size;
+      uint32_t lo = 0, hi = on;  // number of records of the other chunk below rec
+      while (lo < hi) {
+        const uint32_t mid = (lo + hi) >> 1;
+        if (list[ob + mid] < rec) lo = mid + 1; else hi = mid;
+      }
+      place += lo;
+    }
+    const uint32_t e = (uint32_t)rec;
+    keys[c.list_start + place] = tile_bits | (rec >> 32);
+    emission[c.list_start + place] = e;
+    point_list[c.list_start + place] = gauss_of_emission[e];
+  }
 }
 
 #undef GS_SORT_CASE
@@ -412,13 +514,14 @@ tile_sort_kernel(const uint32_t* __restrict__ ranges, const uint64_t* __restrict
 // Tiles the LDS histograms of the counting kernels can hold.
 int bucket_max_tiles() { return 30000; }
 
-// workgroup-by-tile counts, then the tile totals
-size_t bucket_table_bytes(int T) { return ((size_t)BK_MAX_BLOCKS + 1) * (size_t)T * sizeof(uint32_t); }
+// workgroup-by-tile counts, then the tile totals, then the chunk table (T + 1 words)
+size_t bucket_table_bytes(int T) { return (((size_t)BK_MAX_BLOCKS + 2) * (size_t)T + 1) * sizeof(uint32_t); }
 
 int launch_bucket_count(int P, int W, int H, const int* radii, const float* means2D, const uint8_t* compute_locally,
-                        uint32_t* tiles_touched, void* table, uint32_t* ranges, uint32_t* host_words,
-                        hipStream_t stream) {
+                        uint32_t* tiles_touched, void* table, uint32_t* ranges, uint32_t chunk_limit,
+                        uint32_t* host_words, hipStream_t stream) {
   if (P <= 0) return 0;
+  if (chunk_limit == 0 || chunk_limit > (uint32_t)TILE_SORT_LARGE) chunk_limit = TILE_SORT_LARGE;
   const uint32_t gx = (W + GS_TILE_X - 1) / GS_TILE_X, gy = (H + GS_TILE_Y - 1) / GS_TILE_Y;
   const uint32_t T = gx * gy;
   const size_t lds = (size_t)T * (sizeof(uint32_t) + 1);
@@ -437,7 +540,8 @@ int launch_bucket_count(int P, int W, int H, const int* radii, const float* mean
                      (const float2*)means2D, compute_locally, tiles_touched, tab);
   hipLaunchKernelGGL(bucket_columns_kernel, dim3((T + COL_TILES - 1) / COL_TILES), dim3(COL_TILES * COL_RUNS), 0, stream, nb, T,
                      tab, totals);
-  hipLaunchKernelGGL(bucket_ranges_kernel, dim3(1), dim3(1024), 0, stream, T, totals, ranges, host_words);
+  hipLaunchKernelGGL(bucket_ranges_kernel, dim3(1), dim3(1024), 0, stream, T, chunk_limit, totals, ranges, totals + T,
+                     host_words);
   return 0;
 }
 
@@ -454,30 +558,40 @@ int launch_bucket_scatter(int P, int W, int H, const float* means2D, const float
   return 0;
 }
 
-// Sorts every tile's segment; `longest` is the longest list (nothing may exceed TILE_SORT_LARGE).  The register
-// variant by default; with in_registers == 0 the LDS variants (small up to
-// TILE_SORT_SMALL, then large).
-int launch_tile_sort(int T, uint32_t longest, uint32_t in_registers, const uint32_t* ranges, const uint64_t* records,
-                     const uint32_t* gauss_of_emission, uint64_t* keys, uint32_t* emission, uint32_t* point_list,
-                     hipStream_t stream) {
+// Sorts every tile's segment.  `longest` is the longest list and `limit` (at most TILE_SORT_LARGE) the longest
+// one workgroup sorts whole: the register variant by default, with in_registers == 0 the LDS variants (small
+// up to TILE_SORT_SMALL, then large).  Longer lists are the `chunks` chunks that launch_bucket_count laid out
+// with the same limit: sorted in place in `records`, then merged.
+int launch_tile_sort(int T, uint32_t longest, uint32_t limit, uint32_t chunks, uint32_t in_registers,
+                     const uint32_t* ranges, const void* table, uint64_t* records, const uint32_t* gauss_of_emission,
+                     uint64_t* keys, uint32_t* emission, uint32_t* point_list, hipStream_t stream) {
   if (T <= 0 || longest == 0) return 0;
+  if (limit == 0 || limit > (uint32_t)TILE_SORT_LARGE) limit = TILE_SORT_LARGE;
+  const uint32_t whole = longest < limit ? longest : limit;  // the longest list sorted by one workgroup
   if (in_registers == 0) {
+    const uint32_t small_max = limit < (uint32_t)TILE_SORT_SMALL ? limit : (uint32_t)TILE_SORT_SMALL;
     hipLaunchKernelGGL(tile_sort_kernel<TILE_SORT_SMALL>, dim3(T), dim3(TS_THREADS), 0, stream, ranges, records,
-                       gauss_of_emission, keys, emission, point_list, 0u, (uint32_t)TILE_SORT_SMALL);
-    if (longest > (uint32_t)TILE_SORT_SMALL)
+                       gauss_of_emission, keys, emission, point_list, 0u, small_max);
+    if (whole > (uint32_t)TILE_SORT_SMALL)
       hipLaunchKernelGGL(tile_sort_kernel<TILE_SORT_LARGE>, dim3(T), dim3(TS_THREADS), 0, stream, ranges, records,
-                         gauss_of_emission, keys, emission, point_list, (uint32_t)TILE_SORT_SMALL,
-                         (uint32_t)TILE_SORT_LARGE);
-    return 0;
+                         gauss_of_emission, keys, emission, point_list, (uint32_t)TILE_SORT_SMALL, limit);
+  } else {
+    uint32_t m = 256;
+    while (m < whole && m < 2048) m <<= 1;
+    hipLaunchKernelGGL(tile_sort_registers_kernel, dim3(T), dim3(256), (size_t)m * sizeof(uint64_t), stream, ranges,
+                       records, gauss_of_emission, keys, emission, point_list, limit);
+    if (whole > 2048)
+      hipLaunchKernelGGL(tile_sort_registers_long_kernel, dim3(T), dim3(1024),
+                         (size_t)(whole > 4096 ? 8192 : 4096) * sizeof(uint64_t), stream, ranges, records,
+                         gauss_of_emission, keys, emission, point_list, limit);
   }
-  uint32_t m = 256;
-  while (m < longest && m < 2048) m <<= 1;
-  hipLaunchKernelGGL(tile_sort_registers_kernel, dim3(T), dim3(256), (size_t)m * sizeof(uint64_t), stream, ranges,
-                     records, gauss_of_emission, keys, emission, point_list);
-  if (longest > 2048)
-    hipLaunchKernelGGL(tile_sort_registers_long_kernel, dim3(T), dim3(1024),
-                       (size_t)(longest > 4096 ? 8192 : 4096) * sizeof(uint64_t), stream, ranges, records,
+  if (longest > limit && chunks > 0) {
+    const uint32_t* chunk_first = (const uint32_t*)table + ((size_t)BK_MAX_BLOCKS + 1) * (size_t)T;
+    hipLaunchKernelGGL(chunk_sort_kernel, dim3(chunks), dim3(1024), (size_t)(limit > 4096 ? 8192 : 4096) * sizeof(uint64_t),
+                       stream, (uint32_t)T, chunk_first, ranges, records);
+    hipLaunchKernelGGL(chunk_merge_kernel, dim3(chunks), dim3(256), 0, stream, (uint32_t)T, chunk_first, ranges, records,
                        gauss_of_emission, keys, emission, point_list);
+  }
   return 0;
 }
 

@@ -41,7 +41,7 @@ _SIGNATURES = {
     "gs_training_stats": (_i, [_i64, _i, _i64, _i64, _vp, _vp, _vp, _vp, _i] + [_vp] * 6 + [_sz, _vp]),
     "gs_max_radii_update": (_i, [_i64, _vp, _vp, _vp, _vp]),
     "gs_adam_step": (_i, [_i] + [_vp] * 7 + [C.c_double, C.c_double, C.c_double, _f, _vp]),
-    "gs_set_tile_sort_limits": (None, [_i, _i]),
+    "gs_set_tile_sort_limits": (None, [_i, _i, _i]),
     "gs_neural_supported": (_i, [_i]),
     "gs_neural_workspace_bytes": (_sz, [_i64, _i]),
     "gs_neural_opacity_forward": (_i, [_i64, _i] + [_vp] * 8 + [_sz, _vp, _vp]),

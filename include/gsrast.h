@@ -93,13 +93,16 @@ int gs_preprocess_backward(const int* radii, const float* cov3D, const uint8_t* 
                            int debug, gs_stream_t stream);
 
 /* No counterpart in the reference: a test hook.  gs_render_forward builds the per-tile lists either by
- * bucketing the instances by tile and sorting each tile's list on its own (lists of up to 8192 records), or, when
- * a list is longer than that (or the tile grid larger than 30000 tiles), by the reference's own route:
+ * bucketing the instances by tile and sorting each tile's list on its own (one workgroup per list of up to 8192
+ * records; longer lists as chunks of at most 8192 that are merged afterwards, up to 32 chunks per view), or, when
+ * the view has more long lists than that (or the tile grid more than 30000 tiles), by the reference's own route:
  * (tile | depth) keys (rasterizer_impl.cu:74-117), one radix sort over all of them (:675-684), identifyTileRanges
  * (:122-144).  All give the same lists bit for bit.  in_registers = 0 makes the per-tile sort keep its records in
- * LDS instead of registers (default 1); large_limit lowers the list length up to which a per-tile sort is used
- * (default 8192; 0 = always the radix route), so that small scenes can exercise every route. */
-void gs_set_tile_sort_limits(int in_registers, int large_limit);
+ * LDS instead of registers (default 1); large_limit lowers the list length that one workgroup sorts whole
+ * (default 8192; 0 = always the radix route) and max_chunks changes the number of chunks the longer lists of a
+ * view may be cut into (default 32; 0 = a longer list sends the view to the radix route), so that small scenes
+ * can exercise every route. */
+void gs_set_tile_sort_limits(int in_registers, int large_limit, int max_chunks);
 
 /* Replaces Rasterizer::renderForward (CR/rasterizer.h:130-160,
  * CR/rasterizer_impl.cu:586-846): tile count -> prefix sum -> host read-back of

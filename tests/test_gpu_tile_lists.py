@@ -1,6 +1,6 @@
 """The per-tile lists render_gaussians builds (ranges, sorted keys, point_list), by each of its routes: instances
-bucketed by tile and sorted per tile in LDS (small and large variant), and the radix sort over all (tile | depth)
-keys.  Every route must give the oracle's lists bit for bit, and the backward pass must file its per-instance
+bucketed by tile and sorted per tile (in registers or in LDS; a list beyond the limit of one workgroup in chunks
+that are merged), and the radix sort over all (tile | depth) keys.  Every route must give the oracle's lists bit for bit, and the backward pass must file its per-instance
 gradients correctly under each."""
 import ctypes as C
 
@@ -23,7 +23,7 @@ def H():
 def _restore_limits():
     import gsrast_native as gn
     yield
-    gn.lib.gs_set_tile_sort_limits(1, 8192)
+    gn.lib.gs_set_tile_sort_limits(1, 8192, 32)
 
 
 def _mask(kind, gx, gy):
@@ -36,9 +36,11 @@ def _mask(kind, gx, gy):
     return cl
 
 
-# (records in registers?, per-tile limit): defaults; every list through the LDS variants; a list longer than the
-# per-tile limit, found after the counting pass (the radix route takes over); the radix route from the start
-ROUTES = [(1, 8192), (0, 8192), (1, 40), (1, 0)]
+# (records in registers?, longest list one workgroup sorts, chunks the longer lists may be cut into): defaults; every
+# list through the LDS variants; a list too long for the per-tile sort, found after the counting pass (the radix
+# route takes over); the radix route from the start; lists beyond the limit sorted in chunks and merged (few large
+# chunks, the same behind the LDS variants, many chunks of an odd size)
+ROUTES = [(1, 8192, 32), (0, 8192, 32), (1, 40, 0), (1, 0, 32), (1, 40, 1 << 30), (0, 100, 1 << 30), (1, 7, 1 << 30)]
 
 
 @pytest.mark.parametrize("cfg,P,mask", [(0, 30_000, "all"), (1, 120_000, "all"), (1, 60_000, "checker"),
@@ -65,8 +67,8 @@ def test_lists_match_oracle_by_every_route(orc, H, cfg, P, mask):
     ug = gs_scenes.upstream_grads(cam)
     args = {"stats_collector": {}}
     grads = []
-    for small, large in ROUTES:
-        gn.lib.gs_set_tile_sort_limits(small, large)
+    for small, large, chunks in ROUTES:
+        gn.lib.gs_set_tile_sort_limits(small, large, chunks)
         out = _C.render_gaussians(torch.zeros(3, device=DEV), Hh, W, o["means2D"], o["depths"], o["radii"],
                                   o["conic_opacity"], o["rgb"], cl.to(DEV), vm, cp, cam.tanfovx, cam.tanfovy, am,
                                   True, False, args)
@@ -81,9 +83,9 @@ def test_lists_match_oracle_by_every_route(orc, H, cfg, P, mask):
         gn.check(gn.lib.gs_image_state_layout(W, Hh, *[C.byref(x) for x in ioff]), "layout")
         ibase = (imgB.data_ptr() + 255) // 256 * 256 - imgB.data_ptr()
         ranges = imgB[ibase + ioff[3].value: ibase + ioff[3].value + 8 * T].view(torch.int32)
-        assert np.array_equal(H.np_u32(ranges), want["ranges"].reshape(-1)), (small, large)
-        assert np.array_equal(H.np_u32(point_list), want["point_list"]), (small, large)
-        assert np.array_equal(H.np_u64(keys), want["keys"]), (small, large)
+        assert np.array_equal(H.np_u32(ranges), want["ranges"].reshape(-1)), (small, large, chunks)
+        assert np.array_equal(H.np_u32(point_list), want["point_list"]), (small, large, chunks)
+        assert np.array_equal(H.np_u64(keys), want["keys"]), (small, large, chunks)
         assert np.array_equal(n(n_render), (counts[:, 1] - counts[:, 0]).astype(np.int32))
         back = _C.render_gaussians_backward(torch.zeros(3, device=DEV), cam.tanfovx, cam.tanfovy, oam, am, R, geomB,
                                             binB, imgB, cl.to(DEV), ug["color"].to(DEV), ug["all_map"].to(DEV),
@@ -124,8 +126,8 @@ def test_equal_depths_keep_emission_order(orc, H):
     want = orc.bin_and_sort(n(o["radii"]), n(o["means2D"]), n(o["depths"]), cl.numpy().reshape(-1), W, Hh)
     vm, cp = cam.world_view_transform.to(DEV), cam.camera_center.to(DEV)
     am = gs_scenes.build_all_map(gd["means3D"], gd["scales"], gd["rotations"], cam)
-    for small, large in ROUTES:
-        gn.lib.gs_set_tile_sort_limits(small, large)
+    for small, large, chunks in ROUTES:
+        gn.lib.gs_set_tile_sort_limits(small, large, chunks)
         out = _C.render_gaussians(torch.zeros(3, device=DEV), Hh, W, o["means2D"], o["depths"], o["radii"],
                                   o["conic_opacity"], o["rgb"], cl.to(DEV), vm, cp, cam.tanfovx, cam.tanfovy, am,
                                   True, False, {"stats_collector": {}})
@@ -134,13 +136,15 @@ def test_equal_depths_keep_emission_order(orc, H):
         gn.check(gn.lib.gs_binning_state_layout(R, W, Hh, *[C.byref(x) for x in off]), "layout")
         base = (binB.data_ptr() + 255) // 256 * 256 - binB.data_ptr()
         point_list = binB[base + off[0].value: base + off[0].value + 4 * R].view(torch.int32)
-        assert np.array_equal(H.np_u32(point_list), want["point_list"]), (small, large)
+        assert np.array_equal(H.np_u32(point_list), want["point_list"]), (small, large, chunks)
 
 
-@pytest.mark.parametrize("P,expect", [(28_000, "waves4"), (56_000, "waves8"), (110_000, "radix")])
+@pytest.mark.parametrize("P,expect", [(28_000, "waves4"), (56_000, "waves8"), (110_000, "chunks"),
+                                      (110_000, "radix"), (230_000, "chunks3")])
 def test_long_lists(orc, H, P, expect):
     """A small image under many large Gaussians: lists of several thousand records per tile (sixteen waves per
-    tile, 4 or 8 records per lane), and beyond 8192 the radix route, which then takes over by itself."""
+    tile, 4 or 8 records per lane); beyond 8192 the list is sorted in chunks and merged, or, where the view has
+    more such chunks than the bound, the radix route takes over by itself."""
     import gs_scenes
     import gsrast_native as gn
     from diff_gaussian_rasterization import _C
@@ -156,8 +160,13 @@ def test_long_lists(orc, H, P, expect):
     want = orc.bin_and_sort(n(o["radii"]), n(o["means2D"]), n(o["depths"]), cl.numpy().reshape(-1), W, Hh)
     counts = want["ranges"].reshape(-1, 2).astype(np.int64)
     longest = int((counts[:, 1] - counts[:, 0]).max())
-    lo, hi = {"waves4": (2048, 4096), "waves8": (4096, 8192), "radix": (8192, 1 << 30)}[expect]
+    lo, hi = {"waves4": (2048, 4096), "waves8": (4096, 8192), "chunks": (8192, 16384), "radix": (8192, 16384),
+              "chunks3": (16384, 65536)}[expect]
     assert lo < longest <= hi, longest
+    if expect == "radix":
+        gn.lib.gs_set_tile_sort_limits(1, 8192, 0)
+    elif expect.startswith("chunks"):  # nearly every tile of this view has a long list: lift the bound on their number
+        gn.lib.gs_set_tile_sort_limits(1, 8192, 1 << 30)
     vm, cp = cam.world_view_transform.to(DEV), cam.camera_center.to(DEV)
     am = gs_scenes.build_all_map(gd["means3D"], gd["scales"], gd["rotations"], cam)
     out = _C.render_gaussians(torch.zeros(3, device=DEV), Hh, W, o["means2D"], o["depths"], o["radii"],
