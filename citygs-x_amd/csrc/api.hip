@@ -745,8 +745,9 @@ size_t gs_neural_workspace_bytes(int64_t num_anchors, int n_offsets) {
 }
 
 int gs_neural_opacity_forward(int64_t N, int k, const float* anchor, const float* feat, const float* campos,
-                              const float* const* mlp_params, float* neural_opacity, uint8_t* mask, uint32_t* first,
-                              void* workspace, size_t workspace_bytes, int64_t* num_selected, gs_stream_t stream_) {
+                              const float* const* mlp_params, const float* opacity_scale, float* neural_opacity,
+                              uint8_t* mask, uint32_t* first, void* workspace, size_t workspace_bytes,
+                              int64_t* num_selected, gs_stream_t stream_) {
   hipStream_t stream = (hipStream_t)stream_;
   GS_REQUIRE(N >= 0, "gs_neural_opacity_forward: negative anchor count");
   GS_REQUIRE(neural_supported(k), "gs_neural_opacity_forward: n_offsets not among the supported values");
@@ -770,7 +771,7 @@ int gs_neural_opacity_forward(int64_t N, int k, const float* anchor, const float
   uint8_t* counts = (uint8_t*)(base + L.counts);
   {
     StageScope _t("neural_opacity", stream);
-    launch_neural_opacity(N, k, anchor, feat, campos, packed, neural_opacity, mask, counts, stream);
+    launch_neural_opacity(N, k, anchor, feat, campos, packed, opacity_scale, neural_opacity, mask, counts, stream);
   }
   if (check_launch("neural_opacity", stream, false)) return 1;
   uint32_t* total_slot = acquire_total_slot();
@@ -829,11 +830,11 @@ size_t gs_neural_backward_workspace_bytes(int64_t num_anchors, int n_offsets) {
 
 int gs_neural_backward(int64_t N, int k, int64_t S, const float* anchor, const float* feat, const float* offsets,
                        const float* scaling, const float* campos, const float* const* mlp_params,
-                       const float* neural_opacity, const uint32_t* first, const float* color, const float* rot,
-                       const float* aux, const float* dL_dxyz, const float* dL_dcolor, const float* dL_dopacity,
-                       const float* dL_dscaling, const float* dL_drot, float* d_anchor, float* d_feat,
-                       float* d_offsets, float* d_scaling, float* const* d_mlp_params, void* workspace,
-                       size_t workspace_bytes, gs_stream_t stream_) {
+                       const float* opacity_scale, const float* neural_opacity, const uint32_t* first,
+                       const float* color, const float* rot, const float* aux, const float* dL_dxyz,
+                       const float* dL_dcolor, const float* dL_dopacity, const float* dL_dscaling,
+                       const float* dL_drot, float* d_anchor, float* d_feat, float* d_offsets, float* d_scaling,
+                       float* const* d_mlp_params, void* workspace, size_t workspace_bytes, gs_stream_t stream_) {
   hipStream_t stream = (hipStream_t)stream_;
   GS_REQUIRE(N >= 0 && S >= 0, "gs_neural_backward: negative size");
   GS_REQUIRE(neural_supported(k), "gs_neural_backward: n_offsets not among the supported values");
@@ -871,8 +872,8 @@ int gs_neural_backward(int64_t N, int k, int64_t S, const float* anchor, const f
   if (check_launch("neural_pack", stream, false)) return 1;
   {
     StageScope _t("neural_backward", stream);
-    launch_neural_backward(N, k, anchor, feat, offsets, scaling, campos, packed, neural_opacity, first, color, rot,
-                           aux, dL_dxyz, dL_dcolor, dL_dopacity, dL_dscaling, dL_drot, d_anchor, d_feat, d_offsets,
+    launch_neural_backward(N, k, anchor, feat, offsets, scaling, campos, packed, neural_opacity, opacity_scale, first,
+                           color, rot, aux, dL_dxyz, dL_dcolor, dL_dopacity, dL_dscaling, dL_drot, d_anchor, d_feat, d_offsets,
                            d_scaling, d_mlp_params, slot_grads, partials, stream);
   }
   return check_launch("neural_backward", stream, false);

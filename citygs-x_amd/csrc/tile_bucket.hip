@@ -7,8 +7,11 @@
 //   2. one workgroup per tile sorting its segment in LDS by (depth bits, emission index): the emission index
 //      is unique, so the order does not depend on how the scatter happened to fill the segment, and it is the
 //      order a stable sort on the depth bits would leave.
-// No pass over all instances per digit, no look-back chain.  Lists longer than the LDS variant holds are left to
-// the radix sort (the caller decides from the longest list, which this code reports).
+// No pass over all instances per digit, no look-back chain.  A list longer than one workgroup sorts is cut into
+// chunks that are sorted the same way and then merged; a view with many such lists is left to the radix sort
+// (the caller decides from the longest list and the number of chunks, which this code reports).
+#include <atomic>
+
 #include "gs_common.h"
 #include "gs_kernels.h"
 
@@ -525,13 +528,18 @@ int launch_bucket_count(int P, int W, int H, const int* radii, const float* mean
   const uint32_t gx = (W + GS_TILE_X - 1) / GS_TILE_X, gy = (H + GS_TILE_Y - 1) / GS_TILE_Y;
   const uint32_t T = gx * gy;
   const size_t lds = (size_t)T * (sizeof(uint32_t) + 1);
-  static bool raised = false;  // more than 64 KB of dynamic LDS has to be asked for once per kernel
-  if (!raised) {
+  // more than 64 KB of dynamic LDS has to be asked for, once per kernel and device (two threads that both find
+  // the bit clear both ask, which is harmless)
+  static std::atomic<uint64_t> raised{0};
+  int dev = 0;
+  GS_HIP_TRY(hipGetDevice(&dev));
+  const uint64_t dev_bit = 1ull << (dev & 63);
+  if (lds > 64 * 1024 && (dev >= 64 || !(raised.load(std::memory_order_acquire) & dev_bit))) {
     GS_HIP_TRY(hipFuncSetAttribute((const void*)bucket_count_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
                                    bucket_max_tiles() * (int)(sizeof(uint32_t) + 1)));
     GS_HIP_TRY(hipFuncSetAttribute((const void*)bucket_scatter_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
                                    bucket_max_tiles() * (int)(sizeof(uint32_t) + 1)));
-    raised = true;
+    raised.fetch_or(dev_bit, std::memory_order_release);
   }
   const int nb = bucket_blocks(P), per = bucket_per_block(P);
   uint32_t* tab = (uint32_t*)table;

@@ -2,8 +2,8 @@
 as three kernel launches forward (opacity MLP, scan, color/cov MLPs with the post-processing) and two backward,
 in libgsrast.so.  The fused operator is the reference's default model configuration (arguments/__init__.py:94-124):
 feat_dim 32, inputs [feature, view direction]; the drop-in function also serves the appearance embedding and the
-feature bank, which reduce to it; distance or level inputs to the MLPs and dist2level 'progressive' raise
-NotImplementedError."""
+feature bank, which reduce to it, and dist2level 'progressive' (a per-anchor factor on the opacity); distance or
+level inputs to the MLPs raise NotImplementedError."""
 import ctypes as C
 
 import torch
@@ -39,7 +39,7 @@ def _param_shapes(k):
 
 class _NeuralGaussians(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, anchor, feat, offsets, scaling, campos, *params):
+    def forward(ctx, anchor, feat, offsets, scaling, campos, opacity_scale, *params):
         if len(params) != 12:
             raise RuntimeError("expected W1, b1, W2, b2 of the opacity, color and cov MLPs (12 tensors)")
         N = anchor.shape[0]
@@ -51,6 +51,8 @@ class _NeuralGaussians(torch.autograd.Function):
         anchor, feat = _f32(anchor, "anchor", (N, 3)), _f32(feat, "feat", (N, 32))
         offsets, scaling = _f32(offsets, "offsets", (N, k, 3)), _f32(scaling, "scaling", (N, 6))
         campos = _f32(campos, "camera_center", (3,))
+        if opacity_scale is not None:
+            opacity_scale = _f32(opacity_scale.detach(), "opacity_scale", (N,))
         params = [_f32(p, f"MLP parameter {i}", s) for i, (p, s) in enumerate(zip(params, _param_shapes(k)))]
         dev = anchor.device
         stream = C.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
@@ -61,8 +63,10 @@ class _NeuralGaussians(torch.autograd.Function):
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
         table = _table(params)
         S = C.c_int64(0)
-        _n.check(_n.lib.gs_neural_opacity_forward(N, k, _p(anchor), _p(feat), _p(campos), table, _p(neural_opacity),
-                                                  _p(mask), _p(first), _p(ws), ws_bytes, C.byref(S), stream),
+        _n.check(_n.lib.gs_neural_opacity_forward(N, k, _p(anchor), _p(feat), _p(campos), table,
+                                                  _p(opacity_scale),
+                                                  _p(neural_opacity), _p(mask), _p(first), _p(ws), ws_bytes,
+                                                  C.byref(S), stream),
                  "generate_neural_gaussians")
         S = S.value
         xyz, color = torch.empty(S, 3, device=dev), torch.empty(S, 3, device=dev)
@@ -74,6 +78,7 @@ class _NeuralGaussians(torch.autograd.Function):
                                                     stream), "generate_neural_gaussians")
         ctx.save_for_backward(anchor, feat, offsets, scaling, campos, neural_opacity, first, color, rot, aux, *params)
         ctx.sizes = (N, k, S)
+        ctx.opacity_scale = opacity_scale  # carries no gradient (a buffer of the model)
         ctx.mark_non_differentiable(neural_opacity, mask)
         ctx.set_materialize_grads(False)
         return xyz, color, opacity, scal, rot, neural_opacity, mask
@@ -93,20 +98,25 @@ class _NeuralGaussians(torch.autograd.Function):
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
         stream = C.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
         _n.check(_n.lib.gs_neural_backward(N, k, S, _p(anchor), _p(feat), _p(offsets), _p(scaling), _p(campos),
-                                           _table(params), _p(neural_opacity), _p(first), _p(color), _p(rot), _p(aux),
+                                           _table(params),
+                                           _p(ctx.opacity_scale),
+                                           _p(neural_opacity), _p(first), _p(color), _p(rot), _p(aux),
                                            *[_p(u) for u in ups], _p(d_anchor), _p(d_feat), _p(d_offsets),
                                            _p(d_scaling), _table(d_params), _p(ws), ws_bytes, stream),
                  "generate_neural_gaussians backward")
-        return (d_anchor, d_feat, d_offsets, d_scaling, None, *d_params)
+        return (d_anchor, d_feat, d_offsets, d_scaling, None, None, *d_params)
 
 
-def neural_gaussians(anchor, feat, offsets, scaling, camera_center, mlp_opacity, mlp_color, mlp_cov):
+def neural_gaussians(anchor, feat, offsets, scaling, camera_center, mlp_opacity, mlp_color, mlp_cov,
+                     opacity_scale=None):
     """The body of generate_neural_gaussians after the visible_mask gathers (gaussian_renderer/__init__.py:800-896).
     anchor (N,3), feat (N,32), offsets (N,k,3), scaling (N,6) = get_scaling, camera_center (3); each mlp_* is
-    (W1, b1, W2, b2) as nn.Linear holds them.  Returns (xyz, color, opacity, scaling, rot, neural_opacity, mask);
+    (W1, b1, W2, b2) as nn.Linear holds them; opacity_scale (N), if given, multiplies the opacity MLP's output per
+    anchor (:844-848).  Returns (xyz, color, opacity, scaling, rot, neural_opacity, mask);
     differentiable in everything but the camera centre; neural_opacity and mask carry no gradient (the reference
     uses them detached, scene/gaussian_model.py:1183)."""
-    return _NeuralGaussians.apply(anchor, feat, offsets, scaling, camera_center, *mlp_opacity, *mlp_color, *mlp_cov)
+    return _NeuralGaussians.apply(anchor, feat, offsets, scaling, camera_center, opacity_scale, *mlp_opacity,
+                                  *mlp_color, *mlp_cov)
 
 
 def _linear_pair(seq):
@@ -119,18 +129,25 @@ def generate_neural_gaussians(viewpoint_camera, pc, visible_mask=None, is_traini
     the appearance embedding (appearance_dim > 0: every anchor of a view gets the same embedding row, :830-836,
     :866-868, so its part of the first color layer is a per-view addition to that layer's bias) and the feature
     bank (use_feat_bank, :809-823: the view-dependent mix of the feature's resolutions is a few torch lines ahead
-    of the fused operator).  The distance / level inputs and progressive levels raise NotImplementedError."""
-    if (pc.add_opacity_dist or pc.add_color_dist or pc.add_cov_dist or pc.add_level
-            or pc.dist2level == "progressive"):
-        raise NotImplementedError("generate_neural_gaussians: distance or level inputs to the MLPs and progressive "
-                                  "levels are not built")
+    of the fused operator) and dist2level 'progressive' (:844-848: the opacity of an anchor in transition is scaled
+    by its progress ratio).  The distance / level inputs raise NotImplementedError."""
+    if pc.add_opacity_dist or pc.add_color_dist or pc.add_cov_dist or pc.add_level:
+        raise NotImplementedError("generate_neural_gaussians: distance or level inputs to the MLPs are not built")
+    progressive = pc.dist2level == "progressive"
+    opacity_scale = None
     if visible_mask is None:
         anchor, feat, offsets, scaling = pc.get_anchor, pc.get_anchor_feat, pc._offset, pc.get_scaling
+        if progressive:
+            opacity_scale = torch.where(pc.transition_mask, pc._prog_ratio.reshape(-1),
+                                        torch.ones_like(pc._prog_ratio.reshape(-1)))
     else:
         # one nonzero() (one host synchronisation) serves the four gathers; x[visible_mask] would run it four times
         idx = visible_mask.nonzero(as_tuple=True)[0]
         anchor, feat = pc.get_anchor.index_select(0, idx), pc.get_anchor_feat.index_select(0, idx)
         offsets, scaling = pc._offset.index_select(0, idx), pc.get_scaling.index_select(0, idx)
+        if progressive:
+            prog = pc._prog_ratio.reshape(-1).index_select(0, idx)
+            opacity_scale = torch.where(pc.transition_mask.index_select(0, idx), prog, torch.ones_like(prog))
     if pc.use_feat_bank:
         ob_view = anchor - viewpoint_camera.camera_center
         ob_view = ob_view / ob_view.norm(dim=1, keepdim=True)
@@ -147,5 +164,5 @@ def generate_neural_gaussians(viewpoint_camera, pc, visible_mask=None, is_traini
         W1 = color_mlp[0]
         color_mlp = (W1[:, :35].contiguous(), color_mlp[1] + W1[:, 35:] @ row, color_mlp[2], color_mlp[3])
     out = neural_gaussians(anchor, feat, offsets, scaling, viewpoint_camera.camera_center,
-                           _linear_pair(pc.get_opacity_mlp), color_mlp, _linear_pair(pc.get_cov_mlp))
+                           _linear_pair(pc.get_opacity_mlp), color_mlp, _linear_pair(pc.get_cov_mlp), opacity_scale)
     return out if is_training else out[:5]

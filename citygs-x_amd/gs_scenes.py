@@ -212,15 +212,19 @@ def make_anchor_scene(N, k=10, seed=0, feat_dim=32):
     return {"anchor": anchor, "feat": feat, "offsets": offsets, "scaling": scaling, "campos": campos, "mlps": mlps}
 
 
-def neural_gaussians_torch(anchor, feat, offsets, scaling, campos, mlps):
+def neural_gaussians_torch(anchor, feat, offsets, scaling, campos, mlps, prog=None):
     """generate_neural_gaussians (gaussian_renderer/__init__.py:789-899) in its default configuration, with
-    torch operations in the dtype of its inputs: the comparison the fused operator is measured against."""
+    torch operations in the dtype of its inputs: the comparison the fused operator is measured against.  prog
+    (N, 1), if given, is the factor dist2level 'progressive' puts on the opacity (:844-848)."""
     k = offsets.shape[1]
     ob_view = anchor - campos
     ob_view = ob_view / ob_view.norm(dim=1, keepdim=True)
     x = torch.cat([feat, ob_view], dim=1)
     run = lambda m: torch.relu(x @ m[0].t() + m[1]) @ m[2].t() + m[3]
-    neural_opacity = torch.tanh(run(mlps[0])).reshape(-1, 1)
+    neural_opacity = torch.tanh(run(mlps[0]))
+    if prog is not None:
+        neural_opacity = neural_opacity * prog
+    neural_opacity = neural_opacity.reshape(-1, 1)
     mask = (neural_opacity > 0.0).view(-1)
     opacity = neural_opacity[mask]
     color = torch.sigmoid(run(mlps[1])).reshape(-1, 3)

@@ -187,6 +187,9 @@ int gs_all_map_backward(int P, const float* means3D, const float* scales, const 
  * Tanh), mlp_color (3 n_offsets, Sigmoid) and mlp_cov (7 n_offsets), as nn.Linear stores them
  * (scene/gaussian_model.py:131-149).  anchor (N,3), feat (N,32), offsets (N,n_offsets,3), scaling (N,6) = the
  * activated get_scaling, campos (3).  n_offsets must satisfy gs_neural_supported().
+ * opacity_scale (N floats, or NULL for none) serves dist2level 'progressive' (:844-848): neural_opacity =
+ * mlp_opacity(x) * opacity_scale[anchor], where the caller passes _prog_ratio with 1 for the anchors outside
+ * transition_mask; it must be positive wherever the product is (the reference's lies in (0, 1]).
  *
  * Step 1, gs_neural_opacity_forward: writes neural_opacity (N*n_offsets), mask (u8, N*n_offsets) and
  * first (u32, N: selected offsets of all earlier anchors), and returns their number in *num_selected (the host
@@ -201,9 +204,9 @@ int gs_all_map_backward(int P, const float* means3D, const float* scales, const 
 int gs_neural_supported(int n_offsets);
 size_t gs_neural_workspace_bytes(int64_t num_anchors, int n_offsets);
 int gs_neural_opacity_forward(int64_t num_anchors, int n_offsets, const float* anchor, const float* feat,
-                              const float* campos, const float* const* mlp_params, float* neural_opacity,
-                              uint8_t* mask, uint32_t* first, void* workspace, size_t workspace_bytes,
-                              int64_t* num_selected, gs_stream_t stream);
+                              const float* campos, const float* const* mlp_params, const float* opacity_scale,
+                              float* neural_opacity, uint8_t* mask, uint32_t* first, void* workspace,
+                              size_t workspace_bytes, int64_t* num_selected, gs_stream_t stream);
 int gs_neural_gaussians_forward(int64_t num_anchors, int n_offsets, int64_t num_selected, const float* anchor,
                                 const float* feat, const float* offsets, const float* scaling, const float* campos,
                                 const float* neural_opacity, const uint32_t* first, const void* workspace,
@@ -212,11 +215,12 @@ int gs_neural_gaussians_forward(int64_t num_anchors, int n_offsets, int64_t num_
 size_t gs_neural_backward_workspace_bytes(int64_t num_anchors, int n_offsets);
 int gs_neural_backward(int64_t num_anchors, int n_offsets, int64_t num_selected, const float* anchor,
                        const float* feat, const float* offsets, const float* scaling, const float* campos,
-                       const float* const* mlp_params, const float* neural_opacity, const uint32_t* first,
-                       const float* color, const float* rot, const float* aux, const float* dL_dxyz,
-                       const float* dL_dcolor, const float* dL_dopacity, const float* dL_dscaling,
-                       const float* dL_drot, float* d_anchor, float* d_feat, float* d_offsets, float* d_scaling,
-                       float* const* d_mlp_params, void* workspace, size_t workspace_bytes, gs_stream_t stream);
+                       const float* const* mlp_params, const float* opacity_scale, const float* neural_opacity,
+                       const uint32_t* first, const float* color, const float* rot, const float* aux,
+                       const float* dL_dxyz, const float* dL_dcolor, const float* dL_dopacity,
+                       const float* dL_dscaling, const float* dL_drot, float* d_anchor, float* d_feat,
+                       float* d_offsets, float* d_scaling, float* const* d_mlp_params, void* workspace,
+                       size_t workspace_bytes, gs_stream_t stream);
 
 /* Replaces pixelwise_l1_with_mask and pixelwise_ssim_with_mask (utils/loss_utils.py:88-132, 11x11 Gaussian
  * window of create_window :27-43, zero padding; called at gaussian_renderer/loss_distribution.py:267-279).

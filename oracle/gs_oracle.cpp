@@ -1338,6 +1338,8 @@ void oracle_ssim_l1_bwd(int C, int H, int W, const float* img1, const float* img
 // appearance embedding, no distance / level inputs, dist2level 'round'): per visible anchor
 //   x = [feat(32), (anchor - campos)/|anchor - campos| (3)]
 //   neural_opacity = tanh(W2o relu(W1o x + b1o) + b2o)            (k values)       :841-853
+//     (dist2level 'progressive': times prog, the anchor's _prog_ratio or 1 outside transition_mask, :844-848;
+//      prog = NULL stands for no factor)
 //   color = sigmoid(W2c relu(W1c x + b1c) + b2c)                  (k x 3)          :866-870
 //   scale_rot = W2v relu(W1v x + b1v) + b2v                       (k x 7)          :873-877
 // and for every (anchor, offset) with neural_opacity > 0, in that order (:856-858, :886):
@@ -1377,7 +1379,8 @@ void oracle_neural_mlp_fwd(int N, int k, const float* anchor, const float* feat,
                            const float* W1o, const float* b1o, const float* W2o, const float* b2o,
                            const float* W1c, const float* b1c, const float* W2c, const float* b2c,
                            const float* W1v, const float* b1v, const float* W2v, const float* b2v,
-                           float* neural_opacity, uint8_t* mask, float* color, float* scale_rot) {
+                           const float* prog, float* neural_opacity, uint8_t* mask, float* color,
+                           float* scale_rot) {
   const MlpView mo{W1o, b1o, W2o, b2o, k}, mc{W1c, b1c, W2c, b2c, 3 * k}, mv{W1v, b1v, W2v, b2v, 7 * k};
 #pragma omp parallel for schedule(static)
   for (int a = 0; a < N; a++) {
@@ -1386,7 +1389,7 @@ void oracle_neural_mlp_fwd(int N, int k, const float* anchor, const float* feat,
     std::vector<float> out(7 * k);
     mlp_forward(mo, x, hid, out.data());
     for (int j = 0; j < k; j++) {
-      const float t = tanhf(out[j]);
+      const float t = prog ? tanhf(out[j]) * prog[a] : tanhf(out[j]);
       neural_opacity[(size_t)a * k + j] = t;
       mask[(size_t)a * k + j] = t > 0.f;
     }
@@ -1430,7 +1433,7 @@ void oracle_neural_bwd(int N, int k, const float* anchor, const float* feat, con
                        const float* scaling, const float* campos,
                        const float* W1o, const float* b1o, const float* W2o, const float* b2o,
                        const float* W1c, const float* b1c, const float* W2c, const float* b2c,
-                       const float* W1v, const float* b1v, const float* W2v, const float* b2v,
+                       const float* W1v, const float* b1v, const float* W2v, const float* b2v, const float* prog,
                        const float* g_xyz, const float* g_col, const float* g_opacity, const float* g_scal,
                        const float* g_rot, float* d_anchor, float* d_feat, float* d_offsets, float* d_scaling,
                        float* dW1o, float* db1o, float* dW2o, float* db2o, float* dW1c, float* db1c, float* dW2c,
@@ -1460,10 +1463,12 @@ void oracle_neural_bwd(int N, int k, const float* anchor, const float* feat, con
     for (int j = 0; j < k; j++) {
       const size_t s = (size_t)a * k + j;
       for (int c = 0; c < 3; c++) d_offsets[3 * s + c] = 0.f;
-      const float t = tanhf(out[0][j]);
+      const float th = tanhf(out[0][j]);
+      const float pf = prog ? prog[a] : 1.0f;
+      const float t = prog ? th * pf : th;
       if (!(t > 0.f)) continue;
-      // opacity = tanh(pre)
-      gout[0][j] = g_opacity[r] * (1.0f - t * t);
+      // opacity = tanh(pre) * prog
+      gout[0][j] = g_opacity[r] * ((1.0f - th * th) * pf);
       for (int c = 0; c < 3; c++) {
         const float cs = 1.0f / (1.0f + expf(-out[1][3 * j + c]));
         gout[1][3 * j + c] = g_col[3 * r + c] * (cs * (1.0f - cs));

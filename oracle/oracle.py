@@ -417,17 +417,19 @@ def _mlp_args(mlps):
     return flat
 
 
-def neural_gaussians_fwd(anchor, feat, offsets, scaling, campos, mlps):
+def neural_gaussians_fwd(anchor, feat, offsets, scaling, campos, mlps, prog=None):
     """generate_neural_gaussians (gaussian_renderer/__init__.py:789-899), default configuration, on the anchors
-    already selected by visible_mask.  Returns (xyz, color, opacity, scaling, rot, neural_opacity, mask)."""
+    already selected by visible_mask; prog (N), if given, is the per-anchor factor of dist2level 'progressive'
+    (:844-848).  Returns (xyz, color, opacity, scaling, rot, neural_opacity, mask)."""
     anchor, feat, offsets, scaling = _f32(anchor), _f32(feat), _f32(offsets), _f32(scaling)
     cp = _f32(campos).reshape(3)
     N, k = anchor.shape[0], offsets.shape[1]
     w = _mlp_args(mlps)
     nop, mask = np.zeros((N * k, 1), np.float32), np.zeros(N * k, np.uint8)
     col, sr = np.zeros((N * k, 3), np.float32), np.zeros((N * k, 7), np.float32)
-    lib().oracle_neural_mlp_fwd(C.c_int(N), C.c_int(k), _p(anchor), _p(feat), _p(cp), *[_p(x) for x in w], _p(nop),
-                                _p(mask), _p(col), _p(sr))
+    pg = None if prog is None else _f32(prog).reshape(N)
+    lib().oracle_neural_mlp_fwd(C.c_int(N), C.c_int(k), _p(anchor), _p(feat), _p(cp), *[_p(x) for x in w],
+                                None if pg is None else _p(pg), _p(nop), _p(mask), _p(col), _p(sr))
     S = int(mask.sum())
     xyz, c, op = np.zeros((S, 3), np.float32), np.zeros((S, 3), np.float32), np.zeros((S, 1), np.float32)
     sc, rot = np.zeros((S, 3), np.float32), np.zeros((S, 4), np.float32)
@@ -438,7 +440,8 @@ def neural_gaussians_fwd(anchor, feat, offsets, scaling, campos, mlps):
     return xyz, c, op, sc, rot, nop, mask.astype(bool)
 
 
-def neural_gaussians_bwd(anchor, feat, offsets, scaling, campos, mlps, g_xyz, g_color, g_opacity, g_scaling, g_rot):
+def neural_gaussians_bwd(anchor, feat, offsets, scaling, campos, mlps, g_xyz, g_color, g_opacity, g_scaling, g_rot,
+                         prog=None):
     """Gradients of neural_gaussians_fwd's five compacted outputs: (d_anchor, d_feat, d_offsets, d_scaling,
     [12 weight gradients in the order of mlps])."""
     anchor, feat, offsets, scaling = _f32(anchor), _f32(feat), _f32(offsets), _f32(scaling)
@@ -449,7 +452,8 @@ def neural_gaussians_bwd(anchor, feat, offsets, scaling, campos, mlps, g_xyz, g_
     da, df = np.zeros((N, 3), np.float32), np.zeros((N, 32), np.float32)
     do, ds = np.zeros((N, k, 3), np.float32), np.zeros((N, 6), np.float32)
     dw = [np.zeros_like(x) for x in w]
+    pg = None if prog is None else _f32(prog).reshape(N)
     lib().oracle_neural_bwd(C.c_int(N), C.c_int(k), _p(anchor), _p(feat), _p(offsets), _p(scaling), _p(cp),
-                            *[_p(x) for x in w], *[_p(x) for x in gs], _p(da), _p(df), _p(do), _p(ds),
+                            *[_p(x) for x in w], None if pg is None else _p(pg), *[_p(x) for x in gs], _p(da), _p(df), _p(do), _p(ds),
                             *[_p(x) for x in dw])
     return da, df, do, ds, dw

@@ -70,6 +70,41 @@ def test_forward_and_backward_match_oracle(orc, N, k, seed):
         assert _rel(t.grad.cpu().numpy(), w) <= 2e-5, i
 
 
+def _prog(N, seed):
+    gen = torch.Generator().manual_seed(100 + seed)
+    prog = torch.rand(N, 1, generator=gen) * 0.98 + 0.01
+    prog[torch.rand(N, generator=gen) < 0.4] = 1.0
+    prog[torch.rand(N, generator=gen) < 0.1] = 0.0
+    return prog
+
+
+@pytest.mark.parametrize("N,k,seed", [(700, 10, 20), (45, 5, 21), (130, 16, 22)])
+def test_progressive_opacity_factor_matches_oracle(orc, N, k, seed):
+    """dist2level 'progressive' (gaussian_renderer/__init__.py:844-848): a per-anchor factor on the opacity."""
+    from gs_neural import neural_gaussians
+    s = gs_scenes.make_anchor_scene(N, k, seed)
+    prog = _prog(N, seed)
+    anchor, feat, offsets, scaling, campos, mlps = _to_dev(s, grad=True)
+    out = neural_gaussians(anchor, feat, offsets, scaling, campos, *mlps, opacity_scale=prog.reshape(-1).to(DEV))
+    want = orc.neural_gaussians_fwd(*_np_args(s), prog=prog.numpy())
+    got = [o.detach().cpu().numpy() for o in out]
+    assert np.abs(got[5] - want[5]).max() <= 2e-6
+    assert np.array_equal(got[6], want[6])
+    assert not got[6].reshape(N, k)[prog.numpy().ravel() == 0].any()
+    for g, w in zip(got[:5], want[:5]):
+        assert _rel(g, w) <= 5e-6
+    S = int(got[6].sum())
+    gen = torch.Generator().manual_seed(seed)
+    ups = [torch.randn(S, c, generator=gen) for c in (3, 3, 1, 3, 4)]
+    sum((o * u.to(DEV)).sum() for o, u in zip(out[:5], ups)).backward()
+    wd = orc.neural_gaussians_bwd(*_np_args(s), *[u.numpy() for u in ups], prog=prog.numpy())
+    for name, t, w in zip(("anchor", "feat", "offsets", "scaling"), (anchor, feat, offsets, scaling), wd[:4]):
+        assert _rel(t.grad.cpu().numpy(), w) <= 1e-5, name
+    flat = [x for m in mlps for x in m]
+    for i, (t, w) in enumerate(zip(flat, wd[4])):
+        assert _rel(t.grad.cpu().numpy(), w) <= 2e-5, i
+
+
 def test_no_anchor_and_nothing_selected():
     from gs_neural import neural_gaussians
     s = gs_scenes.make_anchor_scene(50, 10, 0)
@@ -154,6 +189,26 @@ def test_drop_in_signature():
         for lin in (q[0], q[2]):
             assert bool(torch.isfinite(lin.weight.grad).all()) and float(lin.weight.grad.abs().max()) > 0.0
     assert float(pc.get_opacity_mlp[2].weight.grad.abs().max()) == 0.0
+    # dist2level 'progressive': the model's ratio where transition_mask is set, 1 elsewhere (:844-848)
+    pc.dist2level = "progressive"
+    pc._prog_ratio = _prog(N, 1).to(DEV).clamp_min(0.01)
+    pc.transition_mask = (torch.rand(N, generator=torch.Generator().manual_seed(2)) < 0.5).to(DEV)
+    prog = pc._prog_ratio[vis].clone()
+    prog[~pc.transition_mask[vis]] = 1.0
+    out = generate_neural_gaussians(cam, pc, vis, is_training=True)
+    ref = gs_scenes.neural_gaussians_torch(pc.get_anchor[vis], pc.get_anchor_feat[vis], pc._offset[vis],
+                                           pc.get_scaling[vis], cam.camera_center,
+                                           [tuple(x.to(DEV) for x in m) for m in s["mlps"]], prog)
+    assert torch.equal(out[6], ref[6])
+    for o, r in zip(out[:6], ref[:6]):
+        assert float((o - r).norm() / r.norm()) <= 5e-6
+    # and without a visibility mask
+    out = generate_neural_gaussians(cam, pc, None, is_training=True)
+    full = torch.where(pc.transition_mask[:, None], pc._prog_ratio, torch.ones_like(pc._prog_ratio))
+    ref = gs_scenes.neural_gaussians_torch(pc.get_anchor, pc.get_anchor_feat, pc._offset, pc.get_scaling,
+                                           cam.camera_center, [tuple(x.to(DEV) for x in m) for m in s["mlps"]], full)
+    assert torch.equal(out[6], ref[6])
+    assert float((out[5] - ref[5]).norm() / ref[5].norm()) <= 5e-6
     pc.add_cov_dist = True
     with pytest.raises(NotImplementedError):
         generate_neural_gaussians(cam, pc, vis)

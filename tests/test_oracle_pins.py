@@ -723,6 +723,47 @@ def test_neural_gaussians_backward_matches_float64_autograd(orc, N, k, seed):
         assert _rel(g, w.grad.numpy()) < 1e-5, i
 
 
+def _prog(N, seed):
+    """Per-anchor opacity factor as dist2level 'progressive' builds it: a ratio in (0, 1), 1 outside the transition
+    mask, and a few anchors switched off altogether (ratio 0)."""
+    gen = torch.Generator().manual_seed(100 + seed)
+    prog = torch.rand(N, 1, generator=gen) * 0.98 + 0.01
+    prog[torch.rand(N, generator=gen) < 0.4] = 1.0
+    prog[torch.rand(N, generator=gen) < 0.1] = 0.0
+    return prog
+
+
+@pytest.mark.parametrize("N,k,seed", [(193, 10, 6), (40, 5, 7)])
+def test_neural_gaussians_progressive_factor_matches_float64_torch(orc, N, k, seed):
+    """The factor scales the dense opacity and the selected one, switches an anchor with ratio 0 off, and reaches
+    the opacity MLP's gradients and nothing else (gaussian_renderer/__init__.py:844-848)."""
+    s, args = _anchor_scene_np(N, k, seed)
+    prog = _prog(N, seed)
+    plain = orc.neural_gaussians_fwd(*args)
+    fwd = orc.neural_gaussians_fwd(*args, prog=prog.numpy())
+    assert np.allclose(fwd[5].reshape(N, k), plain[5].reshape(N, k) * prog.numpy(), rtol=1e-6, atol=0)
+    assert np.array_equal(fwd[6].reshape(N, k), plain[6].reshape(N, k) & (prog.numpy() > 0))
+    assert not fwd[6].reshape(N, k)[prog.numpy().ravel() == 0].any()
+    S = fwd[0].shape[0]
+    gen = torch.Generator().manual_seed(seed)
+    ups = [torch.randn(S, c, generator=gen) for c in (3, 3, 1, 3, 4)]
+    got = orc.neural_gaussians_bwd(*args, *[u.numpy() for u in ups], prog=prog.numpy())
+    leaf = lambda t: t.double().requires_grad_(True)
+    anchor, feat, offsets, scaling = leaf(s["anchor"]), leaf(s["feat"]), leaf(s["offsets"]), leaf(s["scaling"])
+    mlps = [tuple(leaf(x) for x in m) for m in s["mlps"]]
+    out = gs_scenes.neural_gaussians_torch(anchor, feat, offsets, scaling, s["campos"].double(), mlps, prog.double())
+    assert np.array_equal(out[6].numpy(), fwd[6])
+    for g, w in zip(fwd[:6], out[:6]):
+        assert _rel(g, w.detach().numpy()) < 2e-6
+    loss = sum((o * u.double()).sum() for o, u in zip(out[:5], ups))
+    loss.backward()
+    for name, g, w in zip(("anchor", "feat", "offsets", "scaling"), got[:4], (anchor, feat, offsets, scaling)):
+        assert _rel(g, w.grad.numpy()) < 1e-5, name
+    flat = [x for m in mlps for x in m]
+    for i, (g, w) in enumerate(zip(got[4], flat)):
+        assert _rel(g, w.grad.numpy()) < 1e-5, i
+
+
 # ------------------------------------------------------ max-weight depth --
 
 def test_max_weight_depth_known_cases(orc):
