@@ -138,6 +138,61 @@ def test_config1_full_size(H):
     assert float(pb[3][dead].abs().max()) == 0.0  # dL/dshs of culled Gaussians
 
 
+@pytest.mark.parametrize("cfg,P", [(1, 1_000_000), (3, 10_000_000)])
+def test_list_routes_agree_at_full_size(H, cfg, P):
+    """The per-tile lists at BASELINE sizes (config 1; config 3: 10 M Gaussians, 1920x1080, street level, lists of
+    more than 8192 records) come out the same bit for bit by the radix sort over all keys (checked against numpy at
+    small sizes and through its properties at large ones), by the per-tile sort, and by the per-tile sort with
+    every long list cut into chunks and merged."""
+    import gs_scenes
+    import gsrast_native as gn
+    from diff_gaussian_rasterization import _C
+    g, cams = gs_scenes.make_scene(cfg, P=P, n_views=1)
+    cam = cams[0]
+    W, Hh = cam.image_width, cam.image_height
+    d = {k: v.to(DEV) for k, v in g.items() if torch.is_tensor(v)}
+    vm, pm, cp = cam.world_view_transform.to(DEV), cam.full_proj_transform.to(DEV), cam.camera_center.to(DEV)
+    args = {"stats_collector": {}}
+    _, means2D, depths, radii, cov3D, co, rgb, clamped = _C.preprocess_gaussians(
+        d["means3D"], d["scales"], d["rotations"], d["shs"], d["opacities"], 1.0, vm, pm, cam.tanfovx, cam.tanfovy,
+        Hh, W, 3, cp, False, False, args)
+    del d
+    am = torch.zeros(P, 5, device=DEV)
+    gx, gy = (W + 15) // 16, (Hh + 15) // 16
+    T = gx * gy
+    cl = torch.ones(gy, gx, dtype=torch.bool, device=DEV)
+    results = []
+    try:
+        for limits in [(1, 0, 0), (1, 8192, 0), (1, 8192, 1 << 30), (0, 2048, 1 << 30)]:
+            gn.lib.gs_set_tile_sort_limits(*limits)
+            out = _C.render_gaussians(torch.zeros(3, device=DEV), Hh, W, means2D, depths, radii, co, rgb, cl, vm, cp,
+                                      cam.tanfovx, cam.tanfovy, am, False, False, args)
+            R, color, n_render, binB, imgB = out[0], out[1], out[2], out[9], out[10]
+            off = [C.c_size_t() for _ in range(5)]
+            gn.check(gn.lib.gs_binning_state_layout(R, W, Hh, *[C.byref(o) for o in off]), "layout")
+            base = (binB.data_ptr() + 255) // 256 * 256 - binB.data_ptr()
+            point_list = binB[base + off[0].value: base + off[0].value + 4 * R].view(torch.int32).clone()
+            keys = binB[base + off[1].value: base + off[1].value + 8 * R].view(torch.int64).clone()
+            ioff = [C.c_size_t() for _ in range(5)]
+            gn.check(gn.lib.gs_image_state_layout(W, Hh, *[C.byref(o) for o in ioff]), "layout")
+            ibase = (imgB.data_ptr() + 255) // 256 * 256 - imgB.data_ptr()
+            ranges = imgB[ibase + ioff[3].value: ibase + ioff[3].value + 8 * T].view(torch.int32).clone()
+            results.append((limits, R, keys, point_list, ranges, color.clone(), n_render.clone()))
+            del out, binB, imgB
+    finally:
+        gn.lib.gs_set_tile_sort_limits(1, 8192, 32)
+    _, R0, keys0, pl0, ranges0, color0, nr0 = results[0]
+    assert R0 > 1_000_000
+    if cfg == 3:
+        assert int(nr0.max()) > 8192  # so that the third and fourth settings really merge chunks
+    for limits, R, keys, pl, ranges, color, nr in results[1:]:
+        assert R == R0, limits
+        assert torch.equal(ranges, ranges0), limits
+        assert torch.equal(keys, keys0), limits
+        assert torch.equal(pl, pl0), limits
+        assert torch.equal(nr, nr0) and torch.equal(color, color0), limits
+
+
 def test_knn_large_against_brute_force_on_a_sample():
     """distCUDA2 on 3 M points; 512 of them checked against an exhaustive search done with torch."""
     from simple_knn._C import distCUDA2
