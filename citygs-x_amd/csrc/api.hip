@@ -473,11 +473,15 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
     longest = __atomic_load_n(total_slot + 1, __ATOMIC_ACQUIRE);
     chunks = __atomic_load_n(total_slot + 2, __ATOMIC_ACQUIRE);
   } else {
+    uint32_t wrapped = 0;
     GS_HIP_TRY(hipMemcpyAsync(&R_u, point_offsets + (P - 1), sizeof(uint32_t), hipMemcpyDeviceToHost, stream));
+    GS_HIP_TRY(hipMemcpyAsync(&wrapped, scan_overflow_word(scan_temp, P), sizeof(uint32_t), hipMemcpyDeviceToHost,
+                              stream));
     GS_HIP_TRY(hipStreamSynchronize(stream));
+    if (wrapped != 0u) R_u = GS_TOO_MANY_INSTANCES;
   }
-  if (R_u >= 0x7FFFFFFFu) {
-    set_error("gs_render_forward: %u (Gaussian, tile) instances exceed the supported 2^31-2", R_u);
+  if (R_u > GS_MAX_INSTANCES) {
+    set_error("gs_render_forward: more than 2^31-2 (Gaussian, tile) instances in one view");
     return 1;
   }
   const int64_t R = (int64_t)R_u;

@@ -89,16 +89,30 @@ scan_block_sums_kernel(int64_t n, const T* __restrict__ in, uint32_t* __restrict
 }
 
 // One block turns the per-tile sums into exclusive prefixes in place.
+// block_sums[nblocks] receives 1 if the exact grand total exceeds GS_MAX_INSTANCES (the 32-bit sums wrap
+// around), else 0.  A block's own sum is taken as exact: it covers SCAN_TILE elements.
 __global__ void __launch_bounds__(1024) scan_spine_kernel(int nblocks, uint32_t* __restrict__ block_sums) {
   __shared__ uint32_t s_wave[1024 / GS_WAVE];
+  __shared__ double s_exact[1024 / GS_WAVE];
   uint32_t carry = 0;
+  double exact = 0.0;
   for (int start = 0; start < nblocks; start += 1024) {
     const int idx = start + threadIdx.x;
     const uint32_t v = idx < nblocks ? block_sums[idx] : 0u;
+    exact += (double)v;
     uint32_t total;
     const uint32_t ex = block_exclusive_scan<1024>(v, s_wave, total);
     if (idx < nblocks) block_sums[idx] = carry + ex;
     carry += total;
+  }
+#pragma unroll
+  for (int d = GS_WAVE / 2; d >= 1; d >>= 1) exact += __shfl_xor(exact, d, GS_WAVE);
+  if ((threadIdx.x & (GS_WAVE - 1)) == 0) s_exact[threadIdx.x / GS_WAVE] = exact;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    double all = 0.0;
+    for (int w = 0; w < 1024 / GS_WAVE; w++) all += s_exact[w];
+    block_sums[nblocks] = all > (double)GS_MAX_INSTANCES ? 1u : 0u;
   }
 }
 
@@ -132,7 +146,8 @@ scan_apply_kernel(int64_t n, const T* in, const uint32_t* __restrict__ block_pre
   // The owner of the last element also hands the grand total to the host, which may be polling this word
   // (host-visible memory), so the store is made visible system wide.
   if (total_out != nullptr && n - 1 >= base && n - 1 < base + SCAN_ITEMS)
-    __hip_atomic_store(total_out, run, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    __hip_atomic_store(total_out, block_prefix[gridDim.x] != 0u ? GS_TOO_MANY_INSTANCES : run, __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_SYSTEM);
 }
 
 // cuda_rasterizer/rasterizer_impl.cu:74-117.
@@ -211,7 +226,12 @@ int launch_tile_count(int P, int W, int H, const int* radii, const float* means2
 
 size_t scan_temp_bytes(int64_t n) {
   const int64_t nb = (n + SCAN_TILE - 1) / SCAN_TILE;
-  return align_up((size_t)(nb > 0 ? nb : 1) * sizeof(uint32_t), 256);
+  return align_up((size_t)((nb > 0 ? nb : 1) + 1) * sizeof(uint32_t), 256);  // block sums and the overflow word
+}
+
+const uint32_t* scan_overflow_word(const void* temp, int64_t n) {
+  const int64_t nb = (n + SCAN_TILE - 1) / SCAN_TILE;
+  return (const uint32_t*)temp + (nb > 0 ? nb : 1);
 }
 
 template <typename T>

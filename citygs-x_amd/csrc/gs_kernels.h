@@ -45,13 +45,20 @@ int launch_visible_filter(int P, const float* means, const float* scales, float 
 int launch_mark_visible(int P, const float* means, const float* V, uint8_t* present, hipStream_t stream);
 
 // ---- binning ----
+// (Gaussian, tile) instances a view may have (positions are 32-bit, counts are handed to the caller as int), and
+// the count the kernels report in place of a larger, wrapped-around one
+constexpr uint32_t GS_MAX_INSTANCES = 0x7FFFFFFEu;
+constexpr uint32_t GS_TOO_MANY_INSTANCES = 0x7FFFFFFFu;
 int launch_tile_count(int P, int W, int H, const int* radii, const float* means2D, const uint8_t* compute_locally,
                       uint32_t* tiles_touched, hipStream_t stream,
                       uint32_t* zero_words = nullptr, int64_t zero_count = 0);
 size_t scan_temp_bytes(int64_t n);
+// device word of a scan's workspace that is 1 after a scan whose exact total exceeds GS_MAX_INSTANCES, else 0
+const uint32_t* scan_overflow_word(const void* temp, int64_t n);
 int launch_exclusive_sum_u8(int64_t n, const uint8_t* in, uint32_t* out, void* temp, hipStream_t stream,
                             uint32_t* total_out = nullptr);
-// total_out, when given, is a host-visible word that receives the grand total as well
+// total_out, when given, is a host-visible word that receives the grand total as well (GS_TOO_MANY_INSTANCES if
+// the exact total exceeds GS_MAX_INSTANCES; the 32-bit sums themselves wrap around like the reference's)
 int launch_inclusive_sum(int64_t n, const uint32_t* in, uint32_t* out, void* temp, hipStream_t stream,
                          uint32_t* total_out = nullptr);
 int launch_exclusive_sum(int64_t n, const uint32_t* in, uint32_t* out, void* temp, hipStream_t stream);

@@ -133,11 +133,14 @@ __global__ void __launch_bounds__(1024)
 bucket_ranges_kernel(uint32_t T, uint32_t limit, const uint32_t* __restrict__ totals, uint32_t* __restrict__ ranges,
                      uint32_t* __restrict__ chunk_first, uint32_t* __restrict__ host_words) {
   __shared__ uint32_t s_wave[16], s_wave_chunks[16], s_max[16];
+  __shared__ double s_exact[16];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   uint32_t carry = 0, carry_chunks = 0, longest = 0;
+  double exact = 0.0;  // the number of instances without the 32-bit wrap-around of the prefix sums
   for (uint32_t start = 0; start < T; start += 1024) {
     const uint32_t t = start + threadIdx.x;
     const uint32_t v = t < T ? totals[t] : 0u;
+    exact += (double)v;
     const uint32_t c = v > limit ? (v + limit - 1u) / limit : 0u;
     longest = v > longest ? v : longest;
     const uint32_t inc = wave_inclusive_scan_u32(v, lane);
@@ -173,15 +176,26 @@ bucket_ranges_kernel(uint32_t T, uint32_t limit, const uint32_t* __restrict__ to
     const uint32_t o = __shfl_xor(longest, d, GS_WAVE);
     longest = o > longest ? o : longest;
   }
-  if (lane == 0) s_max[wave] = longest;
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) exact += __shfl_xor(exact, d, GS_WAVE);
+  if (lane == 0) {
+    s_max[wave] = longest;
+    s_exact[wave] = exact;
+  }
   __syncthreads();
   if (threadIdx.x == 0) {
     uint32_t m = 0;
-    for (int w = 0; w < 16; w++) m = s_max[w] > m ? s_max[w] : m;
+    double all = 0.0;
+    for (int w = 0; w < 16; w++) {
+      m = s_max[w] > m ? s_max[w] : m;
+      all += s_exact[w];
+    }
     chunk_first[T] = carry_chunks;
+    // more instances than 32-bit positions can address: the host must not go on with the wrapped count
+    const uint32_t reported = all > (double)GS_MAX_INSTANCES ? GS_TOO_MANY_INSTANCES : carry;
     __hip_atomic_store(host_words + 1, m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
     __hip_atomic_store(host_words + 2, carry_chunks, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-    __hip_atomic_store(host_words, carry, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+    __hip_atomic_store(host_words, reported, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
   }
 }
 

@@ -129,7 +129,7 @@ def test_training_size_against_torch_statements():
     a2 = _to_dev(s, grad=True)
     out = neural_gaussians(*a1[:5], *a1[5])
     ref = gs_scenes.neural_gaussians_torch(*a2)
-    assert float((out[5] - ref[5]).abs().max()) <= 5e-6
+    assert float((out[5] - ref[5]).detach().abs().max()) <= 5e-6
     differ = out[6] != ref[6]
     assert int(differ.sum()) <= 20 and float(ref[5].view(-1)[differ].abs().max().item() if differ.any() else 0.0) <= 5e-6
     both = out[6] & ref[6]

@@ -217,3 +217,69 @@ def test_preprocess_backward(H, orc, cfg, P, sh_mode):
         assert np.isfinite(a).all(), k
         assert H.rel_l2(a, r) <= GRAD_TOL, f"{k}: rel L2 {H.rel_l2(a, r)}"
         assert np.array_equal(a, r) or H.rel_l2(a, r) < 1e-6, f"{k} drifted from the op-for-op statement"
+
+
+def _poison(g, seed=0):
+    """Non-finite and absurd parameters in 2 % of the Gaussians (what a diverged optimisation hands the rasterizer)."""
+    P = g["means3D"].shape[0]
+    gen = torch.Generator().manual_seed(seed)
+    idx = torch.randperm(P, generator=gen)[: P // 50].reshape(10, -1)
+    nan, inf = float("nan"), float("inf")
+    g["means3D"][idx[0], 0] = nan
+    g["means3D"][idx[1], 2] = inf
+    g["means3D"][idx[2]] = -inf
+    g["scales"][idx[3], 1] = nan
+    g["scales"][idx[4]] = inf
+    g["scales"][idx[5]] = 1e20
+    g["scales"][idx[6], 0] = -3.0
+    g["rotations"][idx[7], 2] = nan
+    g["rotations"][idx[8]] = 0.0
+    g["opacities"][idx[9]] = nan
+    return idx.reshape(-1)
+
+
+@pytest.mark.parametrize("cfg,P", [(0, 40_000), (1, 100_000)])
+def test_non_finite_parameters_are_contained(H, orc, cfg, P):
+    """NaN, infinite and absurd means, scales, rotations and opacities: every kernel finishes, the integer outputs
+    are the oracle's (a Gaussian whose radius or rectangle cannot be computed is culled, as by the saturating
+    casts of cuda_rasterizer/auxiliary.h:66-76), and whatever the other Gaussians contribute stays finite."""
+    import gs_scenes
+    from diff_gaussian_rasterization import _C
+    DEV = H.DEV
+    g, cam = _scene(cfg, P)
+    bad = _poison(g)
+    got, gd = H.preprocess_fwd(g, cam)
+    ref = H.oracle_preprocess(orc, g, cam)
+    assert np.array_equal(got["radii"].cpu().numpy(), ref["radii"])
+    assert np.array_equal(H.np_u32(got["tiles_touched"]), ref["tiles_touched"])
+    radii = got["radii"]
+    W, Hh = cam.image_width, cam.image_height
+    gx, gy = H.grid(W, Hh)
+    assert int(got["tiles_touched"].max()) <= gx * gy
+    good = torch.ones(P, dtype=torch.bool)
+    good[bad] = False
+    good = good.to(DEV)
+    for k in ("means2D", "depths", "conic_opacity", "rgb"):
+        assert bool(torch.isfinite(got[k][good & (radii > 0)]).all()), k
+    # lists and blending: same lists as the oracle builds from the same per-Gaussian outputs
+    cl = torch.ones(gy, gx, dtype=torch.bool)
+    n = lambda t: t.detach().cpu().numpy()
+    want = orc.bin_and_sort(n(radii), n(got["means2D"]), n(got["depths"]), cl.numpy().reshape(-1), W, Hh)
+    vm, cp = cam.world_view_transform.to(DEV), cam.camera_center.to(DEV)
+    am = torch.zeros(P, 5, device=DEV)
+    args = {"stats_collector": {}}
+    out = _C.render_gaussians(torch.zeros(3, device=DEV), Hh, W, got["means2D"], got["depths"], radii,
+                              got["conic_opacity"], got["rgb"], cl.to(DEV), vm, cp, cam.tanfovx, cam.tanfovy, am,
+                              True, False, args)
+    R, color, n_render, oam, geomB, binB, imgB = out[0], out[1], out[2], out[6], out[8], out[9], out[10]
+    assert R == want["point_list"].shape[0]
+    counts = want["ranges"].reshape(-1, 2).astype(np.int64)
+    assert np.array_equal(n(n_render), (counts[:, 1] - counts[:, 0]).astype(np.int32))
+    ug = gs_scenes.upstream_grads(cam)
+    back = _C.render_gaussians_backward(torch.zeros(3, device=DEV), cam.tanfovx, cam.tanfovy, oam, am, R, geomB, binB,
+                                        imgB, cl.to(DEV), ug["color"].to(DEV), ug["all_map"].to(DEV),
+                                        ug["plane_depth"].to(DEV), got["means2D"], got["conic_opacity"], got["rgb"],
+                                        True, False, args)
+    for t in back:
+        assert t.shape[0] == P
+        assert float(t[radii == 0].abs().max()) == 0.0  # nothing reaches a culled Gaussian

@@ -221,3 +221,33 @@ def test_grid_too_large_for_the_tile_histogram(orc, H):
     ranges = imgB[ibase + ioff[3].value: ibase + ioff[3].value + 8 * T].view(torch.int32)
     assert np.array_equal(H.np_u32(ranges), want["ranges"].reshape(-1))
     assert np.array_equal(H.np_u32(point_list), want["point_list"])
+
+
+@pytest.mark.parametrize("limits", [(1, 8192, 32), (1, 0, 32)])
+def test_more_instances_than_positions_is_an_error(H, limits):
+    """1.2 M splats that each cover all 3888 tiles are 4.7e9 instances: the 32-bit prefix sums wrap around to a
+    plausible count (3.7e8).  The call must fail on the exact count instead of sizing its buffers by the wrapped
+    one, whichever kernels did the counting."""
+    import gsrast_native as gn
+    from diff_gaussian_rasterization import _C
+    P, W, Hh = 1_200_000, 1152, 864
+    gx, gy = H.grid(W, Hh)
+    assert P * gx * gy > 2 ** 32 and (P * gx * gy) % 2 ** 32 < 2 ** 31 - 2
+    means2D = torch.full((P, 2), 500.0, device=DEV)
+    depths = torch.ones(P, device=DEV)
+    radii = torch.full((P,), 5000, dtype=torch.int32, device=DEV)
+    co = torch.tensor([0.01, 0.0, 0.01, 0.5], device=DEV).repeat(P, 1)
+    rgb = torch.zeros(P, 3, device=DEV)
+    cl = torch.ones(gy, gx, dtype=torch.bool, device=DEV)
+    eye = torch.eye(4, device=DEV)
+    gn.lib.gs_set_tile_sort_limits(*limits)
+    with pytest.raises(RuntimeError, match="instances"):
+        _C.render_gaussians(torch.zeros(3, device=DEV), Hh, W, means2D, depths, radii, co, rgb, cl, eye,
+                            torch.zeros(3, device=DEV), 1.0, 0.75, torch.zeros(P, 5, device=DEV), False, False,
+                            {"stats_collector": {}})
+    # a count just inside the limit is still served (here: none at all after the failed call)
+    radii.zero_()
+    out = _C.render_gaussians(torch.zeros(3, device=DEV), Hh, W, means2D, depths, radii, co, rgb, cl, eye,
+                              torch.zeros(3, device=DEV), 1.0, 0.75, torch.zeros(P, 5, device=DEV), False, False,
+                              {"stats_collector": {}})
+    assert out[0] == 0
