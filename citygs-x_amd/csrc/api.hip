@@ -749,9 +749,9 @@ size_t gs_neural_workspace_bytes(int64_t num_anchors, int n_offsets) {
 }
 
 int gs_neural_opacity_forward(int64_t N, int k, const float* anchor, const float* feat, const float* campos,
-                              const float* const* mlp_params, const float* opacity_scale, float* neural_opacity,
-                              uint8_t* mask, uint32_t* first, void* workspace, size_t workspace_bytes,
-                              int64_t* num_selected, gs_stream_t stream_) {
+                              const float* const* mlp_params, const float* opacity_scale, const float* level,
+                              int input_flags, float* neural_opacity, uint8_t* mask, uint32_t* first,
+                              void* workspace, size_t workspace_bytes, int64_t* num_selected, gs_stream_t stream_) {
   hipStream_t stream = (hipStream_t)stream_;
   GS_REQUIRE(N >= 0, "gs_neural_opacity_forward: negative anchor count");
   GS_REQUIRE(neural_supported(k), "gs_neural_opacity_forward: n_offsets not among the supported values");
@@ -759,6 +759,8 @@ int gs_neural_opacity_forward(int64_t N, int k, const float* anchor, const float
   *num_selected = 0;
   GS_REQUIRE(N * (int64_t)k < 0x7FFFFFFFll, "gs_neural_opacity_forward: anchors x offsets exceed 2^31-1");
   GS_REQUIRE(mlp_params && campos, "gs_neural_opacity_forward: null pointer");
+  GS_REQUIRE(input_flags >= 0 && input_flags < 16, "gs_neural_opacity_forward: input_flags has four bits");
+  GS_REQUIRE(!(input_flags & 8) || level || N == 0, "gs_neural_opacity_forward: input_flags asks for the level");
   for (int i = 0; i < 12; i++) GS_REQUIRE(mlp_params[i], "gs_neural_opacity_forward: null MLP parameter");
   GS_REQUIRE(workspace && workspace_bytes >= gs_neural_workspace_bytes(N, k),
              "gs_neural_opacity_forward: workspace missing or too small");
@@ -767,7 +769,7 @@ int gs_neural_opacity_forward(int64_t N, int k, const float* anchor, const float
   float* packed = (float*)(base + L.packed);
   {
     StageScope _t("neural_pack", stream);
-    launch_neural_pack(k, mlp_params, packed, stream);
+    launch_neural_pack(k, mlp_params, input_flags, packed, stream);
   }
   if (check_launch("neural_pack", stream, false)) return 1;
   if (N == 0) return 0;
@@ -775,7 +777,8 @@ int gs_neural_opacity_forward(int64_t N, int k, const float* anchor, const float
   uint8_t* counts = (uint8_t*)(base + L.counts);
   {
     StageScope _t("neural_opacity", stream);
-    launch_neural_opacity(N, k, anchor, feat, campos, packed, opacity_scale, neural_opacity, mask, counts, stream);
+    launch_neural_opacity(N, k, anchor, feat, (input_flags & 8) ? level : nullptr, campos, packed, opacity_scale,
+                          neural_opacity, mask, counts, stream);
   }
   if (check_launch("neural_opacity", stream, false)) return 1;
   uint32_t* total_slot = acquire_total_slot();
@@ -800,7 +803,7 @@ int gs_neural_opacity_forward(int64_t N, int k, const float* anchor, const float
 }
 
 int gs_neural_gaussians_forward(int64_t N, int k, int64_t S, const float* anchor, const float* feat,
-                                const float* offsets, const float* scaling, const float* campos,
+                                const float* offsets, const float* scaling, const float* campos, const float* level,
                                 const float* neural_opacity, const uint32_t* first, const void* workspace,
                                 size_t workspace_bytes, float* xyz, float* color, float* opacity, float* scaling_out,
                                 float* rot, float* aux, gs_stream_t stream_) {
@@ -819,8 +822,8 @@ int gs_neural_gaussians_forward(int64_t N, int k, int64_t S, const float* anchor
   const float* packed = (const float*)(align_ptr((const char*)workspace, 256) + neural_workspace(N, k).packed);
   {
     StageScope _t("neural_gaussians", stream);
-    launch_neural_gaussians(N, k, anchor, feat, offsets, scaling, campos, packed, neural_opacity, first, xyz, color,
-                            opacity, scaling_out, rot, aux, stream);
+    launch_neural_gaussians(N, k, anchor, feat, level, offsets, scaling, campos, packed, neural_opacity, first, xyz,
+                            color, opacity, scaling_out, rot, aux, stream);
   }
   return check_launch("neural_gaussians", stream, false);
 }
@@ -834,22 +837,26 @@ size_t gs_neural_backward_workspace_bytes(int64_t num_anchors, int n_offsets) {
 
 int gs_neural_backward(int64_t N, int k, int64_t S, const float* anchor, const float* feat, const float* offsets,
                        const float* scaling, const float* campos, const float* const* mlp_params,
-                       const float* opacity_scale, const float* neural_opacity, const uint32_t* first,
-                       const float* color, const float* rot, const float* aux, const float* dL_dxyz,
-                       const float* dL_dcolor, const float* dL_dopacity, const float* dL_dscaling,
-                       const float* dL_drot, float* d_anchor, float* d_feat, float* d_offsets, float* d_scaling,
-                       float* const* d_mlp_params, void* workspace, size_t workspace_bytes, gs_stream_t stream_) {
+                       const float* opacity_scale, const float* level, int input_flags,
+                       const float* neural_opacity, const uint32_t* first, const float* color, const float* rot,
+                       const float* aux, const float* dL_dxyz, const float* dL_dcolor, const float* dL_dopacity,
+                       const float* dL_dscaling, const float* dL_drot, float* d_anchor, float* d_feat,
+                       float* d_offsets, float* d_scaling, float* const* d_mlp_params, void* workspace,
+                       size_t workspace_bytes, gs_stream_t stream_) {
   hipStream_t stream = (hipStream_t)stream_;
   GS_REQUIRE(N >= 0 && S >= 0, "gs_neural_backward: negative size");
   GS_REQUIRE(neural_supported(k), "gs_neural_backward: n_offsets not among the supported values");
   GS_REQUIRE(mlp_params && d_mlp_params && campos, "gs_neural_backward: null pointer");
+  GS_REQUIRE(input_flags >= 0 && input_flags < 16, "gs_neural_backward: input_flags has four bits");
+  GS_REQUIRE(!(input_flags & 8) || level || N == 0, "gs_neural_backward: input_flags asks for the level");
   for (int i = 0; i < 12; i++)
     GS_REQUIRE(mlp_params[i] && d_mlp_params[i], "gs_neural_backward: null MLP parameter or gradient");
   if (N == 0) {
     // no anchors: the weight gradients are zero
-    const size_t sizes[4] = {32 * 35, 32, 0, 0};
     for (int i = 0; i < 12; i++) {
-      const int out = (i / 4 == 0 ? 1 : i / 4 == 1 ? 3 : 7) * k;
+      const int m = i / 4;
+      const size_t sizes[4] = {(size_t)32 * (35 + ((input_flags >> m) & 1) + ((input_flags >> 3) & 1)), 32, 0, 0};
+      const int out = (m == 0 ? 1 : m == 1 ? 3 : 7) * k;
       const size_t n = i % 4 == 2 ? (size_t)out * 32 : i % 4 == 3 ? (size_t)out : sizes[i % 4];
       GS_HIP_TRY(hipMemsetAsync(d_mlp_params[i], 0, n * sizeof(float), stream));
     }
@@ -871,12 +878,12 @@ int gs_neural_backward(int64_t N, int k, int64_t S, const float* anchor, const f
   float* partials = (float*)((char*)slot_grads + align_up(neural_slot_grad_floats(k, N) * sizeof(float), 256));
   {
     StageScope _t("neural_pack", stream);
-    launch_neural_pack(k, mlp_params, packed, stream);
+    launch_neural_pack(k, mlp_params, input_flags, packed, stream);
   }
   if (check_launch("neural_pack", stream, false)) return 1;
   {
     StageScope _t("neural_backward", stream);
-    launch_neural_backward(N, k, anchor, feat, offsets, scaling, campos, packed, neural_opacity, opacity_scale, first,
+    launch_neural_backward(N, k, anchor, feat, (input_flags & 8) ? level : nullptr, input_flags, offsets, scaling, campos, packed, neural_opacity, opacity_scale, first,
                            color, rot, aux, dL_dxyz, dL_dcolor, dL_dopacity, dL_dscaling, dL_drot, d_anchor, d_feat, d_offsets,
                            d_scaling, d_mlp_params, slot_grads, partials, stream);
   }

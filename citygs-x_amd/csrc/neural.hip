@@ -1,6 +1,7 @@
 // Neural-Gaussian generation: the three anchor MLPs, the opacity selection and the post-processing of
-// generate_neural_gaussians (gaussian_renderer/__init__.py:789-899) in its default configuration
-// (feat_dim 32, inputs [feat, view direction], scene/gaussian_model.py:131-149), forward and backward.
+// generate_neural_gaussians (gaussian_renderer/__init__.py:789-899) for feat_dim 32 (inputs [feat, view
+// direction] and, where the model asks for them, the distance and the anchor's level,
+// scene/gaussian_model.py:118-149), forward and backward.
 //
 // One wave owns 32 anchors.  Both layers run on the fp32 matrix cores (v_mfma_f32_32x32x2_f32) in the
 // transposed form D[unit][anchor] = W[unit][:] . X[:][anchor]: the anchors sit on the 32 columns, so the
@@ -22,11 +23,12 @@ namespace {
 constexpr int NG_WAVES = 4;          // waves per block of the forward kernels
 constexpr int NG_THREADS = 64 * NG_WAVES;
 constexpr int NG_ANCHORS = 32;       // anchors per wave tile
-constexpr int NG_W1_STEPS = 18;      // 36 input slots: 32 features, 3 view components, 1 constant for the bias
+constexpr int NG_W1_STEPS = 19;      // 38 input slots: 32 features, 3 view components, 1 constant for the bias,
+                                     // the distance and the level (zero weights where an MLP does not take them)
 constexpr int NG_SLOTS = 2 * NG_W1_STEPS;
 constexpr int NG_TILE = 1024;        // one 32x32 accumulator tile
 constexpr int WS = 33;               // row stride of the weight arrays in LDS (conflict-free both ways)
-constexpr int SX_STRIDE = 37;
+constexpr int SX_STRIDE = 39;
 constexpr int SG_STRIDE = 33;
 constexpr int NG_SLOT_GRADS = 11;    // pre-activation gradients per offset: 1 opacity, 3 color, 7 cov
 
@@ -36,7 +38,7 @@ __host__ __device__ constexpr int even_up(int v) { return (v + 1) & ~1; }
 __host__ __device__ constexpr int hrow(int half, int i) { return 8 * (i >> 2) + 4 * half + (i & 3); }
 
 // input slot a lane of the given half supplies at layer-1 step s: 16 consecutive features per half, then the
-// view direction and the constant
+// view direction and the constant, then the distance (half 0) and the level (half 1)
 __host__ __device__ constexpr int xslot(int half, int s) { return s < 16 ? 16 * half + s : 32 + 2 * (s - 16) + half; }
 
 template <int K>
@@ -67,11 +69,29 @@ __host__ __device__ constexpr PackLayout pack_layout(int grows) {
   return PackLayout{0, 3 * NG_SLOTS * WS, 3 * NG_SLOTS * WS + grows * WS, 3 * NG_SLOTS * WS + grows * WS + grows};
 }
 
+// W1 of MLP m has in[m] columns: 32 features, 3 view components, then the distance (column dist_col[m], or -1)
+// and the level (column level_col[m], or -1)
+struct MlpInputs {
+  int in[3], dist_col[3], level_col[3];
+};
+// input_flags: bit m = MLP m (opacity, color, cov) takes the distance, bit 3 = all take the level
+MlpInputs mlp_inputs(int input_flags) {
+  MlpInputs q;
+  for (int m = 0; m < 3; m++) {
+    const bool d = (input_flags >> m) & 1, l = (input_flags >> 3) & 1;
+    q.dist_col[m] = d ? 35 : -1;
+    q.level_col[m] = l ? 35 + (d ? 1 : 0) : -1;
+    q.in[m] = 35 + (d ? 1 : 0) + (l ? 1 : 0);
+  }
+  return q;
+}
 struct MlpParams {
   const float* p[12];  // W1, b1, W2, b2 of the opacity, color and cov MLPs
+  MlpInputs q;
 };
 struct MlpGrads {
   float* p[12];
+  MlpInputs q;
 };
 
 template <int K>
@@ -83,7 +103,10 @@ __global__ void __launch_bounds__(256) neural_pack_kernel(MlpParams w, float* __
   float v = 0.0f;
   if (e < L.w2) {
     const int m = e / (NG_SLOTS * WS), r = e % (NG_SLOTS * WS), slot = r / WS, h = r % WS;
-    if (h < 32) v = slot < 35 ? w.p[4 * m][h * 35 + slot] : w.p[4 * m + 1][h];
+    if (h < 32) {
+      const int col = slot < 35 ? slot : slot == 36 ? w.q.dist_col[m] : slot == 37 ? w.q.level_col[m] : -1;
+      v = slot == 35 ? w.p[4 * m + 1][h] : col >= 0 ? w.p[4 * m][h * w.q.in[m] + col] : 0.0f;
+    }
   } else {
     const bool bias = e >= L.b2;
     const int rel = e - (bias ? L.b2 : L.w2);
@@ -104,24 +127,26 @@ __device__ __forceinline__ void wave_sync() {
 // hardware exp2 and reciprocal: about 1e-6 relative, far inside what float32 MLP outputs carry
 __device__ __forceinline__ float sigmoidf(float x) { return __builtin_amdgcn_rcpf(1.0f + __expf(-x)); }
 
-// The 18 layer-1 B operands of this lane: its anchor's features of its half, the view direction and the constant.
+// The 19 layer-1 B operands of this lane: its anchor's features of its half, the view direction, the constant,
+// the distance and the level.
 // Also returns the unit view direction and the distance (every lane computes both).
 struct XOperand {
   float4 f[4];
-  float ax, ay, az;
+  float ax, ay, az, level;
 };
 __device__ __forceinline__ XOperand fetch_x(bool valid, int64_t a, int half, const float* __restrict__ anchor,
-                                            const float* __restrict__ feat) {
+                                            const float* __restrict__ feat, const float* __restrict__ level) {
   XOperand x;
   if (valid) {
     const float4* f = (const float4*)(feat + a * 32 + 16 * half);
 #pragma unroll
     for (int q = 0; q < 4; q++) x.f[q] = f[q];
     x.ax = anchor[a * 3]; x.ay = anchor[a * 3 + 1]; x.az = anchor[a * 3 + 2];
+    x.level = level != nullptr ? level[a] : 0.0f;
   } else {
 #pragma unroll
     for (int q = 0; q < 4; q++) x.f[q] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-    x.ax = x.ay = x.az = 0.0f;
+    x.ax = x.ay = x.az = x.level = 0.0f;
   }
   return x;
 }
@@ -141,6 +166,7 @@ __device__ __forceinline__ void unpack_x(float (&xb)[NG_W1_STEPS], float (&nv)[3
   }
   xb[16] = half ? nv[1] : nv[0];
   xb[17] = half ? 1.0f : nv[2];
+  xb[18] = half ? x.level : dist;
 }
 
 // relu(W1 x + b1) for the wave's 32 anchors; w1t = this MLP's [slot][WS] array
@@ -152,6 +178,7 @@ __device__ __forceinline__ v16f hidden_layer(const float* w1t, const float (&xb)
   for (int s = 0; s < 16; s++) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(lo[s * WS], xb[s], acc, 0, 0, 0);
   acc = __builtin_amdgcn_mfma_f32_32x32x2f32(hi[0], xb[16], acc, 0, 0, 0);
   acc = __builtin_amdgcn_mfma_f32_32x32x2f32(hi[2 * WS], xb[17], acc, 0, 0, 0);
+  acc = __builtin_amdgcn_mfma_f32_32x32x2f32(hi[4 * WS], xb[18], acc, 0, 0, 0);
 #pragma unroll
   for (int i = 0; i < 16; i++) acc[i] = acc[i] > 0.0f ? acc[i] : 0.0f;
   return acc;
@@ -191,6 +218,7 @@ __device__ __forceinline__ int count_lanes(unsigned long long bits, int lo, int 
 template <int K>
 __global__ void __launch_bounds__(NG_THREADS)
 neural_opacity_kernel(int64_t N, int ntiles, const float* __restrict__ anchor, const float* __restrict__ feat,
+                      const float* __restrict__ level,
                       const float* __restrict__ campos, const float* __restrict__ packed,
                       const float* __restrict__ opacity_scale, float* __restrict__ neural_opacity,
                       uint8_t* __restrict__ mask, uint8_t* __restrict__ counts) {
@@ -210,7 +238,7 @@ neural_opacity_kernel(int64_t N, int ntiles, const float* __restrict__ anchor, c
   for (int tile = blockIdx.x * NG_WAVES + wave; tile < ntiles; tile += gridDim.x * NG_WAVES) {
     const int64_t a = (int64_t)tile * NG_ANCHORS + al;
     float xb[NG_W1_STEPS], nv[3], dist;
-    unpack_x(xb, nv, dist, fetch_x(a < N, a, half, anchor, feat), a < N, half, cam);
+    unpack_x(xb, nv, dist, fetch_x(a < N, a, half, anchor, feat, level), a < N, half, cam);
     const v16f h = hidden_layer(sW1, xb, al, half);
     const v16f o = output_tile<S::OUT0>(sW2, sB2, 0, h, al, half);
     const float ps = (opacity_scale != nullptr && a < N) ? opacity_scale[a] : 1.0f;
@@ -246,7 +274,7 @@ neural_opacity_kernel(int64_t N, int ntiles, const float* __restrict__ anchor, c
 template <int K>
 __global__ void __launch_bounds__(NG_THREADS, 2)
 neural_gaussians_kernel(int64_t N, int ntiles, const float* __restrict__ anchor, const float* __restrict__ feat,
-                        const float* __restrict__ offsets, const float* __restrict__ scaling,
+                        const float* __restrict__ level, const float* __restrict__ offsets, const float* __restrict__ scaling,
                         const float* __restrict__ campos, const float* __restrict__ packed,
                         const float* __restrict__ neural_opacity, const uint32_t* __restrict__ first,
                         float* __restrict__ xyz, float* __restrict__ color, float* __restrict__ opacity,
@@ -277,7 +305,7 @@ neural_gaussians_kernel(int64_t N, int ntiles, const float* __restrict__ anchor,
   uint32_t p_first = 0;
   auto fetch_tile = [&](int t) {
     const int64_t a = (int64_t)t * NG_ANCHORS + al;
-    xo = fetch_x(a < N, a, half, anchor, feat);
+    xo = fetch_x(a < N, a, half, anchor, feat, level);
 #pragma unroll
     for (int c = 0; c < 3; c++) p_sc[c] = a < N ? scaling[a * 6 + 3 * half + c] : 0.0f;
     p_first = a < N ? first[a] : 0u;
@@ -486,7 +514,7 @@ __host__ __device__ constexpr int partial_floats() {
 template <int K>
 __global__ void __launch_bounds__(64 * Shape<K>::BWD_WAVES)
 neural_mlp_backward_kernel(int64_t N, int ntiles, const float* __restrict__ anchor, const float* __restrict__ feat,
-                           const float* __restrict__ campos, const float* __restrict__ packed,
+                           const float* __restrict__ level, const float* __restrict__ campos, const float* __restrict__ packed,
                            const float* __restrict__ slot_grads, float* __restrict__ d_anchor,
                            float* __restrict__ d_feat, float* __restrict__ partials) {
   using S = Shape<K>;
@@ -498,12 +526,15 @@ neural_mlp_backward_kernel(int64_t N, int ntiles, const float* __restrict__ anch
   __shared__ BwdLds<K> lds[NW];
   __shared__ float sW1[3 * NG_SLOTS * WS];
   __shared__ float sW2[S::GROWS * WS];
-  __shared__ __align__(16) float sWview[9 * 32];   // W1[h][32 + c] as [m][c][h]: the view-direction columns
+  // W1's view-direction columns (c = 0..2) and distance column (c = 3) as [m][c][h]
+  __shared__ __align__(16) float sWview[12 * 32];
   __shared__ unsigned short sWhere[TILE_FLOATS];  // where in G each float of a tile's records goes
   for (int e = threadIdx.x; e < 3 * NG_SLOTS * WS; e += NT) sW1[e] = packed[L.w1t + e];
   for (int e = threadIdx.x; e < S::GROWS * WS; e += NT) sW2[e] = packed[L.w2 + e];
-  for (int e = threadIdx.x; e < 9 * 32; e += NT)
-    sWview[e] = packed[L.w1t + ((e / 96) * NG_SLOTS + 32 + (e / 32) % 3) * WS + e % 32];
+  for (int e = threadIdx.x; e < 12 * 32; e += NT) {
+    const int c = (e / 32) % 4;
+    sWview[e] = packed[L.w1t + ((e / 128) * NG_SLOTS + (c < 3 ? 32 + c : 36)) * WS + e % 32];
+  }
   for (int e = threadIdx.x; e < TILE_FLOATS; e += NT) {
     const int slot = e / NG_SLOT_GRADS, comp = e % NG_SLOT_GRADS, ax = slot / K, j = slot % K;
     const int row = comp == 0 ? S::G0 + j : comp < 4 ? S::G1 + 3 * j + (comp - 1) : S::G2 + 7 * j + (comp - 4);
@@ -517,7 +548,7 @@ neural_mlp_backward_kernel(int64_t N, int ntiles, const float* __restrict__ anch
   __syncthreads();
 
   // weight-gradient accumulators: the W2 tiles, the 32 feature columns of W1 per MLP, and one tile that holds the
-  // four remaining columns of W1 (view direction, bias) of all three MLPs as its rows 4 m + c
+  // six remaining columns of W1 (view direction, bias, distance, level) of all three MLPs as its rows 6 m + c
   v16f accW2[S::TILES], accW1[3], accWx;
   float accB2[B2N];
 #pragma unroll
@@ -542,7 +573,7 @@ neural_mlp_backward_kernel(int64_t N, int ntiles, const float* __restrict__ anch
   float da[3] = {0.0f, 0.0f, 0.0f};  // the anchor's direct gradient, as the first kernel left it
   auto fetch_tile = [&](int t) {
     const int64_t a = (int64_t)t * NG_ANCHORS + al;
-    xo = fetch_x(a < N, a, half, anchor, feat);
+    xo = fetch_x(a < N, a, half, anchor, feat, level);
     if (a < N && half == 0) {
 #pragma unroll
       for (int c = 0; c < 3; c++) da[c] = d_anchor[a * 3 + c];
@@ -582,7 +613,8 @@ neural_mlp_backward_kernel(int64_t N, int ntiles, const float* __restrict__ anch
     wave_sync();
 
     v16f dxf = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-    float dv[3] = {0.0f, 0.0f, 0.0f};  // this half's share of the gradient of the view direction
+    // this half's share of the gradient of the view direction (0..2) and of the distance (3)
+    float dv[4] = {0.0f, 0.0f, 0.0f, 0.0f};
     const float* xrow = W.x + al * SX_STRIDE;
 #pragma unroll
     for (int m = 0; m < 3; m++) {
@@ -598,6 +630,7 @@ neural_mlp_backward_kernel(int64_t N, int ntiles, const float* __restrict__ anch
         for (int s = 0; s < 16; s++) h = __builtin_amdgcn_mfma_f32_32x32x2f32(lo[s * WS], xrow[16 * half + s], h, 0, 0, 0);
         h = __builtin_amdgcn_mfma_f32_32x32x2f32(hi[0], xrow[32 + half], h, 0, 0, 0);
         h = __builtin_amdgcn_mfma_f32_32x32x2f32(hi[2 * WS], xrow[34 + half], h, 0, 0, 0);
+        h = __builtin_amdgcn_mfma_f32_32x32x2f32(hi[4 * WS], xrow[36 + half], h, 0, 0, 0);
 #pragma unroll
         for (int i = 0; i < 16; i++) h[i] = h[i] > 0.0f ? h[i] : 0.0f;
       }
@@ -615,18 +648,18 @@ neural_mlp_backward_kernel(int64_t N, int ntiles, const float* __restrict__ anch
       for (int i = 0; i < 16; i++) dh[i] = h[i] > 0.0f ? dh[i] : 0.0f;
       __builtin_amdgcn_sched_barrier(0);
       {
-        // dX += W1^T dHpre: the 32 feature rows on the matrix cores, the 3 view rows as plain sums over the 16
-        // hidden units this lane holds (the other 16 sit in the lane of the other half)
+        // dX += W1^T dHpre: the 32 feature rows on the matrix cores, the 3 view rows and the distance row as plain
+        // sums over the 16 hidden units this lane holds (the other 16 sit in the lane of the other half)
         const float* wf = w1t + al * WS + 4 * half;
 #pragma unroll
         for (int s = 0; s < 16; s++)
           dxf = __builtin_amdgcn_mfma_f32_32x32x2f32(wf[8 * (s >> 2) + (s & 3)], dh[s], dxf, 0, 0, 0);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int c = 0; c < 3; c++)
+        for (int c = 0; c < 4; c++)
 #pragma unroll
           for (int q = 0; q < 4; q++) {
-            const float4 w = *(const float4*)(sWview + (m * 3 + c) * 32 + 8 * q + 4 * half);
+            const float4 w = *(const float4*)(sWview + (m * 4 + c) * 32 + 8 * q + 4 * half);
             dv[c] = __builtin_fmaf(w.x, dh[4 * q], dv[c]);
             dv[c] = __builtin_fmaf(w.y, dh[4 * q + 1], dv[c]);
             dv[c] = __builtin_fmaf(w.z, dh[4 * q + 2], dv[c]);
@@ -657,9 +690,10 @@ neural_mlp_backward_kernel(int64_t N, int ntiles, const float* __restrict__ anch
         const float dhv = dhrow[2 * s + half];
         const float* xr = W.x + (2 * s + half) * SX_STRIDE;
         accW1[m] = __builtin_amdgcn_mfma_f32_32x32x2f32(dhv, xr[al], accW1[m], 0, 0, 0);
-        // rows 4 m .. 4 m + 3 of the shared tile take this MLP's view and bias columns, the other rows add zero
-        const float xv = xr[32 + (al & 3)];
-        accWx = __builtin_amdgcn_mfma_f32_32x32x2f32((al >> 2) == m ? xv : 0.0f, dhv, accWx, 0, 0, 0);
+        // rows 6 m .. 6 m + 5 of the shared tile take this MLP's view, bias, distance and level columns, the
+        // other rows add zero
+        const float xv = xr[32 + (al % 6)];
+        accWx = __builtin_amdgcn_mfma_f32_32x32x2f32((al / 6) == m ? xv : 0.0f, dhv, accWx, 0, 0, 0);
       }
       wave_sync();
     }
@@ -676,16 +710,18 @@ neural_mlp_backward_kernel(int64_t N, int ntiles, const float* __restrict__ anch
 
     // ---- per anchor results
 #pragma unroll
-    for (int c = 0; c < 3; c++) dv[c] += __shfl_xor(dv[c], 32);
+    for (int c = 0; c < 4; c++) dv[c] += __shfl_xor(dv[c], 32);
     if (valid) {
 #pragma unroll
       for (int q = 0; q < 4; q++)
         *(float4*)(d_feat + a * 32 + 8 * q + 4 * half) = make_float4(dxf[4 * q], dxf[4 * q + 1], dxf[4 * q + 2], dxf[4 * q + 3]);
       if (half == 0) {
-        // the view direction n = v / |v| adds (g - n (n.g)) / |v| to the anchor's direct gradient
+        // the view direction n = v / |v| adds (g - n (n.g)) / |v| to the anchor's direct gradient, the distance
+        // |v| adds n g
         const float ng = (nv[0] * dv[0] + nv[1] * dv[1]) + nv[2] * dv[2];
 #pragma unroll
-        for (int c = 0; c < 3; c++) d_anchor[a * 3 + c] = da_now[c] + (dv[c] - nv[c] * ng) / dist;
+        for (int c = 0; c < 3; c++)
+          d_anchor[a * 3 + c] = (da_now[c] + (dv[c] - nv[c] * ng) / dist) + nv[c] * dv[3];
       }
     }
     wave_sync();
@@ -708,11 +744,11 @@ neural_mlp_backward_kernel(int64_t N, int ntiles, const float* __restrict__ anch
       for (int w = 1; w < NW; w++) sum += lds[w].hd[e];
       if (t < S::TILES + 3) {
         dst[e] = sum;
-      } else if (e < 12 * 32) {
-        // row 4 m + c, column h of the shared tile -> column 32 + c of W1 of MLP m: element h * 32 + c of its
-        // second tile
+      } else if (e < 18 * 32) {
+        // row 6 m + c, column h of the shared tile -> input slot 32 + c of W1 of MLP m: element h * 32 + c of
+        // its second tile
         const int row = e >> 5, h = e & 31;
-        out[(S::TILES + 2 * (row >> 2) + 1) * NG_TILE + h * 32 + (row & 3)] = sum;
+        out[(S::TILES + 2 * (row / 6) + 1) * NG_TILE + h * 32 + (row % 6)] = sum;
       }
     }
   }
@@ -735,27 +771,33 @@ template <int K>
 __global__ void __launch_bounds__(256)
 neural_weight_reduce_kernel(int nblocks, const float* __restrict__ partials, MlpGrads d) {
   using S = Shape<K>;
-  constexpr int PER_MLP_1 = 32 * 35 + 32;
-  constexpr int TOTAL = 3 * PER_MLP_1 + 33 * (S::OUT0 + S::OUT1 + S::OUT2);
+  const int per1[3] = {32 * d.q.in[0] + 32, 32 * d.q.in[1] + 32, 32 * d.q.in[2] + 32};
+  const int first_layers = per1[0] + per1[1] + per1[2];
+  const int TOTAL = first_layers + 33 * (S::OUT0 + S::OUT1 + S::OUT2);
   __shared__ float s_part[16][17];
   const int el = threadIdx.x & 15, part = threadIdx.x >> 4;
   const int e = blockIdx.x * 16 + el;
   int src = 0;  // index inside a partial set
   float* dst = nullptr;
   if (e < TOTAL) {
-    if (e < 3 * PER_MLP_1) {
-      const int m = e / PER_MLP_1, r = e % PER_MLP_1;
-      if (r < 32 * 35) {
-        const int h = r / 35, i = r % 35;
-        src = (S::TILES + 2 * m + (i >= 32)) * NG_TILE + h * 32 + (i & 31);
+    if (e < first_layers) {
+      int m = 0, r = e;
+      while (r >= per1[m]) { r -= per1[m]; m++; }
+      const int in = d.q.in[m];
+      if (r < 32 * in) {
+        // column i of W1: a feature (first tile), or input slot 32 + c of the second tile: c = 0..2 the view
+        // direction, 4 the distance, 5 the level (3 is the bias)
+        const int h = r / in, i = r % in;
+        const int c = i < 35 ? i - 32 : i == d.q.dist_col[m] ? 4 : 5;
+        src = i < 32 ? (S::TILES + 2 * m) * NG_TILE + h * 32 + i : (S::TILES + 2 * m + 1) * NG_TILE + h * 32 + c;
         dst = d.p[4 * m] + r;
       } else {
-        const int h = r - 32 * 35;
+        const int h = r - 32 * in;
         src = (S::TILES + 2 * m + 1) * NG_TILE + h * 32 + 3;
         dst = d.p[4 * m + 1] + h;
       }
     } else {
-      int r = e - 3 * PER_MLP_1;
+      int r = e - first_layers;
       int m = 0;
       while (r >= 33 * S::out(m)) { r -= 33 * S::out(m); m++; }
       const int out = S::out(m);
@@ -797,33 +839,34 @@ int blocks_for(int ntiles, int waves_per_block, int per_cu) {
 template <int K>
 struct Launcher {
   using S = Shape<K>;
-  static void pack(const float* const* params, float* packed, hipStream_t stream) {
+  static void pack(const float* const* params, int input_flags, float* packed, hipStream_t stream) {
     MlpParams w;
     for (int i = 0; i < 12; i++) w.p[i] = params[i];
+    w.q = mlp_inputs(input_flags);
     const int total = pack_layout(S::GROWS).total;
     hipLaunchKernelGGL(neural_pack_kernel<K>, dim3((total + 255) / 256), dim3(256), 0, stream, w, packed);
   }
-  static void opacity(int64_t N, const float* anchor, const float* feat, const float* campos, const float* packed,
-                      const float* opacity_scale, float* neural_opacity, uint8_t* mask, uint8_t* counts,
-                      hipStream_t stream) {
+  static void opacity(int64_t N, const float* anchor, const float* feat, const float* level, const float* campos,
+                      const float* packed, const float* opacity_scale, float* neural_opacity, uint8_t* mask,
+                      uint8_t* counts, hipStream_t stream) {
     const int ntiles = (int)((N + NG_ANCHORS - 1) / NG_ANCHORS);
     hipLaunchKernelGGL(neural_opacity_kernel<K>, dim3(blocks_for(ntiles, NG_WAVES, 4)), dim3(NG_THREADS), 0, stream,
-                       N, ntiles, anchor, feat, campos, packed, opacity_scale, neural_opacity, mask, counts);
+                       N, ntiles, anchor, feat, level, campos, packed, opacity_scale, neural_opacity, mask, counts);
   }
-  static void gaussians(int64_t N, const float* anchor, const float* feat, const float* offsets, const float* scaling,
-                        const float* campos, const float* packed, const float* neural_opacity, const uint32_t* first,
+  static void gaussians(int64_t N, const float* anchor, const float* feat, const float* level, const float* offsets,
+                        const float* scaling, const float* campos, const float* packed, const float* neural_opacity, const uint32_t* first,
                         float* xyz, float* color, float* opacity, float* scal, float* rot, float* aux,
                         hipStream_t stream) {
     const int ntiles = (int)((N + NG_ANCHORS - 1) / NG_ANCHORS);
     hipLaunchKernelGGL(neural_gaussians_kernel<K>, dim3(blocks_for(ntiles, NG_WAVES, 2)), dim3(NG_THREADS), 0, stream,
-                       N, ntiles, anchor, feat, offsets, scaling, campos, packed, neural_opacity, first, xyz, color,
-                       opacity, scal, rot, aux);
+                       N, ntiles, anchor, feat, level, offsets, scaling, campos, packed, neural_opacity, first, xyz,
+                       color, opacity, scal, rot, aux);
   }
   static int backward_blocks(int64_t N) {
     return blocks_for((int)((N + NG_ANCHORS - 1) / NG_ANCHORS), S::BWD_WAVES, 1);
   }
-  static void backward(int64_t N, const float* anchor, const float* feat, const float* offsets, const float* scaling,
-                       const float* campos, const float* packed, const float* neural_opacity,
+  static void backward(int64_t N, const float* anchor, const float* feat, const float* level, int input_flags,
+                       const float* offsets, const float* scaling, const float* campos, const float* packed, const float* neural_opacity,
                        const float* opacity_scale, const uint32_t* first, const float* color_out,
                        const float* rot_out, const float* aux, const float* g_xyz, const float* g_color,
                        const float* g_opacity, const float* g_scal, const float* g_rot, float* d_anchor,
@@ -835,10 +878,11 @@ struct Launcher {
                        aux, g_xyz, g_color, g_opacity, g_scal, g_rot, slot_grads, d_anchor, d_offsets, d_scaling);
     const int nblocks = backward_blocks(N);
     hipLaunchKernelGGL(neural_mlp_backward_kernel<K>, dim3(nblocks), dim3(64 * S::BWD_WAVES), 0, stream, N, ntiles,
-                       anchor, feat, campos, packed, slot_grads, d_anchor, d_feat, partials);
+                       anchor, feat, level, campos, packed, slot_grads, d_anchor, d_feat, partials);
     MlpGrads d;
     for (int i = 0; i < 12; i++) d.p[i] = d_params[i];
-    const int total = 3 * (32 * 35 + 32) + 33 * (S::OUT0 + S::OUT1 + S::OUT2);
+    d.q = mlp_inputs(input_flags);
+    const int total = 32 * (d.q.in[0] + d.q.in[1] + d.q.in[2]) + 96 + 33 * (S::OUT0 + S::OUT1 + S::OUT2);
     hipLaunchKernelGGL(neural_weight_reduce_kernel<K>, dim3((total + 15) / 16), dim3(256), 0, stream, nblocks,
                        partials, d);
   }
@@ -880,42 +924,42 @@ size_t neural_partial_floats(int k, int64_t N) {
 // floats of the per-offset gradient records, padded so a 16-byte read at the end stays inside
 size_t neural_slot_grad_floats(int k, int64_t N) { return (size_t)N * (size_t)k * NG_SLOT_GRADS + 4; }
 
-int launch_neural_pack(int k, const float* const* params, float* packed, hipStream_t stream) {
+int launch_neural_pack(int k, const float* const* params, int input_flags, float* packed, hipStream_t stream) {
   switch (k) {
-#define X(KK) case KK: Launcher<KK>::pack(params, packed, stream); return 0;
+#define X(KK) case KK: Launcher<KK>::pack(params, input_flags, packed, stream); return 0;
     NG_FOR_EACH_K(X)
 #undef X
     default: return 1;
   }
 }
 
-int launch_neural_opacity(int64_t N, int k, const float* anchor, const float* feat, const float* campos,
-                          const float* packed, const float* opacity_scale, float* neural_opacity, uint8_t* mask,
+int launch_neural_opacity(int64_t N, int k, const float* anchor, const float* feat, const float* level,
+                          const float* campos, const float* packed, const float* opacity_scale, float* neural_opacity, uint8_t* mask,
                           uint8_t* counts, hipStream_t stream) {
   if (N <= 0) return 0;
   switch (k) {
-#define X(KK) case KK: Launcher<KK>::opacity(N, anchor, feat, campos, packed, opacity_scale, neural_opacity, mask, counts, stream); return 0;
+#define X(KK) case KK: Launcher<KK>::opacity(N, anchor, feat, level, campos, packed, opacity_scale, neural_opacity, mask, counts, stream); return 0;
     NG_FOR_EACH_K(X)
 #undef X
     default: return 1;
   }
 }
 
-int launch_neural_gaussians(int64_t N, int k, const float* anchor, const float* feat, const float* offsets,
-                            const float* scaling, const float* campos, const float* packed,
+int launch_neural_gaussians(int64_t N, int k, const float* anchor, const float* feat, const float* level,
+                            const float* offsets, const float* scaling, const float* campos, const float* packed,
                             const float* neural_opacity, const uint32_t* first, float* xyz, float* color,
                             float* opacity, float* scal, float* rot, float* aux, hipStream_t stream) {
   if (N <= 0) return 0;
   switch (k) {
-#define X(KK) case KK: Launcher<KK>::gaussians(N, anchor, feat, offsets, scaling, campos, packed, neural_opacity, first, xyz, color, opacity, scal, rot, aux, stream); return 0;
+#define X(KK) case KK: Launcher<KK>::gaussians(N, anchor, feat, level, offsets, scaling, campos, packed, neural_opacity, first, xyz, color, opacity, scal, rot, aux, stream); return 0;
     NG_FOR_EACH_K(X)
 #undef X
     default: return 1;
   }
 }
 
-int launch_neural_backward(int64_t N, int k, const float* anchor, const float* feat, const float* offsets,
-                           const float* scaling, const float* campos, const float* packed,
+int launch_neural_backward(int64_t N, int k, const float* anchor, const float* feat, const float* level,
+                           int input_flags, const float* offsets, const float* scaling, const float* campos, const float* packed,
                            const float* neural_opacity, const float* opacity_scale, const uint32_t* first,
                            const float* color_out, const float* rot_out, const float* aux, const float* g_xyz,
                            const float* g_color, const float* g_opacity, const float* g_scal, const float* g_rot,
@@ -923,7 +967,7 @@ int launch_neural_backward(int64_t N, int k, const float* anchor, const float* f
                            float* const* d_params, float* slot_grads, float* partials, hipStream_t stream) {
   if (N <= 0) return 0;
   switch (k) {
-#define X(KK) case KK: Launcher<KK>::backward(N, anchor, feat, offsets, scaling, campos, packed, neural_opacity, opacity_scale, first, color_out, rot_out, aux, g_xyz, g_color, g_opacity, g_scal, g_rot, d_anchor, d_feat, d_offsets, d_scaling, d_params, slot_grads, partials, stream); return 0;
+#define X(KK) case KK: Launcher<KK>::backward(N, anchor, feat, level, input_flags, offsets, scaling, campos, packed, neural_opacity, opacity_scale, first, color_out, rot_out, aux, g_xyz, g_color, g_opacity, g_scal, g_rot, d_anchor, d_feat, d_offsets, d_scaling, d_params, slot_grads, partials, stream); return 0;
     NG_FOR_EACH_K(X)
 #undef X
     default: return 1;

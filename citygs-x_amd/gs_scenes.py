@@ -191,11 +191,13 @@ def build_all_map(means3D, scales, rotations, cam):
     return out
 
 
-def make_anchor_scene(N, k=10, seed=0, feat_dim=32):
+def make_anchor_scene(N, k=10, seed=0, feat_dim=32, input_flags=0):
     """Seeded anchors for the neural-Gaussian generation step: anchor positions, features, offsets,
     activated scalings (N,6), a camera centre and the three MLPs as nn.Linear-shaped tensors
     (scene/gaussian_model.py:131-149: Linear(feat_dim+3, feat_dim), ReLU, Linear(feat_dim, out)) drawn with
-    nn.Linear's default range.  Returns a dict; "mlps" is [(W1, b1, W2, b2)] in the order opacity, color, cov."""
+    nn.Linear's default range.  input_flags widens the first layers by the optional inputs (add_opacity_dist = 1,
+    add_color_dist = 2, add_cov_dist = 4: the distance; add_level = 8: the level, :118-121).  Returns a dict; "mlps"
+    is [(W1, b1, W2, b2)] in the order opacity, color, cov; "level" is the anchors' level (N, 1)."""
     gen = torch.Generator().manual_seed(1000 + seed)
     r = lambda *s: torch.rand(*s, generator=gen)
     n = lambda *s: torch.randn(*s, generator=gen)
@@ -205,30 +207,42 @@ def make_anchor_scene(N, k=10, seed=0, feat_dim=32):
     scaling = torch.exp(n(N, 6) * 0.4 - 1.0)
     campos = torch.tensor([10.0, -20.0, 120.0])
     mlps = []
-    for out in (k, 3 * k, 7 * k):
-        a1, a2 = 1.0 / math.sqrt(feat_dim + 3), 1.0 / math.sqrt(feat_dim)
-        mlps.append(((r(feat_dim, feat_dim + 3) * 2 - 1) * a1, (r(feat_dim) * 2 - 1) * a1,
+    for m, out in enumerate((k, 3 * k, 7 * k)):
+        width = feat_dim + 3 + ((input_flags >> m) & 1) + ((input_flags >> 3) & 1)
+        a1, a2 = 1.0 / math.sqrt(width), 1.0 / math.sqrt(feat_dim)
+        mlps.append(((r(feat_dim, width) * 2 - 1) * a1, (r(feat_dim) * 2 - 1) * a1,
                      (r(out, feat_dim) * 2 - 1) * a2, (r(out) * 2 - 1) * a2))
-    return {"anchor": anchor, "feat": feat, "offsets": offsets, "scaling": scaling, "campos": campos, "mlps": mlps}
+    level = torch.randint(0, 6, (N, 1), generator=gen).float()
+    return {"anchor": anchor, "feat": feat, "offsets": offsets, "scaling": scaling, "campos": campos, "mlps": mlps,
+            "level": level}
 
 
-def neural_gaussians_torch(anchor, feat, offsets, scaling, campos, mlps, prog=None):
+def neural_gaussians_torch(anchor, feat, offsets, scaling, campos, mlps, prog=None, level=None, input_flags=0):
     """generate_neural_gaussians (gaussian_renderer/__init__.py:789-899) in its default configuration, with
     torch operations in the dtype of its inputs: the comparison the fused operator is measured against.  prog
-    (N, 1), if given, is the factor dist2level 'progressive' puts on the opacity (:844-848)."""
+    (N, 1), if given, is the factor dist2level 'progressive' puts on the opacity (:844-848); level (N, 1) and
+    input_flags (add_opacity_dist = 1, add_color_dist = 2, add_cov_dist = 4, add_level = 8) are the MLPs' optional
+    inputs (:824-877)."""
     k = offsets.shape[1]
     ob_view = anchor - campos
-    ob_view = ob_view / ob_view.norm(dim=1, keepdim=True)
-    x = torch.cat([feat, ob_view], dim=1)
-    run = lambda m: torch.relu(x @ m[0].t() + m[1]) @ m[2].t() + m[3]
-    neural_opacity = torch.tanh(run(mlps[0]))
+    ob_dist = ob_view.norm(dim=1, keepdim=True)
+    ob_view = ob_view / ob_dist
+    lv = [level.reshape(-1, 1).to(feat.dtype)] if input_flags & 8 else []
+    with_dist = torch.cat([feat, ob_view, ob_dist] + lv, dim=1)
+    without = torch.cat([feat, ob_view] + lv, dim=1)
+
+    def run(i):
+        m, x = mlps[i], with_dist if (input_flags >> i) & 1 else without
+        return torch.relu(x @ m[0].t() + m[1]) @ m[2].t() + m[3]
+
+    neural_opacity = torch.tanh(run(0))
     if prog is not None:
         neural_opacity = neural_opacity * prog
     neural_opacity = neural_opacity.reshape(-1, 1)
     mask = (neural_opacity > 0.0).view(-1)
     opacity = neural_opacity[mask]
-    color = torch.sigmoid(run(mlps[1])).reshape(-1, 3)
-    scale_rot = run(mlps[2]).reshape(-1, 7)
+    color = torch.sigmoid(run(1)).reshape(-1, 3)
+    scale_rot = run(2).reshape(-1, 7)
     cat = torch.cat([scaling, anchor], dim=-1).repeat_interleave(k, dim=0)
     masked = torch.cat([cat, color, scale_rot, offsets.reshape(-1, 3)], dim=-1)[mask]
     scaling_repeat, repeat_anchor, color, scale_rot, offs = masked.split([6, 3, 3, 7, 3], dim=-1)

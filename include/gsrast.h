@@ -177,19 +177,25 @@ int gs_all_map_backward(int P, const float* means3D, const float* scales, const 
 
 /* Replaces the body of generate_neural_gaussians (gaussian_renderer/__init__.py:789-899) in the reference's
  * default configuration (arguments/__init__.py:94-124: feat_dim 32, no feature bank, no appearance embedding, no
- * distance or level inputs, dist2level 'round'), on the anchors already selected by visible_mask (:794-798):
+ * distance or level inputs, dist2level 'round'; the options further down add to it), on the anchors already
+ * selected by visible_mask (:794-798):
  *   x = [feat, (anchor - campos) / |anchor - campos|]                                   (:801-828)
  *   neural_opacity = mlp_opacity(x), mask = neural_opacity > 0                          (:841-858)
  *   color = mlp_color(x), scale_rot = mlp_cov(x), and for the selected offsets, in (anchor, offset) order,
  *   xyz = anchor + offset * scaling[:3], scaling = scaling[3:] * sigmoid(scale_rot[:3]),
  *   rot = normalize(scale_rot[3:7])                                                     (:866-896)
- * mlp_params: 12 device pointers, {W1 (32x35), b1 (32), W2 (out x 32), b2 (out)} of mlp_opacity (out = n_offsets,
+ * mlp_params: 12 device pointers, {W1 (32x35; see input_flags), b1 (32), W2 (out x 32), b2 (out)} of mlp_opacity (out = n_offsets,
  * Tanh), mlp_color (3 n_offsets, Sigmoid) and mlp_cov (7 n_offsets), as nn.Linear stores them
  * (scene/gaussian_model.py:131-149).  anchor (N,3), feat (N,32), offsets (N,n_offsets,3), scaling (N,6) = the
  * activated get_scaling, campos (3).  n_offsets must satisfy gs_neural_supported().
  * opacity_scale (N floats, or NULL for none) serves dist2level 'progressive' (:844-848): neural_opacity =
  * mlp_opacity(x) * opacity_scale[anchor], where the caller passes _prog_ratio with 1 for the anchors outside
  * transition_mask; it must be positive wherever the product is (the reference's lies in (0, 1]).
+ * input_flags / level serve the MLPs' optional inputs (:824-829, :839-877; scene/gaussian_model.py:118-149):
+ * bit 0 / 1 / 2 (add_opacity_dist / add_color_dist / add_cov_dist) = that MLP takes the distance
+ * |anchor - campos| as input column 35, bit 3 (add_level) = all three take level[anchor] (N floats) as their last
+ * input column; an MLP's W1 is then 32 x 36 or 32 x 37, and so is its gradient.  0 and NULL otherwise.  The
+ * distance carries a gradient to the anchor, the level none.
  *
  * Step 1, gs_neural_opacity_forward: writes neural_opacity (N*n_offsets), mask (u8, N*n_offsets) and
  * first (u32, N: selected offsets of all earlier anchors), and returns their number in *num_selected (the host
@@ -205,22 +211,23 @@ int gs_neural_supported(int n_offsets);
 size_t gs_neural_workspace_bytes(int64_t num_anchors, int n_offsets);
 int gs_neural_opacity_forward(int64_t num_anchors, int n_offsets, const float* anchor, const float* feat,
                               const float* campos, const float* const* mlp_params, const float* opacity_scale,
-                              float* neural_opacity, uint8_t* mask, uint32_t* first, void* workspace,
-                              size_t workspace_bytes, int64_t* num_selected, gs_stream_t stream);
+                              const float* level, int input_flags, float* neural_opacity, uint8_t* mask,
+                              uint32_t* first, void* workspace, size_t workspace_bytes, int64_t* num_selected,
+                              gs_stream_t stream);
 int gs_neural_gaussians_forward(int64_t num_anchors, int n_offsets, int64_t num_selected, const float* anchor,
                                 const float* feat, const float* offsets, const float* scaling, const float* campos,
-                                const float* neural_opacity, const uint32_t* first, const void* workspace,
-                                size_t workspace_bytes, float* xyz, float* color, float* opacity,
-                                float* scaling_out, float* rot, float* aux, gs_stream_t stream);
+                                const float* level, const float* neural_opacity, const uint32_t* first,
+                                const void* workspace, size_t workspace_bytes, float* xyz, float* color,
+                                float* opacity, float* scaling_out, float* rot, float* aux, gs_stream_t stream);
 size_t gs_neural_backward_workspace_bytes(int64_t num_anchors, int n_offsets);
 int gs_neural_backward(int64_t num_anchors, int n_offsets, int64_t num_selected, const float* anchor,
                        const float* feat, const float* offsets, const float* scaling, const float* campos,
-                       const float* const* mlp_params, const float* opacity_scale, const float* neural_opacity,
-                       const uint32_t* first, const float* color, const float* rot, const float* aux,
-                       const float* dL_dxyz, const float* dL_dcolor, const float* dL_dopacity,
-                       const float* dL_dscaling, const float* dL_drot, float* d_anchor, float* d_feat,
-                       float* d_offsets, float* d_scaling, float* const* d_mlp_params, void* workspace,
-                       size_t workspace_bytes, gs_stream_t stream);
+                       const float* const* mlp_params, const float* opacity_scale, const float* level,
+                       int input_flags, const float* neural_opacity, const uint32_t* first, const float* color,
+                       const float* rot, const float* aux, const float* dL_dxyz, const float* dL_dcolor,
+                       const float* dL_dopacity, const float* dL_dscaling, const float* dL_drot, float* d_anchor,
+                       float* d_feat, float* d_offsets, float* d_scaling, float* const* d_mlp_params,
+                       void* workspace, size_t workspace_bytes, gs_stream_t stream);
 
 /* Replaces pixelwise_l1_with_mask and pixelwise_ssim_with_mask (utils/loss_utils.py:88-132, 11x11 Gaussian
  * window of create_window :27-43, zero padding; called at gaussian_renderer/loss_distribution.py:267-279).

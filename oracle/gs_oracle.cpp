@@ -1351,12 +1351,23 @@ void oracle_ssim_l1_bwd(int C, int H, int W, const float* img1, const float* img
 struct MlpView {
   const float *W1, *b1, *W2, *b2;
   int out;
+  int in;         // input width: 35, +1 with the distance, +1 with the level
+  bool has_dist;  // column 35 is the distance |anchor - campos|
+  bool has_level; // the last column is the anchor's level
 };
+
+// input_flags: bit 0 / 1 / 2 = the opacity / color / cov MLP takes the distance (add_opacity_dist,
+// add_color_dist, add_cov_dist, :839-877), bit 3 = all three take the level (add_level, :824-829)
+static MlpView mlp_view(const float* W1, const float* b1, const float* W2, const float* b2, int out, int m,
+                        int input_flags) {
+  const bool d = (input_flags >> m) & 1, l = (input_flags >> 3) & 1;
+  return MlpView{W1, b1, W2, b2, out, 35 + (d ? 1 : 0) + (l ? 1 : 0), d, l};
+}
 
 static void mlp_forward(const MlpView& m, const float* x, float* hidden, float* out) {
   for (int h = 0; h < 32; h++) {
     float a = m.b1[h];
-    for (int i = 0; i < 35; i++) a += m.W1[h * 35 + i] * x[i];
+    for (int i = 0; i < m.in; i++) a += m.W1[h * m.in + i] * x[i];
     hidden[h] = a > 0.f ? a : 0.f;
   }
   for (int o = 0; o < m.out; o++) {
@@ -1366,12 +1377,24 @@ static void mlp_forward(const MlpView& m, const float* x, float* hidden, float* 
   }
 }
 
-static void neural_input(const float* anchor, const float* feat, const float* campos, float* x, float* dist) {
+// x = [feat, view direction, distance, level] (37 values; cat_local_view, :824-829)
+static void neural_input(const float* anchor, const float* feat, const float* campos, float level, float* x,
+                         float* dist) {
   for (int i = 0; i < 32; i++) x[i] = feat[i];
   const float v[3] = {anchor[0] - campos[0], anchor[1] - campos[1], anchor[2] - campos[2]};
   const float d = sqrtf((v[0] * v[0] + v[1] * v[1]) + v[2] * v[2]);
   x[32] = v[0] / d; x[33] = v[1] / d; x[34] = v[2] / d;
+  x[35] = d;
+  x[36] = level;
   *dist = d;
+}
+
+// the columns an MLP takes of x, in its own order
+static void mlp_input(const MlpView& m, const float* x, float* xm) {
+  for (int i = 0; i < 35; i++) xm[i] = x[i];
+  int c = 35;
+  if (m.has_dist) xm[c++] = x[35];
+  if (m.has_level) xm[c++] = x[36];
 }
 
 // dense per-slot results: neural_opacity (N*k), mask (N*k), color (N*k*3, after sigmoid), scale_rot (N*k*7)
@@ -1379,23 +1402,28 @@ void oracle_neural_mlp_fwd(int N, int k, const float* anchor, const float* feat,
                            const float* W1o, const float* b1o, const float* W2o, const float* b2o,
                            const float* W1c, const float* b1c, const float* W2c, const float* b2c,
                            const float* W1v, const float* b1v, const float* W2v, const float* b2v,
-                           const float* prog, float* neural_opacity, uint8_t* mask, float* color,
-                           float* scale_rot) {
-  const MlpView mo{W1o, b1o, W2o, b2o, k}, mc{W1c, b1c, W2c, b2c, 3 * k}, mv{W1v, b1v, W2v, b2v, 7 * k};
+                           const float* prog, const float* level, int input_flags, float* neural_opacity,
+                           uint8_t* mask, float* color, float* scale_rot) {
+  const MlpView mo = mlp_view(W1o, b1o, W2o, b2o, k, 0, input_flags),
+                mc = mlp_view(W1c, b1c, W2c, b2c, 3 * k, 1, input_flags),
+                mv = mlp_view(W1v, b1v, W2v, b2v, 7 * k, 2, input_flags);
 #pragma omp parallel for schedule(static)
   for (int a = 0; a < N; a++) {
-    float x[35], dist, hid[32];
-    neural_input(anchor + 3 * (size_t)a, feat + 32 * (size_t)a, campos, x, &dist);
+    float x[37], xm[37], dist, hid[32];
+    neural_input(anchor + 3 * (size_t)a, feat + 32 * (size_t)a, campos, level ? level[a] : 0.f, x, &dist);
     std::vector<float> out(7 * k);
-    mlp_forward(mo, x, hid, out.data());
+    mlp_input(mo, x, xm);
+    mlp_forward(mo, xm, hid, out.data());
     for (int j = 0; j < k; j++) {
       const float t = prog ? tanhf(out[j]) * prog[a] : tanhf(out[j]);
       neural_opacity[(size_t)a * k + j] = t;
       mask[(size_t)a * k + j] = t > 0.f;
     }
-    mlp_forward(mc, x, hid, out.data());
+    mlp_input(mc, x, xm);
+    mlp_forward(mc, xm, hid, out.data());
     for (int j = 0; j < 3 * k; j++) color[(size_t)a * 3 * k + j] = 1.0f / (1.0f + expf(-out[j]));
-    mlp_forward(mv, x, hid, out.data());
+    mlp_input(mv, x, xm);
+    mlp_forward(mv, xm, hid, out.data());
     for (int j = 0; j < 7 * k; j++) scale_rot[(size_t)a * 7 * k + j] = out[j];
   }
 }
@@ -1434,29 +1462,32 @@ void oracle_neural_bwd(int N, int k, const float* anchor, const float* feat, con
                        const float* W1o, const float* b1o, const float* W2o, const float* b2o,
                        const float* W1c, const float* b1c, const float* W2c, const float* b2c,
                        const float* W1v, const float* b1v, const float* W2v, const float* b2v, const float* prog,
-                       const float* g_xyz, const float* g_col, const float* g_opacity, const float* g_scal,
+                       const float* level, int input_flags, const float* g_xyz, const float* g_col, const float* g_opacity, const float* g_scal,
                        const float* g_rot, float* d_anchor, float* d_feat, float* d_offsets, float* d_scaling,
                        float* dW1o, float* db1o, float* dW2o, float* db2o, float* dW1c, float* db1c, float* dW2c,
                        float* db2c, float* dW1v, float* db1v, float* dW2v, float* db2v) {
-  const MlpView ms[3] = {{W1o, b1o, W2o, b2o, k}, {W1c, b1c, W2c, b2c, 3 * k}, {W1v, b1v, W2v, b2v, 7 * k}};
+  const MlpView ms[3] = {mlp_view(W1o, b1o, W2o, b2o, k, 0, input_flags),
+                         mlp_view(W1c, b1c, W2c, b2c, 3 * k, 1, input_flags),
+                         mlp_view(W1v, b1v, W2v, b2v, 7 * k, 2, input_flags)};
   float* dW1s[3] = {dW1o, dW1c, dW1v};
   float* db1s[3] = {db1o, db1c, db1v};
   float* dW2s[3] = {dW2o, dW2c, dW2v};
   float* db2s[3] = {db2o, db2c, db2v};
   std::vector<std::vector<double>> aW1(3), ab1(3), aW2(3), ab2(3);
   for (int m = 0; m < 3; m++) {
-    aW1[m].assign(32 * 35, 0.0); ab1[m].assign(32, 0.0);
+    aW1[m].assign(32 * (size_t)ms[m].in, 0.0); ab1[m].assign(32, 0.0);
     aW2[m].assign((size_t)ms[m].out * 32, 0.0); ab2[m].assign(ms[m].out, 0.0);
   }
   size_t r = 0;
   for (int a = 0; a < N; a++) {
-    float x[35], dist, hid[3][32];
-    neural_input(anchor + 3 * (size_t)a, feat + 32 * (size_t)a, campos, x, &dist);
+    float x[37], xm[3][37], dist, hid[3][32];
+    neural_input(anchor + 3 * (size_t)a, feat + 32 * (size_t)a, campos, level ? level[a] : 0.f, x, &dist);
     std::vector<float> out[3], gout[3];
     for (int m = 0; m < 3; m++) {
       out[m].resize(ms[m].out);
       gout[m].assign(ms[m].out, 0.f);
-      mlp_forward(ms[m], x, hid[m], out[m].data());
+      mlp_input(ms[m], x, xm[m]);
+      mlp_forward(ms[m], xm[m], hid[m], out[m].data());
     }
     const float* sc = scaling + 6 * (size_t)a;
     float da[3] = {0.f, 0.f, 0.f}, dsc[6] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
@@ -1495,8 +1526,8 @@ void oracle_neural_bwd(int N, int k, const float* anchor, const float* feat, con
       r++;
     }
     // through the three MLPs
-    float dx[35];
-    for (int i = 0; i < 35; i++) dx[i] = 0.f;
+    float dx[36];  // features, view direction, distance (the level is an integer-valued buffer)
+    for (int i = 0; i < 36; i++) dx[i] = 0.f;
     for (int m = 0; m < 3; m++) {
       float dh[32];
       for (int h = 0; h < 32; h++) dh[h] = 0.f;
@@ -1512,9 +1543,10 @@ void oracle_neural_bwd(int N, int k, const float* anchor, const float* feat, con
       for (int h = 0; h < 32; h++) {
         if (!(hid[m][h] > 0.f)) continue;  // ReLU
         ab1[m][h] += dh[h];
-        for (int i = 0; i < 35; i++) {
-          aW1[m][h * 35 + i] += (double)dh[h] * x[i];
-          dx[i] += ms[m].W1[h * 35 + i] * dh[h];
+        const int in = ms[m].in;
+        for (int i = 0; i < in; i++) {
+          aW1[m][h * in + i] += (double)dh[h] * xm[m][i];
+          if (i < 35 || (i == 35 && ms[m].has_dist)) dx[i] += ms[m].W1[h * in + i] * dh[h];
         }
       }
     }
@@ -1522,11 +1554,13 @@ void oracle_neural_bwd(int N, int k, const float* anchor, const float* feat, con
     // view direction v/|v|: d v = (g - n (n.g)) / |v|
     const float nv[3] = {x[32], x[33], x[34]};
     const float ng = (nv[0] * dx[32] + nv[1] * dx[33]) + nv[2] * dx[34];
-    for (int c = 0; c < 3; c++) d_anchor[3 * (size_t)a + c] = da[c] + (dx[32 + c] - nv[c] * ng) / dist;
+    // and the distance |v|: d v = n * g
+    for (int c = 0; c < 3; c++)
+      d_anchor[3 * (size_t)a + c] = (da[c] + (dx[32 + c] - nv[c] * ng) / dist) + nv[c] * dx[35];
     for (int c = 0; c < 6; c++) d_scaling[6 * (size_t)a + c] = dsc[c];
   }
   for (int m = 0; m < 3; m++) {
-    for (int i = 0; i < 32 * 35; i++) dW1s[m][i] = (float)aW1[m][i];
+    for (int i = 0; i < 32 * ms[m].in; i++) dW1s[m][i] = (float)aW1[m][i];
     for (int i = 0; i < 32; i++) db1s[m][i] = (float)ab1[m][i];
     for (size_t i = 0; i < (size_t)ms[m].out * 32; i++) dW2s[m][i] = (float)aW2[m][i];
     for (int i = 0; i < ms[m].out; i++) db2s[m][i] = (float)ab2[m][i];

@@ -409,27 +409,34 @@ def morton(p, mn, mx):
     return int(lib().oracle_morton(_p(p), _p(mn), _p(mx)))
 
 
-def _mlp_args(mlps):
-    """mlps: three (W1 (32,35), b1 (32), W2 (out,32), b2 (out)) tuples in the order opacity, color, cov."""
+def _mlp_args(mlps, input_flags=0):
+    """mlps: three (W1 (32, 35 + extra inputs), b1 (32), W2 (out,32), b2 (out)) tuples in the order opacity, color,
+    cov; extra inputs of MLP m: the distance if bit m of input_flags is set, the level if bit 3 is."""
     flat = []
-    for W1, b1, W2, b2 in mlps:
+    for m, (W1, b1, W2, b2) in enumerate(mlps):
+        assert W1.shape == (32, 35 + ((input_flags >> m) & 1) + ((input_flags >> 3) & 1)), W1.shape
         flat += [_f32(W1), _f32(b1), _f32(W2), _f32(b2)]
     return flat
 
 
-def neural_gaussians_fwd(anchor, feat, offsets, scaling, campos, mlps, prog=None):
+def neural_gaussians_fwd(anchor, feat, offsets, scaling, campos, mlps, prog=None, level=None, input_flags=0):
     """generate_neural_gaussians (gaussian_renderer/__init__.py:789-899), default configuration, on the anchors
     already selected by visible_mask; prog (N), if given, is the per-anchor factor of dist2level 'progressive'
-    (:844-848).  Returns (xyz, color, opacity, scaling, rot, neural_opacity, mask)."""
+    (:844-848); input_flags / level: the MLPs' optional distance and level inputs (add_opacity_dist = 1,
+    add_color_dist = 2, add_cov_dist = 4, add_level = 8; :824-877).
+    Returns (xyz, color, opacity, scaling, rot, neural_opacity, mask)."""
     anchor, feat, offsets, scaling = _f32(anchor), _f32(feat), _f32(offsets), _f32(scaling)
     cp = _f32(campos).reshape(3)
     N, k = anchor.shape[0], offsets.shape[1]
-    w = _mlp_args(mlps)
+    w = _mlp_args(mlps, input_flags)
+    lv = None if level is None else _f32(level).reshape(N)
+    assert lv is not None or not (input_flags & 8)
     nop, mask = np.zeros((N * k, 1), np.float32), np.zeros(N * k, np.uint8)
     col, sr = np.zeros((N * k, 3), np.float32), np.zeros((N * k, 7), np.float32)
     pg = None if prog is None else _f32(prog).reshape(N)
     lib().oracle_neural_mlp_fwd(C.c_int(N), C.c_int(k), _p(anchor), _p(feat), _p(cp), *[_p(x) for x in w],
-                                None if pg is None else _p(pg), _p(nop), _p(mask), _p(col), _p(sr))
+                                None if pg is None else _p(pg), None if lv is None else _p(lv),
+                                C.c_int(input_flags), _p(nop), _p(mask), _p(col), _p(sr))
     S = int(mask.sum())
     xyz, c, op = np.zeros((S, 3), np.float32), np.zeros((S, 3), np.float32), np.zeros((S, 1), np.float32)
     sc, rot = np.zeros((S, 3), np.float32), np.zeros((S, 4), np.float32)
@@ -441,19 +448,21 @@ def neural_gaussians_fwd(anchor, feat, offsets, scaling, campos, mlps, prog=None
 
 
 def neural_gaussians_bwd(anchor, feat, offsets, scaling, campos, mlps, g_xyz, g_color, g_opacity, g_scaling, g_rot,
-                         prog=None):
+                         prog=None, level=None, input_flags=0):
     """Gradients of neural_gaussians_fwd's five compacted outputs: (d_anchor, d_feat, d_offsets, d_scaling,
     [12 weight gradients in the order of mlps])."""
     anchor, feat, offsets, scaling = _f32(anchor), _f32(feat), _f32(offsets), _f32(scaling)
     cp = _f32(campos).reshape(3)
     N, k = anchor.shape[0], offsets.shape[1]
-    w = _mlp_args(mlps)
+    w = _mlp_args(mlps, input_flags)
+    lv = None if level is None else _f32(level).reshape(N)
     gs = [_f32(g_xyz), _f32(g_color), _f32(g_opacity), _f32(g_scaling), _f32(g_rot)]
     da, df = np.zeros((N, 3), np.float32), np.zeros((N, 32), np.float32)
     do, ds = np.zeros((N, k, 3), np.float32), np.zeros((N, 6), np.float32)
     dw = [np.zeros_like(x) for x in w]
     pg = None if prog is None else _f32(prog).reshape(N)
     lib().oracle_neural_bwd(C.c_int(N), C.c_int(k), _p(anchor), _p(feat), _p(offsets), _p(scaling), _p(cp),
-                            *[_p(x) for x in w], None if pg is None else _p(pg), *[_p(x) for x in gs], _p(da), _p(df), _p(do), _p(ds),
+                            *[_p(x) for x in w], None if pg is None else _p(pg), None if lv is None else _p(lv),
+                            C.c_int(input_flags), *[_p(x) for x in gs], _p(da), _p(df), _p(do), _p(ds),
                             *[_p(x) for x in dw])
     return da, df, do, ds, dw

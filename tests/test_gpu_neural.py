@@ -105,6 +105,41 @@ def test_progressive_opacity_factor_matches_oracle(orc, N, k, seed):
         assert _rel(t.grad.cpu().numpy(), w) <= 2e-5, i
 
 
+@pytest.mark.parametrize("N,k,seed,flags", [(600, 10, 30, 15), (100, 5, 31, 1), (100, 4, 32, 2), (100, 3, 33, 4),
+                                            (333, 10, 34, 8), (150, 16, 35, 13), (64, 1, 36, 7)])
+def test_distance_and_level_inputs_match_oracle(orc, N, k, seed, flags):
+    """add_opacity_dist = 1, add_color_dist = 2, add_cov_dist = 4, add_level = 8
+    (gaussian_renderer/__init__.py:824-829, :839-877)."""
+    from gs_neural import neural_gaussians
+    s = gs_scenes.make_anchor_scene(N, k, seed, input_flags=flags)
+    anchor, feat, offsets, scaling, campos, mlps = _to_dev(s, grad=True)
+    out = neural_gaussians(anchor, feat, offsets, scaling, campos, *mlps, level=s["level"].to(DEV),
+                           input_flags=flags)
+    want = orc.neural_gaussians_fwd(*_np_args(s), level=s["level"].numpy(), input_flags=flags)
+    got = [o.detach().cpu().numpy() for o in out]
+    assert np.abs(got[5] - want[5]).max() <= 5e-6
+    differ = got[6] != want[6]
+    assert np.abs(want[5].ravel()[differ]).max(initial=0.0) <= 5e-6
+    both = got[6] & want[6]
+    for g, w, c in zip(got[:5], want[:5], (3, 3, 1, 3, 4)):
+        assert _rel(_dense(g, got[6], c)[both], _dense(w, want[6], c)[both]) <= 1e-5
+    if differ.any():
+        return
+    S = int(got[6].sum())
+    gen = torch.Generator().manual_seed(seed)
+    ups = [torch.randn(S, c, generator=gen) for c in (3, 3, 1, 3, 4)]
+    sum((o * u.to(DEV)).sum() for o, u in zip(out[:5], ups)).backward()
+    wd = orc.neural_gaussians_bwd(*_np_args(s), *[u.numpy() for u in ups], level=s["level"].numpy(),
+                                  input_flags=flags)
+    for name, t, w in zip(("anchor", "feat", "offsets", "scaling"), (anchor, feat, offsets, scaling), wd[:4]):
+        assert t.grad.shape == t.shape
+        assert _rel(t.grad.cpu().numpy(), w) <= 2e-5, name
+    flat = [x for m in mlps for x in m]
+    for i, (t, w) in enumerate(zip(flat, wd[4])):
+        assert t.grad.shape == t.shape
+        assert _rel(t.grad.cpu().numpy(), w) <= 3e-5, i
+
+
 def test_no_anchor_and_nothing_selected():
     from gs_neural import neural_gaussians
     s = gs_scenes.make_anchor_scene(50, 10, 0)
@@ -144,7 +179,7 @@ def test_training_size_against_torch_statements():
             total = total + (o[keep] * u[m][keep]).sum()
         total.backward()
     for o, r in zip(out[:5], ref[:5]):
-        assert float((o[both[out[6]]] - r[both[ref[6]]]).norm() / r.norm()) <= 5e-6
+        assert float((o.detach()[both[out[6]]] - r[both[ref[6]]]).norm() / r.norm()) <= 5e-6
     names = ("anchor", "feat", "offsets", "scaling")
     for name, x, y in zip(names, a1[:4], a2[:4]):
         assert float((x.grad - y.grad).norm() / y.grad.norm()) <= 1e-4, name
@@ -209,9 +244,79 @@ def test_drop_in_signature():
                                            cam.camera_center, [tuple(x.to(DEV) for x in m) for m in s["mlps"]], full)
     assert torch.equal(out[6], ref[6])
     assert float((out[5] - ref[5]).norm() / ref[5].norm()) <= 5e-6
-    pc.add_cov_dist = True
-    with pytest.raises(NotImplementedError):
-        generate_neural_gaussians(cam, pc, vis)
+
+
+def test_drop_in_with_distance_and_level_inputs():
+    """add_opacity_dist, add_cov_dist, add_level, the feature bank with the level and the appearance embedding behind
+    the level column, against the reference's statements run by torch (gaussian_renderer/__init__.py:800-896)."""
+    import types
+    import torch.nn as nn
+    from gs_neural import generate_neural_gaussians
+    N, k, A = 300, 10, 16
+    s = gs_scenes.make_anchor_scene(N, k, 17)
+    torch.manual_seed(5)
+    mlp_op = nn.Sequential(nn.Linear(37, 32), nn.ReLU(True), nn.Linear(32, k), nn.Tanh()).to(DEV)
+    mlp_cov = nn.Sequential(nn.Linear(37, 32), nn.ReLU(True), nn.Linear(32, 7 * k)).to(DEV)
+    mlp_col = nn.Sequential(nn.Linear(36 + A, 32), nn.ReLU(True), nn.Linear(32, 3 * k), nn.Sigmoid()).to(DEV)
+    bank = nn.Sequential(nn.Linear(4, 32), nn.ReLU(True), nn.Linear(32, 3), nn.Softmax(dim=1)).to(DEV)
+    emb = nn.Embedding(5, A).to(DEV)
+    leaf = lambda t: t.to(DEV).requires_grad_(True)
+    pc = types.SimpleNamespace(
+        use_feat_bank=True, appearance_dim=A, add_opacity_dist=True, add_color_dist=False, add_cov_dist=True,
+        add_level=True, dist2level="round", n_offsets=k, get_anchor=leaf(s["anchor"]),
+        get_anchor_feat=leaf(s["feat"]), _offset=leaf(s["offsets"]), get_scaling=leaf(s["scaling"]),
+        get_level=s["level"].to(DEV), get_opacity_mlp=mlp_op, get_color_mlp=mlp_col, get_cov_mlp=mlp_cov,
+        get_featurebank_mlp=bank, get_appearance=emb)
+    cam = types.SimpleNamespace(camera_center=s["campos"].to(DEV), uid=2)
+    vis = (torch.rand(N, generator=torch.Generator().manual_seed(3)) < 0.7).to(DEV)
+
+    def reference():
+        anchor, feat, level = pc.get_anchor[vis], pc.get_anchor_feat[vis], pc.get_level[vis]
+        grid_offsets, grid_scaling = pc._offset[vis], pc.get_scaling[vis]
+        ob_view = anchor - cam.camera_center
+        ob_dist = ob_view.norm(dim=1, keepdim=True)
+        ob_view = ob_view / ob_dist
+        bank_weight = bank(torch.cat([ob_view, level], dim=1)).unsqueeze(dim=1)
+        feat = feat.unsqueeze(dim=-1)
+        feat = feat[:, ::4, :1].repeat([1, 4, 1]) * bank_weight[:, :, :1] + \
+            feat[:, ::2, :1].repeat([1, 2, 1]) * bank_weight[:, :, 1:2] + feat[:, ::1, :1] * bank_weight[:, :, 2:]
+        feat = feat.squeeze(dim=-1)
+        cat_local_view = torch.cat([feat, ob_view, ob_dist, level], dim=1)
+        cat_local_view_wodist = torch.cat([feat, ob_view, level], dim=1)
+        camera_indicies = torch.ones_like(cat_local_view[:, 0], dtype=torch.long) * cam.uid
+        appearance = emb(camera_indicies)
+        neural_opacity = mlp_op(cat_local_view).reshape([-1, 1])
+        mask = (neural_opacity > 0.0).view(-1)
+        opacity = neural_opacity[mask]
+        color = mlp_col(torch.cat([cat_local_view_wodist, appearance], dim=1)).reshape([anchor.shape[0] * k, 3])
+        scale_rot = mlp_cov(cat_local_view).reshape([anchor.shape[0] * k, 7])
+        offsets = grid_offsets.view([-1, 3])
+        cat = torch.cat([grid_scaling, anchor], dim=-1).repeat_interleave(k, dim=0)
+        masked = torch.cat([cat, color, scale_rot, offsets], dim=-1)[mask]
+        scaling_repeat, repeat_anchor, color, scale_rot, offsets = masked.split([6, 3, 3, 7, 3], dim=-1)
+        scaling = scaling_repeat[:, 3:] * torch.sigmoid(scale_rot[:, :3])
+        rot = torch.nn.functional.normalize(scale_rot[:, 3:7])
+        xyz = repeat_anchor + offsets * scaling_repeat[:, :3]
+        return xyz, color, opacity, scaling, rot, neural_opacity, mask
+
+    params = [pc.get_anchor, pc.get_anchor_feat, pc._offset, pc.get_scaling, emb.weight] + \
+        [p for m in (mlp_op, mlp_col, mlp_cov, bank) for p in m.parameters()]
+    gen = torch.Generator().manual_seed(9)
+    results = []
+    for fn in (reference, lambda: generate_neural_gaussians(cam, pc, vis, is_training=True)):
+        for p in params:
+            p.grad = None
+        out = fn()
+        if not results:
+            ups = [torch.randn(out[0].shape[0], c, generator=gen).to(DEV) for c in (3, 3, 1, 3, 4)]
+        sum((o * u).sum() for o, u in zip(out[:5], ups)).backward()
+        results.append(([o.detach().clone() for o in out], [p.grad.detach().clone() for p in params]))
+    (ref_out, ref_grad), (got_out, got_grad) = results
+    assert torch.equal(ref_out[6], got_out[6])
+    for r, g in zip(ref_out[:6], got_out[:6]):
+        assert float((g - r).norm() / r.norm()) <= 1e-5
+    for i, (r, g) in enumerate(zip(ref_grad, got_grad)):
+        assert float((g - r).norm() / r.norm()) <= 2e-4, i
 
 
 def test_drop_in_with_appearance_embedding_and_feature_bank():

@@ -764,6 +764,42 @@ def test_neural_gaussians_progressive_factor_matches_float64_torch(orc, N, k, se
         assert _rel(g, w.grad.numpy()) < 1e-5, i
 
 
+@pytest.mark.parametrize("N,k,seed,flags", [(150, 10, 8, 15), (60, 5, 9, 1), (60, 4, 10, 2), (60, 3, 11, 4),
+                                            (90, 10, 12, 8), (70, 6, 13, 13)])
+def test_neural_gaussians_distance_and_level_inputs_match_float64_torch(orc, N, k, seed, flags):
+    """add_opacity_dist / add_color_dist / add_cov_dist / add_level (gaussian_renderer/__init__.py:824-877): the
+    first layers take the distance and the level as further columns; the distance carries a gradient to the anchor."""
+    s = gs_scenes.make_anchor_scene(N, k, seed, input_flags=flags)
+    n = lambda t: t.numpy()
+    mlps_np = [tuple(n(x) for x in m) for m in s["mlps"]]
+    args = (n(s["anchor"]), n(s["feat"]), n(s["offsets"]), n(s["scaling"]), n(s["campos"]), mlps_np)
+    fwd = orc.neural_gaussians_fwd(*args, level=n(s["level"]), input_flags=flags)
+    S = fwd[0].shape[0]
+    gen = torch.Generator().manual_seed(seed)
+    ups = [torch.randn(S, c, generator=gen) for c in (3, 3, 1, 3, 4)]
+    got = orc.neural_gaussians_bwd(*args, *[u.numpy() for u in ups], level=n(s["level"]), input_flags=flags)
+    leaf = lambda t: t.double().requires_grad_(True)
+    anchor, feat, offsets, scaling = leaf(s["anchor"]), leaf(s["feat"]), leaf(s["offsets"]), leaf(s["scaling"])
+    mlps = [tuple(leaf(x) for x in m) for m in s["mlps"]]
+    out = gs_scenes.neural_gaussians_torch(anchor, feat, offsets, scaling, s["campos"].double(), mlps,
+                                           level=s["level"].double(), input_flags=flags)
+    assert np.array_equal(out[6].numpy(), fwd[6])
+    for g, w in zip(fwd[:6], out[:6]):
+        assert _rel(g, w.detach().numpy()) < 2e-6
+    sum((o * u.double()).sum() for o, u in zip(out[:5], ups)).backward()
+    for name, g, w in zip(("anchor", "feat", "offsets", "scaling"), got[:4], (anchor, feat, offsets, scaling)):
+        assert _rel(g, w.grad.numpy()) < 1e-5, name
+    flat = [x for m in mlps for x in m]
+    for i, (g, w) in enumerate(zip(got[4], flat)):
+        assert g.shape == tuple(w.shape)
+        assert _rel(g, w.grad.numpy()) < 1e-5, i
+    # the optional inputs matter: without them the same weights' leading columns give another result
+    if flags:
+        plain = orc.neural_gaussians_fwd(*args[:5], [(m[0][:, :35].copy(), m[1], m[2], m[3]) for m in mlps_np])
+        same_selection = np.array_equal(plain[6], fwd[6])
+        assert not (same_selection and all(np.allclose(a, b, atol=1e-4) for a, b in zip(plain[:6], fwd[:6])))
+
+
 # ------------------------------------------------------ max-weight depth --
 
 def test_max_weight_depth_known_cases(orc):
