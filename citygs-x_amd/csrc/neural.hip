@@ -891,7 +891,7 @@ struct Launcher {
 }  // namespace
 
 // n_offsets values the kernels are instantiated for
-#define NG_FOR_EACH_K(X) X(1) X(2) X(3) X(4) X(5) X(6) X(8) X(10) X(12) X(16)
+#define NG_FOR_EACH_K(X) X(1) X(2) X(3) X(4) X(5) X(6) X(7) X(8) X(9) X(10) X(11) X(12) X(13) X(14) X(15) X(16)
 
 bool neural_supported(int k) {
   switch (k) {

@@ -36,7 +36,9 @@ def _dense(rows, mask, width):
 
 
 @pytest.mark.parametrize("N,k,seed", [(1000, 10, 0), (33, 10, 1), (1, 10, 2), (300, 5, 3), (97, 4, 4), (64, 16, 5),
-                                      (129, 1, 6), (70, 12, 7), (40, 3, 8), (45, 8, 9), (31, 2, 10), (200, 6, 11)])
+                                      (129, 1, 6), (70, 12, 7), (40, 3, 8), (45, 8, 9), (31, 2, 10), (200, 6, 11),
+                                      (90, 7, 12), (77, 9, 13), (66, 11, 14), (130, 13, 15), (55, 14, 16),
+                                      (100, 15, 17)])
 def test_forward_and_backward_match_oracle(orc, N, k, seed):
     from gs_neural import neural_gaussians
     s = gs_scenes.make_anchor_scene(N, k, seed)
