@@ -181,7 +181,7 @@ def test_training_size_against_torch_statements():
             total = total + (o[keep] * u[m][keep]).sum()
         total.backward()
     for o, r in zip(out[:5], ref[:5]):
-        assert float((o.detach()[both[out[6]]] - r[both[ref[6]]]).norm() / r.norm()) <= 5e-6
+        assert float((o.detach()[both[out[6]]] - r.detach()[both[ref[6]]]).norm() / r.detach().norm()) <= 5e-6
     names = ("anchor", "feat", "offsets", "scaling")
     for name, x, y in zip(names, a1[:4], a2[:4]):
         assert float((x.grad - y.grad).norm() / y.grad.norm()) <= 1e-4, name
