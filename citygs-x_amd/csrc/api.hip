@@ -447,14 +447,14 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
     // the histogram's grand total is the instance count: the host gets it from here, and the prefix over the
     // Gaussians below runs while the host is busy growing the binning buffer
     if (launch_bucket_count(P, width, height, radii, means2D, compute_locally, tiles_touched, bucket_table, ranges,
-                            sort_limit, total_slot, stream))
+                            sort_limit, total_slot, out_observe, stream))
       return 1;
   } else {
     StageScope _t("tile_count", stream);
     // also clears the tile ranges (cudaMemset of CR/rasterizer_impl.cu:687), which nothing reads before
     // identify_tile_ranges fills them
     launch_tile_count(P, width, height, radii, means2D, compute_locally, tiles_touched, stream, ranges,
-                      (int64_t)2 * T);
+                      (int64_t)2 * T, out_observe);
   }
   if (check_launch("tile_count", stream, dbg)) return 1;
   {

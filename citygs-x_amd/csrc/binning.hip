@@ -48,7 +48,8 @@ __device__ __forceinline__ uint32_t block_exclusive_scan(uint32_t v, uint32_t* s
 __global__ void __launch_bounds__(GS_BLOCK_1D)
 tile_count_kernel(int P, uint32_t gx, uint32_t gy, const int* __restrict__ radii,
                   const float2* __restrict__ means2D, const uint8_t* __restrict__ compute_locally,
-                  uint32_t* __restrict__ tiles_touched, uint32_t* __restrict__ zero_words, int64_t zero_count) {
+                  uint32_t* __restrict__ tiles_touched, uint32_t* __restrict__ zero_words, int64_t zero_count,
+                  int* __restrict__ zero_per_gaussian) {
   const int i = blockIdx.x * GS_BLOCK_1D + threadIdx.x;
   // optionally clears another array on the side (the tile ranges of the same call: saves a launch)
   for (int64_t j = i; j < zero_count; j += (int64_t)gridDim.x * GS_BLOCK_1D) zero_words[j] = 0u;
@@ -63,7 +64,10 @@ tile_count_kernel(int P, uint32_t gx, uint32_t gy, const int* __restrict__ radii
   const uint32_t cnt = walk_wave_rects(
       live, rc, gx, none, [&](uint32_t tile) { return compute_locally[tile] != 0; },
       [](const None&, uint32_t, uint32_t) {});
-  if (i < P) tiles_touched[i] = cnt;
+  if (i < P) {
+    tiles_touched[i] = cnt;
+    if (zero_per_gaussian != nullptr) zero_per_gaussian[i] = 0;
+  }
 }
 
 template <typename T>
@@ -215,12 +219,13 @@ tile_ranges_kernel(int64_t L, const uint64_t* __restrict__ keys, uint32_t* __res
 }  // namespace
 
 int launch_tile_count(int P, int W, int H, const int* radii, const float* means2D, const uint8_t* compute_locally,
-                      uint32_t* tiles_touched, hipStream_t stream, uint32_t* zero_words, int64_t zero_count) {
+                      uint32_t* tiles_touched, hipStream_t stream, uint32_t* zero_words, int64_t zero_count,
+                      int* zero_per_gaussian) {
   if (P <= 0) return 0;
   const uint32_t gx = (W + GS_TILE_X - 1) / GS_TILE_X, gy = (H + GS_TILE_Y - 1) / GS_TILE_Y;
   hipLaunchKernelGGL(tile_count_kernel, dim3((P + GS_BLOCK_1D - 1) / GS_BLOCK_1D), dim3(GS_BLOCK_1D), 0, stream, P,
                      gx, gy, radii, (const float2*)means2D, compute_locally, tiles_touched, zero_words,
-                     zero_words ? zero_count : 0);
+                     zero_words ? zero_count : 0, zero_per_gaussian);
   return 0;
 }
 

@@ -51,7 +51,7 @@ constexpr uint32_t GS_MAX_INSTANCES = 0x7FFFFFFEu;
 constexpr uint32_t GS_TOO_MANY_INSTANCES = 0x7FFFFFFFu;
 int launch_tile_count(int P, int W, int H, const int* radii, const float* means2D, const uint8_t* compute_locally,
                       uint32_t* tiles_touched, hipStream_t stream,
-                      uint32_t* zero_words = nullptr, int64_t zero_count = 0);
+                      uint32_t* zero_words = nullptr, int64_t zero_count = 0, int* zero_per_gaussian = nullptr);
 size_t scan_temp_bytes(int64_t n);
 // device word of a scan's workspace that is 1 after a scan whose exact total exceeds GS_MAX_INSTANCES, else 0
 const uint32_t* scan_overflow_word(const void* temp, int64_t n);
@@ -59,6 +59,8 @@ int launch_exclusive_sum_u8(int64_t n, const uint8_t* in, uint32_t* out, void* t
                             uint32_t* total_out = nullptr);
 // total_out, when given, is a host-visible word that receives the grand total as well (GS_TOO_MANY_INSTANCES if
 // the exact total exceeds GS_MAX_INSTANCES; the 32-bit sums themselves wrap around like the reference's)
+// (launch_tile_count and launch_bucket_count: zero_per_gaussian, when given, is an array of P words that the
+// counting kernel clears on the way)
 int launch_inclusive_sum(int64_t n, const uint32_t* in, uint32_t* out, void* temp, hipStream_t stream,
                          uint32_t* total_out = nullptr);
 int launch_exclusive_sum(int64_t n, const uint32_t* in, uint32_t* out, void* temp, hipStream_t stream);
@@ -77,7 +79,7 @@ size_t bucket_table_bytes(int T);
 // the lists of more than chunk_limit records are cut into (word 2)
 int launch_bucket_count(int P, int W, int H, const int* radii, const float* means2D, const uint8_t* compute_locally,
                         uint32_t* tiles_touched, void* table, uint32_t* ranges, uint32_t chunk_limit,
-                        uint32_t* host_words, hipStream_t stream);
+                        uint32_t* host_words, int* zero_per_gaussian, hipStream_t stream);
 int launch_bucket_scatter(int P, int W, int H, const float* means2D, const float* depths, const uint32_t* offsets,
                           const int* radii, const uint8_t* compute_locally, const void* table,
                           const uint32_t* ranges, uint64_t* records, uint32_t* gauss_of_emission,

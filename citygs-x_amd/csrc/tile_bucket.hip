@@ -38,7 +38,8 @@ __host__ __device__ inline int bucket_blocks(int P) {
 __global__ void __launch_bounds__(BK_THREADS)
 bucket_count_kernel(int P, int per_block, uint32_t gx, uint32_t gy, const int* __restrict__ radii,
                     const float2* __restrict__ means2D, const uint8_t* __restrict__ compute_locally,
-                    uint32_t* __restrict__ tiles_touched, uint32_t* __restrict__ table) {
+                    uint32_t* __restrict__ tiles_touched, uint32_t* __restrict__ table,
+                    int* __restrict__ zero_per_gaussian) {
   extern __shared__ uint32_t s_hist[];
   const uint32_t T = gx * gy;
   uint8_t* s_local = reinterpret_cast<uint8_t*>(s_hist + T);  // the tile mask, read once per visited tile
@@ -69,7 +70,11 @@ bucket_count_kernel(int P, int per_block, uint32_t gx, uint32_t gy, const int* _
       const uint32_t cnt = walk_wave_rects(
           live, rc, gx, none, [&](uint32_t tile) { return s_local[tile] != 0; },
           [&](const None&, uint32_t tile, uint32_t) { atomicAdd(&s_hist[tile], 1u); });
-      if (i < last) tiles_touched[i] = cnt;
+      if (i < last) {
+        tiles_touched[i] = cnt;
+        // an array of one word per Gaussian that the caller wants cleared on the way (saves a launch)
+        if (zero_per_gaussian != nullptr) zero_per_gaussian[i] = 0;
+      }
     }
   }
   __syncthreads();
@@ -536,7 +541,7 @@ size_t bucket_table_bytes(int T) { return (((size_t)BK_MAX_BLOCKS + 2) * (size_t
 
 int launch_bucket_count(int P, int W, int H, const int* radii, const float* means2D, const uint8_t* compute_locally,
                         uint32_t* tiles_touched, void* table, uint32_t* ranges, uint32_t chunk_limit,
-                        uint32_t* host_words, hipStream_t stream) {
+                        uint32_t* host_words, int* zero_per_gaussian, hipStream_t stream) {
   if (P <= 0) return 0;
   if (chunk_limit == 0 || chunk_limit > (uint32_t)TILE_SORT_LARGE) chunk_limit = TILE_SORT_LARGE;
   const uint32_t gx = (W + GS_TILE_X - 1) / GS_TILE_X, gy = (H + GS_TILE_Y - 1) / GS_TILE_Y;
@@ -559,7 +564,7 @@ int launch_bucket_count(int P, int W, int H, const int* radii, const float* mean
   uint32_t* tab = (uint32_t*)table;
   uint32_t* totals = tab + (size_t)BK_MAX_BLOCKS * T;
   hipLaunchKernelGGL(bucket_count_kernel, dim3(nb), dim3(BK_THREADS), lds, stream, P, per, gx, gy, radii,
-                     (const float2*)means2D, compute_locally, tiles_touched, tab);
+                     (const float2*)means2D, compute_locally, tiles_touched, tab, zero_per_gaussian);
   hipLaunchKernelGGL(bucket_columns_kernel, dim3((T + COL_TILES - 1) / COL_TILES), dim3(COL_TILES * COL_RUNS), 0, stream, nb, T,
                      tab, totals);
   hipLaunchKernelGGL(bucket_ranges_kernel, dim3(1), dim3(1024), 0, stream, T, chunk_limit, totals, ranges, totals + T,

@@ -185,7 +185,7 @@ def render_gaussians(background, image_height, image_width, means2D, depths, rad
                 torch.zeros(tiles, **i32), torch.zeros(0, **i32), torch.zeros(NUM_ALL_MAP, H, W, **f32),
                 torch.zeros(1, H, W, **f32), empty, empty.clone(), empty.clone())
     out_color = torch.empty(NUM_CHANNELS, H, W, **f32)
-    out_observe = torch.zeros(P, **i32)
+    out_observe = torch.empty(P, **i32)  # cleared by the call itself
     out_all_map = torch.empty(NUM_ALL_MAP, H, W, **f32) if geo else torch.zeros(NUM_ALL_MAP, H, W, **f32)
     out_plane_depth = torch.empty(1, H, W, **f32) if geo else torch.zeros(1, H, W, **f32)
     n_render = torch.empty(tiles, **i32)

@@ -110,7 +110,8 @@ void gs_set_tile_sort_limits(int in_registers, int large_limit, int max_chunks);
  * does at :653) -> key emission -> 64-bit radix sort on 32+bits(tiles) bits
  * -> tile ranges -> blend -> per-tile statistics.
  * out_color (3,H,W); out_all_map (5,H,W) and out_plane_depth (1,H,W) are
- * written only when render_geo != 0; out_observe (P) int32 must arrive zeroed;
+ * written only when render_geo != 0; out_observe (P) int32 is cleared by the call
+ * (the reference's binding allocates it zeroed, rasterize_points.cu:305) and then counted;
  * n_render / n_consider / n_contrib are (tiles) int32, fully written.
  * *num_rendered (host) receives the instance count R.
  * out_max_weight_depth (H*W, optional, NULL to skip) has no counterpart in the reference: per pixel the view-space
