@@ -543,6 +543,12 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
         if (launch_sort_pairs_u64(R, k_start, k_partner, e_start, e_partner, end_bit, sort_temp, stream)) return 1;
       }
       if (check_launch("sort_pairs", stream, dbg)) return 1;
+      if (dbg) {  // (sort_temp is 256-byte aligned already)
+        uint32_t word = 0;
+        GS_HIP_TRY(hipMemcpyAsync(&word, sort_error_word(sort_temp), sizeof(uint32_t), hipMemcpyDeviceToHost, stream));
+        GS_HIP_TRY(hipStreamSynchronize(stream));
+        GS_REQUIRE(word == 0u, "gs_render_forward: the radix sort's bounded look-back wait ran out");
+      }
     }
     {
       StageScope _t("identify_tile_ranges", stream);
@@ -984,6 +990,20 @@ int gs_sort_pairs_u64(int64_t n, uint64_t* keys_in, uint64_t* keys_out, uint32_t
     if (launch_sort_pairs_u64(n, keys_out, keys_in, vals_out, vals_in, end_bit, temp, stream)) return 1;
   }
   return check_launch("sort_pairs_u64", stream, false);
+}
+
+int gs_sort_status(const void* workspace, gs_stream_t stream_) {
+  hipStream_t stream = (hipStream_t)stream_;
+  GS_REQUIRE(workspace, "gs_sort_status: null workspace");
+  const void* temp = align_ptr((const char*)workspace, 256);
+  uint32_t word = 0;
+  GS_HIP_TRY(hipMemcpyAsync(&word, sort_error_word(temp), sizeof(uint32_t), hipMemcpyDeviceToHost, stream));
+  GS_HIP_TRY(hipStreamSynchronize(stream));
+  if (word != 0u) {
+    set_error("radix sort: a bounded wait on an earlier tile's digit counts ran out; the output is not sorted");
+    return 1;
+  }
+  return 0;
 }
 
 int gs_sort_pairs_u32(int64_t n, uint32_t* keys_in, uint32_t* keys_out, uint32_t* vals_in, uint32_t* vals_out,

@@ -139,6 +139,9 @@ int launch_tile_ranges(int64_t L, const uint64_t* keys_sorted, int T, uint32_t* 
 
 // ---- radix sort (stable, LSD, 8-bit digits) ----
 size_t sort_temp_bytes(int64_t n);
+// device word of a sort's workspace that is nonzero after a sort in which a bounded wait of the look-back ran out
+// (the order of the output is then not to be trusted)
+const uint32_t* sort_error_word(const void* temp);
 // Sorts on key bits [0, end_bit), ping-ponging between the (a) and (b) arrays
 // starting from (a).  With an odd number of 8-bit passes the sorted result
 // lands in (b), with an even number back in (a): sort_result_in_b() tells.

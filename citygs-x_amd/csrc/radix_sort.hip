@@ -452,6 +452,8 @@ int sort_pairs_impl(int64_t n, K* keys_a, K* keys_b, uint32_t* vals_a, uint32_t*
 
 size_t sort_temp_bytes(int64_t n) { return sort_layout(n).total_bytes; }
 
+const uint32_t* sort_error_word(const void* temp) { return (const uint32_t*)temp + MAX_PASSES * RADIX + MAX_PASSES; }
+
 int launch_sort_pairs_u64(int64_t n, uint64_t* keys_a, uint64_t* keys_b, uint32_t* vals_a, uint32_t* vals_b,
                           int end_bit, void* temp, hipStream_t stream) {
   return sort_pairs_impl<uint64_t>(n, keys_a, keys_b, vals_a, vals_b, end_bit, temp, stream);

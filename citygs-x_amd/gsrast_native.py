@@ -57,6 +57,7 @@ _SIGNATURES = {
     "gs_inclusive_sum": (_i, [_i64, _vp, _vp, _vp, _sz, _vp]),
     "gs_duplicate_with_keys": (_i, [_i, _i, _i] + [_vp] * 8),
     "gs_sort_workspace_bytes": (_sz, [_i64]),
+    "gs_sort_status": (_i, [_vp, _vp]),
     "gs_sort_pairs_u64": (_i, [_i64, _vp, _vp, _vp, _vp, _i, _vp, _sz, _vp]),
     "gs_sort_pairs_u32": (_i, [_i64, _vp, _vp, _vp, _vp, _i, _vp, _sz, _vp]),
     "gs_identify_tile_ranges": (_i, [_i64, _vp, _i, _vp, _vp]),

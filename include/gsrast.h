@@ -301,6 +301,11 @@ int gs_duplicate_with_keys(int P, int width, int height, const float* means2D, c
  * KNN/simple_knn.cu:210-213): stable.  The input arrays are clobbered; the
  * sorted pairs land in keys_out / vals_out. */
 size_t gs_sort_workspace_bytes(int64_t n);
+/* No counterpart in the reference.  A pass of the sort waits, with a bounded number of polls, for the digit counts
+ * of earlier tiles; if a wait ever ran out the sort sets a word in its workspace instead of hanging.
+ * gs_sort_status waits for the stream and returns 1 (with an error message) if the last sort that used this
+ * workspace set it, else 0.  gs_render_forward checks the word itself when debug != 0. */
+int gs_sort_status(const void* workspace, gs_stream_t stream);
 int gs_sort_pairs_u64(int64_t n, uint64_t* keys_in, uint64_t* keys_out, uint32_t* vals_in, uint32_t* vals_out,
                       int end_bit, void* workspace, size_t workspace_bytes, gs_stream_t stream);
 int gs_sort_pairs_u32(int64_t n, uint32_t* keys_in, uint32_t* keys_out, uint32_t* vals_in, uint32_t* vals_out,

@@ -116,6 +116,8 @@ def sort_pairs_u64(keys, vals, end_bit):
     ws = torch.empty(nb, dtype=torch.uint8, device=DEV)
     gn.check(lib.gs_sort_pairs_u64(n, ptr(kin), ptr(kout), ptr(vin), ptr(vout), end_bit, ptr(ws), nb, stream()),
              "gs_sort_pairs_u64")
+    if n > 0:
+        gn.check(lib.gs_sort_status(ptr(ws), stream()), "gs_sort_status")
     torch.cuda.synchronize()
     return kout, vout
 
@@ -128,6 +130,8 @@ def sort_pairs_u32(keys, vals, end_bit=32):
     ws = torch.empty(nb, dtype=torch.uint8, device=DEV)
     gn.check(lib.gs_sort_pairs_u32(n, ptr(kin), ptr(kout), ptr(vin), ptr(vout), end_bit, ptr(ws), nb, stream()),
              "gs_sort_pairs_u32")
+    if n > 0:
+        gn.check(lib.gs_sort_status(ptr(ws), stream()), "gs_sort_status")
     torch.cuda.synchronize()
     return kout, vout
 
