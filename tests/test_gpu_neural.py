@@ -220,7 +220,7 @@ def test_drop_in_signature():
                                            [tuple(x.to(DEV) for x in m) for m in s["mlps"]])
     assert torch.equal(out[6], ref[6])
     for o, r in zip(out[:6], ref[:6]):
-        assert float((o - r).norm() / r.norm()) <= 5e-6
+        assert float((o.detach() - r.detach()).norm() / r.detach().norm()) <= 5e-6
     (out[1].sum() + out[3].sum()).backward()
     for q in (pc.get_color_mlp, pc.get_cov_mlp):
         for lin in (q[0], q[2]):
@@ -238,7 +238,7 @@ def test_drop_in_signature():
                                            [tuple(x.to(DEV) for x in m) for m in s["mlps"]], prog)
     assert torch.equal(out[6], ref[6])
     for o, r in zip(out[:6], ref[:6]):
-        assert float((o - r).norm() / r.norm()) <= 5e-6
+        assert float((o.detach() - r.detach()).norm() / r.detach().norm()) <= 5e-6
     # and without a visibility mask
     out = generate_neural_gaussians(cam, pc, None, is_training=True)
     full = torch.where(pc.transition_mask[:, None], pc._prog_ratio, torch.ones_like(pc._prog_ratio))
@@ -387,7 +387,7 @@ def test_drop_in_with_appearance_embedding_and_feature_bank():
         else:
             assert torch.equal(out[6], first[6])
             for o, r in zip(first[:6], out[:6]):
-                assert float((o - r).norm() / r.norm()) <= 5e-6
+                assert float((o.detach() - r.detach()).norm() / r.detach().norm()) <= 5e-6
         torch.autograd.backward(list(out[:5]), ups)
         grads.append([p.grad.clone() for p in params])
     for i, (a, b) in enumerate(zip(*grads)):
