@@ -149,7 +149,8 @@ bucket_ranges_kernel(uint32_t T, uint32_t limit, const uint32_t* __restrict__ to
     const uint32_t c = v > limit ? (v + limit - 1u) / limit : 0u;
     longest = v > longest ? v : longest;
     const uint32_t inc = wave_inclusive_scan_u32(v, lane);
-    const uint32_t inc_chunks = wave_inclusive_scan_u32(c, lane);
+    // (a wave without a long list, the usual case, has nothing to scan)
+    const uint32_t inc_chunks = __ballot(c != 0u) != 0ull ? wave_inclusive_scan_u32(c, lane) : 0u;
     if (lane == 63) {
       s_wave[wave] = inc;
       s_wave_chunks[wave] = inc_chunks;
