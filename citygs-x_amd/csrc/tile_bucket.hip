@@ -137,20 +137,28 @@ __device__ __forceinline__ uint32_t wave_inclusive_scan_u32(uint32_t v, int lane
 __global__ void __launch_bounds__(1024)
 bucket_ranges_kernel(uint32_t T, uint32_t limit, const uint32_t* __restrict__ totals, uint32_t* __restrict__ ranges,
                      uint32_t* __restrict__ chunk_first, uint32_t* __restrict__ host_words) {
+  constexpr int ITEMS = 4;  // consecutive tiles per thread: the usual grids (up to 4096 tiles) take one round
   __shared__ uint32_t s_wave[16], s_wave_chunks[16], s_max[16];
   __shared__ double s_exact[16];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   uint32_t carry = 0, carry_chunks = 0, longest = 0;
   double exact = 0.0;  // the number of instances without the 32-bit wrap-around of the prefix sums
-  for (uint32_t start = 0; start < T; start += 1024) {
-    const uint32_t t = start + threadIdx.x;
-    const uint32_t v = t < T ? totals[t] : 0u;
-    exact += (double)v;
-    const uint32_t c = v > limit ? (v + limit - 1u) / limit : 0u;
-    longest = v > longest ? v : longest;
-    const uint32_t inc = wave_inclusive_scan_u32(v, lane);
+  for (uint32_t start = 0; start < T; start += 1024 * ITEMS) {
+    const uint32_t t0 = start + threadIdx.x * ITEMS;
+    uint32_t v[ITEMS], c[ITEMS], sum = 0, sum_chunks = 0;
+#pragma unroll
+    for (int q = 0; q < ITEMS; q++) v[q] = t0 + q < T ? totals[t0 + q] : 0u;
+#pragma unroll
+    for (int q = 0; q < ITEMS; q++) {
+      c[q] = v[q] > limit ? (v[q] + limit - 1u) / limit : 0u;
+      longest = v[q] > longest ? v[q] : longest;
+      exact += (double)v[q];
+      sum += v[q];
+      sum_chunks += c[q];
+    }
+    const uint32_t inc = wave_inclusive_scan_u32(sum, lane);
     // (a wave without a long list, the usual case, has nothing to scan)
-    const uint32_t inc_chunks = __ballot(c != 0u) != 0ull ? wave_inclusive_scan_u32(c, lane) : 0u;
+    const uint32_t inc_chunks = __ballot(sum_chunks != 0u) != 0ull ? wave_inclusive_scan_u32(sum_chunks, lane) : 0u;
     if (lane == 63) {
       s_wave[wave] = inc;
       s_wave_chunks[wave] = inc_chunks;
@@ -168,11 +176,16 @@ bucket_ranges_kernel(uint32_t T, uint32_t limit, const uint32_t* __restrict__ to
       all_chunks += sc;
     }
     __syncthreads();
-    const uint32_t begin = carry + base + inc - v;
-    if (t < T) {
-      ranges[2 * t] = v ? begin : 0u;
-      ranges[2 * t + 1] = v ? begin + v : 0u;
-      chunk_first[t] = carry_chunks + base_chunks + inc_chunks - c;
+    uint32_t begin = carry + base + inc - sum, begin_chunks = carry_chunks + base_chunks + inc_chunks - sum_chunks;
+#pragma unroll
+    for (int q = 0; q < ITEMS; q++) {
+      if (t0 + q < T) {
+        ranges[2 * (t0 + q)] = v[q] ? begin : 0u;
+        ranges[2 * (t0 + q) + 1] = v[q] ? begin + v[q] : 0u;
+        chunk_first[t0 + q] = begin_chunks;
+      }
+      begin += v[q];
+      begin_chunks += c[q];
     }
     carry += all;
     carry_chunks += all_chunks;
