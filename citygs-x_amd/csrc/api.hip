@@ -459,7 +459,9 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
   if (check_launch("tile_count", stream, dbg)) return 1;
   {
     StageScope _t("inclusive_sum", stream);
-    launch_inclusive_sum(P, tiles_touched, point_offsets, scan_temp, stream, bucketed ? nullptr : total_slot);
+    // (on the bucketed route the counting workgroups have summed their chunks already)
+    if (bucketed) launch_bucket_offsets(P, width, height, tiles_touched, bucket_table, point_offsets, stream);
+    else launch_inclusive_sum(P, tiles_touched, point_offsets, scan_temp, stream, total_slot);
   }
   if (check_launch("inclusive_sum", stream, dbg)) return 1;
 

@@ -80,6 +80,8 @@ size_t bucket_table_bytes(int T);
 int launch_bucket_count(int P, int W, int H, const int* radii, const float* means2D, const uint8_t* compute_locally,
                         uint32_t* tiles_touched, void* table, uint32_t* ranges, uint32_t chunk_limit,
                         uint32_t* host_words, int* zero_per_gaussian, hipStream_t stream);
+int launch_bucket_offsets(int P, int W, int H, const uint32_t* tiles_touched, void* table, uint32_t* point_offsets,
+                          hipStream_t stream);
 int launch_bucket_scatter(int P, int W, int H, const float* means2D, const float* depths, const uint32_t* offsets,
                           const int* radii, const uint8_t* compute_locally, const void* table,
                           const uint32_t* ranges, uint64_t* records, uint32_t* gauss_of_emission,

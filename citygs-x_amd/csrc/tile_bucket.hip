@@ -39,8 +39,10 @@ __global__ void __launch_bounds__(BK_THREADS)
 bucket_count_kernel(int P, int per_block, uint32_t gx, uint32_t gy, const int* __restrict__ radii,
                     const float2* __restrict__ means2D, const uint8_t* __restrict__ compute_locally,
                     uint32_t* __restrict__ tiles_touched, uint32_t* __restrict__ table,
-                    int* __restrict__ zero_per_gaussian) {
+                    uint32_t* __restrict__ block_sums, int* __restrict__ zero_per_gaussian) {
   extern __shared__ uint32_t s_hist[];
+  __shared__ uint32_t s_sum[BK_THREADS / GS_WAVE];
+  uint32_t my_sum = 0;  // tiles touched by this thread's Gaussians
   const uint32_t T = gx * gy;
   uint8_t* s_local = reinterpret_cast<uint8_t*>(s_hist + T);  // the tile mask, read once per visited tile
   for (uint32_t t = threadIdx.x; t < T; t += BK_THREADS) {
@@ -72,14 +74,24 @@ bucket_count_kernel(int P, int per_block, uint32_t gx, uint32_t gy, const int* _
           [&](const None&, uint32_t tile, uint32_t) { atomicAdd(&s_hist[tile], 1u); });
       if (i < last) {
         tiles_touched[i] = cnt;
+        my_sum += cnt;
         // an array of one word per Gaussian that the caller wants cleared on the way (saves a launch)
         if (zero_per_gaussian != nullptr) zero_per_gaussian[i] = 0;
       }
     }
   }
+#pragma unroll
+  for (int d = GS_WAVE / 2; d >= 1; d >>= 1) my_sum += __shfl_xor(my_sum, d, GS_WAVE);
+  if ((threadIdx.x & (GS_WAVE - 1)) == 0) s_sum[threadIdx.x / GS_WAVE] = my_sum;
   __syncthreads();
   uint32_t* row = table + (size_t)blockIdx.x * T;
   for (uint32_t t = threadIdx.x; t < T; t += BK_THREADS) row[t] = s_hist[t];
+  // the workgroup's share of the prefix sum over the Gaussians (bucket_offsets_kernel finishes it)
+  if (threadIdx.x == 0) {
+    uint32_t all = 0;
+    for (int w = 0; w < BK_THREADS / GS_WAVE; w++) all += s_sum[w];
+    block_sums[blockIdx.x] = all;
+  }
 }
 
 // 1b. Per tile: the workgroups' counts become exclusive prefixes in place, their sum goes to totals.  A workgroup
@@ -136,11 +148,26 @@ __device__ __forceinline__ uint32_t wave_inclusive_scan_u32(uint32_t v, int lane
 // the host can read them (host_words[1], [2] and [0]; the host polls word 0, so it is written last).
 __global__ void __launch_bounds__(1024)
 bucket_ranges_kernel(uint32_t T, uint32_t limit, const uint32_t* __restrict__ totals, uint32_t* __restrict__ ranges,
-                     uint32_t* __restrict__ chunk_first, uint32_t* __restrict__ host_words) {
+                     uint32_t* __restrict__ chunk_first, uint32_t* __restrict__ block_sums, int nblocks,
+                     uint32_t* __restrict__ host_words) {
   constexpr int ITEMS = 4;  // consecutive tiles per thread: the usual grids (up to 4096 tiles) take one round
   __shared__ uint32_t s_wave[16], s_wave_chunks[16], s_max[16];
   __shared__ double s_exact[16];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  {
+    // the counting workgroups' sums of tiles touched (at most BK_MAX_BLOCKS <= 1024 of them) become exclusive
+    // prefixes in place
+    const uint32_t b = (int)threadIdx.x < nblocks ? block_sums[threadIdx.x] : 0u;
+    const uint32_t inc = wave_inclusive_scan_u32(b, lane);
+    if (lane == 63) s_wave[wave] = inc;
+    __syncthreads();
+    uint32_t base = 0;
+#pragma unroll
+    for (int w = 0; w < 16; w++)
+      if (w < wave) base += s_wave[w];
+    if ((int)threadIdx.x < nblocks) block_sums[threadIdx.x] = base + inc - b;
+    __syncthreads();
+  }
   uint32_t carry = 0, carry_chunks = 0, longest = 0;
   double exact = 0.0;  // the number of instances without the 32-bit wrap-around of the prefix sums
   for (uint32_t start = 0; start < T; start += 1024 * ITEMS) {
@@ -215,6 +242,46 @@ bucket_ranges_kernel(uint32_t T, uint32_t limit, const uint32_t* __restrict__ to
     __hip_atomic_store(host_words + 1, m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
     __hip_atomic_store(host_words + 2, carry_chunks, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
     __hip_atomic_store(host_words, reported, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+  }
+}
+
+// 1c'. Inclusive prefix of tiles_touched over the Gaussians (rasterizer_impl.cu:648), from the counting
+// workgroups' own sums: every workgroup scans its chunk, starting from the prefix bucket_ranges_kernel left.
+__global__ void __launch_bounds__(BK_THREADS)
+bucket_offsets_kernel(int P, int per_block, const uint32_t* __restrict__ tiles_touched,
+                      const uint32_t* __restrict__ block_prefix, uint32_t* __restrict__ point_offsets) {
+  constexpr int ITEMS = 4;
+  __shared__ uint32_t s_wave[BK_THREADS / GS_WAVE];
+  const int lane = threadIdx.x & (GS_WAVE - 1), wave = threadIdx.x / GS_WAVE;
+  const int first = blockIdx.x * per_block;
+  const int last = first + per_block < P ? first + per_block : P;
+  uint32_t carry = block_prefix[blockIdx.x];
+  for (int base = first; base < last; base += BK_THREADS * ITEMS) {
+    const int i0 = base + (int)threadIdx.x * ITEMS;
+    uint32_t v[ITEMS], sum = 0;
+#pragma unroll
+    for (int q = 0; q < ITEMS; q++) {
+      v[q] = i0 + q < last ? tiles_touched[i0 + q] : 0u;
+      sum += v[q];
+    }
+    const uint32_t inc = wave_inclusive_scan_u32(sum, lane);
+    if (lane == GS_WAVE - 1) s_wave[wave] = inc;
+    __syncthreads();
+    uint32_t before = 0, all = 0;
+#pragma unroll
+    for (int w = 0; w < BK_THREADS / GS_WAVE; w++) {
+      const uint32_t s = s_wave[w];
+      if (w < wave) before += s;
+      all += s;
+    }
+    __syncthreads();
+    uint32_t run = carry + before + inc - sum;
+#pragma unroll
+    for (int q = 0; q < ITEMS; q++) {
+      run += v[q];
+      if (i0 + q < last) point_offsets[i0 + q] = run;
+    }
+    carry += all;
   }
 }
 
@@ -550,8 +617,14 @@ tile_sort_kernel(const uint32_t* __restrict__ ranges, const uint64_t* __restrict
 // Tiles the LDS histograms of the counting kernels can hold.
 int bucket_max_tiles() { return 30000; }
 
-// workgroup-by-tile counts, then the tile totals, then the chunk table (T + 1 words)
-size_t bucket_table_bytes(int T) { return (((size_t)BK_MAX_BLOCKS + 2) * (size_t)T + 1) * sizeof(uint32_t); }
+// workgroup-by-tile counts, then the tile totals, then the chunk table (T + 1 words), then the workgroups' sums of
+// tiles touched
+size_t bucket_table_bytes(int T) {
+  return (((size_t)BK_MAX_BLOCKS + 2) * (size_t)T + 1 + BK_MAX_BLOCKS) * sizeof(uint32_t);
+}
+static uint32_t* bucket_block_sums(void* table, uint32_t T) {
+  return (uint32_t*)table + ((size_t)BK_MAX_BLOCKS + 2) * (size_t)T + 1;
+}
 
 int launch_bucket_count(int P, int W, int H, const int* radii, const float* means2D, const uint8_t* compute_locally,
                         uint32_t* tiles_touched, void* table, uint32_t* ranges, uint32_t chunk_limit,
@@ -578,11 +651,22 @@ int launch_bucket_count(int P, int W, int H, const int* radii, const float* mean
   uint32_t* tab = (uint32_t*)table;
   uint32_t* totals = tab + (size_t)BK_MAX_BLOCKS * T;
   hipLaunchKernelGGL(bucket_count_kernel, dim3(nb), dim3(BK_THREADS), lds, stream, P, per, gx, gy, radii,
-                     (const float2*)means2D, compute_locally, tiles_touched, tab, zero_per_gaussian);
+                     (const float2*)means2D, compute_locally, tiles_touched, tab, bucket_block_sums(table, T),
+                     zero_per_gaussian);
   hipLaunchKernelGGL(bucket_columns_kernel, dim3((T + COL_TILES - 1) / COL_TILES), dim3(COL_TILES * COL_RUNS), 0, stream, nb, T,
                      tab, totals);
   hipLaunchKernelGGL(bucket_ranges_kernel, dim3(1), dim3(1024), 0, stream, T, chunk_limit, totals, ranges, totals + T,
-                     host_words);
+                     bucket_block_sums(table, T), nb, host_words);
+  return 0;
+}
+
+// point_offsets = inclusive prefix sum of the tiles_touched that launch_bucket_count left (same P, same table)
+int launch_bucket_offsets(int P, int W, int H, const uint32_t* tiles_touched, void* table, uint32_t* point_offsets,
+                          hipStream_t stream) {
+  if (P <= 0) return 0;
+  const uint32_t gx = (W + GS_TILE_X - 1) / GS_TILE_X, gy = (H + GS_TILE_Y - 1) / GS_TILE_Y;
+  hipLaunchKernelGGL(bucket_offsets_kernel, dim3(bucket_blocks(P)), dim3(BK_THREADS), 0, stream, P,
+                     bucket_per_block(P), tiles_touched, bucket_block_sums(table, gx * gy), point_offsets);
   return 0;
 }
 
