@@ -96,6 +96,10 @@ def cpu_baseline(g, cam, am, ug, runs):
             "sample": f"{runs} full views of the same workload (median); C++/OpenMP oracle incl. python glue"}
 
 
+FORWARD_STAGES = ("preprocess_fwd", "tile_count", "inclusive_sum", "bucket_scatter", "tile_sort",
+                  "duplicate_with_keys", "identify_tile_ranges", "render_fwd")
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -390,6 +394,12 @@ def main():
         "config": {"workload": f"BASELINE config {args.config}: {P} Gaussians, {W}x{H}, SH degree 3, render_geo, "
                                f"1 view per step, seed 0", "instances_R": R, "tiles": gx * gy},
         "gaussian_views_per_s": round(P / (ms_per_step * 1e-3), 1),
+        # the forward half of a step (preprocess, per-tile lists, blend): sum of its stages' event times
+        "forward_ms_per_view": round(sum(stage_report[k]["ms"] * stage_report[k].get("launches_per_step", 1.0)
+                                         for k in FORWARD_STAGES if k in stage_report)
+                                     # (a view on the radix route: one sort of its keys as well)
+                                     + (stage_report["sort_pairs"]["ms"] if "duplicate_with_keys" in stage_report
+                                        and "sort_pairs" in stage_report else 0.0), 4),
         "roofline": roofline,
         "ms_per_step_with_stage_events": round(ms_per_step_instrumented, 4),
         "stages": stage_report,
