@@ -251,3 +251,54 @@ def test_more_instances_than_positions_is_an_error(H, limits):
                               torch.zeros(3, device=DEV), 1.0, 0.75, torch.zeros(P, 5, device=DEV), False, False,
                               {"stats_collector": {}})
     assert out[0] == 0
+
+
+@pytest.mark.parametrize("seed,W,Hh", [(0, 333, 217), (1, 1152, 864), (2, 64, 48), (3, 1920, 1080), (4, 17, 500)])
+def test_random_rectangles_by_every_route(orc, H, seed, W, Hh):
+    """Arbitrary splats handed straight to render_gaussians: radii from 0 to far beyond the image, centres inside,
+    outside and non-finite, many equal depths, a random tile mask, image sizes that leave partial tiles.  Every
+    route must build the oracle's lists."""
+    import gsrast_native as gn
+    from diff_gaussian_rasterization import _C
+    gen = torch.Generator().manual_seed(seed)
+    P = 6000
+    gx, gy = H.grid(W, Hh)
+    T = gx * gy
+    means2D = torch.rand(P, 2, generator=gen) * torch.tensor([1.4 * W, 1.4 * Hh]) - torch.tensor([0.2 * W, 0.2 * Hh])
+    kind = torch.randint(0, 10, (P,), generator=gen)
+    radii = torch.randint(1, 12, (P,), generator=gen, dtype=torch.int32)
+    radii[kind == 0] = 0
+    radii[kind == 1] = torch.randint(40, 200, (int((kind == 1).sum()),), generator=gen, dtype=torch.int32)
+    radii[kind == 2] = 100000  # covers every tile
+    radii[kind == 3] = 2 ** 31 - 1
+    means2D[kind == 4, 0] = float("nan")
+    means2D[kind == 5, 1] = float("inf")
+    means2D[kind == 6] = -1e30
+    depths = (torch.rand(P, generator=gen) * 8).round() / 2 + 0.5  # 17 distinct values
+    cl = torch.rand(gy, gx, generator=gen) < 0.7
+    n = lambda t: t.detach().cpu().numpy()
+    want = orc.bin_and_sort(n(radii), n(means2D), n(depths), cl.numpy().reshape(-1), W, Hh)
+    R_want = int(want["point_list"].shape[0])
+    assert R_want > T  # the splats that cover everything alone give that
+    co = torch.tensor([0.02, 0.0, 0.02, 0.3]).repeat(P, 1).to(DEV)
+    rgb = torch.rand(P, 3, generator=gen).to(DEV)
+    eye = torch.eye(4, device=DEV)
+    for small, large, chunks in ROUTES:
+        gn.lib.gs_set_tile_sort_limits(small, large, chunks)
+        out = _C.render_gaussians(torch.zeros(3, device=DEV), Hh, W, means2D.to(DEV), depths.to(DEV), radii.to(DEV),
+                                  co, rgb, cl.to(DEV), eye, torch.zeros(3, device=DEV), 1.0, 1.0,
+                                  torch.zeros(P, 5, device=DEV), False, False, {"stats_collector": {}})
+        R, binB, imgB = out[0], out[9], out[10]
+        assert R == R_want, (small, large, chunks)
+        off = [C.c_size_t() for _ in range(5)]
+        gn.check(gn.lib.gs_binning_state_layout(R, W, Hh, *[C.byref(x) for x in off]), "layout")
+        base = (binB.data_ptr() + 255) // 256 * 256 - binB.data_ptr()
+        point_list = binB[base + off[0].value: base + off[0].value + 4 * R].view(torch.int32)
+        keys = binB[base + off[1].value: base + off[1].value + 8 * R].view(torch.int64)
+        ioff = [C.c_size_t() for _ in range(5)]
+        gn.check(gn.lib.gs_image_state_layout(W, Hh, *[C.byref(x) for x in ioff]), "layout")
+        ibase = (imgB.data_ptr() + 255) // 256 * 256 - imgB.data_ptr()
+        ranges = imgB[ibase + ioff[3].value: ibase + ioff[3].value + 8 * T].view(torch.int32)
+        assert np.array_equal(H.np_u32(ranges), want["ranges"].reshape(-1)), (small, large, chunks)
+        assert np.array_equal(H.np_u64(keys), want["keys"]), (small, large, chunks)
+        assert np.array_equal(H.np_u32(point_list), want["point_list"]), (small, large, chunks)
