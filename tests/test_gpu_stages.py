@@ -283,3 +283,63 @@ def test_non_finite_parameters_are_contained(H, orc, cfg, P):
     for t in back:
         assert t.shape[0] == P
         assert float(t[radii == 0].abs().max()) == 0.0  # nothing reaches a culled Gaussian
+
+
+@pytest.mark.parametrize("seed,W,Hh,geo", [(0, 100, 70, True), (1, 48, 48, False), (2, 161, 33, True)])
+def test_blend_with_arbitrary_splats(H, orc, seed, W, Hh, geo):
+    """The blend kernels on splats no preprocess would produce: indefinite and degenerate conics (power > 0 is a
+    skip, forward.cu:375-376), opacities above 1 (alpha clamps at 0.99, :383), opaque stacks that end a pixel early,
+    negative and large colours, image sizes with partial tiles.  Forward counters exact, images and gradients
+    within tolerance."""
+    gen = torch.Generator().manual_seed(200 + seed)
+    P = 4000
+    gx, gy = H.grid(W, Hh)
+    means2D = (torch.rand(P, 2, generator=gen) * torch.tensor([W + 20.0, Hh + 20.0]) - 10.0).numpy()
+    radii = torch.randint(1, 30, (P,), generator=gen, dtype=torch.int32).numpy()
+    a = torch.rand(P, generator=gen) * 0.3 + 0.002
+    c = torch.rand(P, generator=gen) * 0.3 + 0.002
+    b = (torch.rand(P, generator=gen) * 2 - 1) * torch.sqrt(a * c) * 1.3  # |b| > sqrt(ac) for some: indefinite
+    kind = torch.randint(0, 12, (P,), generator=gen)
+    a[kind == 0] = 0.0
+    c[kind == 1] = -0.05
+    opac = torch.rand(P, generator=gen) * 1.2
+    opac[kind == 2] = 5.0
+    opac[kind == 3] = 0.0
+    co = torch.stack([a, b, c, opac], 1).numpy()
+    rgb = (torch.randn(P, 3, generator=gen) * 2).numpy()
+    am = (torch.randn(P, 5, generator=gen)).numpy()
+    depths = (torch.rand(P, generator=gen) * 50 + 0.3).numpy()
+    cl = np.ones(gx * gy, bool)
+    bins = orc.bin_and_sort(radii, means2D, depths, cl, W, Hh)
+    bg = np.array([0.1, 0.7, 0.3], np.float32)
+    tanx, tany = 0.8, 0.8 * Hh / W
+    ref = orc.render_fwd(bins["ranges"], bins["point_list"], means2D, rgb, am, co, cl, bg, W, Hh, tanx, tany,
+                         render_geo=geo)
+    got = H.render_fwd(P, W, Hh, tanx, tany, H.as_u32(bins["ranges"]), H.as_u32(bins["point_list"]), H.dev(means2D),
+                       H.dev(rgb), H.dev(am), H.dev(co), H.dev(cl), H.dev(bg), render_geo=geo)
+    for k in ("n_contrib", "n_contrib2loss"):
+        assert np.array_equal(H.np_u32(got[k]), ref[k]), k
+    assert np.array_equal(got["out_observe"].cpu().numpy(), ref["out_observe"])
+    assert (ref["final_T"] < 1e-3).any() and (ref["n_contrib"] < bins["ranges"].reshape(-1, 2)[:, 1].max()).any()
+    assert np.abs(got["final_T"].cpu().numpy() - ref["final_T"]).max() <= IMG_TOL
+    scale = max(1.0, float(np.abs(ref["color"]).max()))
+    assert np.abs(got["color"].cpu().numpy() - ref["color"]).max() <= IMG_TOL * scale
+    if geo:
+        scale = max(1.0, float(np.abs(ref["out_all_map"]).max()))
+        assert np.abs(got["out_all_map"].cpu().numpy() - ref["out_all_map"]).max() <= IMG_TOL * scale
+    gen2 = torch.Generator().manual_seed(seed)
+    gpix = torch.randn(3, Hh, W, generator=gen2).numpy()
+    gmap = torch.randn(5, Hh, W, generator=gen2).numpy()
+    gdep = np.zeros((1, Hh, W), np.float32)  # (plane depth divides by a blended normal: arbitrary here)
+    rb = orc.render_bwd(bins["ranges"], bins["point_list"], means2D, co, rgb, am, ref["out_all_map"], ref["final_T"],
+                        ref["n_contrib"], cl, bg, gpix, gmap, gdep, W, Hh, tanx, tany, render_geo=geo)
+    gb = H.render_bwd(P, W, Hh, tanx, tany, H.dev(bg), H.as_u32(bins["ranges"]), H.as_u32(bins["point_list"]),
+                      H.dev(means2D), H.dev(co), H.dev(rgb), H.dev(am), H.dev(ref["out_all_map"]),
+                      H.dev(ref["final_T"]), H.as_u32(ref["n_contrib"]), H.dev(cl), H.dev(gpix), H.dev(gmap),
+                      H.dev(gdep), H.as_u32(bins["emission_sorted"]), H.as_u32(bins["point_offsets"]), render_geo=geo)
+    pairs = [("dL_dmeans2D", rb["dL_dmeans2D"][:, :2]), ("dL_dconic_opacity", rb["dL_dconic_opacity"]),
+             ("dL_dcolors", rb["dL_dcolors"])] + ([("dL_dall_map", rb["dL_dall_map"])] if geo else [])
+    for k, r in pairs:
+        g_ = gb[k].cpu().numpy()
+        assert np.isfinite(g_).all(), k
+        assert H.rel_l2(g_, r) <= GRAD_TOL, f"{k}: rel L2 {H.rel_l2(g_, r)}"
