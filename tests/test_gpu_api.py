@@ -244,3 +244,42 @@ def test_max_weight_depth_matches_oracle_and_changes_nothing_else(orc, cfg, P, m
     pxn = n(px)
     assert np.array_equal(n(got)[0][pxn], want[0][pxn])
     assert float(got[0][px].max()) > 0
+
+
+def test_debug_mode_gives_the_same_results_by_every_route():
+    """debug=True makes every stage wait for its kernels and report their errors (and check the radix sort's
+    status word); results are those of the normal mode bit for bit, whichever way the per-tile lists are built."""
+    import gs_scenes
+    import gsrast_native as gn
+    from diff_gaussian_rasterization import GaussianRasterizer
+    g, cams = gs_scenes.make_scene(0, P=30_000, n_views=1)
+    cam = cams[0]
+    W, H = cam.image_width, cam.image_height
+    gx, gy = (W + 15) // 16, (H + 15) // 16
+    cl = torch.ones(gy, gx, dtype=torch.bool, device=DEV)
+    ug = {k: v.to(DEV) for k, v in gs_scenes.upstream_grads(cam).items()}
+
+    def run(debug):
+        rast = GaussianRasterizer(_settings(cam)._replace(debug=debug))
+        leaf = {k: g[k].to(DEV).requires_grad_(True) for k in ("means3D", "scales", "rotations", "opacities", "shs")}
+        args = _cuda_args()
+        means2D, rgb, co, radii, depths = rast.preprocess_gaussians(
+            leaf["means3D"], leaf["scales"], leaf["rotations"], leaf["shs"], leaf["opacities"], args)
+        am = gs_scenes.build_all_map(leaf["means3D"], leaf["scales"], leaf["rotations"], cam)
+        m2abs = torch.zeros_like(leaf["means3D"], requires_grad=True) + 0
+        color, n_render, n_consider, n_contrib, obs, oam, opd = rast.render_gaussians(
+            means2D, m2abs, co, rgb, am, depths, radii, cl, cl, args)
+        torch.autograd.backward([color, oam, opd], [ug["color"], ug["all_map"], ug["plane_depth"]])
+        return [color, n_render, n_consider, n_contrib, obs, oam] + [leaf[k].grad for k in sorted(leaf)]
+
+    base = run(False)
+    try:
+        for limits in [(1, 8192, 32), (1, 0, 32), (1, 40, 1 << 30), (0, 100, 1 << 30)]:
+            gn.lib.gs_set_tile_sort_limits(*limits)
+            got = run(True)
+            for i, (a, b) in enumerate(zip(base[:6], got[:6])):
+                assert torch.equal(a, b), (limits, i)
+            for i, (a, b) in enumerate(zip(base[6:], got[6:])):
+                assert float((a - b).norm()) <= 1e-5 * float(a.norm()) + 1e-12, (limits, i)
+    finally:
+        gn.lib.gs_set_tile_sort_limits(1, 8192, 32)
