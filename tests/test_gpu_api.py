@@ -283,3 +283,46 @@ def test_debug_mode_gives_the_same_results_by_every_route():
                 assert float((a - b).norm()) <= 1e-5 * float(a.norm()) + 1e-12, (limits, i)
     finally:
         gn.lib.gs_set_tile_sort_limits(1, 8192, 32)
+
+
+def test_side_stream_gives_the_same_results():
+    """Everything runs on the caller's current stream: the same step on a side stream (default priority), with
+    other work in flight on the default stream, gives the same results."""
+    import gs_scenes
+    from diff_gaussian_rasterization import GaussianRasterizer
+    g, cams = gs_scenes.make_scene(1, P=120_000, n_views=1)
+    cam = cams[0]
+    W, H = cam.image_width, cam.image_height
+    gx, gy = (W + 15) // 16, (H + 15) // 16
+    cl = torch.ones(gy, gx, dtype=torch.bool, device=DEV)
+    ug = {k: v.to(DEV) for k, v in gs_scenes.upstream_grads(cam).items()}
+    dev = {k: g[k].to(DEV) for k in ("means3D", "scales", "rotations", "opacities", "shs")}
+    torch.cuda.synchronize()
+
+    def run():
+        rast = GaussianRasterizer(_settings(cam))
+        leaf = {k: v.clone().requires_grad_(True) for k, v in dev.items()}
+        args = _cuda_args()
+        means2D, rgb, co, radii, depths = rast.preprocess_gaussians(
+            leaf["means3D"], leaf["scales"], leaf["rotations"], leaf["shs"], leaf["opacities"], args)
+        am = gs_scenes.build_all_map(leaf["means3D"], leaf["scales"], leaf["rotations"], cam)
+        m2abs = torch.zeros_like(leaf["means3D"], requires_grad=True) + 0
+        color, n_render, n_consider, n_contrib, obs, oam, opd = rast.render_gaussians(
+            means2D, m2abs, co, rgb, am, depths, radii, cl, cl, args)
+        torch.autograd.backward([color, oam, opd], [ug["color"], ug["all_map"], ug["plane_depth"]])
+        return [color, n_render, n_consider, n_contrib, obs, oam] + [leaf[k].grad for k in sorted(leaf)]
+
+    base = run()
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    busy = torch.randn(4096, 4096, device=DEV)
+    with torch.cuda.stream(side):
+        for _ in range(3):
+            busy = busy @ busy * 1e-3  # keeps the default stream's queue independent of the side stream's
+        got = run()
+    side.synchronize()
+    torch.cuda.synchronize()
+    for i, (a, b) in enumerate(zip(base[:6], got[:6])):
+        assert torch.equal(a, b), i
+    for i, (a, b) in enumerate(zip(base[6:], got[6:])):
+        assert float((a - b).norm()) <= 1e-5 * float(a.norm()) + 1e-12, i
