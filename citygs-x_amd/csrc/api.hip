@@ -891,9 +891,10 @@ int gs_neural_backward(int64_t N, int k, int64_t S, const float* anchor, const f
   if (check_launch("neural_pack", stream, false)) return 1;
   {
     StageScope _t("neural_backward", stream);
-    launch_neural_backward(N, k, anchor, feat, (input_flags & 8) ? level : nullptr, input_flags, offsets, scaling, campos, packed, neural_opacity, opacity_scale, first,
-                           color, rot, aux, dL_dxyz, dL_dcolor, dL_dopacity, dL_dscaling, dL_drot, d_anchor, d_feat, d_offsets,
-                           d_scaling, d_mlp_params, slot_grads, partials, stream);
+    launch_neural_backward(N, k, anchor, feat, (input_flags & 8) ? level : nullptr, input_flags, offsets, scaling,
+                           campos, packed, neural_opacity, opacity_scale, first, color, rot, aux, dL_dxyz, dL_dcolor,
+                           dL_dopacity, dL_dscaling, dL_drot, d_anchor, d_feat, d_offsets, d_scaling, d_mlp_params,
+                           slot_grads, partials, stream);
   }
   return check_launch("neural_backward", stream, false);
 }

@@ -934,11 +934,15 @@ int launch_neural_pack(int k, const float* const* params, int input_flags, float
 }
 
 int launch_neural_opacity(int64_t N, int k, const float* anchor, const float* feat, const float* level,
-                          const float* campos, const float* packed, const float* opacity_scale, float* neural_opacity, uint8_t* mask,
-                          uint8_t* counts, hipStream_t stream) {
+                          const float* campos, const float* packed, const float* opacity_scale,
+                          float* neural_opacity, uint8_t* mask, uint8_t* counts, hipStream_t stream) {
   if (N <= 0) return 0;
   switch (k) {
-#define X(KK) case KK: Launcher<KK>::opacity(N, anchor, feat, level, campos, packed, opacity_scale, neural_opacity, mask, counts, stream); return 0;
+#define X(KK)                                                                                                 \
+  case KK:                                                                                                    \
+    Launcher<KK>::opacity(N, anchor, feat, level, campos, packed, opacity_scale, neural_opacity, mask, counts, \
+                          stream);                                                                            \
+    return 0;
     NG_FOR_EACH_K(X)
 #undef X
     default: return 1;
@@ -951,7 +955,11 @@ int launch_neural_gaussians(int64_t N, int k, const float* anchor, const float* 
                             float* opacity, float* scal, float* rot, float* aux, hipStream_t stream) {
   if (N <= 0) return 0;
   switch (k) {
-#define X(KK) case KK: Launcher<KK>::gaussians(N, anchor, feat, level, offsets, scaling, campos, packed, neural_opacity, first, xyz, color, opacity, scal, rot, aux, stream); return 0;
+#define X(KK)                                                                                                \
+  case KK:                                                                                                   \
+    Launcher<KK>::gaussians(N, anchor, feat, level, offsets, scaling, campos, packed, neural_opacity, first, \
+                            xyz, color, opacity, scal, rot, aux, stream);                                    \
+    return 0;
     NG_FOR_EACH_K(X)
 #undef X
     default: return 1;
@@ -967,7 +975,13 @@ int launch_neural_backward(int64_t N, int k, const float* anchor, const float* f
                            float* const* d_params, float* slot_grads, float* partials, hipStream_t stream) {
   if (N <= 0) return 0;
   switch (k) {
-#define X(KK) case KK: Launcher<KK>::backward(N, anchor, feat, level, input_flags, offsets, scaling, campos, packed, neural_opacity, opacity_scale, first, color_out, rot_out, aux, g_xyz, g_color, g_opacity, g_scal, g_rot, d_anchor, d_feat, d_offsets, d_scaling, d_params, slot_grads, partials, stream); return 0;
+#define X(KK)                                                                                              \
+  case KK:                                                                                                 \
+    Launcher<KK>::backward(N, anchor, feat, level, input_flags, offsets, scaling, campos, packed,          \
+                           neural_opacity, opacity_scale, first, color_out, rot_out, aux, g_xyz, g_color,  \
+                           g_opacity, g_scal, g_rot, d_anchor, d_feat, d_offsets, d_scaling, d_params,     \
+                           slot_grads, partials, stream);                                                  \
+    return 0;
     NG_FOR_EACH_K(X)
 #undef X
     default: return 1;

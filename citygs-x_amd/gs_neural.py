@@ -122,7 +122,8 @@ def neural_gaussians(anchor, feat, offsets, scaling, camera_center, mlp_opacity,
     anchor (N,3), feat (N,32), offsets (N,k,3), scaling (N,6) = get_scaling, camera_center (3); each mlp_* is
     (W1, b1, W2, b2) as nn.Linear holds them; opacity_scale (N), if given, multiplies the opacity MLP's output per
     anchor (:844-848); input_flags (add_opacity_dist = 1, add_color_dist = 2, add_cov_dist = 4: that MLP's W1 has a
-    column for the distance; add_level = 8: all three have a last column for level (N), :824-877).  Returns (xyz, color, opacity, scaling, rot, neural_opacity, mask);
+    column for the distance; add_level = 8: all three have a last column for level (N), :824-877).
+    Returns (xyz, color, opacity, scaling, rot, neural_opacity, mask);
     differentiable in everything but the camera centre; neural_opacity and mask carry no gradient (the reference
     uses them detached, scene/gaussian_model.py:1183)."""
     return _NeuralGaussians.apply(anchor, feat, offsets, scaling, camera_center, opacity_scale, level, input_flags,
