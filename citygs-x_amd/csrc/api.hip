@@ -758,8 +758,9 @@ size_t gs_neural_workspace_bytes(int64_t num_anchors, int n_offsets) {
 
 int gs_neural_opacity_forward(int64_t N, int k, const float* anchor, const float* feat, const float* campos,
                               const float* const* mlp_params, const float* opacity_scale, const float* level,
-                              int input_flags, float* neural_opacity, uint8_t* mask, uint32_t* first,
-                              void* workspace, size_t workspace_bytes, int64_t* num_selected, gs_stream_t stream_) {
+                              int input_flags, float* neural_opacity, float* opacity_tanh, uint8_t* mask,
+                              uint32_t* first, void* workspace, size_t workspace_bytes, int64_t* num_selected,
+                              gs_stream_t stream_) {
   hipStream_t stream = (hipStream_t)stream_;
   GS_REQUIRE(N >= 0, "gs_neural_opacity_forward: negative anchor count");
   GS_REQUIRE(neural_supported(k), "gs_neural_opacity_forward: n_offsets not among the supported values");
@@ -769,6 +770,7 @@ int gs_neural_opacity_forward(int64_t N, int k, const float* anchor, const float
   GS_REQUIRE(mlp_params && campos, "gs_neural_opacity_forward: null pointer");
   GS_REQUIRE(input_flags >= 0 && input_flags < 16, "gs_neural_opacity_forward: input_flags has four bits");
   GS_REQUIRE(!(input_flags & 8) || level || N == 0, "gs_neural_opacity_forward: input_flags asks for the level");
+  GS_REQUIRE(!opacity_scale || opacity_tanh || N == 0, "gs_neural_opacity_forward: opacity_scale needs opacity_tanh");
   for (int i = 0; i < 12; i++) GS_REQUIRE(mlp_params[i], "gs_neural_opacity_forward: null MLP parameter");
   GS_REQUIRE(workspace && workspace_bytes >= gs_neural_workspace_bytes(N, k),
              "gs_neural_opacity_forward: workspace missing or too small");
@@ -786,7 +788,7 @@ int gs_neural_opacity_forward(int64_t N, int k, const float* anchor, const float
   {
     StageScope _t("neural_opacity", stream);
     launch_neural_opacity(N, k, anchor, feat, (input_flags & 8) ? level : nullptr, campos, packed, opacity_scale,
-                          neural_opacity, mask, counts, stream);
+                          neural_opacity, opacity_scale ? opacity_tanh : nullptr, mask, counts, stream);
   }
   if (check_launch("neural_opacity", stream, false)) return 1;
   uint32_t* total_slot = acquire_total_slot();
@@ -846,7 +848,8 @@ size_t gs_neural_backward_workspace_bytes(int64_t num_anchors, int n_offsets) {
 int gs_neural_backward(int64_t N, int k, int64_t S, const float* anchor, const float* feat, const float* offsets,
                        const float* scaling, const float* campos, const float* const* mlp_params,
                        const float* opacity_scale, const float* level, int input_flags,
-                       const float* neural_opacity, const uint32_t* first, const float* color, const float* rot,
+                       const float* neural_opacity, const float* opacity_tanh, const uint32_t* first,
+                       const float* color, const float* rot,
                        const float* aux, const float* dL_dxyz, const float* dL_dcolor, const float* dL_dopacity,
                        const float* dL_dscaling, const float* dL_drot, float* d_anchor, float* d_feat,
                        float* d_offsets, float* d_scaling, float* const* d_mlp_params, void* workspace,
@@ -857,6 +860,7 @@ int gs_neural_backward(int64_t N, int k, int64_t S, const float* anchor, const f
   GS_REQUIRE(mlp_params && d_mlp_params && campos, "gs_neural_backward: null pointer");
   GS_REQUIRE(input_flags >= 0 && input_flags < 16, "gs_neural_backward: input_flags has four bits");
   GS_REQUIRE(!(input_flags & 8) || level || N == 0, "gs_neural_backward: input_flags asks for the level");
+  GS_REQUIRE(!opacity_scale || opacity_tanh || N == 0, "gs_neural_backward: opacity_scale needs opacity_tanh");
   for (int i = 0; i < 12; i++)
     GS_REQUIRE(mlp_params[i] && d_mlp_params[i], "gs_neural_backward: null MLP parameter or gradient");
   if (N == 0) {
@@ -892,7 +896,7 @@ int gs_neural_backward(int64_t N, int k, int64_t S, const float* anchor, const f
   {
     StageScope _t("neural_backward", stream);
     launch_neural_backward(N, k, anchor, feat, (input_flags & 8) ? level : nullptr, input_flags, offsets, scaling,
-                           campos, packed, neural_opacity, opacity_scale, first, color, rot, aux, dL_dxyz, dL_dcolor,
+                           campos, packed, neural_opacity, opacity_scale, opacity_tanh, first, color, rot, aux, dL_dxyz, dL_dcolor,
                            dL_dopacity, dL_dscaling, dL_drot, d_anchor, d_feat, d_offsets, d_scaling, d_mlp_params,
                            slot_grads, partials, stream);
   }

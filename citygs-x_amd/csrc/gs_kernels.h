@@ -113,20 +113,22 @@ size_t neural_partial_floats(int k, int64_t N);
 // three take the anchor's level as their last input column (W1 is then 32 x 36 or 32 x 37); level (N) is read
 // only with bit 3
 int launch_neural_pack(int k, const float* const* params, int input_flags, float* packed, hipStream_t stream);
-// opacity_scale (N, optional): per-anchor factor on the opacity MLP's output
+// opacity_scale (N, optional): per-anchor factor on the opacity MLP's output; opacity_tanh (N*k, with opacity_scale):
+// the output before the factor, which the backward pass needs
 int launch_neural_opacity(int64_t N, int k, const float* anchor, const float* feat, const float* level,
-                          const float* campos, const float* packed, const float* opacity_scale, float* neural_opacity, uint8_t* mask,
-                          uint8_t* counts, hipStream_t stream);
+                          const float* campos, const float* packed, const float* opacity_scale,
+                          float* neural_opacity, float* opacity_tanh, uint8_t* mask, uint8_t* counts,
+                          hipStream_t stream);
 int launch_neural_gaussians(int64_t N, int k, const float* anchor, const float* feat, const float* level,
                             const float* offsets, const float* scaling, const float* campos, const float* packed,
                             const float* neural_opacity, const uint32_t* first, float* xyz, float* color,
                             float* opacity, float* scal, float* rot, float* aux, hipStream_t stream);
 int launch_neural_backward(int64_t N, int k, const float* anchor, const float* feat, const float* level,
                            int input_flags, const float* offsets, const float* scaling, const float* campos, const float* packed,
-                           const float* neural_opacity, const float* opacity_scale, const uint32_t* first,
-                           const float* color_out, const float* rot_out, const float* aux, const float* g_xyz,
-                           const float* g_color, const float* g_opacity, const float* g_scal, const float* g_rot,
-                           float* d_anchor, float* d_feat, float* d_offsets, float* d_scaling,
+                           const float* neural_opacity, const float* opacity_scale, const float* opacity_tanh,
+                           const uint32_t* first, const float* color_out, const float* rot_out, const float* aux,
+                           const float* g_xyz, const float* g_color, const float* g_opacity, const float* g_scal,
+                           const float* g_rot, float* d_anchor, float* d_feat, float* d_offsets, float* d_scaling,
                            float* const* d_params, float* slot_grads, float* partials, hipStream_t stream);
 size_t neural_slot_grad_floats(int k, int64_t N);
 int launch_all_map_fwd(int P, const float* means, const float* scales, const float* rots, const float* V,

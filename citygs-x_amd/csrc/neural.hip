@@ -221,7 +221,7 @@ neural_opacity_kernel(int64_t N, int ntiles, const float* __restrict__ anchor, c
                       const float* __restrict__ level,
                       const float* __restrict__ campos, const float* __restrict__ packed,
                       const float* __restrict__ opacity_scale, float* __restrict__ neural_opacity,
-                      uint8_t* __restrict__ mask, uint8_t* __restrict__ counts) {
+                      float* __restrict__ opacity_tanh, uint8_t* __restrict__ mask, uint8_t* __restrict__ counts) {
   using S = Shape<K>;
   constexpr PackLayout L = pack_layout(S::GROWS);
   __shared__ float sW1[NG_SLOTS * WS];
@@ -241,11 +241,10 @@ neural_opacity_kernel(int64_t N, int ntiles, const float* __restrict__ anchor, c
     unpack_x(xb, nv, dist, fetch_x(a < N, a, half, anchor, feat, level), a < N, half, cam);
     const v16f h = hidden_layer(sW1, xb, al, half);
     const v16f o = output_tile<S::OUT0>(sW2, sB2, 0, h, al, half);
-    const float ps = (opacity_scale != nullptr && a < N) ? opacity_scale[a] : 1.0f;
 #pragma unroll
     for (int i = 0; i < 16; i++) {
       const int row = hrow(half, i);
-      if (row < K) op[al * K + row] = opacity_scale != nullptr ? tanhf(o[i]) * ps : tanhf(o[i]);
+      if (row < K) op[al * K + row] = tanhf(o[i]);
     }
     wave_sync();
 #pragma unroll
@@ -253,12 +252,15 @@ neural_opacity_kernel(int64_t N, int ntiles, const float* __restrict__ anchor, c
       const int idx = g * S::APG * K + lane;  // slot within the tile
       const int64_t slot_anchor = (int64_t)tile * NG_ANCHORS + idx / K;
       const bool ok = lane < S::APG * K && idx < NG_ANCHORS * K && slot_anchor < N;
-      const float t = ok ? op[idx] : 0.0f;
+      const float th = ok ? op[idx] : 0.0f;
+      const float t = (ok && opacity_scale != nullptr) ? th * opacity_scale[slot_anchor] : th;
       const bool sel = t > 0.0f;
       const unsigned long long bits = __ballot(sel);
       if (ok) {
         const int64_t slot = (int64_t)tile * NG_ANCHORS * K + idx;
         neural_opacity[slot] = t;
+        // the backward pass needs 1 - tanh^2 of a saturated unit to the last bit: t / scale would not give it
+        if (opacity_tanh != nullptr) opacity_tanh[slot] = th;
         mask[slot] = sel ? 1 : 0;
         if (idx % K == 0) counts[slot_anchor] = (uint8_t)count_lanes(bits, lane, lane + K);
       }
@@ -407,8 +409,8 @@ template <int K>
 __global__ void __launch_bounds__(NG_THREADS)
 neural_offset_backward_kernel(int64_t N, int ntiles, const float* __restrict__ offsets,
                               const float* __restrict__ scaling, const float* __restrict__ neural_opacity,
-                              const float* __restrict__ opacity_scale, const uint32_t* __restrict__ first,
-                              const float* __restrict__ color_out,
+                              const float* __restrict__ opacity_scale, const float* __restrict__ opacity_tanh,
+                              const uint32_t* __restrict__ first, const float* __restrict__ color_out,
                               const float* __restrict__ rot_out, const float* __restrict__ aux,
                               const float* __restrict__ g_xyz, const float* __restrict__ g_color,
                               const float* __restrict__ g_opacity, const float* __restrict__ g_scal,
@@ -438,7 +440,7 @@ neural_offset_backward_kernel(int64_t N, int ntiles, const float* __restrict__ o
       const float* sc = scaling + sa * 6;
       // opacity = tanh(.) * scale (scale > 0 wherever an offset is selected): d/d pre = scale * (1 - tanh^2)
       const float ps = opacity_scale != nullptr ? opacity_scale[sa] : 1.0f;
-      const float th = opacity_scale != nullptr ? t / ps : t;
+      const float th = opacity_scale != nullptr ? opacity_tanh[slot] : t;
       grad[0] = g_opacity[r] * ((1.0f - th * th) * ps);
       const float4 ax4 = *(const float4*)(aux + r * 4);
       const float sg[3] = {ax4.x, ax4.y, ax4.z};
@@ -847,11 +849,12 @@ struct Launcher {
     hipLaunchKernelGGL(neural_pack_kernel<K>, dim3((total + 255) / 256), dim3(256), 0, stream, w, packed);
   }
   static void opacity(int64_t N, const float* anchor, const float* feat, const float* level, const float* campos,
-                      const float* packed, const float* opacity_scale, float* neural_opacity, uint8_t* mask,
-                      uint8_t* counts, hipStream_t stream) {
+                      const float* packed, const float* opacity_scale, float* neural_opacity, float* opacity_tanh,
+                      uint8_t* mask, uint8_t* counts, hipStream_t stream) {
     const int ntiles = (int)((N + NG_ANCHORS - 1) / NG_ANCHORS);
     hipLaunchKernelGGL(neural_opacity_kernel<K>, dim3(blocks_for(ntiles, NG_WAVES, 4)), dim3(NG_THREADS), 0, stream,
-                       N, ntiles, anchor, feat, level, campos, packed, opacity_scale, neural_opacity, mask, counts);
+                       N, ntiles, anchor, feat, level, campos, packed, opacity_scale, neural_opacity, opacity_tanh, mask,
+                       counts);
   }
   static void gaussians(int64_t N, const float* anchor, const float* feat, const float* level, const float* offsets,
                         const float* scaling, const float* campos, const float* packed, const float* neural_opacity, const uint32_t* first,
@@ -867,15 +870,15 @@ struct Launcher {
   }
   static void backward(int64_t N, const float* anchor, const float* feat, const float* level, int input_flags,
                        const float* offsets, const float* scaling, const float* campos, const float* packed, const float* neural_opacity,
-                       const float* opacity_scale, const uint32_t* first, const float* color_out,
-                       const float* rot_out, const float* aux, const float* g_xyz, const float* g_color,
-                       const float* g_opacity, const float* g_scal, const float* g_rot, float* d_anchor,
-                       float* d_feat, float* d_offsets, float* d_scaling, float* const* d_params, float* slot_grads,
-                       float* partials, hipStream_t stream) {
+                       const float* opacity_scale, const float* opacity_tanh, const uint32_t* first,
+                       const float* color_out, const float* rot_out, const float* aux, const float* g_xyz,
+                       const float* g_color, const float* g_opacity, const float* g_scal, const float* g_rot,
+                       float* d_anchor, float* d_feat, float* d_offsets, float* d_scaling, float* const* d_params,
+                       float* slot_grads, float* partials, hipStream_t stream) {
     const int ntiles = (int)((N + NG_ANCHORS - 1) / NG_ANCHORS);
     hipLaunchKernelGGL(neural_offset_backward_kernel<K>, dim3((ntiles + NG_WAVES - 1) / NG_WAVES), dim3(NG_THREADS), 0,
-                       stream, N, ntiles, offsets, scaling, neural_opacity, opacity_scale, first, color_out, rot_out,
-                       aux, g_xyz, g_color, g_opacity, g_scal, g_rot, slot_grads, d_anchor, d_offsets, d_scaling);
+                       stream, N, ntiles, offsets, scaling, neural_opacity, opacity_scale, opacity_tanh, first, color_out,
+                       rot_out, aux, g_xyz, g_color, g_opacity, g_scal, g_rot, slot_grads, d_anchor, d_offsets, d_scaling);
     const int nblocks = backward_blocks(N);
     hipLaunchKernelGGL(neural_mlp_backward_kernel<K>, dim3(nblocks), dim3(64 * S::BWD_WAVES), 0, stream, N, ntiles,
                        anchor, feat, level, campos, packed, slot_grads, d_anchor, d_feat, partials);
@@ -935,13 +938,14 @@ int launch_neural_pack(int k, const float* const* params, int input_flags, float
 
 int launch_neural_opacity(int64_t N, int k, const float* anchor, const float* feat, const float* level,
                           const float* campos, const float* packed, const float* opacity_scale,
-                          float* neural_opacity, uint8_t* mask, uint8_t* counts, hipStream_t stream) {
+                          float* neural_opacity, float* opacity_tanh, uint8_t* mask, uint8_t* counts,
+                          hipStream_t stream) {
   if (N <= 0) return 0;
   switch (k) {
 #define X(KK)                                                                                                 \
   case KK:                                                                                                    \
-    Launcher<KK>::opacity(N, anchor, feat, level, campos, packed, opacity_scale, neural_opacity, mask, counts, \
-                          stream);                                                                            \
+    Launcher<KK>::opacity(N, anchor, feat, level, campos, packed, opacity_scale, neural_opacity, opacity_tanh, \
+                          mask, counts, stream);                                                              \
     return 0;
     NG_FOR_EACH_K(X)
 #undef X
@@ -968,17 +972,18 @@ int launch_neural_gaussians(int64_t N, int k, const float* anchor, const float* 
 
 int launch_neural_backward(int64_t N, int k, const float* anchor, const float* feat, const float* level,
                            int input_flags, const float* offsets, const float* scaling, const float* campos, const float* packed,
-                           const float* neural_opacity, const float* opacity_scale, const uint32_t* first,
-                           const float* color_out, const float* rot_out, const float* aux, const float* g_xyz,
-                           const float* g_color, const float* g_opacity, const float* g_scal, const float* g_rot,
-                           float* d_anchor, float* d_feat, float* d_offsets, float* d_scaling,
+                           const float* neural_opacity, const float* opacity_scale, const float* opacity_tanh,
+                           const uint32_t* first, const float* color_out, const float* rot_out, const float* aux,
+                           const float* g_xyz, const float* g_color, const float* g_opacity, const float* g_scal,
+                           const float* g_rot, float* d_anchor, float* d_feat, float* d_offsets, float* d_scaling,
                            float* const* d_params, float* slot_grads, float* partials, hipStream_t stream) {
   if (N <= 0) return 0;
   switch (k) {
 #define X(KK)                                                                                              \
   case KK:                                                                                                 \
     Launcher<KK>::backward(N, anchor, feat, level, input_flags, offsets, scaling, campos, packed,          \
-                           neural_opacity, opacity_scale, first, color_out, rot_out, aux, g_xyz, g_color,  \
+                           neural_opacity, opacity_scale, opacity_tanh, first, color_out, rot_out, aux,    \
+                           g_xyz, g_color,                                                                 \
                            g_opacity, g_scal, g_rot, d_anchor, d_feat, d_offsets, d_scaling, d_params,     \
                            slot_grads, partials, stream);                                                  \
     return 0;

@@ -64,6 +64,8 @@ class _NeuralGaussians(torch.autograd.Function):
         dev = anchor.device
         stream = C.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
         neural_opacity = torch.empty(N * k, 1, dtype=torch.float32, device=dev)
+        # with a factor on the opacity the backward pass needs the MLP's own output as well
+        opacity_tanh = torch.empty(N * k, dtype=torch.float32, device=dev) if opacity_scale is not None else None
         mask = torch.empty(N * k, dtype=torch.bool, device=dev)
         first = torch.empty(max(N, 1), dtype=torch.int32, device=dev)
         ws_bytes = _n.lib.gs_neural_workspace_bytes(N, k)
@@ -72,7 +74,7 @@ class _NeuralGaussians(torch.autograd.Function):
         S = C.c_int64(0)
         _n.check(_n.lib.gs_neural_opacity_forward(N, k, _p(anchor), _p(feat), _p(campos), table,
                                                   _p(opacity_scale), _p(level), input_flags,
-                                                  _p(neural_opacity), _p(mask), _p(first), _p(ws), ws_bytes,
+                                                  _p(neural_opacity), _p(opacity_tanh), _p(mask), _p(first), _p(ws), ws_bytes,
                                                   C.byref(S), stream),
                  "generate_neural_gaussians")
         S = S.value
@@ -87,7 +89,7 @@ class _NeuralGaussians(torch.autograd.Function):
         ctx.save_for_backward(anchor, feat, offsets, scaling, campos, neural_opacity, first, color, rot, aux, *params)
         ctx.sizes = (N, k, S)
         ctx.opacity_scale = opacity_scale  # carries no gradient (a buffer of the model)
-        ctx.level, ctx.input_flags = level, input_flags
+        ctx.level, ctx.input_flags, ctx.opacity_tanh = level, input_flags, opacity_tanh
         ctx.mark_non_differentiable(neural_opacity, mask)
         ctx.set_materialize_grads(False)
         return xyz, color, opacity, scal, rot, neural_opacity, mask
@@ -109,7 +111,8 @@ class _NeuralGaussians(torch.autograd.Function):
         _n.check(_n.lib.gs_neural_backward(N, k, S, _p(anchor), _p(feat), _p(offsets), _p(scaling), _p(campos),
                                            _table(params),
                                            _p(ctx.opacity_scale), _p(ctx.level), ctx.input_flags,
-                                           _p(neural_opacity), _p(first), _p(color), _p(rot), _p(aux),
+                                           _p(neural_opacity), _p(ctx.opacity_tanh), _p(first), _p(color), _p(rot),
+                                           _p(aux),
                                            *[_p(u) for u in ups], _p(d_anchor), _p(d_feat), _p(d_offsets),
                                            _p(d_scaling), _table(d_params), _p(ws), ws_bytes, stream),
                  "generate_neural_gaussians backward")

@@ -44,10 +44,10 @@ _SIGNATURES = {
     "gs_set_tile_sort_limits": (None, [_i, _i, _i]),
     "gs_neural_supported": (_i, [_i]),
     "gs_neural_workspace_bytes": (_sz, [_i64, _i]),
-    "gs_neural_opacity_forward": (_i, [_i64, _i] + [_vp] * 6 + [_i] + [_vp] * 4 + [_sz, _vp, _vp]),
+    "gs_neural_opacity_forward": (_i, [_i64, _i] + [_vp] * 6 + [_i] + [_vp] * 5 + [_sz, _vp, _vp]),
     "gs_neural_gaussians_forward": (_i, [_i64, _i, _i64] + [_vp] * 9 + [_sz] + [_vp] * 7),
     "gs_neural_backward_workspace_bytes": (_sz, [_i64, _i]),
-    "gs_neural_backward": (_i, [_i64, _i, _i64] + [_vp] * 8 + [_i] + [_vp] * 16 + [_sz, _vp]),
+    "gs_neural_backward": (_i, [_i64, _i, _i64] + [_vp] * 8 + [_i] + [_vp] * 17 + [_sz, _vp]),
     "gs_all_map_forward": (_i, [_i] + [_vp] * 7),
     "gs_all_map_backward": (_i, [_i] + [_vp] * 9),
     "gs_knn_workspace_bytes": (_sz, [_i]),

@@ -191,7 +191,9 @@ int gs_all_map_backward(int P, const float* means3D, const float* scales, const 
  * activated get_scaling, campos (3).  n_offsets must satisfy gs_neural_supported().
  * opacity_scale (N floats, or NULL for none) serves dist2level 'progressive' (:844-848): neural_opacity =
  * mlp_opacity(x) * opacity_scale[anchor], where the caller passes _prog_ratio with 1 for the anchors outside
- * transition_mask; it must be positive wherever the product is (the reference's lies in (0, 1]).
+ * transition_mask; it must be positive wherever the product is (the reference's lies in (0, 1]).  With it the
+ * call also writes opacity_tanh (N*n_offsets): the MLP's output before the factor, which gs_neural_backward takes
+ * back (1 - tanh^2 of a saturated unit cannot be recovered from the product); NULL without opacity_scale.
  * input_flags / level serve the MLPs' optional inputs (:824-829, :839-877; scene/gaussian_model.py:118-149):
  * bit 0 / 1 / 2 (add_opacity_dist / add_color_dist / add_cov_dist) = that MLP takes the distance
  * |anchor - campos| as input column 35, bit 3 (add_level) = all three take level[anchor] (N floats) as their last
@@ -212,9 +214,9 @@ int gs_neural_supported(int n_offsets);
 size_t gs_neural_workspace_bytes(int64_t num_anchors, int n_offsets);
 int gs_neural_opacity_forward(int64_t num_anchors, int n_offsets, const float* anchor, const float* feat,
                               const float* campos, const float* const* mlp_params, const float* opacity_scale,
-                              const float* level, int input_flags, float* neural_opacity, uint8_t* mask,
-                              uint32_t* first, void* workspace, size_t workspace_bytes, int64_t* num_selected,
-                              gs_stream_t stream);
+                              const float* level, int input_flags, float* neural_opacity, float* opacity_tanh,
+                              uint8_t* mask, uint32_t* first, void* workspace, size_t workspace_bytes,
+                              int64_t* num_selected, gs_stream_t stream);
 int gs_neural_gaussians_forward(int64_t num_anchors, int n_offsets, int64_t num_selected, const float* anchor,
                                 const float* feat, const float* offsets, const float* scaling, const float* campos,
                                 const float* level, const float* neural_opacity, const uint32_t* first,
@@ -224,8 +226,9 @@ size_t gs_neural_backward_workspace_bytes(int64_t num_anchors, int n_offsets);
 int gs_neural_backward(int64_t num_anchors, int n_offsets, int64_t num_selected, const float* anchor,
                        const float* feat, const float* offsets, const float* scaling, const float* campos,
                        const float* const* mlp_params, const float* opacity_scale, const float* level,
-                       int input_flags, const float* neural_opacity, const uint32_t* first, const float* color,
-                       const float* rot, const float* aux, const float* dL_dxyz, const float* dL_dcolor,
+                       int input_flags, const float* neural_opacity, const float* opacity_tanh,
+                       const uint32_t* first, const float* color, const float* rot, const float* aux,
+                       const float* dL_dxyz, const float* dL_dcolor,
                        const float* dL_dopacity, const float* dL_dscaling, const float* dL_drot, float* d_anchor,
                        float* d_feat, float* d_offsets, float* d_scaling, float* const* d_mlp_params,
                        void* workspace, size_t workspace_bytes, gs_stream_t stream);

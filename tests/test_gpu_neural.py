@@ -142,6 +142,35 @@ def test_distance_and_level_inputs_match_oracle(orc, N, k, seed, flags):
         assert _rel(t.grad.cpu().numpy(), w) <= 3e-5, i
 
 
+def test_progressive_factor_with_saturated_opacity_units(orc):
+    """With the distance as an input the opacity MLP's outputs saturate (tanh within an ulp or two of 1), where
+    1 - tanh^2 is a few 1e-7: the backward pass must take it from the tanh the forward pass computed, not from
+    opacity / factor.  The opacity MLP's gradients are tiny here and still the oracle's."""
+    from gs_neural import neural_gaussians
+    N, k, flags, seed = 31, 9, 7, 695985
+    s = gs_scenes.make_anchor_scene(N, k, seed, input_flags=flags)
+    gen = torch.Generator().manual_seed(seed)
+    prog = torch.rand(N, 1, generator=gen) * 0.98 + 0.01
+    prog[torch.rand(N, generator=gen) < 0.3] = 1.0
+    prog[torch.rand(N, generator=gen) < 0.1] = 0.0
+    anchor, feat, offsets, scaling, campos, mlps = _to_dev(s, grad=True)
+    out = neural_gaussians(anchor, feat, offsets, scaling, campos, *mlps, opacity_scale=prog.reshape(-1).to(DEV),
+                           level=s["level"].to(DEV), input_flags=flags)
+    kw = dict(prog=prog.numpy(), level=s["level"].numpy(), input_flags=flags)
+    want = orc.neural_gaussians_fwd(*_np_args(s), **kw)
+    got = [o.detach().cpu().numpy() for o in out]
+    assert np.array_equal(got[6], want[6])
+    th = want[5].reshape(N, k) / np.where(prog.numpy() > 0, prog.numpy(), 1.0)
+    assert (np.abs(th) > 1 - 1e-6).mean() > 0.5  # most units are saturated
+    S = int(got[6].sum())
+    ups = [torch.randn(S, c, generator=gen) for c in (3, 3, 1, 3, 4)]
+    sum((o * u.to(DEV)).sum() for o, u in zip(out[:5], ups)).backward()
+    wd = orc.neural_gaussians_bwd(*_np_args(s), *[u.numpy() for u in ups], **kw)
+    flat = [x for m in mlps for x in m]
+    for i, (t, w) in enumerate(zip(flat, wd[4])):
+        assert _rel(t.grad.cpu().numpy(), w) <= 1e-4, i
+
+
 def test_no_anchor_and_nothing_selected():
     from gs_neural import neural_gaussians
     s = gs_scenes.make_anchor_scene(50, 10, 0)
