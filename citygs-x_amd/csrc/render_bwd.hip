@@ -4,7 +4,7 @@
 // over pixels.
 //
 // Workgroup = one 16x16 tile = four 64-lane waves; a wave owns an 8x8 quadrant
-// and each of its 16-lane rows a 4x4 pixel block.  Per batch of 256 Gaussians
+// and each of its 16-lane rows a 4x4 pixel block.  Per batch of 64 Gaussians
 // (staged in LDS in back-to-front order):
 //   * a wave ballots, for each of its rows, which Gaussians can touch the
 //     row's block (inflated alpha >= 1/255 ellipse against the block) and lie in front of the row's
@@ -13,15 +13,20 @@
 //   * the 16 partial sums of a Gaussian (mean2D x/y, |mean2D| x/y, conic
 //     x/y/w, opacity, colour 3, map 5) are reduced over the row's 16 lanes by
 //     a transposing DPP reduction (15 additions instead of 64) that leaves
-//     component q in lane q, and one LDS float-atomic instruction adds all of
-//     them into a 16x256 accumulator;
-//   * at the end of the batch each thread stores one (tile, Gaussian)
-//     instance's 16 sums as one 64-byte record, at the instance's index in
-//     emission order (the order key emission wrote them: all instances of a
-//     Gaussian are consecutive there).  No global atomics at all.
+//     component q in lane q; rows of the wave that are at the same Gaussian
+//     are merged, and the sums go into the wave's own 16x64 accumulator in
+//     LDS with a plain read-add-write (no atomics: an LDS float atomic costs
+//     about three cycles per active lane here, and the kernel was bound by
+//     them);
+//   * at the end of the batch the four waves' accumulators are added in wave
+//     order and every (tile, Gaussian) instance's 16 sums are stored as one
+//     64-byte record, at the instance's index in emission order (the order
+//     key emission wrote them: all instances of a Gaussian are consecutive
+//     there).  No global atomics either.
 // A second kernel then sums, for every Gaussian, its consecutive records and
-// writes the five gradient tensors: a streaming pass, deterministic from run to
-// run.  (The reference issues 16 global float atomics per pixel and Gaussian,
+// writes the five gradient tensors: a streaming pass.  Every sum is taken in a
+// fixed order, so the gradients are the same bits from run to run.  (The
+// reference issues 16 global float atomics per pixel and Gaussian,
 // cuda_rasterizer/backward.cu:510-563.)
 // The per-pixel arithmetic is, operation for operation, the CPU statement's;
 // only the order in which pixels are summed differs, so gradients agree with a
@@ -34,9 +39,11 @@ namespace gs {
 
 namespace {
 
-constexpr int BATCH = GS_TILE_PIX;
+constexpr int BATCH = GS_TILE_PIX / 4;  // Gaussians staged per round
 constexpr int NV = 16;
 constexpr int CHUNKS = BATCH / 32;
+constexpr int WAVES = GS_TILE_PIX / GS_WAVE;
+static_assert((WAVES * NV * (BATCH + 1)) % 4 == 0, "the accumulators are cleared 16 bytes at a time");
 
 template <bool RENDER_GEO>
 __global__ void __launch_bounds__(GS_TILE_PIX)
@@ -56,7 +63,8 @@ render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
   __shared__ float s_floor[BATCH];
   __shared__ float s_rgb[GS_N_RGB][BATCH];
   __shared__ float s_map[GS_N_MAP][BATCH];
-  __shared__ float s_acc[NV][BATCH + 1];  // +1: the 16 components of one Gaussian fall in 16 different banks
+  // one accumulator per wave; +1: the 16 components of one Gaussian fall in 16 different banks
+  __shared__ __align__(16) float s_acc[WAVES][NV][BATCH + 1];
   __shared__ uint32_t s_list[GS_TILE_PIX / GS_WAVE][4][CHUNKS];
   __shared__ int s_max[GS_TILE_PIX / GS_WAVE];
 
@@ -162,8 +170,8 @@ render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
         for (int ch = 0; ch < GS_N_MAP; ch++) s_map[ch][tid] = all_map[5 * (size_t)g + ch];
       }
     }
-#pragma unroll
-    for (int q = 0; q < NV; q++) s_acc[q][tid] = 0.f;
+    for (int q = tid; q < WAVES * NV * (BATCH + 1) / 4; q += GS_TILE_PIX)
+      reinterpret_cast<float4*>(&s_acc[0][0][0])[q] = make_float4(0.f, 0.f, 0.f, 0.f);
     __syncthreads();
 
     // per-row lists: bit b of word c of row r = slot 32c+b of the batch can touch row r's 4x4 block
@@ -272,17 +280,42 @@ render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
         v[6] = hg * gdy * dy;
         v[7] = G * dL_dalpha;
         // lane q of the row now receives the row's total of component q
-        const float tot = row_transpose_reduce16(v);
-        if (has && tot != 0.f) unsafeAtomicAdd(&s_acc[l16][j], tot);
+        float tot = row_transpose_reduce16(v);
+        // Rows of this wave that are at the same Gaussian in this pass are merged, and the lowest of them
+        // adds the sum to the wave's own accumulator with a plain read-add-write: rows that write hold
+        // different Gaussians, so their addresses differ.  (An LDS float atomic takes about three cycles per
+        // active lane on this hardware, thirteen times the read-add-write.)
+        const int key = has ? j : -1 - row;
+        const int k0 = __builtin_amdgcn_readlane(key, 0), k1 = __builtin_amdgcn_readlane(key, 16);
+        const int k2 = __builtin_amdgcn_readlane(key, 32), k3 = __builtin_amdgcn_readlane(key, 48);
+        constexpr uint64_t R0 = 0xFFFFull, R1 = R0 << 16, R2 = R0 << 32, R3 = R0 << 48;
+        const uint64_t eq16 = (k0 == k1 ? R0 | R1 : 0ull) | (k2 == k3 ? R2 | R3 : 0ull);
+        const uint64_t eq32 = (k0 == k2 ? R0 | R2 : 0ull) | (k1 == k3 ? R1 | R3 : 0ull);
+        const uint64_t eq48 = (k0 == k3 ? R0 | R3 : 0ull) | (k1 == k2 ? R1 | R2 : 0ull);
+        const uint64_t follower = (k1 == k0 ? R1 : 0ull) | ((k2 == k0 || k2 == k1) ? R2 : 0ull) |
+                                  ((k3 == k0 || k3 == k1 || k3 == k2) ? R3 : 0ull);
+        if ((eq16 | eq32 | eq48) != 0ull) {  // wave-uniform
+          const float t16 = __shfl_xor(tot, 16, GS_WAVE), t32 = __shfl_xor(tot, 32, GS_WAVE);
+          const float t48 = __shfl_xor(tot, 48, GS_WAVE);
+          tot += __builtin_amdgcn_inverse_ballot_w64(eq16) ? t16 : 0.f;
+          tot += __builtin_amdgcn_inverse_ballot_w64(eq32) ? t32 : 0.f;
+          tot += __builtin_amdgcn_inverse_ballot_w64(eq48) ? t48 : 0.f;
+        }
+        if (has && !__builtin_amdgcn_inverse_ballot_w64(follower) && tot != 0.f) s_acc[wave][l16][j] += tot;
       }
     }
     __syncthreads();
-    if (tid < count) {
-      float4* rec = instance_grads + 4 * (size_t)s_emis[tid];
-      rec[0] = make_float4(s_acc[0][tid], s_acc[1][tid], s_acc[2][tid], s_acc[3][tid]);
-      rec[1] = make_float4(s_acc[4][tid], s_acc[5][tid], s_acc[6][tid], s_acc[7][tid]);
-      rec[2] = make_float4(s_acc[8][tid], s_acc[9][tid], s_acc[10][tid], s_acc[11][tid]);
-      rec[3] = make_float4(s_acc[12][tid], s_acc[13][tid], s_acc[14][tid], s_acc[15][tid]);
+    // a thread stores a quarter of a record: the four waves' sums of four components, added in wave order
+    for (int q = tid; q < 4 * count; q += GS_TILE_PIX) {
+      const int slot = q >> 2, part = q & 3;
+      float c[4];
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        c[e] = s_acc[0][4 * part + e][slot];
+#pragma unroll
+        for (int w = 1; w < WAVES; w++) c[e] += s_acc[w][4 * part + e][slot];
+      }
+      instance_grads[4 * (size_t)s_emis[slot] + part] = make_float4(c[0], c[1], c[2], c[3]);
     }
   }
 }

@@ -287,7 +287,7 @@ def test_debug_mode_gives_the_same_results_by_every_route():
 
 def test_side_stream_gives_the_same_results():
     """Everything runs on the caller's current stream: the same step on a side stream (default priority), with
-    other work in flight on the default stream, gives the same results."""
+    other work in flight on the default stream, gives the same results, bit for bit."""
     import gs_scenes
     from diff_gaussian_rasterization import GaussianRasterizer
     g, cams = gs_scenes.make_scene(1, P=120_000, n_views=1)
@@ -322,7 +322,6 @@ def test_side_stream_gives_the_same_results():
         got = run()
     side.synchronize()
     torch.cuda.synchronize()
-    for i, (a, b) in enumerate(zip(base[:6], got[:6])):
+    # gradients too: every sum of the backward pass is taken in a fixed order (no float atomics anywhere)
+    for i, (a, b) in enumerate(zip(base, got)):
         assert torch.equal(a, b), i
-    for i, (a, b) in enumerate(zip(base[6:], got[6:])):
-        assert float((a - b).norm()) <= 1e-5 * float(a.norm()) + 1e-12, i
