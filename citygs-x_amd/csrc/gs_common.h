@@ -102,6 +102,16 @@ __device__ __forceinline__ float gs_expf_core(float x) {
   return __builtin_ldexpf(p, (int)n);
 }
 
+// 1.0f / d for a normal d whose reciprocal is normal too: the operation sequence of the IEEE division
+// without its scaling and special-case steps, which change nothing in that range.  Same bits, four
+// instructions fewer.
+__device__ __forceinline__ float gs_rcp_normal(float d) {
+  const float r0 = __builtin_amdgcn_rcpf(d);
+  const float r = __builtin_fmaf(__builtin_fmaf(-d, r0, 1.0f), r0, r0);
+  const float q = __builtin_fmaf(__builtin_fmaf(-d, r, 1.0f), r, r);
+  return __builtin_fmaf(__builtin_fmaf(-d, q, 1.0f), r, q);
+}
+
 // Column-major 3x3 with the product evaluated term by term, left to right
 // (the semantics of the reference's matrix type,
 // third_party/glm/glm/detail/type_mat3x3.inl:486-518).

@@ -237,7 +237,7 @@ render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
         // the result (plane depth divides by a blended normal that may be nearly perpendicular to the
         // ray), so these operations decide how far a gradient can drift.  What follows dL/dalpha is
         // products only.
-        const float rcp1ma = 1.f / (1.f - alpha);
+        const float rcp1ma = gs_rcp_normal(1.f - alpha);  // alpha <= 0.99: the bits of 1.f / (1.f - alpha)
         T = T * rcp1ma;
         const float w = alpha * T;
         const float oml = 1.f - last_alpha;
