@@ -4,12 +4,13 @@
 // over pixels.
 //
 // Workgroup = one 16x16 tile = four 64-lane waves; a wave owns an 8x8 quadrant
-// and each of its 16-lane rows a 4x4 pixel block.  Per batch of 64 Gaussians
-// (staged in LDS in back-to-front order):
-//   * a wave ballots, for each of its rows, which Gaussians can touch the
-//     row's block (inflated alpha >= 1/255 ellipse against the block) and lie in front of the row's
-//     deepest contributor; the four rows then walk their own bit lists
-//     concurrently, so one pass of the loop handles up to four Gaussians;
+// and each of its 16-lane rows a 4x4 pixel block.  Gaussians are staged in LDS
+// 128 at a time, in back-to-front order, and worked on 64 at a time:
+//   * a wave ballots, for each of its rows, which of the 64 Gaussians can touch
+//     the row's block (inflated alpha >= 1/255 ellipse against the block) and
+//     lie in front of the row's deepest contributor; the four rows then walk
+//     their own bit lists concurrently, so one pass of the loop handles up to
+//     four Gaussians;
 //   * the 16 partial sums of a Gaussian (mean2D x/y, |mean2D| x/y, conic
 //     x/y/w, opacity, colour 3, map 5) are reduced over the row's 16 lanes by
 //     a transposing DPP reduction (15 additions instead of 64) that leaves
@@ -18,11 +19,11 @@
 //     LDS with a plain read-add-write (no atomics: an LDS float atomic costs
 //     about three cycles per active lane here, and the kernel was bound by
 //     them);
-//   * at the end of the batch the four waves' accumulators are added in wave
-//     order and every (tile, Gaussian) instance's 16 sums are stored as one
-//     64-byte record, at the instance's index in emission order (the order
-//     key emission wrote them: all instances of a Gaussian are consecutive
-//     there).  No global atomics either.
+//   * then the four waves' accumulators are added in wave order and every
+//     (tile, Gaussian) instance's 16 sums are stored as one 64-byte record, at
+//     the instance's index in emission order (the order key emission wrote
+//     them: all instances of a Gaussian are consecutive there).  No global
+//     atomics either.
 // A second kernel then sums, for every Gaussian, its consecutive records and
 // writes the five gradient tensors: a streaming pass.  Every sum is taken in a
 // fixed order, so the gradients are the same bits from run to run.  (The
@@ -39,11 +40,12 @@ namespace gs {
 
 namespace {
 
-constexpr int BATCH = GS_TILE_PIX / 4;  // Gaussians staged per round
+constexpr int BATCH = GS_TILE_PIX / 2;  // Gaussians staged in LDS per round
+constexpr int SUB = GS_WAVE;        // Gaussians whose sums are in the accumulators at a time: one ballot's worth
 constexpr int NV = 16;
-constexpr int CHUNKS = BATCH / 32;
+constexpr int CHUNKS = SUB / 32;
 constexpr int WAVES = GS_TILE_PIX / GS_WAVE;
-static_assert((WAVES * NV * (BATCH + 1)) % 4 == 0, "the accumulators are cleared 16 bytes at a time");
+static_assert(SUB * 4 == GS_TILE_PIX, "a thread hands over a quarter of one record of the sub-batch");
 
 template <bool RENDER_GEO>
 __global__ void __launch_bounds__(GS_TILE_PIX)
@@ -64,7 +66,7 @@ render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
   __shared__ float s_rgb[GS_N_RGB][BATCH];
   __shared__ float s_map[GS_N_MAP][BATCH];
   // one accumulator per wave; +1: the 16 components of one Gaussian fall in 16 different banks
-  __shared__ __align__(16) float s_acc[WAVES][NV][BATCH + 1];
+  __shared__ float s_acc[WAVES][NV][SUB + 1];
   __shared__ uint32_t s_list[GS_TILE_PIX / GS_WAVE][4][CHUNKS];
   __shared__ int s_max[GS_TILE_PIX / GS_WAVE];
 
@@ -147,10 +149,18 @@ render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
   const int start = tile_last - 1;
   const int rounds = (start + 1 + BATCH - 1) / BATCH;
 
+  // thread tid hands over components 4*part .. 4*part+3 of the sub-batch's slot tid / 4 and clears them
+  const int my_slot = tid >> 2, my_part = tid & 3;
+#pragma unroll
+  for (int w = 0; w < WAVES; w++) {
+#pragma unroll
+    for (int e = 0; e < 4; e++) s_acc[w][4 * my_part + e][my_slot] = 0.f;
+  }
+
   for (int i = 0; i < rounds; i++) {
     const int first_pos = start - i * BATCH;  // position in slot 0
     const int count = first_pos + 1 < BATCH ? first_pos + 1 : BATCH;
-    __syncthreads();
+    // (the barrier that ends the previous batch's last sub-batch has let every wave finish with the staged data)
     if (tid < count) {
       const uint32_t k_sorted = range.x + (uint32_t)(first_pos - tid);
       const uint32_t g = point_list[k_sorted];
@@ -170,152 +180,158 @@ render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
         for (int ch = 0; ch < GS_N_MAP; ch++) s_map[ch][tid] = all_map[5 * (size_t)g + ch];
       }
     }
-    for (int q = tid; q < WAVES * NV * (BATCH + 1) / 4; q += GS_TILE_PIX)
-      reinterpret_cast<float4*>(&s_acc[0][0][0])[q] = make_float4(0.f, 0.f, 0.f, 0.f);
     __syncthreads();
 
-    // per-row lists: bit b of word c of row r = slot 32c+b of the batch can touch row r's 4x4 block
+    for (int base = 0; base < count; base += SUB) {
+      // per-row lists: bit b of word c of row r = slot base+32c+b of the batch can touch row r's 4x4 block
+      {
+        const int jj = base + lane;
+        const bool valid = jj < count;
+        const float2 mu = s_xy[valid ? jj : 0];
+        const float4 cq = s_co[valid ? jj : 0];
+        const float4 cp = s_cp[valid ? jj : 0];
 #pragma unroll
-    for (int k = 0; k < BATCH / GS_WAVE; k++) {
-      const int jj = k * GS_WAVE + lane;
-      const bool valid = jj < count;
-      const float2 mu = s_xy[valid ? jj : 0];
-      const float4 cq = s_co[valid ? jj : 0];
-      const float4 cp = s_cp[valid ? jj : 0];
-#pragma unroll
-      for (int r = 0; r < 4; r++) {
-        const uint64_t hit = __ballot(valid && (first_pos - jj) < row_last_of[r] &&
-                                      ellipse_hits_row(mu, cq, cp, rt.qx0, rt.qy0, r));
-        if (lane == 0) {
-          s_list[wave][r][2 * k] = (uint32_t)hit;
-          s_list[wave][r][2 * k + 1] = (uint32_t)(hit >> 32);
-        }
-      }
-    }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-
-    {
-      int kk = 0;
-      uint32_t m = s_list[wave][row][0];
-      for (;;) {
-        if (m == 0u && kk < CHUNKS - 1) {
-          kk++;
-          m = s_list[wave][row][kk];
-        }
-        const bool has = m != 0u;
-        if (__ballot(has || kk < CHUNKS - 1) == 0ull) break;
-        const int j = has ? kk * 32 + (int)__builtin_ctz(m) : 0;
-        m &= m - 1u;
-        const int pos = first_pos - j;
-        // Straight-line from here on: every lane evaluates its row's Gaussian, and a lane for which the
-        // Gaussian does not count (behind the pixel's last contributor, outside the power window, alpha
-        // below 1/255) takes part with alpha = 0, G = 0.  Such a step leaves T unchanged (T * 1/(1-0)),
-        // contributes zeros to every sum, and only rotates the recurrence state in a way the next real
-        // step undoes exactly (fma(0, c, 1 * accum) == accum), so results are those of skipping it.
-        // Same tests as the forward pass, on the same bits.
-        const float2 xy = s_xy[j];
-        const float4 co = s_co[j];
-        const float dx = xy.x - pfx, dy = xy.y - pfy;
-        const float power = -0.5f * (co.x * dx * dx + co.z * dy * dy) - co.y * dx * dy;
-        // never true for pixels outside the image (last_contributor = 0)
-        const float floor_j = s_floor[j];
-        // (bitwise on purpose: no short-circuit branches in the loop)
-        const bool in = has & (pos < last_contributor) & !(power > 0.0f) & !(power < floor_j);
-        if (__ballot(in) == 0ull) continue;  // wave-uniform
-        const float G_raw = gs_expf_core(power);
-        const float alpha_raw = fminf(0.99f, co.w * G_raw);
-        const bool active = in & !(alpha_raw < 1.0f / 255.0f);
-        if (__ballot(active) == 0ull) continue;  // wave-uniform
-        const float alpha = active ? alpha_raw : 0.f;
-        const float G = active ? G_raw : 0.f;
-
-        float v[NV];
-        // Up to dL/dalpha the operation sequence is exactly the CPU statement's (IEEE reciprocal, explicit
-        // FMAs): upstream gradients of the geometry channels can be many orders of magnitude larger than
-        // the result (plane depth divides by a blended normal that may be nearly perpendicular to the
-        // ray), so these operations decide how far a gradient can drift.  What follows dL/dalpha is
-        // products only.
-        const float rcp1ma = gs_rcp_normal(1.f - alpha);  // alpha <= 0.99: the bits of 1.f / (1.f - alpha)
-        T = T * rcp1ma;
-        const float w = alpha * T;
-        const float oml = 1.f - last_alpha;
-        float dL_dalpha = 0.0f;
-#pragma unroll
-        for (int ch = 0; ch < GS_N_RGB; ch++) {
-          const float c = s_rgb[ch][j];
-          accum_rec[ch] = __builtin_fmaf(last_alpha, last_color[ch], oml * accum_rec[ch]);
-          last_color[ch] = c;
-          dL_dalpha = __builtin_fmaf(c - accum_rec[ch], gpix[ch], dL_dalpha);
-          v[8 + ch] = w * gpix[ch];
-        }
-        if (render_geo) {
-#pragma unroll
-          for (int ch = 0; ch < GS_N_MAP; ch++) {
-            const float c = s_map[ch][j];
-            accum_map[ch] = __builtin_fmaf(last_alpha, last_map[ch], oml * accum_map[ch]);
-            last_map[ch] = c;
-            dL_dalpha = __builtin_fmaf(c - accum_map[ch], gmap[ch], dL_dalpha);
-            v[11 + ch] = w * gmap[ch];
+        for (int r = 0; r < 4; r++) {
+          const uint64_t hit = __ballot(valid && (first_pos - jj) < row_last_of[r] &&
+                                        ellipse_hits_row(mu, cq, cp, rt.qx0, rt.qy0, r));
+          if (lane == 0) {
+            s_list[wave][r][0] = (uint32_t)hit;
+            s_list[wave][r][1] = (uint32_t)(hit >> 32);
           }
-        } else {
-#pragma unroll
-          for (int ch = 0; ch < GS_N_MAP; ch++) v[11 + ch] = 0.f;
         }
-        last_alpha = alpha;
-        dL_dalpha = __builtin_fmaf(dL_dalpha, T, -(bg_term * rcp1ma));
-        dL_dalpha = active ? dL_dalpha : 0.f;
-        const float dL_dG = co.w * dL_dalpha;
-        const float gdx = G * dx, gdy = G * dy;
-        const float dG_ddelx = -gdx * co.x - gdy * co.y;
-        const float dG_ddely = -gdy * co.z - gdx * co.y;
-        v[0] = dL_dG * dG_ddelx * ddelx_dx;
-        v[1] = dL_dG * dG_ddely * ddely_dy;
-        v[2] = fabsf(v[0]);
-        v[3] = fabsf(v[1]);
-        const float hg = -0.5f * dL_dG;
-        v[4] = hg * gdx * dx;
-        v[5] = hg * gdx * dy;
-        v[6] = hg * gdy * dy;
-        v[7] = G * dL_dalpha;
-        // lane q of the row now receives the row's total of component q
-        float tot = row_transpose_reduce16(v);
-        // Rows of this wave that are at the same Gaussian in this pass are merged, and the lowest of them
-        // adds the sum to the wave's own accumulator with a plain read-add-write: rows that write hold
-        // different Gaussians, so their addresses differ.  (An LDS float atomic takes about three cycles per
-        // active lane on this hardware, thirteen times the read-add-write.)
-        const int key = has ? j : -1 - row;
-        const int k0 = __builtin_amdgcn_readlane(key, 0), k1 = __builtin_amdgcn_readlane(key, 16);
-        const int k2 = __builtin_amdgcn_readlane(key, 32), k3 = __builtin_amdgcn_readlane(key, 48);
-        constexpr uint64_t R0 = 0xFFFFull, R1 = R0 << 16, R2 = R0 << 32, R3 = R0 << 48;
-        const uint64_t eq16 = (k0 == k1 ? R0 | R1 : 0ull) | (k2 == k3 ? R2 | R3 : 0ull);
-        const uint64_t eq32 = (k0 == k2 ? R0 | R2 : 0ull) | (k1 == k3 ? R1 | R3 : 0ull);
-        const uint64_t eq48 = (k0 == k3 ? R0 | R3 : 0ull) | (k1 == k2 ? R1 | R2 : 0ull);
-        const uint64_t follower = (k1 == k0 ? R1 : 0ull) | ((k2 == k0 || k2 == k1) ? R2 : 0ull) |
-                                  ((k3 == k0 || k3 == k1 || k3 == k2) ? R3 : 0ull);
-        if ((eq16 | eq32 | eq48) != 0ull) {  // wave-uniform
-          const float t16 = __shfl_xor(tot, 16, GS_WAVE), t32 = __shfl_xor(tot, 32, GS_WAVE);
-          const float t48 = __shfl_xor(tot, 48, GS_WAVE);
-          tot += __builtin_amdgcn_inverse_ballot_w64(eq16) ? t16 : 0.f;
-          tot += __builtin_amdgcn_inverse_ballot_w64(eq32) ? t32 : 0.f;
-          tot += __builtin_amdgcn_inverse_ballot_w64(eq48) ? t48 : 0.f;
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+
+      {
+        int kk = 0;
+        uint32_t m = s_list[wave][row][0];
+        for (;;) {
+          if (m == 0u && kk < CHUNKS - 1) {
+            kk++;
+            m = s_list[wave][row][kk];
+          }
+          const bool has = m != 0u;
+          if (__ballot(has || kk < CHUNKS - 1) == 0ull) break;
+          const int ja = has ? kk * 32 + (int)__builtin_ctz(m) : 0;  // slot of the accumulators
+          const int j = base + ja;                                   // slot of the batch
+          m &= m - 1u;
+          const int pos = first_pos - j;
+          // Straight-line from here on: every lane evaluates its row's Gaussian, and a lane for which the
+          // Gaussian does not count (behind the pixel's last contributor, outside the power window, alpha
+          // below 1/255) takes part with alpha = 0, G = 0.  Such a step leaves T unchanged (T * 1/(1-0)),
+          // contributes zeros to every sum, and only rotates the recurrence state in a way the next real
+          // step undoes exactly (fma(0, c, 1 * accum) == accum), so results are those of skipping it.
+          // Same tests as the forward pass, on the same bits.
+          const float2 xy = s_xy[j];
+          const float4 co = s_co[j];
+          const float dx = xy.x - pfx, dy = xy.y - pfy;
+          const float power = -0.5f * (co.x * dx * dx + co.z * dy * dy) - co.y * dx * dy;
+          // never true for pixels outside the image (last_contributor = 0)
+          const float floor_j = s_floor[j];
+          // (bitwise on purpose: no short-circuit branches in the loop)
+          const bool in = has & (pos < last_contributor) & !(power > 0.0f) & !(power < floor_j);
+          if (__ballot(in) == 0ull) continue;  // wave-uniform
+          const float G_raw = gs_expf_core(power);
+          const float alpha_raw = fminf(0.99f, co.w * G_raw);
+          const bool active = in & !(alpha_raw < 1.0f / 255.0f);
+          if (__ballot(active) == 0ull) continue;  // wave-uniform
+          const float alpha = active ? alpha_raw : 0.f;
+          const float G = active ? G_raw : 0.f;
+
+          float v[NV];
+          // Up to dL/dalpha the operation sequence is exactly the CPU statement's (IEEE reciprocal, explicit
+          // FMAs): upstream gradients of the geometry channels can be many orders of magnitude larger than
+          // the result (plane depth divides by a blended normal that may be nearly perpendicular to the
+          // ray), so these operations decide how far a gradient can drift.  What follows dL/dalpha is
+          // products only.
+          const float rcp1ma = gs_rcp_normal(1.f - alpha);  // alpha <= 0.99: the bits of 1.f / (1.f - alpha)
+          T = T * rcp1ma;
+          const float w = alpha * T;
+          const float oml = 1.f - last_alpha;
+          float dL_dalpha = 0.0f;
+#pragma unroll
+          for (int ch = 0; ch < GS_N_RGB; ch++) {
+            const float c = s_rgb[ch][j];
+            accum_rec[ch] = __builtin_fmaf(last_alpha, last_color[ch], oml * accum_rec[ch]);
+            last_color[ch] = c;
+            dL_dalpha = __builtin_fmaf(c - accum_rec[ch], gpix[ch], dL_dalpha);
+            v[8 + ch] = w * gpix[ch];
+          }
+          if (render_geo) {
+#pragma unroll
+            for (int ch = 0; ch < GS_N_MAP; ch++) {
+              const float c = s_map[ch][j];
+              accum_map[ch] = __builtin_fmaf(last_alpha, last_map[ch], oml * accum_map[ch]);
+              last_map[ch] = c;
+              dL_dalpha = __builtin_fmaf(c - accum_map[ch], gmap[ch], dL_dalpha);
+              v[11 + ch] = w * gmap[ch];
+            }
+          } else {
+#pragma unroll
+            for (int ch = 0; ch < GS_N_MAP; ch++) v[11 + ch] = 0.f;
+          }
+          last_alpha = alpha;
+          dL_dalpha = __builtin_fmaf(dL_dalpha, T, -(bg_term * rcp1ma));
+          dL_dalpha = active ? dL_dalpha : 0.f;
+          const float dL_dG = co.w * dL_dalpha;
+          const float gdx = G * dx, gdy = G * dy;
+          const float dG_ddelx = -gdx * co.x - gdy * co.y;
+          const float dG_ddely = -gdy * co.z - gdx * co.y;
+          v[0] = dL_dG * dG_ddelx * ddelx_dx;
+          v[1] = dL_dG * dG_ddely * ddely_dy;
+          v[2] = fabsf(v[0]);
+          v[3] = fabsf(v[1]);
+          const float hg = -0.5f * dL_dG;
+          v[4] = hg * gdx * dx;
+          v[5] = hg * gdx * dy;
+          v[6] = hg * gdy * dy;
+          v[7] = G * dL_dalpha;
+          // lane q of the row now receives the row's total of component q
+          float tot = row_transpose_reduce16(v);
+          // Rows of this wave that are at the same Gaussian in this pass are merged, and the lowest of them
+          // adds the sum to the wave's own accumulator with a plain read-add-write: rows that write hold
+          // different Gaussians, so their addresses differ.  (An LDS float atomic takes about three cycles per
+          // active lane on this hardware, thirteen times the read-add-write.)
+          const int key = has ? ja : -1 - row;
+          const int k0 = __builtin_amdgcn_readlane(key, 0), k1 = __builtin_amdgcn_readlane(key, 16);
+          const int k2 = __builtin_amdgcn_readlane(key, 32), k3 = __builtin_amdgcn_readlane(key, 48);
+          constexpr uint64_t R0 = 0xFFFFull, R1 = R0 << 16, R2 = R0 << 32, R3 = R0 << 48;
+          const uint64_t eq16 = (k0 == k1 ? R0 | R1 : 0ull) | (k2 == k3 ? R2 | R3 : 0ull);
+          const uint64_t eq32 = (k0 == k2 ? R0 | R2 : 0ull) | (k1 == k3 ? R1 | R3 : 0ull);
+          const uint64_t eq48 = (k0 == k3 ? R0 | R3 : 0ull) | (k1 == k2 ? R1 | R2 : 0ull);
+          const uint64_t follower = (k1 == k0 ? R1 : 0ull) | ((k2 == k0 || k2 == k1) ? R2 : 0ull) |
+                                    ((k3 == k0 || k3 == k1 || k3 == k2) ? R3 : 0ull);
+          if ((eq16 | eq32 | eq48) != 0ull) {  // wave-uniform
+            const float t16 = __shfl_xor(tot, 16, GS_WAVE), t32 = __shfl_xor(tot, 32, GS_WAVE);
+            const float t48 = __shfl_xor(tot, 48, GS_WAVE);
+            tot += __builtin_amdgcn_inverse_ballot_w64(eq16) ? t16 : 0.f;
+            tot += __builtin_amdgcn_inverse_ballot_w64(eq32) ? t32 : 0.f;
+            tot += __builtin_amdgcn_inverse_ballot_w64(eq48) ? t48 : 0.f;
+          }
+          if (has && !__builtin_amdgcn_inverse_ballot_w64(follower) && tot != 0.f) s_acc[wave][l16][ja] += tot;
         }
-        if (has && !__builtin_amdgcn_inverse_ballot_w64(follower) && tot != 0.f) s_acc[wave][l16][j] += tot;
       }
-    }
-    __syncthreads();
-    // a thread stores a quarter of a record: the four waves' sums of four components, added in wave order
-    for (int q = tid; q < 4 * count; q += GS_TILE_PIX) {
-      const int slot = q >> 2, part = q & 3;
-      float c[4];
+      __syncthreads();
+      // a thread stores a quarter of a record: the four waves' sums of four components, added in wave order;
+      // it leaves zeros behind for the next sub-batch
+      {
+        float c[4];
 #pragma unroll
-      for (int e = 0; e < 4; e++) {
-        c[e] = s_acc[0][4 * part + e][slot];
+        for (int e = 0; e < 4; e++) {
+          c[e] = s_acc[0][4 * my_part + e][my_slot];
+          s_acc[0][4 * my_part + e][my_slot] = 0.f;
 #pragma unroll
-        for (int w = 1; w < WAVES; w++) c[e] += s_acc[w][4 * part + e][slot];
+          for (int w = 1; w < WAVES; w++) {
+            c[e] += s_acc[w][4 * my_part + e][my_slot];
+            s_acc[w][4 * my_part + e][my_slot] = 0.f;
+          }
+        }
+        if (base + my_slot < count)
+          instance_grads[4 * (size_t)s_emis[base + my_slot] + my_part] = make_float4(c[0], c[1], c[2], c[3]);
       }
-      instance_grads[4 * (size_t)s_emis[slot] + part] = make_float4(c[0], c[1], c[2], c[3]);
+      __syncthreads();
     }
   }
 }
