@@ -21,6 +21,10 @@
 
 namespace gs {
 
+// Lane mask of a predicate.  Takes the bool itself: the int-taking __ballot makes the compiler materialise the
+// predicate as 0/1 in a vector register and compare it again.
+__device__ __forceinline__ uint64_t gs_ballot(bool p) { return __builtin_amdgcn_ballot_w64(p); }
+
 void set_error(const char* fmt, ...);
 int check_launch(const char* what, hipStream_t stream, bool sync);
 

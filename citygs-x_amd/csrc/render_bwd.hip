@@ -187,13 +187,14 @@ render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
       {
         const int jj = base + lane;
         const bool valid = jj < count;
+        const uint64_t valid_m = gs_ballot(valid);  // (masks of single comparisons, combined in scalar registers)
         const float2 mu = s_xy[valid ? jj : 0];
         const float4 cq = s_co[valid ? jj : 0];
         const float4 cp = s_cp[valid ? jj : 0];
 #pragma unroll
         for (int r = 0; r < 4; r++) {
-          const uint64_t hit = __ballot(valid && (first_pos - jj) < row_last_of[r] &&
-                                        ellipse_hits_row(mu, cq, cp, rt.qx0, rt.qy0, r));
+          const uint64_t hit = valid_m & gs_ballot((first_pos - jj) < row_last_of[r]) &
+                               gs_ballot(ellipse_hits_row(mu, cq, cp, rt.qx0, rt.qy0, r));
           if (lane == 0) {
             s_list[wave][r][0] = (uint32_t)hit;
             s_list[wave][r][1] = (uint32_t)(hit >> 32);
@@ -213,7 +214,8 @@ render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
             m = s_list[wave][row][kk];
           }
           const bool has = m != 0u;
-          if (__ballot(has || kk < CHUNKS - 1) == 0ull) break;
+          const uint64_t has_m = gs_ballot(has);
+          if ((has_m | gs_ballot(kk < CHUNKS - 1)) == 0ull) break;
           const int ja = has ? kk * 32 + (int)__builtin_ctz(m) : 0;  // slot of the accumulators
           const int j = base + ja;                                   // slot of the batch
           m &= m - 1u;
@@ -230,13 +232,15 @@ render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
           const float power = -0.5f * (co.x * dx * dx + co.z * dy * dy) - co.y * dx * dy;
           // never true for pixels outside the image (last_contributor = 0)
           const float floor_j = s_floor[j];
-          // (bitwise on purpose: no short-circuit branches in the loop)
-          const bool in = has & (pos < last_contributor) & !(power > 0.0f) & !(power < floor_j);
-          if (__ballot(in) == 0ull) continue;  // wave-uniform
+          // (lane masks of single comparisons, combined in scalar registers: no short-circuit branches in the loop)
+          const uint64_t in_m = has_m & gs_ballot(pos < last_contributor) & gs_ballot(!(power > 0.0f)) &
+                                gs_ballot(!(power < floor_j));
+          if (in_m == 0ull) continue;  // wave-uniform
           const float G_raw = gs_expf_core(power);
           const float alpha_raw = fminf(0.99f, co.w * G_raw);
-          const bool active = in & !(alpha_raw < 1.0f / 255.0f);
-          if (__ballot(active) == 0ull) continue;  // wave-uniform
+          const uint64_t active_m = in_m & gs_ballot(!(alpha_raw < 1.0f / 255.0f));
+          if (active_m == 0ull) continue;  // wave-uniform
+          const bool active = __builtin_amdgcn_inverse_ballot_w64(active_m);
           const float alpha = active ? alpha_raw : 0.f;
           const float G = active ? G_raw : 0.f;
 
@@ -355,7 +359,7 @@ reduce_instances_kernel(int P, const uint32_t* __restrict__ point_offsets, const
   // whole wave: lane l takes records l, l + 64, ..., then the 64 partial sums are added across the lanes in a fixed
   // order.  Everything else is summed by its own thread, record after record.
   constexpr uint32_t MANY = 32;
-  uint64_t many = __ballot(n > MANY);
+  uint64_t many = gs_ballot(n > MANY);
   while (many != 0ull) {
     const int owner = (int)__builtin_ctzll(many);
     many &= many - 1ull;

@@ -78,7 +78,8 @@ render_fwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
   const size_t pid = (size_t)W * py + px;
   const float pfx = (float)px, pfy = (float)py;
   const float rayx = (pfx - cx) / fx, rayy = (pfy - cy) / fy;
-  bool done = !inside;
+  // pixels that still blend, as a lane mask (wave-uniform, so it lives in scalar registers)
+  uint64_t alive = gs_ballot(inside);
   const int row_shift = 16 * row;
 
   int todo = (int)(range.y - range.x);
@@ -91,7 +92,7 @@ render_fwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
   float best_w = 0.f, best_depth = 0.f;
 
   for (int i = 0; i < rounds; i++, todo -= BATCH) {
-    const uint64_t alive_mask = __ballot(!done);
+    const uint64_t alive_mask = alive;
     if (lane == 0) s_done[wave] = alive_mask == 0ull;
     __syncthreads();
     if (s_done[0] && s_done[1] && s_done[2] && s_done[3]) break;
@@ -125,13 +126,15 @@ render_fwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
       for (int k = 0; k < BATCH / GS_WAVE; k++) {
         const int jj = k * GS_WAVE + lane;
         const bool valid = jj < count;
+        const uint64_t valid_m = gs_ballot(valid);
         const float2 mu = s_xy[valid ? jj : 0];
         const float4 cq = s_co[valid ? jj : 0];
         const float4 cp = s_cp[valid ? jj : 0];
 #pragma unroll
         for (int r = 0; r < 4; r++) {
           const bool row_alive = ((alive_mask >> (16 * r)) & 0xFFFFull) != 0ull;
-          const uint64_t b = __ballot(valid && row_alive && ellipse_hits_row(mu, cq, cp, rt.qx0, rt.qy0, r));
+          // (masks of single comparisons, combined in scalar registers)
+          const uint64_t b = row_alive ? (valid_m & gs_ballot(ellipse_hits_row(mu, cq, cp, rt.qx0, rt.qy0, r))) : 0ull;
           if (lane == 0) {
             s_list[wave][r][2 * k] = (uint32_t)b;
             s_list[wave][r][2 * k + 1] = (uint32_t)(b >> 32);
@@ -150,28 +153,29 @@ render_fwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
           m = s_list[wave][row][kk];
         }
         const bool has = m != 0u;
-        if (__ballot(has || kk < CHUNKS - 1) == 0ull) break;
+        const uint64_t has_m = gs_ballot(has);
+        if ((has_m | gs_ballot(kk < CHUNKS - 1)) == 0ull) break;
         const int j = has ? kk * 32 + (int)__builtin_ctz(m) : 0;
         m &= m - 1u;
 
         // Straight-line: every lane evaluates its row's Gaussian; a lane for which it does not count blends
-        // with weight 0, which leaves its sums unchanged bit for bit (fma(c, 0, C) == C).
+        // with weight 0, which leaves its sums unchanged bit for bit (fma(c, 0, C) == C).  The tests are kept as
+        // lane masks of single comparisons and combined in scalar registers.
         const float2 xy = s_xy[j];
         const float4 co = s_co[j];
         const float dx = xy.x - pfx, dy = xy.y - pfy;
         const float power = -0.5f * (co.x * dx * dx + co.z * dy * dy) - co.y * dx * dy;
         const float floor_j = s_floor[j];
-        // (bitwise on purpose: no short-circuit branches in the loop)
-        const bool in = has & !done & !(power > 0.0f) & !(power < floor_j);
-        if (__ballot(in) == 0ull) continue;
+        const uint64_t in_m = has_m & alive & gs_ballot(!(power > 0.0f)) & gs_ballot(!(power < floor_j));
+        if (in_m == 0ull) continue;
         const float alpha = fminf(0.99f, co.w * gs_expf_core(power));
-        const bool pass = in & !(alpha < 1.0f / 255.0f);
+        const uint64_t pass_m = in_m & gs_ballot(!(alpha < 1.0f / 255.0f));
         const float test_T = T * (1 - alpha);
-        const bool stop = pass & (test_T < 0.0001f);
-        const bool blend = pass & !stop;
-        const uint64_t bmask = __ballot(blend);
+        const uint64_t stop_m = pass_m & gs_ballot(test_T < 0.0001f);
+        const uint64_t bmask = pass_m & ~stop_m;
         if (bmask != 0ull) {
-          if (blend) n2l++;
+          const bool blend = __builtin_amdgcn_inverse_ballot_w64(bmask);
+          n2l += blend ? 1u : 0u;
           // weight once, then one fused multiply-add per channel
           const float w = blend ? alpha * T : 0.f;
 #pragma unroll
@@ -185,7 +189,7 @@ render_fwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
             best_depth = better ? s_depth[j] : best_depth;
             best_w = better ? w : best_w;
           }
-          const uint64_t omask = __ballot(blend && T > 0.5f);
+          const uint64_t omask = bmask & gs_ballot(T > 0.5f);
           if (omask != 0ull) {
             const int cnt = __popc((uint32_t)(omask >> row_shift) & 0xFFFFu);
             if (rt.l16 == 0 && cnt != 0) atomicAdd(&s_obs[j], cnt);
@@ -193,11 +197,10 @@ render_fwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
           T = blend ? test_T : T;
           last = blend ? (uint32_t)(i * BATCH + j + 1) : last;
         }
-        if (__ballot(stop) != 0ull) {
-          if (stop) done = true;
+        if (stop_m != 0ull) {
+          alive &= ~stop_m;
           // a row whose 16 pixels have all saturated drops the rest of its list
-          const uint64_t still = __ballot(!done);
-          if (((uint32_t)(still >> row_shift) & 0xFFFFu) == 0u) {
+          if (((uint32_t)(alive >> row_shift) & 0xFFFFu) == 0u) {
             m = 0u;
             kk = CHUNKS - 1;
           }
