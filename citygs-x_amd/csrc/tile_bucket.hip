@@ -363,22 +363,53 @@ __device__ __forceinline__ void exchange_step(uint64_t (&v)[E], const uint64_t (
   }
 }
 
+// x of lane (lane ^ J), J a power of two below 64, without going through the LDS crossbar: DPP moves inside a
+// 16-lane row (xor 4 = reverse the quads' lanes, then mirror the half rows), v_permlane16_swap / v_permlane32_swap
+// across rows and halves.  A variable-distance __shfl_xor is a ds_bpermute, whose latency every one of the sort's
+// dependent steps would wait for.  All 64 lanes must be active.
+template <int J>
+__device__ __forceinline__ uint32_t xor_lane(uint32_t x, uint32_t lane) {
+  static_assert(J == 1 || J == 2 || J == 4 || J == 8 || J == 16 || J == 32, "distance inside a wave");
+  if constexpr (J == 1) {
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0xB1, 0xF, 0xF, false);  // quad_perm [1,0,3,2]
+  } else if constexpr (J == 2) {
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x4E, 0xF, 0xF, false);  // quad_perm [2,3,0,1]
+  } else if constexpr (J == 4) {
+    const int t = __builtin_amdgcn_update_dpp(0, (int)x, 0x1B, 0xF, 0xF, false);     // quad_perm [3,2,1,0]: lane ^ 3
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, t, 0x141, 0xF, 0xF, false);      // row_half_mirror: lane ^ 7
+  } else if constexpr (J == 8) {
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x128, 0xF, 0xF, false);  // row_ror:8
+  } else if constexpr (J == 16) {
+    // [0]: odd rows replaced by the even rows below them, [1]: even rows replaced by the odd rows above them
+    const auto r = __builtin_amdgcn_permlane16_swap(x, x, false, false);
+    return (lane & 16u) ? r[0] : r[1];
+  } else {
+    // [0]: upper half replaced by the lower half, [1]: lower half replaced by the upper half
+    const auto r = __builtin_amdgcn_permlane32_swap(x, x, false, false);
+    return (lane & 32u) ? r[0] : r[1];
+  }
+}
+
+// One step of the network with the partner in lane ^ J.
+template <int E, int J>
+__device__ __forceinline__ void lane_step(uint64_t (&v)[E], uint32_t row0, uint32_t lane, uint32_t k) {
+  uint64_t other[E];
+#pragma unroll
+  for (int r = 0; r < E; r++) {
+    const uint32_t lo = xor_lane<J>((uint32_t)v[r], lane);
+    const uint32_t hi = xor_lane<J>((uint32_t)(v[r] >> 32), lane);
+    other[r] = ((uint64_t)hi << 32) | lo;
+  }
+  exchange_step<E>(v, other, row0, lane, k, (lane & (uint32_t)J) == 0);
+}
+
 template <int E, int W>
 __device__ __forceinline__ void register_sort(uint64_t (&v)[E], uint32_t wave, uint32_t lane, uint64_t* s_x) {
   constexpr uint32_t M = 64u * E * W;
   const uint32_t row0 = wave * E;
   for (uint32_t k = 2; k <= M; k <<= 1) {
-    for (uint32_t j = k >> 1; j > 0; j >>= 1) {
-      if (j < 64) {
-        uint64_t other[E];
-#pragma unroll
-        for (int r = 0; r < E; r++) {
-          const uint32_t lo = __shfl_xor((uint32_t)v[r], (int)j, 64);
-          const uint32_t hi = __shfl_xor((uint32_t)(v[r] >> 32), (int)j, 64);
-          other[r] = ((uint64_t)hi << 32) | lo;
-        }
-        exchange_step<E>(v, other, row0, lane, k, (lane & j) == 0);
-      } else if (j < 64u * E) {
+    for (uint32_t j = k >> 1; j >= 64; j >>= 1) {
+      if (j < 64u * E) {
         const uint32_t jr = j >> 6;
 #pragma unroll
         for (int b = 1; b < E; b <<= 1) {
@@ -407,6 +438,13 @@ __device__ __forceinline__ void register_sort(uint64_t (&v)[E], uint32_t wave, u
         exchange_step<E>(v, other, row0, lane, k, (wave & jw) == 0);
       }
     }
+    // the steps with the partner in another lane: distances min(k / 2, 32) down to 1
+    if (k >= 64) lane_step<E, 32>(v, row0, lane, k);
+    if (k >= 32) lane_step<E, 16>(v, row0, lane, k);
+    if (k >= 16) lane_step<E, 8>(v, row0, lane, k);
+    if (k >= 8) lane_step<E, 4>(v, row0, lane, k);
+    if (k >= 4) lane_step<E, 2>(v, row0, lane, k);
+    lane_step<E, 1>(v, row0, lane, k);
   }
 }
 
