@@ -30,8 +30,9 @@
 // reference issues 16 global float atomics per pixel and Gaussian,
 // cuda_rasterizer/backward.cu:510-563.)
 // The per-pixel arithmetic is, operation for operation, the CPU statement's;
-// only the order in which pixels are summed differs, so gradients agree with a
-// CPU evaluation to rounding of the sums, not bit for bit.
+// only the order in which pixels are summed differs (and the constant factors
+// W/2, H/2 of the mean2D gradients multiply the sums instead of every term), so
+// gradients agree with a CPU evaluation to rounding of the sums, not bit for bit.
 #include "gs_common.h"
 #include "gs_kernels.h"
 #include "render_common.h"
@@ -142,7 +143,6 @@ render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
   float last_alpha = 0.f;
   float accum_rec[GS_N_RGB] = {0.f, 0.f, 0.f}, accum_map[GS_N_MAP] = {0.f, 0.f, 0.f, 0.f, 0.f};
   float last_color[GS_N_RGB] = {0.f, 0.f, 0.f}, last_map[GS_N_MAP] = {0.f, 0.f, 0.f, 0.f, 0.f};
-  const float ddelx_dx = (float)(0.5 * W), ddely_dy = (float)(0.5 * H);
 
   // Positions are 0-based indices into the tile's list; the walk starts at the tile's deepest contributor.
   // Slot j of batch i holds position start - (i*BATCH + j).
@@ -283,17 +283,17 @@ render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
           const float gdx = G * dx, gdy = G * dy;
           const float dG_ddelx = -gdx * co.x - gdy * co.y;
           const float dG_ddely = -gdy * co.z - gdx * co.y;
-          v[0] = dL_dG * dG_ddelx * ddelx_dx;
-          v[1] = dL_dG * dG_ddely * ddely_dy;
-          v[2] = fabsf(v[0]);
-          v[3] = fabsf(v[1]);
+          // (the factors W/2 and H/2 from pixel to normalised coordinates are applied once per Gaussian, to the
+          // sums, by the reduction kernel; the sums of absolute values are formed inside the row reduction)
+          v[0] = dL_dG * dG_ddelx;
+          v[1] = dL_dG * dG_ddely;
           const float hg = -0.5f * dL_dG;
           v[4] = hg * gdx * dx;
           v[5] = hg * gdx * dy;
           v[6] = hg * gdy * dy;
           v[7] = G * dL_dalpha;
           // lane q of the row now receives the row's total of component q
-          float tot = row_transpose_reduce16(v);
+          float tot = row_transpose_reduce16_abs23(v);
           // Rows of this wave that are at the same Gaussian in this pass are merged, and the lowest of them
           // adds the sum to the wave's own accumulator with a plain read-add-write: rows that write hold
           // different Gaussians, so their addresses differ.  (An LDS float atomic takes about three cycles per
@@ -345,7 +345,7 @@ render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
 // opacity, rgb(3), map(5)].  Every output element is written.
 __global__ void __launch_bounds__(GS_BLOCK_1D)
 reduce_instances_kernel(int P, const uint32_t* __restrict__ point_offsets, const float4* __restrict__ instance_grads,
-                        int render_geo, float2* __restrict__ dL_dmean2D, float* __restrict__ dL_dmean2D_abs,
+                        float ddelx_dx, float ddely_dy, int render_geo, float2* __restrict__ dL_dmean2D, float* __restrict__ dL_dmean2D_abs,
                         float4* __restrict__ dL_dconic_opacity, float* __restrict__ dL_dcolors,
                         float* __restrict__ dL_dall_map) {
   const int i = blockIdx.x * GS_BLOCK_1D + threadIdx.x;
@@ -389,9 +389,10 @@ reduce_instances_kernel(int P, const uint32_t* __restrict__ point_offsets, const
       add(a0, rec[0]); add(a1, rec[1]); add(a2, rec[2]); add(a3, rec[3]);
     }
   }
-  dL_dmean2D[i] = make_float2(a0.x, a0.y);
-  dL_dmean2D_abs[3 * (size_t)i] = a0.z;
-  dL_dmean2D_abs[3 * (size_t)i + 1] = a0.w;
+  // records hold the mean2D sums per pixel unit: d(pixel offset)/d(normalised coordinate) = W/2, H/2
+  dL_dmean2D[i] = make_float2(a0.x * ddelx_dx, a0.y * ddely_dy);
+  dL_dmean2D_abs[3 * (size_t)i] = a0.z * ddelx_dx;
+  dL_dmean2D_abs[3 * (size_t)i + 1] = a0.w * ddely_dy;
   dL_dmean2D_abs[3 * (size_t)i + 2] = 0.f;
   dL_dconic_opacity[i] = a1;
   dL_dcolors[3 * (size_t)i] = a2.x;
@@ -424,7 +425,8 @@ int launch_render_bwd(const RenderBwdArgs& a, hipStream_t stream) {
                        a.compute_locally, a.dL_dpix, a.dL_dout_all_map, a.dL_dout_plane_depth, a.emission_sorted,
                        (float4*)a.instance_grads);
   hipLaunchKernelGGL(reduce_instances_kernel, dim3((a.P + GS_BLOCK_1D - 1) / GS_BLOCK_1D), dim3(GS_BLOCK_1D), 0,
-                     stream, a.P, a.point_offsets, (const float4*)a.instance_grads, a.render_geo,
+                     stream, a.P, a.point_offsets, (const float4*)a.instance_grads, (float)(0.5 * a.W),
+                     (float)(0.5 * a.H), a.render_geo,
                      (float2*)a.dL_dmean2D, a.dL_dmean2D_abs, (float4*)a.dL_dconic_opacity, a.dL_dcolors,
                      a.dL_dall_map);
   return 0;

@@ -247,4 +247,62 @@ __device__ __forceinline__ float row_transpose_reduce16(float* v) {
   return v[0];
 }
 
+// The same with values 2 and 3 defined as |value 0| and |value 1|: their first step reads v[0] and v[1] through the
+// absolute-value source modifier (before those registers are overwritten), so the caller never forms them; v[2] and
+// v[3] need not be set on entry.
+__device__ __forceinline__ float row_transpose_reduce16_abs23(float* v) {
+  const uint64_t bit1_lanes = 0xCCCCCCCCCCCCCCCCull, bit0_lanes = 0xAAAAAAAAAAAAAAAAull;
+  // A DPP operand written by the preceding VALU instruction needs two idle issue slots first; the s_nop 1
+  // between the steps provide them, inside a step no instruction reads a register written less than two
+  // instructions earlier through DPP.
+  asm volatile(
+      "s_nop 1\n\t"
+      // distance 8: lanes 0-7 of a row keep values 0-7, lanes 8-15 keep values 8-15
+      "v_add_f32_dpp %2, |%0|, |%0| row_ror:8 row_mask:0xf bank_mask:0xf\n\t"
+      "v_add_f32_dpp %3, |%1|, |%1| row_ror:8 row_mask:0xf bank_mask:0xf\n\t"
+      "v_add_f32_dpp %0, %0, %0 row_ror:8 row_mask:0xf bank_mask:0xf\n\t"
+      "v_add_f32_dpp %1, %1, %1 row_ror:8 row_mask:0xf bank_mask:0xf\n\t"
+      "v_add_f32_dpp %4, %4, %4 row_ror:8 row_mask:0xf bank_mask:0xf\n\t"
+      "v_add_f32_dpp %5, %5, %5 row_ror:8 row_mask:0xf bank_mask:0xf\n\t"
+      "v_add_f32_dpp %6, %6, %6 row_ror:8 row_mask:0xf bank_mask:0xf\n\t"
+      "v_add_f32_dpp %7, %7, %7 row_ror:8 row_mask:0xf bank_mask:0xf\n\t"
+      "v_add_f32_dpp %0, %8, %8 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+      "v_add_f32_dpp %1, %9, %9 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+      "v_add_f32_dpp %2, %10, %10 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+      "v_add_f32_dpp %3, %11, %11 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+      "v_add_f32_dpp %4, %12, %12 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+      "v_add_f32_dpp %5, %13, %13 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+      "v_add_f32_dpp %6, %14, %14 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+      "v_add_f32_dpp %7, %15, %15 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+      "s_nop 1\n\t"
+      // distance 4: lanes with bit 2 clear (banks 0, 2) keep registers 0-3 and add lane +4's copy,
+      // the others keep registers 4-7 and add lane -4's copy
+      "v_add_f32_dpp %0, %0, %0 row_shl:4 row_mask:0xf bank_mask:0x5\n\t"
+      "v_add_f32_dpp %1, %1, %1 row_shl:4 row_mask:0xf bank_mask:0x5\n\t"
+      "v_add_f32_dpp %2, %2, %2 row_shl:4 row_mask:0xf bank_mask:0x5\n\t"
+      "v_add_f32_dpp %3, %3, %3 row_shl:4 row_mask:0xf bank_mask:0x5\n\t"
+      "v_add_f32_dpp %0, %4, %4 row_shr:4 row_mask:0xf bank_mask:0xa\n\t"
+      "v_add_f32_dpp %1, %5, %5 row_shr:4 row_mask:0xf bank_mask:0xa\n\t"
+      "v_add_f32_dpp %2, %6, %6 row_shr:4 row_mask:0xf bank_mask:0xa\n\t"
+      "v_add_f32_dpp %3, %7, %7 row_shr:4 row_mask:0xf bank_mask:0xa\n\t"
+      "s_nop 1\n\t"
+      // distance 2: + lane^2; lanes with bit 1 set keep registers 2, 3
+      "v_add_f32_dpp %0, %0, %0 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf\n\t"
+      "v_add_f32_dpp %1, %1, %1 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf\n\t"
+      "v_add_f32_dpp %2, %2, %2 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf\n\t"
+      "v_add_f32_dpp %3, %3, %3 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf\n\t"
+      "v_cndmask_b32_e64 %0, %0, %2, %16\n\t"
+      "v_cndmask_b32_e64 %1, %1, %3, %16\n\t"
+      "s_nop 1\n\t"
+      // distance 1: + lane^1; lanes with bit 0 set keep register 1
+      "v_add_f32_dpp %0, %0, %0 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf\n\t"
+      "v_add_f32_dpp %1, %1, %1 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf\n\t"
+      "s_nop 0\n\t"
+      "v_cndmask_b32_e64 %0, %0, %1, %17\n\t"
+      : "+v"(v[0]), "+v"(v[1]), "=&v"(v[2]), "=&v"(v[3]), "+v"(v[4]), "+v"(v[5]), "+v"(v[6]), "+v"(v[7])
+      : "v"(v[8]), "v"(v[9]), "v"(v[10]), "v"(v[11]), "v"(v[12]), "v"(v[13]), "v"(v[14]), "v"(v[15]),
+        "s"(bit1_lanes), "s"(bit0_lanes));
+  return v[0];
+}
+
 }  // namespace gs
