@@ -966,6 +966,16 @@ int gs_inclusive_sum(int64_t n, const uint32_t* in, uint32_t* out, void* workspa
   return check_launch("inclusive_sum", (hipStream_t)stream, false);
 }
 
+int64_t gs_inclusive_sum_static_max(void) { return static_scan_max_elements(); }
+
+int gs_inclusive_sum_static(int64_t n, const uint32_t* in, uint32_t* out, gs_stream_t stream) {
+  GS_REQUIRE(n >= 0, "gs_inclusive_sum_static: negative n");
+  if (n == 0) return 0;
+  GS_REQUIRE(in && out, "gs_inclusive_sum_static: null pointer");
+  if (launch_inclusive_sum_static(n, in, out, (hipStream_t)stream)) return 1;
+  return check_launch("inclusive_sum_static", (hipStream_t)stream, false);
+}
+
 int gs_duplicate_with_keys(int P, int width, int height, const float* means2D, const float* depths,
                            const uint32_t* offsets, const int* radii, const uint8_t* compute_locally, uint64_t* keys,
                            uint32_t* values, gs_stream_t stream) {

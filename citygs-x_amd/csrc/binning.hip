@@ -2,6 +2,8 @@
 // emission and per-tile range detection
 // (cuda_rasterizer/rasterizer_impl.cu:74-144, :264-288, :633-697).
 // All of it is integer / bit work and must match a CPU bit for bit.
+#include <mutex>
+
 #include "gs_common.h"
 #include "gs_kernels.h"
 
@@ -262,6 +264,61 @@ int launch_inclusive_sum(int64_t n, const uint32_t* in, uint32_t* out, void* tem
 
 int launch_exclusive_sum(int64_t n, const uint32_t* in, uint32_t* out, void* temp, hipStream_t stream) {
   return scan_impl(n, in, out, temp, true, nullptr, stream);
+}
+
+// ---- inclusive sum whose spine lives in a static device array (for callers that must not allocate) ----
+// The array is part of the code object: every GPU the library runs on holds its own copy, at its own address,
+// until the process ends.  Host code never passes the array's name to a kernel (there it is a host-side
+// stand-in, not a device address): the device address is looked up once per device with hipGetSymbolAddress
+// and kept in g_static_spine[device].
+constexpr int64_t STATIC_SCAN_MAX = (int64_t)1 << 27;  // elements
+constexpr size_t STATIC_SPINE_WORDS = (size_t)(STATIC_SCAN_MAX / SCAN_TILE) + 1;  // block sums + overflow word
+static __device__ __align__(256) uint32_t scratch[STATIC_SPINE_WORDS];
+
+namespace {
+constexpr int STATIC_MAX_DEVICES = 64;
+std::mutex g_static_mutex;
+uint32_t* g_static_spine[STATIC_MAX_DEVICES] = {};
+}  // namespace
+
+int64_t static_scan_max_elements() { return STATIC_SCAN_MAX; }
+
+// Device address of the current device's copy of the array (looked up on the first call per device).
+static int static_spine(uint32_t** out) {
+  int dev = -1;
+  GS_HIP_TRY(hipGetDevice(&dev));
+  if (dev < 0 || dev >= STATIC_MAX_DEVICES) {
+    set_error("gs_inclusive_sum_static: device ordinal %d outside the supported range [0, %d)", dev,
+              STATIC_MAX_DEVICES);
+    return 1;
+  }
+  std::lock_guard<std::mutex> lock(g_static_mutex);
+  if (g_static_spine[dev] == nullptr) {
+    uint32_t* p = nullptr;
+    GS_HIP_TRY(hipGetSymbolAddress((void**)&p, HIP_SYMBOL(scratch)));
+    if (p == nullptr) {
+      set_error("gs_inclusive_sum_static: hipGetSymbolAddress returned a null address");
+      return 1;
+    }
+    g_static_spine[dev] = p;
+  }
+  *out = g_static_spine[dev];
+  return 0;
+}
+
+// The scan of launch_inclusive_sum with the spine in the static array.  Every word of the spine that a call
+// reads is written by the same call first (block sums by the first kernel, the overflow word by the second),
+// so nothing has to be cleared; calls that overlap on one GPU race on the array.
+int launch_inclusive_sum_static(int64_t n, const uint32_t* in, uint32_t* out, hipStream_t stream) {
+  if (n <= 0) return 0;
+  if (n > STATIC_SCAN_MAX) {
+    set_error("gs_inclusive_sum_static: n = %lld exceeds the static scratch array's capacity of %lld elements",
+              (long long)n, (long long)STATIC_SCAN_MAX);
+    return 1;
+  }
+  uint32_t* spine = nullptr;
+  if (static_spine(&spine)) return 1;
+  return scan_impl(n, in, out, spine, false, nullptr, stream);
 }
 
 // exclusive prefix sums of small counts (a 0/1 mask gives the ranks of its set bytes)

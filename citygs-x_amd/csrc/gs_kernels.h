@@ -64,6 +64,10 @@ int launch_exclusive_sum_u8(int64_t n, const uint8_t* in, uint32_t* out, void* t
 int launch_inclusive_sum(int64_t n, const uint32_t* in, uint32_t* out, void* temp, hipStream_t stream,
                          uint32_t* total_out = nullptr);
 int launch_exclusive_sum(int64_t n, const uint32_t* in, uint32_t* out, void* temp, hipStream_t stream);
+// the inclusive sum with its spine in a static device array instead of a workspace: allocates nothing, takes at
+// most static_scan_max_elements() elements, and calls that overlap on one GPU share (and race on) the array
+int64_t static_scan_max_elements();
+int launch_inclusive_sum_static(int64_t n, const uint32_t* in, uint32_t* out, hipStream_t stream);
 int launch_duplicate_with_keys(int P, int W, int H, const float* means2D, const float* depths,
                                const uint32_t* offsets, const int* radii, const uint8_t* compute_locally,
                                uint64_t* keys, uint32_t* values, uint32_t* emission /*optional*/,

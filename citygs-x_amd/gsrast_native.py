@@ -55,6 +55,8 @@ _SIGNATURES = {
     "gs_tile_count": (_i, [_i, _i, _i, _vp, _vp, _vp, _vp, _vp]),
     "gs_scan_workspace_bytes": (_sz, [_i64]),
     "gs_inclusive_sum": (_i, [_i64, _vp, _vp, _vp, _sz, _vp]),
+    "gs_inclusive_sum_static_max": (_i64, []),
+    "gs_inclusive_sum_static": (_i, [_i64, _vp, _vp, _vp]),
     "gs_duplicate_with_keys": (_i, [_i, _i, _i] + [_vp] * 8),
     "gs_sort_workspace_bytes": (_sz, [_i64]),
     "gs_sort_status": (_i, [_vp, _vp]),

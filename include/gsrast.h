@@ -295,6 +295,18 @@ size_t gs_scan_workspace_bytes(int64_t n);
 int gs_inclusive_sum(int64_t n, const uint32_t* in, uint32_t* out, void* workspace, size_t workspace_bytes,
                      gs_stream_t stream);
 
+/* No counterpart in the reference: gs_inclusive_sum for callers that cannot allocate device memory (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  Same result as gs_inclusive_sum,
+ * no workspace argument: the scan's spine (one word per 2048 elements) lives in a static device array inside the
+ * library, 256 KiB, which every GPU the library runs on holds until the process ends.  n may be at most
+ * gs_inclusive_sum_static_max() = 2^27 elements; a larger n is refused with an error.  The call allocates and
+ * frees nothing (the first call on a device looks the array's device address up).  Every call on a GPU shares
+ * that GPU's array: the call itself writes every word it later reads, so nothing has to be cleared between
+ * calls, but calls that overlap on one GPU (two streams, two threads) race on it and must be serialised by
+ * the caller.  in and out may be the same array. */
+int64_t gs_inclusive_sum_static_max(void);
+int gs_inclusive_sum_static(int64_t n, const uint32_t* in, uint32_t* out, gs_stream_t stream);
+
 /* duplicateWithKeys (CR/rasterizer_impl.cu:74-117). offsets = inclusive sum of tiles_touched. */
 int gs_duplicate_with_keys(int P, int width, int height, const float* means2D, const float* depths,
                            const uint32_t* offsets, const int* radii, const uint8_t* compute_locally,
