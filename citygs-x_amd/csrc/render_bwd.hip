@@ -33,6 +33,8 @@
 // only the order in which pixels are summed differs (and the constant factors
 // W/2, H/2 of the mean2D gradients multiply the sums instead of every term), so
 // gradients agree with a CPU evaluation to rounding of the sums, not bit for bit.
+#include <type_traits>
+
 #include "gs_common.h"
 #include "gs_kernels.h"
 #include "render_common.h"
@@ -49,7 +51,7 @@ constexpr int WAVES = GS_TILE_PIX / GS_WAVE;
 static_assert(SUB * 4 == GS_TILE_PIX, "a thread hands over a quarter of one record of the sub-batch");
 
 template <bool RENDER_GEO>
-__global__ void __launch_bounds__(GS_TILE_PIX)
+__global__ void __launch_bounds__(GS_TILE_PIX) __attribute__((amdgpu_waves_per_eu(5)))
 render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__ point_list, int W, int H, float fx,
                   float fy, const float* __restrict__ bg, const float2* __restrict__ means2D,
                   const float4* __restrict__ conic_opacity, const float* __restrict__ rgb,
@@ -70,6 +72,7 @@ render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
   __shared__ float s_acc[WAVES][NV][SUB + 1];
   __shared__ uint32_t s_list[GS_TILE_PIX / GS_WAVE][4][CHUNKS];
   __shared__ int s_max[GS_TILE_PIX / GS_WAVE];
+  __shared__ int s_bad[GS_TILE_PIX / GS_WAVE];
 
   const int tid = threadIdx.x;
   const RowThread rt = row_thread(blockIdx.x, blockIdx.y);
@@ -161,6 +164,10 @@ render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
     const int first_pos = start - i * BATCH;  // position in slot 0
     const int count = first_pos + 1 < BATCH ? first_pos + 1 : BATCH;
     // (the barrier that ends the previous batch's last sub-batch has let every wave finish with the staged data)
+    // (a lane for which a Gaussian does not count takes part with alpha = 0, which is exact as long as the
+    // Gaussian's colour and geometry channels are finite; a batch holding a non-finite one is walked by the
+    // variant of the loop that leaves such a lane's recurrence state alone instead)
+    bool finite = true;
     if (tid < count) {
       const uint32_t k_sorted = range.x + (uint32_t)(first_pos - tid);
       const uint32_t g = point_list[k_sorted];
@@ -172,15 +179,29 @@ render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
       float pfl;
       s_cp[tid] = cull_params(co, pfl);
       s_floor[tid] = pfl;
-      s_rgb[0][tid] = rgb[3 * (size_t)g];
-      s_rgb[1][tid] = rgb[3 * (size_t)g + 1];
-      s_rgb[2][tid] = rgb[3 * (size_t)g + 2];
+      const float c0 = rgb[3 * (size_t)g], c1 = rgb[3 * (size_t)g + 1], c2 = rgb[3 * (size_t)g + 2];
+      s_rgb[0][tid] = c0;
+      s_rgb[1][tid] = c1;
+      s_rgb[2][tid] = c2;
+      float mag = fmaxf(fmaxf(fabsf(c0), fabsf(c1)), fabsf(c2));
+      finite = c0 == c0 && c1 == c1 && c2 == c2;
       if (render_geo) {
 #pragma unroll
-        for (int ch = 0; ch < GS_N_MAP; ch++) s_map[ch][tid] = all_map[5 * (size_t)g + ch];
+        for (int ch = 0; ch < GS_N_MAP; ch++) {
+          const float v = all_map[5 * (size_t)g + ch];
+          s_map[ch][tid] = v;
+          mag = fmaxf(mag, fabsf(v));
+          finite = finite && v == v;
+        }
       }
+      finite = finite && mag < __builtin_inff();
+    }
+    {
+      const uint64_t bad_m = gs_ballot(!finite);
+      if (lane == 0) s_bad[wave] = bad_m != 0ull;
     }
     __syncthreads();
+    const bool select_state = (s_bad[0] | s_bad[1] | s_bad[2] | s_bad[3]) != 0;
 
     for (int base = 0; base < count; base += SUB) {
       // per-row lists: bit b of word c of row r = slot base+32c+b of the batch can touch row r's 4x4 block
@@ -205,7 +226,12 @@ render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
       __builtin_amdgcn_wave_barrier();
       __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 
-      {
+      // SELECT: a lane for which the Gaussian does not count takes the Gaussian's colour and geometry channels
+      // as 0 (its step then still only rotates the recurrence state: alpha = 0 with a finite colour), so that a
+      // non-finite channel only reaches the pixels that blended it in the forward pass, as in the reference
+      // (cuda_rasterizer/backward.cu:463-472).  Same bits for finite inputs.
+      auto walk = [&](auto select_tag) {
+        constexpr bool SELECT = decltype(select_tag)::value;
         int kk = 0;
         uint32_t m = s_list[wave][row][0];
         for (;;) {
@@ -257,7 +283,7 @@ render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
           float dL_dalpha = 0.0f;
 #pragma unroll
           for (int ch = 0; ch < GS_N_RGB; ch++) {
-            const float c = s_rgb[ch][j];
+            const float c = (!SELECT || active) ? s_rgb[ch][j] : 0.f;
             accum_rec[ch] = __builtin_fmaf(last_alpha, last_color[ch], oml * accum_rec[ch]);
             last_color[ch] = c;
             dL_dalpha = __builtin_fmaf(c - accum_rec[ch], gpix[ch], dL_dalpha);
@@ -266,7 +292,7 @@ render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
           if (render_geo) {
 #pragma unroll
             for (int ch = 0; ch < GS_N_MAP; ch++) {
-              const float c = s_map[ch][j];
+              const float c = (!SELECT || active) ? s_map[ch][j] : 0.f;
               accum_map[ch] = __builtin_fmaf(last_alpha, last_map[ch], oml * accum_map[ch]);
               last_map[ch] = c;
               dL_dalpha = __builtin_fmaf(c - accum_map[ch], gmap[ch], dL_dalpha);
@@ -316,7 +342,9 @@ render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
           }
           if (has && !__builtin_amdgcn_inverse_ballot_w64(follower) && tot != 0.f) s_acc[wave][l16][ja] += tot;
         }
-      }
+      };
+      if (select_state) walk(std::true_type{});
+      else walk(std::false_type{});
       __syncthreads();
       // a thread stores a quarter of a record: the four waves' sums of four components, added in wave order;
       // it leaves zeros behind for the next sub-batch

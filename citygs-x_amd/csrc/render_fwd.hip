@@ -20,6 +20,8 @@
 // counts and images match a CPU evaluation bit for bit; exp() is gs_expf.
 // out_observe increments are counted per row with a ballot, summed per
 // workgroup in LDS and added once per (tile, Gaussian).
+#include <type_traits>
+
 #include "gs_common.h"
 #include "gs_kernels.h"
 #include "render_common.h"
@@ -58,6 +60,7 @@ render_fwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
   __shared__ int s_obs[BATCH];
   __shared__ uint32_t s_list[GS_TILE_PIX / GS_WAVE][4][CHUNKS];
   __shared__ int s_done[GS_TILE_PIX / GS_WAVE];
+  __shared__ int s_bad[GS_TILE_PIX / GS_WAVE];
   __shared__ int s_red[2][GS_TILE_PIX / GS_WAVE];
 
   const int tid = threadIdx.x;
@@ -66,16 +69,29 @@ render_fwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
   const uint32_t tile = blockIdx.y * gridDim.x + blockIdx.x;
   const uint2 range = ranges[tile];
   if (tid == 0) n_render[tile] = (int)(range.y - range.x);
+  const uint32_t px = rt.px, py = rt.py;
+  const bool inside = px < (uint32_t)W && py < (uint32_t)H;
+  const size_t pid = (size_t)W * py + px;
   if (!compute_locally[tile]) {
+    // A tile that is not computed here reads zero in every image, as in the reference, whose binding
+    // allocates the images zero-filled (rasterize_points.cu:303-307) and whose kernel returns before writing.
+    if (inside) {
+      const size_t HW = (size_t)H * W;
+#pragma unroll
+      for (int ch = 0; ch < GS_N_RGB; ch++) out_color[ch * HW + pid] = 0.f;
+      if (render_geo) {
+#pragma unroll
+        for (int ch = 0; ch < GS_N_MAP; ch++) out_all_map[ch * HW + pid] = 0.f;
+        out_plane_depth[pid] = 0.f;
+      }
+      if (MAX_DEPTH) out_max_weight_depth[pid] = 0.f;
+    }
     if (tid == 0) {
       n_consider[tile] = 0;
       n_contrib_tile[tile] = 0;
     }
     return;
   }
-  const uint32_t px = rt.px, py = rt.py;
-  const bool inside = px < (uint32_t)W && py < (uint32_t)H;
-  const size_t pid = (size_t)W * py + px;
   const float pfx = (float)px, pfy = (float)py;
   const float rayx = (pfx - cx) / fx, rayy = (pfy - cy) / fy;
   // pixels that still blend, as a lane mask (wave-uniform, so it lives in scalar registers)
@@ -98,6 +114,10 @@ render_fwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
     if (s_done[0] && s_done[1] && s_done[2] && s_done[3]) break;
 
     const int count = todo < BATCH ? todo : BATCH;
+    // A lane for which a Gaussian does not count blends it with weight 0, which is exact as long as the
+    // Gaussian's colour and geometry channels are finite; a batch that holds a non-finite one is walked by
+    // the variant of the loop that selects instead (below).
+    bool finite = true;
     if (tid < count) {
       const uint32_t g = point_list[range.x + (uint32_t)i * BATCH + tid];
       const float2 xy = means2D[g];
@@ -108,17 +128,31 @@ render_fwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
       s_co[tid] = co;
       s_cp[tid] = cull_params(co, pfl);
       s_floor[tid] = pfl;
-      s_rgb[0][tid] = rgb[3 * (size_t)g];
-      s_rgb[1][tid] = rgb[3 * (size_t)g + 1];
-      s_rgb[2][tid] = rgb[3 * (size_t)g + 2];
+      const float c0 = rgb[3 * (size_t)g], c1 = rgb[3 * (size_t)g + 1], c2 = rgb[3 * (size_t)g + 2];
+      s_rgb[0][tid] = c0;
+      s_rgb[1][tid] = c1;
+      s_rgb[2][tid] = c2;
+      float mag = fmaxf(fmaxf(fabsf(c0), fabsf(c1)), fabsf(c2));
+      finite = c0 == c0 && c1 == c1 && c2 == c2;
       if (render_geo) {
 #pragma unroll
-        for (int ch = 0; ch < GS_N_MAP; ch++) s_map[ch][tid] = all_map[5 * (size_t)g + ch];
+        for (int ch = 0; ch < GS_N_MAP; ch++) {
+          const float v = all_map[5 * (size_t)g + ch];
+          s_map[ch][tid] = v;
+          mag = fmaxf(mag, fabsf(v));
+          finite = finite && v == v;
+        }
       }
+      finite = finite && mag < __builtin_inff();
       if (MAX_DEPTH) s_depth[tid] = depths[g];
+    }
+    {
+      const uint64_t bad_m = gs_ballot(!finite);
+      if (lane == 0) s_bad[wave] = bad_m != 0ull;
     }
     s_obs[tid] = 0;
     __syncthreads();
+    const bool select_blend = (s_bad[0] | s_bad[1] | s_bad[2] | s_bad[3]) != 0;
 
     if (alive_mask != 0ull) {
       // per-row lists: bit b of word c of row r = Gaussian 32c+b of the batch can touch row r's 4x4 block
@@ -145,6 +179,11 @@ render_fwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
       __builtin_amdgcn_wave_barrier();
       __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 
+      // SELECT: a lane that does not blend keeps its sums by a select instead of adding a product with weight 0
+      // (0 * NaN and 0 * inf are NaN): the reference only lets a non-finite colour reach the pixels that blend
+      // it (cuda_rasterizer/forward.cu:381-407).  Same bits for finite inputs.
+      auto walk = [&](auto select_tag) {
+      constexpr bool SELECT = decltype(select_tag)::value;
       int kk = 0;
       uint32_t m = s_list[wave][row][0];
       for (;;) {
@@ -179,10 +218,16 @@ render_fwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
           // weight once, then one fused multiply-add per channel
           const float w = blend ? alpha * T : 0.f;
 #pragma unroll
-          for (int ch = 0; ch < GS_N_RGB; ch++) C[ch] = __builtin_fmaf(s_rgb[ch][j], w, C[ch]);
+          for (int ch = 0; ch < GS_N_RGB; ch++) {
+            const float sum = __builtin_fmaf(s_rgb[ch][j], w, C[ch]);
+            C[ch] = (!SELECT || blend) ? sum : C[ch];
+          }
           if (render_geo) {
 #pragma unroll
-            for (int ch = 0; ch < GS_N_MAP; ch++) Mp[ch] = __builtin_fmaf(s_map[ch][j], w, Mp[ch]);
+            for (int ch = 0; ch < GS_N_MAP; ch++) {
+              const float sum = __builtin_fmaf(s_map[ch][j], w, Mp[ch]);
+              Mp[ch] = (!SELECT || blend) ? sum : Mp[ch];
+            }
           }
           if (MAX_DEPTH) {
             const bool better = w > best_w;  // w is 0 for a lane that does not blend
@@ -206,6 +251,9 @@ render_fwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
           }
         }
       }
+      };
+      if (select_blend) walk(std::true_type{});
+      else walk(std::false_type{});
     }
     __syncthreads();
     if (tid < count) {

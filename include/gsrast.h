@@ -109,8 +109,12 @@ void gs_set_tile_sort_limits(int in_registers, int large_limit, int max_chunks);
  * the instance count (the call blocks on the stream there, as the reference
  * does at :653) -> key emission -> 64-bit radix sort on 32+bits(tiles) bits
  * -> tile ranges -> blend -> per-tile statistics.
- * out_color (3,H,W); out_all_map (5,H,W) and out_plane_depth (1,H,W) are
- * written only when render_geo != 0; out_observe (P) int32 is cleared by the call
+ * out_color (3,H,W) is written in full: pixels of tiles with compute_locally == 0 read 0, as in the reference,
+ * whose binding allocates the images zero-filled (rasterize_points.cu:303-307); so are out_all_map (5,H,W) and
+ * out_plane_depth (1,H,W) when render_geo != 0 (they are not touched otherwise: pass them zero-filled, as the
+ * reference leaves them) and out_max_weight_depth when given.  A Gaussian whose colour or geometry channels are
+ * not finite reaches exactly the pixels that blend it (CR/forward.cu:381-407).
+ * out_observe (P) int32 is cleared by the call
  * (the reference's binding allocates it zeroed, rasterize_points.cu:305) and then counted;
  * n_render / n_consider / n_contrib are (tiles) int32, fully written.
  * *num_rendered (host) receives the instance count R.

@@ -246,6 +246,42 @@ def test_max_weight_depth_matches_oracle_and_changes_nothing_else(orc, cfg, P, m
     assert float(got[0][px].max()) > 0
 
 
+@pytest.mark.parametrize("geo", [True, False])
+def test_pixels_of_tiles_not_computed_locally_read_zero(geo):
+    """The reference allocates its images zero-filled (rasterize_points.cu:303-307) and its kernel skips tiles that
+    are not computed locally, so their pixels read 0; a caller may sum a loss over the whole image.  Same here, in
+    all three images and in the additional depth image, however dirty the allocator's memory is."""
+    import gs_scenes
+    from diff_gaussian_rasterization import GaussianRasterizer
+    g, cams = gs_scenes.make_scene(0, P=20_000, n_views=1)
+    cam = cams[0]
+    W, H = cam.image_width, cam.image_height
+    gx, gy = (W + 15) // 16, (H + 15) // 16
+    cl = torch.ones(gy, gx, dtype=torch.bool, device=DEV)
+    cl[::2, ::2] = False
+    cl[-1, :] = False
+    # leave NaNs behind in the caching allocator's free blocks
+    junk = [torch.full((s, H, W), float("nan"), device=DEV) for s in (3, 5, 1, 1)]
+    del junk
+    rast = GaussianRasterizer(_settings(cam, render_geo=geo, bg=(0.3, 0.6, 0.9)))
+    d = {k: g[k].to(DEV) for k in ("means3D", "scales", "rotations", "opacities", "shs")}
+    args = _cuda_args()
+    args["max_weight_depth"] = True
+    means2D, rgb, co, radii, depths = rast.preprocess_gaussians(d["means3D"], d["scales"], d["rotations"], d["shs"],
+                                                                d["opacities"], args)
+    am = gs_scenes.build_all_map(d["means3D"], d["scales"], d["rotations"], cam)
+    color, n_render, n_consider, n_contrib, obs, oam, opd = rast.render_gaussians(
+        means2D, torch.zeros_like(d["means3D"]), co, rgb, am, depths, radii, cl, cl, args)
+    mwd = args["stats_collector"]["max_weight_depth"]
+    px = cl.repeat_interleave(16, 0).repeat_interleave(16, 1)[:H, :W]
+    for name, img in (("color", color), ("all_map", oam), ("plane_depth", opd), ("max_weight_depth", mwd)):
+        assert bool(torch.isfinite(img).all()), name
+        assert float(img[:, ~px].abs().max()) == 0.0, name
+    assert float(color[:, px].min()) > 0.0  # the local pixels carry at least the background
+    assert int(n_consider.view(gy, gx)[~cl].abs().sum()) == 0 and int(n_contrib.view(gy, gx)[~cl].abs().sum()) == 0
+    assert float((color * px).sum()) == float(color.sum())
+
+
 def test_debug_mode_gives_the_same_results_by_every_route():
     """debug=True makes every stage wait for its kernels and report their errors (and check the radix sort's
     status word); results are those of the normal mode bit for bit, whichever way the per-tile lists are built."""

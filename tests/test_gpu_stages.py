@@ -125,23 +125,26 @@ def test_render_forward(H, orc, cfg, P, mask, geo, bgv):
                        H.dev(pre["means2D"]), H.dev(pre["rgb"]), H.dev(am), H.dev(pre["conic_opacity"]), H.dev(cl),
                        H.dev(bg), render_geo=geo)
     gx, gy = H.grid(W, Hh)
-    # pixels of tiles that are not computed locally are left untouched by both sides
+    # the per-pixel state of tiles that are not computed locally is left untouched by both sides
     pix_local = np.repeat(np.repeat(cl.reshape(gy, gx), 16, 0), 16, 1)[:Hh, :W]
     for k in ("n_contrib", "n_contrib2loss"):
         assert np.array_equal(H.np_u32(got[k])[pix_local], ref[k][pix_local]), k
     assert np.array_equal(got["out_observe"].cpu().numpy(), ref["out_observe"])
     for k in ("n_render", "n_consider", "n_contrib_tile"):
         assert np.array_equal(got[k].cpu().numpy(), ref[k]), k
-    assert np.abs(got["final_T"].cpu().numpy() - ref["final_T"])[pix_local].max() <= IMG_TOL
+    # the transmittance decides the contributor counts: the same bits
+    assert np.array_equal(got["final_T"].cpu().numpy()[pix_local], ref["final_T"][pix_local])
+    # The images are the oracle's bit for bit (same operation order, explicit FMAs, the same exp); the plane
+    # depth is a quotient formed in double precision on both sides, compared element by element.
     keys = ("color", "out_all_map", "out_plane_depth") if geo else ("color",)
     for k in keys:
         a, r = got[k].cpu().numpy()[:, pix_local], ref[k][:, pix_local]
-        if k == "out_plane_depth":
-            # a ratio: compare where the denominator is not tiny
-            ok = np.isfinite(r) & (np.abs(r) < 1e4)
-            assert np.abs(a - r)[ok].max() <= IMG_TOL * np.maximum(1.0, np.abs(r[ok])).max(), k
-        else:
-            assert np.abs(a - r).max() <= IMG_TOL, f"{k}: {np.abs(a - r).max()}"
+        assert np.array_equal(np.isnan(a), np.isnan(r)), k
+        ok = ~np.isnan(r)
+        assert np.array_equal(a[ok], r[ok]), f"{k}: {np.abs(a[ok] - r[ok]).max()}"
+        # pixels of tiles that are not computed locally read zero, as the reference's zero-filled images do
+        # (rasterize_points.cu:303-307); the harness pre-fills every output with 55
+        assert float(np.abs(got[k].cpu().numpy()[:, ~pix_local]).max(initial=0.0)) == 0.0, k
     if not geo:
         assert float(got["out_all_map"].abs().max()) == 0.0 and float(got["out_plane_depth"].abs().max()) == 0.0
 
@@ -173,6 +176,10 @@ def test_render_backward(H, orc, cfg, P, mask, geo):
         a = got[k].cpu().numpy()
         assert np.isfinite(a).all(), k
         assert H.rel_l2(a, r) <= GRAD_TOL, f"{k}: rel L2 {H.rel_l2(a, r)}"
+        # ... and row by row, so that a wrong gradient of a Gaussian with a small one cannot hide behind the
+        # large ones: each element within 1e-3 of its own size plus 1e-5 of the tensor's largest
+        worst = np.abs(a - r) - (GRAD_TOL * np.abs(r) + 1e-5 * np.abs(r).max())
+        assert worst.max() <= 0.0, f"{k}: element {np.unravel_index(worst.argmax(), worst.shape)} off by {worst.max()}"
     a = got["dL_dmeans2D_abs"].cpu().numpy()
     assert (a[:, :2] + 1e-3 * np.abs(a[:, :2]) + 1e-6 >= np.abs(got["dL_dmeans2D"].cpu().numpy())).all()
     assert (a[:, 2] == 0).all()
@@ -343,3 +350,57 @@ def test_blend_with_arbitrary_splats(H, orc, seed, W, Hh, geo):
         g_ = gb[k].cpu().numpy()
         assert np.isfinite(g_).all(), k
         assert H.rel_l2(g_, r) <= GRAD_TOL, f"{k}: rel L2 {H.rel_l2(g_, r)}"
+
+
+@pytest.mark.parametrize("geo", [True, False])
+def test_non_finite_colours_reach_only_the_pixels_that_blend_them(H, orc, geo):
+    """A Gaussian whose colour or geometry channels are NaN or infinite (what a diverging training step hands the
+    rasterizer) poisons exactly the pixels that blend it and the gradients that depend on those pixels, as in the
+    reference (forward.cu:381-407, backward.cu:463-472) and the oracle; every other pixel and gradient keeps the
+    bits / the value it has without it."""
+    import gs_scenes
+    g, cam, pre, cl, b, am = _render_inputs(H, orc, 0, 30_000, "all")
+    W, Hh = cam.image_width, cam.image_height
+    P = 30_000
+    rgb, am = pre["rgb"].copy(), am.copy()
+    vis = np.flatnonzero(pre["radii"] > 0)
+    rng = np.random.default_rng(5)
+    pick = rng.choice(vis, 40, replace=False)
+    rgb[pick[:10], 0] = np.nan
+    rgb[pick[10:20], 2] = np.inf
+    am[pick[20:30], 1] = np.nan
+    am[pick[30:40], 4] = -np.inf
+    bg = np.array([0.1, 0.2, 0.3], np.float32)
+    ref = orc.render_fwd(b["ranges"], b["point_list"], pre["means2D"], rgb, am, pre["conic_opacity"], cl, bg, W, Hh,
+                         cam.tanfovx, cam.tanfovy, render_geo=geo)
+    got = H.render_fwd(P, W, Hh, cam.tanfovx, cam.tanfovy, H.as_u32(b["ranges"]), H.as_u32(b["point_list"]),
+                       H.dev(pre["means2D"]), H.dev(rgb), H.dev(am), H.dev(pre["conic_opacity"]), H.dev(cl),
+                       H.dev(bg), render_geo=geo)
+    for k in ("n_contrib", "n_contrib2loss"):
+        assert np.array_equal(H.np_u32(got[k]), ref[k]), k
+    assert np.array_equal(got["final_T"].cpu().numpy(), ref["final_T"])
+    for k in (("color", "out_all_map") if geo else ("color",)):
+        a, r = got[k].cpu().numpy(), ref[k]
+        assert np.array_equal(np.isnan(a), np.isnan(r)), k
+        assert np.array_equal(a[~np.isnan(r)], r[~np.isnan(r)]), k
+        assert np.isnan(r).any() and np.isnan(r).mean() < 0.2, k  # poisoned pixels exist and stay few
+    ug = gs_scenes.upstream_grads(cam)
+    gpix, gmap = ug["color"].numpy(), ug["all_map"].numpy()
+    gdep = np.zeros((1, Hh, W), np.float32)
+    amp = np.where(np.isfinite(ref["out_all_map"]), ref["out_all_map"], 0.0).astype(np.float32)
+    rb = orc.render_bwd(b["ranges"], b["point_list"], pre["means2D"], pre["conic_opacity"], rgb, am, amp,
+                        ref["final_T"], ref["n_contrib"], cl, bg, gpix, gmap, gdep, W, Hh, cam.tanfovx, cam.tanfovy,
+                        render_geo=geo)
+    gb = H.render_bwd(P, W, Hh, cam.tanfovx, cam.tanfovy, H.dev(bg), H.as_u32(b["ranges"]), H.as_u32(b["point_list"]),
+                      H.dev(pre["means2D"]), H.dev(pre["conic_opacity"]), H.dev(rgb), H.dev(am), H.dev(amp),
+                      H.dev(ref["final_T"]), H.as_u32(ref["n_contrib"]), H.dev(cl), H.dev(gpix), H.dev(gmap),
+                      H.dev(gdep), H.as_u32(b["emission_sorted"]), H.as_u32(b["point_offsets"]), render_geo=geo)
+    pairs = [("dL_dmeans2D", rb["dL_dmeans2D"][:, :2]), ("dL_dconic_opacity", rb["dL_dconic_opacity"]),
+             ("dL_dcolors", rb["dL_dcolors"])] + ([("dL_dall_map", rb["dL_dall_map"])] if geo else [])
+    for k, r in pairs:
+        a = gb[k].cpu().numpy()
+        assert np.array_equal(np.isfinite(a), np.isfinite(r)), (k, int((np.isfinite(a) != np.isfinite(r)).sum()))
+        ok = np.isfinite(r)
+        # (the colour and channel gradients are weight x upstream gradient and stay finite throughout)
+        assert ok.all() if k in ("dL_dcolors", "dL_dall_map") else ((~ok).any() and (~ok).mean() < 0.5), k
+        assert H.rel_l2(a[ok], r[ok]) <= GRAD_TOL, k
