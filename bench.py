@@ -19,6 +19,7 @@ import time
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 sys.path.insert(0, os.path.join(ROOT, "citygs-x_amd"))
+sys.path.insert(0, os.path.join(ROOT, "tests"))  # the seeded scene generator (gs_scenes) is shared with the tests
 
 HBM_PEAK_GBS = 8000.0
 

@@ -43,43 +43,70 @@ int check_launch(const char* what, hipStream_t stream, bool sync) {
 // cuda_rasterizer/timers.cu:11-79): when enabled, every stage of the composite
 // entry points is bracketed by an event pair on its stream; pairs are resolved
 // only when the caller collects them, so enabling it adds no synchronisation.
-// Process-wide and not thread safe: meant for benchmarks and profiling.
+// Process-wide but safe to use from several threads: a stage's pair is filed,
+// under the mutex, only once both events have been recorded.
 struct StageClock {
   struct Rec {
     const char* name;
     hipEvent_t a, b;
   };
-  bool enabled = false;
+  std::atomic<bool> enabled{false};
+  std::mutex mutex;
   std::vector<hipEvent_t> pool;
-  std::vector<Rec> pending;
+  std::vector<Rec> done;
   hipEvent_t take() {
-    if (!pool.empty()) {
-      hipEvent_t e = pool.back();
-      pool.pop_back();
-      return e;
+    {
+      std::lock_guard<std::mutex> lock(mutex);
+      if (!pool.empty()) {
+        hipEvent_t e = pool.back();
+        pool.pop_back();
+        return e;
+      }
     }
     hipEvent_t e = nullptr;
-    if (hipEventCreate(&e) != hipSuccess) return nullptr;
+    if (hipEventCreate(&e) != hipSuccess) {
+      (void)hipGetLastError();
+      return nullptr;
+    }
     return e;
   }
-  void begin(const char* name, hipStream_t s) {
-    if (!enabled) return;
-    Rec r{name, take(), take()};
-    if (!r.a || !r.b) return;
-    (void)hipEventRecord(r.a, s);
-    pending.push_back(r);
+  void give_back(hipEvent_t e) {
+    if (e == nullptr) return;
+    std::lock_guard<std::mutex> lock(mutex);
+    pool.push_back(e);
   }
-  void end(hipStream_t s) {
-    if (!enabled || pending.empty()) return;
-    (void)hipEventRecord(pending.back().b, s);
+  void file(const Rec& r) {
+    std::lock_guard<std::mutex> lock(mutex);
+    done.push_back(r);
   }
 };
 static StageClock g_clock;
 
 struct StageScope {
   hipStream_t s;
-  StageScope(const char* name, hipStream_t stream) : s(stream) { g_clock.begin(name, s); }
-  ~StageScope() { g_clock.end(s); }
+  StageClock::Rec rec{nullptr, nullptr, nullptr};
+  StageScope(const char* name, hipStream_t stream) : s(stream) {
+    if (!g_clock.enabled.load(std::memory_order_relaxed)) return;
+    rec.name = name;
+    rec.a = g_clock.take();
+    rec.b = g_clock.take();
+    if (!rec.a || !rec.b || hipEventRecord(rec.a, s) != hipSuccess) {
+      g_clock.give_back(rec.a);
+      g_clock.give_back(rec.b);
+      rec.a = rec.b = nullptr;
+    }
+  }
+  ~StageScope() {
+    if (!rec.a) return;
+    if (hipEventRecord(rec.b, s) == hipSuccess) {
+      g_clock.file(rec);
+    } else {
+      g_clock.give_back(rec.a);
+      g_clock.give_back(rec.b);
+    }
+  }
+  StageScope(const StageScope&) = delete;
+  StageScope& operator=(const StageScope&) = delete;
 };
 
 namespace {
@@ -323,22 +350,29 @@ std::atomic<uint32_t*> g_total_slots{nullptr};
 std::atomic<unsigned> g_total_next{0};
 std::mutex g_total_mutex;
 
-uint32_t* acquire_total_slot() {
+uint32_t* pinned_words() {
   uint32_t* base = g_total_slots.load(std::memory_order_acquire);
   if (base == nullptr) {
     std::lock_guard<std::mutex> lock(g_total_mutex);
     base = g_total_slots.load(std::memory_order_acquire);
     if (base == nullptr) {
       void* p = nullptr;
-      // 64-byte spacing keeps the words on separate lines
-      if (hipHostMalloc(&p, TOTAL_SLOTS * 64, hipHostMallocDefault) != hipSuccess) {
+      // 64-byte spacing keeps the words on separate lines; one more line holds the fault word (below)
+      if (hipHostMalloc(&p, (TOTAL_SLOTS + 1) * 64, hipHostMallocDefault) != hipSuccess) {
         (void)hipGetLastError();
         return nullptr;  // the caller falls back to a copy and a stream wait
       }
       base = (uint32_t*)p;
+      base[16 * TOTAL_SLOTS] = 0u;
       g_total_slots.store(base, std::memory_order_release);
     }
   }
+  return base;
+}
+
+uint32_t* acquire_total_slot() {
+  uint32_t* base = pinned_words();
+  if (base == nullptr) return nullptr;
   uint32_t* slot = base + 16 * (g_total_next.fetch_add(1, std::memory_order_relaxed) % TOTAL_SLOTS);
   slot[1] = 0u;  // second and third word of the slot: the longest tile list and the number of chunks that the
   slot[2] = 0u;  // longer lists are sorted in, both written before the total
@@ -375,22 +409,44 @@ int wait_for_total(uint32_t* slot, hipStream_t stream, uint32_t* out) {
 }  // namespace
 
 namespace {
-// whether the per-tile sort keeps the records in registers (or in LDS), the list length up to which one
-// workgroup sorts a list whole (0: every view takes the radix sort), and the number of chunks up to which the
-// longer lists of a view are sorted in chunks and merged
-std::atomic<int> g_tile_sort_registers{1};
-std::atomic<int> g_tile_sort_large{TILE_SORT_LARGE};
-std::atomic<int> g_tile_sort_chunks{TILE_SORT_MAX_CHUNKS};
+// A kernel that runs after a radix sort sets this host-visible word when the sort's bounded look-back wait ran
+// out (its output is then not sorted).  The word is sticky: the entry points look at it when they are called,
+// without waiting for anything, so the failure of a sort surfaces at the next call after its kernels have run
+// (and at once in debug mode or when a call times itself, both of which wait for the stream).
+uint32_t* fault_word() {
+  uint32_t* base = pinned_words();
+  return base ? base + 16 * TOTAL_SLOTS : nullptr;
+}
+
+int pending_fault(const char* who) {
+  uint32_t* w = g_total_slots.load(std::memory_order_acquire);
+  if (w == nullptr) return 0;
+  w += 16 * TOTAL_SLOTS;
+  if (__atomic_load_n(w, __ATOMIC_ACQUIRE) == 0u) return 0;
+  __atomic_store_n(w, 0u, __ATOMIC_RELEASE);
+  set_error("%s: an earlier radix sort on this process ran out of its bounded look-back wait; the per-tile lists "
+            "(or neighbour distances) computed from it, and everything derived from them, are not to be trusted",
+            who);
+  return 1;
+}
+
+struct TileSortLimits {
+  int in_registers, large, chunks;
+};
+// The defaults, or what the caller's options ask for: whether the per-tile sort keeps the records in registers
+// (or in LDS), the list length up to which one workgroup sorts a list whole (0: every view takes the radix
+// sort), and the number of chunks up to which the longer lists of a view are sorted in chunks and merged.
+TileSortLimits tile_sort_limits(const gs_render_options* o) {
+  TileSortLimits L = {1, TILE_SORT_LARGE, TILE_SORT_MAX_CHUNKS};
+  if (o == nullptr || o->struct_bytes < sizeof(gs_render_options)) return L;
+  if (o->tile_sort_in_registers >= 0) L.in_registers = o->tile_sort_in_registers != 0;
+  if (o->tile_sort_large_limit >= 0) L.large = o->tile_sort_large_limit < TILE_SORT_LARGE ? o->tile_sort_large_limit : TILE_SORT_LARGE;
+  if (o->tile_sort_max_chunks >= 0) L.chunks = o->tile_sort_max_chunks;
+  return L;
+}
 }  // namespace
 
-void gs_set_tile_sort_limits(int in_registers, int large_limit, int max_chunks) {
-  if (large_limit > TILE_SORT_LARGE) large_limit = TILE_SORT_LARGE;
-  if (large_limit < 0) large_limit = 0;
-  if (max_chunks < 0) max_chunks = 0;
-  g_tile_sort_registers.store(in_registers != 0 ? 1 : 0);
-  g_tile_sort_large.store(large_limit);
-  g_tile_sort_chunks.store(max_chunks);
-}
+int gs_pending_fault(void) { return pending_fault("gs_pending_fault"); }
 
 int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resize_fn binningBuffer,
                       void* binning_user, gs_resize_fn imageBuffer, void* image_user, int P, const float* background,
@@ -400,10 +456,12 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
                       const uint8_t* compute_locally, float* out_color, int* n_render, int* n_consider,
                       int* n_contrib, int* out_observe, float* out_all_map, float* out_plane_depth,
                       float* out_max_weight_depth, int render_geo, int debug, int* num_rendered, float* elapsed_ms,
-                      gs_stream_t stream_) {
+                      const gs_render_options* options, gs_stream_t stream_) {
   (void)viewmatrix;
   (void)cam_pos;
   hipStream_t stream = (hipStream_t)stream_;
+  if (pending_fault("gs_render_forward")) return 1;
+  const TileSortLimits limits = tile_sort_limits(options);
   GS_REQUIRE(P > 0 && width > 0 && height > 0, "gs_render_forward: P, width and height must be positive");
   GS_REQUIRE(geometryBuffer && binningBuffer && imageBuffer, "gs_render_forward: null resize callback");
   GS_REQUIRE(background && means2D && depths && radii && conic_opacity && rgb && compute_locally,
@@ -439,7 +497,7 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
   // sort.  Otherwise: emit (tile | depth) keys, radix-sort all of them, find the tile boundaries.
   uint32_t* total_slot = acquire_total_slot();
   void* bucket_table = ibase + IL.bucket_table;
-  const uint32_t sort_limit = (uint32_t)g_tile_sort_large.load();
+  const uint32_t sort_limit = (uint32_t)limits.large;
   const bool counted_by_tile = T <= bucket_max_tiles() && total_slot != nullptr && sort_limit > 0;
   bool bucketed = counted_by_tile;
   if (bucketed) {
@@ -507,7 +565,7 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
   // A list of more than sort_limit records is sorted in chunks of at most that many and merged.  That serves a
   // view with a few such lists; the merge looks every record up in every other chunk of its list, and a view
   // with many long lists is sorted as fast by the radix sort over all its keys, which then takes over.
-  if (bucketed && longest > sort_limit && chunks > (uint32_t)g_tile_sort_chunks.load()) bucketed = false;
+  if (bucketed && longest > sort_limit && chunks > (uint32_t)limits.chunks) bucketed = false;
   if (bucketed) {
     if (R > 0) {
       {
@@ -518,7 +576,7 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
       if (check_launch("bucket_scatter", stream, dbg)) return 1;
       {
         StageScope _t("tile_sort", stream);
-        launch_tile_sort(T, longest, sort_limit, chunks, (uint32_t)g_tile_sort_registers.load(), ranges, bucket_table,
+        launch_tile_sort(T, longest, sort_limit, chunks, (uint32_t)limits.in_registers, ranges, bucket_table,
                          keys_other, gauss_of_emission, keys, emission, point_list, stream);
       }
       if (check_launch("tile_sort", stream, dbg)) return 1;
@@ -556,7 +614,9 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
       StageScope _t("identify_tile_ranges", stream);
       // ... and gathers the Gaussian ids of the sorted instances on the way (point_list).  The ranges were
       // cleared by the counting kernel of this path, or hold the other path's table and are cleared here.
-      launch_tile_ranges(R, keys, T, ranges, stream, !counted_by_tile, emission, gauss_of_emission, point_list);
+      // It also looks at the sort's error word and raises the sticky fault word if the sort gave up.
+      launch_tile_ranges(R, keys, T, ranges, stream, !counted_by_tile, emission, gauss_of_emission, point_list,
+                         R > 0 ? sort_error_word(sort_temp) : nullptr, fault_word());
     }
     if (check_launch("identify_tile_ranges", stream, dbg)) return 1;
   }
@@ -578,6 +638,8 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
   }
   if (check_launch("render_forward", stream, dbg)) return 1;
   if (timer.end(stream, elapsed_ms)) return 1;
+  // (debug mode and the timer have waited for the stream: a sort that gave up in this call is known by now)
+  if ((dbg || elapsed_ms != nullptr) && pending_fault("gs_render_forward")) return 1;
   return 0;
 }
 
@@ -590,6 +652,7 @@ int gs_render_backward(int P, int R, const float* background, int width, int hei
                        const float* all_map_pixels, int render_geo, int debug, float* instance_grads,
                        size_t instance_grads_bytes, float* elapsed_ms, gs_stream_t stream_) {
   hipStream_t stream = (hipStream_t)stream_;
+  if (pending_fault("gs_render_backward")) return 1;
   GS_REQUIRE(P > 0 && R >= 0 && width > 0 && height > 0, "gs_render_backward: bad sizes");
   GS_REQUIRE(geom_buffer && binning_buffer && img_buffer && compute_locally && background,
              "gs_render_backward: null buffer");
@@ -933,12 +996,14 @@ int gs_all_map_backward(int P, const float* means3D, const float* scales, const 
 int gs_knn_dist2(int P, const float* points, float* mean_dists, void* workspace, size_t workspace_bytes,
                  gs_stream_t stream) {
   GS_REQUIRE(P >= 0, "gs_knn_dist2: negative P");
+  if (pending_fault("gs_knn_dist2")) return 1;
   if (P == 0) return 0;
   GS_REQUIRE(points && mean_dists && workspace, "gs_knn_dist2: null pointer");
   GS_REQUIRE(workspace_bytes >= gs_knn_workspace_bytes(P), "gs_knn_dist2: workspace too small");
   {
     StageScope _t("knn_dist2", (hipStream_t)stream);
-    if (launch_knn_dist2(P, points, mean_dists, align_ptr((char*)workspace, 256), (hipStream_t)stream)) return 1;
+    if (launch_knn_dist2(P, points, mean_dists, align_ptr((char*)workspace, 256), fault_word(), (hipStream_t)stream))
+      return 1;
   }
   return check_launch("knn_dist2", (hipStream_t)stream, false);
 }
@@ -1021,6 +1086,17 @@ int gs_sort_status(const void* workspace, gs_stream_t stream_) {
     return 1;
   }
   return 0;
+}
+
+size_t gs_sort_workspace_error_offset(void) { return sort_error_word_offset(); }
+
+int gs_sort_check_async(const void* workspace, gs_stream_t stream_) {
+  hipStream_t stream = (hipStream_t)stream_;
+  GS_REQUIRE(workspace, "gs_sort_check_async: null workspace");
+  uint32_t* fw = fault_word();
+  GS_REQUIRE(fw, "gs_sort_check_async: no pinned host memory for the fault word");
+  launch_sort_fault_report(sort_error_word(align_ptr((const char*)workspace, 256)), fw, stream);
+  return check_launch("sort_check_async", stream, false);
 }
 
 int gs_sort_pairs_u32(int64_t n, uint32_t* keys_in, uint32_t* keys_out, uint32_t* vals_in, uint32_t* vals_out,
@@ -1114,25 +1190,33 @@ int gs_selftest_reductions(const float* in, float* out_wave, float* out_rows, gs
 }
 
 int gs_stage_timing_enable(int enable) {
-  g_clock.enabled = enable != 0;
+  g_clock.enabled.store(enable != 0);
   return 0;
 }
 
 int gs_stage_timing_collect(char* report, size_t report_bytes) {
   GS_REQUIRE(report && report_bytes > 0, "gs_stage_timing_collect: null report buffer");
+  std::vector<StageClock::Rec> recs;
+  {
+    std::lock_guard<std::mutex> lock(g_clock.mutex);
+    recs.swap(g_clock.done);
+  }
   std::map<std::string, std::pair<double, long>> acc;
   std::vector<std::string> order;
-  for (auto& r : g_clock.pending) {
+  int failed = 0;
+  for (auto& r : recs) {
     float ms = 0.f;
-    GS_HIP_TRY(hipEventSynchronize(r.b));
-    GS_HIP_TRY(hipEventElapsedTime(&ms, r.a, r.b));
-    if (!acc.count(r.name)) order.push_back(r.name);
-    acc[r.name].first += ms;
-    acc[r.name].second += 1;
-    g_clock.pool.push_back(r.a);
-    g_clock.pool.push_back(r.b);
+    if (hipEventSynchronize(r.b) == hipSuccess && hipEventElapsedTime(&ms, r.a, r.b) == hipSuccess) {
+      if (!acc.count(r.name)) order.push_back(r.name);
+      acc[r.name].first += ms;
+      acc[r.name].second += 1;
+    } else {
+      (void)hipGetLastError();
+      failed++;
+    }
+    g_clock.give_back(r.a);
+    g_clock.give_back(r.b);
   }
-  g_clock.pending.clear();
   size_t used = 0;
   report[0] = 0;
   for (auto& name : order) {
@@ -1140,6 +1224,10 @@ int gs_stage_timing_collect(char* report, size_t report_bytes) {
                            acc[name].second);
     if (w < 0 || (size_t)w >= report_bytes - used) break;
     used += (size_t)w;
+  }
+  if (failed) {
+    set_error("gs_stage_timing_collect: %d event pairs could not be read", failed);
+    return 1;
   }
   return 0;
 }

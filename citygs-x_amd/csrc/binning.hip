@@ -200,9 +200,14 @@ __global__ void fill_u32_kernel(int64_t n, uint32_t v, uint32_t* __restrict__ p)
 __global__ void __launch_bounds__(GS_BLOCK_1D)
 tile_ranges_kernel(int64_t L, const uint64_t* __restrict__ keys, uint32_t* __restrict__ ranges,
                    const uint32_t* __restrict__ gather_index, const uint32_t* __restrict__ gather_table,
-                   uint32_t* __restrict__ gather_out) {
+                   uint32_t* __restrict__ gather_out, const uint32_t* __restrict__ sort_error,
+                   uint32_t* __restrict__ fault_word) {
   const int64_t i = (int64_t)blockIdx.x * GS_BLOCK_1D + threadIdx.x;
   if (i >= L) return;
+  // a sort that gave up waiting for an earlier tile's counts left its error word set: tell the host (sticky word
+  // in host-visible memory), which looks at it at its next call
+  if (i == 0 && sort_error != nullptr && fault_word != nullptr && *sort_error != 0u)
+    __hip_atomic_store(fault_word, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
   // optionally also: gather_out[i] = gather_table[gather_index[i]] (the sorted list of Gaussian ids)
   if (gather_out != nullptr) gather_out[i] = gather_table[gather_index[i]];
   const uint32_t cur = (uint32_t)(keys[i] >> 32);
@@ -347,12 +352,12 @@ int launch_gather_u32(int64_t n, const uint32_t* index, const uint32_t* table, u
 
 int launch_tile_ranges(int64_t L, const uint64_t* keys_sorted, int T, uint32_t* ranges, hipStream_t stream,
                        bool already_zero, const uint32_t* gather_index, const uint32_t* gather_table,
-                       uint32_t* gather_out) {
+                       uint32_t* gather_out, const uint32_t* sort_error, uint32_t* fault_word) {
   if (T > 0 && !already_zero)
     hipLaunchKernelGGL(fill_u32_kernel, dim3((2 * T + 255) / 256), dim3(256), 0, stream, (int64_t)2 * T, 0u, ranges);
   if (L > 0)
     hipLaunchKernelGGL(tile_ranges_kernel, dim3((unsigned)((L + GS_BLOCK_1D - 1) / GS_BLOCK_1D)), dim3(GS_BLOCK_1D), 0,
-                       stream, L, keys_sorted, ranges, gather_index, gather_table, gather_out);
+                       stream, L, keys_sorted, ranges, gather_index, gather_table, gather_out, sort_error, fault_word);
   return 0;
 }
 

@@ -141,15 +141,20 @@ int launch_all_map_bwd(int P, const float* means, const float* scales, const flo
                        const float* campos, const float* grad_out, float* dmeans, float* drots,
                        hipStream_t stream);
 // already_zero: the caller cleared `ranges` itself; gather_*: also write gather_out[i] = gather_table[gather_index[i]]
+// sort_error / fault_word: also raise the host-visible fault word if the sort's error word is set
 int launch_tile_ranges(int64_t L, const uint64_t* keys_sorted, int T, uint32_t* ranges, hipStream_t stream,
                        bool already_zero = false, const uint32_t* gather_index = nullptr,
-                       const uint32_t* gather_table = nullptr, uint32_t* gather_out = nullptr);
+                       const uint32_t* gather_table = nullptr, uint32_t* gather_out = nullptr,
+                       const uint32_t* sort_error = nullptr, uint32_t* fault_word = nullptr);
 
 // ---- radix sort (stable, LSD, 8-bit digits) ----
 size_t sort_temp_bytes(int64_t n);
 // device word of a sort's workspace that is nonzero after a sort in which a bounded wait of the look-back ran out
 // (the order of the output is then not to be trusted)
 const uint32_t* sort_error_word(const void* temp);
+size_t sort_error_word_offset();  // its byte offset in the workspace
+// one-thread kernel: stores 1 (system scope) to the host-visible fault_word if *error_word is nonzero
+int launch_sort_fault_report(const uint32_t* error_word, uint32_t* fault_word, hipStream_t stream);
 // Sorts on key bits [0, end_bit), ping-ponging between the (a) and (b) arrays
 // starting from (a).  With an odd number of 8-bit passes the sorted result
 // lands in (b), with an even number back in (a): sort_result_in_b() tells.
@@ -211,6 +216,8 @@ int launch_reduce_selftest(const float* in, float* out_wave, float* out_rows, hi
 
 // ---- k-nearest-neighbour mean squared distance ----
 size_t knn_temp_bytes(int P);
-int launch_knn_dist2(int P, const float* points, float* mean_dist2, void* temp, hipStream_t stream);
+// fault_word (host-visible, optional): raised if the Morton sort's bounded wait ran out
+int launch_knn_dist2(int P, const float* points, float* mean_dist2, void* temp, uint32_t* fault_word,
+                     hipStream_t stream);
 
 }  // namespace gs

@@ -275,7 +275,8 @@ __global__ void __launch_bounds__(GS_BLOCK_1D) box_mean_dist_kernel(int P, const
 
 size_t knn_temp_bytes(int P) { return knn_layout(P).total; }
 
-int launch_knn_dist2(int P, const float* points, float* mean_dist2, void* temp, hipStream_t stream) {
+int launch_knn_dist2(int P, const float* points, float* mean_dist2, void* temp, uint32_t* fault_word,
+                     hipStream_t stream) {
   if (P <= 0) return 0;
   const KnnLayout L = knn_layout(P);
   char* base = (char*)temp;
@@ -298,6 +299,7 @@ int launch_knn_dist2(int P, const float* points, float* mean_dist2, void* temp, 
   hipLaunchKernelGGL(morton_kernel, dim3(blocks), dim3(GS_BLOCK_1D), 0, stream, P, points, minmax, codes_a, idx_a);
   const int end_bit = 32;  // 4 passes (even): the sorted pairs come back in the (a) arrays
   if (launch_sort_pairs_u32(P, codes_a, codes_b, idx_a, idx_b, end_bit, sort_temp, stream)) return 1;
+  launch_sort_fault_report(sort_error_word(sort_temp), fault_word, stream);
   const uint32_t* idx_sorted = sort_result_in_b(end_bit) ? idx_b : idx_a;
   hipLaunchKernelGGL(gather_points_kernel, dim3(blocks), dim3(GS_BLOCK_1D), 0, stream, P, points, idx_sorted,
                      sorted_pts);

@@ -452,7 +452,23 @@ int sort_pairs_impl(int64_t n, K* keys_a, K* keys_b, uint32_t* vals_a, uint32_t*
 
 size_t sort_temp_bytes(int64_t n) { return sort_layout(n).total_bytes; }
 
-const uint32_t* sort_error_word(const void* temp) { return (const uint32_t*)temp + MAX_PASSES * RADIX + MAX_PASSES; }
+size_t sort_error_word_offset() { return (size_t)(MAX_PASSES * RADIX + MAX_PASSES) * sizeof(uint32_t); }
+const uint32_t* sort_error_word(const void* temp) {
+  return (const uint32_t*)((const char*)temp + sort_error_word_offset());
+}
+
+namespace {
+__global__ void sort_fault_report_kernel(const uint32_t* __restrict__ error_word, uint32_t* __restrict__ fault_word) {
+  if (*error_word != 0u) __hip_atomic_store(fault_word, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+}  // namespace
+
+// Raises the host-visible fault word if the sort that last used the workspace gave up waiting.
+int launch_sort_fault_report(const uint32_t* error_word, uint32_t* fault_word, hipStream_t stream) {
+  if (error_word == nullptr || fault_word == nullptr) return 0;
+  hipLaunchKernelGGL(sort_fault_report_kernel, dim3(1), dim3(1), 0, stream, error_word, fault_word);
+  return 0;
+}
 
 int launch_sort_pairs_u64(int64_t n, uint64_t* keys_a, uint64_t* keys_b, uint32_t* vals_a, uint32_t* vals_b,
                           int end_bit, void* temp, hipStream_t stream) {

@@ -168,9 +168,10 @@ class _GrowBuffer:
 
 def render_gaussians(background, image_height, image_width, means2D, depths, radii, conic_opacity, rgb,
                      compute_locally, viewmatrix, campos, tan_fovx, tan_fovy, all_map, render_geo, debug, args):
-    """rasterize_points.cu:276-364.  One addition: with args["max_weight_depth"] set, the per-pixel depth of the
+    """rasterize_points.cu:276-364.  Two additions: with args["max_weight_depth"] set, the per-pixel depth of the
     Gaussian that blends with the largest weight (1, H, W) is left in args["stats_collector"]["max_weight_depth"];
-    the returned tuple is the reference's either way."""
+    args["tile_sort_limits"] = (in_registers, large_limit, max_chunks) chooses, for this call, the way the per-tile
+    lists are built (all ways give the same lists).  The returned tuple is the reference's either way."""
     means2D = _f32c(means2D, "means2D")
     dev = means2D.device
     P = means2D.shape[0]
@@ -202,6 +203,9 @@ def render_gaussians(background, image_height, image_width, means2D, depths, rad
         raise RuntimeError(f"compute_locally must be a bool tensor with {tiles} elements")
     am = _f32c(all_map, "all_map") if geo else None
     want_mwd = isinstance(args, dict) and bool(args.get("max_weight_depth"))
+    # (in_registers, large_limit, max_chunks) for this call only: how the per-tile lists are built (a test hook)
+    limits = args.get("tile_sort_limits") if isinstance(args, dict) else None
+    options = _n.RenderOptions(*limits) if limits is not None else None
     mwd = torch.empty(1, H, W, **f32) if want_mwd else None
     # fp32 arithmetic, as `H / (2.0f * tan_fovy)` at rasterize_points.cu:328-329
     focal_y = np.float32(H) / (np.float32(2.0) * np.float32(tan_fovy))
@@ -216,7 +220,8 @@ def render_gaussians(background, image_height, image_width, means2D, depths, rad
             _ptr(depths), _ptr(radii), _ptr(conic_opacity), _ptr(rgb), _ptr(cl), _ptr(out_color), _ptr(n_render),
             _ptr(n_consider), _ptr(n_contrib), _ptr(out_observe), _ptr(out_all_map), _ptr(out_plane_depth), _ptr(mwd),
             int(geo),
-            int(bool(debug)), C.byref(num_rendered), C.byref(elapsed) if timing else None, _stream(dev)),
+            int(bool(debug)), C.byref(num_rendered), C.byref(elapsed) if timing else None,
+            C.byref(options) if options is not None else None, _stream(dev)),
             "render_gaussians")
     _record_time(args, "forward_render_time", elapsed.value)
     if want_mwd:

@@ -32,7 +32,7 @@ _SIGNATURES = {
     "gs_preprocess_backward": (_i, [_vp] * 3 + [_i] * 5 + [_vp] * 4 + [_f] + [_vp] * 3 + [_f, _f] + [_vp, _i] +
                                [_vp] * 8 + [_i, _vp]),
     "gs_render_forward": (_i, [RESIZE_FN, _vp, RESIZE_FN, _vp, RESIZE_FN, _vp, _i, _vp, _i, _i, _f, _f, _f, _f] +
-                          [_vp] * 17 + [_i, _i, C.POINTER(_i), C.POINTER(_f), _vp]),
+                          [_vp] * 17 + [_i, _i, C.POINTER(_i), C.POINTER(_f), _vp, _vp]),
     "gs_render_backward_workspace_bytes": (_sz, [_i]),
     "gs_render_backward": (_i, [_i, _i, _vp, _i, _i, _f, _f] + [_vp] * 17 + [_i, _i, _vp, _sz, C.POINTER(_f), _vp]),
     "gs_ssim_l1_forward": (_i, [_i, _i, _i] + [_vp] * 9),
@@ -41,7 +41,6 @@ _SIGNATURES = {
     "gs_training_stats": (_i, [_i64, _i, _i64, _i64, _vp, _vp, _vp, _vp, _i] + [_vp] * 6 + [_sz, _vp]),
     "gs_max_radii_update": (_i, [_i64, _vp, _vp, _vp, _vp]),
     "gs_adam_step": (_i, [_i] + [_vp] * 7 + [C.c_double, C.c_double, C.c_double, _f, _vp]),
-    "gs_set_tile_sort_limits": (None, [_i, _i, _i]),
     "gs_neural_supported": (_i, [_i]),
     "gs_neural_workspace_bytes": (_sz, [_i64, _i]),
     "gs_neural_opacity_forward": (_i, [_i64, _i] + [_vp] * 6 + [_i] + [_vp] * 5 + [_sz, _vp, _vp]),
@@ -60,6 +59,9 @@ _SIGNATURES = {
     "gs_duplicate_with_keys": (_i, [_i, _i, _i] + [_vp] * 8),
     "gs_sort_workspace_bytes": (_sz, [_i64]),
     "gs_sort_status": (_i, [_vp, _vp]),
+    "gs_sort_workspace_error_offset": (_sz, []),
+    "gs_sort_check_async": (_i, [_vp, _vp]),
+    "gs_pending_fault": (_i, []),
     "gs_sort_pairs_u64": (_i, [_i64, _vp, _vp, _vp, _vp, _i, _vp, _sz, _vp]),
     "gs_sort_pairs_u32": (_i, [_i64, _vp, _vp, _vp, _vp, _i, _vp, _sz, _vp]),
     "gs_identify_tile_ranges": (_i, [_i64, _vp, _i, _vp, _vp]),
@@ -79,6 +81,16 @@ for _name, (_res, _args) in _SIGNATURES.items():
     _fn.argtypes = _args
 
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)
+
+
+class RenderOptions(C.Structure):
+    """gs_render_options of include/gsrast.h; a negative field keeps the library's default."""
+    _fields_ = [("struct_bytes", C.c_uint32), ("tile_sort_in_registers", C.c_int32),
+                ("tile_sort_large_limit", C.c_int32), ("tile_sort_max_chunks", C.c_int32)]
+
+    def __init__(self, tile_sort_in_registers=-1, tile_sort_large_limit=-1, tile_sort_max_chunks=-1):
+        super().__init__(C.sizeof(RenderOptions), int(tile_sort_in_registers), int(tile_sort_large_limit),
+                         int(tile_sort_max_chunks))
 
 
 def stage_timing(enable):

@@ -92,17 +92,24 @@ int gs_preprocess_backward(const int* radii, const float* cov3D, const uint8_t* 
                            float* dL_dcov3D, float* dL_dscale, float* dL_drot, float* dL_dsh, float* dL_dopacity,
                            int debug, gs_stream_t stream);
 
-/* No counterpart in the reference: a test hook.  gs_render_forward builds the per-tile lists either by
- * bucketing the instances by tile and sorting each tile's list on its own (one workgroup per list of up to 8192
- * records; longer lists as chunks of at most 8192 that are merged afterwards, up to 32 chunks per view), or, when
- * the view has more long lists than that (or the tile grid more than 30000 tiles), by the reference's own route:
- * (tile | depth) keys (rasterizer_impl.cu:74-117), one radix sort over all of them (:675-684), identifyTileRanges
- * (:122-144).  All give the same lists bit for bit.  in_registers = 0 makes the per-tile sort keep its records in
- * LDS instead of registers (default 1); large_limit lowers the list length that one workgroup sorts whole
- * (default 8192; 0 = always the radix route) and max_chunks changes the number of chunks the longer lists of a
- * view may be cut into (default 32; 0 = a longer list sends the view to the radix route), so that small scenes
- * can exercise every route. */
-void gs_set_tile_sort_limits(int in_registers, int large_limit, int max_chunks);
+/* No counterpart in the reference: per-call options of gs_render_forward (NULL = all defaults).  A field below
+ * zero keeps its default; struct_bytes is sizeof(gs_render_options) as the caller compiled it.
+ * gs_render_forward builds the per-tile lists either by bucketing the instances by tile and sorting each tile's
+ * list on its own (one workgroup per list of up to 8192 records; longer lists as chunks of at most 8192 that are
+ * merged afterwards, up to 32 chunks per view), or, when the view has more long lists than that (or the tile grid
+ * more than 30000 tiles), by the reference's own route: (tile | depth) keys (rasterizer_impl.cu:74-117), one radix
+ * sort over all of them (:675-684), identifyTileRanges (:122-144).  All give the same lists bit for bit.
+ * tile_sort_in_registers = 0 makes the per-tile sort keep its records in LDS instead of registers (default 1);
+ * tile_sort_large_limit lowers the list length that one workgroup sorts whole (default and maximum 8192; 0 = always
+ * the radix route) and tile_sort_max_chunks changes the number of chunks the longer lists of a view may be cut into
+ * (default 32; 0 = a longer list sends the view to the radix route), so that small scenes can exercise every
+ * route.  The library keeps no such setting between calls. */
+typedef struct gs_render_options {
+  uint32_t struct_bytes;
+  int32_t tile_sort_in_registers;
+  int32_t tile_sort_large_limit;
+  int32_t tile_sort_max_chunks;
+} gs_render_options;
 
 /* Replaces Rasterizer::renderForward (CR/rasterizer.h:130-160,
  * CR/rasterizer_impl.cu:586-846): tile count -> prefix sum -> host read-back of
@@ -132,7 +139,7 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
                       const float* rgb, const uint8_t* compute_locally, float* out_color, int* n_render,
                       int* n_consider, int* n_contrib, int* out_observe, float* out_all_map,
                       float* out_plane_depth, float* out_max_weight_depth, int render_geo, int debug,
-                      int* num_rendered, float* elapsed_ms, gs_stream_t stream);
+                      int* num_rendered, float* elapsed_ms, const gs_render_options* options, gs_stream_t stream);
 
 /* Replaces Rasterizer::renderBackward (CR/rasterizer.h:162-187,
  * CR/rasterizer_impl.cu:850-932) plus the repacking of
@@ -321,10 +328,22 @@ int gs_duplicate_with_keys(int P, int width, int height, const float* means2D, c
  * sorted pairs land in keys_out / vals_out. */
 size_t gs_sort_workspace_bytes(int64_t n);
 /* No counterpart in the reference.  A pass of the sort waits, with a bounded number of polls, for the digit counts
- * of earlier tiles; if a wait ever ran out the sort sets a word in its workspace instead of hanging.
- * gs_sort_status waits for the stream and returns 1 (with an error message) if the last sort that used this
- * workspace set it, else 0.  gs_render_forward checks the word itself when debug != 0. */
+ * of earlier tiles; if a wait ever ran out the sort sets a word in its workspace (at byte
+ * gs_sort_workspace_error_offset() of the 256-byte aligned workspace) instead of hanging, and its output is not
+ * sorted.  Three ways to learn of it:
+ *   gs_sort_status waits for the stream and returns 1 (with an error message) if the last sort that used this
+ *   workspace set the word, else 0;
+ *   gs_sort_check_async enqueues a one-thread kernel that raises a process-wide sticky fault word in pinned host
+ *   memory if the word is set, and waits for nothing;
+ *   gs_pending_fault returns 1 (with a message) if the fault word is raised, and lowers it.
+ * gs_render_forward (radix route) and gs_knn_dist2 enqueue that check themselves after their sorts, and
+ * gs_render_forward, gs_render_backward and gs_knn_dist2 fail on entry while the fault word is raised (lowering
+ * it): a sort that gave up is therefore reported by the next of these calls made after its kernels have run, and
+ * by the same call when debug != 0 or elapsed_ms is given (both wait for the stream). */
+size_t gs_sort_workspace_error_offset(void);
 int gs_sort_status(const void* workspace, gs_stream_t stream);
+int gs_sort_check_async(const void* workspace, gs_stream_t stream);
+int gs_pending_fault(void);
 int gs_sort_pairs_u64(int64_t n, uint64_t* keys_in, uint64_t* keys_out, uint32_t* vals_in, uint32_t* vals_out,
                       int end_bit, void* workspace, size_t workspace_bytes, gs_stream_t stream);
 int gs_sort_pairs_u32(int64_t n, uint32_t* keys_in, uint32_t* keys_out, uint32_t* vals_in, uint32_t* vals_out,
@@ -374,7 +393,10 @@ int gs_selftest_reductions(const float* in, float* out_wave, float* out_rows, gs
  * is bracketed by an event pair on its stream.  Nothing is synchronised until
  * gs_stage_timing_collect, which waits for the recorded events and writes one
  * line per stage, "name total_ms launches", into report (host buffer), then
- * clears the records.  Process wide, not thread safe. */
+ * clears the records.  Process wide; safe to use while other threads are inside entry points (a stage's pair
+ * is filed under a lock once both events are recorded).  Apart from this switch, the pinned words that carry
+ * instance counts to the host and the sticky fault word of the radix sort, the library holds no state between
+ * calls. */
 int gs_stage_timing_enable(int enable);
 int gs_stage_timing_collect(char* report, size_t report_bytes);
 

@@ -1,4 +1,5 @@
-"""Seeded synthetic scenes and cameras for the rasterizer benchmark and tests.
+"""Seeded synthetic scenes and cameras for the rasterizer tests, smoke check and benchmark (not part of the product
+package).
 
 Cameras are built the way CityGS-X builds them (row-vector convention):
 world_view_transform = W2C^T, full_proj = world_view_transform @ P^T

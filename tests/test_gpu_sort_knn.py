@@ -94,3 +94,41 @@ def test_cross_lane_reductions(H):
     H.gn.check(H.lib.gs_selftest_reductions(H.ptr(tin), H.ptr(ow), H.ptr(orow), H.stream()), "selftest")
     assert np.array_equal(ow.cpu().numpy(), x.sum(0))
     assert np.array_equal(orow.cpu().numpy(), x.reshape(4, 16, 16).sum(1))
+
+
+def test_a_sort_that_gave_up_fails_the_next_call(H):
+    """The radix sort's bounded wait is never made to run out on the GPU; instead the error word it would leave in
+    its workspace is written by hand, and the plumbing behind it is followed: gs_sort_status reports it, the check
+    kernel raises the sticky fault word without any wait, gs_pending_fault / the next composite call fail once and
+    lower it, and the call after that works again."""
+    from simple_knn._C import distCUDA2
+    n = 10_000
+    rng = np.random.default_rng(3)
+    keys = rng.integers(0, 1 << 30, n, dtype=np.uint32)
+    kin, vin = H.as_u32(keys), H.as_u32(np.arange(n, dtype=np.uint32))
+    kout, vout = torch.empty_like(kin), torch.empty_like(vin)
+    nb = H.lib.gs_sort_workspace_bytes(n)
+    ws = torch.empty(nb, dtype=torch.uint8, device=H.DEV)
+    H.gn.check(H.lib.gs_sort_pairs_u32(n, H.ptr(kin), H.ptr(kout), H.ptr(vin), H.ptr(vout), 32, H.ptr(ws), nb,
+                                       H.stream()), "gs_sort_pairs_u32")
+    assert H.lib.gs_sort_status(H.ptr(ws), H.stream()) == 0
+    H.gn.check(H.lib.gs_sort_check_async(H.ptr(ws), H.stream()), "gs_sort_check_async")
+    torch.cuda.synchronize()
+    assert H.lib.gs_pending_fault() == 0
+    # what a sort that gave up leaves behind
+    base = (ws.data_ptr() + 255) // 256 * 256 - ws.data_ptr()
+    off = base + H.lib.gs_sort_workspace_error_offset()
+    ws[off:off + 4].view(torch.int32).fill_(1)
+    assert H.lib.gs_sort_status(H.ptr(ws), H.stream()) == 1 and "not sorted" in H.gn.last_error()
+    H.gn.check(H.lib.gs_sort_check_async(H.ptr(ws), H.stream()), "gs_sort_check_async")
+    torch.cuda.synchronize()
+    pts = torch.rand(1000, 3, device=H.DEV)
+    with pytest.raises(RuntimeError, match="radix sort"):
+        distCUDA2(pts)
+    assert H.lib.gs_pending_fault() == 0  # lowered by the call that reported it
+    assert distCUDA2(pts).shape == (1000,)
+    # raised again: gs_pending_fault itself reports and lowers it
+    H.gn.check(H.lib.gs_sort_check_async(H.ptr(ws), H.stream()), "gs_sort_check_async")
+    torch.cuda.synchronize()
+    assert H.lib.gs_pending_fault() == 1 and "radix sort" in H.gn.last_error()
+    assert H.lib.gs_pending_fault() == 0

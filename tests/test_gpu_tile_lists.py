@@ -19,13 +19,6 @@ def H():
     return gpu_harness
 
 
-@pytest.fixture(autouse=True)
-def _restore_limits():
-    import gsrast_native as gn
-    yield
-    gn.lib.gs_set_tile_sort_limits(1, 8192, 32)
-
-
 def _mask(kind, gx, gy):
     cl = torch.ones(gy, gx, dtype=torch.bool)
     if kind == "rows":
@@ -68,7 +61,7 @@ def test_lists_match_oracle_by_every_route(orc, H, cfg, P, mask):
     args = {"stats_collector": {}}
     grads = []
     for small, large, chunks in ROUTES:
-        gn.lib.gs_set_tile_sort_limits(small, large, chunks)
+        args["tile_sort_limits"] = (small, large, chunks)
         out = _C.render_gaussians(torch.zeros(3, device=DEV), Hh, W, o["means2D"], o["depths"], o["radii"],
                                   o["conic_opacity"], o["rgb"], cl.to(DEV), vm, cp, cam.tanfovx, cam.tanfovy, am,
                                   True, False, args)
@@ -127,10 +120,9 @@ def test_equal_depths_keep_emission_order(orc, H):
     vm, cp = cam.world_view_transform.to(DEV), cam.camera_center.to(DEV)
     am = gs_scenes.build_all_map(gd["means3D"], gd["scales"], gd["rotations"], cam)
     for small, large, chunks in ROUTES:
-        gn.lib.gs_set_tile_sort_limits(small, large, chunks)
         out = _C.render_gaussians(torch.zeros(3, device=DEV), Hh, W, o["means2D"], o["depths"], o["radii"],
                                   o["conic_opacity"], o["rgb"], cl.to(DEV), vm, cp, cam.tanfovx, cam.tanfovy, am,
-                                  True, False, {"stats_collector": {}})
+                                  True, False, {"stats_collector": {}, "tile_sort_limits": (small, large, chunks)})
         R, binB = out[0], out[9]
         off = [C.c_size_t() for _ in range(5)]
         gn.check(gn.lib.gs_binning_state_layout(R, W, Hh, *[C.byref(x) for x in off]), "layout")
@@ -163,15 +155,16 @@ def test_long_lists(orc, H, P, expect):
     lo, hi = {"waves4": (2048, 4096), "waves8": (4096, 8192), "chunks": (8192, 16384), "radix": (8192, 16384),
               "chunks3": (16384, 65536)}[expect]
     assert lo < longest <= hi, longest
+    limits = None
     if expect == "radix":
-        gn.lib.gs_set_tile_sort_limits(1, 8192, 0)
+        limits = (1, 8192, 0)
     elif expect.startswith("chunks"):  # nearly every tile of this view has a long list: lift the bound on their number
-        gn.lib.gs_set_tile_sort_limits(1, 8192, 1 << 30)
+        limits = (1, 8192, 1 << 30)
     vm, cp = cam.world_view_transform.to(DEV), cam.camera_center.to(DEV)
     am = gs_scenes.build_all_map(gd["means3D"], gd["scales"], gd["rotations"], cam)
     out = _C.render_gaussians(torch.zeros(3, device=DEV), Hh, W, o["means2D"], o["depths"], o["radii"],
                               o["conic_opacity"], o["rgb"], cl.to(DEV), vm, cp, cam.tanfovx, cam.tanfovy, am, True,
-                              False, {"stats_collector": {}})
+                              False, {"stats_collector": {}, "tile_sort_limits": limits})
     R, binB, imgB = out[0], out[9], out[10]
     assert R == want["point_list"].shape[0]
     off = [C.c_size_t() for _ in range(5)]
@@ -240,16 +233,15 @@ def test_more_instances_than_positions_is_an_error(H, limits):
     rgb = torch.zeros(P, 3, device=DEV)
     cl = torch.ones(gy, gx, dtype=torch.bool, device=DEV)
     eye = torch.eye(4, device=DEV)
-    gn.lib.gs_set_tile_sort_limits(*limits)
     with pytest.raises(RuntimeError, match="instances"):
         _C.render_gaussians(torch.zeros(3, device=DEV), Hh, W, means2D, depths, radii, co, rgb, cl, eye,
                             torch.zeros(3, device=DEV), 1.0, 0.75, torch.zeros(P, 5, device=DEV), False, False,
-                            {"stats_collector": {}})
+                            {"stats_collector": {}, "tile_sort_limits": limits})
     # a count just inside the limit is still served (here: none at all after the failed call)
     radii.zero_()
     out = _C.render_gaussians(torch.zeros(3, device=DEV), Hh, W, means2D, depths, radii, co, rgb, cl, eye,
                               torch.zeros(3, device=DEV), 1.0, 0.75, torch.zeros(P, 5, device=DEV), False, False,
-                              {"stats_collector": {}})
+                              {"stats_collector": {}, "tile_sort_limits": limits})
     assert out[0] == 0
 
 
@@ -284,10 +276,10 @@ def test_random_rectangles_by_every_route(orc, H, seed, W, Hh):
     rgb = torch.rand(P, 3, generator=gen).to(DEV)
     eye = torch.eye(4, device=DEV)
     for small, large, chunks in ROUTES:
-        gn.lib.gs_set_tile_sort_limits(small, large, chunks)
         out = _C.render_gaussians(torch.zeros(3, device=DEV), Hh, W, means2D.to(DEV), depths.to(DEV), radii.to(DEV),
                                   co, rgb, cl.to(DEV), eye, torch.zeros(3, device=DEV), 1.0, 1.0,
-                                  torch.zeros(P, 5, device=DEV), False, False, {"stats_collector": {}})
+                                  torch.zeros(P, 5, device=DEV), False, False,
+                                  {"stats_collector": {}, "tile_sort_limits": (small, large, chunks)})
         R, binB, imgB = out[0], out[9], out[10]
         assert R == R_want, (small, large, chunks)
         off = [C.c_size_t() for _ in range(5)]
