@@ -17,7 +17,9 @@ def H():
     return gpu_harness
 
 
-@pytest.mark.parametrize("n,end_bit", [(5_000_000, 44), (20_000_001, 45), (33_554_432, 64)])
+# (134 217 728 pairs on 45 bits: the "more than 100 M keys" of BASELINE config 3, whose own generator stays below)
+@pytest.mark.timeout(600)
+@pytest.mark.parametrize("n,end_bit", [(5_000_000, 44), (20_000_001, 45), (33_554_432, 64), (134_217_728, 45)])
 def test_sort_large_is_stable_permutation(H, n, end_bit):
     g = torch.Generator(device=DEV).manual_seed(n)
     tile_bits = min(end_bit - 32, 13)
