@@ -438,7 +438,7 @@ struct TileSortLimits {
 // sort), and the number of chunks up to which the longer lists of a view are sorted in chunks and merged.
 TileSortLimits tile_sort_limits(const gs_render_options* o) {
   TileSortLimits L = {1, TILE_SORT_LARGE, TILE_SORT_MAX_CHUNKS};
-  if (o == nullptr || o->struct_bytes < sizeof(gs_render_options)) return L;
+  if (o == nullptr || o->struct_bytes < 4 * sizeof(uint32_t)) return L;
   if (o->tile_sort_in_registers >= 0) L.in_registers = o->tile_sort_in_registers != 0;
   if (o->tile_sort_large_limit >= 0) L.large = o->tile_sort_large_limit < TILE_SORT_LARGE ? o->tile_sort_large_limit : TILE_SORT_LARGE;
   if (o->tile_sort_max_chunks >= 0) L.chunks = o->tile_sort_max_chunks;
@@ -456,7 +456,7 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
                       const uint8_t* compute_locally, float* out_color, int* n_render, int* n_consider,
                       int* n_contrib, int* out_observe, float* out_all_map, float* out_plane_depth,
                       float* out_max_weight_depth, int render_geo, int debug, int* num_rendered, float* elapsed_ms,
-                      const gs_render_options* options, gs_stream_t stream_) {
+                      const gs_render_options* options, gs_render_result* result, gs_stream_t stream_) {
   (void)viewmatrix;
   (void)cam_pos;
   hipStream_t stream = (hipStream_t)stream_;
@@ -493,19 +493,37 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
   uint32_t* ranges = (uint32_t*)(ibase + IL.ranges);
 
   // Two ways to the sorted per-tile lists.  The default buckets the instances by tile (counting sort) and sorts
-  // every tile's list in LDS; it needs the tile histogram to fit in LDS and every list to fit the per-tile
+  // every tile's list on its own; it needs the tile histogram to fit in LDS and every list to fit the per-tile
   // sort.  Otherwise: emit (tile | depth) keys, radix-sort all of them, find the tile boundaries.
   uint32_t* total_slot = acquire_total_slot();
   void* bucket_table = ibase + IL.bucket_table;
   const uint32_t sort_limit = (uint32_t)limits.large;
   const bool counted_by_tile = T <= bucket_max_tiles() && total_slot != nullptr && sort_limit > 0;
   bool bucketed = counted_by_tile;
+
+  // The instance count decides the size of the binning buffer, and the host learns it only after the counting
+  // kernels have run: a round trip during which the GPU would idle.  A caller that says how many instances and
+  // how long a list it expects (the previous view's figures with a margin) gets the list kernels and the blend
+  // launched right behind the counting kernels, on buffers of the expected size; a device word tells them whether
+  // the view fits (they do nothing otherwise), and the host, which meanwhile has received the counts, either
+  // returns or builds the lists again the ordinary way.
+  int64_t cap_n = 0;
+  uint32_t cap_longest = 0;
+  if (counted_by_tile && !dbg && result != nullptr && result->struct_bytes >= sizeof(gs_render_result) &&
+      options != nullptr && options->struct_bytes >= sizeof(gs_render_options) && options->expected_instances > 0 &&
+      limits.in_registers != 0) {
+    cap_n = options->expected_instances < (int64_t)GS_MAX_INSTANCES ? options->expected_instances
+                                                                     : (int64_t)GS_MAX_INSTANCES;
+    cap_longest = options->expected_longest_list > 0 ? (uint32_t)options->expected_longest_list : sort_limit;
+    if (cap_longest > sort_limit) cap_longest = sort_limit;
+  }
+  const bool ahead = cap_n > 0;
+
   if (bucketed) {
     StageScope _t("tile_count", stream);
-    // the histogram's grand total is the instance count: the host gets it from here, and the prefix over the
-    // Gaussians below runs while the host is busy growing the binning buffer
+    // the histogram's grand total is the instance count: the host gets it from here
     if (launch_bucket_count(P, width, height, radii, means2D, compute_locally, tiles_touched, bucket_table, ranges,
-                            sort_limit, total_slot, out_observe, stream))
+                            sort_limit, total_slot, out_observe, (uint32_t)cap_n, cap_longest, stream))
       return 1;
   } else {
     StageScope _t("tile_count", stream);
@@ -515,18 +533,81 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
                       (int64_t)2 * T, out_observe);
   }
   if (check_launch("tile_count", stream, dbg)) return 1;
-  {
+  if (!bucketed) {
     StageScope _t("inclusive_sum", stream);
-    // (on the bucketed route the counting workgroups have summed their chunks already)
-    if (bucketed) launch_bucket_offsets(P, width, height, tiles_touched, bucket_table, point_offsets, stream);
-    else launch_inclusive_sum(P, tiles_touched, point_offsets, scan_temp, stream, total_slot);
+    launch_inclusive_sum(P, tiles_touched, point_offsets, scan_temp, stream, total_slot);
   }
   if (check_launch("inclusive_sum", stream, dbg)) return 1;
 
-  // The instance count decides the size of the binning buffer, so the host needs it here.  The scan writes
-  // it straight into pinned host memory and the host polls that word: no copy, and no sleeping wait whose
-  // wake-up would leave the GPU idle.  On the bucketed route the count and, in the word beside it, the longest
-  // tile list come from the kernel that builds the tile ranges.
+  EventTimer timer;
+  struct Arrays {
+    uint32_t *point_list, *gauss_of_emission, *emission, *emission_other;
+    uint64_t *keys, *keys_other;
+    void* sort_temp;
+  };
+  auto carve = [&](int64_t n, Arrays& A) -> int {
+    const BinningLayout BL = binning_layout(n);
+    char* bbase = binningBuffer(BL.total, binning_user);
+    GS_REQUIRE(bbase, "gs_render_forward: binning buffer callback returned NULL");
+    bbase = align_ptr(bbase, 256);
+    A.point_list = (uint32_t*)(bbase + BL.point_list);
+    A.keys = (uint64_t*)(bbase + BL.keys);
+    A.gauss_of_emission = (uint32_t*)(bbase + BL.point_list_unsorted);
+    A.keys_other = (uint64_t*)(bbase + BL.keys_unsorted);
+    A.emission = (uint32_t*)(bbase + BL.emission);
+    A.emission_other = (uint32_t*)(bbase + BL.emission_other);
+    A.sort_temp = bbase + BL.sort_temp;
+    return 0;
+  };
+  auto blend = [&](const Arrays& A, bool ahead_of_host) -> int {
+    RenderFwdArgs a;
+    a.P = P; a.W = width; a.H = height;
+    a.fx = focal_x; a.fy = focal_y; a.cx = cx; a.cy = cy;
+    a.ranges = ranges; a.point_list = A.point_list;
+    a.means2D = means2D; a.rgb = rgb; a.all_map = all_map; a.conic_opacity = conic_opacity;
+    a.compute_locally = compute_locally; a.bg = background; a.render_geo = render_geo;
+    a.final_T = accum_alpha; a.n_contrib_px = n_contrib_px; a.n_contrib2loss_px = n_contrib2loss_px;
+    a.out_color = out_color; a.out_observe = out_observe; a.out_all_map = out_all_map;
+    a.out_plane_depth = out_plane_depth;
+    a.depths = depths; a.out_max_weight_depth = out_max_weight_depth;
+    a.n_render = n_render; a.n_consider = n_consider; a.n_contrib_tile = n_contrib;
+    a.fits_word = ahead_of_host ? bucket_fits_word(bucket_table, T) : nullptr;
+    {
+      StageScope _t("render_fwd", stream);
+      launch_render_fwd(a, stream);
+    }
+    return check_launch("render_forward", stream, dbg);
+  };
+  auto lists_by_tile = [&](const Arrays& A, uint32_t longest_for_launch, uint32_t chunks_for_launch,
+                           bool ahead_of_host) -> int {
+    {
+      StageScope _t("bucket_scatter", stream);
+      // (also finishes the prefix sum over the Gaussians: point_offsets)
+      launch_bucket_scatter(P, width, height, means2D, depths, tiles_touched, point_offsets, radii, compute_locally,
+                            bucket_table, ranges, A.keys_other, A.gauss_of_emission, ahead_of_host, stream);
+    }
+    if (check_launch("bucket_scatter", stream, dbg)) return 1;
+    {
+      StageScope _t("tile_sort", stream);
+      launch_tile_sort(T, longest_for_launch, sort_limit, chunks_for_launch, (uint32_t)limits.in_registers, ranges,
+                       bucket_table, A.keys_other, A.gauss_of_emission, A.keys, A.emission, A.point_list,
+                       ahead_of_host, stream);
+    }
+    return check_launch("tile_sort", stream, dbg);
+  };
+
+  Arrays A;
+  if (ahead) {
+    if (carve(cap_n, A)) return 1;
+    if (timer.begin(elapsed_ms != nullptr, stream)) return 1;
+    if (lists_by_tile(A, cap_longest, 0u, true)) return 1;
+    if (blend(A, true)) return 1;
+  }
+
+  // The host needs the instance count: it sizes the binning buffer (unless that was done ahead), and the caller
+  // gets it back.  The counting kernels write it straight into pinned host memory and the host polls that word:
+  // no copy, and no sleeping wait.  On the bucketed route the longest tile list and the number of chunks that
+  // longer lists are cut into arrive in the words beside it.
   uint32_t R_u = 0, longest = 0, chunks = 0;
   if (total_slot != nullptr) {
     if (wait_for_total(total_slot, stream, &R_u)) return 1;
@@ -546,66 +627,60 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
   }
   const int64_t R = (int64_t)R_u;
   *num_rendered = (int)R;
+  if (result != nullptr && result->struct_bytes >= sizeof(gs_render_result)) {
+    result->longest_list = bucketed ? (int32_t)longest : 0;
+    result->binning_capacity = R;
+    result->launched_ahead = 0;
+  }
 
-  const BinningLayout BL = binning_layout(R);
-  char* bbase = binningBuffer(BL.total, binning_user);
-  GS_REQUIRE(bbase, "gs_render_forward: binning buffer callback returned NULL");
-  bbase = align_ptr(bbase, 256);
-  uint32_t* point_list = (uint32_t*)(bbase + BL.point_list);
-  uint64_t* keys = (uint64_t*)(bbase + BL.keys);
-  uint32_t* gauss_of_emission = (uint32_t*)(bbase + BL.point_list_unsorted);
-  uint64_t* keys_other = (uint64_t*)(bbase + BL.keys_unsorted);
-  uint32_t* emission = (uint32_t*)(bbase + BL.emission);
-  uint32_t* emission_other = (uint32_t*)(bbase + BL.emission_other);
-  void* sort_temp = bbase + BL.sort_temp;
+  // (the same test the ranges kernel made on the device)
+  if (ahead && R <= cap_n && longest <= cap_longest) {
+    result->binning_capacity = cap_n;
+    result->launched_ahead = 1;
+    if (timer.end(stream, elapsed_ms)) return 1;
+    return 0;
+  }
 
-  EventTimer timer;
-  if (timer.begin(elapsed_ms != nullptr, stream)) return 1;
+  // The ordinary way (also after kernels launched ahead found that the view does not fit and did nothing).
+  if (carve(R, A)) return 1;
+  if (!ahead && timer.begin(elapsed_ms != nullptr, stream)) return 1;
 
   // A list of more than sort_limit records is sorted in chunks of at most that many and merged.  That serves a
   // view with a few such lists; the merge looks every record up in every other chunk of its list, and a view
   // with many long lists is sorted as fast by the radix sort over all its keys, which then takes over.
   if (bucketed && longest > sort_limit && chunks > (uint32_t)limits.chunks) bucketed = false;
   if (bucketed) {
-    if (R > 0) {
-      {
-        StageScope _t("bucket_scatter", stream);
-        launch_bucket_scatter(P, width, height, means2D, depths, point_offsets, radii, compute_locally, bucket_table,
-                              ranges, keys_other, gauss_of_emission, stream);
-      }
-      if (check_launch("bucket_scatter", stream, dbg)) return 1;
-      {
-        StageScope _t("tile_sort", stream);
-        launch_tile_sort(T, longest, sort_limit, chunks, (uint32_t)limits.in_registers, ranges, bucket_table,
-                         keys_other, gauss_of_emission, keys, emission, point_list, stream);
-      }
-      if (check_launch("tile_sort", stream, dbg)) return 1;
-    }
+    if (lists_by_tile(A, longest, chunks, false)) return 1;
   } else {
+    if (counted_by_tile) {
+      StageScope _t("inclusive_sum", stream);
+      launch_bucket_offsets(P, width, height, tiles_touched, bucket_table, point_offsets, stream);
+    }
     const int end_bit = sort_end_bit(width, height);
     // The sort carries each instance's index in emission order as its payload (the backward pass files
     // per-instance gradients under it); the Gaussian ids of the sorted list are gathered afterwards.
     // It ping-pongs, so start from the array pair that makes it finish in (keys, emission).
     const bool odd = sort_result_in_b(end_bit);
-    uint64_t* k_start = odd ? keys_other : keys;
-    uint32_t* e_start = odd ? emission_other : emission;
-    uint64_t* k_partner = odd ? keys : keys_other;
-    uint32_t* e_partner = odd ? emission : emission_other;
+    uint64_t* k_start = odd ? A.keys_other : A.keys;
+    uint32_t* e_start = odd ? A.emission_other : A.emission;
+    uint64_t* k_partner = odd ? A.keys : A.keys_other;
+    uint32_t* e_partner = odd ? A.emission : A.emission_other;
     if (R > 0) {
       {
         StageScope _t("duplicate_with_keys", stream);
         launch_duplicate_with_keys(P, width, height, means2D, depths, point_offsets, radii, compute_locally, k_start,
-                                   gauss_of_emission, e_start, stream);
+                                   A.gauss_of_emission, e_start, stream);
       }
       if (check_launch("duplicate_with_keys", stream, dbg)) return 1;
       {
         StageScope _t("sort_pairs", stream);
-        if (launch_sort_pairs_u64(R, k_start, k_partner, e_start, e_partner, end_bit, sort_temp, stream)) return 1;
+        if (launch_sort_pairs_u64(R, k_start, k_partner, e_start, e_partner, end_bit, A.sort_temp, stream)) return 1;
       }
       if (check_launch("sort_pairs", stream, dbg)) return 1;
       if (dbg) {  // (sort_temp is 256-byte aligned already)
         uint32_t word = 0;
-        GS_HIP_TRY(hipMemcpyAsync(&word, sort_error_word(sort_temp), sizeof(uint32_t), hipMemcpyDeviceToHost, stream));
+        GS_HIP_TRY(hipMemcpyAsync(&word, sort_error_word(A.sort_temp), sizeof(uint32_t), hipMemcpyDeviceToHost,
+                                  stream));
         GS_HIP_TRY(hipStreamSynchronize(stream));
         GS_REQUIRE(word == 0u, "gs_render_forward: the radix sort's bounded look-back wait ran out");
       }
@@ -615,28 +690,13 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
       // ... and gathers the Gaussian ids of the sorted instances on the way (point_list).  The ranges were
       // cleared by the counting kernel of this path, or hold the other path's table and are cleared here.
       // It also looks at the sort's error word and raises the sticky fault word if the sort gave up.
-      launch_tile_ranges(R, keys, T, ranges, stream, !counted_by_tile, emission, gauss_of_emission, point_list,
-                         R > 0 ? sort_error_word(sort_temp) : nullptr, fault_word());
+      launch_tile_ranges(R, A.keys, T, ranges, stream, !counted_by_tile, A.emission, A.gauss_of_emission,
+                         A.point_list, R > 0 ? sort_error_word(A.sort_temp) : nullptr, fault_word());
     }
     if (check_launch("identify_tile_ranges", stream, dbg)) return 1;
   }
 
-  RenderFwdArgs a;
-  a.P = P; a.W = width; a.H = height;
-  a.fx = focal_x; a.fy = focal_y; a.cx = cx; a.cy = cy;
-  a.ranges = ranges; a.point_list = point_list;
-  a.means2D = means2D; a.rgb = rgb; a.all_map = all_map; a.conic_opacity = conic_opacity;
-  a.compute_locally = compute_locally; a.bg = background; a.render_geo = render_geo;
-  a.final_T = accum_alpha; a.n_contrib_px = n_contrib_px; a.n_contrib2loss_px = n_contrib2loss_px;
-  a.out_color = out_color; a.out_observe = out_observe; a.out_all_map = out_all_map;
-  a.out_plane_depth = out_plane_depth;
-  a.depths = depths; a.out_max_weight_depth = out_max_weight_depth;
-  a.n_render = n_render; a.n_consider = n_consider; a.n_contrib_tile = n_contrib;
-  {
-    StageScope _t("render_fwd", stream);
-    launch_render_fwd(a, stream);
-  }
-  if (check_launch("render_forward", stream, dbg)) return 1;
+  if (blend(A, false)) return 1;
   if (timer.end(stream, elapsed_ms)) return 1;
   // (debug mode and the timer have waited for the stream: a sort that gave up in this call is known by now)
   if ((dbg || elapsed_ms != nullptr) && pending_fault("gs_render_forward")) return 1;
@@ -650,9 +710,11 @@ int gs_render_backward(int P, int R, const float* background, int width, int hei
                        float* dL_dconic_opacity, float* dL_dcolor, float* dL_dall_map, const float* means2D,
                        const float* conic_opacity, const float* rgb, const float* all_maps,
                        const float* all_map_pixels, int render_geo, int debug, float* instance_grads,
-                       size_t instance_grads_bytes, float* elapsed_ms, gs_stream_t stream_) {
+                       size_t instance_grads_bytes, float* elapsed_ms, int64_t binning_capacity,
+                       gs_stream_t stream_) {
   hipStream_t stream = (hipStream_t)stream_;
   if (pending_fault("gs_render_backward")) return 1;
+  GS_REQUIRE(binning_capacity <= 0 || binning_capacity >= R, "gs_render_backward: binning_capacity below R");
   GS_REQUIRE(P > 0 && R >= 0 && width > 0 && height > 0, "gs_render_backward: bad sizes");
   GS_REQUIRE(geom_buffer && binning_buffer && img_buffer && compute_locally && background,
              "gs_render_backward: null buffer");
@@ -663,7 +725,7 @@ int gs_render_backward(int P, int R, const float* background, int width, int hei
              "gs_render_backward: null pointer");
   GS_REQUIRE(!render_geo || (dL_dout_all_map && dL_dout_plane_depth && dL_dall_map && all_maps && all_map_pixels),
              "gs_render_backward: render_geo needs the geometry-map tensors");
-  const BinningLayout BL = binning_layout(R);
+  const BinningLayout BL = binning_layout(binning_capacity > 0 ? binning_capacity : (int64_t)R);
   const ImageLayout IL = image_layout(width, height);
   const GeometryLayout GL = geometry_layout(P);
   const char* gbase = align_ptr(geom_buffer, 256);

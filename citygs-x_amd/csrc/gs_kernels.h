@@ -81,18 +81,25 @@ size_t bucket_table_bytes(int T);
 // tiles_touched per Gaussian, the workgroup-by-tile table, ranges (2 words per tile), and in three host-visible
 // words the number of instances (word 0, written last), the longest list (word 1) and the number of chunks that
 // the lists of more than chunk_limit records are cut into (word 2)
+// cap_instances / cap_longest: what kernels launched ahead of the host's decision were sized for; the ranges kernel
+// leaves 1 in bucket_fits_word(table) if the view has at most that many instances and no longer list, else 0
 int launch_bucket_count(int P, int W, int H, const int* radii, const float* means2D, const uint8_t* compute_locally,
                         uint32_t* tiles_touched, void* table, uint32_t* ranges, uint32_t chunk_limit,
-                        uint32_t* host_words, int* zero_per_gaussian, hipStream_t stream);
+                        uint32_t* host_words, int* zero_per_gaussian, uint32_t cap_instances, uint32_t cap_longest,
+                        hipStream_t stream);
+const uint32_t* bucket_fits_word(const void* table, int T);
 int launch_bucket_offsets(int P, int W, int H, const uint32_t* tiles_touched, void* table, uint32_t* point_offsets,
                           hipStream_t stream);
-int launch_bucket_scatter(int P, int W, int H, const float* means2D, const float* depths, const uint32_t* offsets,
-                          const int* radii, const uint8_t* compute_locally, const void* table,
-                          const uint32_t* ranges, uint64_t* records, uint32_t* gauss_of_emission,
-                          hipStream_t stream);
+// also writes point_offsets (the inclusive prefix sum of tiles_touched).  ahead_of_host: the kernel checks
+// bucket_fits_word itself and does nothing if the view does not fit what it was launched for.
+int launch_bucket_scatter(int P, int W, int H, const float* means2D, const float* depths,
+                          const uint32_t* tiles_touched, uint32_t* point_offsets, const int* radii,
+                          const uint8_t* compute_locally, void* table, const uint32_t* ranges, uint64_t* records,
+                          uint32_t* gauss_of_emission, bool ahead_of_host, hipStream_t stream);
 int launch_tile_sort(int T, uint32_t longest, uint32_t limit, uint32_t chunks, uint32_t in_registers,
                      const uint32_t* ranges, const void* table, uint64_t* records, const uint32_t* gauss_of_emission,
-                     uint64_t* keys, uint32_t* emission, uint32_t* point_list, hipStream_t stream);
+                     uint64_t* keys, uint32_t* emission, uint32_t* point_list, bool ahead_of_host,
+                     hipStream_t stream);
 int launch_gather_u32(int64_t n, const uint32_t* index, const uint32_t* table, uint32_t* out, hipStream_t stream);
 int launch_ssim_l1_fwd(int C, int H, int W, const float* img1, const float* img2, const uint8_t* mask,
                        float* l1_map, float* ssim_map, float* d_mu, float* d_xx, float* d_xy, hipStream_t stream);
@@ -184,6 +191,9 @@ struct RenderFwdArgs {
   int *n_render, *n_consider, *n_contrib_tile;
   const float* depths = nullptr;            // only read when out_max_weight_depth is given
   float* out_max_weight_depth = nullptr;    // optional (H*W)
+  // optional device word: the kernel was launched before the host knew whether the per-tile lists would be
+  // built by the kernels queued ahead of it; it does nothing if the word is 0
+  const uint32_t* fits_word = nullptr;
 };
 int launch_render_fwd(const RenderFwdArgs& a, hipStream_t stream);
 

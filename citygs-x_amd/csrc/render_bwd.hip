@@ -143,9 +143,11 @@ render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
   for (int ch = 0; ch < GS_N_RGB; ch++) bg_dot += bg[ch] * gpix[ch];
 
   const float bg_term = T_final * bg_dot;
-  float last_alpha = 0.f;
+  // Blend of everything behind the Gaussian at hand, per channel.  The reference updates it at the start of a
+  // step from the previous step's alpha and colour (cuda_rasterizer/backward.cu:463-472); here the same
+  // operation, accum = fma(alpha, c, (1 - alpha) * accum), runs at the end of the step that owns that alpha and
+  // colour, which gives the same values and needs neither the previous colours nor the previous alpha.
   float accum_rec[GS_N_RGB] = {0.f, 0.f, 0.f}, accum_map[GS_N_MAP] = {0.f, 0.f, 0.f, 0.f, 0.f};
-  float last_color[GS_N_RGB] = {0.f, 0.f, 0.f}, last_map[GS_N_MAP] = {0.f, 0.f, 0.f, 0.f, 0.f};
 
   // Positions are 0-based indices into the tile's list; the walk starts at the tile's deepest contributor.
   // Slot j of batch i holds position start - (i*BATCH + j).
@@ -249,8 +251,8 @@ render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
           // Straight-line from here on: every lane evaluates its row's Gaussian, and a lane for which the
           // Gaussian does not count (behind the pixel's last contributor, outside the power window, alpha
           // below 1/255) takes part with alpha = 0, G = 0.  Such a step leaves T unchanged (T * 1/(1-0)),
-          // contributes zeros to every sum, and only rotates the recurrence state in a way the next real
-          // step undoes exactly (fma(0, c, 1 * accum) == accum), so results are those of skipping it.
+          // contributes zeros to every sum and leaves the recurrence state as it is
+          // (fma(0, c, 1 * accum) == accum), so results are those of skipping it.
           // Same tests as the forward pass, on the same bits.
           const float2 xy = s_xy[j];
           const float4 co = s_co[j];
@@ -279,30 +281,27 @@ render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
           const float rcp1ma = gs_rcp_normal(1.f - alpha);  // alpha <= 0.99: the bits of 1.f / (1.f - alpha)
           T = T * rcp1ma;
           const float w = alpha * T;
-          const float oml = 1.f - last_alpha;
+          const float oma = 1.f - alpha;
           float dL_dalpha = 0.0f;
 #pragma unroll
           for (int ch = 0; ch < GS_N_RGB; ch++) {
             const float c = (!SELECT || active) ? s_rgb[ch][j] : 0.f;
-            accum_rec[ch] = __builtin_fmaf(last_alpha, last_color[ch], oml * accum_rec[ch]);
-            last_color[ch] = c;
             dL_dalpha = __builtin_fmaf(c - accum_rec[ch], gpix[ch], dL_dalpha);
+            accum_rec[ch] = __builtin_fmaf(alpha, c, oma * accum_rec[ch]);  // (alpha = 0: unchanged)
             v[8 + ch] = w * gpix[ch];
           }
           if (render_geo) {
 #pragma unroll
             for (int ch = 0; ch < GS_N_MAP; ch++) {
               const float c = (!SELECT || active) ? s_map[ch][j] : 0.f;
-              accum_map[ch] = __builtin_fmaf(last_alpha, last_map[ch], oml * accum_map[ch]);
-              last_map[ch] = c;
               dL_dalpha = __builtin_fmaf(c - accum_map[ch], gmap[ch], dL_dalpha);
+              accum_map[ch] = __builtin_fmaf(alpha, c, oma * accum_map[ch]);
               v[11 + ch] = w * gmap[ch];
             }
           } else {
 #pragma unroll
             for (int ch = 0; ch < GS_N_MAP; ch++) v[11 + ch] = 0.f;
           }
-          last_alpha = alpha;
           dL_dalpha = __builtin_fmaf(dL_dalpha, T, -(bg_term * rcp1ma));
           dL_dalpha = active ? dL_dalpha : 0.f;
           const float dL_dG = co.w * dL_dalpha;

@@ -47,8 +47,10 @@ render_fwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
                   int* __restrict__ out_observe, float* __restrict__ out_all_map,
                   float* __restrict__ out_plane_depth, int* __restrict__ n_render, int* __restrict__ n_consider,
                   int* __restrict__ n_contrib_tile, const float* __restrict__ depths,
-                  float* __restrict__ out_max_weight_depth) {
+                  float* __restrict__ out_max_weight_depth, const uint32_t* __restrict__ fits_word) {
   constexpr bool render_geo = RENDER_GEO;
+  // launched ahead of the host's decision on how the per-tile lists are built: nothing to do if they were not
+  if (fits_word != nullptr && *fits_word == 0u) return;
   __shared__ float s_depth[MAX_DEPTH ? BATCH : 1];
   __shared__ int s_id[BATCH];
   __shared__ float2 s_xy[BATCH];
@@ -306,7 +308,7 @@ static void launch_render_fwd_variant(const RenderFwdArgs& a, hipStream_t stream
                      a.point_list, a.W, a.H, a.fx, a.fy, a.cx, a.cy, (const float2*)a.means2D, a.rgb, a.all_map,
                      (const float4*)a.conic_opacity, a.compute_locally, a.bg, a.final_T, a.n_contrib_px,
                      a.n_contrib2loss_px, a.out_color, a.out_observe, a.out_all_map, a.out_plane_depth, a.n_render,
-                     a.n_consider, a.n_contrib_tile, a.depths, a.out_max_weight_depth);
+                     a.n_consider, a.n_contrib_tile, a.depths, a.out_max_weight_depth, a.fits_word);
 }
 
 int launch_render_fwd(const RenderFwdArgs& a, hipStream_t stream) {

@@ -25,7 +25,9 @@ constexpr int BK_BATCH = 4;             // Gaussians a thread loads ahead
 constexpr int TS_THREADS = 256;         // per-tile sort
 
 __host__ __device__ inline int bucket_per_block(int P) {
-  const int per = (P + BK_MAX_BLOCKS - 1) / BK_MAX_BLOCKS;
+  // a multiple of four, so that a thread's four consecutive Gaussians start at a 16-byte boundary of every
+  // per-Gaussian array of words
+  const int per = ((P + BK_MAX_BLOCKS - 1) / BK_MAX_BLOCKS + 3) & ~3;
   return per < BK_MIN_PER_BLOCK ? BK_MIN_PER_BLOCK : per;
 }
 __host__ __device__ inline int bucket_blocks(int P) {
@@ -149,7 +151,8 @@ __device__ __forceinline__ uint32_t wave_inclusive_scan_u32(uint32_t v, int lane
 __global__ void __launch_bounds__(1024)
 bucket_ranges_kernel(uint32_t T, uint32_t limit, const uint32_t* __restrict__ totals, uint32_t* __restrict__ ranges,
                      uint32_t* __restrict__ chunk_first, uint32_t* __restrict__ block_sums, int nblocks,
-                     uint32_t* __restrict__ host_words) {
+                     uint32_t* __restrict__ host_words, uint32_t cap_instances, uint32_t cap_longest,
+                     uint32_t* __restrict__ fits_word) {
   constexpr int ITEMS = 4;  // consecutive tiles per thread: the usual grids (up to 4096 tiles) take one round
   __shared__ uint32_t s_wave[16], s_wave_chunks[16], s_max[16];
   __shared__ double s_exact[16];
@@ -239,6 +242,9 @@ bucket_ranges_kernel(uint32_t T, uint32_t limit, const uint32_t* __restrict__ to
     chunk_first[T] = carry_chunks;
     // more instances than 32-bit positions can address: the host must not go on with the wrapped count
     const uint32_t reported = all > (double)GS_MAX_INSTANCES ? GS_TOO_MANY_INSTANCES : carry;
+    // Kernels launched ahead of the host's decision (buffers sized from the caller's expectation) look at this
+    // word and do nothing unless the view fits what they were launched for.
+    *fits_word = (reported <= cap_instances && m <= cap_longest) ? 1u : 0u;
     __hip_atomic_store(host_words + 1, m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
     __hip_atomic_store(host_words + 2, carry_chunks, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
     __hip_atomic_store(host_words, reported, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
@@ -288,14 +294,23 @@ bucket_offsets_kernel(int P, int per_block, const uint32_t* __restrict__ tiles_t
 // 1d. Every instance goes to its tile's segment: segment start (ranges) + instances of earlier workgroups
 // (table) + a place among this workgroup's own, handed out by an LDS counter.  The record is
 // (depth bits << 32 | emission index); the Gaussian of an emission index goes to a side table
-// (rasterizer_impl.cu:74-117 writes the same pairs in emission order).
+// (rasterizer_impl.cu:74-117 writes the same pairs in emission order).  The kernel also finishes the prefix sum
+// over the Gaussians' tile counts (rasterizer_impl.cu:648) for its own chunk, which is where the emission
+// indices come from: a thread owns four consecutive Gaussians, the workgroup scans the threads' sums, and the
+// inclusive sums go to point_offsets on the way (the backward pass reads them).
+// fits_word (optional): the kernel was launched before the host knew the instance count; it does nothing unless
+// bucket_ranges_kernel found that the view fits the buffers it was launched with.
 __global__ void __launch_bounds__(BK_THREADS)
 bucket_scatter_kernel(int P, int per_block, uint32_t gx, uint32_t gy, const float2* __restrict__ means2D,
-                      const float* __restrict__ depths, const uint32_t* __restrict__ offsets,
+                      const float* __restrict__ depths, const uint32_t* __restrict__ tiles_touched,
+                      const uint32_t* __restrict__ block_prefix, uint32_t* __restrict__ point_offsets,
                       const int* __restrict__ radii, const uint8_t* __restrict__ compute_locally,
                       const uint32_t* __restrict__ table, const uint32_t* __restrict__ ranges,
-                      uint64_t* __restrict__ records, uint32_t* __restrict__ gauss_of_emission) {
+                      uint64_t* __restrict__ records, uint32_t* __restrict__ gauss_of_emission,
+                      const uint32_t* __restrict__ fits_word, int vector_loads) {
   extern __shared__ uint32_t s_next[];
+  __shared__ uint32_t s_wave[BK_THREADS / GS_WAVE];
+  if (fits_word != nullptr && *fits_word == 0u) return;
   const uint32_t T = gx * gy;
   uint8_t* s_local = reinterpret_cast<uint8_t*>(s_next + T);
   const uint32_t* row = table + (size_t)blockIdx.x * T;
@@ -304,27 +319,63 @@ bucket_scatter_kernel(int P, int per_block, uint32_t gx, uint32_t gy, const floa
     s_local[t] = compute_locally[t];
   }
   __syncthreads();
+  const int lane = threadIdx.x & (GS_WAVE - 1), wave = threadIdx.x / GS_WAVE;
   const int first = blockIdx.x * per_block;
   const int last = first + per_block < P ? first + per_block : P;
   struct Owner { uint32_t first, depth_bits, id; };
+  uint32_t carry = block_prefix[blockIdx.x];  // instances of the Gaussians before this round
   for (int base = first; base < last; base += BK_BATCH * BK_THREADS) {
+    const int i0 = base + (int)threadIdx.x * BK_BATCH;
     int r[BK_BATCH];
     float2 p[BK_BATCH];
-    uint32_t e0[BK_BATCH], dbits[BK_BATCH];
+    uint32_t tt[BK_BATCH], dbits[BK_BATCH], sum = 0;
+    static_assert(BK_BATCH == 4, "a thread's Gaussians are loaded as four-word vectors");
+    const bool whole = vector_loads != 0 && i0 + BK_BATCH <= last;
+    if (whole) {
+      // (i0 is a multiple of four and the host found every array 16-byte aligned: 16-byte loads)
+      const int4 rv = *reinterpret_cast<const int4*>(radii + i0);
+      const uint4 tv = *reinterpret_cast<const uint4*>(tiles_touched + i0);
+      const uint4 dv = *reinterpret_cast<const uint4*>(depths + i0);
+      const float4 m01 = *reinterpret_cast<const float4*>(means2D + i0);
+      const float4 m23 = *reinterpret_cast<const float4*>(means2D + i0 + 2);
+      r[0] = rv.x; r[1] = rv.y; r[2] = rv.z; r[3] = rv.w;
+      tt[0] = tv.x; tt[1] = tv.y; tt[2] = tv.z; tt[3] = tv.w;
+      dbits[0] = dv.x; dbits[1] = dv.y; dbits[2] = dv.z; dbits[3] = dv.w;
+      p[0] = make_float2(m01.x, m01.y); p[1] = make_float2(m01.z, m01.w);
+      p[2] = make_float2(m23.x, m23.y); p[3] = make_float2(m23.z, m23.w);
+    } else {
 #pragma unroll
-    for (int q = 0; q < BK_BATCH; q++) {
-      const int i = base + (int)threadIdx.x + q * BK_THREADS;
-      r[q] = i < last ? radii[i] : 0;
-      p[q] = i < last ? means2D[i] : make_float2(0.0f, 0.0f);
-      dbits[q] = i < last ? __float_as_uint(depths[i]) : 0u;
-      e0[q] = (i < last && i > 0) ? offsets[i - 1] : 0u;
+      for (int q = 0; q < BK_BATCH; q++) {
+        const int i = i0 + q;
+        r[q] = i < last ? radii[i] : 0;
+        p[q] = i < last ? means2D[i] : make_float2(0.0f, 0.0f);
+        dbits[q] = i < last ? __float_as_uint(depths[i]) : 0u;
+        tt[q] = i < last ? tiles_touched[i] : 0u;
+      }
     }
 #pragma unroll
+    for (int q = 0; q < BK_BATCH; q++) sum += tt[q];
+    const uint32_t inc = wave_inclusive_scan_u32(sum, lane);
+    if (lane == GS_WAVE - 1) s_wave[wave] = inc;
+    __syncthreads();
+    uint32_t before = 0, all = 0;
+#pragma unroll
+    for (int w = 0; w < BK_THREADS / GS_WAVE; w++) {
+      const uint32_t v = s_wave[w];
+      if (w < wave) before += v;
+      all += v;
+    }
+    __syncthreads();
+    uint32_t run = carry + before + inc - sum;  // emission index of this thread's first instance
+    carry += all;
+#pragma unroll
     for (int q = 0; q < BK_BATCH; q++) {
-      const int i = base + (int)threadIdx.x + q * BK_THREADS;
+      const int i = i0 + q;
       const bool live = i < last && r[q] > 0;
       const Rect rc = live ? get_rect(p[q].x, p[q].y, r[q], gx, gy) : Rect{0u, 0u, 0u, 0u};
-      const Owner mine = {e0[q], dbits[q], (uint32_t)i};
+      const Owner mine = {run, dbits[q], (uint32_t)i};
+      run += tt[q];
+      tt[q] = run;  // from here on: the inclusive sum
       walk_wave_rects(
           live, rc, gx, mine, [&](uint32_t tile) { return s_local[tile] != 0; },
           [&](const Owner& o, uint32_t tile, uint32_t rank) {
@@ -333,6 +384,13 @@ bucket_scatter_kernel(int P, int per_block, uint32_t gx, uint32_t gy, const floa
             records[pos] = ((uint64_t)o.depth_bits << 32) | (uint64_t)e;
             gauss_of_emission[e] = o.id;
           });
+    }
+    if (whole) {
+      *reinterpret_cast<uint4*>(point_offsets + i0) = make_uint4(tt[0], tt[1], tt[2], tt[3]);
+    } else {
+#pragma unroll
+      for (int q = 0; q < BK_BATCH; q++)
+        if (i0 + q < last) point_offsets[i0 + q] = tt[q];
     }
   }
 }
@@ -482,8 +540,10 @@ __device__ __forceinline__ void register_sort_tile(uint32_t t, uint32_t start, u
 __global__ void __launch_bounds__(256)
 tile_sort_registers_kernel(const uint32_t* __restrict__ ranges, const uint64_t* __restrict__ records,
                            const uint32_t* __restrict__ gauss_of_emission, uint64_t* __restrict__ keys,
-                           uint32_t* __restrict__ emission, uint32_t* __restrict__ point_list, uint32_t max_n) {
+                           uint32_t* __restrict__ emission, uint32_t* __restrict__ point_list, uint32_t max_n,
+                           const uint32_t* __restrict__ fits_word) {
   extern __shared__ uint64_t s_exchange[];
+  if (fits_word != nullptr && *fits_word == 0u) return;  // launched ahead of the host's decision: see the scatter
   const uint32_t t = blockIdx.x;
   const uint32_t start = ranges[2 * t];
   const uint32_t n = ranges[2 * t + 1] - start;
@@ -498,8 +558,9 @@ __global__ void __launch_bounds__(1024)
 tile_sort_registers_long_kernel(const uint32_t* __restrict__ ranges, const uint64_t* __restrict__ records,
                                 const uint32_t* __restrict__ gauss_of_emission, uint64_t* __restrict__ keys,
                                 uint32_t* __restrict__ emission, uint32_t* __restrict__ point_list,
-                                uint32_t max_n) {
+                                uint32_t max_n, const uint32_t* __restrict__ fits_word) {
   extern __shared__ uint64_t s_exchange[];
+  if (fits_word != nullptr && *fits_word == 0u) return;
   const uint32_t t = blockIdx.x;
   const uint32_t start = ranges[2 * t];
   const uint32_t n = ranges[2 * t + 1] - start;
@@ -657,16 +718,21 @@ int bucket_max_tiles() { return 30000; }
 
 // workgroup-by-tile counts, then the tile totals, then the chunk table (T + 1 words), then the workgroups' sums of
 // tiles touched
+// ... and the word that says whether the view fits the buffers of kernels launched ahead of the host
 size_t bucket_table_bytes(int T) {
-  return (((size_t)BK_MAX_BLOCKS + 2) * (size_t)T + 1 + BK_MAX_BLOCKS) * sizeof(uint32_t);
+  return (((size_t)BK_MAX_BLOCKS + 2) * (size_t)T + 1 + BK_MAX_BLOCKS + 1) * sizeof(uint32_t);
 }
 static uint32_t* bucket_block_sums(void* table, uint32_t T) {
   return (uint32_t*)table + ((size_t)BK_MAX_BLOCKS + 2) * (size_t)T + 1;
 }
+const uint32_t* bucket_fits_word(const void* table, int T) {
+  return (const uint32_t*)table + ((size_t)BK_MAX_BLOCKS + 2) * (size_t)T + 1 + BK_MAX_BLOCKS;
+}
 
 int launch_bucket_count(int P, int W, int H, const int* radii, const float* means2D, const uint8_t* compute_locally,
                         uint32_t* tiles_touched, void* table, uint32_t* ranges, uint32_t chunk_limit,
-                        uint32_t* host_words, int* zero_per_gaussian, hipStream_t stream) {
+                        uint32_t* host_words, int* zero_per_gaussian, uint32_t cap_instances, uint32_t cap_longest,
+                        hipStream_t stream) {
   if (P <= 0) return 0;
   if (chunk_limit == 0 || chunk_limit > (uint32_t)TILE_SORT_LARGE) chunk_limit = TILE_SORT_LARGE;
   const uint32_t gx = (W + GS_TILE_X - 1) / GS_TILE_X, gy = (H + GS_TILE_Y - 1) / GS_TILE_Y;
@@ -694,11 +760,14 @@ int launch_bucket_count(int P, int W, int H, const int* radii, const float* mean
   hipLaunchKernelGGL(bucket_columns_kernel, dim3((T + COL_TILES - 1) / COL_TILES), dim3(COL_TILES * COL_RUNS), 0, stream, nb, T,
                      tab, totals);
   hipLaunchKernelGGL(bucket_ranges_kernel, dim3(1), dim3(1024), 0, stream, T, chunk_limit, totals, ranges, totals + T,
-                     bucket_block_sums(table, T), nb, host_words);
+                     bucket_block_sums(table, T), nb, host_words, cap_instances, cap_longest,
+                     const_cast<uint32_t*>(bucket_fits_word(table, (int)T)));
   return 0;
 }
 
-// point_offsets = inclusive prefix sum of the tiles_touched that launch_bucket_count left (same P, same table)
+// point_offsets = inclusive prefix sum of the tiles_touched that launch_bucket_count left (same P, same table).
+// launch_bucket_scatter does this itself; this kernel serves a view that was counted by tile and then goes to the
+// radix sort after all.
 int launch_bucket_offsets(int P, int W, int H, const uint32_t* tiles_touched, void* table, uint32_t* point_offsets,
                           hipStream_t stream) {
   if (P <= 0) return 0;
@@ -708,16 +777,20 @@ int launch_bucket_offsets(int P, int W, int H, const uint32_t* tiles_touched, vo
   return 0;
 }
 
-int launch_bucket_scatter(int P, int W, int H, const float* means2D, const float* depths, const uint32_t* offsets,
-                          const int* radii, const uint8_t* compute_locally, const void* table,
-                          const uint32_t* ranges, uint64_t* records, uint32_t* gauss_of_emission,
-                          hipStream_t stream) {
+int launch_bucket_scatter(int P, int W, int H, const float* means2D, const float* depths,
+                          const uint32_t* tiles_touched, uint32_t* point_offsets, const int* radii,
+                          const uint8_t* compute_locally, void* table, const uint32_t* ranges, uint64_t* records,
+                          uint32_t* gauss_of_emission, bool ahead_of_host, hipStream_t stream) {
   if (P <= 0) return 0;
   const uint32_t gx = (W + GS_TILE_X - 1) / GS_TILE_X, gy = (H + GS_TILE_Y - 1) / GS_TILE_Y;
   const size_t lds = (size_t)gx * gy * (sizeof(uint32_t) + 1);
   hipLaunchKernelGGL(bucket_scatter_kernel, dim3(bucket_blocks(P)), dim3(BK_THREADS), lds, stream, P,
-                     bucket_per_block(P), gx, gy, (const float2*)means2D, depths, offsets, radii, compute_locally,
-                     (const uint32_t*)table, ranges, records, gauss_of_emission);
+                     bucket_per_block(P), gx, gy, (const float2*)means2D, depths, tiles_touched,
+                     bucket_block_sums(table, gx * gy), point_offsets, radii, compute_locally, (const uint32_t*)table,
+                     ranges, records, gauss_of_emission,
+                     ahead_of_host ? bucket_fits_word(table, (int)(gx * gy)) : nullptr,
+                     (((uintptr_t)means2D | (uintptr_t)depths | (uintptr_t)tiles_touched | (uintptr_t)point_offsets |
+                       (uintptr_t)radii) & 15u) == 0u ? 1 : 0);
   return 0;
 }
 
@@ -727,8 +800,10 @@ int launch_bucket_scatter(int P, int W, int H, const float* means2D, const float
 // with the same limit: sorted in place in `records`, then merged.
 int launch_tile_sort(int T, uint32_t longest, uint32_t limit, uint32_t chunks, uint32_t in_registers,
                      const uint32_t* ranges, const void* table, uint64_t* records, const uint32_t* gauss_of_emission,
-                     uint64_t* keys, uint32_t* emission, uint32_t* point_list, hipStream_t stream) {
+                     uint64_t* keys, uint32_t* emission, uint32_t* point_list, bool ahead_of_host,
+                     hipStream_t stream) {
   if (T <= 0 || longest == 0) return 0;
+  const uint32_t* fits = ahead_of_host ? bucket_fits_word(table, T) : nullptr;
   if (limit == 0 || limit > (uint32_t)TILE_SORT_LARGE) limit = TILE_SORT_LARGE;
   const uint32_t whole = longest < limit ? longest : limit;  // the longest list sorted by one workgroup
   if (in_registers == 0) {
@@ -742,11 +817,11 @@ int launch_tile_sort(int T, uint32_t longest, uint32_t limit, uint32_t chunks, u
     uint32_t m = 256;
     while (m < whole && m < 2048) m <<= 1;
     hipLaunchKernelGGL(tile_sort_registers_kernel, dim3(T), dim3(256), (size_t)m * sizeof(uint64_t), stream, ranges,
-                       records, gauss_of_emission, keys, emission, point_list, limit);
+                       records, gauss_of_emission, keys, emission, point_list, limit, fits);
     if (whole > 2048)
       hipLaunchKernelGGL(tile_sort_registers_long_kernel, dim3(T), dim3(1024),
                          (size_t)(whole > 4096 ? 8192 : 4096) * sizeof(uint64_t), stream, ranges, records,
-                         gauss_of_emission, keys, emission, point_list, limit);
+                         gauss_of_emission, keys, emission, point_list, limit, fits);
   }
   if (longest > limit && chunks > 0) {
     const uint32_t* chunk_first = (const uint32_t*)table + ((size_t)BK_MAX_BLOCKS + 1) * (size_t)T;

@@ -172,6 +172,19 @@ def render_gaussians(background, image_height, image_width, means2D, depths, rad
     Gaussian that blends with the largest weight (1, H, W) is left in args["stats_collector"]["max_weight_depth"];
     args["tile_sort_limits"] = (in_registers, large_limit, max_chunks) chooses, for this call, the way the per-tile
     lists are built (all ways give the same lists).  The returned tuple is the reference's either way."""
+    return render_gaussians_ex(background, image_height, image_width, means2D, depths, radii, conic_opacity, rgb,
+                               compute_locally, viewmatrix, campos, tan_fovx, tan_fovy, all_map, render_geo, debug,
+                               args)[0]
+
+
+def render_gaussians_ex(background, image_height, image_width, means2D, depths, radii, conic_opacity, rgb,
+                        compute_locally, viewmatrix, campos, tan_fovx, tan_fovy, all_map, render_geo, debug, args,
+                        expected_instances=0, expected_longest_list=0):
+    """render_gaussians plus what the reference's tuple has no slot for: returns (tuple, info) with info =
+    {"longest_list", "binning_capacity", "launched_ahead"}.  With expected_instances > 0 the list kernels and the
+    blend are launched without waiting for the instance count, on a binning buffer laid out for
+    expected_instances; info["binning_capacity"] then has to be handed to render_gaussians_backward (and to
+    gs_binning_state_layout) in place of the instance count.  Results do not depend on the expectation."""
     means2D = _f32c(means2D, "means2D")
     dev = means2D.device
     P = means2D.shape[0]
@@ -182,9 +195,10 @@ def render_gaussians(background, image_height, image_width, means2D, depths, rad
     geo = bool(render_geo)
     if P == 0:
         empty = torch.empty(0, dtype=torch.uint8, device=dev)
-        return (0, torch.zeros(NUM_CHANNELS, H, W, **f32), torch.zeros(tiles, **i32), torch.zeros(tiles, **i32),
-                torch.zeros(tiles, **i32), torch.zeros(0, **i32), torch.zeros(NUM_ALL_MAP, H, W, **f32),
-                torch.zeros(1, H, W, **f32), empty, empty.clone(), empty.clone())
+        return ((0, torch.zeros(NUM_CHANNELS, H, W, **f32), torch.zeros(tiles, **i32), torch.zeros(tiles, **i32),
+                 torch.zeros(tiles, **i32), torch.zeros(0, **i32), torch.zeros(NUM_ALL_MAP, H, W, **f32),
+                 torch.zeros(1, H, W, **f32), empty, empty.clone(), empty.clone()),
+                {"longest_list": 0, "binning_capacity": 0, "launched_ahead": False})
     out_color = torch.empty(NUM_CHANNELS, H, W, **f32)
     out_observe = torch.empty(P, **i32)  # cleared by the call itself
     out_all_map = torch.empty(NUM_ALL_MAP, H, W, **f32) if geo else torch.zeros(NUM_ALL_MAP, H, W, **f32)
@@ -205,7 +219,12 @@ def render_gaussians(background, image_height, image_width, means2D, depths, rad
     want_mwd = isinstance(args, dict) and bool(args.get("max_weight_depth"))
     # (in_registers, large_limit, max_chunks) for this call only: how the per-tile lists are built (a test hook)
     limits = args.get("tile_sort_limits") if isinstance(args, dict) else None
-    options = _n.RenderOptions(*limits) if limits is not None else None
+    options = None
+    if limits is not None or expected_instances > 0:
+        options = _n.RenderOptions(*(limits if limits is not None else (-1, -1, -1)),
+                                   expected_instances=expected_instances,
+                                   expected_longest_list=expected_longest_list)
+    result = _n.RenderResult()
     mwd = torch.empty(1, H, W, **f32) if want_mwd else None
     # fp32 arithmetic, as `H / (2.0f * tan_fovy)` at rasterize_points.cu:328-329
     focal_y = np.float32(H) / (np.float32(2.0) * np.float32(tan_fovy))
@@ -221,20 +240,23 @@ def render_gaussians(background, image_height, image_width, means2D, depths, rad
             _ptr(n_consider), _ptr(n_contrib), _ptr(out_observe), _ptr(out_all_map), _ptr(out_plane_depth), _ptr(mwd),
             int(geo),
             int(bool(debug)), C.byref(num_rendered), C.byref(elapsed) if timing else None,
-            C.byref(options) if options is not None else None, _stream(dev)),
+            C.byref(options) if options is not None else None, C.byref(result), _stream(dev)),
             "render_gaussians")
     _record_time(args, "forward_render_time", elapsed.value)
     if want_mwd:
         args.setdefault("stats_collector", {})["max_weight_depth"] = mwd
-    return (num_rendered.value, out_color, n_render, n_consider, n_contrib, out_observe, out_all_map, out_plane_depth,
-            geom.release(), binning.release(), img.release())
+    info = {"longest_list": int(result.longest_list), "binning_capacity": int(result.binning_capacity),
+            "launched_ahead": bool(result.launched_ahead)}
+    return ((num_rendered.value, out_color, n_render, n_consider, n_contrib, out_observe, out_all_map,
+             out_plane_depth, geom.release(), binning.release(), img.release()), info)
 
 
 def render_gaussians_backward(background, tan_fovx, tan_fovy, all_map_pixels, all_maps, R, geomBuffer, binningBuffer,
                               imageBuffer, compute_locally, dL_dout_color, dL_dout_all_map, dL_dout_plane_depth,
-                              means2D, conic_opacity, rgb, render_geo, debug, args):
+                              means2D, conic_opacity, rgb, render_geo, debug, args, binning_capacity=0):
     """rasterize_points.cu:366-441.  Returns dL_dmeans2D as (P,2); the reference
-    returns (P,3) and its Python wrapper slices [:, :2]."""
+    returns (P,3) and its Python wrapper slices [:, :2].  binning_capacity: info["binning_capacity"] of
+    render_gaussians_ex when that call was given an expectation (0 otherwise)."""
     means2D = _f32c(means2D, "means2D")
     dev = means2D.device
     P = means2D.shape[0]
@@ -265,7 +287,8 @@ def render_gaussians_backward(background, tan_fovx, tan_fovy, all_map_pixels, al
                 _ptr(imageBuffer), _ptr(compute_locally.contiguous()), _ptr(gpix), _ptr(gmap), _ptr(gdep),
                 _ptr(dL_dmeans2D), _ptr(dL_dmeans2D_abs), _ptr(dL_dconic_opacity), _ptr(dL_dcolors), _ptr(dL_dall_map),
                 _ptr(means2D), _ptr(co), _ptr(col), _ptr(am), _ptr(amp), int(geo), int(bool(debug)), _ptr(workspace),
-                ws_bytes, C.byref(elapsed) if timing else None, _stream(dev)), "render_gaussians_backward")
+                ws_bytes, C.byref(elapsed) if timing else None, int(binning_capacity), _stream(dev)),
+                "render_gaussians_backward")
         _record_time(args, "backward_render_time", elapsed.value)
     else:
         _record_time(args, "backward_render_time", 0.0)

@@ -83,6 +83,28 @@ def preprocess_gaussians(means3D, scales, rotations, sh, opacities, raster_setti
 
 # ------------------------------------------------------------------- render --
 
+# What the last view of a given shape needed, (instances, longest list) keyed by (Gaussians, height, width, device):
+# the next view of that shape is launched without waiting for its instance count, on buffers sized for these figures
+# plus a margin (a training loop renders thousands of similar views).  Only the time depends on it, never a result;
+# a stale or missing entry costs one ordinary call.
+_expectations = {}
+_MARGIN = 1.25
+
+
+def _expectation(key):
+    seen = _expectations.get(key)
+    if seen is None:
+        return 0, 0
+    instances, longest = seen
+    if longest <= 0 or longest > 8192:
+        return 0, 0  # a view for the radix sort (no per-tile lists, or lists too long for them): nothing to gain
+    # whole sort variants (256 ... 8192 records per list), so that a slightly longer list still fits
+    cap = 256
+    while cap < min(8192, longest * _MARGIN):
+        cap *= 2
+    return int(instances * _MARGIN) + 65536, cap
+
+
 class _RenderGaussians(torch.autograd.Function):
     @staticmethod
     def forward(ctx, means2D, means2D_abs, conic_opacity, rgb, all_maps, depths, radii, compute_locally,
@@ -90,10 +112,16 @@ class _RenderGaussians(torch.autograd.Function):
         rs = raster_settings
         avoid = bool(cuda_args.get("avoid_pixel_all2all", False)) if cuda_args is not None else False
         mask = extended_compute_locally if avoid else compute_locally
-        (num_rendered, color, n_render, n_consider, n_contrib, out_observe, out_all_map, out_plane_depth, geomBuffer,
-         binningBuffer, imgBuffer) = _C.render_gaussians(
+        key = (means2D.shape[0], rs.image_height, rs.image_width, means2D.device)
+        expected_instances, expected_longest = _expectation(key)
+        ((num_rendered, color, n_render, n_consider, n_contrib, out_observe, out_all_map, out_plane_depth, geomBuffer,
+          binningBuffer, imgBuffer), info) = _C.render_gaussians_ex(
             rs.bg, rs.image_height, rs.image_width, means2D, depths, radii, conic_opacity, rgb, mask, rs.viewmatrix,
-            rs.campos, rs.tanfovx, rs.tanfovy, all_maps, rs.render_geo, rs.debug, cuda_args)
+            rs.campos, rs.tanfovx, rs.tanfovy, all_maps, rs.render_geo, rs.debug, cuda_args,
+            expected_instances=expected_instances, expected_longest_list=expected_longest)
+        if means2D.shape[0] > 0:
+            _expectations[key] = (num_rendered, info["longest_list"])
+        ctx.binning_capacity = info["binning_capacity"]
         ctx.raster_settings = rs
         ctx.cuda_args = cuda_args
         ctx.num_rendered = num_rendered
@@ -119,7 +147,7 @@ class _RenderGaussians(torch.autograd.Function):
         dL_dmeans2D, dL_dmeans2D_abs, dL_dconic_opacity, dL_dcolors, dL_dall_map = _C.render_gaussians_backward(
             rs.bg, rs.tanfovx, rs.tanfovy, all_map_pixels, all_maps, ctx.num_rendered, geomBuffer, binningBuffer,
             imgBuffer, compute_locally, grad_color, grad_out_all_map, grad_out_plane_depth, means2D, conic_opacity,
-            rgb, rs.render_geo, rs.debug, ctx.cuda_args)
+            rgb, rs.render_geo, rs.debug, ctx.cuda_args, binning_capacity=ctx.binning_capacity)
         return (dL_dmeans2D, dL_dmeans2D_abs, dL_dconic_opacity, dL_dcolors, dL_dall_map, None, None, None, None, None,
                 None)
 

@@ -32,9 +32,10 @@ _SIGNATURES = {
     "gs_preprocess_backward": (_i, [_vp] * 3 + [_i] * 5 + [_vp] * 4 + [_f] + [_vp] * 3 + [_f, _f] + [_vp, _i] +
                                [_vp] * 8 + [_i, _vp]),
     "gs_render_forward": (_i, [RESIZE_FN, _vp, RESIZE_FN, _vp, RESIZE_FN, _vp, _i, _vp, _i, _i, _f, _f, _f, _f] +
-                          [_vp] * 17 + [_i, _i, C.POINTER(_i), C.POINTER(_f), _vp, _vp]),
+                          [_vp] * 17 + [_i, _i, C.POINTER(_i), C.POINTER(_f), _vp, _vp, _vp]),
     "gs_render_backward_workspace_bytes": (_sz, [_i]),
-    "gs_render_backward": (_i, [_i, _i, _vp, _i, _i, _f, _f] + [_vp] * 17 + [_i, _i, _vp, _sz, C.POINTER(_f), _vp]),
+    "gs_render_backward": (_i, [_i, _i, _vp, _i, _i, _f, _f] + [_vp] * 17 + [_i, _i, _vp, _sz, C.POINTER(_f), _i64,
+                                _vp]),
     "gs_ssim_l1_forward": (_i, [_i, _i, _i] + [_vp] * 9),
     "gs_ssim_l1_backward": (_i, [_i, _i, _i] + [_vp] * 10),
     "gs_training_stats_workspace_bytes": (_sz, [_i64, _i64]),
@@ -84,13 +85,25 @@ EXPORTED_SYMBOLS = tuple(_SIGNATURES)
 
 
 class RenderOptions(C.Structure):
-    """gs_render_options of include/gsrast.h; a negative field keeps the library's default."""
+    """gs_render_options of include/gsrast.h; a negative limit keeps the library's default, a zero expectation
+    means none."""
     _fields_ = [("struct_bytes", C.c_uint32), ("tile_sort_in_registers", C.c_int32),
-                ("tile_sort_large_limit", C.c_int32), ("tile_sort_max_chunks", C.c_int32)]
+                ("tile_sort_large_limit", C.c_int32), ("tile_sort_max_chunks", C.c_int32),
+                ("expected_instances", C.c_int64), ("expected_longest_list", C.c_int32), ("reserved", C.c_int32)]
 
-    def __init__(self, tile_sort_in_registers=-1, tile_sort_large_limit=-1, tile_sort_max_chunks=-1):
+    def __init__(self, tile_sort_in_registers=-1, tile_sort_large_limit=-1, tile_sort_max_chunks=-1,
+                 expected_instances=0, expected_longest_list=0):
         super().__init__(C.sizeof(RenderOptions), int(tile_sort_in_registers), int(tile_sort_large_limit),
-                         int(tile_sort_max_chunks))
+                         int(tile_sort_max_chunks), int(expected_instances), int(expected_longest_list), 0)
+
+
+class RenderResult(C.Structure):
+    """gs_render_result of include/gsrast.h."""
+    _fields_ = [("struct_bytes", C.c_uint32), ("longest_list", C.c_int32), ("binning_capacity", C.c_int64),
+                ("launched_ahead", C.c_int32), ("reserved", C.c_int32)]
+
+    def __init__(self):
+        super().__init__(C.sizeof(RenderResult), 0, 0, 0, 0)
 
 
 def stage_timing(enable):

@@ -109,7 +109,29 @@ typedef struct gs_render_options {
   int32_t tile_sort_in_registers;
   int32_t tile_sort_large_limit;
   int32_t tile_sort_max_chunks;
+  /* What the caller expects of the view, typically the previous view's figures with a margin (0 = no idea).
+   * With expected_instances > 0 (and a gs_render_result to report into) gs_render_forward does not wait for the
+   * instance count before it goes on: it sizes the binning buffer for expected_instances, launches the list
+   * kernels and the blend right behind the counting kernels, and lets a device-side check turn them into no-ops
+   * if the view has more instances than that or a list longer than expected_longest_list (0 = the longest one
+   * workgroup sorts); in that case the lists are built again the ordinary way, so the result never depends on
+   * the expectation, only the time does. */
+  int64_t expected_instances;
+  int32_t expected_longest_list;
+  int32_t reserved;
 } gs_render_options;
+
+/* What gs_render_forward reports besides the instance count (optional, NULL to skip; struct_bytes as above):
+ * the longest per-tile list (0 on the radix route), whether the list kernels ran ahead of the host, and
+ * binning_capacity: the instance count the arrays inside the binning buffer are laid out for, which is the
+ * instance count itself unless the kernels ran ahead.  gs_render_backward and gs_binning_state_layout take it. */
+typedef struct gs_render_result {
+  uint32_t struct_bytes;
+  int32_t longest_list;
+  int64_t binning_capacity;
+  int32_t launched_ahead;
+  int32_t reserved;
+} gs_render_result;
 
 /* Replaces Rasterizer::renderForward (CR/rasterizer.h:130-160,
  * CR/rasterizer_impl.cu:586-846): tile count -> prefix sum -> host read-back of
@@ -139,7 +161,8 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
                       const float* rgb, const uint8_t* compute_locally, float* out_color, int* n_render,
                       int* n_consider, int* n_contrib, int* out_observe, float* out_all_map,
                       float* out_plane_depth, float* out_max_weight_depth, int render_geo, int debug,
-                      int* num_rendered, float* elapsed_ms, const gs_render_options* options, gs_stream_t stream);
+                      int* num_rendered, float* elapsed_ms, const gs_render_options* options,
+                      gs_render_result* result, gs_stream_t stream);
 
 /* Replaces Rasterizer::renderBackward (CR/rasterizer.h:162-187,
  * CR/rasterizer_impl.cu:850-932) plus the repacking of
@@ -153,7 +176,8 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
  * per (tile, Gaussian) instance into instance_grads, a caller-provided scratch
  * of gs_render_backward_workspace_bytes(R) bytes, and sums each Gaussian's
  * records in a second kernel (no atomics, run-to-run deterministic).
- * elapsed_ms as above (backward_render_time, CR/rasterizer_impl.cu:924-926). */
+ * elapsed_ms as above (backward_render_time, CR/rasterizer_impl.cu:924-926).
+ * binning_capacity: gs_render_result.binning_capacity of the forward call (0 or R if it did not run ahead). */
 size_t gs_render_backward_workspace_bytes(int R);
 int gs_render_backward(int P, int R, const float* background, int width, int height, float tan_fovx,
                        float tan_fovy, const char* geom_buffer, const char* binning_buffer,
@@ -162,7 +186,8 @@ int gs_render_backward(int P, int R, const float* background, int width, int hei
                        float* dL_dmean2D_abs, float* dL_dconic_opacity, float* dL_dcolor, float* dL_dall_map,
                        const float* means2D, const float* conic_opacity, const float* rgb, const float* all_maps,
                        const float* all_map_pixels, int render_geo, int debug, float* instance_grads,
-                       size_t instance_grads_bytes, float* elapsed_ms, gs_stream_t stream);
+                       size_t instance_grads_bytes, float* elapsed_ms, int64_t binning_capacity,
+                       gs_stream_t stream);
 
 /* Replaces SimpleKNN::knn / distCUDA2 (KNN/simple_knn.h:17, KNN/simple_knn.cu:185-221,
  * KNN/spatial.cu:17-35): mean_dists[i] = mean squared distance from point i
@@ -402,7 +427,8 @@ int gs_stage_timing_collect(char* report, size_t report_bytes);
 
 /* Byte offsets of the arrays inside the buffers gs_render_forward fills
  * (the role of ImageState / BinningState::fromChunk, CR/rasterizer_impl.cu:182-205),
- * relative to the 256-byte-aligned start of each buffer.  Host pointers. */
+ * relative to the 256-byte-aligned start of each buffer.  Host pointers.  R of gs_binning_state_layout is the
+ * forward call's binning_capacity (the instance count unless its kernels ran ahead of the host). */
 int gs_image_state_layout(int width, int height, size_t* accum_alpha, size_t* n_contrib, size_t* n_contrib2loss,
                           size_t* ranges, size_t* total_bytes);
 int gs_binning_state_layout(int64_t R, int width, int height, size_t* point_list, size_t* point_list_keys,

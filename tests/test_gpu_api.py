@@ -282,6 +282,100 @@ def test_pixels_of_tiles_not_computed_locally_read_zero(geo):
     assert float((color * px).sum()) == float(color.sum())
 
 
+def test_launching_ahead_of_the_instance_count_changes_no_result(orc):
+    """With an expectation of the view's size, render_gaussians launches the list kernels and the blend without
+    waiting for the instance count.  Whether the expectation holds (kernels ran ahead), is too small in instances
+    or in list length (they turn into no-ops and the lists are built again), or is absent: same outputs and same
+    gradients, bit for bit; the buffers of a call that ran ahead are laid out for its capacity."""
+    import ctypes as C
+    import gs_scenes
+    import gsrast_native as gn
+    from diff_gaussian_rasterization import _C
+    import gpu_harness as H
+    g, cams = gs_scenes.make_scene(1, P=150_000, n_views=1)
+    cam = cams[0]
+    W, Hh = cam.image_width, cam.image_height
+    gx, gy = H.grid(W, Hh)
+    o, gd = H.preprocess_fwd(g, cam)
+    vm, cp = cam.world_view_transform.to(DEV), cam.camera_center.to(DEV)
+    am = gs_scenes.build_all_map(gd["means3D"], gd["scales"], gd["rotations"], cam)
+    cl = torch.ones(gy, gx, dtype=torch.bool, device=DEV)
+    bg = torch.tensor([0.2, 0.1, 0.3], device=DEV)
+    ug = {k: v.to(DEV) for k, v in gs_scenes.upstream_grads(cam).items()}
+
+    def run(expected_instances=0, expected_longest=0):
+        args = {"stats_collector": {}}
+        out, info = _C.render_gaussians_ex(bg, Hh, W, o["means2D"], o["depths"], o["radii"], o["conic_opacity"],
+                                           o["rgb"], cl, vm, cp, cam.tanfovx, cam.tanfovy, am, True, False, args,
+                                           expected_instances=expected_instances,
+                                           expected_longest_list=expected_longest)
+        R, geomB, binB, imgB = out[0], out[8], out[9], out[10]
+        back = _C.render_gaussians_backward(bg, cam.tanfovx, cam.tanfovy, out[6], am, R, geomB, binB, imgB, cl,
+                                            ug["color"], ug["all_map"], ug["plane_depth"], o["means2D"],
+                                            o["conic_opacity"], o["rgb"], True, False, args,
+                                            binning_capacity=info["binning_capacity"])
+        off = [C.c_size_t() for _ in range(5)]
+        gn.check(gn.lib.gs_binning_state_layout(info["binning_capacity"], W, Hh, *[C.byref(x) for x in off]), "layout")
+        base = (binB.data_ptr() + 255) // 256 * 256 - binB.data_ptr()
+        point_list = binB[base + off[0].value: base + off[0].value + 4 * R].view(torch.int32).clone()
+        keys = binB[base + off[1].value: base + off[1].value + 8 * R].view(torch.int64).clone()
+        return out, info, back, point_list, keys
+
+    plain = run()
+    R, longest = plain[0][0], plain[1]["longest_list"]
+    assert not plain[1]["launched_ahead"] and plain[1]["binning_capacity"] == R and 0 < longest <= 2048
+    n = lambda t: t.detach().cpu().numpy()
+    want = orc.bin_and_sort(n(o["radii"]), n(o["means2D"]), n(o["depths"]), np.ones(gx * gy, bool), W, Hh)
+    assert np.array_equal(H.np_u32(plain[3]), want["point_list"])
+    cases = [("holds", R + 1000, 2048, True), ("exact", R, longest, True), ("default list length", 2 * R, 0, True),
+             ("too few instances", R - 1, 2048, False), ("list too long", R + 1000, longest - 1, False)]
+    for name, exp_n, exp_l, ahead in cases:
+        got = run(exp_n, exp_l)
+        assert got[1]["launched_ahead"] == ahead, name
+        assert got[1]["binning_capacity"] == (exp_n if ahead else R), name
+        assert got[1]["longest_list"] == longest and got[0][0] == R, name
+        for a, b in zip(plain[0][1:8], got[0][1:8]):
+            assert torch.equal(a, b), name
+        for a, b in zip(plain[2], got[2]):
+            assert torch.equal(a, b), name
+        assert torch.equal(plain[3], got[3]) and torch.equal(plain[4], got[4]), name
+
+
+def test_the_operator_launches_ahead_from_the_second_view_on():
+    """GaussianRasterizer remembers what the last view of a shape needed and launches the next one ahead; the
+    gradients of the leaves are the same bits as on the first, ordinary call."""
+    import gs_scenes
+    import diff_gaussian_rasterization as dgr
+    g, cams = gs_scenes.make_scene(0, P=25_000, n_views=1)
+    cam = cams[0]
+    W, H = cam.image_width, cam.image_height
+    gx, gy = (W + 15) // 16, (H + 15) // 16
+    cl = torch.ones(gy, gx, dtype=torch.bool, device=DEV)
+    ug = {k: v.to(DEV) for k, v in gs_scenes.upstream_grads(cam).items()}
+    am = gs_scenes.build_all_map(g["means3D"], g["scales"], g["rotations"], cam).to(DEV)
+    dgr._expectations.clear()
+
+    def run():
+        rast = dgr.GaussianRasterizer(_settings(cam))
+        leaf = {k: g[k].to(DEV).requires_grad_(True) for k in ("means3D", "scales", "rotations", "opacities", "shs")}
+        args = _cuda_args()
+        means2D, rgb, co, radii, depths = rast.preprocess_gaussians(
+            leaf["means3D"], leaf["scales"], leaf["rotations"], leaf["shs"], leaf["opacities"], args)
+        m2abs = torch.zeros_like(leaf["means3D"], requires_grad=True) + 0
+        color, n_render, n_consider, n_contrib, obs, oam, opd = rast.render_gaussians(
+            means2D, m2abs, co, rgb, am, depths, radii, cl, cl, args)
+        torch.autograd.backward([color, oam, opd], [ug["color"], ug["all_map"], ug["plane_depth"]])
+        return [color, n_render, n_consider, n_contrib, obs, oam, opd] + [leaf[k].grad for k in sorted(leaf)]
+
+    first = run()
+    key = (25_000, H, W, torch.device(DEV))
+    assert key in dgr._expectations and dgr._expectation(key)[0] > dgr._expectations[key][0]
+    for _ in range(2):
+        again = run()
+        for a, b in zip(first, again):
+            assert torch.equal(a, b)
+
+
 def test_debug_mode_gives_the_same_results_by_every_route():
     """debug=True makes every stage wait for its kernels and report their errors (and check the radix sort's
     status word); results are those of the normal mode bit for bit, whichever way the per-tile lists are built."""
