@@ -158,6 +158,7 @@ GeometryLayout geometry_layout(int P) {
 struct BinningLayout {
   size_t point_list, keys, point_list_unsorted, keys_unsorted, emission, emission_other, sort_temp, total;
 };
+// n = the number of instances the arrays are laid out for
 BinningLayout binning_layout(int64_t R) {
   BinningLayout L;
   const size_t n = (size_t)(R > 0 ? R : 1);
@@ -431,15 +432,14 @@ int pending_fault(const char* who) {
 }
 
 struct TileSortLimits {
-  int in_registers, large, chunks;
+  int large, chunks;
 };
-// The defaults, or what the caller's options ask for: whether the per-tile sort keeps the records in registers
-// (or in LDS), the list length up to which one workgroup sorts a list whole (0: every view takes the radix
-// sort), and the number of chunks up to which the longer lists of a view are sorted in chunks and merged.
+// The defaults, or what the caller's options ask for: the list length up to which one workgroup sorts a list
+// whole (0: every view takes the radix sort), and the number of chunks up to which the longer lists of a view are
+// sorted in chunks and merged.
 TileSortLimits tile_sort_limits(const gs_render_options* o) {
-  TileSortLimits L = {1, TILE_SORT_LARGE, TILE_SORT_MAX_CHUNKS};
-  if (o == nullptr || o->struct_bytes < 4 * sizeof(uint32_t)) return L;
-  if (o->tile_sort_in_registers >= 0) L.in_registers = o->tile_sort_in_registers != 0;
+  TileSortLimits L = {TILE_SORT_LARGE, TILE_SORT_MAX_CHUNKS};
+  if (o == nullptr || o->struct_bytes < 3 * sizeof(uint32_t)) return L;
   if (o->tile_sort_large_limit >= 0) L.large = o->tile_sort_large_limit < TILE_SORT_LARGE ? o->tile_sort_large_limit : TILE_SORT_LARGE;
   if (o->tile_sort_max_chunks >= 0) L.chunks = o->tile_sort_max_chunks;
   return L;
@@ -510,8 +510,7 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
   int64_t cap_n = 0;
   uint32_t cap_longest = 0;
   if (counted_by_tile && !dbg && result != nullptr && result->struct_bytes >= sizeof(gs_render_result) &&
-      options != nullptr && options->struct_bytes >= sizeof(gs_render_options) && options->expected_instances > 0 &&
-      limits.in_registers != 0) {
+      options != nullptr && options->struct_bytes >= sizeof(gs_render_options) && options->expected_instances > 0) {
     cap_n = options->expected_instances < (int64_t)GS_MAX_INSTANCES ? options->expected_instances
                                                                      : (int64_t)GS_MAX_INSTANCES;
     cap_longest = options->expected_longest_list > 0 ? (uint32_t)options->expected_longest_list : sort_limit;
@@ -589,9 +588,8 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
     if (check_launch("bucket_scatter", stream, dbg)) return 1;
     {
       StageScope _t("tile_sort", stream);
-      launch_tile_sort(T, longest_for_launch, sort_limit, chunks_for_launch, (uint32_t)limits.in_registers, ranges,
-                       bucket_table, A.keys_other, A.gauss_of_emission, A.keys, A.emission, A.point_list,
-                       ahead_of_host, stream);
+      launch_tile_sort(T, longest_for_launch, sort_limit, chunks_for_launch, ranges, bucket_table, A.keys_other,
+                       A.gauss_of_emission, A.keys, A.emission, A.point_list, ahead_of_host, stream);
     }
     return check_launch("tile_sort", stream, dbg);
   };

@@ -73,7 +73,6 @@ int launch_duplicate_with_keys(int P, int W, int H, const float* means2D, const 
                                uint64_t* keys, uint32_t* values, uint32_t* emission /*optional*/,
                                hipStream_t stream);
 // ---- binning by tile: counting sort by tile + per-tile LDS sort (tile_bucket.hip) ----
-constexpr int TILE_SORT_SMALL = 2048;  // records per tile the small LDS variant holds
 constexpr int TILE_SORT_LARGE = 8192;  // longest list one workgroup sorts; longer ones are sorted in chunks and merged
 constexpr int TILE_SORT_MAX_CHUNKS = 32;  // chunks of long lists per view the merge takes; beyond: the radix sort
 int bucket_max_tiles();
@@ -90,16 +89,17 @@ int launch_bucket_count(int P, int W, int H, const int* radii, const float* mean
 const uint32_t* bucket_fits_word(const void* table, int T);
 int launch_bucket_offsets(int P, int W, int H, const uint32_t* tiles_touched, void* table, uint32_t* point_offsets,
                           hipStream_t stream);
-// also writes point_offsets (the inclusive prefix sum of tiles_touched).  ahead_of_host: the kernel checks
-// bucket_fits_word itself and does nothing if the view does not fit what it was launched for.
+// records: (depth bits << 32 | emission index) per instance, grouped by tile in any order; gauss_of_emission: the
+// Gaussian of every emission index.  Also writes point_offsets (the inclusive prefix sum of tiles_touched).
+// ahead_of_host: the kernel checks bucket_fits_word itself and does nothing if the view does not fit what it was
+// launched for.
 int launch_bucket_scatter(int P, int W, int H, const float* means2D, const float* depths,
                           const uint32_t* tiles_touched, uint32_t* point_offsets, const int* radii,
                           const uint8_t* compute_locally, void* table, const uint32_t* ranges, uint64_t* records,
                           uint32_t* gauss_of_emission, bool ahead_of_host, hipStream_t stream);
-int launch_tile_sort(int T, uint32_t longest, uint32_t limit, uint32_t chunks, uint32_t in_registers,
-                     const uint32_t* ranges, const void* table, uint64_t* records, const uint32_t* gauss_of_emission,
-                     uint64_t* keys, uint32_t* emission, uint32_t* point_list, bool ahead_of_host,
-                     hipStream_t stream);
+int launch_tile_sort(int T, uint32_t longest, uint32_t limit, uint32_t chunks, const uint32_t* ranges,
+                     const void* table, uint64_t* records, const uint32_t* gauss_of_emission, uint64_t* keys,
+                     uint32_t* emission, uint32_t* point_list, bool ahead_of_host, hipStream_t stream);
 int launch_gather_u32(int64_t n, const uint32_t* index, const uint32_t* table, uint32_t* out, hipStream_t stream);
 int launch_ssim_l1_fwd(int C, int H, int W, const float* img1, const float* img2, const uint8_t* mask,
                        float* l1_map, float* ssim_map, float* d_mu, float* d_xx, float* d_xy, hipStream_t stream);

@@ -22,7 +22,6 @@ constexpr int BK_THREADS = 1024;        // counting and scatter kernels
 constexpr int BK_MAX_BLOCKS = 256;
 constexpr int BK_MIN_PER_BLOCK = 4096;  // Gaussians per workgroup, at least
 constexpr int BK_BATCH = 4;             // Gaussians a thread loads ahead
-constexpr int TS_THREADS = 256;         // per-tile sort
 
 __host__ __device__ inline int bucket_per_block(int P) {
   // a multiple of four, so that a thread's four consecutive Gaussians start at a 16-byte boundary of every
@@ -657,60 +656,6 @@ chunk_merge_kernel(uint32_t T, const uint32_t* __restrict__ chunk_first, const u
 
 #undef GS_SORT_CASE
 
-// 3. The same sort with the records in LDS (kept as the variant the tests can force): one workgroup per tile,
-// bitonic sort of the tile's records in LDS, then the three sorted arrays the
-// rasterizer keeps: the reference's key (tile << 32 | depth bits), the emission index (the backward pass files
-// per-instance gradients under it) and the Gaussian id.  Handles lists of min_n < n <= max_n <= CAP records.
-template <int CAP>
-__global__ void __launch_bounds__(TS_THREADS)
-tile_sort_kernel(const uint32_t* __restrict__ ranges, const uint64_t* __restrict__ records,
-                 const uint32_t* __restrict__ gauss_of_emission, uint64_t* __restrict__ keys,
-                 uint32_t* __restrict__ emission, uint32_t* __restrict__ point_list, uint32_t min_n, uint32_t max_n) {
-  __shared__ uint64_t s[CAP];
-  const uint32_t t = blockIdx.x;
-  const uint32_t start = ranges[2 * t];
-  const uint32_t n = ranges[2 * t + 1] - start;
-  if (n <= min_n || n > max_n) return;
-  uint32_t m = 1;
-  while (m < n) m <<= 1;
-  for (uint32_t i = threadIdx.x; i < m; i += TS_THREADS) s[i] = i < n ? records[start + i] : ~0ull;
-  __syncthreads();
-  // Compare-exchange number idx pairs elements lo and lo + j.  A wave owns the same 64 numbers in every step
-  // (idx = thread + 256 r), and for j <= 64 those touch only the wave's own 128 elements, so such steps follow each
-  // other without a workgroup barrier; one is needed only around the steps with j >= 128.
-  for (uint32_t k = 2; k <= m; k <<= 1) {
-    for (uint32_t j = k >> 1; j > 0; j >>= 1) {
-      for (uint32_t idx = threadIdx.x; idx < (m >> 1); idx += TS_THREADS) {
-        const uint32_t lo = 2 * idx - (idx & (j - 1));
-        const uint32_t hi = lo + j;
-        const uint64_t a = s[lo], b = s[hi];
-        const bool ascending = (lo & k) == 0;
-        if ((a > b) == ascending) {
-          s[lo] = b;
-          s[hi] = a;
-        }
-      }
-      const uint32_t next_j = j > 1 ? (j >> 1) : k;  // first step of the next k is j = k (if there is one)
-      if (j >= 128 || (next_j >= 128 && (j > 1 || 2 * k <= m))) {
-        __syncthreads();
-      } else {
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-      }
-    }
-  }
-  __syncthreads();
-  const uint64_t tile_bits = (uint64_t)t << 32;
-  for (uint32_t i = threadIdx.x; i < n; i += TS_THREADS) {
-    const uint64_t rec = s[i];
-    const uint32_t e = (uint32_t)rec;
-    keys[start + i] = tile_bits | (rec >> 32);
-    emission[start + i] = e;
-    point_list[start + i] = gauss_of_emission[e];
-  }
-}
-
 }  // namespace
 
 // Tiles the LDS histograms of the counting kernels can hold.
@@ -795,34 +740,23 @@ int launch_bucket_scatter(int P, int W, int H, const float* means2D, const float
 }
 
 // Sorts every tile's segment.  `longest` is the longest list and `limit` (at most TILE_SORT_LARGE) the longest
-// one workgroup sorts whole: the register variant by default, with in_registers == 0 the LDS variants (small
-// up to TILE_SORT_SMALL, then large).  Longer lists are the `chunks` chunks that launch_bucket_count laid out
-// with the same limit: sorted in place in `records`, then merged.
-int launch_tile_sort(int T, uint32_t longest, uint32_t limit, uint32_t chunks, uint32_t in_registers,
-                     const uint32_t* ranges, const void* table, uint64_t* records, const uint32_t* gauss_of_emission,
-                     uint64_t* keys, uint32_t* emission, uint32_t* point_list, bool ahead_of_host,
-                     hipStream_t stream) {
+// one workgroup sorts whole.  Longer lists are the `chunks` chunks that launch_bucket_count laid out with the same
+// limit: sorted in place in `records`, then merged.
+int launch_tile_sort(int T, uint32_t longest, uint32_t limit, uint32_t chunks, const uint32_t* ranges,
+                     const void* table, uint64_t* records, const uint32_t* gauss_of_emission, uint64_t* keys,
+                     uint32_t* emission, uint32_t* point_list, bool ahead_of_host, hipStream_t stream) {
   if (T <= 0 || longest == 0) return 0;
   const uint32_t* fits = ahead_of_host ? bucket_fits_word(table, T) : nullptr;
   if (limit == 0 || limit > (uint32_t)TILE_SORT_LARGE) limit = TILE_SORT_LARGE;
   const uint32_t whole = longest < limit ? longest : limit;  // the longest list sorted by one workgroup
-  if (in_registers == 0) {
-    const uint32_t small_max = limit < (uint32_t)TILE_SORT_SMALL ? limit : (uint32_t)TILE_SORT_SMALL;
-    hipLaunchKernelGGL(tile_sort_kernel<TILE_SORT_SMALL>, dim3(T), dim3(TS_THREADS), 0, stream, ranges, records,
-                       gauss_of_emission, keys, emission, point_list, 0u, small_max);
-    if (whole > (uint32_t)TILE_SORT_SMALL)
-      hipLaunchKernelGGL(tile_sort_kernel<TILE_SORT_LARGE>, dim3(T), dim3(TS_THREADS), 0, stream, ranges, records,
-                         gauss_of_emission, keys, emission, point_list, (uint32_t)TILE_SORT_SMALL, limit);
-  } else {
-    uint32_t m = 256;
-    while (m < whole && m < 2048) m <<= 1;
-    hipLaunchKernelGGL(tile_sort_registers_kernel, dim3(T), dim3(256), (size_t)m * sizeof(uint64_t), stream, ranges,
-                       records, gauss_of_emission, keys, emission, point_list, limit, fits);
-    if (whole > 2048)
-      hipLaunchKernelGGL(tile_sort_registers_long_kernel, dim3(T), dim3(1024),
-                         (size_t)(whole > 4096 ? 8192 : 4096) * sizeof(uint64_t), stream, ranges, records,
-                         gauss_of_emission, keys, emission, point_list, limit, fits);
-  }
+  uint32_t m = 256;
+  while (m < whole && m < 2048) m <<= 1;
+  hipLaunchKernelGGL(tile_sort_registers_kernel, dim3(T), dim3(256), (size_t)m * sizeof(uint64_t), stream, ranges,
+                     records, gauss_of_emission, keys, emission, point_list, limit, fits);
+  if (whole > 2048)
+    hipLaunchKernelGGL(tile_sort_registers_long_kernel, dim3(T), dim3(1024),
+                       (size_t)(whole > 4096 ? 8192 : 4096) * sizeof(uint64_t), stream, ranges, records,
+                       gauss_of_emission, keys, emission, point_list, limit, fits);
   if (longest > limit && chunks > 0) {
     const uint32_t* chunk_first = (const uint32_t*)table + ((size_t)BK_MAX_BLOCKS + 1) * (size_t)T;
     hipLaunchKernelGGL(chunk_sort_kernel, dim3(chunks), dim3(1024), (size_t)(limit > 4096 ? 8192 : 4096) * sizeof(uint64_t),

@@ -170,7 +170,7 @@ def render_gaussians(background, image_height, image_width, means2D, depths, rad
                      compute_locally, viewmatrix, campos, tan_fovx, tan_fovy, all_map, render_geo, debug, args):
     """rasterize_points.cu:276-364.  Two additions: with args["max_weight_depth"] set, the per-pixel depth of the
     Gaussian that blends with the largest weight (1, H, W) is left in args["stats_collector"]["max_weight_depth"];
-    args["tile_sort_limits"] = (in_registers, large_limit, max_chunks) chooses, for this call, the way the per-tile
+    args["tile_sort_limits"] = (large_limit, max_chunks) chooses, for this call, the way the per-tile
     lists are built (all ways give the same lists).  The returned tuple is the reference's either way."""
     return render_gaussians_ex(background, image_height, image_width, means2D, depths, radii, conic_opacity, rgb,
                                compute_locally, viewmatrix, campos, tan_fovx, tan_fovy, all_map, render_geo, debug,
@@ -217,11 +217,11 @@ def render_gaussians_ex(background, image_height, image_width, means2D, depths, 
         raise RuntimeError(f"compute_locally must be a bool tensor with {tiles} elements")
     am = _f32c(all_map, "all_map") if geo else None
     want_mwd = isinstance(args, dict) and bool(args.get("max_weight_depth"))
-    # (in_registers, large_limit, max_chunks) for this call only: how the per-tile lists are built (a test hook)
+    # (large_limit, max_chunks) for this call only: how the per-tile lists are built (a test hook)
     limits = args.get("tile_sort_limits") if isinstance(args, dict) else None
     options = None
     if limits is not None or expected_instances > 0:
-        options = _n.RenderOptions(*(limits if limits is not None else (-1, -1, -1)),
+        options = _n.RenderOptions(*(limits if limits is not None else (-1, -1)),
                                    expected_instances=expected_instances,
                                    expected_longest_list=expected_longest_list)
     result = _n.RenderResult()

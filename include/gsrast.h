@@ -99,16 +99,15 @@ int gs_preprocess_backward(const int* radii, const float* cov3D, const uint8_t* 
  * merged afterwards, up to 32 chunks per view), or, when the view has more long lists than that (or the tile grid
  * more than 30000 tiles), by the reference's own route: (tile | depth) keys (rasterizer_impl.cu:74-117), one radix
  * sort over all of them (:675-684), identifyTileRanges (:122-144).  All give the same lists bit for bit.
- * tile_sort_in_registers = 0 makes the per-tile sort keep its records in LDS instead of registers (default 1);
  * tile_sort_large_limit lowers the list length that one workgroup sorts whole (default and maximum 8192; 0 = always
  * the radix route) and tile_sort_max_chunks changes the number of chunks the longer lists of a view may be cut into
  * (default 32; 0 = a longer list sends the view to the radix route), so that small scenes can exercise every
  * route.  The library keeps no such setting between calls. */
 typedef struct gs_render_options {
   uint32_t struct_bytes;
-  int32_t tile_sort_in_registers;
   int32_t tile_sort_large_limit;
   int32_t tile_sort_max_chunks;
+  int32_t expected_longest_list;
   /* What the caller expects of the view, typically the previous view's figures with a margin (0 = no idea).
    * With expected_instances > 0 (and a gs_render_result to report into) gs_render_forward does not wait for the
    * instance count before it goes on: it sizes the binning buffer for expected_instances, launches the list
@@ -117,8 +116,6 @@ typedef struct gs_render_options {
    * workgroup sorts); in that case the lists are built again the ordinary way, so the result never depends on
    * the expectation, only the time does. */
   int64_t expected_instances;
-  int32_t expected_longest_list;
-  int32_t reserved;
 } gs_render_options;
 
 /* What gs_render_forward reports besides the instance count (optional, NULL to skip; struct_bytes as above):

@@ -8,7 +8,7 @@ import torch
 pytestmark = pytest.mark.gpu
 
 DEV = "cuda:0"
-ROUTES = [(1, 8192, 32), (0, 8192, 32), (1, 0, 32), (1, 40, 1 << 30), (1, 7, 1 << 30)]
+ROUTES = [(8192, 32), (0, 32), (40, 1 << 30), (7, 1 << 30), (300, 2)]
 
 
 @pytest.fixture(scope="module")

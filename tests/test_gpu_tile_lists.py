@@ -1,6 +1,5 @@
 """The per-tile lists render_gaussians builds (ranges, sorted keys, point_list), by each of its routes: instances
-bucketed by tile and sorted per tile (in registers or in LDS; a list beyond the limit of one workgroup in chunks
-that are merged), and the radix sort over all (tile | depth) keys.  Every route must give the oracle's lists bit for bit, and the backward pass must file its per-instance
+bucketed by tile and sorted per tile (a list beyond the limit of one workgroup in chunks that are merged), and the radix sort over all (tile | depth) keys.  Every route must give the oracle's lists bit for bit, and the backward pass must file its per-instance
 gradients correctly under each."""
 import ctypes as C
 
@@ -29,11 +28,10 @@ def _mask(kind, gx, gy):
     return cl
 
 
-# (records in registers?, longest list one workgroup sorts, chunks the longer lists may be cut into): defaults; every
-# list through the LDS variants; a list too long for the per-tile sort, found after the counting pass (the radix
-# route takes over); the radix route from the start; lists beyond the limit sorted in chunks and merged (few large
-# chunks, the same behind the LDS variants, many chunks of an odd size)
-ROUTES = [(1, 8192, 32), (0, 8192, 32), (1, 40, 0), (1, 0, 32), (1, 40, 1 << 30), (0, 100, 1 << 30), (1, 7, 1 << 30)]
+# (longest list one workgroup sorts, chunks the longer lists may be cut into): defaults; a list too long for the
+# per-tile sort, found after the counting pass (the radix route takes over); the radix route from the start; lists
+# beyond the limit sorted in chunks and merged (few large chunks, more of them, many chunks of an odd size)
+ROUTES = [(8192, 32), (40, 0), (0, 32), (40, 1 << 30), (100, 1 << 30), (7, 1 << 30)]
 
 
 @pytest.mark.parametrize("cfg,P,mask", [(0, 30_000, "all"), (1, 120_000, "all"), (1, 60_000, "checker"),
@@ -60,8 +58,8 @@ def test_lists_match_oracle_by_every_route(orc, H, cfg, P, mask):
     ug = gs_scenes.upstream_grads(cam)
     args = {"stats_collector": {}}
     grads = []
-    for small, large, chunks in ROUTES:
-        args["tile_sort_limits"] = (small, large, chunks)
+    for large, chunks in ROUTES:
+        args["tile_sort_limits"] = (large, chunks)
         out = _C.render_gaussians(torch.zeros(3, device=DEV), Hh, W, o["means2D"], o["depths"], o["radii"],
                                   o["conic_opacity"], o["rgb"], cl.to(DEV), vm, cp, cam.tanfovx, cam.tanfovy, am,
                                   True, False, args)
@@ -76,9 +74,9 @@ def test_lists_match_oracle_by_every_route(orc, H, cfg, P, mask):
         gn.check(gn.lib.gs_image_state_layout(W, Hh, *[C.byref(x) for x in ioff]), "layout")
         ibase = (imgB.data_ptr() + 255) // 256 * 256 - imgB.data_ptr()
         ranges = imgB[ibase + ioff[3].value: ibase + ioff[3].value + 8 * T].view(torch.int32)
-        assert np.array_equal(H.np_u32(ranges), want["ranges"].reshape(-1)), (small, large, chunks)
-        assert np.array_equal(H.np_u32(point_list), want["point_list"]), (small, large, chunks)
-        assert np.array_equal(H.np_u64(keys), want["keys"]), (small, large, chunks)
+        assert np.array_equal(H.np_u32(ranges), want["ranges"].reshape(-1)), (large, chunks)
+        assert np.array_equal(H.np_u32(point_list), want["point_list"]), (large, chunks)
+        assert np.array_equal(H.np_u64(keys), want["keys"]), (large, chunks)
         assert np.array_equal(n(n_render), (counts[:, 1] - counts[:, 0]).astype(np.int32))
         back = _C.render_gaussians_backward(torch.zeros(3, device=DEV), cam.tanfovx, cam.tanfovy, oam, am, R, geomB,
                                             binB, imgB, cl.to(DEV), ug["color"].to(DEV), ug["all_map"].to(DEV),
@@ -119,16 +117,16 @@ def test_equal_depths_keep_emission_order(orc, H):
     want = orc.bin_and_sort(n(o["radii"]), n(o["means2D"]), n(o["depths"]), cl.numpy().reshape(-1), W, Hh)
     vm, cp = cam.world_view_transform.to(DEV), cam.camera_center.to(DEV)
     am = gs_scenes.build_all_map(gd["means3D"], gd["scales"], gd["rotations"], cam)
-    for small, large, chunks in ROUTES:
+    for large, chunks in ROUTES:
         out = _C.render_gaussians(torch.zeros(3, device=DEV), Hh, W, o["means2D"], o["depths"], o["radii"],
                                   o["conic_opacity"], o["rgb"], cl.to(DEV), vm, cp, cam.tanfovx, cam.tanfovy, am,
-                                  True, False, {"stats_collector": {}, "tile_sort_limits": (small, large, chunks)})
+                                  True, False, {"stats_collector": {}, "tile_sort_limits": (large, chunks)})
         R, binB = out[0], out[9]
         off = [C.c_size_t() for _ in range(5)]
         gn.check(gn.lib.gs_binning_state_layout(R, W, Hh, *[C.byref(x) for x in off]), "layout")
         base = (binB.data_ptr() + 255) // 256 * 256 - binB.data_ptr()
         point_list = binB[base + off[0].value: base + off[0].value + 4 * R].view(torch.int32)
-        assert np.array_equal(H.np_u32(point_list), want["point_list"]), (small, large, chunks)
+        assert np.array_equal(H.np_u32(point_list), want["point_list"]), (large, chunks)
 
 
 @pytest.mark.parametrize("P,expect", [(28_000, "waves4"), (56_000, "waves8"), (110_000, "chunks"),
@@ -157,9 +155,9 @@ def test_long_lists(orc, H, P, expect):
     assert lo < longest <= hi, longest
     limits = None
     if expect == "radix":
-        limits = (1, 8192, 0)
+        limits = (8192, 0)
     elif expect.startswith("chunks"):  # nearly every tile of this view has a long list: lift the bound on their number
-        limits = (1, 8192, 1 << 30)
+        limits = (8192, 1 << 30)
     vm, cp = cam.world_view_transform.to(DEV), cam.camera_center.to(DEV)
     am = gs_scenes.build_all_map(gd["means3D"], gd["scales"], gd["rotations"], cam)
     out = _C.render_gaussians(torch.zeros(3, device=DEV), Hh, W, o["means2D"], o["depths"], o["radii"],
@@ -216,7 +214,7 @@ def test_grid_too_large_for_the_tile_histogram(orc, H):
     assert np.array_equal(H.np_u32(point_list), want["point_list"])
 
 
-@pytest.mark.parametrize("limits", [(1, 8192, 32), (1, 0, 32)])
+@pytest.mark.parametrize("limits", [(8192, 32), (0, 32)])
 def test_more_instances_than_positions_is_an_error(H, limits):
     """1.2 M splats that each cover all 3888 tiles are 4.7e9 instances: the 32-bit prefix sums wrap around to a
     plausible count (3.7e8).  The call must fail on the exact count instead of sizing its buffers by the wrapped
@@ -275,13 +273,13 @@ def test_random_rectangles_by_every_route(orc, H, seed, W, Hh):
     co = torch.tensor([0.02, 0.0, 0.02, 0.3]).repeat(P, 1).to(DEV)
     rgb = torch.rand(P, 3, generator=gen).to(DEV)
     eye = torch.eye(4, device=DEV)
-    for small, large, chunks in ROUTES:
+    for large, chunks in ROUTES:
         out = _C.render_gaussians(torch.zeros(3, device=DEV), Hh, W, means2D.to(DEV), depths.to(DEV), radii.to(DEV),
                                   co, rgb, cl.to(DEV), eye, torch.zeros(3, device=DEV), 1.0, 1.0,
                                   torch.zeros(P, 5, device=DEV), False, False,
-                                  {"stats_collector": {}, "tile_sort_limits": (small, large, chunks)})
+                                  {"stats_collector": {}, "tile_sort_limits": (large, chunks)})
         R, binB, imgB = out[0], out[9], out[10]
-        assert R == R_want, (small, large, chunks)
+        assert R == R_want, (large, chunks)
         off = [C.c_size_t() for _ in range(5)]
         gn.check(gn.lib.gs_binning_state_layout(R, W, Hh, *[C.byref(x) for x in off]), "layout")
         base = (binB.data_ptr() + 255) // 256 * 256 - binB.data_ptr()
@@ -291,6 +289,6 @@ def test_random_rectangles_by_every_route(orc, H, seed, W, Hh):
         gn.check(gn.lib.gs_image_state_layout(W, Hh, *[C.byref(x) for x in ioff]), "layout")
         ibase = (imgB.data_ptr() + 255) // 256 * 256 - imgB.data_ptr()
         ranges = imgB[ibase + ioff[3].value: ibase + ioff[3].value + 8 * T].view(torch.int32)
-        assert np.array_equal(H.np_u32(ranges), want["ranges"].reshape(-1)), (small, large, chunks)
-        assert np.array_equal(H.np_u64(keys), want["keys"]), (small, large, chunks)
-        assert np.array_equal(H.np_u32(point_list), want["point_list"]), (small, large, chunks)
+        assert np.array_equal(H.np_u32(ranges), want["ranges"].reshape(-1)), (large, chunks)
+        assert np.array_equal(H.np_u64(keys), want["keys"]), (large, chunks)
+        assert np.array_equal(H.np_u32(point_list), want["point_list"]), (large, chunks)
