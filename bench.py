@@ -38,6 +38,21 @@ BYTES_PER_GAUSSIAN = {
 # sort_pairs: the radix sort (5 passes of 9-bit digits over 44 key bits), timed on its own on keys of the same
 # distribution: the per-tile lists are built without it unless a list exceeds 8192 records.
 BYTES_PER_INSTANCE = {"sort_pairs": 128, "identify_tile_ranges": 20, "tile_sort": 28}
+# simple-knn (distCUDA2) per point: bounding box 24 B (12 read, twice: partial and final are one pass over the
+# points plus a small second one; the survey's figure), Morton codes 16 B (12 in, 4 out), 32-bit radix sort with
+# index payload 68 B (4 B histogram read + 4 passes x (8 in + 8 out)), gather into Morton order 32 B (4 B index +
+# 12 B point in, 16 B out), box bounds 32 B (the 1024-point boxes and the 64-point leaves each read the 16 B points).
+BYTES_PER_POINT = {"knn_minmax": 24, "knn_morton": 16, "knn_sort": 68, "knn_gather": 32, "knn_boxes": 32}
+# The binning stage as a whole, in the survey's per-unit figures for the reference's algorithm on the same job:
+# per Gaussian tile count 16 + prefix sum 8 + key emission 20 B; per instance 12 B of key/value written, 152 B
+# for a radix sort with 8-bit digits over the 44 key bits, 8 B for the tile ranges.  The per-tile route here moves
+# less: per instance 12 B of records written and read once, then 16 B of sorted keys, emission indices and ids.
+BINNING_REFERENCE_BYTES = (44, 172)   # per Gaussian, per instance
+BINNING_OWN_BYTES = (44, 40)
+BINNING_STAGES = ("tile_count", "inclusive_sum", "bucket_scatter", "tile_sort", "duplicate_with_keys",
+                  "identify_tile_ranges")
+BINNING_KERNELS = ("bucket_count_kernel", "bucket_columns_kernel", "bucket_ranges_kernel", "bucket_scatter_kernel",
+                   "tile_sort_registers_kernel")
 FP32_MATRIX_PEAK_TFLOPS = 157.3
 # Neural-Gaussian generation with 10 offsets: (bytes per anchor, bytes per selected Gaussian, flops per anchor).
 #   opacity:   feat 128 + anchor 12 in; 10 opacities, 10 mask bytes, 1 count out;      2 (35*32 + 32*10) flops
@@ -256,6 +271,13 @@ def main():
                                           C.c_void_p(torch.cuda.current_stream().cuda_stream)), "gs_sort_pairs_u64")
     assert bool((s_kout[1:] >= s_kout[:-1]).all())
     del s_tiles, s_depth, s_keys, s_vals, s_kout, s_vout, s_ws
+    # simple-knn over the 1 M means of this configuration (distCUDA2, run once at initialisation by the caller)
+    from simple_knn._C import distCUDA2
+    knn_pts = leaf["means3D"].detach()
+    torch.cuda._sleep(int(4e7))
+    for _ in range(args.steps):
+        knn_out = distCUDA2(knn_pts)
+    del knn_out
     # neural-Gaussian generation for one view: 200 k visible anchors x 10 offsets through the three MLPs,
     # forward (opacity MLP, scan, color/cov MLPs + post-processing) and backward
     torch.cuda._sleep(int(4e7))
@@ -361,6 +383,8 @@ def main():
             nbytes = BYTES_PER_GAUSSIAN[name] * P
         elif name in BYTES_PER_INSTANCE:
             nbytes = BYTES_PER_INSTANCE[name] * R
+        elif name in BYTES_PER_POINT:
+            nbytes = BYTES_PER_POINT[name] * P
         elif name in ("duplicate_with_keys", "bucket_scatter"):
             nbytes = 20 * P + 12 * R
         elif name == "ssim_l1_fwd":
@@ -395,6 +419,32 @@ def main():
     roofline = {"kernel": "preprocess_fwd_kernel", "bound": "hbm", "achieved": pf.get("GBps"), "peak": HBM_PEAK_GBS,
                 "unit": "GB/s", "frac": pf.get("frac_of_hbm_peak"), "traffic": traffic,
                 "algorithmic_bytes_per_launch": pf.get("algorithmic_bytes")}
+    # The other half of the metric: everything between preprocess and the blend (count, prefix sum, per-tile
+    # lists), one figure for the stage as a whole.
+    bin_ms = sum(stage_report[k]["ms"] * stage_report[k]["launches_per_step"] for k in BINNING_STAGES
+                 if k in stage_report)
+    if "duplicate_with_keys" in stage_report and "sort_pairs" in stage_report:
+        bin_ms += stage_report["sort_pairs"]["ms"]  # (a view on the radix route: one sort of its keys as well)
+    bin_traffic = None
+    if os.path.exists(tpath):
+        try:
+            tj = json.load(open(tpath))
+            if all(k in tj for k in BINNING_KERNELS):
+                bin_traffic = sum(tj[k]["bytes_per_launch"] for k in BINNING_KERNELS)
+        except (OSError, ValueError, KeyError):
+            bin_traffic = None
+    if bin_ms > 0:
+        ref_b = BINNING_REFERENCE_BYTES[0] * P + BINNING_REFERENCE_BYTES[1] * R
+        own_b = BINNING_OWN_BYTES[0] * P + BINNING_OWN_BYTES[1] * R
+        roofline["sort"] = {
+            "kernel": "binning: " + " + ".join(BINNING_KERNELS), "bound": "hbm", "ms": round(bin_ms, 4),
+            "achieved": round(ref_b / (bin_ms * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": round(ref_b / (bin_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "traffic": bin_traffic,
+            "algorithmic_bytes_per_launch": ref_b,
+            "note": "achieved = the bytes the reference's algorithm moves for this job (44 B per Gaussian + 172 B per "
+                    "instance: 8-bit radix sort of 44-bit keys) / the time of the whole stage here",
+            "own_algorithmic_bytes_per_launch": own_b,
+            "own_achieved": round(own_b / (bin_ms * 1e-3) / 1e9, 1)}
 
     out = {
         "metric": "fwd+bwd ms/view @1M Gaussians 1152x864; preprocess+sort HBM GB/s vs peak",

@@ -82,32 +82,26 @@ struct StageClock {
 };
 static StageClock g_clock;
 
-struct StageScope {
-  hipStream_t s;
-  StageClock::Rec rec{nullptr, nullptr, nullptr};
-  StageScope(const char* name, hipStream_t stream) : s(stream) {
-    if (!g_clock.enabled.load(std::memory_order_relaxed)) return;
-    rec.name = name;
-    rec.a = g_clock.take();
-    rec.b = g_clock.take();
-    if (!rec.a || !rec.b || hipEventRecord(rec.a, s) != hipSuccess) {
-      g_clock.give_back(rec.a);
-      g_clock.give_back(rec.b);
-      rec.a = rec.b = nullptr;
-    }
+StageScope::StageScope(const char* stage, hipStream_t stream) : s(stream), name(stage) {
+  if (!g_clock.enabled.load(std::memory_order_relaxed)) return;
+  a = g_clock.take();
+  b = g_clock.take();
+  if (!a || !b || hipEventRecord(a, s) != hipSuccess) {
+    g_clock.give_back(a);
+    g_clock.give_back(b);
+    a = b = nullptr;
   }
-  ~StageScope() {
-    if (!rec.a) return;
-    if (hipEventRecord(rec.b, s) == hipSuccess) {
-      g_clock.file(rec);
-    } else {
-      g_clock.give_back(rec.a);
-      g_clock.give_back(rec.b);
-    }
+}
+
+StageScope::~StageScope() {
+  if (!a) return;
+  if (hipEventRecord(b, s) == hipSuccess) {
+    g_clock.file(StageClock::Rec{name, a, b});
+  } else {
+    g_clock.give_back(a);
+    g_clock.give_back(b);
   }
-  StageScope(const StageScope&) = delete;
-  StageScope& operator=(const StageScope&) = delete;
-};
+}
 
 namespace {
 

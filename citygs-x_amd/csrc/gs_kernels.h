@@ -37,6 +37,19 @@ struct PreprocessBwdArgs {
   float *dL_dmean3D, *dL_dcov3D /*optional*/, *dL_dsh /*optional*/, *dL_dscale, *dL_drot, *dL_dopacity /*optional*/;
 };
 
+// Brackets a stage with an event pair on its stream while stage timing is enabled (gs_stage_timing_enable; the
+// role of the reference's MyTimerOnGPU, cuda_rasterizer/timers.cu:11-79); costs one relaxed load otherwise.  The
+// pairs are read by gs_stage_timing_collect.  `stage` must be a string literal (it is kept by pointer).
+struct StageScope {
+  hipStream_t s;
+  const char* name;
+  hipEvent_t a = nullptr, b = nullptr;
+  StageScope(const char* stage, hipStream_t stream);
+  ~StageScope();
+  StageScope(const StageScope&) = delete;
+  StageScope& operator=(const StageScope&) = delete;
+};
+
 int launch_preprocess_fwd(const PreprocessFwdArgs& a, hipStream_t stream);
 int launch_preprocess_bwd(const PreprocessBwdArgs& a, hipStream_t stream);
 int launch_visible_filter(int P, const float* means, const float* scales, float mod, const float* rots,

@@ -294,21 +294,40 @@ int launch_knn_dist2(int P, const float* points, float* mean_dist2, void* temp, 
   const int blocks = (P + GS_BLOCK_1D - 1) / GS_BLOCK_1D;
   const int nboxes = (P + KNN_BOX - 1) / KNN_BOX;
 
-  hipLaunchKernelGGL(minmax_partial_kernel, dim3(MM_BLOCKS), dim3(MM_THREADS), 0, stream, P, points, partial);
-  hipLaunchKernelGGL(minmax_final_kernel, dim3(1), dim3(MM_THREADS), 0, stream, partial, minmax);
-  hipLaunchKernelGGL(morton_kernel, dim3(blocks), dim3(GS_BLOCK_1D), 0, stream, P, points, minmax, codes_a, idx_a);
+  // (the per-phase scopes only record events while stage timing is enabled)
+  {
+    StageScope _t("knn_minmax", stream);
+    hipLaunchKernelGGL(minmax_partial_kernel, dim3(MM_BLOCKS), dim3(MM_THREADS), 0, stream, P, points, partial);
+    hipLaunchKernelGGL(minmax_final_kernel, dim3(1), dim3(MM_THREADS), 0, stream, partial, minmax);
+  }
+  {
+    StageScope _t("knn_morton", stream);
+    hipLaunchKernelGGL(morton_kernel, dim3(blocks), dim3(GS_BLOCK_1D), 0, stream, P, points, minmax, codes_a, idx_a);
+  }
   const int end_bit = 32;  // 4 passes (even): the sorted pairs come back in the (a) arrays
-  if (launch_sort_pairs_u32(P, codes_a, codes_b, idx_a, idx_b, end_bit, sort_temp, stream)) return 1;
-  launch_sort_fault_report(sort_error_word(sort_temp), fault_word, stream);
+  {
+    StageScope _t("knn_sort", stream);
+    if (launch_sort_pairs_u32(P, codes_a, codes_b, idx_a, idx_b, end_bit, sort_temp, stream)) return 1;
+    launch_sort_fault_report(sort_error_word(sort_temp), fault_word, stream);
+  }
   const uint32_t* idx_sorted = sort_result_in_b(end_bit) ? idx_b : idx_a;
-  hipLaunchKernelGGL(gather_points_kernel, dim3(blocks), dim3(GS_BLOCK_1D), 0, stream, P, points, idx_sorted,
-                     sorted_pts);
-  hipLaunchKernelGGL(box_minmax_kernel, dim3(nboxes), dim3(MM_THREADS), 0, stream, P, sorted_pts, boxes);
-  hipLaunchKernelGGL(leaf_minmax_kernel, dim3(blocks), dim3(GS_BLOCK_1D), 0, stream, P, sorted_pts, leaves);
-  hipLaunchKernelGGL(box_group_kernel, dim3((nboxes + KNN_GROUP - 1) / KNN_GROUP), dim3(GS_WAVE), 0, stream, nboxes,
-                     boxes, groups);
-  hipLaunchKernelGGL(box_mean_dist_kernel, dim3(blocks), dim3(GS_BLOCK_1D), 0, stream, P, sorted_pts, idx_sorted,
-                     boxes, nboxes, groups, leaves, mean_dist2);
+  {
+    StageScope _t("knn_gather", stream);
+    hipLaunchKernelGGL(gather_points_kernel, dim3(blocks), dim3(GS_BLOCK_1D), 0, stream, P, points, idx_sorted,
+                       sorted_pts);
+  }
+  {
+    StageScope _t("knn_boxes", stream);
+    hipLaunchKernelGGL(box_minmax_kernel, dim3(nboxes), dim3(MM_THREADS), 0, stream, P, sorted_pts, boxes);
+    hipLaunchKernelGGL(leaf_minmax_kernel, dim3(blocks), dim3(GS_BLOCK_1D), 0, stream, P, sorted_pts, leaves);
+    hipLaunchKernelGGL(box_group_kernel, dim3((nboxes + KNN_GROUP - 1) / KNN_GROUP), dim3(GS_WAVE), 0, stream, nboxes,
+                       boxes, groups);
+  }
+  {
+    StageScope _t("knn_box_mean_dist", stream);
+    hipLaunchKernelGGL(box_mean_dist_kernel, dim3(blocks), dim3(GS_BLOCK_1D), 0, stream, P, sorted_pts, idx_sorted,
+                       boxes, nboxes, groups, leaves, mean_dist2);
+  }
   return 0;
 }
 
