@@ -71,6 +71,10 @@ def parse():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--config", type=int, default=1, help="BASELINE config index (1 = the headline workload)")
     ap.add_argument("--gaussians", type=int, default=None, help="override the Gaussian count (debugging only)")
+    ap.add_argument("--all-views", action="store_true",
+                    help="time the step for every camera of the configuration's batch and print one JSON object "
+                         "with a per-view list (ms per view, per-stage times, instances, longest list, route); "
+                         "the other BASELINE configurations are parity cases, this is how their figures are made")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-runs", type=int, default=3)
     ap.add_argument("--copy-calibration-mib", type=int, default=0,
@@ -116,6 +120,71 @@ FORWARD_STAGES = ("preprocess_fwd", "tile_count", "inclusive_sum", "bucket_scatt
                   "duplicate_with_keys", "identify_tile_ranges", "render_fwd")
 
 
+def all_views(args):
+    """The same step as the headline measurement, for every camera of the configuration: per view the time of
+    `steps` steps, the per-stage event times of another `steps` steps, and what the view looks like."""
+    import torch
+    import gs_scenes
+    import gsrast_native as gn
+    from diff_gaussian_rasterization import GaussianRasterizationSettings, GaussianRasterizer, _C
+    dev = "cuda:0"
+    g, cams = gs_scenes.make_scene(args.config, P=args.gaussians)
+    P = g["means3D"].shape[0]
+    leaf = {k: g[k].to(dev).requires_grad_(True) for k in ("means3D", "scales", "rotations", "opacities", "shs")}
+    per_view = []
+    for v, cam in enumerate(cams):
+        W, H = cam.image_width, cam.image_height
+        rs = GaussianRasterizationSettings(
+            image_height=H, image_width=W, tanfovx=cam.tanfovx, tanfovy=cam.tanfovy, bg=torch.zeros(3, device=dev),
+            scale_modifier=1.0, viewmatrix=cam.world_view_transform.to(dev),
+            projmatrix=cam.full_proj_transform.to(dev), sh_degree=3, campos=cam.camera_center.to(dev),
+            prefiltered=False, render_geo=True, debug=False)
+        rast = GaussianRasterizer(rs)
+        am = _C.build_all_map(leaf["means3D"].detach(), leaf["scales"].detach(), leaf["rotations"].detach(),
+                              rs.viewmatrix, rs.campos)
+        ug = {k: t.to(dev) for k, t in gs_scenes.upstream_grads(cam, seed=v).items()}
+        gx, gy = (W + 15) // 16, (H + 15) // 16
+        cl = torch.ones(gy, gx, dtype=torch.bool, device=dev)
+        m2abs = torch.zeros(P, 3, device=dev, requires_grad=True)
+        ca = {"avoid_pixel_all2all": False, "stats_collector": {}}
+        info = {}
+
+        def step():
+            for t in leaf.values():
+                t.grad = None
+            m2abs.grad = None
+            means2D, rgb, co, radii, depths = rast.preprocess_gaussians(
+                leaf["means3D"], leaf["scales"], leaf["rotations"], leaf["shs"], leaf["opacities"], ca)
+            color, n_render, _, _, _, oam, opd = rast.render_gaussians(means2D, m2abs, co, rgb, am, depths, radii, cl,
+                                                                       cl, ca)
+            torch.autograd.backward([color, oam, opd], [ug["color"], ug["all_map"], ug["plane_depth"]])
+            info["n_render"], info["radii"] = n_render, radii
+
+        for _ in range(max(args.warmup, 60 if v == 0 else 3)):
+            step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            step()
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t0) * 1e3 / args.steps
+        gn.stage_timing(True)
+        for _ in range(args.steps):
+            step()
+        torch.cuda.synchronize()
+        gn.stage_timing(False)
+        st = gn.stage_timing_collect()
+        stages = {k: round(tot / max(cnt, 1), 4) for k, (tot, cnt) in st.items()}
+        per_view.append({
+            "view": v, "image": f"{W}x{H}", "ms_per_view": round(ms, 4), "instances_R": int(info["n_render"].sum()),
+            "longest_list": int(info["n_render"].max()), "visible_gaussians": int((info["radii"] > 0).sum()),
+            "route": "radix sort over all keys" if "sort_pairs" in stages else "per-tile lists",
+            "stages_ms": stages})
+    print(json.dumps({"metric": "fwd+bwd ms/view, every camera of the batch", "config": args.config,
+                      "gaussians": P, "steps": args.steps, "n_gpus": 1, "dtype": "f32", "data": "synthetic",
+                      "per_view": per_view}))
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -130,6 +199,9 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible; the rasterizer has no CPU path", file=sys.stderr)
         sys.exit(2)
+    if args.all_views:
+        all_views(args)
+        return
     dev = "cuda:0"
     g, cams = gs_scenes.make_scene(args.config, P=args.gaussians, n_views=1)
     cam = cams[0]
