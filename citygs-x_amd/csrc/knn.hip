@@ -216,20 +216,27 @@ __device__ __forceinline__ float box_dist2(const float4& p, const float* bx) {  
   return (diff[0] * diff[0] + diff[1] * diff[1]) + diff[2] * diff[2];
 }
 
-__device__ __forceinline__ void update3(const float4& ref, const float4& p, float* knn) {  // simple_knn.cu:131-145
+// Keeps the three smallest of {knn[0..2], dist(ref, p)} in ascending order (simple_knn.cu:131-145 inserts by
+// compare-and-swap; the minimum / maximum form leaves the same three values).  A NaN distance (a point with a NaN
+// coordinate) is never inserted, as with the reference's `knn[j] > dist`.
+__device__ __forceinline__ void update3(const float4& ref, const float4& p, float* knn) {
   const float dx = p.x - ref.x, dy = p.y - ref.y, dz = p.z - ref.z;
   float dist = (dx * dx + dy * dy) + dz * dz;
-#pragma unroll
-  for (int j = 0; j < 3; j++) {
-    if (knn[j] > dist) {
-      const float t = knn[j];
-      knn[j] = dist;
-      dist = t;
-    }
-  }
+  dist = dist == dist ? dist : FLT_MAX;
+  const float a0 = fminf(knn[0], dist), r0 = fmaxf(knn[0], dist);
+  const float a1 = fminf(knn[1], r0), r1 = fmaxf(knn[1], r0);
+  knn[0] = a0;
+  knn[1] = a1;
+  knn[2] = fminf(knn[2], r1);
 }
 
-// simple-knn/simple_knn.cu:147-183.
+// simple-knn/simple_knn.cu:147-183.  The reference seeds a rejection radius from the three nearest of a point's six
+// neighbours in Morton order and then walks all boxes, skipping those farther away than that radius or than the
+// third-best distance so far.  Here a point first looks at the other points of its own 64-point leaf (its nearest
+// neighbours in Morton order, and the same leaf for every lane of a wave), which makes the third-best distance a
+// tight bound from the start, and then walks groups of boxes, boxes and leaves with the reference's test
+// (simple_knn.cu:161-171) against that bound.  The search is exhaustive within a bound that only ever shrinks to a
+// distance actually found, so the three distances are those of a brute-force search whatever the order.
 __global__ void __launch_bounds__(GS_BLOCK_1D) box_mean_dist_kernel(int P, const float4* __restrict__ sorted_pts,
                                                                     const uint32_t* __restrict__ idx,
                                                                     const float* __restrict__ boxes, int nboxes,
@@ -240,31 +247,37 @@ __global__ void __launch_bounds__(GS_BLOCK_1D) box_mean_dist_kernel(int P, const
   if (k >= P) return;
   const float4 p = sorted_pts[k];
   float best[3] = {FLT_MAX, FLT_MAX, FLT_MAX};
-  const int lo = max(0, k - 3), hi = min(P - 1, k + 3);
-  for (int i = lo; i <= hi; i++) {
-    if (i == k) continue;
-    update3(p, sorted_pts[i], best);
+  const int own = k / KNN_LEAF;
+  {
+    const int l0 = own * KNN_LEAF, le = min(P, l0 + KNN_LEAF);
+    for (int i = l0; i < le; i++) {
+      // (the point itself would contribute distance 0)
+      const float4 q = sorted_pts[i];
+      float keep[3] = {best[0], best[1], best[2]};
+      update3(p, q, best);
+      if (i == k) {
+        best[0] = keep[0];
+        best[1] = keep[1];
+        best[2] = keep[2];
+      }
+    }
   }
-  const float reject = best[2];
-  best[0] = best[1] = best[2] = FLT_MAX;
   const int ngroups = (nboxes + KNN_GROUP - 1) / KNN_GROUP;
   for (int gi = 0; gi < ngroups; gi++) {
     // a group that is too far away holds no box that is near enough
     const float gd = box_dist2(p, groups + 6 * gi);
-    if (gd > reject || gd > best[2]) continue;
+    if (gd > best[2]) continue;
     const int b_end = min(nboxes, (gi + 1) * KNN_GROUP);
     for (int b = gi * KNN_GROUP; b < b_end; b++) {
       const float dist = box_dist2(p, boxes + 6 * b);
-      if (dist > reject || dist > best[2]) continue;
+      if (dist > best[2]) continue;
       const int e = min(P, (b + 1) * KNN_BOX);
       for (int l0 = b * KNN_BOX; l0 < e; l0 += KNN_LEAF) {
+        if (l0 / KNN_LEAF == own) continue;
         const float ld = box_dist2(p, leaves + 6 * (size_t)(l0 / KNN_LEAF));
-        if (ld > reject || ld > best[2]) continue;
+        if (ld > best[2]) continue;
         const int le = min(e, l0 + KNN_LEAF);
-        for (int i = l0; i < le; i++) {
-          if (i == k) continue;
-          update3(p, sorted_pts[i], best);
-        }
+        for (int i = l0; i < le; i++) update3(p, sorted_pts[i], best);
       }
     }
   }

@@ -61,10 +61,24 @@ def test_random_views_match_oracle(orc, H, block):
             bg = torch.tensor(rng.random(3), dtype=torch.float32, device=DEV)
             args = {"stats_collector": {}, "tile_sort_limits": route}
             vm, pm, cp = cam.world_view_transform.to(DEV), cam.full_proj_transform.to(DEV), cam.camera_center.to(DEV)
-            out = _C.render_gaussians(bg, Hh, W, o["means2D"], o["depths"], o["radii"], o["conic_opacity"], o["rgb"],
-                                      cl.to(DEV), vm, cp, cam.tanfovx, cam.tanfovy, am, geo, False, args)
+            # what the caller says it expects of the view: nothing, enough, too little, or exactly right (the list
+            # kernels and the blend are then launched ahead of the instance count, and redone if the view does not fit)
+            R_want = int(want["point_list"].shape[0])
+            counts = want["ranges"].reshape(-1, 2).astype(np.int64)
+            longest_want = int((counts[:, 1] - counts[:, 0]).max())
+            expect = str(rng.choice(["none", "enough", "too few", "exact", "list too long"]))
+            exp_n, exp_l = {"none": (0, 0), "enough": (R_want + int(rng.integers(1, 5000)), 0),
+                            "too few": (max(1, R_want // 2), 0), "exact": (max(1, R_want), longest_want),
+                            "list too long": (R_want + 7, max(1, longest_want // 2))}[expect]
+            tag += f" expect {expect}"
+            out, info = _C.render_gaussians_ex(bg, Hh, W, o["means2D"], o["depths"], o["radii"], o["conic_opacity"],
+                                               o["rgb"], cl.to(DEV), vm, cp, cam.tanfovx, cam.tanfovy, am, geo, False,
+                                               args, expected_instances=exp_n, expected_longest_list=exp_l)
             R, color, n_render, n_consider, n_contrib, obs, oam, opd, geomB, binB, imgB = out
-            assert R == want["point_list"].shape[0], tag
+            assert R == R_want, tag
+            assert info["binning_capacity"] == (exp_n if info["launched_ahead"] else R), tag
+            if exp_n == 0 or exp_n < R_want or 0 < exp_l < longest_want:
+                assert not info["launched_ahead"], tag
             rendered += R > 0
             f = orc.render_fwd(want["ranges"], want["point_list"], ref["means2D"], ref["rgb"], n(am),
                                ref["conic_opacity"], clf, n(bg), W, Hh, cam.tanfovx, cam.tanfovy, render_geo=geo)
@@ -97,7 +111,7 @@ def test_random_views_match_oracle(orc, H, block):
             back = _C.render_gaussians_backward(bg, cam.tanfovx, cam.tanfovy, oam, am, R, geomB, binB, imgB,
                                                 cl.to(DEV), ug["color"].to(DEV), ug["all_map"].to(DEV),
                                                 gdep.to(DEV), o["means2D"], o["conic_opacity"], o["rgb"], geo, False,
-                                                args)
+                                                args, binning_capacity=info["binning_capacity"])
             rb = orc.render_bwd(want["ranges"], want["point_list"], ref["means2D"], ref["conic_opacity"], ref["rgb"],
                                 n(am), f["out_all_map"], f["final_T"], f["n_contrib"], clf, n(bg), n(ug["color"]),
                                 n(ug["all_map"]), n(gdep), W, Hh, cam.tanfovx, cam.tanfovy, render_geo=geo)
