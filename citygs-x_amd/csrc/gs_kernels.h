@@ -85,7 +85,7 @@ int launch_duplicate_with_keys(int P, int W, int H, const float* means2D, const 
                                const uint32_t* offsets, const int* radii, const uint8_t* compute_locally,
                                uint64_t* keys, uint32_t* values, uint32_t* emission /*optional*/,
                                hipStream_t stream);
-// ---- binning by tile: counting sort by tile + per-tile LDS sort (tile_bucket.hip) ----
+// ---- binning by tile: counting sort by tile + per-tile register sort (tile_bucket.hip) ----
 constexpr int TILE_SORT_LARGE = 8192;  // longest list one workgroup sorts; longer ones are sorted in chunks and merged
 constexpr int TILE_SORT_MAX_CHUNKS = 32;  // chunks of long lists per view the merge takes; beyond: the radix sort
 int bucket_max_tiles();

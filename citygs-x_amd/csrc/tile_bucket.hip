@@ -4,7 +4,7 @@
 // and every tile's list is short, so the same list comes out of
 //   1. a counting sort by tile: per-workgroup tile histograms in LDS, a prefix over workgroups and tiles (which
 //      is also the table of tile ranges), and a scatter of every instance into its tile's segment, in any order;
-//   2. one workgroup per tile sorting its segment in LDS by (depth bits, emission index): the emission index
+//   2. one workgroup per tile sorting its segment in registers by (depth bits, emission index): the emission index
 //      is unique, so the order does not depend on how the scatter happened to fill the segment, and it is the
 //      order a stable sort on the depth bits would leave.
 // No pass over all instances per digit, no look-back chain.  A list longer than one workgroup sorts is cut into
