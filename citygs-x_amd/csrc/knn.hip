@@ -16,11 +16,12 @@ namespace {
 constexpr int KNN_BOX = 1024;  // simple-knn/simple_knn.cu:12
 constexpr int KNN_GROUP = 64;  // boxes per group (one group test replaces this many box tests)
 constexpr int KNN_LEAF = 64;   // points per leaf box inside a box (one leaf test replaces this many distances)
+constexpr int KNN_TWIG = 16;   // points per twig box inside a leaf (the finest level)
 constexpr int MM_BLOCKS = 512;
 constexpr int MM_THREADS = 256;
 
 struct KnnLayout {
-  size_t partial, minmax, codes_a, codes_b, idx_a, idx_b, sorted_pts, boxes, groups, leaves, sort_temp, total;
+  size_t partial, minmax, codes_a, codes_b, idx_a, idx_b, sorted_pts, boxes, groups, leaves, twigs, sort_temp, total;
 };
 
 KnnLayout knn_layout(int P) {
@@ -42,6 +43,7 @@ KnnLayout knn_layout(int P) {
   L.sorted_pts = take(sizeof(float4) * n);
   L.boxes = take(sizeof(float) * 6 * nb);
   L.leaves = take(sizeof(float) * 6 * ((n + KNN_LEAF - 1) / KNN_LEAF));
+  L.twigs = take(sizeof(float) * 6 * ((n + KNN_TWIG - 1) / KNN_TWIG));
   L.groups = take(sizeof(float) * 6 * ((nb + KNN_GROUP - 1) / KNN_GROUP));
   L.sort_temp = take(sort_temp_bytes((int64_t)n));
   L.total = off;
@@ -182,10 +184,13 @@ __global__ void __launch_bounds__(GS_WAVE) box_group_kernel(int nboxes, const fl
   }
 }
 
-// Bounding box of every run of KNN_LEAF consecutive sorted points (one wave each): the finest level of the
-// search.  Like the groups, an addition that prunes work without changing which neighbours are found.
+// Bounding box of every run of KNN_LEAF consecutive sorted points (one wave each) and, inside it, of every run
+// of KNN_TWIG points (a 16-lane row each): the two finest levels of the search.  Like the groups, additions that
+// prune work without changing which neighbours are found.
 __global__ void __launch_bounds__(GS_BLOCK_1D) leaf_minmax_kernel(int P, const float4* __restrict__ sorted_pts,
-                                                                  float* __restrict__ leaves) {
+                                                                  float* __restrict__ leaves,
+                                                                  float* __restrict__ twigs) {
+  static_assert(KNN_LEAF == GS_WAVE && KNN_TWIG == 16, "a leaf is a wave, a twig a row of 16 lanes");
   const int i = blockIdx.x * GS_BLOCK_1D + threadIdx.x;
   float v[6] = {FLT_MAX, FLT_MAX, FLT_MAX, -FLT_MAX, -FLT_MAX, -FLT_MAX};
   if (i < P) {
@@ -193,11 +198,18 @@ __global__ void __launch_bounds__(GS_BLOCK_1D) leaf_minmax_kernel(int P, const f
     v[0] = v[3] = p.x; v[1] = v[4] = p.y; v[2] = v[5] = p.z;
   }
 #pragma unroll
-  for (int d = GS_WAVE / 2; d >= 1; d >>= 1) {
+  for (int d = 1; d < GS_WAVE; d <<= 1) {
 #pragma unroll
     for (int c = 0; c < 3; c++) {
       v[c] = fminf(v[c], __shfl_xor(v[c], d, GS_WAVE));
       v[3 + c] = fmaxf(v[3 + c], __shfl_xor(v[3 + c], d, GS_WAVE));
+    }
+    if (d == KNN_TWIG / 2) {
+      const int twig = i / KNN_TWIG;
+      if ((threadIdx.x & (KNN_TWIG - 1)) == 0 && twig * KNN_TWIG < P) {
+#pragma unroll
+        for (int c = 0; c < 6; c++) twigs[6 * (size_t)twig + c] = v[c];
+      }
     }
   }
   const int leaf = i / KNN_LEAF;
@@ -234,7 +246,7 @@ __device__ __forceinline__ void update3(const float4& ref, const float4& p, floa
 // neighbours in Morton order and then walks all boxes, skipping those farther away than that radius or than the
 // third-best distance so far.  Here a point first looks at the other points of its own 64-point leaf (its nearest
 // neighbours in Morton order, and the same leaf for every lane of a wave), which makes the third-best distance a
-// tight bound from the start, and then walks groups of boxes, boxes and leaves with the reference's test
+// tight bound from the start, and then walks groups of boxes, boxes, leaves and 16-point twigs with the reference's test
 // (simple_knn.cu:161-171) against that bound.  The search is exhaustive within a bound that only ever shrinks to a
 // distance actually found, so the three distances are those of a brute-force search whatever the order.
 __global__ void __launch_bounds__(GS_BLOCK_1D) box_mean_dist_kernel(int P, const float4* __restrict__ sorted_pts,
@@ -242,6 +254,7 @@ __global__ void __launch_bounds__(GS_BLOCK_1D) box_mean_dist_kernel(int P, const
                                                                     const float* __restrict__ boxes, int nboxes,
                                                                     const float* __restrict__ groups,
                                                                     const float* __restrict__ leaves,
+                                                                    const float* __restrict__ twigs,
                                                                     float* __restrict__ out) {
   const int k = blockIdx.x * GS_BLOCK_1D + threadIdx.x;
   if (k >= P) return;
@@ -277,7 +290,12 @@ __global__ void __launch_bounds__(GS_BLOCK_1D) box_mean_dist_kernel(int P, const
         const float ld = box_dist2(p, leaves + 6 * (size_t)(l0 / KNN_LEAF));
         if (ld > best[2]) continue;
         const int le = min(e, l0 + KNN_LEAF);
-        for (int i = l0; i < le; i++) update3(p, sorted_pts[i], best);
+        for (int t0 = l0; t0 < le; t0 += KNN_TWIG) {
+          const float td = box_dist2(p, twigs + 6 * (size_t)(t0 / KNN_TWIG));
+          if (td > best[2]) continue;
+          const int te = min(le, t0 + KNN_TWIG);
+          for (int i = t0; i < te; i++) update3(p, sorted_pts[i], best);
+        }
       }
     }
   }
@@ -303,6 +321,7 @@ int launch_knn_dist2(int P, const float* points, float* mean_dist2, void* temp, 
   float* boxes = (float*)(base + L.boxes);
   float* groups = (float*)(base + L.groups);
   float* leaves = (float*)(base + L.leaves);
+  float* twigs = (float*)(base + L.twigs);
   void* sort_temp = base + L.sort_temp;
   const int blocks = (P + GS_BLOCK_1D - 1) / GS_BLOCK_1D;
   const int nboxes = (P + KNN_BOX - 1) / KNN_BOX;
@@ -332,14 +351,14 @@ int launch_knn_dist2(int P, const float* points, float* mean_dist2, void* temp, 
   {
     StageScope _t("knn_boxes", stream);
     hipLaunchKernelGGL(box_minmax_kernel, dim3(nboxes), dim3(MM_THREADS), 0, stream, P, sorted_pts, boxes);
-    hipLaunchKernelGGL(leaf_minmax_kernel, dim3(blocks), dim3(GS_BLOCK_1D), 0, stream, P, sorted_pts, leaves);
+    hipLaunchKernelGGL(leaf_minmax_kernel, dim3(blocks), dim3(GS_BLOCK_1D), 0, stream, P, sorted_pts, leaves, twigs);
     hipLaunchKernelGGL(box_group_kernel, dim3((nboxes + KNN_GROUP - 1) / KNN_GROUP), dim3(GS_WAVE), 0, stream, nboxes,
                        boxes, groups);
   }
   {
     StageScope _t("knn_box_mean_dist", stream);
     hipLaunchKernelGGL(box_mean_dist_kernel, dim3(blocks), dim3(GS_BLOCK_1D), 0, stream, P, sorted_pts, idx_sorted,
-                       boxes, nboxes, groups, leaves, mean_dist2);
+                       boxes, nboxes, groups, leaves, twigs, mean_dist2);
   }
   return 0;
 }
