@@ -260,7 +260,11 @@ __global__ void __launch_bounds__(GS_BLOCK_1D) box_mean_dist_kernel(int P, const
   if (k >= P) return;
   const float4 p = sorted_pts[k];
   float best[3] = {FLT_MAX, FLT_MAX, FLT_MAX};
-  const int own = k / KNN_LEAF;
+  // The lanes of a wave are the points of one leaf, so they walk the tree together: a node is opened when any
+  // lane is within its bound of it, which keeps the walk's control flow and the loads of nodes and points
+  // wave-uniform.  A lane then also sees points that its own test would have skipped; update3 only ever inserts
+  // true distances, so that changes nothing.
+  const int own = __builtin_amdgcn_readfirstlane(k / KNN_LEAF);
   {
     const int l0 = own * KNN_LEAF, le = min(P, l0 + KNN_LEAF);
     for (int i = l0; i < le; i++) {
@@ -279,20 +283,20 @@ __global__ void __launch_bounds__(GS_BLOCK_1D) box_mean_dist_kernel(int P, const
   for (int gi = 0; gi < ngroups; gi++) {
     // a group that is too far away holds no box that is near enough
     const float gd = box_dist2(p, groups + 6 * gi);
-    if (gd > best[2]) continue;
+    if (!__any(!(gd > best[2]))) continue;
     const int b_end = min(nboxes, (gi + 1) * KNN_GROUP);
     for (int b = gi * KNN_GROUP; b < b_end; b++) {
       const float dist = box_dist2(p, boxes + 6 * b);
-      if (dist > best[2]) continue;
+      if (!__any(!(dist > best[2]))) continue;
       const int e = min(P, (b + 1) * KNN_BOX);
       for (int l0 = b * KNN_BOX; l0 < e; l0 += KNN_LEAF) {
         if (l0 / KNN_LEAF == own) continue;
         const float ld = box_dist2(p, leaves + 6 * (size_t)(l0 / KNN_LEAF));
-        if (ld > best[2]) continue;
+        if (!__any(!(ld > best[2]))) continue;
         const int le = min(e, l0 + KNN_LEAF);
         for (int t0 = l0; t0 < le; t0 += KNN_TWIG) {
           const float td = box_dist2(p, twigs + 6 * (size_t)(t0 / KNN_TWIG));
-          if (td > best[2]) continue;
+          if (!__any(!(td > best[2]))) continue;
           const int te = min(le, t0 + KNN_TWIG);
           for (int i = t0; i < te; i++) update3(p, sorted_pts[i], best);
         }

@@ -462,3 +462,49 @@ def test_side_stream_gives_the_same_results():
     # gradients too: every sum of the backward pass is taken in a fixed order (no float atomics anywhere)
     for i, (a, b) in enumerate(zip(base, got)):
         assert torch.equal(a, b), i
+
+
+def test_views_in_flight_on_two_streams_give_the_same_results():
+    """A batch's views alternate between two streams (default priority), so that one view's bandwidth-bound
+    stages run beside the other's blend kernels: every view's outputs and gradients are the bits of the same
+    view rendered alone."""
+    import gs_scenes
+    from diff_gaussian_rasterization import GaussianRasterizer
+    g, cams = gs_scenes.make_scene(2, P=200_000, n_views=4)
+    W, H = cams[0].image_width, cams[0].image_height
+    gx, gy = (W + 15) // 16, (H + 15) // 16
+    cl = torch.ones(gy, gx, dtype=torch.bool, device=DEV)
+    ugs = [{k: v.to(DEV) for k, v in gs_scenes.upstream_grads(c, seed=i).items()} for i, c in enumerate(cams)]
+    dev = {k: g[k].to(DEV) for k in ("means3D", "scales", "rotations", "opacities", "shs")}
+    ams = [gs_scenes.build_all_map(g["means3D"], g["scales"], g["rotations"], c).to(DEV) for c in cams]
+    torch.cuda.synchronize()
+
+    def run(v):
+        rast = GaussianRasterizer(_settings(cams[v]))
+        leaf = {k: t.clone().requires_grad_(True) for k, t in dev.items()}
+        args = _cuda_args()
+        means2D, rgb, co, radii, depths = rast.preprocess_gaussians(
+            leaf["means3D"], leaf["scales"], leaf["rotations"], leaf["shs"], leaf["opacities"], args)
+        m2abs = torch.zeros_like(leaf["means3D"], requires_grad=True) + 0
+        color, n_render, n_consider, n_contrib, obs, oam, opd = rast.render_gaussians(
+            means2D, m2abs, co, rgb, ams[v], depths, radii, cl, cl, args)
+        torch.autograd.backward([color, oam, opd], [ugs[v]["color"], ugs[v]["all_map"], ugs[v]["plane_depth"]])
+        return [color, n_render, n_consider, n_contrib, obs, oam, opd] + [leaf[k].grad for k in sorted(leaf)]
+
+    alone = []
+    for v in range(len(cams)):
+        alone.append(run(v))
+        torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    for s in streams:
+        s.wait_stream(torch.cuda.current_stream())
+    together = []
+    for rep in range(3):  # twelve views, at most two in flight
+        for v in range(len(cams)):
+            with torch.cuda.stream(streams[v % 2]):
+                together.append((v, run(v)))
+    for s in streams:
+        s.synchronize()
+    for v, got in together:
+        for i, (a, b) in enumerate(zip(alone[v], got)):
+            assert torch.equal(a, b), (v, i)
