@@ -85,6 +85,53 @@ def test_knn_dist2(H, orc, P, kind):
         np.testing.assert_allclose(got, _brute(pts), rtol=2e-4, atol=1e-9)
 
 
+def _brute_f32(pts):
+    """The three smallest squared distances of every point in float32 with the kernel's association,
+    ((dx*dx + dy*dy) + dz*dz), and their mean ((a + b) + c) / 3: what any exact search must return, bit for bit.
+    Distances that are not finite count as FLT_MAX, which is also what three missing neighbours read as."""
+    big = np.float32(np.finfo(np.float32).max)
+    out = np.empty(len(pts), np.float32)
+    with np.errstate(all="ignore"):
+        for i, p in enumerate(pts):
+            d = pts - p
+            d2 = (d[:, 0] * d[:, 0] + d[:, 1] * d[:, 1]) + d[:, 2] * d[:, 2]
+            d2 = np.where(np.isnan(d2), big, np.minimum(d2, big)).astype(np.float32)
+            d2[i] = big
+            k = np.sort(np.concatenate([d2, np.full(3, big, np.float32)]))[:3]
+            out[i] = ((k[0] + k[1]) + k[2]) / np.float32(3.0)
+    return out
+
+
+@pytest.mark.parametrize("case", ["one", "two", "three", "four", "63", "64", "65", "129", "identical", "duplicates",
+                                  "line", "plane", "nan_and_inf", "far_outliers", "two_clusters", "2500"])
+def test_knn_edge_cases_match_a_float32_brute_force(H, orc, case):
+    import simple_knn._C as knn
+    rng = np.random.default_rng(len(case) * 7 + ord(case[0]))
+    n = {"one": 1, "two": 2, "three": 3, "four": 4}.get(case, int(case) if case.isdigit() else 1500)
+    pts = rng.uniform(-5, 5, (n, 3)).astype(np.float32)
+    if case == "identical":
+        pts[:] = pts[0]
+    elif case == "duplicates":
+        pts = pts[rng.integers(0, 40, n)]
+    elif case == "line":
+        pts[:, 1:] = 0.25
+    elif case == "plane":
+        pts[:, 2] = -3.0
+    elif case == "nan_and_inf":
+        pts[rng.integers(0, n, 20), rng.integers(0, 3, 20)] = np.nan
+        pts[rng.integers(0, n, 10), rng.integers(0, 3, 10)] = np.inf
+        pts[rng.integers(0, n, 10), rng.integers(0, 3, 10)] = -np.inf
+    elif case == "far_outliers":
+        pts[::97] *= 1.0e6
+    elif case == "two_clusters":
+        pts[: n // 2] = pts[: n // 2] * 1e-3 + 1.0e4
+    got = knn.distCUDA2(torch.from_numpy(pts).to(H.DEV)).cpu().numpy()
+    want = _brute_f32(pts)
+    assert np.array_equal(got, want, equal_nan=True), np.nonzero(got != want)[0][:10]
+    if case not in ("nan_and_inf",):  # (the CPU statement's grid is undefined for non-finite bounds)
+        assert np.array_equal(got, orc.knn_dist2(pts))
+
+
 def test_cross_lane_reductions(H):
     rng = np.random.default_rng(0)
     x = rng.integers(-8, 9, (64, 16)).astype(np.float32)  # small integers: sums are exact in any order
