@@ -39,8 +39,8 @@ BYTES_PER_GAUSSIAN = {
 # distribution: the per-tile lists are built without it unless a list exceeds 8192 records.
 BYTES_PER_INSTANCE = {"sort_pairs": 128, "identify_tile_ranges": 20, "tile_sort": 28}
 # simple-knn (distCUDA2) per point: bounding box 24 B (12 read, twice: partial and final are one pass over the
-# points plus a small second one; the survey's figure), Morton codes 16 B (12 in, 4 out), 32-bit radix sort with
-# index payload 68 B (4 B histogram read + 4 passes x (8 in + 8 out)), gather into Morton order 32 B (4 B index +
+# points plus a small second one; the survey's figure), curve keys 16 B (12 in, 4 out), 32-bit radix sort with
+# index payload 68 B (4 B histogram read + 4 passes x (8 in + 8 out)), gather into sorted order 32 B (4 B index +
 # 12 B point in, 16 B out), box bounds 32 B (the 1024-point boxes and the 64-point leaves each read the 16 B points).
 BYTES_PER_POINT = {"knn_minmax": 24, "knn_keys": 16, "knn_sort": 68, "knn_gather": 32, "knn_boxes": 32}
 # The binning stage as a whole, in the survey's per-unit figures for the reference's algorithm on the same job:
@@ -76,6 +76,9 @@ def parse():
                          "with a per-view list (ms per view, per-stage times, instances, longest list, route); "
                          "the other BASELINE configurations are parity cases, this is how their figures are made")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-views-in-flight", action="store_true",
+                    help="skip the supplementary measurement with two views in flight on two streams (profiling "
+                         "runs: kernels that overlap there would blur the per-kernel averages)")
     ap.add_argument("--cpu-runs", type=int, default=3)
     ap.add_argument("--copy-calibration-mib", type=int, default=0,
                     help="also run three plain device-to-device copies of this many MiB after the timed regions: "
@@ -269,26 +272,28 @@ def main():
     # Not `value`: the same steps with two views in flight, alternating between two streams (default priority)
     # as a caller would run the views of a batch, so that one view's bandwidth-bound stages overlap the other's
     # blend kernels.  Every view has its own parameter copies here because each step resets and refills `.grad`.
-    leaf_b = {k: v.detach().clone().requires_grad_(True) for k, v in leaf.items()}
-    m2abs_b = torch.zeros(P, 3, device=dev, requires_grad=True)
-    lanes = [(torch.cuda.Stream(), leaf, m2abs), (torch.cuda.Stream(), leaf_b, m2abs_b)]
-    for s_, _, _ in lanes:
-        s_.wait_stream(torch.cuda.current_stream())
-
-    def in_flight(n):
-        for i in range(n):
-            s_, lf, m2 = lanes[i % 2]
-            with torch.cuda.stream(s_):
-                step(lf, m2)
+    ms_per_view_two_in_flight = None
+    if not args.no_views_in_flight:
+        leaf_b = {k: v.detach().clone().requires_grad_(True) for k, v in leaf.items()}
+        m2abs_b = torch.zeros(P, 3, device=dev, requires_grad=True)
+        lanes = [(torch.cuda.Stream(), leaf, m2abs), (torch.cuda.Stream(), leaf_b, m2abs_b)]
         for s_, _, _ in lanes:
-            s_.synchronize()
+            s_.wait_stream(torch.cuda.current_stream())
 
-    in_flight(max(2, args.warmup))
-    t0b = time.perf_counter()
-    in_flight(args.steps)
-    ms_per_view_two_in_flight = (time.perf_counter() - t0b) * 1e3 / args.steps
-    torch.cuda.synchronize()
-    del leaf_b, m2abs_b, lanes
+        def in_flight(n):
+            for i in range(n):
+                s_, lf, m2 = lanes[i % 2]
+                with torch.cuda.stream(s_):
+                    step(lf, m2)
+            for s_, _, _ in lanes:
+                s_.synchronize()
+
+        in_flight(max(2, args.warmup))
+        t0b = time.perf_counter()
+        in_flight(args.steps)
+        ms_per_view_two_in_flight = (time.perf_counter() - t0b) * 1e3 / args.steps
+        torch.cuda.synchronize()
+        del leaf_b, m2abs_b, lanes
     # the same `steps` steps again with an event pair around every stage on its stream: the per-kernel
     # durations below come from this region (the event records cost a few microseconds of idle time between
     # kernels, which is why `value` is taken from the region above)
@@ -558,7 +563,8 @@ def main():
                                         and "sort_pairs" in stage_report else 0.0), 4),
         "roofline": roofline,
         # two views in flight on two streams (how the views of a batch can be issued); `value` is one view at a time
-        "ms_per_view_two_views_in_flight": round(ms_per_view_two_in_flight, 4),
+        "ms_per_view_two_views_in_flight": (round(ms_per_view_two_in_flight, 4)
+                                            if ms_per_view_two_in_flight is not None else None),
         "ms_per_step_with_stage_events": round(ms_per_step_instrumented, 4),
         "stages": stage_report,
         "ssim_l1_torch_reference_ms": round(sorted(torch_ssim_ms)[len(torch_ssim_ms) // 2], 4),
