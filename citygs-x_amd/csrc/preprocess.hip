@@ -175,6 +175,82 @@ __device__ __forceinline__ void wave_sync_lds() {
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
+// The same evaluation, one coefficient at a time: B[k] is everything of term k but the coefficient (the products
+// in sh_channel associate from the left, so term k = B[k] * c[k] is the same rounding), and sh_accumulate<K> is
+// the step of the running sum that takes in coefficient K.  Coefficients of degrees above `deg` are left out.
+__device__ __forceinline__ void sh_basis(float x, float y, float z, float* B) {
+  const float xx = x * x, yy = y * y, zz = z * z, xy = x * y, yz = y * z, xz = x * z;
+  B[0] = kC0;
+  B[1] = kC1 * y;
+  B[2] = kC1 * z;
+  B[3] = kC1 * x;
+  B[4] = kC2[0] * xy;
+  B[5] = kC2[1] * yz;
+  B[6] = kC2[2] * (2.0f * zz - xx - yy);
+  B[7] = kC2[3] * xz;
+  B[8] = kC2[4] * (xx - yy);
+  B[9] = kC3[0] * y * (3.0f * xx - yy);
+  B[10] = kC3[1] * xy * z;
+  B[11] = kC3[2] * y * (4.0f * zz - xx - yy);
+  B[12] = kC3[3] * z * (2.0f * zz - 3.0f * xx - 3.0f * yy);
+  B[13] = kC3[4] * x * (4.0f * zz - xx - yy);
+  B[14] = kC3[5] * z * (xx - yy);
+  B[15] = kC3[6] * x * (xx - 3.0f * yy);
+}
+
+template <int K>
+__device__ __forceinline__ float sh_accumulate(int deg, float res, const float* B, float c) {
+  constexpr int degree_of = K == 0 ? 0 : K < 4 ? 1 : K < 9 ? 2 : 3;
+  if (deg < degree_of) return res;
+  if (K == 0) return B[0] * c;
+  if (K == 1 || K == 3) return res - B[K] * c;
+  return res + B[K] * c;
+}
+
+// The 192-byte SH rows of a wave's 64 Gaussians, a third at a time: the 64-byte thirds of all rows are fetched with
+// whole-wave 16-byte loads (four lanes share a 64-byte line and use all of it), parked in LDS (rows of four 16-byte
+// words padded to five, which keeps both access patterns free of bank conflicts) and read back row-wise, a lane its
+// own 16 floats, which it folds into the three running sums before the next third arrives.  A lane that loads its
+// own row directly issues twelve 16-byte loads 192 bytes apart from its neighbours': every line then passes through
+// the first-level cache four times.
+constexpr int SH_THIRD4 = 5;
+
+template <int PHASE>
+__device__ __forceinline__ void sh_third_fetch(const float4* __restrict__ wave_rows, uint64_t need, int lane,
+                                               float4* v) {
+#pragma unroll
+  for (int j = 0; j < 4; j++) {
+    const int idx = j * GS_WAVE + lane, row = idx >> 2, part = idx & 3;
+    v[j] = ((need >> row) & 1ull) ? wave_rows[row * 12 + 4 * PHASE + part] : make_float4(0.f, 0.f, 0.f, 0.f);
+  }
+}
+
+template <int PHASE>
+__device__ __forceinline__ void sh_third_fold(int deg, const float* B, const float4* v, float4* lds, int lane,
+                                              float* res) {
+  wave_sync_lds();  // (everyone has read the previous third)
+#pragma unroll
+  for (int j = 0; j < 4; j++) {
+    const int idx = j * GS_WAVE + lane, row = idx >> 2, part = idx & 3;
+    lds[row * SH_THIRD4 + part] = v[j];
+  }
+  wave_sync_lds();
+  float f[16];
+#pragma unroll
+  for (int k = 0; k < 4; k++) {
+    const float4 w = lds[lane * SH_THIRD4 + k];
+    f[4 * k] = w.x; f[4 * k + 1] = w.y; f[4 * k + 2] = w.z; f[4 * k + 3] = w.w;
+  }
+  // flat element 16 * PHASE + e of the row is coefficient (16 * PHASE + e) / 3 of channel (16 * PHASE + e) % 3
+#define GS_SH_STEP(E)                                                                                         \
+  res[(16 * PHASE + E) % 3] = sh_accumulate<(16 * PHASE + E) / 3>(deg, res[(16 * PHASE + E) % 3], B, f[E]);
+  GS_SH_STEP(0) GS_SH_STEP(1) GS_SH_STEP(2) GS_SH_STEP(3) GS_SH_STEP(4) GS_SH_STEP(5) GS_SH_STEP(6) GS_SH_STEP(7)
+  GS_SH_STEP(8) GS_SH_STEP(9) GS_SH_STEP(10) GS_SH_STEP(11) GS_SH_STEP(12) GS_SH_STEP(13) GS_SH_STEP(14)
+  GS_SH_STEP(15)
+#undef GS_SH_STEP
+}
+
+
 // rows whose bit in `need` is clear are not fetched (their LDS rows read as zero)
 __device__ __forceinline__ void wave_rows_load(const float4* __restrict__ g4, uint64_t need, float4* lds, int lane) {
   float4 v[12];
@@ -214,8 +290,10 @@ preprocess_fwd_kernel(int P, int D, int M, const float* __restrict__ means, cons
                       uint32_t gx, uint32_t gy, int* __restrict__ radii, float2* __restrict__ means2D,
                       float* __restrict__ depths, float* __restrict__ cov3D, float4* __restrict__ conic_opacity,
                       float* __restrict__ rgb, uint8_t* __restrict__ clamped, uint32_t* __restrict__ tiles_touched) {
-  const int i = blockIdx.x * GS_BLOCK_1D + threadIdx.x;
-  if (i >= P) return;
+  __shared__ float4 s_sh[GS_BLOCK_1D / GS_WAVE][GS_WAVE * SH_THIRD4];
+  const int slot = blockIdx.x * GS_BLOCK_1D + threadIdx.x;
+  const bool live = slot < P;
+  const int i = live ? slot : P - 1;  // lanes past the end keep step with a copy of the last Gaussian and store nothing
   CamParams cam;
   load_cam(Vg, PMg, camg, cam);
   const float mean[3] = {means[3 * (size_t)i], means[3 * (size_t)i + 1], means[3 * (size_t)i + 2]};
@@ -226,36 +304,52 @@ preprocess_fwd_kernel(int P, int D, int M, const float* __restrict__ means, cons
   GeomOut g;
   bool in_front;
   const bool ok = geom_forward(mean, sc, mod, q, nullptr, cam, W, H, tanx, tany, fx, fy, gx, gy, cov6, in_front, g);
-  float* c6o = cov3D + 6 * (size_t)i;
-  {
-    float2* c6v = reinterpret_cast<float2*>(c6o);  // 24-byte rows are 8-byte aligned
+  if (live) {
+    float2* c6v = reinterpret_cast<float2*>(cov3D + 6 * (size_t)i);  // 24-byte rows are 8-byte aligned
     c6v[0] = make_float2(cov6[0], cov6[1]);
     c6v[1] = make_float2(cov6[2], cov6[3]);
     c6v[2] = make_float2(cov6[4], cov6[5]);
+    radii[i] = ok ? g.radius : 0;
+    depths[i] = ok ? g.depth : 0.f;
+    means2D[i] = ok ? make_float2(g.px, g.py) : make_float2(0.f, 0.f);
+    conic_opacity[i] = ok ? make_float4(g.conic[0], g.conic[1], g.conic[2], opac[i]) : make_float4(0.f, 0.f, 0.f, 0.f);
+    if (tiles_touched) tiles_touched[i] = ok ? (g.rect.x1 - g.rect.x0) * (g.rect.y1 - g.rect.y0) : 0u;
   }
   float col[3] = {0.f, 0.f, 0.f};
   uint8_t clm[3] = {0, 0, 0};
-  if (ok && shs != nullptr && M > 0) {
+  if (shs != nullptr && M > 0) {  // wave-uniform
     const float dx = mean[0] - cam.campos[0], dy = mean[1] - cam.campos[1], dz = mean[2] - cam.campos[2];
     const float dv[3] = {dx, dy, dz};
     const float len = sqrtf(dot3(dv, dv));
     const float x = dx / len, y = dy / len, z = dz / len;
-    float c[3][16];
-    const float* sh = shs + (size_t)i * M * 3;
     if (M == 16) {
-      // direct 16-byte loads: staging the rows through LDS costs this kernel more occupancy than it saves
-      const float4* sh4 = reinterpret_cast<const float4*>(sh);
-      float flat[48];
+      // colours only for Gaussians that survive culling: the rows of the others are not fetched
+      const int lane = threadIdx.x & (GS_WAVE - 1);
+      const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / GS_WAVE);
+      const uint64_t need = gs_ballot(ok && live);
+      const float4* wave_rows =
+          reinterpret_cast<const float4*>(shs) + 12 * ((size_t)blockIdx.x * GS_BLOCK_1D + (size_t)wave * GS_WAVE);
+      float B[16];
+      sh_basis(x, y, z, B);
+      float res[3] = {0.f, 0.f, 0.f};
+      float4 va[4], vb[4];
+      sh_third_fetch<0>(wave_rows, need, lane, va);
+      sh_third_fetch<1>(wave_rows, need, lane, vb);
+      sh_third_fold<0>(D, B, va, s_sh[wave], lane, res);
+      sh_third_fetch<2>(wave_rows, need, lane, va);
+      sh_third_fold<1>(D, B, vb, s_sh[wave], lane, res);
+      sh_third_fold<2>(D, B, va, s_sh[wave], lane, res);
+      if (ok) {
 #pragma unroll
-      for (int k = 0; k < 12; k++) {
-        const float4 v = sh4[k];
-        flat[4 * k] = v.x; flat[4 * k + 1] = v.y; flat[4 * k + 2] = v.z; flat[4 * k + 3] = v.w;
+        for (int ch = 0; ch < 3; ch++) {
+          const float r = res[ch] + 0.5f;
+          clm[ch] = r < 0.0f;
+          col[ch] = fmaxf(r, 0.0f);
+        }
       }
-#pragma unroll
-      for (int k = 0; k < 16; k++) {
-        c[0][k] = flat[3 * k]; c[1][k] = flat[3 * k + 1]; c[2][k] = flat[3 * k + 2];
-      }
-    } else {
+    } else if (ok) {
+      float c[3][16];
+      const float* sh = shs + (size_t)i * M * 3;
 #pragma unroll
       for (int k = 0; k < 16; k++) {
         const bool have = k < M;
@@ -263,25 +357,21 @@ preprocess_fwd_kernel(int P, int D, int M, const float* __restrict__ means, cons
         c[1][k] = have ? sh[3 * k + 1] : 0.f;
         c[2][k] = have ? sh[3 * k + 2] : 0.f;
       }
-    }
 #pragma unroll
-    for (int ch = 0; ch < 3; ch++) {
-      const float res = sh_channel(D, x, y, z, c[ch]);
-      clm[ch] = res < 0.0f;
-      col[ch] = fmaxf(res, 0.0f);
+      for (int ch = 0; ch < 3; ch++) {
+        const float res = sh_channel(D, x, y, z, c[ch]);
+        clm[ch] = res < 0.0f;
+        col[ch] = fmaxf(res, 0.0f);
+      }
     }
   }
-  radii[i] = ok ? g.radius : 0;
-  depths[i] = ok ? g.depth : 0.f;
-  means2D[i] = ok ? make_float2(g.px, g.py) : make_float2(0.f, 0.f);
-  conic_opacity[i] = ok ? make_float4(g.conic[0], g.conic[1], g.conic[2], opac[i]) : make_float4(0.f, 0.f, 0.f, 0.f);
+  if (!live) return;
   rgb[3 * (size_t)i] = col[0];
   rgb[3 * (size_t)i + 1] = col[1];
   rgb[3 * (size_t)i + 2] = col[2];
   clamped[3 * (size_t)i] = clm[0];
   clamped[3 * (size_t)i + 1] = clm[1];
   clamped[3 * (size_t)i + 2] = clm[2];
-  if (tiles_touched) tiles_touched[i] = ok ? (g.rect.x1 - g.rect.x0) * (g.rect.y1 - g.rect.y0) : 0u;
 }
 
 // cuda_rasterizer/forward.cu:545-620.
