@@ -50,6 +50,15 @@ __device__ __forceinline__ int f2i_sat(float v) {
   return (int)v;
 }
 
+// Workgroups go to the eight XCDs in turn (workgroup b of a launch runs on XCD b % 8), and each XCD has its own L2.
+// This renumbers them so that the workgroups of one XCD hold consecutive indices (XCD 0 the first eighth, and so
+// on, each in launch order): work items that are neighbours in memory then share an L2.  A bijection on [0, n).
+__device__ __forceinline__ uint32_t xcd_contiguous_index(uint32_t b, uint32_t n) {
+  constexpr uint32_t XCDS = 8;
+  const uint32_t x = b % XCDS, rest = n % XCDS;
+  return x * (n / XCDS) + (x < rest ? x : rest) + b / XCDS;
+}
+
 __device__ __forceinline__ uint32_t f2u_sat(float v) {
   if (!(v == v)) return 0u;
   if (v >= 4294967296.0f) return 0xFFFFFFFFu;

@@ -34,6 +34,11 @@ __host__ __device__ inline int bucket_blocks(int P) {
   return (P + per - 1) / per;
 }
 
+// Which chunk of Gaussians a workgroup takes: a tile's records lie in chunk order, so with chunk = workgroup index
+// the records that share a 64-byte line would come from eight different L2s, each of which writes its part of
+// the line back on its own.  Dealt out by xcd_contiguous_index, neighbours in memory meet in one L2.
+__device__ __forceinline__ int chunk_of_workgroup(int b, int n) { return (int)xcd_contiguous_index(b, n); }
+
 // 1a. Per Gaussian the number of tiles it touches (rasterizer_impl.cu:264-288), per workgroup the number of
 // instances of every tile.  The workgroup's Gaussians are a contiguous chunk; the scatter walks the same chunk.
 __global__ void __launch_bounds__(BK_THREADS)
@@ -51,7 +56,8 @@ bucket_count_kernel(int P, int per_block, uint32_t gx, uint32_t gy, const int* _
     s_local[t] = compute_locally[t];
   }
   __syncthreads();
-  const int first = blockIdx.x * per_block;
+  const int chunk = chunk_of_workgroup(blockIdx.x, gridDim.x);
+  const int first = chunk * per_block;
   const int last = first + per_block < P ? first + per_block : P;
   // four Gaussians per round: their loads go out together, then each is walked (the loop bounds are the same
   // for every thread of the workgroup, because the walk is a wave-wide operation)
@@ -85,13 +91,13 @@ bucket_count_kernel(int P, int per_block, uint32_t gx, uint32_t gy, const int* _
   for (int d = GS_WAVE / 2; d >= 1; d >>= 1) my_sum += __shfl_xor(my_sum, d, GS_WAVE);
   if ((threadIdx.x & (GS_WAVE - 1)) == 0) s_sum[threadIdx.x / GS_WAVE] = my_sum;
   __syncthreads();
-  uint32_t* row = table + (size_t)blockIdx.x * T;
+  uint32_t* row = table + (size_t)chunk * T;
   for (uint32_t t = threadIdx.x; t < T; t += BK_THREADS) row[t] = s_hist[t];
   // the workgroup's share of the prefix sum over the Gaussians (bucket_offsets_kernel finishes it)
   if (threadIdx.x == 0) {
     uint32_t all = 0;
     for (int w = 0; w < BK_THREADS / GS_WAVE; w++) all += s_sum[w];
-    block_sums[blockIdx.x] = all;
+    block_sums[chunk] = all;
   }
 }
 
@@ -312,17 +318,18 @@ bucket_scatter_kernel(int P, int per_block, uint32_t gx, uint32_t gy, const floa
   if (fits_word != nullptr && *fits_word == 0u) return;
   const uint32_t T = gx * gy;
   uint8_t* s_local = reinterpret_cast<uint8_t*>(s_next + T);
-  const uint32_t* row = table + (size_t)blockIdx.x * T;
+  const int chunk = chunk_of_workgroup(blockIdx.x, gridDim.x);
+  const uint32_t* row = table + (size_t)chunk * T;
   for (uint32_t t = threadIdx.x; t < T; t += BK_THREADS) {
     s_next[t] = ranges[2 * t] + row[t];
     s_local[t] = compute_locally[t];
   }
   __syncthreads();
   const int lane = threadIdx.x & (GS_WAVE - 1), wave = threadIdx.x / GS_WAVE;
-  const int first = blockIdx.x * per_block;
+  const int first = chunk * per_block;
   const int last = first + per_block < P ? first + per_block : P;
   struct Owner { uint32_t first, depth_bits, id; };
-  uint32_t carry = block_prefix[blockIdx.x];  // instances of the Gaussians before this round
+  uint32_t carry = block_prefix[chunk];  // instances of the Gaussians before this round
   for (int base = first; base < last; base += BK_BATCH * BK_THREADS) {
     const int i0 = base + (int)threadIdx.x * BK_BATCH;
     int r[BK_BATCH];
