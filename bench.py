@@ -288,7 +288,7 @@ def main():
             for s_, _, _ in lanes:
                 s_.synchronize()
 
-        in_flight(max(2, args.warmup))
+        in_flight(max(20, args.warmup))  # (each stream's allocator pool has to fill before the rate is steady)
         t0b = time.perf_counter()
         in_flight(args.steps)
         ms_per_view_two_in_flight = (time.perf_counter() - t0b) * 1e3 / args.steps
