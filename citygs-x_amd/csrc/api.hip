@@ -150,7 +150,7 @@ GeometryLayout geometry_layout(int P) {
 }
 
 struct BinningLayout {
-  size_t point_list, keys, point_list_unsorted, keys_unsorted, emission, emission_other, sort_temp, total;
+  size_t point_list, keys, point_list_unsorted, keys_unsorted, emission, emission_other, sort_temp, block_hits, total;
 };
 // n = the number of instances the arrays are laid out for
 BinningLayout binning_layout(int64_t R) {
@@ -165,6 +165,7 @@ BinningLayout binning_layout(int64_t R) {
   L.emission = take(n * 4);
   L.emission_other = take(n * 4);
   L.sort_temp = take(sort_temp_bytes((int64_t)n));
+  L.block_hits = take(n * 2);  // what the forward blend leaves for the backward blend, per sorted instance
   L.total = off + 256;
   return L;
 }
@@ -537,6 +538,7 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
     uint32_t *point_list, *gauss_of_emission, *emission, *emission_other;
     uint64_t *keys, *keys_other;
     void* sort_temp;
+    uint16_t* block_hits;
   };
   auto carve = [&](int64_t n, Arrays& A) -> int {
     const BinningLayout BL = binning_layout(n);
@@ -550,6 +552,7 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
     A.emission = (uint32_t*)(bbase + BL.emission);
     A.emission_other = (uint32_t*)(bbase + BL.emission_other);
     A.sort_temp = bbase + BL.sort_temp;
+    A.block_hits = (uint16_t*)(bbase + BL.block_hits);
     return 0;
   };
   auto blend = [&](const Arrays& A, bool ahead_of_host) -> int {
@@ -565,6 +568,7 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
     a.depths = depths; a.out_max_weight_depth = out_max_weight_depth;
     a.n_render = n_render; a.n_consider = n_consider; a.n_contrib_tile = n_contrib;
     a.fits_word = ahead_of_host ? bucket_fits_word(bucket_table, T) : nullptr;
+    a.block_hits = A.block_hits;
     {
       StageScope _t("render_fwd", stream);
       launch_render_fwd(a, stream);
@@ -725,6 +729,7 @@ int gs_render_backward(int P, int R, const float* background, int width, int hei
   const char* ibase = align_ptr(img_buffer, 256);
   RenderBwdArgs a;
   a.emission_sorted = (const uint32_t*)(bbase + BL.emission);
+  a.block_hits = (const uint16_t*)(bbase + BL.block_hits);
   a.point_offsets = (const uint32_t*)(gbase + GL.point_offsets);
   a.instance_grads = (float*)align_ptr((const char*)instance_grads, 256);
   a.P = P; a.W = width; a.H = height;

@@ -207,6 +207,10 @@ struct RenderFwdArgs {
   // optional device word: the kernel was launched before the host knew whether the per-tile lists would be
   // built by the kernels queued ahead of it; it does nothing if the word is 0
   const uint32_t* fits_word = nullptr;
+  // optional (R): per sorted instance, which of the tile's sixteen 4x4 pixel blocks the Gaussian can touch (bit
+  // 4 * wave + row), as found by the kernel's own list building; the backward blend reads it instead of testing
+  // again
+  uint16_t* block_hits = nullptr;
 };
 int launch_render_fwd(const RenderFwdArgs& a, hipStream_t stream);
 
@@ -226,6 +230,7 @@ struct RenderBwdArgs {
   const uint32_t* emission_sorted;
   const uint32_t* point_offsets;
   float* instance_grads;  // (R,16) scratch, fully written by the blend kernel
+  const uint16_t* block_hits = nullptr;  // optional (R): left by the forward blend (RenderFwdArgs::block_hits)
   // outputs, fully written by the per-Gaussian reduction
   float* dL_dmean2D;         // (P,2)
   float* dL_dmean2D_abs;     // (P,3)

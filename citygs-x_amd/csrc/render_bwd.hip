@@ -50,7 +50,9 @@ constexpr int CHUNKS = SUB / 32;
 constexpr int WAVES = GS_TILE_PIX / GS_WAVE;
 static_assert(SUB * 4 == GS_TILE_PIX, "a thread hands over a quarter of one record of the sub-batch");
 
-template <bool RENDER_GEO>
+// HITS: the forward blend left, per sorted instance, which 4x4 blocks of the tile the Gaussian can touch; without
+// it the same test is made again here.
+template <bool RENDER_GEO, bool HITS>
 __global__ void __launch_bounds__(GS_TILE_PIX) __attribute__((amdgpu_waves_per_eu(5)))
 render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__ point_list, int W, int H, float fx,
                   float fy, const float* __restrict__ bg, const float2* __restrict__ means2D,
@@ -59,12 +61,14 @@ render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
                   const float* __restrict__ final_Ts, const uint32_t* __restrict__ n_contrib_px,
                   const uint8_t* __restrict__ compute_locally, const float* __restrict__ dL_dpix,
                   const float* __restrict__ dL_dout_all_map, const float* __restrict__ dL_dout_plane_depth,
-                  const uint32_t* __restrict__ emission_sorted, float4* __restrict__ instance_grads) {
+                  const uint32_t* __restrict__ emission_sorted, float4* __restrict__ instance_grads,
+                  const uint16_t* __restrict__ block_hits) {
   constexpr bool render_geo = RENDER_GEO;
   __shared__ uint32_t s_emis[BATCH];
   __shared__ float2 s_xy[BATCH];
   __shared__ float4 s_co[BATCH];
-  __shared__ float4 s_cp[BATCH];
+  __shared__ float4 s_cp[HITS ? 1 : BATCH];
+  __shared__ uint16_t s_hits[HITS ? BATCH : 1];
   __shared__ float s_floor[BATCH];
   __shared__ float s_rgb[GS_N_RGB][BATCH];
   __shared__ float s_map[GS_N_MAP][BATCH];
@@ -179,7 +183,9 @@ render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
       s_xy[tid] = xy;
       s_co[tid] = co;
       float pfl;
-      s_cp[tid] = cull_params(co, pfl);
+      const float4 cp = cull_params(co, pfl);
+      if (HITS) s_hits[tid] = block_hits[k_sorted];
+      else s_cp[tid] = cp;
       s_floor[tid] = pfl;
       const float c0 = rgb[3 * (size_t)g], c1 = rgb[3 * (size_t)g + 1], c2 = rgb[3 * (size_t)g + 2];
       s_rgb[0][tid] = c0;
@@ -211,13 +217,20 @@ render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
         const int jj = base + lane;
         const bool valid = jj < count;
         const uint64_t valid_m = gs_ballot(valid);  // (masks of single comparisons, combined in scalar registers)
-        const float2 mu = s_xy[valid ? jj : 0];
-        const float4 cq = s_co[valid ? jj : 0];
-        const float4 cp = s_cp[valid ? jj : 0];
+        float2 mu = make_float2(0.f, 0.f);
+        float4 cq = make_float4(0.f, 0.f, 0.f, 0.f), cp = cq;
+        uint32_t nibble = 0u;
+        if (HITS) {
+          nibble = (uint32_t)s_hits[valid ? jj : 0] >> (4 * wave);
+        } else {
+          mu = s_xy[valid ? jj : 0];
+          cq = s_co[valid ? jj : 0];
+          cp = s_cp[valid ? jj : 0];
+        }
 #pragma unroll
         for (int r = 0; r < 4; r++) {
-          const uint64_t hit = valid_m & gs_ballot((first_pos - jj) < row_last_of[r]) &
-                               gs_ballot(ellipse_hits_row(mu, cq, cp, rt.qx0, rt.qy0, r));
+          const bool touches = HITS ? ((nibble >> r) & 1u) != 0u : ellipse_hits_row(mu, cq, cp, rt.qx0, rt.qy0, r);
+          const uint64_t hit = valid_m & gs_ballot((first_pos - jj) < row_last_of[r]) & gs_ballot(touches);
           if (lane == 0) {
             s_list[wave][r][0] = (uint32_t)hit;
             s_list[wave][r][1] = (uint32_t)(hit >> 32);
@@ -439,18 +452,19 @@ reduce_instances_kernel(int P, const uint32_t* __restrict__ point_offsets, const
 
 int launch_render_bwd(const RenderBwdArgs& a, hipStream_t stream) {
   const dim3 grid((a.W + GS_TILE_X - 1) / GS_TILE_X, (a.H + GS_TILE_Y - 1) / GS_TILE_Y, 1);
-  if (a.render_geo)
-    hipLaunchKernelGGL(render_bwd_kernel<true>, grid, dim3(GS_TILE_PIX), 0, stream, (const uint2*)a.ranges,
-                       a.point_list, a.W, a.H, a.fx, a.fy, a.bg, (const float2*)a.means2D,
-                       (const float4*)a.conic_opacity, a.rgb, a.all_map, a.all_map_pixels, a.final_T, a.n_contrib_px,
-                       a.compute_locally, a.dL_dpix, a.dL_dout_all_map, a.dL_dout_plane_depth, a.emission_sorted,
-                       (float4*)a.instance_grads);
-  else
-    hipLaunchKernelGGL(render_bwd_kernel<false>, grid, dim3(GS_TILE_PIX), 0, stream, (const uint2*)a.ranges,
-                       a.point_list, a.W, a.H, a.fx, a.fy, a.bg, (const float2*)a.means2D,
-                       (const float4*)a.conic_opacity, a.rgb, a.all_map, a.all_map_pixels, a.final_T, a.n_contrib_px,
-                       a.compute_locally, a.dL_dpix, a.dL_dout_all_map, a.dL_dout_plane_depth, a.emission_sorted,
-                       (float4*)a.instance_grads);
+  auto go = [&](auto kernel) {
+    hipLaunchKernelGGL(kernel, grid, dim3(GS_TILE_PIX), 0, stream, (const uint2*)a.ranges, a.point_list, a.W, a.H,
+                       a.fx, a.fy, a.bg, (const float2*)a.means2D, (const float4*)a.conic_opacity, a.rgb, a.all_map,
+                       a.all_map_pixels, a.final_T, a.n_contrib_px, a.compute_locally, a.dL_dpix, a.dL_dout_all_map,
+                       a.dL_dout_plane_depth, a.emission_sorted, (float4*)a.instance_grads, a.block_hits);
+  };
+  if (a.render_geo) {
+    if (a.block_hits) go(render_bwd_kernel<true, true>);
+    else go(render_bwd_kernel<true, false>);
+  } else {
+    if (a.block_hits) go(render_bwd_kernel<false, true>);
+    else go(render_bwd_kernel<false, false>);
+  }
   hipLaunchKernelGGL(reduce_instances_kernel, dim3((a.P + GS_BLOCK_1D - 1) / GS_BLOCK_1D), dim3(GS_BLOCK_1D), 0,
                      stream, a.P, a.point_offsets, (const float4*)a.instance_grads, (float)(0.5 * a.W),
                      (float)(0.5 * a.H), a.render_geo,

@@ -37,7 +37,7 @@ constexpr int CHUNKS = BATCH / 32;  // 32-bit list words per row and batch
 // that blends with the largest weight alpha * T (the front-most one among equals; 0 where nothing blends).  It
 // leaves every other output as it is.
 template <bool RENDER_GEO, bool MAX_DEPTH>
-__global__ void __launch_bounds__(GS_TILE_PIX)
+__global__ void __launch_bounds__(GS_TILE_PIX) __attribute__((amdgpu_waves_per_eu(7)))
 render_fwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__ point_list, int W, int H, float fx,
                   float fy, float cx, float cy, const float2* __restrict__ means2D, const float* __restrict__ rgb,
                   const float* __restrict__ all_map, const float4* __restrict__ conic_opacity,
@@ -47,7 +47,8 @@ render_fwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
                   int* __restrict__ out_observe, float* __restrict__ out_all_map,
                   float* __restrict__ out_plane_depth, int* __restrict__ n_render, int* __restrict__ n_consider,
                   int* __restrict__ n_contrib_tile, const float* __restrict__ depths,
-                  float* __restrict__ out_max_weight_depth, const uint32_t* __restrict__ fits_word) {
+                  float* __restrict__ out_max_weight_depth, const uint32_t* __restrict__ fits_word,
+                  uint16_t* __restrict__ block_hits) {
   constexpr bool render_geo = RENDER_GEO;
   // launched ahead of the host's decision on how the per-tile lists are built: nothing to do if they were not
   if (fits_word != nullptr && *fits_word == 0u) return;
@@ -256,11 +257,22 @@ render_fwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
       };
       if (select_blend) walk(std::true_type{});
       else walk(std::false_type{});
+    } else if (block_hits != nullptr && lane < 4 * CHUNKS) {
+      s_list[wave][lane / CHUNKS][lane % CHUNKS] = 0u;  // (the lists are also what the backward pass is left)
     }
     __syncthreads();
     if (tid < count) {
       const int c = s_obs[tid];
       if (c != 0) atomicAdd(&out_observe[s_id[tid]], c);
+      if (block_hits != nullptr) {
+        // for the backward pass: this slot's bit of the sixteen row lists (a row that had saturated has an empty
+        // list, and nothing behind a row's last contributor is looked at there)
+        uint32_t hits = 0u;
+#pragma nounroll
+        for (int wr = 0; wr < 4 * (GS_TILE_PIX / GS_WAVE); wr++)  // (one list word at a time: registers are scarce here)
+          hits |= ((s_list[0][0][wr * CHUNKS + (tid >> 5)] >> (tid & 31)) & 1u) << wr;
+        block_hits[range.x + (uint32_t)i * BATCH + tid] = (uint16_t)hits;
+      }
     }
   }
 
@@ -308,7 +320,7 @@ static void launch_render_fwd_variant(const RenderFwdArgs& a, hipStream_t stream
                      a.point_list, a.W, a.H, a.fx, a.fy, a.cx, a.cy, (const float2*)a.means2D, a.rgb, a.all_map,
                      (const float4*)a.conic_opacity, a.compute_locally, a.bg, a.final_T, a.n_contrib_px,
                      a.n_contrib2loss_px, a.out_color, a.out_observe, a.out_all_map, a.out_plane_depth, a.n_render,
-                     a.n_consider, a.n_contrib_tile, a.depths, a.out_max_weight_depth, a.fits_word);
+                     a.n_consider, a.n_contrib_tile, a.depths, a.out_max_weight_depth, a.fits_word, a.block_hits);
 }
 
 int launch_render_fwd(const RenderFwdArgs& a, hipStream_t stream) {
