@@ -404,3 +404,42 @@ def test_non_finite_colours_reach_only_the_pixels_that_blend_them(H, orc, geo):
         # (the colour and channel gradients are weight x upstream gradient and stay finite throughout)
         assert ok.all() if k in ("dL_dcolors", "dL_dall_map") else ((~ok).any() and (~ok).mean() < 0.5), k
         assert H.rel_l2(a[ok], r[ok]) <= GRAD_TOL, k
+
+
+@pytest.mark.parametrize("cfg,P,mask,geo", [(1, 150_000, "all", True), (1, 100_000, "rows", True),
+                                            (3, 60_000, "checker", False)])
+def test_backward_blend_gives_the_same_bits_with_the_forward_lists_and_with_its_own(H, orc, cfg, P, mask, geo):
+    """The whole-view entry points hand the backward blend the row lists the forward blend built (16 bits per
+    sorted instance in the binning buffer); the stage entry points have no such buffer and the backward blend tests
+    every Gaussian against its blocks itself.  Same visits either way, so the five gradient tensors are the same
+    bits."""
+    import gs_scenes
+    from diff_gaussian_rasterization import _C
+    g, cam, pre, cl, b, am = _render_inputs(H, orc, cfg, P, mask)
+    W, Hh = cam.image_width, cam.image_height
+    gx, gy = H.grid(W, Hh)
+    bg = np.array([0.2, 0.4, 0.6], np.float32)
+    ug = gs_scenes.upstream_grads(cam)
+    d = {k: H.dev(pre[k]) for k in ("means2D", "depths", "conic_opacity", "rgb")}
+    radii = torch.from_numpy(pre["radii"].astype(np.int32)).to(H.DEV)
+    t_am, t_cl, t_bg = H.dev(am), torch.from_numpy(cl.reshape(gy, gx)).to(H.DEV), H.dev(bg)
+    gpix, gmap, gdep = (ug[k].to(H.DEV) for k in ("color", "all_map", "plane_depth"))
+    vm, cp = cam.world_view_transform.to(H.DEV), cam.camera_center.to(H.DEV)
+
+    args = {"stats_collector": {}}
+    out, info = _C.render_gaussians_ex(t_bg, Hh, W, d["means2D"], d["depths"], radii, d["conic_opacity"], d["rgb"],
+                                       t_cl, vm, cp, cam.tanfovx, cam.tanfovy, t_am, geo, False, args)
+    whole = _C.render_gaussians_backward(t_bg, cam.tanfovx, cam.tanfovy, out[6], t_am, out[0], out[8], out[9],
+                                         out[10], t_cl, gpix, gmap, gdep, d["means2D"], d["conic_opacity"], d["rgb"],
+                                         geo, False, args, binning_capacity=info["binning_capacity"])
+
+    f = H.render_fwd(P, W, Hh, cam.tanfovx, cam.tanfovy, H.as_u32(b["ranges"]), H.as_u32(b["point_list"]),
+                     d["means2D"], d["rgb"], t_am, d["conic_opacity"], H.dev(cl), t_bg, render_geo=geo)
+    stage = H.render_bwd(P, W, Hh, cam.tanfovx, cam.tanfovy, t_bg, H.as_u32(b["ranges"]), H.as_u32(b["point_list"]),
+                         d["means2D"], d["conic_opacity"], d["rgb"], t_am, f["out_all_map"], f["final_T"],
+                         f["n_contrib"], H.dev(cl), gpix, gmap, gdep, H.as_u32(b["emission_sorted"]),
+                         H.as_u32(b["point_offsets"]), render_geo=geo)
+    names = ["dL_dmeans2D", "dL_dmeans2D_abs", "dL_dconic_opacity", "dL_dcolors"] + (["dL_dall_map"] if geo else [])
+    for k, a in zip(names, whole):
+        assert torch.equal(a, stage[k]), k
+    assert float(stage["dL_dcolors"].abs().max()) > 0.0
