@@ -44,6 +44,23 @@ def test_preprocess_forward(H, orc, cfg, P, sh_mode):
     assert (ref["radii"] > 0).any() and (ref["radii"] == 0).any() or cfg == 0
 
 
+@pytest.mark.parametrize("degree,M", [(0, 16), (1, 16), (2, 16), (3, 16), (0, 1), (1, 4), (2, 9), (1, 9)])
+@pytest.mark.parametrize("P", [1, 63, 64, 65, 33_333])
+def test_preprocess_colours_at_every_degree_and_row_length(H, orc, degree, M, P):
+    """Active SH degrees below the stored one (the caller raises the degree as training goes on), rows shorter than
+    16 coefficients, and Gaussian counts that end inside a wave: colours and clamp flags equal the oracle's bits."""
+    g, cam = _scene(0, P)
+    g = dict(g)
+    g["shs"] = g["shs"][:, :M].contiguous()
+    got, _ = H.preprocess_fwd(g, cam, sh_mode=True, sh_degree=degree)
+    ref = H.oracle_preprocess(orc, g, cam, sh_mode=True, sh_degree=degree)
+    assert np.array_equal(got["radii"].cpu().numpy(), ref["radii"])
+    assert np.array_equal(got["clamped"].cpu().numpy(), ref["clamped"])
+    for k in ("means2D", "cov3D", "conic_opacity", "rgb"):
+        a, b = got[k].cpu().numpy(), ref[k]
+        assert np.array_equal(a, b), f"{k}: max abs diff {np.abs(a - b).max()}"
+
+
 @pytest.mark.parametrize("cfg,P", CASES)
 def test_visible_filter_and_mark_visible(H, orc, cfg, P):
     import ctypes as C
