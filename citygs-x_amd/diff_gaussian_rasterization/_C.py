@@ -4,6 +4,7 @@ names, argument order and return tuples, implemented on libgsrast.so through
 ctypes.  torch is used for device memory and the current stream only.
 """
 import ctypes as C
+import os
 
 import numpy as np
 import torch
@@ -177,6 +178,56 @@ def render_gaussians(background, image_height, image_width, means2D, depths, rad
                                args)[0]
 
 
+def _want_tile_log(args):
+    """cuda_rasterizer/rasterizer_impl.cu:764: in training, with zhx_debug, on the first iteration of every
+    log interval."""
+    if not isinstance(args, dict):
+        return False
+    try:
+        return (str(args.get("mode", "")) == "train" and str(args.get("zhx_debug", "False")) == "True"
+                and int(args.get("iteration", 0)) % int(args.get("log_interval", 0) or 1) == 1)
+    except (TypeError, ValueError):
+        return False
+
+
+def _write_tile_log(args, H, W, n_render, n_consider, n_contrib):
+    """The reference's per-tile debug log (cuda_rasterizer/rasterizer_impl.cu:764-842, file name and line prefix
+    from save_log_in_file, :290-298): for every tile with a non-empty list its range, the list length and the
+    per-pixel averages of the two contributor counts, then one line of totals.  The per-tile sums the reference
+    forms on the host from the per-pixel images are the three per-tile outputs of the forward call."""
+    gx, gy = (W + BLOCK_X - 1) // BLOCK_X, (H + BLOCK_Y - 1) // BLOCK_Y
+    nr = n_render.cpu().numpy().astype(np.int64)
+    nc = n_consider.cpu().numpy().astype(np.int64)
+    n2 = n_contrib.cpu().numpy().astype(np.int64)
+    ends = np.cumsum(nr)
+    it, rk, ws = int(args.get("iteration", 0)), str(args.get("global_rank", "0")), str(args.get("world_size", "1"))
+    lines = []
+    tot_r = tot_c = tot_2 = 0.0
+    pixels = local = 0
+    for t in range(gx * gy):
+        if nr[t] <= 0:
+            continue
+        tx, ty = t % gx, t // gx
+        num_pix = (min(ty * BLOCK_Y + BLOCK_Y, H) - ty * BLOCK_Y) * (min(tx * BLOCK_X + BLOCK_X, W) - tx * BLOCK_X)
+        ave_c = np.float32(nc[t]) / np.float32(num_pix)
+        ave_2 = np.float32(n2[t]) / np.float32(num_pix)
+        ratio = ave_2 / np.float32(nr[t]) if num_pix > 0 else np.float32(0)
+        lines.append("iteration: %d, tile: (%d, %d), range: (%d, %d), num_rendered_this_tile: %d, "
+                     "n_considered_per_pixel: %f, n_contrib2loss_per_pixel: %f, contrib2loss_ratio: %f"
+                     % (it, ty, tx, ends[t], ends[t] - nr[t], nr[t], ave_c, ave_2, ratio))
+        tot_r += float(nr[t]); tot_c += float(nc[t]); tot_2 += float(n2[t])
+        pixels += num_pix
+        local += 1
+    lines.append("iteration: %d, global_rank: %d, world_size: %d, num_tiles: %d, num_pixels: %d, num_rendered: %d, "
+                 "global_ave_n_rendered_per_pix: %f, global_ave_n_considered_per_pix: %f, "
+                 "global_ave_n_contrib2loss_per_pix: %f"
+                 % (it, int(rk), int(ws), local, pixels, int(tot_r), tot_r / max(local, 1), tot_c / max(pixels, 1),
+                    tot_2 / max(pixels, 1)))
+    path = os.path.join(str(args.get("log_folder", ".")), "n_contrib_ws=%s_rk=%s.log" % (ws, rk))
+    with open(path, "a") as f:
+        f.write("\n".join(lines) + "\n")
+
+
 def render_gaussians_ex(background, image_height, image_width, means2D, depths, radii, conic_opacity, rgb,
                         compute_locally, viewmatrix, campos, tan_fovx, tan_fovy, all_map, render_geo, debug, args,
                         expected_instances=0, expected_longest_list=0):
@@ -245,6 +296,8 @@ def render_gaussians_ex(background, image_height, image_width, means2D, depths, 
     _record_time(args, "forward_render_time", elapsed.value)
     if want_mwd:
         args.setdefault("stats_collector", {})["max_weight_depth"] = mwd
+    if _want_tile_log(args):
+        _write_tile_log(args, H, W, n_render, n_consider, n_contrib)
     info = {"longest_list": int(result.longest_list), "binning_capacity": int(result.binning_capacity),
             "launched_ahead": bool(result.launched_ahead)}
     return ((num_rendered.value, out_color, n_render, n_consider, n_contrib, out_observe, out_all_map,

@@ -508,3 +508,50 @@ def test_views_in_flight_on_two_streams_give_the_same_results():
     for v, got in together:
         for i, (a, b) in enumerate(zip(alone[v], got)):
             assert torch.equal(a, b), (v, i)
+
+
+def test_per_tile_debug_log_is_written_like_the_reference(tmp_path):
+    """cuda_args with mode == "train", zhx_debug == "True" and iteration % log_interval == 1 make the forward call
+    append the reference's per-tile log (cuda_rasterizer/rasterizer_impl.cu:764-842): one line per tile with a
+    non-empty list and one line of totals, in its file name and format; other iterations write nothing."""
+    import re
+    import gs_scenes
+    from diff_gaussian_rasterization import GaussianRasterizer
+    g, cams = gs_scenes.make_scene(0, P=20_000, n_views=1)
+    cam = cams[0]
+    W, H = cam.image_width, cam.image_height
+    gx, gy = (W + 15) // 16, (H + 15) // 16
+    rast = GaussianRasterizer(_settings(cam))
+    d = {k: g[k].to(DEV) for k in ("means3D", "scales", "rotations", "opacities", "shs")}
+    cl = torch.ones(gy, gx, dtype=torch.bool, device=DEV)
+    am = gs_scenes.build_all_map(g["means3D"], g["scales"], g["rotations"], cam).to(DEV)
+
+    def run(iteration):
+        args = _cuda_args()
+        args.update(zhx_debug="True", iteration=str(iteration), log_interval="10", log_folder=str(tmp_path))
+        means2D, rgb, co, radii, depths = rast.preprocess_gaussians(d["means3D"], d["scales"], d["rotations"],
+                                                                    d["shs"], d["opacities"], args)
+        m2abs = torch.zeros_like(d["means3D"])
+        return rast.render_gaussians(means2D, m2abs, co, rgb, am, depths, radii, cl, cl, args)
+
+    path = tmp_path / "n_contrib_ws=1_rk=0.log"
+    run(2)
+    assert not path.exists()
+    color, n_render, n_consider, n_contrib, *_ = run(11)
+    lines = path.read_text().splitlines()
+    nr, nc, n2 = (t.cpu().numpy().astype(np.int64) for t in (n_render, n_consider, n_contrib))
+    busy = np.nonzero(nr > 0)[0]
+    assert len(lines) == len(busy) + 1 and len(busy) > 100
+    pat = re.compile(r"iteration: 11, tile: \((\d+), (\d+)\), range: \((\d+), (\d+)\), num_rendered_this_tile: (\d+), "
+                     r"n_considered_per_pixel: ([\d.]+), n_contrib2loss_per_pixel: ([\d.]+), contrib2loss_ratio: ([\d.]+)$")
+    ends = np.cumsum(nr)
+    for line, t in zip(lines, busy):
+        m = pat.match(line)
+        assert m, line
+        ty, tx, end, begin, n = (int(m.group(i)) for i in range(1, 6))
+        assert (ty, tx) == (t // gx, t % gx) and n == nr[t] and end == ends[t] and begin == ends[t] - nr[t]
+        assert abs(float(m.group(6)) - nc[t] / 256.0) < 1e-5 and abs(float(m.group(7)) - n2[t] / 256.0) < 1e-5
+    assert lines[-1].startswith("iteration: 11, global_rank: 0, world_size: 1, num_tiles: %d, num_pixels: %d, "
+                                "num_rendered: %d," % (len(busy), 256 * len(busy), nr.sum()))
+    run(21)
+    assert len(path.read_text().splitlines()) == 2 * (len(busy) + 1)  # appended, like the reference
