@@ -399,7 +399,10 @@ reduce_instances_kernel(int P, const uint32_t* __restrict__ point_offsets, const
   // whole wave: lane l takes records l, l + 64, ..., then the 64 partial sums are added across the lanes in a fixed
   // order.  Everything else is summed by its own thread, record after record.
   constexpr uint32_t MANY = 32;
+  constexpr uint32_t REC_CHUNK = GS_WAVE, REC_STRIDE4 = 5;
+  __shared__ float4 s_rec[GS_BLOCK_1D / GS_WAVE][REC_CHUNK * REC_STRIDE4];
   uint64_t many = gs_ballot(n > MANY);
+  const uint64_t many_in_wave = many;
   while (many != 0ull) {
     const int owner = (int)__builtin_ctzll(many);
     many &= many - 1ull;
@@ -422,13 +425,52 @@ reduce_instances_kernel(int P, const uint32_t* __restrict__ point_offsets, const
     }
     if (lane == owner) { a0 = p0; a1 = p1; a2 = p2; a3 = p3; }
   }
-  if (!live) return;
-  if (n <= MANY) {
-    for (uint32_t k = b; k < e; k++) {
-      const float4* rec = instance_grads + 4 * (size_t)k;
-      add(a0, rec[0]); add(a1, rec[1]); add(a2, rec[2]); add(a3, rec[3]);
+  if (many_in_wave != 0ull) {
+    // (a wave that holds such a Gaussian reads the others' records directly: rare)
+    if (live && n <= MANY) {
+      for (uint32_t k = b; k < e; k++) {
+        const float4* rec = instance_grads + 4 * (size_t)k;
+        add(a0, rec[0]); add(a1, rec[1]); add(a2, rec[2]); add(a3, rec[3]);
+      }
+    }
+  } else {
+    // The records of a wave's 64 Gaussians are one contiguous run.  It is fetched 64 records at a time with
+    // whole-wave 16-byte loads (the four lanes of a record share its 64-byte line), parked in LDS (records
+    // padded to five 16-byte words: neither access pattern has bank conflicts) and every lane then adds up its own
+    // records from there, in order.  With every lane loading its own records directly, a line passed through
+    // the first-level cache once per 16-byte part.
+    float4* mine = s_rec[threadIdx.x / GS_WAVE];
+    const uint32_t run_begin = (uint32_t)__builtin_amdgcn_readfirstlane((int)b);
+    uint32_t run_end = e;
+#pragma unroll
+    for (int d = GS_WAVE / 2; d >= 1; d >>= 1) run_end = max(run_end, (uint32_t)__shfl_xor((int)run_end, d, GS_WAVE));
+    run_end = (uint32_t)__builtin_amdgcn_readfirstlane((int)run_end);
+    for (uint32_t c = run_begin; c < run_end; c += REC_CHUNK) {
+      float4 v[4];
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        const uint32_t idx = (uint32_t)(j * GS_WAVE + lane), r = c + (idx >> 2);
+        v[j] = r < run_end ? instance_grads[4 * (size_t)r + (idx & 3u)] : make_float4(0.f, 0.f, 0.f, 0.f);
+      }
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        const uint32_t idx = (uint32_t)(j * GS_WAVE + lane);
+        mine[(idx >> 2) * REC_STRIDE4 + (idx & 3u)] = v[j];
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      const uint32_t lo = max(b, c), hi = min(e, c + REC_CHUNK);
+      for (uint32_t k = lo; k < hi; k++) {
+        const float4* rec = mine + (k - c) * REC_STRIDE4;
+        add(a0, rec[0]); add(a1, rec[1]); add(a2, rec[2]); add(a3, rec[3]);
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     }
   }
+  if (!live) return;
   // records hold the mean2D sums per pixel unit: d(pixel offset)/d(normalised coordinate) = W/2, H/2
   dL_dmean2D[i] = make_float2(a0.x * ddelx_dx, a0.y * ddely_dy);
   dL_dmean2D_abs[3 * (size_t)i] = a0.z * ddelx_dx;
