@@ -188,9 +188,13 @@ int gs_render_backward(int P, int R, const float* background, int width, int hei
 
 /* Replaces SimpleKNN::knn / distCUDA2 (KNN/simple_knn.h:17, KNN/simple_knn.cu:185-221,
  * KNN/spatial.cu:17-35): mean_dists[i] = mean squared distance from point i
- * to its three nearest other points.  points (P,3).  The reference allocates
- * its temporaries internally; here the caller passes a workspace of
- * gs_knn_workspace_bytes(P) bytes. */
+ * to its three nearest other points (a point with fewer than three finite
+ * distances reads FLT_MAX for the missing ones, as in the reference).  The
+ * result is the exact one, so it does not depend on how the points are
+ * ordered inside the call (a Hilbert curve here, Morton codes in the
+ * reference).  points (P,3).  The reference allocates its temporaries
+ * internally; here the caller passes a workspace of gs_knn_workspace_bytes(P)
+ * bytes. */
 size_t gs_knn_workspace_bytes(int P);
 int gs_knn_dist2(int P, const float* points, float* mean_dists, void* workspace, size_t workspace_bytes,
                  gs_stream_t stream);
@@ -410,8 +414,10 @@ int gs_selftest_reductions(const float* in, float* out_wave, float* out_rows, gs
 /* Optional per-stage GPU timing, the role of the reference's MyTimerOnGPU
  * (CR/timers.cu:11-79; stage names at CR/rasterizer_impl.cu:385-752): while
  * enabled, each stage of the composite entry points (preprocess_fwd,
- * tile_count, inclusive_sum, duplicate_with_keys, sort_pairs,
- * identify_tile_ranges, render_fwd, render_bwd, preprocess_bwd, knn_dist2)
+ * tile_count, bucket_scatter, tile_sort, or on the radix route inclusive_sum,
+ * duplicate_with_keys, sort_pairs, identify_tile_ranges; render_fwd,
+ * render_bwd, preprocess_bwd; knn_dist2 and its phases knn_minmax, knn_keys,
+ * knn_sort, knn_gather, knn_boxes, knn_box_mean_dist)
  * is bracketed by an event pair on its stream.  Nothing is synchronised until
  * gs_stage_timing_collect, which waits for the recorded events and writes one
  * line per stage, "name total_ms launches", into report (host buffer), then
