@@ -39,11 +39,11 @@ BYTES_PER_GAUSSIAN = {
 # distribution: the per-tile lists are built without it unless a list exceeds 8192 records.
 BYTES_PER_INSTANCE = {"sort_pairs": 128, "identify_tile_ranges": 20, "tile_sort": 28}
 # simple-knn (distCUDA2) per point: bounding box 24 B (12 read, twice: partial and final are one pass over the
-# points plus a small second one; the survey's figure), curve keys 16 B (12 in, 4 out), 32-bit radix sort with
+# points plus a small second one: the figure the reference's two reduction passes give), curve keys 16 B (12 in, 4 out), 32-bit radix sort with
 # index payload 68 B (4 B histogram read + 4 passes x (8 in + 8 out)), gather into sorted order 32 B (4 B index +
 # 12 B point in, 16 B out), box bounds 32 B (the 1024-point boxes and the 64-point leaves each read the 16 B points).
 BYTES_PER_POINT = {"knn_minmax": 24, "knn_keys": 16, "knn_sort": 68, "knn_gather": 32, "knn_boxes": 32}
-# The binning stage as a whole, in the survey's per-unit figures for the reference's algorithm on the same job:
+# The binning stage as a whole, in per-unit figures of the reference's algorithm on the same job:
 # per Gaussian tile count 16 + prefix sum 8 + key emission 20 B; per instance 12 B of key/value written, 152 B
 # for a radix sort with 8-bit digits over the 44 key bits, 8 B for the tile ranges.  The per-tile route here moves
 # less: per instance 12 B of records written and read once, then 16 B of sorted keys, emission indices and ids.
