@@ -325,19 +325,22 @@ render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
           behind_dot = __builtin_fmaf(alpha, colour_dot, oma * behind_dot);  // (alpha = 0: unchanged)
           dL_dalpha = __builtin_fmaf(dL_dalpha, T, -(bg_term * rcp1ma));
           dL_dalpha = active ? dL_dalpha : 0.f;
-          const float dL_dG = co.w * dL_dalpha;
-          const float gdx = G * dx, gdy = G * dy;
-          const float dG_ddelx = -gdx * co.x - gdy * co.y;
-          const float dG_ddely = -gdy * co.z - gdx * co.y;
-          // (the factors W/2 and H/2 from pixel to normalised coordinates are applied once per Gaussian, to the
-          // sums, by the reduction kernel; the sums of absolute values are formed inside the row reduction)
-          v[0] = dL_dG * dG_ddelx;
-          v[1] = dL_dG * dG_ddely;
-          const float hg = -0.5f * dL_dG;
-          v[4] = hg * gdx * dx;
-          v[5] = hg * gdx * dy;
-          v[6] = hg * gdy * dy;
-          v[7] = G * dL_dalpha;
+          // The per-Gaussian factors of the geometric gradients stay out of the pixel sums: with
+          // q = G dL/dalpha, u = conic (dx, dy), a pixel's terms are dL/dmean = -opacity q u,
+          // dL/dconic = -opacity/2 q (dx dx, dx dy, dy dy) and dL/dopacity = q
+          // (cuda_rasterizer/backward.cu:520-541), so the row sums q u, q (dx dx, dx dy, dy dy) and q, and the
+          // thread that hands a record over multiplies by -opacity, |opacity| (the sums of absolute values,
+          // formed inside the row reduction) and -opacity/2.  (The factors W/2 and H/2 from pixel to normalised
+          // coordinates are applied once per Gaussian by the reduction kernel.)
+          const float q = G * dL_dalpha;
+          const float ux = __builtin_fmaf(co.y, dy, co.x * dx), uy = __builtin_fmaf(co.y, dx, co.z * dy);
+          v[0] = q * ux;
+          v[1] = q * uy;
+          const float qx = q * dx;
+          v[4] = qx * dx;
+          v[5] = qx * dy;
+          v[6] = (q * dy) * dy;
+          v[7] = q;
           // lane q of the row now receives the row's total of component q
           float tot = row_transpose_reduce16_abs23(v);
           // Rows of this wave that are at the same Gaussian in this pass are merged, and the lowest of them
@@ -380,8 +383,16 @@ render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
             s_acc[w][4 * my_part + e][my_slot] = 0.f;
           }
         }
-        if (base + my_slot < count)
+        if (base + my_slot < count) {
+          const float opacity = s_co[base + my_slot].w;
+          if (my_part == 0) {  // mean2D x, y and their sums of absolute values
+            c[0] *= -opacity; c[1] *= -opacity; c[2] *= fabsf(opacity); c[3] *= fabsf(opacity);
+          } else if (my_part == 1) {  // conic x, y, w; the fourth component is the opacity gradient itself
+            const float h = -0.5f * opacity;
+            c[0] *= h; c[1] *= h; c[2] *= h;
+          }
           instance_grads[4 * (size_t)s_emis[base + my_slot] + my_part] = make_float4(c[0], c[1], c[2], c[3]);
+        }
       }
       __syncthreads();
     }
