@@ -350,20 +350,22 @@ render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
           const int key = has ? ja : -1 - row;
           const int k0 = __builtin_amdgcn_readlane(key, 0), k1 = __builtin_amdgcn_readlane(key, 16);
           const int k2 = __builtin_amdgcn_readlane(key, 32), k3 = __builtin_amdgcn_readlane(key, 48);
-          constexpr uint64_t R0 = 0xFFFFull, R1 = R0 << 16, R2 = R0 << 32, R3 = R0 << 48;
-          const uint64_t eq16 = (k0 == k1 ? R0 | R1 : 0ull) | (k2 == k3 ? R2 | R3 : 0ull);
-          const uint64_t eq32 = (k0 == k2 ? R0 | R2 : 0ull) | (k1 == k3 ? R1 | R3 : 0ull);
-          const uint64_t eq48 = (k0 == k3 ? R0 | R3 : 0ull) | (k1 == k2 ? R1 | R2 : 0ull);
-          const uint64_t follower = (k1 == k0 ? R1 : 0ull) | ((k2 == k0 || k2 == k1) ? R2 : 0ull) |
-                                    ((k3 == k0 || k3 == k1 || k3 == k2) ? R3 : 0ull);
-          if ((eq16 | eq32 | eq48) != 0ull) {  // wave-uniform
+          bool writes = has;
+          if (k0 == k1 || k0 == k2 || k0 == k3 || k1 == k2 || k1 == k3 || k2 == k3) {  // wave-uniform, uncommon
+            constexpr uint64_t R0 = 0xFFFFull, R1 = R0 << 16, R2 = R0 << 32, R3 = R0 << 48;
+            const uint64_t eq16 = (k0 == k1 ? R0 | R1 : 0ull) | (k2 == k3 ? R2 | R3 : 0ull);
+            const uint64_t eq32 = (k0 == k2 ? R0 | R2 : 0ull) | (k1 == k3 ? R1 | R3 : 0ull);
+            const uint64_t eq48 = (k0 == k3 ? R0 | R3 : 0ull) | (k1 == k2 ? R1 | R2 : 0ull);
+            const uint64_t follower = (k1 == k0 ? R1 : 0ull) | ((k2 == k0 || k2 == k1) ? R2 : 0ull) |
+                                      ((k3 == k0 || k3 == k1 || k3 == k2) ? R3 : 0ull);
             const float t16 = __shfl_xor(tot, 16, GS_WAVE), t32 = __shfl_xor(tot, 32, GS_WAVE);
             const float t48 = __shfl_xor(tot, 48, GS_WAVE);
             tot += __builtin_amdgcn_inverse_ballot_w64(eq16) ? t16 : 0.f;
             tot += __builtin_amdgcn_inverse_ballot_w64(eq32) ? t32 : 0.f;
             tot += __builtin_amdgcn_inverse_ballot_w64(eq48) ? t48 : 0.f;
+            writes = has && !__builtin_amdgcn_inverse_ballot_w64(follower);
           }
-          if (has && !__builtin_amdgcn_inverse_ballot_w64(follower) && tot != 0.f) s_acc[wave][l16][ja] += tot;
+          if (writes && tot != 0.f) s_acc[wave][l16][ja] += tot;
         }
       };
       if (select_state) walk(std::true_type{});
