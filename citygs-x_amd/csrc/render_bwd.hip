@@ -70,13 +70,12 @@ render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
                   const uint16_t* __restrict__ block_hits) {
   constexpr bool render_geo = RENDER_GEO;
   __shared__ uint32_t s_emis[BATCH];
-  __shared__ float2 s_xy[BATCH];
+  __shared__ float4 s_xyf[BATCH];  // centre x, y; the power floor; unused
   __shared__ float4 s_co[BATCH];
   __shared__ float4 s_cp[HITS ? 1 : BATCH];
   __shared__ uint16_t s_hits[HITS ? BATCH : 1];
-  __shared__ float s_floor[BATCH];
-  __shared__ float s_rgb[GS_N_RGB][BATCH];
-  __shared__ float s_map[GS_N_MAP][BATCH];
+  // colour, then the five geometry channels: eight floats per Gaussian, read as two 16-byte words
+  __shared__ float4 s_chan[BATCH][RENDER_GEO ? 2 : 1];
   // one accumulator per wave; +1: the 16 components of one Gaussian fall in 16 different banks
   __shared__ float s_acc[WAVES][NV][SUB + 1];
   __shared__ uint32_t s_list[GS_TILE_PIX / GS_WAVE][4][CHUNKS];
@@ -188,28 +187,26 @@ render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
       const float2 xy = means2D[g];
       const float4 co = conic_opacity[g];
       s_emis[tid] = emission_sorted[k_sorted];
-      s_xy[tid] = xy;
       s_co[tid] = co;
       float pfl;
       const float4 cp = cull_params(co, pfl);
       if (HITS) s_hits[tid] = block_hits[k_sorted];
       else s_cp[tid] = cp;
-      s_floor[tid] = pfl;
+      s_xyf[tid] = make_float4(xy.x, xy.y, pfl, 0.f);
       const float c0 = rgb[3 * (size_t)g], c1 = rgb[3 * (size_t)g + 1], c2 = rgb[3 * (size_t)g + 2];
-      s_rgb[0][tid] = c0;
-      s_rgb[1][tid] = c1;
-      s_rgb[2][tid] = c2;
       float mag = fmaxf(fmaxf(fabsf(c0), fabsf(c1)), fabsf(c2));
       finite = c0 == c0 && c1 == c1 && c2 == c2;
+      float m[GS_N_MAP] = {0.f, 0.f, 0.f, 0.f, 0.f};
       if (render_geo) {
 #pragma unroll
         for (int ch = 0; ch < GS_N_MAP; ch++) {
-          const float v = all_map[5 * (size_t)g + ch];
-          s_map[ch][tid] = v;
-          mag = fmaxf(mag, fabsf(v));
-          finite = finite && v == v;
+          m[ch] = all_map[5 * (size_t)g + ch];
+          mag = fmaxf(mag, fabsf(m[ch]));
+          finite = finite && m[ch] == m[ch];
         }
+        s_chan[tid][RENDER_GEO ? 1 : 0] = make_float4(m[1], m[2], m[3], m[4]);
       }
+      s_chan[tid][0] = make_float4(c0, c1, c2, m[0]);
       finite = finite && mag < __builtin_inff();
     }
     {
@@ -231,7 +228,8 @@ render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
         if (HITS) {
           nibble = (uint32_t)s_hits[valid ? jj : 0] >> (4 * wave);
         } else {
-          mu = s_xy[valid ? jj : 0];
+          const float4 xyf = s_xyf[valid ? jj : 0];
+          mu = make_float2(xyf.x, xyf.y);
           cq = s_co[valid ? jj : 0];
           cp = s_cp[valid ? jj : 0];
         }
@@ -275,12 +273,12 @@ render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
           // contributes zeros to every sum and leaves the recurrence state as it is
           // (fma(0, c, 1 * accum) == accum), so results are those of skipping it.
           // Same tests as the forward pass, on the same bits.
-          const float2 xy = s_xy[j];
+          const float4 xy = s_xyf[j];
           const float4 co = s_co[j];
           const float dx = xy.x - pfx, dy = xy.y - pfy;
           const float power = -0.5f * (co.x * dx * dx + co.z * dy * dy) - co.y * dx * dy;
           // never true for pixels outside the image (last_contributor = 0)
-          const float floor_j = s_floor[j];
+          const float floor_j = xy.z;
           // (lane masks of single comparisons, combined in scalar registers: no short-circuit branches in the loop)
           const uint64_t in_m = has_m & gs_ballot(pos < last_contributor) & gs_ballot(!(power > 0.0f)) &
                                 gs_ballot(!(power < floor_j));
@@ -304,22 +302,26 @@ render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
           const float w = alpha * T;
           const float oma = 1.f - alpha;
           float colour_dot = 0.0f;  // S
+          {
+            const float4 c4 = s_chan[j][0];
+            const float c[4] = {c4.x, c4.y, c4.z, c4.w};
 #pragma unroll
-          for (int ch = 0; ch < GS_N_RGB; ch++) {
-            const float c = (!SELECT || active) ? s_rgb[ch][j] : 0.f;
-            colour_dot = __builtin_fmaf(c, gpix[ch], colour_dot);
-            v[8 + ch] = w * gpix[ch];
-          }
-          if (render_geo) {
-#pragma unroll
-            for (int ch = 0; ch < GS_N_MAP; ch++) {
-              const float c = (!SELECT || active) ? s_map[ch][j] : 0.f;
-              colour_dot = __builtin_fmaf(c, gmap[ch], colour_dot);
-              v[11 + ch] = w * gmap[ch];
+            for (int ch = 0; ch < GS_N_RGB; ch++) {
+              colour_dot = __builtin_fmaf((!SELECT || active) ? c[ch] : 0.f, gpix[ch], colour_dot);
+              v[8 + ch] = w * gpix[ch];
             }
-          } else {
+            if (render_geo) {
+              const float4 m4 = s_chan[j][RENDER_GEO ? 1 : 0];
+              const float m[GS_N_MAP] = {c4.w, m4.x, m4.y, m4.z, m4.w};
 #pragma unroll
-            for (int ch = 0; ch < GS_N_MAP; ch++) v[11 + ch] = 0.f;
+              for (int ch = 0; ch < GS_N_MAP; ch++) {
+                colour_dot = __builtin_fmaf((!SELECT || active) ? m[ch] : 0.f, gmap[ch], colour_dot);
+                v[11 + ch] = w * gmap[ch];
+              }
+            } else {
+#pragma unroll
+              for (int ch = 0; ch < GS_N_MAP; ch++) v[11 + ch] = 0.f;
+            }
           }
           float dL_dalpha = colour_dot - behind_dot;
           behind_dot = __builtin_fmaf(alpha, colour_dot, oma * behind_dot);  // (alpha = 0: unchanged)
