@@ -25,10 +25,14 @@ HBM_PEAK_GBS = 8000.0
 
 # Algorithmic bytes per unit of each HBM-bound stage (G = Gaussian, I = (Gaussian,tile) instance).
 BYTES_PER_GAUSSIAN = {
-    "preprocess_fwd": 307 + 4 * 0,  # 44 B geometry in + 192 B SH in + 56 B geometry out + 12 B rgb + 3 B clamped
+    # 44 B geometry in + 192 B SH in + 56 B geometry out + 12 B rgb + 3 B clamped (the 307 B of the reference's
+    # interface) + 36 B: the derivative of the colour with respect to the view direction, which the forward kernel
+    # leaves for the backward kernel in a training step (that kernel then reads these 36 B instead of the 192 B of
+    # coefficients)
+    "preprocess_fwd": 307 + 36,
     "tile_count": 16,
     "inclusive_sum": 8,
-    "preprocess_bwd": 560,
+    "preprocess_bwd": 560 - 192 + 36,
     "all_map_fwd": 60,   # means 12 + scales 12 + rotations 16 in, 20 out
     "all_map_bwd": 88,   # the same 40 + 20 B of upstream gradient in, 12 + 16 out
 }
@@ -518,7 +522,12 @@ def main():
     pf = stage_report.get("preprocess_fwd", {})
     roofline = {"kernel": "preprocess_fwd_kernel", "bound": "hbm", "achieved": pf.get("GBps"), "peak": HBM_PEAK_GBS,
                 "unit": "GB/s", "frac": pf.get("frac_of_hbm_peak"), "traffic": traffic,
-                "algorithmic_bytes_per_launch": pf.get("algorithmic_bytes")}
+                "algorithmic_bytes_per_launch": pf.get("algorithmic_bytes"),
+                "note": "343 B per Gaussian: the 307 B of the reference's interface (44 geometry in, 192 SH in, 56 + 12 "
+                        "+ 3 out) and 36 B of colour derivative kept for the backward kernel, which reads them "
+                        "instead of the 192 B of coefficients"}
+    if pf.get("ms"):
+        roofline["achieved_on_reference_interface_bytes"] = round(307 * P / (pf["ms"] * 1e-3) / 1e9, 1)
     # The other half of the metric: everything between preprocess and the blend (count, prefix sum, per-tile
     # lists), one figure for the stage as a whole.
     bin_ms = sum(stage_report[k]["ms"] * stage_report[k]["launches_per_step"] for k in BINNING_STAGES

@@ -275,7 +275,7 @@ int gs_preprocess_forward(float* means2D, float* depths, int* radii, float* cov3
                           const float* means3D, const float* scales, const float* rotations, const float* shs,
                           const float* opacities, float scale_modifier, const float* viewmatrix,
                           const float* projmatrix, const float* cam_pos, float tan_fovx, float tan_fovy,
-                          int prefiltered, int debug, gs_stream_t stream) {
+                          int prefiltered, int debug, float* dcolor_ddir, gs_stream_t stream) {
   (void)prefiltered;
   GS_REQUIRE(P >= 0 && width > 0 && height > 0, "gs_preprocess_forward: bad sizes");
   if (P == 0) return 0;
@@ -295,6 +295,7 @@ int gs_preprocess_forward(float* means2D, float* depths, int* radii, float* cov3
   a.tanx = tan_fovx; a.tany = tan_fovy;
   a.radii = radii; a.means2D = means2D; a.depths = depths; a.cov3D = cov3D; a.conic_opacity = conic_opacity;
   a.rgb = rgb; a.clamped = clamped; a.tiles_touched = tiles_touched;
+  a.dcolor_ddir = sh_mode ? dcolor_ddir : nullptr;
   {
     StageScope _t("preprocess_fwd", (hipStream_t)stream);
     launch_preprocess_fwd(a, (hipStream_t)stream);
@@ -308,7 +309,7 @@ int gs_preprocess_backward(const int* radii, const float* cov3D, const uint8_t* 
                            const float* campos, float tan_fovx, float tan_fovy, const float* dL_dmean2D,
                            int mean2D_stride, const float* dL_dconic_opacity, const float* dL_dcolor,
                            float* dL_dmean3D, float* dL_dcov3D, float* dL_dscale, float* dL_drot, float* dL_dsh,
-                           float* dL_dopacity, int debug, gs_stream_t stream) {
+                           float* dL_dopacity, int debug, const float* dcolor_ddir, gs_stream_t stream) {
   GS_REQUIRE(P >= 0 && width > 0 && height > 0, "gs_preprocess_backward: bad sizes");
   if (P == 0) return 0;
   GS_REQUIRE(radii && cov3D && means3D && viewmatrix && projmatrix && dL_dmean2D && dL_dconic_opacity && dL_dmean3D,
@@ -316,12 +317,13 @@ int gs_preprocess_backward(const int* radii, const float* cov3D, const uint8_t* 
   GS_REQUIRE(mean2D_stride == 2 || mean2D_stride == 3, "gs_preprocess_backward: mean2D_stride must be 2 or 3");
   GS_REQUIRE((scales == nullptr) == (rotations == nullptr), "gs_preprocess_backward: scales and rotations go together");
   GS_REQUIRE(!scales || (dL_dscale && dL_drot), "gs_preprocess_backward: null scale/rotation gradient");
-  const bool sh_mode = shs != nullptr && M > 0 && dL_dsh != nullptr;
+  const bool sh_mode = (shs != nullptr || dcolor_ddir != nullptr) && M > 0 && dL_dsh != nullptr;
   GS_REQUIRE(!sh_mode || (campos && clamped && dL_dcolor && D >= 0 && D <= 3 && M >= (D + 1) * (D + 1) && M <= 16),
              "gs_preprocess_backward: SH mode needs campos, clamped, dL_dcolor and (D+1)^2 <= M <= 16");
   PreprocessBwdArgs a;
   a.P = P; a.D = D; a.M = sh_mode ? M : 0; a.W = width; a.H = height;
   a.means3D = means3D; a.radii = radii; a.shs = sh_mode ? shs : nullptr; a.clamped = clamped;
+  a.dcolor_ddir = sh_mode ? dcolor_ddir : nullptr;
   a.scales = scales; a.rotations = rotations; a.scale_modifier = scale_modifier;
   a.cov3D = cov3D; a.viewmatrix = viewmatrix; a.projmatrix = projmatrix; a.campos = campos;
   a.tanx = tan_fovx; a.tany = tan_fovy;

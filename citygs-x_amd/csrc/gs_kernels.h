@@ -18,6 +18,10 @@ struct PreprocessFwdArgs {
   float *means2D, *depths, *cov3D, *conic_opacity, *rgb;
   uint8_t* clamped;
   uint32_t* tiles_touched;  // optional
+  // optional (P,3,3): derivative of the three colour channels with respect to the unit view direction,
+  // [axis][channel], written for Gaussians that survive culling (SH mode); the backward kernel takes it in place of
+  // the coefficients
+  float* dcolor_ddir = nullptr;
 };
 
 struct PreprocessBwdArgs {
@@ -35,6 +39,7 @@ struct PreprocessBwdArgs {
   const float* dL_dconic_opacity;  // (P,4) packed [x, y, w, opacity]
   const float* dL_dcolor;          // (P,3), SH mode only
   float *dL_dmean3D, *dL_dcov3D /*optional*/, *dL_dsh /*optional*/, *dL_dscale, *dL_drot, *dL_dopacity /*optional*/;
+  const float* dcolor_ddir = nullptr;  // optional: what the forward kernel left (PreprocessFwdArgs::dcolor_ddir)
 };
 
 // Brackets a stage with an event pair on its stream while stage timing is enabled (gs_stage_timing_enable; the

@@ -175,6 +175,75 @@ __device__ __forceinline__ void wave_sync_lds() {
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
+// Basis values of the 16 SH terms for direction (x, y, z) (those of degrees above D are 0) and, when shv is
+// given, the derivatives of the three colour channels with respect to the direction,
+// dR_[axis][channel] = sum_k d basis_k / d axis * coefficient(k, channel): the derivative of
+// cuda_rasterizer/forward.cu:21-72, evaluated in the order of the reference's 3DGS backward.  shv = the row of
+// 16 x 3 coefficients, flat.  The forward kernel evaluates this once and the backward kernel takes its nine
+// numbers, or evaluates it itself when it is handed the coefficients instead: same code, same bits.
+template <bool WITH_DERIVATIVE>
+__device__ __forceinline__ void sh_basis_and_direction_derivative(int D, float x, float y, float z, const float* shv,
+                                                                  float* basis, float* dRdx, float* dRdy,
+                                                                  float* dRdz) {
+#pragma unroll
+  for (int k = 0; k < 16; k++) basis[k] = 0.f;
+#pragma unroll
+  for (int ch = 0; ch < 3; ch++) dRdx[ch] = dRdy[ch] = dRdz[ch] = 0.f;
+#define SHV(k, ch) (WITH_DERIVATIVE ? shv[3 * (k) + (ch)] : 0.f)
+  basis[0] = kC0;
+  if (D > 0) {
+    basis[1] = -kC1 * y;
+    basis[2] = kC1 * z;
+    basis[3] = -kC1 * x;
+#pragma unroll
+    for (int ch = 0; ch < 3; ch++) {
+      dRdx[ch] = -kC1 * SHV(3, ch);
+      dRdy[ch] = -kC1 * SHV(1, ch);
+      dRdz[ch] = kC1 * SHV(2, ch);
+    }
+    if (D > 1) {
+      const float xx = x * x, yy = y * y, zz = z * z, xy = x * y, yz = y * z, xz = x * z;
+      basis[4] = kC2[0] * xy;
+      basis[5] = kC2[1] * yz;
+      basis[6] = kC2[2] * (2.f * zz - xx - yy);
+      basis[7] = kC2[3] * xz;
+      basis[8] = kC2[4] * (xx - yy);
+#pragma unroll
+      for (int ch = 0; ch < 3; ch++) {
+        dRdx[ch] += kC2[0] * y * SHV(4, ch) + kC2[2] * 2.f * -x * SHV(6, ch) + kC2[3] * z * SHV(7, ch) +
+                    kC2[4] * 2.f * x * SHV(8, ch);
+        dRdy[ch] += kC2[0] * x * SHV(4, ch) + kC2[1] * z * SHV(5, ch) + kC2[2] * 2.f * -y * SHV(6, ch) +
+                    kC2[4] * 2.f * -y * SHV(8, ch);
+        dRdz[ch] += kC2[1] * y * SHV(5, ch) + kC2[2] * 2.f * 2.f * z * SHV(6, ch) + kC2[3] * x * SHV(7, ch);
+      }
+      if (D > 2) {
+        basis[9] = kC3[0] * y * (3.f * xx - yy);
+        basis[10] = kC3[1] * xy * z;
+        basis[11] = kC3[2] * y * (4.f * zz - xx - yy);
+        basis[12] = kC3[3] * z * (2.f * zz - 3.f * xx - 3.f * yy);
+        basis[13] = kC3[4] * x * (4.f * zz - xx - yy);
+        basis[14] = kC3[5] * z * (xx - yy);
+        basis[15] = kC3[6] * x * (xx - 3.f * yy);
+#pragma unroll
+        for (int ch = 0; ch < 3; ch++) {
+          dRdx[ch] += kC3[0] * SHV(9, ch) * 3.f * 2.f * xy + kC3[1] * SHV(10, ch) * yz +
+                      kC3[2] * SHV(11, ch) * -2.f * xy + kC3[3] * SHV(12, ch) * -3.f * 2.f * xz +
+                      kC3[4] * SHV(13, ch) * (-3.f * xx + 4.f * zz - yy) + kC3[5] * SHV(14, ch) * 2.f * xz +
+                      kC3[6] * SHV(15, ch) * 3.f * (xx - yy);
+          dRdy[ch] += kC3[0] * SHV(9, ch) * 3.f * (xx - yy) + kC3[1] * SHV(10, ch) * xz +
+                      kC3[2] * SHV(11, ch) * (-3.f * yy + 4.f * zz - xx) + kC3[3] * SHV(12, ch) * -3.f * 2.f * yz +
+                      kC3[4] * SHV(13, ch) * -2.f * xy + kC3[5] * SHV(14, ch) * -2.f * yz +
+                      kC3[6] * SHV(15, ch) * -3.f * 2.f * xy;
+          dRdz[ch] += kC3[1] * SHV(10, ch) * xy + kC3[2] * SHV(11, ch) * 4.f * 2.f * yz +
+                      kC3[3] * SHV(12, ch) * 3.f * (2.f * zz - xx - yy) + kC3[4] * SHV(13, ch) * 4.f * 2.f * xz +
+                      kC3[5] * SHV(14, ch) * (xx - yy);
+        }
+      }
+    }
+  }
+#undef SHV
+}
+
 // The same evaluation, one coefficient at a time: B[k] is everything of term k but the coefficient (the products
 // in sh_channel associate from the left, so term k = B[k] * c[k] is the same rounding), and sh_accumulate<K> is
 // the step of the running sum that takes in coefficient K.  Coefficients of degrees above `deg` are left out.
@@ -225,9 +294,9 @@ __device__ __forceinline__ void sh_third_fetch(const float4* __restrict__ wave_r
   }
 }
 
-template <int PHASE>
+template <int PHASE, bool KEEP>
 __device__ __forceinline__ void sh_third_fold(int deg, const float* B, const float4* v, float4* lds, int lane,
-                                              float* res) {
+                                              float* res, float* keep) {
   wave_sync_lds();  // (everyone has read the previous third)
 #pragma unroll
   for (int j = 0; j < 4; j++) {
@@ -240,6 +309,10 @@ __device__ __forceinline__ void sh_third_fold(int deg, const float* B, const flo
   for (int k = 0; k < 4; k++) {
     const float4 w = lds[lane * SH_THIRD4 + k];
     f[4 * k] = w.x; f[4 * k + 1] = w.y; f[4 * k + 2] = w.z; f[4 * k + 3] = w.w;
+  }
+  if constexpr (KEEP) {  // (the caller also wants the row itself)
+#pragma unroll
+    for (int e = 0; e < 16; e++) keep[16 * PHASE + e] = f[e];
   }
   // flat element 16 * PHASE + e of the row is coefficient (16 * PHASE + e) / 3 of channel (16 * PHASE + e) % 3
 #define GS_SH_STEP(E)                                                                                         \
@@ -282,14 +355,18 @@ __device__ __forceinline__ void wave_rows_store(float4* __restrict__ g4, int row
   }
 }
 
-__global__ void __launch_bounds__(GS_BLOCK_1D)
+// DERIV: also leave, per surviving Gaussian, the derivative of its colour with respect to the view direction
+// (nine numbers), which is all the backward kernel needs the coefficients for.
+template <bool DERIV>
+__global__ void __launch_bounds__(GS_BLOCK_1D) __attribute__((amdgpu_waves_per_eu(6)))
 preprocess_fwd_kernel(int P, int D, int M, const float* __restrict__ means, const float* __restrict__ scales,
                       float mod, const float* __restrict__ rots, const float* __restrict__ opac,
                       const float* __restrict__ shs, const float* __restrict__ Vg, const float* __restrict__ PMg,
                       const float* __restrict__ camg, int W, int H, float tanx, float tany, float fx, float fy,
                       uint32_t gx, uint32_t gy, int* __restrict__ radii, float2* __restrict__ means2D,
                       float* __restrict__ depths, float* __restrict__ cov3D, float4* __restrict__ conic_opacity,
-                      float* __restrict__ rgb, uint8_t* __restrict__ clamped, uint32_t* __restrict__ tiles_touched) {
+                      float* __restrict__ rgb, uint8_t* __restrict__ clamped, uint32_t* __restrict__ tiles_touched,
+                      float* __restrict__ dcolor_ddir) {
   __shared__ float4 s_sh[GS_BLOCK_1D / GS_WAVE][GS_WAVE * SH_THIRD4];
   const int slot = blockIdx.x * GS_BLOCK_1D + threadIdx.x;
   const bool live = slot < P;
@@ -335,16 +412,39 @@ preprocess_fwd_kernel(int P, int D, int M, const float* __restrict__ means, cons
       float4 va[4], vb[4];
       sh_third_fetch<0>(wave_rows, need, lane, va);
       sh_third_fetch<1>(wave_rows, need, lane, vb);
-      sh_third_fold<0>(D, B, va, s_sh[wave], lane, res);
+      float row[DERIV ? 48 : 1];
+      sh_third_fold<0, DERIV>(D, B, va, s_sh[wave], lane, res, row);
       sh_third_fetch<2>(wave_rows, need, lane, va);
-      sh_third_fold<1>(D, B, vb, s_sh[wave], lane, res);
-      sh_third_fold<2>(D, B, va, s_sh[wave], lane, res);
+      sh_third_fold<1, DERIV>(D, B, vb, s_sh[wave], lane, res, row);
+      sh_third_fold<2, DERIV>(D, B, va, s_sh[wave], lane, res, row);
       if (ok) {
 #pragma unroll
         for (int ch = 0; ch < 3; ch++) {
           const float r = res[ch] + 0.5f;
           clm[ch] = r < 0.0f;
           col[ch] = fmaxf(r, 0.0f);
+        }
+      }
+      if (DERIV) {
+        // the wave's 64 x 9 numbers leave as nine runs of consecutive floats (through the LDS rows the
+        // coefficients came in by); rows of culled Gaussians hold zeros
+        float basis[16], dR[3][3];
+        sh_basis_and_direction_derivative<true>(D, x, y, z, row, basis, dR[0], dR[1], dR[2]);
+        float* lds = reinterpret_cast<float*>(s_sh[wave]);
+        wave_sync_lds();
+#pragma unroll
+        for (int a = 0; a < 3; a++) {
+#pragma unroll
+          for (int ch = 0; ch < 3; ch++) lds[9 * lane + 3 * a + ch] = ok ? dR[a][ch] : 0.f;
+        }
+        wave_sync_lds();
+        const size_t wave_first = (size_t)blockIdx.x * GS_BLOCK_1D + (size_t)wave * GS_WAVE;
+        const size_t rows_left = (size_t)P > wave_first ? (size_t)P - wave_first : 0;
+        float* out = dcolor_ddir + 9 * wave_first;
+#pragma unroll
+        for (int j = 0; j < 9; j++) {
+          const size_t e = (size_t)j * GS_WAVE + (size_t)lane;
+          if (e < 9 * rows_left) out[e] = lds[e];
         }
       }
     } else if (ok) {
@@ -362,6 +462,20 @@ preprocess_fwd_kernel(int P, int D, int M, const float* __restrict__ means, cons
         const float res = sh_channel(D, x, y, z, c[ch]);
         clm[ch] = res < 0.0f;
         col[ch] = fmaxf(res, 0.0f);
+      }
+      if (DERIV && live) {
+        float row[48], basis[16], dR[3][3];
+#pragma unroll
+        for (int k = 0; k < 16; k++) {
+          row[3 * k] = c[0][k]; row[3 * k + 1] = c[1][k]; row[3 * k + 2] = c[2][k];
+        }
+        sh_basis_and_direction_derivative<true>(D, x, y, z, row, basis, dR[0], dR[1], dR[2]);
+        float* dd = dcolor_ddir + 9 * (size_t)i;
+#pragma unroll
+        for (int a = 0; a < 3; a++) {
+#pragma unroll
+          for (int ch = 0; ch < 3; ch++) dd[3 * a + ch] = dR[a][ch];
+        }
       }
     }
   }
@@ -420,6 +534,9 @@ mark_visible_kernel(int P, const float* __restrict__ means, const float* __restr
 // colour derivative (derivative of cuda_rasterizer/forward.cu:21-72, direction
 // normalisation as cuda_rasterizer/auxiliary.h:161-171).  The 3D-covariance
 // gradient stays in registers.  dL_dconic_opacity is packed [x, y, w, opacity].
+// SAVED: the forward kernel's derivative of the colours with respect to the view direction is given, and the
+// coefficient rows are not read.
+template <bool SAVED>
 __global__ void __launch_bounds__(GS_BLOCK_1D)
 preprocess_bwd_kernel(int P, int D, int M, const float* __restrict__ means, const int* __restrict__ radii,
                       const float* __restrict__ shs, const uint8_t* __restrict__ clamped,
@@ -429,13 +546,14 @@ preprocess_bwd_kernel(int P, int D, int M, const float* __restrict__ means, cons
                       const float* __restrict__ dL_dmean2D, int mean2D_stride,
                       const float4* __restrict__ dL_dconic_opacity, const float* __restrict__ dL_dcolor,
                       float* __restrict__ dL_dmean3D, float* __restrict__ dL_dcov3D_out, float* __restrict__ dL_dsh,
-                      float* __restrict__ dL_dscale, float* __restrict__ dL_drot, float* __restrict__ dL_dopacity) {
+                      float* __restrict__ dL_dscale, float* __restrict__ dL_drot, float* __restrict__ dL_dopacity,
+                      const float* __restrict__ dcolor_ddir) {
   __shared__ float4 s_rows[GS_BLOCK_1D / GS_WAVE][SH_WAVE_ROWS4];
   const int lane = threadIdx.x & (GS_WAVE - 1), wave = threadIdx.x / GS_WAVE;
   const int raw_i = blockIdx.x * GS_BLOCK_1D + threadIdx.x;
   const bool in_range = raw_i < P;
   const int i = in_range ? raw_i : P - 1;  // lanes past the end shadow the last Gaussian and store nothing
-  const bool sh_mode = (shs != nullptr) && M > 0 && (dL_dsh != nullptr);
+  const bool sh_mode = (SAVED || shs != nullptr) && M > 0 && (dL_dsh != nullptr);
   const bool sh_staged = sh_mode && M == 16;  // coefficient rows and their gradients go through LDS
   const float4 gco = dL_dconic_opacity[i];
   if (dL_dopacity && in_range) dL_dopacity[i] = gco.w;  // passthrough, rasterize_points.cu:191-194
@@ -444,7 +562,9 @@ preprocess_bwd_kernel(int P, int D, int M, const float* __restrict__ means, cons
   const bool live = in_range && radii[i] > 0;
   const size_t wave_first = (size_t)blockIdx.x * GS_BLOCK_1D + (size_t)wave * GS_WAVE;
   float4* my_row = s_rows[wave] + lane * SH_ROW4;
-  if (sh_staged) {
+  // (the coefficients are only needed for the colours' derivative with respect to the view direction; a caller
+  // that kept the forward pass's nine numbers per Gaussian saves this kernel the 192-byte rows)
+  if (sh_staged && !SAVED) {
     const uint64_t need = __ballot(live);
     if (need != 0ull)
       wave_rows_load(reinterpret_cast<const float4*>(shs) + wave_first * 12, need, s_rows[wave], lane);
@@ -527,18 +647,20 @@ preprocess_bwd_kernel(int P, int D, int M, const float* __restrict__ means, cons
       float* gsh = dL_dsh + (size_t)i * M * 3;
       // the Gaussian's coefficients, in registers; 16-coefficient rows (192 bytes) move as twelve 16-byte words
       float shv[48];
-      if (M == 16) {
+      if (!SAVED) {
+        if (M == 16) {
 #pragma unroll
-        for (int j = 0; j < 12; j++) {
-          const float4 v = my_row[j];
-          shv[4 * j] = v.x;
-          shv[4 * j + 1] = v.y;
-          shv[4 * j + 2] = v.z;
-          shv[4 * j + 3] = v.w;
+          for (int j = 0; j < 12; j++) {
+            const float4 v = my_row[j];
+            shv[4 * j] = v.x;
+            shv[4 * j + 1] = v.y;
+            shv[4 * j + 2] = v.z;
+            shv[4 * j + 3] = v.w;
+          }
+        } else {
+#pragma unroll
+          for (int e = 0; e < 48; e++) shv[e] = e < 3 * M ? sh[e] : 0.f;
         }
-      } else {
-#pragma unroll
-        for (int e = 0; e < 48; e++) shv[e] = e < 3 * M ? sh[e] : 0.f;
       }
       const float d0[3] = {mean[0] - cam.campos[0], mean[1] - cam.campos[1], mean[2] - cam.campos[2]};
       const float s2 = dot3(d0, d0);
@@ -548,62 +670,19 @@ preprocess_bwd_kernel(int P, int D, int M, const float* __restrict__ means, cons
 #pragma unroll
       for (int ch = 0; ch < 3; ch++) gr[ch] = dL_dcolor[3 * (size_t)i + ch] * (clamped[3 * (size_t)i + ch] ? 0.f : 1.f);
       float basis[16];
-#pragma unroll
-      for (int k = 0; k < 16; k++) basis[k] = 0.f;
-      float dRdx[3] = {0.f, 0.f, 0.f}, dRdy[3] = {0.f, 0.f, 0.f}, dRdz[3] = {0.f, 0.f, 0.f};
-#define SHV(k, ch) shv[3 * (k) + (ch)]
-      basis[0] = kC0;
-      if (D > 0) {
-        basis[1] = -kC1 * y;
-        basis[2] = kC1 * z;
-        basis[3] = -kC1 * x;
+      float dRdx[3], dRdy[3], dRdz[3];
+      if (SAVED) {
+        sh_basis_and_direction_derivative<false>(D, x, y, z, nullptr, basis, dRdx, dRdy, dRdz);
+        const float* dd = dcolor_ddir + 9 * (size_t)i;
 #pragma unroll
         for (int ch = 0; ch < 3; ch++) {
-          dRdx[ch] = -kC1 * SHV(3, ch);
-          dRdy[ch] = -kC1 * SHV(1, ch);
-          dRdz[ch] = kC1 * SHV(2, ch);
+          dRdx[ch] = dd[ch];
+          dRdy[ch] = dd[3 + ch];
+          dRdz[ch] = dd[6 + ch];
         }
-        if (D > 1) {
-          const float xx = x * x, yy = y * y, zz = z * z, xy = x * y, yz = y * z, xz = x * z;
-          basis[4] = kC2[0] * xy;
-          basis[5] = kC2[1] * yz;
-          basis[6] = kC2[2] * (2.f * zz - xx - yy);
-          basis[7] = kC2[3] * xz;
-          basis[8] = kC2[4] * (xx - yy);
-#pragma unroll
-          for (int ch = 0; ch < 3; ch++) {
-            dRdx[ch] += kC2[0] * y * SHV(4, ch) + kC2[2] * 2.f * -x * SHV(6, ch) + kC2[3] * z * SHV(7, ch) +
-                        kC2[4] * 2.f * x * SHV(8, ch);
-            dRdy[ch] += kC2[0] * x * SHV(4, ch) + kC2[1] * z * SHV(5, ch) + kC2[2] * 2.f * -y * SHV(6, ch) +
-                        kC2[4] * 2.f * -y * SHV(8, ch);
-            dRdz[ch] += kC2[1] * y * SHV(5, ch) + kC2[2] * 2.f * 2.f * z * SHV(6, ch) + kC2[3] * x * SHV(7, ch);
-          }
-          if (D > 2) {
-            basis[9] = kC3[0] * y * (3.f * xx - yy);
-            basis[10] = kC3[1] * xy * z;
-            basis[11] = kC3[2] * y * (4.f * zz - xx - yy);
-            basis[12] = kC3[3] * z * (2.f * zz - 3.f * xx - 3.f * yy);
-            basis[13] = kC3[4] * x * (4.f * zz - xx - yy);
-            basis[14] = kC3[5] * z * (xx - yy);
-            basis[15] = kC3[6] * x * (xx - 3.f * yy);
-#pragma unroll
-            for (int ch = 0; ch < 3; ch++) {
-              dRdx[ch] += kC3[0] * SHV(9, ch) * 3.f * 2.f * xy + kC3[1] * SHV(10, ch) * yz +
-                          kC3[2] * SHV(11, ch) * -2.f * xy + kC3[3] * SHV(12, ch) * -3.f * 2.f * xz +
-                          kC3[4] * SHV(13, ch) * (-3.f * xx + 4.f * zz - yy) + kC3[5] * SHV(14, ch) * 2.f * xz +
-                          kC3[6] * SHV(15, ch) * 3.f * (xx - yy);
-              dRdy[ch] += kC3[0] * SHV(9, ch) * 3.f * (xx - yy) + kC3[1] * SHV(10, ch) * xz +
-                          kC3[2] * SHV(11, ch) * (-3.f * yy + 4.f * zz - xx) + kC3[3] * SHV(12, ch) * -3.f * 2.f * yz +
-                          kC3[4] * SHV(13, ch) * -2.f * xy + kC3[5] * SHV(14, ch) * -2.f * yz +
-                          kC3[6] * SHV(15, ch) * -3.f * 2.f * xy;
-              dRdz[ch] += kC3[1] * SHV(10, ch) * xy + kC3[2] * SHV(11, ch) * 4.f * 2.f * yz +
-                          kC3[3] * SHV(12, ch) * 3.f * (2.f * zz - xx - yy) + kC3[4] * SHV(13, ch) * 4.f * 2.f * xz +
-                          kC3[5] * SHV(14, ch) * (xx - yy);
-            }
-          }
-        }
+      } else {
+        sh_basis_and_direction_derivative<true>(D, x, y, z, shv, basis, dRdx, dRdy, dRdz);
       }
-#undef SHV
       if (M == 16) {
 #pragma unroll
         for (int j = 0; j < 12; j++)
@@ -703,10 +782,14 @@ int launch_preprocess_fwd(const PreprocessFwdArgs& a, hipStream_t stream) {
   const float fy = a.H / (2.0f * a.tany);  // cuda_rasterizer/rasterizer_impl.cu:371-372
   const float fx = a.W / (2.0f * a.tanx);
   const int blocks = (a.P + GS_BLOCK_1D - 1) / GS_BLOCK_1D;
-  hipLaunchKernelGGL(preprocess_fwd_kernel, dim3(blocks), dim3(GS_BLOCK_1D), 0, stream, a.P, a.D, a.M, a.means3D,
-                     a.scales, a.scale_modifier, a.rotations, a.opacities, a.shs, a.viewmatrix, a.projmatrix,
-                     a.campos, a.W, a.H, a.tanx, a.tany, fx, fy, gx, gy, a.radii, (float2*)a.means2D, a.depths,
-                     a.cov3D, (float4*)a.conic_opacity, a.rgb, a.clamped, a.tiles_touched);
+  auto go = [&](auto kernel) {
+    hipLaunchKernelGGL(kernel, dim3(blocks), dim3(GS_BLOCK_1D), 0, stream, a.P, a.D, a.M, a.means3D, a.scales,
+                       a.scale_modifier, a.rotations, a.opacities, a.shs, a.viewmatrix, a.projmatrix, a.campos, a.W,
+                       a.H, a.tanx, a.tany, fx, fy, gx, gy, a.radii, (float2*)a.means2D, a.depths, a.cov3D,
+                       (float4*)a.conic_opacity, a.rgb, a.clamped, a.tiles_touched, a.dcolor_ddir);
+  };
+  if (a.dcolor_ddir != nullptr && a.shs != nullptr && a.M > 0) go(preprocess_fwd_kernel<true>);
+  else go(preprocess_fwd_kernel<false>);
   return 0;
 }
 
@@ -735,11 +818,15 @@ int launch_preprocess_bwd(const PreprocessBwdArgs& a, hipStream_t stream) {
   const float h_y = a.H / (2.0f * a.tany);
   const float h_x = a.W / (2.0f * a.tanx);
   const int blocks = (a.P + GS_BLOCK_1D - 1) / GS_BLOCK_1D;
-  hipLaunchKernelGGL(preprocess_bwd_kernel, dim3(blocks), dim3(GS_BLOCK_1D), 0, stream, a.P, a.D, a.M, a.means3D,
-                     a.radii, a.shs, a.clamped, a.scales, a.rotations, a.scale_modifier, a.cov3D, a.viewmatrix,
-                     a.projmatrix, a.campos, h_x, h_y, a.tanx, a.tany, a.dL_dmean2D, a.mean2D_stride,
-                     (const float4*)a.dL_dconic_opacity, a.dL_dcolor, a.dL_dmean3D, a.dL_dcov3D, a.dL_dsh,
-                     a.dL_dscale, a.dL_drot, a.dL_dopacity);
+  auto go = [&](auto kernel) {
+    hipLaunchKernelGGL(kernel, dim3(blocks), dim3(GS_BLOCK_1D), 0, stream, a.P, a.D, a.M, a.means3D, a.radii, a.shs,
+                       a.clamped, a.scales, a.rotations, a.scale_modifier, a.cov3D, a.viewmatrix, a.projmatrix,
+                       a.campos, h_x, h_y, a.tanx, a.tany, a.dL_dmean2D, a.mean2D_stride,
+                       (const float4*)a.dL_dconic_opacity, a.dL_dcolor, a.dL_dmean3D, a.dL_dcov3D, a.dL_dsh,
+                       a.dL_dscale, a.dL_drot, a.dL_dopacity, a.dcolor_ddir);
+  };
+  if (a.dcolor_ddir != nullptr) go(preprocess_bwd_kernel<true>);
+  else go(preprocess_bwd_kernel<false>);
   return 0;
 }
 

@@ -79,6 +79,18 @@ def preprocess_gaussians(means3D, scales, rotations, sh, opacity, scale_modifier
                          tan_fovy, image_height, image_width, degree, campos, prefiltered, debug, args):
     """rasterize_points.cu:63-143.  A 3-D `sh` (P,M,3) switches the SH colour
     step on; any other shape keeps the reference behaviour (rgb stays zero)."""
+    return preprocess_gaussians_ex(means3D, scales, rotations, sh, opacity, scale_modifier, viewmatrix, projmatrix,
+                                   tan_fovx, tan_fovy, image_height, image_width, degree, campos, prefiltered, debug,
+                                   args)[0]
+
+
+def preprocess_gaussians_ex(means3D, scales, rotations, sh, opacity, scale_modifier, viewmatrix, projmatrix, tan_fovx,
+                            tan_fovy, image_height, image_width, degree, campos, prefiltered, debug, args,
+                            want_direction_derivative=False):
+    """preprocess_gaussians plus what the reference's tuple has no slot for: returns (tuple, dcolor_ddir).  With
+    want_direction_derivative (and SH colours) dcolor_ddir is the (P,3,3) derivative of every surviving Gaussian's
+    colour with respect to the unit view direction; handed to preprocess_gaussians_backward it replaces the
+    coefficients there (same gradients, and the backward pass does not read the 192-byte rows).  Otherwise None."""
     if means3D.ndimension() != 2 or means3D.size(1) != 3:
         raise RuntimeError("means3D must have dimensions (num_points, 3)")
     means3D = _f32c(means3D, "means3D")
@@ -86,9 +98,9 @@ def preprocess_gaussians(means3D, scales, rotations, sh, opacity, scale_modifier
     P = means3D.shape[0]
     f32 = dict(dtype=torch.float32, device=dev)
     if P == 0:
-        return (0, torch.zeros(0, 2, **f32), torch.zeros(0, **f32), torch.zeros(0, dtype=torch.int32, device=dev),
-                torch.zeros(0, 6, **f32), torch.zeros(0, 4, **f32), torch.zeros(0, 3, **f32),
-                torch.zeros(0, 3, dtype=torch.bool, device=dev))
+        return ((0, torch.zeros(0, 2, **f32), torch.zeros(0, **f32), torch.zeros(0, dtype=torch.int32, device=dev),
+                 torch.zeros(0, 6, **f32), torch.zeros(0, 4, **f32), torch.zeros(0, 3, **f32),
+                 torch.zeros(0, 3, dtype=torch.bool, device=dev)), None)
     means2D = torch.empty(P, 2, **f32)
     depths = torch.empty(P, **f32)
     radii = torch.empty(P, dtype=torch.int32, device=dev)
@@ -101,19 +113,22 @@ def preprocess_gaussians(means3D, scales, rotations, sh, opacity, scale_modifier
     sh_mode = sh is not None and sh.dim() == 3 and sh.shape[0] == P
     M = sh.shape[1] if sh_mode else 0
     shc = _f32c(sh, "sh") if sh_mode else None
+    ddir = torch.empty(P, 3, 3, **f32) if (sh_mode and want_direction_derivative) else None
     with torch.cuda.device(dev):
         _n.check(_lib.gs_preprocess_forward(
             _ptr(means2D), _ptr(depths), _ptr(radii), _ptr(cov3D), _ptr(conic_opacity), _ptr(rgb), _ptr(clamped), None,
             P, int(degree), M, int(image_width), int(image_height), _ptr(means3D), _ptr(scales), _ptr(rotations),
             _ptr(shc), _ptr(opacity), float(scale_modifier), _ptr(vm), _ptr(pm), _ptr(cp), float(tan_fovx),
-            float(tan_fovy), int(bool(prefiltered)), int(bool(debug)), _stream(dev)), "preprocess_gaussians")
-    return 0, means2D, depths, radii, cov3D, conic_opacity, rgb, clamped
+            float(tan_fovy), int(bool(prefiltered)), int(bool(debug)), _ptr(ddir), _stream(dev)),
+            "preprocess_gaussians")
+    return (0, means2D, depths, radii, cov3D, conic_opacity, rgb, clamped), ddir
 
 
 def preprocess_gaussians_backward(radii, cov3D, clamped, means3D, scales, rotations, sh, scale_modifier, viewmatrix,
                                   projmatrix, tan_fovx, tan_fovy, image_height, image_width, degree, campos,
-                                  dL_dmeans2D, dL_dconic_opacity, dL_dcolors, R, debug, args):
-    """rasterize_points.cu:146-234.  dL_dmeans2D may be (P,2) or (P,3)."""
+                                  dL_dmeans2D, dL_dconic_opacity, dL_dcolors, R, debug, args, dcolor_ddir=None):
+    """rasterize_points.cu:146-234.  dL_dmeans2D may be (P,2) or (P,3).  dcolor_ddir: what
+    preprocess_gaussians_ex returned for the same inputs, or None."""
     means3D = _f32c(means3D, "means3D")
     dev = means3D.device
     P = means3D.shape[0]
@@ -142,7 +157,8 @@ def preprocess_gaussians_backward(radii, cov3D, clamped, means3D, scales, rotati
             int(image_width), int(image_height), _ptr(means3D), _ptr(scales), _ptr(rotations), _ptr(shc),
             float(scale_modifier), _ptr(vm), _ptr(pm), _ptr(cp), float(tan_fovx), float(tan_fovy), _ptr(g2),
             int(g2.shape[1]), _ptr(gco), _ptr(gcol), _ptr(dL_dmeans3D), None, _ptr(dL_dscales), _ptr(dL_drotations),
-            _ptr(dL_dsh) if sh_mode else None, _ptr(dL_dopacity), int(bool(debug)), _stream(dev)),
+            _ptr(dL_dsh) if sh_mode else None, _ptr(dL_dopacity), int(bool(debug)),
+            _ptr(dcolor_ddir) if (sh_mode and dcolor_ddir is not None) else None, _stream(dev)),
             "preprocess_gaussians_backward")
     return dL_dmeans3D, dL_dscales, dL_drotations, dL_dsh, dL_dopacity
 

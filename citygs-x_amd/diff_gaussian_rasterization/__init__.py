@@ -45,13 +45,18 @@ class _PreprocessGaussians(torch.autograd.Function):
     @staticmethod
     def forward(ctx, means3D, scales, rotations, sh, opacities, raster_settings, cuda_args):
         rs = raster_settings
-        (num_rendered, means2D, depths, radii, cov3D, conic_opacity, rgb, clamped) = _C.preprocess_gaussians(
+        # (when a backward pass can follow, the forward kernel also leaves the colours' derivative with respect to
+        # the view direction, nine numbers per Gaussian, which is all the backward kernel needs the coefficients for)
+        (num_rendered, means2D, depths, radii, cov3D, conic_opacity, rgb, clamped), ddir = _C.preprocess_gaussians_ex(
             means3D, scales, rotations, sh, opacities, rs.scale_modifier, rs.viewmatrix, rs.projmatrix, rs.tanfovx,
-            rs.tanfovy, rs.image_height, rs.image_width, rs.sh_degree, rs.campos, rs.prefiltered, rs.debug, cuda_args)
+            rs.tanfovy, rs.image_height, rs.image_width, rs.sh_degree, rs.campos, rs.prefiltered, rs.debug, cuda_args,
+            want_direction_derivative=any(ctx.needs_input_grad[:5]))
         ctx.raster_settings = rs
         ctx.cuda_args = cuda_args
         ctx.num_rendered = num_rendered
-        ctx.save_for_backward(means3D, scales, rotations, sh, radii, cov3D, clamped)
+        ctx.has_ddir = ddir is not None
+        ctx.save_for_backward(means3D, scales, rotations, sh, radii, cov3D, clamped,
+                              *([ddir] if ddir is not None else []))
         ctx.mark_non_differentiable(radii, depths)
         # no zero tensors for the outputs nobody differentiates (radii, depths): backward fills in what it needs
         ctx.set_materialize_grads(False)
@@ -60,7 +65,8 @@ class _PreprocessGaussians(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_means2D, grad_rgb, grad_conic_opacity, grad_radii, grad_depths):
         rs = ctx.raster_settings
-        means3D, scales, rotations, sh, radii, cov3D, clamped = ctx.saved_tensors
+        means3D, scales, rotations, sh, radii, cov3D, clamped = ctx.saved_tensors[:7]
+        ddir = ctx.saved_tensors[7] if ctx.has_ddir else None
         P = means3D.shape[0]
         if grad_means2D is None:
             grad_means2D = means3D.new_zeros(P, 2)
@@ -71,7 +77,7 @@ class _PreprocessGaussians(torch.autograd.Function):
         dL_dmeans3D, dL_dscales, dL_drotations, dL_dsh, dL_dopacity = _C.preprocess_gaussians_backward(
             radii, cov3D, clamped, means3D, scales, rotations, sh, rs.scale_modifier, rs.viewmatrix, rs.projmatrix,
             rs.tanfovx, rs.tanfovy, rs.image_height, rs.image_width, rs.sh_degree, rs.campos, grad_means2D,
-            grad_conic_opacity, grad_rgb, ctx.num_rendered, rs.debug, ctx.cuda_args)
+            grad_conic_opacity, grad_rgb, ctx.num_rendered, rs.debug, ctx.cuda_args, dcolor_ddir=ddir)
         if dL_dsh.shape != sh.shape:
             dL_dsh = torch.zeros_like(sh)
         return dL_dmeans3D, dL_dscales, dL_drotations, dL_dsh, dL_dopacity, None, None

@@ -28,9 +28,9 @@ _SIGNATURES = {
     "gs_higher_msb": (C.c_uint32, [C.c_uint32]),
     "gs_mark_visible": (_i, [_i, _vp, _vp, _vp, _vp, _vp]),
     "gs_visible_filter": (_i, [_i, _i, _i, _i, _vp, _vp, _f, _vp, _vp, _vp, _vp, _f, _f, _i, _vp, _i, _vp]),
-    "gs_preprocess_forward": (_i, [_vp] * 8 + [_i] * 5 + [_vp] * 5 + [_f] + [_vp] * 3 + [_f, _f, _i, _i, _vp]),
+    "gs_preprocess_forward": (_i, [_vp] * 8 + [_i] * 5 + [_vp] * 5 + [_f] + [_vp] * 3 + [_f, _f, _i, _i, _vp, _vp]),
     "gs_preprocess_backward": (_i, [_vp] * 3 + [_i] * 5 + [_vp] * 4 + [_f] + [_vp] * 3 + [_f, _f] + [_vp, _i] +
-                               [_vp] * 8 + [_i, _vp]),
+                               [_vp] * 8 + [_i, _vp, _vp]),
     "gs_render_forward": (_i, [RESIZE_FN, _vp, RESIZE_FN, _vp, RESIZE_FN, _vp, _i, _vp, _i, _i, _f, _f, _f, _f] +
                           [_vp] * 17 + [_i, _i, C.POINTER(_i), C.POINTER(_f), _vp, _vp, _vp]),
     "gs_render_backward_workspace_bytes": (_sz, [_i]),

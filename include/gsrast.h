@@ -66,13 +66,19 @@ int gs_visible_filter(int P, int M, int width, int height, const float* means3D,
  * degree D.  tiles_touched (P) uint32 is optional (NULL to skip): the tile
  * rectangle area of each surviving Gaussian (CR/forward.cu:258).
  * prefiltered is accepted and ignored (the reference traps the GPU when a
- * prefiltered Gaussian is culled, CR/auxiliary.h:210-214). */
+ * prefiltered Gaussian is culled, CR/auxiliary.h:210-214).
+ * dcolor_ddir (no counterpart in the reference; NULL to skip): (P,3,3), in SH
+ * mode the derivative of every surviving Gaussian's three colour channels with
+ * respect to the unit view direction, [axis][channel] (rows of culled
+ * Gaussians are not written).  It is all that gs_preprocess_backward needs the
+ * coefficients for: a caller that keeps it (36 bytes per Gaussian) saves the
+ * backward call the 192-byte coefficient rows. */
 int gs_preprocess_forward(float* means2D, float* depths, int* radii, float* cov3D, float* conic_opacity,
                           float* rgb, uint8_t* clamped, uint32_t* tiles_touched, int P, int D, int M, int width,
                           int height, const float* means3D, const float* scales, const float* rotations,
                           const float* shs, const float* opacities, float scale_modifier, const float* viewmatrix,
                           const float* projmatrix, const float* cam_pos, float tan_fovx, float tan_fovy,
-                          int prefiltered, int debug, gs_stream_t stream);
+                          int prefiltered, int debug, float* dcolor_ddir, gs_stream_t stream);
 
 /* Replaces Rasterizer::preprocessBackward (CR/rasterizer.h:86-111,
  * CR/rasterizer_impl.cu:427-489) together with the tensor repacking of
@@ -82,7 +88,9 @@ int gs_preprocess_forward(float* means2D, float* depths, int* radii, float* cov3
  * dL_dmean3D (P,3), dL_dscale (P,3), dL_drot (P,4), dL_dopacity (P) are fully
  * written.  dL_dsh: NULL in reference-compatible mode; (P,M,3) in SH mode,
  * where dL_dcolor (P,3) and clamped are read.  dL_dcov3D (P,6) is optional
- * (NULL: kept in registers). */
+ * (NULL: kept in registers).  dcolor_ddir: NULL, or what gs_preprocess_forward
+ * left for the same inputs and camera; shs is then not read and may be NULL.
+ * Same results either way, bit for bit. */
 int gs_preprocess_backward(const int* radii, const float* cov3D, const uint8_t* clamped, int P, int D, int M,
                            int width, int height, const float* means3D, const float* scales,
                            const float* rotations, const float* shs, float scale_modifier,
@@ -90,7 +98,7 @@ int gs_preprocess_backward(const int* radii, const float* cov3D, const uint8_t* 
                            float tan_fovy, const float* dL_dmean2D, int mean2D_stride,
                            const float* dL_dconic_opacity, const float* dL_dcolor, float* dL_dmean3D,
                            float* dL_dcov3D, float* dL_dscale, float* dL_drot, float* dL_dsh, float* dL_dopacity,
-                           int debug, gs_stream_t stream);
+                           int debug, const float* dcolor_ddir, gs_stream_t stream);
 
 /* No counterpart in the reference: per-call options of gs_render_forward (NULL = all defaults).  A field below
  * zero keeps its default; struct_bytes is sizeof(gs_render_options) as the caller compiled it.

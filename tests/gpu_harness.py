@@ -48,7 +48,7 @@ def grid(W, H):
     return (W + 15) // 16, (H + 15) // 16
 
 
-def preprocess_fwd(g, cam, sh_mode=True, sh_degree=3, want_tiles=True):
+def preprocess_fwd(g, cam, sh_mode=True, sh_degree=3, want_tiles=True, want_ddir=False):
     P = g["means3D"].shape[0]
     W, H = cam.image_width, cam.image_height
     o = dict(
@@ -57,6 +57,8 @@ def preprocess_fwd(g, cam, sh_mode=True, sh_degree=3, want_tiles=True):
         conic_opacity=torch.empty(P, 4, device=DEV), rgb=torch.empty(P, 3, device=DEV),
         clamped=torch.empty(P, 3, dtype=torch.uint8, device=DEV),
         tiles_touched=torch.empty(P, dtype=torch.int32, device=DEV))
+    if want_ddir:
+        o["dcolor_ddir"] = torch.empty(P, 3, 3, device=DEV)
     for v in o.values():
         v.fill_(77)  # the kernel must overwrite every element
     gd = {k: dev(v) for k, v in g.items() if torch.is_tensor(v)}
@@ -66,7 +68,8 @@ def preprocess_fwd(g, cam, sh_mode=True, sh_degree=3, want_tiles=True):
         ptr(o["means2D"]), ptr(o["depths"]), ptr(o["radii"]), ptr(o["cov3D"]), ptr(o["conic_opacity"]), ptr(o["rgb"]),
         ptr(o["clamped"]), ptr(o["tiles_touched"]) if want_tiles else None, P, sh_degree, M, W, H, ptr(gd["means3D"]),
         ptr(gd["scales"]), ptr(gd["rotations"]), ptr(gd["shs"]) if sh_mode else None, ptr(gd["opacities"]), 1.0,
-        ptr(V), ptr(PM), ptr(cp), cam.tanfovx, cam.tanfovy, 0, 1, stream()), "gs_preprocess_forward")
+        ptr(V), ptr(PM), ptr(cp), cam.tanfovx, cam.tanfovy, 0, 1, ptr(o["dcolor_ddir"]) if want_ddir else None,
+        stream()), "gs_preprocess_forward")
     torch.cuda.synchronize()
     return o, gd
 

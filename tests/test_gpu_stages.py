@@ -205,8 +205,12 @@ def test_render_backward(H, orc, cfg, P, mask, geo):
 
 
 @pytest.mark.parametrize("cfg,P", CASES)
-@pytest.mark.parametrize("sh_mode", [True, False])
+@pytest.mark.parametrize("sh_mode", [True, False, "saved"])
 def test_preprocess_backward(H, orc, cfg, P, sh_mode):
+    """sh_mode "saved": the backward call gets the forward call's derivative of the colours with respect to the
+    view direction instead of the coefficients (shs = NULL): the same bits as with the coefficients."""
+    saved = sh_mode == "saved"
+    sh_mode = bool(sh_mode)
     g, cam = _scene(cfg, P)
     W, Hh = cam.image_width, cam.image_height
     pre = H.oracle_preprocess(orc, g, cam, sh_mode=sh_mode)
@@ -227,14 +231,28 @@ def test_preprocess_backward(H, orc, cfg, P, sh_mode):
     # keep every device tensor referenced until the call has run
     t_radii, t_cov, t_clamped = H.dev(pre["radii"]), H.dev(pre["cov3D"]), H.dev(pre["clamped"])
     t_g2, t_gco, t_gcol = H.dev(g2), H.dev(gco), H.dev(gcol)
+    ddir = H.preprocess_fwd(g, cam, want_ddir=True)[0]["dcolor_ddir"] if saved else None
     H.gn.check(H.lib.gs_preprocess_backward(
         H.ptr(t_radii), H.ptr(t_cov), H.ptr(t_clamped), P, 3,
         16 if sh_mode else 0, W, Hh, H.ptr(gd["means3D"]), H.ptr(gd["scales"]), H.ptr(gd["rotations"]),
-        H.ptr(gd["shs"]) if sh_mode else None, 1.0, H.ptr(V), H.ptr(PM), H.ptr(cp), cam.tanfovx, cam.tanfovy,
+        H.ptr(gd["shs"]) if (sh_mode and not saved) else None, 1.0, H.ptr(V), H.ptr(PM), H.ptr(cp), cam.tanfovx,
+        cam.tanfovy,
         H.ptr(t_g2), 2, H.ptr(t_gco), H.ptr(t_gcol), H.ptr(o["dL_dmeans3D"]), H.ptr(o["dL_dcov3D"]),
         H.ptr(o["dL_dscales"]), H.ptr(o["dL_drotations"]), H.ptr(o["dL_dsh"]) if sh_mode else None,
-        H.ptr(o["dL_dopacity"]), 1, H.stream()), "gs_preprocess_backward")
+        H.ptr(o["dL_dopacity"]), 1, H.ptr(ddir) if saved else None, H.stream()), "gs_preprocess_backward")
     torch.cuda.synchronize()
+    if saved:
+        # against the same call with the coefficients: the same bits
+        o2 = {k: torch.full_like(v, 33.0) for k, v in o.items()}
+        H.gn.check(H.lib.gs_preprocess_backward(
+            H.ptr(t_radii), H.ptr(t_cov), H.ptr(t_clamped), P, 3, 16, W, Hh, H.ptr(gd["means3D"]), H.ptr(gd["scales"]),
+            H.ptr(gd["rotations"]), H.ptr(gd["shs"]), 1.0, H.ptr(V), H.ptr(PM), H.ptr(cp), cam.tanfovx, cam.tanfovy,
+            H.ptr(t_g2), 2, H.ptr(t_gco), H.ptr(t_gcol), H.ptr(o2["dL_dmeans3D"]), H.ptr(o2["dL_dcov3D"]),
+            H.ptr(o2["dL_dscales"]), H.ptr(o2["dL_drotations"]), H.ptr(o2["dL_dsh"]), H.ptr(o2["dL_dopacity"]), 1, None,
+            H.stream()), "gs_preprocess_backward")
+        torch.cuda.synchronize()
+        for k in o:
+            assert torch.equal(o[k], o2[k]), k
     keys = ["dL_dmeans3D", "dL_dcov3D", "dL_dscales", "dL_drotations", "dL_dopacity"] + (["dL_dsh"] if sh_mode else [])
     for k in keys:
         a, r = o[k].cpu().numpy(), ref[k]
