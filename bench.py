@@ -516,7 +516,9 @@ def main():
     tpath = os.path.join(ROOT, "profiles", "hbm_traffic.json")
     if os.path.exists(tpath):
         try:
-            traffic = json.load(open(tpath)).get("preprocess_fwd_kernel", {}).get("bytes_per_launch")
+            tj0 = json.load(open(tpath))
+            traffic = (tj0.get("preprocess_fwd_kernel<true>") or tj0.get("preprocess_fwd_kernel", {})).get(
+                "bytes_per_launch")
         except (OSError, ValueError):
             traffic = None
     pf = stage_report.get("preprocess_fwd", {})
