@@ -7,10 +7,11 @@
 // and each of its 16-lane rows a 4x4 pixel block.  Gaussians are staged in LDS
 // 128 at a time, in back-to-front order, and worked on 64 at a time:
 //   * a wave ballots, for each of its rows, which of the 64 Gaussians can touch
-//     the row's block (inflated alpha >= 1/255 ellipse against the block) and
-//     lie in front of the row's deepest contributor; the four rows then walk
-//     their own bit lists concurrently, so one pass of the loop handles up to
-//     four Gaussians;
+//     the row's block (the forward kernel's own answer, 16 bits per instance,
+//     when the caller hands them on; otherwise the inflated alpha >= 1/255
+//     ellipse is tested against the block again) and lie in front of the
+//     row's deepest contributor; the four rows then walk their own bit lists
+//     concurrently, so one pass of the loop handles up to four Gaussians;
 //   * the 16 partial sums of a Gaussian (mean2D x/y, |mean2D| x/y, conic
 //     x/y/w, opacity, colour 3, map 5) are reduced over the row's 16 lanes by
 //     a transposing DPP reduction (15 additions instead of 64) that leaves
@@ -31,9 +32,10 @@
 // cuda_rasterizer/backward.cu:510-563.)
 // The per-pixel arithmetic follows the CPU statement's operation for operation
 // (transmittance, reciprocal, weights, the derivative of the exponent), with
-// three exceptions: the order in which pixels are summed; the constant factors
-// W/2, H/2 of the mean2D gradients, which multiply the sums instead of every
-// term; and the blend of everything behind a Gaussian, which the reference
+// three exceptions: the order in which pixels are summed; the factors that are
+// constant per Gaussian (W/2, H/2, the opacity and -1/2 of the geometric
+// gradients), which multiply the sums instead of every term; and the blend of
+// everything behind a Gaussian, which the reference
 // keeps per channel and this kernel keeps as its dot product with the upstream
 // gradients (one recurrence instead of eight: see `behind_dot`).  Gradients
 // therefore agree with a CPU evaluation to rounding (rel. L2 of the order of
