@@ -69,7 +69,7 @@ def test_training_resolution_against_torch_statements():
     loss2.backward()
     assert torch.equal(l1, rl1)
     assert float((ss.detach() - rss.detach()).abs().max()) <= 2e-5
-    assert abs(float(loss1) - float(loss2)) <= 1e-6
+    assert abs(float(loss1.detach()) - float(loss2.detach())) <= 1e-6
     assert float((x1.grad - x2.grad).norm() / x2.grad.norm()) <= 1e-4
     # the two single-map functions with the reference's names return the same maps
     assert torch.equal(gs_loss.pixelwise_l1_with_mask(a, b, mask), l1.detach())
