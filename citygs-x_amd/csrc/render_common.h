@@ -89,6 +89,21 @@ __device__ __forceinline__ float4 cull_params(float4 co, float& power_floor) {
   return cp;
 }
 
+// cull_params in two words.  A trusted conic keeps (1/A, 1/C), both positive and finite, and its q_max is
+// -2 power_floor (q_max = 2 tau and power_floor = -tau there: tau stays far below 87 for an opacity under 1e30).
+// x = -1 stands for "the opacity alone rules every pixel out", x = +infinity for "the conic cannot be trusted".
+__device__ __forceinline__ float2 pack_cull_params(float4 cp) {
+  if (cp.z < 0.f) return make_float2(-1.0f, 0.f);
+  if (cp.z == __builtin_inff()) return make_float2(__builtin_inff(), 0.f);
+  return make_float2(cp.x, cp.y);
+}
+__device__ __forceinline__ float4 unpack_cull_params(float2 e, float power_floor) {
+  const bool never = e.x < 0.f, always = e.x == __builtin_inff();
+  const bool plain = !(never || always);
+  return make_float4(plain ? e.x : 0.f, plain ? e.y : 0.f,
+                     never ? -1.0f : (always ? __builtin_inff() : -2.0f * power_floor), 0.f);
+}
+
 // Can any point of the pixel block [bx0, bx0+ext] x [by0, by0+ext] have q <= q_max?  q is convex, so over
 // the block it is smallest either at the centre (inside the block: 0) or on one of the two block edges that
 // face the centre; along an edge it is a parabola whose minimiser is clamped to the edge.  The block is

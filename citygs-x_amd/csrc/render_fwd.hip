@@ -7,14 +7,19 @@
 // depth-sorted Gaussians are staged through LDS in batches of 256 (index,
 // centre, conic+opacity, colour, the five geometry channels, the culling
 // parameters and the exponent below which alpha < 1/255 is certain).
-// Per batch a wave ballots, for each of its four rows, which Gaussians'
-// alpha >= 1/255 ellipses (slightly inflated) can reach the row's 4x4 block
-// and leaves those bit lists in LDS; the four rows
-// then walk their own lists concurrently (find-first-set on a per-row mask),
+// Per batch a wave tests, for each of its four rows, which Gaussians' alpha >= 1/255
+// ellipses (slightly inflated) can reach the row's 4x4 block, and compacts the
+// slot numbers of those that can into a byte list per row in LDS (a lane's
+// place in the list is the number of hits in the lanes below it); the four rows
+// then walk their own lists concurrently, entry n of each in pass n,
 // so one pass of the loop blends up to four different Gaussians and a
 // Gaussian that cannot touch a block costs that row nothing.  Pixels keep
 // their own front-to-back order, which is all the blend needs.  A row stops
 // when its 16 pixels have saturated; a batch is not fetched once all have.
+// The same hits, 16 bits per sorted instance, are left for the backward pass.
+// Registers decide how many waves a SIMD holds here (72 allow seven), and a
+// kernel that spills to scratch memory starts its waves much more slowly, so
+// index arithmetic is kept from being hoisted across the blend loop.
 //
 // The per-pixel arithmetic keeps a fixed operation order, so contributor
 // counts and images match a CPU evaluation bit for bit; exp() is gs_expf.
@@ -31,7 +36,14 @@ namespace gs {
 namespace {
 
 constexpr int BATCH = GS_TILE_PIX;
-constexpr int CHUNKS = BATCH / 32;  // 32-bit list words per row and batch
+
+// The value itself, but opaque to the optimizer from here on: what is computed from it stays behind this point
+// instead of being hoisted out of the batch loop, where every hoisted LDS address holds a register through the
+// blend loop (the kernel has none to spare: one more costs a wave per SIMD, or scratch memory).
+__device__ __forceinline__ int not_hoisted(int x) {
+  asm volatile("" : "+v"(x));
+  return x;
+}
 
 // MAX_DEPTH adds one output with no counterpart in the reference: per pixel, the view-space depth of the Gaussian
 // that blends with the largest weight alpha * T (the front-most one among equals; 0 where nothing blends).  It
@@ -53,15 +65,20 @@ render_fwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
   // launched ahead of the host's decision on how the per-tile lists are built: nothing to do if they were not
   if (fits_word != nullptr && *fits_word == 0u) return;
   __shared__ float s_depth[MAX_DEPTH ? BATCH : 1];
-  __shared__ int s_id[BATCH];
   __shared__ float2 s_xy[BATCH];
   __shared__ float4 s_co[BATCH];
-  __shared__ float4 s_cp[BATCH];
+  __shared__ float2 s_cull[BATCH];  // packed_cull_params
   __shared__ float s_floor[BATCH];
   __shared__ float s_rgb[GS_N_RGB][BATCH];
   __shared__ float s_map[GS_N_MAP][BATCH];
-  __shared__ int s_obs[BATCH];
-  __shared__ uint32_t s_list[GS_TILE_PIX / GS_WAVE][4][CHUNKS];
+  // observation counts of slots 2w and 2w + 1 in the low and high half of word w (a count is at most 256)
+  __shared__ uint32_t s_obs[BATCH / 2];
+  // the four rows' lists of every wave: the slots of the batch that can touch the row's block, one byte each, in
+  // depth order; bytes behind a list's end are 0
+  __shared__ __attribute__((aligned(16))) uint32_t s_idx[GS_TILE_PIX / GS_WAVE][4][BATCH / 4];
+  // what the backward pass is left: byte `wave` of word p holds that wave's four row bits for slot 2p (low
+  // half) and slot 2p + 1 (high half)
+  __shared__ uint32_t s_hits[BATCH / 2];
   __shared__ int s_done[GS_TILE_PIX / GS_WAVE];
   __shared__ int s_bad[GS_TILE_PIX / GS_WAVE];
   __shared__ int s_red[2][GS_TILE_PIX / GS_WAVE];
@@ -121,61 +138,92 @@ render_fwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
     // Gaussian's colour and geometry channels are finite; a batch that holds a non-finite one is walked by
     // the variant of the loop that selects instead (below).
     bool finite = true;
-    if (tid < count) {
-      const uint32_t g = point_list[range.x + (uint32_t)i * BATCH + tid];
+    const int ts = not_hoisted(tid);
+    if (ts < count) {
+      const uint32_t g = point_list[range.x + (uint32_t)i * BATCH + ts];
       const float2 xy = means2D[g];
       const float4 co = conic_opacity[g];
       float pfl;
-      s_id[tid] = (int)g;
-      s_xy[tid] = xy;
-      s_co[tid] = co;
-      s_cp[tid] = cull_params(co, pfl);
-      s_floor[tid] = pfl;
+      s_xy[ts] = xy;
+      s_co[ts] = co;
+      s_cull[ts] = pack_cull_params(cull_params(co, pfl));
+      s_floor[ts] = pfl;
       const float c0 = rgb[3 * (size_t)g], c1 = rgb[3 * (size_t)g + 1], c2 = rgb[3 * (size_t)g + 2];
-      s_rgb[0][tid] = c0;
-      s_rgb[1][tid] = c1;
-      s_rgb[2][tid] = c2;
+      s_rgb[0][ts] = c0;
+      s_rgb[1][ts] = c1;
+      s_rgb[2][ts] = c2;
       float mag = fmaxf(fmaxf(fabsf(c0), fabsf(c1)), fabsf(c2));
       finite = c0 == c0 && c1 == c1 && c2 == c2;
       if (render_geo) {
 #pragma unroll
         for (int ch = 0; ch < GS_N_MAP; ch++) {
           const float v = all_map[5 * (size_t)g + ch];
-          s_map[ch][tid] = v;
+          s_map[ch][ts] = v;
           mag = fmaxf(mag, fabsf(v));
           finite = finite && v == v;
         }
       }
       finite = finite && mag < __builtin_inff();
-      if (MAX_DEPTH) s_depth[tid] = depths[g];
+      if (MAX_DEPTH) s_depth[ts] = depths[g];
     }
     {
       const uint64_t bad_m = gs_ballot(!finite);
       if (lane == 0) s_bad[wave] = bad_m != 0ull;
     }
-    s_obs[tid] = 0;
+    if (ts < BATCH / 2) {
+      s_obs[ts] = 0u;
+      s_hits[ts] = 0u;
+    }
+    static_assert(sizeof(s_idx) == 16 * GS_TILE_PIX, "four words of the lists per thread");
+    *reinterpret_cast<uint4*>(&s_idx[0][0][0] + 4 * ts) = make_uint4(0u, 0u, 0u, 0u);
     __syncthreads();
     const bool select_blend = (s_bad[0] | s_bad[1] | s_bad[2] | s_bad[3]) != 0;
 
     if (alive_mask != 0ull) {
-      // per-row lists: bit b of word c of row r = Gaussian 32c+b of the batch can touch row r's 4x4 block
+      // Per-row lists.  A wave looks at 64 slots at a time, lane = slot: the lanes whose Gaussian can touch row
+      // r's 4x4 block append their slot numbers to the row's list, in lane order (a lane's place is the number of
+      // set bits below its own).
+      uint32_t len0 = 0u, len1 = 0u, len2 = 0u, len3 = 0u;  // the lists' lengths (wave-uniform)
+      const int tb = not_hoisted(tid);
+      const int lane_b = tb & (GS_WAVE - 1), wave_b = tb / GS_WAVE;
 #pragma unroll
       for (int k = 0; k < BATCH / GS_WAVE; k++) {
-        const int jj = k * GS_WAVE + lane;
+        if (k * GS_WAVE >= count) break;  // (the last batch of a list is rarely full)
+        const int jj = k * GS_WAVE + lane_b;
         const bool valid = jj < count;
         const uint64_t valid_m = gs_ballot(valid);
         const float2 mu = s_xy[valid ? jj : 0];
         const float4 cq = s_co[valid ? jj : 0];
-        const float4 cp = s_cp[valid ? jj : 0];
+        const float4 cp = unpack_cull_params(s_cull[valid ? jj : 0], s_floor[valid ? jj : 0]);
+        // (the four tests first, in one straight line and unconditionally, so that what they have in common is
+        // computed once; masks of single comparisons, combined in scalar registers)
+        uint64_t hit_m[4];
 #pragma unroll
         for (int r = 0; r < 4; r++) {
           const bool row_alive = ((alive_mask >> (16 * r)) & 0xFFFFull) != 0ull;
-          // (masks of single comparisons, combined in scalar registers)
-          const uint64_t b = row_alive ? (valid_m & gs_ballot(ellipse_hits_row(mu, cq, cp, rt.qx0, rt.qy0, r))) : 0ull;
-          if (lane == 0) {
-            s_list[wave][r][2 * k] = (uint32_t)b;
-            s_list[wave][r][2 * k + 1] = (uint32_t)(b >> 32);
+          hit_m[r] = (row_alive ? valid_m : 0ull) & gs_ballot(ellipse_hits_row(mu, cq, cp, rt.qx0, rt.qy0, r));
+        }
+        uint32_t rows_hit = 0u;
+        auto list_row = [&](auto row_tag, const uint32_t len) {
+          constexpr int r = decltype(row_tag)::value;
+          const uint64_t b = hit_m[r];
+          const uint32_t below = __builtin_amdgcn_mbcnt_hi((uint32_t)(b >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)b, 0u));
+          if (__builtin_amdgcn_inverse_ballot_w64(b)) {
+            reinterpret_cast<uint8_t*>(&s_idx[0][0][0])[(uint32_t)((wave_b * 4 + r) * BATCH) + len + below] = (uint8_t)jj;
+            rows_hit |= 1u << r;
           }
+          return len + (uint32_t)__popcll(b);
+        };
+        len0 = list_row(std::integral_constant<int, 0>{}, len0);
+        len1 = list_row(std::integral_constant<int, 1>{}, len1);
+        len2 = list_row(std::integral_constant<int, 2>{}, len2);
+        len3 = list_row(std::integral_constant<int, 3>{}, len3);
+        if (block_hits != nullptr) {
+          // an even lane stores its own four bits and its odd neighbour's: one byte, no other wave's
+          const uint32_t neighbour = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)rows_hit, 0xB1, 0xF, 0xF, false);
+          if ((lane_b & 1) == 0)
+            reinterpret_cast<uint8_t*>(&s_hits[0])[(4 * (lane_b >> 1) + wave_b) + k * (4 * GS_WAVE / 2)] =
+                (uint8_t)(rows_hit | (neighbour << 4));
         }
       }
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -185,20 +233,21 @@ render_fwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
       // SELECT: a lane that does not blend keeps its sums by a select instead of adding a product with weight 0
       // (0 * NaN and 0 * inf are NaN): the reference only lets a non-finite colour reach the pixels that blend
       // it (cuda_rasterizer/forward.cu:381-407).  Same bits for finite inputs.
-      auto walk = [&](auto select_tag) {
+      len0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)len0);
+      len1 = (uint32_t)__builtin_amdgcn_readfirstlane((int)len1);
+      len2 = (uint32_t)__builtin_amdgcn_readfirstlane((int)len2);
+      len3 = (uint32_t)__builtin_amdgcn_readfirstlane((int)len3);
+      const uint32_t row_len = row == 0 ? len0 : (row == 1 ? len1 : (row == 2 ? len2 : len3));
+      auto walk = [&, len0, len1, len2, len3, row_len](auto select_tag) {
       constexpr bool SELECT = decltype(select_tag)::value;
-      int kk = 0;
-      uint32_t m = s_list[wave][row][0];
-      for (;;) {
-        if (m == 0u && kk < CHUNKS - 1) {
-          kk++;
-          m = s_list[wave][row][kk];
-        }
-        const bool has = m != 0u;
-        const uint64_t has_m = gs_ballot(has);
-        if ((has_m | gs_ballot(kk < CHUNKS - 1)) == 0ull) break;
-        const int j = has ? kk * 32 + (int)__builtin_ctz(m) : 0;
-        m &= m - 1u;
+      uint32_t my_len = row_len;
+      uint32_t passes = max(max(len0, len1), max(len2, len3));  // wave-uniform
+      uint32_t word = 0u;  // four entries of the list
+      for (uint32_t n = 0; n < passes; n++) {
+        if ((n & 3u) == 0u) word = s_idx[wave][row][n >> 2];
+        const uint64_t has_m = gs_ballot(n < my_len);
+        // (slot 0 behind the end of the list: its data are this batch's)
+        const int j = (int)__builtin_amdgcn_ubfe(word, (n & 3u) * 8u, 8u);
 
         // Straight-line: every lane evaluates its row's Gaussian; a lane for which it does not count blends
         // with weight 0, which leaves its sums unchanged bit for bit (fma(c, 0, C) == C).  The tests are kept as
@@ -239,8 +288,8 @@ render_fwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
           }
           const uint64_t omask = bmask & gs_ballot(T > 0.5f);
           if (omask != 0ull) {
-            const int cnt = __popc((uint32_t)(omask >> row_shift) & 0xFFFFu);
-            if (rt.l16 == 0 && cnt != 0) atomicAdd(&s_obs[j], cnt);
+            const uint32_t cnt = (uint32_t)__popc((uint32_t)(omask >> row_shift) & 0xFFFFu);
+            if (rt.l16 == 0 && cnt != 0u) atomicAdd(&s_obs[j >> 1], cnt << (16 * (j & 1)));
           }
           T = blend ? test_T : T;
           last = blend ? (uint32_t)(i * BATCH + j + 1) : last;
@@ -248,30 +297,29 @@ render_fwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
         if (stop_m != 0ull) {
           alive &= ~stop_m;
           // a row whose 16 pixels have all saturated drops the rest of its list
-          if (((uint32_t)(alive >> row_shift) & 0xFFFFu) == 0u) {
-            m = 0u;
-            kk = CHUNKS - 1;
-          }
+          if (((uint32_t)(alive >> row_shift) & 0xFFFFu) == 0u) my_len = 0u;
+          passes = 0u;
+          if (((uint32_t)alive & 0xFFFFu) != 0u) passes = len0;
+          if (((uint32_t)(alive >> 16) & 0xFFFFu) != 0u) passes = max(passes, len1);
+          if (((uint32_t)(alive >> 32) & 0xFFFFu) != 0u) passes = max(passes, len2);
+          if (((uint32_t)(alive >> 48) & 0xFFFFu) != 0u) passes = max(passes, len3);
         }
       }
       };
       if (select_blend) walk(std::true_type{});
       else walk(std::false_type{});
-    } else if (block_hits != nullptr && lane < 4 * CHUNKS) {
-      s_list[wave][lane / CHUNKS][lane % CHUNKS] = 0u;  // (the lists are also what the backward pass is left)
     }
     __syncthreads();
-    if (tid < count) {
-      const int c = s_obs[tid];
-      if (c != 0) atomicAdd(&out_observe[s_id[tid]], c);
+    const int tf = not_hoisted(tid);
+    if (tf < count) {
+      const uint32_t c = (s_obs[tf >> 1] >> (16 * (tf & 1))) & 0xFFFFu;
+      if (c != 0u) atomicAdd(&out_observe[point_list[range.x + (uint32_t)i * BATCH + tf]], (int)c);
+      // for the backward pass: which of the tile's sixteen rows listed this slot (a row that had saturated has an
+      // empty list, and nothing behind a row's last contributor is looked at there)
       if (block_hits != nullptr) {
-        // for the backward pass: this slot's bit of the sixteen row lists (a row that had saturated has an empty
-        // list, and nothing behind a row's last contributor is looked at there)
-        uint32_t hits = 0u;
-#pragma nounroll
-        for (int wr = 0; wr < 4 * (GS_TILE_PIX / GS_WAVE); wr++)  // (one list word at a time: registers are scarce here)
-          hits |= ((s_list[0][0][wr * CHUNKS + (tid >> 5)] >> (tid & 31)) & 1u) << wr;
-        block_hits[range.x + (uint32_t)i * BATCH + tid] = (uint16_t)hits;
+        const uint32_t x = s_hits[tf >> 1] >> (4 * (tf & 1));
+        block_hits[range.x + (uint32_t)i * BATCH + tf] =
+            (uint16_t)((x & 0xFu) | ((x >> 4) & 0xF0u) | ((x >> 8) & 0xF00u) | ((x >> 12) & 0xF000u));
       }
     }
   }
