@@ -10,8 +10,10 @@
 //     the row's block (the forward kernel's own answer, 16 bits per instance,
 //     when the caller hands them on; otherwise the inflated alpha >= 1/255
 //     ellipse is tested against the block again) and lie in front of the
-//     row's deepest contributor; the four rows then walk their own bit lists
-//     concurrently, so one pass of the loop handles up to four Gaussians;
+//     row's deepest contributor, and compacts their slot numbers into a byte
+//     list per row; the four rows then walk their own lists concurrently
+//     (entry n of each in pass n), so one pass of the loop handles up to four
+//     Gaussians;
 //   * the 16 partial sums of a Gaussian (mean2D x/y, |mean2D| x/y, conic
 //     x/y/w, opacity, colour 3, map 5) are reduced over the row's 16 lanes by
 //     a transposing DPP reduction (15 additions instead of 64) that leaves
@@ -53,7 +55,6 @@ namespace {
 constexpr int BATCH = GS_TILE_PIX / 2;  // Gaussians staged in LDS per round
 constexpr int SUB = GS_WAVE;        // Gaussians whose sums are in the accumulators at a time: one ballot's worth
 constexpr int NV = 16;
-constexpr int CHUNKS = SUB / 32;
 constexpr int WAVES = GS_TILE_PIX / GS_WAVE;
 static_assert(SUB * 4 == GS_TILE_PIX, "a thread hands over a quarter of one record of the sub-batch");
 
@@ -80,7 +81,9 @@ render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
   __shared__ float4 s_chan[BATCH][RENDER_GEO ? 2 : 1];
   // one accumulator per wave; +1: the 16 components of one Gaussian fall in 16 different banks
   __shared__ float s_acc[WAVES][NV][SUB + 1];
-  __shared__ uint32_t s_list[GS_TILE_PIX / GS_WAVE][4][CHUNKS];
+  // the four rows' lists of every wave: the slots of the sub-batch that can touch the row's block and are not
+  // behind its deepest contributor, one byte each, in walking order; bytes behind a list's end are 0
+  __shared__ __attribute__((aligned(16))) uint32_t s_idx[GS_TILE_PIX / GS_WAVE][4][SUB / 4];
   __shared__ int s_max[GS_TILE_PIX / GS_WAVE];
   __shared__ int s_bad[GS_TILE_PIX / GS_WAVE];
 
@@ -219,8 +222,12 @@ render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
     const bool select_state = (s_bad[0] | s_bad[1] | s_bad[2] | s_bad[3]) != 0;
 
     for (int base = 0; base < count; base += SUB) {
-      // per-row lists: bit b of word c of row r = slot base+32c+b of the batch can touch row r's 4x4 block
+      // Per-row lists: lane = slot of the sub-batch; the lanes whose Gaussian counts for row r append their slot
+      // numbers to the row's list, in lane order (a lane's place is the number of set bits below its own).
+      uint32_t len0, len1, len2, len3;  // the lists' lengths (wave-uniform)
       {
+        static_assert(sizeof(s_idx[0]) == 4 * GS_WAVE, "a wave clears its own lists, one word per lane");
+        (&s_idx[wave][0][0])[lane] = 0u;
         const int jj = base + lane;
         const bool valid = jj < count;
         const uint64_t valid_m = gs_ballot(valid);  // (masks of single comparisons, combined in scalar registers)
@@ -235,39 +242,44 @@ render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
           cq = s_co[valid ? jj : 0];
           cp = s_cp[valid ? jj : 0];
         }
+        uint64_t hit_m[4];
 #pragma unroll
         for (int r = 0; r < 4; r++) {
           const bool touches = HITS ? ((nibble >> r) & 1u) != 0u : ellipse_hits_row(mu, cq, cp, rt.qx0, rt.qy0, r);
-          const uint64_t hit = valid_m & gs_ballot((first_pos - jj) < row_last_of[r]) & gs_ballot(touches);
-          if (lane == 0) {
-            s_list[wave][r][0] = (uint32_t)hit;
-            s_list[wave][r][1] = (uint32_t)(hit >> 32);
-          }
+          hit_m[r] = valid_m & gs_ballot((first_pos - jj) < row_last_of[r]) & gs_ballot(touches);
         }
+        auto list_row = [&](auto row_tag) {
+          constexpr int r = decltype(row_tag)::value;
+          const uint64_t b = hit_m[r];
+          const uint32_t below = __builtin_amdgcn_mbcnt_hi((uint32_t)(b >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)b, 0u));
+          if (__builtin_amdgcn_inverse_ballot_w64(b)) reinterpret_cast<uint8_t*>(&s_idx[wave][r][0])[below] = (uint8_t)lane;
+          return (uint32_t)__builtin_amdgcn_readfirstlane((int)__popcll(b));
+        };
+        len0 = list_row(std::integral_constant<int, 0>{});
+        len1 = list_row(std::integral_constant<int, 1>{});
+        len2 = list_row(std::integral_constant<int, 2>{});
+        len3 = list_row(std::integral_constant<int, 3>{});
       }
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
       __builtin_amdgcn_wave_barrier();
       __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      const uint32_t my_len = row == 0 ? len0 : (row == 1 ? len1 : (row == 2 ? len2 : len3));
+      const uint32_t passes = max(max(len0, len1), max(len2, len3));  // wave-uniform
 
       // SELECT: a lane for which the Gaussian does not count takes the Gaussian's colour and geometry channels
       // as 0 (its step then still only rotates the recurrence state: alpha = 0 with a finite colour), so that a
       // non-finite channel only reaches the pixels that blended it in the forward pass, as in the reference
       // (cuda_rasterizer/backward.cu:463-472).  Same bits for finite inputs.
-      auto walk = [&](auto select_tag) {
+      auto walk = [&, my_len, passes](auto select_tag) {
         constexpr bool SELECT = decltype(select_tag)::value;
-        int kk = 0;
-        uint32_t m = s_list[wave][row][0];
-        for (;;) {
-          if (m == 0u && kk < CHUNKS - 1) {
-            kk++;
-            m = s_list[wave][row][kk];
-          }
-          const bool has = m != 0u;
+        uint32_t word = 0u;  // four entries of the list
+        for (uint32_t n = 0; n < passes; n++) {
+          if ((n & 3u) == 0u) word = s_idx[wave][row][n >> 2];
+          const bool has = n < my_len;
           const uint64_t has_m = gs_ballot(has);
-          if ((has_m | gs_ballot(kk < CHUNKS - 1)) == 0ull) break;
-          const int ja = has ? kk * 32 + (int)__builtin_ctz(m) : 0;  // slot of the accumulators
-          const int j = base + ja;                                   // slot of the batch
-          m &= m - 1u;
+          // (slot 0 behind the end of the list: its data are this sub-batch's)
+          const int ja = (int)__builtin_amdgcn_ubfe(word, (n & 3u) * 8u, 8u);  // slot of the accumulators
+          const int j = base + ja;                                             // slot of the batch
           const int pos = first_pos - j;
           // Straight-line from here on: every lane evaluates its row's Gaussian, and a lane for which the
           // Gaussian does not count (behind the pixel's last contributor, outside the power window, alpha
