@@ -413,58 +413,74 @@ bucket_scatter_kernel(int P, int per_block, uint32_t gx, uint32_t gy, const floa
 // the indices.  Short dependency chains matter more than instruction count here: every tile is resident at once,
 // so the kernel takes as long as its longest tile, and many waves with few records each finish it soonest.
 
-template <int E>
-__device__ __forceinline__ void exchange_step(uint64_t (&v)[E], const uint64_t (&other)[E], uint32_t row0,
-                                              uint32_t lane, uint32_t k, bool lower) {
-#pragma unroll
-  for (int r = 0; r < E; r++) {
-    const uint32_t i = ((row0 + r) << 6) | lane;
-    const bool ascending = (i & k) == 0;
-    const bool keep_min = lower == ascending;
-    const uint64_t a = v[r], b = other[r];
-    const bool a_less = a < b;
-    v[r] = (a_less == keep_min) ? a : b;
-  }
+// Which element of a pair (a, b) each lane keeps is decided in scalar registers: keep_min is the lane mask of the
+// elements that keep the smaller one, less the lane mask of a < b; a lane keeps a where the two agree.
+__device__ __forceinline__ uint64_t keep_pair(uint64_t a, uint64_t b, uint64_t keep_min) {
+  const uint64_t less = __builtin_amdgcn_ballot_w64(a < b);
+  return __builtin_amdgcn_inverse_ballot_w64(~(less ^ keep_min)) ? a : b;
 }
 
-// x of lane (lane ^ J), J a power of two below 64, without going through the LDS crossbar: DPP moves inside a
-// 16-lane row (xor 4 = reverse the quads' lanes, then mirror the half rows), v_permlane16_swap / v_permlane32_swap
-// across rows and halves.  A variable-distance __shfl_xor is a ds_bpermute, whose latency every one of the sort's
-// dependent steps would wait for.  All 64 lanes must be active.
+// Lanes whose bit J of the lane number is clear: the lower element of every pair at distance J.
 template <int J>
-__device__ __forceinline__ uint32_t xor_lane(uint32_t x, uint32_t lane) {
-  static_assert(J == 1 || J == 2 || J == 4 || J == 8 || J == 16 || J == 32, "distance inside a wave");
+__device__ __forceinline__ constexpr uint64_t lower_lanes() {
+  uint64_t m = 0;
+  for (int l = 0; l < 64; l++)
+    if ((l & J) == 0) m |= 1ull << l;
+  return m;
+}
+
+// x of lane (lane ^ J), J = 1, 2, 4 or 8, by DPP moves inside a 16-lane row (xor 4 = reverse the quads' lanes,
+// then mirror the half rows).  Every lane has a source, so nothing is kept of the old value (with bound_ctrl set
+// the destination needs no initialisation).  A variable-distance __shfl_xor is a ds_bpermute, whose latency
+// every one of the sort's dependent steps would wait for.  All 64 lanes must be active.
+template <int J>
+__device__ __forceinline__ uint32_t xor_lane(uint32_t x) {
+  static_assert(J == 1 || J == 2 || J == 4 || J == 8, "distance inside a 16-lane row");
   if constexpr (J == 1) {
-    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0xB1, 0xF, 0xF, false);  // quad_perm [1,0,3,2]
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0xB1, 0xF, 0xF, true);  // quad_perm [1,0,3,2]
   } else if constexpr (J == 2) {
-    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x4E, 0xF, 0xF, false);  // quad_perm [2,3,0,1]
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x4E, 0xF, 0xF, true);  // quad_perm [2,3,0,1]
   } else if constexpr (J == 4) {
-    const int t = __builtin_amdgcn_update_dpp(0, (int)x, 0x1B, 0xF, 0xF, false);     // quad_perm [3,2,1,0]: lane ^ 3
-    return (uint32_t)__builtin_amdgcn_update_dpp(0, t, 0x141, 0xF, 0xF, false);      // row_half_mirror: lane ^ 7
-  } else if constexpr (J == 8) {
-    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x128, 0xF, 0xF, false);  // row_ror:8
-  } else if constexpr (J == 16) {
-    // [0]: odd rows replaced by the even rows below them, [1]: even rows replaced by the odd rows above them
-    const auto r = __builtin_amdgcn_permlane16_swap(x, x, false, false);
-    return (lane & 16u) ? r[0] : r[1];
+    const int t = __builtin_amdgcn_update_dpp(0, (int)x, 0x1B, 0xF, 0xF, true);     // quad_perm [3,2,1,0]: lane ^ 3
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, t, 0x141, 0xF, 0xF, true);      // row_half_mirror: lane ^ 7
   } else {
-    // [0]: upper half replaced by the lower half, [1]: lower half replaced by the upper half
-    const auto r = __builtin_amdgcn_permlane32_swap(x, x, false, false);
-    return (lane & 32u) ? r[0] : r[1];
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x128, 0xF, 0xF, true);  // row_ror:8
   }
 }
 
-// One step of the network with the partner in lane ^ J.
+// One step of the network with the partner in lane ^ J.  ascending[r]: lane mask of the elements of register r
+// that lie in an ascending run of this stage.
 template <int E, int J>
-__device__ __forceinline__ void lane_step(uint64_t (&v)[E], uint32_t row0, uint32_t lane, uint32_t k) {
-  uint64_t other[E];
+__device__ __forceinline__ void lane_step(uint64_t (&v)[E], const uint64_t (&ascending)[E]) {
+  constexpr uint64_t lower = lower_lanes<J>();
 #pragma unroll
   for (int r = 0; r < E; r++) {
-    const uint32_t lo = xor_lane<J>((uint32_t)v[r], lane);
-    const uint32_t hi = xor_lane<J>((uint32_t)(v[r] >> 32), lane);
-    other[r] = ((uint64_t)hi << 32) | lo;
+    const uint64_t keep_min = ~(lower ^ ascending[r]);  // the lower element of an ascending pair, the upper of a descending
+    if constexpr (J < 16) {
+      const uint32_t lo = xor_lane<J>((uint32_t)v[r]);
+      const uint32_t hi = xor_lane<J>((uint32_t)(v[r] >> 32));
+      v[r] = keep_pair(v[r], ((uint64_t)hi << 32) | lo, keep_min);
+    } else {
+      // v_permlane16_swap / v_permlane32_swap exchange the odd rows (the upper half) of their first operand with
+      // the even rows (the lower half) of the second: from two copies of x they leave the lower element of every
+      // pair in all lanes of the first result and the upper element in the second, so both lanes of a pair
+      // compare the same two values and each keeps its own.
+      const uint32_t xl = (uint32_t)v[r], xh = (uint32_t)(v[r] >> 32);
+      uint64_t a, b;
+      if constexpr (J == 16) {
+        const auto l = __builtin_amdgcn_permlane16_swap(xl, xl, false, false);
+        const auto h = __builtin_amdgcn_permlane16_swap(xh, xh, false, false);
+        a = ((uint64_t)h[0] << 32) | l[0];
+        b = ((uint64_t)h[1] << 32) | l[1];
+      } else {
+        const auto l = __builtin_amdgcn_permlane32_swap(xl, xl, false, false);
+        const auto h = __builtin_amdgcn_permlane32_swap(xh, xh, false, false);
+        a = ((uint64_t)h[0] << 32) | l[0];
+        b = ((uint64_t)h[1] << 32) | l[1];
+      }
+      v[r] = keep_pair(a, b, keep_min);
+    }
   }
-  exchange_step<E>(v, other, row0, lane, k, (lane & (uint32_t)J) == 0);
 }
 
 template <int E, int W>
@@ -472,6 +488,19 @@ __device__ __forceinline__ void register_sort(uint64_t (&v)[E], uint32_t wave, u
   constexpr uint32_t M = 64u * E * W;
   const uint32_t row0 = wave * E;
   for (uint32_t k = 2; k <= M; k <<= 1) {
+    // the direction of this stage's runs: element i = (row << 6 | lane) ascends where (i & k) == 0, which is a
+    // property of the lane below k = 64 and of the register (and wave) from there on
+    uint64_t ascending[E];
+    {
+      const uint64_t by_lane = __builtin_amdgcn_ballot_w64((lane & k) == 0u);
+#pragma unroll
+      for (int r = 0; r < E; r++) {
+        const uint64_t m = k < 64u ? by_lane : ((((row0 + (uint32_t)r) << 6) & k) == 0u ? ~0ull : 0ull);
+        // (wave-uniform: kept in scalar registers)
+        ascending[r] = ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(m >> 32)) << 32) |
+                       (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)m);
+      }
+    }
     for (uint32_t j = k >> 1; j >= 64; j >>= 1) {
       if (j < 64u * E) {
         const uint32_t jr = j >> 6;
@@ -481,12 +510,12 @@ __device__ __forceinline__ void register_sort(uint64_t (&v)[E], uint32_t wave, u
 #pragma unroll
           for (int r = 0; r < E; r++) {
             if (r & b) continue;
-            const uint32_t i = ((row0 + r) << 6) | lane;
-            const bool ascending = (i & k) == 0;
+            // (both registers of a pair lie in the same run)
             const uint64_t x = v[r], y = v[r | b];
-            const bool swap = (x > y) == ascending;
-            v[r] = swap ? y : x;
-            v[r | b] = swap ? x : y;
+            const uint64_t less = __builtin_amdgcn_ballot_w64(x < y);
+            const bool x_first = __builtin_amdgcn_inverse_ballot_w64(~(less ^ ascending[r]));
+            v[r] = x_first ? x : y;
+            v[r | b] = x_first ? y : x;
           }
         }
       } else {
@@ -496,19 +525,21 @@ __device__ __forceinline__ void register_sort(uint64_t (&v)[E], uint32_t wave, u
 #pragma unroll
         for (int r = 0; r < E; r++) s_x[((wave * E + r) << 6) | lane] = v[r];
         __syncthreads();
-        uint64_t other[E];
+        const bool lower = (wave & jw) == 0;
 #pragma unroll
-        for (int r = 0; r < E; r++) other[r] = s_x[(((wave ^ jw) * E + r) << 6) | lane];
-        exchange_step<E>(v, other, row0, lane, k, (wave & jw) == 0);
+        for (int r = 0; r < E; r++) {
+          const uint64_t other = s_x[(((wave ^ jw) * E + r) << 6) | lane];
+          v[r] = keep_pair(v[r], other, lower ? ascending[r] : ~ascending[r]);
+        }
       }
     }
     // the steps with the partner in another lane: distances min(k / 2, 32) down to 1
-    if (k >= 64) lane_step<E, 32>(v, row0, lane, k);
-    if (k >= 32) lane_step<E, 16>(v, row0, lane, k);
-    if (k >= 16) lane_step<E, 8>(v, row0, lane, k);
-    if (k >= 8) lane_step<E, 4>(v, row0, lane, k);
-    if (k >= 4) lane_step<E, 2>(v, row0, lane, k);
-    lane_step<E, 1>(v, row0, lane, k);
+    if (k >= 64) lane_step<E, 32>(v, ascending);
+    if (k >= 32) lane_step<E, 16>(v, ascending);
+    if (k >= 16) lane_step<E, 8>(v, ascending);
+    if (k >= 8) lane_step<E, 4>(v, ascending);
+    if (k >= 4) lane_step<E, 2>(v, ascending);
+    lane_step<E, 1>(v, ascending);
   }
 }
 
