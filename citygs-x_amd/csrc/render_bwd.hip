@@ -243,9 +243,11 @@ render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
           cp = s_cp[valid ? jj : 0];
         }
         uint64_t hit_m[4];
+        bool hits[4] = {false, false, false, false};
+        if (!HITS) ellipse_hits_quadrant(mu, cq, cp, rt.qx0, rt.qy0, hits);
 #pragma unroll
         for (int r = 0; r < 4; r++) {
-          const bool touches = HITS ? ((nibble >> r) & 1u) != 0u : ellipse_hits_row(mu, cq, cp, rt.qx0, rt.qy0, r);
+          const bool touches = HITS ? ((nibble >> r) & 1u) != 0u : hits[r];
           hit_m[r] = valid_m & gs_ballot((first_pos - jj) < row_last_of[r]) & gs_ballot(touches);
         }
         auto list_row = [&](auto row_tag) {

@@ -1,76 +1,20 @@
 // Pieces shared by the forward and backward tile kernels: the pixel layout of a
-// workgroup, the conservative screen-space bounding box used to cull Gaussians
-// per wave, and the 64-lane reduction of 16 values.
+// workgroup, the conservative test that culls Gaussians per 4x4 pixel block, and
+// the reductions of 16 values over a wave and over a 16-lane row.
 #pragma once
 
 #include "gs_common.h"
 
 namespace gs {
 
-// A 16x16 tile is rendered by 256 threads = four 64-lane waves; each wave owns
-// an 8x8 quadrant (lane = 8*row + column inside the quadrant).  Compared with
-// 16x4 strips this keeps a wave's pixels compact, so fewer Gaussians of the
-// tile's list overlap any given wave.
-struct TileThread {
-  int lane, wave;
-  uint32_t px, py;    // this thread's pixel
-  float wx0, wy0, wx1, wy1;  // the wave's pixel rectangle (inclusive), as floats
-};
-
-__device__ __forceinline__ TileThread tile_thread(uint32_t tile_x, uint32_t tile_y) {
-  TileThread t;
-  const int tid = threadIdx.x;
-  t.lane = tid & (GS_WAVE - 1);
-  t.wave = tid / GS_WAVE;
-  const uint32_t qx = (uint32_t)(t.wave & 1) * 8u, qy = (uint32_t)(t.wave >> 1) * 8u;
-  const uint32_t x0 = tile_x * GS_TILE_X + qx, y0 = tile_y * GS_TILE_Y + qy;
-  t.px = x0 + (uint32_t)(t.lane & 7);
-  t.py = y0 + (uint32_t)(t.lane >> 3);
-  t.wx0 = (float)x0;
-  t.wy0 = (float)y0;
-  t.wx1 = (float)(x0 + 7u);
-  t.wy1 = (float)(y0 + 7u);
-  return t;
-}
-
-// Axis-aligned box outside of which a Gaussian cannot pass the blend tests of
-// cuda_rasterizer/forward.cu:381-393 (power <= 0 and opacity*exp(power) >= 1/255).
-// With conic (A,B,C) and tau = ln(255*opacity), alpha >= 1/255 needs
-// A dx^2 + 2B dx dy + C dy^2 <= 2 tau, whose extent along x is sqrt(2 tau C / (AC-B^2)).
-// The box is inflated (tau + 0.01, then 0.1 % and half a pixel) so that fp32
-// rounding in the per-pixel evaluation can never disagree with it; whenever the
-// box cannot be trusted (non-positive determinant, NaN) it is infinite.  Culling
-// with it only skips work, it never changes a result.
-// power_floor receives the exponent below which alpha < 1/255 is certain (never below -87, where
-// gs_expf returns 0 anyway): pixels with power < power_floor can skip the exponential.
-__device__ __forceinline__ float4 cull_box(float2 xy, float4 co, float& power_floor) {
-  const float inf = __builtin_inff();
-  float4 bb = make_float4(-inf, -inf, inf, inf);  // xmin, ymin, xmax, ymax
-  const float o = co.w;
-  power_floor = -87.0f;
-  if (o < 0.0039f) {
-    // opacity below 1/255: alpha = o*exp(power) with power <= 0 can never reach 1/255
-    return make_float4(inf, inf, -inf, -inf);
-  }
-  const float det = co.x * co.z - co.y * co.y;
-  if (o < 1.0e30f) {
-    const float tau = __logf(255.0f * o) + 0.01f;
-    if (tau == tau) power_floor = fmaxf(-tau, -87.0f);
-  }
-  if (det > 0.0f && o < 1.0e30f) {
-    const float tau = __logf(255.0f * o) + 0.01f;
-    const float s = 2.0f * tau / det;
-    const float ex = sqrtf(s * co.z) * 1.001f + 0.5f;
-    const float ey = sqrtf(s * co.x) * 1.001f + 0.5f;
-    if (ex == ex && ey == ey) bb = make_float4(xy.x - ex, xy.y - ey, xy.x + ex, xy.y + ey);
-  }
-  return bb;
-}
-
-// The same region, tested exactly against a block of pixels instead of through its bounding box.
-// cull_params returns (1/A, 1/C, q_max, 0): alpha >= 1/255 needs q(d) = A dx^2 + 2B dx dy + C dy^2 <= q_max
-// = 2 (tau + 0.01).  q_max is +infinity when the conic cannot be trusted (every block then counts as hit)
-// and negative when the opacity alone rules every pixel out.  power_floor as for cull_box.
+// Which Gaussians can pass the blend tests of cuda_rasterizer/forward.cu:381-393 (power <= 0 and
+// opacity * exp(power) >= 1/255) somewhere in a block of pixels.  With conic (A, B, C) and
+// tau = ln(255 * opacity), alpha >= 1/255 needs q(d) = A dx^2 + 2 B dx dy + C dy^2 <= 2 tau.
+// cull_params returns (1/A, 1/C, q_max, 0) with q_max = 2 (tau + 0.01).  q_max is +infinity when the conic
+// cannot be trusted (every block then counts as hit) and negative when the opacity alone rules every pixel out.
+// power_floor receives the exponent below which alpha < 1/255 is certain (never below -87, where gs_expf
+// returns 0 anyway): pixels with power < power_floor can skip the exponential.  Culling with these only skips
+// work, it never changes a result.
 __device__ __forceinline__ float4 cull_params(float4 co, float& power_floor) {
   const float inf = __builtin_inff();
   const float o = co.w;
@@ -104,24 +48,50 @@ __device__ __forceinline__ float4 unpack_cull_params(float2 e, float power_floor
                      never ? -1.0f : (always ? __builtin_inff() : -2.0f * power_floor), 0.f);
 }
 
-// Can any point of the pixel block [bx0, bx0+ext] x [by0, by0+ext] have q <= q_max?  q is convex, so over
-// the block it is smallest either at the centre (inside the block: 0) or on one of the two block edges that
-// face the centre; along an edge it is a parabola whose minimiser is clamped to the edge.  The block is
-// treated as a continuous rectangle, which can only add hits; the 0.01 added to tau covers the rounding
-// differences against the per-pixel evaluation.  NaNs count as hits.
-__device__ __forceinline__ bool ellipse_hits_block(float2 mu, float4 co, float4 cp, float bx0, float by0, float ext) {
-  const float lox = bx0 - mu.x, hix = lox + ext, loy = by0 - mu.y, hiy = loy + ext;
-  const float dxc = fminf(fmaxf(0.f, lox), hix);  // offset of the nearest column / row of the block
-  const float dyc = fminf(fmaxf(0.f, loy), hiy);
-  const float dy1 = fminf(fmaxf(-co.y * dxc * cp.y, loy), hiy);  // best point of the column x = dxc
-  const float q1 = (co.x * dxc * dxc + 2.0f * co.y * dxc * dy1) + co.z * dy1 * dy1;
-  const float dx2 = fminf(fmaxf(-co.y * dyc * cp.x, lox), hix);  // best point of the row y = dyc
-  const float q2 = (co.x * dx2 * dx2 + 2.0f * co.y * dx2 * dyc) + co.z * dyc * dyc;
-  return !(fminf(q1, q2) > cp.z);
-}
-
-__device__ __forceinline__ bool box_hits_wave(const float4 bb, const TileThread& t) {
-  return !(bb.z < t.wx0 || bb.x > t.wx1 || bb.w < t.wy0 || bb.y > t.wy1);
+// The four 4x4 pixel blocks of an 8x8 quadrant at (qx0, qy0), block r at x offset 4 (r & 1), y offset 4 (r >> 1):
+// hit[r] = can any point of block r have q <= q_max?  q is convex, so over a block it is smallest either at the
+// centre (inside the block: 0) or on one of the two block edges that face the centre; along an edge it is a
+// parabola whose minimiser is clamped to the edge.  A block is treated as a continuous rectangle, which can only
+// add hits.  What the two columns and the two rows of blocks have in common is computed once; the parabolas are
+// evaluated in Horner form with fused multiply-adds.
+// Rounding: this evaluation and the per-pixel one (a different operation sequence, at a different point) each
+// carry an error of a few units in the last place of the LARGEST term, which for a long thin Gaussian far from
+// its centre is much larger than q itself.  Every such term is at most S = A X^2 + 2 |B| X Y + C Y^2 with X, Y
+// the largest offsets inside the quadrant, so q_max is raised by 1e-6 S (about 16 units in the last place of S)
+// on top of the 0.02 from tau + 0.01: the test never rejects a block one of whose pixels passes.  NaNs count as
+// hits.
+__device__ __forceinline__ void ellipse_hits_quadrant(float2 mu, float4 co, float4 cp, float qx0, float qy0,
+                                                      bool (&hit)[4]) {
+  const float two_b = 2.0f * co.y;
+  float lox[2], hix[2], dxc[2], t1[2], a1[2], b1[2];  // per column of blocks
+  float loy[2], hiy[2], dyc[2], t2[2], a2[2], b2[2];  // per row of blocks
+#pragma unroll
+  for (int c = 0; c < 2; c++) {
+    lox[c] = (qx0 + (float)(4 * c)) - mu.x;
+    hix[c] = lox[c] + 3.0f;
+    dxc[c] = fminf(fmaxf(0.f, lox[c]), hix[c]);  // offset of the nearest column of the block
+    t1[c] = -co.y * dxc[c] * cp.y;               // where q is smallest along that column
+    a1[c] = co.x * dxc[c] * dxc[c];
+    b1[c] = two_b * dxc[c];
+    loy[c] = (qy0 + (float)(4 * c)) - mu.y;
+    hiy[c] = loy[c] + 3.0f;
+    dyc[c] = fminf(fmaxf(0.f, loy[c]), hiy[c]);  // offset of the nearest row of the block
+    t2[c] = -co.y * dyc[c] * cp.x;               // where q is smallest along that row
+    a2[c] = co.z * dyc[c] * dyc[c];
+    b2[c] = two_b * dyc[c];
+  }
+  const float X = fmaxf(fabsf(lox[0]), fabsf(hix[1])), Y = fmaxf(fabsf(loy[0]), fabsf(hiy[1]));
+  const float S = (co.x * X * X + fabsf(two_b) * X * Y) + co.z * Y * Y;
+  const float limit = cp.z < 0.f ? cp.z : __builtin_fmaf(1.0e-6f, S, cp.z);
+#pragma unroll
+  for (int r = 0; r < 4; r++) {
+    const int c = r & 1, d = r >> 1;
+    const float dy1 = fminf(fmaxf(t1[c], loy[d]), hiy[d]);  // best point of the column x = dxc
+    const float q1 = __builtin_fmaf(__builtin_fmaf(co.z, dy1, b1[c]), dy1, a1[c]);
+    const float dx2 = fminf(fmaxf(t2[d], lox[c]), hix[c]);  // best point of the row y = dyc
+    const float q2 = __builtin_fmaf(__builtin_fmaf(co.x, dx2, b2[d]), dx2, a2[d]);
+    hit[r] = !(fminf(q1, q2) > limit);
+  }
 }
 
 template <int CTRL>
@@ -180,17 +150,6 @@ __device__ __forceinline__ RowThread row_thread(uint32_t tile_x, uint32_t tile_y
   t.qx0 = (float)x0;
   t.qy0 = (float)y0;
   return t;
-}
-
-// Ellipse against the 4x4 block of row r of the quadrant at (qx0, qy0).
-__device__ __forceinline__ bool ellipse_hits_row(float2 mu, float4 co, float4 cp, float qx0, float qy0, int r) {
-  return ellipse_hits_block(mu, co, cp, qx0 + (float)((r & 1) * 4), qy0 + (float)((r >> 1) * 4), 3.0f);
-}
-
-// Box against the 4x4 block of row r of the quadrant at (qx0, qy0).
-__device__ __forceinline__ bool box_hits_row(const float4 bb, float qx0, float qy0, int r) {
-  const float x0 = qx0 + (float)((r & 1) * 4), y0 = qy0 + (float)((r >> 1) * 4);
-  return !(bb.z < x0 || bb.x > x0 + 3.0f || bb.w < y0 || bb.y > y0 + 3.0f);
 }
 
 template <int CTRL, int BANK_MASK>

@@ -198,10 +198,12 @@ render_fwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
         // (the four tests first, in one straight line and unconditionally, so that what they have in common is
         // computed once; masks of single comparisons, combined in scalar registers)
         uint64_t hit_m[4];
+        bool hits[4];
+        ellipse_hits_quadrant(mu, cq, cp, rt.qx0, rt.qy0, hits);
 #pragma unroll
         for (int r = 0; r < 4; r++) {
           const bool row_alive = ((alive_mask >> (16 * r)) & 0xFFFFull) != 0ull;
-          hit_m[r] = (row_alive ? valid_m : 0ull) & gs_ballot(ellipse_hits_row(mu, cq, cp, rt.qx0, rt.qy0, r));
+          hit_m[r] = (row_alive ? valid_m : 0ull) & gs_ballot(hits[r]);
         }
         uint32_t rows_hit = 0u;
         auto list_row = [&](auto row_tag, const uint32_t len) {

@@ -1,6 +1,8 @@
 """GPU parity of every stage of the rasterizer against the CPU oracle, through
 the C ABI.  Integer and index outputs must be identical; images within 1e-4
 absolute; gradients within 1e-3 relative L2."""
+import math
+
 import numpy as np
 import pytest
 import torch
@@ -385,6 +387,48 @@ def test_blend_with_arbitrary_splats(H, orc, seed, W, Hh, geo):
         g_ = gb[k].cpu().numpy()
         assert np.isfinite(g_).all(), k
         assert H.rel_l2(g_, r) <= GRAD_TOL, f"{k}: rel L2 {H.rel_l2(g_, r)}"
+
+
+@pytest.mark.parametrize("seed,reach", [(0, 300.0), (1, 3000.0), (2, 30000.0)])
+def test_long_thin_splats_far_from_their_centre(H, orc, seed, reach):
+    """Splats whose conic has one eigenvalue near the dilation limit (3.3) and one tiny, centred up to `reach`
+    pixels outside the image along their long axis, so that a band a few pixels wide crosses the image.  There
+    the three terms of the exponent (forward.cu:373) are many orders larger than their sum, and the per-pixel
+    value is dominated by rounding: whatever it is, the per-block culling must never drop a splat that one of the
+    block's pixels blends, so counters stay exact against the per-pixel oracle."""
+    gen = torch.Generator().manual_seed(900 + seed)
+    P, W, Hh = 400, 96, 64
+    gx, gy = H.grid(W, Hh)
+    through = torch.rand(P, 2, generator=gen, dtype=torch.float64) * torch.tensor([W - 1.0, Hh - 1.0])
+    ang = torch.rand(P, generator=gen, dtype=torch.float64) * math.pi
+    far = (torch.rand(P, generator=gen, dtype=torch.float64) * 2 - 1) * reach
+    lam_big = torch.rand(P, generator=gen, dtype=torch.float64) * 2.8 + 0.5
+    lam_small = 10.0 ** (-(torch.rand(P, generator=gen, dtype=torch.float64) * 4 + 4))   # 1e-4 .. 1e-8
+    ux, uy = torch.cos(ang), torch.sin(ang)          # the long axis (small eigenvalue)
+    means2D = torch.stack([through[:, 0] + far * ux, through[:, 1] + far * uy], 1).float().numpy()
+    a = (lam_small * ux * ux + lam_big * uy * uy)
+    b = ((lam_small - lam_big) * ux * uy)
+    c = (lam_small * uy * uy + lam_big * ux * ux)
+    opac = torch.rand(P, generator=gen) * 0.7 + 0.3
+    co = torch.stack([a.float(), b.float(), c.float(), opac], 1).numpy()
+    radii = np.full(P, 1 << 20, np.int32)            # every splat is listed in every tile
+    rgb = torch.rand(P, 3, generator=gen).numpy()
+    am = torch.randn(P, 5, generator=gen).numpy()
+    depths = (torch.rand(P, generator=gen) * 50 + 0.3).numpy()
+    cl = np.ones(gx * gy, bool)
+    bins = orc.bin_and_sort(radii, means2D, depths, cl, W, Hh)
+    bg = np.zeros(3, np.float32)
+    tanx, tany = 0.8, 0.8 * Hh / W
+    ref = orc.render_fwd(bins["ranges"], bins["point_list"], means2D, rgb, am, co, cl, bg, W, Hh, tanx, tany,
+                         render_geo=True)
+    got = H.render_fwd(P, W, Hh, tanx, tany, H.as_u32(bins["ranges"]), H.as_u32(bins["point_list"]), H.dev(means2D),
+                       H.dev(rgb), H.dev(am), H.dev(co), H.dev(cl), H.dev(bg), render_geo=True)
+    assert ref["n_contrib2loss"].sum() > 10 * W   # the bands do cross the image
+    for k in ("n_contrib", "n_contrib2loss"):
+        assert np.array_equal(H.np_u32(got[k]), ref[k]), k
+    assert np.array_equal(got["out_observe"].cpu().numpy(), ref["out_observe"])
+    assert np.array_equal(got["final_T"].cpu().numpy(), ref["final_T"])
+    assert np.array_equal(got["color"].cpu().numpy(), ref["color"])
 
 
 @pytest.mark.parametrize("geo", [True, False])
