@@ -431,6 +431,65 @@ def test_long_thin_splats_far_from_their_centre(H, orc, seed, reach):
     assert np.array_equal(got["color"].cpu().numpy(), ref["color"])
 
 
+def test_needles_through_the_whole_forward_pass(H, orc):
+    """Needle-shaped Gaussians (one axis 10^3 to 10^5 times the others, tens to hundreds of metres long) around
+    and in front of the camera: after projection their conics have one eigenvalue at the dilation limit and one
+    near zero, radii of tens of thousands of pixels and centres far outside the image.  Preprocess, lists and
+    blend against the oracle: every integer exact, the images the same bits."""
+    import gs_scenes
+    P = 3000
+    g, cam = _scene(0, P)
+    gen = torch.Generator().manual_seed(77)
+    W, Hh = cam.image_width, cam.image_height
+    g = dict(g)
+    length = 10.0 ** (torch.rand(P, generator=gen) * 1.5 + 0.7)          # 5 .. 160
+    thin = 10.0 ** (-(torch.rand(P, 2, generator=gen) * 2 + 1))            # 1e-1 .. 1e-3
+    g["scales"] = torch.cat([length[:, None], thin], 1)
+    q = torch.randn(P, 4, generator=gen)
+    g["rotations"] = q / q.norm(dim=1, keepdim=True)
+    g["opacities"] = torch.rand(P, 1, generator=gen) * 0.6 + 0.4
+    pre = H.oracle_preprocess(orc, g, cam)
+    got_pre, _ = H.preprocess_fwd(g, cam)
+    assert np.array_equal(got_pre["radii"].cpu().numpy(), pre["radii"])
+    assert np.array_equal(H.np_u32(got_pre["depths"].view(torch.int32)), pre["depths"].view(np.uint32))
+    for k in ("means2D", "conic_opacity", "rgb"):
+        assert np.array_equal(got_pre[k].cpu().numpy(), pre[k], equal_nan=True), k
+    assert (pre["radii"] > 5000).sum() > P // 10   # the needles are what they are meant to be
+    gx, gy = H.grid(W, Hh)
+    cl = np.ones(gx * gy, bool)
+    b = orc.bin_and_sort(pre["radii"], pre["means2D"], pre["depths"], cl, W, Hh)
+    am = gs_scenes.build_all_map(g["means3D"], g["scales"], g["rotations"], cam).numpy()
+    bg = np.zeros(3, np.float32)
+    ref = orc.render_fwd(b["ranges"], b["point_list"], pre["means2D"], pre["rgb"], am, pre["conic_opacity"], cl, bg, W,
+                         Hh, cam.tanfovx, cam.tanfovy, render_geo=True)
+    got = H.render_fwd(P, W, Hh, cam.tanfovx, cam.tanfovy, H.as_u32(b["ranges"]), H.as_u32(b["point_list"]),
+                       H.dev(pre["means2D"]), H.dev(pre["rgb"]), H.dev(am), H.dev(pre["conic_opacity"]), H.dev(cl),
+                       H.dev(bg), render_geo=True)
+    assert ref["n_contrib2loss"].sum() > W * Hh
+    for k in ("n_contrib", "n_contrib2loss"):
+        assert np.array_equal(H.np_u32(got[k]), ref[k]), k
+    assert np.array_equal(got["out_observe"].cpu().numpy(), ref["out_observe"])
+    assert np.array_equal(got["final_T"].cpu().numpy(), ref["final_T"])
+    assert np.array_equal(got["color"].cpu().numpy(), ref["color"])
+    # ... and back: the same contributors, so the sums differ by their order only
+    ug = gs_scenes.upstream_grads(cam)
+    gpix, gmap = ug["color"].numpy(), ug["all_map"].numpy()
+    gdep = np.zeros((1, Hh, W), np.float32)
+    rb = orc.render_bwd(b["ranges"], b["point_list"], pre["means2D"], pre["conic_opacity"], pre["rgb"], am,
+                        ref["out_all_map"], ref["final_T"], ref["n_contrib"], cl, bg, gpix, gmap, gdep, W, Hh,
+                        cam.tanfovx, cam.tanfovy, render_geo=True)
+    gb = H.render_bwd(P, W, Hh, cam.tanfovx, cam.tanfovy, H.dev(bg), H.as_u32(b["ranges"]), H.as_u32(b["point_list"]),
+                      H.dev(pre["means2D"]), H.dev(pre["conic_opacity"]), H.dev(pre["rgb"]), H.dev(am),
+                      H.dev(ref["out_all_map"]), H.dev(ref["final_T"]), H.as_u32(ref["n_contrib"]), H.dev(cl),
+                      H.dev(gpix), H.dev(gmap), H.dev(gdep), H.as_u32(b["emission_sorted"]),
+                      H.as_u32(b["point_offsets"]), render_geo=True)
+    for k, r in (("dL_dmeans2D", rb["dL_dmeans2D"][:, :2]), ("dL_dconic_opacity", rb["dL_dconic_opacity"]),
+                 ("dL_dcolors", rb["dL_dcolors"]), ("dL_dall_map", rb["dL_dall_map"])):
+        a = gb[k].cpu().numpy()
+        assert np.isfinite(a).all(), k
+        assert H.rel_l2(a, r) <= GRAD_TOL, f"{k}: rel L2 {H.rel_l2(a, r)}"
+
+
 @pytest.mark.parametrize("geo", [True, False])
 def test_non_finite_colours_reach_only_the_pixels_that_blend_them(H, orc, geo):
     """A Gaussian whose colour or geometry channels are NaN or infinite (what a diverging training step hands the
