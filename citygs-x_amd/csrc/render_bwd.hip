@@ -267,12 +267,24 @@ render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
       __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
       const uint32_t my_len = row == 0 ? len0 : (row == 1 ? len1 : (row == 2 ? len2 : len3));
       const uint32_t passes = max(max(len0, len1), max(len2, len3));  // wave-uniform
+      // The passes in which two rows of the wave are at the same Gaussian (their sums are merged before they go
+      // to the accumulator) are known as soon as the lists are: bit n of meet_m = entry n of two lists is the
+      // same slot.  Lane n looks at entry n of the four lists.
+      uint64_t meet_m;
+      {
+        const uint8_t* lists = reinterpret_cast<const uint8_t*>(&s_idx[wave][0][0]);
+        const uint32_t e0 = lists[lane], e1 = lists[SUB + lane], e2 = lists[2 * SUB + lane], e3 = lists[3 * SUB + lane];
+        const bool v0 = (uint32_t)lane < len0, v1 = (uint32_t)lane < len1, v2 = (uint32_t)lane < len2,
+                   v3 = (uint32_t)lane < len3;
+        meet_m = gs_ballot((v0 && v1 && e0 == e1) || (v0 && v2 && e0 == e2) || (v0 && v3 && e0 == e3) ||
+                           (v1 && v2 && e1 == e2) || (v1 && v3 && e1 == e3) || (v2 && v3 && e2 == e3));
+      }
 
       // SELECT: a lane for which the Gaussian does not count takes the Gaussian's colour and geometry channels
       // as 0 (its step then still only rotates the recurrence state: alpha = 0 with a finite colour), so that a
       // non-finite channel only reaches the pixels that blended it in the forward pass, as in the reference
       // (cuda_rasterizer/backward.cu:463-472).  Same bits for finite inputs.
-      auto walk = [&, my_len, passes](auto select_tag) {
+      auto walk = [&, my_len, passes, meet_m](auto select_tag) {
         constexpr bool SELECT = decltype(select_tag)::value;
         uint32_t word = 0u;  // four entries of the list
         for (uint32_t n = 0; n < passes; n++) {
@@ -365,11 +377,11 @@ render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
           // adds the sum to the wave's own accumulator with a plain read-add-write: rows that write hold
           // different Gaussians, so their addresses differ.  (An LDS float atomic takes about three cycles per
           // active lane on this hardware, thirteen times the read-add-write.)
-          const int key = has ? ja : -1 - row;
-          const int k0 = __builtin_amdgcn_readlane(key, 0), k1 = __builtin_amdgcn_readlane(key, 16);
-          const int k2 = __builtin_amdgcn_readlane(key, 32), k3 = __builtin_amdgcn_readlane(key, 48);
           bool writes = has;
-          if (k0 == k1 || k0 == k2 || k0 == k3 || k1 == k2 || k1 == k3 || k2 == k3) {  // wave-uniform, uncommon
+          if ((meet_m >> n) & 1ull) {  // wave-uniform, uncommon
+            const int key = has ? ja : -1 - row;
+            const int k0 = __builtin_amdgcn_readlane(key, 0), k1 = __builtin_amdgcn_readlane(key, 16);
+            const int k2 = __builtin_amdgcn_readlane(key, 32), k3 = __builtin_amdgcn_readlane(key, 48);
             constexpr uint64_t R0 = 0xFFFFull, R1 = R0 << 16, R2 = R0 << 32, R3 = R0 << 48;
             const uint64_t eq16 = (k0 == k1 ? R0 | R1 : 0ull) | (k2 == k3 ? R2 | R3 : 0ull);
             const uint64_t eq32 = (k0 == k2 ? R0 | R2 : 0ull) | (k1 == k3 ? R1 | R3 : 0ull);
