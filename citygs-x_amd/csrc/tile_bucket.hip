@@ -401,17 +401,18 @@ bucket_scatter_kernel(int P, int per_block, uint32_t gx, uint32_t gy, const floa
   }
 }
 
-// 2. Per-tile sort, register variant: one workgroup of W waves per tile (4 for lists of up to 2048 records, 16
-// for longer ones).  A wave holds 64 E records, record i = r * 64 + lane in register r of its lane, and the waves
-// hold consecutive runs of 64 E, so a list of up to 64 E W records is sorted with E = 1 .. 8.  In the bitonic
-// network a step pairs i with i ^ j:
+// 2. Per-tile sort, register variant: one workgroup of W waves per tile (4 for lists of up to 256 records, 8 up
+// to 2048, 16 for longer ones).  A wave holds 64 E records, record i = r * 64 + lane in register r of its lane, and
+// the waves hold consecutive runs of 64 E, so a list of up to 64 E W records is sorted with E = 1 .. 8.  In the
+// bitonic network a step pairs i with i ^ j:
 //   j < 64        the partner sits in another lane, same register: one cross-lane read, keep the smaller or larger;
 //   64 <= j < 64E the partner sits in another register of the same lane: no data moves at all;
 //   j >= 64 E     the partner sits in another wave: one exchange through LDS (3 such steps in a whole sort with
-//                 4 waves, 10 with 16).
-// The direction of a step, ((i & k) == 0) ascending, and which of the pair an element keeps are computed from
-// the indices.  Short dependency chains matter more than instruction count here: every tile is resident at once,
-// so the kernel takes as long as its longest tile, and many waves with few records each finish it soonest.
+//                 4 waves, 6 with 8, 10 with 16).
+// A tile takes as long as the instruction stream of one of its waves, and the kernel as long as its longest tiles:
+// a long list is spread over more waves rather than more registers per lane (eight waves with four records per
+// lane for 2048 records, not four with eight).  Sixteen waves for every list were measured too: the launch of so
+// many waves that leave at once costs more than the shorter streams save.
 
 // Which element of a pair (a, b) each lane keeps is decided in scalar registers: keep_min is the lane mask of the
 // elements that keep the smaller one, less the lane mask of a < b; a lane keeps a where the two agree.
@@ -574,7 +575,7 @@ __device__ __forceinline__ void register_sort_tile(uint32_t t, uint32_t start, u
 // 256 records).
 #define GS_SORT_CASE(EE, WW) \
   register_sort_tile<EE, WW>(t, start, n, records, gauss_of_emission, keys, emission, point_list, s_exchange)
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(512)
 tile_sort_registers_kernel(const uint32_t* __restrict__ ranges, const uint64_t* __restrict__ records,
                            const uint32_t* __restrict__ gauss_of_emission, uint64_t* __restrict__ keys,
                            uint32_t* __restrict__ emission, uint32_t* __restrict__ point_list, uint32_t max_n,
@@ -585,10 +586,12 @@ tile_sort_registers_kernel(const uint32_t* __restrict__ ranges, const uint64_t* 
   const uint32_t start = ranges[2 * t];
   const uint32_t n = ranges[2 * t + 1] - start;
   if (n == 0 || n > 2048 || n > max_n) return;
-  if (n <= 256) GS_SORT_CASE(1, 4);
-  else if (n <= 512) GS_SORT_CASE(2, 4);
-  else if (n <= 1024) GS_SORT_CASE(4, 4);
-  else GS_SORT_CASE(8, 4);
+  if (n <= 256) {
+    if (threadIdx.x >= 256) return;  // (half the workgroup is enough; a wave that has left is not waited for)
+    GS_SORT_CASE(1, 4);
+  } else if (n <= 512) GS_SORT_CASE(1, 8);
+  else if (n <= 1024) GS_SORT_CASE(2, 8);
+  else GS_SORT_CASE(4, 8);
 }
 
 __global__ void __launch_bounds__(1024)
@@ -789,7 +792,7 @@ int launch_tile_sort(int T, uint32_t longest, uint32_t limit, uint32_t chunks, c
   const uint32_t whole = longest < limit ? longest : limit;  // the longest list sorted by one workgroup
   uint32_t m = 256;
   while (m < whole && m < 2048) m <<= 1;
-  hipLaunchKernelGGL(tile_sort_registers_kernel, dim3(T), dim3(256), (size_t)m * sizeof(uint64_t), stream, ranges,
+  hipLaunchKernelGGL(tile_sort_registers_kernel, dim3(T), dim3(512), (size_t)m * sizeof(uint64_t), stream, ranges,
                      records, gauss_of_emission, keys, emission, point_list, limit, fits);
   if (whole > 2048)
     hipLaunchKernelGGL(tile_sort_registers_long_kernel, dim3(T), dim3(1024),
