@@ -10,21 +10,25 @@
 // Per batch a wave tests, for each of its four rows, which Gaussians' alpha >= 1/255
 // ellipses (slightly inflated) can reach the row's 4x4 block, and compacts the
 // slot numbers of those that can into a byte list per row in LDS (a lane's
-// place in the list is the number of hits in the lanes below it); the four rows
-// then walk their own lists concurrently, entry n of each in pass n,
-// so one pass of the loop blends up to four different Gaussians and a
-// Gaussian that cannot touch a block costs that row nothing.  Pixels keep
-// their own front-to-back order, which is all the blend needs.  A row stops
-// when its 16 pixels have saturated; a batch is not fetched once all have.
-// The same hits, 16 bits per sorted instance, are left for the backward pass.
-// Registers decide how many waves a SIMD holds here (72 allow seven), and a
+// place in the list is the number of hits in the lanes below it).  A pixel
+// blends about a quarter of its block's list, so the lists are walked 32
+// entries at a time in two steps: every lane marks, one bit per entry, the
+// entries that can reach its own pixel (a fused quadratic form against a
+// limit, eleven instructions an entry), then blends its marked entries in
+// order, the k-th marked one in pass k, whichever entry that is for the other
+// lanes; a chunk takes as many blend passes as its busiest pixel has marks.
+// Pixels keep their own front-to-back order, which is all the blend needs.
+// A row stops when its 16 pixels have saturated; a batch is not fetched once
+// all have.  The rows' hits, 16 bits per sorted instance, are left for the
+// backward pass.
+// Registers decide how many waves a SIMD holds here (80 allow six), and a
 // kernel that spills to scratch memory starts its waves much more slowly, so
 // index arithmetic is kept from being hoisted across the blend loop.
 //
 // The per-pixel arithmetic keeps a fixed operation order, so contributor
 // counts and images match a CPU evaluation bit for bit; exp() is gs_expf.
-// out_observe increments are counted per row with a ballot, summed per
-// workgroup in LDS and added once per (tile, Gaussian).
+// out_observe increments are counted per lane in LDS, two 16-bit counts a
+// word, and added once per (tile, Gaussian).
 #include <type_traits>
 
 #include "gs_common.h"
@@ -36,6 +40,12 @@ namespace gs {
 namespace {
 
 constexpr int BATCH = GS_TILE_PIX;
+constexpr int CHUNK = 32;  // entries of a list marked, then blended, at a time: one bit each in a register
+
+// The exponent of a Gaussian at offset (dx, dy) from its centre (cuda_rasterizer/forward.cu:366).
+__device__ __forceinline__ float gauss_power(const float4 co, const float dx, const float dy) {
+  return -0.5f * (co.x * dx * dx + co.z * dy * dy) - co.y * dx * dy;
+}
 
 // The value itself, but opaque to the optimizer from here on: what is computed from it stays behind this point
 // instead of being hoisted out of the batch loop, where every hoisted LDS address holds a register through the
@@ -49,7 +59,7 @@ __device__ __forceinline__ int not_hoisted(int x) {
 // that blends with the largest weight alpha * T (the front-most one among equals; 0 where nothing blends).  It
 // leaves every other output as it is.
 template <bool RENDER_GEO, bool MAX_DEPTH>
-__global__ void __launch_bounds__(GS_TILE_PIX) __attribute__((amdgpu_waves_per_eu(7)))
+__global__ void __launch_bounds__(GS_TILE_PIX) __attribute__((amdgpu_waves_per_eu(6)))
 render_fwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__ point_list, int W, int H, float fx,
                   float fy, float cx, float cy, const float2* __restrict__ means2D, const float* __restrict__ rgb,
                   const float* __restrict__ all_map, const float4* __restrict__ conic_opacity,
@@ -65,12 +75,14 @@ render_fwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
   // launched ahead of the host's decision on how the per-tile lists are built: nothing to do if they were not
   if (fits_word != nullptr && *fits_word == 0u) return;
   __shared__ float s_depth[MAX_DEPTH ? BATCH : 1];
-  __shared__ float2 s_xy[BATCH];
-  __shared__ float4 s_co[BATCH];
+  // a slot's geometry, (x, y, A, B) and (C, mark limit, opacity, exponent floor), and its channels, (r, g, b, map0)
+  // and (map1 .. map4), in four arrays of 16-byte elements: one address per slot serves them all, and lanes
+  // that read different slots spread over all the banks
+  __shared__ float4 s_geo0[BATCH];
+  __shared__ float4 s_geo1[BATCH];
+  __shared__ float4 s_col0[BATCH];
+  __shared__ float4 s_col1[RENDER_GEO ? BATCH : 1];
   __shared__ float2 s_cull[BATCH];  // packed_cull_params
-  __shared__ float s_floor[BATCH];
-  __shared__ float s_rgb[GS_N_RGB][BATCH];
-  __shared__ float s_map[GS_N_MAP][BATCH];
   // observation counts of slots 2w and 2w + 1 in the low and high half of word w (a count is at most 256)
   __shared__ uint32_t s_obs[BATCH / 2];
   // the four rows' lists of every wave: the slots of the batch that can touch the row's block, one byte each, in
@@ -144,25 +156,33 @@ render_fwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
       const float2 xy = means2D[g];
       const float4 co = conic_opacity[g];
       float pfl;
-      s_xy[ts] = xy;
-      s_co[ts] = co;
       s_cull[ts] = pack_cull_params(cull_params(co, pfl));
-      s_floor[ts] = pfl;
+      // The marking step evaluates the quadratic form A dx^2 + 2 B dx dy + C dy^2 with fused operations, the
+      // blend the exponent -0.5 (A dx^2 + C dy^2) - B dx dy with one rounding per operation; both are within a
+      // few units in the last place of the sum S of the magnitudes of their terms.  A mark limit of twice the
+      // exponent floor plus 2e-6 S, S taken at the tile's pixel farthest from the centre, marks every entry
+      // whose exponent the blend finds at or above the floor (the blend tests the exponent itself again).
+      const float tile_x0 = (float)(blockIdx.x * GS_TILE_X), tile_y0 = (float)(blockIdx.y * GS_TILE_Y);
+      const float far_x = fmaxf(fabsf(xy.x - tile_x0), fabsf(xy.x - (tile_x0 + (float)(GS_TILE_X - 1))));
+      const float far_y = fmaxf(fabsf(xy.y - tile_y0), fabsf(xy.y - (tile_y0 + (float)(GS_TILE_Y - 1))));
+      const float spread = co.x * far_x * far_x + 2.0f * fabsf(co.y) * far_x * far_y + co.z * far_y * far_y;
+      s_geo0[ts] = make_float4(xy.x, xy.y, co.x, co.y);
+      s_geo1[ts] = make_float4(co.z, __builtin_fmaf(2e-6f, spread, -2.0f * pfl), co.w, pfl);
       const float c0 = rgb[3 * (size_t)g], c1 = rgb[3 * (size_t)g + 1], c2 = rgb[3 * (size_t)g + 2];
-      s_rgb[0][ts] = c0;
-      s_rgb[1][ts] = c1;
-      s_rgb[2][ts] = c2;
       float mag = fmaxf(fmaxf(fabsf(c0), fabsf(c1)), fabsf(c2));
       finite = c0 == c0 && c1 == c1 && c2 == c2;
+      float m[GS_N_MAP] = {0.f, 0.f, 0.f, 0.f, 0.f};
       if (render_geo) {
 #pragma unroll
         for (int ch = 0; ch < GS_N_MAP; ch++) {
           const float v = all_map[5 * (size_t)g + ch];
-          s_map[ch][ts] = v;
+          m[ch] = v;
           mag = fmaxf(mag, fabsf(v));
           finite = finite && v == v;
         }
       }
+      s_col0[ts] = make_float4(c0, c1, c2, m[0]);
+      if constexpr (RENDER_GEO) s_col1[ts] = make_float4(m[1], m[2], m[3], m[4]);
       finite = finite && mag < __builtin_inff();
       if (MAX_DEPTH) s_depth[ts] = depths[g];
     }
@@ -192,9 +212,10 @@ render_fwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
         const int jj = k * GS_WAVE + lane_b;
         const bool valid = jj < count;
         const uint64_t valid_m = gs_ballot(valid);
-        const float2 mu = s_xy[valid ? jj : 0];
-        const float4 cq = s_co[valid ? jj : 0];
-        const float4 cp = unpack_cull_params(s_cull[valid ? jj : 0], s_floor[valid ? jj : 0]);
+        const float4 geo0 = s_geo0[valid ? jj : 0], geo1 = s_geo1[valid ? jj : 0];
+        const float2 mu = make_float2(geo0.x, geo0.y);
+        const float4 cq = make_float4(geo0.z, geo0.w, geo1.x, geo1.z);
+        const float4 cp = unpack_cull_params(s_cull[valid ? jj : 0], geo1.w);
         // (the four tests first, in one straight line and unconditionally, so that what they have in common is
         // computed once; masks of single comparisons, combined in scalar registers)
         uint64_t hit_m[4];
@@ -244,68 +265,114 @@ render_fwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
       constexpr bool SELECT = decltype(select_tag)::value;
       uint32_t my_len = row_len;
       uint32_t passes = max(max(len0, len1), max(len2, len3));  // wave-uniform
-      uint32_t word = 0u;  // four entries of the list
-      for (uint32_t n = 0; n < passes; n++) {
-        if ((n & 3u) == 0u) word = s_idx[wave][row][n >> 2];
-        const uint64_t has_m = gs_ballot(n < my_len);
-        // (slot 0 behind the end of the list: its data are this batch's)
-        const int j = (int)__builtin_amdgcn_ubfe(word, (n & 3u) * 8u, 8u);
+      // Of a 4x4 block's list a single pixel blends about a quarter, so the lists are walked a chunk of 32 entries
+      // at a time, in two steps.  First every lane marks, one bit per entry, the entries whose exponent lies in
+      // its window (the cheap part of a blend: centre, conic, two comparisons).  Then each lane blends its own
+      // marked entries in order, the k-th marked one in pass k, whichever entry that is for its neighbours: a
+      // chunk takes as many passes as its busiest pixel has marks.  A pixel's entries keep their order, which is
+      // all the blend needs.
+      float done = __builtin_amdgcn_inverse_ballot_w64(alive) ? 0.f : 1.f;  // 1: this pixel has saturated (or lies outside)
+      const uint8_t* const my_list = reinterpret_cast<const uint8_t*>(&s_idx[wave][row][0]);
+      for (uint32_t base = 0; base < passes; base += CHUNK) {
+        uint32_t marks = 0u;
+        const uint32_t words = min((uint32_t)CHUNK / 4u, (passes - base + 3u) / 4u);
+        // (last entry first: a mark is shifted in at bit 0, as the carry of marks + marks, so entry e of the chunk
+        // ends at bit e)
+        for (int q = (int)words - 1; q >= 0; q--) {
+          const uint32_t word = s_idx[wave][row][(base >> 2) + (uint32_t)q];  // (zero, slot 0, behind the list's end)
+#pragma unroll
+          for (int u = 3; u >= 0; u--) {
+            const int j = (int)__builtin_amdgcn_ubfe(word, 8u * u, 8u);
+            const float4 g0 = s_geo0[j];
+            const float2 g1 = *reinterpret_cast<const float2*>(&s_geo1[j]);  // C and the mark limit
+            const float dx = g0.x - pfx, dy = g0.y - pfy;
+            const float form = __builtin_fmaf(g1.x * dy, dy, __builtin_fmaf(g0.z, dx, g0.w * (dy + dy)) * dx);
+            // marked unless the form exceeds the limit (so a NaN marks, as the blend's own tests let it through)
+            asm("v_cmp_ngt_f32 vcc, %1, %2\n\tv_addc_co_u32 %0, vcc, %0, %0, vcc"
+                : "+v"(marks)
+                : "v"(form), "v"(g1.y)
+                : "vcc");
+          }
+        }
+        {
+          const uint32_t mine = my_len > base ? my_len - base : 0u;  // entries of the chunk that are in the list
+          marks = mine >= (uint32_t)CHUNK ? marks : (marks & ((1u << mine) - 1u));
+          marks = (done != 0.f) ? 0u : marks;
+        }
+        // (the slot of a lane's next marked entry is fetched one pass ahead)
+        uint32_t slot_next = my_list[base + ((uint32_t)__builtin_ctz(marks | 0x80000000u))];
+        // (tested at the bottom: the ballot cannot be copied, so a loop tested at the top is not rotated and pays
+        // a register copy per accumulator and pass)
+        if (gs_ballot(marks != 0u) != 0ull) do {
+          const bool active = marks != 0u;
+          const int j = active ? (int)slot_next : 0;  // (slot 0's data are this batch's)
+          marks &= marks - 1u;
+          slot_next = my_list[base + ((uint32_t)__builtin_ctz(marks | 0x80000000u))];
+          const float4 g0 = s_geo0[j], g1 = s_geo1[j];
+          const float2 xy = make_float2(g0.x, g0.y);
+          const float4 co = make_float4(g0.z, g0.w, g1.x, g1.z);
+          const float floor_j = g1.w;
+          float c[GS_N_RGB + GS_N_MAP] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+          {
+            const float4 c0 = s_col0[j];
+            c[0] = c0.x, c[1] = c0.y, c[2] = c0.z, c[3] = c0.w;
+            if constexpr (RENDER_GEO) {
+              const float4 c1 = s_col1[j];
+              c[4] = c1.x, c[5] = c1.y, c[6] = c1.z, c[7] = c1.w;
+            }
+          }
+          float depth_j = 0.f;
+          if (MAX_DEPTH) depth_j = s_depth[j];
 
-        // Straight-line: every lane evaluates its row's Gaussian; a lane for which it does not count blends
-        // with weight 0, which leaves its sums unchanged bit for bit (fma(c, 0, C) == C).  The tests are kept as
-        // lane masks of single comparisons and combined in scalar registers.
-        const float2 xy = s_xy[j];
-        const float4 co = s_co[j];
-        const float dx = xy.x - pfx, dy = xy.y - pfy;
-        const float power = -0.5f * (co.x * dx * dx + co.z * dy * dy) - co.y * dx * dy;
-        const float floor_j = s_floor[j];
-        const uint64_t in_m = has_m & alive & gs_ballot(!(power > 0.0f)) & gs_ballot(!(power < floor_j));
-        if (in_m == 0ull) continue;
-        const float alpha = fminf(0.99f, co.w * gs_expf_core(power));
-        const uint64_t pass_m = in_m & gs_ballot(!(alpha < 1.0f / 255.0f));
-        const float test_T = T * (1 - alpha);
-        const uint64_t stop_m = pass_m & gs_ballot(test_T < 0.0001f);
-        const uint64_t bmask = pass_m & ~stop_m;
-        if (bmask != 0ull) {
-          const bool blend = __builtin_amdgcn_inverse_ballot_w64(bmask);
-          n2l += blend ? 1u : 0u;
-          // weight once, then one fused multiply-add per channel
+          const float power = gauss_power(co, xy.x - pfx, xy.y - pfy);
+          const float alpha = fminf(0.99f, co.w * gs_expf_core(power));
+          // alpha as far as this lane is concerned: 0 unless it has an entry in this pass and the exponent lies
+          // in the window
+          float a = alpha;
+          a = (power > 0.0f) ? 0.f : a;
+          a = (power < floor_j) ? 0.f : a;
+          a = active ? a : 0.f;
+          a = (a < 1.0f / 255.0f) ? 0.f : a;            // (NaN stays: the reference blends it too)
+          const bool counts = a != 0.f;                  // alpha >= 1/255 and everything above
+          const float test_T = T * (1 - alpha);          // (of use where the entry counts: a == alpha there)
+          const bool stops = counts && test_T < 0.0001f;
+          const bool blend = counts && !stops;
+          // weight once, then one fused multiply-add per channel; w == 0 where the entry does not blend
           const float w = blend ? alpha * T : 0.f;
+          done = stops ? 1.f : done;
+          marks = stops ? 0u : marks;
+          n2l += blend ? 1u : 0u;
 #pragma unroll
           for (int ch = 0; ch < GS_N_RGB; ch++) {
-            const float sum = __builtin_fmaf(s_rgb[ch][j], w, C[ch]);
+            const float sum = __builtin_fmaf(c[ch], w, C[ch]);
             C[ch] = (!SELECT || blend) ? sum : C[ch];
           }
           if (render_geo) {
 #pragma unroll
             for (int ch = 0; ch < GS_N_MAP; ch++) {
-              const float sum = __builtin_fmaf(s_map[ch][j], w, Mp[ch]);
+              const float sum = __builtin_fmaf(c[GS_N_RGB + ch], w, Mp[ch]);
               Mp[ch] = (!SELECT || blend) ? sum : Mp[ch];
             }
           }
           if (MAX_DEPTH) {
             const bool better = w > best_w;  // w is 0 for a lane that does not blend
-            best_depth = better ? s_depth[j] : best_depth;
+            best_depth = better ? depth_j : best_depth;
             best_w = better ? w : best_w;
           }
-          const uint64_t omask = bmask & gs_ballot(T > 0.5f);
-          if (omask != 0ull) {
-            const uint32_t cnt = (uint32_t)__popc((uint32_t)(omask >> row_shift) & 0xFFFFu);
-            if (rt.l16 == 0 && cnt != 0u) atomicAdd(&s_obs[j >> 1], cnt << (16 * (j & 1)));
-          }
+          // observation count of the entry: one for a lane that blends it with T > 0.5
+          if (blend && T > 0.5f) atomicAdd(&s_obs[j >> 1], 1u << (16 * (j & 1)));
           T = blend ? test_T : T;
           last = blend ? (uint32_t)(i * BATCH + j + 1) : last;
-        }
-        if (stop_m != 0ull) {
-          alive &= ~stop_m;
-          // a row whose 16 pixels have all saturated drops the rest of its list
-          if (((uint32_t)(alive >> row_shift) & 0xFFFFu) == 0u) my_len = 0u;
-          passes = 0u;
-          if (((uint32_t)alive & 0xFFFFu) != 0u) passes = len0;
-          if (((uint32_t)(alive >> 16) & 0xFFFFu) != 0u) passes = max(passes, len1);
-          if (((uint32_t)(alive >> 32) & 0xFFFFu) != 0u) passes = max(passes, len2);
-          if (((uint32_t)(alive >> 48) & 0xFFFFu) != 0u) passes = max(passes, len3);
-        }
+        } while (gs_ballot(marks != 0u) != 0ull);
+        // a row whose 16 pixels have all saturated drops the rest of its list
+        alive = gs_ballot(done == 0.f);
+        if (((uint32_t)(alive >> row_shift) & 0xFFFFu) == 0u) my_len = 0u;
+        uint32_t left = 0u;
+        if (((uint32_t)alive & 0xFFFFu) != 0u) left = len0;
+        if (((uint32_t)(alive >> 16) & 0xFFFFu) != 0u) left = max(left, len1);
+        if (((uint32_t)(alive >> 32) & 0xFFFFu) != 0u) left = max(left, len2);
+        if (((uint32_t)(alive >> 48) & 0xFFFFu) != 0u) left = max(left, len3);
+        passes = left;
       }
       };
       if (select_blend) walk(std::true_type{});
