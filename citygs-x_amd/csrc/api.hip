@@ -135,7 +135,7 @@ ImageLayout image_layout(int W, int H) {
 }
 
 struct GeometryLayout {
-  size_t tiles_touched, point_offsets, scan_temp, total;
+  size_t tiles_touched, point_offsets, scan_temp, packed, total;
 };
 GeometryLayout geometry_layout(int P) {
   GeometryLayout L;
@@ -145,6 +145,7 @@ GeometryLayout geometry_layout(int P) {
   L.tiles_touched = take(n * 4);
   L.point_offsets = take(n * 4);
   L.scan_temp = take(scan_temp_bytes((int64_t)n));
+  L.packed = take(n * 64);  // the blend kernels' operands, one 64-byte record per Gaussian
   L.total = off + 256;
   return L;
 }
@@ -479,6 +480,7 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
   uint32_t* tiles_touched = (uint32_t*)(gbase + GL.tiles_touched);
   uint32_t* point_offsets = (uint32_t*)(gbase + GL.point_offsets);
   void* scan_temp = gbase + GL.scan_temp;
+  float* packed = (float*)(gbase + GL.packed);
 
   const ImageLayout IL = image_layout(width, height);
   char* ibase = imageBuffer(IL.total, image_user);
@@ -534,6 +536,15 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
     launch_inclusive_sum(P, tiles_touched, point_offsets, scan_temp, stream, total_slot);
   }
   if (check_launch("inclusive_sum", stream, dbg)) return 1;
+  {
+    // The blend kernels (this call's and the backward call's) fetch a Gaussian's operands as one 64-byte record.
+    // Queued behind the counting kernels: where the host has to wait for the instance count before it can size
+    // the binning buffer, the GPU packs meanwhile.
+    StageScope _t("pack_operands", stream);
+    launch_pack_blend_operands(P, radii, means2D, conic_opacity, rgb, render_geo ? all_map : nullptr, depths, packed,
+                               stream);
+  }
+  if (check_launch("pack_operands", stream, dbg)) return 1;
 
   EventTimer timer;
   struct Arrays {
@@ -571,6 +582,7 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
     a.n_render = n_render; a.n_consider = n_consider; a.n_contrib_tile = n_contrib;
     a.fits_word = ahead_of_host ? bucket_fits_word(bucket_table, T) : nullptr;
     a.block_hits = A.block_hits;
+    a.packed = packed;
     {
       StageScope _t("render_fwd", stream);
       launch_render_fwd(a, stream);
@@ -733,6 +745,7 @@ int gs_render_backward(int P, int R, const float* background, int width, int hei
   a.emission_sorted = (const uint32_t*)(bbase + BL.emission);
   a.block_hits = (const uint16_t*)(bbase + BL.block_hits);
   a.point_offsets = (const uint32_t*)(gbase + GL.point_offsets);
+  a.packed = (const float*)(gbase + GL.packed);  // (of the arrays the forward call was given)
   a.instance_grads = (float*)align_ptr((const char*)instance_grads, 256);
   a.P = P; a.W = width; a.H = height;
   a.fy = height / (2.0f * tan_fovy);  // cuda_rasterizer/rasterizer_impl.cu:885-886

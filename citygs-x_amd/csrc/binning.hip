@@ -191,6 +191,50 @@ gather_u32_kernel(int64_t n, const uint32_t* __restrict__ index, const uint32_t*
   if (i < n) out[i] = table[index[i]];
 }
 
+// One thread per Gaussian.  A wave's 64 records (4 KB, contiguous) pass through LDS so that every store
+// instruction writes one contiguous kilobyte: lane l stores 16-byte word (l & 3) of record 16 k + (l >> 2) in
+// round k.  (In LDS a record's four words sit 1040 bytes apart, so that neither the writes, record-major, nor the
+// reads, word-minor, pile up on a few banks.)  A wave none of whose Gaussians is visible stores nothing; in a wave
+// with some, the invisible ones' records are written too (zeros for the colour of a culled Gaussian do no harm:
+// no tile lists it).
+__global__ void __launch_bounds__(GS_BLOCK_1D)
+pack_blend_operands_kernel(int P, const int* __restrict__ radii, const float2* __restrict__ means2D,
+                           const float4* __restrict__ conic_opacity, const float* __restrict__ rgb,
+                           const float* __restrict__ all_map, const float* __restrict__ depths,
+                           float4* __restrict__ packed) {
+  constexpr int WORD_STRIDE = GS_WAVE + 1;  // in 16-byte units
+  __shared__ float4 s_rec[GS_BLOCK_1D / GS_WAVE][4 * WORD_STRIDE];
+  const int lane = threadIdx.x & (GS_WAVE - 1), wave = threadIdx.x / GS_WAVE;
+  const int i = blockIdx.x * GS_BLOCK_1D + threadIdx.x;
+  const bool live = i < P && radii[i] > 0;
+  if (gs_ballot(live) == 0ull) return;
+  const int ic = i < P ? i : P - 1;
+  const float2 xy = means2D[ic];
+  const float4 co = conic_opacity[ic];
+  const float c0 = rgb[3 * (size_t)ic], c1 = rgb[3 * (size_t)ic + 1], c2 = rgb[3 * (size_t)ic + 2];
+  float m[5] = {0.f, 0.f, 0.f, 0.f, 0.f};
+  if (all_map != nullptr) {
+#pragma unroll
+    for (int ch = 0; ch < 5; ch++) m[ch] = all_map[5 * (size_t)ic + ch];
+  }
+  const float d = depths != nullptr ? depths[ic] : 0.f;
+  float4* mine = &s_rec[wave][0];
+  mine[0 * WORD_STRIDE + lane] = make_float4(xy.x, xy.y, co.x, co.y);
+  mine[1 * WORD_STRIDE + lane] = make_float4(co.z, co.w, c0, c1);
+  mine[2 * WORD_STRIDE + lane] = make_float4(c2, m[0], m[1], m[2]);
+  mine[3 * WORD_STRIDE + lane] = make_float4(m[3], m[4], d, 0.f);
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  const int first = blockIdx.x * GS_BLOCK_1D + wave * GS_WAVE;  // the wave's first Gaussian
+  float4* out = packed + 4 * (size_t)first;
+#pragma unroll
+  for (int k = 0; k < 4; k++) {
+    const int rec = 16 * k + (lane >> 2), word = lane & 3;
+    if (first + rec < P) out[64 * k + lane] = mine[word * WORD_STRIDE + rec];
+  }
+}
+
 __global__ void fill_u32_kernel(int64_t n, uint32_t v, uint32_t* __restrict__ p) {
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i < n) p[i] = v;
@@ -340,6 +384,16 @@ int launch_duplicate_with_keys(int P, int W, int H, const float* means2D, const 
   hipLaunchKernelGGL(duplicate_with_keys_kernel, dim3((P + GS_BLOCK_1D - 1) / GS_BLOCK_1D), dim3(GS_BLOCK_1D), 0,
                      stream, P, gx, gy, (const float2*)means2D, depths, offsets, radii, compute_locally, keys, values,
                      emission);
+  return 0;
+}
+
+int launch_pack_blend_operands(int P, const int* radii, const float* means2D, const float* conic_opacity,
+                               const float* rgb, const float* all_map, const float* depths, float* packed,
+                               hipStream_t stream) {
+  if (P <= 0) return 0;
+  hipLaunchKernelGGL(pack_blend_operands_kernel, dim3((P + GS_BLOCK_1D - 1) / GS_BLOCK_1D), dim3(GS_BLOCK_1D), 0,
+                     stream, P, radii, (const float2*)means2D, (const float4*)conic_opacity, rgb, all_map, depths,
+                     (float4*)packed);
   return 0;
 }
 

@@ -118,6 +118,12 @@ int launch_bucket_scatter(int P, int W, int H, const float* means2D, const float
 int launch_tile_sort(int T, uint32_t longest, uint32_t limit, uint32_t chunks, const uint32_t* ranges,
                      const void* table, uint64_t* records, const uint32_t* gauss_of_emission, uint64_t* keys,
                      uint32_t* emission, uint32_t* point_list, bool ahead_of_host, hipStream_t stream);
+// What the blend kernels read of a Gaussian, in one 64-byte record per Gaussian: (x, y, A, B), (C, opacity, r, g),
+// (b, map0, map1, map2), (map3, map4, depth, 0); all_map and depths may be null (zeros).  Records of Gaussians with
+// radius 0 are left as they are (no tile lists them).
+int launch_pack_blend_operands(int P, const int* radii, const float* means2D, const float* conic_opacity,
+                               const float* rgb, const float* all_map, const float* depths, float* packed,
+                               hipStream_t stream);
 int launch_gather_u32(int64_t n, const uint32_t* index, const uint32_t* table, uint32_t* out, hipStream_t stream);
 int launch_ssim_l1_fwd(int C, int H, int W, const float* img1, const float* img2, const uint8_t* mask,
                        float* l1_map, float* ssim_map, float* d_mu, float* d_xx, float* d_xy, hipStream_t stream);
@@ -216,6 +222,9 @@ struct RenderFwdArgs {
   // 4 * wave + row), as found by the kernel's own list building; the backward blend reads it instead of testing
   // again
   uint16_t* block_hits = nullptr;
+  // optional (P,4) 16-byte words: pack_blend_operands' records; the kernel then fetches a Gaussian's operands as
+  // one 64-byte line instead of gathering them from means2D, conic_opacity, rgb, all_map (and depths)
+  const float* packed = nullptr;
 };
 int launch_render_fwd(const RenderFwdArgs& a, hipStream_t stream);
 
@@ -236,6 +245,7 @@ struct RenderBwdArgs {
   const uint32_t* point_offsets;
   float* instance_grads;  // (R,16) scratch, fully written by the blend kernel
   const uint16_t* block_hits = nullptr;  // optional (R): left by the forward blend (RenderFwdArgs::block_hits)
+  const float* packed = nullptr;         // optional (P,4) 16-byte words: see RenderFwdArgs::packed
   // outputs, fully written by the per-Gaussian reduction
   float* dL_dmean2D;         // (P,2)
   float* dL_dmean2D_abs;     // (P,3)

@@ -70,7 +70,7 @@ render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
                   const uint8_t* __restrict__ compute_locally, const float* __restrict__ dL_dpix,
                   const float* __restrict__ dL_dout_all_map, const float* __restrict__ dL_dout_plane_depth,
                   const uint32_t* __restrict__ emission_sorted, float4* __restrict__ instance_grads,
-                  const uint16_t* __restrict__ block_hits) {
+                  const uint16_t* __restrict__ block_hits, const float4* __restrict__ packed) {
   constexpr bool render_geo = RENDER_GEO;
   __shared__ uint32_t s_emis[BATCH];
   __shared__ float4 s_xyf[BATCH];  // centre x, y; the power floor; unused
@@ -189,23 +189,45 @@ render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
     if (tid < count) {
       const uint32_t k_sorted = range.x + (uint32_t)(first_pos - tid);
       const uint32_t g = point_list[k_sorted];
-      const float2 xy = means2D[g];
-      const float4 co = conic_opacity[g];
+      // A Gaussian's operands: one 64-byte record where the forward call packed them (a single line of memory,
+      // every byte of it used), else gathered from the four arrays; all loads issued before anything is computed.
+      float2 xy;
+      float4 co;
+      float c0, c1, c2;
+      float m[GS_N_MAP] = {0.f, 0.f, 0.f, 0.f, 0.f};
+      if (packed != nullptr) {
+        const float4* rec = packed + 4 * (size_t)g;
+        const float4 r0 = rec[0], r1 = rec[1], r2 = rec[2];
+        xy = make_float2(r0.x, r0.y);
+        co = make_float4(r0.z, r0.w, r1.x, r1.y);
+        c0 = r1.z, c1 = r1.w, c2 = r2.x;
+        m[0] = r2.y, m[1] = r2.z, m[2] = r2.w;
+        if (render_geo) {
+          const float4 r3 = rec[3];
+          m[3] = r3.x, m[4] = r3.y;
+        }
+      } else {
+        xy = means2D[g];
+        co = conic_opacity[g];
+        c0 = rgb[3 * (size_t)g], c1 = rgb[3 * (size_t)g + 1], c2 = rgb[3 * (size_t)g + 2];
+        if (render_geo) {
+#pragma unroll
+          for (int ch = 0; ch < GS_N_MAP; ch++) m[ch] = all_map[5 * (size_t)g + ch];
+        }
+      }
       s_emis[tid] = emission_sorted[k_sorted];
       s_co[tid] = co;
-      float pfl;
-      const float4 cp = cull_params(co, pfl);
+      float pfl, mark_limit;
+      const float4 cp = block_test_params(co, xy, (float)(blockIdx.x * GS_TILE_X), (float)(blockIdx.y * GS_TILE_Y),
+                                          pfl, mark_limit);
       if (HITS) s_hits[tid] = block_hits[k_sorted];
       else s_cp[tid] = cp;
       s_xyf[tid] = make_float4(xy.x, xy.y, pfl, 0.f);
-      const float c0 = rgb[3 * (size_t)g], c1 = rgb[3 * (size_t)g + 1], c2 = rgb[3 * (size_t)g + 2];
       float mag = fmaxf(fmaxf(fabsf(c0), fabsf(c1)), fabsf(c2));
       finite = c0 == c0 && c1 == c1 && c2 == c2;
-      float m[GS_N_MAP] = {0.f, 0.f, 0.f, 0.f, 0.f};
       if (render_geo) {
 #pragma unroll
         for (int ch = 0; ch < GS_N_MAP; ch++) {
-          m[ch] = all_map[5 * (size_t)g + ch];
           mag = fmaxf(mag, fabsf(m[ch]));
           finite = finite && m[ch] == m[ch];
         }
@@ -244,7 +266,7 @@ render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
         }
         uint64_t hit_m[4];
         bool hits[4] = {false, false, false, false};
-        if (!HITS) ellipse_hits_quadrant(mu, cq, cp, rt.qx0, rt.qy0, hits);
+        if (!HITS) ellipse_hits_quadrant(mu, cq, cp.x, cp.y, cp.z, rt.qx0, rt.qy0, hits);
 #pragma unroll
         for (int r = 0; r < 4; r++) {
           const bool touches = HITS ? ((nibble >> r) & 1u) != 0u : hits[r];
@@ -549,7 +571,8 @@ int launch_render_bwd(const RenderBwdArgs& a, hipStream_t stream) {
     hipLaunchKernelGGL(kernel, grid, dim3(GS_TILE_PIX), 0, stream, (const uint2*)a.ranges, a.point_list, a.W, a.H,
                        a.fx, a.fy, a.bg, (const float2*)a.means2D, (const float4*)a.conic_opacity, a.rgb, a.all_map,
                        a.all_map_pixels, a.final_T, a.n_contrib_px, a.compute_locally, a.dL_dpix, a.dL_dout_all_map,
-                       a.dL_dout_plane_depth, a.emission_sorted, (float4*)a.instance_grads, a.block_hits);
+                       a.dL_dout_plane_depth, a.emission_sorted, (float4*)a.instance_grads, a.block_hits,
+                       (const float4*)a.packed);
   };
   if (a.render_geo) {
     if (a.block_hits) go(render_bwd_kernel<true, true>);

@@ -33,35 +33,36 @@ __device__ __forceinline__ float4 cull_params(float4 co, float& power_floor) {
   return cp;
 }
 
-// cull_params in two words.  A trusted conic keeps (1/A, 1/C), both positive and finite, and its q_max is
-// -2 power_floor (q_max = 2 tau and power_floor = -tau there: tau stays far below 87 for an opacity under 1e30).
-// x = -1 stands for "the opacity alone rules every pixel out", x = +infinity for "the conic cannot be trusted".
-__device__ __forceinline__ float2 pack_cull_params(float4 cp) {
-  if (cp.z < 0.f) return make_float2(-1.0f, 0.f);
-  if (cp.z == __builtin_inff()) return make_float2(__builtin_inff(), 0.f);
-  return make_float2(cp.x, cp.y);
-}
-__device__ __forceinline__ float4 unpack_cull_params(float2 e, float power_floor) {
-  const bool never = e.x < 0.f, always = e.x == __builtin_inff();
-  const bool plain = !(never || always);
-  return make_float4(plain ? e.x : 0.f, plain ? e.y : 0.f,
-                     never ? -1.0f : (always ? __builtin_inff() : -2.0f * power_floor), 0.f);
+// What the block tests of a tile's kernels need of a Gaussian centred at xy: (1/A, 1/C, limit on q, 0), and, in
+// mark_limit, the limit on q for a single pixel of the tile (the forward blend marks the pixels an entry can reach
+// with it).  Both limits are q_max plus a margin for rounding: the block test, the pixel mark and the blend itself
+// evaluate q by different operation sequences at different points, each within a few units in the last place of
+// the LARGEST term, which for a long thin Gaussian far from its centre is much larger than q itself.  Every such
+// term is at most S = A X^2 + 2 |B| X Y + C Y^2 with X, Y the largest offsets of a pixel of the tile from the
+// centre; the margin is 2e-6 S (about 32 units in the last place of S), on top of the 0.02 from tau + 0.01.  The
+// block limit is negative when the opacity alone rules every pixel out and +infinity when the conic cannot be
+// trusted.  The same numbers in the forward and the backward kernel, so both build the same lists.
+__device__ __forceinline__ float4 block_test_params(float4 co, float2 xy, float tile_x0, float tile_y0,
+                                                    float& power_floor, float& mark_limit) {
+  const float4 cp = cull_params(co, power_floor);
+  const float far_x = fmaxf(fabsf(xy.x - tile_x0), fabsf(xy.x - (tile_x0 + (float)(GS_TILE_X - 1))));
+  const float far_y = fmaxf(fabsf(xy.y - tile_y0), fabsf(xy.y - (tile_y0 + (float)(GS_TILE_Y - 1))));
+  const float spread = co.x * far_x * far_x + 2.0f * fabsf(co.y) * far_x * far_y + co.z * far_y * far_y;
+  // (q_max = 2 (tau + 0.01) is -2 power_floor wherever the conic is trusted)
+  mark_limit = __builtin_fmaf(2e-6f, spread, -2.0f * power_floor);
+  const bool never = cp.z < 0.f, untrusted = cp.z == __builtin_inff();
+  return make_float4(cp.x, cp.y, never ? -1.0f : (untrusted ? cp.z : mark_limit), 0.f);
 }
 
 // The four 4x4 pixel blocks of an 8x8 quadrant at (qx0, qy0), block r at x offset 4 (r & 1), y offset 4 (r >> 1):
-// hit[r] = can any point of block r have q <= q_max?  q is convex, so over a block it is smallest either at the
+// hit[r] = can any point of block r have q <= limit?  q is convex, so over a block it is smallest either at the
 // centre (inside the block: 0) or on one of the two block edges that face the centre; along an edge it is a
 // parabola whose minimiser is clamped to the edge.  A block is treated as a continuous rectangle, which can only
 // add hits.  What the two columns and the two rows of blocks have in common is computed once; the parabolas are
-// evaluated in Horner form with fused multiply-adds.
-// Rounding: this evaluation and the per-pixel one (a different operation sequence, at a different point) each
-// carry an error of a few units in the last place of the LARGEST term, which for a long thin Gaussian far from
-// its centre is much larger than q itself.  Every such term is at most S = A X^2 + 2 |B| X Y + C Y^2 with X, Y
-// the largest offsets inside the quadrant, so q_max is raised by 1e-6 S (about 16 units in the last place of S)
-// on top of the 0.02 from tau + 0.01: the test never rejects a block one of whose pixels passes.  NaNs count as
+// evaluated in Horner form with fused multiply-adds.  inv_a, inv_c and limit: block_test_params.  NaNs count as
 // hits.
-__device__ __forceinline__ void ellipse_hits_quadrant(float2 mu, float4 co, float4 cp, float qx0, float qy0,
-                                                      bool (&hit)[4]) {
+__device__ __forceinline__ void ellipse_hits_quadrant(float2 mu, float4 co, float inv_a, float inv_c, float limit,
+                                                      float qx0, float qy0, bool (&hit)[4]) {
   const float two_b = 2.0f * co.y;
   float lox[2], hix[2], dxc[2], t1[2], a1[2], b1[2];  // per column of blocks
   float loy[2], hiy[2], dyc[2], t2[2], a2[2], b2[2];  // per row of blocks
@@ -70,19 +71,16 @@ __device__ __forceinline__ void ellipse_hits_quadrant(float2 mu, float4 co, floa
     lox[c] = (qx0 + (float)(4 * c)) - mu.x;
     hix[c] = lox[c] + 3.0f;
     dxc[c] = fminf(fmaxf(0.f, lox[c]), hix[c]);  // offset of the nearest column of the block
-    t1[c] = -co.y * dxc[c] * cp.y;               // where q is smallest along that column
+    t1[c] = -co.y * dxc[c] * inv_c;              // where q is smallest along that column
     a1[c] = co.x * dxc[c] * dxc[c];
     b1[c] = two_b * dxc[c];
     loy[c] = (qy0 + (float)(4 * c)) - mu.y;
     hiy[c] = loy[c] + 3.0f;
     dyc[c] = fminf(fmaxf(0.f, loy[c]), hiy[c]);  // offset of the nearest row of the block
-    t2[c] = -co.y * dyc[c] * cp.x;               // where q is smallest along that row
+    t2[c] = -co.y * dyc[c] * inv_a;              // where q is smallest along that row
     a2[c] = co.z * dyc[c] * dyc[c];
     b2[c] = two_b * dyc[c];
   }
-  const float X = fmaxf(fabsf(lox[0]), fabsf(hix[1])), Y = fmaxf(fabsf(loy[0]), fabsf(hiy[1]));
-  const float S = (co.x * X * X + fabsf(two_b) * X * Y) + co.z * Y * Y;
-  const float limit = cp.z < 0.f ? cp.z : __builtin_fmaf(1.0e-6f, S, cp.z);
 #pragma unroll
   for (int r = 0; r < 4; r++) {
     const int c = r & 1, d = r >> 1;

@@ -70,7 +70,7 @@ render_fwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
                   float* __restrict__ out_plane_depth, int* __restrict__ n_render, int* __restrict__ n_consider,
                   int* __restrict__ n_contrib_tile, const float* __restrict__ depths,
                   float* __restrict__ out_max_weight_depth, const uint32_t* __restrict__ fits_word,
-                  uint16_t* __restrict__ block_hits) {
+                  uint16_t* __restrict__ block_hits, const float4* __restrict__ packed) {
   constexpr bool render_geo = RENDER_GEO;
   // launched ahead of the host's decision on how the per-tile lists are built: nothing to do if they were not
   if (fits_word != nullptr && *fits_word == 0u) return;
@@ -82,7 +82,8 @@ render_fwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
   __shared__ float4 s_geo1[BATCH];
   __shared__ float4 s_col0[BATCH];
   __shared__ float4 s_col1[RENDER_GEO ? BATCH : 1];
-  __shared__ float2 s_cull[BATCH];  // packed_cull_params
+  // block_test_params
+  __shared__ float4 s_cull[BATCH];
   // observation counts of slots 2w and 2w + 1 in the low and high half of word w (a count is at most 256)
   __shared__ uint32_t s_obs[BATCH / 2];
   // the four rows' lists of every wave: the slots of the batch that can touch the row's block, one byte each, in
@@ -153,38 +154,54 @@ render_fwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
     const int ts = not_hoisted(tid);
     if (ts < count) {
       const uint32_t g = point_list[range.x + (uint32_t)i * BATCH + ts];
-      const float2 xy = means2D[g];
-      const float4 co = conic_opacity[g];
-      float pfl;
-      s_cull[ts] = pack_cull_params(cull_params(co, pfl));
-      // The marking step evaluates the quadratic form A dx^2 + 2 B dx dy + C dy^2 with fused operations, the
-      // blend the exponent -0.5 (A dx^2 + C dy^2) - B dx dy with one rounding per operation; both are within a
-      // few units in the last place of the sum S of the magnitudes of their terms.  A mark limit of twice the
-      // exponent floor plus 2e-6 S, S taken at the tile's pixel farthest from the centre, marks every entry
-      // whose exponent the blend finds at or above the floor (the blend tests the exponent itself again).
-      const float tile_x0 = (float)(blockIdx.x * GS_TILE_X), tile_y0 = (float)(blockIdx.y * GS_TILE_Y);
-      const float far_x = fmaxf(fabsf(xy.x - tile_x0), fabsf(xy.x - (tile_x0 + (float)(GS_TILE_X - 1))));
-      const float far_y = fmaxf(fabsf(xy.y - tile_y0), fabsf(xy.y - (tile_y0 + (float)(GS_TILE_Y - 1))));
-      const float spread = co.x * far_x * far_x + 2.0f * fabsf(co.y) * far_x * far_y + co.z * far_y * far_y;
+      // A Gaussian's operands: one 64-byte record where the caller had them packed (a single line of memory,
+      // every byte of it used), else gathered from the five arrays.  All loads are issued before anything is
+      // computed: one round trip to memory.
+      float2 xy;
+      float4 co;
+      float c0, c1, c2, depth_g = 0.f;
+      float m[GS_N_MAP] = {0.f, 0.f, 0.f, 0.f, 0.f};
+      if (packed != nullptr) {
+        const float4* rec = packed + 4 * (size_t)g;
+        const float4 r0 = rec[0], r1 = rec[1], r2 = rec[2];
+        xy = make_float2(r0.x, r0.y);
+        co = make_float4(r0.z, r0.w, r1.x, r1.y);
+        c0 = r1.z, c1 = r1.w, c2 = r2.x;
+        m[0] = r2.y, m[1] = r2.z, m[2] = r2.w;
+        if (render_geo || MAX_DEPTH) {
+          const float4 r3 = rec[3];
+          m[3] = r3.x, m[4] = r3.y, depth_g = r3.z;
+        }
+      } else {
+        xy = means2D[g];
+        co = conic_opacity[g];
+        c0 = rgb[3 * (size_t)g], c1 = rgb[3 * (size_t)g + 1], c2 = rgb[3 * (size_t)g + 2];
+        if (render_geo) {
+#pragma unroll
+          for (int ch = 0; ch < GS_N_MAP; ch++) m[ch] = all_map[5 * (size_t)g + ch];
+        }
+        if (MAX_DEPTH) depth_g = depths[g];
+      }
+      // (the marking step evaluates the quadratic form with fused operations, the blend the exponent with one
+      // rounding per operation: the mark limit's margin covers both, and the blend tests the exponent itself again)
+      float pfl, mark_limit;
+      s_cull[ts] = block_test_params(co, xy, (float)(blockIdx.x * GS_TILE_X), (float)(blockIdx.y * GS_TILE_Y), pfl,
+                                     mark_limit);
       s_geo0[ts] = make_float4(xy.x, xy.y, co.x, co.y);
-      s_geo1[ts] = make_float4(co.z, __builtin_fmaf(2e-6f, spread, -2.0f * pfl), co.w, pfl);
-      const float c0 = rgb[3 * (size_t)g], c1 = rgb[3 * (size_t)g + 1], c2 = rgb[3 * (size_t)g + 2];
+      s_geo1[ts] = make_float4(co.z, mark_limit, co.w, pfl);
       float mag = fmaxf(fmaxf(fabsf(c0), fabsf(c1)), fabsf(c2));
       finite = c0 == c0 && c1 == c1 && c2 == c2;
-      float m[GS_N_MAP] = {0.f, 0.f, 0.f, 0.f, 0.f};
       if (render_geo) {
 #pragma unroll
         for (int ch = 0; ch < GS_N_MAP; ch++) {
-          const float v = all_map[5 * (size_t)g + ch];
-          m[ch] = v;
-          mag = fmaxf(mag, fabsf(v));
-          finite = finite && v == v;
+          mag = fmaxf(mag, fabsf(m[ch]));
+          finite = finite && m[ch] == m[ch];
         }
       }
       s_col0[ts] = make_float4(c0, c1, c2, m[0]);
       if constexpr (RENDER_GEO) s_col1[ts] = make_float4(m[1], m[2], m[3], m[4]);
       finite = finite && mag < __builtin_inff();
-      if (MAX_DEPTH) s_depth[ts] = depths[g];
+      if (MAX_DEPTH) s_depth[ts] = depth_g;
     }
     {
       const uint64_t bad_m = gs_ballot(!finite);
@@ -212,15 +229,16 @@ render_fwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
         const int jj = k * GS_WAVE + lane_b;
         const bool valid = jj < count;
         const uint64_t valid_m = gs_ballot(valid);
-        const float4 geo0 = s_geo0[valid ? jj : 0], geo1 = s_geo1[valid ? jj : 0];
+        const int js = valid ? jj : 0;
+        const float4 geo0 = s_geo0[js];
         const float2 mu = make_float2(geo0.x, geo0.y);
-        const float4 cq = make_float4(geo0.z, geo0.w, geo1.x, geo1.z);
-        const float4 cp = unpack_cull_params(s_cull[valid ? jj : 0], geo1.w);
+        const float4 cq = make_float4(geo0.z, geo0.w, s_geo1[js].x, 0.f);
+        const float4 cu = s_cull[js];
         // (the four tests first, in one straight line and unconditionally, so that what they have in common is
         // computed once; masks of single comparisons, combined in scalar registers)
         uint64_t hit_m[4];
         bool hits[4];
-        ellipse_hits_quadrant(mu, cq, cp, rt.qx0, rt.qy0, hits);
+        ellipse_hits_quadrant(mu, cq, cu.x, cu.y, cu.z, rt.qx0, rt.qy0, hits);
 #pragma unroll
         for (int r = 0; r < 4; r++) {
           const bool row_alive = ((alive_mask >> (16 * r)) & 0xFFFFull) != 0ull;
@@ -437,7 +455,8 @@ static void launch_render_fwd_variant(const RenderFwdArgs& a, hipStream_t stream
                      a.point_list, a.W, a.H, a.fx, a.fy, a.cx, a.cy, (const float2*)a.means2D, a.rgb, a.all_map,
                      (const float4*)a.conic_opacity, a.compute_locally, a.bg, a.final_T, a.n_contrib_px,
                      a.n_contrib2loss_px, a.out_color, a.out_observe, a.out_all_map, a.out_plane_depth, a.n_render,
-                     a.n_consider, a.n_contrib_tile, a.depths, a.out_max_weight_depth, a.fits_word, a.block_hits);
+                     a.n_consider, a.n_contrib_tile, a.depths, a.out_max_weight_depth, a.fits_word, a.block_hits,
+                     (const float4*)a.packed);
 }
 
 int launch_render_fwd(const RenderFwdArgs& a, hipStream_t stream) {
