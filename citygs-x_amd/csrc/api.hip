@@ -135,7 +135,7 @@ ImageLayout image_layout(int W, int H) {
 }
 
 struct GeometryLayout {
-  size_t tiles_touched, point_offsets, scan_temp, packed, total;
+  size_t tiles_touched, point_offsets, scan_temp, packed_valid, packed, total;
 };
 GeometryLayout geometry_layout(int P) {
   GeometryLayout L;
@@ -145,7 +145,8 @@ GeometryLayout geometry_layout(int P) {
   L.tiles_touched = take(n * 4);
   L.point_offsets = take(n * 4);
   L.scan_temp = take(scan_temp_bytes((int64_t)n));
-  L.packed = take(n * 64);  // the blend kernels' operands, one 64-byte record per Gaussian
+  L.packed_valid = take(4);  // one word: whether the forward call packed the records below
+  L.packed = take(n * 64);   // the blend kernels' operands, one 64-byte record per Gaussian
   L.total = off + 256;
   return L;
 }
@@ -481,6 +482,7 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
   uint32_t* point_offsets = (uint32_t*)(gbase + GL.point_offsets);
   void* scan_temp = gbase + GL.scan_temp;
   float* packed = (float*)(gbase + GL.packed);
+  uint32_t* packed_valid = (uint32_t*)(gbase + GL.packed_valid);
 
   const ImageLayout IL = image_layout(width, height);
   char* ibase = imageBuffer(IL.total, image_user);
@@ -536,15 +538,22 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
     launch_inclusive_sum(P, tiles_touched, point_offsets, scan_temp, stream, total_slot);
   }
   if (check_launch("inclusive_sum", stream, dbg)) return 1;
-  {
-    // The blend kernels (this call's and the backward call's) fetch a Gaussian's operands as one 64-byte record.
-    // Queued behind the counting kernels: where the host has to wait for the instance count before it can size
-    // the binning buffer, the GPU packs meanwhile.
+  // The blend kernels (this call's and the backward call's) can fetch a Gaussian's operands as one 64-byte record
+  // instead of gathering parts of five lines of memory.  Packing the records costs about 20 us per million
+  // Gaussians and saves about 25 us per million instances: done for a view with enough instances per Gaussian.
+  bool use_packed = false, pack_decided = false;
+  auto decide_packing = [&](int64_t instances) -> int {
+    if (pack_decided) return 0;
+    pack_decided = true;
+    use_packed = instances * 5 > (int64_t)P * 4;
     StageScope _t("pack_operands", stream);
-    launch_pack_blend_operands(P, radii, means2D, conic_opacity, rgb, render_geo ? all_map : nullptr, depths, packed,
-                               stream);
-  }
-  if (check_launch("pack_operands", stream, dbg)) return 1;
+    if (use_packed)
+      launch_pack_blend_operands(P, radii, means2D, conic_opacity, rgb, render_geo ? all_map : nullptr, depths, packed,
+                                 packed_valid, stream);
+    else
+      launch_fill_u32(1, 0u, packed_valid, stream);
+    return check_launch("pack_operands", stream, dbg);
+  };
 
   EventTimer timer;
   struct Arrays {
@@ -582,7 +591,7 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
     a.n_render = n_render; a.n_consider = n_consider; a.n_contrib_tile = n_contrib;
     a.fits_word = ahead_of_host ? bucket_fits_word(bucket_table, T) : nullptr;
     a.block_hits = A.block_hits;
-    a.packed = packed;
+    a.packed = use_packed ? packed : nullptr;
     {
       StageScope _t("render_fwd", stream);
       launch_render_fwd(a, stream);
@@ -610,6 +619,7 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
   if (ahead) {
     if (carve(cap_n, A)) return 1;
     if (timer.begin(elapsed_ms != nullptr, stream)) return 1;
+    if (decide_packing(cap_n)) return 1;  // (on the expected count; the margin in it is the caller's)
     if (lists_by_tile(A, cap_longest, 0u, true)) return 1;
     if (blend(A, true)) return 1;
   }
@@ -654,6 +664,7 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
   // The ordinary way (also after kernels launched ahead found that the view does not fit and did nothing).
   if (carve(R, A)) return 1;
   if (!ahead && timer.begin(elapsed_ms != nullptr, stream)) return 1;
+  if (decide_packing(R)) return 1;
 
   // A list of more than sort_limit records is sorted in chunks of at most that many and merged.  That serves a
   // view with a few such lists; the merge looks every record up in every other chunk of its list, and a view
@@ -746,6 +757,7 @@ int gs_render_backward(int P, int R, const float* background, int width, int hei
   a.block_hits = (const uint16_t*)(bbase + BL.block_hits);
   a.point_offsets = (const uint32_t*)(gbase + GL.point_offsets);
   a.packed = (const float*)(gbase + GL.packed);  // (of the arrays the forward call was given)
+  a.packed_valid = (const uint32_t*)(gbase + GL.packed_valid);
   a.instance_grads = (float*)align_ptr((const char*)instance_grads, 256);
   a.P = P; a.W = width; a.H = height;
   a.fy = height / (2.0f * tan_fovy);  // cuda_rasterizer/rasterizer_impl.cu:885-886

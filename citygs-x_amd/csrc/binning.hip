@@ -191,47 +191,62 @@ gather_u32_kernel(int64_t n, const uint32_t* __restrict__ index, const uint32_t*
   if (i < n) out[i] = table[index[i]];
 }
 
-// One thread per Gaussian.  A wave's 64 records (4 KB, contiguous) pass through LDS so that every store
+// One thread per Gaussian; only visible Gaussians (radius > 0) are read and written: no tile lists the others.  A
+// wave whose 64 Gaussians are all visible passes its records (4 KB, contiguous) through LDS so that every store
 // instruction writes one contiguous kilobyte: lane l stores 16-byte word (l & 3) of record 16 k + (l >> 2) in
 // round k.  (In LDS a record's four words sit 1040 bytes apart, so that neither the writes, record-major, nor the
-// reads, word-minor, pile up on a few banks.)  A wave none of whose Gaussians is visible stores nothing; in a wave
-// with some, the invisible ones' records are written too (zeros for the colour of a culled Gaussian do no harm:
-// no tile lists it).
+// reads, word-minor, pile up on a few banks.)  In any other wave a visible lane stores its own record, four
+// 16-byte stores that fill one 64-byte line.
 __global__ void __launch_bounds__(GS_BLOCK_1D)
 pack_blend_operands_kernel(int P, const int* __restrict__ radii, const float2* __restrict__ means2D,
                            const float4* __restrict__ conic_opacity, const float* __restrict__ rgb,
                            const float* __restrict__ all_map, const float* __restrict__ depths,
-                           float4* __restrict__ packed) {
+                           float4* __restrict__ packed, uint32_t* __restrict__ valid_word) {
+  if (valid_word != nullptr && blockIdx.x == 0 && threadIdx.x == 0) *valid_word = 1u;
   constexpr int WORD_STRIDE = GS_WAVE + 1;  // in 16-byte units
   __shared__ float4 s_rec[GS_BLOCK_1D / GS_WAVE][4 * WORD_STRIDE];
   const int lane = threadIdx.x & (GS_WAVE - 1), wave = threadIdx.x / GS_WAVE;
   const int i = blockIdx.x * GS_BLOCK_1D + threadIdx.x;
   const bool live = i < P && radii[i] > 0;
-  if (gs_ballot(live) == 0ull) return;
-  const int ic = i < P ? i : P - 1;
-  const float2 xy = means2D[ic];
-  const float4 co = conic_opacity[ic];
-  const float c0 = rgb[3 * (size_t)ic], c1 = rgb[3 * (size_t)ic + 1], c2 = rgb[3 * (size_t)ic + 2];
-  float m[5] = {0.f, 0.f, 0.f, 0.f, 0.f};
-  if (all_map != nullptr) {
+  const uint64_t live_m = gs_ballot(live);
+  if (live_m == 0ull) return;
+  float4 w0 = make_float4(0.f, 0.f, 0.f, 0.f), w1 = w0, w2 = w0, w3 = w0;
+  if (live) {
+    const float2 xy = means2D[i];
+    const float4 co = conic_opacity[i];
+    const float c0 = rgb[3 * (size_t)i], c1 = rgb[3 * (size_t)i + 1], c2 = rgb[3 * (size_t)i + 2];
+    float m[5] = {0.f, 0.f, 0.f, 0.f, 0.f};
+    if (all_map != nullptr) {
 #pragma unroll
-    for (int ch = 0; ch < 5; ch++) m[ch] = all_map[5 * (size_t)ic + ch];
+      for (int ch = 0; ch < 5; ch++) m[ch] = all_map[5 * (size_t)i + ch];
+    }
+    const float d = depths != nullptr ? depths[i] : 0.f;
+    w0 = make_float4(xy.x, xy.y, co.x, co.y);
+    w1 = make_float4(co.z, co.w, c0, c1);
+    w2 = make_float4(c2, m[0], m[1], m[2]);
+    w3 = make_float4(m[3], m[4], d, 0.f);
   }
-  const float d = depths != nullptr ? depths[ic] : 0.f;
+  // (a wave with a few invisible Gaussians still takes the contiguous route: their records are zeros)
+  if (__popcll(live_m) < 48) {
+    if (live) {
+      float4* rec = packed + 4 * (size_t)i;
+      rec[0] = w0; rec[1] = w1; rec[2] = w2; rec[3] = w3;
+    }
+    return;
+  }
   float4* mine = &s_rec[wave][0];
-  mine[0 * WORD_STRIDE + lane] = make_float4(xy.x, xy.y, co.x, co.y);
-  mine[1 * WORD_STRIDE + lane] = make_float4(co.z, co.w, c0, c1);
-  mine[2 * WORD_STRIDE + lane] = make_float4(c2, m[0], m[1], m[2]);
-  mine[3 * WORD_STRIDE + lane] = make_float4(m[3], m[4], d, 0.f);
+  mine[0 * WORD_STRIDE + lane] = w0;
+  mine[1 * WORD_STRIDE + lane] = w1;
+  mine[2 * WORD_STRIDE + lane] = w2;
+  mine[3 * WORD_STRIDE + lane] = w3;
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
   __builtin_amdgcn_wave_barrier();
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-  const int first = blockIdx.x * GS_BLOCK_1D + wave * GS_WAVE;  // the wave's first Gaussian
-  float4* out = packed + 4 * (size_t)first;
+  float4* out = packed + 4 * (size_t)(blockIdx.x * GS_BLOCK_1D + wave * GS_WAVE);  // the wave's first record
 #pragma unroll
   for (int k = 0; k < 4; k++) {
-    const int rec = 16 * k + (lane >> 2), word = lane & 3;
-    if (first + rec < P) out[64 * k + lane] = mine[word * WORD_STRIDE + rec];
+    const int rec = 16 * k + (lane >> 2);
+    if (blockIdx.x * GS_BLOCK_1D + wave * GS_WAVE + rec < P) out[64 * k + lane] = mine[(lane & 3) * WORD_STRIDE + rec];
   }
 }
 
@@ -389,11 +404,17 @@ int launch_duplicate_with_keys(int P, int W, int H, const float* means2D, const 
 
 int launch_pack_blend_operands(int P, const int* radii, const float* means2D, const float* conic_opacity,
                                const float* rgb, const float* all_map, const float* depths, float* packed,
-                               hipStream_t stream) {
+                               uint32_t* valid_word, hipStream_t stream) {
   if (P <= 0) return 0;
   hipLaunchKernelGGL(pack_blend_operands_kernel, dim3((P + GS_BLOCK_1D - 1) / GS_BLOCK_1D), dim3(GS_BLOCK_1D), 0,
                      stream, P, radii, (const float2*)means2D, (const float4*)conic_opacity, rgb, all_map, depths,
-                     (float4*)packed);
+                     (float4*)packed, valid_word);
+  return 0;
+}
+
+int launch_fill_u32(int64_t n, uint32_t value, uint32_t* p, hipStream_t stream) {
+  if (n <= 0) return 0;
+  hipLaunchKernelGGL(fill_u32_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, n, value, p);
   return 0;
 }
 

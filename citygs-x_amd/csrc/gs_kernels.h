@@ -121,9 +121,11 @@ int launch_tile_sort(int T, uint32_t longest, uint32_t limit, uint32_t chunks, c
 // What the blend kernels read of a Gaussian, in one 64-byte record per Gaussian: (x, y, A, B), (C, opacity, r, g),
 // (b, map0, map1, map2), (map3, map4, depth, 0); all_map and depths may be null (zeros).  Records of Gaussians with
 // radius 0 are left as they are (no tile lists them).
+// valid_word (optional): set to 1 by the kernel.
 int launch_pack_blend_operands(int P, const int* radii, const float* means2D, const float* conic_opacity,
                                const float* rgb, const float* all_map, const float* depths, float* packed,
-                               hipStream_t stream);
+                               uint32_t* valid_word, hipStream_t stream);
+int launch_fill_u32(int64_t n, uint32_t value, uint32_t* p, hipStream_t stream);
 int launch_gather_u32(int64_t n, const uint32_t* index, const uint32_t* table, uint32_t* out, hipStream_t stream);
 int launch_ssim_l1_fwd(int C, int H, int W, const float* img1, const float* img2, const uint8_t* mask,
                        float* l1_map, float* ssim_map, float* d_mu, float* d_xx, float* d_xy, hipStream_t stream);
@@ -246,6 +248,8 @@ struct RenderBwdArgs {
   float* instance_grads;  // (R,16) scratch, fully written by the blend kernel
   const uint16_t* block_hits = nullptr;  // optional (R): left by the forward blend (RenderFwdArgs::block_hits)
   const float* packed = nullptr;         // optional (P,4) 16-byte words: see RenderFwdArgs::packed
+  // optional device word beside `packed`: non-zero if the forward call did pack the records (it decides per view)
+  const uint32_t* packed_valid = nullptr;
   // outputs, fully written by the per-Gaussian reduction
   float* dL_dmean2D;         // (P,2)
   float* dL_dmean2D_abs;     // (P,3)

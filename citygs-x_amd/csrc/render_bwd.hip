@@ -70,7 +70,11 @@ render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
                   const uint8_t* __restrict__ compute_locally, const float* __restrict__ dL_dpix,
                   const float* __restrict__ dL_dout_all_map, const float* __restrict__ dL_dout_plane_depth,
                   const uint32_t* __restrict__ emission_sorted, float4* __restrict__ instance_grads,
-                  const uint16_t* __restrict__ block_hits, const float4* __restrict__ packed) {
+                  const uint16_t* __restrict__ block_hits, const float4* __restrict__ packed_records,
+                  const uint32_t* __restrict__ packed_valid) {
+  // (whether the forward call packed the records is its decision per view: a word beside them says)
+  const float4* packed = (packed_records != nullptr && (packed_valid == nullptr || *packed_valid != 0u))
+                             ? packed_records : nullptr;
   constexpr bool render_geo = RENDER_GEO;
   __shared__ uint32_t s_emis[BATCH];
   __shared__ float4 s_xyf[BATCH];  // centre x, y; the power floor; unused
@@ -190,51 +194,51 @@ render_bwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
       const uint32_t k_sorted = range.x + (uint32_t)(first_pos - tid);
       const uint32_t g = point_list[k_sorted];
       // A Gaussian's operands: one 64-byte record where the forward call packed them (a single line of memory,
-      // every byte of it used), else gathered from the four arrays; all loads issued before anything is computed.
-      float2 xy;
-      float4 co;
-      float c0, c1, c2;
-      float m[GS_N_MAP] = {0.f, 0.f, 0.f, 0.f, 0.f};
+      // every byte of it used), else gathered from the four arrays.  (Each route loads and then stages by itself:
+      // with the loaded values merged across the two routes the compiler splits the gathers into single words.)
+      auto stage = [&](const float2 xy, const float4 co, const float c0, const float c1, const float c2,
+                       const float (&m)[GS_N_MAP]) {
+        s_emis[tid] = emission_sorted[k_sorted];
+        s_co[tid] = co;
+        float pfl, mark_limit;
+        const float4 cp = block_test_params(co, xy, (float)(blockIdx.x * GS_TILE_X), (float)(blockIdx.y * GS_TILE_Y),
+                                            pfl, mark_limit);
+        if (HITS) s_hits[tid] = block_hits[k_sorted];
+        else s_cp[tid] = cp;
+        s_xyf[tid] = make_float4(xy.x, xy.y, pfl, 0.f);
+        float mag = fmaxf(fmaxf(fabsf(c0), fabsf(c1)), fabsf(c2));
+        bool fin = c0 == c0 && c1 == c1 && c2 == c2;
+        if (render_geo) {
+#pragma unroll
+          for (int ch = 0; ch < GS_N_MAP; ch++) {
+            mag = fmaxf(mag, fabsf(m[ch]));
+            fin = fin && m[ch] == m[ch];
+          }
+          s_chan[tid][RENDER_GEO ? 1 : 0] = make_float4(m[1], m[2], m[3], m[4]);
+        }
+        s_chan[tid][0] = make_float4(c0, c1, c2, m[0]);
+        return fin && mag < __builtin_inff();
+      };
       if (packed != nullptr) {
         const float4* rec = packed + 4 * (size_t)g;
         const float4 r0 = rec[0], r1 = rec[1], r2 = rec[2];
-        xy = make_float2(r0.x, r0.y);
-        co = make_float4(r0.z, r0.w, r1.x, r1.y);
-        c0 = r1.z, c1 = r1.w, c2 = r2.x;
-        m[0] = r2.y, m[1] = r2.z, m[2] = r2.w;
+        float m[GS_N_MAP] = {r2.y, r2.z, r2.w, 0.f, 0.f};
         if (render_geo) {
           const float4 r3 = rec[3];
           m[3] = r3.x, m[4] = r3.y;
         }
+        finite = stage(make_float2(r0.x, r0.y), make_float4(r0.z, r0.w, r1.x, r1.y), r1.z, r1.w, r2.x, m);
       } else {
-        xy = means2D[g];
-        co = conic_opacity[g];
-        c0 = rgb[3 * (size_t)g], c1 = rgb[3 * (size_t)g + 1], c2 = rgb[3 * (size_t)g + 2];
+        const float2 xy = means2D[g];
+        const float4 co = conic_opacity[g];
+        const float c0 = rgb[3 * (size_t)g], c1 = rgb[3 * (size_t)g + 1], c2 = rgb[3 * (size_t)g + 2];
+        float m[GS_N_MAP] = {0.f, 0.f, 0.f, 0.f, 0.f};
         if (render_geo) {
 #pragma unroll
           for (int ch = 0; ch < GS_N_MAP; ch++) m[ch] = all_map[5 * (size_t)g + ch];
         }
+        finite = stage(xy, co, c0, c1, c2, m);
       }
-      s_emis[tid] = emission_sorted[k_sorted];
-      s_co[tid] = co;
-      float pfl, mark_limit;
-      const float4 cp = block_test_params(co, xy, (float)(blockIdx.x * GS_TILE_X), (float)(blockIdx.y * GS_TILE_Y),
-                                          pfl, mark_limit);
-      if (HITS) s_hits[tid] = block_hits[k_sorted];
-      else s_cp[tid] = cp;
-      s_xyf[tid] = make_float4(xy.x, xy.y, pfl, 0.f);
-      float mag = fmaxf(fmaxf(fabsf(c0), fabsf(c1)), fabsf(c2));
-      finite = c0 == c0 && c1 == c1 && c2 == c2;
-      if (render_geo) {
-#pragma unroll
-        for (int ch = 0; ch < GS_N_MAP; ch++) {
-          mag = fmaxf(mag, fabsf(m[ch]));
-          finite = finite && m[ch] == m[ch];
-        }
-        s_chan[tid][RENDER_GEO ? 1 : 0] = make_float4(m[1], m[2], m[3], m[4]);
-      }
-      s_chan[tid][0] = make_float4(c0, c1, c2, m[0]);
-      finite = finite && mag < __builtin_inff();
     }
     {
       const uint64_t bad_m = gs_ballot(!finite);
@@ -572,7 +576,7 @@ int launch_render_bwd(const RenderBwdArgs& a, hipStream_t stream) {
                        a.fx, a.fy, a.bg, (const float2*)a.means2D, (const float4*)a.conic_opacity, a.rgb, a.all_map,
                        a.all_map_pixels, a.final_T, a.n_contrib_px, a.compute_locally, a.dL_dpix, a.dL_dout_all_map,
                        a.dL_dout_plane_depth, a.emission_sorted, (float4*)a.instance_grads, a.block_hits,
-                       (const float4*)a.packed);
+                       (const float4*)a.packed, a.packed_valid);
   };
   if (a.render_geo) {
     if (a.block_hits) go(render_bwd_kernel<true, true>);

@@ -59,7 +59,7 @@ __device__ __forceinline__ int not_hoisted(int x) {
 // that blends with the largest weight alpha * T (the front-most one among equals; 0 where nothing blends).  It
 // leaves every other output as it is.
 template <bool RENDER_GEO, bool MAX_DEPTH>
-__global__ void __launch_bounds__(GS_TILE_PIX) __attribute__((amdgpu_waves_per_eu(6)))
+__global__ void __launch_bounds__(GS_TILE_PIX) __attribute__((amdgpu_waves_per_eu(MAX_DEPTH ? 5 : 6)))
 render_fwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__ point_list, int W, int H, float fx,
                   float fy, float cx, float cy, const float2* __restrict__ means2D, const float* __restrict__ rgb,
                   const float* __restrict__ all_map, const float4* __restrict__ conic_opacity,
@@ -155,53 +155,53 @@ render_fwd_kernel(const uint2* __restrict__ ranges, const uint32_t* __restrict__
     if (ts < count) {
       const uint32_t g = point_list[range.x + (uint32_t)i * BATCH + ts];
       // A Gaussian's operands: one 64-byte record where the caller had them packed (a single line of memory,
-      // every byte of it used), else gathered from the five arrays.  All loads are issued before anything is
-      // computed: one round trip to memory.
-      float2 xy;
-      float4 co;
-      float c0, c1, c2, depth_g = 0.f;
-      float m[GS_N_MAP] = {0.f, 0.f, 0.f, 0.f, 0.f};
+      // every byte of it used), else gathered from the five arrays.  (Each route loads and then stages by itself:
+      // with the loaded values merged across the two routes the compiler splits the gathers into single words.)
+      auto stage = [&](const float2 xy, const float4 co, const float c0, const float c1, const float c2,
+                       const float (&m)[GS_N_MAP], const float depth_g) {
+        // (the marking step evaluates the quadratic form with fused operations, the blend the exponent with one
+        // rounding per operation: the mark limit's margin covers both, and the blend tests the exponent itself
+        // again)
+        float pfl, mark_limit;
+        s_cull[ts] = block_test_params(co, xy, (float)(blockIdx.x * GS_TILE_X), (float)(blockIdx.y * GS_TILE_Y), pfl,
+                                       mark_limit);
+        s_geo0[ts] = make_float4(xy.x, xy.y, co.x, co.y);
+        s_geo1[ts] = make_float4(co.z, mark_limit, co.w, pfl);
+        float mag = fmaxf(fmaxf(fabsf(c0), fabsf(c1)), fabsf(c2));
+        bool fin = c0 == c0 && c1 == c1 && c2 == c2;
+        if (render_geo) {
+#pragma unroll
+          for (int ch = 0; ch < GS_N_MAP; ch++) {
+            mag = fmaxf(mag, fabsf(m[ch]));
+            fin = fin && m[ch] == m[ch];
+          }
+        }
+        s_col0[ts] = make_float4(c0, c1, c2, m[0]);
+        if constexpr (RENDER_GEO) s_col1[ts] = make_float4(m[1], m[2], m[3], m[4]);
+        if (MAX_DEPTH) s_depth[ts] = depth_g;
+        return fin && mag < __builtin_inff();
+      };
       if (packed != nullptr) {
         const float4* rec = packed + 4 * (size_t)g;
         const float4 r0 = rec[0], r1 = rec[1], r2 = rec[2];
-        xy = make_float2(r0.x, r0.y);
-        co = make_float4(r0.z, r0.w, r1.x, r1.y);
-        c0 = r1.z, c1 = r1.w, c2 = r2.x;
-        m[0] = r2.y, m[1] = r2.z, m[2] = r2.w;
+        float m[GS_N_MAP] = {r2.y, r2.z, r2.w, 0.f, 0.f};
+        float depth_g = 0.f;
         if (render_geo || MAX_DEPTH) {
           const float4 r3 = rec[3];
           m[3] = r3.x, m[4] = r3.y, depth_g = r3.z;
         }
+        finite = stage(make_float2(r0.x, r0.y), make_float4(r0.z, r0.w, r1.x, r1.y), r1.z, r1.w, r2.x, m, depth_g);
       } else {
-        xy = means2D[g];
-        co = conic_opacity[g];
-        c0 = rgb[3 * (size_t)g], c1 = rgb[3 * (size_t)g + 1], c2 = rgb[3 * (size_t)g + 2];
+        const float2 xy = means2D[g];
+        const float4 co = conic_opacity[g];
+        const float c0 = rgb[3 * (size_t)g], c1 = rgb[3 * (size_t)g + 1], c2 = rgb[3 * (size_t)g + 2];
+        float m[GS_N_MAP] = {0.f, 0.f, 0.f, 0.f, 0.f};
         if (render_geo) {
 #pragma unroll
           for (int ch = 0; ch < GS_N_MAP; ch++) m[ch] = all_map[5 * (size_t)g + ch];
         }
-        if (MAX_DEPTH) depth_g = depths[g];
+        finite = stage(xy, co, c0, c1, c2, m, MAX_DEPTH ? depths[g] : 0.f);
       }
-      // (the marking step evaluates the quadratic form with fused operations, the blend the exponent with one
-      // rounding per operation: the mark limit's margin covers both, and the blend tests the exponent itself again)
-      float pfl, mark_limit;
-      s_cull[ts] = block_test_params(co, xy, (float)(blockIdx.x * GS_TILE_X), (float)(blockIdx.y * GS_TILE_Y), pfl,
-                                     mark_limit);
-      s_geo0[ts] = make_float4(xy.x, xy.y, co.x, co.y);
-      s_geo1[ts] = make_float4(co.z, mark_limit, co.w, pfl);
-      float mag = fmaxf(fmaxf(fabsf(c0), fabsf(c1)), fabsf(c2));
-      finite = c0 == c0 && c1 == c1 && c2 == c2;
-      if (render_geo) {
-#pragma unroll
-        for (int ch = 0; ch < GS_N_MAP; ch++) {
-          mag = fmaxf(mag, fabsf(m[ch]));
-          finite = finite && m[ch] == m[ch];
-        }
-      }
-      s_col0[ts] = make_float4(c0, c1, c2, m[0]);
-      if constexpr (RENDER_GEO) s_col1[ts] = make_float4(m[1], m[2], m[3], m[4]);
-      finite = finite && mag < __builtin_inff();
-      if (MAX_DEPTH) s_depth[ts] = depth_g;
     }
     {
       const uint64_t bad_m = gs_ballot(!finite);
