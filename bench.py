@@ -31,6 +31,9 @@ BYTES_PER_GAUSSIAN = {
     # coefficients)
     "preprocess_fwd": 307 + 36,
     "tile_count": 16,
+    # radius 4 + centre 8 + conic and opacity 16 + colour 12 + geometry channels 20 + depth 4 in, one 64 B record out
+    # (visible Gaussians only: the figure is an upper bound)
+    "pack_operands": 64 + 64,
     "inclusive_sum": 8,
     "preprocess_bwd": 560 - 192 + 36,
     "all_map_fwd": 60,   # means 12 + scales 12 + rotations 16 in, 20 out
@@ -123,7 +126,7 @@ def cpu_baseline(g, cam, am, ug, runs):
             "sample": f"{runs} full views of the same workload (median); C++/OpenMP oracle incl. python glue"}
 
 
-FORWARD_STAGES = ("preprocess_fwd", "tile_count", "inclusive_sum", "bucket_scatter", "tile_sort",
+FORWARD_STAGES = ("preprocess_fwd", "tile_count", "inclusive_sum", "pack_operands", "bucket_scatter", "tile_sort",
                   "duplicate_with_keys", "identify_tile_ranges", "render_fwd")
 
 
