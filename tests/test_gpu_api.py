@@ -422,6 +422,56 @@ def test_debug_mode_gives_the_same_results_by_every_route():
         assert torch.equal(a, b)
 
 
+def test_packed_and_gathered_operands_give_the_same_results():
+    """The forward call packs the blend kernels' operands into one record per Gaussian when the view has more than
+    0.8 instances per Gaussian, and lets both blend kernels gather them from the caller's arrays otherwise.  The
+    same Gaussians with and without a crowd of Gaussians behind the camera (which adds no instance and tips the
+    decision) must render and differentiate to the same bits."""
+    import gs_scenes
+    from diff_gaussian_rasterization import GaussianRasterizer
+    g, cams = gs_scenes.make_scene(1, P=40_000, n_views=1)
+    cam = cams[0]
+    W, H = cam.image_width, cam.image_height
+    gx, gy = (W + 15) // 16, (H + 15) // 16
+    cl = torch.ones(gy, gx, dtype=torch.bool, device=DEV)
+    ug = {k: v.to(DEV) for k, v in gs_scenes.upstream_grads(cam).items()}
+    P = g["means3D"].shape[0]
+
+    def run(extra):
+        h = {k: g[k] for k in ("means3D", "scales", "rotations", "opacities", "shs")}
+        if extra:
+            # behind the camera: culled by the preprocess, radius 0, no instance
+            eye = cam.camera_center.reshape(1, 3).cpu()
+            look = torch.zeros(1, 3) - eye
+            behind = eye - 5.0 * look / look.norm() + 0.1 * torch.randn(extra, 3, generator=torch.Generator().manual_seed(1))
+            h = {"means3D": torch.cat([h["means3D"], behind]),
+                 "scales": torch.cat([h["scales"], h["scales"][:1].expand(extra, -1)]),
+                 "rotations": torch.cat([h["rotations"], h["rotations"][:1].expand(extra, -1)]),
+                 "opacities": torch.cat([h["opacities"], h["opacities"][:1].expand(extra, -1)]),
+                 "shs": torch.cat([h["shs"], h["shs"][:1].expand(extra, -1, -1)])}
+        rast = GaussianRasterizer(_settings(cam))
+        leaf = {k: v.to(DEV).requires_grad_(True) for k, v in h.items()}
+        args = _cuda_args()
+        means2D, rgb, co, radii, depths = rast.preprocess_gaussians(
+            leaf["means3D"], leaf["scales"], leaf["rotations"], leaf["shs"], leaf["opacities"], args)
+        assert int((radii[P:] > 0).sum()) == 0
+        am = gs_scenes.build_all_map(leaf["means3D"], leaf["scales"], leaf["rotations"], cam)
+        m2abs = torch.zeros_like(leaf["means3D"], requires_grad=True) + 0
+        color, n_render, n_consider, n_contrib, obs, oam, opd = rast.render_gaussians(
+            means2D, m2abs, co, rgb, am, depths, radii, cl, cl, args)
+        torch.autograd.backward([color, oam, opd], [ug["color"], ug["all_map"], ug["plane_depth"]])
+        R = int(n_render.sum())
+        return R, [color, n_render, n_consider, n_contrib, obs[:P], oam, opd] + [leaf[k].grad[:P] for k in sorted(leaf)]
+
+    R, packed = run(0)
+    assert R * 5 > P * 4, "the plain scene is meant to take the packed route"
+    extra = 2 * R  # more than R / 0.8 - P
+    R2, gathered = run(extra)
+    assert R2 == R and R2 * 5 <= (P + extra) * 4
+    for a, b in zip(packed, gathered):
+        assert torch.equal(a, b)
+
+
 def test_side_stream_gives_the_same_results():
     """Everything runs on the caller's current stream: the same step on a side stream (default priority), with
     other work in flight on the default stream, gives the same results, bit for bit."""
