@@ -26,7 +26,9 @@ __device__ __forceinline__ float4 cull_params(float4 co, float& power_floor) {
     if (tau == tau) {
       power_floor = fmaxf(-tau, -87.0f);
       const float det = co.x * co.z - co.y * co.y;
-      const float ia = 1.0f / co.x, ic = 1.0f / co.z;
+      // (the hardware reciprocal: 1/A and 1/C only place the point of a block edge where q is evaluated, and q
+      // there exceeds the edge's minimum by the square of the placement error)
+      const float ia = __builtin_amdgcn_rcpf(co.x), ic = __builtin_amdgcn_rcpf(co.z);
       if (det > 0.0f && co.x > 0.0f && co.z > 0.0f && ia < inf && ic < inf) cp = make_float4(ia, ic, 2.0f * tau, 0.f);
     }
   }
