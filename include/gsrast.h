@@ -157,7 +157,9 @@ typedef struct gs_render_result {
  * where nothing blends; asking for it changes no other output.
  * elapsed_ms (host, optional): if non-NULL the call times key emission + sort
  * + blend with events and blocks until done (the forward_render_time the
- * reference stores at CR/rasterizer_impl.cu:754-755). */
+ * reference stores at CR/rasterizer_impl.cu:754-755).
+ * The geometry buffer is asked for 72 bytes per Gaussian plus the prefix sum's workspace (the reference's holds the
+ * preprocess outputs as well, CR/rasterizer_impl.cu:160-188; here those are the caller's tensors). */
 int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resize_fn binningBuffer,
                       void* binning_user, gs_resize_fn imageBuffer, void* image_user, int P,
                       const float* background, int width, int height, float focal_x, float focal_y, float cx,
@@ -173,7 +175,10 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
  * CR/rasterizer_impl.cu:850-932) plus the repacking of
  * RenderGaussiansBackwardCUDA (DGR/rasterize_points.cu:428-440).  The three
  * buffers are the ones gs_render_forward filled (the geometry buffer is read
- * too: it holds the per-Gaussian instance offsets).  Gradient outputs are
+ * too: it holds the per-Gaussian instance offsets and, for a view with more than 0.8 instances per Gaussian, one
+ * 64-byte record per visible Gaussian with the values of means2D, conic_opacity, rgb and all_maps that the forward
+ * call was given, which the kernel then reads instead of those arrays: pass the forward call's arrays, as the
+ * reference does).  Gradient outputs are
  * fully written and need no initialisation: dL_dmean2D (P,2), dL_dmean2D_abs
  * (P,3), dL_dconic_opacity (P,4) packed [x, y, w, opacity], dL_dcolor (P,3),
  * dL_dall_map (P,5).  Where the reference adds every pixel's contribution
