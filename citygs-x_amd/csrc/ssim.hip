@@ -94,8 +94,14 @@ ssim_l1_fwd_kernel(int H, int W, const float* __restrict__ img1, const float* __
   __shared__ float s_a[STY][SPITCH];
   __shared__ float s_b[STY][SPITCH];
   __shared__ float s_h[5][STY][SBX];
-  const size_t plane = (size_t)blockIdx.z * H * W;
-  const int x0 = blockIdx.x * SBX, y0 = blockIdx.y * SBY;
+  // Workgroups go to the eight XCDs in turn; dealt out this way an XCD holds a contiguous run of blocks, so the
+  // halo that neighbouring blocks share is fetched into one second-level cache once, not into up to eight.
+  const uint32_t blocks_xy = gridDim.x * gridDim.y;
+  const uint32_t b = xcd_contiguous_index(blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z),
+                                          blocks_xy * gridDim.z);
+  const uint32_t bz = b / blocks_xy, by = (b % blocks_xy) / gridDim.x, bx = b % gridDim.x;
+  const size_t plane = (size_t)bz * H * W;
+  const int x0 = bx * SBX, y0 = by * SBY;
   {
     float va[STAGE_ROUNDS], vb[STAGE_ROUNDS];
 #pragma unroll
@@ -159,8 +165,14 @@ ssim_l1_bwd_kernel(int H, int W, const float* __restrict__ img1, const float* __
                    const float* __restrict__ d_xx, const float* __restrict__ d_xy, float* __restrict__ dimg1) {
   __shared__ float s_d[3][STY][SPITCH];
   __shared__ float s_h[3][STY][SBX];
-  const size_t plane = (size_t)blockIdx.z * H * W;
-  const int x0 = blockIdx.x * SBX, y0 = blockIdx.y * SBY;
+  // Workgroups go to the eight XCDs in turn; dealt out this way an XCD holds a contiguous run of blocks, so the
+  // halo that neighbouring blocks share is fetched into one second-level cache once, not into up to eight.
+  const uint32_t blocks_xy = gridDim.x * gridDim.y;
+  const uint32_t b = xcd_contiguous_index(blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z),
+                                          blocks_xy * gridDim.z);
+  const uint32_t bz = b / blocks_xy, by = (b % blocks_xy) / gridDim.x, bx = b % gridDim.x;
+  const size_t plane = (size_t)bz * H * W;
+  const int x0 = bx * SBX, y0 = by * SBY;
   {
     float vg[STAGE_ROUNDS], v0[STAGE_ROUNDS], v1[STAGE_ROUNDS], v2[STAGE_ROUNDS];
 #pragma unroll
