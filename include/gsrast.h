@@ -428,7 +428,7 @@ int gs_selftest_reductions(const float* in, float* out_wave, float* out_rows, gs
  * (CR/timers.cu:11-79; stage names at CR/rasterizer_impl.cu:385-752): while
  * enabled, each stage of the composite entry points (preprocess_fwd,
  * tile_count, bucket_scatter, tile_sort, or on the radix route inclusive_sum,
- * duplicate_with_keys, sort_pairs, identify_tile_ranges; render_fwd,
+ * duplicate_with_keys, sort_pairs, identify_tile_ranges; pack_operands; render_fwd,
  * render_bwd, preprocess_bwd; knn_dist2 and its phases knn_minmax, knn_keys,
  * knn_sort, knn_gather, knn_boxes, knn_box_mean_dist)
  * is bracketed by an event pair on its stream.  Nothing is synchronised until
