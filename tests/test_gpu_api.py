@@ -422,11 +422,13 @@ def test_debug_mode_gives_the_same_results_by_every_route():
         assert torch.equal(a, b)
 
 
-def test_packed_and_gathered_operands_give_the_same_results():
+@pytest.mark.parametrize("poison", [False, True])
+def test_packed_and_gathered_operands_give_the_same_results(poison):
     """The forward call packs the blend kernels' operands into one record per Gaussian when the view has more than
     0.8 instances per Gaussian, and lets both blend kernels gather them from the caller's arrays otherwise.  The
     same Gaussians with and without a crowd of Gaussians behind the camera (which adds no instance and tips the
-    decision) must render and differentiate to the same bits."""
+    decision) must render and differentiate to the same bits; so must a view in which some Gaussians carry NaN or
+    infinite colours and geometry channels (NaNs in the same places, the same bits everywhere else)."""
     import gs_scenes
     from diff_gaussian_rasterization import GaussianRasterizer
     g, cams = gs_scenes.make_scene(1, P=40_000, n_views=1)
@@ -456,6 +458,17 @@ def test_packed_and_gathered_operands_give_the_same_results():
             leaf["means3D"], leaf["scales"], leaf["rotations"], leaf["shs"], leaf["opacities"], args)
         assert int((radii[P:] > 0).sum()) == 0
         am = gs_scenes.build_all_map(leaf["means3D"], leaf["scales"], leaf["rotations"], cam)
+        if poison:
+            vis = torch.nonzero(radii[:P] > 0)[:, 0]
+            pick = vis[torch.randperm(vis.numel(), generator=torch.Generator().manual_seed(3))[:40].to(vis.device)]
+            rgb = rgb.detach().clone()
+            am = am.detach().clone()
+            rgb[pick[:10], 0] = float("nan")
+            rgb[pick[10:20], 2] = float("inf")
+            am[pick[20:30], 1] = float("nan")
+            am[pick[30:40], 4] = float("-inf")
+            rgb.requires_grad_(True)
+            am.requires_grad_(True)
         m2abs = torch.zeros_like(leaf["means3D"], requires_grad=True) + 0
         color, n_render, n_consider, n_contrib, obs, oam, opd = rast.render_gaussians(
             means2D, m2abs, co, rgb, am, depths, radii, cl, cl, args)
@@ -469,7 +482,13 @@ def test_packed_and_gathered_operands_give_the_same_results():
     R2, gathered = run(extra)
     assert R2 == R and R2 * 5 <= (P + extra) * 4
     for a, b in zip(packed, gathered):
-        assert torch.equal(a, b)
+        if a.is_floating_point():
+            assert torch.equal(torch.isnan(a), torch.isnan(b))
+            assert torch.equal(torch.nan_to_num(a, nan=0.0), torch.nan_to_num(b, nan=0.0))
+        else:
+            assert torch.equal(a, b)
+    if poison:
+        assert bool(torch.isnan(packed[0]).any()) and float(torch.isnan(packed[0]).float().mean()) < 0.2
 
 
 def test_side_stream_gives_the_same_results():
