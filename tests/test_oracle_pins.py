@@ -406,6 +406,67 @@ def test_render_forward_backward_match_autograd(orc, seed, geo):
     assert (bo["dL_dmeans2D_abs"][:, :2] >= np.abs(bo["dL_dmeans2D"][:, :2]) * (1 - 1e-5) - 1e-7).all()
 
 
+@pytest.mark.parametrize("seed,geo", [(3, True), (4, False)])
+def test_render_backward_abs_gradient_is_a_sum_of_per_pixel_magnitudes(orc, seed, geo):
+    """dL_dmeans2D_abs (backward.cu:553-554) adds up, pixel by pixel, the magnitude of that pixel's own
+    contribution to the mean2D gradient.  Pinned by differentiating every pixel's loss term on its own
+    (float64 autograd through torch_ref.render) and summing the magnitudes; upstream gradients of mixed sign
+    make the pixels' contributions cancel, so taking the magnitude of the finished sum instead gives a
+    different number, which the last lines check."""
+    W = H = 16
+    P = 30
+    cam = _cam(W, H)
+    gen = torch.Generator().manual_seed(seed)
+    means2D = torch.rand(P, 2, generator=gen, dtype=torch.float64) * 18.0 - 1.0
+    s = torch.rand(P, generator=gen, dtype=torch.float64) * 3 + 1.5
+    ang = torch.rand(P, generator=gen, dtype=torch.float64) * math.pi
+    ecc = torch.rand(P, generator=gen, dtype=torch.float64) * 0.6 + 0.4
+    ca, sa = torch.cos(ang), torch.sin(ang)
+    ia, ib = 1 / s ** 2, 1 / (s * ecc) ** 2
+    conic = torch.stack([ca * ca * ia + sa * sa * ib, ca * sa * (ia - ib), sa * sa * ia + ca * ca * ib], -1)
+    co = torch.cat([conic, torch.rand(P, 1, generator=gen, dtype=torch.float64) * 0.6 + 0.05], 1)
+    rgb = torch.rand(P, 3, generator=gen, dtype=torch.float64)
+    amap = torch.randn(P, 5, generator=gen, dtype=torch.float64)
+    amap[:, :2] *= 0.2
+    amap[:, 2] = 1.0
+    amap[:, :3] = torch.nn.functional.normalize(amap[:, :3], dim=-1)
+    amap[:, 3] = 1.0
+    amap[:, 4] = amap[:, 4].abs() + 1.0
+    depths = torch.rand(P, generator=gen) * 10 + 1
+    radii = torch.ceil(3 * s).int()
+    bg = torch.tensor([0.3, 0.1, 0.7], dtype=torch.float64)
+    cl = np.ones(1, bool)
+    f32 = lambda t: t.detach().float().numpy()
+    b = orc.bin_and_sort(radii.numpy(), f32(means2D), depths.numpy(), cl, W, H)
+    fo = orc.render_fwd(b["ranges"], b["point_list"], f32(means2D), f32(rgb), f32(amap), f32(co), cl, f32(bg), W, H,
+                        cam.tanfovx, cam.tanfovy, geo)
+    gpix = torch.randn(3, H, W, generator=gen, dtype=torch.float64)
+    gmap = torch.randn(5, H, W, generator=gen, dtype=torch.float64)
+    gdep = torch.randn(1, H, W, generator=gen, dtype=torch.float64)
+    m = means2D.clone().requires_grad_(True)
+    ft = tr.render(m, co, rgb, amap, b["ranges"], b["point_list"], bg, W, H, cam.tanfovx, cam.tanfovy, geo)
+    assert np.array_equal(fo["n_contrib"], ft["n_contrib"].numpy().astype(np.uint32))
+    per_pixel = (ft["color"] * gpix).sum(0)
+    if geo:
+        per_pixel = per_pixel + (ft["out_all_map"] * gmap).sum(0) + (ft["out_plane_depth"] * gdep).sum(0)
+    scale = torch.tensor([0.5 * W, 0.5 * H], dtype=torch.float64)
+    sum_of_abs = torch.zeros(P, 2, dtype=torch.float64)
+    plain_sum = torch.zeros(P, 2, dtype=torch.float64)
+    for y in range(H):
+        for x in range(W):
+            (gp,) = torch.autograd.grad(per_pixel[y, x], m, retain_graph=True)
+            sum_of_abs += (gp * scale).abs()
+            plain_sum += gp * scale
+    bo = orc.render_bwd(b["ranges"], b["point_list"], f32(means2D), f32(co), f32(rgb), f32(amap), fo["out_all_map"],
+                        fo["final_T"], fo["n_contrib"], cl, f32(bg), f32(gpix), f32(gmap), f32(gdep), W, H, cam.tanfovx,
+                        cam.tanfovy, geo)
+    assert _rel(bo["dL_dmeans2D"][:, :2], plain_sum.numpy()) <= 1e-4
+    assert _rel(bo["dL_dmeans2D_abs"][:, :2], sum_of_abs.numpy()) <= 1e-4
+    assert (bo["dL_dmeans2D_abs"][:, 2] == 0).all()
+    # the case tells the two readings apart: the magnitude of the finished sum is far from the sum of magnitudes
+    assert _rel(np.abs(bo["dL_dmeans2D"][:, :2]), sum_of_abs.numpy()) > 0.2
+
+
 def test_render_masked_tiles_are_untouched(orc):
     g, cams = gs_scenes.make_scene(0, P=3000)
     cam = cams[0]
