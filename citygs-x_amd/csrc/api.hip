@@ -152,7 +152,8 @@ GeometryLayout geometry_layout(int P) {
 }
 
 struct BinningLayout {
-  size_t point_list, keys, point_list_unsorted, keys_unsorted, emission, emission_other, sort_temp, block_hits, total;
+  size_t point_list, keys, point_list_unsorted, keys_unsorted, emission, emission_other, sort_temp, block_hits,
+      radix_scratch, total;
 };
 // n = the number of instances the arrays are laid out for
 BinningLayout binning_layout(int64_t R) {
@@ -162,12 +163,16 @@ BinningLayout binning_layout(int64_t R) {
   auto take = [&](size_t b) { size_t o = off; off += align_up(b, 256); return o; };
   L.point_list = take(n * 4);
   L.keys = take(n * 8);
-  L.point_list_unsorted = take(n * 4);
+  // The next three lie back to back: on the per-tile route they are one array of 16-byte records (16 n bytes from
+  // keys_unsorted on), on the radix route the unsorted keys, the Gaussian of every emission index and the sort's
+  // second payload array.
   L.keys_unsorted = take(n * 8);
-  L.emission = take(n * 4);
+  L.point_list_unsorted = take(n * 4);
   L.emission_other = take(n * 4);
+  L.emission = take(n * 4);
   L.sort_temp = take(sort_temp_bytes((int64_t)n));
   L.block_hits = take(n * 2);  // what the forward blend leaves for the backward blend, per sorted instance
+  L.radix_scratch = take(n * 8);  // second array of the per-tile radix sort for lists it sorts in blocks
   L.total = off + 256;
   return L;
 }
@@ -374,8 +379,8 @@ uint32_t* acquire_total_slot() {
   uint32_t* base = pinned_words();
   if (base == nullptr) return nullptr;
   uint32_t* slot = base + 16 * (g_total_next.fetch_add(1, std::memory_order_relaxed) % TOTAL_SLOTS);
-  slot[1] = 0u;  // second and third word of the slot: the longest tile list and the number of chunks that the
-  slot[2] = 0u;  // longer lists are sorted in, both written before the total
+  slot[1] = 0u;  // second and third word of the slot: the longest tile list and the numbers of lists for the
+  slot[2] = 0u;  // per-tile radix sort's two kernels, both written before the total
   __atomic_store_n(slot, TOTAL_PENDING, __ATOMIC_RELEASE);
   return slot;
 }
@@ -431,16 +436,16 @@ int pending_fault(const char* who) {
 }
 
 struct TileSortLimits {
-  int large, chunks;
+  int small, block;
 };
-// The defaults, or what the caller's options ask for: the list length up to which one workgroup sorts a list
-// whole (0: every view takes the radix sort), and the number of chunks up to which the longer lists of a view are
-// sorted in chunks and merged.
+// The defaults, or what the caller's options ask for: the list length up to which a list is sorted in registers
+// (0: the view takes the radix sort over all its keys), and the number of records the per-tile radix sort holds
+// in one block (longer lists are sorted block by block through memory).
 TileSortLimits tile_sort_limits(const gs_render_options* o) {
-  TileSortLimits L = {TILE_SORT_LARGE, TILE_SORT_MAX_CHUNKS};
+  TileSortLimits L = {TILE_SORT_SMALL, tile_radix_block_records()};
   if (o == nullptr || o->struct_bytes < 3 * sizeof(uint32_t)) return L;
-  if (o->tile_sort_large_limit >= 0) L.large = o->tile_sort_large_limit < TILE_SORT_LARGE ? o->tile_sort_large_limit : TILE_SORT_LARGE;
-  if (o->tile_sort_max_chunks >= 0) L.chunks = o->tile_sort_max_chunks;
+  if (o->tile_sort_small_limit >= 0) L.small = o->tile_sort_small_limit < TILE_SORT_SMALL ? o->tile_sort_small_limit : TILE_SORT_SMALL;
+  if (o->tile_sort_block_records > 0 && o->tile_sort_block_records < L.block) L.block = o->tile_sort_block_records;
   return L;
 }
 }  // namespace
@@ -494,13 +499,12 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
   uint32_t* ranges = (uint32_t*)(ibase + IL.ranges);
 
   // Two ways to the sorted per-tile lists.  The default buckets the instances by tile (counting sort) and sorts
-  // every tile's list on its own; it needs the tile histogram to fit in LDS and every list to fit the per-tile
-  // sort.  Otherwise: emit (tile | depth) keys, radix-sort all of them, find the tile boundaries.
+  // every tile's list on its own; it needs the tile histogram to fit in LDS.  Otherwise: emit (tile | depth) keys,
+  // radix-sort all of them, find the tile boundaries.
   uint32_t* total_slot = acquire_total_slot();
   void* bucket_table = ibase + IL.bucket_table;
-  const uint32_t sort_limit = (uint32_t)limits.large;
-  const bool counted_by_tile = T <= bucket_max_tiles() && total_slot != nullptr && sort_limit > 0;
-  bool bucketed = counted_by_tile;
+  const uint32_t sort_limit = (uint32_t)limits.small;
+  const bool bucketed = T <= bucket_max_tiles() && total_slot != nullptr && sort_limit > 0;
 
   // The instance count decides the size of the binning buffer, and the host learns it only after the counting
   // kernels have run: a round trip during which the GPU would idle.  A caller that says how many instances and
@@ -510,12 +514,12 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
   // returns or builds the lists again the ordinary way.
   int64_t cap_n = 0;
   uint32_t cap_longest = 0;
-  if (counted_by_tile && !dbg && result != nullptr && result->struct_bytes >= sizeof(gs_render_result) &&
+  if (bucketed && !dbg && result != nullptr && result->struct_bytes >= sizeof(gs_render_result) &&
       options != nullptr && options->struct_bytes >= sizeof(gs_render_options) && options->expected_instances > 0) {
     cap_n = options->expected_instances < (int64_t)GS_MAX_INSTANCES ? options->expected_instances
                                                                      : (int64_t)GS_MAX_INSTANCES;
-    cap_longest = options->expected_longest_list > 0 ? (uint32_t)options->expected_longest_list : sort_limit;
-    if (cap_longest > sort_limit) cap_longest = sort_limit;
+    // (0: any length; the sort kernels launched and their LDS depend on it)
+    cap_longest = options->expected_longest_list > 0 ? (uint32_t)options->expected_longest_list : GS_MAX_INSTANCES;
   }
   const bool ahead = cap_n > 0;
 
@@ -523,7 +527,8 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
     StageScope _t("tile_count", stream);
     // the histogram's grand total is the instance count: the host gets it from here
     if (launch_bucket_count(P, width, height, radii, means2D, compute_locally, tiles_touched, bucket_table, ranges,
-                            sort_limit, total_slot, out_observe, (uint32_t)cap_n, cap_longest, stream))
+                            sort_limit, (uint32_t)limits.block, total_slot, out_observe, (uint32_t)cap_n, cap_longest,
+                            stream))
       return 1;
   } else {
     StageScope _t("tile_count", stream);
@@ -558,7 +563,7 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
   EventTimer timer;
   struct Arrays {
     uint32_t *point_list, *gauss_of_emission, *emission, *emission_other;
-    uint64_t *keys, *keys_other;
+    uint64_t *keys, *keys_other, *radix_scratch;
     void* sort_temp;
     uint16_t* block_hits;
   };
@@ -575,6 +580,7 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
     A.emission_other = (uint32_t*)(bbase + BL.emission_other);
     A.sort_temp = bbase + BL.sort_temp;
     A.block_hits = (uint16_t*)(bbase + BL.block_hits);
+    A.radix_scratch = (uint64_t*)(bbase + BL.radix_scratch);
     return 0;
   };
   auto blend = [&](const Arrays& A, bool ahead_of_host) -> int {
@@ -598,19 +604,22 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
     }
     return check_launch("render_forward", stream, dbg);
   };
-  auto lists_by_tile = [&](const Arrays& A, uint32_t longest_for_launch, uint32_t chunks_for_launch,
+  auto lists_by_tile = [&](const Arrays& A, uint32_t longest_for_launch, uint32_t radix_tiles,
                            bool ahead_of_host) -> int {
     {
       StageScope _t("bucket_scatter", stream);
-      // (also finishes the prefix sum over the Gaussians: point_offsets)
+      // (also finishes the prefix sum over the Gaussians: point_offsets; the 16-byte records take the place of
+      // the three unsorted arrays of the other route)
       launch_bucket_scatter(P, width, height, means2D, depths, tiles_touched, point_offsets, radii, compute_locally,
-                            bucket_table, ranges, A.keys_other, A.gauss_of_emission, ahead_of_host, stream);
+                            bucket_table, ranges, A.keys_other, ahead_of_host, stream);
     }
     if (check_launch("bucket_scatter", stream, dbg)) return 1;
     {
       StageScope _t("tile_sort", stream);
-      launch_tile_sort(T, longest_for_launch, sort_limit, chunks_for_launch, ranges, bucket_table, A.keys_other,
-                       A.gauss_of_emission, A.keys, A.emission, A.point_list, ahead_of_host, stream);
+      if (launch_tile_sort(T, longest_for_launch, radix_tiles, sort_limit, (uint32_t)limits.block, ranges,
+                           bucket_table, A.keys_other, A.radix_scratch, A.keys, A.emission, A.point_list,
+                           ahead_of_host, stream))
+        return 1;
     }
     return check_launch("tile_sort", stream, dbg);
   };
@@ -620,19 +629,19 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
     if (carve(cap_n, A)) return 1;
     if (timer.begin(elapsed_ms != nullptr, stream)) return 1;
     if (decide_packing(cap_n)) return 1;  // (on the expected count; the margin in it is the caller's)
-    if (lists_by_tile(A, cap_longest, 0u, true)) return 1;
+    if (lists_by_tile(A, cap_longest, 0xFFFFFFFFu, true)) return 1;
     if (blend(A, true)) return 1;
   }
 
   // The host needs the instance count: it sizes the binning buffer (unless that was done ahead), and the caller
   // gets it back.  The counting kernels write it straight into pinned host memory and the host polls that word:
-  // no copy, and no sleeping wait.  On the bucketed route the longest tile list and the number of chunks that
-  // longer lists are cut into arrive in the words beside it.
-  uint32_t R_u = 0, longest = 0, chunks = 0;
+  // no copy, and no sleeping wait.  On the bucketed route the longest tile list and the numbers of lists that go
+  // to the per-tile radix sort's two kernels arrive in the words beside it.
+  uint32_t R_u = 0, longest = 0, radix_tiles = 0;
   if (total_slot != nullptr) {
     if (wait_for_total(total_slot, stream, &R_u)) return 1;
     longest = __atomic_load_n(total_slot + 1, __ATOMIC_ACQUIRE);
-    chunks = __atomic_load_n(total_slot + 2, __ATOMIC_ACQUIRE);
+    radix_tiles = __atomic_load_n(total_slot + 2, __ATOMIC_ACQUIRE);
   } else {
     uint32_t wrapped = 0;
     GS_HIP_TRY(hipMemcpyAsync(&R_u, point_offsets + (P - 1), sizeof(uint32_t), hipMemcpyDeviceToHost, stream));
@@ -666,17 +675,9 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
   if (!ahead && timer.begin(elapsed_ms != nullptr, stream)) return 1;
   if (decide_packing(R)) return 1;
 
-  // A list of more than sort_limit records is sorted in chunks of at most that many and merged.  That serves a
-  // view with a few such lists; the merge looks every record up in every other chunk of its list, and a view
-  // with many long lists is sorted as fast by the radix sort over all its keys, which then takes over.
-  if (bucketed && longest > sort_limit && chunks > (uint32_t)limits.chunks) bucketed = false;
   if (bucketed) {
-    if (lists_by_tile(A, longest, chunks, false)) return 1;
+    if (lists_by_tile(A, longest, radix_tiles, false)) return 1;
   } else {
-    if (counted_by_tile) {
-      StageScope _t("inclusive_sum", stream);
-      launch_bucket_offsets(P, width, height, tiles_touched, bucket_table, point_offsets, stream);
-    }
     const int end_bit = sort_end_bit(width, height);
     // The sort carries each instance's index in emission order as its payload (the backward pass files
     // per-instance gradients under it); the Gaussian ids of the sorted list are gathered afterwards.
@@ -711,7 +712,7 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
       // ... and gathers the Gaussian ids of the sorted instances on the way (point_list).  The ranges were
       // cleared by the counting kernel of this path, or hold the other path's table and are cleared here.
       // It also looks at the sort's error word and raises the sticky fault word if the sort gave up.
-      launch_tile_ranges(R, A.keys, T, ranges, stream, !counted_by_tile, A.emission, A.gauss_of_emission,
+      launch_tile_ranges(R, A.keys, T, ranges, stream, true, A.emission, A.gauss_of_emission,
                          A.point_list, R > 0 ? sort_error_word(A.sort_temp) : nullptr, fault_word());
     }
     if (check_launch("identify_tile_ranges", stream, dbg)) return 1;

@@ -90,34 +90,41 @@ int launch_duplicate_with_keys(int P, int W, int H, const float* means2D, const 
                                const uint32_t* offsets, const int* radii, const uint8_t* compute_locally,
                                uint64_t* keys, uint32_t* values, uint32_t* emission /*optional*/,
                                hipStream_t stream);
-// ---- binning by tile: counting sort by tile + per-tile register sort (tile_bucket.hip) ----
-constexpr int TILE_SORT_LARGE = 8192;  // longest list one workgroup sorts; longer ones are sorted in chunks and merged
-constexpr int TILE_SORT_MAX_CHUNKS = 32;  // chunks of long lists per view the merge takes; beyond: the radix sort
+// ---- binning by tile: counting sort by tile + per-tile sorts (tile_bucket.hip, tile_radix.hip) ----
+constexpr int TILE_SORT_SMALL = 2048;  // longest list the register sort takes; longer ones go to the radix sort
 int bucket_max_tiles();
 size_t bucket_table_bytes(int T);
-// tiles_touched per Gaussian, the workgroup-by-tile table, ranges (2 words per tile), and in three host-visible
-// words the number of instances (word 0, written last), the longest list (word 1) and the number of chunks that
-// the lists of more than chunk_limit records are cut into (word 2)
+// tiles_touched per Gaussian, the workgroup-by-tile table, ranges (2 words per tile), the lists of tiles with more
+// than small_limit records (0 = TILE_SORT_SMALL) for the radix sort's kernels, and in three host-visible words the
+// number of instances (word 0, written last), the longest list (word 1) and the numbers of tiles in those lists
+// (word 2: larger kernel's << 16 | smaller kernel's).  block_limit (0 = the maximum): the records the radix sort
+// holds in one block, see launch_tile_sort.
 // cap_instances / cap_longest: what kernels launched ahead of the host's decision were sized for; the ranges kernel
 // leaves 1 in bucket_fits_word(table) if the view has at most that many instances and no longer list, else 0
 int launch_bucket_count(int P, int W, int H, const int* radii, const float* means2D, const uint8_t* compute_locally,
-                        uint32_t* tiles_touched, void* table, uint32_t* ranges, uint32_t chunk_limit,
-                        uint32_t* host_words, int* zero_per_gaussian, uint32_t cap_instances, uint32_t cap_longest,
-                        hipStream_t stream);
+                        uint32_t* tiles_touched, void* table, uint32_t* ranges, uint32_t small_limit,
+                        uint32_t block_limit, uint32_t* host_words, int* zero_per_gaussian, uint32_t cap_instances,
+                        uint32_t cap_longest, hipStream_t stream);
 const uint32_t* bucket_fits_word(const void* table, int T);
-int launch_bucket_offsets(int P, int W, int H, const uint32_t* tiles_touched, void* table, uint32_t* point_offsets,
-                          hipStream_t stream);
-// records: (depth bits << 32 | emission index) per instance, grouped by tile in any order; gauss_of_emission: the
-// Gaussian of every emission index.  Also writes point_offsets (the inclusive prefix sum of tiles_touched).
+// records: one 16-byte record (Gaussian, emission index, depth bits, 0) per instance, grouped by tile in any
+// order.  Also writes point_offsets (the inclusive prefix sum of tiles_touched).
 // ahead_of_host: the kernel checks bucket_fits_word itself and does nothing if the view does not fit what it was
 // launched for.
 int launch_bucket_scatter(int P, int W, int H, const float* means2D, const float* depths,
                           const uint32_t* tiles_touched, uint32_t* point_offsets, const int* radii,
-                          const uint8_t* compute_locally, void* table, const uint32_t* ranges, uint64_t* records,
-                          uint32_t* gauss_of_emission, bool ahead_of_host, hipStream_t stream);
-int launch_tile_sort(int T, uint32_t longest, uint32_t limit, uint32_t chunks, const uint32_t* ranges,
-                     const void* table, uint64_t* records, const uint32_t* gauss_of_emission, uint64_t* keys,
-                     uint32_t* emission, uint32_t* point_list, bool ahead_of_host, hipStream_t stream);
+                          const uint8_t* compute_locally, void* table, const uint32_t* ranges, void* records,
+                          bool ahead_of_host, hipStream_t stream);
+// scratch: 8 bytes per instance, used for lists of more than block_limit records
+int launch_tile_sort(int T, uint32_t longest, uint32_t radix_tiles, uint32_t small_limit, uint32_t block_limit,
+                     const uint32_t* ranges, const void* table, const void* records, uint64_t* scratch,
+                     uint64_t* keys, uint32_t* emission, uint32_t* point_list, bool ahead_of_host,
+                     hipStream_t stream);
+int tile_radix_mid_records();    // records one workgroup of the radix sort's smaller kernel holds (4096)
+int tile_radix_block_records();  // ... and of its larger kernel (16384): longer lists are sorted in blocks
+int launch_tile_radix_sort(int T, bool mid, bool lng, const uint32_t* ranges, const uint32_t* tile_lists,
+                           const uint32_t* counts, uint32_t block_limit, const void* records, uint64_t* ping,
+                           uint64_t* pong, uint64_t* keys, uint32_t* emission, uint32_t* point_list,
+                           const uint32_t* fits_word, hipStream_t stream);
 // What the blend kernels read of a Gaussian, in one 64-byte record per Gaussian: (x, y, A, B), (C, opacity, r, g),
 // (b, map0, map1, map2), (map3, map4, depth, 0); all_map and depths may be null (zeros).  Records of Gaussians with
 // radius 0 are left as they are (no tile lists them).

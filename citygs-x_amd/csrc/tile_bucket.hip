@@ -7,13 +7,14 @@
 //   2. one workgroup per tile sorting its segment in registers by (depth bits, emission index): the emission index
 //      is unique, so the order does not depend on how the scatter happened to fill the segment, and it is the
 //      order a stable sort on the depth bits would leave.
-// No pass over all instances per digit, no look-back chain.  A list longer than one workgroup sorts is cut into
-// chunks that are sorted the same way and then merged; a view with many such lists is left to the radix sort
-// (the caller decides from the longest list and the number of chunks, which this code reports).
+// No pass over all instances per digit, no look-back chain.  Lists of up to 2048 records are sorted in registers
+// by a bitonic network (below); longer ones by a radix sort on the depth bits that stays inside the CU
+// (tile_radix.hip).  The ranges kernel sorts the tiles into those classes.
 #include <atomic>
 
 #include "gs_common.h"
 #include "gs_kernels.h"
+#include "tile_lists.h"
 
 namespace gs {
 namespace {
@@ -93,7 +94,7 @@ bucket_count_kernel(int P, int per_block, uint32_t gx, uint32_t gy, const int* _
   __syncthreads();
   uint32_t* row = table + (size_t)chunk * T;
   for (uint32_t t = threadIdx.x; t < T; t += BK_THREADS) row[t] = s_hist[t];
-  // the workgroup's share of the prefix sum over the Gaussians (bucket_offsets_kernel finishes it)
+  // the workgroup's share of the prefix sum over the Gaussians (the scatter kernel finishes it)
   if (threadIdx.x == 0) {
     uint32_t all = 0;
     for (int w = 0; w < BK_THREADS / GS_WAVE; w++) all += s_sum[w];
@@ -149,17 +150,18 @@ __device__ __forceinline__ uint32_t wave_inclusive_scan_u32(uint32_t v, int lane
 }
 
 // 1c. One workgroup: exclusive prefix of the tile totals = the tile ranges (rasterizer_impl.cu:122-144 leaves
-// (0, 0) for a tile without instances).  A list of more than `limit` records is sorted in chunks that are merged
-// afterwards: chunk_first[t] = number of chunks of the tiles before t (chunk_first[T] = all chunks; a tile within
-// the limit has none).  The longest list, the number of chunks and then the number of instances are stored where
-// the host can read them (host_words[1], [2] and [0]; the host polls word 0, so it is written last).
+// (0, 0) for a tile without instances).  Tiles whose lists are too long for the register sort are entered in two
+// lists for the radix sort's kernels: lists of more than small_limit and at most mid_limit records ascending from
+// tile_lists[0], longer ones descending from tile_lists[T - 1]; tile_lists[T] = (number of the longer ones << 16
+// | number of the others) (T is at most 30000).  The longest list, that word and then the number of instances are
+// stored where the host can read them (host_words[1], [2] and [0]; the host polls word 0, so it is written last).
 __global__ void __launch_bounds__(1024)
-bucket_ranges_kernel(uint32_t T, uint32_t limit, const uint32_t* __restrict__ totals, uint32_t* __restrict__ ranges,
-                     uint32_t* __restrict__ chunk_first, uint32_t* __restrict__ block_sums, int nblocks,
-                     uint32_t* __restrict__ host_words, uint32_t cap_instances, uint32_t cap_longest,
-                     uint32_t* __restrict__ fits_word) {
+bucket_ranges_kernel(uint32_t T, uint32_t small_limit, uint32_t mid_limit, const uint32_t* __restrict__ totals,
+                     uint32_t* __restrict__ ranges, uint32_t* __restrict__ tile_lists,
+                     uint32_t* __restrict__ block_sums, int nblocks, uint32_t* __restrict__ host_words,
+                     uint32_t cap_instances, uint32_t cap_longest, uint32_t* __restrict__ fits_word) {
   constexpr int ITEMS = 4;  // consecutive tiles per thread: the usual grids (up to 4096 tiles) take one round
-  __shared__ uint32_t s_wave[16], s_wave_chunks[16], s_max[16];
+  __shared__ uint32_t s_wave[16], s_wave_class[16], s_max[16];
   __shared__ double s_exact[16];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   {
@@ -176,54 +178,55 @@ bucket_ranges_kernel(uint32_t T, uint32_t limit, const uint32_t* __restrict__ to
     if ((int)threadIdx.x < nblocks) block_sums[threadIdx.x] = base + inc - b;
     __syncthreads();
   }
-  uint32_t carry = 0, carry_chunks = 0, longest = 0;
+  uint32_t carry = 0, carry_class = 0, longest = 0;
   double exact = 0.0;  // the number of instances without the 32-bit wrap-around of the prefix sums
   for (uint32_t start = 0; start < T; start += 1024 * ITEMS) {
     const uint32_t t0 = start + threadIdx.x * ITEMS;
-    uint32_t v[ITEMS], c[ITEMS], sum = 0, sum_chunks = 0;
+    uint32_t v[ITEMS], c[ITEMS], sum = 0, sum_class = 0;
 #pragma unroll
     for (int q = 0; q < ITEMS; q++) v[q] = t0 + q < T ? totals[t0 + q] : 0u;
 #pragma unroll
     for (int q = 0; q < ITEMS; q++) {
-      c[q] = v[q] > limit ? (v[q] + limit - 1u) / limit : 0u;
+      c[q] = v[q] > mid_limit ? 0x10000u : (v[q] > small_limit ? 1u : 0u);
       longest = v[q] > longest ? v[q] : longest;
       exact += (double)v[q];
       sum += v[q];
-      sum_chunks += c[q];
+      sum_class += c[q];
     }
     const uint32_t inc = wave_inclusive_scan_u32(sum, lane);
     // (a wave without a long list, the usual case, has nothing to scan)
-    const uint32_t inc_chunks = __ballot(sum_chunks != 0u) != 0ull ? wave_inclusive_scan_u32(sum_chunks, lane) : 0u;
+    const uint32_t inc_class = __ballot(sum_class != 0u) != 0ull ? wave_inclusive_scan_u32(sum_class, lane) : 0u;
     if (lane == 63) {
       s_wave[wave] = inc;
-      s_wave_chunks[wave] = inc_chunks;
+      s_wave_class[wave] = inc_class;
     }
     __syncthreads();
-    uint32_t base = 0, all = 0, base_chunks = 0, all_chunks = 0;
+    uint32_t base = 0, all = 0, base_class = 0, all_class = 0;
 #pragma unroll
     for (int w = 0; w < 16; w++) {
-      const uint32_t s = s_wave[w], sc = s_wave_chunks[w];
+      const uint32_t s = s_wave[w], sc = s_wave_class[w];
       if (w < wave) {
         base += s;
-        base_chunks += sc;
+        base_class += sc;
       }
       all += s;
-      all_chunks += sc;
+      all_class += sc;
     }
     __syncthreads();
-    uint32_t begin = carry + base + inc - sum, begin_chunks = carry_chunks + base_chunks + inc_chunks - sum_chunks;
+    uint32_t begin = carry + base + inc - sum, begin_class = carry_class + base_class + inc_class - sum_class;
 #pragma unroll
     for (int q = 0; q < ITEMS; q++) {
       if (t0 + q < T) {
         ranges[2 * (t0 + q)] = v[q] ? begin : 0u;
         ranges[2 * (t0 + q) + 1] = v[q] ? begin + v[q] : 0u;
-        chunk_first[t0 + q] = begin_chunks;
+        if (c[q] == 1u) tile_lists[begin_class & 0xFFFFu] = t0 + q;
+        if (c[q] == 0x10000u) tile_lists[T - 1u - (begin_class >> 16)] = t0 + q;
       }
       begin += v[q];
-      begin_chunks += c[q];
+      begin_class += c[q];
     }
     carry += all;
-    carry_chunks += all_chunks;
+    carry_class += all_class;
   }
 #pragma unroll
   for (int d = 32; d >= 1; d >>= 1) {
@@ -244,62 +247,23 @@ bucket_ranges_kernel(uint32_t T, uint32_t limit, const uint32_t* __restrict__ to
       m = s_max[w] > m ? s_max[w] : m;
       all += s_exact[w];
     }
-    chunk_first[T] = carry_chunks;
+    tile_lists[T] = carry_class;
     // more instances than 32-bit positions can address: the host must not go on with the wrapped count
     const uint32_t reported = all > (double)GS_MAX_INSTANCES ? GS_TOO_MANY_INSTANCES : carry;
     // Kernels launched ahead of the host's decision (buffers sized from the caller's expectation) look at this
     // word and do nothing unless the view fits what they were launched for.
     *fits_word = (reported <= cap_instances && m <= cap_longest) ? 1u : 0u;
     __hip_atomic_store(host_words + 1, m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-    __hip_atomic_store(host_words + 2, carry_chunks, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    __hip_atomic_store(host_words + 2, carry_class, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
     __hip_atomic_store(host_words, reported, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
   }
 }
 
-// 1c'. Inclusive prefix of tiles_touched over the Gaussians (rasterizer_impl.cu:648), from the counting
-// workgroups' own sums: every workgroup scans its chunk, starting from the prefix bucket_ranges_kernel left.
-__global__ void __launch_bounds__(BK_THREADS)
-bucket_offsets_kernel(int P, int per_block, const uint32_t* __restrict__ tiles_touched,
-                      const uint32_t* __restrict__ block_prefix, uint32_t* __restrict__ point_offsets) {
-  constexpr int ITEMS = 4;
-  __shared__ uint32_t s_wave[BK_THREADS / GS_WAVE];
-  const int lane = threadIdx.x & (GS_WAVE - 1), wave = threadIdx.x / GS_WAVE;
-  const int first = blockIdx.x * per_block;
-  const int last = first + per_block < P ? first + per_block : P;
-  uint32_t carry = block_prefix[blockIdx.x];
-  for (int base = first; base < last; base += BK_THREADS * ITEMS) {
-    const int i0 = base + (int)threadIdx.x * ITEMS;
-    uint32_t v[ITEMS], sum = 0;
-#pragma unroll
-    for (int q = 0; q < ITEMS; q++) {
-      v[q] = i0 + q < last ? tiles_touched[i0 + q] : 0u;
-      sum += v[q];
-    }
-    const uint32_t inc = wave_inclusive_scan_u32(sum, lane);
-    if (lane == GS_WAVE - 1) s_wave[wave] = inc;
-    __syncthreads();
-    uint32_t before = 0, all = 0;
-#pragma unroll
-    for (int w = 0; w < BK_THREADS / GS_WAVE; w++) {
-      const uint32_t s = s_wave[w];
-      if (w < wave) before += s;
-      all += s;
-    }
-    __syncthreads();
-    uint32_t run = carry + before + inc - sum;
-#pragma unroll
-    for (int q = 0; q < ITEMS; q++) {
-      run += v[q];
-      if (i0 + q < last) point_offsets[i0 + q] = run;
-    }
-    carry += all;
-  }
-}
-
 // 1d. Every instance goes to its tile's segment: segment start (ranges) + instances of earlier workgroups
-// (table) + a place among this workgroup's own, handed out by an LDS counter.  The record is
-// (depth bits << 32 | emission index); the Gaussian of an emission index goes to a side table
-// (rasterizer_impl.cu:74-117 writes the same pairs in emission order).  The kernel also finishes the prefix sum
+// (table) + a place among this workgroup's own, handed out by an LDS counter.  The record is one 16-byte store
+// (Gaussian, emission index, depth bits, 0) (rasterizer_impl.cu:74-117 writes the same instances in emission
+// order); the per-tile sorts read the depth bits and look the other two up once a record's place is known, inside
+// the tile's own segment.  The kernel also finishes the prefix sum
 // over the Gaussians' tile counts (rasterizer_impl.cu:648) for its own chunk, which is where the emission
 // indices come from: a thread owns four consecutive Gaussians, the workgroup scans the threads' sums, and the
 // inclusive sums go to point_offsets on the way (the backward pass reads them).
@@ -311,8 +275,8 @@ bucket_scatter_kernel(int P, int per_block, uint32_t gx, uint32_t gy, const floa
                       const uint32_t* __restrict__ block_prefix, uint32_t* __restrict__ point_offsets,
                       const int* __restrict__ radii, const uint8_t* __restrict__ compute_locally,
                       const uint32_t* __restrict__ table, const uint32_t* __restrict__ ranges,
-                      uint64_t* __restrict__ records, uint32_t* __restrict__ gauss_of_emission,
-                      const uint32_t* __restrict__ fits_word, int vector_loads) {
+                      TileRecord* __restrict__ records, const uint32_t* __restrict__ fits_word,
+                      int vector_loads) {
   extern __shared__ uint32_t s_next[];
   __shared__ uint32_t s_wave[BK_THREADS / GS_WAVE];
   if (fits_word != nullptr && *fits_word == 0u) return;
@@ -387,8 +351,7 @@ bucket_scatter_kernel(int P, int per_block, uint32_t gx, uint32_t gy, const floa
           [&](const Owner& o, uint32_t tile, uint32_t rank) {
             const uint32_t e = o.first + rank;
             const uint32_t pos = atomicAdd(&s_next[tile], 1u);
-            records[pos] = ((uint64_t)o.depth_bits << 32) | (uint64_t)e;
-            gauss_of_emission[e] = o.id;
+            records[pos] = make_uint4(o.id, e, o.depth_bits, 0u);
           });
     }
     if (whole) {
@@ -544,10 +507,11 @@ __device__ __forceinline__ void register_sort(uint64_t (&v)[E], uint32_t wave, u
   }
 }
 
+// Sorts (depth bits << 32 | place in the segment) and hands every entry to emit_list_entry, which puts runs of
+// equal depth bits into emission order.  s_x: at least 64 E W words.
 template <int E, int W>
 __device__ __forceinline__ void register_sort_tile(uint32_t t, uint32_t start, uint32_t n,
-                                                   const uint64_t* __restrict__ records,
-                                                   const uint32_t* __restrict__ gauss_of_emission,
+                                                   const TileRecord* __restrict__ records,
                                                    uint64_t* __restrict__ keys, uint32_t* __restrict__ emission,
                                                    uint32_t* __restrict__ point_list, uint64_t* s_x) {
   const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -555,37 +519,50 @@ __device__ __forceinline__ void register_sort_tile(uint32_t t, uint32_t start, u
 #pragma unroll
   for (int r = 0; r < E; r++) {
     const uint32_t i = ((wave * E + r) << 6) | lane;
-    v[r] = i < n ? records[start + i] : ~0ull;
+    v[r] = i < n ? ((uint64_t)records[start + i].z << 32) | (uint64_t)i : ~0ull;
   }
   register_sort<E, W>(v, wave, lane, s_x);
-  const uint64_t tile_bits = (uint64_t)t << 32;
+  uint32_t gaussian[E];
 #pragma unroll
   for (int r = 0; r < E; r++) {
     const uint32_t i = ((wave * E + r) << 6) | lane;
+    gaussian[r] = 0u;
     if (i < n) {
-      const uint32_t e = (uint32_t)v[r];
-      keys[start + i] = tile_bits | (v[r] >> 32);
-      emission[start + i] = e;
-      point_list[start + i] = gauss_of_emission[e];
+      const uint2 ge = *reinterpret_cast<const uint2*>(records + start + (uint32_t)v[r]);
+      gaussian[r] = ge.x;
+      v[r] = (v[r] & 0xFFFFFFFF00000000ull) | (uint64_t)ge.y;
     }
+  }
+  __syncthreads();  // (the sort's last exchange between waves has been read by everybody)
+#pragma unroll
+  for (int r = 0; r < E; r++) {
+    const uint32_t i = ((wave * E + r) << 6) | lane;
+    if (i < n) s_x[i] = v[r];
+  }
+  __syncthreads();
+  const uint64_t* sorted = s_x;
+#pragma unroll
+  for (int r = 0; r < E; r++) {
+    const uint32_t i = ((wave * E + r) << 6) | lane;
+    if (i < n)
+      emit_list_entry(t, start, n, i, gaussian[r], [&](uint32_t q) { return sorted[q]; }, keys, emission, point_list);
   }
 }
 
 // Dynamic LDS: 8 bytes per record of the longest list the kernel takes, rounded up to a power of two (at least
-// 256 records).
-#define GS_SORT_CASE(EE, WW) \
-  register_sort_tile<EE, WW>(t, start, n, records, gauss_of_emission, keys, emission, point_list, s_exchange)
+// 256 records).  Lists of more than max_n records are left to the radix sort's kernels.
+#define GS_SORT_CASE(EE, WW) register_sort_tile<EE, WW>(t, start, n, records, keys, emission, point_list, s_exchange)
 __global__ void __launch_bounds__(512)
-tile_sort_registers_kernel(const uint32_t* __restrict__ ranges, const uint64_t* __restrict__ records,
-                           const uint32_t* __restrict__ gauss_of_emission, uint64_t* __restrict__ keys,
-                           uint32_t* __restrict__ emission, uint32_t* __restrict__ point_list, uint32_t max_n,
+tile_sort_registers_kernel(const uint32_t* __restrict__ ranges, const TileRecord* __restrict__ records,
+                           uint64_t* __restrict__ keys, uint32_t* __restrict__ emission,
+                           uint32_t* __restrict__ point_list, uint32_t max_n,
                            const uint32_t* __restrict__ fits_word) {
   extern __shared__ uint64_t s_exchange[];
   if (fits_word != nullptr && *fits_word == 0u) return;  // launched ahead of the host's decision: see the scatter
   const uint32_t t = blockIdx.x;
   const uint32_t start = ranges[2 * t];
   const uint32_t n = ranges[2 * t + 1] - start;
-  if (n == 0 || n > 2048 || n > max_n) return;
+  if (n == 0 || n > (uint32_t)TILE_SORT_SMALL || n > max_n) return;
   if (n <= 256) {
     if (threadIdx.x >= 256) return;  // (half the workgroup is enough; a wave that has left is not waited for)
     GS_SORT_CASE(1, 4);
@@ -593,108 +570,6 @@ tile_sort_registers_kernel(const uint32_t* __restrict__ ranges, const uint64_t* 
   else if (n <= 1024) GS_SORT_CASE(2, 8);
   else GS_SORT_CASE(4, 8);
 }
-
-__global__ void __launch_bounds__(1024)
-tile_sort_registers_long_kernel(const uint32_t* __restrict__ ranges, const uint64_t* __restrict__ records,
-                                const uint32_t* __restrict__ gauss_of_emission, uint64_t* __restrict__ keys,
-                                uint32_t* __restrict__ emission, uint32_t* __restrict__ point_list,
-                                uint32_t max_n, const uint32_t* __restrict__ fits_word) {
-  extern __shared__ uint64_t s_exchange[];
-  if (fits_word != nullptr && *fits_word == 0u) return;
-  const uint32_t t = blockIdx.x;
-  const uint32_t start = ranges[2 * t];
-  const uint32_t n = ranges[2 * t + 1] - start;
-  if (n <= 2048 || n > max_n) return;
-  if (n <= 4096) GS_SORT_CASE(4, 16);
-  else GS_SORT_CASE(8, 16);
-}
-
-// 2b. Lists beyond the limit of the per-tile sort: the list is cut into chunk_first[t + 1] - chunk_first[t]
-// chunks of equal size (the last one may be shorter), one workgroup sorts each chunk in place, and the merge
-// below puts every record at its final place.
-struct Chunk { uint32_t tile, list_start, list_n, size, index, count; };
-__device__ __forceinline__ Chunk find_chunk(uint32_t b, uint32_t T, const uint32_t* __restrict__ chunk_first,
-                                            const uint32_t* __restrict__ ranges) {
-  // the tile t with chunk_first[t] <= b < chunk_first[t + 1]
-  uint32_t lo = 0, hi = T;
-  while (hi - lo > 1) {
-    const uint32_t mid = (lo + hi) >> 1;
-    if (chunk_first[mid] <= b) lo = mid; else hi = mid;
-  }
-  Chunk c;
-  c.tile = lo;
-  c.list_start = ranges[2 * lo];
-  c.list_n = ranges[2 * lo + 1] - c.list_start;
-  c.count = chunk_first[lo + 1] - chunk_first[lo];
-  c.index = b - chunk_first[lo];
-  c.size = (c.list_n + c.count - 1u) / c.count;
-  return c;
-}
-
-template <int E, int W>
-__device__ __forceinline__ void register_sort_in_place(uint64_t* __restrict__ records, uint32_t n, uint64_t* s_x) {
-  const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  uint64_t v[E];
-#pragma unroll
-  for (int r = 0; r < E; r++) {
-    const uint32_t i = ((wave * E + r) << 6) | lane;
-    v[r] = i < n ? records[i] : ~0ull;
-  }
-  register_sort<E, W>(v, wave, lane, s_x);
-#pragma unroll
-  for (int r = 0; r < E; r++) {
-    const uint32_t i = ((wave * E + r) << 6) | lane;
-    if (i < n) records[i] = v[r];
-  }
-}
-
-__global__ void __launch_bounds__(1024)
-chunk_sort_kernel(uint32_t T, const uint32_t* __restrict__ chunk_first, const uint32_t* __restrict__ ranges,
-                  uint64_t* __restrict__ records) {
-  extern __shared__ uint64_t s_exchange[];
-  const Chunk c = find_chunk(blockIdx.x, T, chunk_first, ranges);
-  const uint32_t begin = c.index * c.size;
-  if (begin >= c.list_n) return;
-  const uint32_t n = c.list_n - begin < c.size ? c.list_n - begin : c.size;
-  uint64_t* mine = records + c.list_start + begin;
-  if (n <= 4096) register_sort_in_place<4, 16>(mine, n, s_exchange);
-  else register_sort_in_place<8, 16>(mine, n, s_exchange);
-}
-
-// A record's final place in its tile's list: its place in its own chunk plus, for every other chunk of the
-// list, the number of that chunk's records below it (records are distinct: they end in the emission index).
-__global__ void __launch_bounds__(256)
-chunk_merge_kernel(uint32_t T, const uint32_t* __restrict__ chunk_first, const uint32_t* __restrict__ ranges,
-                   const uint64_t* __restrict__ records, const uint32_t* __restrict__ gauss_of_emission,
-                   uint64_t* __restrict__ keys, uint32_t* __restrict__ emission, uint32_t* __restrict__ point_list) {
-  const Chunk c = find_chunk(blockIdx.x, T, chunk_first, ranges);
-  const uint32_t begin = c.index * c.size;
-  if (begin >= c.list_n) return;
-  const uint32_t n = c.list_n - begin < c.size ? c.list_n - begin : c.size;
-  const uint64_t* list = records + c.list_start;
-  const uint64_t tile_bits = (uint64_t)c.tile << 32;
-  for (uint32_t i = threadIdx.x; i < n; i += 256) {
-    const uint64_t rec = list[begin + i];
-    uint32_t place = i;
-    for (uint32_t other = 0; other < c.count; other++) {
-      if (other == c.index) continue;
-      const uint32_t ob = other * c.size;
-      if (ob >= c.list_n) break;
-      const uint32_t on = c.list_n - ob < c.size ? c.list_n - ob : c.size;
-      uint32_t lo = 0, hi = on;  // number of records of the other chunk below rec
-      while (lo < hi) {
-        const uint32_t mid = (lo + hi) >> 1;
-        if (list[ob + mid] < rec) lo = mid + 1; else hi = mid;
-      }
-      place += lo;
-    }
-    const uint32_t e = (uint32_t)rec;
-    keys[c.list_start + place] = tile_bits | (rec >> 32);
-    emission[c.list_start + place] = e;
-    point_list[c.list_start + place] = gauss_of_emission[e];
-  }
-}
-
 #undef GS_SORT_CASE
 
 }  // namespace
@@ -702,9 +577,9 @@ chunk_merge_kernel(uint32_t T, const uint32_t* __restrict__ chunk_first, const u
 // Tiles the LDS histograms of the counting kernels can hold.
 int bucket_max_tiles() { return 30000; }
 
-// workgroup-by-tile counts, then the tile totals, then the chunk table (T + 1 words), then the workgroups' sums of
-// tiles touched
-// ... and the word that says whether the view fits the buffers of kernels launched ahead of the host
+// workgroup-by-tile counts, then the tile totals, then the tile lists of the radix sort's kernels (T + 1 words), then
+// the workgroups' sums of tiles touched and the word that says whether the view fits the buffers of kernels
+// launched ahead of the host
 size_t bucket_table_bytes(int T) {
   return (((size_t)BK_MAX_BLOCKS + 2) * (size_t)T + 1 + BK_MAX_BLOCKS + 1) * sizeof(uint32_t);
 }
@@ -716,11 +591,15 @@ const uint32_t* bucket_fits_word(const void* table, int T) {
 }
 
 int launch_bucket_count(int P, int W, int H, const int* radii, const float* means2D, const uint8_t* compute_locally,
-                        uint32_t* tiles_touched, void* table, uint32_t* ranges, uint32_t chunk_limit,
-                        uint32_t* host_words, int* zero_per_gaussian, uint32_t cap_instances, uint32_t cap_longest,
-                        hipStream_t stream) {
+                        uint32_t* tiles_touched, void* table, uint32_t* ranges, uint32_t small_limit,
+                        uint32_t block_limit, uint32_t* host_words, int* zero_per_gaussian, uint32_t cap_instances,
+                        uint32_t cap_longest, hipStream_t stream) {
   if (P <= 0) return 0;
-  if (chunk_limit == 0 || chunk_limit > (uint32_t)TILE_SORT_LARGE) chunk_limit = TILE_SORT_LARGE;
+  if (small_limit == 0 || small_limit > (uint32_t)TILE_SORT_SMALL) small_limit = TILE_SORT_SMALL;
+  // the lists one workgroup of the radix sort's smaller kernel holds; longer ones go to the larger kernel
+  uint32_t mid_limit = (uint32_t)tile_radix_mid_records();
+  if (block_limit != 0 && block_limit < mid_limit) mid_limit = block_limit;
+  if (mid_limit < small_limit) mid_limit = small_limit;
   const uint32_t gx = (W + GS_TILE_X - 1) / GS_TILE_X, gy = (H + GS_TILE_Y - 1) / GS_TILE_Y;
   const uint32_t T = gx * gy;
   const size_t lds = (size_t)T * (sizeof(uint32_t) + 1);
@@ -745,65 +624,52 @@ int launch_bucket_count(int P, int W, int H, const int* radii, const float* mean
                      zero_per_gaussian);
   hipLaunchKernelGGL(bucket_columns_kernel, dim3((T + COL_TILES - 1) / COL_TILES), dim3(COL_TILES * COL_RUNS), 0, stream, nb, T,
                      tab, totals);
-  hipLaunchKernelGGL(bucket_ranges_kernel, dim3(1), dim3(1024), 0, stream, T, chunk_limit, totals, ranges, totals + T,
+  hipLaunchKernelGGL(bucket_ranges_kernel, dim3(1), dim3(1024), 0, stream, T, small_limit, mid_limit, totals, ranges,
+                     totals + T,
                      bucket_block_sums(table, T), nb, host_words, cap_instances, cap_longest,
                      const_cast<uint32_t*>(bucket_fits_word(table, (int)T)));
   return 0;
 }
 
-// point_offsets = inclusive prefix sum of the tiles_touched that launch_bucket_count left (same P, same table).
-// launch_bucket_scatter does this itself; this kernel serves a view that was counted by tile and then goes to the
-// radix sort after all.
-int launch_bucket_offsets(int P, int W, int H, const uint32_t* tiles_touched, void* table, uint32_t* point_offsets,
-                          hipStream_t stream) {
-  if (P <= 0) return 0;
-  const uint32_t gx = (W + GS_TILE_X - 1) / GS_TILE_X, gy = (H + GS_TILE_Y - 1) / GS_TILE_Y;
-  hipLaunchKernelGGL(bucket_offsets_kernel, dim3(bucket_blocks(P)), dim3(BK_THREADS), 0, stream, P,
-                     bucket_per_block(P), tiles_touched, bucket_block_sums(table, gx * gy), point_offsets);
-  return 0;
-}
-
 int launch_bucket_scatter(int P, int W, int H, const float* means2D, const float* depths,
                           const uint32_t* tiles_touched, uint32_t* point_offsets, const int* radii,
-                          const uint8_t* compute_locally, void* table, const uint32_t* ranges, uint64_t* records,
-                          uint32_t* gauss_of_emission, bool ahead_of_host, hipStream_t stream) {
+                          const uint8_t* compute_locally, void* table, const uint32_t* ranges, void* records,
+                          bool ahead_of_host, hipStream_t stream) {
   if (P <= 0) return 0;
   const uint32_t gx = (W + GS_TILE_X - 1) / GS_TILE_X, gy = (H + GS_TILE_Y - 1) / GS_TILE_Y;
   const size_t lds = (size_t)gx * gy * (sizeof(uint32_t) + 1);
   hipLaunchKernelGGL(bucket_scatter_kernel, dim3(bucket_blocks(P)), dim3(BK_THREADS), lds, stream, P,
                      bucket_per_block(P), gx, gy, (const float2*)means2D, depths, tiles_touched,
                      bucket_block_sums(table, gx * gy), point_offsets, radii, compute_locally, (const uint32_t*)table,
-                     ranges, records, gauss_of_emission,
+                     ranges, (TileRecord*)records,
                      ahead_of_host ? bucket_fits_word(table, (int)(gx * gy)) : nullptr,
                      (((uintptr_t)means2D | (uintptr_t)depths | (uintptr_t)tiles_touched | (uintptr_t)point_offsets |
                        (uintptr_t)radii) & 15u) == 0u ? 1 : 0);
   return 0;
 }
 
-// Sorts every tile's segment.  `longest` is the longest list and `limit` (at most TILE_SORT_LARGE) the longest
-// one workgroup sorts whole.  Longer lists are the `chunks` chunks that launch_bucket_count laid out with the same
-// limit: sorted in place in `records`, then merged.
-int launch_tile_sort(int T, uint32_t longest, uint32_t limit, uint32_t chunks, const uint32_t* ranges,
-                     const void* table, uint64_t* records, const uint32_t* gauss_of_emission, uint64_t* keys,
-                     uint32_t* emission, uint32_t* point_list, bool ahead_of_host, hipStream_t stream) {
+// Sorts every tile's segment of `records`.  `longest` is the longest list the launch has to be ready for and
+// `radix_tiles` what the ranges kernel reported (number of lists for the radix sort's larger kernel << 16 | number
+// for its smaller one; a caller that does not know passes 0xFFFFFFFF): the kernels that have nothing to do are
+// not launched.  small_limit (at most TILE_SORT_SMALL) and block_limit as given to launch_bucket_count.
+int launch_tile_sort(int T, uint32_t longest, uint32_t radix_tiles, uint32_t small_limit, uint32_t block_limit,
+                     const uint32_t* ranges, const void* table, const void* records, uint64_t* scratch,
+                     uint64_t* keys, uint32_t* emission, uint32_t* point_list, bool ahead_of_host,
+                     hipStream_t stream) {
   if (T <= 0 || longest == 0) return 0;
   const uint32_t* fits = ahead_of_host ? bucket_fits_word(table, T) : nullptr;
-  if (limit == 0 || limit > (uint32_t)TILE_SORT_LARGE) limit = TILE_SORT_LARGE;
-  const uint32_t whole = longest < limit ? longest : limit;  // the longest list sorted by one workgroup
+  if (small_limit == 0 || small_limit > (uint32_t)TILE_SORT_SMALL) small_limit = TILE_SORT_SMALL;
+  const uint32_t whole = longest < small_limit ? longest : small_limit;  // the longest list sorted in registers
   uint32_t m = 256;
-  while (m < whole && m < 2048) m <<= 1;
+  while (m < whole) m <<= 1;
   hipLaunchKernelGGL(tile_sort_registers_kernel, dim3(T), dim3(512), (size_t)m * sizeof(uint64_t), stream, ranges,
-                     records, gauss_of_emission, keys, emission, point_list, limit, fits);
-  if (whole > 2048)
-    hipLaunchKernelGGL(tile_sort_registers_long_kernel, dim3(T), dim3(1024),
-                       (size_t)(whole > 4096 ? 8192 : 4096) * sizeof(uint64_t), stream, ranges, records,
-                       gauss_of_emission, keys, emission, point_list, limit, fits);
-  if (longest > limit && chunks > 0) {
-    const uint32_t* chunk_first = (const uint32_t*)table + ((size_t)BK_MAX_BLOCKS + 1) * (size_t)T;
-    hipLaunchKernelGGL(chunk_sort_kernel, dim3(chunks), dim3(1024), (size_t)(limit > 4096 ? 8192 : 4096) * sizeof(uint64_t),
-                       stream, (uint32_t)T, chunk_first, ranges, records);
-    hipLaunchKernelGGL(chunk_merge_kernel, dim3(chunks), dim3(256), 0, stream, (uint32_t)T, chunk_first, ranges, records,
-                       gauss_of_emission, keys, emission, point_list);
+                     (const TileRecord*)records, keys, emission, point_list, small_limit, fits);
+  if (longest > small_limit) {
+    const uint32_t* tile_lists = (const uint32_t*)table + ((size_t)BK_MAX_BLOCKS + 1) * (size_t)T;
+    if (launch_tile_radix_sort(T, (radix_tiles & 0xFFFFu) != 0u, (radix_tiles >> 16) != 0u, ranges, tile_lists,
+                               tile_lists + T, block_limit, records, keys, scratch, keys, emission, point_list, fits,
+                               stream))
+      return 1;
   }
   return 0;
 }

@@ -187,8 +187,9 @@ def render_gaussians(background, image_height, image_width, means2D, depths, rad
                      compute_locally, viewmatrix, campos, tan_fovx, tan_fovy, all_map, render_geo, debug, args):
     """rasterize_points.cu:276-364.  Two additions: with args["max_weight_depth"] set, the per-pixel depth of the
     Gaussian that blends with the largest weight (1, H, W) is left in args["stats_collector"]["max_weight_depth"];
-    args["tile_sort_limits"] = (large_limit, max_chunks) chooses, for this call, the way the per-tile
-    lists are built (all ways give the same lists).  The returned tuple is the reference's either way."""
+    args["tile_sort_limits"] = (small_limit, block_records) chooses, for this call, the way the per-tile
+    lists are built (the longest list sorted in registers, 0 = one radix sort over all keys; the records the
+    per-tile radix sort holds at once; all ways give the same lists).  The returned tuple is the reference's either way."""
     return render_gaussians_ex(background, image_height, image_width, means2D, depths, radii, conic_opacity, rgb,
                                compute_locally, viewmatrix, campos, tan_fovx, tan_fovy, all_map, render_geo, debug,
                                args)[0]
@@ -284,7 +285,7 @@ def render_gaussians_ex(background, image_height, image_width, means2D, depths, 
         raise RuntimeError(f"compute_locally must be a bool tensor with {tiles} elements")
     am = _f32c(all_map, "all_map") if geo else None
     want_mwd = isinstance(args, dict) and bool(args.get("max_weight_depth"))
-    # (large_limit, max_chunks) for this call only: how the per-tile lists are built (a test hook)
+    # (small_limit, block_records) for this call only: how the per-tile lists are built (a test hook)
     limits = args.get("tile_sort_limits") if isinstance(args, dict) else None
     options = None
     if limits is not None or expected_instances > 0:

@@ -102,13 +102,14 @@ def _expectation(key):
     if seen is None:
         return 0, 0
     instances, longest = seen
-    if longest <= 0 or longest > 8192:
-        return 0, 0  # a view for the radix sort (no per-tile lists, or lists too long for them): nothing to gain
-    # whole sort variants (256 ... 8192 records per list), so that a slightly longer list still fits
+    if longest <= 0:
+        return 0, 0  # a view without per-tile lists (a tile grid too large for them): nothing to gain
+    # whole variants of the register sort (256 ... 2048 records per list), so that a slightly longer list still
+    # fits; beyond them any length (0): the radix sort's kernels are launched as well
     cap = 256
-    while cap < min(8192, longest * _MARGIN):
+    while cap < longest * _MARGIN:
         cap *= 2
-    return int(instances * _MARGIN) + 65536, cap
+    return int(instances * _MARGIN) + 65536, (cap if cap <= 2048 else 0)
 
 
 class _RenderGaussians(torch.autograd.Function):

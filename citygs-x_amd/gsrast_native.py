@@ -87,13 +87,13 @@ EXPORTED_SYMBOLS = tuple(_SIGNATURES)
 class RenderOptions(C.Structure):
     """gs_render_options of include/gsrast.h; a negative limit keeps the library's default, a zero expectation
     means none."""
-    _fields_ = [("struct_bytes", C.c_uint32), ("tile_sort_large_limit", C.c_int32),
-                ("tile_sort_max_chunks", C.c_int32), ("expected_longest_list", C.c_int32),
+    _fields_ = [("struct_bytes", C.c_uint32), ("tile_sort_small_limit", C.c_int32),
+                ("tile_sort_block_records", C.c_int32), ("expected_longest_list", C.c_int32),
                 ("expected_instances", C.c_int64)]
 
-    def __init__(self, tile_sort_large_limit=-1, tile_sort_max_chunks=-1, expected_instances=0,
+    def __init__(self, tile_sort_small_limit=-1, tile_sort_block_records=-1, expected_instances=0,
                  expected_longest_list=0):
-        super().__init__(C.sizeof(RenderOptions), int(tile_sort_large_limit), int(tile_sort_max_chunks),
+        super().__init__(C.sizeof(RenderOptions), int(tile_sort_small_limit), int(tile_sort_block_records),
                          int(expected_longest_list), int(expected_instances))
 
 

@@ -102,26 +102,27 @@ int gs_preprocess_backward(const int* radii, const float* cov3D, const uint8_t* 
 
 /* No counterpart in the reference: per-call options of gs_render_forward (NULL = all defaults).  A field below
  * zero keeps its default; struct_bytes is sizeof(gs_render_options) as the caller compiled it.
- * gs_render_forward builds the per-tile lists either by bucketing the instances by tile and sorting each tile's
- * list on its own (one workgroup per list of up to 8192 records; longer lists as chunks of at most 8192 that are
- * merged afterwards, up to 32 chunks per view), or, when the view has more long lists than that (or the tile grid
- * more than 30000 tiles), by the reference's own route: (tile | depth) keys (rasterizer_impl.cu:74-117), one radix
- * sort over all of them (:675-684), identifyTileRanges (:122-144).  All give the same lists bit for bit.
- * tile_sort_large_limit lowers the list length that one workgroup sorts whole (default and maximum 8192; 0 = always
- * the radix route) and tile_sort_max_chunks changes the number of chunks the longer lists of a view may be cut into
- * (default 32; 0 = a longer list sends the view to the radix route), so that small scenes can exercise every
- * route.  The library keeps no such setting between calls. */
+ * gs_render_forward builds the per-tile lists by bucketing the instances by tile (a counting sort) and sorting
+ * each tile's list on its own: lists of up to 2048 records in registers, longer ones by a radix sort on the depth
+ * bits that one workgroup runs inside its CU (up to 16384 records at once; a longer list block by block through
+ * memory).  A tile grid of more than 30000 tiles takes the reference's own route instead: (tile | depth) keys
+ * (rasterizer_impl.cu:74-117), one radix sort over all of them (:675-684), identifyTileRanges (:122-144).  All
+ * give the same lists bit for bit.
+ * tile_sort_small_limit lowers the list length that is sorted in registers (default and maximum 2048; 0 = the
+ * view takes the reference's route) and tile_sort_block_records the number of records the per-tile radix sort
+ * holds at once (default and maximum 16384; 0 or below = default), so that small scenes can exercise every route.
+ * The library keeps no such setting between calls. */
 typedef struct gs_render_options {
   uint32_t struct_bytes;
-  int32_t tile_sort_large_limit;
-  int32_t tile_sort_max_chunks;
+  int32_t tile_sort_small_limit;
+  int32_t tile_sort_block_records;
   int32_t expected_longest_list;
   /* What the caller expects of the view, typically the previous view's figures with a margin (0 = no idea).
    * With expected_instances > 0 (and a gs_render_result to report into) gs_render_forward does not wait for the
    * instance count before it goes on: it sizes the binning buffer for expected_instances, launches the list
    * kernels and the blend right behind the counting kernels, and lets a device-side check turn them into no-ops
-   * if the view has more instances than that or a list longer than expected_longest_list (0 = the longest one
-   * workgroup sorts); in that case the lists are built again the ordinary way, so the result never depends on
+   * if the view has more instances than that or a list longer than expected_longest_list (0 = any length; a
+   * figure of at most 2048 spares the launch of the radix sort's kernels); in that case the lists are built again the ordinary way, so the result never depends on
    * the expectation, only the time does. */
   int64_t expected_instances;
 } gs_render_options;

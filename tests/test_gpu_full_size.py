@@ -144,8 +144,8 @@ def test_config1_full_size(H):
 def test_list_routes_agree_at_full_size(H, cfg, P):
     """The per-tile lists at BASELINE sizes (config 1; config 3: 10 M Gaussians, 1920x1080, street level, lists of
     more than 8192 records) come out the same bit for bit by the radix sort over all keys (checked against numpy at
-    small sizes and through its properties at large ones), by the per-tile sort, and by the per-tile sort with
-    every long list cut into chunks (of 8192 and of 2048 records) and merged."""
+    small sizes and through its properties at large ones), by the per-tile sorts, by the per-tile radix sort from
+    256 records on, and by the per-tile radix sort going block by block (3000 records) through memory."""
     import gs_scenes
     import gsrast_native as gn
     from diff_gaussian_rasterization import _C
@@ -165,7 +165,7 @@ def test_list_routes_agree_at_full_size(H, cfg, P):
     cl = torch.ones(gy, gx, dtype=torch.bool, device=DEV)
     results = []
     if True:
-        for limits in [(0, 0), (8192, 0), (8192, 1 << 30), (2048, 1 << 30)]:
+        for limits in [(0, 0), (-1, -1), (256, 0), (-1, 3000)]:
             args["tile_sort_limits"] = limits
             out = _C.render_gaussians(torch.zeros(3, device=DEV), Hh, W, means2D, depths, radii, co, rgb, cl, vm, cp,
                                       cam.tanfovx, cam.tanfovy, am, False, False, args)

@@ -1,6 +1,7 @@
 """The per-tile lists render_gaussians builds (ranges, sorted keys, point_list), by each of its routes: instances
-bucketed by tile and sorted per tile (a list beyond the limit of one workgroup in chunks that are merged), and the radix sort over all (tile | depth) keys.  Every route must give the oracle's lists bit for bit, and the backward pass must file its per-instance
-gradients correctly under each."""
+bucketed by tile and sorted per tile (in registers, by the per-tile radix sort inside one CU, or by the per-tile radix
+sort block by block through memory), and the radix sort over all (tile | depth) keys.  Every route must give the
+oracle's lists bit for bit, and the backward pass must file its per-instance gradients correctly under each."""
 import ctypes as C
 
 import numpy as np
@@ -28,10 +29,10 @@ def _mask(kind, gx, gy):
     return cl
 
 
-# (longest list one workgroup sorts, chunks the longer lists may be cut into): defaults; a list too long for the
-# per-tile sort, found after the counting pass (the radix route takes over); the radix route from the start; lists
-# beyond the limit sorted in chunks and merged (few large chunks, more of them, many chunks of an odd size)
-ROUTES = [(8192, 32), (40, 0), (0, 32), (40, 1 << 30), (100, 1 << 30), (7, 1 << 30)]
+# (longest list sorted in registers, records the per-tile radix sort holds at once): defaults; lists of more than 40
+# records by the per-tile radix sort's two kernels; the radix sort over all keys; lists of more than 40 records by
+# the smaller kernel up to 64 and block by block beyond (blocks of 64, of 128, and many blocks of an odd size)
+ROUTES = [(-1, -1), (40, 0), (0, 0), (40, 64), (100, 128), (7, 7)]
 
 
 @pytest.mark.parametrize("cfg,P,mask", [(0, 30_000, "all"), (1, 120_000, "all"), (1, 60_000, "checker"),
@@ -54,7 +55,7 @@ def test_lists_match_oracle_by_every_route(orc, H, cfg, P, mask):
     R_want = int(want["point_list"].shape[0])
     counts = want["ranges"].reshape(-1, 2).astype(np.int64)
     longest = int((counts[:, 1] - counts[:, 0]).max())
-    assert longest > 40  # so that the third route really exceeds its large limit
+    assert longest > 64  # so that the blocked routes really sort lists of more than one block
     ug = gs_scenes.upstream_grads(cam)
     args = {"stats_collector": {}}
     grads = []
@@ -129,12 +130,12 @@ def test_equal_depths_keep_emission_order(orc, H):
         assert np.array_equal(H.np_u32(point_list), want["point_list"]), (large, chunks)
 
 
-@pytest.mark.parametrize("P,expect", [(28_000, "waves4"), (56_000, "waves8"), (110_000, "chunks"),
-                                      (110_000, "radix"), (230_000, "chunks3")])
+@pytest.mark.parametrize("P,expect", [(28_000, "mid"), (56_000, "long"), (110_000, "long2"),
+                                      (110_000, "radix"), (230_000, "blocks"), (230_000, "blocks4k")])
 def test_long_lists(orc, H, P, expect):
-    """A small image under many large Gaussians: lists of several thousand records per tile (sixteen waves per
-    tile, 4 or 8 records per lane); beyond 8192 the list is sorted in chunks and merged, or, where the view has
-    more such chunks than the bound, the radix route takes over by itself."""
+    """A small image under many large Gaussians: lists of several thousand records per tile.  Up to 4096 the
+    smaller kernel of the per-tile radix sort takes them, up to 16384 the larger one, both inside the CU; beyond
+    that (or beyond the block size the call asks for) the larger kernel sorts block by block through memory."""
     import gs_scenes
     import gsrast_native as gn
     from diff_gaussian_rasterization import _C
@@ -150,14 +151,14 @@ def test_long_lists(orc, H, P, expect):
     want = orc.bin_and_sort(n(o["radii"]), n(o["means2D"]), n(o["depths"]), cl.numpy().reshape(-1), W, Hh)
     counts = want["ranges"].reshape(-1, 2).astype(np.int64)
     longest = int((counts[:, 1] - counts[:, 0]).max())
-    lo, hi = {"waves4": (2048, 4096), "waves8": (4096, 8192), "chunks": (8192, 16384), "radix": (8192, 16384),
-              "chunks3": (16384, 65536)}[expect]
+    lo, hi = {"mid": (2048, 4096), "long": (4096, 8192), "long2": (8192, 16384), "radix": (8192, 16384),
+              "blocks": (16384, 65536), "blocks4k": (16384, 65536)}[expect]
     assert lo < longest <= hi, longest
     limits = None
     if expect == "radix":
-        limits = (8192, 0)
-    elif expect.startswith("chunks"):  # nearly every tile of this view has a long list: lift the bound on their number
-        limits = (8192, 1 << 30)
+        limits = (0, 0)
+    elif expect == "blocks4k":
+        limits = (-1, 5000)
     vm, cp = cam.world_view_transform.to(DEV), cam.camera_center.to(DEV)
     am = gs_scenes.build_all_map(gd["means3D"], gd["scales"], gd["rotations"], cam)
     out = _C.render_gaussians(torch.zeros(3, device=DEV), Hh, W, o["means2D"], o["depths"], o["radii"],
@@ -214,7 +215,7 @@ def test_grid_too_large_for_the_tile_histogram(orc, H):
     assert np.array_equal(H.np_u32(point_list), want["point_list"])
 
 
-@pytest.mark.parametrize("limits", [(8192, 32), (0, 32)])
+@pytest.mark.parametrize("limits", [(-1, -1), (0, 0)])
 def test_more_instances_than_positions_is_an_error(H, limits):
     """1.2 M splats that each cover all 3888 tiles are 4.7e9 instances: the 32-bit prefix sums wrap around to a
     plausible count (3.7e8).  The call must fail on the exact count instead of sizing its buffers by the wrapped
