@@ -172,7 +172,7 @@ BinningLayout binning_layout(int64_t R) {
   L.emission = take(n * 4);
   L.sort_temp = take(sort_temp_bytes((int64_t)n));
   L.block_hits = take(n * 2);  // what the forward blend leaves for the backward blend, per sorted instance
-  L.radix_scratch = take(n * 8);  // second array of the per-tile radix sort for lists it sorts in blocks
+  L.radix_scratch = take(n * 24);  // per-tile radix sort: lists beyond one block, split (16 B) and in blocks (8 B)
   L.total = off + 256;
   return L;
 }
@@ -563,8 +563,9 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
   EventTimer timer;
   struct Arrays {
     uint32_t *point_list, *gauss_of_emission, *emission, *emission_other;
-    uint64_t *keys, *keys_other, *radix_scratch;
-    void* sort_temp;
+    uint64_t *keys, *keys_other;
+    void *sort_temp, *radix_scratch;
+    int64_t capacity;
     uint16_t* block_hits;
   };
   auto carve = [&](int64_t n, Arrays& A) -> int {
@@ -580,7 +581,8 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
     A.emission_other = (uint32_t*)(bbase + BL.emission_other);
     A.sort_temp = bbase + BL.sort_temp;
     A.block_hits = (uint16_t*)(bbase + BL.block_hits);
-    A.radix_scratch = (uint64_t*)(bbase + BL.radix_scratch);
+    A.radix_scratch = bbase + BL.radix_scratch;
+    A.capacity = n > 0 ? n : 1;
     return 0;
   };
   auto blend = [&](const Arrays& A, bool ahead_of_host) -> int {
@@ -617,8 +619,8 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
     {
       StageScope _t("tile_sort", stream);
       if (launch_tile_sort(T, longest_for_launch, radix_tiles, sort_limit, (uint32_t)limits.block, ranges,
-                           bucket_table, A.keys_other, A.radix_scratch, A.keys, A.emission, A.point_list,
-                           ahead_of_host, stream))
+                           bucket_table, A.keys_other, A.radix_scratch, A.capacity, A.keys, A.emission,
+                           A.point_list, ahead_of_host, stream))
         return 1;
     }
     return check_launch("tile_sort", stream, dbg);

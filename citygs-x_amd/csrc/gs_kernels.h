@@ -114,16 +114,16 @@ int launch_bucket_scatter(int P, int W, int H, const float* means2D, const float
                           const uint32_t* tiles_touched, uint32_t* point_offsets, const int* radii,
                           const uint8_t* compute_locally, void* table, const uint32_t* ranges, void* records,
                           bool ahead_of_host, hipStream_t stream);
-// scratch: 8 bytes per instance, used for lists of more than block_limit records
+// scratch: 24 bytes per instance, used for lists of more than block_limit records
 int launch_tile_sort(int T, uint32_t longest, uint32_t radix_tiles, uint32_t small_limit, uint32_t block_limit,
-                     const uint32_t* ranges, const void* table, const void* records, uint64_t* scratch,
+                     const uint32_t* ranges, const void* table, const void* records, void* scratch, int64_t capacity,
                      uint64_t* keys, uint32_t* emission, uint32_t* point_list, bool ahead_of_host,
                      hipStream_t stream);
 int tile_radix_mid_records();    // records one workgroup of the radix sort's smaller kernel holds (4096)
 int tile_radix_block_records();  // ... and of its larger kernel (16384): longer lists are sorted in blocks
 int launch_tile_radix_sort(int T, bool mid, bool lng, const uint32_t* ranges, const uint32_t* tile_lists,
-                           const uint32_t* counts, uint32_t block_limit, const void* records, uint64_t* ping,
-                           uint64_t* pong, uint64_t* keys, uint32_t* emission, uint32_t* point_list,
+                           const uint32_t* counts, uint32_t block_limit, const void* records, void* parted,
+                           uint64_t* ping, uint64_t* pong, uint64_t* keys, uint32_t* emission, uint32_t* point_list,
                            const uint32_t* fits_word, hipStream_t stream);
 // What the blend kernels read of a Gaussian, in one 64-byte record per Gaussian: (x, y, A, B), (C, opacity, r, g),
 // (b, map0, map1, map2), (map3, map4, depth, 0); all_map and depths may be null (zeros).  Records of Gaussians with

@@ -274,8 +274,12 @@ sort_onesweep_kernel(int64_t n, const K* __restrict__ keys_in, K* __restrict__ k
   // of them waits for an earlier one's result, so all items are in flight together.
   // Step 1: the lanes of the wave that hold the same digit find each other through a 64-bit lane mask per
   // digit: every lane ORs its bit in, reads the mask back, and clears it for the next item.
-  volatile unsigned long long* vmask = s_mask[wave];
-  volatile uint32_t* vcount = s_wcount[wave];
+  // (typed as LDS pointers: through plain pointers these volatile accesses come out as flat loads and stores,
+  // which are slower and wait on the memory counters as well)
+  typedef __attribute__((address_space(3))) unsigned long long lds_mask;
+  typedef __attribute__((address_space(3))) uint32_t lds_u32;
+  volatile lds_mask* vmask = (lds_mask*)&s_mask[wave][0];
+  volatile lds_u32* vcount = (lds_u32*)&s_wcount[wave][0];
   const unsigned long long lane_bit = 1ull << lane;
   const unsigned long long lt_mask = lane_bit - 1ull;
   uint32_t match[SORT_ITEMS];  // rank in the wave | valid << 17; later the place in the regrouped tile

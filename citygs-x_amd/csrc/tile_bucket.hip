@@ -651,9 +651,10 @@ int launch_bucket_scatter(int P, int W, int H, const float* means2D, const float
 // Sorts every tile's segment of `records`.  `longest` is the longest list the launch has to be ready for and
 // `radix_tiles` what the ranges kernel reported (number of lists for the radix sort's larger kernel << 16 | number
 // for its smaller one; a caller that does not know passes 0xFFFFFFFF): the kernels that have nothing to do are
-// not launched.  small_limit (at most TILE_SORT_SMALL) and block_limit as given to launch_bucket_count.
+// not launched.  small_limit (at most TILE_SORT_SMALL) and block_limit as given to launch_bucket_count; `scratch`
+// holds 24 bytes for each of the `capacity` instances the binning arrays are laid out for.
 int launch_tile_sort(int T, uint32_t longest, uint32_t radix_tiles, uint32_t small_limit, uint32_t block_limit,
-                     const uint32_t* ranges, const void* table, const void* records, uint64_t* scratch,
+                     const uint32_t* ranges, const void* table, const void* records, void* scratch, int64_t capacity,
                      uint64_t* keys, uint32_t* emission, uint32_t* point_list, bool ahead_of_host,
                      hipStream_t stream) {
   if (T <= 0 || longest == 0) return 0;
@@ -666,9 +667,11 @@ int launch_tile_sort(int T, uint32_t longest, uint32_t radix_tiles, uint32_t sma
                      (const TileRecord*)records, keys, emission, point_list, small_limit, fits);
   if (longest > small_limit) {
     const uint32_t* tile_lists = (const uint32_t*)table + ((size_t)BK_MAX_BLOCKS + 1) * (size_t)T;
+    // scratch: `capacity` 16-byte records for the lists that are split first, then as many 8-byte words
+    uint64_t* pong = (uint64_t*)((char*)scratch + (size_t)capacity * 16);
     if (launch_tile_radix_sort(T, (radix_tiles & 0xFFFFu) != 0u, (radix_tiles >> 16) != 0u, ranges, tile_lists,
-                               tile_lists + T, block_limit, records, keys, scratch, keys, emission, point_list, fits,
-                               stream))
+                               tile_lists + T, block_limit, records, scratch, keys, pong, keys, emission, point_list,
+                               fits, stream))
       return 1;
   }
   return 0;

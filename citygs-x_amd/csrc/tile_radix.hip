@@ -18,11 +18,21 @@
 #include "gs_kernels.h"
 #include "tile_lists.h"
 
+#ifndef TR_MARK
+#define TR_MARK(i)
+#endif
+
 namespace gs {
 namespace {
 
 constexpr int TR_DIGITS = 256;
 constexpr int TR_PASSES = 4;
+
+// Pointers into LDS, typed as such: through a plain pointer the volatile accesses of the ranking come out as
+// flat loads and stores, which are slower and wait on the memory counters as well.
+typedef __attribute__((address_space(3))) uint64_t lds_u64;
+typedef __attribute__((address_space(3))) uint32_t lds_u32;
+typedef __attribute__((address_space(3))) unsigned long long lds_mask;
 
 __device__ __forceinline__ uint32_t tr_wave_inclusive_scan(uint32_t v, int lane) {
 #pragma unroll
@@ -40,22 +50,25 @@ struct TileRadixLds {
   static constexpr int BLOCK = THREADS * ITEMS;
   static_assert(BLOCK >= WAVES * TR_DIGITS, "the lane masks of the ranking live in the regrouping buffer");
   static_assert(ITEMS % 4 == 0, "items are ranked four at a time");
-  uint64_t* rec;    // [BLOCK] regrouping buffer; during the ranking its head holds the lane masks [WAVES][256]
-  uint32_t* count;  // [WAVES][256] per wave and digit: running count, then place of the wave's first such record
-  uint32_t* total;  // [256] records of the block per digit
-  uint32_t* first;  // [256] place in the regrouped block of the first record of a digit
-  uint32_t* base;   // [4][256] blocked sort: where the next record of a digit goes in the segment, per pass
-  uint32_t* scan;   // [16]
-  __device__ explicit TileRadixLds(uint64_t* p) {
+  lds_u64* rec;    // [BLOCK] regrouping buffer; during the ranking its head holds the lane masks [WAVES][256]
+  lds_u32* count;  // [WAVES][256] per wave and digit: running count, then place of the wave's first such record
+  lds_u32* total;  // [256] records of the block per digit
+  lds_u32* first;  // [256] place in the regrouped block of the first record of a digit
+  lds_u32* base;   // [4][256] blocked sort: where the next record of a digit goes in the segment, per pass
+  lds_u32* scan;   // [16]
+  lds_u32* bins;   // [257] partitioned sort: first place of every leading-digit bin in the list, then its length
+  __device__ explicit TileRadixLds(lds_u64* p) {
     rec = p;
-    count = reinterpret_cast<uint32_t*>(p + BLOCK);
+    count = (lds_u32*)(p + BLOCK);
     total = count + WAVES * TR_DIGITS;
     first = total + TR_DIGITS;
     base = first + TR_DIGITS;
     scan = base + TR_PASSES * TR_DIGITS;
+    bins = scan + 16;
   }
   static constexpr size_t bytes() {
-    return (size_t)BLOCK * 8 + (size_t)(WAVES * TR_DIGITS + 2 * TR_DIGITS + TR_PASSES * TR_DIGITS + 16) * 4;
+    return (size_t)BLOCK * 8 +
+           (size_t)(WAVES * TR_DIGITS + 2 * TR_DIGITS + TR_PASSES * TR_DIGITS + 16 + TR_DIGITS + 4) * 4;
   }
 };
 
@@ -67,16 +80,17 @@ __device__ __forceinline__ void radix_block_pass(const uint64_t (&rec)[ITEMS], u
                                                  const TileRadixLds<WAVES, ITEMS>& L) {
   constexpr int THREADS = WAVES * GS_WAVE;
   const int tid = threadIdx.x, lane = tid & (GS_WAVE - 1), wave = tid / GS_WAVE;
-  unsigned long long* s_mask = reinterpret_cast<unsigned long long*>(L.rec);
+  lds_mask* s_mask = (lds_mask*)L.rec;
   for (int i = tid; i < WAVES * TR_DIGITS; i += THREADS) {
     s_mask[i] = 0ull;
     L.count[i] = 0u;
   }
   __syncthreads();
+  TR_MARK(1);
   // LDS operations of one wave execute in program order, which the two steps rely on; none of them waits for an
   // earlier one's result, so the items of a batch are in flight together.
-  volatile unsigned long long* vmask = s_mask + wave * TR_DIGITS;
-  volatile uint32_t* vcount = L.count + wave * TR_DIGITS;
+  volatile lds_mask* vmask = s_mask + wave * TR_DIGITS;
+  volatile lds_u32* vcount = L.count + wave * TR_DIGITS;
   const unsigned long long lane_bit = 1ull << lane;
   const unsigned long long lt_mask = lane_bit - 1ull;
   const uint32_t wave_first = (uint32_t)wave * GS_WAVE * E;
@@ -92,17 +106,38 @@ __device__ __forceinline__ void radix_block_pass(const uint64_t (&rec)[ITEMS], u
   for (int h = 0; h < ITEMS / BATCH; h++) {
     if ((uint32_t)(h * BATCH) >= E) continue;  // (uniform over the workgroup)
     unsigned long long same[BATCH];
-    // Step 1: every lane ORs its bit into the mask of its digit, reads the mask back and clears it.
+    // Step 1: the lanes that hold the same digit find each other.  A digit that many lanes share (the leading
+    // bits of depths inside one tile take few values) would serialise the LDS atomic below lane after lane, so
+    // up to three such digits are taken out first with one ballot each; the other lanes OR their bit into the
+    // mask of their digit, read the mask back and clear it.
 #pragma unroll
     for (int j = 0; j < BATCH; j++) {
       const int k = h * BATCH + j;
       const uint32_t d = (uint32_t)(rec[k] >> shift) & (TR_DIGITS - 1);
-      if (valid[k]) atomicOr(&s_mask[wave * TR_DIGITS + d], lane_bit);
-      __builtin_amdgcn_wave_barrier();
-      same[j] = valid[k] ? vmask[d] : 0ull;
-      __builtin_amdgcn_wave_barrier();
-      if (valid[k]) vmask[d] = 0ull;
-      __builtin_amdgcn_wave_barrier();
+      uint64_t rest = gs_ballot(valid[k]);
+      unsigned long long mine = 0ull;
+      bool placed = !valid[k];
+#pragma unroll
+      for (int round = 0; round < 3; round++) {
+        if (rest == 0ull) break;
+        const uint32_t d0 = (uint32_t)__builtin_amdgcn_readlane((int)d, (int)__builtin_ctzll(rest));
+        const uint64_t m = gs_ballot(valid[k] && d == d0);
+        if (__popcll(m) < 8) break;
+        if (valid[k] && d == d0) {
+          mine = m;
+          placed = true;
+        }
+        rest &= ~m;
+      }
+      same[j] = mine;
+      if (rest != 0ull) {
+        if (!placed) atomicOr((unsigned long long*)&s_mask[wave * TR_DIGITS + d], lane_bit);
+        __builtin_amdgcn_wave_barrier();
+        if (!placed) same[j] = vmask[d];
+        __builtin_amdgcn_wave_barrier();
+        if (!placed) vmask[d] = 0ull;
+        __builtin_amdgcn_wave_barrier();
+      }
     }
     // Step 2: all matching lanes read the wave's running count of the digit, the lowest of them adds their number.
 #pragma unroll
@@ -112,12 +147,15 @@ __device__ __forceinline__ void radix_block_pass(const uint64_t (&rec)[ITEMS], u
       const unsigned long long lower = same[j] & lt_mask;
       const uint32_t before = valid[k] ? vcount[d] : 0u;
       __builtin_amdgcn_wave_barrier();
-      if (valid[k] && lower == 0ull) atomicAdd(&L.count[wave * TR_DIGITS + d], (uint32_t)__popcll(same[j]));
+      if (valid[k] && lower == 0ull)
+        atomicAdd((uint32_t*)&L.count[wave * TR_DIGITS + d], (uint32_t)__popcll(same[j]));
       __builtin_amdgcn_wave_barrier();
       match[k] = before + (uint32_t)__popcll(lower);
     }
   }
+  TR_MARK(2);
   __syncthreads();
+  TR_MARK(3);
   // thread d < 256: the block's records of digit d, their first place, and every wave's first place
   uint32_t tot = 0, inc = 0;
   if (tid < TR_DIGITS) {
@@ -143,6 +181,7 @@ __device__ __forceinline__ void radix_block_pass(const uint64_t (&rec)[ITEMS], u
     }
   }
   __syncthreads();
+  TR_MARK(4);
 #pragma unroll
   for (int k = 0; k < ITEMS; k++) {
     if (!valid[k]) continue;
@@ -150,6 +189,41 @@ __device__ __forceinline__ void radix_block_pass(const uint64_t (&rec)[ITEMS], u
     L.rec[L.count[wave * TR_DIGITS + d] + match[k]] = rec[k];
   }
   __syncthreads();
+  TR_MARK(5);
+}
+
+
+// Smallest and largest of the threads' values over the workgroup (every thread calls this; `lo_words` and
+// `hi_words` are 16 words of LDS each, free for the duration).
+template <int WAVES>
+__device__ __forceinline__ void workgroup_min_max(uint32_t& lo, uint32_t& hi, lds_u32* lo_words, lds_u32* hi_words) {
+  const int lane = threadIdx.x & (GS_WAVE - 1), wave = threadIdx.x / GS_WAVE;
+#pragma unroll
+  for (int d = GS_WAVE / 2; d >= 1; d >>= 1) {
+    const uint32_t a = __shfl_xor(lo, d, GS_WAVE), b = __shfl_xor(hi, d, GS_WAVE);
+    lo = a < lo ? a : lo;
+    hi = b > hi ? b : hi;
+  }
+  if (lane == 0) {
+    lo_words[wave] = lo;
+    hi_words[wave] = hi;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int w = 0; w < WAVES; w++) {
+    const uint32_t a = lo_words[w], b = hi_words[w];
+    lo = a < lo ? a : lo;
+    hi = b > hi ? b : hi;
+  }
+  __syncthreads();
+}
+
+// Passes a list whose depth bits span `range` (largest minus smallest) needs: the sort runs on depth bits minus
+// the smallest, whose digits above the range are all zero.  At least one, so that the pass's output exists.
+__device__ __forceinline__ int passes_for_range(uint32_t range) {
+  int p = 1;
+  while (p < TR_PASSES && (range >> (8 * p)) != 0u) p++;
+  return p;
 }
 
 // A list of at most BLOCK records.
@@ -163,15 +237,27 @@ __device__ __forceinline__ void sort_resident(uint32_t tile, uint32_t start, uin
   const uint32_t E = (n + THREADS - 1) / THREADS;
   const uint32_t wave_first = (uint32_t)wave * GS_WAVE * E;
   uint64_t rec[ITEMS];
+  uint32_t dmin = 0xFFFFFFFFu, dmax = 0u;
 #pragma unroll
   for (int k = 0; k < ITEMS; k++) {
     const uint32_t i = wave_first + (uint32_t)k * GS_WAVE + (uint32_t)lane;
-    rec[k] = ((uint32_t)k < E && i < n) ? ((uint64_t)records[start + i].z << 32) | (uint64_t)i : ~0ull;
+    rec[k] = ~0ull;
+    if ((uint32_t)k < E && i < n) {
+      const uint32_t depth_bits = records[start + i].z;
+      dmin = depth_bits < dmin ? depth_bits : dmin;
+      dmax = depth_bits > dmax ? depth_bits : dmax;
+      rec[k] = ((uint64_t)depth_bits << 32) | (uint64_t)i;
+    }
   }
+  TR_MARK(0);
+  workgroup_min_max<WAVES>(dmin, dmax, L.scan, L.total);
+  const int passes = passes_for_range(dmax - dmin);
+#pragma unroll
+  for (int k = 0; k < ITEMS; k++) rec[k] -= (uint64_t)dmin << 32;  // (records that do not exist are never looked at)
 #pragma unroll 1
-  for (int p = 0; p < TR_PASSES; p++) {
+  for (int p = 0; p < passes; p++) {
     radix_block_pass<WAVES, ITEMS>(rec, E, n, 32 + 8 * p, L);
-    if (p + 1 < TR_PASSES) {
+    if (p + 1 < passes) {
 #pragma unroll
       for (int k = 0; k < ITEMS; k++) {
         const uint32_t i = wave_first + (uint32_t)k * GS_WAVE + (uint32_t)lane;
@@ -180,18 +266,35 @@ __device__ __forceinline__ void sort_resident(uint32_t tile, uint32_t start, uin
       __syncthreads();
     }
   }
-  // L.rec: (depth bits << 32 | place in the segment) in the final order but for runs of equal depth bits.  Replace
-  // the place by the emission index, keep the Gaussian, and write the lists.
+  // L.rec: ((depth bits - smallest) << 32 | place in the segment) in the final order but for runs of equal depth
+  // bits.  The Gaussian and the emission index of every entry are looked up through LDS: the sorted entries wait in
+  // registers while the segment's (Gaussian, emission index) pairs are read in order into the buffer (a gather
+  // from memory, even from the L2, costs as much as all four passes); then the buffer takes (depth bits << 32 |
+  // emission index) in sorted order for the last step.
+#pragma unroll
+  for (int k = 0; k < ITEMS; k++) {
+    const uint32_t i = (uint32_t)k * THREADS + (uint32_t)tid;
+    rec[k] = i < n ? L.rec[i] : 0ull;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int k = 0; k < ITEMS; k++) {
+    const uint32_t i = (uint32_t)k * THREADS + (uint32_t)tid;
+    if (i < n) {
+      const uint2 ge = *reinterpret_cast<const uint2*>(records + start + i);
+      L.rec[i] = ((uint64_t)ge.y << 32) | (uint64_t)ge.x;
+    }
+  }
+  __syncthreads();
   uint32_t gaussian[ITEMS];
 #pragma unroll
   for (int k = 0; k < ITEMS; k++) {
     const uint32_t i = (uint32_t)k * THREADS + (uint32_t)tid;
     gaussian[k] = 0u;
     if (i < n) {
-      const uint64_t r = L.rec[i];
-      const uint2 ge = *reinterpret_cast<const uint2*>(records + start + (uint32_t)r);
-      gaussian[k] = ge.x;
-      rec[k] = (r & 0xFFFFFFFF00000000ull) | (uint64_t)ge.y;
+      const uint64_t ge = L.rec[(uint32_t)rec[k]];
+      gaussian[k] = (uint32_t)ge;
+      rec[k] = ((rec[k] & 0xFFFFFFFF00000000ull) + ((uint64_t)dmin << 32)) | (ge >> 32);
     }
   }
   __syncthreads();
@@ -201,7 +304,8 @@ __device__ __forceinline__ void sort_resident(uint32_t tile, uint32_t start, uin
     if (i < n) L.rec[i] = rec[k];
   }
   __syncthreads();
-  const uint64_t* sorted = L.rec;
+  TR_MARK(6);
+  const lds_u64* sorted = L.rec;
 #pragma unroll 1
   for (int k = 0; k < ITEMS; k++) {
     const uint32_t i = (uint32_t)k * THREADS + (uint32_t)tid;
@@ -209,10 +313,11 @@ __device__ __forceinline__ void sort_resident(uint32_t tile, uint32_t start, uin
       emit_list_entry(tile, start, n, i, gaussian[k], [&](uint32_t q) { return sorted[q]; }, keys, emission,
                       point_list);
   }
+  TR_MARK(7);
 }
 
-// A list of more than `blk` records (blk <= BLOCK): four passes over its blocks, from the segment's records into
-// `ping`, then ping -> pong -> ping -> pong; the lists are written from pong.
+// A list of more than `blk` records (blk <= BLOCK): up to four passes over its blocks, the first from the segment's
+// records, then between ping and pong, ending in pong; the lists are written from pong.
 template <int WAVES, int ITEMS>
 __device__ __forceinline__ void sort_blocked(uint32_t tile, uint32_t start, uint32_t n, uint32_t blk,
                                              const TileRecord* __restrict__ records, uint64_t* ping, uint64_t* pong,
@@ -221,29 +326,59 @@ __device__ __forceinline__ void sort_blocked(uint32_t tile, uint32_t start, uint
                                              const TileRadixLds<WAVES, ITEMS>& L) {
   constexpr int THREADS = WAVES * GS_WAVE;
   const int tid = threadIdx.x, lane = tid & (GS_WAVE - 1), wave = tid / GS_WAVE;
+  // (one workgroup has few loads in flight: every sweep over the list keeps SWEEP of them per thread going)
+  constexpr int SWEEP = 8;
+  uint32_t dmin = 0xFFFFFFFFu, dmax = 0u;
+  for (uint32_t i0 = 0; i0 < n; i0 += THREADS * SWEEP) {
+    uint32_t depth_bits[SWEEP];
+#pragma unroll
+    for (int u = 0; u < SWEEP; u++) {
+      const uint32_t i = i0 + (uint32_t)u * THREADS + (uint32_t)tid;
+      depth_bits[u] = i < n ? records[start + i].z : dmax;
+    }
+#pragma unroll
+    for (int u = 0; u < SWEEP; u++) {
+      const uint32_t i = i0 + (uint32_t)u * THREADS + (uint32_t)tid;
+      if (i < n) {
+        dmin = depth_bits[u] < dmin ? depth_bits[u] : dmin;
+        dmax = depth_bits[u] > dmax ? depth_bits[u] : dmax;
+      }
+    }
+  }
+  workgroup_min_max<WAVES>(dmin, dmax, L.scan, L.total);
+  const int passes = passes_for_range(dmax - dmin);
   for (int i = tid; i < TR_PASSES * TR_DIGITS; i += THREADS) L.base[i] = 0u;
   __syncthreads();
-  // the digit histograms of all four passes from one read of the depth bits
-  for (uint32_t i0 = 0; i0 < n; i0 += THREADS) {
-    const uint32_t i = i0 + (uint32_t)tid;
-    const bool valid = i < n;
-    const uint32_t depth_bits = valid ? records[start + i].z : 0u;
+  // the digit histograms of all passes from one more read of the depth bits
+  for (uint32_t i0 = 0; i0 < n; i0 += THREADS * SWEEP) {
+    uint32_t depth_bits[SWEEP];
 #pragma unroll
-    for (int p = 0; p < TR_PASSES; p++) {
-      const uint32_t d = (depth_bits >> (8 * p)) & (TR_DIGITS - 1);
-      // a digit shared by the whole wave (exponent bits) would serialise the LDS atomic 64 ways: one lane adds
-      const uint64_t vm = gs_ballot(valid);
-      const uint32_t d0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)d);
-      if (vm != 0ull && gs_ballot(valid && d == d0) == vm && (vm & 1ull)) {
-        if (lane == 0) atomicAdd(&L.base[p * TR_DIGITS + d0], (uint32_t)__popcll(vm));
-      } else if (valid) {
-        atomicAdd(&L.base[p * TR_DIGITS + d], 1u);
+    for (int u = 0; u < SWEEP; u++) {
+      const uint32_t i = i0 + (uint32_t)u * THREADS + (uint32_t)tid;
+      depth_bits[u] = i < n ? records[start + i].z : dmin;
+    }
+#pragma unroll
+    for (int u = 0; u < SWEEP; u++) {
+      const bool valid = i0 + (uint32_t)u * THREADS + (uint32_t)tid < n;
+      const uint32_t key = depth_bits[u] - dmin;
+#pragma unroll
+      for (int p = 0; p < TR_PASSES; p++) {
+        if (p >= passes) break;
+        const uint32_t d = (key >> (8 * p)) & (TR_DIGITS - 1);
+        // a digit shared by the whole wave (leading bits) would serialise the LDS atomic 64 ways: one lane adds
+        const uint64_t vm = gs_ballot(valid);
+        const uint32_t d0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)d);
+        if (vm != 0ull && gs_ballot(valid && d == d0) == vm && (vm & 1ull)) {
+          if (lane == 0) atomicAdd((uint32_t*)&L.base[p * TR_DIGITS + d0], (uint32_t)__popcll(vm));
+        } else if (valid) {
+          atomicAdd((uint32_t*)&L.base[p * TR_DIGITS + d], 1u);
+        }
       }
     }
   }
   __syncthreads();
 #pragma unroll 1
-  for (int p = 0; p < TR_PASSES; p++) {
+  for (int p = 0; p < passes; p++) {
     uint32_t v = 0, inc = 0;
     if (tid < TR_DIGITS) {
       v = L.base[p * TR_DIGITS + tid];
@@ -262,9 +397,11 @@ __device__ __forceinline__ void sort_blocked(uint32_t tile, uint32_t start, uint
   }
   const uint32_t nblocks = (n + blk - 1u) / blk;
 #pragma unroll 1
-  for (int p = 0; p < TR_PASSES; p++) {
-    const uint64_t* src = (p & 1) ? ping : pong;  // (pass 0 reads the segment's records instead)
-    uint64_t* dst = (p & 1) ? pong : ping;
+  for (int p = 0; p < passes; p++) {
+    // the last pass writes pong (the lists, one of which may be ping itself, are written from there)
+    const bool to_pong = ((passes - 1 - p) & 1) == 0;
+    const uint64_t* src = to_pong ? ping : pong;  // (pass 0 reads the segment's records instead)
+    uint64_t* dst = to_pong ? pong : ping;
     const int shift = 32 + 8 * p;
 #pragma unroll 1
     for (uint32_t b = 0; b < nblocks; b++) {
@@ -278,7 +415,8 @@ __device__ __forceinline__ void sort_blocked(uint32_t tile, uint32_t start, uint
         const uint32_t i = wave_first + (uint32_t)k * GS_WAVE + (uint32_t)lane;
         rec[k] = ~0ull;
         if ((uint32_t)k < E && i < cnt)
-          rec[k] = p == 0 ? ((uint64_t)records[start + b0 + i].z << 32) | (uint64_t)(b0 + i) : src[start + b0 + i];
+          rec[k] = p == 0 ? ((uint64_t)(records[start + b0 + i].z - dmin) << 32) | (uint64_t)(b0 + i)
+                          : src[start + b0 + i];
       }
       radix_block_pass<WAVES, ITEMS>(rec, E, cnt, shift, L);
 #pragma unroll
@@ -294,36 +432,156 @@ __device__ __forceinline__ void sort_blocked(uint32_t tile, uint32_t start, uint
       if (tid < TR_DIGITS) L.base[p * TR_DIGITS + tid] += L.total[tid];
       // (the next block's pass begins with a barrier of its own before anything reads L.base again)
     }
-    // what this workgroup has written is read back by other threads of it: stores complete, then barrier, then
-    // drop whatever stale lines of the two arrays the CU's vector cache holds
-    __threadfence();
+    // What this workgroup has written is read back by other threads of it, and by nobody else before the kernel
+    // ends: the barrier's workgroup-scope release and acquire is all that takes (the waves of a workgroup share
+    // their CU's vector cache; a device-scope fence here would write the whole L2's dirty lines back every time).
     __syncthreads();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
   }
   const uint64_t* sorted = pong + start;
   const TileRecord* seg = records + start;
-  for (uint32_t i0 = 0; i0 < n; i0 += THREADS) {
-    const uint32_t i = i0 + (uint32_t)tid;
-    if (i >= n) continue;
-    // (emission index of a sorted entry: through its place in the segment)
-    auto entry = [&](uint32_t q) {
-      const uint64_t r = sorted[q];
-      return (r & 0xFFFFFFFF00000000ull) | (uint64_t)seg[(uint32_t)r].y;
-    };
-    // Depth bits of the neighbours decide whether the entry is part of a run; only then are emission indices of
+  // (emission index of a sorted entry: through its place in the segment)
+  auto entry = [&](uint32_t q) {
+    const uint64_t r = sorted[q];
+    return ((r & 0xFFFFFFFF00000000ull) + ((uint64_t)dmin << 32)) | (uint64_t)seg[(uint32_t)r].y;
+  };
+  for (uint32_t i0 = 0; i0 < n; i0 += THREADS * SWEEP) {
+    // Depth bits of the neighbours decide whether an entry is part of a run; only then are emission indices of
     // other entries needed, so the neighbours are compared on the sorted array alone first.
-    const uint64_t r = sorted[i];
-    const uint32_t depth_bits = (uint32_t)(r >> 32);
-    const bool tie = (i > 0u && (uint32_t)(sorted[i - 1u] >> 32) == depth_bits) ||
-                     (i + 1u < n && (uint32_t)(sorted[i + 1u] >> 32) == depth_bits);
-    const uint2 ge = *reinterpret_cast<const uint2*>(seg + (uint32_t)r);
-    if (tie) {
-      emit_list_entry(tile, start, n, i, ge.x, entry, keys, emission, point_list);
-    } else {
-      keys[start + i] = ((uint64_t)tile << 32) | (uint64_t)depth_bits;
-      emission[start + i] = ge.y;
-      point_list[start + i] = ge.x;
+    uint64_t r[SWEEP], before[SWEEP], after[SWEEP];
+    uint2 ge[SWEEP];
+#pragma unroll
+    for (int u = 0; u < SWEEP; u++) {
+      const uint32_t i = i0 + (uint32_t)u * THREADS + (uint32_t)tid;
+      r[u] = i < n ? sorted[i] : 0ull;
+      before[u] = (i < n && i > 0u) ? sorted[i - 1u] : 0ull;
+      after[u] = i + 1u < n ? sorted[i + 1u] : 0ull;
     }
+#pragma unroll
+    for (int u = 0; u < SWEEP; u++) {
+      const uint32_t i = i0 + (uint32_t)u * THREADS + (uint32_t)tid;
+      ge[u] = i < n ? *reinterpret_cast<const uint2*>(seg + (uint32_t)r[u]) : make_uint2(0u, 0u);
+    }
+#pragma unroll
+    for (int u = 0; u < SWEEP; u++) {
+      const uint32_t i = i0 + (uint32_t)u * THREADS + (uint32_t)tid;
+      if (i >= n) continue;
+      const uint32_t key = (uint32_t)(r[u] >> 32);
+      const bool tie = (i > 0u && (uint32_t)(before[u] >> 32) == key) || (i + 1u < n && (uint32_t)(after[u] >> 32) == key);
+      if (tie) {
+        emit_list_entry(tile, start, n, i, ge[u].x, entry, keys, emission, point_list);
+      } else {
+        keys[start + i] = ((uint64_t)tile << 32) | (uint64_t)(key + dmin);
+        emission[start + i] = ge[u].y;
+        point_list[start + i] = ge[u].x;
+      }
+    }
+  }
+}
+
+// A list of more than `blk` records: split by the leading eight bits of (depth bits - smallest) into bins, moved
+// bin by bin into `parted` (any order inside a bin), and runs of consecutive bins that hold at most blk records
+// together are sorted like short lists, inside the CU.  A single bin beyond blk records (many instances within
+// 1/256 of the list's depth range) goes block by block through memory.  Runs of equal depth bits never straddle
+// two bins, so the last step of the sorts still sees them whole.
+template <int WAVES, int ITEMS>
+__device__ __forceinline__ void sort_partitioned(uint32_t tile, uint32_t start, uint32_t n, uint32_t blk,
+                                                 const TileRecord* __restrict__ records, TileRecord* parted,
+                                                 uint64_t* ping, uint64_t* pong, uint64_t* keys, uint32_t* emission,
+                                                 uint32_t* point_list, const TileRadixLds<WAVES, ITEMS>& L) {
+  constexpr int THREADS = WAVES * GS_WAVE;
+  constexpr int SWEEP = 8;  // loads a thread keeps in flight in every sweep over the list
+  const int tid = threadIdx.x, lane = tid & (GS_WAVE - 1), wave = tid / GS_WAVE;
+  uint32_t dmin = 0xFFFFFFFFu, dmax = 0u;
+  for (uint32_t i0 = 0; i0 < n; i0 += THREADS * SWEEP) {
+    uint32_t depth_bits[SWEEP];
+#pragma unroll
+    for (int u = 0; u < SWEEP; u++) {
+      const uint32_t i = i0 + (uint32_t)u * THREADS + (uint32_t)tid;
+      depth_bits[u] = i < n ? records[start + i].z : dmax;
+    }
+#pragma unroll
+    for (int u = 0; u < SWEEP; u++) {
+      const uint32_t i = i0 + (uint32_t)u * THREADS + (uint32_t)tid;
+      if (i < n) {
+        dmin = depth_bits[u] < dmin ? depth_bits[u] : dmin;
+        dmax = depth_bits[u] > dmax ? depth_bits[u] : dmax;
+      }
+    }
+  }
+  workgroup_min_max<WAVES>(dmin, dmax, L.scan, L.total);
+  const uint32_t range = dmax - dmin;
+  const int bits = range != 0u ? 32 - __builtin_clz(range) : 0;
+  const int shift = bits > 8 ? bits - 8 : 0;
+  for (int i = tid; i <= TR_DIGITS; i += THREADS) L.bins[i] = 0u;
+  __syncthreads();
+  for (uint32_t i0 = 0; i0 < n; i0 += THREADS * SWEEP) {
+    uint32_t depth_bits[SWEEP];
+#pragma unroll
+    for (int u = 0; u < SWEEP; u++) {
+      const uint32_t i = i0 + (uint32_t)u * THREADS + (uint32_t)tid;
+      depth_bits[u] = i < n ? records[start + i].z : dmin;
+    }
+#pragma unroll
+    for (int u = 0; u < SWEEP; u++) {
+      const bool valid = i0 + (uint32_t)u * THREADS + (uint32_t)tid < n;
+      const uint32_t d = (depth_bits[u] - dmin) >> shift;
+      // a digit shared by the whole wave would serialise the LDS atomic 64 ways: one lane adds
+      const uint64_t vm = gs_ballot(valid);
+      const uint32_t d0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)d);
+      if (vm != 0ull && gs_ballot(valid && d == d0) == vm && (vm & 1ull)) {
+        if (lane == 0) atomicAdd((uint32_t*)&L.bins[d0], (uint32_t)__popcll(vm));
+      } else if (valid) {
+        atomicAdd((uint32_t*)&L.bins[d], 1u);
+      }
+    }
+  }
+  __syncthreads();
+  {
+    uint32_t v = 0, inc = 0;
+    if (tid < TR_DIGITS) {
+      v = L.bins[tid];
+      inc = tr_wave_inclusive_scan(v, lane);
+      if (lane == GS_WAVE - 1) L.scan[wave] = inc;
+    }
+    __syncthreads();
+    if (tid < TR_DIGITS) {
+      uint32_t before = 0;
+#pragma unroll
+      for (int w = 0; w < TR_DIGITS / GS_WAVE; w++)
+        if (w < wave) before += L.scan[w];
+      L.bins[tid] = before + inc - v;
+      L.first[tid] = before + inc - v;  // where the bin's next record goes
+      if (tid == TR_DIGITS - 1) L.bins[TR_DIGITS] = before + inc;
+    }
+    __syncthreads();
+  }
+  for (uint32_t i0 = 0; i0 < n; i0 += THREADS * SWEEP) {
+    TileRecord r[SWEEP];
+#pragma unroll
+    for (int u = 0; u < SWEEP; u++) {
+      const uint32_t i = i0 + (uint32_t)u * THREADS + (uint32_t)tid;
+      r[u] = i < n ? records[start + i] : make_uint4(0u, 0u, dmin, 0u);
+    }
+#pragma unroll
+    for (int u = 0; u < SWEEP; u++) {
+      const uint32_t i = i0 + (uint32_t)u * THREADS + (uint32_t)tid;
+      if (i < n) parted[start + atomicAdd((uint32_t*)&L.first[(r[u].z - dmin) >> shift], 1u)] = r[u];
+    }
+  }
+  __syncthreads();  // (the moved records are read back by this workgroup only: see sort_blocked)
+  uint32_t g0 = 0;
+  while (g0 < (uint32_t)TR_DIGITS) {
+    const uint32_t first = L.bins[g0];
+    uint32_t g1 = g0 + 1u;
+    while (g1 < (uint32_t)TR_DIGITS && L.bins[g1 + 1u] - first <= blk) g1++;
+    const uint32_t cnt = (uint32_t)__builtin_amdgcn_readfirstlane((int)(L.bins[g1] - first));
+    g0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)g1);
+    if (cnt == 0u) continue;
+    if (cnt <= blk)
+      sort_resident<WAVES, ITEMS>(tile, start + first, cnt, parted, keys, emission, point_list, L);
+    else
+      sort_blocked<WAVES, ITEMS>(tile, start + first, cnt, blk, parted, ping, pong, keys, emission, point_list, L);
+    __syncthreads();
   }
 }
 
@@ -332,12 +590,12 @@ template <int WAVES, int ITEMS>
 __global__ void __launch_bounds__(WAVES * GS_WAVE)
 tile_radix_sort_kernel(const uint32_t* __restrict__ ranges, const uint32_t* __restrict__ tile_list, int step,
                        const uint32_t* __restrict__ list_count, uint32_t count_shift, uint32_t block_limit,
-                       const TileRecord* __restrict__ records, uint64_t* ping, uint64_t* pong,
-                       uint64_t* __restrict__ keys, uint32_t* __restrict__ emission,
-                       uint32_t* __restrict__ point_list, const uint32_t* __restrict__ fits_word) {
+                       const TileRecord* __restrict__ records, TileRecord* parted, uint64_t* ping, uint64_t* pong,
+                       uint64_t* keys, uint32_t* emission, uint32_t* point_list,
+                       const uint32_t* __restrict__ fits_word) {
   extern __shared__ uint64_t s_tile_radix[];
   if (fits_word != nullptr && *fits_word == 0u) return;  // launched ahead of the host's decision: see the scatter
-  const TileRadixLds<WAVES, ITEMS> L(s_tile_radix);
+  const TileRadixLds<WAVES, ITEMS> L((lds_u64*)s_tile_radix);
   const uint32_t count = (*list_count >> count_shift) & 0xFFFFu;
   uint32_t blk = block_limit < (uint32_t)TileRadixLds<WAVES, ITEMS>::BLOCK ? block_limit
                                                                            : (uint32_t)TileRadixLds<WAVES, ITEMS>::BLOCK;
@@ -349,8 +607,8 @@ tile_radix_sort_kernel(const uint32_t* __restrict__ ranges, const uint32_t* __re
     if (n == 0u) continue;
     if (n <= blk)
       sort_resident<WAVES, ITEMS>(t, start, n, records, keys, emission, point_list, L);
-    else
-      sort_blocked<WAVES, ITEMS>(t, start, n, blk, records, ping, pong, keys, emission, point_list, L);
+    else if constexpr (WAVES == 16)
+      sort_partitioned<WAVES, ITEMS>(t, start, n, blk, records, parted, ping, pong, keys, emission, point_list, L);
     __syncthreads();  // the next tile overwrites the LDS the last step has been reading
   }
 }
@@ -363,11 +621,12 @@ int tile_radix_block_records() { return TileRadixLds<16, 16>::BLOCK; }
 // Sorts the tiles of the two lists the ranges kernel of the counting sort made: `mid` lists (ascending from
 // tile_lists[0], their number in the low half of *counts) by workgroups of 8 waves that hold up to 4096 records,
 // `long` lists (descending from tile_lists[T - 1], their number in the high half) by workgroups of 16 waves that
-// hold up to 16384 records and sort longer lists in blocks of block_limit (at most 16384) records through
-// `ping` (which may be `keys`) and `pong` (at least as long as the longest such list's segment end).
+// hold up to 16384 records; a longer list (or one beyond block_limit records, at most 16384) is first split by its
+// leading depth bits into `parted` (16 bytes per instance), and a part that is still too long goes block by block
+// through `ping` (which may be `keys`) and `pong` (8 bytes per instance each).
 int launch_tile_radix_sort(int T, bool mid, bool lng, const uint32_t* ranges, const uint32_t* tile_lists,
-                           const uint32_t* counts, uint32_t block_limit, const void* records, uint64_t* ping,
-                           uint64_t* pong, uint64_t* keys, uint32_t* emission, uint32_t* point_list,
+                           const uint32_t* counts, uint32_t block_limit, const void* records, void* parted,
+                           uint64_t* ping, uint64_t* pong, uint64_t* keys, uint32_t* emission, uint32_t* point_list,
                            const uint32_t* fits_word, hipStream_t stream) {
   if (T <= 0) return 0;
   // more than 64 KB of dynamic LDS has to be asked for, once per device
@@ -388,12 +647,12 @@ int launch_tile_radix_sort(int T, bool mid, bool lng, const uint32_t* ranges, co
   const uint32_t mid_block = Mid::BLOCK;
   if (mid)
     hipLaunchKernelGGL((tile_radix_sort_kernel<8, 8>), dim3(T < 2048 ? T : 2048), dim3(8 * GS_WAVE), mid_lds, stream,
-                       ranges, tile_lists, 1, counts, 0u, mid_block, (const TileRecord*)records, ping, pong, keys,
-                       emission, point_list, fits_word);
+                       ranges, tile_lists, 1, counts, 0u, mid_block, (const TileRecord*)records, (TileRecord*)parted,
+                       ping, pong, keys, emission, point_list, fits_word);
   if (lng)
     hipLaunchKernelGGL((tile_radix_sort_kernel<16, 16>), dim3(T < 1024 ? T : 1024), dim3(16 * GS_WAVE), long_lds,
                        stream, ranges, tile_lists + (T - 1), -1, counts, 16u, block_limit, (const TileRecord*)records,
-                       ping, pong, keys, emission, point_list, fits_word);
+                       (TileRecord*)parted, ping, pong, keys, emission, point_list, fits_word);
   return 0;
 }
 
