@@ -680,6 +680,11 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
   if (bucketed) {
     if (lists_by_tile(A, longest, radix_tiles, false)) return 1;
   } else {
+    if (R > sort_max_pairs()) {
+      set_error("gs_render_forward: %lld instances in a view that takes the radix sort over all keys, which takes "
+                "at most 2^30-2", (long long)R);
+      return 1;
+    }
     const int end_bit = sort_end_bit(width, height);
     // The sort carries each instance's index in emission order as its payload (the backward pass files
     // per-instance gradients under it); the Gaussian ids of the sorted list are gathered afterwards.
@@ -1144,10 +1149,13 @@ int gs_duplicate_with_keys(int P, int width, int height, const float* means2D, c
 
 size_t gs_sort_workspace_bytes(int64_t n) { return sort_temp_bytes(n) + 256; }
 
+int64_t gs_sort_max_pairs(void) { return sort_max_pairs(); }
+
 int gs_sort_pairs_u64(int64_t n, uint64_t* keys_in, uint64_t* keys_out, uint32_t* vals_in, uint32_t* vals_out,
                       int end_bit, void* workspace, size_t workspace_bytes, gs_stream_t stream_) {
   hipStream_t stream = (hipStream_t)stream_;
   GS_REQUIRE(n >= 0 && end_bit >= 1 && end_bit <= 64, "gs_sort_pairs_u64: bad n or end_bit");
+  GS_REQUIRE(n <= sort_max_pairs(), "gs_sort_pairs_u64: more than 2^30-2 pairs");
   if (n == 0) return 0;
   GS_REQUIRE(keys_in && keys_out && vals_in && vals_out && workspace, "gs_sort_pairs_u64: null pointer");
   GS_REQUIRE(workspace_bytes >= gs_sort_workspace_bytes(n), "gs_sort_pairs_u64: workspace too small");
@@ -1192,6 +1200,7 @@ int gs_sort_pairs_u32(int64_t n, uint32_t* keys_in, uint32_t* keys_out, uint32_t
                       int end_bit, void* workspace, size_t workspace_bytes, gs_stream_t stream_) {
   hipStream_t stream = (hipStream_t)stream_;
   GS_REQUIRE(n >= 0 && end_bit >= 1 && end_bit <= 32, "gs_sort_pairs_u32: bad n or end_bit");
+  GS_REQUIRE(n <= sort_max_pairs(), "gs_sort_pairs_u32: more than 2^30-2 pairs");
   if (n == 0) return 0;
   GS_REQUIRE(keys_in && keys_out && vals_in && vals_out && workspace, "gs_sort_pairs_u32: null pointer");
   GS_REQUIRE(workspace_bytes >= gs_sort_workspace_bytes(n), "gs_sort_pairs_u32: workspace too small");

@@ -189,6 +189,7 @@ int launch_tile_ranges(int64_t L, const uint64_t* keys_sorted, int T, uint32_t* 
 
 // ---- radix sort (stable, LSD, 8-bit digits) ----
 size_t sort_temp_bytes(int64_t n);
+int64_t sort_max_pairs();  // 2^30 - 2
 // device word of a sort's workspace that is nonzero after a sort in which a bounded wait of the look-back ran out
 // (the order of the output is then not to be trusted)
 const uint32_t* sort_error_word(const void* temp);

@@ -412,7 +412,7 @@ template <typename K>
 int sort_pairs_impl(int64_t n, K* keys_a, K* keys_b, uint32_t* vals_a, uint32_t* vals_b, int end_bit, void* temp,
                     hipStream_t stream) {
   if (n <= 0) return 0;
-  if (n >= (int64_t)VALUE_MASK) {
+  if (n > sort_max_pairs()) {
     set_error("radix sort: %lld pairs exceed the supported 2^30-2", (long long)n);
     return 1;
   }
@@ -455,6 +455,9 @@ int sort_pairs_impl(int64_t n, K* keys_a, K* keys_b, uint32_t* vals_a, uint32_t*
 }  // namespace
 
 size_t sort_temp_bytes(int64_t n) { return sort_layout(n).total_bytes; }
+
+// A look-back word carries a 30-bit count beside its two flag bits, and a count can be the whole input.
+int64_t sort_max_pairs() { return (int64_t)VALUE_MASK - 1; }
 
 size_t sort_error_word_offset() { return (size_t)(MAX_PASSES * RADIX + MAX_PASSES) * sizeof(uint32_t); }
 const uint32_t* sort_error_word(const void* temp) {

@@ -59,6 +59,7 @@ _SIGNATURES = {
     "gs_inclusive_sum_static": (_i, [_i64, _vp, _vp, _vp]),
     "gs_duplicate_with_keys": (_i, [_i, _i, _i] + [_vp] * 8),
     "gs_sort_workspace_bytes": (_sz, [_i64]),
+    "gs_sort_max_pairs": (_i64, []),
     "gs_sort_status": (_i, [_vp, _vp]),
     "gs_sort_workspace_error_offset": (_sz, []),
     "gs_sort_check_async": (_i, [_vp, _vp]),

@@ -152,7 +152,10 @@ typedef struct gs_render_result {
  * out_observe (P) int32 is cleared by the call
  * (the reference's binding allocates it zeroed, rasterize_points.cu:305) and then counted;
  * n_render / n_consider / n_contrib are (tiles) int32, fully written.
- * *num_rendered (host) receives the instance count R.
+ * *num_rendered (host) receives the instance count R.  A view may have up to 2^31-2 instances (positions are
+ * 32-bit, as in the reference, whose prefix sum wraps beyond that: here the call fails instead); a view that takes
+ * the radix sort over all keys (a grid of more than 30000 tiles, or tile_sort_small_limit = 0) up to 2^30-2, the
+ * capacity of that sort (gs_sort_max_pairs).
  * out_max_weight_depth (H*W, optional, NULL to skip) has no counterpart in the reference: per pixel the view-space
  * depth (depths[g]) of the Gaussian that blends with the largest weight alpha * T, the front-most among equals, 0
  * where nothing blends; asking for it changes no other output.
@@ -365,7 +368,9 @@ int gs_duplicate_with_keys(int P, int width, int height, const float* means2D, c
 
 /* cub::DeviceRadixSort::SortPairs on bits [0, end_bit) (CR/rasterizer_impl.cu:679-684,
  * KNN/simple_knn.cu:210-213): stable.  The input arrays are clobbered; the
- * sorted pairs land in keys_out / vals_out. */
+ * sorted pairs land in keys_out / vals_out.  At most gs_sort_max_pairs() = 2^30-2 pairs (the look-back words of a
+ * pass carry 30-bit counts beside their two flag bits); more is refused with an error before anything is launched. */
+int64_t gs_sort_max_pairs(void);
 size_t gs_sort_workspace_bytes(int64_t n);
 /* No counterpart in the reference.  A pass of the sort waits, with a bounded number of polls, for the digit counts
  * of earlier tiles; if a wait ever ran out the sort sets a word in its workspace (at byte

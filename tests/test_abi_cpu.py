@@ -55,6 +55,30 @@ def test_state_layouts_are_aligned_and_disjoint():
     assert gn.lib.gs_knn_workspace_bytes(1000) > 1000 * 16
 
 
+def test_layouts_and_capacities_at_the_instance_limit():
+    """A view may hold up to 2^31-2 instances: at that count every array of the binning buffer still starts
+    behind the one before it (no offset is formed in 32 bits), the per-instance workspaces are sized in 64 bits,
+    and the radix sort over all keys, whose capacity is 2^30-2 pairs, refuses more before launching anything."""
+    import gsrast_native as gn
+    R = 2 ** 31 - 2
+    sz = [C.c_size_t() for _ in range(5)]
+    assert gn.lib.gs_binning_state_layout(R, 1920, 1080, *[C.byref(s) for s in sz]) == 0
+    pl, k, plu, ku, tot = [s.value for s in sz]
+    offs = sorted([(pl, 4 * R), (k, 8 * R), (plu, 4 * R), (ku, 8 * R)])
+    for (o1, l1), (o2, _) in zip(offs, offs[1:]):
+        assert o1 + l1 <= o2 and o1 % 256 == 0
+    # point list, keys, 16-byte records, emission indices, block hits, 24 bytes of per-tile radix sort scratch
+    assert tot >= (4 + 8 + 16 + 4 + 2 + 24) * R
+    assert gn.lib.gs_render_backward_workspace_bytes(R) == 64 * R + 256
+    assert gn.lib.gs_sort_max_pairs() == 2 ** 30 - 2
+    assert gn.lib.gs_sort_workspace_bytes(2 ** 30 - 2) > 5 * 512 * 4 * ((2 ** 30 - 2) // 4096)
+    one = C.c_void_p(256)  # never dereferenced: the count is refused first
+    assert gn.lib.gs_sort_pairs_u64(2 ** 30 - 1, one, one, one, one, 44, one, 1 << 40, None) != 0
+    assert "2^30-2" in gn.last_error()
+    assert gn.lib.gs_sort_pairs_u32(2 ** 31, one, one, one, one, 32, one, 1 << 40, None) != 0
+    assert "2^30-2" in gn.last_error()
+
+
 def test_argument_validation_without_a_gpu():
     import gsrast_native as gn
     assert gn.lib.gs_preprocess_forward(*([None] * 8), 10, 3, 16, 0, 480, *([None] * 5), 1.0, None, None, None, 0.5, 0.5,

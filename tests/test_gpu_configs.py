@@ -156,7 +156,7 @@ def _buffer_views(gn, geomB, binB, imgB, P, R, W, Hh, T):
     return point_list, keys, tiles_touched, final_T
 
 
-def _full_size_view(H, d, cam, view, render_geo=True, args=None):
+def _full_size_view(H, d, cam, view, render_geo=True, args=None, scale_modifier=1.0):
     """One view of a full-size configuration, forward and backward, checked through properties: list order and
     counts, image ranges, repeatability bit for bit forward, linearity and exact zeros backward.  Returns what the
     caller's later stages use."""
@@ -172,8 +172,8 @@ def _full_size_view(H, d, cam, view, render_geo=True, args=None):
     T = gx * gy
     cl = torch.ones(gy, gx, dtype=torch.bool, device=DEV)
     _, means2D, depths, radii, cov3D, co, rgb, clamped = _C.preprocess_gaussians(
-        d["means3D"], d["scales"], d["rotations"], d["shs"], d["opacities"], 1.0, vm, pm, cam.tanfovx, cam.tanfovy,
-        Hh, W, 3, cp, False, False, args)
+        d["means3D"], d["scales"], d["rotations"], d["shs"], d["opacities"], scale_modifier, vm, pm, cam.tanfovx,
+        cam.tanfovy, Hh, W, 3, cp, False, False, args)
     am = _C.build_all_map(d["means3D"], d["scales"], d["rotations"], vm, cp)
     bg = torch.zeros(3, device=DEV)
 
@@ -236,8 +236,8 @@ def _full_size_view(H, d, cam, view, render_geo=True, args=None):
         assert float(t[dead].abs().max()) == 0.0, tag
     assert bool((b1[1][:, :2] * (1 + 1e-3) + 1e-6 >= b1[0].abs()).all()) and float(b1[1][:, 2].abs().max()) == 0.0, tag
     pb = _C.preprocess_gaussians_backward(radii, cov3D, clamped, d["means3D"], d["scales"], d["rotations"], d["shs"],
-                                          1.0, vm, pm, cam.tanfovx, cam.tanfovy, Hh, W, 3, cp, b1[0], b1[2], b1[3],
-                                          R, False, args)
+                                          scale_modifier, vm, pm, cam.tanfovx, cam.tanfovy, Hh, W, 3, cp, b1[0], b1[2],
+                                          b1[3], R, False, args)
     for t in pb:
         assert bool(torch.isfinite(t).all()), tag
         assert float(t[dead].abs().max()) == 0.0, tag
@@ -280,6 +280,49 @@ def test_config3_full_size_all_views_forward_and_backward_with_geometry(H):
         r = _full_size_view(H, d, cam, v)
         longest = max(longest, r["longest"])
     assert longest > 8192  # the regime in which a list no longer fits one workgroup's sort
+
+
+@pytest.mark.timeout(900)
+def test_config3_hundred_million_instances(H):
+    """The regime BASELINE config 3 names (lists of more than 5000 Gaussians per tile, more than 100 M keys), which
+    its own generator stays a factor 12 below: the street-level view with the most instances, its Gaussians enlarged
+    by the rasterizer's scale modifier until the view has at least 10^8 instances; forward and backward with the
+    geometry maps through the property checks of every full-size view.  Positions, layouts and record indices
+    are 32-bit up to 2^31-2 instances; this view exercises them at a twentieth of that."""
+    import gsrast_native as gn
+    from diff_gaussian_rasterization import _C
+    d, cams = _load(3)
+    cam = cams[6]
+    W, Hh = cam.image_width, cam.image_height
+    P = d["means3D"].shape[0]
+    vm, pm, cp = cam.world_view_transform.to(DEV), cam.full_proj_transform.to(DEV), cam.camera_center.to(DEV)
+    gx, gy = (W + 15) // 16, (Hh + 15) // 16
+    cl = torch.ones(gy * gx, dtype=torch.bool, device=DEV)
+    tt = torch.empty(P, dtype=torch.int32, device=DEV)
+    mod, R = 2.0, 0
+    while True:
+        _, means2D, depths, radii, _, _, _, _ = _C.preprocess_gaussians(
+            d["means3D"], d["scales"], d["rotations"], d["shs"], d["opacities"], mod, vm, pm, cam.tanfovx, cam.tanfovy,
+            Hh, W, 3, cp, False, False, {})
+        gn.check(gn.lib.gs_tile_count(P, W, Hh, H.ptr(radii), H.ptr(means2D), H.ptr(cl), H.ptr(tt), H.stream()),
+                 "gs_tile_count")
+        R = int(tt.to(torch.int64).sum())
+        if R >= 100_000_000:
+            break
+        assert mod < 40.0, (mod, R)
+        mod *= 1.25 if R > 50_000_000 else 1.5
+    del means2D, depths, radii, tt
+    assert R < 400_000_000, (mod, R)  # (a few tens of GB of buffers at most)
+    print(f"scale modifier {mod:.3f}: {R} instances", flush=True)
+    gn.stage_timing(True)
+    r = _full_size_view(H, d, cam, 6, scale_modifier=mod)
+    torch.cuda.synchronize()
+    gn.stage_timing(False)
+    st = gn.stage_timing_collect()
+    assert r["R"] == R and r["longest"] > 16384
+    print("stages (ms per launch, launches): " +
+          ", ".join(f"{k} {tot / max(cnt, 1):.3f} x{cnt}" for k, (tot, cnt) in st.items()), flush=True)
+    print(f"longest list {r['longest']}", flush=True)
 
 
 @pytest.mark.timeout(1100)
