@@ -286,8 +286,7 @@ int gs_preprocess_forward(float* means2D, float* depths, int* radii, float* cov3
   (void)prefiltered;
   GS_REQUIRE(P >= 0 && width > 0 && height > 0, "gs_preprocess_forward: bad sizes");
   if (P == 0) return 0;
-  GS_REQUIRE(means2D && depths && radii && cov3D && conic_opacity && rgb && clamped,
-             "gs_preprocess_forward: null output");
+  GS_REQUIRE(means2D && depths && radii && conic_opacity && rgb && clamped, "gs_preprocess_forward: null output");
   GS_REQUIRE(means3D && scales && rotations && opacities && viewmatrix && projmatrix,
              "gs_preprocess_forward: null input");
   const bool sh_mode = shs != nullptr && M > 0;
@@ -319,8 +318,9 @@ int gs_preprocess_backward(const int* radii, const float* cov3D, const uint8_t* 
                            float* dL_dopacity, int debug, const float* dcolor_ddir, gs_stream_t stream) {
   GS_REQUIRE(P >= 0 && width > 0 && height > 0, "gs_preprocess_backward: bad sizes");
   if (P == 0) return 0;
-  GS_REQUIRE(radii && cov3D && means3D && viewmatrix && projmatrix && dL_dmean2D && dL_dconic_opacity && dL_dmean3D,
+  GS_REQUIRE(radii && means3D && viewmatrix && projmatrix && dL_dmean2D && dL_dconic_opacity && dL_dmean3D,
              "gs_preprocess_backward: null pointer");
+  GS_REQUIRE(cov3D || (scales && rotations), "gs_preprocess_backward: without cov3D, scales and rotations are needed");
   GS_REQUIRE(mean2D_stride == 2 || mean2D_stride == 3, "gs_preprocess_backward: mean2D_stride must be 2 or 3");
   GS_REQUIRE((scales == nullptr) == (rotations == nullptr), "gs_preprocess_backward: scales and rotations go together");
   GS_REQUIRE(!scales || (dL_dscale && dL_drot), "gs_preprocess_backward: null scale/rotation gradient");

@@ -382,10 +382,12 @@ preprocess_fwd_kernel(int P, int D, int M, const float* __restrict__ means, cons
   bool in_front;
   const bool ok = geom_forward(mean, sc, mod, q, nullptr, cam, W, H, tanx, tany, fx, fy, gx, gy, cov6, in_front, g);
   if (live) {
-    float2* c6v = reinterpret_cast<float2*>(cov3D + 6 * (size_t)i);  // 24-byte rows are 8-byte aligned
-    c6v[0] = make_float2(cov6[0], cov6[1]);
-    c6v[1] = make_float2(cov6[2], cov6[3]);
-    c6v[2] = make_float2(cov6[4], cov6[5]);
+    if (cov3D != nullptr) {  // (a caller that hands scales and rotations to the backward pass needs no copy)
+      float2* c6v = reinterpret_cast<float2*>(cov3D + 6 * (size_t)i);  // 24-byte rows are 8-byte aligned
+      c6v[0] = make_float2(cov6[0], cov6[1]);
+      c6v[1] = make_float2(cov6[2], cov6[3]);
+      c6v[2] = make_float2(cov6[4], cov6[5]);
+    }
     radii[i] = ok ? g.radius : 0;
     depths[i] = ok ? g.depth : 0.f;
     means2D[i] = ok ? make_float2(g.px, g.py) : make_float2(0.f, 0.f);
@@ -574,10 +576,17 @@ preprocess_bwd_kernel(int P, int D, int M, const float* __restrict__ means, cons
     load_cam(Vg, PMg, camg, cam);
     const float mean[3] = {means[3 * (size_t)i], means[3 * (size_t)i + 1], means[3 * (size_t)i + 2]};
     float c6[6];
-    {
+    if (cov3D != nullptr) {
       const float2* c6v = reinterpret_cast<const float2*>(cov3D + 6 * (size_t)i);
       const float2 a = c6v[0], b = c6v[1], c = c6v[2];
       c6[0] = a.x; c6[1] = a.y; c6[2] = b.x; c6[3] = b.y; c6[4] = c.x; c6[5] = c.y;
+    } else {
+      // the forward pass's own operations on the same inputs: the same bits it would have stored
+      const float sc[3] = {scales[3 * (size_t)i], scales[3 * (size_t)i + 1], scales[3 * (size_t)i + 2]};
+      const float4 q4 = reinterpret_cast<const float4*>(rots)[i];
+      const float q[4] = {q4.x, q4.y, q4.z, q4.w};
+      M3 unused_m, unused_r;
+      cov3d_from_scale_rot(sc, mod, q, c6, &unused_m, &unused_r);
     }
     Cov2DCtx cc;
     cov2d(mean, h_x, h_y, tanx, tany, c6, cam.V, cc);

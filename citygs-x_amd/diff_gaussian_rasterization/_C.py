@@ -86,11 +86,13 @@ def preprocess_gaussians(means3D, scales, rotations, sh, opacity, scale_modifier
 
 def preprocess_gaussians_ex(means3D, scales, rotations, sh, opacity, scale_modifier, viewmatrix, projmatrix, tan_fovx,
                             tan_fovy, image_height, image_width, degree, campos, prefiltered, debug, args,
-                            want_direction_derivative=False):
+                            want_direction_derivative=False, want_cov3D=True):
     """preprocess_gaussians plus what the reference's tuple has no slot for: returns (tuple, dcolor_ddir).  With
     want_direction_derivative (and SH colours) dcolor_ddir is the (P,3,3) derivative of every surviving Gaussian's
     colour with respect to the unit view direction; handed to preprocess_gaussians_backward it replaces the
-    coefficients there (same gradients, and the backward pass does not read the 192-byte rows).  Otherwise None."""
+    coefficients there (same gradients, and the backward pass does not read the 192-byte rows).  Otherwise None.
+    want_cov3D=False leaves the cov3D slot of the tuple None: preprocess_gaussians_backward, given None, forms the
+    covariances again from scales and rotations (the same bits), and neither pass moves the 24 bytes per Gaussian."""
     if means3D.ndimension() != 2 or means3D.size(1) != 3:
         raise RuntimeError("means3D must have dimensions (num_points, 3)")
     means3D = _f32c(means3D, "means3D")
@@ -104,7 +106,7 @@ def preprocess_gaussians_ex(means3D, scales, rotations, sh, opacity, scale_modif
     means2D = torch.empty(P, 2, **f32)
     depths = torch.empty(P, **f32)
     radii = torch.empty(P, dtype=torch.int32, device=dev)
-    cov3D = torch.empty(P, 6, **f32)
+    cov3D = torch.empty(P, 6, **f32) if want_cov3D else None
     conic_opacity = torch.empty(P, 4, **f32)
     rgb = torch.empty(P, 3, **f32)
     clamped = torch.empty(P, 3, dtype=torch.bool, device=dev)
@@ -153,7 +155,8 @@ def preprocess_gaussians_backward(radii, cov3D, clamped, means3D, scales, rotati
     shc = _f32c(sh, "sh") if sh_mode else None
     with torch.cuda.device(dev):
         _n.check(_lib.gs_preprocess_backward(
-            _ptr(radii.contiguous()), _ptr(cov3D.contiguous()), _ptr(clamped.contiguous()), P, int(degree), M,
+            _ptr(radii.contiguous()), _ptr(cov3D.contiguous() if cov3D is not None else None),
+            _ptr(clamped.contiguous()), P, int(degree), M,
             int(image_width), int(image_height), _ptr(means3D), _ptr(scales), _ptr(rotations), _ptr(shc),
             float(scale_modifier), _ptr(vm), _ptr(pm), _ptr(cp), float(tan_fovx), float(tan_fovy), _ptr(g2),
             int(g2.shape[1]), _ptr(gco), _ptr(gcol), _ptr(dL_dmeans3D), None, _ptr(dL_dscales), _ptr(dL_drotations),

@@ -50,7 +50,9 @@ class _PreprocessGaussians(torch.autograd.Function):
         (num_rendered, means2D, depths, radii, cov3D, conic_opacity, rgb, clamped), ddir = _C.preprocess_gaussians_ex(
             means3D, scales, rotations, sh, opacities, rs.scale_modifier, rs.viewmatrix, rs.projmatrix, rs.tanfovx,
             rs.tanfovy, rs.image_height, rs.image_width, rs.sh_degree, rs.campos, rs.prefiltered, rs.debug, cuda_args,
-            want_direction_derivative=any(ctx.needs_input_grad[:5]))
+            want_direction_derivative=any(ctx.needs_input_grad[:5]), want_cov3D=False)
+        # (cov3D is None: the backward kernel forms the covariances again from scales and rotations, which it reads
+        # anyway, instead of both passes moving 24 bytes per Gaussian)
         ctx.raster_settings = rs
         ctx.cuda_args = cuda_args
         ctx.num_rendered = num_rendered
@@ -89,12 +91,15 @@ def preprocess_gaussians(means3D, scales, rotations, sh, opacities, raster_setti
 
 # ------------------------------------------------------------------- render --
 
-# What the last view of a given shape needed, (instances, longest list) keyed by (Gaussians, height, width, device):
-# the next view of that shape is launched without waiting for its instance count, on buffers sized for these figures
-# plus a margin (a training loop renders thousands of similar views).  Only the time depends on it, never a result;
-# a stale or missing entry costs one ordinary call.
+# What the last view of a given image size needed, (instances, longest list) keyed by (height, width, device): the
+# next view of that size is launched without waiting for its instance count, on buffers sized for these figures plus
+# a margin (a training loop renders thousands of similar views; the number of Gaussians changes at every
+# densification, so it is not part of the key).  Only the time depends on it, never a result; a stale or missing
+# entry costs one ordinary call.  A handful of image sizes at most are alive in a run: the oldest entry goes
+# when there are more than _MAX_EXPECTATIONS.
 _expectations = {}
 _MARGIN = 1.25
+_MAX_EXPECTATIONS = 16
 
 
 def _expectation(key):
@@ -112,6 +117,13 @@ def _expectation(key):
     return int(instances * _MARGIN) + 65536, (cap if cap <= 2048 else 0)
 
 
+def _remember(key, instances, longest):
+    _expectations.pop(key, None)  # (re-inserted at the end: the dict keeps insertion order)
+    _expectations[key] = (instances, longest)
+    while len(_expectations) > _MAX_EXPECTATIONS:
+        _expectations.pop(next(iter(_expectations)))
+
+
 class _RenderGaussians(torch.autograd.Function):
     @staticmethod
     def forward(ctx, means2D, means2D_abs, conic_opacity, rgb, all_maps, depths, radii, compute_locally,
@@ -119,7 +131,7 @@ class _RenderGaussians(torch.autograd.Function):
         rs = raster_settings
         avoid = bool(cuda_args.get("avoid_pixel_all2all", False)) if cuda_args is not None else False
         mask = extended_compute_locally if avoid else compute_locally
-        key = (means2D.shape[0], rs.image_height, rs.image_width, means2D.device)
+        key = (rs.image_height, rs.image_width, means2D.device)
         expected_instances, expected_longest = _expectation(key)
         ((num_rendered, color, n_render, n_consider, n_contrib, out_observe, out_all_map, out_plane_depth, geomBuffer,
           binningBuffer, imgBuffer), info) = _C.render_gaussians_ex(
@@ -127,7 +139,11 @@ class _RenderGaussians(torch.autograd.Function):
             rs.campos, rs.tanfovx, rs.tanfovy, all_maps, rs.render_geo, rs.debug, cuda_args,
             expected_instances=expected_instances, expected_longest_list=expected_longest)
         if means2D.shape[0] > 0:
-            _expectations[key] = (num_rendered, info["longest_list"])
+            _remember(key, num_rendered, info["longest_list"])
+        if isinstance(cuda_args, dict) and isinstance(cuda_args.get("stats_collector"), dict):
+            # (beside the reference's timing keys: whether this view's list kernels ran ahead of its instance count)
+            cuda_args["stats_collector"]["launched_ahead"] = info["launched_ahead"]
+            cuda_args["stats_collector"]["num_rendered"] = num_rendered
         ctx.binning_capacity = info["binning_capacity"]
         ctx.raster_settings = rs
         ctx.cuda_args = cuda_args

@@ -60,7 +60,8 @@ int gs_visible_filter(int P, int M, int width, int height, const float* means3D,
  * CR/rasterizer_impl.cu:336-425).  Shapes: means2D (P,2), depths (P), radii
  * (P) int32, cov3D (P,6), conic_opacity (P,4), rgb (P,3), clamped (P,3) bytes.
  * Every output element is written (zeros for culled Gaussians), so outputs
- * need no initialisation.  shs == NULL or M == 0: colour is left zero, as in
+ * need no initialisation.  cov3D may be NULL (not stored): gs_preprocess_backward
+ * then forms the covariances again from scales and rotations.  shs == NULL or M == 0: colour is left zero, as in
  * the reference (its SH call is commented out, CR/forward.cu:243-250);
  * otherwise shs is (P,M,3) and rgb/clamped follow CR/forward.cu:21-72 at
  * degree D.  tiles_touched (P) uint32 is optional (NULL to skip): the tile
@@ -88,7 +89,9 @@ int gs_preprocess_forward(float* means2D, float* depths, int* radii, float* cov3
  * dL_dmean3D (P,3), dL_dscale (P,3), dL_drot (P,4), dL_dopacity (P) are fully
  * written.  dL_dsh: NULL in reference-compatible mode; (P,M,3) in SH mode,
  * where dL_dcolor (P,3) and clamped are read.  dL_dcov3D (P,6) is optional
- * (NULL: kept in registers).  dcolor_ddir: NULL, or what gs_preprocess_forward
+ * (NULL: kept in registers).  cov3D: what gs_preprocess_forward stored, or NULL with
+ * scales and rotations given (the covariances are then formed again, the same bits).
+ * dcolor_ddir: NULL, or what gs_preprocess_forward
  * left for the same inputs and camera; shs is then not read and may be NULL.
  * Same results either way, bit for bit. */
 int gs_preprocess_backward(const int* radii, const float* cov3D, const uint8_t* clamped, int P, int D, int M,

@@ -368,12 +368,17 @@ def test_the_operator_launches_ahead_from_the_second_view_on():
         return [color, n_render, n_consider, n_contrib, obs, oam, opd] + [leaf[k].grad for k in sorted(leaf)]
 
     first = run()
-    key = (25_000, H, W, torch.device(DEV))
+    key = (H, W, torch.device(DEV))
     assert key in dgr._expectations and dgr._expectation(key)[0] > dgr._expectations[key][0]
     for _ in range(2):
         again = run()
         for a, b in zip(first, again):
             assert torch.equal(a, b)
+    # the table of expectations stays small whatever sizes come by
+    for k in range(3 * dgr._MAX_EXPECTATIONS):
+        dgr._remember((100 + k, 100, torch.device(DEV)), 1000, 100)
+    assert len(dgr._expectations) == dgr._MAX_EXPECTATIONS and (100, 100, torch.device(DEV)) not in dgr._expectations
+    dgr._expectations.clear()
 
 
 def test_debug_mode_gives_the_same_results_by_every_route():

@@ -255,6 +255,18 @@ def test_preprocess_backward(H, orc, cfg, P, sh_mode):
         torch.cuda.synchronize()
         for k in o:
             assert torch.equal(o[k], o2[k]), k
+    # without the stored covariances (formed again from scales and rotations): the same bits
+    o3 = {k: torch.full_like(v, 33.0) for k, v in o.items()}
+    H.gn.check(H.lib.gs_preprocess_backward(
+        H.ptr(t_radii), None, H.ptr(t_clamped), P, 3, 16 if sh_mode else 0, W, Hh, H.ptr(gd["means3D"]),
+        H.ptr(gd["scales"]), H.ptr(gd["rotations"]), H.ptr(gd["shs"]) if (sh_mode and not saved) else None, 1.0,
+        H.ptr(V), H.ptr(PM), H.ptr(cp), cam.tanfovx, cam.tanfovy, H.ptr(t_g2), 2, H.ptr(t_gco), H.ptr(t_gcol),
+        H.ptr(o3["dL_dmeans3D"]), H.ptr(o3["dL_dcov3D"]), H.ptr(o3["dL_dscales"]), H.ptr(o3["dL_drotations"]),
+        H.ptr(o3["dL_dsh"]) if sh_mode else None, H.ptr(o3["dL_dopacity"]), 1, H.ptr(ddir) if saved else None,
+        H.stream()), "gs_preprocess_backward")
+    torch.cuda.synchronize()
+    for k in o:
+        assert torch.equal(o[k], o3[k]), k
     keys = ["dL_dmeans3D", "dL_dcov3D", "dL_dscales", "dL_drotations", "dL_dopacity"] + (["dL_dsh"] if sh_mode else [])
     for k in keys:
         a, r = o[k].cpu().numpy(), ref[k]
