@@ -357,7 +357,9 @@ int gs_inclusive_sum(int64_t n, const uint32_t* in, uint32_t* out, void* workspa
  * no workspace argument: the scan's spine (one word per 2048 elements) lives in a static device array inside the
  * library, 256 KiB, which every GPU the library runs on holds until the process ends.  n may be at most
  * gs_inclusive_sum_static_max() = 2^27 elements; a larger n is refused with an error.  The call allocates and
- * frees nothing (the first call on a device looks the array's device address up).  Every call on a GPU shares
+ * frees nothing.  The first call on a device looks the array's device address up (a mutex, hipGetDevice and
+ * hipGetSymbolAddress: not a sequence to record into a graph), so make one call per device outside any capture
+ * before relying on it there.  Every call on a GPU shares
  * that GPU's array: the call itself writes every word it later reads, so nothing has to be cleared between
  * calls, but calls that overlap on one GPU (two streams, two threads) race on it and must be serialised by
  * the caller.  in and out may be the same array. */
@@ -427,7 +429,8 @@ int gs_render_tiles_backward(int P, int width, int height, float tan_fovx, float
                              float* instance_grads, float* dL_dmean2D, float* dL_dmean2D_abs,
                              float* dL_dconic_opacity, float* dL_dcolor, float* dL_dall_map, gs_stream_t stream);
 
-/* Diagnostic with no counterpart in the reference: runs the two cross-lane
+/* A test hook, not part of the path (no counterpart in the reference, nothing in the library calls it; it is
+ * exported so that the test suite can check the inline-assembly reductions on their own): runs the two cross-lane
  * reductions of the blend kernels on one 64-lane wave.  in is (64,16) floats;
  * out_wave (16) receives the sums over all 64 lanes, out_rows (4,16) the sums
  * over each 16-lane row.  Synchronises the stream. */

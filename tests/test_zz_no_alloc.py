@@ -22,15 +22,22 @@ def _both(H, x):
     H.gn.check(H.lib.gs_inclusive_sum(n, H.ptr(xin), H.ptr(ref), H.ptr(ws), nb, H.stream()), "gs_inclusive_sum")
     out = torch.full((n,), -2, dtype=torch.int32, device=H.DEV)
     torch.cuda.synchronize()
-    before = torch.cuda.memory_allocated()
+    # free device memory as the driver sees it (an allocation inside the library would not show in torch's own
+    # counters), and torch's counters for the wrapper side
+    free_before, before = torch.cuda.mem_get_info()[0], torch.cuda.memory_allocated()
     H.gn.check(H.lib.gs_inclusive_sum_static(n, H.ptr(xin), H.ptr(out), H.stream()), "gs_inclusive_sum_static")
     torch.cuda.synchronize()
     assert torch.cuda.memory_allocated() == before
+    assert torch.cuda.mem_get_info()[0] == free_before
     return H.np_u32(ref), H.np_u32(out)
 
 
 def test_static_scan_matches_workspace_scan_twice_in_a_row(H):
     rng = np.random.default_rng(7)
+    # (the first call on a device looks the static array's address up; the calls measured below come after it)
+    t0 = H.as_u32(np.array([1, 2, 3], np.uint32))
+    H.gn.check(H.lib.gs_inclusive_sum_static(3, H.ptr(t0), H.ptr(t0), H.stream()), "gs_inclusive_sum_static")
+    torch.cuda.synchronize()
     # two calls in a row on the same GPU (they share the static array), the second with a smaller input
     for n in (3_000_001, 70_003):
         x = rng.integers(0, 9, n, dtype=np.uint32)
