@@ -89,6 +89,10 @@ def parse():
                          "previous, different view needed), and report the share of views whose list kernels ran "
                          "ahead of the instance count, the time per view, and the time per view when no view may "
                          "run ahead (the cost of a miss)")
+    ap.add_argument("--with-all-map", action="store_true",
+                    help="with --all-views: build the geometry channels inside every step with the fused op, forward "
+                         "and backward, linked to the preprocess outputs as a caller links them "
+                         "(build_all_map(..., blend_records_of=means2D)), instead of preparing them once per camera")
     ap.add_argument("--vary-gaussians", action="store_true",
                     help="with --interleave: every other step renders only the first 90 %% of the Gaussians, as the "
                          "count changes at every densification of a training run")
@@ -146,7 +150,7 @@ def all_views(args):
     import torch
     import gs_scenes
     import gsrast_native as gn
-    from diff_gaussian_rasterization import GaussianRasterizationSettings, GaussianRasterizer, _C
+    from diff_gaussian_rasterization import GaussianRasterizationSettings, GaussianRasterizer, _C, build_all_map
     dev = "cuda:0"
     g, cams = gs_scenes.make_scene(args.config, P=args.gaussians)
     P = g["means3D"].shape[0]
@@ -170,7 +174,7 @@ def all_views(args):
         ca = {"avoid_pixel_all2all": False, "stats_collector": {}}
         info = {}
 
-        def step(n_gaussians=None, rast=rast, am=am, ug=ug, cl=cl, m2abs=m2abs, ca=ca, info=info):
+        def step(n_gaussians=None, rast=rast, rs=rs, am=am, ug=ug, cl=cl, m2abs=m2abs, ca=ca, info=info):
             """One view; n_gaussians: render only the first so many Gaussians (a scene between two densifications)."""
             lf = leaf if n_gaussians is None else {k: t[:n_gaussians] for k, t in leaf.items()}
             a_m = am if n_gaussians is None else am[:n_gaussians]
@@ -180,6 +184,9 @@ def all_views(args):
             m2abs.grad = None
             means2D, rgb, co, radii, depths = rast.preprocess_gaussians(
                 lf["means3D"], lf["scales"], lf["rotations"], lf["shs"], lf["opacities"], ca)
+            if args.with_all_map:
+                a_m = build_all_map(lf["means3D"], lf["scales"], lf["rotations"], rs.viewmatrix, rs.campos,
+                                    blend_records_of=means2D)
             color, n_render, _, _, _, oam, opd = rast.render_gaussians(means2D, m2, co, rgb, a_m, depths, radii, cl,
                                                                        cl, ca)
             torch.autograd.backward([color, oam, opd], [ug["color"], ug["all_map"], ug["plane_depth"]])
@@ -208,6 +215,7 @@ def all_views(args):
             "route": "radix sort over all keys" if "sort_pairs" in stages else "per-tile lists",
             "stages_ms": stages})
     out = {"metric": "fwd+bwd ms/view, every camera of the batch", "config": args.config, "gaussians": P,
+           "all_map_built_inside_the_step": bool(args.with_all_map),
            "steps": args.steps, "n_gpus": 1, "dtype": "f32", "data": "synthetic", "per_view": per_view}
     if args.interleave:
         out["interleaved"] = interleaved(args, steppers, P)
@@ -298,7 +306,7 @@ def main():
     info = {}
 
     from diff_gaussian_rasterization import build_all_map
-    vmat, cpos = cam.world_view_transform.to(dev), cam.camera_center.to(dev)
+    vmat, cpos = rs.viewmatrix, rs.campos  # (the camera's own tensors, as the caller passes them to both ops)
 
     def step(leaf=leaf, m2abs=m2abs, with_all_map=False):
         """with_all_map: the geometry channels are built inside the step by the fused op, forward and backward, as
@@ -310,7 +318,8 @@ def main():
         means2D, rgb, co, radii, depths = rast.preprocess_gaussians(leaf["means3D"], leaf["scales"],
                                                                     leaf["rotations"], leaf["shs"],
                                                                     leaf["opacities"], ca)
-        a_m = build_all_map(leaf["means3D"], leaf["scales"], leaf["rotations"], vmat, cpos) if with_all_map else am
+        a_m = (build_all_map(leaf["means3D"], leaf["scales"], leaf["rotations"], vmat, cpos, blend_records_of=means2D)
+               if with_all_map else am)
         color, n_render, _, _, _, oam, opd = rast.render_gaussians(means2D, m2abs, co, rgb, a_m, depths, radii, cl, cl,
                                                                    ca)
         torch.autograd.backward([color, oam, opd], [ug["color"], ug["all_map"], ug["plane_depth"]])

@@ -137,7 +137,8 @@ ImageLayout image_layout(int W, int H) {
 struct GeometryLayout {
   size_t tiles_touched, point_offsets, scan_temp, packed_valid, packed, total;
 };
-GeometryLayout geometry_layout(int P) {
+// own_records: the library packs the blend kernels' operand records itself (the caller brought none)
+GeometryLayout geometry_layout(int P, bool own_records = true) {
   GeometryLayout L;
   const size_t n = (size_t)(P > 0 ? P : 1);
   size_t off = 0;
@@ -146,7 +147,8 @@ GeometryLayout geometry_layout(int P) {
   L.point_offsets = take(n * 4);
   L.scan_temp = take(scan_temp_bytes((int64_t)n));
   L.packed_valid = take(4);  // one word: whether the forward call packed the records below
-  L.packed = take(n * 64);   // the blend kernels' operands, one 64-byte record per Gaussian
+  // the blend kernels' operands, one 64-byte record per Gaussian (last, so that no other offset depends on it)
+  L.packed = take(own_records ? n * 64 : 0);
   L.total = off + 256;
   return L;
 }
@@ -282,9 +284,12 @@ int gs_preprocess_forward(float* means2D, float* depths, int* radii, float* cov3
                           const float* means3D, const float* scales, const float* rotations, const float* shs,
                           const float* opacities, float scale_modifier, const float* viewmatrix,
                           const float* projmatrix, const float* cam_pos, float tan_fovx, float tan_fovy,
-                          int prefiltered, int debug, float* dcolor_ddir, gs_stream_t stream) {
+                          int prefiltered, int debug, float* dcolor_ddir, float* blend_records,
+                          gs_stream_t stream) {
   (void)prefiltered;
   GS_REQUIRE(P >= 0 && width > 0 && height > 0, "gs_preprocess_forward: bad sizes");
+  GS_REQUIRE(((uintptr_t)blend_records & 15u) == 0u, "gs_preprocess_forward: blend_records must be 16-byte aligned");
+  GS_REQUIRE(blend_records == nullptr || cam_pos != nullptr, "gs_preprocess_forward: blend_records needs cam_pos");
   if (P == 0) return 0;
   GS_REQUIRE(means2D && depths && radii && conic_opacity && rgb && clamped, "gs_preprocess_forward: null output");
   GS_REQUIRE(means3D && scales && rotations && opacities && viewmatrix && projmatrix,
@@ -302,6 +307,7 @@ int gs_preprocess_forward(float* means2D, float* depths, int* radii, float* cov3
   a.radii = radii; a.means2D = means2D; a.depths = depths; a.cov3D = cov3D; a.conic_opacity = conic_opacity;
   a.rgb = rgb; a.clamped = clamped; a.tiles_touched = tiles_touched;
   a.dcolor_ddir = sh_mode ? dcolor_ddir : nullptr;
+  a.blend_records = blend_records;
   {
     StageScope _t("preprocess_fwd", (hipStream_t)stream);
     launch_preprocess_fwd(a, (hipStream_t)stream);
@@ -479,7 +485,12 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
   tile_grid(width, height, gx, gy);
   const int T = gx * gy;
 
-  const GeometryLayout GL = geometry_layout(P);
+  // The blend kernels' operand records: the caller's (complete: gs_preprocess_forward and gs_all_map_forward wrote
+  // their parts), or packed here for a view with enough instances per Gaussian.
+  const float* caller_records =
+      (options != nullptr && options->struct_bytes >= sizeof(gs_render_options)) ? options->blend_records : nullptr;
+  GS_REQUIRE(((uintptr_t)caller_records & 15u) == 0u, "gs_render_forward: blend_records must be 16-byte aligned");
+  const GeometryLayout GL = geometry_layout(P, caller_records == nullptr);
   char* gbase = geometryBuffer(GL.total, geometry_user);
   GS_REQUIRE(gbase, "gs_render_forward: geometry buffer callback returned NULL");
   gbase = align_ptr(gbase, 256);
@@ -550,6 +561,13 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
   auto decide_packing = [&](int64_t instances) -> int {
     if (pack_decided) return 0;
     pack_decided = true;
+    if (caller_records != nullptr) {
+      // (the word beside the library's own records says "none": a backward call that is not handed the caller's
+      // records again gathers the operands from the arrays)
+      use_packed = true;
+      launch_fill_u32(1, 0u, packed_valid, stream);
+      return check_launch("pack_operands", stream, dbg);
+    }
     use_packed = instances * 5 > (int64_t)P * 4;
     StageScope _t("pack_operands", stream);
     if (use_packed)
@@ -599,7 +617,7 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
     a.n_render = n_render; a.n_consider = n_consider; a.n_contrib_tile = n_contrib;
     a.fits_word = ahead_of_host ? bucket_fits_word(bucket_table, T) : nullptr;
     a.block_hits = A.block_hits;
-    a.packed = use_packed ? packed : nullptr;
+    a.packed = use_packed ? (caller_records != nullptr ? caller_records : packed) : nullptr;
     {
       StageScope _t("render_fwd", stream);
       launch_render_fwd(a, stream);
@@ -630,7 +648,8 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
   if (ahead) {
     if (carve(cap_n, A)) return 1;
     if (timer.begin(elapsed_ms != nullptr, stream)) return 1;
-    if (decide_packing(cap_n)) return 1;  // (on the expected count; the margin in it is the caller's)
+    // (on the expected count less a fifth: the caller's expectation carries a margin of a quarter)
+    if (decide_packing(cap_n - cap_n / 5)) return 1;
     if (lists_by_tile(A, cap_longest, 0xFFFFFFFFu, true)) return 1;
     if (blend(A, true)) return 1;
   }
@@ -740,7 +759,7 @@ int gs_render_backward(int P, int R, const float* background, int width, int hei
                        const float* conic_opacity, const float* rgb, const float* all_maps,
                        const float* all_map_pixels, int render_geo, int debug, float* instance_grads,
                        size_t instance_grads_bytes, float* elapsed_ms, int64_t binning_capacity,
-                       gs_stream_t stream_) {
+                       const float* blend_records, gs_stream_t stream_) {
   hipStream_t stream = (hipStream_t)stream_;
   if (pending_fault("gs_render_backward")) return 1;
   GS_REQUIRE(binning_capacity <= 0 || binning_capacity >= R, "gs_render_backward: binning_capacity below R");
@@ -764,8 +783,10 @@ int gs_render_backward(int P, int R, const float* background, int width, int hei
   a.emission_sorted = (const uint32_t*)(bbase + BL.emission);
   a.block_hits = (const uint16_t*)(bbase + BL.block_hits);
   a.point_offsets = (const uint32_t*)(gbase + GL.point_offsets);
-  a.packed = (const float*)(gbase + GL.packed);  // (of the arrays the forward call was given)
-  a.packed_valid = (const uint32_t*)(gbase + GL.packed_valid);
+  // (records of the arrays the forward call was given: the caller's own, or what the forward call packed)
+  GS_REQUIRE(((uintptr_t)blend_records & 15u) == 0u, "gs_render_backward: blend_records must be 16-byte aligned");
+  a.packed = blend_records != nullptr ? blend_records : (const float*)(gbase + GL.packed);
+  a.packed_valid = blend_records != nullptr ? nullptr : (const uint32_t*)(gbase + GL.packed_valid);
   a.instance_grads = (float*)align_ptr((const char*)instance_grads, 256);
   a.P = P; a.W = width; a.H = height;
   a.fy = height / (2.0f * tan_fovy);  // cuda_rasterizer/rasterizer_impl.cu:885-886

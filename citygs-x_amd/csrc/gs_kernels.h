@@ -22,6 +22,10 @@ struct PreprocessFwdArgs {
   // [axis][channel], written for Gaussians that survive culling (SH mode); the backward kernel takes it in place of
   // the coefficients
   float* dcolor_ddir = nullptr;
+  // optional (P,16): the blend kernels' operand records (see launch_pack_blend_operands) of the surviving
+  // Gaussians, complete: the geometry channels are formed from means3D, scales, rotations, viewmatrix and campos
+  // as launch_all_map_fwd forms them
+  float* blend_records = nullptr;
 };
 
 struct PreprocessBwdArgs {

@@ -7,6 +7,7 @@
 // for the rounding policy).  One thread per Gaussian; every output element is
 // written by the kernel (zeros for culled Gaussians), so callers may hand in
 // uninitialised buffers.
+#include "all_map_common.h"
 #include "gs_common.h"
 #include "gs_kernels.h"
 
@@ -357,8 +358,12 @@ __device__ __forceinline__ void wave_rows_store(float4* __restrict__ g4, int row
 
 // DERIV: also leave, per surviving Gaussian, the derivative of its colour with respect to the view direction
 // (nine numbers), which is all the backward kernel needs the coefficients for.
-template <bool DERIV>
-__global__ void __launch_bounds__(GS_BLOCK_1D) __attribute__((amdgpu_waves_per_eu(6)))
+// RECORDS: also write the blend kernels' operand record of every surviving Gaussian, (x, y, conic.x, conic.y)
+// (conic.w, opacity, r, g) (b, map0, map1, map2) (map3, map4, depth, 0), the geometry channels formed here by the
+// all_map kernel's own operations on the same inputs; a wave's 64 records leave through LDS as contiguous lines.
+// (six waves per SIMD; five with the records: six would spill there, and a kernel that spills starts its waves slowly)
+template <bool DERIV, bool RECORDS>
+__global__ void __launch_bounds__(GS_BLOCK_1D) __attribute__((amdgpu_waves_per_eu(RECORDS ? 5 : 6)))
 preprocess_fwd_kernel(int P, int D, int M, const float* __restrict__ means, const float* __restrict__ scales,
                       float mod, const float* __restrict__ rots, const float* __restrict__ opac,
                       const float* __restrict__ shs, const float* __restrict__ Vg, const float* __restrict__ PMg,
@@ -366,8 +371,11 @@ preprocess_fwd_kernel(int P, int D, int M, const float* __restrict__ means, cons
                       uint32_t gx, uint32_t gy, int* __restrict__ radii, float2* __restrict__ means2D,
                       float* __restrict__ depths, float* __restrict__ cov3D, float4* __restrict__ conic_opacity,
                       float* __restrict__ rgb, uint8_t* __restrict__ clamped, uint32_t* __restrict__ tiles_touched,
-                      float* __restrict__ dcolor_ddir) {
+                      float* __restrict__ dcolor_ddir, float* __restrict__ blend_records) {
   __shared__ float4 s_sh[GS_BLOCK_1D / GS_WAVE][GS_WAVE * SH_THIRD4];
+  // RECORDS: what the record takes of the geometry, parked per lane while the colour is evaluated (held in
+  // registers it would make the kernel spill; fetched again at the end it would keep every wave waiting for loads)
+  __shared__ float s_keep[RECORDS ? GS_BLOCK_1D / GS_WAVE : 1][RECORDS ? 12 * GS_WAVE : 1];
   const int slot = blockIdx.x * GS_BLOCK_1D + threadIdx.x;
   const bool live = slot < P;
   const int i = live ? slot : P - 1;  // lanes past the end keep step with a copy of the last Gaussian and store nothing
@@ -394,6 +402,23 @@ preprocess_fwd_kernel(int P, int D, int M, const float* __restrict__ means, cons
     conic_opacity[i] = ok ? make_float4(g.conic[0], g.conic[1], g.conic[2], opac[i]) : make_float4(0.f, 0.f, 0.f, 0.f);
     if (tiles_touched) tiles_touched[i] = ok ? (g.rect.x1 - g.rect.x0) * (g.rect.y1 - g.rect.y0) : 0u;
   }
+  if (RECORDS && ok) {  // (culled Gaussians have no record)
+    float chan[5];
+    AllMapGeom ag;
+    all_map_geom(mean, sc, q4, cam.V, cam.campos, ag);
+    all_map_channels(ag, chan);
+    float* keep = s_keep[threadIdx.x / GS_WAVE] + (threadIdx.x & (GS_WAVE - 1));
+    keep[0 * GS_WAVE] = g.px;
+    keep[1 * GS_WAVE] = g.py;
+    keep[2 * GS_WAVE] = g.conic[0];
+    keep[3 * GS_WAVE] = g.conic[1];
+    keep[4 * GS_WAVE] = g.conic[2];
+    keep[5 * GS_WAVE] = opac[i];
+    keep[6 * GS_WAVE] = g.depth;
+#pragma unroll
+    for (int k = 0; k < 5; k++) keep[(7 + k) * GS_WAVE] = chan[k];
+  }
+
   float col[3] = {0.f, 0.f, 0.f};
   uint8_t clm[3] = {0, 0, 0};
   if (shs != nullptr && M > 0) {  // wave-uniform
@@ -478,6 +503,32 @@ preprocess_fwd_kernel(int P, int D, int M, const float* __restrict__ means, cons
 #pragma unroll
           for (int ch = 0; ch < 3; ch++) dd[3 * a + ch] = dR[a][ch];
         }
+      }
+    }
+  }
+  if (RECORDS) {
+    // lane l stores 16-byte word (l & 3) of record 16 k + (l >> 2) in round k; in LDS a record's four words sit
+    // 65 words apart, so that neither the writes, record-major, nor the reads, word-minor, pile up on a few banks
+    constexpr int WORD_STRIDE = GS_WAVE + 1;
+    static_assert(4 * WORD_STRIDE <= GS_WAVE * SH_THIRD4, "the records are staged where the coefficient rows were");
+    const int lane = threadIdx.x & (GS_WAVE - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / GS_WAVE);
+    const uint64_t ok_m = gs_ballot(ok && live);
+    if (ok_m != 0ull) {
+      float4* mine = s_sh[wave];
+      wave_sync_lds();  // (everyone has read what the buffer last held)
+      const float* keep = s_keep[wave] + lane;
+      mine[0 * WORD_STRIDE + lane] = make_float4(keep[0 * GS_WAVE], keep[1 * GS_WAVE], keep[2 * GS_WAVE], keep[3 * GS_WAVE]);
+      mine[1 * WORD_STRIDE + lane] = make_float4(keep[4 * GS_WAVE], keep[5 * GS_WAVE], col[0], col[1]);
+      mine[2 * WORD_STRIDE + lane] = make_float4(col[2], keep[7 * GS_WAVE], keep[8 * GS_WAVE], keep[9 * GS_WAVE]);
+      mine[3 * WORD_STRIDE + lane] = make_float4(keep[10 * GS_WAVE], keep[11 * GS_WAVE], keep[6 * GS_WAVE], 0.f);
+      wave_sync_lds();
+      float4* out = reinterpret_cast<float4*>(blend_records) +
+                    4 * ((size_t)blockIdx.x * GS_BLOCK_1D + (size_t)wave * GS_WAVE);  // the wave's first record
+#pragma unroll
+      for (int k = 0; k < 4; k++) {
+        const int rec = 16 * k + (lane >> 2);
+        if ((ok_m >> rec) & 1ull) out[64 * k + lane] = mine[(lane & 3) * WORD_STRIDE + rec];
       }
     }
   }
@@ -795,10 +846,16 @@ int launch_preprocess_fwd(const PreprocessFwdArgs& a, hipStream_t stream) {
     hipLaunchKernelGGL(kernel, dim3(blocks), dim3(GS_BLOCK_1D), 0, stream, a.P, a.D, a.M, a.means3D, a.scales,
                        a.scale_modifier, a.rotations, a.opacities, a.shs, a.viewmatrix, a.projmatrix, a.campos, a.W,
                        a.H, a.tanx, a.tany, fx, fy, gx, gy, a.radii, (float2*)a.means2D, a.depths, a.cov3D,
-                       (float4*)a.conic_opacity, a.rgb, a.clamped, a.tiles_touched, a.dcolor_ddir);
+                       (float4*)a.conic_opacity, a.rgb, a.clamped, a.tiles_touched, a.dcolor_ddir, a.blend_records);
   };
-  if (a.dcolor_ddir != nullptr && a.shs != nullptr && a.M > 0) go(preprocess_fwd_kernel<true>);
-  else go(preprocess_fwd_kernel<false>);
+  const bool deriv = a.dcolor_ddir != nullptr && a.shs != nullptr && a.M > 0;
+  if (a.blend_records != nullptr) {
+    if (deriv) go(preprocess_fwd_kernel<true, true>);
+    else go(preprocess_fwd_kernel<false, true>);
+  } else {
+    if (deriv) go(preprocess_fwd_kernel<true, false>);
+    else go(preprocess_fwd_kernel<false, false>);
+  }
   return 0;
 }
 

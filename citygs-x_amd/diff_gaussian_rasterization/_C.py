@@ -86,13 +86,16 @@ def preprocess_gaussians(means3D, scales, rotations, sh, opacity, scale_modifier
 
 def preprocess_gaussians_ex(means3D, scales, rotations, sh, opacity, scale_modifier, viewmatrix, projmatrix, tan_fovx,
                             tan_fovy, image_height, image_width, degree, campos, prefiltered, debug, args,
-                            want_direction_derivative=False, want_cov3D=True):
+                            want_direction_derivative=False, want_cov3D=True, blend_records=None):
     """preprocess_gaussians plus what the reference's tuple has no slot for: returns (tuple, dcolor_ddir).  With
     want_direction_derivative (and SH colours) dcolor_ddir is the (P,3,3) derivative of every surviving Gaussian's
     colour with respect to the unit view direction; handed to preprocess_gaussians_backward it replaces the
     coefficients there (same gradients, and the backward pass does not read the 192-byte rows).  Otherwise None.
     want_cov3D=False leaves the cov3D slot of the tuple None: preprocess_gaussians_backward, given None, forms the
-    covariances again from scales and rotations (the same bits), and neither pass moves the 24 bytes per Gaussian."""
+    covariances again from scales and rotations (the same bits), and neither pass moves the 24 bytes per Gaussian.
+    blend_records: an optional (P,16) float32 tensor that receives the blend kernels' operand records of the
+    surviving Gaussians, geometry channels included (those build_all_map gives for the same means3D, scales,
+    rotations, viewmatrix and campos); see render_gaussians_ex."""
     if means3D.ndimension() != 2 or means3D.size(1) != 3:
         raise RuntimeError("means3D must have dimensions (num_points, 3)")
     means3D = _f32c(means3D, "means3D")
@@ -121,7 +124,8 @@ def preprocess_gaussians_ex(means3D, scales, rotations, sh, opacity, scale_modif
             _ptr(means2D), _ptr(depths), _ptr(radii), _ptr(cov3D), _ptr(conic_opacity), _ptr(rgb), _ptr(clamped), None,
             P, int(degree), M, int(image_width), int(image_height), _ptr(means3D), _ptr(scales), _ptr(rotations),
             _ptr(shc), _ptr(opacity), float(scale_modifier), _ptr(vm), _ptr(pm), _ptr(cp), float(tan_fovx),
-            float(tan_fovy), int(bool(prefiltered)), int(bool(debug)), _ptr(ddir), _stream(dev)),
+            float(tan_fovy), int(bool(prefiltered)), int(bool(debug)), _ptr(ddir), _ptr(blend_records),
+            _stream(dev)),
             "preprocess_gaussians")
     return (0, means2D, depths, radii, cov3D, conic_opacity, rgb, clamped), ddir
 
@@ -250,12 +254,15 @@ def _write_tile_log(args, H, W, n_render, n_consider, n_contrib):
 
 def render_gaussians_ex(background, image_height, image_width, means2D, depths, radii, conic_opacity, rgb,
                         compute_locally, viewmatrix, campos, tan_fovx, tan_fovy, all_map, render_geo, debug, args,
-                        expected_instances=0, expected_longest_list=0):
+                        expected_instances=0, expected_longest_list=0, blend_records=None):
     """render_gaussians plus what the reference's tuple has no slot for: returns (tuple, info) with info =
     {"longest_list", "binning_capacity", "launched_ahead"}.  With expected_instances > 0 the list kernels and the
     blend are launched without waiting for the instance count, on a binning buffer laid out for
     expected_instances; info["binning_capacity"] then has to be handed to render_gaussians_backward (and to
-    gs_binning_state_layout) in place of the instance count.  Results do not depend on the expectation."""
+    gs_binning_state_layout) in place of the instance count.  Results do not depend on the expectation.
+    blend_records: the (P,16) operand records that preprocess_gaussians_ex wrote for exactly these inputs, all_map
+    being build_all_map of the same Gaussians and camera (the blend kernels then read them and nothing is
+    packed); the same tensor goes to render_gaussians_backward."""
     means2D = _f32c(means2D, "means2D")
     dev = means2D.device
     P = means2D.shape[0]
@@ -291,10 +298,14 @@ def render_gaussians_ex(background, image_height, image_width, means2D, depths, 
     # (small_limit, block_records) for this call only: how the per-tile lists are built (a test hook)
     limits = args.get("tile_sort_limits") if isinstance(args, dict) else None
     options = None
-    if limits is not None or expected_instances > 0:
+    if blend_records is not None and (blend_records.shape != (P, 16) or blend_records.dtype != torch.float32
+                                      or not blend_records.is_contiguous() or blend_records.device != dev):
+        raise RuntimeError("blend_records must be a contiguous (P, 16) float32 tensor on the same device")
+    if limits is not None or expected_instances > 0 or blend_records is not None:
         options = _n.RenderOptions(*(limits if limits is not None else (-1, -1)),
                                    expected_instances=expected_instances,
-                                   expected_longest_list=expected_longest_list)
+                                   expected_longest_list=expected_longest_list,
+                                   blend_records=blend_records.data_ptr() if blend_records is not None else None)
     result = _n.RenderResult()
     mwd = torch.empty(1, H, W, **f32) if want_mwd else None
     # fp32 arithmetic, as `H / (2.0f * tan_fovy)` at rasterize_points.cu:328-329
@@ -326,10 +337,12 @@ def render_gaussians_ex(background, image_height, image_width, means2D, depths, 
 
 def render_gaussians_backward(background, tan_fovx, tan_fovy, all_map_pixels, all_maps, R, geomBuffer, binningBuffer,
                               imageBuffer, compute_locally, dL_dout_color, dL_dout_all_map, dL_dout_plane_depth,
-                              means2D, conic_opacity, rgb, render_geo, debug, args, binning_capacity=0):
+                              means2D, conic_opacity, rgb, render_geo, debug, args, binning_capacity=0,
+                              blend_records=None):
     """rasterize_points.cu:366-441.  Returns dL_dmeans2D as (P,2); the reference
     returns (P,3) and its Python wrapper slices [:, :2].  binning_capacity: info["binning_capacity"] of
-    render_gaussians_ex when that call was given an expectation (0 otherwise)."""
+    render_gaussians_ex when that call was given an expectation (0 otherwise); blend_records: the tensor that call
+    was given, if any."""
     means2D = _f32c(means2D, "means2D")
     dev = means2D.device
     P = means2D.shape[0]
@@ -360,7 +373,8 @@ def render_gaussians_backward(background, tan_fovx, tan_fovy, all_map_pixels, al
                 _ptr(imageBuffer), _ptr(compute_locally.contiguous()), _ptr(gpix), _ptr(gmap), _ptr(gdep),
                 _ptr(dL_dmeans2D), _ptr(dL_dmeans2D_abs), _ptr(dL_dconic_opacity), _ptr(dL_dcolors), _ptr(dL_dall_map),
                 _ptr(means2D), _ptr(co), _ptr(col), _ptr(am), _ptr(amp), int(geo), int(bool(debug)), _ptr(workspace),
-                ws_bytes, C.byref(elapsed) if timing else None, int(binning_capacity), _stream(dev)),
+                ws_bytes, C.byref(elapsed) if timing else None, int(binning_capacity), _ptr(blend_records),
+                _stream(dev)),
                 "render_gaussians_backward")
         _record_time(args, "backward_render_time", elapsed.value)
     else:

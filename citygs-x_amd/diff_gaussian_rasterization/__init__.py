@@ -12,6 +12,7 @@ preprocess evaluate colour from spherical harmonics at `sh_degree` and return
 the matching dL/dshs; any other `shs` shape keeps the reference behaviour
 (colour output zero, zero gradient of the same shape as `shs`).
 """
+import weakref
 from typing import NamedTuple
 
 import torch
@@ -39,6 +40,59 @@ class GaussianRasterizationSettings(NamedTuple):
     debug: bool
 
 
+# ------------------------------------------------------------ blend records --
+
+# The blend kernels read a Gaussian's operands (centre, conic, opacity, colour, geometry channels, depth) as one
+# 64-byte record.  The library packs those records itself from the separate tensors, one more pass per view, unless
+# preprocess_gaussians has written them on the way: it has every value but the geometry channels at hand, and
+# those it forms as build_all_map does, from the same parameters and camera.  The records travel as an attribute
+# of the means2D tensor.  render_gaussians uses them only if every tensor it is given is the very tensor the
+# records were written from, unmodified since (tensor identity and version counters), and, with geometry channels
+# to render, if all_map is what build_all_map(..., blend_records_of=means2D) returned for the very parameter
+# tensors and camera preprocess_gaussians had; otherwise the library packs.  Nothing a caller sees changes: same
+# tensors, same values.
+
+class _BlendRecords:
+    __slots__ = ("records", "refs", "versions", "sources", "source_versions", "all_map_ref", "all_map_version")
+
+    def __init__(self, records, parts, sources):
+        self.records = records
+        self.refs = [weakref.ref(t) for t in parts]
+        self.versions = [t._version for t in parts]
+        # means3D, scales, rotations, viewmatrix, campos as preprocess_gaussians had them
+        self.sources = [weakref.ref(t) for t in sources]
+        self.source_versions = [t._version for t in sources]
+        self.all_map_ref = None
+        self.all_map_version = -1
+
+    def same_sources(self, sources):
+        return all(ref() is t and t._version == v for ref, v, t in zip(self.sources, self.source_versions, sources))
+
+    def usable(self, parts, all_maps, render_geo):
+        for ref, version, t in zip(self.refs, self.versions, parts):
+            if ref() is not t or t._version != version:
+                return False
+        if render_geo and (self.all_map_ref is None or self.all_map_ref() is not all_maps
+                           or all_maps._version != self.all_map_version):
+            return False
+        return True
+
+
+_linked_all_map_seen = [False]  # the caller builds all_map with blend_records_of=...: records are worth starting
+_pending_blend = [None]         # from _PreprocessGaussians.forward to the wrapper that tags its outputs
+
+
+def _records_wanted(rs, P, device):
+    """Whether preprocess should write the records: the last view of this image size had enough instances per
+    Gaussian for records to pay (written on the way they cost about a third of the library's packing pass, which
+    pays from 0.8 instances per Gaussian), and render_gaussians will be able to use them (no geometry channels to
+    render, or the caller builds them through build_all_map(..., blend_records_of=means2D))."""
+    seen = _expectations.get((rs.image_height, rs.image_width, device))
+    if seen is None or seen[0] * 10 <= P * 3:
+        return False
+    return (not rs.render_geo) or _linked_all_map_seen[0]
+
+
 # --------------------------------------------------------------- preprocess --
 
 class _PreprocessGaussians(torch.autograd.Function):
@@ -47,10 +101,15 @@ class _PreprocessGaussians(torch.autograd.Function):
         rs = raster_settings
         # (when a backward pass can follow, the forward kernel also leaves the colours' derivative with respect to
         # the view direction, nine numbers per Gaussian, which is all the backward kernel needs the coefficients for)
+        P = means3D.shape[0]
+        records = (torch.empty(P, 16, dtype=torch.float32, device=means3D.device)
+                   if P > 0 and _records_wanted(rs, P, means3D.device) else None)
         (num_rendered, means2D, depths, radii, cov3D, conic_opacity, rgb, clamped), ddir = _C.preprocess_gaussians_ex(
             means3D, scales, rotations, sh, opacities, rs.scale_modifier, rs.viewmatrix, rs.projmatrix, rs.tanfovx,
             rs.tanfovy, rs.image_height, rs.image_width, rs.sh_degree, rs.campos, rs.prefiltered, rs.debug, cuda_args,
-            want_direction_derivative=any(ctx.needs_input_grad[:5]), want_cov3D=False)
+            want_direction_derivative=any(ctx.needs_input_grad[:5]), want_cov3D=False, blend_records=records)
+        _pending_blend[0] = ((records, (means3D, scales, rotations, rs.viewmatrix, rs.campos))
+                             if records is not None else None)
         # (cov3D is None: the backward kernel forms the covariances again from scales and rotations, which it reads
         # anyway, instead of both passes moving 24 bytes per Gaussian)
         ctx.raster_settings = rs
@@ -86,7 +145,13 @@ class _PreprocessGaussians(torch.autograd.Function):
 
 
 def preprocess_gaussians(means3D, scales, rotations, sh, opacities, raster_settings, cuda_args):
-    return _PreprocessGaussians.apply(means3D, scales, rotations, sh, opacities, raster_settings, cuda_args)
+    _pending_blend[0] = None
+    means2D, rgb, conic_opacity, radii, depths = _PreprocessGaussians.apply(means3D, scales, rotations, sh, opacities,
+                                                                            raster_settings, cuda_args)
+    pending, _pending_blend[0] = _pending_blend[0], None
+    if pending is not None:
+        means2D._gs_blend = _BlendRecords(pending[0], (means2D, conic_opacity, rgb, depths), pending[1])
+    return means2D, rgb, conic_opacity, radii, depths
 
 
 # ------------------------------------------------------------------- render --
@@ -133,11 +198,19 @@ class _RenderGaussians(torch.autograd.Function):
         mask = extended_compute_locally if avoid else compute_locally
         key = (rs.image_height, rs.image_width, means2D.device)
         expected_instances, expected_longest = _expectation(key)
+        blend = getattr(means2D, "_gs_blend", None)
+        records = (blend.records if blend is not None and blend.usable((means2D, conic_opacity, rgb, depths), all_maps,
+                                                                       rs.render_geo) else None)
+        if blend is not None and records is None and rs.render_geo:
+            # records were written and cannot be used: the caller does not (or no longer) build all_map through
+            # build_all_map(..., blend_records_of=means2D); stop writing them until it does
+            _linked_all_map_seen[0] = False
         ((num_rendered, color, n_render, n_consider, n_contrib, out_observe, out_all_map, out_plane_depth, geomBuffer,
           binningBuffer, imgBuffer), info) = _C.render_gaussians_ex(
             rs.bg, rs.image_height, rs.image_width, means2D, depths, radii, conic_opacity, rgb, mask, rs.viewmatrix,
             rs.campos, rs.tanfovx, rs.tanfovy, all_maps, rs.render_geo, rs.debug, cuda_args,
-            expected_instances=expected_instances, expected_longest_list=expected_longest)
+            expected_instances=expected_instances, expected_longest_list=expected_longest, blend_records=records)
+        ctx.blend_records = records
         if means2D.shape[0] > 0:
             _remember(key, num_rendered, info["longest_list"])
         if isinstance(cuda_args, dict) and isinstance(cuda_args.get("stats_collector"), dict):
@@ -170,7 +243,8 @@ class _RenderGaussians(torch.autograd.Function):
         dL_dmeans2D, dL_dmeans2D_abs, dL_dconic_opacity, dL_dcolors, dL_dall_map = _C.render_gaussians_backward(
             rs.bg, rs.tanfovx, rs.tanfovy, all_map_pixels, all_maps, ctx.num_rendered, geomBuffer, binningBuffer,
             imgBuffer, compute_locally, grad_color, grad_out_all_map, grad_out_plane_depth, means2D, conic_opacity,
-            rgb, rs.render_geo, rs.debug, ctx.cuda_args, binning_capacity=ctx.binning_capacity)
+            rgb, rs.render_geo, rs.debug, ctx.cuda_args, binning_capacity=ctx.binning_capacity,
+            blend_records=ctx.blend_records)
         return (dL_dmeans2D, dL_dmeans2D_abs, dL_dconic_opacity, dL_dcolors, dL_dall_map, None, None, None, None, None,
                 None)
 
@@ -197,11 +271,22 @@ class _BuildAllMap(torch.autograd.Function):
         return dL_dmeans3D, None, dL_drotations, None, None
 
 
-def build_all_map(means3D, scales, rotations, viewmatrix, campos):
+def build_all_map(means3D, scales, rotations, viewmatrix, campos, blend_records_of=None):
     """[normal in the camera frame, 1, |normal . p_cam|] per Gaussian: a drop-in for the torch lines
     gaussian_renderer/__init__.py:1501-1518 (pass the camera's world_view_transform and camera_center).
-    Differentiable in means3D and rotations, like those lines; `scales` only picks the axis."""
-    return _BuildAllMap.apply(means3D, scales, rotations, viewmatrix, campos)
+    Differentiable in means3D and rotations, like those lines; `scales` only picks the axis.
+    blend_records_of (optional): the means2D tensor preprocess_gaussians returned for the same parameter tensors
+    and camera (the settings' viewmatrix and campos tensors).  preprocess_gaussians then writes the blend kernels'
+    operand records with these very channels in them (from the next view on), and render_gaussians, given these
+    very tensors, skips the pass that packs them.  The returned tensor is the same either way."""
+    all_map = _BuildAllMap.apply(means3D, scales, rotations, viewmatrix, campos)
+    if blend_records_of is not None:
+        _linked_all_map_seen[0] = True
+        blend = getattr(blend_records_of, "_gs_blend", None)
+        if blend is not None and blend.same_sources((means3D, scales, rotations, viewmatrix, campos)):
+            blend.all_map_ref = weakref.ref(all_map)
+            blend.all_map_version = all_map._version
+    return all_map
 
 
 # ------------------------------------------------------------------- module --

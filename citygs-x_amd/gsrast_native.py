@@ -28,14 +28,15 @@ _SIGNATURES = {
     "gs_higher_msb": (C.c_uint32, [C.c_uint32]),
     "gs_mark_visible": (_i, [_i, _vp, _vp, _vp, _vp, _vp]),
     "gs_visible_filter": (_i, [_i, _i, _i, _i, _vp, _vp, _f, _vp, _vp, _vp, _vp, _f, _f, _i, _vp, _i, _vp]),
-    "gs_preprocess_forward": (_i, [_vp] * 8 + [_i] * 5 + [_vp] * 5 + [_f] + [_vp] * 3 + [_f, _f, _i, _i, _vp, _vp]),
+    "gs_preprocess_forward": (_i, [_vp] * 8 + [_i] * 5 + [_vp] * 5 + [_f] + [_vp] * 3 + [_f, _f, _i, _i, _vp, _vp,
+                                   _vp]),
     "gs_preprocess_backward": (_i, [_vp] * 3 + [_i] * 5 + [_vp] * 4 + [_f] + [_vp] * 3 + [_f, _f] + [_vp, _i] +
                                [_vp] * 8 + [_i, _vp, _vp]),
     "gs_render_forward": (_i, [RESIZE_FN, _vp, RESIZE_FN, _vp, RESIZE_FN, _vp, _i, _vp, _i, _i, _f, _f, _f, _f] +
                           [_vp] * 17 + [_i, _i, C.POINTER(_i), C.POINTER(_f), _vp, _vp, _vp]),
     "gs_render_backward_workspace_bytes": (_sz, [_i]),
     "gs_render_backward": (_i, [_i, _i, _vp, _i, _i, _f, _f] + [_vp] * 17 + [_i, _i, _vp, _sz, C.POINTER(_f), _i64,
-                                _vp]),
+                                _vp, _vp]),
     "gs_ssim_l1_forward": (_i, [_i, _i, _i] + [_vp] * 9),
     "gs_ssim_l1_backward": (_i, [_i, _i, _i] + [_vp] * 10),
     "gs_training_stats_workspace_bytes": (_sz, [_i64, _i64]),
@@ -90,12 +91,12 @@ class RenderOptions(C.Structure):
     means none."""
     _fields_ = [("struct_bytes", C.c_uint32), ("tile_sort_small_limit", C.c_int32),
                 ("tile_sort_block_records", C.c_int32), ("expected_longest_list", C.c_int32),
-                ("expected_instances", C.c_int64)]
+                ("expected_instances", C.c_int64), ("blend_records", C.c_void_p)]
 
     def __init__(self, tile_sort_small_limit=-1, tile_sort_block_records=-1, expected_instances=0,
-                 expected_longest_list=0):
+                 expected_longest_list=0, blend_records=None):
         super().__init__(C.sizeof(RenderOptions), int(tile_sort_small_limit), int(tile_sort_block_records),
-                         int(expected_longest_list), int(expected_instances))
+                         int(expected_longest_list), int(expected_instances), blend_records)
 
 
 class RenderResult(C.Structure):

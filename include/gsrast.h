@@ -73,13 +73,21 @@ int gs_visible_filter(int P, int M, int width, int height, const float* means3D,
  * respect to the unit view direction, [axis][channel] (rows of culled
  * Gaussians are not written).  It is all that gs_preprocess_backward needs the
  * coefficients for: a caller that keeps it (36 bytes per Gaussian) saves the
- * backward call the 192-byte coefficient rows. */
+ * backward call the 192-byte coefficient rows.
+ * blend_records (no counterpart in the reference; NULL to skip): (P,16) floats, 16-byte aligned: the blend
+ * kernels' operand records, one 64-byte record per Gaussian, (x, y, conic.x, conic.y) (conic.w, opacity, r, g)
+ * (b, map0, map1, map2) (map3, map4, depth, 0).  This call writes the record of every surviving Gaussian in
+ * full: the five geometry channels are the ones gs_all_map_forward gives for the same means3D, scales (as
+ * passed here), rotations, viewmatrix and cam_pos, bit for bit.  A caller that blends with exactly those
+ * channels hands the records to gs_render_forward (gs_render_options.blend_records) and gs_render_backward and
+ * saves them the pass that packs the same records from the separate arrays. */
 int gs_preprocess_forward(float* means2D, float* depths, int* radii, float* cov3D, float* conic_opacity,
                           float* rgb, uint8_t* clamped, uint32_t* tiles_touched, int P, int D, int M, int width,
                           int height, const float* means3D, const float* scales, const float* rotations,
                           const float* shs, const float* opacities, float scale_modifier, const float* viewmatrix,
                           const float* projmatrix, const float* cam_pos, float tan_fovx, float tan_fovy,
-                          int prefiltered, int debug, float* dcolor_ddir, gs_stream_t stream);
+                          int prefiltered, int debug, float* dcolor_ddir, float* blend_records,
+                          gs_stream_t stream);
 
 /* Replaces Rasterizer::preprocessBackward (CR/rasterizer.h:86-111,
  * CR/rasterizer_impl.cu:427-489) together with the tensor repacking of
@@ -125,9 +133,15 @@ typedef struct gs_render_options {
    * instance count before it goes on: it sizes the binning buffer for expected_instances, launches the list
    * kernels and the blend right behind the counting kernels, and lets a device-side check turn them into no-ops
    * if the view has more instances than that or a list longer than expected_longest_list (0 = any length; a
-   * figure of at most 2048 spares the launch of the radix sort's kernels); in that case the lists are built again the ordinary way, so the result never depends on
-   * the expectation, only the time does. */
+   * figure of at most 2048 spares the launch of the radix sort's kernels); in that case the lists are built
+   * again the ordinary way, so the result never depends on the expectation, only the time does. */
   int64_t expected_instances;
+  /* The blend kernels' operand records of this view's Gaussians as gs_preprocess_forward wrote them (their
+   * geometry channels must be the all_map this call is given; with render_geo == 0 they are not read), or NULL:
+   * the call then packs
+   * them itself when the view has more than 0.8 instances per Gaussian.  The same pointer goes to
+   * gs_render_backward; the records must stay as they are until that call has run. */
+  const float* blend_records;
 } gs_render_options;
 
 /* What gs_render_forward reports besides the instance count (optional, NULL to skip; struct_bytes as above):
@@ -194,7 +208,8 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
  * of gs_render_backward_workspace_bytes(R) bytes, and sums each Gaussian's
  * records in a second kernel (no atomics, run-to-run deterministic).
  * elapsed_ms as above (backward_render_time, CR/rasterizer_impl.cu:924-926).
- * binning_capacity: gs_render_result.binning_capacity of the forward call (0 or R if it did not run ahead). */
+ * binning_capacity: gs_render_result.binning_capacity of the forward call (0 or R if it did not run ahead).
+ * blend_records: gs_render_options.blend_records of the forward call (NULL if that call was given none). */
 size_t gs_render_backward_workspace_bytes(int R);
 int gs_render_backward(int P, int R, const float* background, int width, int height, float tan_fovx,
                        float tan_fovy, const char* geom_buffer, const char* binning_buffer,
@@ -204,7 +219,7 @@ int gs_render_backward(int P, int R, const float* background, int width, int hei
                        const float* means2D, const float* conic_opacity, const float* rgb, const float* all_maps,
                        const float* all_map_pixels, int render_geo, int debug, float* instance_grads,
                        size_t instance_grads_bytes, float* elapsed_ms, int64_t binning_capacity,
-                       gs_stream_t stream);
+                       const float* blend_records, gs_stream_t stream);
 
 /* Replaces SimpleKNN::knn / distCUDA2 (KNN/simple_knn.h:17, KNN/simple_knn.cu:185-221,
  * KNN/spatial.cu:17-35): mean_dists[i] = mean squared distance from point i

@@ -69,7 +69,7 @@ def preprocess_fwd(g, cam, sh_mode=True, sh_degree=3, want_tiles=True, want_ddir
         ptr(o["clamped"]), ptr(o["tiles_touched"]) if want_tiles else None, P, sh_degree, M, W, H, ptr(gd["means3D"]),
         ptr(gd["scales"]), ptr(gd["rotations"]), ptr(gd["shs"]) if sh_mode else None, ptr(gd["opacities"]), 1.0,
         ptr(V), ptr(PM), ptr(cp), cam.tanfovx, cam.tanfovy, 0, 1, ptr(o["dcolor_ddir"]) if want_ddir else None,
-        stream()), "gs_preprocess_forward")
+        None, stream()), "gs_preprocess_forward")
     torch.cuda.synchronize()
     return o, gd
 

@@ -82,7 +82,7 @@ def test_layouts_and_capacities_at_the_instance_limit():
 def test_argument_validation_without_a_gpu():
     import gsrast_native as gn
     assert gn.lib.gs_preprocess_forward(*([None] * 8), 10, 3, 16, 0, 480, *([None] * 5), 1.0, None, None, None, 0.5, 0.5,
-                                        0, 0, None, None) != 0
+                                        0, 0, None, None, None) != 0
     assert "bad sizes" in gn.last_error()
     assert gn.lib.gs_sort_pairs_u64(5, None, None, None, None, 70, None, 0, None) != 0
     assert "end_bit" in gn.last_error()

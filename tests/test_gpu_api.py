@@ -427,6 +427,71 @@ def test_debug_mode_gives_the_same_results_by_every_route():
         assert torch.equal(a, b)
 
 
+@pytest.mark.parametrize("geo", [True, False])
+def test_records_written_by_the_producers_give_the_same_results(geo):
+    """From the second view of an image size on, preprocess_gaussians starts the blend kernels' operand records and
+    build_all_map(..., blend_records_of=means2D) finishes them, so that render_gaussians packs nothing.  Outputs and
+    gradients are the bits of the first view (whose records the library packed); a tensor that is replaced or
+    modified on the way makes render_gaussians fall back to packing, again with the same bits."""
+    import gs_scenes
+    import diff_gaussian_rasterization as dgr
+    import gsrast_native as gn
+    g, cams = gs_scenes.make_scene(1, P=40_000, n_views=1)
+    cam = cams[0]
+    W, H = cam.image_width, cam.image_height
+    gx, gy = (W + 15) // 16, (H + 15) // 16
+    cl = torch.ones(gy, gx, dtype=torch.bool, device=DEV)
+    ug = {k: v.to(DEV) for k, v in gs_scenes.upstream_grads(cam).items()}
+    dgr._expectations.clear()
+    dgr._linked_all_map_seen[0] = False
+
+    def run(disturb=None):
+        rs = _settings(cam, render_geo=geo)
+        rast = dgr.GaussianRasterizer(rs)
+        leaf = {k: g[k].to(DEV).requires_grad_(True) for k in ("means3D", "scales", "rotations", "opacities", "shs")}
+        args = _cuda_args()
+        means2D, rgb, co, radii, depths = rast.preprocess_gaussians(
+            leaf["means3D"], leaf["scales"], leaf["rotations"], leaf["shs"], leaf["opacities"], args)
+        started = getattr(means2D, "_gs_blend", None) is not None
+        am = dgr.build_all_map(leaf["means3D"], leaf["scales"], leaf["rotations"], rs.viewmatrix, rs.campos,
+                               blend_records_of=means2D)
+        if disturb == "replace":
+            am = am * 1.0  # the same values in another tensor
+        elif disturb == "modify":
+            with torch.no_grad():
+                rgb.mul_(1.0)  # (an in-place operation on one of the tensors the records were written from)
+        m2abs = torch.zeros_like(leaf["means3D"], requires_grad=True) + 0
+        gn.stage_timing(True)
+        color, n_render, n_consider, n_contrib, obs, oam, opd = rast.render_gaussians(
+            means2D, m2abs, co, rgb, am, depths, radii, cl, cl, args)
+        torch.autograd.backward([color, oam, opd] if geo else [color],
+                                [ug["color"], ug["all_map"], ug["plane_depth"]] if geo else [ug["color"]])
+        torch.cuda.synchronize()
+        gn.stage_timing(False)
+        packed_by_library = gn.stage_timing_collect().get("pack_operands", (0.0, 0))[1] > 0
+        outs = [color, n_render, n_consider, n_contrib, obs, oam, opd] + [leaf[k].grad for k in sorted(leaf)]
+        return started, packed_by_library, outs
+
+    started, packed_by_library, first = run()
+    assert not started and packed_by_library  # nothing is known about this image size yet
+    used = 0
+    for disturb in (None, None, "replace", None, None, "modify", None, None):
+        started, packed_by_library, again = run(disturb)
+        if disturb == "modify" or not started:
+            assert packed_by_library, disturb
+        elif disturb is None:
+            assert not packed_by_library
+            used += 1
+        elif disturb == "replace":
+            # (with no geometry channels to render, the all_map tensor is not part of the records)
+            assert packed_by_library == geo
+        for a, b in zip(first, again):
+            assert torch.equal(a, b), disturb
+    assert used >= 3
+    dgr._expectations.clear()
+    dgr._linked_all_map_seen[0] = False
+
+
 @pytest.mark.parametrize("poison", [False, True])
 def test_packed_and_gathered_operands_give_the_same_results(poison):
     """The forward call packs the blend kernels' operands into one record per Gaussian when the view has more than
