@@ -609,8 +609,8 @@ def main():
     if os.path.exists(tpath):
         try:
             tj0 = json.load(open(tpath))
-            traffic = (tj0.get("preprocess_fwd_kernel<true>") or tj0.get("preprocess_fwd_kernel", {})).get(
-                "bytes_per_launch")
+            traffic = (tj0.get("preprocess_fwd_kernel<true, false>") or tj0.get("preprocess_fwd_kernel<true>")
+                       or {}).get("bytes_per_launch")
         except (OSError, ValueError):
             traffic = None
     pf = stage_report.get("preprocess_fwd", {})

@@ -18,10 +18,6 @@
 #include "gs_kernels.h"
 #include "tile_lists.h"
 
-#ifndef TR_MARK
-#define TR_MARK(i)
-#endif
-
 namespace gs {
 namespace {
 
@@ -86,7 +82,6 @@ __device__ __forceinline__ void radix_block_pass(const uint64_t (&rec)[ITEMS], u
     L.count[i] = 0u;
   }
   __syncthreads();
-  TR_MARK(1);
   // LDS operations of one wave execute in program order, which the two steps rely on; none of them waits for an
   // earlier one's result, so the items of a batch are in flight together.
   volatile lds_mask* vmask = s_mask + wave * TR_DIGITS;
@@ -153,9 +148,7 @@ __device__ __forceinline__ void radix_block_pass(const uint64_t (&rec)[ITEMS], u
       match[k] = before + (uint32_t)__popcll(lower);
     }
   }
-  TR_MARK(2);
   __syncthreads();
-  TR_MARK(3);
   // thread d < 256: the block's records of digit d, their first place, and every wave's first place
   uint32_t tot = 0, inc = 0;
   if (tid < TR_DIGITS) {
@@ -181,7 +174,6 @@ __device__ __forceinline__ void radix_block_pass(const uint64_t (&rec)[ITEMS], u
     }
   }
   __syncthreads();
-  TR_MARK(4);
 #pragma unroll
   for (int k = 0; k < ITEMS; k++) {
     if (!valid[k]) continue;
@@ -189,7 +181,6 @@ __device__ __forceinline__ void radix_block_pass(const uint64_t (&rec)[ITEMS], u
     L.rec[L.count[wave * TR_DIGITS + d] + match[k]] = rec[k];
   }
   __syncthreads();
-  TR_MARK(5);
 }
 
 
@@ -249,7 +240,6 @@ __device__ __forceinline__ void sort_resident(uint32_t tile, uint32_t start, uin
       rec[k] = ((uint64_t)depth_bits << 32) | (uint64_t)i;
     }
   }
-  TR_MARK(0);
   workgroup_min_max<WAVES>(dmin, dmax, L.scan, L.total);
   const int passes = passes_for_range(dmax - dmin);
 #pragma unroll
@@ -304,7 +294,6 @@ __device__ __forceinline__ void sort_resident(uint32_t tile, uint32_t start, uin
     if (i < n) L.rec[i] = rec[k];
   }
   __syncthreads();
-  TR_MARK(6);
   const lds_u64* sorted = L.rec;
 #pragma unroll 1
   for (int k = 0; k < ITEMS; k++) {
@@ -313,7 +302,6 @@ __device__ __forceinline__ void sort_resident(uint32_t tile, uint32_t start, uin
       emit_list_entry(tile, start, n, i, gaussian[k], [&](uint32_t q) { return sorted[q]; }, keys, emission,
                       point_list);
   }
-  TR_MARK(7);
 }
 
 // A list of more than `blk` records (blk <= BLOCK): up to four passes over its blocks, the first from the segment's
