@@ -179,8 +179,9 @@ typedef struct gs_render_result {
  * elapsed_ms (host, optional): if non-NULL the call times key emission + sort
  * + blend with events and blocks until done (the forward_render_time the
  * reference stores at CR/rasterizer_impl.cu:754-755).
- * The geometry buffer is asked for 72 bytes per Gaussian plus the prefix sum's workspace (the reference's holds the
- * preprocess outputs as well, CR/rasterizer_impl.cu:160-188; here those are the caller's tensors). */
+ * The geometry buffer is asked for 72 bytes per Gaussian (tile counts, their prefix sum, and room for the blend
+ * operand records, reserved whether or not this call packs them) plus the prefix sum's workspace (the reference's
+ * holds the preprocess outputs as well, CR/rasterizer_impl.cu:160-188; here those are the caller's tensors). */
 int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resize_fn binningBuffer,
                       void* binning_user, gs_resize_fn imageBuffer, void* image_user, int P,
                       const float* background, int width, int height, float focal_x, float focal_y, float cx,

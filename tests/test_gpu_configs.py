@@ -279,7 +279,7 @@ def test_config3_full_size_all_views_forward_and_backward_with_geometry(H):
         assert (cam.image_width, cam.image_height) == (1920, 1080)
         r = _full_size_view(H, d, cam, v)
         longest = max(longest, r["longest"])
-    assert longest > 8192  # the regime in which a list no longer fits one workgroup's sort
+    assert longest > 8192  # the regime of the per-tile radix sort's larger kernel
 
 
 @pytest.mark.timeout(900)

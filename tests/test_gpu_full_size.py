@@ -164,27 +164,26 @@ def test_list_routes_agree_at_full_size(H, cfg, P):
     T = gx * gy
     cl = torch.ones(gy, gx, dtype=torch.bool, device=DEV)
     results = []
-    if True:
-        for limits in [(0, 0), (-1, -1), (256, 0), (-1, 3000)]:
-            args["tile_sort_limits"] = limits
-            out = _C.render_gaussians(torch.zeros(3, device=DEV), Hh, W, means2D, depths, radii, co, rgb, cl, vm, cp,
-                                      cam.tanfovx, cam.tanfovy, am, False, False, args)
-            R, color, n_render, binB, imgB = out[0], out[1], out[2], out[9], out[10]
-            off = [C.c_size_t() for _ in range(5)]
-            gn.check(gn.lib.gs_binning_state_layout(R, W, Hh, *[C.byref(o) for o in off]), "layout")
-            base = (binB.data_ptr() + 255) // 256 * 256 - binB.data_ptr()
-            point_list = binB[base + off[0].value: base + off[0].value + 4 * R].view(torch.int32).clone()
-            keys = binB[base + off[1].value: base + off[1].value + 8 * R].view(torch.int64).clone()
-            ioff = [C.c_size_t() for _ in range(5)]
-            gn.check(gn.lib.gs_image_state_layout(W, Hh, *[C.byref(o) for o in ioff]), "layout")
-            ibase = (imgB.data_ptr() + 255) // 256 * 256 - imgB.data_ptr()
-            ranges = imgB[ibase + ioff[3].value: ibase + ioff[3].value + 8 * T].view(torch.int32).clone()
-            results.append((limits, R, keys, point_list, ranges, color.clone(), n_render.clone()))
-            del out, binB, imgB
+    for limits in [(0, 0), (-1, -1), (256, 0), (-1, 3000)]:
+        args["tile_sort_limits"] = limits
+        out = _C.render_gaussians(torch.zeros(3, device=DEV), Hh, W, means2D, depths, radii, co, rgb, cl, vm, cp,
+                                  cam.tanfovx, cam.tanfovy, am, False, False, args)
+        R, color, n_render, binB, imgB = out[0], out[1], out[2], out[9], out[10]
+        off = [C.c_size_t() for _ in range(5)]
+        gn.check(gn.lib.gs_binning_state_layout(R, W, Hh, *[C.byref(o) for o in off]), "layout")
+        base = (binB.data_ptr() + 255) // 256 * 256 - binB.data_ptr()
+        point_list = binB[base + off[0].value: base + off[0].value + 4 * R].view(torch.int32).clone()
+        keys = binB[base + off[1].value: base + off[1].value + 8 * R].view(torch.int64).clone()
+        ioff = [C.c_size_t() for _ in range(5)]
+        gn.check(gn.lib.gs_image_state_layout(W, Hh, *[C.byref(o) for o in ioff]), "layout")
+        ibase = (imgB.data_ptr() + 255) // 256 * 256 - imgB.data_ptr()
+        ranges = imgB[ibase + ioff[3].value: ibase + ioff[3].value + 8 * T].view(torch.int32).clone()
+        results.append((limits, R, keys, point_list, ranges, color.clone(), n_render.clone()))
+        del out, binB, imgB
     _, R0, keys0, pl0, ranges0, color0, nr0 = results[0]
     assert R0 > 1_000_000
     if cfg == 3:
-        assert int(nr0.max()) > 8192  # so that the third and fourth settings really merge chunks
+        assert int(nr0.max()) > 8192  # so that the last setting really goes block by block through memory
     for limits, R, keys, pl, ranges, color, nr in results[1:]:
         assert R == R0, limits
         assert torch.equal(ranges, ranges0), limits
