@@ -42,12 +42,12 @@ inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 // ------------------------------------------------------------ device math --
 
 __device__ __forceinline__ int f2i_sat(float v) {
-  // float -> int32 with the conversion instruction's semantics spelled out:
-  // truncate toward zero, clamp to the int32 range, NaN -> 0.
-  if (!(v == v)) return 0;
-  if (v >= 2147483648.0f) return 2147483647;
-  if (v <= -2147483648.0f) return (-2147483647 - 1);
-  return (int)v;
+  // float -> int32: truncate toward zero, clamp to the int32 range, NaN -> 0.  That is what the conversion
+  // instruction does by itself; as C++ (three comparisons around a cast, whose out-of-range cases the language
+  // leaves undefined) it came out as three nested branches per conversion.
+  int r;
+  asm("v_cvt_i32_f32 %0, %1" : "=v"(r) : "v"(v));
+  return r;
 }
 
 // Workgroups go to the eight XCDs in turn (workgroup b of a launch runs on XCD b % 8), and each XCD has its own L2.
@@ -60,10 +60,10 @@ __device__ __forceinline__ uint32_t xcd_contiguous_index(uint32_t b, uint32_t n)
 }
 
 __device__ __forceinline__ uint32_t f2u_sat(float v) {
-  if (!(v == v)) return 0u;
-  if (v >= 4294967296.0f) return 0xFFFFFFFFu;
-  if (v <= 0.0f) return 0u;
-  return (uint32_t)v;
+  // float -> uint32: truncate, clamp to [0, 2^32 - 1], NaN -> 0 (the conversion instruction's own behaviour)
+  uint32_t r;
+  asm("v_cvt_u32_f32 %0, %1" : "=v"(r) : "v"(v));
+  return r;
 }
 
 // Store for data that is written once and not read again on the GPU for a long while (gradients of leaf
@@ -254,6 +254,109 @@ __device__ __forceinline__ uint32_t walk_wave_rects(bool live, const Rect& rc, u
       }
   }
   return count;
+}
+
+// Inclusive scans over the 64 lanes of a wave by DPP moves: four shifts inside the 16-lane rows, then the last
+// lane of rows 0 and 2 goes to rows 1 and 3 and lane 31 to rows 2 and 3 (a lane without a source takes the
+// identity, 0).  All 64 lanes must be active.
+#define GS_WAVE_SCAN_STEP(OP, CTRL, ROWS) \
+  v = OP(v, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, ROWS, 0xF, false))
+__device__ __forceinline__ uint32_t gs_scan_add_op(uint32_t a, uint32_t b) { return a + b; }
+__device__ __forceinline__ uint32_t gs_scan_max_op(uint32_t a, uint32_t b) { return a > b ? a : b; }
+__device__ __forceinline__ uint32_t wave_scan_add(uint32_t v) {
+  GS_WAVE_SCAN_STEP(gs_scan_add_op, 0x111, 0xF);  // row_shr:1
+  GS_WAVE_SCAN_STEP(gs_scan_add_op, 0x112, 0xF);  // row_shr:2
+  GS_WAVE_SCAN_STEP(gs_scan_add_op, 0x114, 0xF);  // row_shr:4
+  GS_WAVE_SCAN_STEP(gs_scan_add_op, 0x118, 0xF);  // row_shr:8
+  GS_WAVE_SCAN_STEP(gs_scan_add_op, 0x142, 0xA);  // row_bcast:15 into rows 1 and 3
+  GS_WAVE_SCAN_STEP(gs_scan_add_op, 0x143, 0xC);  // row_bcast:31 into rows 2 and 3
+  return v;
+}
+__device__ __forceinline__ uint32_t wave_scan_max(uint32_t v) {
+  GS_WAVE_SCAN_STEP(gs_scan_max_op, 0x111, 0xF);
+  GS_WAVE_SCAN_STEP(gs_scan_max_op, 0x112, 0xF);
+  GS_WAVE_SCAN_STEP(gs_scan_max_op, 0x114, 0xF);
+  GS_WAVE_SCAN_STEP(gs_scan_max_op, 0x118, 0xF);
+  GS_WAVE_SCAN_STEP(gs_scan_max_op, 0x142, 0xA);
+  GS_WAVE_SCAN_STEP(gs_scan_max_op, 0x143, 0xC);
+  return v;
+}
+#undef GS_WAVE_SCAN_STEP
+
+// A pointer into LDS typed as such: volatile accesses through a plain pointer come out as flat loads and stores.
+typedef __attribute__((address_space(3))) uint32_t lds_word;
+
+// walk_wave_rects for a wave all of whose tiles are computed locally (no tile mask), with the work spread evenly:
+// the rectangles of at most GS_BIG_RECT tiles are laid end to end (a prefix sum of their areas over the lanes) and
+// lane l of round k takes instance 64 k + l of that sequence, whichever Gaussian it belongs to, instead of every
+// lane looping over its own rectangle while the lanes with smaller ones wait.  The owner of an instance is found
+// through `heads` (64 words of LDS of the wave's own): every owner enters its lane number at the place of its
+// first instance, and a running maximum over the places carries it to the instances behind.  What visit needs of
+// the owner comes by cross-lane reads.  rank = the instance's place in its rectangle's row-major order, which
+// with every tile local is the rank walk_wave_rects gives.  Larger rectangles are walked as there.
+template <typename Payload, typename Visit>
+__device__ __forceinline__ uint32_t walk_wave_rects_flat(bool live, const Rect& rc, uint32_t gx, const Payload& mine,
+                                                         lds_word* heads, Visit visit) {
+  static_assert(sizeof(Payload) % 4 == 0, "payload of 32-bit words");
+  static_assert(GS_BIG_RECT <= 16, "areas and ranks are packed into 5 and 11 bits");
+  const int lane = threadIdx.x & (GS_WAVE - 1);
+  const uint32_t w = live ? rc.x1 - rc.x0 : 0u, h = live ? rc.y1 - rc.y0 : 0u;
+  const uint32_t area = w * h;
+  uint64_t big = __ballot(area > GS_BIG_RECT);
+  while (big != 0ull) {
+    const int owner = (int)__builtin_ctzll(big);
+    big &= big - 1ull;
+    const uint32_t ox0 = __shfl(rc.x0, owner, GS_WAVE), oy0 = __shfl(rc.y0, owner, GS_WAVE);
+    const uint32_t ow = __shfl(w, owner, GS_WAVE), on = __shfl(area, owner, GS_WAVE);
+    Payload theirs;
+    {
+      const uint32_t* src = reinterpret_cast<const uint32_t*>(&mine);
+      uint32_t* dst = reinterpret_cast<uint32_t*>(&theirs);
+#pragma unroll
+      for (int k = 0; k < (int)(sizeof(Payload) / 4); k++) dst[k] = __shfl(src[k], owner, GS_WAVE);
+    }
+    for (uint32_t q0 = 0; q0 < on; q0 += GS_WAVE) {
+      const uint32_t q = q0 + (uint32_t)lane;
+      const uint32_t ry = q / ow, rx = q - ry * ow;
+      if (q < on) visit(theirs, (oy0 + ry) * gx + (ox0 + rx), q);
+    }
+  }
+  const uint32_t small = area <= GS_BIG_RECT ? area : 0u;
+  const uint32_t incl = wave_scan_add(small), excl = incl - small;
+  const uint32_t total = (uint32_t)__builtin_amdgcn_readlane((int)incl, GS_WAVE - 1);
+  // what an instance needs of its owner: the rectangle's corner, and in one word its width (5 bits), the place of
+  // its first instance (11 bits) and m = floor(2^15 / width) + 1, with which (q m) >> 15 = q / width for q < 16
+  const uint32_t corner = rc.x0 | (rc.y0 << 16);
+  const uint32_t m = w != 0u ? (uint32_t)(32768.0f / (float)w) + 1u : 0u;  // (exact: w <= 16)
+  const uint32_t shape = w | (excl << 5) | (m << 16);
+  volatile lds_word* vheads = heads;
+  uint32_t carried = 0;  // owner of the last instance of the previous round, plus one
+  for (uint32_t base = 0; base < total; base += GS_WAVE) {
+    vheads[lane] = 0u;
+    __builtin_amdgcn_wave_barrier();
+    if (small != 0u && excl >= base && excl < base + GS_WAVE) vheads[excl - base] = (uint32_t)lane + 1u;
+    __builtin_amdgcn_wave_barrier();
+    uint32_t owner1 = wave_scan_max(vheads[lane]);
+    __builtin_amdgcn_wave_barrier();
+    owner1 = owner1 > carried ? owner1 : carried;
+    carried = (uint32_t)__builtin_amdgcn_readlane((int)owner1, GS_WAVE - 1);
+    const int src_lane = (int)owner1 - 1;  // (at least 0: the first instance of the sequence is a head)
+    const uint32_t o_corner = __shfl(corner, src_lane, GS_WAVE), o_shape = __shfl(shape, src_lane, GS_WAVE);
+    Payload theirs;
+    {
+      const uint32_t* src = reinterpret_cast<const uint32_t*>(&mine);
+      uint32_t* dst = reinterpret_cast<uint32_t*>(&theirs);
+#pragma unroll
+      for (int k = 0; k < (int)(sizeof(Payload) / 4); k++) dst[k] = __shfl(src[k], src_lane, GS_WAVE);
+    }
+    const uint32_t slot = base + (uint32_t)lane;
+    if (slot < total) {
+      const uint32_t ow = o_shape & 31u, q = slot - ((o_shape >> 5) & 2047u);
+      const uint32_t ry = (q * (o_shape >> 16)) >> 15, rx = q - ry * ow;
+      visit(theirs, ((o_corner >> 16) + ry) * gx + ((o_corner & 0xFFFFu) + rx), q);
+    }
+  }
+  return area;
 }
 
 }  // namespace gs

@@ -49,14 +49,20 @@ bucket_count_kernel(int P, int per_block, uint32_t gx, uint32_t gy, const int* _
                     uint32_t* __restrict__ block_sums, int* __restrict__ zero_per_gaussian) {
   extern __shared__ uint32_t s_hist[];
   __shared__ uint32_t s_sum[BK_THREADS / GS_WAVE];
+  __shared__ uint32_t s_heads[BK_THREADS];
   uint32_t my_sum = 0;  // tiles touched by this thread's Gaussians
   const uint32_t T = gx * gy;
   uint8_t* s_local = reinterpret_cast<uint8_t*>(s_hist + T);  // the tile mask, read once per visited tile
+  int masked = 0;
   for (uint32_t t = threadIdx.x; t < T; t += BK_THREADS) {
     s_hist[t] = 0u;
-    s_local[t] = compute_locally[t];
+    const uint8_t c = compute_locally[t];
+    s_local[t] = c;
+    masked |= c == 0 ? 1 : 0;
   }
-  __syncthreads();
+  // (also the barrier behind the loop) without a tile mask the rectangles are walked with the work spread evenly
+  const bool all_local = __syncthreads_or(masked) == 0;
+  lds_word* heads = (lds_word*)s_heads + (threadIdx.x / GS_WAVE) * GS_WAVE;
   const int chunk = chunk_of_workgroup(blockIdx.x, gridDim.x);
   const int first = chunk * per_block;
   const int last = first + per_block < P ? first + per_block : P;
@@ -77,9 +83,12 @@ bucket_count_kernel(int P, int per_block, uint32_t gx, uint32_t gy, const int* _
       const int i = base + (int)threadIdx.x + q * BK_THREADS;
       const bool live = i < last && r[q] > 0;
       const Rect rc = live ? get_rect(p[q].x, p[q].y, r[q], gx, gy) : Rect{0u, 0u, 0u, 0u};
-      const uint32_t cnt = walk_wave_rects(
-          live, rc, gx, none, [&](uint32_t tile) { return s_local[tile] != 0; },
-          [&](const None&, uint32_t tile, uint32_t) { atomicAdd(&s_hist[tile], 1u); });
+      const uint32_t cnt =
+          all_local ? walk_wave_rects_flat(live, rc, gx, none, heads,
+                                           [&](const None&, uint32_t tile, uint32_t) { atomicAdd(&s_hist[tile], 1u); })
+                    : walk_wave_rects(
+                          live, rc, gx, none, [&](uint32_t tile) { return s_local[tile] != 0; },
+                          [&](const None&, uint32_t tile, uint32_t) { atomicAdd(&s_hist[tile], 1u); });
       if (i < last) {
         tiles_touched[i] = cnt;
         my_sum += cnt;
@@ -279,17 +288,22 @@ bucket_scatter_kernel(int P, int per_block, uint32_t gx, uint32_t gy, const floa
                       int vector_loads) {
   extern __shared__ uint32_t s_next[];
   __shared__ uint32_t s_wave[BK_THREADS / GS_WAVE];
+  __shared__ uint32_t s_heads[BK_THREADS];
   if (fits_word != nullptr && *fits_word == 0u) return;
   const uint32_t T = gx * gy;
   uint8_t* s_local = reinterpret_cast<uint8_t*>(s_next + T);
   const int chunk = chunk_of_workgroup(blockIdx.x, gridDim.x);
   const uint32_t* row = table + (size_t)chunk * T;
+  int masked = 0;
   for (uint32_t t = threadIdx.x; t < T; t += BK_THREADS) {
     s_next[t] = ranges[2 * t] + row[t];
-    s_local[t] = compute_locally[t];
+    const uint8_t c = compute_locally[t];
+    s_local[t] = c;
+    masked |= c == 0 ? 1 : 0;
   }
-  __syncthreads();
+  const bool all_local = __syncthreads_or(masked) == 0;  // (as in the counting kernel; also the barrier)
   const int lane = threadIdx.x & (GS_WAVE - 1), wave = threadIdx.x / GS_WAVE;
+  lds_word* heads = (lds_word*)s_heads + wave * GS_WAVE;
   const int first = chunk * per_block;
   const int last = first + per_block < P ? first + per_block : P;
   struct Owner { uint32_t first, depth_bits, id; };
@@ -346,13 +360,13 @@ bucket_scatter_kernel(int P, int per_block, uint32_t gx, uint32_t gy, const floa
       const Owner mine = {run, dbits[q], (uint32_t)i};
       run += tt[q];
       tt[q] = run;  // from here on: the inclusive sum
-      walk_wave_rects(
-          live, rc, gx, mine, [&](uint32_t tile) { return s_local[tile] != 0; },
-          [&](const Owner& o, uint32_t tile, uint32_t rank) {
-            const uint32_t e = o.first + rank;
-            const uint32_t pos = atomicAdd(&s_next[tile], 1u);
-            records[pos] = make_uint4(o.id, e, o.depth_bits, 0u);
-          });
+      const auto emit = [&](const Owner& o, uint32_t tile, uint32_t rank) {
+        const uint32_t e = o.first + rank;
+        const uint32_t pos = atomicAdd(&s_next[tile], 1u);
+        records[pos] = make_uint4(o.id, e, o.depth_bits, 0u);
+      };
+      if (all_local) walk_wave_rects_flat(live, rc, gx, mine, heads, emit);
+      else walk_wave_rects(live, rc, gx, mine, [&](uint32_t tile) { return s_local[tile] != 0; }, emit);
     }
     if (whole) {
       *reinterpret_cast<uint4*>(point_offsets + i0) = make_uint4(tt[0], tt[1], tt[2], tt[3]);
