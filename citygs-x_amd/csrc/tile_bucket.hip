@@ -379,21 +379,28 @@ bucket_scatter_kernel(int P, int per_block, uint32_t gx, uint32_t gy, const floa
 }
 
 // 2. Per-tile sort, register variant: one workgroup of W waves per tile (4 for lists of up to 256 records, 8 up
-// to 2048, 16 for longer ones).  A wave holds 64 E records, record i = r * 64 + lane in register r of its lane, and
-// the waves hold consecutive runs of 64 E, so a list of up to 64 E W records is sorted with E = 1 .. 8.  In the
-// bitonic network a step pairs i with i ^ j:
+// to 2048).  A wave holds 64 E keys, key i = r * 64 + lane in register r of its lane, and the waves hold
+// consecutive runs of 64 E, so a list of up to 64 E W records is sorted with E = 1 .. 4.  In the bitonic network
+// a step pairs i with i ^ j:
 //   j < 64        the partner sits in another lane, same register: one cross-lane read, keep the smaller or larger;
 //   64 <= j < 64E the partner sits in another register of the same lane: no data moves at all;
 //   j >= 64 E     the partner sits in another wave: one exchange through LDS (3 such steps in a whole sort with
-//                 4 waves, 6 with 8, 10 with 16).
+//                 4 waves, 6 with 8).
 // A tile takes as long as the instruction stream of one of its waves, and the kernel as long as its longest tiles:
 // a long list is spread over more waves rather than more registers per lane (eight waves with four records per
-// lane for 2048 records, not four with eight).  Sixteen waves for every list were measured too: the launch of so
-// many waves that leave at once costs more than the shorter streams save.
+// lane for 2048 records, not four with eight).
+//
+// The key is one 32-bit word: (depth bits - smallest depth bits of the list) >> shift in the high bits, the
+// record's place in the unsorted segment in the low log2(64 E W) bits; shift is what it takes to fit the list's
+// range of depth bits (0 when it fits as it is).  A step then costs three vector instructions per key (one move,
+// one comparison, one select) where a 64-bit key cost five.  Keys whose depths agree in the bits kept end up next
+// to each other in the order of their places; the last step (emit_list_entry) puts every such run into its true
+// order, by all depth bits and then the emission index, exactly as it does for runs of equal depth bits.  Depths
+// inside a tile are spread over the view's range, so with the 21 to 24 bits kept runs are as rare as before.
 
 // Which element of a pair (a, b) each lane keeps is decided in scalar registers: keep_min is the lane mask of the
 // elements that keep the smaller one, less the lane mask of a < b; a lane keeps a where the two agree.
-__device__ __forceinline__ uint64_t keep_pair(uint64_t a, uint64_t b, uint64_t keep_min) {
+__device__ __forceinline__ uint32_t keep_pair(uint32_t a, uint32_t b, uint64_t keep_min) {
   const uint64_t less = __builtin_amdgcn_ballot_w64(a < b);
   return __builtin_amdgcn_inverse_ballot_w64(~(less ^ keep_min)) ? a : b;
 }
@@ -429,40 +436,31 @@ __device__ __forceinline__ uint32_t xor_lane(uint32_t x) {
 // One step of the network with the partner in lane ^ J.  ascending[r]: lane mask of the elements of register r
 // that lie in an ascending run of this stage.
 template <int E, int J>
-__device__ __forceinline__ void lane_step(uint64_t (&v)[E], const uint64_t (&ascending)[E]) {
+__device__ __forceinline__ void lane_step(uint32_t (&v)[E], const uint64_t (&ascending)[E]) {
   constexpr uint64_t lower = lower_lanes<J>();
 #pragma unroll
   for (int r = 0; r < E; r++) {
     const uint64_t keep_min = ~(lower ^ ascending[r]);  // the lower element of an ascending pair, the upper of a descending
     if constexpr (J < 16) {
-      const uint32_t lo = xor_lane<J>((uint32_t)v[r]);
-      const uint32_t hi = xor_lane<J>((uint32_t)(v[r] >> 32));
-      v[r] = keep_pair(v[r], ((uint64_t)hi << 32) | lo, keep_min);
+      v[r] = keep_pair(v[r], xor_lane<J>(v[r]), keep_min);
     } else {
       // v_permlane16_swap / v_permlane32_swap exchange the odd rows (the upper half) of their first operand with
       // the even rows (the lower half) of the second: from two copies of x they leave the lower element of every
       // pair in all lanes of the first result and the upper element in the second, so both lanes of a pair
       // compare the same two values and each keeps its own.
-      const uint32_t xl = (uint32_t)v[r], xh = (uint32_t)(v[r] >> 32);
-      uint64_t a, b;
       if constexpr (J == 16) {
-        const auto l = __builtin_amdgcn_permlane16_swap(xl, xl, false, false);
-        const auto h = __builtin_amdgcn_permlane16_swap(xh, xh, false, false);
-        a = ((uint64_t)h[0] << 32) | l[0];
-        b = ((uint64_t)h[1] << 32) | l[1];
+        const auto p = __builtin_amdgcn_permlane16_swap(v[r], v[r], false, false);
+        v[r] = keep_pair(p[0], p[1], keep_min);
       } else {
-        const auto l = __builtin_amdgcn_permlane32_swap(xl, xl, false, false);
-        const auto h = __builtin_amdgcn_permlane32_swap(xh, xh, false, false);
-        a = ((uint64_t)h[0] << 32) | l[0];
-        b = ((uint64_t)h[1] << 32) | l[1];
+        const auto p = __builtin_amdgcn_permlane32_swap(v[r], v[r], false, false);
+        v[r] = keep_pair(p[0], p[1], keep_min);
       }
-      v[r] = keep_pair(a, b, keep_min);
     }
   }
 }
 
 template <int E, int W>
-__device__ __forceinline__ void register_sort(uint64_t (&v)[E], uint32_t wave, uint32_t lane, uint64_t* s_x) {
+__device__ __forceinline__ void register_sort(uint32_t (&v)[E], uint32_t wave, uint32_t lane, uint32_t* s_x) {
   constexpr uint32_t M = 64u * E * W;
   const uint32_t row0 = wave * E;
   for (uint32_t k = 2; k <= M; k <<= 1) {
@@ -489,7 +487,7 @@ __device__ __forceinline__ void register_sort(uint64_t (&v)[E], uint32_t wave, u
           for (int r = 0; r < E; r++) {
             if (r & b) continue;
             // (both registers of a pair lie in the same run)
-            const uint64_t x = v[r], y = v[r | b];
+            const uint32_t x = v[r], y = v[r | b];
             const uint64_t less = __builtin_amdgcn_ballot_w64(x < y);
             const bool x_first = __builtin_amdgcn_inverse_ballot_w64(~(less ^ ascending[r]));
             v[r] = x_first ? x : y;
@@ -506,7 +504,7 @@ __device__ __forceinline__ void register_sort(uint64_t (&v)[E], uint32_t wave, u
         const bool lower = (wave & jw) == 0;
 #pragma unroll
         for (int r = 0; r < E; r++) {
-          const uint64_t other = s_x[(((wave ^ jw) * E + r) << 6) | lane];
+          const uint32_t other = s_x[(((wave ^ jw) * E + r) << 6) | lane];
           v[r] = keep_pair(v[r], other, lower ? ascending[r] : ~ascending[r]);
         }
       }
@@ -521,37 +519,73 @@ __device__ __forceinline__ void register_sort(uint64_t (&v)[E], uint32_t wave, u
   }
 }
 
-// Sorts (depth bits << 32 | place in the segment) and hands every entry to emit_list_entry, which puts runs of
-// equal depth bits into emission order.  s_x: at least 64 E W words.
+// Sorts the tile's one-word keys and hands every entry to emit_list_entry, which puts runs of keys with the same
+// depth field into their order by all depth bits and then emission index.  s_x: at least 64 E W 8-byte words.
 template <int E, int W>
 __device__ __forceinline__ void register_sort_tile(uint32_t t, uint32_t start, uint32_t n,
                                                    const TileRecord* __restrict__ records,
                                                    uint64_t* __restrict__ keys, uint32_t* __restrict__ emission,
                                                    uint32_t* __restrict__ point_list, uint64_t* s_x) {
+  constexpr uint32_t M = 64u * E * W;
+  constexpr int PLACE_BITS = M == 256 ? 8 : M == 512 ? 9 : M == 1024 ? 10 : 11;
+  static_assert(M == 1u << PLACE_BITS, "a list of 256 to 2048 places");
   const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  uint64_t v[E];
+  uint32_t* s_words = reinterpret_cast<uint32_t*>(s_x);
+  uint32_t v[E];
+  uint32_t lo = 0xFFFFFFFFu, hi = 0u;
 #pragma unroll
   for (int r = 0; r < E; r++) {
     const uint32_t i = ((wave * E + r) << 6) | lane;
-    v[r] = i < n ? ((uint64_t)records[start + i].z << 32) | (uint64_t)i : ~0ull;
+    v[r] = i < n ? records[start + i].z : 0u;
+    if (i < n) {
+      lo = v[r] < lo ? v[r] : lo;
+      hi = v[r] > hi ? v[r] : hi;
+    }
   }
-  register_sort<E, W>(v, wave, lane, s_x);
+  // smallest and largest depth bits of the list: over the wave by a scan (its last lane holds the result), over
+  // the waves through LDS
+  lo = ~(uint32_t)__builtin_amdgcn_readlane((int)wave_scan_max(~lo), GS_WAVE - 1);
+  hi = (uint32_t)__builtin_amdgcn_readlane((int)wave_scan_max(hi), GS_WAVE - 1);
+  if (lane == 0) {
+    s_words[wave] = lo;
+    s_words[W + wave] = hi;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int w = 0; w < W; w++) {
+    const uint32_t a = s_words[w], b = s_words[W + w];
+    lo = a < lo ? a : lo;
+    hi = b > hi ? b : hi;
+  }
+  const uint32_t range = hi - lo;  // (n >= 1, so lo <= hi)
+  const int range_bits = range != 0u ? 32 - __builtin_clz(range) : 0;
+  const uint32_t shift = range_bits + PLACE_BITS > 32 ? (uint32_t)(range_bits + PLACE_BITS - 32) : 0u;
+#pragma unroll
+  for (int r = 0; r < E; r++) {
+    const uint32_t i = ((wave * E + r) << 6) | lane;
+    v[r] = i < n ? ((((v[r] - lo) >> shift) << PLACE_BITS) | i) : 0xFFFFFFFFu;
+  }
+  // (a real key is below the padding's: a key of all ones would be the list's last place, which is padding
+  // unless the list fills all M places, and then there is none)
+  register_sort<E, W>(v, wave, lane, s_words);  // (starts its first exchange behind a barrier: lo and hi are read)
   uint32_t gaussian[E];
+  uint64_t entry[E];
 #pragma unroll
   for (int r = 0; r < E; r++) {
     const uint32_t i = ((wave * E + r) << 6) | lane;
     gaussian[r] = 0u;
+    entry[r] = 0ull;
     if (i < n) {
-      const uint2 ge = *reinterpret_cast<const uint2*>(records + start + (uint32_t)v[r]);
-      gaussian[r] = ge.x;
-      v[r] = (v[r] & 0xFFFFFFFF00000000ull) | (uint64_t)ge.y;
+      const TileRecord rec = records[start + (v[r] & (M - 1u))];
+      gaussian[r] = rec.x;
+      entry[r] = ((uint64_t)rec.z << 32) | (uint64_t)rec.y;
     }
   }
   __syncthreads();  // (the sort's last exchange between waves has been read by everybody)
 #pragma unroll
   for (int r = 0; r < E; r++) {
     const uint32_t i = ((wave * E + r) << 6) | lane;
-    if (i < n) s_x[i] = v[r];
+    if (i < n) s_x[i] = entry[r];
   }
   __syncthreads();
   const uint64_t* sorted = s_x;
@@ -559,7 +593,8 @@ __device__ __forceinline__ void register_sort_tile(uint32_t t, uint32_t start, u
   for (int r = 0; r < E; r++) {
     const uint32_t i = ((wave * E + r) << 6) | lane;
     if (i < n)
-      emit_list_entry(t, start, n, i, gaussian[r], [&](uint32_t q) { return sorted[q]; }, keys, emission, point_list);
+      emit_list_entry(t, start, n, i, gaussian[r], [&](uint32_t q) { return sorted[q]; }, keys, emission, point_list,
+                      lo, shift);
   }
 }
 
