@@ -21,8 +21,15 @@
 namespace gs {
 namespace {
 
-constexpr int TR_DIGITS = 256;
+constexpr int TR_DIGITS = 256;  // digit values of the passes that go through memory and of the split by leading bits
 constexpr int TR_PASSES = 4;
+// Lists that one workgroup holds are sorted on one-word keys: a depth field of TR_FIELD_BITS bits over the
+// record's place in the unsorted list, in two passes (or one) on digits of TR_KEY_DIGIT_BITS bits.
+constexpr int TR_PLACE_BITS = 14;
+constexpr int TR_FIELD_BITS = 32 - TR_PLACE_BITS;
+constexpr int TR_KEY_DIGIT_BITS = 9;
+constexpr int TR_KEY_DIGITS = 1 << TR_KEY_DIGIT_BITS;
+static_assert(2 * TR_KEY_DIGIT_BITS == TR_FIELD_BITS, "two passes cover the depth field");
 
 // Pointers into LDS, typed as such: through a plain pointer the volatile accesses of the ranking come out as
 // flat loads and stores, which are slower and wait on the memory counters as well.
@@ -39,53 +46,81 @@ __device__ __forceinline__ uint32_t tr_wave_inclusive_scan(uint32_t v, int lane)
   return v;
 }
 
-// The workgroup's LDS, carved from one dynamic allocation.
+// What one pass works in: the regrouping buffer (whose head holds the lane masks [WAVES][digits] during the
+// ranking), per wave and digit the running count and then the place of the wave's first such record, per digit
+// the records of the block and the place of the first, and 16 words for the scan over the digits.
+template <typename RecPtr>
+struct PassLds {
+  RecPtr rec;
+  lds_mask* mask;
+  lds_u32* count;
+  lds_u32* total;
+  lds_u32* first;
+  lds_u32* scan;
+};
+
+// The workgroup's LDS, carved from one dynamic allocation.  Two views of the leading region: `rec`, BLOCK 8-byte
+// words (the passes on 64-bit records that go through memory; the last step of every sort), and for the passes on
+// one-word keys `key` (BLOCK words) under the lane masks [WAVES][512] with the counts [WAVES][512] behind them.
 template <int WAVES, int ITEMS>
 struct TileRadixLds {
   static constexpr int THREADS = WAVES * GS_WAVE;
   static constexpr int BLOCK = THREADS * ITEMS;
   static_assert(BLOCK >= WAVES * TR_DIGITS, "the lane masks of the ranking live in the regrouping buffer");
+  static_assert(BLOCK <= WAVES * TR_KEY_DIGITS * 2, "the one-word keys are regrouped under their lane masks");
+  static_assert(BLOCK <= 1 << TR_PLACE_BITS, "a record's place fits the key's low bits");
+  static_assert(THREADS >= TR_KEY_DIGITS, "one thread per digit in the scan");
   static_assert(ITEMS % 4 == 0, "items are ranked four at a time");
-  lds_u64* rec;    // [BLOCK] regrouping buffer; during the ranking its head holds the lane masks [WAVES][256]
-  lds_u32* count;  // [WAVES][256] per wave and digit: running count, then place of the wave's first such record
-  lds_u32* total;  // [256] records of the block per digit
-  lds_u32* first;  // [256] place in the regrouped block of the first record of a digit
-  lds_u32* base;   // [4][256] blocked sort: where the next record of a digit goes in the segment, per pass
-  lds_u32* scan;   // [16]
-  lds_u32* bins;   // [257] partitioned sort: first place of every leading-digit bin in the list, then its length
+  static constexpr size_t LEAD_BYTES =
+      (size_t)BLOCK * 8 > (size_t)WAVES * TR_KEY_DIGITS * 12 ? (size_t)BLOCK * 8 : (size_t)WAVES * TR_KEY_DIGITS * 12;
+  lds_u64* rec;        // [BLOCK]
+  lds_u32* key;        // [BLOCK], the same memory
+  lds_u32* key_count;  // [WAVES][512], behind the masks of the one-word passes
+  lds_u32* count;      // [WAVES][256]
+  lds_u32* total;      // [512]
+  lds_u32* first;      // [512]
+  lds_u32* base;       // [4][256] blocked sort: where the next record of a digit goes in the segment, per pass
+  lds_u32* scan;       // [16]
+  lds_u32* bins;       // [257] partitioned sort: first place of every leading-digit bin in the list, then its length
   __device__ explicit TileRadixLds(lds_u64* p) {
     rec = p;
-    count = (lds_u32*)(p + BLOCK);
+    key = (lds_u32*)p;
+    key_count = (lds_u32*)p + WAVES * TR_KEY_DIGITS * 2;
+    count = (lds_u32*)p + LEAD_BYTES / 4;
     total = count + WAVES * TR_DIGITS;
-    first = total + TR_DIGITS;
-    base = first + TR_DIGITS;
+    first = total + TR_KEY_DIGITS;
+    base = first + TR_KEY_DIGITS;
     scan = base + TR_PASSES * TR_DIGITS;
     bins = scan + 16;
   }
   static constexpr size_t bytes() {
-    return (size_t)BLOCK * 8 +
-           (size_t)(WAVES * TR_DIGITS + 2 * TR_DIGITS + TR_PASSES * TR_DIGITS + 16 + TR_DIGITS + 4) * 4;
+    return LEAD_BYTES +
+           (size_t)(WAVES * TR_DIGITS + 2 * TR_KEY_DIGITS + TR_PASSES * TR_DIGITS + 16 + TR_DIGITS + 4) * 4;
   }
+  __device__ PassLds<lds_u64*> wide() const { return {rec, (lds_mask*)rec, count, total, first, scan}; }
+  __device__ PassLds<lds_u32*> narrow() const { return {key, (lds_mask*)rec, key_count, total, first, scan}; }
 };
 
 // One pass over one block: the `count` records (record k of a lane sits at place wave * 64 E + k * 64 + lane of
 // the block, E records per lane) end up in L.rec ordered by the digit at `shift`, records of equal digit in their
 // old order.  Every thread of the workgroup calls this; it starts by overwriting L.rec and ends behind a barrier.
-template <int WAVES, int ITEMS>
-__device__ __forceinline__ void radix_block_pass(const uint64_t (&rec)[ITEMS], uint32_t E, uint32_t count, int shift,
-                                                 const TileRadixLds<WAVES, ITEMS>& L) {
+template <int WAVES, int ITEMS, int DIGIT_BITS, typename Rec, typename RecPtr>
+__device__ __forceinline__ void radix_block_pass(const Rec (&rec)[ITEMS], uint32_t E, uint32_t count, int shift,
+                                                 const PassLds<RecPtr>& L) {
   constexpr int THREADS = WAVES * GS_WAVE;
+  constexpr int DIGITS = 1 << DIGIT_BITS;
+  static_assert(THREADS >= DIGITS, "one thread per digit in the scan");
   const int tid = threadIdx.x, lane = tid & (GS_WAVE - 1), wave = tid / GS_WAVE;
-  lds_mask* s_mask = (lds_mask*)L.rec;
-  for (int i = tid; i < WAVES * TR_DIGITS; i += THREADS) {
+  lds_mask* s_mask = L.mask;
+  for (int i = tid; i < WAVES * DIGITS; i += THREADS) {
     s_mask[i] = 0ull;
     L.count[i] = 0u;
   }
   __syncthreads();
   // LDS operations of one wave execute in program order, which the two steps rely on; none of them waits for an
   // earlier one's result, so the items of a batch are in flight together.
-  volatile lds_mask* vmask = s_mask + wave * TR_DIGITS;
-  volatile lds_u32* vcount = L.count + wave * TR_DIGITS;
+  volatile lds_mask* vmask = s_mask + wave * DIGITS;
+  volatile lds_u32* vcount = L.count + wave * DIGITS;
   const unsigned long long lane_bit = 1ull << lane;
   const unsigned long long lt_mask = lane_bit - 1ull;
   const uint32_t wave_first = (uint32_t)wave * GS_WAVE * E;
@@ -108,7 +143,7 @@ __device__ __forceinline__ void radix_block_pass(const uint64_t (&rec)[ITEMS], u
 #pragma unroll
     for (int j = 0; j < BATCH; j++) {
       const int k = h * BATCH + j;
-      const uint32_t d = (uint32_t)(rec[k] >> shift) & (TR_DIGITS - 1);
+      const uint32_t d = (uint32_t)(rec[k] >> shift) & (DIGITS - 1);
       uint64_t rest = gs_ballot(valid[k]);
       unsigned long long mine = 0ull;
       bool placed = !valid[k];
@@ -126,7 +161,7 @@ __device__ __forceinline__ void radix_block_pass(const uint64_t (&rec)[ITEMS], u
       }
       same[j] = mine;
       if (rest != 0ull) {
-        if (!placed) atomicOr((unsigned long long*)&s_mask[wave * TR_DIGITS + d], lane_bit);
+        if (!placed) atomicOr((unsigned long long*)&s_mask[wave * DIGITS + d], lane_bit);
         __builtin_amdgcn_wave_barrier();
         if (!placed) same[j] = vmask[d];
         __builtin_amdgcn_wave_barrier();
@@ -138,12 +173,12 @@ __device__ __forceinline__ void radix_block_pass(const uint64_t (&rec)[ITEMS], u
 #pragma unroll
     for (int j = 0; j < BATCH; j++) {
       const int k = h * BATCH + j;
-      const uint32_t d = (uint32_t)(rec[k] >> shift) & (TR_DIGITS - 1);
+      const uint32_t d = (uint32_t)(rec[k] >> shift) & (DIGITS - 1);
       const unsigned long long lower = same[j] & lt_mask;
       const uint32_t before = valid[k] ? vcount[d] : 0u;
       __builtin_amdgcn_wave_barrier();
       if (valid[k] && lower == 0ull)
-        atomicAdd((uint32_t*)&L.count[wave * TR_DIGITS + d], (uint32_t)__popcll(same[j]));
+        atomicAdd((uint32_t*)&L.count[wave * DIGITS + d], (uint32_t)__popcll(same[j]));
       __builtin_amdgcn_wave_barrier();
       match[k] = before + (uint32_t)__popcll(lower);
     }
@@ -151,25 +186,25 @@ __device__ __forceinline__ void radix_block_pass(const uint64_t (&rec)[ITEMS], u
   __syncthreads();
   // thread d < 256: the block's records of digit d, their first place, and every wave's first place
   uint32_t tot = 0, inc = 0;
-  if (tid < TR_DIGITS) {
+  if (tid < DIGITS) {
 #pragma unroll
-    for (int w = 0; w < WAVES; w++) tot += L.count[w * TR_DIGITS + tid];
+    for (int w = 0; w < WAVES; w++) tot += L.count[w * DIGITS + tid];
     inc = tr_wave_inclusive_scan(tot, lane);
     if (lane == GS_WAVE - 1) L.scan[wave] = inc;
   }
   __syncthreads();
-  if (tid < TR_DIGITS) {
+  if (tid < DIGITS) {
     uint32_t before = 0;
 #pragma unroll
-    for (int w = 0; w < TR_DIGITS / GS_WAVE; w++)
+    for (int w = 0; w < DIGITS / GS_WAVE; w++)
       if (w < wave) before += L.scan[w];
     uint32_t run = before + inc - tot;
     L.total[tid] = tot;
     L.first[tid] = run;
 #pragma unroll
     for (int w = 0; w < WAVES; w++) {
-      const uint32_t c = L.count[w * TR_DIGITS + tid];
-      L.count[w * TR_DIGITS + tid] = run;
+      const uint32_t c = L.count[w * DIGITS + tid];
+      L.count[w * DIGITS + tid] = run;
       run += c;
     }
   }
@@ -177,8 +212,8 @@ __device__ __forceinline__ void radix_block_pass(const uint64_t (&rec)[ITEMS], u
 #pragma unroll
   for (int k = 0; k < ITEMS; k++) {
     if (!valid[k]) continue;
-    const uint32_t d = (uint32_t)(rec[k] >> shift) & (TR_DIGITS - 1);
-    L.rec[L.count[wave * TR_DIGITS + d] + match[k]] = rec[k];
+    const uint32_t d = (uint32_t)(rec[k] >> shift) & (DIGITS - 1);
+    L.rec[L.count[wave * DIGITS + d] + match[k]] = rec[k];
   }
   __syncthreads();
 }
@@ -217,81 +252,117 @@ __device__ __forceinline__ int passes_for_range(uint32_t range) {
   return p;
 }
 
-// A list of at most BLOCK records.
+// A list of at most BLOCK records, sorted inside the CU on one-word keys: the leading TR_FIELD_BITS bits of (depth
+// bits - smallest of the list) over the record's place in the unsorted list, so two passes on 9-bit digits (one, if
+// the list's depth bits span 9 bits or fewer) order it by the depth field with equal fields in the order of their
+// places.  Where depths agree in the bits kept, the last step (emit_list_entry) orders the run by all depth bits
+// and the emission index, as it does for equal depth bits; with 18 bits kept over a list's own range such runs
+// stay short.
 template <int WAVES, int ITEMS>
 __device__ __forceinline__ void sort_resident(uint32_t tile, uint32_t start, uint32_t n,
                                               const TileRecord* __restrict__ records, uint64_t* __restrict__ keys,
                                               uint32_t* __restrict__ emission, uint32_t* __restrict__ point_list,
                                               const TileRadixLds<WAVES, ITEMS>& L) {
   constexpr int THREADS = WAVES * GS_WAVE;
+  constexpr uint32_t PLACE_MASK = (1u << TR_PLACE_BITS) - 1u;
   const int tid = threadIdx.x, lane = tid & (GS_WAVE - 1), wave = tid / GS_WAVE;
   const uint32_t E = (n + THREADS - 1) / THREADS;
   const uint32_t wave_first = (uint32_t)wave * GS_WAVE * E;
-  uint64_t rec[ITEMS];
+  uint32_t key[ITEMS];
   uint32_t dmin = 0xFFFFFFFFu, dmax = 0u;
 #pragma unroll
   for (int k = 0; k < ITEMS; k++) {
     const uint32_t i = wave_first + (uint32_t)k * GS_WAVE + (uint32_t)lane;
-    rec[k] = ~0ull;
+    key[k] = 0u;
     if ((uint32_t)k < E && i < n) {
-      const uint32_t depth_bits = records[start + i].z;
-      dmin = depth_bits < dmin ? depth_bits : dmin;
-      dmax = depth_bits > dmax ? depth_bits : dmax;
-      rec[k] = ((uint64_t)depth_bits << 32) | (uint64_t)i;
+      key[k] = records[start + i].z;
+      dmin = key[k] < dmin ? key[k] : dmin;
+      dmax = key[k] > dmax ? key[k] : dmax;
     }
   }
   workgroup_min_max<WAVES>(dmin, dmax, L.scan, L.total);
-  const int passes = passes_for_range(dmax - dmin);
+  const uint32_t range = dmax - dmin;
+  const int bits = range != 0u ? 32 - __builtin_clz(range) : 0;
+  const uint32_t drop = bits > TR_FIELD_BITS ? (uint32_t)(bits - TR_FIELD_BITS) : 0u;
+  const int passes = bits > TR_KEY_DIGIT_BITS ? 2 : 1;
 #pragma unroll
-  for (int k = 0; k < ITEMS; k++) rec[k] -= (uint64_t)dmin << 32;  // (records that do not exist are never looked at)
+  for (int k = 0; k < ITEMS; k++) {
+    const uint32_t i = wave_first + (uint32_t)k * GS_WAVE + (uint32_t)lane;
+    // (keys of records that do not exist are never looked at)
+    key[k] = (((key[k] - dmin) >> drop) << TR_PLACE_BITS) | (i & PLACE_MASK);
+  }
+  const PassLds<lds_u32*> view = L.narrow();
 #pragma unroll 1
   for (int p = 0; p < passes; p++) {
-    radix_block_pass<WAVES, ITEMS>(rec, E, n, 32 + 8 * p, L);
+    radix_block_pass<WAVES, ITEMS, TR_KEY_DIGIT_BITS>(key, E, n, TR_PLACE_BITS + TR_KEY_DIGIT_BITS * p, view);
     if (p + 1 < passes) {
 #pragma unroll
       for (int k = 0; k < ITEMS; k++) {
         const uint32_t i = wave_first + (uint32_t)k * GS_WAVE + (uint32_t)lane;
-        if ((uint32_t)k < E && i < n) rec[k] = L.rec[i];
+        if ((uint32_t)k < E && i < n) key[k] = L.key[i];
       }
       __syncthreads();
     }
   }
-  // L.rec: ((depth bits - smallest) << 32 | place in the segment) in the final order but for runs of equal depth
-  // bits.  The Gaussian and the emission index of every entry are looked up through LDS: the sorted entries wait in
-  // registers while the segment's (Gaussian, emission index) pairs are read in order into the buffer (a gather
-  // from memory, even from the L2, costs as much as all four passes); then the buffer takes (depth bits << 32 |
-  // emission index) in sorted order for the last step.
+  // L.key: the keys in their final order but for runs of equal depth field.  Gaussian, emission index and depth
+  // bits of every entry are looked up through LDS: the sorted keys wait in registers while the list's (Gaussian,
+  // emission index) pairs, and then its depth bits, are read in order into the buffer (a gather from memory, even
+  // from the L2, costs as much as the passes); then the buffer takes (depth bits << 32 | emission index) in sorted
+  // order for the last step.
 #pragma unroll
   for (int k = 0; k < ITEMS; k++) {
     const uint32_t i = (uint32_t)k * THREADS + (uint32_t)tid;
-    rec[k] = i < n ? L.rec[i] : 0ull;
+    key[k] = i < n ? L.key[i] & PLACE_MASK : 0u;  // from here on: the entry's place in the unsorted list
   }
   __syncthreads();
+  uint32_t depth[ITEMS];
 #pragma unroll
-  for (int k = 0; k < ITEMS; k++) {
-    const uint32_t i = (uint32_t)k * THREADS + (uint32_t)tid;
-    if (i < n) {
-      const uint2 ge = *reinterpret_cast<const uint2*>(records + start + i);
-      L.rec[i] = ((uint64_t)ge.y << 32) | (uint64_t)ge.x;
+  for (int k0 = 0; k0 < ITEMS; k0 += 4) {
+    // (four loads in flight at a time: with all of them hoisted to the front the kernel spills)
+    TileRecord r[4];
+#pragma unroll
+    for (int u = 0; u < 4; u++) {
+      const uint32_t i = (uint32_t)(k0 + u) * THREADS + (uint32_t)tid;
+      r[u] = i < n ? records[start + i] : make_uint4(0u, 0u, 0u, 0u);
     }
+#pragma unroll
+    for (int u = 0; u < 4; u++) {
+      const uint32_t i = (uint32_t)(k0 + u) * THREADS + (uint32_t)tid;
+      if (i < n) L.rec[i] = ((uint64_t)r[u].y << 32) | (uint64_t)r[u].x;
+      depth[k0 + u] = r[u].z;
+    }
+    __builtin_amdgcn_sched_barrier(0);
   }
   __syncthreads();
-  uint32_t gaussian[ITEMS];
+  uint32_t gaussian[ITEMS], index[ITEMS];
 #pragma unroll
   for (int k = 0; k < ITEMS; k++) {
     const uint32_t i = (uint32_t)k * THREADS + (uint32_t)tid;
     gaussian[k] = 0u;
+    index[k] = 0u;
     if (i < n) {
-      const uint64_t ge = L.rec[(uint32_t)rec[k]];
+      const uint64_t ge = L.rec[key[k]];
       gaussian[k] = (uint32_t)ge;
-      rec[k] = ((rec[k] & 0xFFFFFFFF00000000ull) + ((uint64_t)dmin << 32)) | (ge >> 32);
+      index[k] = (uint32_t)(ge >> 32);
     }
   }
   __syncthreads();
 #pragma unroll
   for (int k = 0; k < ITEMS; k++) {
     const uint32_t i = (uint32_t)k * THREADS + (uint32_t)tid;
-    if (i < n) L.rec[i] = rec[k];
+    if (i < n) L.key[i] = depth[k];
+  }
+  __syncthreads();
+#pragma unroll
+  for (int k = 0; k < ITEMS; k++) {
+    const uint32_t i = (uint32_t)k * THREADS + (uint32_t)tid;
+    if (i < n) depth[k] = L.key[key[k]];
+  }
+  __syncthreads();
+#pragma unroll
+  for (int k = 0; k < ITEMS; k++) {
+    const uint32_t i = (uint32_t)k * THREADS + (uint32_t)tid;
+    if (i < n) L.rec[i] = ((uint64_t)depth[k] << 32) | (uint64_t)index[k];
   }
   __syncthreads();
   const lds_u64* sorted = L.rec;
@@ -300,7 +371,7 @@ __device__ __forceinline__ void sort_resident(uint32_t tile, uint32_t start, uin
     const uint32_t i = (uint32_t)k * THREADS + (uint32_t)tid;
     if (i < n)
       emit_list_entry(tile, start, n, i, gaussian[k], [&](uint32_t q) { return sorted[q]; }, keys, emission,
-                      point_list);
+                      point_list, dmin, drop);
   }
 }
 
@@ -406,7 +477,7 @@ __device__ __forceinline__ void sort_blocked(uint32_t tile, uint32_t start, uint
           rec[k] = p == 0 ? ((uint64_t)(records[start + b0 + i].z - dmin) << 32) | (uint64_t)(b0 + i)
                           : src[start + b0 + i];
       }
-      radix_block_pass<WAVES, ITEMS>(rec, E, cnt, shift, L);
+      radix_block_pass<WAVES, ITEMS, 8>(rec, E, cnt, shift, L.wide());
 #pragma unroll
       for (int k = 0; k < ITEMS; k++) {
         const uint32_t q = (uint32_t)k * THREADS + (uint32_t)tid;
