@@ -1,17 +1,19 @@
-// Per-tile sort of the longer lists: a stable least-significant-digit radix sort on the 32 depth bits, one
-// workgroup per tile, 8-bit digits, four passes.  The counting sort by tile (tile_bucket.hip) has left every
-// tile's instances in one segment of 16-byte records; what remains of the reference's sort of (tile << 32 | depth)
-// keys (cuda_rasterizer/rasterizer_impl.cu:675-684) is the order by depth bits inside each segment, ties in
-// emission order.
+// Per-tile sort of the longer lists: a stable least-significant-digit radix sort on the depth bits, one workgroup
+// per tile.  The counting sort by tile (tile_bucket.hip) has left every tile's instances in one segment of 16-byte
+// records; what remains of the reference's sort of (tile << 32 | depth) keys
+// (cuda_rasterizer/rasterizer_impl.cu:675-684) is the order by depth bits inside each segment, ties in emission
+// order.
 //
-// A list that fits one block (THREADS x ITEMS records) never leaves the CU: the workgroup holds (depth bits << 32 |
-// place in the segment) in registers, ranks the records of a pass per wave (lanes that hold the same digit find
-// each other through a 64-bit lane mask per digit in LDS, a running count per wave and digit makes the rank stable),
-// turns the waves' digit counts into places by one scan, moves every record to its place through LDS and reads
-// its next batch back.  A longer list is sorted block by block against running digit bases, ping-ponging between
-// two arrays in memory (its segment stays in the L2 of the workgroup's XCD).  The last step looks the Gaussian and
-// the emission index of every sorted record up in the segment (a gather inside the tile's own records, not over
-// the view's) and writes the three lists, putting runs of equal depth bits into emission order (tile_lists.h).
+// A list that fits one block (THREADS x ITEMS records) never leaves the CU: the workgroup holds one-word keys (the
+// leading 18 bits of depth bits minus the list's smallest, over the record's place in the segment) in registers,
+// ranks the keys of a pass per wave (lanes that hold the same digit find each other through a 64-bit lane mask per
+// digit in LDS, a running count per wave and digit makes the rank stable), turns the waves' digit counts into
+// places by one scan, moves every key to its place through LDS and reads its next batch back: two passes on 9-bit
+// digits.  A longer list is first split by its leading depth bits into parts that fit; a part that still does not
+// is sorted block by block on 64-bit records (depth bits << 32 | place) with 8-bit digits against running digit
+// bases, ping-ponging between two arrays in memory.  The last step looks Gaussian, emission index and depth bits of
+// every sorted entry up in the segment (a gather inside the tile's own records, through LDS) and writes the three
+// lists, putting runs of equal depth field into their order by depth bits and emission index (tile_lists.h).
 #include <atomic>
 
 #include "gs_common.h"
