@@ -293,3 +293,41 @@ def test_random_rectangles_by_every_route(orc, H, seed, W, Hh):
         assert np.array_equal(H.np_u32(ranges), want["ranges"].reshape(-1)), (large, chunks)
         assert np.array_equal(H.np_u64(keys), want["keys"]), (large, chunks)
         assert np.array_equal(H.np_u32(point_list), want["point_list"]), (large, chunks)
+
+
+@pytest.mark.parametrize("P", [1500, 3500, 9000, 20000])
+def test_depths_that_agree_in_their_leading_bits(orc, H, P):
+    """The per-tile sorts order their lists on the leading bits of the depth (relative to the list's smallest) and
+    leave the rest to their last step.  Here every splat covers every tile and the depths form two clusters, at 1
+    and at 64, whose members differ in their last 9 bits only (some not at all): all of a cluster shares the
+    leading bits at every list length (registers, both radix kernels, a split list), so the whole order inside a
+    cluster is made by that last step, by all depth bits and then the emission index."""
+    import gsrast_native as gn
+    from diff_gaussian_rasterization import _C
+    gen = torch.Generator().manual_seed(P)
+    W, Hh = 64, 48
+    gx, gy = H.grid(W, Hh)
+    T = gx * gy
+    means2D = torch.rand(P, 2, generator=gen) * torch.tensor([float(W), float(Hh)])
+    radii = torch.full((P,), 1000, dtype=torch.int32)
+    base = torch.where(torch.rand(P, generator=gen) < 0.5, torch.tensor(1.0), torch.tensor(64.0))
+    ulps = torch.randint(0, 300, (P,), generator=gen, dtype=torch.int32)
+    depths = (base.view(torch.int32) + ulps).view(torch.float32)
+    cl = torch.ones(gy, gx, dtype=torch.bool)
+    n = lambda t: t.detach().cpu().numpy()
+    want = orc.bin_and_sort(n(radii), n(means2D), n(depths), cl.numpy().reshape(-1), W, Hh)
+    assert int(want["point_list"].shape[0]) == P * T
+    co = torch.tensor([0.02, 0.0, 0.02, 0.3]).repeat(P, 1).to(DEV)
+    eye = torch.eye(4, device=DEV)
+    out = _C.render_gaussians(torch.zeros(3, device=DEV), Hh, W, means2D.to(DEV), depths.to(DEV), radii.to(DEV), co,
+                              torch.zeros(P, 3, device=DEV), cl.to(DEV), eye, torch.zeros(3, device=DEV), 1.0, 1.0,
+                              torch.zeros(P, 5, device=DEV), False, False, {"stats_collector": {}})
+    R, binB, imgB = out[0], out[9], out[10]
+    assert R == P * T
+    off = [C.c_size_t() for _ in range(5)]
+    gn.check(gn.lib.gs_binning_state_layout(R, W, Hh, *[C.byref(x) for x in off]), "layout")
+    b0 = (binB.data_ptr() + 255) // 256 * 256 - binB.data_ptr()
+    point_list = binB[b0 + off[0].value: b0 + off[0].value + 4 * R].view(torch.int32)
+    keys = binB[b0 + off[1].value: b0 + off[1].value + 8 * R].view(torch.int64)
+    assert np.array_equal(H.np_u64(keys), want["keys"])
+    assert np.array_equal(H.np_u32(point_list), want["point_list"])
