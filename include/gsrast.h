@@ -115,8 +115,8 @@ int gs_preprocess_backward(const int* radii, const float* cov3D, const uint8_t* 
  * zero keeps its default; struct_bytes is sizeof(gs_render_options) as the caller compiled it.
  * gs_render_forward builds the per-tile lists by bucketing the instances by tile (a counting sort) and sorting
  * each tile's list on its own: lists of up to 2048 records in registers, longer ones by a radix sort on the depth
- * bits that one workgroup runs inside its CU (up to 16384 records at once; a longer list block by block through
- * memory).  A tile grid of more than 30000 tiles takes the reference's own route instead: (tile | depth) keys
+ * bits that one workgroup runs inside its CU (up to 16384 records at once; a longer list is first split by its
+ * leading depth bits into parts that fit).  A tile grid of more than 30000 tiles takes the reference's own route instead: (tile | depth) keys
  * (rasterizer_impl.cu:74-117), one radix sort over all of them (:675-684), identifyTileRanges (:122-144).  All
  * give the same lists bit for bit.
  * tile_sort_small_limit lowers the list length that is sorted in registers (default and maximum 2048; 0 = the
