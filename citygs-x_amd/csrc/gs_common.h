@@ -210,13 +210,14 @@ __device__ __forceinline__ Rect get_rect(float px, float py, int radius, uint32_
 // big rectangle it is handed from the owner lane to all lanes while the wave is still convergent.  Every lane of
 // the wave must call this (it uses ballots and cross-lane reads).
 #define GS_BIG_RECT 16
+// The rectangles of more than GS_BIG_RECT tiles among the wave's 64, one after the other, each by the whole wave:
+// 64 tiles per step, ranks by ballot.  Returns, to the owner lane of such a rectangle, its count of local tiles
+// (0 to every other lane).
 template <typename Payload, typename Mask, typename Visit>
-__device__ __forceinline__ uint32_t walk_wave_rects(bool live, const Rect& rc, uint32_t gx, const Payload& mine,
-                                                    Mask is_local, Visit visit) {
+__device__ __forceinline__ uint32_t walk_wave_big_rects(uint32_t area, const Rect& rc, uint32_t w, uint32_t gx,
+                                                        const Payload& mine, Mask is_local, Visit visit) {
   static_assert(sizeof(Payload) % 4 == 0, "payload of 32-bit words");
   const int lane = threadIdx.x & (GS_WAVE - 1);
-  const uint32_t w = live ? rc.x1 - rc.x0 : 0u, h = live ? rc.y1 - rc.y0 : 0u;
-  const uint32_t area = w * h;
   uint32_t count = 0;
   uint64_t big = __ballot(area > GS_BIG_RECT);
   while (big != 0ull) {
@@ -243,6 +244,15 @@ __device__ __forceinline__ uint32_t walk_wave_rects(bool live, const Rect& rc, u
     }
     if (lane == owner) count = before;
   }
+  return count;
+}
+
+template <typename Payload, typename Mask, typename Visit>
+__device__ __forceinline__ uint32_t walk_wave_rects(bool live, const Rect& rc, uint32_t gx, const Payload& mine,
+                                                    Mask is_local, Visit visit) {
+  const uint32_t w = live ? rc.x1 - rc.x0 : 0u, h = live ? rc.y1 - rc.y0 : 0u;
+  const uint32_t area = w * h;
+  uint32_t count = walk_wave_big_rects(area, rc, w, gx, mine, is_local, visit);
   if (area != 0u && area <= GS_BIG_RECT) {
     for (uint32_t y = rc.y0; y < rc.y1; y++)
       for (uint32_t x = rc.x0; x < rc.x1; x++) {
@@ -302,25 +312,7 @@ __device__ __forceinline__ uint32_t walk_wave_rects_flat(bool live, const Rect& 
   const int lane = threadIdx.x & (GS_WAVE - 1);
   const uint32_t w = live ? rc.x1 - rc.x0 : 0u, h = live ? rc.y1 - rc.y0 : 0u;
   const uint32_t area = w * h;
-  uint64_t big = __ballot(area > GS_BIG_RECT);
-  while (big != 0ull) {
-    const int owner = (int)__builtin_ctzll(big);
-    big &= big - 1ull;
-    const uint32_t ox0 = __shfl(rc.x0, owner, GS_WAVE), oy0 = __shfl(rc.y0, owner, GS_WAVE);
-    const uint32_t ow = __shfl(w, owner, GS_WAVE), on = __shfl(area, owner, GS_WAVE);
-    Payload theirs;
-    {
-      const uint32_t* src = reinterpret_cast<const uint32_t*>(&mine);
-      uint32_t* dst = reinterpret_cast<uint32_t*>(&theirs);
-#pragma unroll
-      for (int k = 0; k < (int)(sizeof(Payload) / 4); k++) dst[k] = __shfl(src[k], owner, GS_WAVE);
-    }
-    for (uint32_t q0 = 0; q0 < on; q0 += GS_WAVE) {
-      const uint32_t q = q0 + (uint32_t)lane;
-      const uint32_t ry = q / ow, rx = q - ry * ow;
-      if (q < on) visit(theirs, (oy0 + ry) * gx + (ox0 + rx), q);
-    }
-  }
+  (void)walk_wave_big_rects(area, rc, w, gx, mine, [](uint32_t) { return true; }, visit);
   const uint32_t small = area <= GS_BIG_RECT ? area : 0u;
   const uint32_t incl = wave_scan_add(small), excl = incl - small;
   const uint32_t total = (uint32_t)__builtin_amdgcn_readlane((int)incl, GS_WAVE - 1);
