@@ -695,7 +695,9 @@ int launch_tile_radix_sort(int T, bool mid, bool lng, const uint32_t* ranges, co
   int dev = 0;
   GS_HIP_TRY(hipGetDevice(&dev));
   const uint64_t dev_bit = 1ull << (dev & 63);
-  if (lng && (dev >= 64 || !(raised.load(std::memory_order_acquire) & dev_bit))) {
+  if ((mid || lng) && (dev >= 64 || !(raised.load(std::memory_order_acquire) & dev_bit))) {
+    GS_HIP_TRY(hipFuncSetAttribute((const void*)tile_radix_sort_kernel<8, 8>,
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)TileRadixLds<8, 8>::bytes()));
     GS_HIP_TRY(hipFuncSetAttribute((const void*)tile_radix_sort_kernel<16, 16>,
                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)TileRadixLds<16, 16>::bytes()));
     raised.fetch_or(dev_bit, std::memory_order_release);
