@@ -162,15 +162,18 @@ __device__ __forceinline__ uint32_t wave_inclusive_scan_u32(uint32_t v, int lane
 // (0, 0) for a tile without instances).  Tiles whose lists are too long for the register sort are entered in two
 // lists for the radix sort's kernels: lists of more than small_limit and at most mid_limit records ascending from
 // tile_lists[0], longer ones descending from tile_lists[T - 1]; tile_lists[T] = (number of the longer ones << 16
-// | number of the others) (T is at most 30000).  The longest list, that word and then the number of instances are
+// | number of the others) (T is at most 30000).  The lists beyond block_limit records, which are split before they
+// are sorted and take several times as long, are entered a second time in a list of their own, so that the larger
+// kernel can start with them: their number in tile_lists[T + 1], the tiles ascending from tile_lists[T + 2].  The longest list, that word and then the number of instances are
 // stored where the host can read them (host_words[1], [2] and [0]; the host polls word 0, so it is written last).
 __global__ void __launch_bounds__(1024)
-bucket_ranges_kernel(uint32_t T, uint32_t small_limit, uint32_t mid_limit, const uint32_t* __restrict__ totals,
+bucket_ranges_kernel(uint32_t T, uint32_t small_limit, uint32_t mid_limit, uint32_t block_limit,
+                     const uint32_t* __restrict__ totals,
                      uint32_t* __restrict__ ranges, uint32_t* __restrict__ tile_lists,
                      uint32_t* __restrict__ block_sums, int nblocks, uint32_t* __restrict__ host_words,
                      uint32_t cap_instances, uint32_t cap_longest, uint32_t* __restrict__ fits_word) {
   constexpr int ITEMS = 4;  // consecutive tiles per thread: the usual grids (up to 4096 tiles) take one round
-  __shared__ uint32_t s_wave[16], s_wave_class[16], s_max[16];
+  __shared__ uint32_t s_wave[16], s_wave_class[16], s_wave_split[16], s_max[16];
   __shared__ double s_exact[16];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   {
@@ -187,16 +190,17 @@ bucket_ranges_kernel(uint32_t T, uint32_t small_limit, uint32_t mid_limit, const
     if ((int)threadIdx.x < nblocks) block_sums[threadIdx.x] = base + inc - b;
     __syncthreads();
   }
-  uint32_t carry = 0, carry_class = 0, longest = 0;
+  uint32_t carry = 0, carry_class = 0, carry_split = 0, longest = 0;
   double exact = 0.0;  // the number of instances without the 32-bit wrap-around of the prefix sums
   for (uint32_t start = 0; start < T; start += 1024 * ITEMS) {
     const uint32_t t0 = start + threadIdx.x * ITEMS;
-    uint32_t v[ITEMS], c[ITEMS], sum = 0, sum_class = 0;
+    uint32_t v[ITEMS], c[ITEMS], sum = 0, sum_class = 0, sum_split = 0;
 #pragma unroll
     for (int q = 0; q < ITEMS; q++) v[q] = t0 + q < T ? totals[t0 + q] : 0u;
 #pragma unroll
     for (int q = 0; q < ITEMS; q++) {
       c[q] = v[q] > mid_limit ? 0x10000u : (v[q] > small_limit ? 1u : 0u);
+      sum_split += v[q] > block_limit ? 1u : 0u;
       longest = v[q] > longest ? v[q] : longest;
       exact += (double)v[q];
       sum += v[q];
@@ -205,24 +209,29 @@ bucket_ranges_kernel(uint32_t T, uint32_t small_limit, uint32_t mid_limit, const
     const uint32_t inc = wave_inclusive_scan_u32(sum, lane);
     // (a wave without a long list, the usual case, has nothing to scan)
     const uint32_t inc_class = __ballot(sum_class != 0u) != 0ull ? wave_inclusive_scan_u32(sum_class, lane) : 0u;
+    const uint32_t inc_split = __ballot(sum_split != 0u) != 0ull ? wave_inclusive_scan_u32(sum_split, lane) : 0u;
     if (lane == 63) {
       s_wave[wave] = inc;
       s_wave_class[wave] = inc_class;
+      s_wave_split[wave] = inc_split;
     }
     __syncthreads();
-    uint32_t base = 0, all = 0, base_class = 0, all_class = 0;
+    uint32_t base = 0, all = 0, base_class = 0, all_class = 0, base_split = 0, all_split = 0;
 #pragma unroll
     for (int w = 0; w < 16; w++) {
-      const uint32_t s = s_wave[w], sc = s_wave_class[w];
+      const uint32_t s = s_wave[w], sc = s_wave_class[w], ss = s_wave_split[w];
       if (w < wave) {
         base += s;
         base_class += sc;
+        base_split += ss;
       }
       all += s;
       all_class += sc;
+      all_split += ss;
     }
     __syncthreads();
     uint32_t begin = carry + base + inc - sum, begin_class = carry_class + base_class + inc_class - sum_class;
+    uint32_t begin_split = carry_split + base_split + inc_split - sum_split;
 #pragma unroll
     for (int q = 0; q < ITEMS; q++) {
       if (t0 + q < T) {
@@ -230,12 +239,15 @@ bucket_ranges_kernel(uint32_t T, uint32_t small_limit, uint32_t mid_limit, const
         ranges[2 * (t0 + q) + 1] = v[q] ? begin + v[q] : 0u;
         if (c[q] == 1u) tile_lists[begin_class & 0xFFFFu] = t0 + q;
         if (c[q] == 0x10000u) tile_lists[T - 1u - (begin_class >> 16)] = t0 + q;
+        if (v[q] > block_limit) tile_lists[T + 2u + begin_split] = t0 + q;
       }
       begin += v[q];
       begin_class += c[q];
+      begin_split += v[q] > block_limit ? 1u : 0u;
     }
     carry += all;
     carry_class += all_class;
+    carry_split += all_split;
   }
 #pragma unroll
   for (int d = 32; d >= 1; d >>= 1) {
@@ -257,6 +269,7 @@ bucket_ranges_kernel(uint32_t T, uint32_t small_limit, uint32_t mid_limit, const
       all += s_exact[w];
     }
     tile_lists[T] = carry_class;
+    tile_lists[T + 1u] = carry_split;
     // more instances than 32-bit positions can address: the host must not go on with the wrapped count
     const uint32_t reported = all > (double)GS_MAX_INSTANCES ? GS_TOO_MANY_INSTANCES : carry;
     // Kernels launched ahead of the host's decision (buffers sized from the caller's expectation) look at this
@@ -626,17 +639,17 @@ tile_sort_registers_kernel(const uint32_t* __restrict__ ranges, const TileRecord
 // Tiles the LDS histograms of the counting kernels can hold.
 int bucket_max_tiles() { return 30000; }
 
-// workgroup-by-tile counts, then the tile totals, then the tile lists of the radix sort's kernels (T + 1 words), then
+// workgroup-by-tile counts, then the tile totals, then the tile lists of the radix sort's kernels (2 T + 2 words), then
 // the workgroups' sums of tiles touched and the word that says whether the view fits the buffers of kernels
 // launched ahead of the host
 size_t bucket_table_bytes(int T) {
-  return (((size_t)BK_MAX_BLOCKS + 2) * (size_t)T + 1 + BK_MAX_BLOCKS + 1) * sizeof(uint32_t);
+  return (((size_t)BK_MAX_BLOCKS + 3) * (size_t)T + 2 + BK_MAX_BLOCKS + 1) * sizeof(uint32_t);
 }
 static uint32_t* bucket_block_sums(void* table, uint32_t T) {
-  return (uint32_t*)table + ((size_t)BK_MAX_BLOCKS + 2) * (size_t)T + 1;
+  return (uint32_t*)table + ((size_t)BK_MAX_BLOCKS + 3) * (size_t)T + 2;
 }
 const uint32_t* bucket_fits_word(const void* table, int T) {
-  return (const uint32_t*)table + ((size_t)BK_MAX_BLOCKS + 2) * (size_t)T + 1 + BK_MAX_BLOCKS;
+  return (const uint32_t*)table + ((size_t)BK_MAX_BLOCKS + 3) * (size_t)T + 2 + BK_MAX_BLOCKS;
 }
 
 int launch_bucket_count(int P, int W, int H, const int* radii, const float* means2D, const uint8_t* compute_locally,
@@ -649,6 +662,10 @@ int launch_bucket_count(int P, int W, int H, const int* radii, const float* mean
   uint32_t mid_limit = (uint32_t)tile_radix_mid_records();
   if (block_limit != 0 && block_limit < mid_limit) mid_limit = block_limit;
   if (mid_limit < small_limit) mid_limit = small_limit;
+  // ... and the lists the larger kernel holds; longer ones are split first
+  uint32_t split_limit = (uint32_t)tile_radix_block_records();
+  if (block_limit != 0 && block_limit < split_limit) split_limit = block_limit;
+  if (split_limit < mid_limit) split_limit = mid_limit;
   const uint32_t gx = (W + GS_TILE_X - 1) / GS_TILE_X, gy = (H + GS_TILE_Y - 1) / GS_TILE_Y;
   const uint32_t T = gx * gy;
   const size_t lds = (size_t)T * (sizeof(uint32_t) + 1);
@@ -673,8 +690,8 @@ int launch_bucket_count(int P, int W, int H, const int* radii, const float* mean
                      zero_per_gaussian);
   hipLaunchKernelGGL(bucket_columns_kernel, dim3((T + COL_TILES - 1) / COL_TILES), dim3(COL_TILES * COL_RUNS), 0, stream, nb, T,
                      tab, totals);
-  hipLaunchKernelGGL(bucket_ranges_kernel, dim3(1), dim3(1024), 0, stream, T, small_limit, mid_limit, totals, ranges,
-                     totals + T,
+  hipLaunchKernelGGL(bucket_ranges_kernel, dim3(1), dim3(1024), 0, stream, T, small_limit, mid_limit, split_limit,
+                     totals, ranges, totals + T,
                      bucket_block_sums(table, T), nb, host_words, cap_instances, cap_longest,
                      const_cast<uint32_t*>(bucket_fits_word(table, (int)T)));
   return 0;
