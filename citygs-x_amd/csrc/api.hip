@@ -539,7 +539,7 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
     // the histogram's grand total is the instance count: the host gets it from here
     if (launch_bucket_count(P, width, height, radii, means2D, compute_locally, tiles_touched, bucket_table, ranges,
                             sort_limit, (uint32_t)limits.block, total_slot, out_observe, (uint32_t)cap_n, cap_longest,
-                            stream))
+                            packed_valid, stream))
       return 1;
   } else {
     StageScope _t("tile_count", stream);
@@ -565,10 +565,12 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
       // (the word beside the library's own records says "none": a backward call that is not handed the caller's
       // records again gathers the operands from the arrays)
       use_packed = true;
+      if (bucketed) return 0;  // (the counting kernels have cleared the word)
       launch_fill_u32(1, 0u, packed_valid, stream);
       return check_launch("pack_operands", stream, dbg);
     }
     use_packed = instances * 5 > (int64_t)P * 4;
+    if (!use_packed && bucketed) return 0;  // (likewise)
     StageScope _t("pack_operands", stream);
     if (use_packed)
       launch_pack_blend_operands(P, radii, means2D, conic_opacity, rgb, render_geo ? all_map : nullptr, depths, packed,

@@ -108,7 +108,7 @@ size_t bucket_table_bytes(int T);
 int launch_bucket_count(int P, int W, int H, const int* radii, const float* means2D, const uint8_t* compute_locally,
                         uint32_t* tiles_touched, void* table, uint32_t* ranges, uint32_t small_limit,
                         uint32_t block_limit, uint32_t* host_words, int* zero_per_gaussian, uint32_t cap_instances,
-                        uint32_t cap_longest, hipStream_t stream);
+                        uint32_t cap_longest, uint32_t* clear_word, hipStream_t stream);
 const uint32_t* bucket_fits_word(const void* table, int T);
 // records: one 16-byte record (Gaussian, emission index, depth bits, 0) per instance, grouped by tile in any
 // order.  Also writes point_offsets (the inclusive prefix sum of tiles_touched).

@@ -171,7 +171,8 @@ bucket_ranges_kernel(uint32_t T, uint32_t small_limit, uint32_t mid_limit, uint3
                      const uint32_t* __restrict__ totals,
                      uint32_t* __restrict__ ranges, uint32_t* __restrict__ tile_lists,
                      uint32_t* __restrict__ block_sums, int nblocks, uint32_t* __restrict__ host_words,
-                     uint32_t cap_instances, uint32_t cap_longest, uint32_t* __restrict__ fits_word) {
+                     uint32_t cap_instances, uint32_t cap_longest, uint32_t* __restrict__ fits_word,
+                     uint32_t* __restrict__ clear_word) {
   constexpr int ITEMS = 4;  // consecutive tiles per thread: the usual grids (up to 4096 tiles) take one round
   __shared__ uint32_t s_wave[16], s_wave_class[16], s_wave_split[16], s_max[16];
   __shared__ double s_exact[16];
@@ -270,6 +271,7 @@ bucket_ranges_kernel(uint32_t T, uint32_t small_limit, uint32_t mid_limit, uint3
     }
     tile_lists[T] = carry_class;
     tile_lists[T + 1u] = carry_split;
+    if (clear_word != nullptr) *clear_word = 0u;  // (a word the caller wants cleared on the way: saves a launch)
     // more instances than 32-bit positions can address: the host must not go on with the wrapped count
     const uint32_t reported = all > (double)GS_MAX_INSTANCES ? GS_TOO_MANY_INSTANCES : carry;
     // Kernels launched ahead of the host's decision (buffers sized from the caller's expectation) look at this
@@ -655,7 +657,7 @@ const uint32_t* bucket_fits_word(const void* table, int T) {
 int launch_bucket_count(int P, int W, int H, const int* radii, const float* means2D, const uint8_t* compute_locally,
                         uint32_t* tiles_touched, void* table, uint32_t* ranges, uint32_t small_limit,
                         uint32_t block_limit, uint32_t* host_words, int* zero_per_gaussian, uint32_t cap_instances,
-                        uint32_t cap_longest, hipStream_t stream) {
+                        uint32_t cap_longest, uint32_t* clear_word, hipStream_t stream) {
   if (P <= 0) return 0;
   if (small_limit == 0 || small_limit > (uint32_t)TILE_SORT_SMALL) small_limit = TILE_SORT_SMALL;
   // the lists one workgroup of the radix sort's smaller kernel holds; longer ones go to the larger kernel
@@ -693,7 +695,7 @@ int launch_bucket_count(int P, int W, int H, const int* radii, const float* mean
   hipLaunchKernelGGL(bucket_ranges_kernel, dim3(1), dim3(1024), 0, stream, T, small_limit, mid_limit, split_limit,
                      totals, ranges, totals + T,
                      bucket_block_sums(table, T), nb, host_words, cap_instances, cap_longest,
-                     const_cast<uint32_t*>(bucket_fits_word(table, (int)T)));
+                     const_cast<uint32_t*>(bucket_fits_word(table, (int)T)), clear_word);
   return 0;
 }
 
