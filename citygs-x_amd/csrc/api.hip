@@ -135,10 +135,9 @@ ImageLayout image_layout(int W, int H) {
 }
 
 struct GeometryLayout {
-  size_t tiles_touched, point_offsets, scan_temp, packed_valid, packed, total;
+  size_t tiles_touched, point_offsets, scan_temp, packed_valid, total;
 };
-// own_records: the library packs the blend kernels' operand records itself (the caller brought none)
-GeometryLayout geometry_layout(int P, bool own_records = true) {
+GeometryLayout geometry_layout(int P) {
   GeometryLayout L;
   const size_t n = (size_t)(P > 0 ? P : 1);
   size_t off = 0;
@@ -146,19 +145,18 @@ GeometryLayout geometry_layout(int P, bool own_records = true) {
   L.tiles_touched = take(n * 4);
   L.point_offsets = take(n * 4);
   L.scan_temp = take(scan_temp_bytes((int64_t)n));
-  L.packed_valid = take(4);  // one word: whether the forward call packed the records below
-  // the blend kernels' operands, one 64-byte record per Gaussian (last, so that no other offset depends on it)
-  L.packed = take(own_records ? n * 64 : 0);
+  L.packed_valid = take(4);  // one word: whether the forward call packed operand records (binning buffer)
   L.total = off + 256;
   return L;
 }
 
 struct BinningLayout {
   size_t point_list, keys, point_list_unsorted, keys_unsorted, emission, emission_other, sort_temp, block_hits,
-      radix_scratch, total;
+      radix_scratch, packed, total;
 };
-// n = the number of instances the arrays are laid out for
-BinningLayout binning_layout(int64_t R) {
+// n = the number of instances the arrays are laid out for; packed_gaussians: the Gaussians the forward call packs
+// operand records for (0 when it packs none, or when only the offsets are asked for)
+BinningLayout binning_layout(int64_t R, int64_t packed_gaussians = 0) {
   BinningLayout L;
   const size_t n = (size_t)(R > 0 ? R : 1);
   size_t off = 0;
@@ -175,6 +173,9 @@ BinningLayout binning_layout(int64_t R) {
   L.sort_temp = take(sort_temp_bytes((int64_t)n));
   L.block_hits = take(n * 2);  // what the forward blend leaves for the backward blend, per sorted instance
   L.radix_scratch = take(n * 24);  // per-tile radix sort: lists beyond one block, split (16 B) and in blocks (8 B)
+  // the blend kernels' operands, one 64-byte record per Gaussian, if the forward call packs them (last, so that
+  // no other offset depends on whether it does)
+  L.packed = take(packed_gaussians > 0 ? (size_t)packed_gaussians * 64 : 0);
   L.total = off + 256;
   return L;
 }
@@ -490,14 +491,13 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
   const float* caller_records =
       (options != nullptr && options->struct_bytes >= sizeof(gs_render_options)) ? options->blend_records : nullptr;
   GS_REQUIRE(((uintptr_t)caller_records & 15u) == 0u, "gs_render_forward: blend_records must be 16-byte aligned");
-  const GeometryLayout GL = geometry_layout(P, caller_records == nullptr);
+  const GeometryLayout GL = geometry_layout(P);
   char* gbase = geometryBuffer(GL.total, geometry_user);
   GS_REQUIRE(gbase, "gs_render_forward: geometry buffer callback returned NULL");
   gbase = align_ptr(gbase, 256);
   uint32_t* tiles_touched = (uint32_t*)(gbase + GL.tiles_touched);
   uint32_t* point_offsets = (uint32_t*)(gbase + GL.point_offsets);
   void* scan_temp = gbase + GL.scan_temp;
-  float* packed = (float*)(gbase + GL.packed);
   uint32_t* packed_valid = (uint32_t*)(gbase + GL.packed_valid);
 
   const ImageLayout IL = image_layout(width, height);
@@ -557,27 +557,12 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
   // The blend kernels (this call's and the backward call's) can fetch a Gaussian's operands as one 64-byte record
   // instead of gathering parts of five lines of memory.  Packing the records costs about 20 us per million
   // Gaussians and saves about 25 us per million instances: done for a view with enough instances per Gaussian.
+  // The library's own records live at the end of the binning buffer, which is sized once the decision is made.
   bool use_packed = false, pack_decided = false;
-  auto decide_packing = [&](int64_t instances) -> int {
-    if (pack_decided) return 0;
+  auto decide_packing = [&](int64_t instances) {
+    if (pack_decided) return;
     pack_decided = true;
-    if (caller_records != nullptr) {
-      // (the word beside the library's own records says "none": a backward call that is not handed the caller's
-      // records again gathers the operands from the arrays)
-      use_packed = true;
-      if (bucketed) return 0;  // (the counting kernels have cleared the word)
-      launch_fill_u32(1, 0u, packed_valid, stream);
-      return check_launch("pack_operands", stream, dbg);
-    }
-    use_packed = instances * 5 > (int64_t)P * 4;
-    if (!use_packed && bucketed) return 0;  // (likewise)
-    StageScope _t("pack_operands", stream);
-    if (use_packed)
-      launch_pack_blend_operands(P, radii, means2D, conic_opacity, rgb, render_geo ? all_map : nullptr, depths, packed,
-                                 packed_valid, stream);
-    else
-      launch_fill_u32(1, 0u, packed_valid, stream);
-    return check_launch("pack_operands", stream, dbg);
+    use_packed = caller_records != nullptr || instances * 5 > (int64_t)P * 4;
   };
 
   EventTimer timer;
@@ -587,9 +572,10 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
     void *sort_temp, *radix_scratch;
     int64_t capacity;
     uint16_t* block_hits;
+    float* packed;
   };
   auto carve = [&](int64_t n, Arrays& A) -> int {
-    const BinningLayout BL = binning_layout(n);
+    const BinningLayout BL = binning_layout(n, (use_packed && caller_records == nullptr) ? (int64_t)P : 0);
     char* bbase = binningBuffer(BL.total, binning_user);
     GS_REQUIRE(bbase, "gs_render_forward: binning buffer callback returned NULL");
     bbase = align_ptr(bbase, 256);
@@ -602,8 +588,23 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
     A.sort_temp = bbase + BL.sort_temp;
     A.block_hits = (uint16_t*)(bbase + BL.block_hits);
     A.radix_scratch = bbase + BL.radix_scratch;
+    A.packed = (float*)(bbase + BL.packed);
     A.capacity = n > 0 ? n : 1;
     return 0;
+  };
+  // Packs the library's own records into the arrays just carved.  With the caller's records, or none, the word
+  // beside them must say "none" (a backward call that is not handed the caller's records again then gathers the
+  // operands from the arrays): the counting kernels of the per-tile route have cleared it on their way.
+  auto pack_records = [&](const Arrays& A) -> int {
+    if (caller_records != nullptr || !use_packed) {
+      if (bucketed) return 0;
+      launch_fill_u32(1, 0u, packed_valid, stream);
+      return check_launch("pack_operands", stream, dbg);
+    }
+    StageScope _t("pack_operands", stream);
+    launch_pack_blend_operands(P, radii, means2D, conic_opacity, rgb, render_geo ? all_map : nullptr, depths,
+                               A.packed, packed_valid, stream);
+    return check_launch("pack_operands", stream, dbg);
   };
   auto blend = [&](const Arrays& A, bool ahead_of_host) -> int {
     RenderFwdArgs a;
@@ -619,7 +620,7 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
     a.n_render = n_render; a.n_consider = n_consider; a.n_contrib_tile = n_contrib;
     a.fits_word = ahead_of_host ? bucket_fits_word(bucket_table, T) : nullptr;
     a.block_hits = A.block_hits;
-    a.packed = use_packed ? (caller_records != nullptr ? caller_records : packed) : nullptr;
+    a.packed = use_packed ? (caller_records != nullptr ? caller_records : A.packed) : nullptr;
     {
       StageScope _t("render_fwd", stream);
       launch_render_fwd(a, stream);
@@ -648,10 +649,11 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
 
   Arrays A;
   if (ahead) {
+    // (on the expected count less a fifth: the caller's expectation carries a margin of a quarter)
+    decide_packing(cap_n - cap_n / 5);
     if (carve(cap_n, A)) return 1;
     if (timer.begin(elapsed_ms != nullptr, stream)) return 1;
-    // (on the expected count less a fifth: the caller's expectation carries a margin of a quarter)
-    if (decide_packing(cap_n - cap_n / 5)) return 1;
+    if (pack_records(A)) return 1;
     if (lists_by_tile(A, cap_longest, 0xFFFFFFFFu, true)) return 1;
     if (blend(A, true)) return 1;
   }
@@ -694,9 +696,11 @@ int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resiz
   }
 
   // The ordinary way (also after kernels launched ahead found that the view does not fit and did nothing).
+  // (after kernels launched ahead: the records are packed again, the buffer may be another one)
+  decide_packing(R);
   if (carve(R, A)) return 1;
   if (!ahead && timer.begin(elapsed_ms != nullptr, stream)) return 1;
-  if (decide_packing(R)) return 1;
+  if (pack_records(A)) return 1;
 
   if (bucketed) {
     if (lists_by_tile(A, longest, radix_tiles, false)) return 1;
@@ -787,7 +791,7 @@ int gs_render_backward(int P, int R, const float* background, int width, int hei
   a.point_offsets = (const uint32_t*)(gbase + GL.point_offsets);
   // (records of the arrays the forward call was given: the caller's own, or what the forward call packed)
   GS_REQUIRE(((uintptr_t)blend_records & 15u) == 0u, "gs_render_backward: blend_records must be 16-byte aligned");
-  a.packed = blend_records != nullptr ? blend_records : (const float*)(gbase + GL.packed);
+  a.packed = blend_records != nullptr ? blend_records : (const float*)(bbase + BL.packed);
   a.packed_valid = blend_records != nullptr ? nullptr : (const uint32_t*)(gbase + GL.packed_valid);
   a.instance_grads = (float*)align_ptr((const char*)instance_grads, 256);
   a.P = P; a.W = width; a.H = height;

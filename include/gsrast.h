@@ -179,9 +179,11 @@ typedef struct gs_render_result {
  * elapsed_ms (host, optional): if non-NULL the call times key emission + sort
  * + blend with events and blocks until done (the forward_render_time the
  * reference stores at CR/rasterizer_impl.cu:754-755).
- * The geometry buffer is asked for 72 bytes per Gaussian (tile counts, their prefix sum, and room for the blend
- * operand records, reserved whether or not this call packs them) plus the prefix sum's workspace (the reference's
- * holds the preprocess outputs as well, CR/rasterizer_impl.cu:160-188; here those are the caller's tensors). */
+ * The geometry buffer is asked for 8 bytes per Gaussian (tile counts and their prefix sum) plus the prefix sum's
+ * workspace (the reference's holds the preprocess outputs as well, CR/rasterizer_impl.cu:160-188; here those are
+ * the caller's tensors).  The binning buffer is asked for 64 bytes per Gaussian beyond what
+ * gs_binning_state_layout reports when this call packs the blend kernels' operand records itself (a view with
+ * more than 0.8 instances per Gaussian and no blend_records from the caller). */
 int gs_render_forward(gs_resize_fn geometryBuffer, void* geometry_user, gs_resize_fn binningBuffer,
                       void* binning_user, gs_resize_fn imageBuffer, void* image_user, int P,
                       const float* background, int width, int height, float focal_x, float focal_y, float cx,
