@@ -393,6 +393,173 @@ bucket_scatter_kernel(int P, int per_block, uint32_t gx, uint32_t gy, const floa
   }
 }
 
+// 1d'. The same scatter for a view in which a workgroup walks its chunk of Gaussians in one round (at most
+// BK_BATCH * BK_THREADS of them) and its instances fit the LDS: the records are staged in LDS, ordered by tile (the
+// counting kernels' table gives the workgroup's own count per tile: the next workgroup's prefix minus its own), and
+// written out tile by tile, so that the records a workgroup adds to one tile's segment leave as one run, all
+// workgroups at about the same time.  Every 16-byte record written on its own costs the memory a 64-byte write;
+// runs that meet in the L2 cost their bytes.  A workgroup with more than `cap` instances stores directly, as the
+// kernel above does.
+// Dynamic LDS: 9 bytes per tile and 12 bytes per staged record.
+__global__ void __launch_bounds__(BK_THREADS)
+bucket_scatter_staged_kernel(int P, int per_block, int nblocks, uint32_t gx, uint32_t gy,
+                             const float2* __restrict__ means2D, const float* __restrict__ depths,
+                             const uint32_t* __restrict__ tiles_touched, const uint32_t* __restrict__ block_prefix,
+                             uint32_t* __restrict__ point_offsets, const int* __restrict__ radii,
+                             const uint8_t* __restrict__ compute_locally, const uint32_t* __restrict__ table,
+                             const uint32_t* __restrict__ totals, const uint32_t* __restrict__ ranges,
+                             TileRecord* __restrict__ records, const uint32_t* __restrict__ fits_word,
+                             int vector_loads, uint32_t cap) {
+  extern __shared__ uint32_t s_mem[];
+  __shared__ uint32_t s_wave[BK_THREADS / GS_WAVE], s_wave_tiles[BK_THREADS / GS_WAVE];
+  __shared__ uint32_t s_heads[BK_THREADS];
+  if (fits_word != nullptr && *fits_word == 0u) return;
+  const uint32_t T = gx * gy;
+  uint32_t* s_next = s_mem;         // [T] where the workgroup's first record of a tile goes in memory
+  uint32_t* s_cursor = s_mem + T;   // [T] next free place of a tile: in the staging arrays, or in memory
+  uint32_t* stage_g = s_cursor + T; // [cap] x 3: Gaussian, emission index, depth bits
+  uint32_t* stage_e = stage_g + cap;
+  uint32_t* stage_z = stage_e + cap;
+  uint8_t* s_local = reinterpret_cast<uint8_t*>(stage_z + cap);
+  const int lane = threadIdx.x & (GS_WAVE - 1), wave = threadIdx.x / GS_WAVE;
+  const int chunk = chunk_of_workgroup(blockIdx.x, gridDim.x);
+  const uint32_t* row = table + (size_t)chunk * T;
+  const uint32_t* next_row = chunk + 1 < nblocks ? table + (size_t)(chunk + 1) * T : totals;
+  const int first = chunk * per_block;
+  const int last = first + per_block < P ? first + per_block : P;
+  // (the workgroup's Gaussians are asked for first: their latency passes behind the set-up of the tiles)
+  const int i0 = first + (int)threadIdx.x * BK_BATCH;
+  int r[BK_BATCH];
+  float2 p[BK_BATCH];
+  uint32_t tt[BK_BATCH], dbits[BK_BATCH], sum = 0;
+  static_assert(BK_BATCH == 4, "a thread's Gaussians are loaded as four-word vectors");
+  const bool whole = vector_loads != 0 && i0 + BK_BATCH <= last;
+  if (whole) {
+    const int4 rv = *reinterpret_cast<const int4*>(radii + i0);
+    const uint4 tv = *reinterpret_cast<const uint4*>(tiles_touched + i0);
+    const uint4 dv = *reinterpret_cast<const uint4*>(depths + i0);
+    const float4 m01 = *reinterpret_cast<const float4*>(means2D + i0);
+    const float4 m23 = *reinterpret_cast<const float4*>(means2D + i0 + 2);
+    r[0] = rv.x; r[1] = rv.y; r[2] = rv.z; r[3] = rv.w;
+    tt[0] = tv.x; tt[1] = tv.y; tt[2] = tv.z; tt[3] = tv.w;
+    dbits[0] = dv.x; dbits[1] = dv.y; dbits[2] = dv.z; dbits[3] = dv.w;
+    p[0] = make_float2(m01.x, m01.y); p[1] = make_float2(m01.z, m01.w);
+    p[2] = make_float2(m23.x, m23.y); p[3] = make_float2(m23.z, m23.w);
+  } else {
+#pragma unroll
+    for (int q = 0; q < BK_BATCH; q++) {
+      const int i = i0 + q;
+      r[q] = i < last ? radii[i] : 0;
+      p[q] = i < last ? means2D[i] : make_float2(0.0f, 0.0f);
+      dbits[q] = i < last ? __float_as_uint(depths[i]) : 0u;
+      tt[q] = i < last ? tiles_touched[i] : 0u;
+    }
+  }
+  int masked = 0;
+  constexpr int TILES_AHEAD = 4;  // tiles a thread has in flight: a usual grid is set up with one memory latency
+  for (uint32_t t0 = threadIdx.x; t0 < T; t0 += TILES_AHEAD * BK_THREADS) {
+    uint32_t before[TILES_AHEAD], upto[TILES_AHEAD], begin[TILES_AHEAD];
+    uint8_t c[TILES_AHEAD];
+#pragma unroll
+    for (int u = 0; u < TILES_AHEAD; u++) {
+      const uint32_t t = t0 + (uint32_t)u * BK_THREADS;
+      before[u] = t < T ? row[t] : 0u;
+      upto[u] = t < T ? next_row[t] : 0u;
+      begin[u] = t < T ? ranges[2 * t] : 0u;
+      c[u] = t < T ? compute_locally[t] : (uint8_t)1;
+    }
+#pragma unroll
+    for (int u = 0; u < TILES_AHEAD; u++) {
+      const uint32_t t = t0 + (uint32_t)u * BK_THREADS;
+      if (t < T) {
+        s_next[t] = begin[u] + before[u];
+        s_cursor[t] = upto[u] - before[u];  // the workgroup's own instances of the tile
+        s_local[t] = c[u];
+        masked |= c[u] == 0 ? 1 : 0;
+      }
+    }
+  }
+  const bool all_local = __syncthreads_or(masked) == 0;
+  // exclusive prefix of the counts over the tiles, in place: a thread owns `per` consecutive tiles
+  const uint32_t per = (T + BK_THREADS - 1) / BK_THREADS, t_first = threadIdx.x * per;
+  uint32_t own = 0;
+  for (uint32_t k = 0; k < per; k++)
+    if (t_first + k < T) own += s_cursor[t_first + k];
+  const uint32_t own_inc = wave_inclusive_scan_u32(own, lane);
+  // (the prefix sum over the Gaussians' tile counts shares the barrier)
+#pragma unroll
+  for (int q = 0; q < BK_BATCH; q++) sum += tt[q];
+  const uint32_t inc = wave_inclusive_scan_u32(sum, lane);
+  if (lane == GS_WAVE - 1) {
+    s_wave_tiles[wave] = own_inc;
+    s_wave[wave] = inc;
+  }
+  __syncthreads();
+  uint32_t tiles_before = 0, total = 0, before = 0;
+#pragma unroll
+  for (int w = 0; w < BK_THREADS / GS_WAVE; w++) {
+    const uint32_t v = s_wave_tiles[w];
+    if (w < wave) {
+      tiles_before += v;
+      before += s_wave[w];
+    }
+    total += v;
+  }
+  const bool staged = total <= cap;  // (the same for the whole workgroup)
+  {
+    uint32_t run = tiles_before + own_inc - own;
+    for (uint32_t k = 0; k < per; k++)
+      if (t_first + k < T) {
+        const uint32_t v = s_cursor[t_first + k];
+        s_cursor[t_first + k] = staged ? run : s_next[t_first + k];
+        run += v;
+      }
+  }
+  __syncthreads();
+  lds_word* heads = (lds_word*)s_heads + wave * GS_WAVE;
+  struct Owner { uint32_t first, depth_bits, id; };
+  {
+    uint32_t run = block_prefix[chunk] + before + inc - sum;  // emission index of this thread's first instance
+#pragma unroll
+    for (int q = 0; q < BK_BATCH; q++) {
+      const int i = i0 + q;
+      const bool live = i < last && r[q] > 0;
+      const Rect rc = live ? get_rect(p[q].x, p[q].y, r[q], gx, gy) : Rect{0u, 0u, 0u, 0u};
+      const Owner mine = {run, dbits[q], (uint32_t)i};
+      run += tt[q];
+      tt[q] = run;  // from here on: the inclusive sum
+      const auto emit = [&](const Owner& o, uint32_t tile, uint32_t rank) {
+        const uint32_t e = o.first + rank;
+        const uint32_t pos = atomicAdd(&s_cursor[tile], 1u);
+        if (staged) {
+          stage_g[pos] = o.id;
+          stage_e[pos] = e;
+          stage_z[pos] = o.depth_bits;
+        } else {
+          records[pos] = make_uint4(o.id, e, o.depth_bits, 0u);
+        }
+      };
+      if (all_local) walk_wave_rects_flat(live, rc, gx, mine, heads, emit);
+      else walk_wave_rects(live, rc, gx, mine, [&](uint32_t tile) { return s_local[tile] != 0; }, emit);
+    }
+    if (whole) {
+      *reinterpret_cast<uint4*>(point_offsets + i0) = make_uint4(tt[0], tt[1], tt[2], tt[3]);
+    } else {
+#pragma unroll
+      for (int q = 0; q < BK_BATCH; q++)
+        if (i0 + q < last) point_offsets[i0 + q] = tt[q];
+    }
+  }
+  if (!staged) return;
+  __syncthreads();
+  // every tile's run: staged at [cursor of the tile before, cursor of the tile), to memory from s_next on
+  for (uint32_t t = threadIdx.x; t < T; t += BK_THREADS) {
+    const uint32_t lo = t > 0u ? s_cursor[t - 1u] : 0u, hi = s_cursor[t];
+    TileRecord* dst = records + s_next[t];
+    for (uint32_t k = lo; k < hi; k++) dst[k - lo] = make_uint4(stage_g[k], stage_e[k], stage_z[k], 0u);
+  }
+}
+
 // 2. Per-tile sort, register variant: one workgroup of W waves per tile (4 for lists of up to 256 records, 8 up
 // to 2048).  A wave holds 64 E keys, key i = r * 64 + lane in register r of its lane, and the waves hold
 // consecutive runs of 64 E, so a list of up to 64 E W records is sorted with E = 1 .. 4.  In the bitonic network
@@ -706,13 +873,36 @@ int launch_bucket_scatter(int P, int W, int H, const float* means2D, const float
   if (P <= 0) return 0;
   const uint32_t gx = (W + GS_TILE_X - 1) / GS_TILE_X, gy = (H + GS_TILE_Y - 1) / GS_TILE_Y;
   const size_t lds = (size_t)gx * gy * (sizeof(uint32_t) + 1);
+  const int vector_loads = (((uintptr_t)means2D | (uintptr_t)depths | (uintptr_t)tiles_touched |
+                             (uintptr_t)point_offsets | (uintptr_t)radii) & 15u) == 0u ? 1 : 0;
+  // One round per workgroup and room in the LDS for its records: they are staged and leave tile by tile.
+  const size_t tiles_bytes = (size_t)gx * gy * (2 * sizeof(uint32_t) + 1);
+  const size_t lds_room = 150 * 1024;
+  if (bucket_per_block(P) <= BK_BATCH * BK_THREADS && tiles_bytes + 12 * 4096 <= lds_room) {
+    const uint32_t cap = (uint32_t)((lds_room - tiles_bytes) / 12) & ~63u;
+    const uint32_t T = gx * gy;
+    const uint32_t* tab = (const uint32_t*)table;
+    static std::atomic<uint64_t> raised{0};
+    int dev = 0;
+    GS_HIP_TRY(hipGetDevice(&dev));
+    const uint64_t dev_bit = 1ull << (dev & 63);
+    if (dev >= 64 || !(raised.load(std::memory_order_acquire) & dev_bit)) {
+      GS_HIP_TRY(hipFuncSetAttribute((const void*)bucket_scatter_staged_kernel,
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_room));
+      raised.fetch_or(dev_bit, std::memory_order_release);
+    }
+    hipLaunchKernelGGL(bucket_scatter_staged_kernel, dim3(bucket_blocks(P)), dim3(BK_THREADS),
+                       tiles_bytes + (size_t)cap * 12, stream, P, bucket_per_block(P), bucket_blocks(P), gx, gy,
+                       (const float2*)means2D, depths, tiles_touched, bucket_block_sums(table, T), point_offsets, radii,
+                       compute_locally, tab, tab + (size_t)BK_MAX_BLOCKS * T, ranges, (TileRecord*)records,
+                       ahead_of_host ? bucket_fits_word(table, (int)T) : nullptr, vector_loads, cap);
+    return 0;
+  }
   hipLaunchKernelGGL(bucket_scatter_kernel, dim3(bucket_blocks(P)), dim3(BK_THREADS), lds, stream, P,
                      bucket_per_block(P), gx, gy, (const float2*)means2D, depths, tiles_touched,
                      bucket_block_sums(table, gx * gy), point_offsets, radii, compute_locally, (const uint32_t*)table,
                      ranges, (TileRecord*)records,
-                     ahead_of_host ? bucket_fits_word(table, (int)(gx * gy)) : nullptr,
-                     (((uintptr_t)means2D | (uintptr_t)depths | (uintptr_t)tiles_touched | (uintptr_t)point_offsets |
-                       (uintptr_t)radii) & 15u) == 0u ? 1 : 0);
+                     ahead_of_host ? bucket_fits_word(table, (int)(gx * gy)) : nullptr, vector_loads);
   return 0;
 }
 
