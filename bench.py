@@ -59,7 +59,8 @@ BINNING_REFERENCE_BYTES = (44, 172)   # per Gaussian, per instance
 BINNING_OWN_BYTES = (44, 48)
 BINNING_STAGES = ("tile_count", "inclusive_sum", "bucket_scatter", "tile_sort", "duplicate_with_keys",
                   "identify_tile_ranges")
-BINNING_KERNELS = ("bucket_count_kernel", "bucket_columns_kernel", "bucket_ranges_kernel", "bucket_scatter_kernel",
+BINNING_KERNELS = ("bucket_count_kernel", "bucket_columns_kernel", "bucket_ranges_kernel",
+                   "bucket_scatter_staged_kernel",  # (bucket_scatter_kernel beyond one round per workgroup)
                    "tile_sort_registers_kernel")  # (views with lists above 2048 records: + tile_radix_sort_kernel)
 FP32_MATRIX_PEAK_TFLOPS = 157.3
 # Neural-Gaussian generation with 10 offsets: (bytes per anchor, bytes per selected Gaussian, flops per anchor).
